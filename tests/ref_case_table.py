@@ -1,0 +1,48 @@
+"""The operator cases oracle/ref_driver.cpp emits through the reference's own lowering and
+C code generator, with seeded inputs and the oracle composition each one must equal bit for bit.
+
+Each entry: name -> (input shapes in parameter order, function(oracle, inputs) -> expected output).
+"""
+import importlib
+
+import numpy as np
+
+synth = importlib.import_module("hdkx-aicompiler_amd.synth")
+
+
+def _conv(stride, pad, bias, relu):
+    def f(o, ins):
+        return o.conv_chain(ins[0], ins[1], ins[2] if bias else None, stride, pad, None, relu)
+    return f
+
+
+CASES = {
+    "kxc_ref_conv_cfg1": ([(1, 64, 56, 56), (64, 64, 3, 3), (64,)], _conv(1, 1, True, True)),
+    "kxc_ref_conv7x7s2": ([(2, 3, 32, 32), (16, 3, 7, 7), (16,)], _conv(2, 3, True, True)),
+    "kxc_ref_conv3x3s1": ([(2, 8, 14, 14), (16, 8, 3, 3), (16,)], _conv(1, 1, True, True)),
+    "kxc_ref_conv3x3s2": ([(2, 8, 14, 14), (16, 8, 3, 3), (16,)], _conv(2, 1, True, True)),
+    "kxc_ref_conv1x1s2": ([(2, 8, 14, 14), (16, 8, 1, 1), (16,)], _conv(2, 0, True, False)),
+    "kxc_ref_conv_nobias": ([(1, 4, 9, 11), (5, 4, 3, 3)], _conv(1, 1, False, False)),
+    "kxc_ref_conv_add_relu": ([(2, 8, 14, 14), (8, 8, 3, 3), (8,), (2, 8, 14, 14)],
+                              lambda o, i: o.conv_chain(i[0], i[1], i[2], 1, 1, i[3], True)),
+    "kxc_ref_maxpool3x3s2": ([(2, 4, 16, 16)], lambda o, i: o.pool2d(i[0], 3, 2, 1)),
+    "kxc_ref_maxpool_ceil": ([(1, 2, 7, 9)], lambda o, i: o.pool2d(i[0], 3, 2, 1, ceil_mode=True)),
+    "kxc_ref_avgpool3x3s2": ([(2, 4, 16, 16)], lambda o, i: o.pool2d(i[0], 3, 2, 1, avg=True)),
+    "kxc_ref_gap7x7": ([(4, 32, 7, 7)], lambda o, i: o.gap(i[0])),
+    "kxc_ref_add_relu": ([(4, 16, 7, 7), (4, 16, 7, 7)], lambda o, i: o.relu(o.add(i[0], i[1]))),
+    "kxc_ref_add_bcast": ([(2, 3, 4), (3, 1)], lambda o, i: o.add(i[0], i[1])),
+    "kxc_ref_dense": ([(8, 64), (40, 64)], lambda o, i: o.dense(i[0], i[1])),
+    "kxc_ref_gemm_fc": ([(8, 64), (40, 64), (40,)], lambda o, i: o.gemm(i[0], i[1], i[2], 1.0, 1.0, 1)),
+    "kxc_ref_gemm_ab": ([(4, 10), (10, 6), (6,)], lambda o, i: o.gemm(i[0], i[1], i[2], 0.5, 2.0, 0)),
+    "kxc_ref_head": ([(4, 32, 7, 7), (10, 32), (10,)],
+                     lambda o, i: o.gemm(o.gap(i[0]).reshape(4, 32), i[1], i[2], 1.0, 1.0, 1)),
+}
+
+
+def case_inputs(name):
+    shapes, _ = CASES[name]
+    base = 7000 + 10 * sorted(CASES).index(name)
+    if name == "kxc_ref_conv_cfg1":  # BASELINE configuration 1, seeds 1000..1002
+        return [synth.uniform(shapes[0], 1000), synth.normal(shapes[1], 1001, float(np.sqrt(2.0 / 576))),
+                synth.uniform(shapes[2], 1002, -0.1, 0.1)]
+    return [synth.uniform(s, base + t) for t, s in enumerate(shapes)]
