@@ -1,0 +1,229 @@
+#!/usr/bin/env python3
+"""Benchmark of the lowered-operator hot path on one MI355X.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--no-cpu] [--ops]
+
+A step is one forward pass of the ResNet-18 launch plan (fp32, batch 64, [64,3,224,224] input,
+seeded synthetic weights/input already resident in HBM) enqueued on one stream through the C ABI.
+Prints ONE JSON line: whole-job throughput (img/s), the roofline position of the dominant kernel
+(the 3x3/1 convolution of layer1, timed with events on the launch stream), per-layer and
+per-operator figures, and the single-core CPU baseline (the CPU checker in oracle/, timed on a
+bounded sample: one image).
+"""
+import argparse
+import importlib
+import json
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
+
+PEAK_FP32_MFMA_TFLOPS = 157.3
+PEAK_HBM_GBS = 8000.0
+
+
+def _event_time_ms(torch, fn, iters, warmup):
+    """Average duration of fn() in ms, HIP events recorded on the stream fn launches on."""
+    for _ in range(warmup):
+        fn()
+    torch.cuda.synchronize()
+    start = torch.cuda.Event(enable_timing=True)
+    stop = torch.cuda.Event(enable_timing=True)
+    start.record()
+    for _ in range(iters):
+        fn()
+    stop.record()
+    torch.cuda.synchronize()
+    return start.elapsed_time(stop) / iters
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=20)
+    ap.add_argument("--warmup", type=int, default=5)
+    ap.add_argument("--batch", type=int, default=64)
+    ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
+    ap.add_argument("--no-layers", action="store_true", help="skip the per-layer / per-operator timings")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        print("bench.py: this build runs on exactly one GPU (no collectives, no sharding); "
+              "--gpus %d is not supported" % args.gpus, file=sys.stderr)
+        sys.exit(2)
+
+    import numpy as np
+    import torch
+    pkg = importlib.import_module("hdkx-aicompiler_amd")
+    r18 = importlib.import_module("hdkx-aicompiler_amd.resnet18")
+    synth = pkg.synth
+    if not torch.cuda.is_available():
+        print("bench.py: no GPU visible", file=sys.stderr)
+        sys.exit(3)
+    torch.cuda.set_device(0)
+    attrs = pkg.device_attributes(0)
+    dev = lambda a: torch.from_numpy(np.ascontiguousarray(a)).cuda()
+
+    batch = args.batch
+    consts_h = synth.resnet18_consts(4)
+    x_h = synth.resnet18_input(4, batch)
+    consts = [dev(c) for c in consts_h]
+    x = dev(x_h)
+    out = torch.empty((batch, 1000), device="cuda")
+    plan, info = r18.build_plan(batch, 224)
+    tensors = [x] + consts + [out]
+    packed = plan.packed(tensors)
+    stream = torch.cuda.current_stream().cuda_stream
+
+    def step():
+        plan.run_packed(packed, stream)
+
+    for _ in range(args.warmup):
+        step()
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(args.steps):
+        step()
+    torch.cuda.synchronize()
+    t1 = time.perf_counter()
+    ms_per_step = (t1 - t0) * 1e3 / args.steps
+    img_s = batch / (ms_per_step * 1e-3)
+    flop_step = r18.flops_per_image() * batch
+    logits_ok = bool(torch.isfinite(out).all().item())
+
+    # ---- dominant kernel: layer1 3x3/1 conv, [64,64,56,56] * [64,64,3,3], fused bias + ReLU
+    lx = dev(synth.uniform((batch, 64, 56, 56), 4100))
+    lw = dev(synth.normal((64, 64, 3, 3), 4101, float(np.sqrt(2.0 / 576))))
+    lb = dev(synth.uniform((64,), 4103, -0.1, 0.1))
+    ly = torch.empty((batch, 64, 56, 56), device="cuda")
+    conv_ms = _event_time_ms(torch, lambda: pkg.conv2d(lx, lw, lb, None, 1, 1, 1, True, out=ly), 30, 5)
+    conv_flop = 2.0 * batch * 64 * 56 * 56 * 64 * 9
+    conv_tflops = conv_flop / (conv_ms * 1e-3) / 1e12
+    roofline = {"bound": "mfma", "kernel": "conv_mfma_kernel<3,3> (layer1: [%d,64,56,56]x[64,64,3,3] s1 p1 +bias+relu)" % batch,
+                "variant": pkg.conv2d_variant((batch, 64, 56, 56), (64, 64, 3, 3), 1, 1),
+                "achieved": round(conv_tflops, 3), "peak": PEAK_FP32_MFMA_TFLOPS, "unit": "TFLOP/s",
+                "frac": round(conv_tflops / PEAK_FP32_MFMA_TFLOPS, 4), "avg_launch_ms": round(conv_ms, 4),
+                "flop_per_launch": conv_flop, "traffic": None}
+
+    result = {
+        "metric": "resnet18_fp32_bs64_img_per_s", "value": round(img_s, 2), "unit": "img/s",
+        "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "ms_per_step": round(ms_per_step, 4),
+        "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "f32", "data": "synthetic",
+        "config": {"workload": "ResNet-18 fp32 inference, batch %d, input [%d,3,224,224], BN folded, seeded Kaiming weights "
+                               "(BASELINE configs[3])" % (batch, batch),
+                   "launches_per_step": len(info["launches"]), "workspace_bytes": info["workspace_bytes"]},
+        "end_to_end_tflops": round(flop_step / (ms_per_step * 1e-3) / 1e12, 3),
+        "end_to_end_frac_of_fp32_mfma_peak": round(flop_step / (ms_per_step * 1e-3) / 1e12 / PEAK_FP32_MFMA_TFLOPS, 4),
+        "logits_finite": logits_ok,
+        "device": {"name": attrs.device_name.decode(), "arch": attrs.arch.decode(), "cus": int(attrs.multi_processor_count),
+                   "clock_khz": int(attrs.max_clock_rate_khz)},
+        "roofline": roofline,
+    }
+
+    if not args.no_layers:
+        result["conv_layers"] = bench_conv_layers(torch, pkg, synth, dev, batch)
+        result["ops"] = bench_ops(torch, pkg, synth, dev)
+        result["resnet18_bs1_img_per_s"] = bench_batch1(torch, pkg, r18, synth, dev)
+
+    if not args.no_cpu:
+        result["cpu_baseline"] = cpu_baseline(np, synth)
+        result["gpu_over_cpu"] = round(img_s / result["cpu_baseline"]["value"], 1)
+    print(json.dumps(result))
+
+
+CONV_LAYERS = [  # name, C, H, O, k, s, p, count per network, residual
+    ("conv1", 3, 224, 64, 7, 2, 3, 1, False),
+    ("layer1.3x3", 64, 56, 64, 3, 1, 1, 4, False),
+    ("layer2.0.conv1", 64, 56, 128, 3, 2, 1, 1, False),
+    ("layer2.3x3", 128, 28, 128, 3, 1, 1, 3, True),
+    ("layer2.0.down", 64, 56, 128, 1, 2, 0, 1, False),
+    ("layer3.0.conv1", 128, 28, 256, 3, 2, 1, 1, False),
+    ("layer3.3x3", 256, 14, 256, 3, 1, 1, 3, True),
+    ("layer3.0.down", 128, 28, 256, 1, 2, 0, 1, False),
+    ("layer4.0.conv1", 256, 14, 512, 3, 2, 1, 1, False),
+    ("layer4.3x3", 512, 7, 512, 3, 1, 1, 3, True),
+    ("layer4.0.down", 256, 14, 512, 1, 2, 0, 1, False),
+]
+
+
+def bench_conv_layers(torch, pkg, synth, dev, batch):
+    rows = []
+    for i, (name, c, h, o, k, s, p, count, res) in enumerate(CONV_LAYERS):
+        x = dev(synth.uniform((batch, c, h, h), 4200 + i))
+        w = dev(synth.normal((o, c, k, k), 4300 + i, float((2.0 / (c * k * k)) ** 0.5)))
+        b = dev(synth.uniform((o,), 4400 + i, -0.1, 0.1))
+        oh = (h + 2 * p - k) // s + 1
+        y = torch.empty((batch, o, oh, oh), device="cuda")
+        skip = torch.zeros_like(y) if res else None
+        ms = _event_time_ms(torch, lambda: pkg.conv2d(x, w, b, skip, s, p, 1, True, out=y), 20, 3)
+        flop = 2.0 * batch * o * oh * oh * c * k * k
+        rows.append({"layer": name, "variant": pkg.conv2d_variant((batch, c, h, h), (o, c, k, k), s, p), "count": count,
+                     "ms": round(ms, 4), "tflops": round(flop / (ms * 1e-3) / 1e12, 2),
+                     "frac_fp32_mfma_peak": round(flop / (ms * 1e-3) / 1e12 / PEAK_FP32_MFMA_TFLOPS, 4)})
+    return rows
+
+
+def bench_ops(torch, pkg, synth, dev):
+    """BASELINE configs[1]: the bandwidth-bound operators at ResNet-18 shapes, algorithmic bytes / time."""
+    rows = []
+    x = dev(synth.uniform((64, 64, 112, 112), 2000))
+    y = torch.empty((64, 64, 56, 56), device="cuda")
+    ms = _event_time_ms(torch, lambda: pkg.pool2d(x, 3, 2, 1, out=y), 30, 5)
+    rows.append(_bw_row("maxpool3x3s2 [64,64,112,112]", 256901120, ms))
+    del x, y
+    a = dev(synth.uniform((64, 128, 28, 28), 2010)); b = dev(synth.uniform((64, 128, 28, 28), 2011))
+    ms = _event_time_ms(torch, lambda: pkg.binary(0, a, b, relu=True), 30, 5)
+    rows.append(_bw_row("add+relu [64,128,28,28]", 77070336, ms))
+    g = dev(synth.uniform((64, 512, 7, 7), 2020))
+    ms = _event_time_ms(torch, lambda: pkg.global_avg_pool2d(g), 30, 5)
+    rows.append(_bw_row("global_avg_pool [64,512,7,7]", 6553600, ms))
+    fa = dev(synth.uniform((64, 512), 2030)); fw = dev(synth.uniform((1000, 512), 2031)); fb = dev(synth.uniform((1000,), 2032))
+    ms = _event_time_ms(torch, lambda: pkg.gemm(fa, fw, fb), 30, 5)
+    rows.append({"op": "dense [64,512]x[1000,512]T+bias", "ms": round(ms, 4), "gflops": round(65536000 / (ms * 1e-3) / 1e9, 1),
+                 "gbs": round(2439072 / (ms * 1e-3) / 1e9, 1)})
+    # a plain device-to-device copy of the max-pool input size, as the achievable-bandwidth yardstick
+    src = torch.empty(205520896 // 4, device="cuda"); dst = torch.empty_like(src)
+    ms = _event_time_ms(torch, lambda: dst.copy_(src), 20, 3)
+    rows.append(_bw_row("copy 205.5 MB (yardstick, read+write)", 2 * 205520896, ms))
+    return rows
+
+
+def _bw_row(name, nbytes, ms):
+    gbs = nbytes / (ms * 1e-3) / 1e9
+    return {"op": name, "ms": round(ms, 4), "gbs": round(gbs, 1), "frac_hbm_peak": round(gbs / PEAK_HBM_GBS, 4)}
+
+
+def bench_batch1(torch, pkg, r18, synth, dev):
+    consts = [dev(c) for c in synth.resnet18_consts(3)]
+    x = dev(synth.resnet18_input(3, 1))
+    out = torch.empty((1, 1000), device="cuda")
+    plan, _ = r18.build_plan(1, 224)
+    packed = plan.packed([x] + consts + [out])
+    stream = torch.cuda.current_stream().cuda_stream
+    ms = _event_time_ms(torch, lambda: plan.run_packed(packed, stream), 50, 10)
+    plan.close()
+    return {"value": round(1e3 / ms, 1), "ms_per_image": round(ms, 4)}
+
+
+def cpu_baseline(np, synth):
+    """The CPU checker (oracle/, -O3, strict fp32) on one core: ResNet-18 forward of ONE image."""
+    sys.path.insert(0, os.path.join(ROOT, "tests"))
+    from oracle_lib import Oracle
+    orc = Oracle(fast=True)
+    consts = synth.resnet18_consts(4)
+    x = synth.resnet18_input(4, 1)
+    times = []
+    for _ in range(3):
+        t0 = time.perf_counter()
+        orc.resnet18(x, consts)
+        times.append(time.perf_counter() - t0)
+    t = sorted(times)[1]
+    return {"value": round(1.0 / t, 4), "unit": "img/s", "cores": 1, "kind": "port",
+            "sample": "ResNet-18 fp32 forward of 1 image (first image of the batch), median of 3 runs, "
+                      "gcc -O3 -march=native -ffp-contract=off",
+            "seconds_per_image": round(t, 3), "host_cpus": os.cpu_count()}
+
+
+if __name__ == "__main__":
+    main()

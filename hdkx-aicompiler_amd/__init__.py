@@ -1,0 +1,16 @@
+"""MI355X (gfx950) backend for the kxc compiler's lowered-operator hot path.
+
+The product is the C-ABI library ``lib/libkxc_hip.so`` (declared in ``include/kxc_hip.h``) and the
+C++ host layer in ``host/``.  This Python package is a thin ctypes binding of that ABI, used by the
+tests and the benchmark; PyTorch appears only as a provider of device memory and streams.
+
+The directory name carries a hyphen, so import it with
+``importlib.import_module("hdkx-aicompiler_amd")``.
+"""
+from . import synth  # noqa: F401
+from .hipabi import (  # noqa: F401
+    KxcHipError, lib, library_path, conv2d, relu, binary, bias_add, pool2d, global_avg_pool2d, gemm,
+    flatten, quantize, qconv2d, qdense, maxpool2d_i8, global_avg_pool2d_i8, conv2d_variant,
+    device_attributes, Plan, Buf, ConvDesc, PoolDesc, QConvDesc,
+    CONV_BIAS, CONV_RESIDUAL, CONV_RELU, CONV_FORCE_DIRECT,
+)

@@ -1,0 +1,57 @@
+"""Builds libkxc_hip.so (the C-ABI library of hand-written gfx950 kernels) with hipcc.
+
+Usage: python build.py            (from anywhere; output goes to <package>/lib/libkxc_hip.so)
+The benchmark, tests and smoke check load the built library and only call this when it is missing;
+__graft_entry__.build() always calls it.
+"""
+import concurrent.futures
+import os
+import subprocess
+import sys
+
+PKG = os.path.dirname(os.path.abspath(__file__))
+ROOT = os.path.dirname(PKG)
+CSRC = os.path.join(PKG, "csrc")
+LIBDIR = os.path.join(PKG, "lib")
+OBJDIR = os.path.join(PKG, "build")
+LIB = os.path.join(LIBDIR, "libkxc_hip.so")
+
+SOURCES = ["device_api.hip", "eltwise.hip", "pool.hip", "gemm.hip", "conv2d_f32.hip", "qconv_i8.hip",
+           "module.hip", "plan.hip"]
+
+HIPCC = os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")
+FLAGS = ["-O3", "--offload-arch=gfx950", "-fPIC", "-std=c++17", "-I" + os.path.join(ROOT, "include"),
+         # packed fp32 instructions are kept out of every kernel
+         "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
+         "-Wall", "-Wno-unused-function"]
+
+
+def _compile(src):
+    obj = os.path.join(OBJDIR, src.replace(".hip", ".o"))
+    cmd = [HIPCC] + FLAGS + ["-c", os.path.join(CSRC, src), "-o", obj]
+    r = subprocess.run(cmd, capture_output=True, text=True)
+    err = "\n".join(l for l in r.stderr.splitlines() if "packed-fp32-ops" not in l)
+    if r.returncode != 0:
+        raise RuntimeError("hipcc failed for %s:\n%s" % (src, err))
+    return obj, err
+
+
+def build(verbose=True):
+    os.makedirs(LIBDIR, exist_ok=True)
+    os.makedirs(OBJDIR, exist_ok=True)
+    with concurrent.futures.ThreadPoolExecutor(max_workers=8) as ex:
+        results = list(ex.map(_compile, SOURCES))
+    for obj, err in results:
+        if verbose and err.strip():
+            print(err, file=sys.stderr)
+    cmd = [HIPCC, "--offload-arch=gfx950", "-shared", "-fPIC", "-o", LIB] + [o for o, _ in results] + ["-lhiprtc"]
+    r = subprocess.run(cmd, capture_output=True, text=True)
+    if r.returncode != 0:
+        raise RuntimeError("link failed:\n" + r.stderr)
+    if verbose:
+        print("built", LIB)
+    return LIB
+
+
+if __name__ == "__main__":
+    build()

@@ -1,0 +1,57 @@
+// common.h -- shared host-side helpers of libkxc_hip.so (error reporting, stream resolution).
+#pragma once
+
+#include <hip/hip_runtime.h>
+
+#include <cstdarg>
+#include <cstdint>
+#include <cstdio>
+#include <string>
+
+#include "kxc_hip.h"
+
+namespace kxc_hip {
+
+// Per-thread message of the last failure (returned by kxc_hip_last_error).
+std::string& LastError();
+// Per-thread current stream (DeviceAPI::SetStream semantics: thread local).
+hipStream_t& CurrentStream();
+
+inline int32_t Fail(int32_t code, const char* fmt, ...) {
+    char buf[1024];
+    va_list ap;
+    va_start(ap, fmt);
+    vsnprintf(buf, sizeof(buf), fmt, ap);
+    va_end(ap);
+    LastError() = buf;
+    return code;
+}
+
+inline hipStream_t ResolveStream(void* stream) {
+    return stream ? reinterpret_cast<hipStream_t>(stream) : CurrentStream();
+}
+
+// Launch-error check: hipGetLastError after a triple-chevron launch.
+inline int32_t CheckLaunch(const char* what) {
+    hipError_t e = hipGetLastError();
+    if (e != hipSuccess) return Fail(KXC_HIP_ERR_RUNTIME, "%s launch failed: %s", what, hipGetErrorString(e));
+    return KXC_HIP_OK;
+}
+
+constexpr int64_t kMaxGridX = 2147483647LL;
+
+inline int64_t CeilDiv(int64_t a, int64_t b) { return (a + b - 1) / b; }
+
+}  // namespace kxc_hip
+
+#define KXC_HIP_CALL(expr, what)                                                              \
+    do {                                                                                      \
+        hipError_t _e = (expr);                                                               \
+        if (_e != hipSuccess)                                                                 \
+            return ::kxc_hip::Fail(KXC_HIP_ERR_RUNTIME, "%s failed: %s", what, hipGetErrorString(_e)); \
+    } while (0)
+
+#define KXC_HIP_REQUIRE(cond, ...)                                              \
+    do {                                                                        \
+        if (!(cond)) return ::kxc_hip::Fail(KXC_HIP_ERR_INVALID, __VA_ARGS__);  \
+    } while (0)

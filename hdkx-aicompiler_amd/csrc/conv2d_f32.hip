@@ -1,0 +1,444 @@
+// conv2d_f32.hip -- nn_conv2d (NCHW data, OIHW weights, fp32) for gfx950.
+//
+// Two kernels behind one entry point:
+//
+//  * conv_mfma_kernel: implicit GEMM on the fp32 matrix cores (v_mfma_f32_32x32x2_f32),
+//    D[o][pixel] += W[o][k] * X[k][pixel], k = (channel, rh, rw).
+//      - Output pixels are flattened over (n, oh, ow); a workgroup owns TO output channels by TP
+//        consecutive pixels.  The weights are the MFMA "A" operand and the pixels the "B"
+//        operand, so the 32 lanes of a half-wave hold 32 consecutive pixels of ONE output
+//        channel: NCHW stores (and residual loads) are 128-byte contiguous runs.
+//      - The input is NOT expanded to an im2col matrix.  For each chunk of CC input channels the
+//        workgroup stages the raw input rows its pixels touch (with the zero padding
+//        materialised) in LDS as patch[channel][padded_row][padded_col]; the operand for tap
+//        (rh, rw) is the same patch read at a shifted address, so every input element is
+//        fetched from memory once per workgroup instead of KH*KW times.  Rows are addressed in
+//        "padded row space" Q = n*(H+2*pad_h) + ih + pad_h, which makes a tile that crosses
+//        image boundaries (7x7 and 14x14 feature maps) just a longer run of rows.
+//      - One MFMA consumes two k values, one per half-wave.  They are chosen as the SAME tap of
+//        two adjacent channels, so a lane's LDS address is (per-lane base) + (uniform offset)
+//        for both operands; the reduction order differs from the CPU loop only in that way and
+//        in the blocking of channels, which is what the 1e-3 tolerance is for.
+//      - Chunks are double buffered: the next chunk's global loads are issued before the MFMA
+//        loop over the current one and written to the other LDS buffer after it.
+//      - The epilogue adds bias, the residual operand, and applies ReLU, each as one rounded
+//        fp32 operation in the order of the unfused operator chain.
+//
+//  * conv_direct_kernel: one thread per output element, the CPU loop nest's exact order
+//    (rc, rh, rw ascending from 0.0f, multiply and add rounded separately, padded taps add
+//    0.0f * w).  Bit-identical to the CPU backend; used for shapes the MFMA tiling does not
+//    cover (output channels not a multiple of 32, very wide rows) and on request.
+#include <cstdlib>
+#include <cstring>
+
+#include "common.h"
+
+using namespace kxc_hip;
+
+namespace {
+
+typedef float floatx16 __attribute__((ext_vector_type(16)));
+
+struct ConvArgs {
+    const float* x;
+    const float* w;
+    const float* bias;
+    const float* res;
+    float* y;
+    int32_t N, C, H, W, O, OH, OW;
+    int32_t sh, sw, ph, pw, dh, dw;
+    int32_t Hp, Wp;      // padded input extent: H + 2*ph, W + 2*pw
+    int32_t M;           // N*OH*OW output pixels
+    int32_t OHW;
+    int32_t chs;         // LDS floats per patch channel (>= rows*Wp, padded)
+    int32_t nchunks;     // ceil(C / CC)
+    uint32_t flags;
+};
+
+__device__ __forceinline__ float relu_sel(float v) { return (v > 0.0f) ? v : 0.0f; }
+
+// ------------------------------------------------------------------------------------------
+// MFMA kernel.  KH,KW: filter; CC: channels per LDS chunk (even); WO x WP waves, each wave
+// RO x RP blocks of 32x32; PPT: patch positions per thread (upper bound, checked on the host).
+// ------------------------------------------------------------------------------------------
+template <int KH, int KW, int CC, int WO, int WP, int RO, int RP, int PPT>
+__global__ void __launch_bounds__(64 * WO * WP)
+conv_mfma_kernel(const ConvArgs a) {
+    constexpr int NT = 64 * WO * WP;
+    constexpr int TO = 32 * RO * WO;
+    constexpr int TP = 32 * RP * WP;
+    constexpr int KHW = KH * KW;
+    constexpr int KC = CC * KHW;                 // k values per chunk
+    constexpr int KS = KC | 1;                   // odd LDS row stride for the weight tile
+    constexpr int WPT = (TO * KC + NT - 1) / NT; // weight elements per thread per chunk
+
+    extern __shared__ float lds[];
+    const int xs_size = CC * a.chs;
+    float* xs0 = lds;
+    // layout: [xs0][ws0][xs1][ws1]; the second pair exists only when there is more than one chunk
+    float* xs1 = lds + xs_size + TO * KS;
+    float* ws0 = lds + xs_size;
+    float* ws1 = xs1 + xs_size;
+
+    const int tid = threadIdx.x;
+    const int lane = tid & 63;
+    const int wave = tid >> 6;
+    const int wave_o = wave / WP;
+    const int wave_p = wave % WP;
+    const int half = lane >> 5;
+    const int r = lane & 31;
+
+    // blockIdx.x walks pixel tiles fastest so that concurrently resident workgroups share weights.
+    const int m0 = blockIdx.x * TP;
+    const int o0 = blockIdx.y * TO;
+
+    // ---- geometry of this tile in padded row space
+    const int m_last = min(m0 + TP, a.M) - 1;
+    int qmin, qlast;
+    {
+        const int n = m0 / a.OHW, rem = m0 - n * a.OHW;
+        qmin = n * a.Hp + (rem / a.OW) * a.sh;
+        const int n2 = m_last / a.OHW, rem2 = m_last - n2 * a.OHW;
+        qlast = n2 * a.Hp + (rem2 / a.OW) * a.sh + (KH - 1) * a.dh;
+    }
+    const int P = (qlast - qmin + 1) * a.Wp;      // patch positions per channel (<= chs, <= PPT*NT)
+    const int HW = a.H * a.W;
+
+    // ---- per-thread patch positions: global offset inside channel 0 (or -1 for padding)
+    int goff[PPT];
+#pragma unroll
+    for (int i = 0; i < PPT; ++i) {
+        const int pos = tid + i * NT;
+        const int q = pos / a.Wp, col = pos - q * a.Wp;
+        const int Q = qmin + q;
+        const int n = Q / a.Hp, ih = Q - n * a.Hp - a.ph, iw = col - a.pw;
+        const bool ok = pos < P && n < a.N && ih >= 0 && ih < a.H && iw >= 0 && iw < a.W;
+        goff[i] = ok ? ((n * a.C) * a.H + ih) * a.W + iw : -1;
+    }
+
+    // ---- per-lane operand bases
+    int xbase[RP];
+    int ybase[RP];      // offset of (n, o=0, oh, ow) in y, or -1 when the pixel is past the end
+#pragma unroll
+    for (int j = 0; j < RP; ++j) {
+        const int m = m0 + (wave_p * RP + j) * 32 + r;
+        const int mc = min(m, a.M - 1);
+        const int n = mc / a.OHW, rem = mc - n * a.OHW;
+        const int oh = rem / a.OW, ow = rem - oh * a.OW;
+        xbase[j] = (n * a.Hp + oh * a.sh - qmin) * a.Wp + ow * a.sw + half * a.chs;
+        ybase[j] = (m < a.M) ? n * a.O * a.OHW + rem : -1;
+    }
+    int wbase[RO];
+#pragma unroll
+    for (int i = 0; i < RO; ++i) wbase[i] = ((wave_o * RO + i) * 32 + r) * KS + half * KHW;
+
+    floatx16 acc[RO][RP];
+#pragma unroll
+    for (int i = 0; i < RO; ++i)
+#pragma unroll
+        for (int j = 0; j < RP; ++j)
+#pragma unroll
+            for (int g = 0; g < 16; ++g) acc[i][j][g] = 0.0f;
+
+    float xreg[CC][PPT];
+    float wreg[WPT];
+
+    auto load_chunk = [&](int chunk) {
+        const int c0 = chunk * CC;
+#pragma unroll
+        for (int cl = 0; cl < CC; ++cl) {
+            const bool cok = (c0 + cl) < a.C;
+#pragma unroll
+            for (int i = 0; i < PPT; ++i)
+                xreg[cl][i] = (cok && goff[i] >= 0) ? a.x[goff[i] + (c0 + cl) * HW] : 0.0f;
+        }
+#pragma unroll
+        for (int i = 0; i < WPT; ++i) {
+            const int e = tid + i * NT;
+            const int ol = e / KC, kk = e - ol * KC;
+            const int cl = kk / KHW;
+            const bool ok = e < TO * KC && (o0 + ol) < a.O && (c0 + cl) < a.C;
+            wreg[i] = ok ? a.w[((o0 + ol) * a.C + c0) * KHW + kk] : 0.0f;
+        }
+    };
+    auto store_chunk = [&](float* xs, float* ws) {
+#pragma unroll
+        for (int cl = 0; cl < CC; ++cl)
+#pragma unroll
+            for (int i = 0; i < PPT; ++i) {
+                const int pos = tid + i * NT;
+                if (pos < P) xs[cl * a.chs + pos] = xreg[cl][i];
+            }
+#pragma unroll
+        for (int i = 0; i < WPT; ++i) {
+            const int e = tid + i * NT;
+            const int ol = e / KC, kk = e - ol * KC;
+            if (e < TO * KC) ws[ol * KS + kk] = wreg[i];
+        }
+    };
+
+    load_chunk(0);
+    store_chunk(xs0, ws0);
+    __syncthreads();
+
+    for (int chunk = 0; chunk < a.nchunks; ++chunk) {
+        const float* xs = (chunk & 1) ? xs1 : xs0;
+        const float* ws = (chunk & 1) ? ws1 : ws0;
+        const bool more = (chunk + 1) < a.nchunks;
+        if (more) load_chunk(chunk + 1);
+
+#pragma unroll
+        for (int cp = 0; cp < CC / 2; ++cp) {
+#pragma unroll
+            for (int rh = 0; rh < KH; ++rh) {
+#pragma unroll
+                for (int rw = 0; rw < KW; ++rw) {
+                    const int koff_x = (2 * cp) * a.chs + rh * a.dh * a.Wp + rw * a.dw;
+                    const int koff_w = (2 * cp) * KHW + rh * KW + rw;
+                    float av[RO], bv[RP];
+#pragma unroll
+                    for (int i = 0; i < RO; ++i) av[i] = ws[wbase[i] + koff_w];
+#pragma unroll
+                    for (int j = 0; j < RP; ++j) bv[j] = xs[xbase[j] + koff_x];
+#pragma unroll
+                    for (int i = 0; i < RO; ++i)
+#pragma unroll
+                        for (int j = 0; j < RP; ++j)
+                            acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x2f32(av[i], bv[j], acc[i][j], 0, 0, 0);
+                }
+            }
+        }
+
+        if (more) store_chunk((chunk & 1) ? xs0 : xs1, (chunk & 1) ? ws0 : ws1);
+        __syncthreads();
+    }
+
+    // ---- epilogue: accumulator register g of a block holds row 8*(g/4) + 4*half + g%4, column r
+    const bool has_bias = (a.flags & KXC_HIP_CONV_BIAS) != 0;
+    const bool has_res = (a.flags & KXC_HIP_CONV_RESIDUAL) != 0;
+    const bool do_relu = (a.flags & KXC_HIP_CONV_RELU) != 0;
+#pragma unroll
+    for (int i = 0; i < RO; ++i) {
+#pragma unroll
+        for (int g = 0; g < 16; ++g) {
+            const int o = o0 + (wave_o * RO + i) * 32 + 8 * (g / 4) + 4 * half + (g % 4);
+            if (o >= a.O) continue;
+            const float bval = has_bias ? a.bias[o] : 0.0f;
+#pragma unroll
+            for (int j = 0; j < RP; ++j) {
+                if (ybase[j] < 0) continue;
+                const int off = ybase[j] + o * a.OHW;
+                float v = acc[i][j][g];
+                if (has_bias) v = __fadd_rn(v, bval);
+                if (has_res) v = __fadd_rn(v, a.res[off]);
+                if (do_relu) v = relu_sel(v);
+                a.y[off] = v;
+            }
+        }
+    }
+}
+
+// ------------------------------------------------------------------------------------------
+// Direct kernel: the CPU loop nest, one thread per output element.
+// ------------------------------------------------------------------------------------------
+__global__ void __launch_bounds__(256) conv_direct_kernel(const ConvArgs a, int32_t KH, int32_t KW, int64_t total) {
+    const int64_t stride = static_cast<int64_t>(gridDim.x) * 256;
+    const bool has_bias = (a.flags & KXC_HIP_CONV_BIAS) != 0;
+    const bool has_res = (a.flags & KXC_HIP_CONV_RESIDUAL) != 0;
+    const bool do_relu = (a.flags & KXC_HIP_CONV_RELU) != 0;
+    for (int64_t e = static_cast<int64_t>(blockIdx.x) * 256 + threadIdx.x; e < total; e += stride) {
+        const int32_t ow = static_cast<int32_t>(e % a.OW);
+        int64_t t = e / a.OW;
+        const int32_t oh = static_cast<int32_t>(t % a.OH);
+        t /= a.OH;
+        const int32_t o = static_cast<int32_t>(t % a.O);
+        const int64_t n = t / a.O;
+        const float* xn = a.x + n * a.C * a.H * a.W;
+        const float* wo = a.w + static_cast<int64_t>(o) * a.C * KH * KW;
+        float acc = 0.0f;
+        for (int32_t rc = 0; rc < a.C; ++rc)
+            for (int32_t rh = 0; rh < KH; ++rh) {
+                const int32_t ih = oh * a.sh + rh * a.dh - a.ph;
+                for (int32_t rw = 0; rw < KW; ++rw) {
+                    const int32_t iw = ow * a.sw + rw * a.dw - a.pw;
+                    const bool inb = ih >= 0 && ih < a.H && iw >= 0 && iw < a.W;
+                    const float v = inb ? xn[(static_cast<int64_t>(rc) * a.H + ih) * a.W + iw] : 0.0f;
+                    acc = __fadd_rn(acc, __fmul_rn(v, wo[(rc * KH + rh) * KW + rw]));
+                }
+            }
+        if (has_bias) acc = __fadd_rn(acc, a.bias[o]);
+        if (has_res) acc = __fadd_rn(acc, a.res[e]);
+        if (do_relu) acc = relu_sel(acc);
+        a.y[e] = acc;
+    }
+}
+
+// ------------------------------------------------------------------------------------------
+// Host side: variant table and selection.
+// ------------------------------------------------------------------------------------------
+struct Variant {
+    const char* name;
+    int kh, kw, cc, to, tp, nt, ppt;
+    void (*kernel)(const ConvArgs);
+};
+
+#define KXC_VARIANT(KH, KW, CC, WO, WP, RO, RP, PPT)                                                   \
+    {"mfma_k" #KH "x" #KW "_c" #CC "_o" #WO "x" #RO "_p" #WP "x" #RP, KH, KW, CC, 32 * RO * WO, 32 * RP * WP, \
+     64 * WO * WP, PPT, conv_mfma_kernel<KH, KW, CC, WO, WP, RO, RP, PPT>}
+
+// Ordered by preference (largest tile first); the host takes the first one that fits the shape
+// and fills the GPU.
+const Variant kVariants[] = {
+    KXC_VARIANT(3, 3, 4, 1, 4, 2, 2, 4),   // 64 x 256
+    KXC_VARIANT(3, 3, 4, 1, 4, 2, 1, 4),   // 64 x 128
+    KXC_VARIANT(3, 3, 4, 2, 2, 1, 1, 6),   // 64 x 64
+    KXC_VARIANT(3, 3, 4, 1, 4, 1, 1, 4),   // 32 x 128
+    KXC_VARIANT(1, 1, 8, 1, 4, 2, 2, 6),   // 64 x 256
+    KXC_VARIANT(1, 1, 8, 1, 4, 2, 1, 4),   // 64 x 128
+    KXC_VARIANT(1, 1, 8, 2, 2, 1, 1, 6),   // 64 x 64
+    KXC_VARIANT(1, 1, 8, 1, 4, 1, 1, 4),   // 32 x 128
+    KXC_VARIANT(7, 7, 4, 1, 4, 2, 1, 12),  // 64 x 128 (3 input channels padded to 4)
+    KXC_VARIANT(7, 7, 4, 1, 4, 1, 1, 12),  // 32 x 128
+};
+constexpr int kNumVariants = sizeof(kVariants) / sizeof(kVariants[0]);
+
+struct Choice {
+    const Variant* v = nullptr;
+    int32_t chs = 0;
+    size_t lds_bytes = 0;
+};
+
+// Largest padded-row span any pixel tile of size tp touches.
+int32_t MaxTileRows(const ConvArgs& a, int kh, int tp) {
+    int32_t best = 0;
+    for (int64_t m0 = 0; m0 < a.M; m0 += tp) {
+        const int64_t ml = (m0 + tp < a.M ? m0 + tp : a.M) - 1;
+        const int32_t n = static_cast<int32_t>(m0 / a.OHW), rem = static_cast<int32_t>(m0 - static_cast<int64_t>(n) * a.OHW);
+        const int32_t n2 = static_cast<int32_t>(ml / a.OHW), rem2 = static_cast<int32_t>(ml - static_cast<int64_t>(n2) * a.OHW);
+        const int32_t qmin = n * a.Hp + (rem / a.OW) * a.sh;
+        const int32_t qlast = n2 * a.Hp + (rem2 / a.OW) * a.sh + (kh - 1) * a.dh;
+        if (qlast - qmin + 1 > best) best = qlast - qmin + 1;
+    }
+    return best;
+}
+
+constexpr size_t kMaxLdsBytes = 160 * 1024;  // LDS of one gfx950 compute unit
+constexpr int64_t kFillTiles = 512;          // two workgroups per CU on 256 CUs
+
+bool Fits(const Variant& v, const ConvArgs& a, Choice* out) {
+    const int32_t rows = MaxTileRows(a, v.kh, v.tp);
+    const int64_t P = static_cast<int64_t>(rows) * a.Wp;
+    if (P > static_cast<int64_t>(v.ppt) * v.nt) return false;
+    // Channel stride: a multiple of 64 floats plus 32, so the two half-waves (which read channels
+    // c and c+1 at the same position) fall into different halves of the LDS banks.
+    const int32_t chs = static_cast<int32_t>((P + 63) / 64 * 64 + 32);
+    const int ks = (v.cc * v.kh * v.kw) | 1;
+    const int buffers = (a.C + v.cc - 1) / v.cc > 1 ? 2 : 1;   // a single chunk needs no second buffer
+    const size_t lds = buffers * (static_cast<size_t>(v.cc) * chs + static_cast<size_t>(v.to) * ks) * sizeof(float);
+    if (lds > kMaxLdsBytes) return false;
+    out->v = &v;
+    out->chs = chs;
+    out->lds_bytes = lds;
+    return true;
+}
+
+// Picks the MFMA variant for a shape, or leaves choice.v == nullptr for the direct kernel.
+void Select(const ConvArgs& a, int kh, int kw, Choice* choice) {
+    choice->v = nullptr;
+    if (a.O < 32 || a.M < 32) return;
+    // int32 offsets inside the kernel
+    const int64_t x_elems = static_cast<int64_t>(a.N) * a.C * a.H * a.W;
+    const int64_t y_elems = static_cast<int64_t>(a.N) * a.O * a.OHW;
+    const int64_t q_rows = static_cast<int64_t>(a.N + 1) * a.Hp + kh * a.dh;
+    if (x_elems >= (1LL << 31) || y_elems >= (1LL << 31) || q_rows * a.Wp >= (1LL << 31)) return;
+    const char* forced = std::getenv("KXC_HIP_CONV_VARIANT");
+    Choice best;
+    int64_t best_tiles = -1;
+    for (int i = 0; i < kNumVariants; ++i) {
+        const Variant& v = kVariants[i];
+        if (v.kh != kh || v.kw != kw) continue;
+        if (forced && *forced && std::strcmp(forced, v.name) != 0) continue;
+        if (v.to > a.O) continue;                 // do not spend matrix work on absent output channels
+        Choice c;
+        if (!Fits(v, a, &c)) continue;
+        const int64_t tiles = CeilDiv(a.M, v.tp) * CeilDiv(a.O, v.to);
+        if (tiles >= kFillTiles) { *choice = c; return; }   // first (largest) tile that fills the chip
+        if (tiles > best_tiles) { best_tiles = tiles; best = c; }
+    }
+    *choice = best;
+}
+
+int32_t FillArgs(const kxc_hip_conv2d_desc* d, ConvArgs* a, const char* who) {
+    KXC_HIP_REQUIRE(d != nullptr, "%s: desc is NULL", who);
+    KXC_HIP_REQUIRE(d->n >= 0 && d->c > 0 && d->h > 0 && d->w > 0 && d->o > 0 && d->kh > 0 && d->kw > 0,
+                    "%s: bad shape", who);
+    KXC_HIP_REQUIRE(d->stride_h > 0 && d->stride_w > 0 && d->dil_h > 0 && d->dil_w > 0,
+                    "%s: nn_conv2d stride and dilation must be positive", who);
+    KXC_HIP_REQUIRE(d->pad_h >= 0 && d->pad_w >= 0, "%s: negative padding", who);
+    // WindowOutputDim (src/relay/type_infer.cc:166-184)
+    const int64_t nh = static_cast<int64_t>(d->h) + 2 * d->pad_h - (static_cast<int64_t>(d->dil_h) * (d->kh - 1) + 1);
+    const int64_t nw = static_cast<int64_t>(d->w) + 2 * d->pad_w - (static_cast<int64_t>(d->dil_w) * (d->kw - 1) + 1);
+    KXC_HIP_REQUIRE(nh >= 0 && nw >= 0, "%s: nn_conv2d window is larger than input", who);
+    std::memset(a, 0, sizeof(*a));
+    a->N = d->n; a->C = d->c; a->H = d->h; a->W = d->w; a->O = d->o;
+    a->OH = static_cast<int32_t>(nh / d->stride_h + 1);
+    a->OW = static_cast<int32_t>(nw / d->stride_w + 1);
+    a->sh = d->stride_h; a->sw = d->stride_w; a->ph = d->pad_h; a->pw = d->pad_w; a->dh = d->dil_h; a->dw = d->dil_w;
+    a->Hp = d->h + 2 * d->pad_h; a->Wp = d->w + 2 * d->pad_w;
+    a->OHW = a->OH * a->OW;
+    const int64_t M = static_cast<int64_t>(d->n) * a->OHW;
+    a->M = M < (1LL << 31) ? static_cast<int32_t>(M) : 0;
+    a->flags = d->flags;
+    return KXC_HIP_OK;
+}
+
+}  // namespace
+
+extern "C" {
+
+const char* kxc_hip_conv2d_variant(const kxc_hip_conv2d_desc* desc) {
+    ConvArgs a;
+    if (FillArgs(desc, &a, "kxc_hip_conv2d_variant") != KXC_HIP_OK) return "invalid";
+    if (desc->flags & KXC_HIP_CONV_FORCE_DIRECT) return "direct";
+    Choice c;
+    Select(a, desc->kh, desc->kw, &c);
+    return c.v ? c.v->name : "direct";
+}
+
+int32_t kxc_hip_conv2d_nchw_f32(const kxc_hip_conv2d_desc* desc, const float* x, const float* w, const float* bias,
+                                const float* residual, float* y, void* stream) {
+    ConvArgs a;
+    if (int32_t rc = FillArgs(desc, &a, "kxc_hip_conv2d_nchw_f32")) return rc;
+    const int64_t total = static_cast<int64_t>(a.N) * a.O * a.OHW;
+    if (total == 0) return KXC_HIP_OK;
+    KXC_HIP_REQUIRE(x && w && y, "kxc_hip_conv2d_nchw_f32: NULL pointer");
+    KXC_HIP_REQUIRE(!(desc->flags & KXC_HIP_CONV_BIAS) || bias, "kxc_hip_conv2d_nchw_f32: bias flag without bias");
+    KXC_HIP_REQUIRE(!(desc->flags & KXC_HIP_CONV_RESIDUAL) || residual,
+                    "kxc_hip_conv2d_nchw_f32: residual flag without residual");
+    a.x = x; a.w = w; a.bias = bias; a.res = residual; a.y = y;
+    hipStream_t s = ResolveStream(stream);
+
+    Choice c;
+    if (!(desc->flags & KXC_HIP_CONV_FORCE_DIRECT) && a.M > 0) Select(a, desc->kh, desc->kw, &c);
+    if (c.v) {
+        a.chs = c.chs;
+        a.nchunks = (a.C + c.v->cc - 1) / c.v->cc;
+        dim3 grid(static_cast<unsigned>(CeilDiv(a.M, c.v->tp)), static_cast<unsigned>(CeilDiv(a.O, c.v->to)));
+        KXC_HIP_REQUIRE(grid.y <= 65535u, "kxc_hip_conv2d_nchw_f32: too many output channels");
+        if (c.lds_bytes > 64 * 1024) {
+            // above the default 64 KiB the dynamic LDS size has to be granted per kernel
+            KXC_HIP_CALL(hipFuncSetAttribute(reinterpret_cast<const void*>(c.v->kernel),
+                                             hipFuncAttributeMaxDynamicSharedMemorySize,
+                                             static_cast<int>(c.lds_bytes)),
+                         "hipFuncSetAttribute(MaxDynamicSharedMemorySize)");
+        }
+        hipLaunchKernelGGL(c.v->kernel, grid, dim3(c.v->nt), c.lds_bytes, s, a);
+        return CheckLaunch(c.v->name);
+    }
+    int64_t g = CeilDiv(total, 256);
+    if (g > 256 * 64) g = 256 * 64;
+    conv_direct_kernel<<<static_cast<int>(g), 256, 0, s>>>(a, desc->kh, desc->kw, total);
+    return CheckLaunch("conv_direct");
+}
+
+}  // extern "C"

@@ -1,0 +1,432 @@
+// plan.hip -- launch plan: the body of one compiled function as a list of kernel launches on one
+// stream.  Fills the gap the reference leaves in its execution plan, whose executor only copies
+// buffers (src/base/disco/executor.cc:122-157): every node here is a real launch, named by a
+// kernel_symbol as KernelExecNode would carry it (include/base/execution_plan.h:42-50).
+// Intermediates live in ONE workspace allocated at finalize time (the CPU backend mallocs and frees
+// every intermediate on every call, src/codegen/codegen_llvm.cc:578-623).
+#include <cstring>
+#include <string>
+#include <vector>
+
+#include "common.h"
+
+using namespace kxc_hip;
+
+namespace {
+
+enum class NodeKind {
+    kConv2D, kPool2D, kGlobalAvgPool, kGemm, kBinary, kRelu, kCopy,
+    kQConv2D, kQuantize, kMaxPoolI8, kGlobalAvgPoolI8, kQDense, kModuleKernel
+};
+
+struct Node {
+    NodeKind kind;
+    std::string symbol;
+    kxc_hip_buf bufs[6];
+    kxc_hip_conv2d_desc conv;
+    kxc_hip_qconv2d_desc qconv;
+    kxc_hip_pool2d_desc pool;
+    int64_t dims[4];
+    float f[2];
+    int32_t i32[4];
+    int64_t a_shape[6], b_shape[6];
+    // module kernel
+    void* function = nullptr;
+    uint32_t grid[3], block[3], shared_bytes = 0;
+    std::vector<kxc_hip_buf> params;
+};
+
+}  // namespace
+
+struct kxc_hip_plan {
+    int32_t device_id = 0;
+    int32_t num_args = 0;
+    std::vector<Node> nodes;
+    void* workspace = nullptr;
+    size_t workspace_bytes = 0;
+    bool finalized = false;
+};
+
+namespace {
+
+int32_t CheckBuf(const kxc_hip_plan* p, kxc_hip_buf b, bool optional, const char* who) {
+    if (b.kind == KXC_HIP_BUF_NONE) {
+        KXC_HIP_REQUIRE(optional, "%s: a required operand is absent", who);
+        return KXC_HIP_OK;
+    }
+    if (b.kind == KXC_HIP_BUF_ARG) {
+        KXC_HIP_REQUIRE(b.index_or_offset >= 0 && b.index_or_offset < p->num_args,
+                        "%s: packed argument index %lld out of range [0,%d)", who,
+                        static_cast<long long>(b.index_or_offset), p->num_args);
+        return KXC_HIP_OK;
+    }
+    KXC_HIP_REQUIRE(b.kind == KXC_HIP_BUF_WORKSPACE, "%s: bad buffer kind %d", who, b.kind);
+    KXC_HIP_REQUIRE(b.index_or_offset >= 0 && (b.index_or_offset % 256) == 0,
+                    "%s: workspace offsets must be non-negative multiples of 256", who);
+    return KXC_HIP_OK;
+}
+
+inline void* Resolve(const kxc_hip_plan* p, kxc_hip_buf b, void** args) {
+    if (b.kind == KXC_HIP_BUF_ARG) return args[b.index_or_offset];
+    if (b.kind == KXC_HIP_BUF_WORKSPACE) return static_cast<char*>(p->workspace) + b.index_or_offset;
+    return nullptr;
+}
+
+int32_t Begin(kxc_hip_plan* p, const char* who) {
+    KXC_HIP_REQUIRE(p != nullptr, "%s: plan is NULL", who);
+    KXC_HIP_REQUIRE(!p->finalized, "%s: plan is already finalized", who);
+    return KXC_HIP_OK;
+}
+
+}  // namespace
+
+#define KXC_PLAN_BEGIN(who) if (int32_t _rc = Begin(plan, who)) return _rc
+#define KXC_PLAN_BUF(b, optional, who) if (int32_t _rc = CheckBuf(plan, b, optional, who)) return _rc
+
+extern "C" {
+
+int32_t kxc_hip_plan_create(int32_t device_id, int32_t num_packed_args, kxc_hip_plan** out) {
+    KXC_HIP_REQUIRE(out != nullptr, "kxc_hip_plan_create: out is NULL");
+    KXC_HIP_REQUIRE(num_packed_args >= 0, "kxc_hip_plan_create: negative argument count");
+    kxc_hip_plan* p = new kxc_hip_plan();
+    p->device_id = device_id;
+    p->num_args = num_packed_args;
+    *out = p;
+    return KXC_HIP_OK;
+}
+
+int32_t kxc_hip_plan_destroy(kxc_hip_plan* plan) {
+    if (!plan) return KXC_HIP_OK;
+    hipError_t e = hipSuccess;
+    if (plan->workspace) e = hipFree(plan->workspace);
+    delete plan;
+    KXC_HIP_CALL(e, "plan workspace free");
+    return KXC_HIP_OK;
+}
+
+int32_t kxc_hip_plan_add_conv2d(kxc_hip_plan* plan, const kxc_hip_conv2d_desc* desc, kxc_hip_buf x, kxc_hip_buf w,
+                                kxc_hip_buf bias, kxc_hip_buf residual, kxc_hip_buf y) {
+    const char* who = "kxc_hip_plan_add_conv2d";
+    KXC_PLAN_BEGIN(who);
+    KXC_HIP_REQUIRE(desc != nullptr, "%s: desc is NULL", who);
+    KXC_PLAN_BUF(x, false, who); KXC_PLAN_BUF(w, false, who); KXC_PLAN_BUF(y, false, who);
+    KXC_PLAN_BUF(bias, !(desc->flags & KXC_HIP_CONV_BIAS), who);
+    KXC_PLAN_BUF(residual, !(desc->flags & KXC_HIP_CONV_RESIDUAL), who);
+    Node n{};
+    n.kind = NodeKind::kConv2D;
+    n.conv = *desc;
+    n.bufs[0] = x; n.bufs[1] = w; n.bufs[2] = bias; n.bufs[3] = residual; n.bufs[4] = y;
+    n.symbol = std::string("kxc_conv2d_nchw_f32.") + kxc_hip_conv2d_variant(desc);
+    if (desc->flags & KXC_HIP_CONV_BIAS) n.symbol += "+bias";
+    if (desc->flags & KXC_HIP_CONV_RESIDUAL) n.symbol += "+add";
+    if (desc->flags & KXC_HIP_CONV_RELU) n.symbol += "+relu";
+    plan->nodes.push_back(n);
+    return KXC_HIP_OK;
+}
+
+int32_t kxc_hip_plan_add_pool2d(kxc_hip_plan* plan, const kxc_hip_pool2d_desc* desc, kxc_hip_buf x, kxc_hip_buf y) {
+    const char* who = "kxc_hip_plan_add_pool2d";
+    KXC_PLAN_BEGIN(who);
+    KXC_HIP_REQUIRE(desc != nullptr, "%s: desc is NULL", who);
+    KXC_PLAN_BUF(x, false, who); KXC_PLAN_BUF(y, false, who);
+    Node n{};
+    n.kind = NodeKind::kPool2D;
+    n.pool = *desc;
+    n.bufs[0] = x; n.bufs[1] = y;
+    n.symbol = desc->is_avg ? "kxc_avg_pool2d_f32" : "kxc_max_pool2d_f32";
+    plan->nodes.push_back(n);
+    return KXC_HIP_OK;
+}
+
+int32_t kxc_hip_plan_add_global_avg_pool2d(kxc_hip_plan* plan, int64_t nn, int64_t c, int64_t h, int64_t w,
+                                           kxc_hip_buf x, kxc_hip_buf y) {
+    const char* who = "kxc_hip_plan_add_global_avg_pool2d";
+    KXC_PLAN_BEGIN(who);
+    KXC_PLAN_BUF(x, false, who); KXC_PLAN_BUF(y, false, who);
+    Node n{};
+    n.kind = NodeKind::kGlobalAvgPool;
+    n.dims[0] = nn; n.dims[1] = c; n.dims[2] = h; n.dims[3] = w;
+    n.bufs[0] = x; n.bufs[1] = y;
+    n.symbol = "kxc_global_avg_pool2d_f32";
+    plan->nodes.push_back(n);
+    return KXC_HIP_OK;
+}
+
+int32_t kxc_hip_plan_add_gemm(kxc_hip_plan* plan, int64_t m, int64_t nn, int64_t k, float alpha, float beta,
+                              int32_t transB, int64_t c_len, kxc_hip_buf a, kxc_hip_buf b, kxc_hip_buf c, kxc_hip_buf y) {
+    const char* who = "kxc_hip_plan_add_gemm";
+    KXC_PLAN_BEGIN(who);
+    KXC_PLAN_BUF(a, false, who); KXC_PLAN_BUF(b, false, who); KXC_PLAN_BUF(c, true, who); KXC_PLAN_BUF(y, false, who);
+    Node n{};
+    n.kind = NodeKind::kGemm;
+    n.dims[0] = m; n.dims[1] = nn; n.dims[2] = k; n.dims[3] = c_len;
+    n.f[0] = alpha; n.f[1] = beta; n.i32[0] = transB;
+    n.bufs[0] = a; n.bufs[1] = b; n.bufs[2] = c; n.bufs[3] = y;
+    n.symbol = "kxc_gemm_f32";
+    plan->nodes.push_back(n);
+    return KXC_HIP_OK;
+}
+
+int32_t kxc_hip_plan_add_binary(kxc_hip_plan* plan, int32_t op, const int64_t* a_shape, int32_t a_ndim,
+                                const int64_t* b_shape, int32_t b_ndim, int32_t relu, kxc_hip_buf a, kxc_hip_buf b,
+                                kxc_hip_buf y) {
+    const char* who = "kxc_hip_plan_add_binary";
+    KXC_PLAN_BEGIN(who);
+    KXC_HIP_REQUIRE(op >= 0 && op <= 3 && a_ndim >= 0 && a_ndim <= 6 && b_ndim >= 0 && b_ndim <= 6, "%s: bad op or rank", who);
+    KXC_HIP_REQUIRE((a_ndim == 0 || a_shape) && (b_ndim == 0 || b_shape), "%s: shape is NULL", who);
+    KXC_PLAN_BUF(a, false, who); KXC_PLAN_BUF(b, false, who); KXC_PLAN_BUF(y, false, who);
+    Node n{};
+    n.kind = NodeKind::kBinary;
+    n.i32[0] = op; n.i32[1] = a_ndim; n.i32[2] = b_ndim; n.i32[3] = relu;
+    for (int i = 0; i < a_ndim; ++i) n.a_shape[i] = a_shape[i];
+    for (int i = 0; i < b_ndim; ++i) n.b_shape[i] = b_shape[i];
+    n.bufs[0] = a; n.bufs[1] = b; n.bufs[2] = y;
+    static const char* names[4] = {"kxc_add_f32", "kxc_subtract_f32", "kxc_multiply_f32", "kxc_divide_f32"};
+    n.symbol = names[op];
+    if (relu) n.symbol += "+relu";
+    plan->nodes.push_back(n);
+    return KXC_HIP_OK;
+}
+
+int32_t kxc_hip_plan_add_relu(kxc_hip_plan* plan, int64_t count, kxc_hip_buf x, kxc_hip_buf y) {
+    const char* who = "kxc_hip_plan_add_relu";
+    KXC_PLAN_BEGIN(who);
+    KXC_PLAN_BUF(x, false, who); KXC_PLAN_BUF(y, false, who);
+    Node n{};
+    n.kind = NodeKind::kRelu;
+    n.dims[0] = count;
+    n.bufs[0] = x; n.bufs[1] = y;
+    n.symbol = "kxc_relu_f32";
+    plan->nodes.push_back(n);
+    return KXC_HIP_OK;
+}
+
+int32_t kxc_hip_plan_add_copy(kxc_hip_plan* plan, int64_t nbytes, kxc_hip_buf x, kxc_hip_buf y) {
+    const char* who = "kxc_hip_plan_add_copy";
+    KXC_PLAN_BEGIN(who);
+    KXC_HIP_REQUIRE(nbytes >= 0, "%s: negative size", who);
+    KXC_PLAN_BUF(x, false, who); KXC_PLAN_BUF(y, false, who);
+    Node n{};
+    n.kind = NodeKind::kCopy;
+    n.dims[0] = nbytes;
+    n.bufs[0] = x; n.bufs[1] = y;
+    n.symbol = "kxc_copy";
+    plan->nodes.push_back(n);
+    return KXC_HIP_OK;
+}
+
+int32_t kxc_hip_plan_add_qconv2d(kxc_hip_plan* plan, const kxc_hip_qconv2d_desc* desc, kxc_hip_buf x, kxc_hip_buf w,
+                                 kxc_hip_buf bias, kxc_hip_buf mult, kxc_hip_buf residual, kxc_hip_buf y) {
+    const char* who = "kxc_hip_plan_add_qconv2d";
+    KXC_PLAN_BEGIN(who);
+    KXC_HIP_REQUIRE(desc != nullptr, "%s: desc is NULL", who);
+    KXC_PLAN_BUF(x, false, who); KXC_PLAN_BUF(w, false, who); KXC_PLAN_BUF(mult, false, who); KXC_PLAN_BUF(y, false, who);
+    KXC_PLAN_BUF(bias, !(desc->flags & KXC_HIP_CONV_BIAS), who);
+    KXC_PLAN_BUF(residual, !(desc->flags & KXC_HIP_CONV_RESIDUAL), who);
+    Node n{};
+    n.kind = NodeKind::kQConv2D;
+    n.qconv = *desc;
+    n.bufs[0] = x; n.bufs[1] = w; n.bufs[2] = bias; n.bufs[3] = mult; n.bufs[4] = residual; n.bufs[5] = y;
+    n.symbol = "kxc_qconv2d_nchw_i8";
+    plan->nodes.push_back(n);
+    return KXC_HIP_OK;
+}
+
+int32_t kxc_hip_plan_add_quantize(kxc_hip_plan* plan, int64_t count, float scale, kxc_hip_buf x, kxc_hip_buf q) {
+    const char* who = "kxc_hip_plan_add_quantize";
+    KXC_PLAN_BEGIN(who);
+    KXC_PLAN_BUF(x, false, who); KXC_PLAN_BUF(q, false, who);
+    Node n{};
+    n.kind = NodeKind::kQuantize;
+    n.dims[0] = count; n.f[0] = scale;
+    n.bufs[0] = x; n.bufs[1] = q;
+    n.symbol = "kxc_quantize_f32_i8";
+    plan->nodes.push_back(n);
+    return KXC_HIP_OK;
+}
+
+int32_t kxc_hip_plan_add_maxpool2d_i8(kxc_hip_plan* plan, const kxc_hip_pool2d_desc* desc, kxc_hip_buf x, kxc_hip_buf y) {
+    const char* who = "kxc_hip_plan_add_maxpool2d_i8";
+    KXC_PLAN_BEGIN(who);
+    KXC_HIP_REQUIRE(desc != nullptr, "%s: desc is NULL", who);
+    KXC_PLAN_BUF(x, false, who); KXC_PLAN_BUF(y, false, who);
+    Node n{};
+    n.kind = NodeKind::kMaxPoolI8;
+    n.pool = *desc;
+    n.bufs[0] = x; n.bufs[1] = y;
+    n.symbol = "kxc_max_pool2d_i8";
+    plan->nodes.push_back(n);
+    return KXC_HIP_OK;
+}
+
+int32_t kxc_hip_plan_add_global_avg_pool2d_i8(kxc_hip_plan* plan, int64_t nn, int64_t c, int64_t h, int64_t w, float mult,
+                                              kxc_hip_buf x, kxc_hip_buf y) {
+    const char* who = "kxc_hip_plan_add_global_avg_pool2d_i8";
+    KXC_PLAN_BEGIN(who);
+    KXC_PLAN_BUF(x, false, who); KXC_PLAN_BUF(y, false, who);
+    Node n{};
+    n.kind = NodeKind::kGlobalAvgPoolI8;
+    n.dims[0] = nn; n.dims[1] = c; n.dims[2] = h; n.dims[3] = w; n.f[0] = mult;
+    n.bufs[0] = x; n.bufs[1] = y;
+    n.symbol = "kxc_global_avg_pool2d_i8";
+    plan->nodes.push_back(n);
+    return KXC_HIP_OK;
+}
+
+int32_t kxc_hip_plan_add_qdense(kxc_hip_plan* plan, int64_t m, int64_t nn, int64_t k, kxc_hip_buf a, kxc_hip_buf b,
+                                kxc_hip_buf bias, kxc_hip_buf mult, kxc_hip_buf y) {
+    const char* who = "kxc_hip_plan_add_qdense";
+    KXC_PLAN_BEGIN(who);
+    KXC_PLAN_BUF(a, false, who); KXC_PLAN_BUF(b, false, who); KXC_PLAN_BUF(bias, true, who);
+    KXC_PLAN_BUF(mult, false, who); KXC_PLAN_BUF(y, false, who);
+    Node n{};
+    n.kind = NodeKind::kQDense;
+    n.dims[0] = m; n.dims[1] = nn; n.dims[2] = k;
+    n.bufs[0] = a; n.bufs[1] = b; n.bufs[2] = bias; n.bufs[3] = mult; n.bufs[4] = y;
+    n.symbol = "kxc_qdense_i8";
+    plan->nodes.push_back(n);
+    return KXC_HIP_OK;
+}
+
+int32_t kxc_hip_plan_add_module_kernel(kxc_hip_plan* plan, void* function, const char* symbol, const uint32_t grid[3],
+                                       const uint32_t block[3], uint32_t shared_bytes, const kxc_hip_buf* params,
+                                       int32_t num_params) {
+    const char* who = "kxc_hip_plan_add_module_kernel";
+    KXC_PLAN_BEGIN(who);
+    KXC_HIP_REQUIRE(function && grid && block && num_params >= 0 && (num_params == 0 || params), "%s: NULL argument", who);
+    KXC_HIP_REQUIRE(grid[0] > 0 && grid[1] > 0 && grid[2] > 0 && block[0] > 0 && block[1] > 0 && block[2] > 0,
+                    "%s: empty grid or block", who);
+    KXC_HIP_REQUIRE(static_cast<uint64_t>(block[0]) * block[1] * block[2] <= 1024, "%s: more than 1024 threads per block", who);
+    Node n{};
+    n.kind = NodeKind::kModuleKernel;
+    n.function = function;
+    for (int i = 0; i < 3; ++i) { n.grid[i] = grid[i]; n.block[i] = block[i]; }
+    n.shared_bytes = shared_bytes;
+    for (int i = 0; i < num_params; ++i) {
+        KXC_PLAN_BUF(params[i], false, who);
+        n.params.push_back(params[i]);
+    }
+    n.symbol = symbol ? symbol : "kxc_module_kernel";
+    plan->nodes.push_back(n);
+    return KXC_HIP_OK;
+}
+
+int32_t kxc_hip_plan_finalize(kxc_hip_plan* plan, size_t workspace_bytes) {
+    KXC_HIP_REQUIRE(plan != nullptr, "kxc_hip_plan_finalize: plan is NULL");
+    KXC_HIP_REQUIRE(!plan->finalized, "kxc_hip_plan_finalize: plan is already finalized");
+    for (const Node& n : plan->nodes) {
+        auto check = [&](kxc_hip_buf b) {
+            return !(b.kind == KXC_HIP_BUF_WORKSPACE && static_cast<size_t>(b.index_or_offset) >= workspace_bytes &&
+                     workspace_bytes > 0) &&
+                   !(b.kind == KXC_HIP_BUF_WORKSPACE && workspace_bytes == 0);
+        };
+        for (const kxc_hip_buf& b : n.bufs)
+            KXC_HIP_REQUIRE(b.kind != KXC_HIP_BUF_WORKSPACE || check(b),
+                            "kxc_hip_plan_finalize: node %s uses a workspace offset beyond %zu bytes", n.symbol.c_str(),
+                            workspace_bytes);
+        for (const kxc_hip_buf& b : n.params)
+            KXC_HIP_REQUIRE(b.kind != KXC_HIP_BUF_WORKSPACE || check(b),
+                            "kxc_hip_plan_finalize: node %s uses a workspace offset beyond %zu bytes", n.symbol.c_str(),
+                            workspace_bytes);
+    }
+    if (workspace_bytes > 0) {
+        KXC_HIP_CALL(hipSetDevice(plan->device_id), "HIP SetDevice");
+        KXC_HIP_CALL(hipMalloc(&plan->workspace, workspace_bytes), "plan workspace allocation");
+    }
+    plan->workspace_bytes = workspace_bytes;
+    plan->finalized = true;
+    return KXC_HIP_OK;
+}
+
+int32_t kxc_hip_plan_run(kxc_hip_plan* plan, void** args, void* stream) {
+    KXC_HIP_REQUIRE(plan != nullptr, "kxc_hip_plan_run: plan is NULL");
+    KXC_HIP_REQUIRE(plan->finalized, "kxc_hip_plan_run: plan is not finalized");
+    KXC_HIP_REQUIRE(plan->num_args == 0 || args != nullptr, "kxc_hip_plan_run: packed_args is NULL");
+    for (int i = 0; i < plan->num_args; ++i)
+        KXC_HIP_REQUIRE(args[i] != nullptr, "kxc_hip_plan_run: packed argument %d is NULL", i);
+    void* s = stream ? stream : static_cast<void*>(CurrentStream());
+    for (Node& n : plan->nodes) {
+        int32_t rc = KXC_HIP_OK;
+        auto B = [&](int i) { return Resolve(plan, n.bufs[i], args); };
+        switch (n.kind) {
+            case NodeKind::kConv2D:
+                rc = kxc_hip_conv2d_nchw_f32(&n.conv, static_cast<const float*>(B(0)), static_cast<const float*>(B(1)),
+                                             static_cast<const float*>(B(2)), static_cast<const float*>(B(3)),
+                                             static_cast<float*>(B(4)), s);
+                break;
+            case NodeKind::kPool2D:
+                rc = kxc_hip_pool2d_f32(&n.pool, static_cast<const float*>(B(0)), static_cast<float*>(B(1)), s);
+                break;
+            case NodeKind::kGlobalAvgPool:
+                rc = kxc_hip_global_avg_pool2d_f32(static_cast<const float*>(B(0)), static_cast<float*>(B(1)), n.dims[0],
+                                                   n.dims[1], n.dims[2], n.dims[3], s);
+                break;
+            case NodeKind::kGemm:
+                rc = kxc_hip_gemm_f32(static_cast<const float*>(B(0)), static_cast<const float*>(B(1)),
+                                      static_cast<const float*>(B(2)), static_cast<float*>(B(3)), n.dims[0], n.dims[1],
+                                      n.dims[2], n.f[0], n.f[1], n.i32[0], n.dims[3], s);
+                break;
+            case NodeKind::kBinary:
+                rc = kxc_hip_broadcast_binary_f32(n.i32[0], static_cast<const float*>(B(0)), n.a_shape, n.i32[1],
+                                                  static_cast<const float*>(B(1)), n.b_shape, n.i32[2],
+                                                  static_cast<float*>(B(2)), n.i32[3], s);
+                break;
+            case NodeKind::kRelu:
+                rc = kxc_hip_relu_f32(static_cast<const float*>(B(0)), static_cast<float*>(B(1)), n.dims[0], s);
+                break;
+            case NodeKind::kCopy: {
+                hipError_t e = hipMemcpyAsync(B(1), B(0), static_cast<size_t>(n.dims[0]), hipMemcpyDeviceToDevice,
+                                              reinterpret_cast<hipStream_t>(s));
+                if (e != hipSuccess) rc = Fail(KXC_HIP_ERR_RUNTIME, "plan copy failed: %s", hipGetErrorString(e));
+                break;
+            }
+            case NodeKind::kQConv2D:
+                rc = kxc_hip_qconv2d_nchw_i8(&n.qconv, static_cast<const int8_t*>(B(0)), static_cast<const int8_t*>(B(1)),
+                                             static_cast<const int32_t*>(B(2)), static_cast<const float*>(B(3)),
+                                             static_cast<const int8_t*>(B(4)), static_cast<int8_t*>(B(5)), s);
+                break;
+            case NodeKind::kQuantize:
+                rc = kxc_hip_quantize_f32_i8(static_cast<const float*>(B(0)), static_cast<int8_t*>(B(1)), n.dims[0], n.f[0], s);
+                break;
+            case NodeKind::kMaxPoolI8:
+                rc = kxc_hip_maxpool2d_i8(&n.pool, static_cast<const int8_t*>(B(0)), static_cast<int8_t*>(B(1)), s);
+                break;
+            case NodeKind::kGlobalAvgPoolI8:
+                rc = kxc_hip_global_avg_pool2d_i8(static_cast<const int8_t*>(B(0)), static_cast<int8_t*>(B(1)), n.dims[0],
+                                                  n.dims[1], n.dims[2], n.dims[3], n.f[0], s);
+                break;
+            case NodeKind::kQDense:
+                rc = kxc_hip_qdense_i8(static_cast<const int8_t*>(B(0)), static_cast<const int8_t*>(B(1)),
+                                       static_cast<const int32_t*>(B(2)), static_cast<const float*>(B(3)),
+                                       static_cast<float*>(B(4)), n.dims[0], n.dims[1], n.dims[2], s);
+                break;
+            case NodeKind::kModuleKernel: {
+                // every parameter is a device pointer; hipModuleLaunchKernel wants the address of each
+                std::vector<void*> values(n.params.size());
+                std::vector<void*> addrs(n.params.size());
+                for (size_t i = 0; i < n.params.size(); ++i) {
+                    values[i] = Resolve(plan, n.params[i], args);
+                    addrs[i] = &values[i];
+                }
+                rc = kxc_hip_module_launch(n.function, n.grid, n.block, n.shared_bytes, s, addrs.data());
+                break;
+            }
+        }
+        if (rc != KXC_HIP_OK) {
+            const std::string inner = LastError();
+            return Fail(rc, "plan node %s: %s", n.symbol.c_str(), inner.c_str());
+        }
+    }
+    return KXC_HIP_OK;
+}
+
+int32_t kxc_hip_plan_num_nodes(const kxc_hip_plan* plan) { return plan ? static_cast<int32_t>(plan->nodes.size()) : 0; }
+
+const char* kxc_hip_plan_node_symbol(const kxc_hip_plan* plan, int32_t i) {
+    if (!plan || i < 0 || i >= static_cast<int32_t>(plan->nodes.size())) return "";
+    return plan->nodes[i].symbol.c_str();
+}
+
+void* kxc_hip_plan_workspace(const kxc_hip_plan* plan) { return plan ? plan->workspace : nullptr; }
+
+}  // extern "C"

@@ -1,0 +1,361 @@
+"""ctypes binding of include/kxc_hip.h.
+
+Every wrapper takes torch tensors that already live on the GPU and passes their device pointers
+through the C ABI; a non-zero status raises KxcHipError carrying kxc_hip_last_error(), the way the
+reference's C++ layers throw std::runtime_error.  There is no CPU fallback: if the library is
+missing, loading fails loudly.
+"""
+import ctypes as C
+import os
+
+PKG = os.path.dirname(os.path.abspath(__file__))
+_LIB_PATH = os.path.join(PKG, "lib", "libkxc_hip.so")
+_lib = None
+
+CONV_BIAS, CONV_RESIDUAL, CONV_RELU, CONV_FORCE_DIRECT = 1, 2, 4, 0x100
+BUF_ARG, BUF_WORKSPACE, BUF_NONE = 0, 1, 2
+
+
+class KxcHipError(RuntimeError):
+    pass
+
+
+class ConvDesc(C.Structure):
+    _fields_ = [(n, C.c_int32) for n in ("n", "c", "h", "w", "o", "kh", "kw", "stride_h", "stride_w",
+                                         "pad_h", "pad_w", "dil_h", "dil_w")] + [("flags", C.c_uint32)]
+
+
+class QConvDesc(C.Structure):
+    _fields_ = [(n, C.c_int32) for n in ("n", "c", "h", "w", "o", "kh", "kw", "stride_h", "stride_w",
+                                         "pad_h", "pad_w")] + [("flags", C.c_uint32), ("res_mult", C.c_float)]
+
+
+class PoolDesc(C.Structure):
+    _fields_ = [(n, C.c_int32) for n in ("n", "c", "h", "w", "kh", "kw", "stride_h", "stride_w",
+                                         "pad_top", "pad_left", "pad_bottom", "pad_right", "ceil_mode", "is_avg")]
+
+
+class Buf(C.Structure):
+    _fields_ = [("kind", C.c_int32), ("index_or_offset", C.c_int64)]
+
+    @staticmethod
+    def arg(i):
+        return Buf(BUF_ARG, i)
+
+    @staticmethod
+    def ws(offset):
+        return Buf(BUF_WORKSPACE, offset)
+
+    @staticmethod
+    def none():
+        return Buf(BUF_NONE, 0)
+
+
+class DeviceAttrs(C.Structure):
+    _fields_ = [("exists", C.c_int32), ("warp_size", C.c_int32),
+                ("max_threads_per_block", C.c_int64), ("max_shared_memory_per_block", C.c_int64),
+                ("max_shared_memory_per_multiprocessor", C.c_int64), ("multi_processor_count", C.c_int64),
+                ("max_clock_rate_khz", C.c_int64), ("max_registers_per_block", C.c_int64),
+                ("l2_cache_size_bytes", C.c_int64), ("total_global_memory", C.c_int64),
+                ("available_global_memory", C.c_int64), ("max_threads_per_multiprocessor", C.c_int64),
+                ("compute_version_major", C.c_int32), ("compute_version_minor", C.c_int32),
+                ("api_version", C.c_int32), ("driver_version", C.c_int32),
+                ("device_name", C.c_char * 128), ("arch", C.c_char * 32), ("status", C.c_char * 128)]
+
+
+def library_path():
+    return _LIB_PATH
+
+
+def lib():
+    """The loaded C-ABI library.  Builds it first only when no built library exists."""
+    global _lib
+    if _lib is None:
+        if not os.path.exists(_LIB_PATH):
+            from . import build as _build
+            _build.build(verbose=False)
+        _lib = C.CDLL(_LIB_PATH)
+        _lib.kxc_hip_last_error.restype = C.c_char_p
+        _lib.kxc_hip_target_kind.restype = C.c_char_p
+        _lib.kxc_hip_conv2d_variant.restype = C.c_char_p
+        _lib.kxc_hip_plan_node_symbol.restype = C.c_char_p
+        _lib.kxc_hip_plan_workspace.restype = C.c_void_p
+    return _lib
+
+
+def _check(rc):
+    if rc != 0:
+        raise KxcHipError(lib().kxc_hip_last_error().decode())
+
+
+def _p(t):
+    return C.c_void_p(t.data_ptr()) if t is not None else C.c_void_p(0)
+
+
+def _stream():
+    import torch
+    return C.c_void_p(torch.cuda.current_stream().cuda_stream)
+
+
+def _need(t, dtype, name):
+    import torch
+    if t is None:
+        return
+    if not (t.is_cuda and t.is_contiguous() and t.dtype == dtype):
+        raise KxcHipError("%s must be a contiguous %s tensor on the GPU" % (name, dtype))
+
+
+def device_attributes(device_id=0):
+    a = DeviceAttrs()
+    _check(lib().kxc_hip_device_attributes(C.c_int32(device_id), C.byref(a)))
+    return a
+
+
+def conv_desc(x_shape, w_shape, stride, pad, dil=1, flags=0):
+    n, c, h, w = x_shape
+    o, _, kh, kw = w_shape
+    return ConvDesc(n, c, h, w, o, kh, kw, stride, stride, pad, pad, dil, dil, flags)
+
+
+def conv_out_shape(d):
+    oh = (d.h + 2 * d.pad_h - ((d.kh - 1) * d.dil_h + 1)) // d.stride_h + 1
+    ow = (d.w + 2 * d.pad_w - ((d.kw - 1) * d.dil_w + 1)) // d.stride_w + 1
+    return (d.n, d.o, oh, ow)
+
+
+def conv2d_variant(x_shape, w_shape, stride, pad, dil=1, flags=0):
+    d = conv_desc(x_shape, w_shape, stride, pad, dil, flags)
+    return lib().kxc_hip_conv2d_variant(C.byref(d)).decode()
+
+
+def conv2d(x, w, bias=None, residual=None, stride=1, pad=0, dil=1, relu=False, force_direct=False, out=None):
+    import torch
+    _need(x, torch.float32, "x"); _need(w, torch.float32, "w")
+    _need(bias, torch.float32, "bias"); _need(residual, torch.float32, "residual")
+    if x.shape[1] != w.shape[1]:
+        raise KxcHipError("nn_conv2d input channel mismatch")
+    flags = (CONV_BIAS if bias is not None else 0) | (CONV_RESIDUAL if residual is not None else 0) | \
+            (CONV_RELU if relu else 0) | (CONV_FORCE_DIRECT if force_direct else 0)
+    d = conv_desc(tuple(x.shape), tuple(w.shape), stride, pad, dil, flags)
+    y = out if out is not None else torch.empty(conv_out_shape(d), dtype=torch.float32, device=x.device)
+    _check(lib().kxc_hip_conv2d_nchw_f32(C.byref(d), _p(x), _p(w), _p(bias), _p(residual), _p(y), _stream()))
+    return y
+
+
+def relu(x):
+    import torch
+    _need(x, torch.float32, "x")
+    y = torch.empty_like(x)
+    _check(lib().kxc_hip_relu_f32(_p(x), _p(y), C.c_int64(x.numel()), _stream()))
+    return y
+
+
+def binary(op, a, b, relu=False):
+    import torch
+    _need(a, torch.float32, "a"); _need(b, torch.float32, "b")
+    shape = torch.broadcast_shapes(a.shape, b.shape)
+    y = torch.empty(shape, dtype=torch.float32, device=a.device)
+    sa = (C.c_int64 * max(1, a.dim()))(*a.shape); sb = (C.c_int64 * max(1, b.dim()))(*b.shape)
+    _check(lib().kxc_hip_broadcast_binary_f32(C.c_int32(op), _p(a), sa, C.c_int32(a.dim()), _p(b), sb,
+                                              C.c_int32(b.dim()), _p(y), C.c_int32(int(relu)), _stream()))
+    return y
+
+
+def bias_add(x, bias, relu=False):
+    import torch
+    _need(x, torch.float32, "x"); _need(bias, torch.float32, "bias")
+    y = torch.empty_like(x)
+    n, o = x.shape[:2]
+    hw = x.numel() // max(1, n * o)
+    _check(lib().kxc_hip_bias_add_nchw_f32(_p(x), _p(bias), _p(y), C.c_int64(n), C.c_int64(o), C.c_int64(hw),
+                                           C.c_int32(int(relu)), _stream()))
+    return y
+
+
+def pool_desc(x_shape, k, s, pad, ceil_mode=False, avg=False):
+    n, c, h, w = x_shape
+    if isinstance(pad, int):
+        pad = (pad, pad, pad, pad)
+    return PoolDesc(n, c, h, w, k, k, s, s, pad[0], pad[1], pad[2], pad[3], int(ceil_mode), int(avg))
+
+
+def pool_out_shape(d):
+    hn = d.h + d.pad_top + d.pad_bottom - d.kh
+    wn = d.w + d.pad_left + d.pad_right - d.kw
+    if d.ceil_mode:
+        return (d.n, d.c, (hn + d.stride_h - 1) // d.stride_h + 1, (wn + d.stride_w - 1) // d.stride_w + 1)
+    return (d.n, d.c, hn // d.stride_h + 1, wn // d.stride_w + 1)
+
+
+def pool2d(x, k, s, pad, ceil_mode=False, avg=False, out=None):
+    import torch
+    _need(x, torch.float32, "x")
+    d = pool_desc(tuple(x.shape), k, s, pad, ceil_mode, avg)
+    y = out if out is not None else torch.empty(pool_out_shape(d), dtype=torch.float32, device=x.device)
+    _check(lib().kxc_hip_pool2d_f32(C.byref(d), _p(x), _p(y), _stream()))
+    return y
+
+
+def global_avg_pool2d(x):
+    import torch
+    _need(x, torch.float32, "x")
+    n, c, h, w = x.shape
+    y = torch.empty((n, c, 1, 1), dtype=torch.float32, device=x.device)
+    _check(lib().kxc_hip_global_avg_pool2d_f32(_p(x), _p(y), C.c_int64(n), C.c_int64(c), C.c_int64(h), C.c_int64(w),
+                                               _stream()))
+    return y
+
+
+def gemm(a, b, c=None, alpha=1.0, beta=1.0, transB=1):
+    import torch
+    _need(a, torch.float32, "a"); _need(b, torch.float32, "b"); _need(c, torch.float32, "c")
+    m, k = a.shape
+    n = b.shape[0] if transB else b.shape[1]
+    y = torch.empty((m, n), dtype=torch.float32, device=a.device)
+    _check(lib().kxc_hip_gemm_f32(_p(a), _p(b), _p(c), _p(y), C.c_int64(m), C.c_int64(n), C.c_int64(k),
+                                  C.c_float(alpha), C.c_float(beta), C.c_int32(transB),
+                                  C.c_int64(c.numel() if c is not None else 0), _stream()))
+    return y
+
+
+def flatten(x):
+    import torch
+    _need(x, torch.float32, "x")
+    y = torch.empty((x.shape[0], x.numel() // max(1, x.shape[0])), dtype=torch.float32, device=x.device)
+    _check(lib().kxc_hip_flatten_f32(_p(x), _p(y), C.c_int64(x.numel()), _stream()))
+    return y
+
+
+def quantize(x, scale):
+    import torch
+    _need(x, torch.float32, "x")
+    q = torch.empty(x.shape, dtype=torch.int8, device=x.device)
+    _check(lib().kxc_hip_quantize_f32_i8(_p(x), _p(q), C.c_int64(x.numel()), C.c_float(scale), _stream()))
+    return q
+
+
+def qconv2d(x, w, bias, mult, residual=None, res_mult=0.0, stride=1, pad=0, relu=True, force_direct=False):
+    import torch
+    _need(x, torch.int8, "x"); _need(w, torch.int8, "w"); _need(bias, torch.int32, "bias")
+    _need(mult, torch.float32, "mult"); _need(residual, torch.int8, "residual")
+    n, c, h, wd = x.shape
+    o, _, kh, kw = w.shape
+    flags = (CONV_BIAS if bias is not None else 0) | (CONV_RESIDUAL if residual is not None else 0) | \
+            (CONV_RELU if relu else 0) | (CONV_FORCE_DIRECT if force_direct else 0)
+    d = QConvDesc(n, c, h, wd, o, kh, kw, stride, stride, pad, pad, flags, res_mult)
+    oh = (h + 2 * pad - kh) // stride + 1; ow = (wd + 2 * pad - kw) // stride + 1
+    y = torch.empty((n, o, oh, ow), dtype=torch.int8, device=x.device)
+    _check(lib().kxc_hip_qconv2d_nchw_i8(C.byref(d), _p(x), _p(w), _p(bias), _p(mult), _p(residual), _p(y), _stream()))
+    return y
+
+
+def qdense(a, b, bias, mult):
+    import torch
+    _need(a, torch.int8, "a"); _need(b, torch.int8, "b"); _need(bias, torch.int32, "bias"); _need(mult, torch.float32, "mult")
+    m, k = a.shape
+    n = b.shape[0]
+    y = torch.empty((m, n), dtype=torch.float32, device=a.device)
+    _check(lib().kxc_hip_qdense_i8(_p(a), _p(b), _p(bias), _p(mult), _p(y), C.c_int64(m), C.c_int64(n), C.c_int64(k),
+                                   _stream()))
+    return y
+
+
+def maxpool2d_i8(x, k, s, pad):
+    import torch
+    _need(x, torch.int8, "x")
+    d = pool_desc(tuple(x.shape), k, s, pad)
+    y = torch.empty(pool_out_shape(d), dtype=torch.int8, device=x.device)
+    _check(lib().kxc_hip_maxpool2d_i8(C.byref(d), _p(x), _p(y), _stream()))
+    return y
+
+
+def global_avg_pool2d_i8(x, mult):
+    import torch
+    _need(x, torch.int8, "x")
+    n, c, h, w = x.shape
+    y = torch.empty((n, c, 1, 1), dtype=torch.int8, device=x.device)
+    _check(lib().kxc_hip_global_avg_pool2d_i8(_p(x), _p(y), C.c_int64(n), C.c_int64(c), C.c_int64(h), C.c_int64(w),
+                                              C.c_float(mult), _stream()))
+    return y
+
+
+class Plan:
+    """kxc_hip_plan: a list of launches over packed arguments and one workspace."""
+
+    def __init__(self, num_args, device_id=0):
+        self._h = C.c_void_p()
+        _check(lib().kxc_hip_plan_create(C.c_int32(device_id), C.c_int32(num_args), C.byref(self._h)))
+        self.num_args = num_args
+
+    def close(self):
+        if self._h:
+            lib().kxc_hip_plan_destroy(self._h)
+            self._h = C.c_void_p()
+
+    def __del__(self):
+        try:
+            self.close()
+        except Exception:
+            pass
+
+    def add_conv2d(self, desc, x, w, bias, residual, y):
+        _check(lib().kxc_hip_plan_add_conv2d(self._h, C.byref(desc), x, w, bias, residual, y))
+
+    def add_pool2d(self, desc, x, y):
+        _check(lib().kxc_hip_plan_add_pool2d(self._h, C.byref(desc), x, y))
+
+    def add_global_avg_pool2d(self, n, c, h, w, x, y):
+        _check(lib().kxc_hip_plan_add_global_avg_pool2d(self._h, C.c_int64(n), C.c_int64(c), C.c_int64(h), C.c_int64(w), x, y))
+
+    def add_gemm(self, m, n, k, alpha, beta, transB, c_len, a, b, c, y):
+        _check(lib().kxc_hip_plan_add_gemm(self._h, C.c_int64(m), C.c_int64(n), C.c_int64(k), C.c_float(alpha),
+                                           C.c_float(beta), C.c_int32(transB), C.c_int64(c_len), a, b, c, y))
+
+    def add_binary(self, op, a_shape, b_shape, relu, a, b, y):
+        sa = (C.c_int64 * max(1, len(a_shape)))(*a_shape); sb = (C.c_int64 * max(1, len(b_shape)))(*b_shape)
+        _check(lib().kxc_hip_plan_add_binary(self._h, C.c_int32(op), sa, C.c_int32(len(a_shape)), sb,
+                                             C.c_int32(len(b_shape)), C.c_int32(int(relu)), a, b, y))
+
+    def add_relu(self, n, x, y):
+        _check(lib().kxc_hip_plan_add_relu(self._h, C.c_int64(n), x, y))
+
+    def add_copy(self, nbytes, x, y):
+        _check(lib().kxc_hip_plan_add_copy(self._h, C.c_int64(nbytes), x, y))
+
+    def add_qconv2d(self, desc, x, w, bias, mult, residual, y):
+        _check(lib().kxc_hip_plan_add_qconv2d(self._h, C.byref(desc), x, w, bias, mult, residual, y))
+
+    def add_quantize(self, n, scale, x, q):
+        _check(lib().kxc_hip_plan_add_quantize(self._h, C.c_int64(n), C.c_float(scale), x, q))
+
+    def add_maxpool2d_i8(self, desc, x, y):
+        _check(lib().kxc_hip_plan_add_maxpool2d_i8(self._h, C.byref(desc), x, y))
+
+    def add_global_avg_pool2d_i8(self, n, c, h, w, mult, x, y):
+        _check(lib().kxc_hip_plan_add_global_avg_pool2d_i8(self._h, C.c_int64(n), C.c_int64(c), C.c_int64(h),
+                                                           C.c_int64(w), C.c_float(mult), x, y))
+
+    def add_qdense(self, m, n, k, a, b, bias, mult, y):
+        _check(lib().kxc_hip_plan_add_qdense(self._h, C.c_int64(m), C.c_int64(n), C.c_int64(k), a, b, bias, mult, y))
+
+    def finalize(self, workspace_bytes):
+        _check(lib().kxc_hip_plan_finalize(self._h, C.c_size_t(workspace_bytes)))
+
+    def run(self, tensors, stream=None):
+        """tensors: the packed arguments (inputs, constants, outputs) as GPU tensors."""
+        args = (C.c_void_p * len(tensors))(*[t.data_ptr() for t in tensors])
+        s = C.c_void_p(stream) if stream is not None else _stream()
+        _check(lib().kxc_hip_plan_run(self._h, args, s))
+
+    def packed(self, tensors):
+        return (C.c_void_p * len(tensors))(*[t.data_ptr() for t in tensors])
+
+    def run_packed(self, args, stream):
+        _check(lib().kxc_hip_plan_run(self._h, args, C.c_void_p(stream)))
+
+    def symbols(self):
+        n = lib().kxc_hip_plan_num_nodes(self._h)
+        return [lib().kxc_hip_plan_node_symbol(self._h, C.c_int32(i)).decode() for i in range(n)]
+
+    def workspace_ptr(self):
+        return lib().kxc_hip_plan_workspace(self._h)

@@ -1,0 +1,263 @@
+/*
+ * kxc_hip.h -- C ABI of libkxc_hip.so, the MI355X (gfx950) backend for the
+ * kxc compiler's lowered-operator hot path.
+ *
+ * Plain C: pointers, sizes and POD structs only.  Every data pointer passed to
+ * an operator is a DEVICE pointer (from kxc_hip_alloc or any other HIP
+ * allocation); `stream` is a hipStream_t passed as void* (NULL = the calling
+ * thread's current stream set with kxc_hip_set_stream, else the null stream).
+ * Every entry point returns 0 on success and a non-zero code on failure; the
+ * message is then available from kxc_hip_last_error() on the same thread.
+ * Operators only enqueue work; they do not synchronise.
+ *
+ * Each declaration cites the reference interface (relative to the reference
+ * checkout) that it implements on the GPU or that would bind it.
+ */
+#ifndef KXC_HIP_H_
+#define KXC_HIP_H_
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define KXC_HIP_OK 0
+#define KXC_HIP_ERR_INVALID 1      /* bad argument / unsupported shape */
+#define KXC_HIP_ERR_RUNTIME 2      /* a HIP runtime call failed */
+#define KXC_HIP_ERR_COMPILE 3      /* hipRTC compilation failed */
+#define KXC_HIP_ERR_NO_DEVICE 4    /* no usable GPU */
+
+/* Message of the last failure on the calling thread ("" if none). */
+const char* kxc_hip_last_error(void);
+/* ABI version of this library (bumped on incompatible changes). */
+int32_t kxc_hip_abi_version(void);
+
+/* ========================================================================
+ * 1. Device API -- the calls a HIPDeviceAPI subclass of the reference's
+ *    DeviceAPI (include/base/device_api.h:77-123) forwards to, one for one
+ *    with CUDADeviceAPI (src/base/device/cuda_device_api.cc:75-328).
+ * ===================================================================== */
+
+/* DeviceAttributes (include/base/device_api.h:42-63) as a POD. */
+typedef struct kxc_hip_device_attrs {
+    int32_t exists;                      /* 0 when no device / no runtime; never an error */
+    int32_t warp_size;                   /* 64 on gfx950 */
+    int64_t max_threads_per_block;
+    int64_t max_shared_memory_per_block; /* LDS bytes a workgroup may use */
+    int64_t max_shared_memory_per_multiprocessor;
+    int64_t multi_processor_count;       /* compute units */
+    int64_t max_clock_rate_khz;
+    int64_t max_registers_per_block;
+    int64_t l2_cache_size_bytes;
+    int64_t total_global_memory;
+    int64_t available_global_memory;
+    int64_t max_threads_per_multiprocessor;
+    int32_t compute_version_major;
+    int32_t compute_version_minor;
+    int32_t api_version;
+    int32_t driver_version;
+    char device_name[128];
+    char arch[32];                       /* "gfx950" */
+    char status[128];                    /* reason text when exists == 0 */
+} kxc_hip_device_attrs;
+
+/* GetTargetKind (cuda_device_api.cc:218-221 returns "cuda"): returns "hip". */
+const char* kxc_hip_target_kind(void);
+/* Device enumeration (src/base/device_api.cc:344,395-402).  *count = 0 without a GPU. */
+int32_t kxc_hip_device_count(int32_t* count);
+/* GetDeviceAttributes (cuda_device_api.cc:159-216): never fails, exists = 0 + status text instead. */
+int32_t kxc_hip_device_attributes(int32_t device_id, kxc_hip_device_attrs* out);
+/* SetDevice (cuda_device_api.cc:77-88). */
+int32_t kxc_hip_set_device(int32_t device_id);
+/* AllocDataSpace / FreeDataSpace (cuda_device_api.cc:90-114); alignment <= 256 is always met. */
+int32_t kxc_hip_alloc(int32_t device_id, size_t nbytes, size_t alignment, void** out_ptr);
+int32_t kxc_hip_free(int32_t device_id, void* ptr);
+/* CopyDataFromTo with offsets and stream (cuda_device_api.cc:122-157).
+ * kind: 0 host->device, 1 device->host, 2 device->device, 3 host->host.
+ * stream NULL and no current stream: synchronous copy. */
+int32_t kxc_hip_copy(const void* from, size_t from_offset, void* to, size_t to_offset,
+                     size_t nbytes, int32_t kind, int32_t device_id, void* stream);
+/* CreateStream / FreeStream / SetStream / GetCurrentStream / StreamSync /
+ * SyncStreamFromTo (cuda_device_api.cc:223-328).  The current stream is per thread.
+ * kxc_hip_stream_sync(dev, NULL) with no current stream synchronises the whole device. */
+int32_t kxc_hip_stream_create(int32_t device_id, void** out_stream);
+int32_t kxc_hip_stream_destroy(int32_t device_id, void* stream);
+int32_t kxc_hip_set_stream(int32_t device_id, void* stream);
+int32_t kxc_hip_get_stream(int32_t device_id, void** out_stream);
+int32_t kxc_hip_stream_sync(int32_t device_id, void* stream);
+int32_t kxc_hip_stream_wait(int32_t device_id, void* src_stream, void* dst_stream);
+
+/* ========================================================================
+ * 2. Hand-written operators.  Each is the GPU implementation of one
+ *    FRelayToTE compute definition (the CPU definition stays the fallback).
+ * ===================================================================== */
+
+#define KXC_HIP_CONV_BIAS 1u       /* + bias[o]              (convolution.cc:72-74)            */
+#define KXC_HIP_CONV_RESIDUAL 2u   /* + residual[n,o,h,w]    (add(conv_out, skip), math.cc:41-47) */
+#define KXC_HIP_CONV_RELU 4u       /* (v > 0) ? v : 0        (nn.h:19-30)                      */
+#define KXC_HIP_CONV_FORCE_DIRECT 0x100u /* use the one-thread-per-output kernel (reference order) */
+
+/* nn_conv2d: Conv2DCompute (src/relay/op/nn/convolution.cc:38-75) ->
+ * topi::conv2d_nchw (include/te/topi/nn.h:107-158); shapes by Conv2DInferType
+ * (src/relay/type_infer.cc:346-400).  x [n,c,h,w], w [o,c,kh,kw], y [n,o,oh,ow].
+ * The fused epilogue applies, in the reference chain's order, bias, residual
+ * add (conv_out + residual), ReLU; each one rounded fp32 operation. */
+typedef struct kxc_hip_conv2d_desc {
+    int32_t n, c, h, w;
+    int32_t o, kh, kw;
+    int32_t stride_h, stride_w;
+    int32_t pad_h, pad_w;            /* padding[0], padding[1], applied to both sides (convolution.cc:53-54) */
+    int32_t dil_h, dil_w;
+    uint32_t flags;
+} kxc_hip_conv2d_desc;
+int32_t kxc_hip_conv2d_nchw_f32(const kxc_hip_conv2d_desc* desc, const float* x, const float* w,
+                                const float* bias, const float* residual, float* y, void* stream);
+/* Name of the kernel variant the library would launch for this shape ("mfma_..." or "direct"). */
+const char* kxc_hip_conv2d_variant(const kxc_hip_conv2d_desc* desc);
+
+/* nn_relu: ReluCompute (src/relay/op/nn/activation.cc:14-19). */
+int32_t kxc_hip_relu_f32(const float* x, float* y, int64_t n, void* stream);
+/* add / subtract / multiply / divide: broadcast.h:90-113 via math.cc:41-95.
+ * op 0..3; shapes right-aligned, ndim <= 6; relu != 0 fuses a following nn_relu. */
+int32_t kxc_hip_broadcast_binary_f32(int32_t op, const float* a, const int64_t* a_shape, int32_t a_ndim,
+                                     const float* b, const int64_t* b_shape, int32_t b_ndim,
+                                     float* y, int32_t relu, void* stream);
+/* T_conv2d_bias_add on its own (convolution.cc:72-74): y[n,o,:] = x[n,o,:] + bias[o]. */
+int32_t kxc_hip_bias_add_nchw_f32(const float* x, const float* bias, float* y,
+                                  int64_t n, int64_t o, int64_t hw, int32_t relu, void* stream);
+
+/* nn_max_pool2d / nn_avg_pool2d: MaxPool2DCompute / AvgPool2DCompute
+ * (src/relay/op/nn/pooling.cc:50-86) -> topi::pool2d (nn.h:161-258). */
+typedef struct kxc_hip_pool2d_desc {
+    int32_t n, c, h, w;
+    int32_t kh, kw, stride_h, stride_w;
+    int32_t pad_top, pad_left, pad_bottom, pad_right;
+    int32_t ceil_mode;
+    int32_t is_avg;                  /* 0 max, 1 avg */
+} kxc_hip_pool2d_desc;
+int32_t kxc_hip_pool2d_f32(const kxc_hip_pool2d_desc* desc, const float* x, float* y, void* stream);
+
+/* nn_global_avg_pool2d: GlobalAvgPool2DCompute (pooling.cc:88-98) -> nn.h:260-287. */
+int32_t kxc_hip_global_avg_pool2d_f32(const float* x, float* y, int64_t n, int64_t c, int64_t h,
+                                      int64_t w, void* stream);
+
+/* nn_dense (DenseCompute, src/relay/op/nn/dense.cc:27-32) and nn_gemm (GemmCompute :34-61):
+ * y[m,n] = alpha * sum_k a[m,k]*b[n,k] (transB=1) or a[m,k]*b[k,n] (transB=0), + beta*c[n].
+ * c may be NULL (nn_dense); c_len is n or 1. */
+int32_t kxc_hip_gemm_f32(const float* a, const float* b, const float* c, float* y,
+                         int64_t m, int64_t n, int64_t k, float alpha, float beta,
+                         int32_t transB, int64_t c_len, void* stream);
+
+/* nn_flatten (FlattenCompute, src/relay/op/tensor/transform.cc:140-182): a row-major copy.
+ * (Inside a launch plan a flatten is an alias and launches nothing.) */
+int32_t kxc_hip_flatten_f32(const float* x, float* y, int64_t n, void* stream);
+
+/* ---- int8 family.  The reference has no quantised operator; these implement the
+ *      definition in oracle/kxc_oracle.h (qnn-style conv/dense with int32 accumulate and
+ *      per-output-channel fp32 requantisation, round half to even). ---- */
+int32_t kxc_hip_quantize_f32_i8(const float* x, int8_t* q, int64_t n, float scale, void* stream);
+typedef struct kxc_hip_qconv2d_desc {
+    int32_t n, c, h, w;
+    int32_t o, kh, kw;
+    int32_t stride_h, stride_w;
+    int32_t pad_h, pad_w;
+    uint32_t flags;                  /* KXC_HIP_CONV_BIAS | _RESIDUAL | _RELU | _FORCE_DIRECT */
+    float res_mult;
+} kxc_hip_qconv2d_desc;
+int32_t kxc_hip_qconv2d_nchw_i8(const kxc_hip_qconv2d_desc* desc, const int8_t* x, const int8_t* w,
+                                const int32_t* bias, const float* mult, const int8_t* residual,
+                                int8_t* y, void* stream);
+int32_t kxc_hip_qdense_i8(const int8_t* a, const int8_t* b, const int32_t* bias, const float* mult,
+                          float* y, int64_t m, int64_t n, int64_t k, void* stream);
+int32_t kxc_hip_maxpool2d_i8(const kxc_hip_pool2d_desc* desc, const int8_t* x, int8_t* y, void* stream);
+int32_t kxc_hip_global_avg_pool2d_i8(const int8_t* x, int8_t* y, int64_t n, int64_t c, int64_t h,
+                                     int64_t w, float mult, void* stream);
+
+/* ========================================================================
+ * 3. Module loader -- run-time compiled kernels (the TIR->HIP emitter's output).
+ *    Mirrors the only device-code launch site in the reference, an NVRTC +
+ *    cuLaunchKernel sequence (test/cupti_smoke_test.cpp:143-205), and is what a
+ *    HIP CompiledKernelNode (include/codegen/compiled_kernel.h:19-41) owns.
+ * ===================================================================== */
+typedef struct kxc_hip_module kxc_hip_module;   /* opaque */
+/* hipRTC-compile `source` for gfx950 and load it.  log (may be NULL) receives the compiler log. */
+int32_t kxc_hip_module_compile(const char* source, const char* name, kxc_hip_module** out,
+                               char* log, size_t log_capacity);
+/* Compile only (no GPU needed): code object size in *out_size; used by build-time checks. */
+int32_t kxc_hip_module_compile_only(const char* source, const char* name, size_t* out_size,
+                                    char* log, size_t log_capacity);
+int32_t kxc_hip_module_get_function(kxc_hip_module* module, const char* symbol, void** out_function);
+/* hipModuleLaunchKernel(f, grid, block, shared_bytes, stream, kernel_params, NULL). */
+int32_t kxc_hip_module_launch(void* function, const uint32_t grid[3], const uint32_t block[3],
+                              uint32_t shared_bytes, void* stream, void** kernel_params);
+int32_t kxc_hip_module_free(kxc_hip_module* module);
+
+/* ========================================================================
+ * 4. Launch plan -- the kernel-launch half of the reference's ExecutionPlan
+ *    (include/base/execution_plan.h:42-50,102-130; its executor only copies
+ *    buffers, src/base/disco/executor.cc:122-157).  One plan = the body of one
+ *    compiled function `int32_t kxc_kernel_main(void** packed_args)`
+ *    (src/codegen/compiled_kernel.cc:41-55): a list of launches on ONE stream
+ *    over buffers that are either caller arguments or slots of a workspace the
+ *    plan owns (allocated once, no per-run allocation).
+ * ===================================================================== */
+typedef struct kxc_hip_plan kxc_hip_plan;       /* opaque */
+
+/* A buffer operand: packed_args[index] (kind 0), byte offset into the plan
+ * workspace (kind 1), or absent (kind 2, e.g. no bias). */
+typedef struct kxc_hip_buf {
+    int32_t kind;
+    int64_t index_or_offset;
+} kxc_hip_buf;
+#define KXC_HIP_BUF_ARG 0
+#define KXC_HIP_BUF_WORKSPACE 1
+#define KXC_HIP_BUF_NONE 2
+
+int32_t kxc_hip_plan_create(int32_t device_id, int32_t num_packed_args, kxc_hip_plan** out);
+int32_t kxc_hip_plan_destroy(kxc_hip_plan* plan);
+/* Node builders; `symbol` is stored as KernelExecNode::kernel_symbol would be. */
+int32_t kxc_hip_plan_add_conv2d(kxc_hip_plan* plan, const kxc_hip_conv2d_desc* desc, kxc_hip_buf x,
+                                kxc_hip_buf w, kxc_hip_buf bias, kxc_hip_buf residual, kxc_hip_buf y);
+int32_t kxc_hip_plan_add_pool2d(kxc_hip_plan* plan, const kxc_hip_pool2d_desc* desc, kxc_hip_buf x,
+                                kxc_hip_buf y);
+int32_t kxc_hip_plan_add_global_avg_pool2d(kxc_hip_plan* plan, int64_t n, int64_t c, int64_t h,
+                                           int64_t w, kxc_hip_buf x, kxc_hip_buf y);
+int32_t kxc_hip_plan_add_gemm(kxc_hip_plan* plan, int64_t m, int64_t n, int64_t k, float alpha,
+                              float beta, int32_t transB, int64_t c_len, kxc_hip_buf a,
+                              kxc_hip_buf b, kxc_hip_buf c, kxc_hip_buf y);
+int32_t kxc_hip_plan_add_binary(kxc_hip_plan* plan, int32_t op, const int64_t* a_shape,
+                                int32_t a_ndim, const int64_t* b_shape, int32_t b_ndim, int32_t relu,
+                                kxc_hip_buf a, kxc_hip_buf b, kxc_hip_buf y);
+int32_t kxc_hip_plan_add_relu(kxc_hip_plan* plan, int64_t n, kxc_hip_buf x, kxc_hip_buf y);
+int32_t kxc_hip_plan_add_copy(kxc_hip_plan* plan, int64_t nbytes, kxc_hip_buf x, kxc_hip_buf y);
+int32_t kxc_hip_plan_add_qconv2d(kxc_hip_plan* plan, const kxc_hip_qconv2d_desc* desc, kxc_hip_buf x,
+                                 kxc_hip_buf w, kxc_hip_buf bias, kxc_hip_buf mult,
+                                 kxc_hip_buf residual, kxc_hip_buf y);
+int32_t kxc_hip_plan_add_quantize(kxc_hip_plan* plan, int64_t n, float scale, kxc_hip_buf x, kxc_hip_buf q);
+int32_t kxc_hip_plan_add_maxpool2d_i8(kxc_hip_plan* plan, const kxc_hip_pool2d_desc* desc,
+                                      kxc_hip_buf x, kxc_hip_buf y);
+int32_t kxc_hip_plan_add_global_avg_pool2d_i8(kxc_hip_plan* plan, int64_t n, int64_t c, int64_t h,
+                                              int64_t w, float mult, kxc_hip_buf x, kxc_hip_buf y);
+int32_t kxc_hip_plan_add_qdense(kxc_hip_plan* plan, int64_t m, int64_t n, int64_t k, kxc_hip_buf a,
+                                kxc_hip_buf b, kxc_hip_buf bias, kxc_hip_buf mult, kxc_hip_buf y);
+/* A run-time compiled kernel (section 3): params[i] is a buffer operand, passed as a pointer. */
+int32_t kxc_hip_plan_add_module_kernel(kxc_hip_plan* plan, void* function, const char* symbol,
+                                       const uint32_t grid[3], const uint32_t block[3],
+                                       uint32_t shared_bytes, const kxc_hip_buf* params,
+                                       int32_t num_params);
+/* Allocate the workspace (bytes = the largest offset + size the nodes use). */
+int32_t kxc_hip_plan_finalize(kxc_hip_plan* plan, size_t workspace_bytes);
+/* Enqueue every node on `stream`; returns after enqueue (no synchronisation). */
+int32_t kxc_hip_plan_run(kxc_hip_plan* plan, void** packed_args, void* stream);
+int32_t kxc_hip_plan_num_nodes(const kxc_hip_plan* plan);
+/* kernel_symbol of node i (static storage owned by the plan). */
+const char* kxc_hip_plan_node_symbol(const kxc_hip_plan* plan, int32_t i);
+/* Device address of the workspace (NULL before finalize): lets tests read intermediates. */
+void* kxc_hip_plan_workspace(const kxc_hip_plan* plan);
+
+#ifdef __cplusplus
+}
+#endif
+#endif  /* KXC_HIP_H_ */
