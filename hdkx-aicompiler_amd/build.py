@@ -23,6 +23,9 @@ HIPCC = os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")
 FLAGS = ["-O3", "--offload-arch=gfx950", "-fPIC", "-std=c++17", "-I" + os.path.join(ROOT, "include"),
          # packed fp32 instructions are kept out of every kernel
          "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
+         # no multiply-add contraction anywhere: the reference-order kernels must round every multiply
+         # and add separately like the CPU backend (HIP's __fmul_rn/__fadd_rn do not prevent fusion)
+         "-ffp-contract=off",
          "-Wall", "-Wno-unused-function"]
 
 

@@ -167,7 +167,7 @@ def test_conv_full_batch_properties(pkg, synth):
     assert_close(host(fast), host(slow), what="layer1 batch 64")
     y12 = pkg.conv2d(x, w1 + w2, None, None, 1, 1)
     y1 = pkg.conv2d(x, w1, None, None, 1, 1); y2 = pkg.conv2d(x, w2, None, None, 1, 1)
-    assert_close(host(y12), host(y1 + y2), tol=1e-4, what="linearity")
+    assert_close(host(y12), host(y1 + y2), what="linearity")
     one = pkg.conv2d(x[17:18].contiguous(), w1, b, None, 1, 1, 1, True)
     assert_close(host(one), host(fast[17:18]), tol=1e-5, what="batch independence")
 
@@ -295,10 +295,10 @@ def _run_plan(pkg, batch, hw, config, fuse=True):
 def test_resnet18_small_image(pkg, fast_orc):
     x, consts, got, info = _run_plan(pkg, 2, 64, 3)
     want = fast_orc.resnet18(x, consts)
-    assert_close(got, want, what="resnet18 64x64 logits")
+    assert_close(got, want, what="resnet18 64x64 logits", floor="scale")
     assert len(info["launches"]) == 23
     x, consts, got2, info2 = _run_plan(pkg, 2, 64, 3, fuse=False)
-    assert_close(got2, want, what="resnet18 64x64 logits (unfused launches)")
+    assert_close(got2, want, what="resnet18 64x64 logits (unfused launches)", floor="scale")
     assert len(info2["launches"]) > 23
 
 
@@ -306,7 +306,7 @@ def test_resnet18_batch1_224(pkg, fast_orc):
     """BASELINE configuration 3: full ResNet-18 at batch 1, logits within 1e-3 of the CPU path."""
     x, consts, got, info = _run_plan(pkg, 1, 224, 3)
     want = fast_orc.resnet18(x, consts)
-    assert_close(got, want, what="resnet18 224 logits")
+    assert_close(got, want, what="resnet18 224 logits", floor="scale")
     assert int(np.argmax(got)) == int(np.argmax(want))
 
 
@@ -319,4 +319,4 @@ def test_resnet18_batch64_properties(pkg, fast_orc):
     assert np.isfinite(got).all()
     for n in (0, 63):
         want = fast_orc.resnet18(x[n:n + 1], consts)
-        assert_close(got[n:n + 1], want, what="resnet18 batch 64, image %d" % n)
+        assert_close(got[n:n + 1], want, what="resnet18 batch 64, image %d" % n, floor="scale")
