@@ -52,6 +52,7 @@ struct ConvArgs {
     int32_t OHW;
     int32_t chs;         // LDS floats per patch channel (>= rows*Wp, padded)
     int32_t nchunks;     // ceil(C / CC)
+    uint32_t x_bytes, w_bytes;
     uint32_t flags;
 };
 
@@ -59,30 +60,48 @@ __device__ __forceinline__ float relu_sel(float v) { return (v > 0.0f) ? v : 0.0
 
 // ------------------------------------------------------------------------------------------
 // MFMA kernel.  KH,KW: filter; CC: channels per LDS chunk (even); WO x WP waves, each wave
-// RO x RP blocks of 32x32; PPT: patch positions per thread (upper bound, checked on the host).
+// RO x RP blocks of 32x32; PPT: 64-float patch segments per wave per channel (upper bound,
+// checked on the host).
+//
+// Both LDS tiles are filled by buffer loads that write straight to LDS (buffer_load_dword ... lds):
+// lane l of a wave writes LDS float (segment base + l), its global byte offset comes from a
+// per-thread table computed once, and the chunk's channel offset is the instruction's scalar
+// offset.  Table entries for padding / out-of-tile positions hold an offset beyond the buffer,
+// for which the hardware returns 0 -- zero padding costs no branch and no select, and the loads
+// need no staging registers: they run while the matrix cores work on the other LDS buffer.
 // ------------------------------------------------------------------------------------------
+constexpr uint32_t kOobOffset = 0x80000000u;   // beyond any buffer this kernel accepts (< 2 GiB)
+
+__device__ __forceinline__ __amdgpu_buffer_rsrc_t make_rsrc(const void* p, uint32_t bytes) {
+    return __builtin_amdgcn_make_buffer_rsrc(const_cast<void*>(p), 0, static_cast<int>(bytes), 0x00020000);
+}
+
+typedef __attribute__((address_space(3))) void* lds_ptr_t;
+
 template <int KH, int KW, int CC, int WO, int WP, int RO, int RP, int PPT>
 __global__ void __launch_bounds__(64 * WO * WP)
 conv_mfma_kernel(const ConvArgs a) {
-    constexpr int NT = 64 * WO * WP;
+    constexpr int NW = WO * WP;
     constexpr int TO = 32 * RO * WO;
     constexpr int TP = 32 * RP * WP;
     constexpr int KHW = KH * KW;
-    constexpr int KC = CC * KHW;                 // k values per chunk
-    constexpr int KS = KC | 1;                   // odd LDS row stride for the weight tile
-    constexpr int WPT = (TO * KC + NT - 1) / NT; // weight elements per thread per chunk
+    constexpr int KS2 = ((CC / 2) * KHW) | 1;                 // odd row stride of one weight plane
+    constexpr int PL = (TO * KS2 + 63) / 64 * 64 + 32;        // plane stride: 32 mod 64
+    constexpr int WSZ = 2 * PL;                               // floats in the weight tile (multiple of 64)
+    constexpr int WSEG = WSZ / 64;                            // 64-float segments of the weight tile
+    constexpr int WPT = (WSEG + NW - 1) / NW;                 // weight segments per wave
 
     extern __shared__ float lds[];
-    const int xs_size = CC * a.chs;
-    float* xs0 = lds;
+    const int xs_size = CC * a.chs;                           // multiple of 32; tiles start 128-byte aligned
     // layout: [xs0][ws0][xs1][ws1]; the second pair exists only when there is more than one chunk
-    float* xs1 = lds + xs_size + TO * KS;
-    float* ws0 = lds + xs_size;
-    float* ws1 = xs1 + xs_size;
+    float* const xs0 = lds;
+    float* const ws0 = lds + xs_size;
+    float* const xs1 = ws0 + WSZ;
+    float* const ws1 = xs1 + xs_size;
 
     const int tid = threadIdx.x;
     const int lane = tid & 63;
-    const int wave = tid >> 6;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int wave_o = wave / WP;
     const int wave_p = wave % WP;
     const int half = lane >> 5;
@@ -101,20 +120,40 @@ conv_mfma_kernel(const ConvArgs a) {
         const int n2 = m_last / a.OHW, rem2 = m_last - n2 * a.OHW;
         qlast = n2 * a.Hp + (rem2 / a.OW) * a.sh + (KH - 1) * a.dh;
     }
-    const int P = (qlast - qmin + 1) * a.Wp;      // patch positions per channel (<= chs, <= PPT*NT)
+    const int P = (qlast - qmin + 1) * a.Wp;      // patch positions per channel (<= chs - 32)
+    const int xsegs = (P + 63) >> 6;              // 64-float segments per channel
     const int HW = a.H * a.W;
 
-    // ---- per-thread patch positions: global offset inside channel 0 (or -1 for padding)
-    int goff[PPT];
+    const __amdgpu_buffer_rsrc_t xr = make_rsrc(a.x, a.x_bytes);
+    const __amdgpu_buffer_rsrc_t wr = make_rsrc(a.w, a.w_bytes);
+
+    // ---- per-thread load tables (byte offsets; kOobOffset reads as 0)
+    uint32_t goff[PPT];
 #pragma unroll
     for (int i = 0; i < PPT; ++i) {
-        const int pos = tid + i * NT;
+        const int pos = (wave + i * NW) * 64 + lane;
         const int q = pos / a.Wp, col = pos - q * a.Wp;
         const int Q = qmin + q;
         const int n = Q / a.Hp, ih = Q - n * a.Hp - a.ph, iw = col - a.pw;
         const bool ok = pos < P && n < a.N && ih >= 0 && ih < a.H && iw >= 0 && iw < a.W;
-        goff[i] = ok ? ((n * a.C) * a.H + ih) * a.W + iw : -1;
+        goff[i] = ok ? static_cast<uint32_t>(((n * a.C) * a.H + ih) * a.W + iw) * 4u : kOobOffset;
     }
+    // weight tile element L = plane*PL + row*KS2 + col, col = pair*KHW + tap, channel = 2*pair + plane
+    uint32_t woff[WPT];
+    auto weight_table = [&](int channels_left) {
+#pragma unroll
+        for (int i = 0; i < WPT; ++i) {
+            const int L = (wave + i * NW) * 64 + lane;
+            const int plane = L >= PL ? 1 : 0;
+            const int rem = L - plane * PL;
+            const int row = rem / KS2, col = rem - row * KS2;
+            const int pair = col / KHW, tap = col - pair * KHW;
+            const int cl = 2 * pair + plane;
+            const bool ok = L < WSZ && row < TO && col < (CC / 2) * KHW && (o0 + row) < a.O && cl < channels_left;
+            woff[i] = ok ? static_cast<uint32_t>(((o0 + row) * a.C + cl) * KHW + tap) * 4u : kOobOffset;
+        }
+    };
+    weight_table(min(CC, a.C));
 
     // ---- per-lane operand bases
     int xbase[RP];
@@ -130,7 +169,7 @@ conv_mfma_kernel(const ConvArgs a) {
     }
     int wbase[RO];
 #pragma unroll
-    for (int i = 0; i < RO; ++i) wbase[i] = ((wave_o * RO + i) * 32 + r) * KS + half * KHW;
+    for (int i = 0; i < RO; ++i) wbase[i] = half * PL + ((wave_o * RO + i) * 32 + r) * KS2;
 
     floatx16 acc[RO][RP];
 #pragma unroll
@@ -140,52 +179,46 @@ conv_mfma_kernel(const ConvArgs a) {
 #pragma unroll
             for (int g = 0; g < 16; ++g) acc[i][j][g] = 0.0f;
 
-    float xreg[CC][PPT];
-    float wreg[WPT];
-
-    auto load_chunk = [&](int chunk) {
+    auto issue_loads = [&](int chunk, float* xs, float* ws) {
         const int c0 = chunk * CC;
+        if (c0 + CC > a.C && chunk > 0) weight_table(a.C - c0);   // partial last chunk (rare)
 #pragma unroll
         for (int cl = 0; cl < CC; ++cl) {
-            const bool cok = (c0 + cl) < a.C;
+            if (c0 + cl < a.C) {
+                const uint32_t soff = static_cast<uint32_t>(c0 + cl) * static_cast<uint32_t>(HW) * 4u;
 #pragma unroll
-            for (int i = 0; i < PPT; ++i)
-                xreg[cl][i] = (cok && goff[i] >= 0) ? a.x[goff[i] + (c0 + cl) * HW] : 0.0f;
-        }
+                for (int i = 0; i < PPT; ++i) {
+                    const int seg = wave + i * NW;
+                    if (seg < xsegs)
+                        __builtin_amdgcn_raw_ptr_buffer_load_lds(xr, (lds_ptr_t)(xs + cl * a.chs + seg * 64), 4,
+                                                                 goff[i], soff, 0, 0);
+                }
+            } else {
+                // channel beyond C: zero plane (the matching weights are zero too, keep the product exact)
 #pragma unroll
-        for (int i = 0; i < WPT; ++i) {
-            const int e = tid + i * NT;
-            const int ol = e / KC, kk = e - ol * KC;
-            const int cl = kk / KHW;
-            const bool ok = e < TO * KC && (o0 + ol) < a.O && (c0 + cl) < a.C;
-            wreg[i] = ok ? a.w[((o0 + ol) * a.C + c0) * KHW + kk] : 0.0f;
-        }
-    };
-    auto store_chunk = [&](float* xs, float* ws) {
-#pragma unroll
-        for (int cl = 0; cl < CC; ++cl)
-#pragma unroll
-            for (int i = 0; i < PPT; ++i) {
-                const int pos = tid + i * NT;
-                if (pos < P) xs[cl * a.chs + pos] = xreg[cl][i];
+                for (int i = 0; i < PPT; ++i) {
+                    const int seg = wave + i * NW;
+                    if (seg < xsegs) xs[cl * a.chs + seg * 64 + lane] = 0.0f;
+                }
             }
+        }
+        const uint32_t wsoff = static_cast<uint32_t>(c0) * KHW * 4u;
 #pragma unroll
         for (int i = 0; i < WPT; ++i) {
-            const int e = tid + i * NT;
-            const int ol = e / KC, kk = e - ol * KC;
-            if (e < TO * KC) ws[ol * KS + kk] = wreg[i];
+            const int seg = wave + i * NW;
+            if (seg < WSEG)
+                __builtin_amdgcn_raw_ptr_buffer_load_lds(wr, (lds_ptr_t)(ws + seg * 64), 4, woff[i], wsoff, 0, 0);
         }
     };
 
-    load_chunk(0);
-    store_chunk(xs0, ws0);
+    issue_loads(0, xs0, ws0);
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
     __syncthreads();
 
     for (int chunk = 0; chunk < a.nchunks; ++chunk) {
         const float* xs = (chunk & 1) ? xs1 : xs0;
         const float* ws = (chunk & 1) ? ws1 : ws0;
-        const bool more = (chunk + 1) < a.nchunks;
-        if (more) load_chunk(chunk + 1);
+        if (chunk + 1 < a.nchunks) issue_loads(chunk + 1, (chunk & 1) ? xs0 : xs1, (chunk & 1) ? ws0 : ws1);
 
 #pragma unroll
         for (int cp = 0; cp < CC / 2; ++cp) {
@@ -194,7 +227,7 @@ conv_mfma_kernel(const ConvArgs a) {
 #pragma unroll
                 for (int rw = 0; rw < KW; ++rw) {
                     const int koff_x = (2 * cp) * a.chs + rh * a.dh * a.Wp + rw * a.dw;
-                    const int koff_w = (2 * cp) * KHW + rh * KW + rw;
+                    const int koff_w = cp * KHW + rh * KW + rw;
                     float av[RO], bv[RP];
 #pragma unroll
                     for (int i = 0; i < RO; ++i) av[i] = ws[wbase[i] + koff_w];
@@ -209,7 +242,7 @@ conv_mfma_kernel(const ConvArgs a) {
             }
         }
 
-        if (more) store_chunk((chunk & 1) ? xs0 : xs1, (chunk & 1) ? ws0 : ws1);
+        asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
         __syncthreads();
     }
 
@@ -278,26 +311,41 @@ __global__ void __launch_bounds__(256) conv_direct_kernel(const ConvArgs a, int3
 // ------------------------------------------------------------------------------------------
 struct Variant {
     const char* name;
-    int kh, kw, cc, to, tp, nt, ppt;
+    int kh, kw, cc, to, tp, nw, ppt;
     void (*kernel)(const ConvArgs);
 };
 
 #define KXC_VARIANT(KH, KW, CC, WO, WP, RO, RP, PPT)                                                   \
     {"mfma_k" #KH "x" #KW "_c" #CC "_o" #WO "x" #RO "_p" #WP "x" #RP, KH, KW, CC, 32 * RO * WO, 32 * RP * WP, \
-     64 * WO * WP, PPT, conv_mfma_kernel<KH, KW, CC, WO, WP, RO, RP, PPT>}
+     WO * WP, PPT, conv_mfma_kernel<KH, KW, CC, WO, WP, RO, RP, PPT>}
 
-// Ordered by preference (largest tile first); the host takes the first one that fits the shape
-// and fills the GPU.
+// name = mfma_k<filter>_c<channels per chunk>_o<waves x blocks along output channels>_p<waves x blocks
+// along pixels>; tile = 32*blocks*waves in each direction.
 const Variant kVariants[] = {
-    KXC_VARIANT(3, 3, 4, 1, 4, 2, 2, 4),   // 64 x 256
+    KXC_VARIANT(3, 3, 4, 1, 4, 2, 2, 4),   // 64 x 256, 4 waves of 64x64
+    KXC_VARIANT(3, 3, 4, 1, 8, 2, 1, 2),   // 64 x 256, 8 waves of 64x32
+    KXC_VARIANT(3, 3, 4, 1, 7, 2, 1, 2),   // 64 x 224
+    KXC_VARIANT(3, 3, 4, 1, 6, 2, 1, 3),   // 64 x 192
+    KXC_VARIANT(3, 3, 4, 1, 5, 2, 1, 3),   // 64 x 160
     KXC_VARIANT(3, 3, 4, 1, 4, 2, 1, 4),   // 64 x 128
+    KXC_VARIANT(3, 3, 4, 1, 3, 2, 1, 6),   // 64 x 96
+    KXC_VARIANT(3, 3, 4, 1, 2, 2, 2, 8),   // 64 x 128, 2 waves of 64x64
     KXC_VARIANT(3, 3, 4, 2, 2, 1, 1, 6),   // 64 x 64
     KXC_VARIANT(3, 3, 4, 1, 4, 1, 1, 4),   // 32 x 128
+    KXC_VARIANT(3, 3, 8, 1, 4, 2, 2, 4),   // 8-channel chunks
+    KXC_VARIANT(3, 3, 8, 1, 8, 2, 1, 2),
+    KXC_VARIANT(3, 3, 8, 1, 6, 2, 1, 3),
+    KXC_VARIANT(3, 3, 8, 1, 5, 2, 1, 3),
+    KXC_VARIANT(3, 3, 8, 1, 4, 2, 1, 4),
+    KXC_VARIANT(3, 3, 8, 2, 2, 1, 1, 6),
     KXC_VARIANT(1, 1, 8, 1, 4, 2, 2, 6),   // 64 x 256
     KXC_VARIANT(1, 1, 8, 1, 4, 2, 1, 4),   // 64 x 128
     KXC_VARIANT(1, 1, 8, 2, 2, 1, 1, 6),   // 64 x 64
     KXC_VARIANT(1, 1, 8, 1, 4, 1, 1, 4),   // 32 x 128
+    KXC_VARIANT(1, 1, 16, 1, 4, 2, 1, 4),
+    KXC_VARIANT(1, 1, 16, 2, 2, 1, 1, 6),
     KXC_VARIANT(7, 7, 4, 1, 4, 2, 1, 12),  // 64 x 128 (3 input channels padded to 4)
+    KXC_VARIANT(7, 7, 4, 1, 8, 2, 1, 8),   // 64 x 256
     KXC_VARIANT(7, 7, 4, 1, 4, 1, 1, 12),  // 32 x 128
 };
 constexpr int kNumVariants = sizeof(kVariants) / sizeof(kVariants[0]);
@@ -323,18 +371,21 @@ int32_t MaxTileRows(const ConvArgs& a, int kh, int tp) {
 }
 
 constexpr size_t kMaxLdsBytes = 160 * 1024;  // LDS of one gfx950 compute unit
-constexpr int64_t kFillTiles = 512;          // two workgroups per CU on 256 CUs
+constexpr int kNumCUs = 256;
 
 bool Fits(const Variant& v, const ConvArgs& a, Choice* out) {
     const int32_t rows = MaxTileRows(a, v.kh, v.tp);
     const int64_t P = static_cast<int64_t>(rows) * a.Wp;
-    if (P > static_cast<int64_t>(v.ppt) * v.nt) return false;
+    const int64_t segs = (P + 63) / 64;
+    if (segs > static_cast<int64_t>(v.ppt) * v.nw) return false;
     // Channel stride: a multiple of 64 floats plus 32, so the two half-waves (which read channels
     // c and c+1 at the same position) fall into different halves of the LDS banks.
-    const int32_t chs = static_cast<int32_t>((P + 63) / 64 * 64 + 32);
-    const int ks = (v.cc * v.kh * v.kw) | 1;
+    const int32_t chs = static_cast<int32_t>(segs * 64 + 32);
+    const int khw = v.kh * v.kw;
+    const int ks2 = ((v.cc / 2) * khw) | 1;
+    const int pl = (v.to * ks2 + 63) / 64 * 64 + 32;
     const int buffers = (a.C + v.cc - 1) / v.cc > 1 ? 2 : 1;   // a single chunk needs no second buffer
-    const size_t lds = buffers * (static_cast<size_t>(v.cc) * chs + static_cast<size_t>(v.to) * ks) * sizeof(float);
+    const size_t lds = buffers * (static_cast<size_t>(v.cc) * chs + 2 * static_cast<size_t>(pl)) * sizeof(float);
     if (lds > kMaxLdsBytes) return false;
     out->v = &v;
     out->chs = chs;
@@ -342,18 +393,27 @@ bool Fits(const Variant& v, const ConvArgs& a, Choice* out) {
     return true;
 }
 
+// Cost model: workgroups are spread over 256 CUs, so the launch takes about
+// ceil(tiles / CUs) tile times; a tile costs its matrix work plus the LDS fill, which is
+// amortised better by larger tiles.
+double Cost(const Variant& v, const ConvArgs& a) {
+    const int64_t tiles = CeilDiv(a.M, v.tp) * CeilDiv(a.O, v.to);
+    const double rounds = static_cast<double>(CeilDiv(tiles, kNumCUs));
+    return rounds * v.tp * v.to * (1.0 + 40.0 / v.tp + 12.0 / v.to);
+}
+
 // Picks the MFMA variant for a shape, or leaves choice.v == nullptr for the direct kernel.
 void Select(const ConvArgs& a, int kh, int kw, Choice* choice) {
     choice->v = nullptr;
     if (a.O < 32 || a.M < 32) return;
-    // int32 offsets inside the kernel
-    const int64_t x_elems = static_cast<int64_t>(a.N) * a.C * a.H * a.W;
+    // 32-bit byte offsets inside the kernel
+    const int64_t x_bytes = static_cast<int64_t>(a.N) * a.C * a.H * a.W * 4;
     const int64_t y_elems = static_cast<int64_t>(a.N) * a.O * a.OHW;
+    const int64_t w_bytes = static_cast<int64_t>(a.O) * a.C * kh * kw * 4;
     const int64_t q_rows = static_cast<int64_t>(a.N + 1) * a.Hp + kh * a.dh;
-    if (x_elems >= (1LL << 31) || y_elems >= (1LL << 31) || q_rows * a.Wp >= (1LL << 31)) return;
+    if (x_bytes >= (1LL << 31) || y_elems >= (1LL << 31) || w_bytes >= (1LL << 31) || q_rows * a.Wp >= (1LL << 31)) return;
     const char* forced = std::getenv("KXC_HIP_CONV_VARIANT");
-    Choice best;
-    int64_t best_tiles = -1;
+    double best_cost = 0.0;
     for (int i = 0; i < kNumVariants; ++i) {
         const Variant& v = kVariants[i];
         if (v.kh != kh || v.kw != kw) continue;
@@ -361,11 +421,9 @@ void Select(const ConvArgs& a, int kh, int kw, Choice* choice) {
         if (v.to > a.O) continue;                 // do not spend matrix work on absent output channels
         Choice c;
         if (!Fits(v, a, &c)) continue;
-        const int64_t tiles = CeilDiv(a.M, v.tp) * CeilDiv(a.O, v.to);
-        if (tiles >= kFillTiles) { *choice = c; return; }   // first (largest) tile that fills the chip
-        if (tiles > best_tiles) { best_tiles = tiles; best = c; }
+        const double cost = Cost(v, a);
+        if (!choice->v || cost < best_cost) { *choice = c; best_cost = cost; }
     }
-    *choice = best;
 }
 
 int32_t FillArgs(const kxc_hip_conv2d_desc* d, ConvArgs* a, const char* who) {
@@ -416,6 +474,8 @@ int32_t kxc_hip_conv2d_nchw_f32(const kxc_hip_conv2d_desc* desc, const float* x,
     KXC_HIP_REQUIRE(!(desc->flags & KXC_HIP_CONV_RESIDUAL) || residual,
                     "kxc_hip_conv2d_nchw_f32: residual flag without residual");
     a.x = x; a.w = w; a.bias = bias; a.res = residual; a.y = y;
+    a.x_bytes = static_cast<uint32_t>(static_cast<int64_t>(a.N) * a.C * a.H * a.W * 4);       // < 2 GiB on the MFMA path
+    a.w_bytes = static_cast<uint32_t>(static_cast<int64_t>(a.O) * a.C * desc->kh * desc->kw * 4);
     hipStream_t s = ResolveStream(stream);
 
     Choice c;
@@ -432,7 +492,7 @@ int32_t kxc_hip_conv2d_nchw_f32(const kxc_hip_conv2d_desc* desc, const float* x,
                                              static_cast<int>(c.lds_bytes)),
                          "hipFuncSetAttribute(MaxDynamicSharedMemorySize)");
         }
-        hipLaunchKernelGGL(c.v->kernel, grid, dim3(c.v->nt), c.lds_bytes, s, a);
+        hipLaunchKernelGGL(c.v->kernel, grid, dim3(64 * c.v->nw), c.lds_bytes, s, a);
         return CheckLaunch(c.v->name);
     }
     int64_t g = CeilDiv(total, 256);
