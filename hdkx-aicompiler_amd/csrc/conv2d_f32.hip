@@ -90,6 +90,8 @@ conv_mfma_kernel(const ConvArgs a) {
     constexpr int WSZ = 2 * PL;                               // floats in the weight tile (multiple of 64)
     constexpr int WSEG = WSZ / 64;                            // 64-float segments of the weight tile
     constexpr int WPT = (WSEG + NW - 1) / NW;                 // weight segments per wave
+    constexpr int NS = (CC / 2) * KHW;                        // matrix k-steps per chunk
+    constexpr int PF = (RO * RP >= 4) ? 1 : (RO * RP == 2 ? 2 : 3);   // operand prefetch distance in k-steps
 
     extern __shared__ float lds[];
     const int xs_size = CC * a.chs;                           // multiple of 32; tiles start 128-byte aligned
@@ -220,30 +222,46 @@ conv_mfma_kernel(const ConvArgs a) {
         const float* ws = (chunk & 1) ? ws1 : ws0;
         if (chunk + 1 < a.nchunks) issue_loads(chunk + 1, (chunk & 1) ? xs0 : xs1, (chunk & 1) ? ws0 : ws1);
 
+        // k-steps of this chunk: step = pair * KHW + tap.  Operands are fetched from LDS PF steps ahead of
+        // the matrix instruction that consumes them (rotating register sets; all indices are compile-time
+        // after unrolling), so the LDS latency is covered by the PF matrix instructions in between.
+        auto fetch = [&](int step, float (&av)[RO], float (&bv)[RP]) {
+            const int cp = step / KHW, tap = step - cp * KHW;
+            const int rh = tap / KW, rw = tap - rh * KW;
+            const int koff_x = (2 * cp) * a.chs + rh * a.dh * a.Wp + rw * a.dw;
+            const int koff_w = cp * KHW + tap;
 #pragma unroll
-        for (int cp = 0; cp < CC / 2; ++cp) {
+            for (int i = 0; i < RO; ++i) av[i] = ws[wbase[i] + koff_w];
 #pragma unroll
-            for (int rh = 0; rh < KH; ++rh) {
+            for (int j = 0; j < RP; ++j) bv[j] = xs[xbase[j] + koff_x];
+#ifdef KXC_DBG_NO_LDS_READS
 #pragma unroll
-                for (int rw = 0; rw < KW; ++rw) {
-                    const int koff_x = (2 * cp) * a.chs + rh * a.dh * a.Wp + rw * a.dw;
-                    const int koff_w = cp * KHW + rh * KW + rw;
-                    float av[RO], bv[RP];
+            for (int i = 0; i < RO; ++i) av[i] = (float)(wbase[i] + koff_w);
 #pragma unroll
-                    for (int i = 0; i < RO; ++i) av[i] = ws[wbase[i] + koff_w];
+            for (int j = 0; j < RP; ++j) bv[j] = (float)(xbase[j] + koff_x);
+#endif
+        };
+        float av[PF + 1][RO], bv[PF + 1][RP];
 #pragma unroll
-                    for (int j = 0; j < RP; ++j) bv[j] = xs[xbase[j] + koff_x];
+        for (int p = 0; p < PF; ++p)
+            if (p < NS) fetch(p, av[p % (PF + 1)], bv[p % (PF + 1)]);
 #pragma unroll
-                    for (int i = 0; i < RO; ++i)
+        for (int step = 0; step < NS; ++step) {
+            if (step + PF < NS) fetch(step + PF, av[(step + PF) % (PF + 1)], bv[(step + PF) % (PF + 1)]);
+            __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
-                        for (int j = 0; j < RP; ++j)
-                            acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x2f32(av[i], bv[j], acc[i][j], 0, 0, 0);
-                }
-            }
+            for (int i = 0; i < RO; ++i)
+#pragma unroll
+                for (int j = 0; j < RP; ++j)
+                    acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x2f32(av[step % (PF + 1)][i], bv[step % (PF + 1)][j],
+                                                                     acc[i][j], 0, 0, 0);
+            __builtin_amdgcn_sched_barrier(0);
         }
 
+#ifndef KXC_DBG_NO_BARRIER
         asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
         __syncthreads();
+#endif
     }
 
     // ---- epilogue: accumulator register g of a block holds row 8*(g/4) + 4*half + g%4, column r
@@ -265,6 +283,9 @@ conv_mfma_kernel(const ConvArgs a) {
                 if (has_bias) v = __fadd_rn(v, bval);
                 if (has_res) v = __fadd_rn(v, a.res[off]);
                 if (do_relu) v = relu_sel(v);
+#ifdef KXC_DBG_NO_STORE
+                if (v == 123456.789f)
+#endif
                 a.y[off] = v;
             }
         }
@@ -321,32 +342,33 @@ struct Variant {
 
 // name = mfma_k<filter>_c<channels per chunk>_o<waves x blocks along output channels>_p<waves x blocks
 // along pixels>; tile = 32*blocks*waves in each direction.
+//
+// Measured on MI355X (batch 64 ResNet-18 layers): one 32x32 block per wave with many waves per SIMD
+// beats larger register tiles -- the matrix pipe is kept busy by wave-level parallelism, and small
+// workgroups (32 output channels x 128 pixels, 28 KiB of LDS) fit five to a CU and balance the
+// 256 CUs well.  Per filter size the table is in order of preference; Select() takes the first
+// entry that fits the shape, except that launches too small to fill the GPU take the entry with
+// the most workgroups.
 const Variant kVariants[] = {
+    KXC_VARIANT(3, 3, 4, 1, 4, 1, 1, 4),   // 32 x 128, 4 waves            (default)
+    KXC_VARIANT(3, 3, 4, 1, 8, 1, 1, 2),   // 32 x 256, 8 waves            (14x14 maps: fewer weight refills)
+    KXC_VARIANT(3, 3, 2, 1, 4, 1, 1, 4),   // 32 x 128, 2-channel chunks   (stride-2 56->28: smaller patch)
+    KXC_VARIANT(3, 3, 4, 1, 2, 1, 1, 8),   // 32 x 64, 2 waves             (small launches)
+    KXC_VARIANT(3, 3, 4, 2, 4, 1, 1, 4),   // 64 x 128, 8 waves
+    KXC_VARIANT(3, 3, 4, 2, 8, 1, 1, 2),   // 64 x 256, 16 waves
+    KXC_VARIANT(3, 3, 4, 1, 4, 2, 1, 4),   // 64 x 128, 4 waves of 64x32
     KXC_VARIANT(3, 3, 4, 1, 4, 2, 2, 4),   // 64 x 256, 4 waves of 64x64
-    KXC_VARIANT(3, 3, 4, 1, 8, 2, 1, 2),   // 64 x 256, 8 waves of 64x32
-    KXC_VARIANT(3, 3, 4, 1, 7, 2, 1, 2),   // 64 x 224
-    KXC_VARIANT(3, 3, 4, 1, 6, 2, 1, 3),   // 64 x 192
-    KXC_VARIANT(3, 3, 4, 1, 5, 2, 1, 3),   // 64 x 160
-    KXC_VARIANT(3, 3, 4, 1, 4, 2, 1, 4),   // 64 x 128
-    KXC_VARIANT(3, 3, 4, 1, 3, 2, 1, 6),   // 64 x 96
-    KXC_VARIANT(3, 3, 4, 1, 2, 2, 2, 8),   // 64 x 128, 2 waves of 64x64
-    KXC_VARIANT(3, 3, 4, 2, 2, 1, 1, 6),   // 64 x 64
-    KXC_VARIANT(3, 3, 4, 1, 4, 1, 1, 4),   // 32 x 128
-    KXC_VARIANT(3, 3, 8, 1, 4, 2, 2, 4),   // 8-channel chunks
-    KXC_VARIANT(3, 3, 8, 1, 8, 2, 1, 2),
-    KXC_VARIANT(3, 3, 8, 1, 6, 2, 1, 3),
-    KXC_VARIANT(3, 3, 8, 1, 5, 2, 1, 3),
-    KXC_VARIANT(3, 3, 8, 1, 4, 2, 1, 4),
-    KXC_VARIANT(3, 3, 8, 2, 2, 1, 1, 6),
-    KXC_VARIANT(1, 1, 8, 1, 4, 2, 2, 6),   // 64 x 256
+    KXC_VARIANT(3, 3, 8, 1, 8, 1, 1, 2),   // 8-channel chunks
     KXC_VARIANT(1, 1, 8, 1, 4, 2, 1, 4),   // 64 x 128
+    KXC_VARIANT(1, 1, 8, 1, 4, 2, 2, 6),   // 64 x 256
     KXC_VARIANT(1, 1, 8, 2, 2, 1, 1, 6),   // 64 x 64
     KXC_VARIANT(1, 1, 8, 1, 4, 1, 1, 4),   // 32 x 128
-    KXC_VARIANT(1, 1, 16, 1, 4, 2, 1, 4),
     KXC_VARIANT(1, 1, 16, 2, 2, 1, 1, 6),
-    KXC_VARIANT(7, 7, 4, 1, 4, 2, 1, 12),  // 64 x 128 (3 input channels padded to 4)
-    KXC_VARIANT(7, 7, 4, 1, 8, 2, 1, 8),   // 64 x 256
-    KXC_VARIANT(7, 7, 4, 1, 4, 1, 1, 12),  // 32 x 128
+    KXC_VARIANT(7, 7, 2, 1, 8, 1, 1, 8),   // 32 x 256; 2-channel chunks: two chunks for RGB, loads overlap compute
+    KXC_VARIANT(7, 7, 2, 1, 7, 1, 1, 8),   // 32 x 224: two full output rows of a 112-wide map
+    KXC_VARIANT(7, 7, 4, 1, 8, 1, 1, 8),   // 32 x 256, one chunk (3 input channels padded to 4)
+    KXC_VARIANT(7, 7, 2, 1, 4, 1, 1, 12),  // 32 x 128
+    KXC_VARIANT(7, 7, 4, 1, 4, 1, 1, 12),
 };
 constexpr int kNumVariants = sizeof(kVariants) / sizeof(kVariants[0]);
 
@@ -393,15 +415,6 @@ bool Fits(const Variant& v, const ConvArgs& a, Choice* out) {
     return true;
 }
 
-// Cost model: workgroups are spread over 256 CUs, so the launch takes about
-// ceil(tiles / CUs) tile times; a tile costs its matrix work plus the LDS fill, which is
-// amortised better by larger tiles.
-double Cost(const Variant& v, const ConvArgs& a) {
-    const int64_t tiles = CeilDiv(a.M, v.tp) * CeilDiv(a.O, v.to);
-    const double rounds = static_cast<double>(CeilDiv(tiles, kNumCUs));
-    return rounds * v.tp * v.to * (1.0 + 40.0 / v.tp + 12.0 / v.to);
-}
-
 // Picks the MFMA variant for a shape, or leaves choice.v == nullptr for the direct kernel.
 void Select(const ConvArgs& a, int kh, int kw, Choice* choice) {
     choice->v = nullptr;
@@ -413,16 +426,31 @@ void Select(const ConvArgs& a, int kh, int kw, Choice* choice) {
     const int64_t q_rows = static_cast<int64_t>(a.N + 1) * a.Hp + kh * a.dh;
     if (x_bytes >= (1LL << 31) || y_elems >= (1LL << 31) || w_bytes >= (1LL << 31) || q_rows * a.Wp >= (1LL << 31)) return;
     const char* forced = std::getenv("KXC_HIP_CONV_VARIANT");
-    double best_cost = 0.0;
-    for (int i = 0; i < kNumVariants; ++i) {
-        const Variant& v = kVariants[i];
-        if (v.kh != kh || v.kw != kw) continue;
-        if (forced && *forced && std::strcmp(forced, v.name) != 0) continue;
-        if (v.to > a.O) continue;                 // do not spend matrix work on absent output channels
-        Choice c;
-        if (!Fits(v, a, &c)) continue;
-        const double cost = Cost(v, a);
-        if (!choice->v || cost < best_cost) { *choice = c; best_cost = cost; }
+    // Shape rules on top of the table order (measured, see the table's comment).
+    const char* preferred = nullptr;
+    if (kh == 3 && a.OW <= 14 && a.M >= 8192) preferred = "mfma_k3x3_c4_o1x1_p8x1";
+    if (kh == 3 && a.sh == 2 && a.W >= 56) preferred = "mfma_k3x3_c2_o1x1_p4x1";
+    Choice first_fit, most_tiles;
+    int64_t most = -1;
+    for (int pass = 0; pass < 2 && !choice->v; ++pass) {
+        for (int i = 0; i < kNumVariants; ++i) {
+            const Variant& v = kVariants[i];
+            if (v.kh != kh || v.kw != kw) continue;
+            if (forced && *forced && std::strcmp(forced, v.name) != 0) continue;
+            if (pass == 0 && !(forced && *forced) && (!preferred || std::strcmp(preferred, v.name) != 0)) continue;
+            if (v.to > a.O && v.to > 32) continue;    // do not spend matrix work on absent output channels
+            Choice c;
+            if (!Fits(v, a, &c)) continue;
+            const int64_t tiles = CeilDiv(a.M, v.tp) * CeilDiv(a.O, v.to);
+            if (pass == 0 || (forced && *forced)) { *choice = c; return; }
+            if (!first_fit.v) first_fit = c;
+            if (tiles > most) { most = tiles; most_tiles = c; }
+            if (first_fit.v && most >= 2 * kNumCUs) break;
+        }
+        if (pass == 1) {
+            const int64_t ff_tiles = first_fit.v ? CeilDiv(a.M, first_fit.v->tp) * CeilDiv(a.O, first_fit.v->to) : 0;
+            *choice = (ff_tiles >= kNumCUs || !most_tiles.v) ? first_fit : most_tiles;
+        }
     }
 }
 

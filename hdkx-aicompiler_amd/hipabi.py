@@ -9,7 +9,8 @@ import ctypes as C
 import os
 
 PKG = os.path.dirname(os.path.abspath(__file__))
-_LIB_PATH = os.path.join(PKG, "lib", "libkxc_hip.so")
+# KXC_HIP_LIB points at an alternative build of the same library (kernel experiments).
+_LIB_PATH = os.environ.get("KXC_HIP_LIB") or os.path.join(PKG, "lib", "libkxc_hip.so")
 _lib = None
 
 CONV_BIAS, CONV_RESIDUAL, CONV_RELU, CONV_FORCE_DIRECT = 1, 2, 4, 0x100
