@@ -1,0 +1,58 @@
+// codegen.h -- TIR -> C text for the host, TIR -> HIP source for gfx950.
+//
+// CodeGenC mirrors the reference's C back end (src/codegen/codegen_c.cc:54-276): one function
+// `int32_t <name>(void** packed_args)` of scalar serial loops.  Differences on purpose: buffer
+// names are made unique (the reference declares same-named arrays twice for a graph that calls an
+// operator twice) and intermediates are heap-allocated like its LLVM back end does
+// (src/codegen/codegen_llvm.cc:578-623) instead of living on the stack.
+//
+// CodeGenHIP is the GPU emitter the reference reserves an enum value for
+// (include/codegen/codegen.h:19-23, kCUDA "future extension").  Every top-level compute stage of
+// the PrimFunc becomes one `extern "C" __global__` kernel:
+//   * the stage's data-parallel loop nest is flattened to one index; a workgroup is 256 threads =
+//     four 64-lane wavefronts, the innermost data axis is the lane-fastest one (coalesced stores),
+//     and a grid-stride loop covers the rest;
+//   * reduce loops stay inside the thread, in the CPU order, accumulating through the output
+//     element exactly as the lowered TIR does -- so a generated kernel is bit-identical to the CPU
+//     loop nest (the source is compiled without multiply-add contraction);
+//   * LDS staging: a reduction whose source rows are contiguous in memory (global average pool,
+//     reduce_mean over trailing axes, row sums) is scheduled as a cooperative, coalesced load of the
+//     workgroup's rows into LDS followed by per-thread sequential sums from LDS (odd row stride, no
+//     bank conflicts), which keeps the order and removes the strided global reads.
+#pragma once
+
+#include "kxc/tir.h"
+
+namespace kxc {
+namespace codegen {
+
+enum class CodeGenBackend { kLLVM, kC, kCUDA, kHIP };
+
+class CodeGenC {
+public:
+    std::string Generate(const tir::PrimFunc& func, const std::string& name = "main");
+};
+
+struct HIPKernelSpec {
+    std::string symbol;
+    uint32_t grid[3] = {1, 1, 1};
+    uint32_t block[3] = {256, 1, 1};
+    uint32_t shared_bytes = 0;
+    // kernel parameters: the buffer variables of the PrimFunc (parameters or Allocate'd intermediates)
+    std::vector<const tir::ExprNode*> buffers;
+    std::string schedule;     // "flat" or "lds_row_reduce"
+};
+
+struct HIPModuleSource {
+    std::string source;
+    std::vector<HIPKernelSpec> kernels;      // in execution order
+};
+
+class CodeGenHIP {
+public:
+    // prefix: made part of every kernel symbol so several PrimFuncs can share one module
+    HIPModuleSource Generate(const tir::PrimFunc& func, const std::string& prefix = "kxc");
+};
+
+}  // namespace codegen
+}  // namespace kxc

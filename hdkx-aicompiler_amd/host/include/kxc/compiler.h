@@ -1,0 +1,86 @@
+// compiler.h -- CompileConfig, Compiler::Compile, CompiledModule::Run.
+// The user-visible entry of the reference (include/api/compiler.h:32-92, include/api/compile_config.h:34-68):
+// a test that compiles for the CPU with CompileConfig::JIT(BuildTarget(kCPU)) runs on the GPU by
+// changing only the target to BuildTarget(kGPU).  Compile selects the back end from
+// config->target->kind: "hip" builds a launch plan of hand-written kernels (operators that register
+// FHIPDispatch, with bias / residual add / ReLU fused into convolutions) and run-time compiled
+// kernels from the TIR -> HIP generator (everything else); any other kind compiles the whole
+// function to C with the host compiler.
+//
+// Run ABI (src/codegen/compiled_kernel.cc:41-55): packed_args = inputs, constants in lowering order,
+// outputs.  For the "hip" target every pointer is a DEVICE pointer; Run enqueues the plan on the
+// current stream and synchronises it before returning, because callers read outputs right after.
+#pragma once
+
+#include <memory>
+
+#include "kxc/codegen.h"
+#include "kxc/device_api.h"
+#include "kxc/lower.h"
+
+namespace kxc {
+namespace api {
+
+enum class CompileMode { kAOT, kJIT, kAdaptive };
+
+struct CompileConfigNode {
+    CompileMode mode{CompileMode::kAOT};
+    int opt_level{2};
+    Target target;
+    codegen::CodeGenBackend backend{codegen::CodeGenBackend::kLLVM};
+    // HIP back end switches
+    bool hip_use_handwritten{true};    // false: every operator goes through the TIR -> HIP generator
+    bool hip_fuse{true};               // fold bias / residual add / ReLU into convolution launches
+    bool sync_after_run{true};
+};
+class CompileConfig : public Ref<CompileConfigNode> {
+public:
+    CompileConfig() = default;
+    explicit CompileConfig(std::shared_ptr<CompileConfigNode> n) : Ref<CompileConfigNode>(std::move(n)) {}
+    static CompileConfig AOT(Target target, int opt_level = 3);
+    static CompileConfig JIT(Target target);
+};
+
+// One launch of a compiled module, as an execution-plan node would describe it
+// (include/base/execution_plan.h:42-50): operator, kernel symbol, value ids.
+struct KernelExecInfo {
+    std::string op_name;
+    std::string kernel_symbol;
+    std::vector<int> input_values;
+    std::vector<int> output_values;
+};
+
+class CompiledModuleImpl;
+
+class CompiledModule {
+public:
+    CompiledModule() = default;
+    explicit CompiledModule(std::shared_ptr<CompiledModuleImpl> impl) : impl_(std::move(impl)) {}
+    void Run(const std::vector<void*>& packed_args);
+    bool IsReady() const;
+    std::string GetStatus() const;
+    const tir::PrimFunc& GetPrimFunc() const;
+    // Generated source: C for the host back end, HIP for the GPU back end.
+    const std::string& GetSource() const;
+    void SaveCSource(const std::string& path) const;
+    // Constants of the graph in parameter order (host data), to be passed again at every Run.
+    const Array<runtime::NDArray>& GetConstants() const;
+    int64_t input_count() const;
+    int64_t constant_count() const;
+    // The launches Run performs, in order.
+    const std::vector<KernelExecInfo>& GetKernelExecs() const;
+    // Execution-plan description (schema of src/base/execution_plan.cc:674-877: integers plus kernel_symbol).
+    std::string ExecutionPlanJSON() const;
+    size_t workspace_bytes() const;
+
+private:
+    std::shared_ptr<CompiledModuleImpl> impl_;
+};
+
+class Compiler {
+public:
+    static CompiledModule Compile(Function func, CompileConfig config);
+};
+
+}  // namespace api
+}  // namespace kxc

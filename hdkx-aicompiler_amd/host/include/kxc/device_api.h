@@ -1,0 +1,102 @@
+// device_api.h -- Device, DeviceAPI (CPU and HIP), Target.
+// Interface of the reference's include/base/device.h:20-62, include/base/device_api.h:42-151 and
+// include/base/target.h:34-35.  kGPU is served by HIPDeviceAPI, a thin C++ face of the C-ABI
+// library's device calls (the reference wires kGPU to its CUDA implementation,
+// src/base/device_api.cc:164-178): target kind "hip", arch "gfx950", warp_size 64.
+#pragma once
+
+#include "kxc/base.h"
+
+namespace kxc {
+
+enum DeviceTypeCode { kCPU = 0, kGPU = 1, kOpenCL = 2, kMetal = 3, kUnknown = -1 };
+
+class Device {
+public:
+    Device() = default;
+    Device(DeviceTypeCode type, int id) : type_(type), id_(id) {}
+    DeviceTypeCode device_type() const { return type_; }
+    int device_id() const { return id_; }
+
+private:
+    DeviceTypeCode type_ = kCPU;
+    int id_ = 0;
+};
+
+using StreamHandle = void*;
+
+struct DeviceAttributes {
+    int exists{0};
+    int64_t max_threads_per_block{1};
+    int64_t warp_size{1};
+    int64_t max_shared_memory_per_block{0};
+    std::string compute_version{"0.0"};
+    std::string device_name;
+    int64_t max_clock_rate_khz{0};
+    int64_t max_registers_per_block{0};
+    int64_t api_version{0};
+    int64_t driver_version{0};
+    int64_t l2_cache_size_bytes{0};
+    int64_t total_global_memory{0};
+    int64_t available_global_memory{0};
+    int64_t max_shared_memory_per_multiprocessor{0};
+    int64_t max_threads_per_multiprocessor{0};
+    int64_t compute_version_major{0};
+    int64_t compute_version_minor{0};
+    int64_t multi_processor_count{1};
+    std::string arch;
+    std::string status;
+};
+
+struct DeviceInfo {
+    DeviceTypeCode device_type{kUnknown};
+    int device_id{-1};
+    std::string device_type_name;
+    std::string target_kind;
+    bool available{false};
+    std::string status;
+    DeviceAttributes attrs;
+};
+
+class DeviceAPI {
+public:
+    virtual ~DeviceAPI() = default;
+    virtual void SetDevice(const Device& device) = 0;
+    virtual void* AllocDataSpace(const Device& device, size_t nbytes, size_t alignment) = 0;
+    virtual void FreeDataSpace(const Device& device, void* ptr) = 0;
+    virtual void CopyDataFromTo(const Device& from_dev, const void* from_ptr, const Device& to_dev, void* to_ptr,
+                                size_t nbytes) = 0;
+    virtual void CopyDataFromTo(const void* from_ptr, size_t from_offset, void* to_ptr, size_t to_offset, size_t nbytes,
+                                const Device& from_dev, const Device& to_dev, StreamHandle stream);
+    virtual DeviceAttributes GetDeviceAttributes(const Device& device) = 0;
+    virtual std::string GetTargetKind(const Device& device) const = 0;
+    virtual StreamHandle CreateStream(const Device& device);
+    virtual void FreeStream(const Device& device, StreamHandle stream);
+    virtual void SetStream(const Device& device, StreamHandle stream);
+    virtual StreamHandle GetCurrentStream(const Device& device);
+    virtual void StreamSync(const Device& device, StreamHandle stream);
+    virtual void SyncStreamFromTo(const Device& device, StreamHandle src, StreamHandle dst);
+    virtual void* AllocWorkspace(const Device& device, size_t nbytes, size_t alignment);
+    virtual void FreeWorkspace(const Device& device, void* ptr);
+};
+
+DeviceAPI* GetCPUDeviceAPI();
+DeviceAPI* GetHIPDeviceAPI();
+DeviceAPI* GetDeviceAPI(DeviceTypeCode type);
+std::vector<DeviceInfo> GetAllDeviceInfo();
+std::string GetAllDeviceInfoJSON();
+
+struct TargetNode {
+    std::string kind;            // "llvm" for the CPU (the reference's name), "hip" for the GPU
+    Device device;
+    DeviceAttributes attrs;
+};
+class Target : public Ref<TargetNode> {
+public:
+    Target() = default;
+    explicit Target(std::shared_ptr<TargetNode> n) : Ref<TargetNode>(std::move(n)) {}
+};
+// src/base/target.cc:34-51: kind and attributes come from the device API.
+Target BuildTarget(DeviceTypeCode type, int device_id = 0);
+
+}  // namespace kxc

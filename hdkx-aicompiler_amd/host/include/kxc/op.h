@@ -1,0 +1,184 @@
+// op.h -- operator registry, attribute types and the per-operator hooks.
+//
+// Same registration DSL and hook types as the reference (include/relay/op_macros.h:16-40,
+// include/relay/op_attr_types.h:17-23, include/relay/op.h:29-54,104-382):
+//   KXC_REGISTER_OP(nn_conv2d).describe(..).set_num_inputs(-1).add_argument(..)
+//       .set_attr<FInferType>("FInferType", ..).set_attr<FRelayToTE>("FRelayToTE", ..)
+// plus one hook of this backend registered alongside them: "FHIPDispatch", which maps a call (and
+// what was fused into it) to a hand-written gfx950 kernel of the C-ABI library.  Operators without
+// it go through FRelayToTE -> TIR -> the HIP code generator.
+#pragma once
+
+#include <any>
+#include <functional>
+#include <unordered_map>
+
+#include "kxc/relay.h"
+#include "kxc/te.h"
+
+struct kxc_hip_plan;   // C ABI (kxc_hip.h)
+
+namespace kxc {
+namespace relay {
+
+struct ArgumentInfo {
+    std::string name, type, description;
+};
+
+struct OpNode : RelayExprNode {
+    std::string name;
+    std::string description;
+    Array<ArgumentInfo> arguments;
+    int num_inputs = -1;
+    std::unordered_map<std::string, std::any> attrs;
+};
+
+class Op : public Expr {
+public:
+    Op() = default;
+    explicit Op(std::shared_ptr<OpNode> n) { ptr_ = n; }
+    const OpNode* operator->() const { return static_cast<const OpNode*>(ptr_.get()); }
+    // Looks the operator up in the global table, creating an empty entry if absent (src/base/op.cc:19-39).
+    static const Op& Get(const std::string& name);
+};
+
+using FInferType = std::function<Type(const Attrs&, const Array<Type>&)>;
+using FRelayToTE = std::function<te::Tensor(const Attrs&, const Array<te::Tensor>&, const Type&)>;
+
+// ---- this backend's hook -------------------------------------------------------------------
+// A device buffer operand of a launch: a packed argument or a workspace slot.
+struct HIPBuffer {
+    int kind = 2;            // KXC_HIP_BUF_ARG / _WORKSPACE / _NONE
+    int64_t index_or_offset = 0;
+};
+struct HIPDispatchContext {
+    Attrs attrs;
+    Array<Type> input_types;
+    Type out_type;
+    Array<HIPBuffer> inputs;
+    HIPBuffer output;
+    // what the graph pass fused behind this call (only offered to operators that declare "THIPFusable")
+    bool fused_relu = false;
+    bool has_residual = false;
+    HIPBuffer residual;
+};
+// Appends the launch(es) for one call to the plan; returns the kernel_symbol, or "" to decline (the
+// call is then compiled through the code generator).
+using FHIPDispatch = std::function<std::string(const HIPDispatchContext&, kxc_hip_plan*)>;
+
+class OpRegEntry {
+public:
+    explicit OpRegEntry(std::shared_ptr<OpNode> op) : op_(std::move(op)) {}
+    OpRegEntry& describe(const std::string& text) { op_->description = text; return *this; }
+    OpRegEntry& set_num_inputs(int n) { op_->num_inputs = n; return *this; }
+    OpRegEntry& add_argument(const std::string& name, const std::string& type, const std::string& desc) {
+        op_->arguments.push_back({name, type, desc});
+        return *this;
+    }
+    template <typename T>
+    OpRegEntry& set_attr(const std::string& key, const T& value) {
+        op_->attrs[key] = value;
+        return *this;
+    }
+    static OpRegEntry Register(const std::string& name);
+
+private:
+    std::shared_ptr<OpNode> op_;
+};
+
+#define KXC_OP_CONCAT_(a, b) a##b
+#define KXC_OP_CONCAT(a, b) KXC_OP_CONCAT_(a, b)
+#define KXC_REGISTER_OP(OpName) \
+    static ::kxc::relay::OpRegEntry KXC_OP_CONCAT(kxc_op_reg_, __COUNTER__) = ::kxc::relay::OpRegEntry::Register(#OpName)
+
+// Force the built-in operator registrations to be linked (static initialisers in ops.cc).
+void EnsureBuiltinOpsRegistered();
+
+// ------------------------------------------------------------------ attribute types
+#define KXC_ATTRS_REF(TypeName)                                                                      \
+    class TypeName : public Attrs {                                                                  \
+    public:                                                                                          \
+        TypeName() = default;                                                                        \
+        explicit TypeName(std::shared_ptr<TypeName##Node> n) : Attrs(n) {}                           \
+        const TypeName##Node* operator->() const { return static_cast<const TypeName##Node*>(ptr_.get()); }
+
+struct Conv2DAttrsNode : AttrsNode {
+    std::vector<int64_t> strides, padding, dilation, kernel_size;
+    int groups = 1, channels = 0;
+    std::string data_layout, kernel_layout, out_layout, out_dtype;
+};
+KXC_ATTRS_REF(Conv2DAttrs)
+    static Conv2DAttrs Create(std::vector<int64_t> strides, std::vector<int64_t> padding, std::vector<int64_t> dilation,
+                              int groups, int channels, std::vector<int64_t> kernel_size, std::string data_layout,
+                              std::string kernel_layout, std::string out_layout, std::string out_dtype);
+};
+
+struct MaxPool2DAttrsNode : AttrsNode {
+    std::vector<int64_t> strides, padding, dilation, pool_size;
+    std::string layout;
+    bool ceil_mode = false;
+};
+KXC_ATTRS_REF(MaxPool2DAttrs)
+    // strides first, pool_size fourth (include/relay/op.h:172-174)
+    static MaxPool2DAttrs Create(std::vector<int64_t> strides, std::vector<int64_t> padding, std::vector<int64_t> dilation,
+                                 std::vector<int64_t> pool_size, std::string layout, bool ceil_mode);
+};
+
+struct DenseAttrsNode : AttrsNode { int64_t units = 0; std::string out_dtype; };
+KXC_ATTRS_REF(DenseAttrs)
+    static DenseAttrs Create(int64_t units, std::string out_dtype);
+};
+
+struct GemmAttrsNode : AttrsNode { float alpha = 1.0f, beta = 1.0f; int transA = 0, transB = 0; };
+KXC_ATTRS_REF(GemmAttrs)
+    static GemmAttrs Create(float alpha = 1.0f, float beta = 1.0f, int transA = 0, int transB = 0);
+};
+
+struct FlattenAttrsNode : AttrsNode { int axis = 1; };
+KXC_ATTRS_REF(FlattenAttrs)
+    static FlattenAttrs Create(int axis = 1);
+};
+
+struct ReshapeAttrsNode : AttrsNode { std::vector<int64_t> newshape; };
+KXC_ATTRS_REF(ReshapeAttrs)
+    static ReshapeAttrs Create(std::vector<int64_t> newshape);
+};
+
+struct TransposeAttrsNode : AttrsNode { std::vector<int64_t> axes; };
+KXC_ATTRS_REF(TransposeAttrs)
+    static TransposeAttrs Create(std::vector<int64_t> axes);
+};
+
+struct ReduceMeanAttrsNode : AttrsNode { std::vector<int64_t> axes; int keepdims = 0; };
+KXC_ATTRS_REF(ReduceMeanAttrs)
+    static ReduceMeanAttrs Create(std::vector<int64_t> axes, int keepdims);
+};
+
+#define KXC_SIMPLE_ATTRS(TypeName)                \
+    struct TypeName##Node : AttrsNode {};         \
+    KXC_ATTRS_REF(TypeName)                       \
+        static TypeName Create() { return TypeName(std::make_shared<TypeName##Node>()); } \
+    };
+KXC_SIMPLE_ATTRS(ReluAttrs)
+KXC_SIMPLE_ATTRS(AddAttrs)
+KXC_SIMPLE_ATTRS(GlobalAvgPool2DAttrs)
+
+// ------------------------------------------------------------------ shape rules (src/relay/type_infer.cc)
+Type Conv2DInferType(const Attrs& attrs, const Array<Type>& inputs);
+Type Pool2DInferType(const Attrs& attrs, const Array<Type>& inputs);
+Type GlobalAvgPool2DInferType(const Attrs& attrs, const Array<Type>& inputs);
+Type DenseInferType(const Attrs& attrs, const Array<Type>& inputs);
+Type GemmInferType(const Attrs& attrs, const Array<Type>& inputs);
+Type MatmulInferType(const Attrs& attrs, const Array<Type>& inputs);
+Type UnarySameInferType(const Attrs& attrs, const Array<Type>& inputs);
+Type BroadcastInferType(const Attrs& attrs, const Array<Type>& inputs);
+Type FlattenInferType(const Attrs& attrs, const Array<Type>& inputs);
+Type ReshapeInferType(const Attrs& attrs, const Array<Type>& inputs);
+Type TransposeInferType(const Attrs& attrs, const Array<Type>& inputs);
+Type ReduceMeanInferType(const Attrs& attrs, const Array<Type>& inputs);
+
+// InferTypePass (src/relay/transforms/infer_type.cc:41-222): fills checked_type_ of every node.
+Function InferTypePass(const Function& f);
+
+}  // namespace relay
+}  // namespace kxc

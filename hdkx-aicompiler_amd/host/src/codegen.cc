@@ -1,0 +1,430 @@
+// codegen.cc -- see codegen.h.
+#include "kxc/codegen.h"
+
+#include <cmath>
+#include <cstdio>
+#include <functional>
+#include <map>
+#include <set>
+#include <sstream>
+#include <unordered_map>
+
+namespace kxc {
+namespace codegen {
+
+using tir::DataType;
+using tir::ExprKind;
+using tir::ExprNode;
+using tir::PrimExpr;
+using tir::Stmt;
+using tir::StmtKind;
+
+namespace {
+
+// builtin = true: spell integer types with language keywords (run-time compiled device code has no <stdint.h>)
+std::string CType(DataType t, bool builtin = false) {
+    if (t.is_float()) return t.bits == 64 ? "double" : "float";
+    if (t.is_bool()) return "bool";
+    if (builtin) {
+        const int bits = t.bits == 1 ? 8 : t.bits;
+        const char* base = bits == 8 ? "char" : bits == 16 ? "short" : bits == 32 ? "int" : "long long";
+        return std::string(t.is_uint() ? "unsigned " : (bits == 8 ? "signed " : "")) + base;
+    }
+    const std::string base = "int" + std::to_string(t.bits == 1 ? 8 : t.bits) + "_t";
+    return t.is_uint() ? "u" + base : base;
+}
+
+// Assigns every variable node a C identifier that is unique within one generated function/module.
+class Names {
+public:
+    std::string Get(const ExprNode* v) {
+        auto it = names_.find(v);
+        if (it != names_.end()) return it->second;
+        std::string base;
+        for (char c : v->name) base += (std::isalnum(static_cast<unsigned char>(c)) || c == '_') ? c : '_';
+        if (base.empty() || std::isdigit(static_cast<unsigned char>(base[0]))) base = "v_" + base;
+        std::string name = base;
+        for (int k = 1; used_.count(name); ++k) name = base + "_" + std::to_string(k);
+        used_.insert(name);
+        names_[v] = name;
+        return name;
+    }
+    void Reserve(const std::string& s) { used_.insert(s); }
+    bool builtin_types = false;
+
+private:
+    std::unordered_map<const ExprNode*, std::string> names_;
+    std::set<std::string> used_;
+};
+
+// Expression text shared by both generators.  C's usual arithmetic conversions promote mixed operands
+// to the wider / floating type, which is the reference's promotion rule
+// (src/codegen/codegen_llvm.cc:189-217,266-273); Min/Max are compare + select with an ordered compare
+// (:317-334), Select is a conditional (:391-442).
+std::string EmitExpr(const PrimExpr& e, Names* names) {
+    if (!e.defined()) return "0";
+    auto A = [&](int i) { return EmitExpr(e->args[i], names); };
+    char buf[64];
+    switch (e->kind) {
+        case ExprKind::kIntImm:
+            if (e->dtype.is_bool()) return e->ivalue ? "true" : "false";
+            if (e->dtype.bits == 64) return "((" + CType(e->dtype, names->builtin_types) + ")" + std::to_string(e->ivalue) + "LL)";
+            return std::to_string(e->ivalue);
+        case ExprKind::kFloatImm:
+            if (std::isinf(e->fvalue)) return e->fvalue > 0 ? "INFINITY" : "(-INFINITY)";
+            if (std::isnan(e->fvalue)) return "NAN";
+            std::snprintf(buf, sizeof(buf), e->dtype.bits == 32 ? "%.9ef" : "%.17e", e->fvalue);
+            return buf;
+        case ExprKind::kVar: return names->Get(e.get());
+        case ExprKind::kAdd: return "(" + A(0) + " + " + A(1) + ")";
+        case ExprKind::kSub: return "(" + A(0) + " - " + A(1) + ")";
+        case ExprKind::kMul: return "(" + A(0) + " * " + A(1) + ")";
+        case ExprKind::kDiv: return "(" + A(0) + " / " + A(1) + ")";
+        case ExprKind::kMod:
+            if (PromoteTypes(e->args[0].dtype(), e->args[1].dtype()).is_float()) return "fmod(" + A(0) + ", " + A(1) + ")";
+            return "(" + A(0) + " % " + A(1) + ")";
+        case ExprKind::kMin: { std::string a = A(0), b = A(1); return "((" + a + ") < (" + b + ") ? (" + a + ") : (" + b + "))"; }
+        case ExprKind::kMax: { std::string a = A(0), b = A(1); return "((" + a + ") > (" + b + ") ? (" + a + ") : (" + b + "))"; }
+        case ExprKind::kEQ: return "(" + A(0) + " == " + A(1) + ")";
+        case ExprKind::kLT: return "(" + A(0) + " < " + A(1) + ")";
+        case ExprKind::kAnd: return "(" + A(0) + " && " + A(1) + ")";
+        case ExprKind::kOr: return "(" + A(0) + " || " + A(1) + ")";
+        case ExprKind::kNot: return "(!" + A(0) + ")";
+        case ExprKind::kLoad: return A(0) + "[" + A(1) + "]";
+        case ExprKind::kSelect: return "(" + A(0) + " ? " + A(1) + " : " + A(2) + ")";
+        case ExprKind::kCall: {
+            if (e->name == "cast") return "((" + CType(e->dtype, names->builtin_types) + ")(" + A(0) + "))";
+            static const std::map<std::string, std::string> f32 = {{"exp", "expf"}, {"log", "logf"}, {"sqrt", "sqrtf"},
+                {"floor", "floorf"}, {"ceil", "ceilf"}, {"fabs", "fabsf"}, {"tanh", "tanhf"}};
+            std::string name = e->name;
+            if (name.rfind("tir.", 0) == 0) name = name.substr(4);
+            auto it = f32.find(name);
+            if (it == f32.end()) throw std::runtime_error("code generator: unsupported intrinsic " + e->name);
+            std::string fn = e->dtype.bits == 64 ? name : it->second;
+            std::string out = fn + "(";
+            for (size_t i = 0; i < e->args.size(); ++i) out += (i ? ", " : "") + A(static_cast<int>(i));
+            return out + ")";
+        }
+        default: throw std::runtime_error("code generator: TE-only expression reached the back end");
+    }
+}
+
+void EmitStmt(const Stmt& s, Names* names, std::ostringstream& os, int indent) {
+    if (!s.defined()) return;
+    const std::string pad(indent, ' ');
+    switch (s->kind) {
+        case StmtKind::kFor: {
+            const std::string v = names->Get(s->var.get());
+            const std::string lo = EmitExpr(s->a, names), ext = EmitExpr(s->b, names);
+            os << pad << "for (int " << v << " = " << lo << "; " << v << " < (" << lo << " + " << ext << "); ++" << v
+               << ") {\n";
+            EmitStmt(s->body[0], names, os, indent + 2);
+            os << pad << "}\n";
+            break;
+        }
+        case StmtKind::kStore:
+            os << pad << names->Get(s->var.get()) << "[" << EmitExpr(s->b, names) << "] = " << EmitExpr(s->a, names) << ";\n";
+            break;
+        case StmtKind::kLetStmt:
+            os << pad << "{\n" << pad << "  const " << CType(s->var.dtype(), names->builtin_types) << " " << names->Get(s->var.get()) << " = "
+               << EmitExpr(s->a, names) << ";\n";
+            EmitStmt(s->body[0], names, os, indent + 2);
+            os << pad << "}\n";
+            break;
+        case StmtKind::kIfThenElse:
+            os << pad << "if (" << EmitExpr(s->a, names) << ") {\n";
+            EmitStmt(s->body[0], names, os, indent + 2);
+            if (s->body.size() > 1) {
+                os << pad << "} else {\n";
+                EmitStmt(s->body[1], names, os, indent + 2);
+            }
+            os << pad << "}\n";
+            break;
+        case StmtKind::kSeqStmt:
+            for (const auto& b : s->body) EmitStmt(b, names, os, indent);
+            break;
+        case StmtKind::kEvaluate: os << pad << EmitExpr(s->a, names) << ";\n"; break;
+        case StmtKind::kAllocate: throw std::runtime_error("code generator: Allocate inside a compute stage");
+    }
+}
+
+// Peels the Allocate nest off a PrimFunc body and returns the top-level stages.
+void SplitStages(const Stmt& body, std::vector<Stmt>* allocs, std::vector<Stmt>* stages) {
+    Stmt cur = body;
+    while (cur.defined() && cur->kind == StmtKind::kAllocate) {
+        allocs->push_back(cur);
+        cur = cur->body[0];
+    }
+    if (!cur.defined()) return;
+    if (cur->kind == StmtKind::kSeqStmt) {
+        for (const auto& s : cur->body) {
+            if (s.defined() && s->kind == StmtKind::kAllocate) throw std::runtime_error("code generator: nested Allocate in a sequence");
+            stages->push_back(s);
+        }
+    } else {
+        stages->push_back(cur);
+    }
+}
+
+void CollectBuffers(const PrimExpr& e, std::vector<const ExprNode*>* out) {
+    if (!e.defined()) return;
+    if (e->kind == ExprKind::kLoad) {
+        const ExprNode* b = e->args[0].get();
+        if (std::find(out->begin(), out->end(), b) == out->end()) out->push_back(b);
+        CollectBuffers(e->args[1], out);
+        return;
+    }
+    for (const auto& a : e->args) CollectBuffers(a, out);
+}
+void CollectBuffers(const Stmt& s, std::vector<const ExprNode*>* out, std::vector<const ExprNode*>* written) {
+    if (!s.defined()) return;
+    if (s->kind == StmtKind::kStore) {
+        const ExprNode* b = s->var.get();
+        if (std::find(out->begin(), out->end(), b) == out->end()) out->push_back(b);
+        if (std::find(written->begin(), written->end(), b) == written->end()) written->push_back(b);
+    }
+    CollectBuffers(s->a, out);
+    CollectBuffers(s->b, out);
+    for (const auto& b : s->body) CollectBuffers(b, out, written);
+}
+
+}  // namespace
+
+// =================================================================== host C
+std::string CodeGenC::Generate(const tir::PrimFunc& func, const std::string& name) {
+    Names names;
+    names.Reserve("packed_args");
+    std::ostringstream os;
+    os << "#include <stdint.h>\n#include <stdbool.h>\n#include <stdlib.h>\n#include <math.h>\n\n";
+    os << "int32_t " << name << "(void** packed_args) {\n";
+    for (size_t i = 0; i < func->params.size(); ++i) {
+        const auto& p = func->params[i];
+        os << "  " << CType(p.dtype()) << "* restrict " << names.Get(p.get()) << " = (" << CType(p.dtype())
+           << "*)packed_args[" << i << "];\n";
+    }
+    std::vector<Stmt> allocs, stages;
+    SplitStages(func->body, &allocs, &stages);
+    std::vector<std::string> to_free;
+    for (const auto& a : allocs) {
+        int64_t count = 1;
+        for (const auto& e : a->extents) {
+            int64_t v;
+            if (!tir::GetConstInt(e, &v)) throw std::runtime_error("CodeGenC: non-constant allocation extent");
+            count *= v;
+        }
+        const std::string v = names.Get(a->var.get());
+        os << "  " << CType(a->dtype) << "* restrict " << v << " = (" << CType(a->dtype) << "*)malloc((size_t)"
+           << count << " * sizeof(" << CType(a->dtype) << "));\n";
+        os << "  if (!" << v << ") return 1;\n";
+        to_free.push_back(v);
+    }
+    for (const auto& st : stages) EmitStmt(st, &names, os, 2);
+    for (auto it = to_free.rbegin(); it != to_free.rend(); ++it) os << "  free(" << *it << ");\n";
+    os << "  return 0;\n}\n";
+    return os.str();
+}
+
+// =================================================================== gfx950 HIP
+namespace {
+
+struct Affine {
+    bool ok = true;
+    int64_t constant = 0;
+    std::map<const ExprNode*, int64_t> coef;
+};
+
+Affine AnalyzeAffine(const PrimExpr& e) {
+    Affine r;
+    if (!e.defined()) { r.ok = false; return r; }
+    switch (e->kind) {
+        case ExprKind::kIntImm: r.constant = e->ivalue; return r;
+        case ExprKind::kVar: r.coef[e.get()] = 1; return r;
+        case ExprKind::kAdd: case ExprKind::kSub: {
+            Affine a = AnalyzeAffine(e->args[0]), b = AnalyzeAffine(e->args[1]);
+            if (!a.ok || !b.ok) { r.ok = false; return r; }
+            const int64_t sign = e->kind == ExprKind::kAdd ? 1 : -1;
+            r = a;
+            r.constant += sign * b.constant;
+            for (auto& kv : b.coef) r.coef[kv.first] += sign * kv.second;
+            return r;
+        }
+        case ExprKind::kMul: {
+            Affine a = AnalyzeAffine(e->args[0]), b = AnalyzeAffine(e->args[1]);
+            if (!a.ok || !b.ok) { r.ok = false; return r; }
+            if (!a.coef.empty() && !b.coef.empty()) { r.ok = false; return r; }
+            const Affine& lin = a.coef.empty() ? b : a;
+            const int64_t k = a.coef.empty() ? a.constant : b.constant;
+            r.constant = lin.constant * k;
+            for (auto& kv : lin.coef) r.coef[kv.first] = kv.second * k;
+            return r;
+        }
+        default: r.ok = false; return r;
+    }
+}
+
+struct LoopNest {
+    std::vector<tir::Var> vars;
+    std::vector<int64_t> extents;
+    Stmt body;
+};
+
+// Strips the outer data-parallel loops (constant extent, zero minimum).
+LoopNest PeelLoops(Stmt s, bool stop_at_seq) {
+    LoopNest n;
+    while (s.defined() && s->kind == StmtKind::kFor) {
+        int64_t lo, ext;
+        if (!tir::GetConstInt(s->a, &lo) || !tir::GetConstInt(s->b, &ext) || lo != 0) break;
+        n.vars.push_back(s->var);
+        n.extents.push_back(ext);
+        s = s->body[0];
+        if (stop_at_seq && s.defined() && s->kind == StmtKind::kSeqStmt) break;
+    }
+    n.body = s;
+    return n;
+}
+
+// Recognises  for data axes { out[o] = init; for reduce axes { out[o] = out[o] (+) src[o*R + r] } }  with
+// contiguous rows: every data-axis coefficient of the source index is R times its coefficient in the
+// output index and the reduce axes enumerate 0..R-1 in row-major order.
+bool MatchRowReduce(const LoopNest& data, Stmt* init_out, PrimExpr* src_load, int64_t* R, int* reduce_kind,
+                    const ExprNode** out_buf) {
+    const Stmt& b = data.body;
+    if (!b.defined() || b->kind != StmtKind::kSeqStmt || b->body.size() != 2) return false;
+    const Stmt& init = b->body[0];
+    if (init->kind != StmtKind::kStore) return false;
+    LoopNest red = PeelLoops(b->body[1], false);
+    if (red.vars.empty() || !red.body.defined() || red.body->kind != StmtKind::kStore) return false;
+    const Stmt& upd = red.body;
+    if (upd->var.get() != init->var.get()) return false;
+    const PrimExpr& v = upd->a;
+    if (v->kind != ExprKind::kAdd) return false;            // sums only: the staged loop keeps the order
+    const PrimExpr& old = v->args[0];
+    const PrimExpr& src = v->args[1];
+    if (old->kind != ExprKind::kLoad || old->args[0].get() != init->var.get()) return false;
+    if (src->kind != ExprKind::kLoad || src->args[0].get() == init->var.get()) return false;
+    int64_t rows = 1;
+    for (auto e : red.extents) rows *= e;
+    if (rows < 2 || rows > 63) return false;                 // 256 rows of (R|1) floats must fit 64 KiB of LDS
+    if (!src.dtype().is_float() || src.dtype().bits != 32) return false;
+    Affine oi = AnalyzeAffine(init->b), ui = AnalyzeAffine(upd->b), si = AnalyzeAffine(src->args[1]);
+    if (!oi.ok || !ui.ok || !si.ok || oi.constant != 0 || si.constant != 0) return false;
+    if (oi.coef != ui.coef || oi.constant != ui.constant) return false;
+    // output index must be the flattened data index
+    int64_t stride = 1;
+    for (int i = static_cast<int>(data.vars.size()) - 1; i >= 0; --i) {
+        const int64_t c = oi.coef.count(data.vars[i].get()) ? oi.coef.at(data.vars[i].get()) : 0;
+        if (data.extents[i] != 1 && c != stride) return false;
+        const int64_t sc = si.coef.count(data.vars[i].get()) ? si.coef.at(data.vars[i].get()) : 0;
+        if (data.extents[i] != 1 && sc != stride * rows) return false;
+        stride *= data.extents[i];
+    }
+    int64_t rs = 1;
+    for (int i = static_cast<int>(red.vars.size()) - 1; i >= 0; --i) {
+        const int64_t c = si.coef.count(red.vars[i].get()) ? si.coef.at(red.vars[i].get()) : 0;
+        if (red.extents[i] != 1 && c != rs) return false;
+        if (oi.coef.count(red.vars[i].get()) && oi.coef.at(red.vars[i].get()) != 0) return false;
+        rs *= red.extents[i];
+    }
+    *init_out = init;
+    *src_load = src;
+    *R = rows;
+    *reduce_kind = 0;
+    *out_buf = init->var.get();
+    return true;
+}
+
+}  // namespace
+
+HIPModuleSource CodeGenHIP::Generate(const tir::PrimFunc& func, const std::string& prefix) {
+    HIPModuleSource out;
+    Names names;
+    names.builtin_types = true;
+    std::ostringstream os;
+    os << "// generated by kxc CodeGenHIP for gfx950 (wave64)\n";
+    os << "#ifndef INFINITY\n#define INFINITY __builtin_inff()\n#endif\n#ifndef NAN\n#define NAN __builtin_nanf(\"\")\n#endif\n\n";
+
+    std::vector<Stmt> allocs, stages;
+    SplitStages(func->body, &allocs, &stages);
+    std::map<const ExprNode*, DataType> buffer_types;
+    for (const auto& p : func->params) buffer_types[p.get()] = p.dtype();
+    for (const auto& a : allocs) buffer_types[a->var.get()] = a->dtype;
+
+    int index = 0;
+    for (const auto& stage : stages) {
+        HIPKernelSpec spec;
+        std::vector<const ExprNode*> written;
+        CollectBuffers(stage, &spec.buffers, &written);
+        for (const ExprNode* b : spec.buffers)
+            if (!buffer_types.count(b)) throw std::runtime_error("CodeGenHIP: stage uses an undeclared buffer '" + b->name + "'");
+        const std::string target = written.empty() ? "stage" : names.Get(written[0]);
+        spec.symbol = prefix + "_s" + std::to_string(index++) + "_" + target;
+        names.Reserve(spec.symbol);
+
+        LoopNest data = PeelLoops(stage, true);
+        int64_t total = 1;
+        for (auto e : data.extents) total *= e;
+        if (total <= 0) total = 1;
+
+        os << "extern \"C\" __global__ void __launch_bounds__(256) " << spec.symbol << "(";
+        for (size_t i = 0; i < spec.buffers.size(); ++i) {
+            const ExprNode* b = spec.buffers[i];
+            const bool is_written = std::find(written.begin(), written.end(), b) != written.end();
+            os << (i ? ", " : "") << (is_written ? "" : "const ") << CType(buffer_types[b], true) << "* __restrict__ " << names.Get(b);
+        }
+        os << ") {\n";
+
+        Stmt init;
+        PrimExpr src;
+        int64_t R = 0;
+        int rkind = 0;
+        const ExprNode* obuf = nullptr;
+        if (MatchRowReduce(data, &init, &src, &R, &rkind, &obuf)) {
+            // ---- LDS-staged contiguous row reduction
+            const int64_t rp = R | 1;
+            spec.schedule = "lds_row_reduce";
+            spec.shared_bytes = 0;   // static LDS
+            const std::string o = names.Get(obuf), s = names.Get(src->args[0].get());
+            os << "  __shared__ float tile[" << 256 * rp << "];\n";
+            os << "  const long long total = " << total << "LL;\n";
+            os << "  for (long long base = (long long)blockIdx.x * 256; base < total; base += (long long)gridDim.x * 256) {\n";
+            os << "    const int rows = (int)((total - base) < 256 ? (total - base) : 256);\n";
+            os << "    for (int e = threadIdx.x; e < rows * " << R << "; e += 256) {\n";
+            os << "      const int row = e / " << R << ";\n";
+            os << "      tile[row * " << rp << " + (e - row * " << R << ")] = " << s << "[base * " << R << " + e];\n";
+            os << "    }\n    __syncthreads();\n";
+            os << "    if ((int)threadIdx.x < rows) {\n";
+            os << "      " << CType(buffer_types[obuf], true) << " acc = " << EmitExpr(init->a, &names) << ";\n";
+            os << "      for (int r = 0; r < " << R << "; ++r) acc = acc + tile[threadIdx.x * " << rp << " + r];\n";
+            os << "      " << o << "[base + threadIdx.x] = acc;\n";
+            os << "    }\n    __syncthreads();\n  }\n";
+        } else {
+            // ---- flat schedule: one output element per thread per grid-stride step
+            spec.schedule = "flat";
+            os << "  for (long long gid = (long long)blockIdx.x * 256 + threadIdx.x; gid < " << total
+               << "LL; gid += (long long)gridDim.x * 256) {\n";
+            // innermost data axis is lane-fastest
+            os << "    long long rem = gid;\n";
+            for (int i = static_cast<int>(data.vars.size()) - 1; i >= 0; --i) {
+                const std::string v = names.Get(data.vars[i].get());
+                if (i == 0) os << "    const int " << v << " = (int)rem;\n";
+                else {
+                    os << "    const int " << v << " = (int)(rem % " << data.extents[i] << "LL);\n";
+                    os << "    rem /= " << data.extents[i] << "LL;\n";
+                }
+            }
+            EmitStmt(data.body, &names, os, 4);
+            os << "  }\n";
+        }
+        os << "}\n\n";
+        int64_t blocks = (total + 255) / 256;
+        if (blocks > 256 * 32) blocks = 256 * 32;       // grid-stride beyond 32 workgroups per CU
+        if (blocks < 1) blocks = 1;
+        spec.grid[0] = static_cast<uint32_t>(blocks);
+        out.kernels.push_back(spec);
+    }
+    out.source = os.str();
+    return out;
+}
+
+}  // namespace codegen
+}  // namespace kxc

@@ -1,0 +1,524 @@
+// compiler.cc -- Compiler::Compile and CompiledModule (see compiler.h).
+#include "kxc/compiler.h"
+
+#include <dlfcn.h>
+#include <unistd.h>
+
+#include <atomic>
+#include <cstdio>
+#include <cstdlib>
+#include <fstream>
+#include <sstream>
+#include <unordered_map>
+#include <unordered_set>
+
+#include "kxc_hip.h"
+
+namespace kxc {
+namespace api {
+
+using relay::OpNode;
+
+constexpr const char* kKernelEntrySymbol = "kxc_kernel_main";   // src/api/compiler.cc:30
+
+CompileConfig CompileConfig::AOT(Target target, int opt_level) {
+    auto n = std::make_shared<CompileConfigNode>();
+    n->mode = CompileMode::kAOT;
+    n->opt_level = opt_level;
+    n->target = target;
+    return CompileConfig(n);
+}
+CompileConfig CompileConfig::JIT(Target target) {
+    auto n = std::make_shared<CompileConfigNode>();
+    n->mode = CompileMode::kJIT;
+    n->opt_level = 1;
+    n->target = target;
+    return CompileConfig(n);
+}
+
+class CompiledModuleImpl {
+public:
+    CompileConfig config;
+    tir::PrimFunc prim_func;
+    std::string source;
+    Array<runtime::NDArray> constants;
+    int64_t input_count = 0, constant_count = 0;
+    std::vector<KernelExecInfo> execs;
+    std::string status = "not compiled";
+    int num_values = 0;
+    std::vector<int> input_value_ids, constant_value_ids;
+    int output_value = -1;
+    // host back end
+    void* dl_handle = nullptr;
+    int32_t (*fn)(void**) = nullptr;
+    std::string so_path;
+    // hip back end
+    kxc_hip_plan* plan = nullptr;
+    std::vector<kxc_hip_module*> modules;
+    size_t workspace_bytes = 0;
+    bool ready = false;
+
+    ~CompiledModuleImpl() {
+        if (plan) kxc_hip_plan_destroy(plan);
+        for (auto* m : modules) kxc_hip_module_free(m);
+        if (dl_handle) dlclose(dl_handle);
+        if (!so_path.empty()) std::remove(so_path.c_str());
+    }
+};
+
+namespace {
+
+// ------------------------------------------------------------------ host back end
+void CompileHost(const Function& typed, const CompileConfig& config, CompiledModuleImpl* m) {
+    relay::LoweredFunc lowered = relay::LowerToTIRDetailed(typed);
+    m->prim_func = tir::RunTIRPassPipeline(lowered.func, {"fold_constant", "simplify_expr"});
+    m->constants = lowered.constants;
+    m->input_count = m->prim_func->int_attrs.at("kxc.input_count");
+    m->constant_count = m->prim_func->int_attrs.at("kxc.constant_count");
+    codegen::CodeGenC cg;
+    m->source = cg.Generate(m->prim_func, kKernelEntrySymbol);
+    static std::atomic<int> counter{0};
+    const char* tmp = std::getenv("TMPDIR");
+    const std::string base = std::string(tmp && *tmp ? tmp : "/tmp") + "/kxc_jit_" + std::to_string(getpid()) + "_" +
+                             std::to_string(counter.fetch_add(1));
+    const std::string c_path = base + ".c";
+    m->so_path = base + ".so";
+    {
+        std::ofstream out(c_path);
+        out << m->source;
+    }
+    const int level = config->opt_level < 0 ? 0 : config->opt_level > 3 ? 3 : config->opt_level;
+    // strict fp32: no contraction, no fast-math -- results do not depend on the optimisation level
+    const std::string cmd = "cc -std=gnu11 -O" + std::to_string(level) +
+                            " -fno-fast-math -ffp-contract=off -shared -fPIC -w -o " + m->so_path + " " + c_path + " -lm 2>&1";
+    FILE* pipe = popen(cmd.c_str(), "r");
+    if (!pipe) throw std::runtime_error("host compiler could not be started");
+    std::string log;
+    char buf[512];
+    while (fgets(buf, sizeof(buf), pipe)) log += buf;
+    const int rc = pclose(pipe);
+    std::remove(c_path.c_str());
+    if (rc != 0) throw std::runtime_error("host compilation of the generated C failed:\n" + log);
+    m->dl_handle = dlopen(m->so_path.c_str(), RTLD_NOW | RTLD_LOCAL);
+    if (!m->dl_handle) throw std::runtime_error(std::string("dlopen failed: ") + dlerror());
+    m->fn = reinterpret_cast<int32_t (*)(void**)>(dlsym(m->dl_handle, kKernelEntrySymbol));
+    if (!m->fn) throw std::runtime_error("generated library lacks kxc_kernel_main");
+    KernelExecInfo e;
+    e.op_name = "main";
+    e.kernel_symbol = kKernelEntrySymbol;
+    m->execs.push_back(e);
+    m->ready = true;
+    m->status = "ready (host C back end)";
+}
+
+// ------------------------------------------------------------------ hip back end
+struct Arena {
+    std::vector<std::pair<int64_t, int64_t>> free_list;   // offset, size
+    int64_t top = 0;
+    std::pair<int64_t, int64_t> Alloc(int64_t nbytes) {
+        const int64_t size = (std::max<int64_t>(nbytes, 1) + 255) / 256 * 256;
+        for (size_t i = 0; i < free_list.size(); ++i) {
+            if (free_list[i].second >= size) {
+                const int64_t off = free_list[i].first;
+                if (free_list[i].second == size) free_list.erase(free_list.begin() + i);
+                else { free_list[i].first += size; free_list[i].second -= size; }
+                return {off, size};
+            }
+        }
+        const int64_t off = top;
+        top += size;
+        return {off, size};
+    }
+    void Release(std::pair<int64_t, int64_t> blk) {
+        free_list.push_back(blk);
+        std::sort(free_list.begin(), free_list.end());
+        std::vector<std::pair<int64_t, int64_t>> merged;
+        for (auto& b : free_list) {
+            if (!merged.empty() && merged.back().first + merged.back().second == b.first) merged.back().second += b.second;
+            else merged.push_back(b);
+        }
+        free_list.swap(merged);
+    }
+};
+
+struct Group {
+    const CallNode* head = nullptr;     // the operator that is launched
+    const CallNode* tail = nullptr;     // the last call folded into it (its value is the group's output)
+    const RelayExprNode* residual = nullptr;
+    bool fused_relu = false;
+};
+
+template <typename T>
+const T* OpAttr(const OpNode* op, const char* key) {
+    auto it = op->attrs.find(key);
+    return it == op->attrs.end() ? nullptr : std::any_cast<T>(&it->second);
+}
+bool OpFlag(const OpNode* op, const char* key) {
+    const bool* b = OpAttr<bool>(op, key);
+    return b && *b;
+}
+const TensorTypeNode* TT(const Type& t) { return t.As<TensorTypeNode>(); }
+int64_t TypeBytes(const Type& t) { return Product(TT(t)->shape) * tir::DTypeFromString(TT(t)->dtype).bytes(); }
+
+class HipBuilder {
+public:
+    HipBuilder(const Function& f, const CompileConfig& cfg, CompiledModuleImpl* m, bool dry) : f_(f), cfg_(cfg), m_(m), dry_(dry) {}
+
+    void Build() {
+        Number();
+        FormGroups();
+        if (kxc_hip_plan_create(cfg_->target->device.device_id(), static_cast<int32_t>(num_args_), &m_->plan))
+            throw std::runtime_error(std::string("plan creation failed: ") + kxc_hip_last_error());
+        Emit();
+        m_->workspace_bytes = static_cast<size_t>(arena_.top);
+        if (!dry_) {
+            if (kxc_hip_plan_finalize(m_->plan, m_->workspace_bytes))
+                throw std::runtime_error(std::string("plan finalize failed: ") + kxc_hip_last_error());
+            m_->ready = true;
+            m_->status = "ready (hip back end, " + std::to_string(m_->execs.size()) + " launches)";
+        } else {
+            m_->status = "compiled without loading (no GPU): " + std::to_string(m_->execs.size()) + " launches";
+        }
+    }
+
+private:
+    // ---- value numbering: one id per Relay expression; DFS in argument order (the lowering's order)
+    void Number() {
+        for (const auto& p : f_->params) {
+            value_id_[p.get()] = next_value_++;
+            m_->input_value_ids.push_back(value_id_[p.get()]);
+            arg_index_[p.get()] = static_cast<int>(arg_index_.size());
+        }
+        num_inputs_ = static_cast<int>(f_->params.size());
+        Visit(f_->body);
+        num_args_ = num_inputs_ + static_cast<int>(constants_.size()) + 1;
+        for (size_t k = 0; k < constants_.size(); ++k) arg_index_[constants_[k]] = num_inputs_ + static_cast<int>(k);
+        m_->num_values = next_value_;
+        m_->output_value = value_id_.at(f_->body.get());
+    }
+    void Visit(const Expr& e) {
+        if (value_id_.count(e.get())) return;
+        if (const auto* c = e.As<ConstantNode>()) {
+            value_id_[e.get()] = next_value_++;
+            m_->constant_value_ids.push_back(value_id_[e.get()]);
+            constants_.push_back(e.get());
+            m_->constants.push_back(c->data);
+            return;
+        }
+        const auto* call = e.As<CallNode>();
+        if (!call) throw std::runtime_error("hip back end: unsupported Relay node (free variable or non-call expression)");
+        for (const auto& a : call->args) {
+            Visit(a);
+            consumers_[a.get()].push_back(call);
+        }
+        value_id_[e.get()] = next_value_++;
+        topo_.push_back(call);
+        expr_of_[call] = e;
+    }
+
+    const CallNode* SoleConsumer(const RelayExprNode* e) const {
+        auto it = consumers_.find(e);
+        if (it == consumers_.end() || it->second.size() != 1 || e == f_->body.get()) return nullptr;
+        return it->second[0];
+    }
+    static bool IsOp(const CallNode* c, const char* name) {
+        const auto* op = c->op.As<OpNode>();
+        return op && op->name == name;
+    }
+    static bool IsF32(const Type& t) { return TT(t) && TT(t)->dtype == "float32"; }
+
+    // ---- fusion: conv(+bias) -> [add(conv_out, skip)] -> [relu];  binary -> [relu]
+    void FormGroups() {
+        std::unordered_set<const CallNode*> absorbed;
+        for (const CallNode* c : topo_) {
+            if (absorbed.count(c)) continue;
+            const auto* op = c->op.As<OpNode>();
+            Group g;
+            g.head = g.tail = c;
+            const bool dispatchable = cfg_->hip_use_handwritten && OpAttr<relay::FHIPDispatch>(op, "FHIPDispatch") &&
+                                      IsF32(c->checked_type_);
+            if (cfg_->hip_fuse && dispatchable) {
+                if (OpFlag(op, "THIPFusable")) {
+                    const CallNode* n = SoleConsumer(g.tail);
+                    if (n && !absorbed.count(n) && IsOp(n, "add") && n->args.size() == 2 && n->args[0].get() != n->args[1].get()) {
+                        const RelayExprNode* other = n->args[0].get() == g.tail ? n->args[1].get() : n->args[0].get();
+                        if (TT(other->checked_type_)->shape == TT(c->checked_type_)->shape && IsF32(other->checked_type_)) {
+                            g.residual = other;
+                            g.tail = n;
+                            absorbed.insert(n);
+                        }
+                    }
+                    n = SoleConsumer(g.tail);
+                    if (n && !absorbed.count(n) && IsOp(n, "nn_relu")) { g.fused_relu = true; g.tail = n; absorbed.insert(n); }
+                } else if (OpFlag(op, "THIPFusableRelu") && TT(c->checked_type_)->shape.size() <= 6) {
+                    const CallNode* n = SoleConsumer(g.tail);
+                    if (n && !absorbed.count(n) && IsOp(n, "nn_relu")) { g.fused_relu = true; g.tail = n; absorbed.insert(n); }
+                }
+            }
+            group_of_tail_[g.tail] = groups_.size();
+            groups_.push_back(g);
+        }
+    }
+
+    // ---- buffers
+    relay::HIPBuffer BufferOf(const RelayExprNode* e) {
+        e = Resolve(e);
+        auto a = arg_index_.find(e);
+        if (a != arg_index_.end()) return {KXC_HIP_BUF_ARG, a->second};
+        auto s = slot_.find(e);
+        if (s == slot_.end()) {
+            const auto* c = dynamic_cast<const CallNode*>(e);
+            const auto* op = c ? c->op.As<OpNode>() : nullptr;
+            throw std::runtime_error("hip back end: value " + std::to_string(value_id_.count(e) ? value_id_.at(e) : -1) +
+                                     " (" + (op ? op->name : std::string("?")) + ") used before it is produced");
+        }
+        return {KXC_HIP_BUF_WORKSPACE, s->second.first};
+    }
+    const RelayExprNode* Resolve(const RelayExprNode* e) const {
+        auto it = alias_.find(e);
+        while (it != alias_.end()) { e = it->second; it = alias_.find(e); }
+        return e;
+    }
+
+    void Emit() {
+        // emission order = topo order of the group tails
+        std::vector<size_t> order;
+        for (const CallNode* c : topo_) {
+            auto it = group_of_tail_.find(c);
+            if (it != group_of_tail_.end()) order.push_back(it->second);
+        }
+        // last reader of every (resolved) value, in emission steps; alias ops are transparent
+        std::unordered_map<const RelayExprNode*, int> last_use;
+        std::vector<bool> is_alias(groups_.size(), false);
+        for (size_t step = 0; step < order.size(); ++step) {
+            const Group& g = groups_[order[step]];
+            const auto* op = g.head->op.As<OpNode>();
+            if (OpFlag(op, "THIPAlias") && g.tail != f_->body.get() && g.head == g.tail) {
+                is_alias[order[step]] = true;
+                alias_[g.head] = g.head->args[0].get();
+            }
+        }
+        for (size_t step = 0; step < order.size(); ++step) {
+            const Group& g = groups_[order[step]];
+            if (is_alias[order[step]]) continue;
+            for (const auto& a : g.head->args) last_use[Resolve(a.get())] = static_cast<int>(step);
+            if (g.residual) last_use[Resolve(g.residual)] = static_cast<int>(step);
+        }
+        last_use[Resolve(f_->body.get())] = static_cast<int>(order.size());
+
+        for (size_t step = 0; step < order.size(); ++step) {
+            const Group& g = groups_[order[step]];
+            if (is_alias[order[step]]) continue;
+            const auto* op = g.head->op.As<OpNode>();
+            // output buffer
+            relay::HIPBuffer out;
+            if (g.tail == f_->body.get()) {
+                out = {KXC_HIP_BUF_ARG, num_args_ - 1};
+            } else {
+                slot_[g.tail] = arena_.Alloc(TypeBytes(g.tail->checked_type_));
+                out = {KXC_HIP_BUF_WORKSPACE, slot_[g.tail].first};
+            }
+            relay::HIPDispatchContext ctx;
+            ctx.attrs = g.head->attrs;
+            for (const auto& a : g.head->args) {
+                ctx.input_types.push_back(a.checked_type());
+                ctx.inputs.push_back(BufferOf(a.get()));
+            }
+            ctx.out_type = g.tail->checked_type_;
+            ctx.output = out;
+            ctx.fused_relu = g.fused_relu;
+            ctx.has_residual = g.residual != nullptr;
+            if (g.residual) ctx.residual = BufferOf(g.residual);
+
+            KernelExecInfo info;
+            info.op_name = op->name;
+            for (const auto& a : g.head->args) info.input_values.push_back(value_id_.at(a.get()));
+            if (g.residual) info.input_values.push_back(value_id_.at(g.residual));
+            info.output_values.push_back(value_id_.at(g.tail));
+
+            std::string symbol;
+            const auto* dispatch = cfg_->hip_use_handwritten ? OpAttr<relay::FHIPDispatch>(op, "FHIPDispatch") : nullptr;
+            if (OpFlag(op, "THIPAlias")) {
+                // a view that is the function's result: materialise it with a copy
+                if (kxc_hip_plan_add_copy(m_->plan, TypeBytes(g.tail->checked_type_), {ctx.inputs[0].kind, ctx.inputs[0].index_or_offset},
+                                          {out.kind, out.index_or_offset}))
+                    throw std::runtime_error(std::string("plan copy failed: ") + kxc_hip_last_error());
+                symbol = "kxc_copy";
+            } else if (dispatch) {
+                symbol = (*dispatch)(ctx, m_->plan);
+            }
+            if (!symbol.empty()) {
+                info.kernel_symbol = symbol;
+                m_->execs.push_back(info);
+            } else {
+                if (g.fused_relu || g.residual) throw std::runtime_error("hip back end: operator declined a fused launch: " + op->name);
+                EmitGenerated(g, ctx, info, static_cast<int>(step));
+            }
+            // release everything whose last reader has now been enqueued
+            for (auto it = slot_.begin(); it != slot_.end();) {
+                auto lu = last_use.find(it->first);
+                if (lu == last_use.end() || lu->second <= static_cast<int>(step)) {
+                    if (lu == last_use.end() && it->first == g.tail) { ++it; continue; }   // produced now, unread: keep until end
+                    arena_.Release(it->second);
+                    it = slot_.erase(it);
+                } else {
+                    ++it;
+                }
+            }
+        }
+    }
+
+    // ---- operators without a hand-written kernel: FRelayToTE -> TIR -> CodeGenHIP -> hipRTC
+    void EmitGenerated(const Group& g, const relay::HIPDispatchContext& ctx, const KernelExecInfo& info, int step) {
+        Array<Var> params;
+        Array<Expr> args;
+        for (size_t i = 0; i < g.head->args.size(); ++i) {
+            Var v("in" + std::to_string(i), g.head->args[i].checked_type());
+            params.push_back(v);
+            args.push_back(v);
+        }
+        Function mini(params, Call(g.head->op, args, g.head->attrs));
+        relay::LoweredFunc lowered = relay::LowerToTIRDetailed(relay::InferTypePass(mini));
+        tir::PrimFunc pf = tir::RunTIRPassPipeline(lowered.func, {"fold_constant", "simplify_expr"});
+        codegen::CodeGenHIP cg;
+        codegen::HIPModuleSource src = cg.Generate(pf, "kxc_g" + std::to_string(step));
+        m_->source += src.source;
+        // buffers: mini-function parameters map to the group's operands, intermediates to scratch slots
+        std::unordered_map<const tir::ExprNode*, relay::HIPBuffer> buf;
+        for (size_t i = 0; i < g.head->args.size(); ++i) buf[pf->params[i].get()] = ctx.inputs[i];
+        buf[pf->params.back().get()] = ctx.output;
+        std::vector<std::pair<int64_t, int64_t>> scratch;
+        for (const auto& im : lowered.intermediates) {
+            scratch.push_back(arena_.Alloc(im.elements * im.dtype.bytes()));
+            buf[im.var] = {KXC_HIP_BUF_WORKSPACE, scratch.back().first};
+        }
+        kxc_hip_module* module = nullptr;
+        std::vector<char> log(16384, 0);
+        if (dry_) {
+            size_t size = 0;
+            if (kxc_hip_module_compile_only(src.source.c_str(), "kxc_generated.hip", &size, log.data(), log.size()))
+                throw std::runtime_error(std::string("generated HIP source does not compile: ") + kxc_hip_last_error());
+        } else {
+            if (kxc_hip_module_compile(src.source.c_str(), "kxc_generated.hip", &module, log.data(), log.size()))
+                throw std::runtime_error(std::string("generated HIP source does not compile: ") + kxc_hip_last_error());
+            m_->modules.push_back(module);
+        }
+        for (const auto& k : src.kernels) {
+            KernelExecInfo e = info;
+            e.kernel_symbol = k.symbol + " [generated:" + k.schedule + "]";
+            m_->execs.push_back(e);
+            if (dry_) continue;
+            void* fn = nullptr;
+            if (kxc_hip_module_get_function(module, k.symbol.c_str(), &fn))
+                throw std::runtime_error(std::string("generated kernel not found: ") + kxc_hip_last_error());
+            std::vector<kxc_hip_buf> params_buf;
+            for (const tir::ExprNode* b : k.buffers) {
+                auto it = buf.find(b);
+                if (it == buf.end()) throw std::runtime_error("generated kernel uses an unmapped buffer");
+                params_buf.push_back({it->second.kind, it->second.index_or_offset});
+            }
+            if (kxc_hip_plan_add_module_kernel(m_->plan, fn, k.symbol.c_str(), k.grid, k.block, k.shared_bytes, params_buf.data(),
+                                               static_cast<int32_t>(params_buf.size())))
+                throw std::runtime_error(std::string("plan_add_module_kernel failed: ") + kxc_hip_last_error());
+        }
+        for (auto& s : scratch) arena_.Release(s);
+    }
+
+    const Function& f_;
+    const CompileConfig& cfg_;
+    CompiledModuleImpl* m_;
+    bool dry_;
+    int next_value_ = 0, num_inputs_ = 0, num_args_ = 0;
+    std::unordered_map<const RelayExprNode*, int> value_id_, arg_index_;
+    std::vector<const RelayExprNode*> constants_;
+    std::unordered_map<const RelayExprNode*, std::vector<const CallNode*>> consumers_;
+    std::vector<const CallNode*> topo_;
+    std::unordered_map<const CallNode*, Expr> expr_of_;
+    std::vector<Group> groups_;
+    std::unordered_map<const CallNode*, size_t> group_of_tail_;
+    std::unordered_map<const RelayExprNode*, const RelayExprNode*> alias_;
+    std::unordered_map<const RelayExprNode*, std::pair<int64_t, int64_t>> slot_;
+    Arena arena_;
+};
+
+}  // namespace
+
+CompiledModule Compiler::Compile(Function func, CompileConfig config) {
+    if (!config.defined() || !config->target.defined()) throw std::runtime_error("Compiler::Compile: config has no target");
+    auto impl = std::make_shared<CompiledModuleImpl>();
+    impl->config = config;
+    Function typed = relay::InferTypePass(func);
+    if (config->target->kind == "hip") {
+        // the whole-function TIR is kept for inspection (GetPrimFunc) and fixes the parameter order
+        relay::LoweredFunc whole = relay::LowerToTIRDetailed(typed);
+        impl->prim_func = tir::RunTIRPassPipeline(whole.func, {"fold_constant", "simplify_expr"});
+        impl->input_count = impl->prim_func->int_attrs.at("kxc.input_count");
+        impl->constant_count = impl->prim_func->int_attrs.at("kxc.constant_count");
+        const bool dry = config->target->attrs.exists == 0;
+        HipBuilder builder(typed, config, impl.get(), dry);
+        builder.Build();
+        if (static_cast<int64_t>(impl->constants.size()) != impl->constant_count)
+            throw std::runtime_error("hip back end: constant order disagrees with the lowering");
+    } else {
+        CompileHost(typed, config, impl.get());
+    }
+    return CompiledModule(impl);
+}
+
+void CompiledModule::Run(const std::vector<void*>& packed_args) {
+    if (!impl_ || !impl_->ready) throw std::runtime_error("CompiledModule::Run: module is not ready: " + GetStatus());
+    const size_t expect = static_cast<size_t>(impl_->input_count + impl_->constant_count + 1);
+    if (packed_args.size() != expect)
+        throw std::runtime_error("CompiledModule::Run: expected " + std::to_string(expect) + " packed arguments, got " +
+                                 std::to_string(packed_args.size()));
+    if (impl_->fn) {
+        const int32_t rc = impl_->fn(const_cast<void**>(packed_args.data()));
+        if (rc != 0) throw std::runtime_error("Kernel kxc_kernel_main returned error code " + std::to_string(rc));
+        return;
+    }
+    if (kxc_hip_plan_run(impl_->plan, const_cast<void**>(packed_args.data()), nullptr))
+        throw std::runtime_error(std::string("Kernel kxc_kernel_main failed: ") + kxc_hip_last_error());
+    if (impl_->config->sync_after_run) {
+        if (kxc_hip_stream_sync(impl_->config->target->device.device_id(), nullptr))
+            throw std::runtime_error(std::string("HIP StreamSync failed: ") + kxc_hip_last_error());
+    }
+}
+
+bool CompiledModule::IsReady() const { return impl_ && impl_->ready; }
+std::string CompiledModule::GetStatus() const { return impl_ ? impl_->status : "empty"; }
+const tir::PrimFunc& CompiledModule::GetPrimFunc() const { return impl_->prim_func; }
+const std::string& CompiledModule::GetSource() const { return impl_->source; }
+void CompiledModule::SaveCSource(const std::string& path) const {
+    std::ofstream out(path);
+    if (!out) throw std::runtime_error("SaveCSource: cannot open " + path);
+    out << impl_->source;
+}
+const Array<runtime::NDArray>& CompiledModule::GetConstants() const { return impl_->constants; }
+int64_t CompiledModule::input_count() const { return impl_->input_count; }
+int64_t CompiledModule::constant_count() const { return impl_->constant_count; }
+const std::vector<KernelExecInfo>& CompiledModule::GetKernelExecs() const { return impl_->execs; }
+size_t CompiledModule::workspace_bytes() const { return impl_->workspace_bytes; }
+
+std::string CompiledModule::ExecutionPlanJSON() const {
+    std::ostringstream os;
+    os << "{\"schema_version\":1,\"num_values\":" << impl_->num_values << ",\"output_value\":" << impl_->output_value
+       << ",\"input_value_ids\":[";
+    for (size_t i = 0; i < impl_->input_value_ids.size(); ++i) os << (i ? "," : "") << impl_->input_value_ids[i];
+    os << "],\"constant_value_ids\":[";
+    for (size_t i = 0; i < impl_->constant_value_ids.size(); ++i) os << (i ? "," : "") << impl_->constant_value_ids[i];
+    os << "],\"nodes\":[";
+    for (size_t i = 0; i < impl_->execs.size(); ++i) {
+        const auto& e = impl_->execs[i];
+        os << (i ? "," : "") << "{\"kind\":\"kernel_exec\",\"op_name\":\"" << e.op_name << "\",\"kernel_symbol\":\""
+           << e.kernel_symbol << "\",\"input_values\":[";
+        for (size_t k = 0; k < e.input_values.size(); ++k) os << (k ? "," : "") << e.input_values[k];
+        os << "],\"output_values\":[";
+        for (size_t k = 0; k < e.output_values.size(); ++k) os << (k ? "," : "") << e.output_values[k];
+        os << "],\"worker_set\":[0]}";
+    }
+    os << "]}";
+    return os.str();
+}
+
+}  // namespace api
+}  // namespace kxc

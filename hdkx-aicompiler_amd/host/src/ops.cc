@@ -1,0 +1,352 @@
+// ops.cc -- built-in operator registrations: shape rule, TE compute definition (the CPU / generic
+// definition, src/relay/op/nn/*.cc and src/relay/op/tensor/*.cc of the reference) and, where a
+// hand-written gfx950 kernel exists, the FHIPDispatch hook that adds its launch to a plan.
+#include <algorithm>
+
+#include "kxc/op.h"
+#include "kxc/topi.h"
+#include "kxc_hip.h"
+
+namespace kxc {
+namespace relay {
+
+namespace {
+
+int Read2D(const std::vector<int64_t>& v, int idx, int dflt) {
+    return idx >= 0 && static_cast<size_t>(idx) < v.size() ? static_cast<int>(v[idx]) : dflt;
+}
+std::vector<int> ReadPair(const std::vector<int64_t>& v, int dflt) {
+    if (v.size() >= 2) return {static_cast<int>(v[0]), static_cast<int>(v[1])};
+    return {dflt, dflt};
+}
+std::vector<int> ReadPad4(const std::vector<int64_t>& v) {
+    if (v.size() >= 4) return {static_cast<int>(v[0]), static_cast<int>(v[1]), static_cast<int>(v[2]), static_cast<int>(v[3])};
+    if (v.size() >= 2) return {static_cast<int>(v[0]), static_cast<int>(v[1]), static_cast<int>(v[0]), static_cast<int>(v[1])};
+    return {0, 0, 0, 0};
+}
+const TensorTypeNode* TT(const Type& t) { return t.As<TensorTypeNode>(); }
+kxc_hip_buf B(const HIPBuffer& b) { return kxc_hip_buf{b.kind, b.index_or_offset}; }
+bool IsF32(const Type& t) { return TT(t) && TT(t)->dtype == "float32"; }
+void Check(int32_t rc, const char* what) {
+    if (rc != 0) throw std::runtime_error(std::string(what) + ": " + kxc_hip_last_error());
+}
+
+// ---------------------------------------------------------------- nn_conv2d (src/relay/op/nn/convolution.cc:38-75)
+te::Tensor Conv2DCompute(const Attrs& attrs, const Array<te::Tensor>& in, const Type&) {
+    if (in.size() < 2 || in.size() > 3) throw std::runtime_error("nn_conv2d expects 2 or 3 inputs (data, weight[, bias])");
+    const auto* p = attrs.As<Conv2DAttrsNode>();
+    if (!p) throw std::runtime_error("nn_conv2d expects Conv2DAttrs");
+    if (p->data_layout != "NCHW" && !p->data_layout.empty()) throw std::runtime_error("nn_conv2d currently only supports NCHW");
+    if (in[0]->shape.size() != 4 || in[1]->shape.size() != 4)
+        throw std::runtime_error("nn_conv2d currently expects NCHW/OIHW rank-4 tensors");
+    if (in.size() == 3 && in[2]->shape.size() != 1) throw std::runtime_error("nn_conv2d bias must be rank-1");
+    // padding[0], padding[1] are applied on both sides (convolution.cc:53-54)
+    te::Tensor conv = te::topi::conv2d_nchw(in[0], in[1], Read2D(p->strides, 0, 1), Read2D(p->strides, 1, 1),
+                                            Read2D(p->padding, 0, 0), Read2D(p->padding, 1, 0), Read2D(p->dilation, 0, 1),
+                                            Read2D(p->dilation, 1, 1), "T_conv2d");
+    if (in.size() == 2) return conv;
+    te::Tensor bias = in[2];
+    return te::compute(conv->shape, [&](const Array<tir::Var>& ax) { return conv(ax) + bias(ax[1]); }, "T_conv2d_bias_add");
+}
+
+std::string Conv2DDispatch(const HIPDispatchContext& c, kxc_hip_plan* plan) {
+    const auto* p = c.attrs.As<Conv2DAttrsNode>();
+    if (!p || !IsF32(c.input_types[0]) || !IsF32(c.out_type)) return "";
+    const auto* x = TT(c.input_types[0]);
+    const auto* w = TT(c.input_types[1]);
+    kxc_hip_conv2d_desc d{};
+    d.n = static_cast<int32_t>(x->shape[0]); d.c = static_cast<int32_t>(x->shape[1]);
+    d.h = static_cast<int32_t>(x->shape[2]); d.w = static_cast<int32_t>(x->shape[3]);
+    d.o = static_cast<int32_t>(w->shape[0]); d.kh = static_cast<int32_t>(w->shape[2]); d.kw = static_cast<int32_t>(w->shape[3]);
+    d.stride_h = Read2D(p->strides, 0, 1); d.stride_w = Read2D(p->strides, 1, 1);
+    d.pad_h = Read2D(p->padding, 0, 0); d.pad_w = Read2D(p->padding, 1, 0);
+    d.dil_h = Read2D(p->dilation, 0, 1); d.dil_w = Read2D(p->dilation, 1, 1);
+    const bool has_bias = c.inputs.size() == 3;
+    d.flags = (has_bias ? KXC_HIP_CONV_BIAS : 0u) | (c.has_residual ? KXC_HIP_CONV_RESIDUAL : 0u) |
+              (c.fused_relu ? KXC_HIP_CONV_RELU : 0u);
+    const kxc_hip_buf none{KXC_HIP_BUF_NONE, 0};
+    Check(kxc_hip_plan_add_conv2d(plan, &d, B(c.inputs[0]), B(c.inputs[1]), has_bias ? B(c.inputs[2]) : none,
+                                  c.has_residual ? B(c.residual) : none, B(c.output)),
+          "nn_conv2d dispatch");
+    return std::string("kxc_conv2d_nchw_f32.") + kxc_hip_conv2d_variant(&d) + (has_bias ? "+bias" : "") +
+           (c.has_residual ? "+add" : "") + (c.fused_relu ? "+relu" : "");
+}
+
+// ---------------------------------------------------------------- pooling (src/relay/op/nn/pooling.cc:50-98)
+te::Tensor PoolCompute(const char* op, const char* type, const char* tname, const Attrs& attrs, const Array<te::Tensor>& in) {
+    if (in.size() != 1) throw std::runtime_error(std::string(op) + " expects exactly 1 input");
+    const auto* p = attrs.As<MaxPool2DAttrsNode>();
+    if (!p) throw std::runtime_error(std::string(op) + " expects MaxPool2DAttrs");
+    if ((p->layout != "NCHW" && !p->layout.empty()) || in[0]->shape.size() != 4)
+        throw std::runtime_error(std::string(op) + " expects NCHW rank-4 input");
+    return te::topi::pool2d(in[0], ReadPair(p->pool_size, 1), ReadPair(p->strides, 1), ReadPad4(p->padding), type,
+                            p->ceil_mode, tname);
+}
+
+std::string PoolDispatch(bool is_avg, const HIPDispatchContext& c, kxc_hip_plan* plan) {
+    const auto* p = c.attrs.As<MaxPool2DAttrsNode>();
+    if (!p || !IsF32(c.input_types[0])) return "";
+    const auto* x = TT(c.input_types[0]);
+    const auto ks = ReadPair(p->pool_size, 1), st = ReadPair(p->strides, 1), pd = ReadPad4(p->padding);
+    kxc_hip_pool2d_desc d{};
+    d.n = static_cast<int32_t>(x->shape[0]); d.c = static_cast<int32_t>(x->shape[1]);
+    d.h = static_cast<int32_t>(x->shape[2]); d.w = static_cast<int32_t>(x->shape[3]);
+    d.kh = ks[0]; d.kw = ks[1]; d.stride_h = st[0]; d.stride_w = st[1];
+    d.pad_top = pd[0]; d.pad_left = pd[1]; d.pad_bottom = pd[2]; d.pad_right = pd[3];
+    d.ceil_mode = p->ceil_mode ? 1 : 0;
+    d.is_avg = is_avg ? 1 : 0;
+    Check(kxc_hip_plan_add_pool2d(plan, &d, B(c.inputs[0]), B(c.output)), "pool2d dispatch");
+    return is_avg ? "kxc_avg_pool2d_f32" : "kxc_max_pool2d_f32";
+}
+
+std::string GapDispatch(const HIPDispatchContext& c, kxc_hip_plan* plan) {
+    if (!IsF32(c.input_types[0])) return "";
+    const auto* x = TT(c.input_types[0]);
+    Check(kxc_hip_plan_add_global_avg_pool2d(plan, x->shape[0], x->shape[1], x->shape[2], x->shape[3], B(c.inputs[0]),
+                                             B(c.output)),
+          "nn_global_avg_pool2d dispatch");
+    return "kxc_global_avg_pool2d_f32";
+}
+
+// ---------------------------------------------------------------- dense / gemm (src/relay/op/nn/dense.cc:17-61)
+te::Tensor ScaleTensor(const te::Tensor& t, double scale, const std::string& name) {
+    if (scale == 1.0) return t;
+    return te::compute(t->shape, [&](const Array<tir::Var>& ax) { return t(ax) * te::topi::make_const(t->dtype, scale); }, name);
+}
+
+te::Tensor GemmCompute(const Attrs& attrs, const Array<te::Tensor>& in, const Type&) {
+    if (in.size() != 3) throw std::runtime_error("nn_gemm expects exactly 3 inputs");
+    const auto* p = attrs.As<GemmAttrsNode>();
+    if (!p) throw std::runtime_error("nn_gemm expects GemmAttrs");
+    if (p->transA != 0) throw std::runtime_error("nn_gemm currently does not support transA=1");
+    te::Tensor out = p->transB == 1 ? te::topi::dense(in[0], in[1], "T_gemm_dense") : te::topi::matmul(in[0], in[1], "T_gemm_matmul");
+    out = ScaleTensor(out, p->alpha, "T_gemm_alpha");
+    te::Tensor bias = in[2];
+    if (p->beta != 1.0) bias = ScaleTensor(in[2], p->beta, "T_gemm_beta");
+    return te::topi::add(out, bias, "T_gemm_out");
+}
+
+std::string GemmDispatch(const HIPDispatchContext& c, kxc_hip_plan* plan) {
+    const auto* p = c.attrs.As<GemmAttrsNode>();
+    if (!p || p->transA != 0 || !IsF32(c.input_types[0])) return "";
+    const auto* a = TT(c.input_types[0]);
+    const auto* o = TT(c.out_type);
+    const auto* bias = TT(c.input_types[2]);
+    const int64_t c_len = Product(bias->shape);
+    if (bias->shape.size() > 1 || (c_len != o->shape[1] && c_len != 1)) return "";   // general bias shapes: generic path
+    Check(kxc_hip_plan_add_gemm(plan, o->shape[0], o->shape[1], a->shape[1], p->alpha, p->beta, p->transB, c_len,
+                                B(c.inputs[0]), B(c.inputs[1]), B(c.inputs[2]), B(c.output)),
+          "nn_gemm dispatch");
+    return "kxc_gemm_f32";
+}
+
+std::string DenseDispatch(bool transB, const HIPDispatchContext& c, kxc_hip_plan* plan) {
+    if (!IsF32(c.input_types[0])) return "";
+    const auto* a = TT(c.input_types[0]);
+    const auto* o = TT(c.out_type);
+    const kxc_hip_buf none{KXC_HIP_BUF_NONE, 0};
+    Check(kxc_hip_plan_add_gemm(plan, o->shape[0], o->shape[1], a->shape[1], 1.0f, 1.0f, transB ? 1 : 0, 0, B(c.inputs[0]),
+                                B(c.inputs[1]), none, B(c.output)),
+          "nn_dense dispatch");
+    return "kxc_gemm_f32";
+}
+
+// ---------------------------------------------------------------- elementwise
+std::string BinaryDispatch(int op, const HIPDispatchContext& c, kxc_hip_plan* plan) {
+    if (!IsF32(c.input_types[0]) || !IsF32(c.input_types[1])) return "";
+    const auto* a = TT(c.input_types[0]);
+    const auto* b = TT(c.input_types[1]);
+    if (a->shape.size() > 6 || b->shape.size() > 6) return "";
+    Check(kxc_hip_plan_add_binary(plan, op, a->shape.data(), static_cast<int32_t>(a->shape.size()), b->shape.data(),
+                                  static_cast<int32_t>(b->shape.size()), c.fused_relu ? 1 : 0, B(c.inputs[0]), B(c.inputs[1]),
+                                  B(c.output)),
+          "broadcast dispatch");
+    static const char* names[4] = {"kxc_add_f32", "kxc_subtract_f32", "kxc_multiply_f32", "kxc_divide_f32"};
+    return std::string(names[op]) + (c.fused_relu ? "+relu" : "");
+}
+
+std::string ReluDispatch(const HIPDispatchContext& c, kxc_hip_plan* plan) {
+    if (!IsF32(c.input_types[0])) return "";
+    Check(kxc_hip_plan_add_relu(plan, Product(TT(c.input_types[0])->shape), B(c.inputs[0]), B(c.output)), "nn_relu dispatch");
+    return "kxc_relu_f32";
+}
+
+FRelayToTE BinaryCompute(int op, const char* name) {
+    return [op, name](const Attrs&, const Array<te::Tensor>& in, const Type&) {
+        if (in.size() != 2) throw std::runtime_error(std::string(name) + " expects exactly 2 inputs");
+        static const char* tnames[4] = {"T_add", "T_subtract", "T_multiply", "T_divide"};
+        return te::topi::broadcast_binary(op, in[0], in[1], tnames[op]);
+    };
+}
+
+bool g_registered = false;
+
+}  // namespace
+
+void EnsureBuiltinOpsRegistered() {
+    static bool done = [] {
+        g_registered = true;
+        OpRegEntry::Register("nn_conv2d")
+            .describe("2D convolution, NCHW data and OIHW weights, optional rank-1 bias.")
+            .set_num_inputs(-1)
+            .add_argument("data", "Tensor", "The input tensor.")
+            .add_argument("weight", "Tensor", "The weight tensor.")
+            .set_attr<std::string>("TAttrs", "Conv2DAttrs")
+            .set_attr<FInferType>("FInferType", Conv2DInferType)
+            .set_attr<FRelayToTE>("FRelayToTE", Conv2DCompute)
+            .set_attr<bool>("THIPFusable", true)
+            .set_attr<FHIPDispatch>("FHIPDispatch", Conv2DDispatch);
+        OpRegEntry::Register("nn_relu")
+            .describe("Rectified Linear Unit activation")
+            .set_num_inputs(1)
+            .add_argument("data", "Tensor", "The input tensor.")
+            .set_attr<std::string>("TAttrs", "ReluAttrs")
+            .set_attr<FInferType>("FInferType", UnarySameInferType)
+            .set_attr<FRelayToTE>("FRelayToTE", [](const Attrs&, const Array<te::Tensor>& in, const Type&) {
+                if (in.size() != 1) throw std::runtime_error("nn_relu expects exactly 1 input");
+                return te::topi::relu(in[0], "T_relu");
+            })
+            .set_attr<FHIPDispatch>("FHIPDispatch", ReluDispatch);
+        OpRegEntry::Register("nn_max_pool2d")
+            .describe("2D max pooling operation.")
+            .set_num_inputs(1)
+            .add_argument("data", "Tensor", "The input tensor.")
+            .set_attr<std::string>("TAttrs", "MaxPool2DAttrs")
+            .set_attr<FInferType>("FInferType", Pool2DInferType)
+            .set_attr<FRelayToTE>("FRelayToTE", [](const Attrs& a, const Array<te::Tensor>& in, const Type&) {
+                return PoolCompute("nn_max_pool2d", "max", "T_max_pool2d", a, in);
+            })
+            .set_attr<FHIPDispatch>("FHIPDispatch", [](const HIPDispatchContext& c, kxc_hip_plan* p) { return PoolDispatch(false, c, p); });
+        OpRegEntry::Register("nn_avg_pool2d")
+            .describe("2D average pooling operation.")
+            .set_num_inputs(1)
+            .add_argument("data", "Tensor", "The input tensor.")
+            .set_attr<std::string>("TAttrs", "MaxPool2DAttrs")
+            .set_attr<FInferType>("FInferType", Pool2DInferType)
+            .set_attr<FRelayToTE>("FRelayToTE", [](const Attrs& a, const Array<te::Tensor>& in, const Type&) {
+                return PoolCompute("nn_avg_pool2d", "avg", "T_avg_pool2d", a, in);
+            })
+            .set_attr<FHIPDispatch>("FHIPDispatch", [](const HIPDispatchContext& c, kxc_hip_plan* p) { return PoolDispatch(true, c, p); });
+        OpRegEntry::Register("nn_global_avg_pool2d")
+            .describe("Global average pooling: reduces H and W to 1x1 by averaging.")
+            .set_num_inputs(1)
+            .add_argument("data", "Tensor", "The input tensor.")
+            .set_attr<std::string>("TAttrs", "GlobalAvgPool2DAttrs")
+            .set_attr<FInferType>("FInferType", GlobalAvgPool2DInferType)
+            .set_attr<FRelayToTE>("FRelayToTE", [](const Attrs&, const Array<te::Tensor>& in, const Type&) {
+                if (in.size() != 1) throw std::runtime_error("nn_global_avg_pool2d expects exactly 1 input");
+                if (in[0]->shape.size() != 4) throw std::runtime_error("nn_global_avg_pool2d expects NCHW rank-4 input");
+                return te::topi::global_avg_pool2d(in[0], "T_global_avg_pool2d");
+            })
+            .set_attr<FHIPDispatch>("FHIPDispatch", GapDispatch);
+        OpRegEntry::Register("nn_dense")
+            .describe("Dense (fully connected) layer")
+            .set_num_inputs(2)
+            .add_argument("data", "Tensor", "The input tensor.")
+            .add_argument("weight", "Tensor", "The weight tensor.")
+            .set_attr<std::string>("TAttrs", "DenseAttrs")
+            .set_attr<FInferType>("FInferType", DenseInferType)
+            .set_attr<FRelayToTE>("FRelayToTE", [](const Attrs&, const Array<te::Tensor>& in, const Type&) {
+                if (in.size() != 2) throw std::runtime_error("nn_dense expects exactly 2 inputs");
+                return te::topi::dense(in[0], in[1], "T_dense");
+            })
+            .set_attr<FHIPDispatch>("FHIPDispatch", [](const HIPDispatchContext& c, kxc_hip_plan* p) { return DenseDispatch(true, c, p); });
+        OpRegEntry::Register("matmul")
+            .describe("Matrix multiplication [M,K] x [K,N]")
+            .set_num_inputs(2)
+            .add_argument("lhs", "Tensor", "The first input tensor.")
+            .add_argument("rhs", "Tensor", "The second input tensor.")
+            .set_attr<FInferType>("FInferType", MatmulInferType)
+            .set_attr<FRelayToTE>("FRelayToTE", [](const Attrs&, const Array<te::Tensor>& in, const Type&) {
+                if (in.size() != 2) throw std::runtime_error("matmul expects exactly 2 inputs");
+                return te::topi::matmul(in[0], in[1], "T_matmul");
+            })
+            .set_attr<FHIPDispatch>("FHIPDispatch", [](const HIPDispatchContext& c, kxc_hip_plan* p) { return DenseDispatch(false, c, p); });
+        OpRegEntry::Register("nn_gemm")
+            .describe("General matrix multiplication.")
+            .set_num_inputs(3)
+            .add_argument("A", "Tensor", "The first input tensor.")
+            .add_argument("B", "Tensor", "The second input tensor.")
+            .add_argument("C", "Tensor", "The third input tensor (bias).")
+            .set_attr<std::string>("TAttrs", "GemmAttrs")
+            .set_attr<FInferType>("FInferType", GemmInferType)
+            .set_attr<FRelayToTE>("FRelayToTE", GemmCompute)
+            .set_attr<FHIPDispatch>("FHIPDispatch", GemmDispatch);
+        struct Bin { const char* name; int op; };
+        for (Bin b : {Bin{"add", 0}, Bin{"subtract", 1}, Bin{"mul", 2}, Bin{"multiply", 2}, Bin{"divide", 3}}) {
+            const int op = b.op;
+            OpRegEntry::Register(b.name)
+                .describe("Elementwise binary operator with numpy-style broadcasting")
+                .set_num_inputs(2)
+                .add_argument("lhs", "Tensor", "The first input tensor.")
+                .add_argument("rhs", "Tensor", "The second input tensor.")
+                .set_attr<FInferType>("FInferType", BroadcastInferType)
+                .set_attr<FRelayToTE>("FRelayToTE", BinaryCompute(op, b.name))
+                .set_attr<bool>("THIPFusableRelu", true)
+                .set_attr<FHIPDispatch>("FHIPDispatch", [op](const HIPDispatchContext& c, kxc_hip_plan* p) { return BinaryDispatch(op, c, p); });
+        }
+        for (const char* fn : {"sqrt", "exp", "log"}) {
+            const std::string name = fn;
+            OpRegEntry::Register(name)
+                .describe("Elementwise " + name)
+                .set_num_inputs(1)
+                .add_argument("data", "Tensor", "The input tensor.")
+                .set_attr<FInferType>("FInferType", UnarySameInferType)
+                .set_attr<FRelayToTE>("FRelayToTE", [name](const Attrs&, const Array<te::Tensor>& in, const Type&) {
+                    if (in.size() != 1) throw std::runtime_error(name + " expects exactly 1 input");
+                    return te::topi::unary_call(in[0], name, "T_" + name);
+                });
+        }
+        OpRegEntry::Register("nn_flatten")
+            .describe("Flattens all axes from `axis` on into one")
+            .set_num_inputs(1)
+            .add_argument("data", "Tensor", "The input tensor.")
+            .set_attr<std::string>("TAttrs", "FlattenAttrs")
+            .set_attr<FInferType>("FInferType", FlattenInferType)
+            .set_attr<FRelayToTE>("FRelayToTE", [](const Attrs&, const Array<te::Tensor>& in, const Type& out) {
+                return te::topi::reshape(in[0], out.As<TensorTypeNode>()->shape, "T_flatten");
+            })
+            .set_attr<bool>("THIPAlias", true);      // row-major view of the same memory: no launch
+        OpRegEntry::Register("reshape")
+            .describe("Row-major reshape")
+            .set_num_inputs(1)
+            .add_argument("data", "Tensor", "The input tensor.")
+            .set_attr<std::string>("TAttrs", "ReshapeAttrs")
+            .set_attr<FInferType>("FInferType", ReshapeInferType)
+            .set_attr<FRelayToTE>("FRelayToTE", [](const Attrs&, const Array<te::Tensor>& in, const Type& out) {
+                return te::topi::reshape(in[0], out.As<TensorTypeNode>()->shape, "T_reshape");
+            })
+            .set_attr<bool>("THIPAlias", true);
+        OpRegEntry::Register("transpose")
+            .describe("Axis permutation")
+            .set_num_inputs(1)
+            .add_argument("data", "Tensor", "The input tensor.")
+            .set_attr<std::string>("TAttrs", "TransposeAttrs")
+            .set_attr<FInferType>("FInferType", TransposeInferType)
+            .set_attr<FRelayToTE>("FRelayToTE", [](const Attrs& attrs, const Array<te::Tensor>& in, const Type&) {
+                const auto* a = attrs.As<TransposeAttrsNode>();
+                std::vector<int> axes;
+                if (a) for (auto v : a->axes) axes.push_back(static_cast<int>(v));
+                if (axes.empty()) for (int i = static_cast<int>(in[0]->shape.size()) - 1; i >= 0; --i) axes.push_back(i);
+                return te::topi::transpose(in[0], axes, "T_transpose");
+            });
+        OpRegEntry::Register("reduce_mean")
+            .describe("Mean over the given axes")
+            .set_num_inputs(1)
+            .add_argument("data", "Tensor", "The input tensor.")
+            .set_attr<std::string>("TAttrs", "ReduceMeanAttrs")
+            .set_attr<FInferType>("FInferType", ReduceMeanInferType)
+            .set_attr<FRelayToTE>("FRelayToTE", [](const Attrs& attrs, const Array<te::Tensor>& in, const Type&) {
+                const auto* a = attrs.As<ReduceMeanAttrsNode>();
+                if (!a) throw std::runtime_error("reduce_mean expects ReduceMeanAttrs");
+                std::vector<int> axes;
+                for (auto v : a->axes) axes.push_back(static_cast<int>(v));
+                return te::topi::reduce_mean(in[0], axes, a->keepdims != 0, "T_reduce_mean");
+            });
+        return true;
+    }();
+    (void)done;
+}
+
+}  // namespace relay
+}  // namespace kxc
