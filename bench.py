@@ -57,6 +57,7 @@ def main():
     import torch
     pkg = importlib.import_module("hdkx-aicompiler_amd")
     r18 = importlib.import_module("hdkx-aicompiler_amd.resnet18")
+    hostapi = importlib.import_module("hdkx-aicompiler_amd.hostapi")
     synth = pkg.synth
     if not torch.cuda.is_available():
         print("bench.py: no GPU visible", file=sys.stderr)
@@ -71,13 +72,15 @@ def main():
     consts = [dev(c) for c in consts_h]
     x = dev(x_h)
     out = torch.empty((batch, 1000), device="cuda")
-    plan, info = r18.build_plan(batch, 224)
+    # The ResNet-18 Relay graph, compiled by the C++ host layer's Compiler::Compile for the "hip" target.
+    module = hostapi.CompiledResNet18(batch, 224, "hip", sync_after_run=False)
+    info = {"launches": module.launches(), "workspace_bytes": module.workspace_bytes()}
     tensors = [x] + consts + [out]
-    packed = plan.packed(tensors)
+    packed = module.packed(tensors)
     stream = torch.cuda.current_stream().cuda_stream
 
     def step():
-        plan.run_packed(packed, stream)
+        module.run_packed(packed, stream)
 
     for _ in range(args.warmup):
         step()
@@ -112,6 +115,7 @@ def main():
         "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "f32", "data": "synthetic",
         "config": {"workload": "ResNet-18 fp32 inference, batch %d, input [%d,3,224,224], BN folded, seeded Kaiming weights "
                                "(BASELINE configs[3])" % (batch, batch),
+                   "compiled_by": "C++ host layer, Compiler::Compile(Relay graph, target hip)",
                    "launches_per_step": len(info["launches"]), "workspace_bytes": info["workspace_bytes"]},
         "end_to_end_tflops": round(flop_step / (ms_per_step * 1e-3) / 1e12, 3),
         "end_to_end_frac_of_fp32_mfma_peak": round(flop_step / (ms_per_step * 1e-3) / 1e12 / PEAK_FP32_MFMA_TFLOPS, 4),
@@ -124,7 +128,7 @@ def main():
     if not args.no_layers:
         result["conv_layers"] = bench_conv_layers(torch, pkg, synth, dev, batch)
         result["ops"] = bench_ops(torch, pkg, synth, dev)
-        result["resnet18_bs1_img_per_s"] = bench_batch1(torch, pkg, r18, synth, dev)
+        result["resnet18_bs1_img_per_s"] = bench_batch1(torch, pkg, hostapi, synth, dev)
 
     if not args.no_cpu:
         result["cpu_baseline"] = cpu_baseline(np, synth)
@@ -194,15 +198,15 @@ def _bw_row(name, nbytes, ms):
     return {"op": name, "ms": round(ms, 4), "gbs": round(gbs, 1), "frac_hbm_peak": round(gbs / PEAK_HBM_GBS, 4)}
 
 
-def bench_batch1(torch, pkg, r18, synth, dev):
+def bench_batch1(torch, pkg, hostapi, synth, dev):
     consts = [dev(c) for c in synth.resnet18_consts(3)]
     x = dev(synth.resnet18_input(3, 1))
     out = torch.empty((1, 1000), device="cuda")
-    plan, _ = r18.build_plan(1, 224)
-    packed = plan.packed([x] + consts + [out])
+    module = hostapi.CompiledResNet18(1, 224, "hip", sync_after_run=False)
+    packed = module.packed([x] + consts + [out])
     stream = torch.cuda.current_stream().cuda_stream
-    ms = _event_time_ms(torch, lambda: plan.run_packed(packed, stream), 50, 10)
-    plan.close()
+    ms = _event_time_ms(torch, lambda: module.run_packed(packed, stream), 50, 10)
+    module.close()
     return {"value": round(1e3 / ms, 1), "ms_per_image": round(ms, 4)}
 
 

@@ -1,0 +1,65 @@
+// capi.cc -- a small C face of the host layer so that non-C++ callers (the benchmark, tests) can compile
+// a graph for a target and run it with device pointers.  Errors are returned as codes; the message is
+// kept per thread.
+#include <cstring>
+
+#include "kxc/compiler.h"
+#include "kxc/models.h"
+
+namespace {
+thread_local std::string g_error;
+struct ModuleHandle {
+    kxc::api::CompiledModule module;
+    std::string symbols;     // newline-separated kernel symbols
+    std::string plan_json;
+};
+}  // namespace
+
+extern "C" {
+
+const char* kxc_host_last_error(void) { return g_error.c_str(); }
+
+// target: "hip" or "cpu".  sync_after_run = 0 leaves synchronisation to the caller (benchmarks).
+int kxc_host_compile_resnet18(const char* target, long long batch, long long hw, int use_handwritten, int fuse,
+                              int sync_after_run, void** out_module) {
+    try {
+        const bool gpu = std::strcmp(target, "cpu") != 0;
+        auto config = kxc::api::CompileConfig::AOT(kxc::BuildTarget(gpu ? kxc::kGPU : kxc::kCPU));
+        config->hip_use_handwritten = use_handwritten != 0;
+        config->hip_fuse = fuse != 0;
+        config->sync_after_run = sync_after_run != 0;
+        auto* h = new ModuleHandle();
+        h->module = kxc::api::Compiler::Compile(kxc::models::BuildResNet18(batch, hw), config);
+        for (const auto& e : h->module.GetKernelExecs()) h->symbols += e.op_name + " " + e.kernel_symbol + "\n";
+        h->plan_json = h->module.ExecutionPlanJSON();
+        *out_module = h;
+        return 0;
+    } catch (const std::exception& e) {
+        g_error = e.what();
+        return 1;
+    }
+}
+
+int kxc_host_module_run(void* module, void** packed_args, int num_args) {
+    try {
+        static_cast<ModuleHandle*>(module)->module.Run(std::vector<void*>(packed_args, packed_args + num_args));
+        return 0;
+    } catch (const std::exception& e) {
+        g_error = e.what();
+        return 1;
+    }
+}
+
+int kxc_host_module_is_ready(void* module) { return static_cast<ModuleHandle*>(module)->module.IsReady() ? 1 : 0; }
+const char* kxc_host_module_status(void* module) {
+    g_error = static_cast<ModuleHandle*>(module)->module.GetStatus();
+    return g_error.c_str();
+}
+const char* kxc_host_module_symbols(void* module) { return static_cast<ModuleHandle*>(module)->symbols.c_str(); }
+const char* kxc_host_module_plan_json(void* module) { return static_cast<ModuleHandle*>(module)->plan_json.c_str(); }
+long long kxc_host_module_workspace_bytes(void* module) {
+    return static_cast<long long>(static_cast<ModuleHandle*>(module)->module.workspace_bytes());
+}
+void kxc_host_module_free(void* module) { delete static_cast<ModuleHandle*>(module); }
+
+}  // extern "C"

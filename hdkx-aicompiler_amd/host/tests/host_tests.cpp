@@ -17,6 +17,7 @@
 #include <iostream>
 
 #include "kxc/compiler.h"
+#include "kxc/models.h"
 #include "kxc/topi.h"
 
 namespace {
@@ -320,44 +321,6 @@ int RunDeviceInfo() {
 }
 
 // ------------------------------------------------------------------ ResNet-18 (test/resnet18_ir_dump.cpp:191-452)
-struct ResNet {
-    std::vector<kxc::runtime::NDArray> consts;     // creation order = depth-first argument order
-    kxc::Expr Conv(kxc::Expr x, int64_t c, int64_t o, int k, int s, int p) {
-        kxc::runtime::NDArray w({o, c, k, k}, "float32"), b({o}, "float32");
-        consts.push_back(w);
-        consts.push_back(b);
-        auto attrs = kxc::relay::Conv2DAttrs::Create({s, s}, {p, p, p, p}, {1, 1}, 1, static_cast<int>(o), {k, k}, "NCHW", "OIHW", "", "");
-        return kxc::Call(Op::Get("nn_conv2d"), {x, kxc::Constant(w), kxc::Constant(b)}, attrs);
-    }
-    static kxc::Expr Relu(kxc::Expr x) { return kxc::Call(Op::Get("nn_relu"), {x}, kxc::relay::ReluAttrs::Create()); }
-    kxc::Expr Block(kxc::Expr x, int64_t c, int64_t o, int stride, bool down) {
-        kxc::Expr a = Relu(Conv(x, c, o, 3, stride, 1));
-        kxc::Expr b = Conv(a, o, o, 3, 1, 1);
-        kxc::Expr id = down ? Conv(x, c, o, 1, stride, 0) : x;
-        return Relu(kxc::Call(Op::Get("add"), {b, id}, kxc::relay::AddAttrs::Create()));
-    }
-    kxc::Function Build(int64_t batch, int64_t hw) {
-        kxc::Var input("input", kxc::TensorType({batch, 3, hw, hw}, "float32"));
-        kxc::Expr x = Relu(Conv(input, 3, 64, 7, 2, 3));
-        x = kxc::Call(Op::Get("nn_max_pool2d"), {x},
-                      kxc::relay::MaxPool2DAttrs::Create({2, 2}, {1, 1, 1, 1}, {1, 1}, {3, 3}, "NCHW", false));
-        const int64_t ch[4] = {64, 128, 256, 512};
-        int64_t cin = 64;
-        for (int st = 0; st < 4; ++st) {
-            x = Block(x, cin, ch[st], st == 0 ? 1 : 2, st != 0);
-            x = Block(x, ch[st], ch[st], 1, false);
-            cin = ch[st];
-        }
-        x = kxc::Call(Op::Get("nn_global_avg_pool2d"), {x}, kxc::relay::GlobalAvgPool2DAttrs::Create());
-        x = kxc::Call(Op::Get("nn_flatten"), {x}, kxc::relay::FlattenAttrs::Create(1));
-        kxc::runtime::NDArray fw({1000, 512}, "float32"), fb({1000}, "float32");
-        consts.push_back(fw);
-        consts.push_back(fb);
-        x = kxc::Call(Op::Get("nn_gemm"), {x, kxc::Constant(fw), kxc::Constant(fb)}, kxc::relay::GemmAttrs::Create(1.0f, 1.0f, 0, 1));
-        return kxc::Function({input}, x);
-    }
-};
-
 std::vector<char> ReadFile(const std::string& path, size_t expect) {
     std::ifstream in(path, std::ios::binary);
     if (!in) throw std::runtime_error("cannot open " + path);
@@ -367,8 +330,8 @@ std::vector<char> ReadFile(const std::string& path, size_t expect) {
 }
 
 int RunResNet18(const std::string& dir, int64_t batch, int64_t hw) {
-    ResNet net;
-    kxc::Function func = net.Build(batch, hw);
+    std::vector<kxc::runtime::NDArray> net_consts;
+    kxc::Function func = kxc::models::BuildResNet18(batch, hw, &net_consts);
     auto config = MakeConfig();
     auto module = kxc::api::Compiler::Compile(func, config);
     std::cout << "status: " << module.GetStatus() << "\n";
@@ -377,7 +340,7 @@ int RunResNet18(const std::string& dir, int64_t batch, int64_t hw) {
     // the constants come back in parameter order, which is the graph's depth-first argument order
     const auto& consts = module.GetConstants();
     for (size_t k = 0; k < consts.size(); ++k)
-        Check(consts[k].get() == net.consts[k].get(), "constant " + std::to_string(k) + " is out of lowering order");
+        Check(consts[k].get() == net_consts[k].get(), "constant " + std::to_string(k) + " is out of lowering order");
     {
         std::ofstream plan(dir + "/plan.json");
         plan << module.ExecutionPlanJSON();
@@ -454,8 +417,7 @@ int RunCodegen() {
     Check(gap_hip.source.find("/ ((long long)49LL)") != std::string::npos || gap_hip.source.find("49") != std::string::npos, "division by H*W");
     // a ResNet-18 compile for the hip target without a GPU: plan and fusion are built, nothing is loaded
     g_mode = "hip";
-    ResNet net;
-    auto module = kxc::api::Compiler::Compile(net.Build(1, 224), MakeConfig());
+    auto module = kxc::api::Compiler::Compile(kxc::models::BuildResNet18(1, 224), MakeConfig());
     Check(module.GetKernelExecs().size() == 23, "49 Relay calls become 23 launches, got " + std::to_string(module.GetKernelExecs().size()));
     int fused_add = 0, fused_relu = 0;
     for (const auto& e : module.GetKernelExecs()) {

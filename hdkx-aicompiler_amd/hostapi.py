@@ -1,0 +1,70 @@
+"""ctypes binding of the C++ host layer's C face (host/src/capi.cc): compile a Relay graph for a target
+and run it with device pointers."""
+import ctypes as C
+import os
+
+from . import hipabi
+
+PKG = os.path.dirname(os.path.abspath(__file__))
+_HOST_LIB = os.path.join(PKG, "lib", "libkxc_host.so")
+_lib = None
+
+
+def lib():
+    global _lib
+    if _lib is None:
+        hipabi.lib()     # the C-ABI library must be loaded first (the host library links against it)
+        if not os.path.exists(_HOST_LIB):
+            import subprocess
+            subprocess.check_call(["make", "-C", os.path.join(PKG, "host"), "-j8"])
+        _lib = C.CDLL(_HOST_LIB, mode=C.RTLD_GLOBAL)
+        _lib.kxc_host_last_error.restype = C.c_char_p
+        _lib.kxc_host_module_status.restype = C.c_char_p
+        _lib.kxc_host_module_symbols.restype = C.c_char_p
+        _lib.kxc_host_module_plan_json.restype = C.c_char_p
+        _lib.kxc_host_module_workspace_bytes.restype = C.c_longlong
+    return _lib
+
+
+class CompiledResNet18:
+    """ResNet-18 Relay graph compiled by Compiler::Compile for "hip" (or "cpu")."""
+
+    def __init__(self, batch, hw=224, target="hip", use_handwritten=True, fuse=True, sync_after_run=False):
+        self._h = C.c_void_p()
+        rc = lib().kxc_host_compile_resnet18(target.encode(), C.c_longlong(batch), C.c_longlong(hw),
+                                             int(use_handwritten), int(fuse), int(sync_after_run), C.byref(self._h))
+        if rc != 0:
+            raise hipabi.KxcHipError(lib().kxc_host_last_error().decode())
+        self.num_args = 44
+
+    @property
+    def ready(self):
+        return bool(lib().kxc_host_module_is_ready(self._h))
+
+    @property
+    def status(self):
+        return lib().kxc_host_module_status(self._h).decode()
+
+    def launches(self):
+        return [l for l in lib().kxc_host_module_symbols(self._h).decode().split("\n") if l]
+
+    def plan_json(self):
+        return lib().kxc_host_module_plan_json(self._h).decode()
+
+    def workspace_bytes(self):
+        return int(lib().kxc_host_module_workspace_bytes(self._h))
+
+    def packed(self, tensors):
+        return (C.c_void_p * len(tensors))(*[t.data_ptr() for t in tensors])
+
+    def run_packed(self, args, stream=None):
+        """Enqueue on `stream` (a hipStream_t as int): it becomes the calling thread's current stream."""
+        if stream is not None:
+            hipabi.lib().kxc_hip_set_stream(0, C.c_void_p(stream))
+        if lib().kxc_host_module_run(self._h, args, len(args)) != 0:
+            raise hipabi.KxcHipError(lib().kxc_host_last_error().decode())
+
+    def close(self):
+        if self._h:
+            lib().kxc_host_module_free(self._h)
+            self._h = C.c_void_p()

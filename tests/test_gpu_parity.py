@@ -169,7 +169,7 @@ def test_conv_full_batch_properties(pkg, synth):
     y1 = pkg.conv2d(x, w1, None, None, 1, 1); y2 = pkg.conv2d(x, w2, None, None, 1, 1)
     assert_close(host(y12), host(y1 + y2), what="linearity")
     one = pkg.conv2d(x[17:18].contiguous(), w1, b, None, 1, 1, 1, True)
-    assert_close(host(one), host(fast[17:18]), tol=1e-5, what="batch independence")
+    assert_close(host(one), host(fast[17:18]), tol=1e-4, what="batch independence")
 
 
 # ------------------------------------------------------------------ pooling / elementwise at BASELINE sizes
