@@ -39,6 +39,19 @@ def _event_time_ms(torch, fn, iters, warmup):
     return start.elapsed_time(stop) / iters
 
 
+def _profiled_traffic_bytes():
+    """HBM bytes per launch of the dominant kernel, as measured with the rocprofv3 FETCH_SIZE and
+    WRITE_SIZE passes whose summary is kept beside this file (counters cannot be read from inside a run)."""
+    path = os.path.join(os.path.dirname(os.path.abspath(__file__)), "profiles", "conv3x3_layer1_bs64_counters.md")
+    try:
+        for line in open(path):
+            if line.startswith("TRAFFIC_BYTES_PER_LAUNCH="):
+                return int(line.split("=", 1)[1])
+    except OSError:
+        pass
+    return None
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -107,7 +120,9 @@ def main():
                 "variant": pkg.conv2d_variant((batch, 64, 56, 56), (64, 64, 3, 3), 1, 1),
                 "achieved": round(conv_tflops, 3), "peak": PEAK_FP32_MFMA_TFLOPS, "unit": "TFLOP/s",
                 "frac": round(conv_tflops / PEAK_FP32_MFMA_TFLOPS, 4), "avg_launch_ms": round(conv_ms, 4),
-                "flop_per_launch": conv_flop, "traffic": None}
+                "flop_per_launch": conv_flop, "traffic": _profiled_traffic_bytes() if batch == 64 else None,
+                "traffic_unit": "bytes per launch (FETCH_SIZE + WRITE_SIZE, calibrated on a copy; from profiles/)",
+                "algorithmic_bytes_per_launch": 4 * (2 * batch * 64 * 56 * 56 + 64 * 64 * 9 + 64)}
 
     result = {
         "metric": "resnet18_fp32_bs64_img_per_s", "value": round(img_s, 2), "unit": "img/s",
