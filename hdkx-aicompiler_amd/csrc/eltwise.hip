@@ -120,6 +120,23 @@ __global__ void __launch_bounds__(kBlock) quantize_kernel(const float* __restric
     }
 }
 
+// max |x| over a tensor (NaN ignored): per-wave reduction, then one atomic per wave on the bit pattern
+// (non-negative floats order like unsigned integers).  *out must be 0 on entry.
+__global__ void __launch_bounds__(kBlock) absmax_kernel(const float* __restrict__ x, int64_t n, unsigned int* out) {
+    const int64_t stride = static_cast<int64_t>(gridDim.x) * kBlock;
+    float m = 0.0f;
+    for (int64_t i = static_cast<int64_t>(blockIdx.x) * kBlock + threadIdx.x; i < n; i += stride) {
+        const float v = fabsf(x[i]);
+        m = (v > m) ? v : m;
+    }
+#pragma unroll
+    for (int off = 32; off > 0; off >>= 1) {
+        const float o = __shfl_down(m, off, 64);
+        m = (o > m) ? o : m;
+    }
+    if ((threadIdx.x & 63) == 0) atomicMax(out, __float_as_uint(m));
+}
+
 inline int GridFor(int64_t work_items) {
     // Enough workgroups for ~8 per CU at 256 CUs; grid-stride loops take the rest.
     int64_t g = CeilDiv(work_items, kBlock);
@@ -257,6 +274,17 @@ int32_t kxc_hip_quantize_f32_i8(const float* x, int8_t* q, int64_t n, float scal
     KXC_HIP_REQUIRE(scale > 0.0f, "kxc_hip_quantize_f32_i8: scale must be positive");
     quantize_kernel<<<GridFor(n), kBlock, 0, ResolveStream(stream)>>>(x, q, n, scale);
     return CheckLaunch("quantize");
+}
+
+int32_t kxc_hip_absmax_f32(const float* x, int64_t n, float* out, void* stream) {
+    KXC_HIP_REQUIRE(n >= 0, "kxc_hip_absmax_f32: negative size");
+    KXC_HIP_REQUIRE(out != nullptr, "kxc_hip_absmax_f32: NULL output");
+    hipStream_t s = ResolveStream(stream);
+    KXC_HIP_CALL(hipMemsetAsync(out, 0, sizeof(float), s), "hipMemsetAsync");
+    if (n == 0) return KXC_HIP_OK;
+    KXC_HIP_REQUIRE(x != nullptr, "kxc_hip_absmax_f32: NULL pointer");
+    absmax_kernel<<<GridFor(n), kBlock, 0, s>>>(x, n, reinterpret_cast<unsigned int*>(out));
+    return CheckLaunch("absmax");
 }
 
 }  // extern "C"

@@ -288,6 +288,52 @@ int32_t kxc_hip_plan_add_qdense(kxc_hip_plan* plan, int64_t m, int64_t nn, int64
     return KXC_HIP_OK;
 }
 
+// ---- the same int8 operators on the channel-blocked "c16" layout (qconv_c16_i8.hip); i32[0] = 1 marks them
+int32_t kxc_hip_plan_add_qconv2d_c16(kxc_hip_plan* plan, const kxc_hip_qconv2d_desc* desc, kxc_hip_buf x,
+                                     kxc_hip_buf w_packed, kxc_hip_buf bias, kxc_hip_buf mult, kxc_hip_buf residual,
+                                     kxc_hip_buf y) {
+    const char* who = "kxc_hip_plan_add_qconv2d_c16";
+    if (int32_t rc = kxc_hip_plan_add_qconv2d(plan, desc, x, w_packed, bias, mult, residual, y)) return rc;
+    Node& n = plan->nodes.back();
+    const char* variant = kxc_hip_qconv2d_c16_variant(desc);
+    if (std::strcmp(variant, "none") == 0) {
+        const std::string inner = LastError();
+        plan->nodes.pop_back();
+        return Fail(KXC_HIP_ERR_INVALID, "%s: %s", who, inner.c_str());
+    }
+    n.i32[0] = 1;
+    n.symbol = std::string("kxc_qconv2d_c16_i8:") + variant;
+    return KXC_HIP_OK;
+}
+
+int32_t kxc_hip_plan_add_quantize_c16(kxc_hip_plan* plan, int64_t nn, int64_t c, int64_t hw, float scale, kxc_hip_buf x,
+                                      kxc_hip_buf q) {
+    if (int32_t rc = kxc_hip_plan_add_quantize(plan, nn, scale, x, q)) return rc;
+    Node& n = plan->nodes.back();
+    n.dims[0] = nn; n.dims[1] = c; n.dims[2] = hw;
+    n.i32[0] = 1;
+    n.symbol = "kxc_quantize_f32_nchw_to_c16_i8";
+    return KXC_HIP_OK;
+}
+
+int32_t kxc_hip_plan_add_maxpool2d_c16_i8(kxc_hip_plan* plan, const kxc_hip_pool2d_desc* desc, kxc_hip_buf x,
+                                          kxc_hip_buf y) {
+    if (int32_t rc = kxc_hip_plan_add_maxpool2d_i8(plan, desc, x, y)) return rc;
+    Node& n = plan->nodes.back();
+    n.i32[0] = 1;
+    n.symbol = "kxc_max_pool2d_c16_i8";
+    return KXC_HIP_OK;
+}
+
+int32_t kxc_hip_plan_add_global_avg_pool2d_c16_i8(kxc_hip_plan* plan, int64_t nn, int64_t c, int64_t h, int64_t w,
+                                                  float mult, kxc_hip_buf x, kxc_hip_buf y) {
+    if (int32_t rc = kxc_hip_plan_add_global_avg_pool2d_i8(plan, nn, c, h, w, mult, x, y)) return rc;
+    Node& n = plan->nodes.back();
+    n.i32[0] = 1;
+    n.symbol = "kxc_global_avg_pool2d_c16_i8";
+    return KXC_HIP_OK;
+}
+
 int32_t kxc_hip_plan_add_module_kernel(kxc_hip_plan* plan, void* function, const char* symbol, const uint32_t grid[3],
                                        const uint32_t block[3], uint32_t shared_bytes, const kxc_hip_buf* params,
                                        int32_t num_params) {
@@ -381,17 +427,37 @@ int32_t kxc_hip_plan_run(kxc_hip_plan* plan, void** args, void* stream) {
                 break;
             }
             case NodeKind::kQConv2D:
+                if (n.i32[0] == 1) {
+                    rc = kxc_hip_qconv2d_c16_i8(&n.qconv, static_cast<const int8_t*>(B(0)), static_cast<const int8_t*>(B(1)),
+                                                static_cast<const int32_t*>(B(2)), static_cast<const float*>(B(3)),
+                                                static_cast<const int8_t*>(B(4)), static_cast<int8_t*>(B(5)), s);
+                    break;
+                }
                 rc = kxc_hip_qconv2d_nchw_i8(&n.qconv, static_cast<const int8_t*>(B(0)), static_cast<const int8_t*>(B(1)),
                                              static_cast<const int32_t*>(B(2)), static_cast<const float*>(B(3)),
                                              static_cast<const int8_t*>(B(4)), static_cast<int8_t*>(B(5)), s);
                 break;
             case NodeKind::kQuantize:
+                if (n.i32[0] == 1) {
+                    rc = kxc_hip_quantize_f32_nchw_to_c16_i8(static_cast<const float*>(B(0)), static_cast<int8_t*>(B(1)),
+                                                             n.dims[0], n.dims[1], n.dims[2], n.f[0], s);
+                    break;
+                }
                 rc = kxc_hip_quantize_f32_i8(static_cast<const float*>(B(0)), static_cast<int8_t*>(B(1)), n.dims[0], n.f[0], s);
                 break;
             case NodeKind::kMaxPoolI8:
+                if (n.i32[0] == 1) {
+                    rc = kxc_hip_maxpool2d_c16_i8(&n.pool, static_cast<const int8_t*>(B(0)), static_cast<int8_t*>(B(1)), s);
+                    break;
+                }
                 rc = kxc_hip_maxpool2d_i8(&n.pool, static_cast<const int8_t*>(B(0)), static_cast<int8_t*>(B(1)), s);
                 break;
             case NodeKind::kGlobalAvgPoolI8:
+                if (n.i32[0] == 1) {
+                    rc = kxc_hip_global_avg_pool2d_c16_i8(static_cast<const int8_t*>(B(0)), static_cast<int8_t*>(B(1)),
+                                                          n.dims[0], n.dims[1], n.dims[2], n.dims[3], n.f[0], s);
+                    break;
+                }
                 rc = kxc_hip_global_avg_pool2d_i8(static_cast<const int8_t*>(B(0)), static_cast<int8_t*>(B(1)), n.dims[0],
                                                   n.dims[1], n.dims[2], n.dims[3], n.f[0], s);
                 break;

@@ -1,0 +1,682 @@
+// qconv_c16_i8.hip -- int8 convolution on the gfx950 int8 matrix cores (v_mfma_i32_32x32x32_i8), with the
+// operators around it, on a channel-blocked activation layout.
+//
+// Layout "c16": an int8 activation of logical shape [N, C, H, W] is stored as [N][CB][H][W][16] with
+// CB = ceil(C/16); element (n, c, h, w) lives at (((n*CB + c/16)*H + h)*W + w)*16 + c%16 and the bytes
+// of channels >= C are zero.  One pixel's 16 channels are one 16-byte word: exactly the k-slice one lane
+// feeds to the 32x32x32 matrix instruction, so a filter tap is ONE aligned ds_read_b128 per lane and no
+// byte gather or transpose exists anywhere.  The reference compiler has no int8 operator, so there is no
+// external layout to match; the NCHW entry points remain for interchange, with converters below.
+//
+// Arithmetic (identical to the NCHW kernel and the CPU definition):
+//   acc = sum x*w in int32 (exact, order free) [+ bias[o]];  v = (float)acc * mult[o];
+//   [v = v + (float)res * res_mult];  y = clamp(rint_half_even(v), relu ? 0 : -128, 127).
+//
+// Kernel structure: D[o][pixel] += W[o][k] * X[k][pixel]; pixels are flattened over (n, oh, ow).  A
+// workgroup of WP waves owns 32*RO output channels by 32*WP consecutive pixels; every wave computes RO
+// 32x32 blocks that share one pixel operand.  Per chunk of CBC channel blocks the workgroup stages in LDS
+//   * the input rows its pixels touch, in "padded row space" Q = n*(H+2*pad) + ih + pad, as 16-byte
+//     positions patch[cb][Q - Qmin][col + pad]  (zero padding comes from the buffer descriptor's
+//     out-of-range rule, so it costs nothing), and
+//   * the weights, which the host has pre-packed in exactly the order the lanes read them
+//     ([o block][chunk][k-step][lane][16 bytes]), so the copy is linear.
+// Both are written by LDS-direct buffer loads of 16 bytes per lane and double buffered.
+// A k-step is 32 reduction values: lane half h takes linear index q = 2*step + h of the chunk's
+// (tap, channel block) pairs, q = tap*CBC + cb_local; indices past the end carry zero weights.
+#include <cstring>
+#include <vector>
+
+#include "common.h"
+
+using namespace kxc_hip;
+
+namespace {
+
+typedef int intx4 __attribute__((ext_vector_type(4)));
+typedef int intx16 __attribute__((ext_vector_type(16)));
+typedef __attribute__((address_space(3))) void* lds_ptr_t;
+
+constexpr uint32_t kOob = 0x80000000u;
+constexpr int kBlock = 256;
+
+__device__ __forceinline__ __amdgpu_buffer_rsrc_t make_rsrc(const void* p, uint32_t bytes) {
+    return __builtin_amdgcn_make_buffer_rsrc(const_cast<void*>(p), 0, static_cast<int>(bytes), 0x00020000);
+}
+
+// 16 bytes per lane from a buffer straight into LDS (lane l writes lds + 16*l).  The 16-byte form exists on
+// gfx950 only; the host pass of the compiler does not know the target and rejects the size, so it sees an
+// empty body.
+__device__ __forceinline__ void load16_to_lds(__amdgpu_buffer_rsrc_t rsrc, lds_ptr_t lds, uint32_t voffset,
+                                              uint32_t soffset) {
+#if defined(__HIP_DEVICE_COMPILE__)
+    __builtin_amdgcn_raw_ptr_buffer_load_lds(rsrc, lds, 16, voffset, soffset, 0, 0);
+#endif
+}
+
+__device__ __forceinline__ int32_t requant_i32(int32_t acc, float mult, bool has_res, int32_t res, float res_mult,
+                                               bool relu) {
+    float v = __fmul_rn(static_cast<float>(acc), mult);
+    if (has_res) v = __fadd_rn(v, __fmul_rn(static_cast<float>(res), res_mult));
+    float r = rintf(v);
+    r = (v == v) ? r : 0.0f;
+    r = fminf(fmaxf(r, relu ? 0.0f : -128.0f), 127.0f);
+    return static_cast<int32_t>(r);
+}
+
+struct QArgs {
+    const int8_t* x;
+    const int8_t* wp;
+    const int32_t* bias;
+    const float* mult;
+    const int8_t* res;
+    int8_t* y;
+    int32_t N, CB, H, W, O, OH, OW;
+    int32_t sh, sw, ph, pw;
+    int32_t Hp, Wp, M, OHW;
+    int32_t chs;          // 16-byte positions per channel block plane in LDS (multiple of 64)
+    int32_t nchunks;
+    uint32_t x_bytes, w_bytes;
+    int32_t p_tiles, o_tiles, num_tiles, tiles_per_xcd;
+    float res_mult;
+    uint32_t flags;
+};
+
+template <int KH, int KW, int CBC, int WP, int RO, int PPT>
+__global__ void __launch_bounds__(64 * WP) qconv_mfma_kernel(const QArgs a) {
+    constexpr int KHW = KH * KW;
+    constexpr int NS = (KHW * CBC + 1) / 2;          // matrix k-steps per chunk
+    constexpr int TP = 32 * WP;
+    constexpr int WSEG = RO * NS;                    // 1 KiB weight segments per chunk
+    constexpr int WPT = (WSEG + WP - 1) / WP;
+
+    extern __shared__ __attribute__((aligned(16))) char lds[];
+    const int tid = threadIdx.x;
+    const int lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int half = lane >> 5;
+    const int r = lane & 31;
+
+    const int xs_bytes = CBC * a.chs * 16;
+    const int buf_bytes = xs_bytes + WSEG * 1024;
+    char* const buf0 = lds;
+    char* const buf1 = lds + buf_bytes;              // present only when nchunks > 1
+
+    // consecutive workgroups go to the 8 XCDs round-robin; give every XCD (own L2) a contiguous run of tiles
+    const int tile = (blockIdx.x & 7) * a.tiles_per_xcd + (blockIdx.x >> 3);
+    if (tile >= a.num_tiles || static_cast<int>(blockIdx.x >> 3) >= a.tiles_per_xcd) return;
+    const int p_tile = tile / a.o_tiles, o_tile = tile - p_tile * a.o_tiles;
+    const int m0 = p_tile * TP;
+    const int ob0 = o_tile * RO;                     // first 32-channel output block
+
+    const int m_last = min(m0 + TP, a.M) - 1;
+    int qmin, qlast;
+    {
+        const int n = m0 / a.OHW, rem = m0 - n * a.OHW;
+        qmin = n * a.Hp + (rem / a.OW) * a.sh;
+        const int n2 = m_last / a.OHW, rem2 = m_last - n2 * a.OHW;
+        qlast = n2 * a.Hp + (rem2 / a.OW) * a.sh + (KH - 1);
+    }
+    const int P = (qlast - qmin + 1) * a.Wp;         // positions per plane (<= chs)
+    const int xsegs = (P + 63) >> 6;
+    const uint32_t plane_bytes = static_cast<uint32_t>(a.H) * a.W * 16u;
+
+    const __amdgpu_buffer_rsrc_t xr = make_rsrc(a.x, a.x_bytes);
+    const __amdgpu_buffer_rsrc_t wr = make_rsrc(a.wp, a.w_bytes);
+
+    uint32_t goff[PPT];
+#pragma unroll
+    for (int i = 0; i < PPT; ++i) {
+        const int pos = (wave + i * WP) * 64 + lane;
+        const int q = pos / a.Wp, col = pos - q * a.Wp;
+        const int Q = qmin + q;
+        const int n = Q / a.Hp, ih = Q - n * a.Hp - a.ph, iw = col - a.pw;
+        const bool ok = pos < P && n < a.N && ih >= 0 && ih < a.H && iw >= 0 && iw < a.W;
+        goff[i] = ok ? (static_cast<uint32_t>(n) * a.CB * a.H * a.W + static_cast<uint32_t>(ih * a.W + iw)) * 16u : kOob;
+    }
+
+    // per-lane operand base: byte address of the pixel's (tap 0, channel block 0) position
+    const int m = m0 + wave * 32 + r;
+    int xbase;
+    int ypix;            // position index (n*OB16*OHW + pixel) of this lane's output pixel for block 0, or -1
+    int ostride;         // positions between consecutive 16-channel output blocks
+    {
+        const int mc = min(m, a.M - 1);
+        const int n = mc / a.OHW, rem = mc - n * a.OHW;
+        const int oh = rem / a.OW, ow = rem - oh * a.OW;
+        xbase = ((n * a.Hp + oh * a.sh - qmin) * a.Wp + ow * a.sw) * 16;
+        if (CBC > 1) xbase += half * a.chs * 16;
+        ostride = a.OHW;
+        ypix = (m < a.M) ? n * (a.O >> 4) * a.OHW + rem : -1;
+    }
+
+    intx16 acc[RO];
+#pragma unroll
+    for (int i = 0; i < RO; ++i)
+#pragma unroll
+        for (int g = 0; g < 16; ++g) acc[i][g] = 0;
+
+    // packed weights: [(o block)][chunk][NS][64][16]
+    const uint32_t w_chunk_bytes = NS * 1024u;
+    auto issue_loads = [&](int chunk, char* buf) {
+#pragma unroll
+        for (int cl = 0; cl < CBC; ++cl) {
+            const int cb = chunk * CBC + cl;
+            if (cb < a.CB) {
+                const uint32_t soff = static_cast<uint32_t>(cb) * plane_bytes;
+#pragma unroll
+                for (int i = 0; i < PPT; ++i) {
+                    const int seg = wave + i * WP;
+                    if (seg < xsegs)
+                        load16_to_lds(xr, (lds_ptr_t)(buf + (cl * a.chs + seg * 64) * 16), goff[i], soff);
+                }
+            }   // a missing channel block keeps stale bytes; its packed weights are zero and integers have no NaN
+        }
+#pragma unroll
+        for (int i = 0; i < WPT; ++i) {
+            const int seg = wave + i * WP;
+            if (seg < WSEG) {
+                const int ro = seg / NS, st = seg - ro * NS;
+                const uint32_t soff = (static_cast<uint32_t>(ob0 + ro) * a.nchunks + chunk) * w_chunk_bytes + st * 1024u;
+                load16_to_lds(wr, (lds_ptr_t)(buf + xs_bytes + seg * 1024), static_cast<uint32_t>(lane) * 16u, soff);
+            }
+        }
+    };
+
+    issue_loads(0, buf0);
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+    __syncthreads();
+
+    for (int chunk = 0; chunk < a.nchunks; ++chunk) {
+        const char* buf = (chunk & 1) ? buf1 : buf0;
+        if (chunk + 1 < a.nchunks) issue_loads(chunk + 1, (chunk & 1) ? buf0 : buf1);
+        const char* ws = buf + xs_bytes + lane * 16;
+        auto tap_off = [&](int tap) {
+            const int t = tap < KHW ? tap : KHW - 1;
+            const int rh = t / KW, rw = t - rh * KW;
+            return (rh * a.Wp + rw) * 16;
+        };
+        auto fetch_b = [&](int step) -> intx4 {
+            int off;
+            if constexpr (CBC == 1) {
+                off = half ? tap_off(2 * step + 1) : tap_off(2 * step);
+            } else {
+                constexpr int H2 = CBC / 2;
+                off = tap_off(step / H2) + 2 * (step % H2) * a.chs * 16;
+            }
+            return *reinterpret_cast<const intx4*>(buf + xbase + off);
+        };
+        intx4 bcur = fetch_b(0);
+        intx4 acur[RO];
+#pragma unroll
+        for (int i = 0; i < RO; ++i) acur[i] = *reinterpret_cast<const intx4*>(ws + (i * NS) * 1024);
+#pragma unroll
+        for (int step = 0; step < NS; ++step) {
+            intx4 bnext = bcur;
+            intx4 anext[RO];
+#pragma unroll
+            for (int i = 0; i < RO; ++i) anext[i] = acur[i];
+            if (step + 1 < NS) {
+                bnext = fetch_b(step + 1);
+#pragma unroll
+                for (int i = 0; i < RO; ++i)
+                    anext[i] = *reinterpret_cast<const intx4*>(ws + (i * NS + step + 1) * 1024);
+            }
+#pragma unroll
+            for (int i = 0; i < RO; ++i) acc[i] = __builtin_amdgcn_mfma_i32_32x32x32_i8(acur[i], bcur, acc[i], 0, 0, 0);
+            bcur = bnext;
+#pragma unroll
+            for (int i = 0; i < RO; ++i) acur[i] = anext[i];
+        }
+        asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+        __syncthreads();
+    }
+
+    // ---- epilogue.  Accumulator register g of a block is output channel 8*(g/4) + 4*half + g%4 (within
+    // the block of 32) at pixel r: registers 4j..4j+3 are four consecutive channels = one dword of the c16
+    // word of this pixel.
+    if (ypix < 0) return;
+    const bool has_bias = (a.flags & KXC_HIP_CONV_BIAS) != 0;
+    const bool has_res = (a.flags & KXC_HIP_CONV_RESIDUAL) != 0;
+    const bool do_relu = (a.flags & KXC_HIP_CONV_RELU) != 0;
+#pragma unroll
+    for (int i = 0; i < RO; ++i) {
+        const int obase = (ob0 + i) * 32;
+        if (obase >= a.O) continue;
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+            const int o = obase + 8 * j + 4 * half;                 // first of 4 consecutive channels
+            if (o >= a.O) continue;
+            // byte offset of channels o..o+3 of this pixel
+            const int64_t off = (static_cast<int64_t>(ypix) + static_cast<int64_t>(o >> 4) * ostride) * 16 + (o & 15);
+            uint32_t resw = 0;
+            if (has_res) resw = *reinterpret_cast<const uint32_t*>(a.res + off);
+            const float4 mv = *reinterpret_cast<const float4*>(a.mult + o);
+            int4 bv = make_int4(0, 0, 0, 0);
+            if (has_bias) bv = *reinterpret_cast<const int4*>(a.bias + o);
+            const float ms[4] = {mv.x, mv.y, mv.z, mv.w};
+            const int bs[4] = {bv.x, bv.y, bv.z, bv.w};
+            uint32_t outw = 0;
+#pragma unroll
+            for (int e = 0; e < 4; ++e) {
+                const int32_t rq = static_cast<int32_t>(static_cast<int8_t>((resw >> (8 * e)) & 0xff));
+                const int32_t q = requant_i32(acc[i][4 * j + e] + bs[e], ms[e], has_res, rq, a.res_mult, do_relu);
+                outw |= (static_cast<uint32_t>(q) & 0xffu) << (8 * e);
+            }
+            *reinterpret_cast<uint32_t*>(a.y + off) = outw;
+        }
+    }
+}
+
+// ------------------------------------------------------------------ weight packing
+struct PackArgs {
+    const int8_t* w;      // OIHW
+    int8_t* wp;
+    int32_t O, C, KHW, CBC, NS, nchunks, oblocks;
+};
+
+__global__ void __launch_bounds__(kBlock) pack_weights_kernel(const PackArgs a, int64_t total_slots) {
+    const int64_t s = static_cast<int64_t>(blockIdx.x) * kBlock + threadIdx.x;
+    if (s >= total_slots) return;
+    const int lane = static_cast<int>(s & 63);
+    int64_t t = s >> 6;
+    const int step = static_cast<int>(t % a.NS); t /= a.NS;
+    const int chunk = static_cast<int>(t % a.nchunks);
+    const int ob = static_cast<int>(t / a.nchunks);
+    const int o = ob * 32 + (lane & 31), h = lane >> 5;
+    const int q = 2 * step + h;
+    const int tap = q / a.CBC, cbl = q - tap * a.CBC;
+    const int cb = chunk * a.CBC + cbl;
+    int8_t out[16];
+#pragma unroll
+    for (int j = 0; j < 16; ++j) {
+        const int c = cb * 16 + j;
+        out[j] = (tap < a.KHW && c < a.C && o < a.O) ? a.w[(static_cast<int64_t>(o) * a.C + c) * a.KHW + tap] : 0;
+    }
+    *reinterpret_cast<int4*>(a.wp + s * 16) = *reinterpret_cast<const int4*>(out);
+}
+
+// ------------------------------------------------------------------ layout conversion and quantisation
+// One thread per 16-byte position of the c16 tensor.
+__global__ void __launch_bounds__(kBlock) nchw_to_c16_kernel(const int8_t* __restrict__ x, int8_t* __restrict__ y,
+                                                             int32_t C, int32_t CB, int64_t HW, int64_t total) {
+    const int64_t s = static_cast<int64_t>(blockIdx.x) * kBlock + threadIdx.x;
+    if (s >= total) return;
+    const int64_t p = s % HW;
+    const int64_t t = s / HW;
+    const int cb = static_cast<int>(t % CB);
+    const int64_t n = t / CB;
+    int8_t out[16];
+#pragma unroll
+    for (int j = 0; j < 16; ++j) {
+        const int c = cb * 16 + j;
+        out[j] = c < C ? x[(n * C + c) * HW + p] : 0;
+    }
+    *reinterpret_cast<int4*>(y + s * 16) = *reinterpret_cast<const int4*>(out);
+}
+
+__global__ void __launch_bounds__(kBlock) c16_to_nchw_kernel(const int8_t* __restrict__ x, int8_t* __restrict__ y,
+                                                             int32_t C, int32_t CB, int64_t HW, int64_t total) {
+    const int64_t e = static_cast<int64_t>(blockIdx.x) * kBlock + threadIdx.x;   // NCHW element
+    if (e >= total) return;
+    const int64_t p = e % HW;
+    const int64_t t = e / HW;
+    const int c = static_cast<int>(t % C);
+    const int64_t n = t / C;
+    y[e] = x[((n * CB + (c >> 4)) * HW + p) * 16 + (c & 15)];
+}
+
+__global__ void __launch_bounds__(kBlock) quantize_to_c16_kernel(const float* __restrict__ x, int8_t* __restrict__ y,
+                                                                 int32_t C, int32_t CB, int64_t HW, int64_t total,
+                                                                 float scale) {
+    const int64_t s = static_cast<int64_t>(blockIdx.x) * kBlock + threadIdx.x;
+    if (s >= total) return;
+    const int64_t p = s % HW;
+    const int64_t t = s / HW;
+    const int cb = static_cast<int>(t % CB);
+    const int64_t n = t / CB;
+    int8_t out[16];
+#pragma unroll
+    for (int j = 0; j < 16; ++j) {
+        const int c = cb * 16 + j;
+        int32_t q = 0;
+        if (c < C) {
+            const float v = __fdiv_rn(x[(n * C + c) * HW + p], scale);
+            float rr = rintf(v);
+            rr = (v == v) ? rr : 0.0f;
+            rr = fminf(fmaxf(rr, -127.0f), 127.0f);
+            q = static_cast<int32_t>(rr);
+        }
+        out[j] = static_cast<int8_t>(q);
+    }
+    *reinterpret_cast<int4*>(y + s * 16) = *reinterpret_cast<const int4*>(out);
+}
+
+// ------------------------------------------------------------------ pooling on c16
+struct PoolArgs {
+    int32_t N, CB, H, W, OH, OW, KH, KW, sh, sw, pt, pl;
+};
+
+// One thread per output position (16 channels): byte-wise signed max over the window.
+__global__ void __launch_bounds__(kBlock) maxpool_c16_kernel(const int8_t* __restrict__ x, int8_t* __restrict__ y,
+                                                             const PoolArgs d, int64_t total) {
+    const int64_t s = static_cast<int64_t>(blockIdx.x) * kBlock + threadIdx.x;
+    if (s >= total) return;
+    const int ow = static_cast<int>(s % d.OW);
+    int64_t t = s / d.OW;
+    const int oh = static_cast<int>(t % d.OH);
+    const int64_t plane = t / d.OH;                  // n*CB + cb
+    const int8_t* xp = x + plane * d.H * d.W * 16;
+    int32_t m[16];
+#pragma unroll
+    for (int j = 0; j < 16; ++j) m[j] = -128;
+    for (int rh = 0; rh < d.KH; ++rh) {
+        const int ih = oh * d.sh + rh - d.pt;
+        if (ih < 0 || ih >= d.H) continue;
+        for (int rw = 0; rw < d.KW; ++rw) {
+            const int iw = ow * d.sw + rw - d.pl;
+            if (iw < 0 || iw >= d.W) continue;
+            const int4 v = *reinterpret_cast<const int4*>(xp + (static_cast<int64_t>(ih) * d.W + iw) * 16);
+            const int vw[4] = {v.x, v.y, v.z, v.w};
+#pragma unroll
+            for (int j = 0; j < 16; ++j) {
+                const int32_t b = static_cast<int32_t>(static_cast<int8_t>((vw[j >> 2] >> (8 * (j & 3))) & 0xff));
+                m[j] = b > m[j] ? b : m[j];
+            }
+        }
+    }
+    uint32_t o[4] = {0, 0, 0, 0};
+#pragma unroll
+    for (int j = 0; j < 16; ++j) o[j >> 2] |= (static_cast<uint32_t>(m[j]) & 0xffu) << (8 * (j & 3));
+    *reinterpret_cast<int4*>(y + s * 16) = make_int4(o[0], o[1], o[2], o[3]);
+}
+
+// One thread per (n, channel block): sums the plane, requantises; output [N][CB*16] (= c16 with H = W = 1).
+__global__ void __launch_bounds__(kBlock) gap_c16_kernel(const int8_t* __restrict__ x, int8_t* __restrict__ y,
+                                                         int64_t planes, int32_t hw, float mult) {
+    const int64_t p = static_cast<int64_t>(blockIdx.x) * kBlock + threadIdx.x;
+    if (p >= planes) return;
+    const int8_t* src = x + p * hw * 16;
+    int32_t sum[16];
+#pragma unroll
+    for (int j = 0; j < 16; ++j) sum[j] = 0;
+    for (int i = 0; i < hw; ++i) {
+        const int4 v = *reinterpret_cast<const int4*>(src + static_cast<int64_t>(i) * 16);
+        const int vw[4] = {v.x, v.y, v.z, v.w};
+#pragma unroll
+        for (int j = 0; j < 16; ++j)
+            sum[j] += static_cast<int32_t>(static_cast<int8_t>((vw[j >> 2] >> (8 * (j & 3))) & 0xff));
+    }
+    uint32_t o[4] = {0, 0, 0, 0};
+#pragma unroll
+    for (int j = 0; j < 16; ++j) {
+        const int32_t q = requant_i32(sum[j], mult, false, 0, 0.0f, false);
+        o[j >> 2] |= (static_cast<uint32_t>(q) & 0xffu) << (8 * (j & 3));
+    }
+    *reinterpret_cast<int4*>(y + p * 16) = make_int4(o[0], o[1], o[2], o[3]);
+}
+
+// ------------------------------------------------------------------ host side
+struct QVariant {
+    const char* name;
+    int kh, kw, cbc, wp, ro, ppt;
+    void (*kernel)(const QArgs);
+};
+
+#define KXC_QV(KH, KW, CBC, WP, RO, PPT)                                                             \
+    { "qmfma_k" #KH "x" #KW "_cb" #CBC "_p" #WP "_o" #RO, KH, KW, CBC, WP, RO, PPT,                      \
+      qconv_mfma_kernel<KH, KW, CBC, WP, RO, PPT> }
+
+const QVariant kQVariants[] = {
+    KXC_QV(3, 3, 2, 4, 2, 4),
+    KXC_QV(3, 3, 2, 4, 1, 4),
+    KXC_QV(3, 3, 2, 2, 1, 4),
+    KXC_QV(1, 1, 4, 4, 2, 6),
+    KXC_QV(1, 1, 4, 4, 1, 6),
+    KXC_QV(1, 1, 4, 2, 1, 6),
+    KXC_QV(3, 3, 1, 4, 1, 4),      // at most 16 input channels: k-steps pair filter taps
+    KXC_QV(3, 3, 1, 2, 1, 4),
+    KXC_QV(1, 1, 1, 4, 1, 6),
+    KXC_QV(1, 1, 1, 2, 1, 6),
+    KXC_QV(7, 7, 1, 4, 2, 12),
+    KXC_QV(7, 7, 1, 2, 2, 12),
+};
+
+int CbcFor(int c, int kh, int kw) {
+    const int cb = (c + 15) / 16;
+    if (cb == 1) return 1;
+    if (kh == 1 && kw == 1) return 4;
+    return 2;
+}
+
+struct QLaunch {
+    const QVariant* v = nullptr;
+    QArgs args;
+    int grid = 0;
+    size_t lds_bytes = 0;
+};
+
+// Largest number of patch rows any pixel tile of TP pixels touches.
+int MaxRows(const QArgs& a, int KH, int TP) {
+    int best = 0;
+    for (int m0 = 0; m0 < a.M; m0 += TP) {
+        const int ml = (m0 + TP < a.M ? m0 + TP : a.M) - 1;
+        const int n = m0 / a.OHW, rem = m0 - n * a.OHW;
+        const int n2 = ml / a.OHW, rem2 = ml - n2 * a.OHW;
+        const int qmin = n * a.Hp + (rem / a.OW) * a.sh;
+        const int qlast = n2 * a.Hp + (rem2 / a.OW) * a.sh + KH - 1;
+        if (qlast - qmin + 1 > best) best = qlast - qmin + 1;
+    }
+    return best;
+}
+
+int32_t PrepareUncached(const kxc_hip_qconv2d_desc* d, QLaunch* L, const char* who);
+
+// The selection walks every pixel tile once; a forward pass repeats the same few descriptors, so the last
+// results are kept per thread (pointers are filled in by the caller afterwards).
+int32_t Prepare(const kxc_hip_qconv2d_desc* d, QLaunch* L, const char* who) {
+    KXC_HIP_REQUIRE(d != nullptr, "%s: desc is NULL", who);
+    struct Entry { kxc_hip_qconv2d_desc desc; QLaunch launch; };
+    thread_local std::vector<Entry> cache;
+    for (const Entry& e : cache)
+        if (std::memcmp(&e.desc, d, sizeof(*d)) == 0) { *L = e.launch; return KXC_HIP_OK; }
+    if (int32_t rc = PrepareUncached(d, L, who)) return rc;
+    if (cache.size() >= 128) cache.clear();
+    Entry e;
+    std::memcpy(&e.desc, d, sizeof(*d));
+    e.launch = *L;
+    cache.push_back(e);
+    return KXC_HIP_OK;
+}
+
+int32_t PrepareUncached(const kxc_hip_qconv2d_desc* d, QLaunch* L, const char* who) {
+    KXC_HIP_REQUIRE(d->n >= 0 && d->c > 0 && d->h > 0 && d->w > 0 && d->o > 0 && d->kh > 0 && d->kw > 0,
+                    "%s: bad shape", who);
+    KXC_HIP_REQUIRE(d->stride_h > 0 && d->stride_w > 0 && d->pad_h >= 0 && d->pad_w >= 0, "%s: bad stride or padding", who);
+    const int64_t nh = static_cast<int64_t>(d->h) + 2 * d->pad_h - d->kh;
+    const int64_t nw = static_cast<int64_t>(d->w) + 2 * d->pad_w - d->kw;
+    KXC_HIP_REQUIRE(nh >= 0 && nw >= 0, "%s: window is larger than input", who);
+    KXC_HIP_REQUIRE(d->o % 32 == 0, "%s: output channels must be a multiple of 32 (got %d)", who, d->o);
+    KXC_HIP_REQUIRE(static_cast<int64_t>(d->c) * d->kh * d->kw <= 2147483647LL / (128 * 128),
+                    "%s: reduction too long for int32 accumulation", who);
+    QArgs& a = L->args;
+    std::memset(&a, 0, sizeof(a));
+    a.N = d->n; a.CB = (d->c + 15) / 16; a.H = d->h; a.W = d->w; a.O = d->o;
+    a.OH = static_cast<int32_t>(nh / d->stride_h + 1);
+    a.OW = static_cast<int32_t>(nw / d->stride_w + 1);
+    a.sh = d->stride_h; a.sw = d->stride_w; a.ph = d->pad_h; a.pw = d->pad_w;
+    a.Hp = a.H + 2 * a.ph; a.Wp = a.W + 2 * a.pw;
+    a.OHW = a.OH * a.OW;
+    const int64_t M = static_cast<int64_t>(a.N) * a.OHW;
+    const int64_t xb = static_cast<int64_t>(a.N) * a.CB * a.H * a.W * 16;
+    KXC_HIP_REQUIRE(M < (1LL << 30) && xb < (1LL << 31) && M * (a.O / 16) * 16 < (1LL << 31) &&
+                    static_cast<int64_t>(a.N + 1) * a.Hp * a.Wp < (1LL << 30),
+                    "%s: tensor too large for 32-bit addressing", who);
+    a.M = static_cast<int32_t>(M);
+    a.x_bytes = static_cast<uint32_t>(xb);
+    a.res_mult = d->res_mult;
+    a.flags = d->flags;
+    const int cbc = CbcFor(d->c, d->kh, d->kw);
+    a.nchunks = (a.CB + cbc - 1) / cbc;
+    if (M == 0) return KXC_HIP_OK;
+    // pick the first variant that fits, preferring enough workgroups to fill 256 CUs a few times over
+    const QVariant* best = nullptr;
+    int best_chs = 0;
+    for (const QVariant& v : kQVariants) {
+        if (v.kh != d->kh || v.kw != d->kw || v.cbc != cbc) continue;
+        if ((a.O / 32) % v.ro != 0) continue;
+        const int TP = 32 * v.wp;
+        const int rows = MaxRows(a, v.kh, TP);
+        const int positions = rows * a.Wp;
+        const int segs = (positions + 63) / 64;
+        if (segs > v.ppt * v.wp) continue;
+        const int chs = segs * 64;
+        const int NS = (v.kh * v.kw * cbc + 1) / 2;
+        const size_t buf = static_cast<size_t>(cbc) * chs * 16 + static_cast<size_t>(v.ro) * NS * 1024;
+        const size_t lds = buf * (a.nchunks > 1 ? 2 : 1);
+        if (lds > 160 * 1024) continue;
+        const int64_t tiles = CeilDiv(M, TP) * ((a.O / 32) / v.ro);
+        if (best == nullptr) { best = &v; best_chs = chs; L->lds_bytes = lds; }
+        if (tiles >= 2 * 256) { best = &v; best_chs = chs; L->lds_bytes = lds; break; }
+    }
+    KXC_HIP_REQUIRE(best != nullptr, "%s: no matrix-core variant for a %dx%d filter on this shape", who, d->kh, d->kw);
+    a.chs = best_chs;
+    a.p_tiles = static_cast<int32_t>(CeilDiv(M, 32 * best->wp));
+    a.o_tiles = (a.O / 32) / best->ro;
+    a.num_tiles = a.p_tiles * a.o_tiles;
+    a.tiles_per_xcd = (a.num_tiles + 7) / 8;
+    L->grid = a.tiles_per_xcd * 8;
+    L->v = best;
+    const int NS = (best->kh * best->kw * cbc + 1) / 2;
+    a.w_bytes = static_cast<uint32_t>(static_cast<int64_t>(a.O / 32) * a.nchunks * NS * 1024);
+    return KXC_HIP_OK;
+}
+
+}  // namespace
+
+extern "C" {
+
+int32_t kxc_hip_qconv2d_c16_packed_bytes(const kxc_hip_qconv2d_desc* d, size_t* out_bytes) {
+    KXC_HIP_REQUIRE(d != nullptr && out_bytes != nullptr, "kxc_hip_qconv2d_c16_packed_bytes: NULL argument");
+    KXC_HIP_REQUIRE(d->c > 0 && d->o > 0 && d->kh > 0 && d->kw > 0 && d->o % 32 == 0,
+                    "kxc_hip_qconv2d_c16_packed_bytes: bad shape (output channels must be a multiple of 32)");
+    const int cbc = CbcFor(d->c, d->kh, d->kw);
+    const int cb = (d->c + 15) / 16;
+    const int64_t nchunks = (cb + cbc - 1) / cbc;
+    const int64_t NS = (static_cast<int64_t>(d->kh) * d->kw * cbc + 1) / 2;
+    *out_bytes = static_cast<size_t>((d->o / 32) * nchunks * NS * 1024);
+    return KXC_HIP_OK;
+}
+
+int32_t kxc_hip_qconv2d_c16_pack_weights(const kxc_hip_qconv2d_desc* d, const int8_t* w_oihw, int8_t* packed,
+                                         void* stream) {
+    size_t bytes = 0;
+    if (int32_t rc = kxc_hip_qconv2d_c16_packed_bytes(d, &bytes)) return rc;
+    KXC_HIP_REQUIRE(w_oihw && packed, "kxc_hip_qconv2d_c16_pack_weights: NULL pointer");
+    PackArgs p;
+    p.w = w_oihw; p.wp = packed; p.O = d->o; p.C = d->c; p.KHW = d->kh * d->kw;
+    p.CBC = CbcFor(d->c, d->kh, d->kw);
+    p.NS = (p.KHW * p.CBC + 1) / 2;
+    p.nchunks = ((d->c + 15) / 16 + p.CBC - 1) / p.CBC;
+    p.oblocks = d->o / 32;
+    const int64_t slots = static_cast<int64_t>(bytes / 16);
+    pack_weights_kernel<<<static_cast<int>(CeilDiv(slots, kBlock)), kBlock, 0, ResolveStream(stream)>>>(p, slots);
+    return CheckLaunch("qconv2d_c16_pack_weights");
+}
+
+const char* kxc_hip_qconv2d_c16_variant(const kxc_hip_qconv2d_desc* d) {
+    QLaunch L;
+    if (Prepare(d, &L, "kxc_hip_qconv2d_c16_variant") != KXC_HIP_OK) return "none";
+    return L.v ? L.v->name : "empty";
+}
+
+int32_t kxc_hip_qconv2d_c16_i8(const kxc_hip_qconv2d_desc* d, const int8_t* x, const int8_t* w_packed,
+                               const int32_t* bias, const float* mult, const int8_t* residual, int8_t* y,
+                               void* stream) {
+    QLaunch L;
+    if (int32_t rc = Prepare(d, &L, "kxc_hip_qconv2d_c16_i8")) return rc;
+    if (L.args.M == 0) return KXC_HIP_OK;
+    KXC_HIP_REQUIRE(x && w_packed && mult && y, "kxc_hip_qconv2d_c16_i8: NULL pointer");
+    KXC_HIP_REQUIRE(!(d->flags & KXC_HIP_CONV_BIAS) || bias, "kxc_hip_qconv2d_c16_i8: bias flag without bias");
+    KXC_HIP_REQUIRE(!(d->flags & KXC_HIP_CONV_RESIDUAL) || residual, "kxc_hip_qconv2d_c16_i8: residual flag without residual");
+    QArgs& a = L.args;
+    a.x = x; a.wp = w_packed; a.bias = bias; a.mult = mult; a.res = residual; a.y = y;
+    if (L.lds_bytes > 64 * 1024) {
+        KXC_HIP_CALL(hipFuncSetAttribute(reinterpret_cast<const void*>(L.v->kernel),
+                                         hipFuncAttributeMaxDynamicSharedMemorySize, static_cast<int>(L.lds_bytes)),
+                     "hipFuncSetAttribute");
+    }
+    hipLaunchKernelGGL(L.v->kernel, dim3(L.grid), dim3(64 * L.v->wp), L.lds_bytes, ResolveStream(stream), a);
+    return CheckLaunch(L.v->name);
+}
+
+int32_t kxc_hip_i8_nchw_to_c16(const int8_t* x, int8_t* y, int64_t n, int64_t c, int64_t hw, void* stream) {
+    KXC_HIP_REQUIRE(n >= 0 && c > 0 && hw >= 0, "kxc_hip_i8_nchw_to_c16: bad shape");
+    const int64_t cb = (c + 15) / 16, total = n * cb * hw;
+    if (total == 0) return KXC_HIP_OK;
+    KXC_HIP_REQUIRE(x && y, "kxc_hip_i8_nchw_to_c16: NULL pointer");
+    KXC_HIP_REQUIRE(CeilDiv(total, kBlock) <= kMaxGridX, "kxc_hip_i8_nchw_to_c16: tensor too large");
+    nchw_to_c16_kernel<<<static_cast<int>(CeilDiv(total, kBlock)), kBlock, 0, ResolveStream(stream)>>>(
+        x, y, static_cast<int32_t>(c), static_cast<int32_t>(cb), hw, total);
+    return CheckLaunch("i8_nchw_to_c16");
+}
+
+int32_t kxc_hip_i8_c16_to_nchw(const int8_t* x, int8_t* y, int64_t n, int64_t c, int64_t hw, void* stream) {
+    KXC_HIP_REQUIRE(n >= 0 && c > 0 && hw >= 0, "kxc_hip_i8_c16_to_nchw: bad shape");
+    const int64_t cb = (c + 15) / 16, total = n * c * hw;
+    if (total == 0) return KXC_HIP_OK;
+    KXC_HIP_REQUIRE(x && y, "kxc_hip_i8_c16_to_nchw: NULL pointer");
+    KXC_HIP_REQUIRE(CeilDiv(total, kBlock) <= kMaxGridX, "kxc_hip_i8_c16_to_nchw: tensor too large");
+    c16_to_nchw_kernel<<<static_cast<int>(CeilDiv(total, kBlock)), kBlock, 0, ResolveStream(stream)>>>(
+        x, y, static_cast<int32_t>(c), static_cast<int32_t>(cb), hw, total);
+    return CheckLaunch("i8_c16_to_nchw");
+}
+
+int32_t kxc_hip_quantize_f32_nchw_to_c16_i8(const float* x, int8_t* y, int64_t n, int64_t c, int64_t hw, float scale,
+                                            void* stream) {
+    KXC_HIP_REQUIRE(n >= 0 && c > 0 && hw >= 0, "kxc_hip_quantize_f32_nchw_to_c16_i8: bad shape");
+    KXC_HIP_REQUIRE(scale > 0.0f, "kxc_hip_quantize_f32_nchw_to_c16_i8: scale must be positive");
+    const int64_t cb = (c + 15) / 16, total = n * cb * hw;
+    if (total == 0) return KXC_HIP_OK;
+    KXC_HIP_REQUIRE(x && y, "kxc_hip_quantize_f32_nchw_to_c16_i8: NULL pointer");
+    KXC_HIP_REQUIRE(CeilDiv(total, kBlock) <= kMaxGridX, "kxc_hip_quantize_f32_nchw_to_c16_i8: tensor too large");
+    quantize_to_c16_kernel<<<static_cast<int>(CeilDiv(total, kBlock)), kBlock, 0, ResolveStream(stream)>>>(
+        x, y, static_cast<int32_t>(c), static_cast<int32_t>(cb), hw, total, scale);
+    return CheckLaunch("quantize_f32_nchw_to_c16_i8");
+}
+
+int32_t kxc_hip_maxpool2d_c16_i8(const kxc_hip_pool2d_desc* p, const int8_t* x, int8_t* y, void* stream) {
+    KXC_HIP_REQUIRE(p != nullptr, "kxc_hip_maxpool2d_c16_i8: desc is NULL");
+    KXC_HIP_REQUIRE(p->n >= 0 && p->c > 0 && p->h > 0 && p->w > 0, "kxc_hip_maxpool2d_c16_i8: bad input shape");
+    KXC_HIP_REQUIRE(p->kh > 0 && p->kw > 0 && p->stride_h > 0 && p->stride_w > 0, "kxc_hip_maxpool2d_c16_i8: bad window");
+    KXC_HIP_REQUIRE(p->pad_top >= 0 && p->pad_left >= 0 && p->pad_bottom >= 0 && p->pad_right >= 0,
+                    "kxc_hip_maxpool2d_c16_i8: negative padding");
+    KXC_HIP_REQUIRE(!p->is_avg, "kxc_hip_maxpool2d_c16_i8: average pooling is not defined for int8");
+    const int hn = p->h + p->pad_top + p->pad_bottom - p->kh;
+    const int wn = p->w + p->pad_left + p->pad_right - p->kw;
+    KXC_HIP_REQUIRE(hn >= 0 && wn >= 0, "kxc_hip_maxpool2d_c16_i8: pool2d window is larger than input");
+    PoolArgs d;
+    d.N = p->n; d.CB = (p->c + 15) / 16; d.H = p->h; d.W = p->w;
+    d.OH = p->ceil_mode ? (hn + p->stride_h - 1) / p->stride_h + 1 : hn / p->stride_h + 1;
+    d.OW = p->ceil_mode ? (wn + p->stride_w - 1) / p->stride_w + 1 : wn / p->stride_w + 1;
+    d.KH = p->kh; d.KW = p->kw; d.sh = p->stride_h; d.sw = p->stride_w; d.pt = p->pad_top; d.pl = p->pad_left;
+    const int64_t total = static_cast<int64_t>(d.N) * d.CB * d.OH * d.OW;
+    if (total == 0) return KXC_HIP_OK;
+    KXC_HIP_REQUIRE(x && y, "kxc_hip_maxpool2d_c16_i8: NULL pointer");
+    KXC_HIP_REQUIRE(CeilDiv(total, kBlock) <= kMaxGridX, "kxc_hip_maxpool2d_c16_i8: tensor too large");
+    maxpool_c16_kernel<<<static_cast<int>(CeilDiv(total, kBlock)), kBlock, 0, ResolveStream(stream)>>>(x, y, d, total);
+    return CheckLaunch("maxpool2d_c16_i8");
+}
+
+int32_t kxc_hip_global_avg_pool2d_c16_i8(const int8_t* x, int8_t* y, int64_t n, int64_t c, int64_t h, int64_t w,
+                                         float mult, void* stream) {
+    KXC_HIP_REQUIRE(n >= 0 && c > 0 && h > 0 && w > 0, "kxc_hip_global_avg_pool2d_c16_i8: bad shape");
+    KXC_HIP_REQUIRE(h * w <= 2147483647LL / 128, "kxc_hip_global_avg_pool2d_c16_i8: plane too large for int32 sum");
+    const int64_t planes = n * ((c + 15) / 16);
+    if (planes == 0) return KXC_HIP_OK;
+    KXC_HIP_REQUIRE(x && y, "kxc_hip_global_avg_pool2d_c16_i8: NULL pointer");
+    gap_c16_kernel<<<static_cast<int>(CeilDiv(planes, kBlock)), kBlock, 0, ResolveStream(stream)>>>(
+        x, y, planes, static_cast<int32_t>(h * w), mult);
+    return CheckLaunch("global_avg_pool2d_c16_i8");
+}
+
+}  // extern "C"

@@ -79,6 +79,7 @@ def lib():
         _lib.kxc_hip_last_error.restype = C.c_char_p
         _lib.kxc_hip_target_kind.restype = C.c_char_p
         _lib.kxc_hip_conv2d_variant.restype = C.c_char_p
+        _lib.kxc_hip_qconv2d_c16_variant.restype = C.c_char_p
         _lib.kxc_hip_plan_node_symbol.restype = C.c_char_p
         _lib.kxc_hip_plan_workspace.restype = C.c_void_p
     return _lib
@@ -235,6 +236,15 @@ def quantize(x, scale):
     return q
 
 
+def absmax(x):
+    """max |x| of a GPU fp32 tensor, as a Python float (synchronises)."""
+    import torch
+    _need(x, torch.float32, "x")
+    out = torch.empty((1,), dtype=torch.float32, device=x.device)
+    _check(lib().kxc_hip_absmax_f32(_p(x), C.c_int64(x.numel()), _p(out), _stream()))
+    return float(out.item())
+
+
 def qconv2d(x, w, bias, mult, residual=None, res_mult=0.0, stride=1, pad=0, relu=True, force_direct=False):
     import torch
     _need(x, torch.int8, "x"); _need(w, torch.int8, "w"); _need(bias, torch.int32, "bias")
@@ -277,6 +287,99 @@ def global_avg_pool2d_i8(x, mult):
     y = torch.empty((n, c, 1, 1), dtype=torch.int8, device=x.device)
     _check(lib().kxc_hip_global_avg_pool2d_i8(_p(x), _p(y), C.c_int64(n), C.c_int64(c), C.c_int64(h), C.c_int64(w),
                                               C.c_float(mult), _stream()))
+    return y
+
+
+# ---- int8 on the channel-blocked "c16" layout ([N][ceil(C/16)][H][W][16])
+
+def c16_shape(n, c, h, w):
+    return (n, (c + 15) // 16, h, w, 16)
+
+
+def i8_nchw_to_c16(x):
+    import torch
+    _need(x, torch.int8, "x")
+    n, c, h, w = x.shape
+    y = torch.empty(c16_shape(n, c, h, w), dtype=torch.int8, device=x.device)
+    _check(lib().kxc_hip_i8_nchw_to_c16(_p(x), _p(y), C.c_int64(n), C.c_int64(c), C.c_int64(h * w), _stream()))
+    return y
+
+
+def i8_c16_to_nchw(x, c):
+    import torch
+    _need(x, torch.int8, "x")
+    n, cb, h, w, _ = x.shape
+    y = torch.empty((n, c, h, w), dtype=torch.int8, device=x.device)
+    _check(lib().kxc_hip_i8_c16_to_nchw(_p(x), _p(y), C.c_int64(n), C.c_int64(c), C.c_int64(h * w), _stream()))
+    return y
+
+
+def quantize_to_c16(x, scale):
+    import torch
+    _need(x, torch.float32, "x")
+    n, c, h, w = x.shape
+    y = torch.empty(c16_shape(n, c, h, w), dtype=torch.int8, device=x.device)
+    _check(lib().kxc_hip_quantize_f32_nchw_to_c16_i8(_p(x), _p(y), C.c_int64(n), C.c_int64(c), C.c_int64(h * w),
+                                                     C.c_float(scale), _stream()))
+    return y
+
+
+def qconv_desc(n, c, h, w, o, kh, kw, stride, pad, flags=0, res_mult=0.0):
+    return QConvDesc(n, c, h, w, o, kh, kw, stride, stride, pad, pad, flags, res_mult)
+
+
+def qconv2d_c16_variant(d):
+    return lib().kxc_hip_qconv2d_c16_variant(C.byref(d)).decode()
+
+
+def qconv2d_c16_pack_weights(w):
+    """OIHW int8 weights (GPU) -> the packed order the matrix-core kernel reads."""
+    import torch
+    _need(w, torch.int8, "w")
+    o, c, kh, kw = w.shape
+    d = qconv_desc(1, c, kh, kw, o, kh, kw, 1, 0)
+    nbytes = C.c_size_t()
+    _check(lib().kxc_hip_qconv2d_c16_packed_bytes(C.byref(d), C.byref(nbytes)))
+    packed = torch.empty((nbytes.value,), dtype=torch.int8, device=w.device)
+    _check(lib().kxc_hip_qconv2d_c16_pack_weights(C.byref(d), _p(w), _p(packed), _stream()))
+    return packed
+
+
+def qconv2d_c16(x, c, w_packed, w_shape, bias, mult, residual=None, res_mult=0.0, stride=1, pad=0, relu=True):
+    """x: c16 tensor of logical channel count c; returns the c16 output."""
+    import torch
+    _need(x, torch.int8, "x"); _need(w_packed, torch.int8, "w_packed"); _need(bias, torch.int32, "bias")
+    _need(mult, torch.float32, "mult"); _need(residual, torch.int8, "residual")
+    n, cb, h, wd, _ = x.shape
+    o, _, kh, kw = w_shape
+    flags = (CONV_BIAS if bias is not None else 0) | (CONV_RESIDUAL if residual is not None else 0) | \
+            (CONV_RELU if relu else 0)
+    d = qconv_desc(n, c, h, wd, o, kh, kw, stride, pad, flags, res_mult)
+    oh = (h + 2 * pad - kh) // stride + 1; ow = (wd + 2 * pad - kw) // stride + 1
+    y = torch.empty(c16_shape(n, o, oh, ow), dtype=torch.int8, device=x.device)
+    _check(lib().kxc_hip_qconv2d_c16_i8(C.byref(d), _p(x), _p(w_packed), _p(bias), _p(mult), _p(residual), _p(y),
+                                        _stream()))
+    return y
+
+
+def maxpool2d_c16_i8(x, c, k, s, pad):
+    import torch
+    _need(x, torch.int8, "x")
+    n, cb, h, w, _ = x.shape
+    d = pool_desc((n, c, h, w), k, s, pad)
+    _, _, oh, ow = pool_out_shape(d)
+    y = torch.empty(c16_shape(n, c, oh, ow), dtype=torch.int8, device=x.device)
+    _check(lib().kxc_hip_maxpool2d_c16_i8(C.byref(d), _p(x), _p(y), _stream()))
+    return y
+
+
+def global_avg_pool2d_c16_i8(x, c, mult):
+    import torch
+    _need(x, torch.int8, "x")
+    n, cb, h, w, _ = x.shape
+    y = torch.empty((n, cb * 16), dtype=torch.int8, device=x.device)
+    _check(lib().kxc_hip_global_avg_pool2d_c16_i8(_p(x), _p(y), C.c_int64(n), C.c_int64(c), C.c_int64(h), C.c_int64(w),
+                                                  C.c_float(mult), _stream()))
     return y
 
 
@@ -335,6 +438,19 @@ class Plan:
     def add_global_avg_pool2d_i8(self, n, c, h, w, mult, x, y):
         _check(lib().kxc_hip_plan_add_global_avg_pool2d_i8(self._h, C.c_int64(n), C.c_int64(c), C.c_int64(h),
                                                            C.c_int64(w), C.c_float(mult), x, y))
+
+    def add_qconv2d_c16(self, desc, x, w_packed, bias, mult, residual, y):
+        _check(lib().kxc_hip_plan_add_qconv2d_c16(self._h, C.byref(desc), x, w_packed, bias, mult, residual, y))
+
+    def add_quantize_c16(self, n, c, hw, scale, x, q):
+        _check(lib().kxc_hip_plan_add_quantize_c16(self._h, C.c_int64(n), C.c_int64(c), C.c_int64(hw), C.c_float(scale), x, q))
+
+    def add_maxpool2d_c16_i8(self, desc, x, y):
+        _check(lib().kxc_hip_plan_add_maxpool2d_c16_i8(self._h, C.byref(desc), x, y))
+
+    def add_global_avg_pool2d_c16_i8(self, n, c, h, w, mult, x, y):
+        _check(lib().kxc_hip_plan_add_global_avg_pool2d_c16_i8(self._h, C.c_int64(n), C.c_int64(c), C.c_int64(h),
+                                                               C.c_int64(w), C.c_float(mult), x, y))
 
     def add_qdense(self, m, n, k, a, b, bias, mult, y):
         _check(lib().kxc_hip_plan_add_qdense(self._h, C.c_int64(m), C.c_int64(n), C.c_int64(k), a, b, bias, mult, y))

@@ -158,6 +158,9 @@ int32_t kxc_hip_flatten_f32(const float* x, float* y, int64_t n, void* stream);
  *      definition in oracle/kxc_oracle.h (qnn-style conv/dense with int32 accumulate and
  *      per-output-channel fp32 requantisation, round half to even). ---- */
 int32_t kxc_hip_quantize_f32_i8(const float* x, int8_t* q, int64_t n, float scale, void* stream);
+/* Calibration helper: *out (device float) = max |x[i]| (0 for an empty tensor; NaN ignored).  Per-tensor
+ * symmetric scales are max-abs / 127. */
+int32_t kxc_hip_absmax_f32(const float* x, int64_t n, float* out, void* stream);
 typedef struct kxc_hip_qconv2d_desc {
     int32_t n, c, h, w;
     int32_t o, kh, kw;
@@ -174,6 +177,32 @@ int32_t kxc_hip_qdense_i8(const int8_t* a, const int8_t* b, const int32_t* bias,
 int32_t kxc_hip_maxpool2d_i8(const kxc_hip_pool2d_desc* desc, const int8_t* x, int8_t* y, void* stream);
 int32_t kxc_hip_global_avg_pool2d_i8(const int8_t* x, int8_t* y, int64_t n, int64_t c, int64_t h,
                                      int64_t w, float mult, void* stream);
+
+/* ---- int8 on the channel-blocked "c16" layout: logical [N,C,H,W] stored as [N][ceil(C/16)][H][W][16]
+ *      (element (n,c,h,w) at (((n*CB + c/16)*H + h)*W + w)*16 + c%16, channels >= C are zero).  One pixel's 16
+ *      channels are the 16-byte k-slice a lane feeds to v_mfma_i32_32x32x32_i8, so the convolution runs on
+ *      the int8 matrix cores with no byte gathers.  Same arithmetic as the NCHW entry points; like them these
+ *      have no counterpart in the reference (no int8 operator exists there). ---- */
+/* Size in bytes of the packed weight buffer for a convolution (output channels must be a multiple of 32). */
+int32_t kxc_hip_qconv2d_c16_packed_bytes(const kxc_hip_qconv2d_desc* desc, size_t* out_bytes);
+/* Repack OIHW int8 weights (device) into the order the matrix-core kernel reads them (device, once per model). */
+int32_t kxc_hip_qconv2d_c16_pack_weights(const kxc_hip_qconv2d_desc* desc, const int8_t* w_oihw, int8_t* packed,
+                                         void* stream);
+/* Name of the kernel variant the shape selects ("none" when no matrix-core variant covers it). */
+const char* kxc_hip_qconv2d_c16_variant(const kxc_hip_qconv2d_desc* desc);
+/* x, residual, y in c16; w_packed from kxc_hip_qconv2d_c16_pack_weights; bias int32[O], mult float[O]. */
+int32_t kxc_hip_qconv2d_c16_i8(const kxc_hip_qconv2d_desc* desc, const int8_t* x, const int8_t* w_packed,
+                               const int32_t* bias, const float* mult, const int8_t* residual, int8_t* y,
+                               void* stream);
+/* Layout converters and the quantising converter (fp32 NCHW -> int8 c16, same rounding as kxc_hip_quantize_f32_i8). */
+int32_t kxc_hip_i8_nchw_to_c16(const int8_t* x, int8_t* y, int64_t n, int64_t c, int64_t hw, void* stream);
+int32_t kxc_hip_i8_c16_to_nchw(const int8_t* x, int8_t* y, int64_t n, int64_t c, int64_t hw, void* stream);
+int32_t kxc_hip_quantize_f32_nchw_to_c16_i8(const float* x, int8_t* y, int64_t n, int64_t c, int64_t hw,
+                                            float scale, void* stream);
+int32_t kxc_hip_maxpool2d_c16_i8(const kxc_hip_pool2d_desc* desc, const int8_t* x, int8_t* y, void* stream);
+/* Output is [N][ceil(C/16)*16] int8 (c16 with H = W = 1, i.e. plain row-major when C is a multiple of 16). */
+int32_t kxc_hip_global_avg_pool2d_c16_i8(const int8_t* x, int8_t* y, int64_t n, int64_t c, int64_t h,
+                                         int64_t w, float mult, void* stream);
 
 /* ========================================================================
  * 3. Module loader -- run-time compiled kernels (the TIR->HIP emitter's output).
@@ -240,6 +269,15 @@ int32_t kxc_hip_plan_add_maxpool2d_i8(kxc_hip_plan* plan, const kxc_hip_pool2d_d
                                       kxc_hip_buf x, kxc_hip_buf y);
 int32_t kxc_hip_plan_add_global_avg_pool2d_i8(kxc_hip_plan* plan, int64_t n, int64_t c, int64_t h,
                                               int64_t w, float mult, kxc_hip_buf x, kxc_hip_buf y);
+int32_t kxc_hip_plan_add_qconv2d_c16(kxc_hip_plan* plan, const kxc_hip_qconv2d_desc* desc, kxc_hip_buf x,
+                                     kxc_hip_buf w_packed, kxc_hip_buf bias, kxc_hip_buf mult,
+                                     kxc_hip_buf residual, kxc_hip_buf y);
+int32_t kxc_hip_plan_add_quantize_c16(kxc_hip_plan* plan, int64_t n, int64_t c, int64_t hw, float scale,
+                                      kxc_hip_buf x, kxc_hip_buf q);
+int32_t kxc_hip_plan_add_maxpool2d_c16_i8(kxc_hip_plan* plan, const kxc_hip_pool2d_desc* desc,
+                                          kxc_hip_buf x, kxc_hip_buf y);
+int32_t kxc_hip_plan_add_global_avg_pool2d_c16_i8(kxc_hip_plan* plan, int64_t n, int64_t c, int64_t h,
+                                                  int64_t w, float mult, kxc_hip_buf x, kxc_hip_buf y);
 int32_t kxc_hip_plan_add_qdense(kxc_hip_plan* plan, int64_t m, int64_t n, int64_t k, kxc_hip_buf a,
                                 kxc_hip_buf b, kxc_hip_buf bias, kxc_hip_buf mult, kxc_hip_buf y);
 /* A run-time compiled kernel (section 3): params[i] is a buffer operand, passed as a pointer. */

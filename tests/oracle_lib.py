@@ -187,6 +187,38 @@ class Oracle:
                                                  C.c_float(mult))
         return y
 
+    def qresnet18(self, x, model, gap_mult):
+        """Quantised ResNet-18 as a chain of the CPU int8 operators (NCHW).  `model` is the dict of quantised
+        constants and scales the product's preparation step produced: both sides consume the same numbers.
+        Returns (logits fp32, {tap name: int8 NCHW tensor})."""
+        by = {L["name"]: L for L in model["layers"]}
+        taps = {}
+
+        def conv(t, name, res=None):
+            L = by[name]
+            y = self.qconv(t, L["wq"], L["bias_q"], L["mult"], L["stride"], L["pad"], res,
+                           L["res_mult"] if res is not None else 0.0, L["relu"])
+            taps[name] = y
+            return y
+
+        q = self.quantize(x, model["input_scale"])
+        taps["input"] = q
+        y = conv(q, "conv1")
+        cur = self.qmaxpool(y, 3, 2, 1)
+        taps["maxpool"] = cur
+        for stage in range(4):
+            for blk in range(2):
+                first = blk == 0 and stage > 0
+                name = "l%d.%d" % (stage + 1, blk)
+                a = conv(cur, name + ".conv1")
+                idn = conv(cur, name + ".down") if first else cur
+                cur = conv(a, name + ".conv2", idn)
+        g = self.qgap(cur, gap_mult)
+        taps["gap"] = g
+        fc = model["fc"]
+        logits = self.qdense(g.reshape(g.shape[0], -1), fc["wq"], fc["bias_q"], fc["mult"])
+        return logits, taps
+
     # ---- network ----
     TAP_NAMES = ("conv1_relu", "maxpool", "layer1", "layer2", "layer3", "layer4", "gap", "flatten", "logits")
 
