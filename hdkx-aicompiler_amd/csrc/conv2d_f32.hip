@@ -39,6 +39,10 @@ namespace {
 
 typedef float floatx16 __attribute__((ext_vector_type(16)));
 
+struct FastDiv {
+    uint32_t mul, shift;
+};
+
 struct ConvArgs {
     const float* x;
     const float* w;
@@ -55,9 +59,16 @@ struct ConvArgs {
     uint32_t x_bytes, w_bytes;
     int32_t p_tiles, o_tiles, num_tiles, tiles_per_xcd, o_fastest;
     uint32_t flags;
+    FastDiv div_wp, div_hp, div_ohw, div_ow, div_otiles, div_ptiles;
 };
 
 __device__ __forceinline__ float relu_sel(float v) { return (v > 0.0f) ? v : 0.0f; }
+
+// Division of x < 2^31 by a launch-invariant divisor as a multiply and a shift (the magic number comes from
+// the host): a hardware-less integer division costs ~35 instructions and the tile set-up needs about twenty.
+__device__ __forceinline__ int fast_div(int x, FastDiv f) {
+    return static_cast<int>((static_cast<uint64_t>(static_cast<uint32_t>(x)) * f.mul) >> f.shift);
+}
 
 // ------------------------------------------------------------------------------------------
 // MFMA kernel.  KH,KW: filter; CC: channels per LDS chunk (even); WO x WP waves, each wave
@@ -125,8 +136,8 @@ conv_mfma_kernel(const ConvArgs a) {
     int tile = (blockIdx.x & 7) * a.tiles_per_xcd + (blockIdx.x >> 3);
     if (tile >= a.num_tiles || (blockIdx.x >> 3) >= a.tiles_per_xcd) return;
     int p_tile, o_tile;
-    if (a.o_fastest) { p_tile = tile / a.o_tiles; o_tile = tile - p_tile * a.o_tiles; }
-    else { o_tile = tile / a.p_tiles; p_tile = tile - o_tile * a.p_tiles; }
+    if (a.o_fastest) { p_tile = fast_div(tile, a.div_otiles); o_tile = tile - p_tile * a.o_tiles; }
+    else { o_tile = fast_div(tile, a.div_ptiles); p_tile = tile - o_tile * a.p_tiles; }
     const int m0 = p_tile * TP;
     const int o0 = o_tile * TO;
 
@@ -134,10 +145,10 @@ conv_mfma_kernel(const ConvArgs a) {
     const int m_last = min(m0 + TP, a.M) - 1;
     int qmin, qlast;
     {
-        const int n = m0 / a.OHW, rem = m0 - n * a.OHW;
-        qmin = n * a.Hp + (rem / a.OW) * a.sh;
-        const int n2 = m_last / a.OHW, rem2 = m_last - n2 * a.OHW;
-        qlast = n2 * a.Hp + (rem2 / a.OW) * a.sh + (KH - 1) * a.dh;
+        const int n = fast_div(m0, a.div_ohw), rem = m0 - n * a.OHW;
+        qmin = n * a.Hp + fast_div(rem, a.div_ow) * a.sh;
+        const int n2 = fast_div(m_last, a.div_ohw), rem2 = m_last - n2 * a.OHW;
+        qlast = n2 * a.Hp + fast_div(rem2, a.div_ow) * a.sh + (KH - 1) * a.dh;
     }
     const int P = (qlast - qmin + 1) * a.Wp;      // patch positions per channel (<= chs - 32)
     const int xsegs = (P + 63) >> 6;              // 64-float segments per channel
@@ -151,9 +162,9 @@ conv_mfma_kernel(const ConvArgs a) {
 #pragma unroll
     for (int i = 0; i < PPT; ++i) {
         const int pos = (wave + i * NW) * 64 + lane;
-        const int q = pos / a.Wp, col = pos - q * a.Wp;
+        const int q = fast_div(pos, a.div_wp), col = pos - q * a.Wp;
         const int Q = qmin + q;
-        const int n = Q / a.Hp, ih = Q - n * a.Hp - a.ph, iw = col - a.pw;
+        const int n = fast_div(Q, a.div_hp), ih = Q - n * a.Hp - a.ph, iw = col - a.pw;
         const bool ok = pos < P && n < a.N && ih >= 0 && ih < a.H && iw >= 0 && iw < a.W;
         goff[i] = ok ? static_cast<uint32_t>(((n * a.C) * a.H + ih) * a.W + iw) * 4u : kOobOffset;
     }
@@ -181,8 +192,8 @@ conv_mfma_kernel(const ConvArgs a) {
     for (int j = 0; j < RP; ++j) {
         const int m = m0 + (wave_p * RP + j) * 32 + r;
         const int mc = min(m, a.M - 1);
-        const int n = mc / a.OHW, rem = mc - n * a.OHW;
-        const int oh = rem / a.OW, ow = rem - oh * a.OW;
+        const int n = fast_div(mc, a.div_ohw), rem = mc - n * a.OHW;
+        const int oh = fast_div(rem, a.div_ow), ow = rem - oh * a.OW;
         xbase[j] = (n * a.Hp + oh * a.sh - qmin) * a.Wp + ow * a.sw + half * a.chs;
         ybase[j] = (m < a.M) ? n * a.O * a.OHW + rem : -1;
     }
@@ -525,6 +536,17 @@ void Select(const ConvArgs& a, int kh, int kw, Choice* choice) {
     }
 }
 
+// floor(x / d) == (x * mul) >> shift for every 0 <= x < 2^31: shift = 31 + ceil(log2 d), mul = floor(2^shift / d) + 1.
+FastDiv MakeFastDiv(int32_t d) {
+    FastDiv f{1u << 31, 31};
+    if (d <= 0) return f;
+    uint32_t s = 0;
+    while ((1LL << s) < d) ++s;
+    f.shift = 31 + s;
+    f.mul = static_cast<uint32_t>((1ULL << f.shift) / static_cast<uint64_t>(d) + 1);
+    return f;
+}
+
 int32_t FillArgs(const kxc_hip_conv2d_desc* d, ConvArgs* a, const char* who) {
     KXC_HIP_REQUIRE(d != nullptr, "%s: desc is NULL", who);
     KXC_HIP_REQUIRE(d->n >= 0 && d->c > 0 && d->h > 0 && d->w > 0 && d->o > 0 && d->kh > 0 && d->kw > 0,
@@ -588,6 +610,8 @@ int32_t kxc_hip_conv2d_nchw_f32(const kxc_hip_conv2d_desc* desc, const float* x,
         KXC_HIP_REQUIRE(tiles < (1LL << 30), "kxc_hip_conv2d_nchw_f32: too many tiles");
         a.num_tiles = static_cast<int32_t>(tiles);
         a.tiles_per_xcd = static_cast<int32_t>(CeilDiv(tiles, 8));
+        a.div_wp = MakeFastDiv(a.Wp); a.div_hp = MakeFastDiv(a.Hp); a.div_ohw = MakeFastDiv(a.OHW);
+        a.div_ow = MakeFastDiv(a.OW); a.div_otiles = MakeFastDiv(a.o_tiles); a.div_ptiles = MakeFastDiv(a.p_tiles);
         // weights of one output-channel tile: to * C * kh * kw * 4 bytes; keep the larger operand resident
         const int64_t w_tile_bytes = static_cast<int64_t>(c.v->to) * a.C * desc->kh * desc->kw * 4;
         a.o_fastest = w_tile_bytes * a.o_tiles <= (2 << 20) ? 1 : 0;
