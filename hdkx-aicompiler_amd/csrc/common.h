@@ -38,6 +38,18 @@ inline int32_t CheckLaunch(const char* what) {
     return KXC_HIP_OK;
 }
 
+// Geometry of the calling thread's most recent kernel launch, for the profiled plan run: the launch sites
+// pass their grid, block and dynamic-LDS arguments through these.
+struct LaunchNote {
+    uint32_t grid[3] = {0, 0, 0};
+    uint32_t block[3] = {0, 0, 0};
+    uint32_t dynamic_lds = 0;
+};
+LaunchNote& LastLaunch();
+inline dim3 NoteGrid(dim3 g) { LaunchNote& n = LastLaunch(); n.grid[0] = g.x; n.grid[1] = g.y; n.grid[2] = g.z; return g; }
+inline dim3 NoteBlock(dim3 b) { LaunchNote& n = LastLaunch(); n.block[0] = b.x; n.block[1] = b.y; n.block[2] = b.z; return b; }
+inline size_t NoteLds(size_t bytes) { LastLaunch().dynamic_lds = static_cast<uint32_t>(bytes); return bytes; }
+
 constexpr int64_t kMaxGridX = 2147483647LL;
 
 inline int64_t CeilDiv(int64_t a, int64_t b) { return (a + b - 1) / b; }

@@ -624,12 +624,12 @@ int32_t kxc_hip_conv2d_nchw_f32(const kxc_hip_conv2d_desc* desc, const float* x,
                                              static_cast<int>(c.lds_bytes)),
                          "hipFuncSetAttribute(MaxDynamicSharedMemorySize)");
         }
-        hipLaunchKernelGGL(c.v->kernel, grid, dim3(64 * c.v->nw * c.v->ks), c.lds_bytes, s, a);
+        hipLaunchKernelGGL(c.v->kernel, NoteGrid(grid), NoteBlock(dim3(64 * c.v->nw * c.v->ks)), NoteLds(c.lds_bytes), s, a);
         return CheckLaunch(c.v->name);
     }
     int64_t g = CeilDiv(total, 256);
     if (g > 256 * 64) g = 256 * 64;
-    conv_direct_kernel<<<static_cast<int>(g), 256, 0, s>>>(a, desc->kh, desc->kw, total);
+    conv_direct_kernel<<<NoteGrid(static_cast<int>(g)), NoteBlock(256), NoteLds(0), s>>>(a, desc->kh, desc->kw, total);
     return CheckLaunch("conv_direct");
 }
 

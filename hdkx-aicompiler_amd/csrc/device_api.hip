@@ -11,6 +11,10 @@ std::string& LastError() {
     static thread_local std::string msg;
     return msg;
 }
+LaunchNote& LastLaunch() {
+    static thread_local LaunchNote note;
+    return note;
+}
 hipStream_t& CurrentStream() {
     static thread_local hipStream_t s = nullptr;
     return s;

@@ -155,12 +155,12 @@ int32_t LaunchSameShape(const float* a, const float* b, float* y, int64_t n, boo
         // unaligned: go through the generic kernel with a flat 1-d description
         BroadcastDims d{};
         d.ndim = 1; d.out_shape[0] = n; d.a_stride[0] = 1; d.b_stride[0] = 1;
-        if (relu) broadcast_kernel<OP, true><<<grid, kBlock, 0, s>>>(a, b, y, d, n);
-        else broadcast_kernel<OP, false><<<grid, kBlock, 0, s>>>(a, b, y, d, n);
+        if (relu) broadcast_kernel<OP, true><<<NoteGrid(grid), NoteBlock(kBlock), NoteLds(0), s>>>(a, b, y, d, n);
+        else broadcast_kernel<OP, false><<<NoteGrid(grid), NoteBlock(kBlock), NoteLds(0), s>>>(a, b, y, d, n);
     } else if (relu) {
-        same_shape_kernel<OP, true><<<grid, kBlock, 0, s>>>(a, b, y, n4, n);
+        same_shape_kernel<OP, true><<<NoteGrid(grid), NoteBlock(kBlock), NoteLds(0), s>>>(a, b, y, n4, n);
     } else {
-        same_shape_kernel<OP, false><<<grid, kBlock, 0, s>>>(a, b, y, n4, n);
+        same_shape_kernel<OP, false><<<NoteGrid(grid), NoteBlock(kBlock), NoteLds(0), s>>>(a, b, y, n4, n);
     }
     return CheckLaunch("broadcast_binary");
 }
@@ -169,8 +169,8 @@ template <int OP>
 int32_t LaunchBroadcast(const float* a, const float* b, float* y, const BroadcastDims& d, int64_t total, bool relu,
                         hipStream_t s) {
     const int grid = GridFor(total);
-    if (relu) broadcast_kernel<OP, true><<<grid, kBlock, 0, s>>>(a, b, y, d, total);
-    else broadcast_kernel<OP, false><<<grid, kBlock, 0, s>>>(a, b, y, d, total);
+    if (relu) broadcast_kernel<OP, true><<<NoteGrid(grid), NoteBlock(kBlock), NoteLds(0), s>>>(a, b, y, d, total);
+    else broadcast_kernel<OP, false><<<NoteGrid(grid), NoteBlock(kBlock), NoteLds(0), s>>>(a, b, y, d, total);
     return CheckLaunch("broadcast_binary");
 }
 
@@ -184,9 +184,9 @@ int32_t kxc_hip_relu_f32(const float* x, float* y, int64_t n, void* stream) {
     KXC_HIP_REQUIRE(x && y, "kxc_hip_relu_f32: NULL pointer");
     hipStream_t s = ResolveStream(stream);
     if (Aligned16(x) && Aligned16(y) && n >= 4) {
-        relu_kernel<<<GridFor(n / 4), kBlock, 0, s>>>(x, y, n / 4, n);
+        relu_kernel<<<NoteGrid(GridFor(n / 4)), NoteBlock(kBlock), NoteLds(0), s>>>(x, y, n / 4, n);
     } else {
-        relu_scalar_kernel<<<GridFor(n), kBlock, 0, s>>>(x, y, n);
+        relu_scalar_kernel<<<NoteGrid(GridFor(n)), NoteBlock(kBlock), NoteLds(0), s>>>(x, y, n);
     }
     return CheckLaunch("relu");
 }
@@ -246,8 +246,8 @@ int32_t kxc_hip_bias_add_nchw_f32(const float* x, const float* bias, float* y, i
     if (total == 0) return KXC_HIP_OK;
     KXC_HIP_REQUIRE(x && bias && y, "kxc_hip_bias_add_nchw_f32: NULL pointer");
     hipStream_t s = ResolveStream(stream);
-    if (relu) bias_add_kernel<true><<<GridFor(total), kBlock, 0, s>>>(x, bias, y, o, hw, total);
-    else bias_add_kernel<false><<<GridFor(total), kBlock, 0, s>>>(x, bias, y, o, hw, total);
+    if (relu) bias_add_kernel<true><<<NoteGrid(GridFor(total)), NoteBlock(kBlock), NoteLds(0), s>>>(x, bias, y, o, hw, total);
+    else bias_add_kernel<false><<<NoteGrid(GridFor(total)), NoteBlock(kBlock), NoteLds(0), s>>>(x, bias, y, o, hw, total);
     return CheckLaunch("bias_add");
 }
 
@@ -262,7 +262,7 @@ int32_t kxc_hip_flatten_f32(const float* x, float* y, int64_t n, void* stream) {
                      "flatten copy");
         return KXC_HIP_OK;
     }
-    copy_kernel<<<GridFor(n4), kBlock, 0, s>>>(reinterpret_cast<const float4*>(x), reinterpret_cast<float4*>(y), n4,
+    copy_kernel<<<NoteGrid(GridFor(n4)), NoteBlock(kBlock), NoteLds(0), s>>>(reinterpret_cast<const float4*>(x), reinterpret_cast<float4*>(y), n4,
                                                 x, y, n);
     return CheckLaunch("flatten");
 }
@@ -272,7 +272,7 @@ int32_t kxc_hip_quantize_f32_i8(const float* x, int8_t* q, int64_t n, float scal
     if (n == 0) return KXC_HIP_OK;
     KXC_HIP_REQUIRE(x && q, "kxc_hip_quantize_f32_i8: NULL pointer");
     KXC_HIP_REQUIRE(scale > 0.0f, "kxc_hip_quantize_f32_i8: scale must be positive");
-    quantize_kernel<<<GridFor(n), kBlock, 0, ResolveStream(stream)>>>(x, q, n, scale);
+    quantize_kernel<<<NoteGrid(GridFor(n)), NoteBlock(kBlock), NoteLds(0), ResolveStream(stream)>>>(x, q, n, scale);
     return CheckLaunch("quantize");
 }
 
@@ -283,7 +283,7 @@ int32_t kxc_hip_absmax_f32(const float* x, int64_t n, float* out, void* stream) 
     KXC_HIP_CALL(hipMemsetAsync(out, 0, sizeof(float), s), "hipMemsetAsync");
     if (n == 0) return KXC_HIP_OK;
     KXC_HIP_REQUIRE(x != nullptr, "kxc_hip_absmax_f32: NULL pointer");
-    absmax_kernel<<<GridFor(n), kBlock, 0, s>>>(x, n, reinterpret_cast<unsigned int*>(out));
+    absmax_kernel<<<NoteGrid(GridFor(n)), NoteBlock(kBlock), NoteLds(0), s>>>(x, n, reinterpret_cast<unsigned int*>(out));
     return CheckLaunch("absmax");
 }
 

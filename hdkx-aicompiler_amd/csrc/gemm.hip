@@ -141,14 +141,14 @@ int32_t kxc_hip_gemm_f32(const float* a, const float* b, const float* c, float* 
     if (transB && k > 0 && (k % 32) == 0 && aligned && m < (1 << 20) && n < (1 << 20) && k < (1 << 30)) {
         dim3 grid(static_cast<unsigned>(CeilDiv(n, 32)), static_cast<unsigned>(CeilDiv(m, 32)));
         KXC_HIP_REQUIRE(grid.y <= 65535u, "kxc_hip_gemm_f32: m too large");
-        gemm_nt_mfma_kernel<<<grid, 256, 0, s>>>(a, b, c, y, static_cast<int32_t>(m), static_cast<int32_t>(n),
+        gemm_nt_mfma_kernel<<<NoteGrid(grid), NoteBlock(256), NoteLds(0), s>>>(a, b, c, y, static_cast<int32_t>(m), static_cast<int32_t>(n),
                                                   static_cast<int32_t>(k), alpha, beta, c_len, scale_a, scale_c);
         return CheckLaunch("gemm_nt_mfma");
     }
     int64_t g = CeilDiv(m * n, 256);
     if (g > 256 * 32) g = 256 * 32;
-    if (transB) gemm_direct_kernel<true><<<static_cast<int>(g), 256, 0, s>>>(a, b, c, y, m, n, k, alpha, beta, c_len, scale_a, scale_c);
-    else gemm_direct_kernel<false><<<static_cast<int>(g), 256, 0, s>>>(a, b, c, y, m, n, k, alpha, beta, c_len, scale_a, scale_c);
+    if (transB) gemm_direct_kernel<true><<<NoteGrid(static_cast<int>(g)), NoteBlock(256), NoteLds(0), s>>>(a, b, c, y, m, n, k, alpha, beta, c_len, scale_a, scale_c);
+    else gemm_direct_kernel<false><<<NoteGrid(static_cast<int>(g)), NoteBlock(256), NoteLds(0), s>>>(a, b, c, y, m, n, k, alpha, beta, c_len, scale_a, scale_c);
     return CheckLaunch("gemm_direct");
 }
 
@@ -160,7 +160,7 @@ int32_t kxc_hip_qdense_i8(const int8_t* a, const int8_t* b, const int32_t* bias,
     KXC_HIP_REQUIRE(k <= 2147483647LL / (128 * 128), "kxc_hip_qdense_i8: k too large for int32 accumulation");
     int64_t g = CeilDiv(m * n, 256);
     if (g > 256 * 32) g = 256 * 32;
-    qdense_kernel<<<static_cast<int>(g), 256, 0, ResolveStream(stream)>>>(a, b, bias, mult, y, m, n, k);
+    qdense_kernel<<<NoteGrid(static_cast<int>(g)), NoteBlock(256), NoteLds(0), ResolveStream(stream)>>>(a, b, bias, mult, y, m, n, k);
     return CheckLaunch("qdense");
 }
 

@@ -135,6 +135,9 @@ int32_t kxc_hip_module_launch(void* function, const uint32_t grid[3], const uint
                     "kxc_hip_module_launch: empty grid or block");
     KXC_HIP_REQUIRE(static_cast<uint64_t>(block[0]) * block[1] * block[2] <= 1024,
                     "kxc_hip_module_launch: more than 1024 threads per block");
+    NoteGrid(dim3(grid[0], grid[1], grid[2]));
+    NoteBlock(dim3(block[0], block[1], block[2]));
+    NoteLds(shared_bytes);
     KXC_HIP_CALL(hipModuleLaunchKernel(reinterpret_cast<hipFunction_t>(function), grid[0], grid[1], grid[2], block[0],
                                        block[1], block[2], shared_bytes, ResolveStream(stream), kernel_params, nullptr),
                  "hipModuleLaunchKernel");

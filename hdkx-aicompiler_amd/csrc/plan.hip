@@ -4,6 +4,7 @@
 // kernel_symbol as KernelExecNode would carry it (include/base/execution_plan.h:42-50).
 // Intermediates live in ONE workspace allocated at finalize time (the CPU backend mallocs and frees
 // every intermediate on every call, src/codegen/codegen_llvm.cc:578-623).
+#include <cstdio>
 #include <cstring>
 #include <string>
 #include <vector>
@@ -384,14 +385,22 @@ int32_t kxc_hip_plan_finalize(kxc_hip_plan* plan, size_t workspace_bytes) {
     return KXC_HIP_OK;
 }
 
-int32_t kxc_hip_plan_run(kxc_hip_plan* plan, void** args, void* stream) {
-    KXC_HIP_REQUIRE(plan != nullptr, "kxc_hip_plan_run: plan is NULL");
-    KXC_HIP_REQUIRE(plan->finalized, "kxc_hip_plan_run: plan is not finalized");
-    KXC_HIP_REQUIRE(plan->num_args == 0 || args != nullptr, "kxc_hip_plan_run: packed_args is NULL");
+}  // extern "C"
+
+namespace {
+
+int32_t CheckRunArgs(kxc_hip_plan* plan, void** args, const char* who) {
+    KXC_HIP_REQUIRE(plan != nullptr, "%s: plan is NULL", who);
+    KXC_HIP_REQUIRE(plan->finalized, "%s: plan is not finalized", who);
+    KXC_HIP_REQUIRE(plan->num_args == 0 || args != nullptr, "%s: packed_args is NULL", who);
     for (int i = 0; i < plan->num_args; ++i)
-        KXC_HIP_REQUIRE(args[i] != nullptr, "kxc_hip_plan_run: packed argument %d is NULL", i);
-    void* s = stream ? stream : static_cast<void*>(CurrentStream());
-    for (Node& n : plan->nodes) {
+        KXC_HIP_REQUIRE(args[i] != nullptr, "%s: packed argument %d is NULL", who, i);
+    return KXC_HIP_OK;
+}
+
+// Enqueues one node on stream s.
+int32_t RunNode(kxc_hip_plan* plan, Node& n, void** args, void* s) {
+    {
         int32_t rc = KXC_HIP_OK;
         auto B = [&](int i) { return Resolve(plan, n.bufs[i], args); };
         switch (n.kind) {
@@ -484,6 +493,67 @@ int32_t kxc_hip_plan_run(kxc_hip_plan* plan, void** args, void* stream) {
         }
     }
     return KXC_HIP_OK;
+}
+
+}  // namespace
+
+extern "C" {
+
+int32_t kxc_hip_plan_run(kxc_hip_plan* plan, void** args, void* stream) {
+    if (int32_t rc = CheckRunArgs(plan, args, "kxc_hip_plan_run")) return rc;
+    void* s = stream ? stream : static_cast<void*>(CurrentStream());
+    for (Node& n : plan->nodes)
+        if (int32_t rc = RunNode(plan, n, args, s)) return rc;
+    return KXC_HIP_OK;
+}
+
+int32_t kxc_hip_plan_run_profiled(kxc_hip_plan* plan, void** args, void* stream, kxc_hip_launch_record* records,
+                                  int32_t capacity, int32_t* count) {
+    const char* who = "kxc_hip_plan_run_profiled";
+    if (int32_t rc = CheckRunArgs(plan, args, who)) return rc;
+    KXC_HIP_REQUIRE(count != nullptr && (capacity == 0 || records != nullptr), "%s: NULL output", who);
+    const int32_t nodes = static_cast<int32_t>(plan->nodes.size());
+    *count = nodes;
+    KXC_HIP_REQUIRE(capacity >= nodes, "%s: %d records needed, room for %d", who, nodes, capacity);
+    void* s = stream ? stream : static_cast<void*>(CurrentStream());
+    hipStream_t hs = reinterpret_cast<hipStream_t>(s);
+    // one event before every node and one after the last: node i ran between events i and i+1
+    std::vector<hipEvent_t> ev(static_cast<size_t>(nodes) + 1, nullptr);
+    int32_t rc = KXC_HIP_OK;
+    for (auto& e : ev)
+        if (hipEventCreate(&e) != hipSuccess) { rc = Fail(KXC_HIP_ERR_RUNTIME, "%s: hipEventCreate failed", who); break; }
+    for (int32_t i = 0; rc == KXC_HIP_OK && i < nodes; ++i) {
+        Node& n = plan->nodes[i];
+        if (hipEventRecord(ev[i], hs) != hipSuccess) { rc = Fail(KXC_HIP_ERR_RUNTIME, "%s: hipEventRecord failed", who); break; }
+        LastLaunch() = LaunchNote();
+        rc = RunNode(plan, n, args, s);
+        if (rc != KXC_HIP_OK) break;
+        kxc_hip_launch_record& r = records[i];
+        std::memset(&r, 0, sizeof(r));
+        std::snprintf(r.kernel_symbol, sizeof(r.kernel_symbol), "%s", n.symbol.c_str());
+        r.kind = n.kind == NodeKind::kCopy ? KXC_HIP_RECORD_MEMCPY : KXC_HIP_RECORD_KERNEL;
+        const LaunchNote& note = LastLaunch();
+        for (int k = 0; k < 3; ++k) { r.grid[k] = note.grid[k]; r.block[k] = note.block[k]; }
+        r.dynamic_shared_memory = note.dynamic_lds;
+        if (n.kind == NodeKind::kCopy) r.bytes = n.dims[0];
+    }
+    if (rc == KXC_HIP_OK && hipEventRecord(ev[nodes], hs) != hipSuccess)
+        rc = Fail(KXC_HIP_ERR_RUNTIME, "%s: hipEventRecord failed", who);
+    if (rc == KXC_HIP_OK && hipEventSynchronize(ev[nodes]) != hipSuccess)
+        rc = Fail(KXC_HIP_ERR_RUNTIME, "%s: hipEventSynchronize failed", who);
+    for (int32_t i = 0; rc == KXC_HIP_OK && i < nodes; ++i) {
+        float start_ms = 0.0f, dur_ms = 0.0f;
+        if (hipEventElapsedTime(&start_ms, ev[0], ev[i]) != hipSuccess ||
+            hipEventElapsedTime(&dur_ms, ev[i], ev[i + 1]) != hipSuccess) {
+            rc = Fail(KXC_HIP_ERR_RUNTIME, "%s: hipEventElapsedTime failed", who);
+            break;
+        }
+        records[i].start_ns = static_cast<int64_t>(static_cast<double>(start_ms) * 1e6);
+        records[i].duration_ns = static_cast<int64_t>(static_cast<double>(dur_ms) * 1e6);
+    }
+    for (auto& e : ev)
+        if (e) (void)hipEventDestroy(e);
+    return rc;
 }
 
 int32_t kxc_hip_plan_num_nodes(const kxc_hip_plan* plan) { return plan ? static_cast<int32_t>(plan->nodes.size()) : 0; }

@@ -256,12 +256,12 @@ int32_t kxc_hip_pool2d_f32(const kxc_hip_pool2d_desc* desc, const float* x, floa
         const int64_t threads = planes * row_groups * col_groups;
         const int64_t blocks = CeilDiv(threads, kBlock);
         KXC_HIP_REQUIRE(blocks <= kMaxGridX, "kxc_hip_pool2d_f32: tensor too large");
-        maxpool3x3s2_kernel<kRows><<<static_cast<int>(blocks), kBlock, 0, s>>>(x, y, d.h, d.w, d.oh, d.ow, col_groups,
+        maxpool3x3s2_kernel<kRows><<<NoteGrid(static_cast<int>(blocks)), NoteBlock(kBlock), NoteLds(0), s>>>(x, y, d.h, d.w, d.oh, d.ow, col_groups,
                                                                                row_groups, threads);
         return CheckLaunch("maxpool3x3s2");
     }
-    if (desc->is_avg) pool_generic_kernel<true><<<GridFor(total), kBlock, 0, s>>>(x, y, d, total);
-    else pool_generic_kernel<false><<<GridFor(total), kBlock, 0, s>>>(x, y, d, total);
+    if (desc->is_avg) pool_generic_kernel<true><<<NoteGrid(GridFor(total)), NoteBlock(kBlock), NoteLds(0), s>>>(x, y, d, total);
+    else pool_generic_kernel<false><<<NoteGrid(GridFor(total)), NoteBlock(kBlock), NoteLds(0), s>>>(x, y, d, total);
     return CheckLaunch("pool2d");
 }
 
@@ -278,11 +278,11 @@ int32_t kxc_hip_global_avg_pool2d_f32(const float* x, float* y, int64_t n, int64
         const int64_t blocks = CeilDiv(planes, kGapPlanes);
         KXC_HIP_REQUIRE(blocks <= kMaxGridX, "kxc_hip_global_avg_pool2d_f32: tensor too large");
         const size_t lds = static_cast<size_t>(kGapPlanes) * hw_pad * sizeof(float);   // <= 33 KiB
-        gap_lds_kernel<<<static_cast<int>(blocks), kGapPlanes, lds, s>>>(x, y, planes, static_cast<int32_t>(hw), hw_pad);
+        gap_lds_kernel<<<NoteGrid(static_cast<int>(blocks)), NoteBlock(kGapPlanes), NoteLds(lds), s>>>(x, y, planes, static_cast<int32_t>(hw), hw_pad);
         return CheckLaunch("global_avg_pool2d");
     }
     KXC_HIP_REQUIRE(planes <= kMaxGridX, "kxc_hip_global_avg_pool2d_f32: tensor too large");
-    gap_wave_kernel<<<static_cast<int>(planes), 64, 0, s>>>(x, y, planes, hw);
+    gap_wave_kernel<<<NoteGrid(static_cast<int>(planes)), NoteBlock(64), NoteLds(0), s>>>(x, y, planes, hw);
     return CheckLaunch("global_avg_pool2d");
 }
 
@@ -293,7 +293,7 @@ int32_t kxc_hip_maxpool2d_i8(const kxc_hip_pool2d_desc* desc, const int8_t* x, i
     const int64_t total = static_cast<int64_t>(d.n) * d.c * d.oh * d.ow;
     if (total == 0) return KXC_HIP_OK;
     KXC_HIP_REQUIRE(x && y, "kxc_hip_maxpool2d_i8: NULL pointer");
-    maxpool_i8_kernel<<<GridFor(total), kBlock, 0, ResolveStream(stream)>>>(x, y, d, total);
+    maxpool_i8_kernel<<<NoteGrid(GridFor(total)), NoteBlock(kBlock), NoteLds(0), ResolveStream(stream)>>>(x, y, d, total);
     return CheckLaunch("maxpool2d_i8");
 }
 
@@ -304,7 +304,7 @@ int32_t kxc_hip_global_avg_pool2d_i8(const int8_t* x, int8_t* y, int64_t n, int6
     if (planes == 0) return KXC_HIP_OK;
     KXC_HIP_REQUIRE(x && y, "kxc_hip_global_avg_pool2d_i8: NULL pointer");
     KXC_HIP_REQUIRE(h * w <= 2147483647LL / 128, "kxc_hip_global_avg_pool2d_i8: plane too large for int32 sum");
-    gap_i8_kernel<<<static_cast<int>(CeilDiv(planes, kBlock)), kBlock, 0, ResolveStream(stream)>>>(
+    gap_i8_kernel<<<NoteGrid(static_cast<int>(CeilDiv(planes, kBlock))), NoteBlock(kBlock), NoteLds(0), ResolveStream(stream)>>>(
         x, y, planes, static_cast<int32_t>(h * w), mult);
     return CheckLaunch("global_avg_pool2d_i8");
 }

@@ -579,7 +579,7 @@ int32_t kxc_hip_qconv2d_c16_pack_weights(const kxc_hip_qconv2d_desc* d, const in
     p.nchunks = ((d->c + 15) / 16 + p.CBC - 1) / p.CBC;
     p.oblocks = d->o / 32;
     const int64_t slots = static_cast<int64_t>(bytes / 16);
-    pack_weights_kernel<<<static_cast<int>(CeilDiv(slots, kBlock)), kBlock, 0, ResolveStream(stream)>>>(p, slots);
+    pack_weights_kernel<<<NoteGrid(static_cast<int>(CeilDiv(slots, kBlock))), NoteBlock(kBlock), NoteLds(0), ResolveStream(stream)>>>(p, slots);
     return CheckLaunch("qconv2d_c16_pack_weights");
 }
 
@@ -605,7 +605,7 @@ int32_t kxc_hip_qconv2d_c16_i8(const kxc_hip_qconv2d_desc* d, const int8_t* x, c
                                          hipFuncAttributeMaxDynamicSharedMemorySize, static_cast<int>(L.lds_bytes)),
                      "hipFuncSetAttribute");
     }
-    hipLaunchKernelGGL(L.v->kernel, dim3(L.grid), dim3(64 * L.v->wp), L.lds_bytes, ResolveStream(stream), a);
+    hipLaunchKernelGGL(L.v->kernel, NoteGrid(dim3(L.grid)), NoteBlock(dim3(64 * L.v->wp)), NoteLds(L.lds_bytes), ResolveStream(stream), a);
     return CheckLaunch(L.v->name);
 }
 
@@ -615,7 +615,7 @@ int32_t kxc_hip_i8_nchw_to_c16(const int8_t* x, int8_t* y, int64_t n, int64_t c,
     if (total == 0) return KXC_HIP_OK;
     KXC_HIP_REQUIRE(x && y, "kxc_hip_i8_nchw_to_c16: NULL pointer");
     KXC_HIP_REQUIRE(CeilDiv(total, kBlock) <= kMaxGridX, "kxc_hip_i8_nchw_to_c16: tensor too large");
-    nchw_to_c16_kernel<<<static_cast<int>(CeilDiv(total, kBlock)), kBlock, 0, ResolveStream(stream)>>>(
+    nchw_to_c16_kernel<<<NoteGrid(static_cast<int>(CeilDiv(total, kBlock))), NoteBlock(kBlock), NoteLds(0), ResolveStream(stream)>>>(
         x, y, static_cast<int32_t>(c), static_cast<int32_t>(cb), hw, total);
     return CheckLaunch("i8_nchw_to_c16");
 }
@@ -626,7 +626,7 @@ int32_t kxc_hip_i8_c16_to_nchw(const int8_t* x, int8_t* y, int64_t n, int64_t c,
     if (total == 0) return KXC_HIP_OK;
     KXC_HIP_REQUIRE(x && y, "kxc_hip_i8_c16_to_nchw: NULL pointer");
     KXC_HIP_REQUIRE(CeilDiv(total, kBlock) <= kMaxGridX, "kxc_hip_i8_c16_to_nchw: tensor too large");
-    c16_to_nchw_kernel<<<static_cast<int>(CeilDiv(total, kBlock)), kBlock, 0, ResolveStream(stream)>>>(
+    c16_to_nchw_kernel<<<NoteGrid(static_cast<int>(CeilDiv(total, kBlock))), NoteBlock(kBlock), NoteLds(0), ResolveStream(stream)>>>(
         x, y, static_cast<int32_t>(c), static_cast<int32_t>(cb), hw, total);
     return CheckLaunch("i8_c16_to_nchw");
 }
@@ -639,7 +639,7 @@ int32_t kxc_hip_quantize_f32_nchw_to_c16_i8(const float* x, int8_t* y, int64_t n
     if (total == 0) return KXC_HIP_OK;
     KXC_HIP_REQUIRE(x && y, "kxc_hip_quantize_f32_nchw_to_c16_i8: NULL pointer");
     KXC_HIP_REQUIRE(CeilDiv(total, kBlock) <= kMaxGridX, "kxc_hip_quantize_f32_nchw_to_c16_i8: tensor too large");
-    quantize_to_c16_kernel<<<static_cast<int>(CeilDiv(total, kBlock)), kBlock, 0, ResolveStream(stream)>>>(
+    quantize_to_c16_kernel<<<NoteGrid(static_cast<int>(CeilDiv(total, kBlock))), NoteBlock(kBlock), NoteLds(0), ResolveStream(stream)>>>(
         x, y, static_cast<int32_t>(c), static_cast<int32_t>(cb), hw, total, scale);
     return CheckLaunch("quantize_f32_nchw_to_c16_i8");
 }
@@ -663,7 +663,7 @@ int32_t kxc_hip_maxpool2d_c16_i8(const kxc_hip_pool2d_desc* p, const int8_t* x, 
     if (total == 0) return KXC_HIP_OK;
     KXC_HIP_REQUIRE(x && y, "kxc_hip_maxpool2d_c16_i8: NULL pointer");
     KXC_HIP_REQUIRE(CeilDiv(total, kBlock) <= kMaxGridX, "kxc_hip_maxpool2d_c16_i8: tensor too large");
-    maxpool_c16_kernel<<<static_cast<int>(CeilDiv(total, kBlock)), kBlock, 0, ResolveStream(stream)>>>(x, y, d, total);
+    maxpool_c16_kernel<<<NoteGrid(static_cast<int>(CeilDiv(total, kBlock))), NoteBlock(kBlock), NoteLds(0), ResolveStream(stream)>>>(x, y, d, total);
     return CheckLaunch("maxpool2d_c16_i8");
 }
 
@@ -674,7 +674,7 @@ int32_t kxc_hip_global_avg_pool2d_c16_i8(const int8_t* x, int8_t* y, int64_t n, 
     const int64_t planes = n * ((c + 15) / 16);
     if (planes == 0) return KXC_HIP_OK;
     KXC_HIP_REQUIRE(x && y, "kxc_hip_global_avg_pool2d_c16_i8: NULL pointer");
-    gap_c16_kernel<<<static_cast<int>(CeilDiv(planes, kBlock)), kBlock, 0, ResolveStream(stream)>>>(
+    gap_c16_kernel<<<NoteGrid(static_cast<int>(CeilDiv(planes, kBlock))), NoteBlock(kBlock), NoteLds(0), ResolveStream(stream)>>>(
         x, y, planes, static_cast<int32_t>(h * w), mult);
     return CheckLaunch("global_avg_pool2d_c16_i8");
 }

@@ -100,7 +100,7 @@ int32_t kxc_hip_qconv2d_nchw_i8(const kxc_hip_qconv2d_desc* d, const int8_t* x, 
     a.x = x; a.w = w; a.bias = bias; a.mult = mult; a.res = residual; a.y = y;
     int64_t g = CeilDiv(total, 256);
     if (g > 256 * 64) g = 256 * 64;
-    qconv_direct_kernel<<<static_cast<int>(g), 256, 0, ResolveStream(stream)>>>(a, total);
+    qconv_direct_kernel<<<NoteGrid(static_cast<int>(g)), NoteBlock(256), NoteLds(0), ResolveStream(stream)>>>(a, total);
     return CheckLaunch("qconv_direct");
 }
 

@@ -1,5 +1,6 @@
 // compiler.cc -- Compiler::Compile and CompiledModule (see compiler.h).
 #include "kxc/compiler.h"
+#include "kxc/profiling.h"
 
 #include <dlfcn.h>
 #include <unistd.h>
@@ -447,7 +448,20 @@ CompiledModule Compiler::Compile(Function func, CompileConfig config) {
     if (!config.defined() || !config->target.defined()) throw std::runtime_error("Compiler::Compile: config has no target");
     auto impl = std::make_shared<CompiledModuleImpl>();
     impl->config = config;
-    Function typed = relay::InferTypePass(func);
+    profiling::EventSpec cspec;
+    cspec.component = "compiler";
+    cspec.event_type = "compile";
+    cspec.device = config->target->kind;
+    profiling::ScopedSpan compile_span = profiling::CurrentSpan(cspec);
+    Function typed;
+    {
+        profiling::EventSpec e;
+        e.component = "relay.transform";
+        e.event_type = "pass";
+        e.pass_name = "InferType";
+        profiling::ScopedSpan span = profiling::CurrentSpan(e);
+        typed = relay::InferTypePass(func);
+    }
     if (config->target->kind == "hip") {
         // the whole-function TIR is kept for inspection (GetPrimFunc) and fixes the parameter order
         relay::LoweredFunc whole = relay::LowerToTIRDetailed(typed);
@@ -455,14 +469,34 @@ CompiledModule Compiler::Compile(Function func, CompileConfig config) {
         impl->input_count = impl->prim_func->int_attrs.at("kxc.input_count");
         impl->constant_count = impl->prim_func->int_attrs.at("kxc.constant_count");
         const bool dry = config->target->attrs.exists == 0;
-        HipBuilder builder(typed, config, impl.get(), dry);
-        builder.Build();
+        {
+            profiling::EventSpec e;
+            e.component = "backend.hip";
+            e.event_type = "build_plan";
+            e.device = "hip:" + std::to_string(config->target->device.device_id());
+            profiling::ScopedSpan span = profiling::CurrentSpan(e);
+            HipBuilder builder(typed, config, impl.get(), dry);
+            builder.Build();
+            span.AddMetric("launches", static_cast<double>(impl->execs.size()));
+            span.AddMetric("workspace_bytes", static_cast<double>(impl->workspace_bytes));
+        }
         if (static_cast<int64_t>(impl->constants.size()) != impl->constant_count)
             throw std::runtime_error("hip back end: constant order disagrees with the lowering");
     } else {
+        profiling::EventSpec e;
+        e.component = "codegen";
+        e.event_type = "host_c_compile";
+        profiling::ScopedSpan span = profiling::CurrentSpan(e);
         CompileHost(typed, config, impl.get());
     }
-    return CompiledModule(impl);
+    CompiledModule module(impl);
+    if (auto ctx = profiling::CurrentContext()) {
+        if (ctx->options().enabled && ctx->options().record_execution_plan_details && config->target->kind == "hip")
+            ctx->WriteArtifact("execution_plan.json", module.ExecutionPlanJSON());
+        if (profiling::ShouldCaptureIR(ctx, true, false) && !impl->source.empty())
+            ctx->WriteArtifact(config->target->kind == "hip" ? "generated_kernels.hip" : "kernel_main.c", impl->source);
+    }
+    return module;
 }
 
 void CompiledModule::Run(const std::vector<void*>& packed_args) {
@@ -475,6 +509,44 @@ void CompiledModule::Run(const std::vector<void*>& packed_args) {
         const int32_t rc = impl_->fn(const_cast<void**>(packed_args.data()));
         if (rc != 0) throw std::runtime_error("Kernel kxc_kernel_main returned error code " + std::to_string(rc));
         return;
+    }
+    auto ctx = profiling::CurrentContext();
+    if (ctx && ctx->options().enabled && ctx->options().enable_gpu_activity) {
+        // One "runtime" span for the call, one "backend.hip" event per launch from the plan's HIP events.
+        profiling::EventSpec rspec;
+        rspec.component = "runtime";
+        rspec.event_type = "kernel_run";
+        rspec.kernel_symbol = "kxc_kernel_main";
+        const std::string device = "hip:" + std::to_string(impl_->config->target->device.device_id());
+        rspec.device = device;
+        profiling::ScopedSpan run_span(ctx, rspec);
+        std::vector<kxc_hip_launch_record> records(impl_->execs.size() + 8);
+        int32_t count = 0;
+        const std::int64_t t0 = ctx->NowNs();
+        if (kxc_hip_plan_run_profiled(impl_->plan, const_cast<void**>(packed_args.data()), nullptr, records.data(),
+                                      static_cast<int32_t>(records.size()), &count)) {
+            run_span.SetStatus("error");
+            throw std::runtime_error(std::string("Kernel kxc_kernel_main failed: ") + kxc_hip_last_error());
+        }
+        for (int32_t i = 0; i < count; ++i) {
+            const kxc_hip_launch_record& r = records[i];
+            profiling::EventSpec e;
+            e.component = "backend.hip";
+            e.event_type = r.kind == KXC_HIP_RECORD_MEMCPY ? "hip_memcpy" : "hip_kernel";
+            e.device = device;
+            e.kernel_symbol = r.kernel_symbol;
+            if (static_cast<size_t>(i) < impl_->execs.size()) e.op_name = impl_->execs[i].op_name;
+            e.fields["backend.hip.launch_index"] = std::to_string(i);
+            e.fields["backend.hip.timing_source"] = "hip_events";
+            e.metrics["grid_x"] = r.grid[0]; e.metrics["grid_y"] = r.grid[1]; e.metrics["grid_z"] = r.grid[2];
+            e.metrics["block_x"] = r.block[0]; e.metrics["block_y"] = r.block[1]; e.metrics["block_z"] = r.block[2];
+            e.metrics["dynamic_shared_memory"] = r.dynamic_shared_memory;
+            if (r.kind == KXC_HIP_RECORD_MEMCPY) e.metrics["bytes"] = static_cast<double>(r.bytes);
+            ctx->RecordCompletedSpan(e, profiling::CurrentRunId(), ctx->NextSpanId(), run_span.span_id(), t0 + r.start_ns,
+                                     t0 + r.start_ns + r.duration_ns);
+        }
+        run_span.AddMetric("launches", count);
+        return;     // the profiled run has already waited for the last launch
     }
     if (kxc_hip_plan_run(impl_->plan, const_cast<void**>(packed_args.data()), nullptr))
         throw std::runtime_error(std::string("Kernel kxc_kernel_main failed: ") + kxc_hip_last_error());

@@ -1,5 +1,6 @@
 // device_api.cc -- CPUDeviceAPI, HIPDeviceAPI (over the C ABI), device enumeration, BuildTarget.
 #include "kxc/device_api.h"
+#include "kxc/profiling.h"
 
 #include <cstdlib>
 #include <cstring>
@@ -53,6 +54,18 @@ public:
     std::string GetTargetKind(const Device&) const override { return "llvm"; }
 };
 
+// Every device call is a "device_api" span with its byte count, as in the reference's CUDA device API
+// (src/base/device/cuda_device_api.cc:90-157); without an active profiling context this is a no-op.
+profiling::ScopedSpan ApiSpan(const char* event_type, const Device& d, double bytes = -1.0) {
+    if (!profiling::CurrentContext()) return profiling::ScopedSpan();
+    profiling::EventSpec e;
+    e.component = "device_api";
+    e.event_type = event_type;
+    e.device = "hip:" + std::to_string(d.device_id());
+    if (bytes >= 0.0) e.metrics["bytes"] = bytes;
+    return profiling::CurrentSpan(e);
+}
+
 [[noreturn]] void ThrowHip(const char* what) {
     throw std::runtime_error(std::string("HIP ") + what + " failed: " + kxc_hip_last_error());
 }
@@ -65,10 +78,12 @@ public:
     }
     void* AllocDataSpace(const Device& d, size_t nbytes, size_t alignment) override {
         void* p = nullptr;
+        profiling::ScopedSpan span = ApiSpan("alloc_data_space", d, static_cast<double>(nbytes));
         if (kxc_hip_alloc(d.device_id(), nbytes, alignment, &p)) ThrowHip("AllocDataSpace");
         return p;
     }
     void FreeDataSpace(const Device& d, void* ptr) override {
+        profiling::ScopedSpan span = ApiSpan("free_data_space", d);
         if (kxc_hip_free(d.device_id(), ptr)) ThrowHip("FreeDataSpace");
     }
     void CopyDataFromTo(const Device& from_dev, const void* from_ptr, const Device& to_dev, void* to_ptr, size_t nbytes) override {
@@ -79,6 +94,8 @@ public:
         const bool fg = from_dev.device_type() == kGPU, tg = to_dev.device_type() == kGPU;
         const int kind = (!fg && tg) ? 0 : (fg && !tg) ? 1 : (fg && tg) ? 2 : 3;
         const int dev = tg ? to_dev.device_id() : from_dev.device_id();
+        profiling::ScopedSpan span = ApiSpan("copy_data_from_to", tg ? to_dev : from_dev, static_cast<double>(nbytes));
+        span.AddField("device_api.copy_kind", kind == 0 ? "host_to_device" : kind == 1 ? "device_to_host" : kind == 2 ? "device_to_device" : "host_to_host");
         if (kxc_hip_copy(from_ptr, from_offset, to_ptr, to_offset, nbytes, kind, dev, stream)) ThrowHip("CopyDataFromTo");
     }
     DeviceAttributes GetDeviceAttributes(const Device& d) override {
@@ -125,6 +142,7 @@ public:
         return s;
     }
     void StreamSync(const Device& d, StreamHandle s) override {
+        profiling::ScopedSpan span = ApiSpan("stream_sync", d);
         if (kxc_hip_stream_sync(d.device_id(), s)) ThrowHip("StreamSync");
     }
     void SyncStreamFromTo(const Device& d, StreamHandle src, StreamHandle dst) override {

@@ -18,6 +18,7 @@
 
 #include "kxc/compiler.h"
 #include "kxc/models.h"
+#include "kxc/profiling.h"
 #include "kxc/topi.h"
 
 namespace {
@@ -432,12 +433,37 @@ int RunCodegen() {
 
 }  // namespace
 
+// profile <cpu|hip|hipgen> <bundle dir>: the CNN known-answer model under an active profiling context; the
+// bundle lands in <bundle dir> (the Python tests read it back).
+int RunProfile(const std::string& dir) {
+    kxc::profiling::ProfileOptions options;
+    options.enabled = true;
+    options.bundle_dir = dir;
+    options.ir_capture_mode = kxc::profiling::IRCaptureMode::kVerbose;
+    options = kxc::profiling::ApplyEnvironmentOverrides(options);
+    auto ctx = kxc::profiling::ProfileContext::Create(options);
+    {
+        kxc::profiling::ActivationScope scope(ctx, ctx->NextRunId("host_tests"));
+        kxc::profiling::EventSpec spec;
+        spec.component = "test";
+        spec.event_type = "model_cnn";
+        kxc::profiling::ScopedSpan span(ctx, spec);
+        TestModelCNN();
+        ctx->RecordLog(kxc::profiling::LogSeverity::kInfo, "test", "model_cnn passed",
+                       kxc::profiling::MakeFields({{"mode", g_mode}}));
+    }
+    ctx->Flush();
+    std::cout << "profile bundle: " << ctx->bundle_dir() << " events=" << ctx->event_count() << "\n";
+    return 0;
+}
+
 int main(int argc, char** argv) {
     try {
         const std::string cmd = argc > 1 ? argv[1] : "";
         if (cmd == "op_numeric") { g_mode = argc > 2 ? argv[2] : "cpu"; return RunOpNumeric(); }
         if (cmd == "device_info") return RunDeviceInfo();
         if (cmd == "codegen") return RunCodegen();
+        if (cmd == "profile" && argc >= 4) { g_mode = argv[2]; return RunProfile(argv[3]); }
         if (cmd == "resnet18" && argc >= 6) { g_mode = argv[2]; return RunResNet18(argv[3], std::atoll(argv[4]), std::atoll(argv[5])); }
         std::cerr << "usage: host_tests op_numeric <cpu|hip|hipgen> | device_info | codegen | resnet18 <cpu|hip|hipgen> <dir> <batch> <hw>\n";
         return 2;

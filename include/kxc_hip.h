@@ -289,6 +289,23 @@ int32_t kxc_hip_plan_add_module_kernel(kxc_hip_plan* plan, void* function, const
 int32_t kxc_hip_plan_finalize(kxc_hip_plan* plan, size_t workspace_bytes);
 /* Enqueue every node on `stream`; returns after enqueue (no synchronisation). */
 int32_t kxc_hip_plan_run(kxc_hip_plan* plan, void** packed_args, void* stream);
+/* The same run with a HIP event between consecutive launches: fills one record per plan node (kernel symbol,
+ * launch geometry, start relative to the first launch, duration) and returns after the last launch has
+ * finished.  The records carry what the reference's profiler adapter puts into a "cuda_kernel" event
+ * (src/base/profiling.cc:623-651: grid_x..block_z, dynamic_shared_memory, start, end); the host layer turns
+ * them into component "backend.hip" events.  *count = number of nodes; fails if capacity is smaller. */
+#define KXC_HIP_RECORD_KERNEL 0
+#define KXC_HIP_RECORD_MEMCPY 1
+typedef struct kxc_hip_launch_record {
+    char kernel_symbol[120];
+    int32_t kind;                    /* KXC_HIP_RECORD_* */
+    uint32_t grid[3], block[3];
+    uint32_t dynamic_shared_memory;
+    int64_t bytes;                   /* copies only */
+    int64_t start_ns, duration_ns;
+} kxc_hip_launch_record;
+int32_t kxc_hip_plan_run_profiled(kxc_hip_plan* plan, void** packed_args, void* stream,
+                                  kxc_hip_launch_record* records, int32_t capacity, int32_t* count);
 int32_t kxc_hip_plan_num_nodes(const kxc_hip_plan* plan);
 /* kernel_symbol of node i (static storage owned by the plan). */
 const char* kxc_hip_plan_node_symbol(const kxc_hip_plan* plan, int32_t i);

@@ -116,3 +116,65 @@ def test_resnet18_generated_kernels_equal_oracle_bit_for_bit(synth):
         got = np.fromfile(os.path.join(d, "logits.bin"), np.float32).reshape(1, 1000)
     want = Oracle(fast=True).resnet18(x, consts)
     assert np.array_equal(bits(got), bits(want))
+
+
+# ------------------------------------------------------------------ profiling bundle
+EVENT_KEYS = ("trace_id", "session_id", "run_id", "span_id", "parent_span_id", "component", "event_type", "phase",
+              "ts_ns", "duration_ns", "status", "severity", "device", "worker_id", "op_name", "pass_name",
+              "kernel_symbol", "shape_signature", "message", "fields", "metrics")
+
+
+def _read_bundle(d):
+    for name in ("manifest.json", "events.jsonl", "trace.json", "summary.json", "diagnosis.json", "diagnosis.md"):
+        assert os.path.exists(os.path.join(d, name)), name
+    events = [json.loads(line) for line in open(os.path.join(d, "events.jsonl")) if line.strip()]
+    manifest = json.load(open(os.path.join(d, "manifest.json")))
+    trace = json.load(open(os.path.join(d, "trace.json")))
+    summary = json.load(open(os.path.join(d, "summary.json")))
+    assert manifest["schema_version"] == 1 and manifest["event_count"] == len(events) == summary["event_count"]
+    assert len(trace["traceEvents"]) == len(events)
+    for e in events:
+        # the stable event fields of the reference's bundle (src/base/profiling.cc:740-771)
+        assert tuple(e.keys()) == EVENT_KEYS
+        assert e["fields"]["schema_version"] == "1" and e["duration_ns"] >= 0
+    return events, manifest, summary
+
+
+def test_profiling_bundle_cpu_target():
+    with tempfile.TemporaryDirectory() as d:
+        run("profile", "cpu", d)
+        events, manifest, summary = _read_bundle(d)
+        comps = {e["component"] for e in events}
+        assert {"compiler", "relay.transform", "codegen", "test"} <= comps
+        spans = {e["span_id"]: e for e in events}
+        infer = [e for e in events if e["pass_name"] == "InferType"][0]
+        assert spans[infer["parent_span_id"]]["event_type"] == "compile"       # nesting follows the call stack
+        assert os.path.exists(os.path.join(d, "artifacts", "kernel_main.c"))
+
+
+@pytest.mark.gpu
+def test_profiling_bundle_hip_events():
+    """A profiled Run yields one backend.hip event per launch with the kernel symbol and the launch geometry the
+    reference's adapter records for CUDA kernels (grid_x..block_z, dynamic_shared_memory), device_api spans
+    with byte counts, and the execution plan as an artifact."""
+    with tempfile.TemporaryDirectory() as d:
+        run("profile", "hip", d)
+        events, manifest, summary = _read_bundle(d)
+        assert manifest["gpu_activity_source"] == "hip_events"
+        kernels = [e for e in events if e["component"] == "backend.hip" and e["event_type"] == "hip_kernel"]
+        plan = json.load(open(os.path.join(d, "artifacts", "execution_plan.json")))
+        assert len(kernels) == len(plan["nodes"]) >= 3
+        run_span = [e for e in events if e["component"] == "runtime" and e["event_type"] == "kernel_run"][0]
+        for k, node in zip(kernels, plan["nodes"]):
+            assert k["kernel_symbol"] == node["kernel_symbol"] and k["kernel_symbol"]
+            assert k["parent_span_id"] == run_span["span_id"] and k["device"] == "hip:0"
+            m = k["metrics"]
+            assert m["grid_x"] >= 1 and m["block_x"] >= 64 and m["grid_y"] == m["grid_z"] == m["block_y"] == m["block_z"] == 1
+            assert "dynamic_shared_memory" in m and k["duration_ns"] > 0
+        assert any(k["kernel_symbol"].startswith("mfma_") or k["kernel_symbol"] == "direct" or "conv" in k["kernel_symbol"]
+                   for k in kernels)
+        starts = [k["ts_ns"] for k in kernels]
+        assert starts == sorted(starts)
+        copies = [e for e in events if e["component"] == "device_api" and e["event_type"] == "copy_data_from_to"]
+        assert copies and all(c["metrics"]["bytes"] > 0 for c in copies)
+        assert summary["component_counts"]["backend.hip"] >= len(kernels)
