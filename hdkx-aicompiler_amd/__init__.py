@@ -11,7 +11,7 @@ from . import synth  # noqa: F401
 from .hipabi import (  # noqa: F401
     KxcHipError, lib, library_path, conv2d, relu, binary, bias_add, pool2d, global_avg_pool2d, gemm,
     flatten, quantize, qconv2d, qdense, maxpool2d_i8, global_avg_pool2d_i8, conv2d_variant,
-    absmax, i8_nchw_to_c16, i8_c16_to_nchw, quantize_to_c16, qconv_desc, qconv2d_c16_variant, qconv2d_c16_pack_weights,
+    absmax, quantize_to_c4, qconv2d_c4_pack_weights, qconv2d_c4, i8_nchw_to_c16, i8_c16_to_nchw, quantize_to_c16, qconv_desc, qconv2d_c16_variant, qconv2d_c16_pack_weights,
     qconv2d_c16, maxpool2d_c16_i8, global_avg_pool2d_c16_i8, c16_shape, pool_desc, pool_out_shape,
     device_attributes, Plan, Buf, ConvDesc, PoolDesc, QConvDesc,
     CONV_BIAS, CONV_RESIDUAL, CONV_RELU, CONV_FORCE_DIRECT,

@@ -307,6 +307,32 @@ int32_t kxc_hip_plan_add_qconv2d_c16(kxc_hip_plan* plan, const kxc_hip_qconv2d_d
     return KXC_HIP_OK;
 }
 
+int32_t kxc_hip_plan_add_qconv2d_c4(kxc_hip_plan* plan, const kxc_hip_qconv2d_desc* desc, kxc_hip_buf x_c4,
+                                    kxc_hip_buf w_packed, kxc_hip_buf bias, kxc_hip_buf mult, kxc_hip_buf y_c16) {
+    const char* who = "kxc_hip_plan_add_qconv2d_c4";
+    KXC_HIP_REQUIRE(desc != nullptr, "%s: desc is NULL", who);
+    KXC_HIP_REQUIRE(!(desc->flags & KXC_HIP_CONV_RESIDUAL), "%s: no residual operand on the first layer", who);
+    size_t bytes = 0;
+    if (int32_t rc = kxc_hip_qconv2d_c4_packed_bytes(desc, &bytes)) return rc;
+    kxc_hip_buf none;
+    none.kind = KXC_HIP_BUF_NONE; none.index_or_offset = 0;
+    if (int32_t rc = kxc_hip_plan_add_qconv2d(plan, desc, x_c4, w_packed, bias, mult, none, y_c16)) return rc;
+    Node& n = plan->nodes.back();
+    n.i32[0] = 2;
+    n.symbol = "kxc_qconv2d_c4_i8:qmfma_k7x7s2_c4";
+    return KXC_HIP_OK;
+}
+
+int32_t kxc_hip_plan_add_quantize_c4(kxc_hip_plan* plan, int64_t nn, int64_t c, int64_t hw, float scale, kxc_hip_buf x,
+                                     kxc_hip_buf q) {
+    if (int32_t rc = kxc_hip_plan_add_quantize(plan, nn, scale, x, q)) return rc;
+    Node& n = plan->nodes.back();
+    n.dims[0] = nn; n.dims[1] = c; n.dims[2] = hw;
+    n.i32[0] = 2;
+    n.symbol = "kxc_quantize_f32_nchw_to_c4_i8";
+    return KXC_HIP_OK;
+}
+
 int32_t kxc_hip_plan_add_quantize_c16(kxc_hip_plan* plan, int64_t nn, int64_t c, int64_t hw, float scale, kxc_hip_buf x,
                                       kxc_hip_buf q) {
     if (int32_t rc = kxc_hip_plan_add_quantize(plan, nn, scale, x, q)) return rc;
@@ -436,6 +462,12 @@ int32_t RunNode(kxc_hip_plan* plan, Node& n, void** args, void* s) {
                 break;
             }
             case NodeKind::kQConv2D:
+                if (n.i32[0] == 2) {
+                    rc = kxc_hip_qconv2d_c4_i8(&n.qconv, static_cast<const int8_t*>(B(0)), static_cast<const int8_t*>(B(1)),
+                                               static_cast<const int32_t*>(B(2)), static_cast<const float*>(B(3)),
+                                               static_cast<int8_t*>(B(5)), s);
+                    break;
+                }
                 if (n.i32[0] == 1) {
                     rc = kxc_hip_qconv2d_c16_i8(&n.qconv, static_cast<const int8_t*>(B(0)), static_cast<const int8_t*>(B(1)),
                                                 static_cast<const int32_t*>(B(2)), static_cast<const float*>(B(3)),
@@ -447,6 +479,11 @@ int32_t RunNode(kxc_hip_plan* plan, Node& n, void** args, void* s) {
                                              static_cast<const int8_t*>(B(4)), static_cast<int8_t*>(B(5)), s);
                 break;
             case NodeKind::kQuantize:
+                if (n.i32[0] == 2) {
+                    rc = kxc_hip_quantize_f32_nchw_to_c4_i8(static_cast<const float*>(B(0)), static_cast<int8_t*>(B(1)),
+                                                            n.dims[0], n.dims[1], n.dims[2], n.f[0], s);
+                    break;
+                }
                 if (n.i32[0] == 1) {
                     rc = kxc_hip_quantize_f32_nchw_to_c16_i8(static_cast<const float*>(B(0)), static_cast<int8_t*>(B(1)),
                                                              n.dims[0], n.dims[1], n.dims[2], n.f[0], s);

@@ -81,6 +81,42 @@ struct QArgs {
     uint32_t flags;
 };
 
+// Epilogue shared by the matrix-core kernels.  Accumulator register g of a 32x32 block is output channel
+// 8*(g/4) + 4*half + g%4 (within the block of 32) at the lane's pixel: registers 4j..4j+3 are four
+// consecutive channels = one dword of the pixel's c16 word.  ypix = n*(O/16)*OHW + pixel index.
+template <int RO>
+__device__ __forceinline__ void epilogue_c16(const intx16 (&acc)[RO], const QArgs& a, int ypix, int ob0, int half) {
+    const bool has_bias = (a.flags & KXC_HIP_CONV_BIAS) != 0;
+    const bool has_res = (a.flags & KXC_HIP_CONV_RESIDUAL) != 0;
+    const bool do_relu = (a.flags & KXC_HIP_CONV_RELU) != 0;
+#pragma unroll
+    for (int i = 0; i < RO; ++i) {
+        const int obase = (ob0 + i) * 32;
+        if (obase >= a.O) continue;
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+            const int o = obase + 8 * j + 4 * half;                 // first of 4 consecutive channels
+            if (o >= a.O) continue;
+            const int64_t off = (static_cast<int64_t>(ypix) + static_cast<int64_t>(o >> 4) * a.OHW) * 16 + (o & 15);
+            uint32_t resw = 0;
+            if (has_res) resw = *reinterpret_cast<const uint32_t*>(a.res + off);
+            const float4 mv = *reinterpret_cast<const float4*>(a.mult + o);
+            int4 bv = make_int4(0, 0, 0, 0);
+            if (has_bias) bv = *reinterpret_cast<const int4*>(a.bias + o);
+            const float ms[4] = {mv.x, mv.y, mv.z, mv.w};
+            const int bs[4] = {bv.x, bv.y, bv.z, bv.w};
+            uint32_t outw = 0;
+#pragma unroll
+            for (int e = 0; e < 4; ++e) {
+                const int32_t rq = static_cast<int32_t>(static_cast<int8_t>((resw >> (8 * e)) & 0xff));
+                const int32_t q = requant_i32(acc[i][4 * j + e] + bs[e], ms[e], has_res, rq, a.res_mult, do_relu);
+                outw |= (static_cast<uint32_t>(q) & 0xffu) << (8 * e);
+            }
+            *reinterpret_cast<uint32_t*>(a.y + off) = outw;
+        }
+    }
+}
+
 template <int KH, int KW, int CBC, int WP, int RO, int PPT>
 __global__ void __launch_bounds__(64 * WP) qconv_mfma_kernel(const QArgs a) {
     constexpr int KHW = KH * KW;
@@ -138,14 +174,12 @@ __global__ void __launch_bounds__(64 * WP) qconv_mfma_kernel(const QArgs a) {
     const int m = m0 + wave * 32 + r;
     int xbase;
     int ypix;            // position index (n*OB16*OHW + pixel) of this lane's output pixel for block 0, or -1
-    int ostride;         // positions between consecutive 16-channel output blocks
     {
         const int mc = min(m, a.M - 1);
         const int n = mc / a.OHW, rem = mc - n * a.OHW;
         const int oh = rem / a.OW, ow = rem - oh * a.OW;
         xbase = ((n * a.Hp + oh * a.sh - qmin) * a.Wp + ow * a.sw) * 16;
         if (CBC > 1) xbase += half * a.chs * 16;
-        ostride = a.OHW;
         ypix = (m < a.M) ? n * (a.O >> 4) * a.OHW + rem : -1;
     }
 
@@ -231,40 +265,145 @@ __global__ void __launch_bounds__(64 * WP) qconv_mfma_kernel(const QArgs a) {
         __syncthreads();
     }
 
-    // ---- epilogue.  Accumulator register g of a block is output channel 8*(g/4) + 4*half + g%4 (within
-    // the block of 32) at pixel r: registers 4j..4j+3 are four consecutive channels = one dword of the c16
-    // word of this pixel.
     if (ypix < 0) return;
-    const bool has_bias = (a.flags & KXC_HIP_CONV_BIAS) != 0;
-    const bool has_res = (a.flags & KXC_HIP_CONV_RESIDUAL) != 0;
-    const bool do_relu = (a.flags & KXC_HIP_CONV_RELU) != 0;
+    epilogue_c16<RO>(acc, a, ypix, ob0, half);
+}
+
+// ------------------------------------------------------------------------------------------------
+// First layer: 7x7, stride 2, padding 3, at most 4 input channels, on the "c4" input layout
+// [N][H][W][4] (4 bytes per pixel, channels >= C zero).  A 16-byte k-slice is four horizontally adjacent
+// pixels x 4 channels, so a k-step (32 values) is ONE filter row: lane half h covers the taps
+// kw = 4h-1 .. 4h+2 (the window is widened by one tap on the left, with zero weight, so that it starts on
+// an 8-byte boundary).  7 k-steps per 32x32 block instead of the 25 that padding 3 channels to a 16-channel
+// block costs, and a quarter of the input bytes.  LDS rows hold [4 zero pixels][W pixels][4 zero pixels]
+// as 16-byte positions; a tile's rows are loaded once (single chunk).  Output is c16.
+template <int WP, int RO, int PPT>
+__global__ void __launch_bounds__(64 * WP) qconv_k7s2_c4_kernel(const QArgs a) {
+    constexpr int KH = 7;
+    constexpr int TP = 32 * WP;
+    constexpr int WSEG = RO * KH;
+    constexpr int WPT = (WSEG + WP - 1) / WP;
+    extern __shared__ __attribute__((aligned(16))) char lds[];
+    const int tid = threadIdx.x;
+    const int lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int half = lane >> 5;
+    const int r = lane & 31;
+    const int W4 = (a.W >> 2) + 2;                  // 16-byte positions per LDS row
+    const int xs_bytes = a.chs * 16;
+
+    const int tile = (blockIdx.x & 7) * a.tiles_per_xcd + (blockIdx.x >> 3);
+    if (tile >= a.num_tiles || static_cast<int>(blockIdx.x >> 3) >= a.tiles_per_xcd) return;
+    const int p_tile = tile / a.o_tiles, o_tile = tile - p_tile * a.o_tiles;
+    const int m0 = p_tile * TP;
+    const int ob0 = o_tile * RO;
+    const int m_last = min(m0 + TP, a.M) - 1;
+    int qmin, qlast;
+    {
+        const int n = m0 / a.OHW, rem = m0 - n * a.OHW;
+        qmin = n * a.Hp + (rem / a.OW) * 2;
+        const int n2 = m_last / a.OHW, rem2 = m_last - n2 * a.OHW;
+        qlast = n2 * a.Hp + (rem2 / a.OW) * 2 + (KH - 1);
+    }
+    const int P = (qlast - qmin + 1) * W4;
+    const int xsegs = (P + 63) >> 6;
+    const __amdgpu_buffer_rsrc_t xr = make_rsrc(a.x, a.x_bytes);
+    const __amdgpu_buffer_rsrc_t wr = make_rsrc(a.wp, a.w_bytes);
 #pragma unroll
-    for (int i = 0; i < RO; ++i) {
-        const int obase = (ob0 + i) * 32;
-        if (obase >= a.O) continue;
-#pragma unroll
-        for (int j = 0; j < 4; ++j) {
-            const int o = obase + 8 * j + 4 * half;                 // first of 4 consecutive channels
-            if (o >= a.O) continue;
-            // byte offset of channels o..o+3 of this pixel
-            const int64_t off = (static_cast<int64_t>(ypix) + static_cast<int64_t>(o >> 4) * ostride) * 16 + (o & 15);
-            uint32_t resw = 0;
-            if (has_res) resw = *reinterpret_cast<const uint32_t*>(a.res + off);
-            const float4 mv = *reinterpret_cast<const float4*>(a.mult + o);
-            int4 bv = make_int4(0, 0, 0, 0);
-            if (has_bias) bv = *reinterpret_cast<const int4*>(a.bias + o);
-            const float ms[4] = {mv.x, mv.y, mv.z, mv.w};
-            const int bs[4] = {bv.x, bv.y, bv.z, bv.w};
-            uint32_t outw = 0;
-#pragma unroll
-            for (int e = 0; e < 4; ++e) {
-                const int32_t rq = static_cast<int32_t>(static_cast<int8_t>((resw >> (8 * e)) & 0xff));
-                const int32_t q = requant_i32(acc[i][4 * j + e] + bs[e], ms[e], has_res, rq, a.res_mult, do_relu);
-                outw |= (static_cast<uint32_t>(q) & 0xffu) << (8 * e);
-            }
-            *reinterpret_cast<uint32_t*>(a.y + off) = outw;
+    for (int i = 0; i < PPT; ++i) {
+        const int seg = wave + i * WP;
+        if (seg < xsegs) {
+            const int pos = seg * 64 + lane;
+            const int q = pos / W4, c4 = pos - q * W4;
+            const int Q = qmin + q;
+            const int n = Q / a.Hp, ih = Q - n * a.Hp - 3;
+            const bool ok = pos < P && n < a.N && ih >= 0 && ih < a.H && c4 >= 1 && c4 <= (a.W >> 2);
+            const uint32_t off = ok ? static_cast<uint32_t>((n * a.H + ih) * a.W + (c4 - 1) * 4) * 4u : kOob;
+            load16_to_lds(xr, (lds_ptr_t)(lds + seg * 1024), off, 0);
         }
     }
+#pragma unroll
+    for (int i = 0; i < WPT; ++i) {
+        const int seg = wave + i * WP;
+        if (seg < WSEG) {
+            const int ro = seg / KH, st = seg - ro * KH;
+            load16_to_lds(wr, (lds_ptr_t)(lds + xs_bytes + seg * 1024), static_cast<uint32_t>(lane) * 16u,
+                          (static_cast<uint32_t>(ob0 + ro) * KH + st) * 1024u);
+        }
+    }
+    const int m = m0 + wave * 32 + r;
+    int xbase, ypix;
+    {
+        const int mc = min(m, a.M - 1);
+        const int n = mc / a.OHW, rem = mc - n * a.OHW;
+        const int oh = rem / a.OW, ow = rem - oh * a.OW;
+        xbase = (n * a.Hp + oh * 2 - qmin) * W4 * 16 + ow * 8 + half * 16;
+        ypix = (m < a.M) ? n * (a.O >> 4) * a.OHW + rem : -1;
+    }
+    intx16 acc[RO];
+#pragma unroll
+    for (int i = 0; i < RO; ++i)
+#pragma unroll
+        for (int g = 0; g < 16; ++g) acc[i][g] = 0;
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+    __syncthreads();
+    const char* ws = lds + xs_bytes + lane * 16;
+#pragma unroll
+    for (int kh = 0; kh < KH; ++kh) {
+        const int2 lo = *reinterpret_cast<const int2*>(lds + xbase + kh * W4 * 16);        // 8-byte aligned
+        const int2 hi = *reinterpret_cast<const int2*>(lds + xbase + kh * W4 * 16 + 8);
+        intx4 b;
+        b[0] = lo.x; b[1] = lo.y; b[2] = hi.x; b[3] = hi.y;
+#pragma unroll
+        for (int i = 0; i < RO; ++i) {
+            const intx4 wv = *reinterpret_cast<const intx4*>(ws + (i * KH + kh) * 1024);
+            acc[i] = __builtin_amdgcn_mfma_i32_32x32x32_i8(wv, b, acc[i], 0, 0, 0);
+        }
+    }
+    if (ypix < 0) return;
+    epilogue_c16<RO>(acc, a, ypix, ob0, half);
+}
+
+// Weights of the first-layer kernel: [o block][kh][lane][16]; lane (o, half), byte j = pixel j/4, channel j%4,
+// tap kw = 4*half + j/4 - 1.
+__global__ void __launch_bounds__(kBlock) pack_weights_k7_c4_kernel(const int8_t* __restrict__ w, int8_t* __restrict__ wp,
+                                                                    int32_t O, int32_t C, int64_t total_slots) {
+    const int64_t s = static_cast<int64_t>(blockIdx.x) * kBlock + threadIdx.x;
+    if (s >= total_slots) return;
+    const int lane = static_cast<int>(s & 63);
+    const int64_t t = s >> 6;
+    const int kh = static_cast<int>(t % 7);
+    const int ob = static_cast<int>(t / 7);
+    const int o = ob * 32 + (lane & 31), h = lane >> 5;
+    int8_t out[16];
+#pragma unroll
+    for (int j = 0; j < 16; ++j) {
+        const int kw = 4 * h + (j >> 2) - 1, c = j & 3;
+        out[j] = (kw >= 0 && kw < 7 && c < C && o < O) ? w[((static_cast<int64_t>(o) * C + c) * 7 + kh) * 7 + kw] : 0;
+    }
+    *reinterpret_cast<int4*>(wp + s * 16) = *reinterpret_cast<const int4*>(out);
+}
+
+// fp32 NCHW -> int8 c4 ([N][H][W][4]); one thread per pixel.
+__global__ void __launch_bounds__(kBlock) quantize_to_c4_kernel(const float* __restrict__ x, int8_t* __restrict__ y,
+                                                                int32_t C, int64_t HW, int64_t total, float scale) {
+    const int64_t s = static_cast<int64_t>(blockIdx.x) * kBlock + threadIdx.x;
+    if (s >= total) return;
+    const int64_t p = s % HW, n = s / HW;
+    uint32_t word = 0;
+#pragma unroll
+    for (int c = 0; c < 4; ++c) {
+        int32_t q = 0;
+        if (c < C) {
+            const float v = __fdiv_rn(x[(n * C + c) * HW + p], scale);
+            float rr = rintf(v);
+            rr = (v == v) ? rr : 0.0f;
+            rr = fminf(fmaxf(rr, -127.0f), 127.0f);
+            q = static_cast<int32_t>(rr);
+        }
+        word |= (static_cast<uint32_t>(q) & 0xffu) << (8 * c);
+    }
+    reinterpret_cast<uint32_t*>(y)[s] = word;
 }
 
 // ------------------------------------------------------------------ weight packing
@@ -677,6 +816,124 @@ int32_t kxc_hip_global_avg_pool2d_c16_i8(const int8_t* x, int8_t* y, int64_t n, 
     gap_c16_kernel<<<NoteGrid(static_cast<int>(CeilDiv(planes, kBlock))), NoteBlock(kBlock), NoteLds(0), ResolveStream(stream)>>>(
         x, y, planes, static_cast<int32_t>(h * w), mult);
     return CheckLaunch("global_avg_pool2d_c16_i8");
+}
+
+}  // extern "C"
+
+// ---- first layer on the c4 layout
+namespace {
+
+struct K7Variant { const char* name; int wp, ro, ppt; void (*kernel)(const QArgs); };
+const K7Variant kK7Variants[] = {
+    {"qmfma_k7x7s2_c4_p4_o2", 4, 2, 4, qconv_k7s2_c4_kernel<4, 2, 4>},
+    {"qmfma_k7x7s2_c4_p4_o1", 4, 1, 4, qconv_k7s2_c4_kernel<4, 1, 4>},
+    {"qmfma_k7x7s2_c4_p2_o1", 2, 1, 8, qconv_k7s2_c4_kernel<2, 1, 8>},
+};
+
+int32_t PrepareK7(const kxc_hip_qconv2d_desc* d, QLaunch* L, const K7Variant** out, const char* who) {
+    KXC_HIP_REQUIRE(d != nullptr, "%s: desc is NULL", who);
+    KXC_HIP_REQUIRE(d->kh == 7 && d->kw == 7 && d->stride_h == 2 && d->stride_w == 2 && d->pad_h == 3 && d->pad_w == 3,
+                    "%s: only a 7x7 filter with stride 2 and padding 3 runs on the c4 layout", who);
+    KXC_HIP_REQUIRE(d->c >= 1 && d->c <= 4, "%s: at most 4 input channels (got %d)", who, d->c);
+    KXC_HIP_REQUIRE(d->n >= 0 && d->h >= 1 && d->w >= 4 && d->w % 4 == 0, "%s: width must be a positive multiple of 4", who);
+    KXC_HIP_REQUIRE(d->o > 0 && d->o % 32 == 0, "%s: output channels must be a multiple of 32 (got %d)", who, d->o);
+    KXC_HIP_REQUIRE(!(d->flags & KXC_HIP_CONV_RESIDUAL), "%s: no residual operand on the first layer", who);
+    QArgs& a = L->args;
+    std::memset(&a, 0, sizeof(a));
+    a.N = d->n; a.CB = 1; a.H = d->h; a.W = d->w; a.O = d->o;
+    a.OH = (d->h + 6 - 7) / 2 + 1;
+    a.OW = (d->w + 6 - 7) / 2 + 1;
+    a.sh = a.sw = 2; a.ph = a.pw = 3;
+    a.Hp = a.H + 6; a.Wp = a.W + 6;
+    a.OHW = a.OH * a.OW;
+    const int64_t M = static_cast<int64_t>(a.N) * a.OHW;
+    const int64_t xb = static_cast<int64_t>(a.N) * a.H * a.W * 4;
+    KXC_HIP_REQUIRE(M < (1LL << 30) && xb < (1LL << 31) && M * a.O < (1LL << 31) &&
+                    static_cast<int64_t>(a.N + 1) * a.Hp * (a.W / 4 + 2) < (1LL << 26),
+                    "%s: tensor too large for 32-bit addressing", who);
+    a.M = static_cast<int32_t>(M);
+    a.x_bytes = static_cast<uint32_t>(xb);
+    a.flags = d->flags;
+    a.nchunks = 1;
+    a.w_bytes = static_cast<uint32_t>((a.O / 32) * 7 * 1024);
+    *out = nullptr;
+    if (M == 0) return KXC_HIP_OK;
+    const int W4 = a.W / 4 + 2;
+    for (const K7Variant& v : kK7Variants) {
+        if ((a.O / 32) % v.ro != 0) continue;
+        const int rows = MaxRows(a, 7, 32 * v.wp);
+        const int segs = (rows * W4 + 63) / 64;
+        if (segs > v.ppt * v.wp) continue;
+        const size_t lds = static_cast<size_t>(segs) * 1024 + static_cast<size_t>(v.ro) * 7 * 1024;
+        if (lds > 160 * 1024) continue;
+        const int64_t tiles = CeilDiv(M, 32 * v.wp) * ((a.O / 32) / v.ro);
+        if (*out == nullptr || tiles >= 2 * 256) {
+            *out = &v; a.chs = segs * 64; L->lds_bytes = lds;
+            if (tiles >= 2 * 256) break;
+        }
+    }
+    KXC_HIP_REQUIRE(*out != nullptr, "%s: image rows too wide for the first-layer kernel (width %d)", who, d->w);
+    a.p_tiles = static_cast<int32_t>(CeilDiv(M, 32 * (*out)->wp));
+    a.o_tiles = (a.O / 32) / (*out)->ro;
+    a.num_tiles = a.p_tiles * a.o_tiles;
+    a.tiles_per_xcd = (a.num_tiles + 7) / 8;
+    L->grid = a.tiles_per_xcd * 8;
+    return KXC_HIP_OK;
+}
+
+}  // namespace
+
+extern "C" {
+
+int32_t kxc_hip_qconv2d_c4_packed_bytes(const kxc_hip_qconv2d_desc* d, size_t* out_bytes) {
+    KXC_HIP_REQUIRE(d != nullptr && out_bytes != nullptr, "kxc_hip_qconv2d_c4_packed_bytes: NULL argument");
+    KXC_HIP_REQUIRE(d->kh == 7 && d->kw == 7 && d->c >= 1 && d->c <= 4 && d->o > 0 && d->o % 32 == 0,
+                    "kxc_hip_qconv2d_c4_packed_bytes: needs a 7x7 filter, at most 4 input channels, output channels a multiple of 32");
+    *out_bytes = static_cast<size_t>(d->o / 32) * 7 * 1024;
+    return KXC_HIP_OK;
+}
+
+int32_t kxc_hip_qconv2d_c4_pack_weights(const kxc_hip_qconv2d_desc* d, const int8_t* w_oihw, int8_t* packed, void* stream) {
+    size_t bytes = 0;
+    if (int32_t rc = kxc_hip_qconv2d_c4_packed_bytes(d, &bytes)) return rc;
+    KXC_HIP_REQUIRE(w_oihw && packed, "kxc_hip_qconv2d_c4_pack_weights: NULL pointer");
+    const int64_t slots = static_cast<int64_t>(bytes / 16);
+    pack_weights_k7_c4_kernel<<<NoteGrid(static_cast<int>(CeilDiv(slots, kBlock))), NoteBlock(kBlock), NoteLds(0),
+                                ResolveStream(stream)>>>(w_oihw, packed, d->o, d->c, slots);
+    return CheckLaunch("qconv2d_c4_pack_weights");
+}
+
+int32_t kxc_hip_qconv2d_c4_i8(const kxc_hip_qconv2d_desc* d, const int8_t* x_c4, const int8_t* w_packed,
+                              const int32_t* bias, const float* mult, int8_t* y_c16, void* stream) {
+    QLaunch L;
+    const K7Variant* v = nullptr;
+    if (int32_t rc = PrepareK7(d, &L, &v, "kxc_hip_qconv2d_c4_i8")) return rc;
+    if (L.args.M == 0) return KXC_HIP_OK;
+    KXC_HIP_REQUIRE(x_c4 && w_packed && mult && y_c16, "kxc_hip_qconv2d_c4_i8: NULL pointer");
+    KXC_HIP_REQUIRE(!(d->flags & KXC_HIP_CONV_BIAS) || bias, "kxc_hip_qconv2d_c4_i8: bias flag without bias");
+    QArgs& a = L.args;
+    a.x = x_c4; a.wp = w_packed; a.bias = bias; a.mult = mult; a.res = nullptr; a.y = y_c16;
+    if (L.lds_bytes > 64 * 1024) {
+        KXC_HIP_CALL(hipFuncSetAttribute(reinterpret_cast<const void*>(v->kernel),
+                                         hipFuncAttributeMaxDynamicSharedMemorySize, static_cast<int>(L.lds_bytes)),
+                     "hipFuncSetAttribute");
+    }
+    hipLaunchKernelGGL(v->kernel, NoteGrid(dim3(L.grid)), NoteBlock(dim3(64 * v->wp)), NoteLds(L.lds_bytes),
+                       ResolveStream(stream), a);
+    return CheckLaunch(v->name);
+}
+
+int32_t kxc_hip_quantize_f32_nchw_to_c4_i8(const float* x, int8_t* y, int64_t n, int64_t c, int64_t hw, float scale,
+                                           void* stream) {
+    KXC_HIP_REQUIRE(n >= 0 && c >= 1 && c <= 4 && hw >= 0, "kxc_hip_quantize_f32_nchw_to_c4_i8: needs 1..4 channels");
+    KXC_HIP_REQUIRE(scale > 0.0f, "kxc_hip_quantize_f32_nchw_to_c4_i8: scale must be positive");
+    const int64_t total = n * hw;
+    if (total == 0) return KXC_HIP_OK;
+    KXC_HIP_REQUIRE(x && y, "kxc_hip_quantize_f32_nchw_to_c4_i8: NULL pointer");
+    KXC_HIP_REQUIRE(CeilDiv(total, kBlock) <= kMaxGridX, "kxc_hip_quantize_f32_nchw_to_c4_i8: tensor too large");
+    quantize_to_c4_kernel<<<NoteGrid(static_cast<int>(CeilDiv(total, kBlock))), NoteBlock(kBlock), NoteLds(0),
+                            ResolveStream(stream)>>>(x, y, static_cast<int32_t>(c), hw, total, scale);
+    return CheckLaunch("quantize_f32_nchw_to_c4_i8");
 }
 
 }  // extern "C"

@@ -362,6 +362,44 @@ def qconv2d_c16(x, c, w_packed, w_shape, bias, mult, residual=None, res_mult=0.0
     return y
 
 
+def quantize_to_c4(x, scale):
+    """fp32 NCHW (at most 4 channels) -> int8 [N][H][W][4]."""
+    import torch
+    _need(x, torch.float32, "x")
+    n, c, h, w = x.shape
+    y = torch.empty((n, h, w, 4), dtype=torch.int8, device=x.device)
+    _check(lib().kxc_hip_quantize_f32_nchw_to_c4_i8(_p(x), _p(y), C.c_int64(n), C.c_int64(c), C.c_int64(h * w),
+                                                    C.c_float(scale), _stream()))
+    return y
+
+
+def qconv2d_c4_pack_weights(w):
+    import torch
+    _need(w, torch.int8, "w")
+    o, c, kh, kw = w.shape
+    d = qconv_desc(1, c, kh, kw, o, kh, kw, 2, 3)
+    nbytes = C.c_size_t()
+    _check(lib().kxc_hip_qconv2d_c4_packed_bytes(C.byref(d), C.byref(nbytes)))
+    packed = torch.empty((nbytes.value,), dtype=torch.int8, device=w.device)
+    _check(lib().kxc_hip_qconv2d_c4_pack_weights(C.byref(d), _p(w), _p(packed), _stream()))
+    return packed
+
+
+def qconv2d_c4(x, c, w_packed, w_shape, bias, mult, relu=True):
+    """First layer: x in c4 ([N][H][W][4]), 7x7 / stride 2 / padding 3; returns the c16 output."""
+    import torch
+    _need(x, torch.int8, "x"); _need(w_packed, torch.int8, "w_packed"); _need(bias, torch.int32, "bias")
+    _need(mult, torch.float32, "mult")
+    n, h, wd, _ = x.shape
+    o = w_shape[0]
+    flags = (CONV_BIAS if bias is not None else 0) | (CONV_RELU if relu else 0)
+    d = qconv_desc(n, c, h, wd, o, 7, 7, 2, 3, flags)
+    oh = (h + 6 - 7) // 2 + 1; ow = (wd + 6 - 7) // 2 + 1
+    y = torch.empty(c16_shape(n, o, oh, ow), dtype=torch.int8, device=x.device)
+    _check(lib().kxc_hip_qconv2d_c4_i8(C.byref(d), _p(x), _p(w_packed), _p(bias), _p(mult), _p(y), _stream()))
+    return y
+
+
 def maxpool2d_c16_i8(x, c, k, s, pad):
     import torch
     _need(x, torch.int8, "x")
@@ -441,6 +479,12 @@ class Plan:
 
     def add_qconv2d_c16(self, desc, x, w_packed, bias, mult, residual, y):
         _check(lib().kxc_hip_plan_add_qconv2d_c16(self._h, C.byref(desc), x, w_packed, bias, mult, residual, y))
+
+    def add_qconv2d_c4(self, desc, x, w_packed, bias, mult, y):
+        _check(lib().kxc_hip_plan_add_qconv2d_c4(self._h, C.byref(desc), x, w_packed, bias, mult, y))
+
+    def add_quantize_c4(self, n, c, hw, scale, x, q):
+        _check(lib().kxc_hip_plan_add_quantize_c4(self._h, C.c_int64(n), C.c_int64(c), C.c_int64(hw), C.c_float(scale), x, q))
 
     def add_quantize_c16(self, n, c, hw, scale, x, q):
         _check(lib().kxc_hip_plan_add_quantize_c16(self._h, C.c_int64(n), C.c_int64(c), C.c_int64(hw), C.c_float(scale), x, q))

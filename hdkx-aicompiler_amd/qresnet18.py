@@ -126,8 +126,11 @@ class QuantizedResNet18:
         self.batch, self.hw = batch, hw
         dev = lambda a: torch.from_numpy(np.ascontiguousarray(a)).to(device)
         self.consts = []          # packed args after the input: per layer w_packed, bias, mult; fc w, bias, mult
-        for L in model["layers"]:
-            self.consts += [H.qconv2d_c16_pack_weights(dev(L["wq"])), dev(L["bias_q"]), dev(L["mult"])]
+        # the 7x7/2 first layer runs on the 4-channel input layout when the width allows it
+        self.first_c4 = hw % 4 == 0 and model["layers"][0]["k"] == 7 and model["layers"][0]["cin"] <= 4
+        for i, L in enumerate(model["layers"]):
+            pack = H.qconv2d_c4_pack_weights if (i == 0 and self.first_c4) else H.qconv2d_c16_pack_weights
+            self.consts += [pack(dev(L["wq"])), dev(L["bias_q"]), dev(L["mult"])]
         self.consts += [dev(model["fc"]["wq"]), dev(model["fc"]["bias_q"]), dev(model["fc"]["mult"])]
         nargs = 1 + len(self.consts) + 1
         plan = H.Plan(nargs)
@@ -158,9 +161,19 @@ class QuantizedResNet18:
                                  residual["buf"] if residual is not None else Buf.none(), y["buf"])
             return y
 
-        xq = new_act(batch, 3, hw, hw)
-        plan.add_quantize_c16(batch, 3, hw * hw, model["input_scale"], arg(0), xq["buf"])
-        y = conv(xq, "conv1")
+        if self.first_c4:
+            L0 = model["layers"][0]
+            off, size = arena.alloc(batch * hw * hw * 4)
+            xq = {"buf": Buf.ws(off), "off": off, "size": size}
+            plan.add_quantize_c4(batch, 3, hw * hw, model["input_scale"], arg(0), xq["buf"])
+            d = H.qconv_desc(batch, 3, hw, hw, L0["cout"], 7, 7, 2, 3, CONV_BIAS | CONV_RELU)
+            oh = (hw + 6 - 7) // 2 + 1
+            y = new_act(batch, L0["cout"], oh, oh)
+            plan.add_qconv2d_c4(d, xq["buf"], arg(1), arg(2), arg(3), y["buf"])
+        else:
+            xq = new_act(batch, 3, hw, hw)
+            plan.add_quantize_c16(batch, 3, hw * hw, model["input_scale"], arg(0), xq["buf"])
+            y = conv(xq, "conv1")
         free_act(xq)
         n, c, h, w = y["shape"]
         pd = H.pool_desc((n, c, h, w), 3, 2, 1)

@@ -199,6 +199,16 @@ int32_t kxc_hip_i8_nchw_to_c16(const int8_t* x, int8_t* y, int64_t n, int64_t c,
 int32_t kxc_hip_i8_c16_to_nchw(const int8_t* x, int8_t* y, int64_t n, int64_t c, int64_t hw, void* stream);
 int32_t kxc_hip_quantize_f32_nchw_to_c16_i8(const float* x, int8_t* y, int64_t n, int64_t c, int64_t hw,
                                             float scale, void* stream);
+/* First layer (7x7, stride 2, padding 3, at most 4 input channels, width a multiple of 4) on the "c4" input
+ * layout [N][H][W][4] (4 bytes per pixel, channels >= C zero): a k-step of the matrix instruction is one
+ * filter row of 8 taps x 4 channels.  Output is c16.  Weights are packed by the _c4_pack_weights call. */
+int32_t kxc_hip_qconv2d_c4_packed_bytes(const kxc_hip_qconv2d_desc* desc, size_t* out_bytes);
+int32_t kxc_hip_qconv2d_c4_pack_weights(const kxc_hip_qconv2d_desc* desc, const int8_t* w_oihw, int8_t* packed,
+                                        void* stream);
+int32_t kxc_hip_qconv2d_c4_i8(const kxc_hip_qconv2d_desc* desc, const int8_t* x_c4, const int8_t* w_packed,
+                              const int32_t* bias, const float* mult, int8_t* y_c16, void* stream);
+int32_t kxc_hip_quantize_f32_nchw_to_c4_i8(const float* x, int8_t* y, int64_t n, int64_t c, int64_t hw,
+                                           float scale, void* stream);
 int32_t kxc_hip_maxpool2d_c16_i8(const kxc_hip_pool2d_desc* desc, const int8_t* x, int8_t* y, void* stream);
 /* Output is [N][ceil(C/16)*16] int8 (c16 with H = W = 1, i.e. plain row-major when C is a multiple of 16). */
 int32_t kxc_hip_global_avg_pool2d_c16_i8(const int8_t* x, int8_t* y, int64_t n, int64_t c, int64_t h,
@@ -272,6 +282,10 @@ int32_t kxc_hip_plan_add_global_avg_pool2d_i8(kxc_hip_plan* plan, int64_t n, int
 int32_t kxc_hip_plan_add_qconv2d_c16(kxc_hip_plan* plan, const kxc_hip_qconv2d_desc* desc, kxc_hip_buf x,
                                      kxc_hip_buf w_packed, kxc_hip_buf bias, kxc_hip_buf mult,
                                      kxc_hip_buf residual, kxc_hip_buf y);
+int32_t kxc_hip_plan_add_qconv2d_c4(kxc_hip_plan* plan, const kxc_hip_qconv2d_desc* desc, kxc_hip_buf x_c4,
+                                    kxc_hip_buf w_packed, kxc_hip_buf bias, kxc_hip_buf mult, kxc_hip_buf y_c16);
+int32_t kxc_hip_plan_add_quantize_c4(kxc_hip_plan* plan, int64_t n, int64_t c, int64_t hw, float scale,
+                                     kxc_hip_buf x, kxc_hip_buf q);
 int32_t kxc_hip_plan_add_quantize_c16(kxc_hip_plan* plan, int64_t n, int64_t c, int64_t hw, float scale,
                                       kxc_hip_buf x, kxc_hip_buf q);
 int32_t kxc_hip_plan_add_maxpool2d_c16_i8(kxc_hip_plan* plan, const kxc_hip_pool2d_desc* desc,

@@ -97,6 +97,32 @@ def test_qconv_c16_against_cpu(pkg, orc, shape, residual):
     assert len(np.unique(want)) > 20
 
 
+@pytest.mark.parametrize("shape", [(2, 3, 224, 224, 64), (1, 3, 64, 64, 64), (3, 4, 20, 36, 32), (2, 1, 9, 8, 96)],
+                         ids=lambda s: "x".join(map(str, s)))
+def test_qconv_first_layer_c4_against_cpu(pkg, orc, shape):
+    """7x7 / stride 2 / padding 3 on the 4-channel input layout: same integers as the NCHW definition."""
+    n, c, h, w, o = shape
+    rng = np.random.default_rng(hash(shape) % (2 ** 31))
+    x = rng.integers(-128, 128, (n, c, h, w), dtype=np.int8)
+    wq = rng.integers(-127, 128, (o, c, 7, 7), dtype=np.int8)
+    bias = rng.integers(-20000, 20000, (o,), dtype=np.int32)
+    mult = rng.uniform(0.5, 2.0, (o,)).astype(np.float32) * np.float32(1.0 / (8.0 * np.sqrt(c * 49) * 64))
+    want = orc.qconv(x, wq, bias, mult, 2, 3, None, 0.0, True)
+    x4 = np.zeros((n, h, w, 4), np.int8)
+    x4[..., :c] = x.transpose(0, 2, 3, 1)
+    got = pkg.qconv2d_c4(dev(x4), c, pkg.qconv2d_c4_pack_weights(dev(wq)), wq.shape, dev(bias), dev(mult), True)
+    assert_bit_exact(from_c16(pkg, got, o), want, "first layer c4 %s" % (shape,))
+    assert len(np.unique(want)) > 20
+
+
+def test_quantize_to_c4(pkg, orc, synth):
+    x = synth.normal((2, 3, 12, 16), 902, 1.0)
+    q = host(pkg.quantize_to_c4(dev(x), 0.0171))
+    want = orc.quantize(x, 0.0171)
+    assert_bit_exact(q[..., :3], want.transpose(0, 2, 3, 1), "quantize to c4")
+    assert (q[..., 3] == 0).all()
+
+
 def test_qconv_c16_closed_forms(pkg):
     # all-ones input and weights, unit multiplier: the output counts the taps inside the image times C
     c, o = 32, 32
@@ -187,7 +213,8 @@ def test_qresnet18_small_every_layer(pkg, orc):
     assert_bit_exact(host(out), want_logits, "quantised logits (plan)")
     # the quantisation must be meaningful: logits close to the fp32 network's in the large
     assert np.isfinite(want_logits).all() and np.abs(want_logits).max() > 0
-    assert len(net.launches) == 24 and net.launches[1].startswith("kxc_qconv2d_c16_i8:qmfma")
+    assert len(net.launches) == 24 and net.launches[1].startswith("kxc_qconv2d_c4_i8:qmfma")
+    assert net.launches[3].startswith("kxc_qconv2d_c16_i8:qmfma")
 
 
 def test_qresnet18_batch64_images(pkg, orc):
