@@ -60,6 +60,8 @@ def main():
     ap.add_argument("--batch", type=int, default=64)
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--no-layers", action="store_true", help="skip the per-layer / per-operator timings")
+    ap.add_argument("--int8-only", action="store_true",
+                    help="run only the quantised ResNet-18 leg (for profiling its kernels) and print its JSON")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py: this build runs on exactly one GPU (no collectives, no sharding); "
@@ -80,6 +82,9 @@ def main():
     dev = lambda a: torch.from_numpy(np.ascontiguousarray(a)).cuda()
 
     batch = args.batch
+    if args.int8_only:
+        print(json.dumps(bench_int8(torch, pkg, synth, dev, np, batch)))
+        return
     consts_h = synth.resnet18_consts(4)
     x_h = synth.resnet18_input(4, batch)
     consts = [dev(c) for c in consts_h]
@@ -144,6 +149,7 @@ def main():
         result["conv_layers"] = bench_conv_layers(torch, pkg, synth, dev, batch)
         result["ops"] = bench_ops(torch, pkg, synth, dev)
         result["resnet18_bs1_img_per_s"] = bench_batch1(torch, pkg, hostapi, synth, dev)
+        result["int8"] = bench_int8(torch, pkg, synth, dev, np, batch)
 
     if not args.no_cpu:
         result["cpu_baseline"] = cpu_baseline(np, synth)
@@ -223,6 +229,27 @@ def bench_batch1(torch, pkg, hostapi, synth, dev):
     ms = _event_time_ms(torch, lambda: module.run_packed(packed, stream), 50, 10)
     module.close()
     return {"value": round(1e3 / ms, 1), "ms_per_image": round(ms, 4)}
+
+
+def bench_int8(torch, pkg, synth, dev, np, batch):
+    """BASELINE configs[4]: quantised ResNet-18, batch 64, int8 matrix cores (calibrated on the same batch)."""
+    qr = importlib.import_module("hdkx-aicompiler_amd.qresnet18")
+    consts = synth.resnet18_consts(5)
+    x = dev(synth.resnet18_input(5, batch))
+    amax = qr.calibrate(x, [dev(c) for c in consts])
+    model = qr.prepare(consts, amax)
+    net = qr.QuantizedResNet18(model, batch, 224)
+    out = torch.empty((batch, 1000), device="cuda")
+    packed = net.packed(x, out)
+    stream = torch.cuda.current_stream().cuda_stream
+    ms = _event_time_ms(torch, lambda: net.plan.run_packed(packed, stream), 50, 10)
+    r18 = importlib.import_module("hdkx-aicompiler_amd.resnet18")
+    ops = float(r18.flops_per_image()) * batch          # 2 integer operations per multiply-accumulate
+    return {"metric": "resnet18_int8_bs%d_img_per_s" % batch, "value": round(batch / (ms * 1e-3), 1), "ms_per_step": round(ms, 4),
+            "int8_tops": round(ops / (ms * 1e-3) / 1e12, 1), "frac_int8_mfma_peak": round(ops / (ms * 1e-3) / 1e12 / 5000.0, 4),
+            "launches_per_step": len(net.launches), "workspace_bytes": net.workspace_bytes,
+            "logits_finite": bool(torch.isfinite(out).all().item()),
+            "parity": "bit-exact against the CPU int8 chain (tests/test_gpu_int8.py); definition is this build's own"}
 
 
 def cpu_baseline(np, synth):

@@ -50,6 +50,25 @@ inline dim3 NoteGrid(dim3 g) { LaunchNote& n = LastLaunch(); n.grid[0] = g.x; n.
 inline dim3 NoteBlock(dim3 b) { LaunchNote& n = LastLaunch(); n.block[0] = b.x; n.block[1] = b.y; n.block[2] = b.z; return b; }
 inline size_t NoteLds(size_t bytes) { LastLaunch().dynamic_lds = static_cast<uint32_t>(bytes); return bytes; }
 
+// floor(x / d) for 0 <= x < 2^31 as a multiply and a shift: shift = 31 + ceil(log2 d), mul = floor(2^shift / d) + 1.
+// The kernels' tile set-up divides by launch-invariant values about twenty times; an integer division without
+// hardware support costs ~35 instructions, this costs three.
+struct FastDiv {
+    uint32_t mul, shift;
+};
+inline FastDiv MakeFastDiv(int32_t d) {
+    FastDiv f{1u << 31, 31};
+    if (d <= 0) return f;
+    uint32_t s = 0;
+    while ((1LL << s) < d) ++s;
+    f.shift = 31 + s;
+    f.mul = static_cast<uint32_t>((1ULL << f.shift) / static_cast<uint64_t>(d) + 1);
+    return f;
+}
+__device__ __forceinline__ int fast_div(int x, FastDiv f) {
+    return static_cast<int>((static_cast<uint64_t>(static_cast<uint32_t>(x)) * f.mul) >> f.shift);
+}
+
 constexpr int64_t kMaxGridX = 2147483647LL;
 
 inline int64_t CeilDiv(int64_t a, int64_t b) { return (a + b - 1) / b; }

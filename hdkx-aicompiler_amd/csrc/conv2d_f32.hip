@@ -39,10 +39,6 @@ namespace {
 
 typedef float floatx16 __attribute__((ext_vector_type(16)));
 
-struct FastDiv {
-    uint32_t mul, shift;
-};
-
 struct ConvArgs {
     const float* x;
     const float* w;
@@ -63,12 +59,6 @@ struct ConvArgs {
 };
 
 __device__ __forceinline__ float relu_sel(float v) { return (v > 0.0f) ? v : 0.0f; }
-
-// Division of x < 2^31 by a launch-invariant divisor as a multiply and a shift (the magic number comes from
-// the host): a hardware-less integer division costs ~35 instructions and the tile set-up needs about twenty.
-__device__ __forceinline__ int fast_div(int x, FastDiv f) {
-    return static_cast<int>((static_cast<uint64_t>(static_cast<uint32_t>(x)) * f.mul) >> f.shift);
-}
 
 // ------------------------------------------------------------------------------------------
 // MFMA kernel.  KH,KW: filter; CC: channels per LDS chunk (even); WO x WP waves, each wave
@@ -534,17 +524,6 @@ void Select(const ConvArgs& a, int kh, int kw, Choice* choice) {
             }
         }
     }
-}
-
-// floor(x / d) == (x * mul) >> shift for every 0 <= x < 2^31: shift = 31 + ceil(log2 d), mul = floor(2^shift / d) + 1.
-FastDiv MakeFastDiv(int32_t d) {
-    FastDiv f{1u << 31, 31};
-    if (d <= 0) return f;
-    uint32_t s = 0;
-    while ((1LL << s) < d) ++s;
-    f.shift = 31 + s;
-    f.mul = static_cast<uint32_t>((1ULL << f.shift) / static_cast<uint64_t>(d) + 1);
-    return f;
 }
 
 int32_t FillArgs(const kxc_hip_conv2d_desc* d, ConvArgs* a, const char* who) {

@@ -123,6 +123,102 @@ __global__ void __launch_bounds__(256) qdense_kernel(const int8_t* __restrict__ 
     }
 }
 
+// int8 dense, one wave per output column j and 64 rows at a time.  Lane l owns bytes [16l, 16l+16) of every
+// 1 KiB slice of K: the weight row is read once, every activation row as one coalesced 16-byte load per lane,
+// products go through the 4-way int8 dot instruction, and the 64 per-lane partial sums of the 64 rows are
+// combined with a transposing butterfly (63 exchanges instead of 64 x 6) that leaves row r's total in lane r.
+__global__ void __launch_bounds__(256) qdense_wave_kernel(const int8_t* __restrict__ a, const int8_t* __restrict__ b,
+                                                          const int32_t* __restrict__ bias, const float* __restrict__ mult,
+                                                          float* __restrict__ y, int32_t M, int32_t N, int32_t K) {
+    const int lane = threadIdx.x & 63;
+    const int j = blockIdx.x * 4 + (threadIdx.x >> 6);
+    if (j >= N) return;
+    const int32_t bj = bias ? bias[j] : 0;
+    const float mj = mult[j];
+    for (int i0 = 0; i0 < M; i0 += 64) {
+        int32_t acc[64];
+#pragma unroll
+        for (int r = 0; r < 64; ++r) acc[r] = 0;
+        for (int k0 = 0; k0 < K; k0 += 1024) {
+            const int kk = k0 + lane * 16;
+            if (kk < K) {
+                const int4 vb = *reinterpret_cast<const int4*>(b + static_cast<int64_t>(j) * K + kk);
+#pragma unroll
+                for (int r = 0; r < 64; ++r) {
+                    if (i0 + r < M) {
+                        const int4 va = *reinterpret_cast<const int4*>(a + static_cast<int64_t>(i0 + r) * K + kk);
+                        int32_t t = acc[r];
+                        t = __builtin_amdgcn_sdot4(va.x, vb.x, t, false);
+                        t = __builtin_amdgcn_sdot4(va.y, vb.y, t, false);
+                        t = __builtin_amdgcn_sdot4(va.z, vb.z, t, false);
+                        t = __builtin_amdgcn_sdot4(va.w, vb.w, t, false);
+                        acc[r] = t;
+                    }
+                }
+            }
+        }
+#pragma unroll
+        for (int s = 32; s >= 1; s >>= 1) {
+            const bool upper = (lane & s) != 0;
+#pragma unroll
+            for (int t = 0; t < s; ++t) {
+                const int32_t send = upper ? acc[t] : acc[t + s];
+                const int32_t keep = upper ? acc[t + s] : acc[t];
+                acc[t] = keep + __shfl_xor(send, s, 64);
+            }
+        }
+        const int row = i0 + lane;
+        if (row < M) y[static_cast<int64_t>(row) * N + j] = __fmul_rn(static_cast<float>(acc[0] + bj), mj);
+    }
+}
+
+// int8 dense on the int8 matrix cores: one wave per 32x32 block of y, D[i][j] += A[i][k] * B[j][k].  Both
+// operands are k-contiguous in memory, so a lane's 16-byte k-slice of the 32x32x32 instruction is one global
+// load each (no LDS): lane (r, half) reads a[i0+r][32*step + 16*half ..] and b[j0+r][same].  Rows / columns
+// past the end are clamped for the loads and skipped at the store.
+typedef int intx4_t __attribute__((ext_vector_type(4)));
+typedef int intx16_t __attribute__((ext_vector_type(16)));
+__global__ void __launch_bounds__(64) qdense_mfma_kernel(const int8_t* __restrict__ a, const int8_t* __restrict__ b,
+                                                         const int32_t* __restrict__ bias, const float* __restrict__ mult,
+                                                         float* __restrict__ y, int32_t M, int32_t N, int32_t K,
+                                                         int32_t col_blocks) {
+    const int lane = threadIdx.x;
+    const int r = lane & 31, half = lane >> 5;
+    const int ib = blockIdx.x / col_blocks, jb = blockIdx.x - ib * col_blocks;
+    const int i0 = ib * 32, j0 = jb * 32;
+    const int8_t* ap = a + static_cast<int64_t>(min(i0 + r, M - 1)) * K + 16 * half;
+    const int8_t* bp = b + static_cast<int64_t>(min(j0 + r, N - 1)) * K + 16 * half;
+    intx16_t acc;
+#pragma unroll
+    for (int g = 0; g < 16; ++g) acc[g] = 0;
+    const int steps = K >> 5;
+    int s = 0;
+    for (; s + 4 <= steps; s += 4) {
+        intx4_t av[4], bv[4];
+#pragma unroll
+        for (int u = 0; u < 4; ++u) {
+            av[u] = *reinterpret_cast<const intx4_t*>(ap + (s + u) * 32);
+            bv[u] = *reinterpret_cast<const intx4_t*>(bp + (s + u) * 32);
+        }
+#pragma unroll
+        for (int u = 0; u < 4; ++u) acc = __builtin_amdgcn_mfma_i32_32x32x32_i8(av[u], bv[u], acc, 0, 0, 0);
+    }
+    for (; s < steps; ++s) {
+        const intx4_t av = *reinterpret_cast<const intx4_t*>(ap + s * 32);
+        const intx4_t bv = *reinterpret_cast<const intx4_t*>(bp + s * 32);
+        acc = __builtin_amdgcn_mfma_i32_32x32x32_i8(av, bv, acc, 0, 0, 0);
+    }
+    const int j = j0 + r;
+    if (j >= N) return;
+    const int32_t bj = bias ? bias[j] : 0;
+    const float mj = mult[j];
+#pragma unroll
+    for (int g = 0; g < 16; ++g) {
+        const int i = i0 + 8 * (g / 4) + 4 * half + (g % 4);
+        if (i < M) y[static_cast<int64_t>(i) * N + j] = __fmul_rn(static_cast<float>(acc[g] + bj), mj);
+    }
+}
+
 }  // namespace
 
 extern "C" {
@@ -158,6 +254,21 @@ int32_t kxc_hip_qdense_i8(const int8_t* a, const int8_t* b, const int32_t* bias,
     if (m == 0 || n == 0) return KXC_HIP_OK;
     KXC_HIP_REQUIRE(a && b && mult && y, "kxc_hip_qdense_i8: NULL pointer");
     KXC_HIP_REQUIRE(k <= 2147483647LL / (128 * 128), "kxc_hip_qdense_i8: k too large for int32 accumulation");
+    const bool aligned16 = ((reinterpret_cast<uintptr_t>(a) | reinterpret_cast<uintptr_t>(b)) & 15u) == 0;
+    if (k % 32 == 0 && k > 0 && aligned16 && m < (1LL << 30) && n < (1LL << 30) &&
+        CeilDiv(m, 32) * CeilDiv(n, 32) <= kMaxGridX) {
+        const int32_t col_blocks = static_cast<int32_t>(CeilDiv(n, 32));
+        qdense_mfma_kernel<<<NoteGrid(static_cast<int>(CeilDiv(m, 32) * col_blocks)), NoteBlock(64), NoteLds(0),
+                             ResolveStream(stream)>>>(a, b, bias, mult, y, static_cast<int32_t>(m),
+                                                      static_cast<int32_t>(n), static_cast<int32_t>(k), col_blocks);
+        return CheckLaunch("qdense_mfma");
+    }
+    if (k % 16 == 0 && m < (1LL << 31) && n < (1LL << 31) && CeilDiv(n, 4) <= kMaxGridX &&
+        ((reinterpret_cast<uintptr_t>(a) | reinterpret_cast<uintptr_t>(b)) & 15u) == 0) {
+        qdense_wave_kernel<<<NoteGrid(static_cast<int>(CeilDiv(n, 4))), NoteBlock(256), NoteLds(0), ResolveStream(stream)>>>(
+            a, b, bias, mult, y, static_cast<int32_t>(m), static_cast<int32_t>(n), static_cast<int32_t>(k));
+        return CheckLaunch("qdense_wave");
+    }
     int64_t g = CeilDiv(m * n, 256);
     if (g > 256 * 32) g = 256 * 32;
     qdense_kernel<<<NoteGrid(static_cast<int>(g)), NoteBlock(256), NoteLds(0), ResolveStream(stream)>>>(a, b, bias, mult, y, m, n, k);

@@ -79,6 +79,7 @@ struct QArgs {
     int32_t p_tiles, o_tiles, num_tiles, tiles_per_xcd;
     float res_mult;
     uint32_t flags;
+    FastDiv div_wp, div_hp, div_ohw, div_ow, div_otiles;   // div_wp: positions per LDS row (pixels, or pixel quads on c4)
 };
 
 // Epilogue shared by the matrix-core kernels.  Accumulator register g of a 32x32 block is output channel
@@ -140,17 +141,17 @@ __global__ void __launch_bounds__(64 * WP) qconv_mfma_kernel(const QArgs a) {
     // consecutive workgroups go to the 8 XCDs round-robin; give every XCD (own L2) a contiguous run of tiles
     const int tile = (blockIdx.x & 7) * a.tiles_per_xcd + (blockIdx.x >> 3);
     if (tile >= a.num_tiles || static_cast<int>(blockIdx.x >> 3) >= a.tiles_per_xcd) return;
-    const int p_tile = tile / a.o_tiles, o_tile = tile - p_tile * a.o_tiles;
+    const int p_tile = fast_div(tile, a.div_otiles), o_tile = tile - p_tile * a.o_tiles;
     const int m0 = p_tile * TP;
     const int ob0 = o_tile * RO;                     // first 32-channel output block
 
     const int m_last = min(m0 + TP, a.M) - 1;
     int qmin, qlast;
     {
-        const int n = m0 / a.OHW, rem = m0 - n * a.OHW;
-        qmin = n * a.Hp + (rem / a.OW) * a.sh;
-        const int n2 = m_last / a.OHW, rem2 = m_last - n2 * a.OHW;
-        qlast = n2 * a.Hp + (rem2 / a.OW) * a.sh + (KH - 1);
+        const int n = fast_div(m0, a.div_ohw), rem = m0 - n * a.OHW;
+        qmin = n * a.Hp + fast_div(rem, a.div_ow) * a.sh;
+        const int n2 = fast_div(m_last, a.div_ohw), rem2 = m_last - n2 * a.OHW;
+        qlast = n2 * a.Hp + fast_div(rem2, a.div_ow) * a.sh + (KH - 1);
     }
     const int P = (qlast - qmin + 1) * a.Wp;         // positions per plane (<= chs)
     const int xsegs = (P + 63) >> 6;
@@ -163,9 +164,9 @@ __global__ void __launch_bounds__(64 * WP) qconv_mfma_kernel(const QArgs a) {
 #pragma unroll
     for (int i = 0; i < PPT; ++i) {
         const int pos = (wave + i * WP) * 64 + lane;
-        const int q = pos / a.Wp, col = pos - q * a.Wp;
+        const int q = fast_div(pos, a.div_wp), col = pos - q * a.Wp;
         const int Q = qmin + q;
-        const int n = Q / a.Hp, ih = Q - n * a.Hp - a.ph, iw = col - a.pw;
+        const int n = fast_div(Q, a.div_hp), ih = Q - n * a.Hp - a.ph, iw = col - a.pw;
         const bool ok = pos < P && n < a.N && ih >= 0 && ih < a.H && iw >= 0 && iw < a.W;
         goff[i] = ok ? (static_cast<uint32_t>(n) * a.CB * a.H * a.W + static_cast<uint32_t>(ih * a.W + iw)) * 16u : kOob;
     }
@@ -176,8 +177,8 @@ __global__ void __launch_bounds__(64 * WP) qconv_mfma_kernel(const QArgs a) {
     int ypix;            // position index (n*OB16*OHW + pixel) of this lane's output pixel for block 0, or -1
     {
         const int mc = min(m, a.M - 1);
-        const int n = mc / a.OHW, rem = mc - n * a.OHW;
-        const int oh = rem / a.OW, ow = rem - oh * a.OW;
+        const int n = fast_div(mc, a.div_ohw), rem = mc - n * a.OHW;
+        const int oh = fast_div(rem, a.div_ow), ow = rem - oh * a.OW;
         xbase = ((n * a.Hp + oh * a.sh - qmin) * a.Wp + ow * a.sw) * 16;
         if (CBC > 1) xbase += half * a.chs * 16;
         ypix = (m < a.M) ? n * (a.O >> 4) * a.OHW + rem : -1;
@@ -294,16 +295,16 @@ __global__ void __launch_bounds__(64 * WP) qconv_k7s2_c4_kernel(const QArgs a) {
 
     const int tile = (blockIdx.x & 7) * a.tiles_per_xcd + (blockIdx.x >> 3);
     if (tile >= a.num_tiles || static_cast<int>(blockIdx.x >> 3) >= a.tiles_per_xcd) return;
-    const int p_tile = tile / a.o_tiles, o_tile = tile - p_tile * a.o_tiles;
+    const int p_tile = fast_div(tile, a.div_otiles), o_tile = tile - p_tile * a.o_tiles;
     const int m0 = p_tile * TP;
     const int ob0 = o_tile * RO;
     const int m_last = min(m0 + TP, a.M) - 1;
     int qmin, qlast;
     {
-        const int n = m0 / a.OHW, rem = m0 - n * a.OHW;
-        qmin = n * a.Hp + (rem / a.OW) * 2;
-        const int n2 = m_last / a.OHW, rem2 = m_last - n2 * a.OHW;
-        qlast = n2 * a.Hp + (rem2 / a.OW) * 2 + (KH - 1);
+        const int n = fast_div(m0, a.div_ohw), rem = m0 - n * a.OHW;
+        qmin = n * a.Hp + fast_div(rem, a.div_ow) * 2;
+        const int n2 = fast_div(m_last, a.div_ohw), rem2 = m_last - n2 * a.OHW;
+        qlast = n2 * a.Hp + fast_div(rem2, a.div_ow) * 2 + (KH - 1);
     }
     const int P = (qlast - qmin + 1) * W4;
     const int xsegs = (P + 63) >> 6;
@@ -314,9 +315,9 @@ __global__ void __launch_bounds__(64 * WP) qconv_k7s2_c4_kernel(const QArgs a) {
         const int seg = wave + i * WP;
         if (seg < xsegs) {
             const int pos = seg * 64 + lane;
-            const int q = pos / W4, c4 = pos - q * W4;
+            const int q = fast_div(pos, a.div_wp), c4 = pos - q * W4;
             const int Q = qmin + q;
-            const int n = Q / a.Hp, ih = Q - n * a.Hp - 3;
+            const int n = fast_div(Q, a.div_hp), ih = Q - n * a.Hp - 3;
             const bool ok = pos < P && n < a.N && ih >= 0 && ih < a.H && c4 >= 1 && c4 <= (a.W >> 2);
             const uint32_t off = ok ? static_cast<uint32_t>((n * a.H + ih) * a.W + (c4 - 1) * 4) * 4u : kOob;
             load16_to_lds(xr, (lds_ptr_t)(lds + seg * 1024), off, 0);
@@ -335,8 +336,8 @@ __global__ void __launch_bounds__(64 * WP) qconv_k7s2_c4_kernel(const QArgs a) {
     int xbase, ypix;
     {
         const int mc = min(m, a.M - 1);
-        const int n = mc / a.OHW, rem = mc - n * a.OHW;
-        const int oh = rem / a.OW, ow = rem - oh * a.OW;
+        const int n = fast_div(mc, a.div_ohw), rem = mc - n * a.OHW;
+        const int oh = fast_div(rem, a.div_ow), ow = rem - oh * a.OW;
         xbase = (n * a.Hp + oh * 2 - qmin) * W4 * 16 + ow * 8 + half * 16;
         ypix = (m < a.M) ? n * (a.O >> 4) * a.OHW + rem : -1;
     }
@@ -529,29 +530,25 @@ __global__ void __launch_bounds__(kBlock) maxpool_c16_kernel(const int8_t* __res
     *reinterpret_cast<int4*>(y + s * 16) = make_int4(o[0], o[1], o[2], o[3]);
 }
 
-// One thread per (n, channel block): sums the plane, requantises; output [N][CB*16] (= c16 with H = W = 1).
+// Four threads per (n, channel block) plane, each summing one dword (4 channels) of every position; output
+// [N][CB*16] (= c16 with H = W = 1).
 __global__ void __launch_bounds__(kBlock) gap_c16_kernel(const int8_t* __restrict__ x, int8_t* __restrict__ y,
                                                          int64_t planes, int32_t hw, float mult) {
-    const int64_t p = static_cast<int64_t>(blockIdx.x) * kBlock + threadIdx.x;
-    if (p >= planes) return;
-    const int8_t* src = x + p * hw * 16;
-    int32_t sum[16];
-#pragma unroll
-    for (int j = 0; j < 16; ++j) sum[j] = 0;
+    const int64_t t = static_cast<int64_t>(blockIdx.x) * kBlock + threadIdx.x;
+    if (t >= planes * 4) return;
+    const uint32_t* src = reinterpret_cast<const uint32_t*>(x) + (t >> 2) * hw * 4 + (t & 3);
+    int32_t sum[4] = {0, 0, 0, 0};
+#pragma unroll 7
     for (int i = 0; i < hw; ++i) {
-        const int4 v = *reinterpret_cast<const int4*>(src + static_cast<int64_t>(i) * 16);
-        const int vw[4] = {v.x, v.y, v.z, v.w};
+        const uint32_t v = src[static_cast<int64_t>(i) * 4];
 #pragma unroll
-        for (int j = 0; j < 16; ++j)
-            sum[j] += static_cast<int32_t>(static_cast<int8_t>((vw[j >> 2] >> (8 * (j & 3))) & 0xff));
+        for (int j = 0; j < 4; ++j) sum[j] += static_cast<int32_t>(static_cast<int8_t>((v >> (8 * j)) & 0xff));
     }
-    uint32_t o[4] = {0, 0, 0, 0};
+    uint32_t o = 0;
 #pragma unroll
-    for (int j = 0; j < 16; ++j) {
-        const int32_t q = requant_i32(sum[j], mult, false, 0, 0.0f, false);
-        o[j >> 2] |= (static_cast<uint32_t>(q) & 0xffu) << (8 * (j & 3));
-    }
-    *reinterpret_cast<int4*>(y + p * 16) = make_int4(o[0], o[1], o[2], o[3]);
+    for (int j = 0; j < 4; ++j)
+        o |= (static_cast<uint32_t>(requant_i32(sum[j], mult, false, 0, 0.0f, false)) & 0xffu) << (8 * j);
+    reinterpret_cast<uint32_t*>(y)[t] = o;
 }
 
 // ------------------------------------------------------------------ host side
@@ -683,6 +680,8 @@ int32_t PrepareUncached(const kxc_hip_qconv2d_desc* d, QLaunch* L, const char* w
     a.o_tiles = (a.O / 32) / best->ro;
     a.num_tiles = a.p_tiles * a.o_tiles;
     a.tiles_per_xcd = (a.num_tiles + 7) / 8;
+    a.div_wp = MakeFastDiv(a.Wp); a.div_hp = MakeFastDiv(a.Hp); a.div_ohw = MakeFastDiv(a.OHW);
+    a.div_ow = MakeFastDiv(a.OW); a.div_otiles = MakeFastDiv(a.o_tiles);
     L->grid = a.tiles_per_xcd * 8;
     L->v = best;
     const int NS = (best->kh * best->kw * cbc + 1) / 2;
@@ -813,7 +812,7 @@ int32_t kxc_hip_global_avg_pool2d_c16_i8(const int8_t* x, int8_t* y, int64_t n, 
     const int64_t planes = n * ((c + 15) / 16);
     if (planes == 0) return KXC_HIP_OK;
     KXC_HIP_REQUIRE(x && y, "kxc_hip_global_avg_pool2d_c16_i8: NULL pointer");
-    gap_c16_kernel<<<NoteGrid(static_cast<int>(CeilDiv(planes, kBlock))), NoteBlock(kBlock), NoteLds(0), ResolveStream(stream)>>>(
+    gap_c16_kernel<<<NoteGrid(static_cast<int>(CeilDiv(planes * 4, kBlock))), NoteBlock(kBlock), NoteLds(0), ResolveStream(stream)>>>(
         x, y, planes, static_cast<int32_t>(h * w), mult);
     return CheckLaunch("global_avg_pool2d_c16_i8");
 }
@@ -877,6 +876,8 @@ int32_t PrepareK7(const kxc_hip_qconv2d_desc* d, QLaunch* L, const K7Variant** o
     a.o_tiles = (a.O / 32) / (*out)->ro;
     a.num_tiles = a.p_tiles * a.o_tiles;
     a.tiles_per_xcd = (a.num_tiles + 7) / 8;
+    a.div_wp = MakeFastDiv(W4); a.div_hp = MakeFastDiv(a.Hp); a.div_ohw = MakeFastDiv(a.OHW);
+    a.div_ow = MakeFastDiv(a.OW); a.div_otiles = MakeFastDiv(a.o_tiles);
     L->grid = a.tiles_per_xcd * 8;
     return KXC_HIP_OK;
 }

@@ -231,3 +231,16 @@ def test_qresnet18_batch64_images(pkg, orc):
     for n in (0, 63):
         want, _ = orc.qresnet18(x[n:n + 1], model, net.gap_mult)
         assert_bit_exact(first[n:n + 1], want, "quantised resnet18 batch 64, image %d" % n)
+
+
+@pytest.mark.parametrize("m,n,k", [(64, 1000, 512), (70, 37, 1056), (33, 65, 32), (70, 37, 1040), (1, 5, 16), (9, 12, 24)])
+def test_qdense_shapes(pkg, orc, m, n, k):
+    """Matrix-core kernel (k a multiple of 32, ragged rows and columns), wave-per-column kernel (k a multiple
+    of 16, more than one 1 KiB slice) and the scalar fallback (k = 24)."""
+    rng = np.random.default_rng(m * 1000 + k)
+    a = rng.integers(-128, 128, (m, k), dtype=np.int8)
+    b = rng.integers(-127, 128, (n, k), dtype=np.int8)
+    bias = rng.integers(-5000, 5000, (n,), dtype=np.int32)
+    mult = rng.uniform(1e-4, 1e-3, (n,)).astype(np.float32)
+    assert_bit_exact(host(pkg.qdense(dev(a), dev(b), dev(bias), dev(mult))), orc.qdense(a, b, bias, mult),
+                     "qdense %dx%dx%d" % (m, n, k))
