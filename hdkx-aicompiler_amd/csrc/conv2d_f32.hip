@@ -85,7 +85,7 @@ typedef __attribute__((address_space(3))) void* lds_ptr_t;
 // order at the end (deterministic).  It multiplies the waves per output block for launches that have too
 // few 32x32 blocks to occupy 1024 SIMDs (7x7 feature maps, batch 1).
 template <int KH, int KW, int CC, int WO, int WP, int RO, int RP, int PPT, int KS>
-__global__ void __launch_bounds__(64 * WO * WP * KS)
+__global__ void __launch_bounds__(64 * WO * WP * KS) __attribute__((amdgpu_waves_per_eu(2)))
 conv_mfma_kernel(const ConvArgs a) {
     constexpr int NW = WO * WP;                               // waves per reduction group
     constexpr int TO = 32 * RO * WO;

@@ -33,7 +33,7 @@ __device__ __forceinline__ float epilogue(float acc, float alpha, float beta, co
     return v;
 }
 
-__global__ void __launch_bounds__(256) gemm_nt_mfma_kernel(const float* __restrict__ a, const float* __restrict__ b,
+__global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2))) gemm_nt_mfma_kernel(const float* __restrict__ a, const float* __restrict__ b,
                                                            const float* __restrict__ c, float* __restrict__ y,
                                                            int32_t M, int32_t N, int32_t K, float alpha, float beta,
                                                            int64_t c_len, int scale_a, int scale_c) {
@@ -178,7 +178,7 @@ __global__ void __launch_bounds__(256) qdense_wave_kernel(const int8_t* __restri
 // past the end are clamped for the loads and skipped at the store.
 typedef int intx4_t __attribute__((ext_vector_type(4)));
 typedef int intx16_t __attribute__((ext_vector_type(16)));
-__global__ void __launch_bounds__(64) qdense_mfma_kernel(const int8_t* __restrict__ a, const int8_t* __restrict__ b,
+__global__ void __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(2))) qdense_mfma_kernel(const int8_t* __restrict__ a, const int8_t* __restrict__ b,
                                                          const int32_t* __restrict__ bias, const float* __restrict__ mult,
                                                          float* __restrict__ y, int32_t M, int32_t N, int32_t K,
                                                          int32_t col_blocks) {

@@ -119,7 +119,7 @@ __device__ __forceinline__ void epilogue_c16(const intx16 (&acc)[RO], const QArg
 }
 
 template <int KH, int KW, int CBC, int WP, int RO, int PPT>
-__global__ void __launch_bounds__(64 * WP) qconv_mfma_kernel(const QArgs a) {
+__global__ void __launch_bounds__(64 * WP) __attribute__((amdgpu_waves_per_eu(2))) qconv_mfma_kernel(const QArgs a) {
     constexpr int KHW = KH * KW;
     constexpr int NS = (KHW * CBC + 1) / 2;          // matrix k-steps per chunk
     constexpr int TP = 32 * WP;
@@ -279,7 +279,7 @@ __global__ void __launch_bounds__(64 * WP) qconv_mfma_kernel(const QArgs a) {
 // block costs, and a quarter of the input bytes.  LDS rows hold [4 zero pixels][W pixels][4 zero pixels]
 // as 16-byte positions; a tile's rows are loaded once (single chunk).  Output is c16.
 template <int WP, int RO, int PPT>
-__global__ void __launch_bounds__(64 * WP) qconv_k7s2_c4_kernel(const QArgs a) {
+__global__ void __launch_bounds__(64 * WP) __attribute__((amdgpu_waves_per_eu(2))) qconv_k7s2_c4_kernel(const QArgs a) {
     constexpr int KH = 7;
     constexpr int TP = 32 * WP;
     constexpr int WSEG = RO * KH;
