@@ -487,6 +487,8 @@ void Select(const ConvArgs& a, int kh, int kw, Choice* choice) {
     const char* preferred = nullptr;
     if (kh == 3 && a.OW <= 14 && a.M >= 8192) preferred = "mfma_k3x3_c4_o1x1_p8x1";
     if (kh == 3 && a.sh == 2 && a.W >= 56) preferred = "mfma_k3x3_c2_o1x1_p4x1";
+    if (kh == 3 && a.sh == 1 && a.W >= 56 && a.O % 64 == 0 && a.M >= 65536) preferred = "mfma_k3x3_c4_o1x2_p4x1";
+    if (kh == 1 && a.W >= 56 && a.O % 64 == 0 && a.M >= 32768) preferred = "mfma_k1x1_c8_o1x2_p4x2";
     // Pass 0 takes the rule's variant (or the forced one).  Pass 1 takes the first table entry that fits,
     // unless that launch would leave most SIMDs idle (fewer than three waves per SIMD): then the reduction is
     // split inside the workgroup -- two ways on the 32x128 tile if that is enough, else four or eight ways on

@@ -5,7 +5,9 @@
 // Intermediates live in ONE workspace allocated at finalize time (the CPU backend mallocs and frees
 // every intermediate on every call, src/codegen/codegen_llvm.cc:578-623).
 #include <cstdio>
+#include <cstdlib>
 #include <cstring>
+#include <sstream>
 #include <string>
 #include <vector>
 
@@ -591,6 +593,136 @@ int32_t kxc_hip_plan_run_profiled(kxc_hip_plan* plan, void** args, void* stream,
     for (auto& e : ev)
         if (e) (void)hipEventDestroy(e);
     return rc;
+}
+
+// ---- serialisation: one text line per node, every field as a number (floats as hex floats, exact)
+int32_t kxc_hip_plan_serialize(const kxc_hip_plan* plan, char* buffer, size_t capacity, size_t* needed) {
+    KXC_HIP_REQUIRE(plan != nullptr && needed != nullptr, "kxc_hip_plan_serialize: NULL argument");
+    KXC_HIP_REQUIRE(plan->finalized, "kxc_hip_plan_serialize: plan is not finalized");
+    std::string out;
+    char tmp[96];
+    auto I = [&](long long v) { std::snprintf(tmp, sizeof(tmp), " %lld", v); out += tmp; };
+    auto F = [&](float v) { std::snprintf(tmp, sizeof(tmp), " %a", static_cast<double>(v)); out += tmp; };
+    out += "kxc_hip_plan 1";
+    I(plan->num_args); I(static_cast<long long>(plan->workspace_bytes)); I(static_cast<long long>(plan->nodes.size()));
+    out += "\n";
+    for (const Node& n : plan->nodes) {
+        KXC_HIP_REQUIRE(n.symbol.find_first_of(" \n\t") == std::string::npos,
+                        "kxc_hip_plan_serialize: kernel symbol '%s' contains white space", n.symbol.c_str());
+        out += "node";
+        I(static_cast<int>(n.kind));
+        out += " " + n.symbol;
+        for (const kxc_hip_buf& b : n.bufs) { I(b.kind); I(b.index_or_offset); }
+        const kxc_hip_conv2d_desc& c = n.conv;
+        for (long long v : {(long long)c.n, (long long)c.c, (long long)c.h, (long long)c.w, (long long)c.o, (long long)c.kh,
+                            (long long)c.kw, (long long)c.stride_h, (long long)c.stride_w, (long long)c.pad_h, (long long)c.pad_w,
+                            (long long)c.dil_h, (long long)c.dil_w, (long long)c.flags}) I(v);
+        const kxc_hip_qconv2d_desc& q = n.qconv;
+        for (long long v : {(long long)q.n, (long long)q.c, (long long)q.h, (long long)q.w, (long long)q.o, (long long)q.kh,
+                            (long long)q.kw, (long long)q.stride_h, (long long)q.stride_w, (long long)q.pad_h, (long long)q.pad_w,
+                            (long long)q.flags}) I(v);
+        F(q.res_mult);
+        const kxc_hip_pool2d_desc& pd = n.pool;
+        for (long long v : {(long long)pd.n, (long long)pd.c, (long long)pd.h, (long long)pd.w, (long long)pd.kh, (long long)pd.kw,
+                            (long long)pd.stride_h, (long long)pd.stride_w, (long long)pd.pad_top, (long long)pd.pad_left,
+                            (long long)pd.pad_bottom, (long long)pd.pad_right, (long long)pd.ceil_mode, (long long)pd.is_avg}) I(v);
+        for (int64_t v : n.dims) I(v);
+        for (float v : n.f) F(v);
+        for (int32_t v : n.i32) I(v);
+        for (int64_t v : n.a_shape) I(v);
+        for (int64_t v : n.b_shape) I(v);
+        for (uint32_t v : n.grid) I(v);
+        for (uint32_t v : n.block) I(v);
+        I(n.shared_bytes);
+        I(static_cast<long long>(n.params.size()));
+        for (const kxc_hip_buf& b : n.params) { I(b.kind); I(b.index_or_offset); }
+        out += "\n";
+    }
+    *needed = out.size() + 1;
+    if (buffer == nullptr || capacity == 0) return KXC_HIP_OK;
+    KXC_HIP_REQUIRE(capacity >= *needed, "kxc_hip_plan_serialize: %zu bytes needed, room for %zu", *needed, capacity);
+    std::memcpy(buffer, out.c_str(), *needed);
+    return KXC_HIP_OK;
+}
+
+int32_t kxc_hip_plan_deserialize(const char* text, int32_t device_id, kxc_hip_module* const* modules, int32_t num_modules,
+                                 kxc_hip_plan** out_plan) {
+    const char* who = "kxc_hip_plan_deserialize";
+    KXC_HIP_REQUIRE(text != nullptr && out_plan != nullptr, "%s: NULL argument", who);
+    std::istringstream in{std::string(text)};
+    std::string magic;
+    long long version = 0, num_args = 0, workspace = 0, count = 0;
+    in >> magic >> version >> num_args >> workspace >> count;
+    KXC_HIP_REQUIRE(in && magic == "kxc_hip_plan" && version == 1, "%s: not a version-1 plan", who);
+    KXC_HIP_REQUIRE(num_args >= 0 && num_args < (1 << 20) && workspace >= 0 && count >= 0 && count < (1 << 24),
+                    "%s: implausible header", who);
+    kxc_hip_plan* plan = nullptr;
+    if (int32_t rc = kxc_hip_plan_create(device_id, static_cast<int32_t>(num_args), &plan)) return rc;
+    auto fail = [&](const char* what) {
+        kxc_hip_plan_destroy(plan);
+        return Fail(KXC_HIP_ERR_INVALID, "%s: %s", who, what);
+    };
+    for (long long k = 0; k < count; ++k) {
+        std::string tag;
+        long long kind = -1;
+        Node n{};
+        in >> tag >> kind >> n.symbol;
+        if (!in || tag != "node" || kind < 0 || kind > static_cast<long long>(NodeKind::kModuleKernel)) return fail("bad node line");
+        n.kind = static_cast<NodeKind>(kind);
+        long long v = 0;
+        auto I = [&]() { in >> v; return v; };
+        auto F = [&]() { std::string t; in >> t; return static_cast<float>(std::strtod(t.c_str(), nullptr)); };
+        for (kxc_hip_buf& b : n.bufs) { b.kind = static_cast<int32_t>(I()); b.index_or_offset = I(); }
+        kxc_hip_conv2d_desc& c = n.conv;
+        c.n = I(); c.c = I(); c.h = I(); c.w = I(); c.o = I(); c.kh = I(); c.kw = I(); c.stride_h = I(); c.stride_w = I();
+        c.pad_h = I(); c.pad_w = I(); c.dil_h = I(); c.dil_w = I(); c.flags = static_cast<uint32_t>(I());
+        kxc_hip_qconv2d_desc& q = n.qconv;
+        q.n = I(); q.c = I(); q.h = I(); q.w = I(); q.o = I(); q.kh = I(); q.kw = I(); q.stride_h = I(); q.stride_w = I();
+        q.pad_h = I(); q.pad_w = I(); q.flags = static_cast<uint32_t>(I()); q.res_mult = F();
+        kxc_hip_pool2d_desc& pd = n.pool;
+        pd.n = I(); pd.c = I(); pd.h = I(); pd.w = I(); pd.kh = I(); pd.kw = I(); pd.stride_h = I(); pd.stride_w = I();
+        pd.pad_top = I(); pd.pad_left = I(); pd.pad_bottom = I(); pd.pad_right = I(); pd.ceil_mode = I(); pd.is_avg = I();
+        for (int64_t& d : n.dims) d = I();
+        for (float& f : n.f) f = F();
+        for (int32_t& i : n.i32) i = static_cast<int32_t>(I());
+        for (int64_t& d : n.a_shape) d = I();
+        for (int64_t& d : n.b_shape) d = I();
+        for (uint32_t& g : n.grid) g = static_cast<uint32_t>(I());
+        for (uint32_t& b : n.block) b = static_cast<uint32_t>(I());
+        n.shared_bytes = static_cast<uint32_t>(I());
+        const long long np = I();
+        if (!in || np < 0 || np > 4096) return fail("bad parameter count");
+        for (long long i = 0; i < np; ++i) {
+            kxc_hip_buf b;
+            b.kind = static_cast<int32_t>(I()); b.index_or_offset = I();
+            n.params.push_back(b);
+        }
+        if (!in) return fail("truncated node line");
+        auto buf_ok = [&](const kxc_hip_buf& b) {
+            if (b.kind == KXC_HIP_BUF_ARG) return b.index_or_offset >= 0 && b.index_or_offset < num_args;
+            if (b.kind == KXC_HIP_BUF_WORKSPACE) return b.index_or_offset >= 0 && b.index_or_offset < workspace;
+            return b.kind == KXC_HIP_BUF_NONE;
+        };
+        for (const kxc_hip_buf& b : n.bufs) if (!buf_ok(b)) return fail("buffer operand out of range");
+        for (const kxc_hip_buf& b : n.params) if (!buf_ok(b)) return fail("kernel parameter out of range");
+        if (n.kind == NodeKind::kModuleKernel) {
+            // generated kernels are found by name in the modules the caller compiled from the saved source
+            for (int32_t m = 0; m < num_modules && !n.function; ++m) {
+                void* fn = nullptr;
+                if (modules && modules[m] && kxc_hip_module_get_function(modules[m], n.symbol.c_str(), &fn) == KXC_HIP_OK) n.function = fn;
+            }
+            if (!n.function) return fail(("generated kernel not found in the given modules: " + n.symbol).c_str());
+            if (static_cast<uint64_t>(n.block[0]) * n.block[1] * n.block[2] > 1024 || n.grid[0] == 0 || n.block[0] == 0)
+                return fail("bad launch geometry");
+        }
+        plan->nodes.push_back(n);
+    }
+    if (int32_t rc = kxc_hip_plan_finalize(plan, static_cast<size_t>(workspace))) {
+        kxc_hip_plan_destroy(plan);
+        return rc;
+    }
+    *out_plan = plan;
+    return KXC_HIP_OK;
 }
 
 int32_t kxc_hip_plan_num_nodes(const kxc_hip_plan* plan) { return plan ? static_cast<int32_t>(plan->nodes.size()) : 0; }

@@ -69,7 +69,8 @@ public:
     int64_t constant_count() const;
     // The launches Run performs, in order.
     const std::vector<KernelExecInfo>& GetKernelExecs() const;
-    // Execution-plan description (schema of src/base/execution_plan.cc:674-877: integers plus kernel_symbol).
+    // Execution-plan description: the schema of src/base/execution_plan.cc:674-877 (value ids, op_name,
+    // kernel_symbol per node) plus a "kxc_hip" object with everything LoadExecutionPlan needs.
     std::string ExecutionPlanJSON() const;
     size_t workspace_bytes() const;
 
@@ -80,6 +81,10 @@ private:
 class Compiler {
 public:
     static CompiledModule Compile(Function func, CompileConfig config);
+    // Rebuilds a runnable module for the hip target from CompiledModule::ExecutionPlanJSON() without the
+    // graph: saved kernel sources are compiled again, the launches come from the saved launch plan.  The
+    // caller passes the same packed arguments (inputs, constants, outputs) to Run as for the original.
+    static CompiledModule LoadExecutionPlan(const std::string& plan_json, CompileConfig config);
 };
 
 }  // namespace api

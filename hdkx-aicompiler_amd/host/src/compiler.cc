@@ -1,6 +1,7 @@
 // compiler.cc -- Compiler::Compile and CompiledModule (see compiler.h).
 #include "kxc/compiler.h"
 #include "kxc/profiling.h"
+#include "json_reader.h"
 
 #include <dlfcn.h>
 #include <unistd.h>
@@ -56,6 +57,7 @@ public:
     // hip back end
     kxc_hip_plan* plan = nullptr;
     std::vector<kxc_hip_module*> modules;
+    std::vector<std::string> module_sources;     // one per entry of modules (dry builds keep the sources only)
     size_t workspace_bytes = 0;
     bool ready = false;
 
@@ -395,6 +397,7 @@ private:
         }
         kxc_hip_module* module = nullptr;
         std::vector<char> log(16384, 0);
+        m_->module_sources.push_back(src.source);
         if (dry_) {
             size_t size = 0;
             if (kxc_hip_module_compile_only(src.source.c_str(), "kxc_generated.hip", &size, log.data(), log.size()))
@@ -581,15 +584,84 @@ std::string CompiledModule::ExecutionPlanJSON() const {
     os << "],\"nodes\":[";
     for (size_t i = 0; i < impl_->execs.size(); ++i) {
         const auto& e = impl_->execs[i];
-        os << (i ? "," : "") << "{\"kind\":\"kernel_exec\",\"op_name\":\"" << e.op_name << "\",\"kernel_symbol\":\""
-           << e.kernel_symbol << "\",\"input_values\":[";
+        os << (i ? "," : "") << "{\"kind\":\"kernel\",\"input_values\":[";
         for (size_t k = 0; k < e.input_values.size(); ++k) os << (k ? "," : "") << e.input_values[k];
         os << "],\"output_values\":[";
         for (size_t k = 0; k < e.output_values.size(); ++k) os << (k ? "," : "") << e.output_values[k];
-        os << "],\"worker_set\":[0]}";
+        os << "],\"worker_set\":[0],\"op_name\":\"" << json::Escape(e.op_name) << "\",\"kernel_symbol\":\""
+           << json::Escape(e.kernel_symbol) << "\"}";
     }
-    os << "]}";
+    os << "]";
+    // Beyond the reference's schema (src/base/execution_plan.cc:674-877 keeps value ids and kernel symbols):
+    // what is needed to run the function again without compiling it -- see Compiler::LoadExecutionPlan.
+    os << ",\"kxc_hip\":{\"target_kind\":\"" << json::Escape(impl_->config->target->kind) << "\",\"input_count\":"
+       << impl_->input_count << ",\"constant_count\":" << impl_->constant_count << ",\"workspace_bytes\":"
+       << impl_->workspace_bytes << ",\"generated_modules\":[";
+    for (size_t i = 0; i < impl_->module_sources.size(); ++i)
+        os << (i ? "," : "") << "\"" << json::Escape(impl_->module_sources[i]) << "\"";
+    os << "]";
+    if (impl_->plan && impl_->ready) {     // a build without a GPU records launches but cannot run them
+        size_t needed = 0;
+        if (kxc_hip_plan_serialize(impl_->plan, nullptr, 0, &needed))
+            throw std::runtime_error(std::string("ExecutionPlanJSON: ") + kxc_hip_last_error());
+        std::string text(needed, '\0');
+        if (kxc_hip_plan_serialize(impl_->plan, &text[0], text.size(), &needed))
+            throw std::runtime_error(std::string("ExecutionPlanJSON: ") + kxc_hip_last_error());
+        text.resize(needed - 1);
+        os << ",\"launch_plan\":\"" << json::Escape(text) << "\"";
+    }
+    os << "}}";
     return os.str();
+}
+
+CompiledModule Compiler::LoadExecutionPlan(const std::string& plan_json, CompileConfig config) {
+    if (!config.defined() || !config->target.defined() || config->target->kind != "hip")
+        throw std::runtime_error("LoadExecutionPlan: a hip target is required");
+    if (config->target->attrs.exists == 0) throw std::runtime_error("LoadExecutionPlan: no GPU to load the plan on");
+    profiling::EventSpec spec;
+    spec.component = "compiler";
+    spec.event_type = "load_execution_plan";
+    profiling::ScopedSpan span = profiling::CurrentSpan(spec);
+    const json::Value root = json::Reader(plan_json).Parse();
+    if (root.at("schema_version").integer != 1) throw std::runtime_error("LoadExecutionPlan: unsupported schema_version");
+    const json::Value& hip = root.at("kxc_hip");
+    if (hip.at("target_kind").string != "hip" || !hip.has("launch_plan"))
+        throw std::runtime_error("LoadExecutionPlan: the plan carries no launch description for the hip target");
+    auto impl = std::make_shared<CompiledModuleImpl>();
+    impl->config = config;
+    impl->input_count = hip.at("input_count").integer;
+    impl->constant_count = hip.at("constant_count").integer;
+    impl->num_values = static_cast<int>(root.at("num_values").integer);
+    impl->output_value = static_cast<int>(root.at("output_value").integer);
+    for (const auto& v : root.at("input_value_ids").array) impl->input_value_ids.push_back(static_cast<int>(v.integer));
+    for (const auto& v : root.at("constant_value_ids").array) impl->constant_value_ids.push_back(static_cast<int>(v.integer));
+    for (const auto& n : root.at("nodes").array) {
+        if (n.at("kind").string != "kernel") throw std::runtime_error("LoadExecutionPlan: only kernel nodes can be replayed");
+        KernelExecInfo e;
+        e.op_name = n.at("op_name").string;
+        e.kernel_symbol = n.at("kernel_symbol").string;
+        for (const auto& v : n.at("input_values").array) e.input_values.push_back(static_cast<int>(v.integer));
+        for (const auto& v : n.at("output_values").array) e.output_values.push_back(static_cast<int>(v.integer));
+        impl->execs.push_back(e);
+    }
+    std::vector<char> log(16384, 0);
+    for (const auto& m : hip.at("generated_modules").array) {
+        kxc_hip_module* module = nullptr;
+        if (kxc_hip_module_compile(m.string.c_str(), "kxc_generated.hip", &module, log.data(), log.size()))
+            throw std::runtime_error(std::string("LoadExecutionPlan: saved kernel source does not compile: ") + kxc_hip_last_error());
+        impl->modules.push_back(module);
+        impl->module_sources.push_back(m.string);
+        impl->source += m.string;
+    }
+    if (kxc_hip_plan_deserialize(hip.at("launch_plan").string.c_str(), config->target->device.device_id(), impl->modules.data(),
+                                 static_cast<int32_t>(impl->modules.size()), &impl->plan))
+        throw std::runtime_error(std::string("LoadExecutionPlan: ") + kxc_hip_last_error());
+    if (kxc_hip_plan_num_nodes(impl->plan) != static_cast<int32_t>(impl->execs.size()))
+        throw std::runtime_error("LoadExecutionPlan: node list and launch plan disagree");
+    impl->workspace_bytes = static_cast<size_t>(hip.at("workspace_bytes").integer);
+    impl->ready = true;
+    impl->status = "loaded from an execution plan";
+    return CompiledModule(impl);
 }
 
 }  // namespace api

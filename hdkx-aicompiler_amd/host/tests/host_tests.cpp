@@ -10,6 +10,7 @@
 //                                            builds the ResNet-18 graph, reads input.bin and const_<k>.bin
 //                                            from <dir>, runs, writes logits.bin and plan.json
 #include <cmath>
+#include <sstream>
 #include <cstdio>
 #include <cstring>
 #include <fstream>
@@ -374,6 +375,20 @@ int RunResNet18(const std::string& dir, int64_t batch, int64_t hw) {
         module.Run(args);
         module.Run(args);      // a second run reuses the plan and its workspace
         api->CopyDataFromTo(dev, args.back(), cpu, logits.data(), logits.size() * sizeof(float));
+        // the saved execution plan runs again without the graph and without compiling it
+        std::ifstream saved(dir + "/plan.json");
+        std::stringstream text;
+        text << saved.rdbuf();
+        auto replay = kxc::api::Compiler::LoadExecutionPlan(text.str(), config);
+        Check(replay.IsReady() && replay.GetKernelExecs().size() == module.GetKernelExecs().size(), "replayed module");
+        std::vector<float> zeros(logits.size(), 0.0f), again(logits.size(), -1.0f);
+        api->CopyDataFromTo(cpu, zeros.data(), dev, args.back(), zeros.size() * sizeof(float));
+        replay.Run(args);
+        api->CopyDataFromTo(dev, args.back(), cpu, again.data(), again.size() * sizeof(float));
+        Check(std::memcmp(again.data(), logits.data(), logits.size() * sizeof(float)) == 0,
+              "replayed execution plan must reproduce the compiled module bit for bit");
+        Check(replay.ExecutionPlanJSON() == text.str(), "a loaded plan serialises to the same JSON");
+        std::cout << "execution plan replayed: " << replay.GetKernelExecs().size() << " launches, identical output\n";
         for (auto* p : args) api->FreeDataSpace(dev, p);
     }
     std::ofstream out(dir + "/logits.bin", std::ios::binary);

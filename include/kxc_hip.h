@@ -299,6 +299,14 @@ int32_t kxc_hip_plan_add_module_kernel(kxc_hip_plan* plan, void* function, const
                                        const uint32_t grid[3], const uint32_t block[3],
                                        uint32_t shared_bytes, const kxc_hip_buf* params,
                                        int32_t num_params);
+/* Text form of a finalized plan (every launch with its descriptor, operands and geometry), so that a compiled
+ * function can be stored and run again without compiling: the launch-level counterpart of the reference's
+ * execution-plan JSON (src/base/execution_plan.cc:674-877), which keeps only value ids and kernel_symbol.
+ * With buffer == NULL only *needed is set.  Deserialising allocates the workspace on device_id; generated
+ * kernels are looked up by name in `modules` (compiled by the caller from the saved source). */
+int32_t kxc_hip_plan_serialize(const kxc_hip_plan* plan, char* buffer, size_t capacity, size_t* needed);
+int32_t kxc_hip_plan_deserialize(const char* text, int32_t device_id, kxc_hip_module* const* modules,
+                                 int32_t num_modules, kxc_hip_plan** out_plan);
 /* Allocate the workspace (bytes = the largest offset + size the nodes use). */
 int32_t kxc_hip_plan_finalize(kxc_hip_plan* plan, size_t workspace_bytes);
 /* Enqueue every node on `stream`; returns after enqueue (no synchronisation). */
