@@ -199,36 +199,37 @@ conv_mfma_kernel(const ConvArgs a) {
 #pragma unroll
             for (int g = 0; g < 16; ++g) acc[i][j][g] = 0.0f;
 
-    auto issue_loads = [&](int chunk, float* xs, float* ws) {
+    // The loads of one chunk as NOPS separate operations (CC*PPT patch segments, then WPT weight segments), so
+    // that the main loop can issue them a few at a time between matrix instructions instead of in one burst
+    // during which the wave feeds nothing to the matrix pipe.
+    constexpr int NOPS = CC * PPT + WPT;
+    auto issue_op = [&](int j, int chunk, float* xs, float* ws) {
         const int c0 = chunk * CC;
-        if (c0 + CC > a.C && chunk >= KS) weight_table(a.C - c0);   // partial last chunk (rare)
-#pragma unroll
-        for (int cl = 0; cl < CC; ++cl) {
-            if (c0 + cl < a.C) {
-                const uint32_t soff = static_cast<uint32_t>(c0 + cl) * static_cast<uint32_t>(HW) * 4u;
-#pragma unroll
-                for (int i = 0; i < PPT; ++i) {
-                    const int seg = wave + i * NW;
-                    if (seg < xsegs)
-                        __builtin_amdgcn_raw_ptr_buffer_load_lds(xr, (lds_ptr_t)(xs + cl * a.chs + seg * 64), 4,
-                                                                 goff[i], soff, 0, 0);
-                }
-            } else {
-                // channel beyond C: zero plane (the matching weights are zero too, keep the product exact)
-#pragma unroll
-                for (int i = 0; i < PPT; ++i) {
-                    const int seg = wave + i * NW;
-                    if (seg < xsegs) xs[cl * a.chs + seg * 64 + lane] = 0.0f;
+        if (j < CC * PPT) {
+            const int cl = j / PPT, i = j - cl * PPT;
+            const int seg = wave + i * NW;
+            if (seg < xsegs) {
+                if (c0 + cl < a.C) {
+                    const uint32_t soff = static_cast<uint32_t>(c0 + cl) * static_cast<uint32_t>(HW) * 4u;
+                    __builtin_amdgcn_raw_ptr_buffer_load_lds(xr, (lds_ptr_t)(xs + cl * a.chs + seg * 64), 4, goff[i], soff, 0, 0);
+                } else {
+                    // channel beyond C: zero plane (the matching weights are zero too, keep the product exact)
+                    xs[cl * a.chs + seg * 64 + lane] = 0.0f;
                 }
             }
-        }
-        const uint32_t wsoff = static_cast<uint32_t>(c0) * KHW * 4u;
-#pragma unroll
-        for (int i = 0; i < WPT; ++i) {
+        } else {
+            const int i = j - CC * PPT;
             const int seg = wave + i * NW;
-            if (seg < WSEG)
+            if (seg < WSEG) {
+                const uint32_t wsoff = static_cast<uint32_t>(c0) * KHW * 4u;
                 __builtin_amdgcn_raw_ptr_buffer_load_lds(wr, (lds_ptr_t)(ws + seg * 64), 4, woff[i], wsoff, 0, 0);
+            }
         }
+    };
+    auto issue_loads = [&](int chunk, float* xs, float* ws) {
+        if (chunk * CC + CC > a.C && chunk >= KS) weight_table(a.C - chunk * CC);   // partial last chunk (rare)
+#pragma unroll
+        for (int j = 0; j < NOPS; ++j) issue_op(j, chunk, xs, ws);
     };
 
     if (kgroup < a.nchunks) issue_loads(kgroup, xs0, ws0);
@@ -239,8 +240,12 @@ conv_mfma_kernel(const ConvArgs a) {
         const int chunk = it * KS + kgroup;
         const float* xs = (it & 1) ? xs1 : xs0;
         const float* ws = (it & 1) ? ws1 : ws0;
-        if (chunk + KS < a.nchunks) issue_loads(chunk + KS, (it & 1) ? xs0 : xs1, (it & 1) ? ws0 : ws1);
+        const bool has_next = chunk + KS < a.nchunks;
+        float* const nxs = (it & 1) ? xs0 : xs1;
+        float* const nws = (it & 1) ? ws0 : ws1;
+        if (has_next && (chunk + KS) * CC + CC > a.C) weight_table(a.C - (chunk + KS) * CC);   // partial last chunk (rare)
         if (chunk < a.nchunks) {
+        constexpr int OPS_PER_STEP = (NOPS + NS - 1) / NS;
 
         // k-steps of this chunk: step = pair * KHW + tap.  Operands are fetched from LDS PF steps ahead of
         // the matrix instruction that consumes them (rotating register sets; all indices are compile-time
@@ -275,6 +280,13 @@ conv_mfma_kernel(const ConvArgs a) {
                 for (int j = 0; j < RP; ++j)
                     acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x2f32(av[step % (PF + 1)][i], bv[step % (PF + 1)][j],
                                                                      acc[i][j], 0, 0, 0);
+            __builtin_amdgcn_sched_barrier(0);
+            // next chunk's loads, a few per k-step, issued while this step's matrix instructions execute
+            if (has_next) {
+#pragma unroll
+                for (int u = 0; u < OPS_PER_STEP; ++u)
+                    if (step * OPS_PER_STEP + u < NOPS) issue_op(step * OPS_PER_STEP + u, chunk + KS, nxs, nws);
+            }
             __builtin_amdgcn_sched_barrier(0);
         }
         }
