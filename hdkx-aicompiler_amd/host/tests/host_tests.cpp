@@ -19,6 +19,7 @@
 
 #include "kxc/compiler.h"
 #include "kxc/models.h"
+#include "kxc/onnx_importer.h"
 #include "kxc/profiling.h"
 #include "kxc/topi.h"
 
@@ -448,6 +449,84 @@ int RunCodegen() {
 
 }  // namespace
 
+// onnx <cpu|hip|hipgen> <dir>: loads <dir>/model.import.json + <dir>/model.params.bin (the reference's ONNX import
+// wire format), compiles the imported function for the target and runs it on the input pattern of the
+// reference's acceptance test (test/onnx_importer_test.cpp:138-144); writes <dir>/logits.bin.
+int RunOnnx(const std::string& dir) {
+    kxc::frontend::ImportedONNXModel imported =
+        kxc::frontend::LoadONNXImportSpec(dir + "/model.import.json", dir + "/model.params.bin");
+    Check(imported.function.defined(), "importer should construct a Relay Function");
+    Check(imported.input_names.size() == 1 && imported.output_names.size() == 1, "one input, one output");
+    Check(imported.params.size() == imported.param_order.size(), "every parameter is kept");
+    std::cout << "imported: " << imported.param_order.size() << " params, input " << imported.input_names[0] << ", output "
+              << imported.output_names[0] << "\n";
+    auto config = MakeConfig();
+    auto module = kxc::api::Compiler::Compile(imported.function, config);
+    Check(module.input_count() == 1, "one function input");
+    Check(static_cast<size_t>(module.constant_count()) == imported.param_order.size(), "every parameter becomes a constant argument");
+    if (!module.IsReady()) { std::cout << "module not loadable here (no GPU)\n"; return 0; }
+    // shapes of the input and the output come from the typed function
+    kxc::Function typed = kxc::relay::InferTypePass(imported.function);
+    auto elements = [](const kxc::Type& t) {
+        size_t n = 1;
+        for (auto d : static_cast<const kxc::TensorTypeNode*>(t.get())->shape) n *= static_cast<size_t>(d);
+        return n;
+    };
+    const size_t in_elems = elements(typed->params[0]->type_annotation), out_elems = elements(typed->body.checked_type());
+    std::vector<float> input(in_elems), output(out_elems, 0.0f);
+    for (size_t i = 0; i < in_elems; ++i) input[i] = (static_cast<float>(i % 251) - 125.0f) / 125.0f;
+    std::vector<std::vector<char>> consts;
+    for (const auto& c : module.GetConstants()) {
+        std::vector<char> bytes(c.nbytes());
+        c.CopyToBytes(bytes.data(), bytes.size());
+        consts.push_back(std::move(bytes));
+    }
+    std::vector<Buf> bufs;
+    bufs.push_back(In(input));
+    for (auto& c : consts) bufs.push_back({c.data(), c.size(), false});
+    bufs.push_back(Out(output));
+    std::vector<void*> args;
+    if (g_mode == "cpu") {
+        for (auto& b : bufs) args.push_back(b.host);
+        module.Run(args);
+    } else {
+        kxc::DeviceAPI* api = kxc::GetDeviceAPI(kxc::kGPU);
+        kxc::Device dev(kxc::kGPU, 0), cpu(kxc::kCPU, 0);
+        for (auto& b : bufs) {
+            void* d = api->AllocDataSpace(dev, b.bytes, 256);
+            if (!b.out) api->CopyDataFromTo(cpu, b.host, dev, d, b.bytes);
+            args.push_back(d);
+        }
+        module.Run(args);
+        api->CopyDataFromTo(dev, args.back(), cpu, output.data(), output.size() * sizeof(float));
+        for (auto* p : args) api->FreeDataSpace(dev, p);
+    }
+    std::ofstream out(dir + "/logits.bin", std::ios::binary);
+    out.write(reinterpret_cast<const char*>(output.data()), static_cast<std::streamsize>(output.size() * sizeof(float)));
+    std::cout << "launches: " << module.GetKernelExecs().size() << "; wrote " << dir << "/logits.bin\n";
+    return 0;
+}
+
+// onnx_errors <dir>: malformed specs raise the reference's messages.
+int RunOnnxErrors(const std::string& dir) {
+    auto expect = [&](const std::string& file, const std::string& needle) {
+        try {
+            kxc::frontend::LoadONNXImportSpec(dir + "/" + file, dir + "/model.params.bin");
+        } catch (const std::exception& e) {
+            Check(std::string(e.what()).find(needle) != std::string::npos, file + ": expected '" + needle + "', got '" + e.what() + "'");
+            return;
+        }
+        throw std::runtime_error(file + ": expected an error");
+    };
+    expect("bad_format.json", "Unsupported ONNX import spec format");
+    expect("bad_op.json", "Unsupported Relay op in ONNX import spec: identity");
+    expect("bad_input.json", "Missing input value 'nowhere' for node 'relu0'");
+    expect("bad_range.json", "Param bytes range out of bounds for: conv1.weight");
+    expect("bad_order.json", "param_order does not match params metadata");
+    std::cout << "onnx error messages ok\n";
+    return 0;
+}
+
 // profile <cpu|hip|hipgen> <bundle dir>: the CNN known-answer model under an active profiling context; the
 // bundle lands in <bundle dir> (the Python tests read it back).
 int RunProfile(const std::string& dir) {
@@ -478,6 +557,8 @@ int main(int argc, char** argv) {
         if (cmd == "op_numeric") { g_mode = argc > 2 ? argv[2] : "cpu"; return RunOpNumeric(); }
         if (cmd == "device_info") return RunDeviceInfo();
         if (cmd == "codegen") return RunCodegen();
+        if (cmd == "onnx" && argc >= 4) { g_mode = argv[2]; return RunOnnx(argv[3]); }
+        if (cmd == "onnx_errors" && argc >= 3) return RunOnnxErrors(argv[2]);
         if (cmd == "profile" && argc >= 4) { g_mode = argv[2]; return RunProfile(argv[3]); }
         if (cmd == "resnet18" && argc >= 6) { g_mode = argv[2]; return RunResNet18(argv[3], std::atoll(argv[4]), std::atoll(argv[5])); }
         std::cerr << "usage: host_tests op_numeric <cpu|hip|hipgen> | device_info | codegen | resnet18 <cpu|hip|hipgen> <dir> <batch> <hw>\n";

@@ -180,3 +180,59 @@ def test_profiling_bundle_hip_events():
         copies = [e for e in events if e["component"] == "device_api" and e["event_type"] == "copy_data_from_to"]
         assert copies and all(c["metrics"]["bytes"] > 0 for c in copies)
         assert summary["component_counts"]["backend.hip"] >= len(kernels)
+
+
+# ------------------------------------------------------------------ ONNX import wire format
+def _onnx_case(synth, d, batch, hw):
+    import copy
+    import onnx_spec
+    consts = synth.resnet18_consts(3)
+    spec, blob = onnx_spec.resnet18_spec(batch, hw, consts)
+    onnx_spec.write(d, spec, blob)
+    return consts, onnx_spec.reference_input(batch, hw), spec
+
+
+def test_onnx_import_cpu_backend_bit_exact(synth):
+    """import.json + params.bin -> Relay function -> CPU back end: the imported ResNet-18 reproduces the CPU
+    oracle bit for bit on the reference's acceptance input pattern (parameters keep their bytes and their order)."""
+    with tempfile.TemporaryDirectory() as d:
+        consts, x, _ = _onnx_case(synth, d, 1, 32)
+        out = run("onnx", "cpu", d)
+        assert "imported: 42 params, input input, output logits" in out
+        got = np.fromfile(os.path.join(d, "logits.bin"), np.float32).reshape(1, 1000)
+        want = Oracle().resnet18(x, consts)
+        assert (bits(got) == bits(want)).all()
+
+
+def test_onnx_import_error_messages(synth):
+    import copy
+    with tempfile.TemporaryDirectory() as d:
+        _, _, spec = _onnx_case(synth, d, 1, 32)
+
+        def variant(name, edit):
+            s = copy.deepcopy(spec)
+            edit(s)
+            with open(os.path.join(d, name), "w") as f:
+                json.dump(s, f)
+
+        variant("bad_format.json", lambda s: s.update(format="kxc.onnx_import.v0"))
+        variant("bad_op.json", lambda s: s["function"]["nodes"][1].update(op_name="identity"))
+        variant("bad_input.json", lambda s: s["function"]["nodes"][1].update(name="relu0", inputs=["nowhere"]))
+        variant("bad_range.json", lambda s: s["params"][0].update(offset=10 ** 12))
+        variant("bad_order.json", lambda s: s.update(param_order=list(reversed(s["param_order"]))))
+        assert "onnx error messages ok" in run("onnx_errors", d)
+
+
+@pytest.mark.gpu
+def test_onnx_import_runs_on_hip(synth):
+    """The same files on the HIP target: the reference's acceptance criterion (max abs error <= 1e-3 or max
+    relative error <= 1e-3 with denominator max(1, |ref|), test/onnx_importer_test.cpp:146-179) against the CPU oracle."""
+    with tempfile.TemporaryDirectory() as d:
+        consts, x, _ = _onnx_case(synth, d, 2, 224)
+        out = run("onnx", "hip", d)
+        assert "launches: 23" in out
+        got = np.fromfile(os.path.join(d, "logits.bin"), np.float32).reshape(2, 1000)
+        want = Oracle(fast=True).resnet18(x, consts)
+        abs_err = np.abs(got - want)
+        rel_err = abs_err / np.maximum(1.0, np.abs(want))
+        assert abs_err.max() <= 1e-3 or rel_err.max() <= 1e-3, (abs_err.max(), rel_err.max())
