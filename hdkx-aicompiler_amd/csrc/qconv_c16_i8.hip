@@ -123,8 +123,6 @@ __global__ void __launch_bounds__(64 * WP) __attribute__((amdgpu_waves_per_eu(2)
     constexpr int KHW = KH * KW;
     constexpr int NS = (KHW * CBC + 1) / 2;          // matrix k-steps per chunk
     constexpr int TP = 32 * WP;
-    constexpr int WSEG = RO * NS;                    // 1 KiB weight segments per chunk
-    constexpr int WPT = (WSEG + WP - 1) / WP;
 
     extern __shared__ __attribute__((aligned(16))) char lds[];
     const int tid = threadIdx.x;
@@ -134,7 +132,7 @@ __global__ void __launch_bounds__(64 * WP) __attribute__((amdgpu_waves_per_eu(2)
     const int r = lane & 31;
 
     const int xs_bytes = CBC * a.chs * 16;
-    const int buf_bytes = xs_bytes + WSEG * 1024;
+    const int buf_bytes = xs_bytes;
     char* const buf0 = lds;
     char* const buf1 = lds + buf_bytes;              // present only when nchunks > 1
 
@@ -190,8 +188,6 @@ __global__ void __launch_bounds__(64 * WP) __attribute__((amdgpu_waves_per_eu(2)
 #pragma unroll
         for (int g = 0; g < 16; ++g) acc[i][g] = 0;
 
-    // packed weights: [(o block)][chunk][NS][64][16]
-    const uint32_t w_chunk_bytes = NS * 1024u;
     auto issue_loads = [&](int chunk, char* buf) {
 #pragma unroll
         for (int cl = 0; cl < CBC; ++cl) {
@@ -206,25 +202,36 @@ __global__ void __launch_bounds__(64 * WP) __attribute__((amdgpu_waves_per_eu(2)
                 }
             }   // a missing channel block keeps stale bytes; its packed weights are zero and integers have no NaN
         }
-#pragma unroll
-        for (int i = 0; i < WPT; ++i) {
-            const int seg = wave + i * WP;
-            if (seg < WSEG) {
-                const int ro = seg / NS, st = seg - ro * NS;
-                const uint32_t soff = (static_cast<uint32_t>(ob0 + ro) * a.nchunks + chunk) * w_chunk_bytes + st * 1024u;
-                load16_to_lds(wr, (lds_ptr_t)(buf + xs_bytes + seg * 1024), static_cast<uint32_t>(lane) * 16u, soff);
-            }
-        }
+        __builtin_amdgcn_sched_barrier(0);
+        asm volatile("" ::: "memory");      // the weight loads below stay behind these in program order
     };
 
+    // Weights do not pass through LDS: the packed layout [o block][chunk][k-step][lane][16] makes a wave's
+    // operand for linear step t = chunk*NS + step ONE contiguous 1 KiB load, shared by the workgroup's waves
+    // through the vector cache.  A ring of D steps is kept in flight across chunk boundaries; loads past the
+    // last step fall outside the buffer and return 0 without a branch.  With the weights out of LDS a workgroup
+    // needs only the patch (12 KiB per buffer for a 56-wide map), which triples the resident workgroups per CU.
+    constexpr int D = (NS % 3 == 0) ? 3 : (NS % 5 == 0 ? 5 : (NS % 2 == 0 ? 2 : 1));
+    const uint32_t total_steps = static_cast<uint32_t>(a.nchunks) * NS;
+    uint32_t wvoff[RO];
+#pragma unroll
+    for (int i = 0; i < RO; ++i) wvoff[i] = static_cast<uint32_t>(ob0 + i) * total_steps * 1024u + static_cast<uint32_t>(lane) * 16u;
+    auto load_a = [&](int i, uint32_t t) -> intx4 {
+        return __builtin_amdgcn_raw_buffer_load_b128(wr, wvoff[i] + (t < total_steps ? t * 1024u : kOob), 0, 0);
+    };
+    intx4 ring[D][RO];
+
     issue_loads(0, buf0);
-    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+#pragma unroll
+    for (int d = 0; d < D; ++d)
+#pragma unroll
+        for (int i = 0; i < RO; ++i) ring[d][i] = load_a(i, d);
+    asm volatile("s_waitcnt vmcnt(%0)" ::"n"(D * RO) : "memory");     // the patch has landed, the ring may still fly
     __syncthreads();
 
     for (int chunk = 0; chunk < a.nchunks; ++chunk) {
         const char* buf = (chunk & 1) ? buf1 : buf0;
         if (chunk + 1 < a.nchunks) issue_loads(chunk + 1, (chunk & 1) ? buf0 : buf1);
-        const char* ws = buf + xs_bytes + lane * 16;
         auto tap_off = [&](int tap) {
             const int t = tap < KHW ? tap : KHW - 1;
             const int rh = t / KW, rw = t - rh * KW;
@@ -240,29 +247,21 @@ __global__ void __launch_bounds__(64 * WP) __attribute__((amdgpu_waves_per_eu(2)
             }
             return *reinterpret_cast<const intx4*>(buf + xbase + off);
         };
+        const uint32_t t0 = static_cast<uint32_t>(chunk) * NS;
         intx4 bcur = fetch_b(0);
-        intx4 acur[RO];
-#pragma unroll
-        for (int i = 0; i < RO; ++i) acur[i] = *reinterpret_cast<const intx4*>(ws + (i * NS) * 1024);
 #pragma unroll
         for (int step = 0; step < NS; ++step) {
             intx4 bnext = bcur;
-            intx4 anext[RO];
+            if (step + 1 < NS) bnext = fetch_b(step + 1);
 #pragma unroll
-            for (int i = 0; i < RO; ++i) anext[i] = acur[i];
-            if (step + 1 < NS) {
-                bnext = fetch_b(step + 1);
+            for (int i = 0; i < RO; ++i)
+                acc[i] = __builtin_amdgcn_mfma_i32_32x32x32_i8(ring[step % D][i], bcur, acc[i], 0, 0, 0);
 #pragma unroll
-                for (int i = 0; i < RO; ++i)
-                    anext[i] = *reinterpret_cast<const intx4*>(ws + (i * NS + step + 1) * 1024);
-            }
-#pragma unroll
-            for (int i = 0; i < RO; ++i) acc[i] = __builtin_amdgcn_mfma_i32_32x32x32_i8(acur[i], bcur, acc[i], 0, 0, 0);
+            for (int i = 0; i < RO; ++i) ring[step % D][i] = load_a(i, t0 + step + D);
             bcur = bnext;
-#pragma unroll
-            for (int i = 0; i < RO; ++i) acur[i] = anext[i];
         }
-        asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+        // every load older than the D*RO ring refills just issued has completed: that includes the next patch
+        asm volatile("s_waitcnt vmcnt(%0)" ::"n"(D * RO) : "memory");
         __syncthreads();
     }
 
@@ -666,8 +665,7 @@ int32_t PrepareUncached(const kxc_hip_qconv2d_desc* d, QLaunch* L, const char* w
         const int segs = (positions + 63) / 64;
         if (segs > v.ppt * v.wp) continue;
         const int chs = segs * 64;
-        const int NS = (v.kh * v.kw * cbc + 1) / 2;
-        const size_t buf = static_cast<size_t>(cbc) * chs * 16 + static_cast<size_t>(v.ro) * NS * 1024;
+        const size_t buf = static_cast<size_t>(cbc) * chs * 16;      // the patch only; weights stream from memory
         const size_t lds = buf * (a.nchunks > 1 ? 2 : 1);
         if (lds > 160 * 1024) continue;
         const int64_t tiles = CeilDiv(M, TP) * ((a.O / 32) / v.ro);
