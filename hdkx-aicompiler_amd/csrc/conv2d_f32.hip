@@ -48,6 +48,7 @@ struct ConvArgs {
     int32_t N, C, H, W, O, OH, OW;
     int32_t sh, sw, ph, pw, dh, dw;
     int32_t Hp, Wp;      // padded input extent: H + 2*ph, W + 2*pw
+    int32_t Hv, row_step;   // rows the matrix kernel sees and their distance in input rows (see RowView)
     int32_t M;           // N*OH*OW output pixels
     int32_t OHW;
     int32_t chs;         // LDS floats per patch channel (>= rows*Wp, padded)
@@ -155,8 +156,8 @@ conv_mfma_kernel(const ConvArgs a) {
         const int q = fast_div(pos, a.div_wp), col = pos - q * a.Wp;
         const int Q = qmin + q;
         const int n = fast_div(Q, a.div_hp), ih = Q - n * a.Hp - a.ph, iw = col - a.pw;
-        const bool ok = pos < P && n < a.N && ih >= 0 && ih < a.H && iw >= 0 && iw < a.W;
-        goff[i] = ok ? static_cast<uint32_t>(((n * a.C) * a.H + ih) * a.W + iw) * 4u : kOobOffset;
+        const bool ok = pos < P && n < a.N && ih >= 0 && ih < a.Hv && iw >= 0 && iw < a.W;
+        goff[i] = ok ? static_cast<uint32_t>(((n * a.C) * a.H + ih * a.row_step) * a.W + iw) * 4u : kOobOffset;
     }
     // weight tile element L = plane*PL + row*KS2 + col, col = pair*KHW + tap, channel = 2*pair + plane
     uint32_t woff[WPT];
@@ -429,6 +430,9 @@ const Variant kVariants[] = {
     KXC_VARIANT(1, 1, 8, 2, 2, 1, 1, 6),   // 64 x 64
     KXC_VARIANT(1, 1, 8, 1, 4, 1, 1, 4),   // 32 x 128
     KXC_VARIANT(1, 1, 16, 2, 2, 1, 1, 6),
+    KXC_VARIANT_KS(1, 1, 8, 1, 4, 1, 1, 4, 2),   // reduction split inside the workgroup for small launches
+    KXC_VARIANT_KS(1, 1, 8, 1, 4, 1, 1, 4, 4),
+    KXC_VARIANT_KS(1, 1, 8, 1, 2, 1, 1, 8, 8),
     KXC_VARIANT(7, 7, 2, 1, 8, 1, 1, 8),   // 32 x 256; 2-channel chunks: two chunks for RGB, loads overlap compute
     KXC_VARIANT(7, 7, 2, 1, 7, 1, 1, 8),   // 32 x 224: two full output rows of a 112-wide map
     KXC_VARIANT(7, 7, 4, 1, 8, 1, 1, 8),   // 32 x 256, one chunk (3 input channels padded to 4)
@@ -506,8 +510,11 @@ void Select(const ConvArgs& a, int kh, int kw, Choice* choice) {
     // split inside the workgroup -- two ways on the 32x128 tile if that is enough, else four or eight ways on
     // the 32x64 tile (measured: layer4 43% -> 53% of peak, batch-1 layers 1.6x faster).
     constexpr int64_t kEnoughWaves = 3 * 4 * kNumCUs;
-    static const char* const kSplitOrder[] = {"mfma_k3x3_c4_o1x1_p4x1_ks2", "mfma_k3x3_c4_o1x1_p2x1_ks4",
-                                              "mfma_k3x3_c4_o1x1_p2x1_ks8"};
+    static const char* const kSplitOrder3x3[] = {"mfma_k3x3_c4_o1x1_p4x1_ks2", "mfma_k3x3_c4_o1x1_p2x1_ks4",
+                                                 "mfma_k3x3_c4_o1x1_p2x1_ks8"};
+    static const char* const kSplitOrder1x1[] = {"mfma_k1x1_c8_o1x1_p4x1_ks2", "mfma_k1x1_c8_o1x1_p4x1_ks4",
+                                                 "mfma_k1x1_c8_o1x1_p2x1_ks8"};
+    const char* const* kSplitOrder = kh == 1 ? kSplitOrder1x1 : kSplitOrder3x3;
     Choice first_fit;
     int64_t first_waves = 0;
     Choice split[3];
@@ -557,11 +564,18 @@ int32_t FillArgs(const kxc_hip_conv2d_desc* d, ConvArgs* a, const char* who) {
     a->OW = static_cast<int32_t>(nw / d->stride_w + 1);
     a->sh = d->stride_h; a->sw = d->stride_w; a->ph = d->pad_h; a->pw = d->pad_w; a->dh = d->dil_h; a->dw = d->dil_w;
     a->Hp = d->h + 2 * d->pad_h; a->Wp = d->w + 2 * d->pad_w;
+    a->Hv = d->h; a->row_step = 1;
     a->OHW = a->OH * a->OW;
     const int64_t M = static_cast<int64_t>(d->n) * a->OHW;
     a->M = M < (1LL << 31) ? static_cast<int32_t>(M) : 0;
     a->flags = d->flags;
     return KXC_HIP_OK;
+}
+
+void ApplyRowView(ConvArgs* a, int kh) {
+    if (kh == 1 && a->ph == 0 && a->sh > 1) {
+        a->Hv = a->OH; a->Hp = a->OH; a->row_step = a->sh; a->sh = 1;
+    }
 }
 
 }  // namespace
@@ -572,6 +586,7 @@ const char* kxc_hip_conv2d_variant(const kxc_hip_conv2d_desc* desc) {
     ConvArgs a;
     if (FillArgs(desc, &a, "kxc_hip_conv2d_variant") != KXC_HIP_OK) return "invalid";
     if (desc->flags & KXC_HIP_CONV_FORCE_DIRECT) return "direct";
+    ApplyRowView(&a, desc->kh);
     Choice c;
     Select(a, desc->kh, desc->kw, &c);
     return c.v ? c.v->name : "direct";
@@ -592,6 +607,11 @@ int32_t kxc_hip_conv2d_nchw_f32(const kxc_hip_conv2d_desc* desc, const float* x,
     a.w_bytes = static_cast<uint32_t>(static_cast<int64_t>(a.O) * a.C * desc->kh * desc->kw * 4);
     hipStream_t s = ResolveStream(stream);
 
+    // A filter one row high with a vertical stride touches only every stride-th input row (the 1x1/2
+    // downsample convolutions): the matrix kernel then sees an image of OH rows that are stride rows apart, so
+    // the skipped rows are neither loaded nor staged.
+    ConvArgs direct_args = a;
+    ApplyRowView(&a, desc->kh);
     Choice c;
     if (!(desc->flags & KXC_HIP_CONV_FORCE_DIRECT) && a.M > 0) Select(a, desc->kh, desc->kw, &c);
     if (c.v) {
@@ -622,7 +642,7 @@ int32_t kxc_hip_conv2d_nchw_f32(const kxc_hip_conv2d_desc* desc, const float* x,
     }
     int64_t g = CeilDiv(total, 256);
     if (g > 256 * 64) g = 256 * 64;
-    conv_direct_kernel<<<NoteGrid(static_cast<int>(g)), NoteBlock(256), NoteLds(0), s>>>(a, desc->kh, desc->kw, total);
+    conv_direct_kernel<<<NoteGrid(static_cast<int>(g)), NoteBlock(256), NoteLds(0), s>>>(direct_args, desc->kh, desc->kw, total);
     return CheckLaunch("conv_direct");
 }
 
