@@ -33,6 +33,10 @@ struct Node {
     float f[2];
     int32_t i32[4];
     int64_t a_shape[6], b_shape[6];
+    // concurrency: lane 1 = runs on the plan's side stream, concurrently with the main-lane nodes enqueued
+    // after it; `join` = this (main-lane) node first waits for every side-lane node enqueued before it
+    int32_t lane = 0, join = 0;
+    hipEvent_t fork_event = nullptr, done_event = nullptr;
     // module kernel
     void* function = nullptr;
     uint32_t grid[3], block[3], shared_bytes = 0;
@@ -48,6 +52,7 @@ struct kxc_hip_plan {
     void* workspace = nullptr;
     size_t workspace_bytes = 0;
     bool finalized = false;
+    hipStream_t side_stream = nullptr;     // created at finalize when a node uses lane 1 (default priority)
 };
 
 namespace {
@@ -102,6 +107,11 @@ int32_t kxc_hip_plan_destroy(kxc_hip_plan* plan) {
     if (!plan) return KXC_HIP_OK;
     hipError_t e = hipSuccess;
     if (plan->workspace) e = hipFree(plan->workspace);
+    for (Node& n : plan->nodes) {
+        if (n.fork_event) (void)hipEventDestroy(n.fork_event);
+        if (n.done_event) (void)hipEventDestroy(n.done_event);
+    }
+    if (plan->side_stream) (void)hipStreamDestroy(plan->side_stream);
     delete plan;
     KXC_HIP_CALL(e, "plan workspace free");
     return KXC_HIP_OK;
@@ -409,6 +419,15 @@ int32_t kxc_hip_plan_finalize(kxc_hip_plan* plan, size_t workspace_bytes) {
         KXC_HIP_CALL(hipMalloc(&plan->workspace, workspace_bytes), "plan workspace allocation");
     }
     plan->workspace_bytes = workspace_bytes;
+    for (Node& n : plan->nodes) {
+        if (n.lane != 1) continue;
+        if (!plan->side_stream) {
+            KXC_HIP_CALL(hipSetDevice(plan->device_id), "HIP SetDevice");
+            KXC_HIP_CALL(hipStreamCreateWithFlags(&plan->side_stream, hipStreamNonBlocking), "plan side stream");
+        }
+        KXC_HIP_CALL(hipEventCreateWithFlags(&n.fork_event, hipEventDisableTiming), "plan event");
+        KXC_HIP_CALL(hipEventCreateWithFlags(&n.done_event, hipEventDisableTiming), "plan event");
+    }
     plan->finalized = true;
     return KXC_HIP_OK;
 }
@@ -541,8 +560,37 @@ extern "C" {
 int32_t kxc_hip_plan_run(kxc_hip_plan* plan, void** args, void* stream) {
     if (int32_t rc = CheckRunArgs(plan, args, "kxc_hip_plan_run")) return rc;
     void* s = stream ? stream : static_cast<void*>(CurrentStream());
-    for (Node& n : plan->nodes)
+    hipStream_t main_stream = reinterpret_cast<hipStream_t>(s);
+    std::vector<Node*> unjoined;      // side-lane nodes the main lane has not waited for yet
+    for (Node& n : plan->nodes) {
+        if (n.lane == 1 && plan->side_stream) {
+            // everything enqueued so far on the main lane happens before the side node; the side node then runs
+            // concurrently with the main-lane nodes that follow, until a node marked `join`
+            KXC_HIP_CALL(hipEventRecord(n.fork_event, main_stream), "hipEventRecord");
+            KXC_HIP_CALL(hipStreamWaitEvent(plan->side_stream, n.fork_event, 0), "hipStreamWaitEvent");
+            if (int32_t rc = RunNode(plan, n, args, plan->side_stream)) return rc;
+            KXC_HIP_CALL(hipEventRecord(n.done_event, plan->side_stream), "hipEventRecord");
+            unjoined.push_back(&n);
+            continue;
+        }
+        if (n.join) {
+            for (Node* side : unjoined) KXC_HIP_CALL(hipStreamWaitEvent(main_stream, side->done_event, 0), "hipStreamWaitEvent");
+            unjoined.clear();
+        }
         if (int32_t rc = RunNode(plan, n, args, s)) return rc;
+    }
+    for (Node* side : unjoined) KXC_HIP_CALL(hipStreamWaitEvent(main_stream, side->done_event, 0), "hipStreamWaitEvent");
+    return KXC_HIP_OK;
+}
+
+int32_t kxc_hip_plan_set_concurrency(kxc_hip_plan* plan, int32_t node, int32_t lane, int32_t join) {
+    const char* who = "kxc_hip_plan_set_concurrency";
+    KXC_PLAN_BEGIN(who);
+    KXC_HIP_REQUIRE(node >= 0 && node < static_cast<int32_t>(plan->nodes.size()), "%s: node %d out of range", who, node);
+    KXC_HIP_REQUIRE((lane == 0 || lane == 1) && (join == 0 || join == 1) && !(lane == 1 && join == 1),
+                    "%s: lane must be 0 or 1, join 0 or 1, and a side-lane node cannot join", who);
+    plan->nodes[node].lane = lane;
+    plan->nodes[node].join = join;
     return KXC_HIP_OK;
 }
 
@@ -634,6 +682,7 @@ int32_t kxc_hip_plan_serialize(const kxc_hip_plan* plan, char* buffer, size_t ca
         for (uint32_t v : n.grid) I(v);
         for (uint32_t v : n.block) I(v);
         I(n.shared_bytes);
+        I(n.lane); I(n.join);
         I(static_cast<long long>(n.params.size()));
         for (const kxc_hip_buf& b : n.params) { I(b.kind); I(b.index_or_offset); }
         out += "\n";
@@ -690,6 +739,8 @@ int32_t kxc_hip_plan_deserialize(const char* text, int32_t device_id, kxc_hip_mo
         for (uint32_t& g : n.grid) g = static_cast<uint32_t>(I());
         for (uint32_t& b : n.block) b = static_cast<uint32_t>(I());
         n.shared_bytes = static_cast<uint32_t>(I());
+        n.lane = static_cast<int32_t>(I()); n.join = static_cast<int32_t>(I());
+        if (n.lane < 0 || n.lane > 1 || n.join < 0 || n.join > 1) return fail("bad concurrency flags");
         const long long np = I();
         if (!in || np < 0 || np > 4096) return fail("bad parameter count");
         for (long long i = 0; i < np; ++i) {

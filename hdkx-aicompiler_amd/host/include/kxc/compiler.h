@@ -31,6 +31,7 @@ struct CompileConfigNode {
     // HIP back end switches
     bool hip_use_handwritten{true};    // false: every operator goes through the TIR -> HIP generator
     bool hip_fuse{true};               // fold bias / residual add / ReLU into convolution launches
+    bool hip_concurrent_branches{true};   // run a block's downsample convolution beside its first 3x3 convolution
     bool sync_after_run{true};
 };
 class CompileConfig : public Ref<CompileConfigNode> {

@@ -290,6 +290,32 @@ private:
             auto it = group_of_tail_.find(c);
             if (it != group_of_tail_.end()) order.push_back(it->second);
         }
+        // Independent branches: a hand-written convolution whose value is only the residual operand of a later
+        // fused convolution (a block's 1x1 downsample) and that does not depend on the group emitted just before
+        // it moves in front of that group and runs on the plan's side lane, concurrently with it; the consumer
+        // joins.  side_of[g] = group that joins, or -1.
+        std::vector<int> side_join(groups_.size(), -1);
+        std::vector<bool> joins(groups_.size(), false);
+        const char* conc_env = std::getenv("KXC_HIP_CONCURRENT_BRANCHES");     // "0" switches the side lane off
+        if (cfg_->hip_fuse && cfg_->hip_use_handwritten && cfg_->hip_concurrent_branches && !dry_ && !(conc_env && conc_env[0] == '0')) {
+            for (size_t step = 1; step < order.size(); ++step) {
+                const Group& g = groups_[order[step]];
+                const Group& prev = groups_[order[step - 1]];
+                if (!IsOp(g.head, "nn_conv2d") || !IsOp(prev.head, "nn_conv2d") || g.residual || !IsF32(g.head->checked_type_)) continue;
+                if (side_join[order[step - 1]] >= 0 || joins[order[step - 1]]) continue;
+                bool depends = false;
+                for (const auto& a : g.head->args) depends = depends || Resolve(a.get()) == prev.tail;
+                if (depends) continue;
+                int consumer = -1;
+                for (size_t later = step + 1; later < order.size() && consumer < 0; ++later)
+                    if (groups_[order[later]].residual == g.tail) consumer = static_cast<int>(order[later]);
+                const CallNode* sole = SoleConsumer(g.tail);
+                if (consumer < 0 || !sole || !IsOp(sole, "add")) continue;
+                side_join[order[step]] = consumer;
+                joins[consumer] = true;
+                std::swap(order[step - 1], order[step]);
+            }
+        }
         // last reader of every (resolved) value, in emission steps; alias ops are transparent
         std::unordered_map<const RelayExprNode*, int> last_use;
         std::vector<bool> is_alias(groups_.size(), false);
@@ -308,6 +334,17 @@ private:
             if (g.residual) last_use[Resolve(g.residual)] = static_cast<int>(step);
         }
         last_use[Resolve(f_->body.get())] = static_cast<int>(order.size());
+        // a side-lane launch may still be reading its operands until the join has been enqueued
+        for (size_t step = 0; step < order.size(); ++step) {
+            if (side_join[order[step]] < 0) continue;
+            int join_step = static_cast<int>(step);
+            for (size_t later = step + 1; later < order.size(); ++later)
+                if (static_cast<int>(order[later]) == side_join[order[step]]) join_step = static_cast<int>(later);
+            for (const auto& a : groups_[order[step]].head->args) {
+                int& lu = last_use[Resolve(a.get())];
+                if (lu < join_step) lu = join_step;
+            }
+        }
 
         for (size_t step = 0; step < order.size(); ++step) {
             const Group& g = groups_[order[step]];
@@ -340,6 +377,7 @@ private:
             info.output_values.push_back(value_id_.at(g.tail));
 
             std::string symbol;
+            const int32_t first_node = kxc_hip_plan_num_nodes(m_->plan);
             const auto* dispatch = cfg_->hip_use_handwritten ? OpAttr<relay::FHIPDispatch>(op, "FHIPDispatch") : nullptr;
             if (OpFlag(op, "THIPAlias")) {
                 // a view that is the function's result: materialise it with a copy
@@ -353,6 +391,11 @@ private:
             if (!symbol.empty()) {
                 info.kernel_symbol = symbol;
                 m_->execs.push_back(info);
+                const int32_t added = kxc_hip_plan_num_nodes(m_->plan) - first_node;
+                const bool side = side_join[order[step]] >= 0 && added == 1;
+                if ((side || joins[order[step]]) && added >= 1 &&
+                    kxc_hip_plan_set_concurrency(m_->plan, first_node, side ? 1 : 0, joins[order[step]] ? 1 : 0))
+                    throw std::runtime_error(std::string("plan_set_concurrency failed: ") + kxc_hip_last_error());
             } else {
                 if (g.fused_relu || g.residual) throw std::runtime_error("hip back end: operator declined a fused launch: " + op->name);
                 EmitGenerated(g, ctx, info, static_cast<int>(step));

@@ -307,6 +307,13 @@ int32_t kxc_hip_plan_add_module_kernel(kxc_hip_plan* plan, void* function, const
 int32_t kxc_hip_plan_serialize(const kxc_hip_plan* plan, char* buffer, size_t capacity, size_t* needed);
 int32_t kxc_hip_plan_deserialize(const char* text, int32_t device_id, kxc_hip_module* const* modules,
                                  int32_t num_modules, kxc_hip_plan** out_plan);
+/* Concurrency inside a plan.  lane = 1 puts node `node` (index in order of the add calls) on the plan's side
+ * stream: it starts after everything added before it and runs concurrently with the main-lane nodes added
+ * after it.  join = 1 on a main-lane node makes it wait first for every side-lane node added before it.  The
+ * caller guarantees that no main-lane node between a side node and its join reads the side node's output or
+ * overwrites a buffer the side node uses.  Without a join the plan run ends with one.  (Independent branches of
+ * a graph -- a residual block's 1x1 downsample next to its 3x3 convolution -- overlap this way.) */
+int32_t kxc_hip_plan_set_concurrency(kxc_hip_plan* plan, int32_t node, int32_t lane, int32_t join);
 /* Allocate the workspace (bytes = the largest offset + size the nodes use). */
 int32_t kxc_hip_plan_finalize(kxc_hip_plan* plan, size_t workspace_bytes);
 /* Enqueue every node on `stream`; returns after enqueue (no synchronisation). */
