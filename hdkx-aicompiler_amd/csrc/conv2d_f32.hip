@@ -85,19 +85,24 @@ typedef __attribute__((address_space(3))) void* lds_ptr_t;
 // LDS tiles and works on chunks g, g+KS, ...; the partial accumulators are added through LDS in group
 // order at the end (deterministic).  It multiplies the waves per output block for launches that have too
 // few 32x32 blocks to occupy 1024 SIMDs (7x7 feature maps, batch 1).
-template <int KH, int KW, int CC, int WO, int WP, int RO, int RP, int PPT, int KS>
+//
+// TPAIR: how the two k values of one matrix instruction are chosen.  false: the same filter tap of two adjacent
+// channels (CC even).  true: two consecutive taps of ONE channel (an odd tap count gets a zero-weight partner):
+// for a 3-channel 7x7 first layer that is 75 k-steps instead of the 98 that pairing channels 2 and "3" costs.
+template <int KH, int KW, int CC, int WO, int WP, int RO, int RP, int PPT, int KS, bool TPAIR = false>
 __global__ void __launch_bounds__(64 * WO * WP * KS) __attribute__((amdgpu_waves_per_eu(2)))
 conv_mfma_kernel(const ConvArgs a) {
     constexpr int NW = WO * WP;                               // waves per reduction group
     constexpr int TO = 32 * RO * WO;
     constexpr int TP = 32 * RP * WP;
     constexpr int KHW = KH * KW;
-    constexpr int KS2 = ((CC / 2) * KHW) | 1;                 // odd row stride of one weight plane
+    constexpr int TPS = (KHW + 1) / 2;                        // tap pairs per channel (TPAIR)
+    constexpr int NS = TPAIR ? CC * TPS : (CC / 2) * KHW;     // matrix k-steps per chunk
+    constexpr int KS2 = NS | 1;                               // odd row stride of one weight plane
     constexpr int PL = (TO * KS2 + 63) / 64 * 64 + 32;        // plane stride: 32 mod 64
     constexpr int WSZ = 2 * PL;                               // floats in the weight tile (multiple of 64)
     constexpr int WSEG = WSZ / 64;                            // 64-float segments of the weight tile
     constexpr int WPT = (WSEG + NW - 1) / NW;                 // weight segments per wave
-    constexpr int NS = (CC / 2) * KHW;                        // matrix k-steps per chunk
     constexpr int PF = (RO * RP >= 4) ? 1 : (RO * RP == 2 ? 2 : 3);   // operand prefetch distance in k-steps
 
     extern __shared__ float lds[];
@@ -159,7 +164,8 @@ conv_mfma_kernel(const ConvArgs a) {
         const bool ok = pos < P && n < a.N && ih >= 0 && ih < a.Hv && iw >= 0 && iw < a.W;
         goff[i] = ok ? static_cast<uint32_t>(((n * a.C) * a.H + ih * a.row_step) * a.W + iw) * 4u : kOobOffset;
     }
-    // weight tile element L = plane*PL + row*KS2 + col, col = pair*KHW + tap, channel = 2*pair + plane
+    // weight tile element L = plane*PL + row*KS2 + col; col = pair*KHW + tap with channel = 2*pair + plane, or
+    // (TPAIR) col = channel*TPS + s with tap = 2*s + plane
     uint32_t woff[WPT];
     auto weight_table = [&](int channels_left) {
 #pragma unroll
@@ -168,9 +174,10 @@ conv_mfma_kernel(const ConvArgs a) {
             const int plane = L >= PL ? 1 : 0;
             const int rem = L - plane * PL;
             const int row = rem / KS2, col = rem - row * KS2;
-            const int pair = col / KHW, tap = col - pair * KHW;
-            const int cl = 2 * pair + plane;
-            const bool ok = L < WSZ && row < TO && col < (CC / 2) * KHW && (o0 + row) < a.O && cl < channels_left;
+            int cl, tap;
+            if (TPAIR) { cl = col / TPS; tap = 2 * (col - cl * TPS) + plane; }
+            else { const int pair = col / KHW; tap = col - pair * KHW; cl = 2 * pair + plane; }
+            const bool ok = L < WSZ && row < TO && col < NS && tap < KHW && (o0 + row) < a.O && cl < channels_left;
             woff[i] = ok ? static_cast<uint32_t>(((o0 + row) * a.C + cl) * KHW + tap) * 4u : kOobOffset;
         }
     };
@@ -185,7 +192,7 @@ conv_mfma_kernel(const ConvArgs a) {
         const int mc = min(m, a.M - 1);
         const int n = fast_div(mc, a.div_ohw), rem = mc - n * a.OHW;
         const int oh = fast_div(rem, a.div_ow), ow = rem - oh * a.OW;
-        xbase[j] = (n * a.Hp + oh * a.sh - qmin) * a.Wp + ow * a.sw + half * a.chs;
+        xbase[j] = (n * a.Hp + oh * a.sh - qmin) * a.Wp + ow * a.sw + (TPAIR ? 0 : half * a.chs);
         ybase[j] = (m < a.M) ? n * a.O * a.OHW + rem : -1;
     }
     int wbase[RO];
@@ -252,10 +259,21 @@ conv_mfma_kernel(const ConvArgs a) {
         // the matrix instruction that consumes them (rotating register sets; all indices are compile-time
         // after unrolling), so the LDS latency is covered by the PF matrix instructions in between.
         auto fetch = [&](int step, float (&av)[RO], float (&bv)[RP]) {
-            const int cp = step / KHW, tap = step - cp * KHW;
-            const int rh = tap / KW, rw = tap - rh * KW;
-            const int koff_x = (2 * cp) * a.chs + rh * a.dh * a.Wp + rw * a.dw;
-            const int koff_w = cp * KHW + tap;
+            int koff_x, koff_w;
+            if (TPAIR) {
+                // lane half h reads tap 2*s + h of channel c; a tap past the end (zero weight) re-reads the last one
+                const int c = step / TPS, s2 = 2 * (step - c * TPS);
+                const int t0 = s2, t1 = s2 + 1 < KHW ? s2 + 1 : KHW - 1;
+                const int off0 = (t0 / KW) * a.dh * a.Wp + (t0 % KW) * a.dw;
+                const int off1 = (t1 / KW) * a.dh * a.Wp + (t1 % KW) * a.dw;
+                koff_x = c * a.chs + (half ? off1 : off0);
+                koff_w = step;
+            } else {
+                const int cp = step / KHW, tap = step - cp * KHW;
+                const int rh = tap / KW, rw = tap - rh * KW;
+                koff_x = (2 * cp) * a.chs + rh * a.dh * a.Wp + rw * a.dw;
+                koff_w = cp * KHW + tap;
+            }
 #pragma unroll
             for (int i = 0; i < RO; ++i) av[i] = ws[wbase[i] + koff_w];
 #pragma unroll
@@ -392,16 +410,19 @@ __global__ void __launch_bounds__(256) conv_direct_kernel(const ConvArgs a, int3
 // ------------------------------------------------------------------------------------------
 struct Variant {
     const char* name;
-    int kh, kw, cc, to, tp, nw, ppt, ks;
+    int kh, kw, cc, to, tp, nw, ppt, ks, tpair;
     void (*kernel)(const ConvArgs);
 };
 
 #define KXC_VARIANT(KH, KW, CC, WO, WP, RO, RP, PPT)                                                   \
     {"mfma_k" #KH "x" #KW "_c" #CC "_o" #WO "x" #RO "_p" #WP "x" #RP, KH, KW, CC, 32 * RO * WO, 32 * RP * WP, \
-     WO * WP, PPT, 1, conv_mfma_kernel<KH, KW, CC, WO, WP, RO, RP, PPT, 1>}
+     WO * WP, PPT, 1, 0, conv_mfma_kernel<KH, KW, CC, WO, WP, RO, RP, PPT, 1>}
 #define KXC_VARIANT_KS(KH, KW, CC, WO, WP, RO, RP, PPT, KS)                                            \
     {"mfma_k" #KH "x" #KW "_c" #CC "_o" #WO "x" #RO "_p" #WP "x" #RP "_ks" #KS, KH, KW, CC, 32 * RO * WO,   \
-     32 * RP * WP, WO * WP, PPT, KS, conv_mfma_kernel<KH, KW, CC, WO, WP, RO, RP, PPT, KS>}
+     32 * RP * WP, WO * WP, PPT, KS, 0, conv_mfma_kernel<KH, KW, CC, WO, WP, RO, RP, PPT, KS>}
+#define KXC_VARIANT_TP(KH, KW, CC, WO, WP, RO, RP, PPT)                                                \
+    {"mfma_k" #KH "x" #KW "_t" #CC "_o" #WO "x" #RO "_p" #WP "x" #RP, KH, KW, CC, 32 * RO * WO, 32 * RP * WP, \
+     WO * WP, PPT, 1, 1, conv_mfma_kernel<KH, KW, CC, WO, WP, RO, RP, PPT, 1, true>}
 
 // name = mfma_k<filter>_c<channels per chunk>_o<waves x blocks along output channels>_p<waves x blocks
 // along pixels>; tile = 32*blocks*waves in each direction.
@@ -433,6 +454,12 @@ const Variant kVariants[] = {
     KXC_VARIANT_KS(1, 1, 8, 1, 4, 1, 1, 4, 2),   // reduction split inside the workgroup for small launches
     KXC_VARIANT_KS(1, 1, 8, 1, 4, 1, 1, 4, 4),
     KXC_VARIANT_KS(1, 1, 8, 1, 2, 1, 1, 8, 8),
+    KXC_VARIANT_TP(7, 7, 1, 1, 8, 2, 1, 8),   // 64 x 256, taps paired, one channel per chunk (double buffered): RGB first layer
+    KXC_VARIANT_TP(7, 7, 1, 1, 8, 1, 1, 8),   // 32 x 256, one channel per chunk
+    KXC_VARIANT_TP(7, 7, 1, 1, 4, 1, 1, 12),  // 32 x 128, one channel per chunk
+    KXC_VARIANT_TP(7, 7, 3, 1, 8, 1, 1, 8),   // 32 x 256, all three channels in one chunk
+    KXC_VARIANT_TP(7, 7, 3, 1, 4, 1, 1, 12),  // 32 x 128
+    KXC_VARIANT_TP(7, 7, 3, 1, 8, 2, 1, 8),   // 64 x 256
     KXC_VARIANT(7, 7, 2, 1, 8, 1, 1, 8),   // 32 x 256; 2-channel chunks: two chunks for RGB, loads overlap compute
     KXC_VARIANT(7, 7, 2, 1, 7, 1, 1, 8),   // 32 x 224: two full output rows of a 112-wide map
     KXC_VARIANT(7, 7, 4, 1, 8, 1, 1, 8),   // 32 x 256, one chunk (3 input channels padded to 4)
@@ -473,7 +500,8 @@ bool Fits(const Variant& v, const ConvArgs& a, Choice* out) {
     // c and c+1 at the same position) fall into different halves of the LDS banks.
     const int32_t chs = static_cast<int32_t>(segs * 64 + 32);
     const int khw = v.kh * v.kw;
-    const int ks2 = ((v.cc / 2) * khw) | 1;
+    if (v.tpair && a.C % 2 == 0) return false;     // pairing taps pays when channels cannot be paired evenly
+    const int ks2 = (v.tpair ? v.cc * ((khw + 1) / 2) : (v.cc / 2) * khw) | 1;
     const int pl = (v.to * ks2 + 63) / 64 * 64 + 32;
     const int nchunks = (a.C + v.cc - 1) / v.cc;
     if (v.ks > 1 && nchunks < 2 * v.ks) return false;          // not enough reduction to split
