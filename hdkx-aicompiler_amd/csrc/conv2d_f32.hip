@@ -111,7 +111,7 @@ conv_mfma_kernel(const ConvArgs a) {
     const int wave_all = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int kgroup = wave_all / NW;
     const int wave = wave_all - kgroup * NW;
-    const int xs_size = CC * a.chs;                           // multiple of 32; tiles start 128-byte aligned
+    const int xs_size = (CC * a.chs + 31) & ~31;              // rounded so that every tile starts 128-byte aligned
     const int iters = (a.nchunks + KS - 1) / KS;              // chunk steps of every reduction group
     // per group: [xs0][ws0][xs1][ws1]; the second pair exists only when a group has more than one chunk
     float* const xs0 = lds + kgroup * (iters > 1 ? 2 : 1) * (xs_size + WSZ);
@@ -498,7 +498,9 @@ bool Fits(const Variant& v, const ConvArgs& a, Choice* out) {
     if (segs > static_cast<int64_t>(v.ppt) * v.nw) return false;
     // Channel stride: a multiple of 64 floats plus 32, so the two half-waves (which read channels
     // c and c+1 at the same position) fall into different halves of the LDS banks.
-    const int32_t chs = static_cast<int32_t>(segs * 64 + 32);
+    // With a horizontal stride of 2 the lanes of a half-wave already use every other bank, so the second
+    // half-wave is skewed by one more float to land on the odd banks.
+    const int32_t chs = static_cast<int32_t>(segs * 64 + 32) + ((a.sw % 2 == 0 && !v.tpair) ? 1 : 0);
     const int khw = v.kh * v.kw;
     if (v.tpair && a.C % 2 == 0) return false;     // pairing taps pays when channels cannot be paired evenly
     const int ks2 = (v.tpair ? v.cc * ((khw + 1) / 2) : (v.cc / 2) * khw) | 1;
@@ -506,7 +508,8 @@ bool Fits(const Variant& v, const ConvArgs& a, Choice* out) {
     const int nchunks = (a.C + v.cc - 1) / v.cc;
     if (v.ks > 1 && nchunks < 2 * v.ks) return false;          // not enough reduction to split
     const int buffers = (nchunks + v.ks - 1) / v.ks > 1 ? 2 : 1;   // a single chunk step needs no second buffer
-    size_t lds = static_cast<size_t>(v.ks) * buffers * (static_cast<size_t>(v.cc) * chs + 2 * static_cast<size_t>(pl)) * sizeof(float);
+    const size_t xs_size = (static_cast<size_t>(v.cc) * chs + 31) & ~static_cast<size_t>(31);
+    size_t lds = static_cast<size_t>(v.ks) * buffers * (xs_size + 2 * static_cast<size_t>(pl)) * sizeof(float);
     const size_t red = static_cast<size_t>(v.ks - 1) * v.to * v.tp * sizeof(float);   // partial accumulators
     if (red > lds) lds = red;
     if (lds > kMaxLdsBytes) return false;
@@ -531,6 +534,7 @@ void Select(const ConvArgs& a, int kh, int kw, Choice* choice) {
     const char* preferred = nullptr;
     if (kh == 3 && a.OW <= 14 && a.M >= 8192) preferred = "mfma_k3x3_c4_o1x1_p8x1";
     if (kh == 3 && a.sh == 2 && a.W >= 56) preferred = "mfma_k3x3_c2_o1x1_p4x1";
+    if (kh == 3 && a.sh == 2 && a.W >= 28 && a.W < 56 && a.O % 64 == 0 && a.M >= 8192) preferred = "mfma_k3x3_c4_o2x1_p8x1";
     if (kh == 3 && a.sh == 1 && a.W >= 56 && a.O % 64 == 0 && a.M >= 65536) preferred = "mfma_k3x3_c4_o1x2_p4x1";
     if (kh == 1 && a.W >= 56 && a.O % 64 == 0 && a.M >= 32768) preferred = "mfma_k1x1_c8_o1x2_p4x2";
     // Pass 0 takes the rule's variant (or the forced one).  Pass 1 takes the first table entry that fits,
