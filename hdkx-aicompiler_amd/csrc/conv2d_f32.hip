@@ -30,6 +30,8 @@
 //    cover (output channels not a multiple of 32, very wide rows) and on request.
 #include <cstdlib>
 #include <cstring>
+#include <mutex>
+#include <vector>
 
 #include "common.h"
 
@@ -49,6 +51,11 @@ struct ConvArgs {
     int32_t sh, sw, ph, pw, dh, dw;
     int32_t Hp, Wp;      // padded input extent: H + 2*ph, W + 2*pw
     int32_t Hv, row_step;   // rows the matrix kernel sees and their distance in input rows (see RowView)
+    // reduction split over workgroups: workgroup (tile, split) reduces chunks [split*cps, min((split+1)*cps, nchunks))
+    // and writes raw partial sums to partial[split][N*O*OH*OW]; a second kernel adds them up (gsplit == 1: off)
+    float* partial;
+    int32_t gsplit, cps;
+    int64_t out_elems;
     int32_t M;           // N*OH*OW output pixels
     int32_t OHW;
     int32_t chs;         // LDS floats per patch channel (>= rows*Wp, padded)
@@ -56,7 +63,7 @@ struct ConvArgs {
     uint32_t x_bytes, w_bytes;
     int32_t p_tiles, o_tiles, num_tiles, tiles_per_xcd, o_fastest;
     uint32_t flags;
-    FastDiv div_wp, div_hp, div_ohw, div_ow, div_otiles, div_ptiles;
+    FastDiv div_wp, div_hp, div_ohw, div_ow, div_otiles, div_ptiles, div_gsplit;
 };
 
 __device__ __forceinline__ float relu_sel(float v) { return (v > 0.0f) ? v : 0.0f; }
@@ -112,7 +119,18 @@ conv_mfma_kernel(const ConvArgs a) {
     const int kgroup = wave_all / NW;
     const int wave = wave_all - kgroup * NW;
     const int xs_size = (CC * a.chs + 31) & ~31;              // rounded so that every tile starts 128-byte aligned
-    const int iters = (a.nchunks + KS - 1) / KS;              // chunk steps of every reduction group
+    // Workgroup -> (tile, split).  The dispatcher hands consecutive workgroups to the 8 XCDs round-robin and every
+    // XCD has its own L2, so workgroup L works on logical unit (L % 8) * units_per_xcd + L / 8: each XCD owns a
+    // contiguous run of tiles and the halo rows / weight slices neighbouring tiles share are fetched into one L2
+    // instead of eight.  Within the run the output-channel tile or the pixel tile varies fastest (host's choice:
+    // whichever operand is larger stays put).
+    const int unit = (blockIdx.x & 7) * a.tiles_per_xcd + (blockIdx.x >> 3);
+    if (unit >= a.num_tiles * a.gsplit || static_cast<int>(blockIdx.x >> 3) >= a.tiles_per_xcd) return;
+    const int tile = a.gsplit > 1 ? fast_div(unit, a.div_gsplit) : unit;
+    const int split = unit - tile * a.gsplit;
+    const int c_lo = split * a.cps;                           // this workgroup's chunks: [c_lo, c_hi)
+    const int c_hi = min(a.nchunks, c_lo + a.cps);
+    const int iters = (c_hi - c_lo + KS - 1) / KS;            // chunk steps of every reduction group
     // per group: [xs0][ws0][xs1][ws1]; the second pair exists only when a group has more than one chunk
     float* const xs0 = lds + kgroup * (iters > 1 ? 2 : 1) * (xs_size + WSZ);
     float* const ws0 = xs0 + xs_size;
@@ -124,13 +142,6 @@ conv_mfma_kernel(const ConvArgs a) {
     const int half = lane >> 5;
     const int r = lane & 31;
 
-    // Workgroup -> tile mapping.  The dispatcher hands consecutive workgroups to the 8 XCDs round-robin and
-    // every XCD has its own L2, so workgroup L works on logical tile (L % 8) * tiles_per_xcd + L / 8: each XCD
-    // owns a contiguous run of tiles and the halo rows / weight slices neighbouring tiles share are fetched
-    // into one L2 instead of eight.  Within the run the output-channel tile or the pixel tile varies fastest
-    // (host's choice: whichever operand is larger stays put).
-    int tile = (blockIdx.x & 7) * a.tiles_per_xcd + (blockIdx.x >> 3);
-    if (tile >= a.num_tiles || (blockIdx.x >> 3) >= a.tiles_per_xcd) return;
     int p_tile, o_tile;
     if (a.o_fastest) { p_tile = fast_div(tile, a.div_otiles); o_tile = tile - p_tile * a.o_tiles; }
     else { o_tile = fast_div(tile, a.div_ptiles); p_tile = tile - o_tile * a.p_tiles; }
@@ -181,7 +192,7 @@ conv_mfma_kernel(const ConvArgs a) {
             woff[i] = ok ? static_cast<uint32_t>(((o0 + row) * a.C + cl) * KHW + tap) * 4u : kOobOffset;
         }
     };
-    weight_table(min(CC, a.C - kgroup * CC));
+    weight_table(min(CC, a.C - (c_lo + kgroup) * CC));
 
     // ---- per-lane operand bases
     int xbase[RP];
@@ -235,24 +246,24 @@ conv_mfma_kernel(const ConvArgs a) {
         }
     };
     auto issue_loads = [&](int chunk, float* xs, float* ws) {
-        if (chunk * CC + CC > a.C && chunk >= KS) weight_table(a.C - chunk * CC);   // partial last chunk (rare)
+        if (chunk * CC + CC > a.C && chunk >= c_lo + KS) weight_table(a.C - chunk * CC);   // partial last chunk (rare)
 #pragma unroll
         for (int j = 0; j < NOPS; ++j) issue_op(j, chunk, xs, ws);
     };
 
-    if (kgroup < a.nchunks) issue_loads(kgroup, xs0, ws0);
+    if (c_lo + kgroup < c_hi) issue_loads(c_lo + kgroup, xs0, ws0);
     asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
     __syncthreads();
 
     for (int it = 0; it < iters; ++it) {
-        const int chunk = it * KS + kgroup;
+        const int chunk = c_lo + it * KS + kgroup;
         const float* xs = (it & 1) ? xs1 : xs0;
         const float* ws = (it & 1) ? ws1 : ws0;
-        const bool has_next = chunk + KS < a.nchunks;
+        const bool has_next = chunk + KS < c_hi;
         float* const nxs = (it & 1) ? xs0 : xs1;
         float* const nws = (it & 1) ? ws0 : ws1;
         if (has_next && (chunk + KS) * CC + CC > a.C) weight_table(a.C - (chunk + KS) * CC);   // partial last chunk (rare)
-        if (chunk < a.nchunks) {
+        if (chunk < c_hi) {
         constexpr int OPS_PER_STEP = (NOPS + NS - 1) / NS;
 
         // k-steps of this chunk: step = pair * KHW + tap.  Operands are fetched from LDS PF steps ahead of
@@ -343,6 +354,23 @@ conv_mfma_kernel(const ConvArgs a) {
     }
 
     // ---- epilogue: accumulator register g of a block holds row 8*(g/4) + 4*half + g%4, column r
+    if (a.gsplit > 1) {
+        // raw partial sums of this split; conv_split_reduce_kernel finishes the layer
+        float* const part = a.partial + static_cast<int64_t>(split) * a.out_elems;
+        if (KS == 1 || kgroup == 0) {
+#pragma unroll
+            for (int i = 0; i < RO; ++i)
+#pragma unroll
+                for (int g = 0; g < 16; ++g) {
+                    const int o = o0 + (wave_o * RO + i) * 32 + 8 * (g / 4) + 4 * half + (g % 4);
+                    if (o >= a.O) continue;
+#pragma unroll
+                    for (int j = 0; j < RP; ++j)
+                        if (ybase[j] >= 0) part[ybase[j] + o * a.OHW] = acc[i][j][g];
+                }
+        }
+        return;
+    }
     const bool has_bias = (a.flags & KXC_HIP_CONV_BIAS) != 0;
     const bool has_res = (a.flags & KXC_HIP_CONV_RESIDUAL) != 0;
     const bool do_relu = (a.flags & KXC_HIP_CONV_RELU) != 0;
@@ -368,6 +396,19 @@ conv_mfma_kernel(const ConvArgs a) {
             }
         }
     }
+}
+
+// Second half of a layer whose reduction was split over workgroups: y = relu(((p0 + p1) + ... ) + bias + residual),
+// the partial sums added in split order (deterministic), then the same epilogue as the unsplit kernel.
+__global__ void __launch_bounds__(256) conv_split_reduce_kernel(const ConvArgs a) {
+    const int64_t e = static_cast<int64_t>(blockIdx.x) * 256 + threadIdx.x;
+    if (e >= a.out_elems) return;
+    float v = a.partial[e];
+    for (int s = 1; s < a.gsplit; ++s) v = __fadd_rn(v, a.partial[static_cast<int64_t>(s) * a.out_elems + e]);
+    if (a.flags & KXC_HIP_CONV_BIAS) v = __fadd_rn(v, a.bias[(e / a.OHW) % a.O]);
+    if (a.flags & KXC_HIP_CONV_RESIDUAL) v = __fadd_rn(v, a.res[e]);
+    if (a.flags & KXC_HIP_CONV_RELU) v = relu_sel(v);
+    a.y[e] = v;
 }
 
 // ------------------------------------------------------------------------------------------
@@ -579,6 +620,31 @@ void Select(const ConvArgs& a, int kh, int kw, Choice* choice) {
     }
 }
 
+// Scratch for the partial sums of a workgroup-split reduction: one grow-only buffer per (device, stream), so
+// that launches on different streams never share one.  Growing frees the old buffer (hipFree waits for the
+// device) and allocates a larger one; in steady state no call allocates.
+int32_t SplitScratch(hipStream_t stream, size_t bytes, float** out) {
+    struct Entry { int device; hipStream_t stream; float* ptr; size_t bytes; };
+    static std::mutex mu;
+    static std::vector<Entry> entries;
+    int dev = 0;
+    KXC_HIP_CALL(hipGetDevice(&dev), "hipGetDevice");
+    std::lock_guard<std::mutex> lock(mu);
+    Entry* e = nullptr;
+    for (Entry& it : entries)
+        if (it.device == dev && it.stream == stream) e = &it;
+    if (!e) { entries.push_back({dev, stream, nullptr, 0}); e = &entries.back(); }
+    if (e->bytes < bytes) {
+        if (e->ptr) KXC_HIP_CALL(hipFree(e->ptr), "hipFree(split scratch)");
+        e->ptr = nullptr; e->bytes = 0;
+        const size_t want = (bytes + (1u << 20) - 1) & ~static_cast<size_t>((1u << 20) - 1);
+        KXC_HIP_CALL(hipMalloc(reinterpret_cast<void**>(&e->ptr), want), "hipMalloc(split scratch)");
+        e->bytes = want;
+    }
+    *out = e->ptr;
+    return KXC_HIP_OK;
+}
+
 int32_t FillArgs(const kxc_hip_conv2d_desc* d, ConvArgs* a, const char* who) {
     KXC_HIP_REQUIRE(d != nullptr, "%s: desc is NULL", who);
     KXC_HIP_REQUIRE(d->n >= 0 && d->c > 0 && d->h > 0 && d->w > 0 && d->o > 0 && d->kh > 0 && d->kw > 0,
@@ -654,7 +720,28 @@ int32_t kxc_hip_conv2d_nchw_f32(const kxc_hip_conv2d_desc* desc, const float* x,
         const int64_t tiles = static_cast<int64_t>(a.p_tiles) * a.o_tiles;
         KXC_HIP_REQUIRE(tiles < (1LL << 30), "kxc_hip_conv2d_nchw_f32: too many tiles");
         a.num_tiles = static_cast<int32_t>(tiles);
-        a.tiles_per_xcd = static_cast<int32_t>(CeilDiv(tiles, 8));
+        // Launches that still leave most SIMDs idle (batch 1, deep layers: a handful of tiles, a long reduction)
+        // split the reduction over workgroups as well; every workgroup keeps at least two chunks per wave group.
+        a.gsplit = 1;
+        a.cps = a.nchunks;
+        a.out_elems = total;
+        {
+            const int64_t waves = tiles * c.v->nw * c.v->ks;
+            int split = 1;
+            while (split < 16 && waves * split < 2048 && a.nchunks / (split * 2) >= 2 * c.v->ks) split *= 2;
+            if (const char* e = std::getenv("KXC_HIP_CONV_GSPLIT")) { const int f = std::atoi(e); if (f >= 1 && f <= a.nchunks) split = f; }
+            if (split > 1) {
+                a.cps = static_cast<int32_t>(CeilDiv(a.nchunks, split));
+                a.gsplit = static_cast<int32_t>(CeilDiv(a.nchunks, a.cps));      // no empty split
+                if (a.gsplit > 1) {
+                    if (int32_t rc = SplitScratch(s, static_cast<size_t>(a.gsplit) * total * sizeof(float), &a.partial)) return rc;
+                } else {
+                    a.cps = a.nchunks;
+                }
+            }
+        }
+        a.div_gsplit = MakeFastDiv(a.gsplit);
+        a.tiles_per_xcd = static_cast<int32_t>(CeilDiv(tiles * a.gsplit, 8));
         a.div_wp = MakeFastDiv(a.Wp); a.div_hp = MakeFastDiv(a.Hp); a.div_ohw = MakeFastDiv(a.OHW);
         a.div_ow = MakeFastDiv(a.OW); a.div_otiles = MakeFastDiv(a.o_tiles); a.div_ptiles = MakeFastDiv(a.p_tiles);
         // weights of one output-channel tile: to * C * kh * kw * 4 bytes; keep the larger operand resident
@@ -670,7 +757,12 @@ int32_t kxc_hip_conv2d_nchw_f32(const kxc_hip_conv2d_desc* desc, const float* x,
                          "hipFuncSetAttribute(MaxDynamicSharedMemorySize)");
         }
         hipLaunchKernelGGL(c.v->kernel, NoteGrid(grid), NoteBlock(dim3(64 * c.v->nw * c.v->ks)), NoteLds(c.lds_bytes), s, a);
-        return CheckLaunch(c.v->name);
+        if (int32_t rc = CheckLaunch(c.v->name)) return rc;
+        if (a.gsplit > 1) {
+            conv_split_reduce_kernel<<<NoteGrid(static_cast<int>(CeilDiv(total, 256))), NoteBlock(256), NoteLds(0), s>>>(a);
+            return CheckLaunch("conv_split_reduce");
+        }
+        return KXC_HIP_OK;
     }
     int64_t g = CeilDiv(total, 256);
     if (g > 256 * 64) g = 256 * 64;

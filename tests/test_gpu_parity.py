@@ -134,6 +134,29 @@ def test_conv_mfma_against_oracle(pkg, fast_orc, synth, shape):
     assert_close(got, want, what=variant + " (bare)")
 
 
+@pytest.mark.parametrize("shape,forced", [((1, 512, 7, 7, 512, 3, 1, 1), None), ((1, 256, 14, 14, 256, 3, 1, 1), None),
+                                          ((1, 256, 14, 14, 512, 1, 2, 0), None), ((1, 256, 14, 14, 512, 3, 2, 1), None),
+                                          ((2, 128, 28, 28, 128, 3, 1, 1), "3"), ((2, 128, 28, 28, 128, 3, 1, 1), "5"),
+                                          ((1, 70, 9, 11, 64, 3, 1, 1), "2")],
+                         ids=lambda v: "x".join(map(str, v)) if isinstance(v, tuple) else str(v))
+def test_conv_reduction_split_over_workgroups(pkg, fast_orc, synth, monkeypatch, shape, forced):
+    """Small launches with a long reduction (batch-1 deep layers) split the channels over workgroups and add the
+    partial sums in a second kernel: same tolerance, bias / residual / ReLU applied once, deterministic."""
+    n, c, h, w, o, k, s, p = shape
+    if forced is not None:
+        monkeypatch.setenv("KXC_HIP_CONV_GSPLIT", forced)
+    x = synth.uniform((n, c, h, w), 6100)
+    wt = synth.normal((o, c, k, k), 6101, float(np.sqrt(2.0 / (c * k * k))))
+    b = synth.uniform((o,), 6102, -0.1, 0.1)
+    oh, ow = (h + 2 * p - k) // s + 1, (w + 2 * p - k) // s + 1
+    skip = synth.uniform((n, o, oh, ow), 6103)
+    want = fast_orc.conv_chain(x, wt, b, s, p, skip=skip, relu=True)
+    got1 = host(pkg.conv2d(dev(x), dev(wt), dev(b), dev(skip), s, p, 1, True))
+    got2 = host(pkg.conv2d(dev(x), dev(wt), dev(b), dev(skip), s, p, 1, True))
+    assert_close(got1, want, what="split reduction %s" % (shape,))
+    assert_bit_exact(got2, got1, "split reduction is deterministic")
+
+
 def test_conv_dilation(pkg, orc, synth):
     x = synth.uniform((1, 8, 20, 20), 300); w = synth.uniform((32, 8, 3, 3), 301)
     want = orc.conv2d(x, w, 1, 2, 2)
