@@ -53,6 +53,13 @@ struct kxc_hip_plan {
     size_t workspace_bytes = 0;
     bool finalized = false;
     hipStream_t side_stream = nullptr;     // created at finalize when a node uses lane 1 (default priority)
+    // HIP graph replay (kxc_hip_plan_enable_graph): the run after the first one on a capturable stream is
+    // captured; later runs with the same argument pointers launch the instantiated graph
+    bool graph_enabled = false;
+    int eager_runs = 0;
+    hipGraph_t graph = nullptr;
+    hipGraphExec_t graph_exec = nullptr;
+    std::vector<void*> graph_args;
 };
 
 namespace {
@@ -112,6 +119,8 @@ int32_t kxc_hip_plan_destroy(kxc_hip_plan* plan) {
         if (n.done_event) (void)hipEventDestroy(n.done_event);
     }
     if (plan->side_stream) (void)hipStreamDestroy(plan->side_stream);
+    if (plan->graph_exec) (void)hipGraphExecDestroy(plan->graph_exec);
+    if (plan->graph) (void)hipGraphDestroy(plan->graph);
     delete plan;
     KXC_HIP_CALL(e, "plan workspace free");
     return KXC_HIP_OK;
@@ -557,10 +566,14 @@ int32_t RunNode(kxc_hip_plan* plan, Node& n, void** args, void* s) {
 
 extern "C" {
 
-int32_t kxc_hip_plan_run(kxc_hip_plan* plan, void** args, void* stream) {
-    if (int32_t rc = CheckRunArgs(plan, args, "kxc_hip_plan_run")) return rc;
-    void* s = stream ? stream : static_cast<void*>(CurrentStream());
-    hipStream_t main_stream = reinterpret_cast<hipStream_t>(s);
+}  // extern "C"
+
+namespace {
+
+// Enqueues every node: main lane on `main_stream`, side-lane nodes on the plan's side stream between a fork and a
+// join event (also the pattern stream capture records as parallel graph branches).
+int32_t EnqueueAll(kxc_hip_plan* plan, void** args, hipStream_t main_stream) {
+    void* s = static_cast<void*>(main_stream);
     std::vector<Node*> unjoined;      // side-lane nodes the main lane has not waited for yet
     for (Node& n : plan->nodes) {
         if (n.lane == 1 && plan->side_stream) {
@@ -580,6 +593,62 @@ int32_t kxc_hip_plan_run(kxc_hip_plan* plan, void** args, void* stream) {
         if (int32_t rc = RunNode(plan, n, args, s)) return rc;
     }
     for (Node* side : unjoined) KXC_HIP_CALL(hipStreamWaitEvent(main_stream, side->done_event, 0), "hipStreamWaitEvent");
+    return KXC_HIP_OK;
+}
+
+void DropGraph(kxc_hip_plan* plan) {
+    if (plan->graph_exec) (void)hipGraphExecDestroy(plan->graph_exec);
+    if (plan->graph) (void)hipGraphDestroy(plan->graph);
+    plan->graph_exec = nullptr;
+    plan->graph = nullptr;
+    plan->graph_args.clear();
+}
+
+}  // namespace
+
+extern "C" {
+
+int32_t kxc_hip_plan_run(kxc_hip_plan* plan, void** args, void* stream) {
+    if (int32_t rc = CheckRunArgs(plan, args, "kxc_hip_plan_run")) return rc;
+    hipStream_t main_stream = reinterpret_cast<hipStream_t>(stream ? stream : static_cast<void*>(CurrentStream()));
+    // Graph replay needs a real stream (the null stream cannot be captured) and one eager run before the
+    // capture, so that everything that allocates lazily (split-reduction scratch, function attributes) exists.
+    if (!plan->graph_enabled || main_stream == nullptr) return EnqueueAll(plan, args, main_stream);
+    const std::vector<void*> now(args, args + plan->num_args);
+    if (plan->graph_exec && now == plan->graph_args) {
+        KXC_HIP_CALL(hipGraphLaunch(plan->graph_exec, main_stream), "hipGraphLaunch");
+        return KXC_HIP_OK;
+    }
+    if (plan->eager_runs < 1) {
+        ++plan->eager_runs;
+        return EnqueueAll(plan, args, main_stream);
+    }
+    DropGraph(plan);
+    KXC_HIP_CALL(hipStreamBeginCapture(main_stream, hipStreamCaptureModeThreadLocal), "hipStreamBeginCapture");
+    const int32_t rc = EnqueueAll(plan, args, main_stream);
+    hipGraph_t graph = nullptr;
+    const hipError_t end = hipStreamEndCapture(main_stream, &graph);
+    if (rc != KXC_HIP_OK) {
+        if (graph) (void)hipGraphDestroy(graph);
+        return rc;
+    }
+    if (end != hipSuccess || graph == nullptr)
+        return Fail(KXC_HIP_ERR_RUNTIME, "kxc_hip_plan_run: stream capture failed: %s", hipGetErrorString(end));
+    plan->graph = graph;
+    const hipError_t inst = hipGraphInstantiate(&plan->graph_exec, plan->graph, nullptr, nullptr, 0);
+    if (inst != hipSuccess) {
+        DropGraph(plan);
+        return Fail(KXC_HIP_ERR_RUNTIME, "kxc_hip_plan_run: hipGraphInstantiate failed: %s", hipGetErrorString(inst));
+    }
+    plan->graph_args = now;
+    KXC_HIP_CALL(hipGraphLaunch(plan->graph_exec, main_stream), "hipGraphLaunch");     // the capture itself ran nothing
+    return KXC_HIP_OK;
+}
+
+int32_t kxc_hip_plan_enable_graph(kxc_hip_plan* plan, int32_t enable) {
+    KXC_HIP_REQUIRE(plan != nullptr, "kxc_hip_plan_enable_graph: plan is NULL");
+    plan->graph_enabled = enable != 0;
+    if (!plan->graph_enabled) DropGraph(plan);
     return KXC_HIP_OK;
 }
 

@@ -499,6 +499,9 @@ class Plan:
     def add_qdense(self, m, n, k, a, b, bias, mult, y):
         _check(lib().kxc_hip_plan_add_qdense(self._h, C.c_int64(m), C.c_int64(n), C.c_int64(k), a, b, bias, mult, y))
 
+    def enable_graph(self, enable=True):
+        _check(lib().kxc_hip_plan_enable_graph(self._h, C.c_int32(1 if enable else 0)))
+
     def finalize(self, workspace_bytes):
         _check(lib().kxc_hip_plan_finalize(self._h, C.c_size_t(workspace_bytes)))
 

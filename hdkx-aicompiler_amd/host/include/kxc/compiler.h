@@ -74,6 +74,9 @@ public:
     // kernel_symbol per node) plus a "kxc_hip" object with everything LoadExecutionPlan needs.
     std::string ExecutionPlanJSON() const;
     size_t workspace_bytes() const;
+    // hip target: later runs on a non-null stream with unchanged argument pointers replay a captured HIP graph
+    // (one launch call per Run instead of one per kernel; for launch-bound, small-batch functions).
+    void EnableGraphReplay(bool enable);
 
 private:
     std::shared_ptr<CompiledModuleImpl> impl_;

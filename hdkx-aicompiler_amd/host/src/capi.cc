@@ -50,6 +50,16 @@ int kxc_host_module_run(void* module, void** packed_args, int num_args) {
     }
 }
 
+int kxc_host_module_enable_graph(void* module, int enable) {
+    try {
+        static_cast<ModuleHandle*>(module)->module.EnableGraphReplay(enable != 0);
+        return 0;
+    } catch (const std::exception& e) {
+        g_error = e.what();
+        return 1;
+    }
+}
+
 int kxc_host_module_is_ready(void* module) { return static_cast<ModuleHandle*>(module)->module.IsReady() ? 1 : 0; }
 const char* kxc_host_module_status(void* module) {
     g_error = static_cast<ModuleHandle*>(module)->module.GetStatus();

@@ -616,6 +616,10 @@ int64_t CompiledModule::input_count() const { return impl_->input_count; }
 int64_t CompiledModule::constant_count() const { return impl_->constant_count; }
 const std::vector<KernelExecInfo>& CompiledModule::GetKernelExecs() const { return impl_->execs; }
 size_t CompiledModule::workspace_bytes() const { return impl_->workspace_bytes; }
+void CompiledModule::EnableGraphReplay(bool enable) {
+    if (!impl_ || !impl_->plan) throw std::runtime_error("EnableGraphReplay: not a loaded hip module");
+    if (kxc_hip_plan_enable_graph(impl_->plan, enable ? 1 : 0)) throw std::runtime_error(std::string("EnableGraphReplay: ") + kxc_hip_last_error());
+}
 
 std::string CompiledModule::ExecutionPlanJSON() const {
     std::ostringstream os;

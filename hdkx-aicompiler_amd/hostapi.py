@@ -58,10 +58,19 @@ class CompiledResNet18:
         return (C.c_void_p * len(tensors))(*[t.data_ptr() for t in tensors])
 
     def run_packed(self, args, stream=None):
-        """Enqueue on `stream` (a hipStream_t as int): it becomes the calling thread's current stream."""
+        """Enqueue on `stream` (a hipStream_t as int), which is the thread's current stream for the call."""
         if stream is not None:
             hipabi.lib().kxc_hip_set_stream(0, C.c_void_p(stream))
-        if lib().kxc_host_module_run(self._h, args, len(args)) != 0:
+        try:
+            if lib().kxc_host_module_run(self._h, args, len(args)) != 0:
+                raise hipabi.KxcHipError(lib().kxc_host_last_error().decode())
+        finally:
+            if stream is not None:
+                hipabi.lib().kxc_hip_set_stream(0, C.c_void_p(0))     # do not leave it as the thread's current stream
+
+    def enable_graph_replay(self, enable=True):
+        """Later runs on a non-null stream with the same argument pointers replay a captured HIP graph."""
+        if lib().kxc_host_module_enable_graph(self._h, 1 if enable else 0) != 0:
             raise hipabi.KxcHipError(lib().kxc_host_last_error().decode())
 
     def close(self):

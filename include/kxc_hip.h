@@ -318,6 +318,11 @@ int32_t kxc_hip_plan_set_concurrency(kxc_hip_plan* plan, int32_t node, int32_t l
 int32_t kxc_hip_plan_finalize(kxc_hip_plan* plan, size_t workspace_bytes);
 /* Enqueue every node on `stream`; returns after enqueue (no synchronisation). */
 int32_t kxc_hip_plan_run(kxc_hip_plan* plan, void** packed_args, void* stream);
+/* HIP graph replay for launch-bound plans (batch-1 inference: ~25 launches of ~15 us).  When enabled, the second
+ * run on a non-null stream is recorded by stream capture (side-lane nodes become parallel branches) and every
+ * later run with the same packed-argument pointers is one hipGraphLaunch; other pointers re-capture.  The first
+ * run stays eager so that lazily allocated scratch exists before the capture.  The plan records no memset node. */
+int32_t kxc_hip_plan_enable_graph(kxc_hip_plan* plan, int32_t enable);
 /* The same run with a HIP event between consecutive launches: fills one record per plan node (kernel symbol,
  * launch geometry, start relative to the first launch, duration) and returns after the last launch has
  * finished.  The records carry what the reference's profiler adapter puts into a "cuda_kernel" event

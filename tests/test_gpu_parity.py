@@ -343,3 +343,43 @@ def test_resnet18_batch64_properties(pkg, fast_orc):
     for n in (0, 63):
         want = fast_orc.resnet18(x[n:n + 1], consts)
         assert_close(got[n:n + 1], want, what="resnet18 batch 64, image %d" % n, floor="scale")
+
+
+def test_plan_hip_graph_replay(pkg):
+    """A launch plan replayed as a captured HIP graph gives the eager result on every replay, with eager work and
+    synchronisations in between, and re-captures when an argument pointer changes.  Batch 1 exercises the
+    workgroup-split reduction (scratch buffer, second kernel) inside the graph."""
+    import importlib
+    r = importlib.import_module("hdkx-aicompiler_amd.resnet18")
+    synth = importlib.import_module("hdkx-aicompiler_amd.synth")
+    consts = [dev(c) for c in synth.resnet18_consts(3)]
+    x = dev(synth.resnet18_input(3, 1, 224))
+    plan, info = r.build_plan(1, 224, True)
+    out = torch.empty((1, 1000), device="cuda")
+    plan.run([x] + consts + [out])
+    torch.cuda.synchronize()
+    eager = host(out).copy()
+    assert np.isfinite(eager).all() and np.abs(eager).max() > 0
+    stream = torch.cuda.Stream()
+    plan.enable_graph(True)
+    with torch.cuda.stream(stream):
+        for replay in range(5):
+            out.zero_()
+            plan.run([x] + consts + [out], stream.cuda_stream)     # run 0 eager, run 1 captures, runs 2.. replay
+            stream.synchronize()
+            assert_bit_exact(host(out), eager, "graph replay %d" % replay)
+            # eager work of the program between replays
+            y = pkg.conv2d(x, consts[0], consts[1], None, 2, 3, 1, True)
+            torch.cuda.synchronize()
+            assert torch.isfinite(y).all()
+        other = torch.empty((1, 1000), device="cuda")             # different output pointer: captured again
+        for replay in range(3):
+            other.zero_()
+            plan.run([x] + consts + [other], stream.cuda_stream)
+            stream.synchronize()
+            assert_bit_exact(host(other), eager, "graph replay with a new output buffer %d" % replay)
+    plan.enable_graph(False)
+    plan.run([x] + consts + [out])
+    torch.cuda.synchronize()
+    assert_bit_exact(host(out), eager, "eager again")
+    plan.close()
