@@ -728,7 +728,10 @@ int32_t kxc_hip_conv2d_nchw_f32(const kxc_hip_conv2d_desc* desc, const float* x,
         {
             const int64_t waves = tiles * c.v->nw * c.v->ks;
             int split = 1;
-            while (split < 16 && waves * split < 2048 && a.nchunks / (split * 2) >= 2 * c.v->ks) split *= 2;
+            // (only while the partial sums stay small next to the caches: the split re-reads them once)
+            while (split < 16 && waves * split < 2048 && a.nchunks / (split * 2) >= 2 * c.v->ks &&
+                   total * static_cast<int64_t>(sizeof(float)) * split * 2 <= (8LL << 20))
+                split *= 2;
             if (const char* e = std::getenv("KXC_HIP_CONV_GSPLIT")) { const int f = std::atoi(e); if (f >= 1 && f <= a.nchunks) split = f; }
             if (split > 1) {
                 a.cps = static_cast<int32_t>(CeilDiv(a.nchunks, split));
