@@ -1,0 +1,484 @@
+// conv2d_wino_f32.hip -- nn_conv2d for 3x3 filters, stride 1, dilation 1 (NCHW, OIHW, fp32) as Winograd
+// F(2x2, 3x3) on the fp32 matrix cores of gfx950.
+//
+//   Y = A^T [ (G g G^T) (.) (B^T d B) ] A      per 4x4 input patch d, 3x3 filter g, 2x2 output block Y
+//
+// 16 multiplies per 2x2 output block and channel instead of 36: the matrix work of a layer drops by 2.25x.  The
+// sixteen element-wise products are sixteen independent matrix products  M_f[o][tile] = sum_c U_f[o][c] V_f[c][tile]
+// (f = position in the 4x4 transform domain), which is what the matrix cores run.
+//
+//  * The filter transform U = G g G^T is done once per weight tensor by wino_weight_kernel into a packed buffer
+//    whose blocks are byte-for-byte the LDS image the main kernel wants: [32 output channels][4 input channels]
+//    as [c][o/16][f/4][o%16][f%4], 8 KiB per block, so that a workgroup fills its weight tile with 16-byte
+//    loads that write straight to LDS, and a lane's four f values of one (o, c) are one 16-byte LDS read.
+//  * The input transform V = B^T d B runs inside the main kernel: per step of 4 input channels every thread
+//    loads 3 rows x 4 columns of one tile's patch into registers (two threads share a tile: rows 0-2 give
+//    transform rows 0-1, rows 1-3 give rows 2-3), transforms them with 16 additions and writes two 16-byte
+//    vectors to LDS.  Padding costs nothing: offsets of positions outside the image point beyond the buffer,
+//    where a buffer load returns 0.  The loads for step s+2 are issued while step s multiplies.
+//  * v_mfma_f32_16x16x4_f32: a wave owns 32 output channels x 16 tiles x all 16 f -- 32 accumulators of 4
+//    registers.  Because every f of one (o, tile) lands in the same lane, the output transform A^T M A and the
+//    epilogue (bias, residual, ReLU) run in registers and the 2x2 block is stored as two 8-byte runs; the 16
+//    lanes of a quarter-wave hold consecutive tiles, i.e. 128 contiguous bytes of an output row.
+//
+// The sums are formed in a different order than the direct loop nest (and G introduces factors 1/2, 1/4), so
+// results agree with the CPU backend within the fp32 tolerance of the operator (about 1e-6 relative on
+// ResNet-sized reductions), not bit for bit.
+#include <cstdlib>
+#include <cstring>
+
+#include "common.h"
+
+using namespace kxc_hip;
+
+namespace {
+
+typedef float floatx4 __attribute__((ext_vector_type(4)));
+typedef float floatx2 __attribute__((ext_vector_type(2)));
+typedef __attribute__((address_space(3))) void* lds_ptr_t;
+
+constexpr uint32_t kOob = 0x80000000u;     // beyond any buffer this kernel accepts (< 2 GiB): reads as 0
+
+struct WinoArgs {
+    const float* x;
+    const float* u;
+    const float* bias;
+    const float* res;
+    float* y;
+    int32_t N, C, H, W, O, OH, OW, ph, pw;
+    int32_t TW, TI, NT;              // tiles per output row, per image, in total
+    int32_t HW, OHW;
+    int32_t csteps;                  // C / 4
+    int32_t t_groups, k_groups, num_units, units_per_xcd, k_fastest;
+    uint32_t x_bytes, u_bytes, flags;
+    FastDiv div_ti, div_tw, div_kgroups, div_tgroups;
+};
+
+__device__ __forceinline__ __amdgpu_buffer_rsrc_t make_rsrc(const void* p, uint32_t bytes) {
+    return __builtin_amdgcn_make_buffer_rsrc(const_cast<void*>(p), 0, static_cast<int>(bytes), 0x00020000);
+}
+
+// 16 bytes per lane from a buffer straight into LDS (lane l writes lds + 16*l).  The 16-byte form exists on
+// gfx950 only; the host pass of the compiler does not know the target and rejects the size, so it sees an
+// empty body.
+__device__ __forceinline__ void load16_to_lds(__amdgpu_buffer_rsrc_t rsrc, lds_ptr_t lds, uint32_t voffset,
+                                              uint32_t soffset) {
+#if defined(__HIP_DEVICE_COMPILE__)
+    __builtin_amdgcn_raw_ptr_buffer_load_lds(rsrc, lds, 16, voffset, soffset, 0, 0);
+#endif
+}
+
+__device__ __forceinline__ float load_f32(__amdgpu_buffer_rsrc_t rsrc, uint32_t voffset, uint32_t soffset) {
+    return __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(rsrc, voffset, soffset, 0));
+}
+
+__device__ __forceinline__ float relu_sel(float v) { return (v > 0.0f) ? v : 0.0f; }
+
+// ------------------------------------------------------------------------------------------
+// Filter transform.  One thread per (o, c), o < 32*ceil(O/32) (absent output channels give zero blocks).
+// packed index: ((o/32 * csteps + c/4) * 2048) + (((c%4)*2 + (o%32)/16)*4 + i)*64 + (o%16)*4 + j  for U[i][j]
+// ------------------------------------------------------------------------------------------
+__global__ void __launch_bounds__(256) wino_weight_kernel(const float* __restrict__ w, float* __restrict__ u, int32_t O,
+                                                          int32_t C, int32_t o_padded) {
+    const int e = blockIdx.x * 256 + threadIdx.x;
+    if (e >= o_padded * C) return;
+    const int o = e / C, c = e - o * C;
+    float g[3][3];
+#pragma unroll
+    for (int i = 0; i < 3; ++i)
+#pragma unroll
+        for (int j = 0; j < 3; ++j) g[i][j] = o < O ? w[(static_cast<int64_t>(o) * C + c) * 9 + i * 3 + j] : 0.0f;
+    float t[4][3];      // G g
+#pragma unroll
+    for (int j = 0; j < 3; ++j) {
+        t[0][j] = g[0][j];
+        t[1][j] = 0.5f * ((g[0][j] + g[2][j]) + g[1][j]);
+        t[2][j] = 0.5f * ((g[0][j] + g[2][j]) - g[1][j]);
+        t[3][j] = g[2][j];
+    }
+    const int csteps = C / 4;
+    float* const dst = u + (static_cast<int64_t>(o / 32) * csteps + c / 4) * 2048 + (((c % 4) * 2 + (o % 32) / 16) * 4) * 64 +
+                       (o % 16) * 4;
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+        floatx4 v;
+        v[0] = t[i][0];
+        v[1] = 0.5f * ((t[i][0] + t[i][2]) + t[i][1]);
+        v[2] = 0.5f * ((t[i][0] + t[i][2]) - t[i][1]);
+        v[3] = t[i][2];
+        *reinterpret_cast<floatx4*>(dst + i * 64) = v;
+    }
+}
+
+// ------------------------------------------------------------------------------------------
+// Main kernel.  WK x WT waves; a wave owns 32 output channels x 16 tiles; the workgroup 32*WK x 16*WT.
+// One step = 4 input channels.  LDS per buffer: U [WK][c4][o/16: 2][f/4: 4][o%16][f%4] and
+// V [c4][WT][f/4: 4][tile%16][f%4]; two of each.
+// ------------------------------------------------------------------------------------------
+template <int WK, int WT>
+__global__ void __launch_bounds__(64 * WK * WT) __attribute__((amdgpu_waves_per_eu(2)))
+wino_kernel(const WinoArgs a) {
+    constexpr int NTH = 64 * WK * WT;
+    constexpr int TT = 16 * WT;
+    constexpr int U_FLOATS = 2048 * WK;
+    constexpr int V_FLOATS = 1024 * WT;
+    constexpr int ULOADS = U_FLOATS / 4 / NTH;     // 16-byte loads per thread and step
+    constexpr int ITEMS = 2 / WK;                   // (tile, channel, half) items per thread and step
+    static_assert(WK == 1 || WK == 2, "a thread transforms one or two input items per step");
+    static_assert((U_FLOATS / 4) % NTH == 0, "weight tile must divide over the threads");
+
+    extern __shared__ float lds[];
+    const int tid = threadIdx.x;
+    const int lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int wave_k = wave / WT, wave_t = wave % WT;
+    // Consecutive workgroups go to the 8 XCDs round-robin; each XCD (own L2) takes a contiguous run of units.
+    const int unit = (blockIdx.x & 7) * a.units_per_xcd + (blockIdx.x >> 3);
+    if (unit >= a.num_units || static_cast<int>(blockIdx.x >> 3) >= a.units_per_xcd) return;
+    int kg, tg;
+    if (a.k_fastest) { tg = fast_div(unit, a.div_kgroups); kg = unit - tg * a.k_groups; }
+    else { kg = fast_div(unit, a.div_tgroups); tg = unit - kg * a.t_groups; }
+    const int t0 = tg * TT;
+
+    const __amdgpu_buffer_rsrc_t xr = make_rsrc(a.x, a.x_bytes);
+    const __amdgpu_buffer_rsrc_t ur = make_rsrc(a.u, a.u_bytes);
+
+    // ---- input items: item = tid + i*NTH -> tile = item % TT, channel = (item / TT) % 4, half = item / (4*TT)
+    uint32_t goff[ITEMS][12];
+    int vdst[ITEMS];
+#pragma unroll
+    for (int i = 0; i < ITEMS; ++i) {
+        const int item = tid + i * NTH;
+        const int tile_l = item % TT, cl = (item / TT) % 4, half = item / (4 * TT);
+        const int tile = t0 + tile_l;
+        const int n = fast_div(tile, a.div_ti), rem = tile - n * a.TI;
+        const int ty = fast_div(rem, a.div_tw), tx = rem - ty * a.TW;
+#pragma unroll
+        for (int r = 0; r < 3; ++r) {
+            const int ih = 2 * ty - a.ph + half + r;
+#pragma unroll
+            for (int j = 0; j < 4; ++j) {
+                const int iw = 2 * tx - a.pw + j;
+                const bool ok = tile < a.NT && ih >= 0 && ih < a.H && iw >= 0 && iw < a.W;
+                goff[i][r * 4 + j] = ok ? static_cast<uint32_t>(((n * a.C + cl) * a.H + ih) * a.W + iw) * 4u : kOob;
+            }
+        }
+        vdst[i] = ((cl * WT + tile_l / 16) * 4 + 2 * half) * 64 + (tile_l % 16) * 4;
+    }
+    // ---- weight tile loads: 16-byte unit idx = j*NTH + tid of the tile; block h = idx / 512 is k32 group kg*WK + h
+    uint32_t uoff[ULOADS];
+#pragma unroll
+    for (int j = 0; j < ULOADS; ++j) {
+        const int idx = j * NTH + tid;
+        const int h = idx / 512, within = idx - h * 512;
+        uoff[j] = static_cast<uint32_t>((kg * WK + h) * a.csteps) * 8192u + static_cast<uint32_t>(within) * 16u;
+    }
+
+    const int a_base = wave_k * 2048 + (lane >> 4) * 512 + (lane & 15) * 4;
+    const int b_base = ((lane >> 4) * WT + wave_t) * 256 + (lane & 15) * 4;
+
+    floatx4 acc[16][2];
+#pragma unroll
+    for (int f = 0; f < 16; ++f)
+#pragma unroll
+        for (int kb = 0; kb < 2; ++kb) acc[f][kb] = floatx4{0.0f, 0.0f, 0.0f, 0.0f};
+
+    float d[ITEMS][12];
+    auto load_raw = [&](int s) {
+        const uint32_t soff = static_cast<uint32_t>(s) * static_cast<uint32_t>(a.HW) * 16u;   // 4 channels of HW floats
+#pragma unroll
+        for (int i = 0; i < ITEMS; ++i)
+#pragma unroll
+            for (int q = 0; q < 12; ++q) d[i][q] = load_f32(xr, goff[i][q], soff);
+#ifdef KXC_WDBG_NO_RAW
+#pragma unroll
+        for (int i = 0; i < ITEMS; ++i)
+#pragma unroll
+            for (int q = 0; q < 12; ++q) d[i][q] = (float)(goff[i][q] + soff);
+#endif
+    };
+    auto issue_u = [&](int s, float* buf) {
+#pragma unroll
+        for (int j = 0; j < ULOADS; ++j)
+#ifndef KXC_WDBG_NO_U
+            load16_to_lds(ur, (lds_ptr_t)(buf + (j * NTH + wave * 64) * 4), uoff[j], static_cast<uint32_t>(s) * 8192u);
+#else
+            ;
+#endif
+    };
+    auto transform = [&](float* buf) {
+#pragma unroll
+        for (int i = 0; i < ITEMS; ++i) {
+            const int half = (tid + i * NTH) / (4 * TT);        // uniform over the wave
+            float ta[4], tb[4];
+#pragma unroll
+            for (int j = 0; j < 4; ++j) {
+                const float e0 = d[i][j], e1 = d[i][4 + j], e2 = d[i][8 + j];
+                ta[j] = half == 0 ? e0 - e2 : e1 - e0;
+                tb[j] = half == 0 ? e1 + e2 : e0 - e2;
+            }
+            floatx4 va, vb;
+            va[0] = ta[0] - ta[2]; va[1] = ta[1] + ta[2]; va[2] = ta[2] - ta[1]; va[3] = ta[1] - ta[3];
+            vb[0] = tb[0] - tb[2]; vb[1] = tb[1] + tb[2]; vb[2] = tb[2] - tb[1]; vb[3] = tb[1] - tb[3];
+            *reinterpret_cast<floatx4*>(buf + vdst[i]) = va;
+            *reinterpret_cast<floatx4*>(buf + vdst[i] + 64) = vb;
+        }
+    };
+    // Operands of one group of four f values: two 16-byte reads of U (output-channel blocks 0 and 1) and one of V.
+    // Two register sets: the reads for group fg+1 are issued before the matrix instructions of group fg.
+    floatx4 ra[2][2], rb[2];
+    auto fetch = [&](const float* ub, const float* vb, int fg, int set) {
+        ra[set][0] = *reinterpret_cast<const floatx4*>(ub + a_base + fg * 64);
+        ra[set][1] = *reinterpret_cast<const floatx4*>(ub + a_base + 256 + fg * 64);
+        rb[set] = *reinterpret_cast<const floatx4*>(vb + b_base + fg * 64);
+    };
+    auto mm = [&](int fg, int set) {
+#pragma unroll
+        for (int f = 0; f < 4; ++f) {
+#ifdef KXC_WDBG_NO_MFMA
+            acc[fg * 4 + f][0][0] += ra[set][0][f] + rb[set][f];
+            acc[fg * 4 + f][1][0] += ra[set][1][f];
+#else
+            acc[fg * 4 + f][0] = __builtin_amdgcn_mfma_f32_16x16x4f32(ra[set][0][f], rb[set][f], acc[fg * 4 + f][0], 0, 0, 0);
+            acc[fg * 4 + f][1] = __builtin_amdgcn_mfma_f32_16x16x4f32(ra[set][1][f], rb[set][f], acc[fg * 4 + f][1], 0, 0, 0);
+#endif
+        }
+    };
+
+    // LDS: two weight tiles and two transformed-input tiles.  The compiler orders every barrier after the
+    // LDS-writing loads issued before it, so a weight tile is requested at the top of the step before the one that
+    // uses it and has that whole step to arrive; the raw input (registers) is requested two steps ahead.
+    float* const ub0 = lds;
+    float* const ub1 = lds + U_FLOATS;
+    float* const vb0 = lds + 2 * U_FLOATS;
+    float* const vb1 = vb0 + V_FLOATS;
+    const int last = a.csteps - 1;
+
+    // ---- prologue: weight tile and transformed input of step 0; raw input of step 1 in flight
+    issue_u(0, ub0);
+    load_raw(0);
+    transform(vb0);
+    load_raw(min(1, last));
+    __builtin_amdgcn_sched_barrier(0);
+    __syncthreads();
+
+    for (int s = 0; s < a.csteps; ++s) {
+        const float* const ucur = (s & 1) ? ub1 : ub0;
+        const float* const vcur = (s & 1) ? vb1 : vb0;
+        float* const unxt = (s & 1) ? ub0 : ub1;
+        float* const vnxt = (s & 1) ? vb0 : vb1;
+        // Steps past the end re-load the last step (never used), which keeps the loop free of branches.
+        issue_u(min(s + 1, last), unxt);
+        fetch(ucur, vcur, 0, 0);
+        __builtin_amdgcn_sched_barrier(0);
+        fetch(ucur, vcur, 1, 1);
+        mm(0, 0);
+        __builtin_amdgcn_sched_barrier(0);
+        // group 1 multiplies while the raw input of step s+1 (requested one step ago) is transformed: the vector
+        // instructions are spread between the matrix instructions, which run 8 passes each
+        fetch(ucur, vcur, 2, 0);
+        mm(1, 1);
+        transform(vnxt);
+#pragma unroll
+        for (int q = 0; q < 8; ++q) {
+            __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);      // one matrix instruction
+            __builtin_amdgcn_sched_group_barrier(0x002, 6, 0);      // six vector ALU instructions
+        }
+        __builtin_amdgcn_sched_barrier(0);
+        fetch(ucur, vcur, 3, 1);
+        mm(2, 0);
+        load_raw(min(s + 2, last));
+#pragma unroll
+        for (int q = 0; q < 8; ++q) {
+            __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+            __builtin_amdgcn_sched_group_barrier(0x020, 2, 0);      // two vector memory reads
+        }
+        __builtin_amdgcn_sched_barrier(0);
+        mm(3, 1);
+        __builtin_amdgcn_sched_barrier(0);
+        __syncthreads();
+    }
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+
+    // ---- epilogue: accumulator register g of block kb holds output channel 16*kb + 4*(lane/16) + g, tile lane%16
+    const int tile = t0 + wave_t * 16 + (lane & 15);
+    if (tile >= a.NT) return;
+#ifdef KXC_WDBG_NO_EPI
+    if (acc[0][0][0] != 123456.789f) return;
+#endif
+    const int n = fast_div(tile, a.div_ti), rem = tile - n * a.TI;
+    const int ty = fast_div(rem, a.div_tw), tx = rem - ty * a.TW;
+    const int oh = 2 * ty, ow = 2 * tx;
+    const bool row1 = oh + 1 < a.OH, col1 = ow + 1 < a.OW;
+    const bool vec2 = (a.OW & 1) == 0;
+    const bool has_bias = (a.flags & KXC_HIP_CONV_BIAS) != 0;
+    const bool has_res = (a.flags & KXC_HIP_CONV_RESIDUAL) != 0;
+    const bool do_relu = (a.flags & KXC_HIP_CONV_RELU) != 0;
+#pragma unroll
+    for (int kb = 0; kb < 2; ++kb) {
+#pragma unroll
+        for (int g = 0; g < 4; ++g) {
+            const int o = (kg * WK + wave_k) * 32 + kb * 16 + 4 * (lane >> 4) + g;
+            if (o >= a.O) continue;
+            // A^T M A with A^T = [1 1 1 0; 0 1 -1 -1]
+            float r0[4], r1[4];
+#pragma unroll
+            for (int j = 0; j < 4; ++j) {
+                const float m0 = acc[j][kb][g], m1 = acc[4 + j][kb][g], m2 = acc[8 + j][kb][g], m3 = acc[12 + j][kb][g];
+                r0[j] = (m0 + m1) + m2;
+                r1[j] = (m1 - m2) - m3;
+            }
+            float y00 = (r0[0] + r0[1]) + r0[2], y01 = (r0[1] - r0[2]) - r0[3];
+            float y10 = (r1[0] + r1[1]) + r1[2], y11 = (r1[1] - r1[2]) - r1[3];
+            const int off = ((n * a.O + o) * a.OH + oh) * a.OW + ow;
+            if (has_bias) {
+                const float bval = a.bias[o];
+                y00 = __fadd_rn(y00, bval); y01 = __fadd_rn(y01, bval); y10 = __fadd_rn(y10, bval); y11 = __fadd_rn(y11, bval);
+            }
+            if (vec2) {
+                if (has_res) {
+                    const floatx2 q0 = *reinterpret_cast<const floatx2*>(a.res + off);
+                    y00 = __fadd_rn(y00, q0[0]); y01 = __fadd_rn(y01, q0[1]);
+                    if (row1) {
+                        const floatx2 q1 = *reinterpret_cast<const floatx2*>(a.res + off + a.OW);
+                        y10 = __fadd_rn(y10, q1[0]); y11 = __fadd_rn(y11, q1[1]);
+                    }
+                }
+                if (do_relu) { y00 = relu_sel(y00); y01 = relu_sel(y01); y10 = relu_sel(y10); y11 = relu_sel(y11); }
+                *reinterpret_cast<floatx2*>(a.y + off) = floatx2{y00, y01};
+                if (row1) *reinterpret_cast<floatx2*>(a.y + off + a.OW) = floatx2{y10, y11};
+            } else {
+                if (has_res) {
+                    y00 = __fadd_rn(y00, a.res[off]);
+                    if (col1) y01 = __fadd_rn(y01, a.res[off + 1]);
+                    if (row1) y10 = __fadd_rn(y10, a.res[off + a.OW]);
+                    if (row1 && col1) y11 = __fadd_rn(y11, a.res[off + a.OW + 1]);
+                }
+                if (do_relu) { y00 = relu_sel(y00); y01 = relu_sel(y01); y10 = relu_sel(y10); y11 = relu_sel(y11); }
+                a.y[off] = y00;
+                if (col1) a.y[off + 1] = y01;
+                if (row1) a.y[off + a.OW] = y10;
+                if (row1 && col1) a.y[off + a.OW + 1] = y11;
+            }
+        }
+    }
+}
+
+struct WinoVariant {
+    const char* name;
+    int wk, wt;
+    void (*kernel)(const WinoArgs);
+};
+#define KXC_WINO(WK, WT) {"winograd_f2k3_o" #WK "_t" #WT, WK, WT, wino_kernel<WK, WT>}
+// name = winograd_f2k3_o<waves along output channels (32 each)>_t<waves along tiles (16 each)>
+const WinoVariant kWino[] = {
+    KXC_WINO(2, 2),   // 64 channels x 32 tiles, 4 waves, 48 KiB of LDS (default)
+    KXC_WINO(2, 4),   // 64 x 64, 8 waves
+    KXC_WINO(1, 4),   // 32 x 64, 4 waves
+    KXC_WINO(2, 1),   // 64 x 16, 2 waves
+    KXC_WINO(1, 2),   // 32 x 32, 2 waves
+};
+constexpr int kNumWino = sizeof(kWino) / sizeof(kWino[0]);
+
+bool Supported(const kxc_hip_conv2d_desc* d) {
+    if (!d || d->kh != 3 || d->kw != 3 || d->stride_h != 1 || d->stride_w != 1 || d->dil_h != 1 || d->dil_w != 1) return false;
+    if (d->n <= 0 || d->c <= 0 || d->c % 4 != 0 || d->o <= 0 || d->pad_h < 0 || d->pad_w < 0) return false;
+    const int64_t oh = static_cast<int64_t>(d->h) + 2 * d->pad_h - 2, ow = static_cast<int64_t>(d->w) + 2 * d->pad_w - 2;
+    if (oh <= 0 || ow <= 0) return false;
+    const int64_t x_bytes = static_cast<int64_t>(d->n) * d->c * d->h * d->w * 4;
+    const int64_t y_elems = static_cast<int64_t>(d->n) * d->o * oh * ow;
+    const int64_t u_bytes = CeilDiv(d->o, 32) * 32 * static_cast<int64_t>(d->c) * 64;
+    const int64_t tiles = static_cast<int64_t>(d->n) * CeilDiv(oh, 2) * CeilDiv(ow, 2);
+    return x_bytes < (1LL << 31) && y_elems < (1LL << 31) && u_bytes < (1LL << 31) && tiles < (1LL << 30);
+}
+
+const WinoVariant* SelectWino(const kxc_hip_conv2d_desc* d) {
+    if (const char* e = std::getenv("KXC_HIP_WINOGRAD_VARIANT")) {
+        for (int i = 0; i < kNumWino; ++i)
+            if (std::strcmp(e, kWino[i].name) == 0) return &kWino[i];
+    }
+    return &kWino[0];
+}
+
+}  // namespace
+
+extern "C" {
+
+int32_t kxc_hip_conv2d_winograd_supported(const kxc_hip_conv2d_desc* desc) { return Supported(desc) ? 1 : 0; }
+
+int32_t kxc_hip_conv2d_winograd_preferred(const kxc_hip_conv2d_desc* desc) {
+    if (!Supported(desc)) return 0;
+    const WinoVariant* v = SelectWino(desc);
+    const int64_t oh = static_cast<int64_t>(desc->h) + 2 * desc->pad_h - 2, ow = static_cast<int64_t>(desc->w) + 2 * desc->pad_w - 2;
+    const int64_t tiles = static_cast<int64_t>(desc->n) * CeilDiv(oh, 2) * CeilDiv(ow, 2);
+    const int64_t units = CeilDiv(tiles, 16 * v->wt) * CeilDiv(desc->o, 32 * v->wk);
+    int64_t min_units = 256;                     // one workgroup per compute unit
+    if (const char* e = std::getenv("KXC_HIP_WINOGRAD_MIN_UNITS")) min_units = std::atoll(e);
+    return units >= min_units ? 1 : 0;
+}
+
+const char* kxc_hip_conv2d_winograd_variant(const kxc_hip_conv2d_desc* desc) {
+    return Supported(desc) ? SelectWino(desc)->name : "unsupported";
+}
+
+int32_t kxc_hip_conv2d_winograd_weight_bytes(const kxc_hip_conv2d_desc* desc, size_t* out_bytes) {
+    KXC_HIP_REQUIRE(desc && out_bytes, "kxc_hip_conv2d_winograd_weight_bytes: NULL argument");
+    KXC_HIP_REQUIRE(Supported(desc), "kxc_hip_conv2d_winograd_weight_bytes: shape is not a 3x3 stride-1 convolution with C %% 4 == 0");
+    *out_bytes = static_cast<size_t>(CeilDiv(desc->o, 32)) * 32 * static_cast<size_t>(desc->c) * 16 * sizeof(float);
+    return KXC_HIP_OK;
+}
+
+int32_t kxc_hip_conv2d_winograd_transform_weights(const kxc_hip_conv2d_desc* desc, const float* w, float* u, void* stream) {
+    KXC_HIP_REQUIRE(desc && Supported(desc), "kxc_hip_conv2d_winograd_transform_weights: unsupported shape");
+    KXC_HIP_REQUIRE(w && u, "kxc_hip_conv2d_winograd_transform_weights: NULL pointer");
+    const int32_t o_padded = static_cast<int32_t>(CeilDiv(desc->o, 32) * 32);
+    const int64_t total = static_cast<int64_t>(o_padded) * desc->c;
+    wino_weight_kernel<<<NoteGrid(static_cast<int>(CeilDiv(total, 256))), NoteBlock(256), NoteLds(0), ResolveStream(stream)>>>(
+        w, u, static_cast<int32_t>(desc->o), static_cast<int32_t>(desc->c), o_padded);
+    return CheckLaunch("wino_weight_kernel");
+}
+
+int32_t kxc_hip_conv2d_winograd_nchw_f32(const kxc_hip_conv2d_desc* desc, const float* x, const float* u, const float* bias,
+                                         const float* residual, float* y, void* stream) {
+    KXC_HIP_REQUIRE(desc && Supported(desc), "kxc_hip_conv2d_winograd_nchw_f32: unsupported shape");
+    KXC_HIP_REQUIRE(x && u && y, "kxc_hip_conv2d_winograd_nchw_f32: NULL pointer");
+    KXC_HIP_REQUIRE(!(desc->flags & KXC_HIP_CONV_BIAS) || bias, "kxc_hip_conv2d_winograd_nchw_f32: bias flag without bias");
+    KXC_HIP_REQUIRE(!(desc->flags & KXC_HIP_CONV_RESIDUAL) || residual,
+                    "kxc_hip_conv2d_winograd_nchw_f32: residual flag without residual");
+    const WinoVariant* v = SelectWino(desc);
+    WinoArgs a;
+    std::memset(&a, 0, sizeof(a));
+    a.x = x; a.u = u; a.bias = bias; a.res = residual; a.y = y;
+    a.N = static_cast<int32_t>(desc->n); a.C = static_cast<int32_t>(desc->c); a.H = static_cast<int32_t>(desc->h);
+    a.W = static_cast<int32_t>(desc->w); a.O = static_cast<int32_t>(desc->o);
+    a.ph = static_cast<int32_t>(desc->pad_h); a.pw = static_cast<int32_t>(desc->pad_w);
+    a.OH = a.H + 2 * a.ph - 2; a.OW = a.W + 2 * a.pw - 2;
+    a.TW = (a.OW + 1) / 2;
+    a.TI = ((a.OH + 1) / 2) * a.TW;
+    a.NT = a.N * a.TI;
+    a.HW = a.H * a.W; a.OHW = a.OH * a.OW;
+    a.csteps = a.C / 4;
+    a.x_bytes = static_cast<uint32_t>(static_cast<int64_t>(a.N) * a.C * a.HW * 4);
+    a.u_bytes = static_cast<uint32_t>(CeilDiv(a.O, 32) * 32 * static_cast<int64_t>(a.C) * 64);
+    a.flags = desc->flags;
+    a.t_groups = static_cast<int32_t>(CeilDiv(a.NT, 16 * v->wt));
+    a.k_groups = static_cast<int32_t>(CeilDiv(a.O, 32 * v->wk));
+    a.num_units = a.t_groups * a.k_groups;
+    a.units_per_xcd = static_cast<int32_t>(CeilDiv(a.num_units, 8));
+    // transformed weights of all output channels small next to an L2: neighbouring units share the input tile
+    a.k_fastest = a.u_bytes <= (2u << 20) ? 1 : 0;
+    if (const char* e = std::getenv("KXC_HIP_WINOGRAD_KFAST")) a.k_fastest = std::atoi(e);
+    a.div_ti = MakeFastDiv(a.TI); a.div_tw = MakeFastDiv(a.TW);
+    a.div_kgroups = MakeFastDiv(a.k_groups); a.div_tgroups = MakeFastDiv(a.t_groups);
+    const size_t lds_bytes = 2 * static_cast<size_t>(2048 * v->wk + 1024 * v->wt) * sizeof(float);
+    if (lds_bytes > 64 * 1024) {
+        KXC_HIP_CALL(hipFuncSetAttribute(reinterpret_cast<const void*>(v->kernel), hipFuncAttributeMaxDynamicSharedMemorySize,
+                                         static_cast<int>(lds_bytes)),
+                     "hipFuncSetAttribute(MaxDynamicSharedMemorySize)");
+    }
+    hipLaunchKernelGGL(v->kernel, NoteGrid(dim3(static_cast<unsigned>(a.units_per_xcd * 8))),
+                       NoteBlock(dim3(64 * v->wk * v->wt)), NoteLds(lds_bytes), ResolveStream(stream), a);
+    return CheckLaunch(v->name);
+}
+
+}  // extern "C"

@@ -37,6 +37,8 @@ struct Node {
     // after it; `join` = this (main-lane) node first waits for every side-lane node enqueued before it
     int32_t lane = 0, join = 0;
     hipEvent_t fork_event = nullptr, done_event = nullptr;
+    // Winograd convolution (i32[0] == 1 on a kConv2D node): the weight pointer whose transform bufs[5] holds
+    const void* transformed_from = nullptr;
     // module kernel
     void* function = nullptr;
     uint32_t grid[3], block[3], shared_bytes = 0;
@@ -143,6 +145,31 @@ int32_t kxc_hip_plan_add_conv2d(kxc_hip_plan* plan, const kxc_hip_conv2d_desc* d
     if (desc->flags & KXC_HIP_CONV_RESIDUAL) n.symbol += "+add";
     if (desc->flags & KXC_HIP_CONV_RELU) n.symbol += "+relu";
     plan->nodes.push_back(n);
+    return KXC_HIP_OK;
+}
+
+int32_t kxc_hip_plan_add_conv2d_winograd(kxc_hip_plan* plan, const kxc_hip_conv2d_desc* desc, kxc_hip_buf x, kxc_hip_buf w,
+                                         kxc_hip_buf bias, kxc_hip_buf residual, kxc_hip_buf y, kxc_hip_buf u) {
+    const char* who = "kxc_hip_plan_add_conv2d_winograd";
+    KXC_PLAN_BEGIN(who);
+    KXC_HIP_REQUIRE(desc != nullptr, "%s: desc is NULL", who);
+    KXC_HIP_REQUIRE(kxc_hip_conv2d_winograd_supported(desc), "%s: not a 3x3 stride-1 convolution with c %% 4 == 0", who);
+    KXC_HIP_REQUIRE(u.kind == KXC_HIP_BUF_WORKSPACE, "%s: the transformed weights live in the plan workspace", who);
+    KXC_PLAN_BUF(u, false, who);
+    if (int32_t rc = kxc_hip_plan_add_conv2d(plan, desc, x, w, bias, residual, y)) return rc;
+    Node& n = plan->nodes.back();
+    n.i32[0] = 1;
+    n.bufs[5] = u;
+    n.symbol = std::string("kxc_conv2d_nchw_f32.") + kxc_hip_conv2d_winograd_variant(desc);
+    if (desc->flags & KXC_HIP_CONV_BIAS) n.symbol += "+bias";
+    if (desc->flags & KXC_HIP_CONV_RESIDUAL) n.symbol += "+add";
+    if (desc->flags & KXC_HIP_CONV_RELU) n.symbol += "+relu";
+    return KXC_HIP_OK;
+}
+
+int32_t kxc_hip_plan_invalidate_constants(kxc_hip_plan* plan) {
+    KXC_HIP_REQUIRE(plan != nullptr, "kxc_hip_plan_invalidate_constants: plan is NULL");
+    for (Node& n : plan->nodes) n.transformed_from = nullptr;
     return KXC_HIP_OK;
 }
 
@@ -461,6 +488,19 @@ int32_t RunNode(kxc_hip_plan* plan, Node& n, void** args, void* s) {
         auto B = [&](int i) { return Resolve(plan, n.bufs[i], args); };
         switch (n.kind) {
             case NodeKind::kConv2D:
+                if (n.i32[0] == 1) {
+                    // weights are module constants: transformed when first seen (or when another tensor is passed)
+                    if (n.transformed_from != B(1)) {
+                        rc = kxc_hip_conv2d_winograd_transform_weights(&n.conv, static_cast<const float*>(B(1)),
+                                                                       static_cast<float*>(B(5)), s);
+                        if (rc) break;
+                        n.transformed_from = B(1);
+                    }
+                    rc = kxc_hip_conv2d_winograd_nchw_f32(&n.conv, static_cast<const float*>(B(0)), static_cast<const float*>(B(5)),
+                                                          static_cast<const float*>(B(2)), static_cast<const float*>(B(3)),
+                                                          static_cast<float*>(B(4)), s);
+                    break;
+                }
                 rc = kxc_hip_conv2d_nchw_f32(&n.conv, static_cast<const float*>(B(0)), static_cast<const float*>(B(1)),
                                              static_cast<const float*>(B(2)), static_cast<const float*>(B(3)),
                                              static_cast<float*>(B(4)), s);
@@ -825,6 +865,9 @@ int32_t kxc_hip_plan_deserialize(const char* text, int32_t device_id, kxc_hip_mo
         };
         for (const kxc_hip_buf& b : n.bufs) if (!buf_ok(b)) return fail("buffer operand out of range");
         for (const kxc_hip_buf& b : n.params) if (!buf_ok(b)) return fail("kernel parameter out of range");
+        if (n.kind == NodeKind::kConv2D && n.i32[0] == 1 &&
+            (!kxc_hip_conv2d_winograd_supported(&n.conv) || n.bufs[5].kind != KXC_HIP_BUF_WORKSPACE))
+            return fail("bad Winograd convolution node");
         if (n.kind == NodeKind::kModuleKernel) {
             // generated kernels are found by name in the modules the caller compiled from the saved source
             for (int32_t m = 0; m < num_modules && !n.function; ++m) {

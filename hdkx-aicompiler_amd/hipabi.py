@@ -79,6 +79,7 @@ def lib():
         _lib.kxc_hip_last_error.restype = C.c_char_p
         _lib.kxc_hip_target_kind.restype = C.c_char_p
         _lib.kxc_hip_conv2d_variant.restype = C.c_char_p
+        _lib.kxc_hip_conv2d_winograd_variant.restype = C.c_char_p
         _lib.kxc_hip_qconv2d_c16_variant.restype = C.c_char_p
         _lib.kxc_hip_plan_node_symbol.restype = C.c_char_p
         _lib.kxc_hip_plan_workspace.restype = C.c_void_p
@@ -141,6 +142,52 @@ def conv2d(x, w, bias=None, residual=None, stride=1, pad=0, dil=1, relu=False, f
     d = conv_desc(tuple(x.shape), tuple(w.shape), stride, pad, dil, flags)
     y = out if out is not None else torch.empty(conv_out_shape(d), dtype=torch.float32, device=x.device)
     _check(lib().kxc_hip_conv2d_nchw_f32(C.byref(d), _p(x), _p(w), _p(bias), _p(residual), _p(y), _stream()))
+    return y
+
+
+def conv2d_winograd_supported(x_shape, w_shape, stride, pad, dil=1):
+    d = conv_desc(x_shape, w_shape, stride, pad, dil, 0)
+    return bool(lib().kxc_hip_conv2d_winograd_supported(C.byref(d)))
+
+
+def conv2d_winograd_preferred(x_shape, w_shape, stride=1, pad=1, dil=1):
+    d = conv_desc(x_shape, w_shape, stride, pad, dil, 0)
+    return bool(lib().kxc_hip_conv2d_winograd_preferred(C.byref(d)))
+
+
+def conv2d_winograd_weight_bytes(x_shape, w_shape, pad=1):
+    d = conv_desc(x_shape, w_shape, 1, pad, 1, 0)
+    nbytes = C.c_size_t(0)
+    _check(lib().kxc_hip_conv2d_winograd_weight_bytes(C.byref(d), C.byref(nbytes)))
+    return nbytes.value
+
+
+def conv2d_winograd_variant(x_shape, w_shape, stride=1, pad=1, dil=1):
+    d = conv_desc(x_shape, w_shape, stride, pad, dil, 0)
+    return lib().kxc_hip_conv2d_winograd_variant(C.byref(d)).decode()
+
+
+def conv2d_winograd_transform_weights(x_shape, w, pad=1):
+    """OIHW 3x3 weights -> the transformed, packed form kxc_hip_conv2d_winograd_nchw_f32 reads."""
+    import torch
+    _need(w, torch.float32, "w")
+    d = conv_desc(tuple(x_shape), tuple(w.shape), 1, pad, 1, 0)
+    nbytes = C.c_size_t(0)
+    _check(lib().kxc_hip_conv2d_winograd_weight_bytes(C.byref(d), C.byref(nbytes)))
+    u = torch.empty(nbytes.value // 4, dtype=torch.float32, device=w.device)
+    _check(lib().kxc_hip_conv2d_winograd_transform_weights(C.byref(d), _p(w), _p(u), _stream()))
+    return u
+
+
+def conv2d_winograd(x, u, w_shape, bias=None, residual=None, pad=1, relu=False, out=None):
+    import torch
+    _need(x, torch.float32, "x"); _need(u, torch.float32, "u")
+    _need(bias, torch.float32, "bias"); _need(residual, torch.float32, "residual")
+    flags = (CONV_BIAS if bias is not None else 0) | (CONV_RESIDUAL if residual is not None else 0) | \
+            (CONV_RELU if relu else 0)
+    d = conv_desc(tuple(x.shape), tuple(w_shape), 1, pad, 1, flags)
+    y = out if out is not None else torch.empty(conv_out_shape(d), dtype=torch.float32, device=x.device)
+    _check(lib().kxc_hip_conv2d_winograd_nchw_f32(C.byref(d), _p(x), _p(u), _p(bias), _p(residual), _p(y), _stream()))
     return y
 
 
@@ -443,6 +490,12 @@ class Plan:
     def add_conv2d(self, desc, x, w, bias, residual, y):
         _check(lib().kxc_hip_plan_add_conv2d(self._h, C.byref(desc), x, w, bias, residual, y))
 
+    def add_conv2d_winograd(self, desc, x, w, bias, residual, y, u):
+        _check(lib().kxc_hip_plan_add_conv2d_winograd(self._h, C.byref(desc), x, w, bias, residual, y, u))
+
+    def invalidate_constants(self):
+        _check(lib().kxc_hip_plan_invalidate_constants(self._h))
+
     def add_pool2d(self, desc, x, y):
         _check(lib().kxc_hip_plan_add_pool2d(self._h, C.byref(desc), x, y))
 
@@ -516,6 +569,26 @@ class Plan:
 
     def run_packed(self, args, stream):
         _check(lib().kxc_hip_plan_run(self._h, args, C.c_void_p(stream)))
+
+    def serialize(self):
+        """The finalized plan as text (kxc_hip_plan_serialize)."""
+        need = C.c_size_t(0)
+        _check(lib().kxc_hip_plan_serialize(self._h, None, C.c_size_t(0), C.byref(need)))
+        buf = C.create_string_buffer(need.value)
+        _check(lib().kxc_hip_plan_serialize(self._h, buf, C.c_size_t(need.value), C.byref(need)))
+        return buf.value.decode()
+
+    @classmethod
+    def deserialize(cls, text, device_id=0):
+        """A plan without generated-kernel nodes rebuilt from serialize() output, finalized."""
+        self = cls.__new__(cls)
+        self._h = C.c_void_p()
+        _check(lib().kxc_hip_plan_deserialize(text.encode(), C.c_int32(device_id), None, C.c_int32(0), C.byref(self._h)))
+        self.num_args = None
+        return self
+
+    def node_symbol(self, i):
+        return lib().kxc_hip_plan_node_symbol(self._h, C.c_int32(i)).decode()
 
     def symbols(self):
         n = lib().kxc_hip_plan_num_nodes(self._h)

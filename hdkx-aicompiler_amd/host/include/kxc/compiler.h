@@ -32,6 +32,7 @@ struct CompileConfigNode {
     bool hip_use_handwritten{true};    // false: every operator goes through the TIR -> HIP generator
     bool hip_fuse{true};               // fold bias / residual add / ReLU into convolution launches
     bool hip_concurrent_branches{true};   // run a block's downsample convolution beside its first 3x3 convolution
+    bool hip_winograd{true};              // 3x3 stride-1 convolutions with constant weights as Winograd F(2x2,3x3) where faster
     bool sync_after_run{true};
 };
 class CompileConfig : public Ref<CompileConfigNode> {

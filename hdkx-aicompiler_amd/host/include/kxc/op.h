@@ -61,6 +61,11 @@ struct HIPDispatchContext {
     bool fused_relu = false;
     bool has_residual = false;
     HIPBuffer residual;
+    // input_constant[i]: input i is a module constant (same tensor on every run).  alloc_persistent(bytes) hands
+    // out a workspace region that lives as long as the module, for a re-laid-out copy of such a constant; it is
+    // empty when the configuration rules that out.
+    std::vector<bool> input_constant;
+    std::function<HIPBuffer(int64_t)> alloc_persistent;
 };
 // Appends the launch(es) for one call to the plan; returns the kernel_symbol, or "" to decline (the
 // call is then compiled through the code generator).

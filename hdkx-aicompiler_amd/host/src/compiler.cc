@@ -364,6 +364,16 @@ private:
                 ctx.input_types.push_back(a.checked_type());
                 ctx.inputs.push_back(BufferOf(a.get()));
             }
+            for (const auto& a : g.head->args) ctx.input_constant.push_back(dynamic_cast<const ConstantNode*>(Resolve(a.get())) != nullptr);
+            const char* wino_env = std::getenv("KXC_HIP_WINOGRAD");                 // "0" switches Winograd off
+            if (cfg_->hip_winograd && !(wino_env && wino_env[0] == '0'))
+                ctx.alloc_persistent = [this](int64_t bytes) {
+                    // above everything handed out so far and never released: no activation of an earlier or later
+                    // step ever shares the region, so what the first run wrote there is still valid in the next
+                    const int64_t off = arena_.top;
+                    arena_.top += (std::max<int64_t>(bytes, 1) + 255) / 256 * 256;
+                    return relay::HIPBuffer{KXC_HIP_BUF_WORKSPACE, off};
+                };
             ctx.out_type = g.tail->checked_type_;
             ctx.output = out;
             ctx.fused_relu = g.fused_relu;

@@ -65,6 +65,18 @@ std::string Conv2DDispatch(const HIPDispatchContext& c, kxc_hip_plan* plan) {
     d.flags = (has_bias ? KXC_HIP_CONV_BIAS : 0u) | (c.has_residual ? KXC_HIP_CONV_RESIDUAL : 0u) |
               (c.fused_relu ? KXC_HIP_CONV_RELU : 0u);
     const kxc_hip_buf none{KXC_HIP_BUF_NONE, 0};
+    // 3x3 stride-1 convolutions with constant weights run as Winograd F(2x2,3x3) when the library expects that to
+    // be faster for the shape; the transformed weights get a workspace region of their own.
+    if (c.alloc_persistent && c.input_constant.size() > 1 && c.input_constant[1] && kxc_hip_conv2d_winograd_preferred(&d)) {
+        size_t u_bytes = 0;
+        Check(kxc_hip_conv2d_winograd_weight_bytes(&d, &u_bytes), "nn_conv2d dispatch");
+        const HIPBuffer u = c.alloc_persistent(static_cast<int64_t>(u_bytes));
+        Check(kxc_hip_plan_add_conv2d_winograd(plan, &d, B(c.inputs[0]), B(c.inputs[1]), has_bias ? B(c.inputs[2]) : none,
+                                               c.has_residual ? B(c.residual) : none, B(c.output), B(u)),
+              "nn_conv2d dispatch");
+        return std::string("kxc_conv2d_nchw_f32.") + kxc_hip_conv2d_winograd_variant(&d) + (has_bias ? "+bias" : "") +
+               (c.has_residual ? "+add" : "") + (c.fused_relu ? "+relu" : "");
+    }
     Check(kxc_hip_plan_add_conv2d(plan, &d, B(c.inputs[0]), B(c.inputs[1]), has_bias ? B(c.inputs[2]) : none,
                                   c.has_residual ? B(c.residual) : none, B(c.output)),
           "nn_conv2d dispatch");

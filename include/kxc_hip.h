@@ -117,6 +117,24 @@ int32_t kxc_hip_conv2d_nchw_f32(const kxc_hip_conv2d_desc* desc, const float* x,
 /* Name of the kernel variant the library would launch for this shape ("mfma_..." or "direct"). */
 const char* kxc_hip_conv2d_variant(const kxc_hip_conv2d_desc* desc);
 
+/* nn_conv2d with a 3x3 filter, stride 1, dilation 1 and c % 4 == 0 as Winograd F(2x2, 3x3) on the matrix cores:
+ * same operator and epilogue as kxc_hip_conv2d_nchw_f32 (convolution.cc:38-75, nn.h:107-158) with 2.25x fewer
+ * multiplies; the sums are formed in a different order, results agree within the operator's fp32 tolerance.
+ * The filter is passed in transformed form: `u` holds weight_bytes bytes written by ..._transform_weights from
+ * the OIHW tensor (the reference keeps weights as module constants, CompiledModule::GetConstants,
+ * include/compiler.h:83, so a caller transforms them once per module).
+ *   ..._supported: 1 when the shape qualifies, else 0 (no error is recorded). */
+int32_t kxc_hip_conv2d_winograd_supported(const kxc_hip_conv2d_desc* desc);
+int32_t kxc_hip_conv2d_winograd_weight_bytes(const kxc_hip_conv2d_desc* desc, size_t* out_bytes);
+int32_t kxc_hip_conv2d_winograd_transform_weights(const kxc_hip_conv2d_desc* desc, const float* w_oihw, float* u,
+                                                  void* stream);
+int32_t kxc_hip_conv2d_winograd_nchw_f32(const kxc_hip_conv2d_desc* desc, const float* x, const float* u,
+                                         const float* bias, const float* residual, float* y, void* stream);
+const char* kxc_hip_conv2d_winograd_variant(const kxc_hip_conv2d_desc* desc);
+/* 1 when the shape qualifies and the launch is large enough for this path to beat kxc_hip_conv2d_nchw_f32
+ * (measured on MI355X: at least one workgroup per compute unit), else 0. */
+int32_t kxc_hip_conv2d_winograd_preferred(const kxc_hip_conv2d_desc* desc);
+
 /* nn_relu: ReluCompute (src/relay/op/nn/activation.cc:14-19). */
 int32_t kxc_hip_relu_f32(const float* x, float* y, int64_t n, void* stream);
 /* add / subtract / multiply / divide: broadcast.h:90-113 via math.cc:41-95.
@@ -259,6 +277,15 @@ int32_t kxc_hip_plan_destroy(kxc_hip_plan* plan);
 /* Node builders; `symbol` is stored as KernelExecNode::kernel_symbol would be. */
 int32_t kxc_hip_plan_add_conv2d(kxc_hip_plan* plan, const kxc_hip_conv2d_desc* desc, kxc_hip_buf x,
                                 kxc_hip_buf w, kxc_hip_buf bias, kxc_hip_buf residual, kxc_hip_buf y);
+/* The same operator through kxc_hip_conv2d_winograd_nchw_f32.  `w` is the OIHW weight tensor as the reference
+ * passes it (a module constant among the packed arguments); `u` is a workspace region of
+ * kxc_hip_conv2d_winograd_weight_bytes bytes that no other node uses.  The node transforms w into u on the first
+ * run and again whenever a different pointer arrives for w; a caller that rewrites the weights in place calls
+ * kxc_hip_plan_invalidate_constants. */
+int32_t kxc_hip_plan_add_conv2d_winograd(kxc_hip_plan* plan, const kxc_hip_conv2d_desc* desc, kxc_hip_buf x,
+                                         kxc_hip_buf w, kxc_hip_buf bias, kxc_hip_buf residual, kxc_hip_buf y,
+                                         kxc_hip_buf u);
+int32_t kxc_hip_plan_invalidate_constants(kxc_hip_plan* plan);
 int32_t kxc_hip_plan_add_pool2d(kxc_hip_plan* plan, const kxc_hip_pool2d_desc* desc, kxc_hip_buf x,
                                 kxc_hip_buf y);
 int32_t kxc_hip_plan_add_global_avg_pool2d(kxc_hip_plan* plan, int64_t n, int64_t c, int64_t h,

@@ -157,6 +157,112 @@ def test_conv_reduction_split_over_workgroups(pkg, fast_orc, synth, monkeypatch,
     assert_bit_exact(got2, got1, "split reduction is deterministic")
 
 
+# ------------------------------------------------------------------ Winograd F(2x2,3x3)
+WINOGRAD_SHAPES = [
+    (2, 64, 56, 56, 64, 1),       # layer1
+    (3, 128, 28, 28, 128, 1),     # layer2
+    (5, 256, 14, 14, 256, 1),     # layer3: tile groups cross image boundaries
+    (7, 512, 7, 7, 512, 1),       # layer4: odd output size, partial 2x2 blocks
+    (1, 8, 9, 33, 40, 1),         # ragged: output channels not a multiple of 32, odd width
+    (2, 12, 10, 6, 96, 0),        # no padding
+    (1, 4, 5, 4, 16, 2),          # padding wider than the filter needs
+    (3, 20, 1, 1, 32, 1),         # one pixel
+]
+
+
+@pytest.mark.parametrize("shape", WINOGRAD_SHAPES, ids=lambda s: "x".join(map(str, s)))
+def test_conv_winograd_against_oracle(pkg, fast_orc, synth, shape):
+    """The Winograd path of nn_conv2d (3x3, stride 1) against the CPU loop nest: fp32 tolerance, with and without
+    the fused bias / residual / ReLU."""
+    n, c, h, w, o, p = shape
+    assert pkg.conv2d_winograd_supported((n, c, h, w), (o, c, 3, 3), 1, p)
+    seed = 7000 + WINOGRAD_SHAPES.index(shape) * 5
+    x = synth.uniform((n, c, h, w), seed)
+    wt = synth.normal((o, c, 3, 3), seed + 1, float(np.sqrt(2.0 / (c * 9))))
+    b = synth.uniform((o,), seed + 2, -0.1, 0.1)
+    oh, ow = h + 2 * p - 2, w + 2 * p - 2
+    skip = synth.uniform((n, o, oh, ow), seed + 3)
+    u = pkg.conv2d_winograd_transform_weights((n, c, h, w), dev(wt), p)
+    assert u.numel() * 4 == pkg.conv2d_winograd_weight_bytes((n, c, h, w), (o, c, 3, 3), p)
+    want = fast_orc.conv_chain(x, wt, b, 1, p, skip, True)
+    got = host(pkg.conv2d_winograd(dev(x), u, wt.shape, dev(b), dev(skip), p, True))
+    assert_close(got, want, what="winograd %s" % (shape,))
+    want = fast_orc.conv2d(x, wt, 1, p)
+    got = host(pkg.conv2d_winograd(dev(x), u, wt.shape, None, None, p, False))
+    assert_close(got, want, what="winograd bare %s" % (shape,))
+
+
+def test_conv_winograd_exact_on_small_integers(pkg, orc):
+    """Small integers keep every transformed value, product and partial sum exact (the filter transform's halves
+    and quarters included), so the result must equal the direct loop nest bit for bit: isolates indexing."""
+    rng = np.random.default_rng(12)
+    for (n, c, h, w, o, p) in [(3, 16, 14, 14, 64, 1), (9, 8, 7, 7, 64, 1), (2, 4, 9, 12, 48, 0)]:
+        x = rng.integers(-3, 4, (n, c, h, w)).astype(np.float32)
+        wt = (4 * rng.integers(-2, 3, (o, c, 3, 3))).astype(np.float32)
+        b = rng.integers(-5, 6, (o,)).astype(np.float32)
+        want = orc.conv_chain(x, wt, b, 1, p, None, True)
+        u = pkg.conv2d_winograd_transform_weights(x.shape, dev(wt), p)
+        assert_bit_exact(host(pkg.conv2d_winograd(dev(x), u, wt.shape, dev(b), None, p, True)), want, str((n, c, h, w, o, p)))
+
+
+def test_conv_winograd_unsupported_shapes_are_refused(pkg):
+    assert not pkg.conv2d_winograd_supported((1, 8, 8, 8), (16, 8, 3, 3), 2, 1)        # stride
+    assert not pkg.conv2d_winograd_supported((1, 8, 8, 8), (16, 8, 1, 1), 1, 0)        # filter size
+    assert not pkg.conv2d_winograd_supported((1, 6, 8, 8), (16, 6, 3, 3), 1, 1)        # channels not a multiple of 4
+    assert not pkg.conv2d_winograd_supported((1, 8, 8, 8), (16, 8, 3, 3), 1, 1, 2)     # dilation
+    assert not pkg.conv2d_winograd_preferred((1, 64, 56, 56), (64, 64, 3, 3))          # batch 1: direct path is faster
+    assert pkg.conv2d_winograd_preferred((64, 64, 56, 56), (64, 64, 3, 3))
+    x = torch.zeros((1, 6, 8, 8), device="cuda"); u = torch.zeros((1024,), device="cuda")
+    with pytest.raises(pkg.KxcHipError):
+        pkg.conv2d_winograd(x, u, (16, 6, 3, 3))
+
+
+def test_conv_winograd_full_batch_properties(pkg, synth):
+    """BASELINE-size layers (batch 64): Winograd vs the implicit-GEMM kernel on the GPU, linearity in the weights
+    and batch independence."""
+    for (c, hw, o) in [(64, 56, 64), (512, 7, 512)]:
+        x = dev(synth.uniform((64, c, hw, hw), 7100))
+        w1 = dev(synth.normal((o, c, 3, 3), 7101, float(np.sqrt(2.0 / (9 * c)))))
+        w2 = dev(synth.normal((o, c, 3, 3), 7102, float(np.sqrt(2.0 / (9 * c)))))
+        b = dev(synth.uniform((o,), 7103, -0.1, 0.1))
+        u1 = pkg.conv2d_winograd_transform_weights(x.shape, w1); u2 = pkg.conv2d_winograd_transform_weights(x.shape, w2)
+        u12 = pkg.conv2d_winograd_transform_weights(x.shape, w1 + w2)
+        fast = pkg.conv2d_winograd(x, u1, w1.shape, b, None, 1, True)
+        other = pkg.conv2d(x, w1, b, None, 1, 1, 1, True)
+        assert_close(host(fast), host(other), what="winograd vs implicit GEMM, batch 64")
+        y12 = pkg.conv2d_winograd(x, u12, w1.shape); y1 = pkg.conv2d_winograd(x, u1, w1.shape); y2 = pkg.conv2d_winograd(x, u2, w1.shape)
+        assert_close(host(y12), host(y1 + y2), what="linearity")
+        one = pkg.conv2d_winograd(x[17:18].contiguous(), u1, w1.shape, b, None, 1, True)
+        assert_close(host(one), host(fast[17:18]), tol=1e-4, what="batch independence")
+
+
+def test_plan_winograd_node_transforms_constants_once(pkg, synth, fast_orc):
+    """A plan's Winograd node takes the OIHW weights as a packed argument, transforms them on the first run and when
+    another tensor is passed; the serialised plan keeps the node."""
+    n, c, h, o = 4, 16, 12, 64
+    x = synth.uniform((n, c, h, h), 7200)
+    w1 = synth.normal((o, c, 3, 3), 7201, 0.1); w2 = synth.normal((o, c, 3, 3), 7202, 0.1)
+    b = synth.uniform((o,), 7203, -0.1, 0.1)
+    d = pkg.ConvDesc(n, c, h, h, o, 3, 3, 1, 1, 1, 1, 1, 1, pkg.CONV_BIAS | pkg.CONV_RELU)
+    ubytes = pkg.conv2d_winograd_weight_bytes((n, c, h, h), (o, c, 3, 3))
+    plan = pkg.Plan(4)
+    plan.add_conv2d_winograd(d, pkg.Buf.arg(0), pkg.Buf.arg(1), pkg.Buf.arg(2), pkg.Buf.none(), pkg.Buf.arg(3), pkg.Buf.ws(0))
+    plan.finalize(ubytes)
+    assert "winograd" in plan.node_symbol(0)
+    xd, w1d, w2d, bd = dev(x), dev(w1), dev(w2), dev(b)
+    y = torch.empty((n, o, h, h), device="cuda")
+    for wd, wh in ((w1d, w1), (w1d, w1), (w2d, w2)):
+        plan.run([xd, wd, bd, y]); torch.cuda.synchronize()
+        assert_close(host(y), fast_orc.conv_chain(x, wh, b, 1, 1, None, True), what="plan winograd")
+    w2d.copy_(w1d); plan.invalidate_constants()          # rewritten in place: the caller says so
+    plan.run([xd, w2d, bd, y]); torch.cuda.synchronize()
+    assert_close(host(y), fast_orc.conv_chain(x, w1, b, 1, 1, None, True), what="plan winograd after invalidate")
+    again = pkg.Plan.deserialize(plan.serialize(), 0)
+    y2 = torch.empty_like(y)
+    again.run([xd, w1d, bd, y2]); torch.cuda.synchronize()
+    assert_bit_exact(host(y2), host(y), "deserialised winograd plan")
+
+
 def test_conv_dilation(pkg, orc, synth):
     x = synth.uniform((1, 8, 20, 20), 300); w = synth.uniform((32, 8, 3, 3), 301)
     want = orc.conv2d(x, w, 1, 2, 2)

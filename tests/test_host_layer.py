@@ -20,9 +20,10 @@ def _ensure_built():
         subprocess.check_call(["make", "-C", HOST, "-j8"])
 
 
-def run(*args, timeout=600):
+def run(*args, timeout=600, env=None):
     _ensure_built()
-    r = subprocess.run([BIN] + list(args), capture_output=True, text=True, timeout=timeout)
+    r = subprocess.run([BIN] + list(args), capture_output=True, text=True, timeout=timeout,
+                       env=dict(os.environ, **env) if env else None)
     assert r.returncode == 0, r.stdout[-3000:] + r.stderr[-3000:]
     return r.stdout
 
@@ -80,6 +81,16 @@ def test_resnet18_hip_plan_without_gpu():
     assert sum(s.startswith("kxc_conv2d") and s.endswith("+bias") for s in syms) == 3   # downsamples
     assert len(plan["constant_value_ids"]) == 42 and len(plan["input_value_ids"]) == 1
     assert all(n["kind"] == "kernel" and n["worker_set"] == [0] for n in plan["nodes"])
+    # at batch 64 every 3x3 stride-1 convolution (constant weights) takes the Winograd kernel, the rest do not
+    assert sum(".winograd_f2k3" in s for s in syms) == 13 and sum(".mfma_" in s for s in syms) == 7
+    with tempfile.TemporaryDirectory() as d:
+        run("resnet18", "hip", d, "64", "224", env={"KXC_HIP_WINOGRAD": "0"})
+        off = json.load(open(os.path.join(d, "plan.json")))
+    assert not any("winograd" in n["kernel_symbol"] for n in off["nodes"])
+    with tempfile.TemporaryDirectory() as d:
+        run("resnet18", "hip", d, "1", "224")
+        one = json.load(open(os.path.join(d, "plan.json")))
+    assert not any("winograd" in n["kernel_symbol"] for n in one["nodes"])     # batch 1: too small to pay
 
 
 # ------------------------------------------------------------------ GPU
@@ -104,6 +115,22 @@ def test_resnet18_hip_matches_oracle(synth):
         got = np.fromfile(os.path.join(d, "logits.bin"), np.float32).reshape(2, 1000)
     want = Oracle(fast=True).resnet18(x, consts)
     assert_close(got, want, what="C++ host layer, ResNet-18 logits", floor="scale")
+
+
+@pytest.mark.gpu
+def test_resnet18_hip_winograd_matches_oracle(synth):
+    """The same network with every 3x3 stride-1 convolution on the Winograd kernel (forced at this small batch):
+    logits within the fp32 tolerance, and the saved plan replays to the identical output."""
+    from gpu_util import assert_close
+    with tempfile.TemporaryDirectory() as d:
+        x, consts = _write_resnet_inputs(synth, d, 3, 2, 224)
+        out = run("resnet18", "hip", d, "2", "224", env={"KXC_HIP_WINOGRAD_MIN_UNITS": "0"})
+        assert "execution plan replayed: 23 launches, identical output" in out
+        plan = json.load(open(os.path.join(d, "plan.json")))
+        assert sum(".winograd_f2k3" in n["kernel_symbol"] for n in plan["nodes"]) == 13
+        got = np.fromfile(os.path.join(d, "logits.bin"), np.float32).reshape(2, 1000)
+    want = Oracle(fast=True).resnet18(x, consts)
+    assert_close(got, want, what="C++ host layer, ResNet-18 logits (Winograd)", floor="scale")
 
 
 @pytest.mark.gpu
