@@ -6,7 +6,8 @@
 A step is one forward pass of the ResNet-18 launch plan (fp32, batch 64, [64,3,224,224] input,
 seeded synthetic weights/input already resident in HBM) enqueued on one stream through the C ABI.
 Prints ONE JSON line: whole-job throughput (img/s), the roofline position of the dominant kernel
-(the 3x3/1 convolution of layer1, timed with events on the launch stream), per-layer and
+(the 3x3/1 convolution of layer1 -- the Winograd kernel the plan runs, with the implicit-GEMM kernel beside it --
+timed with events on the launch stream), per-layer and
 per-operator figures, and the single-core CPU baseline (the CPU checker in oracle/, timed on a
 bounded sample: one image).
 """
@@ -39,10 +40,10 @@ def _event_time_ms(torch, fn, iters, warmup):
     return start.elapsed_time(stop) / iters
 
 
-def _profiled_traffic_bytes():
+def _profiled_traffic_bytes(name):
     """HBM bytes per launch of the dominant kernel, as measured with the rocprofv3 FETCH_SIZE and
     WRITE_SIZE passes whose summary is kept beside this file (counters cannot be read from inside a run)."""
-    path = os.path.join(os.path.dirname(os.path.abspath(__file__)), "profiles", "conv3x3_layer1_bs64_counters.md")
+    path = os.path.join(os.path.dirname(os.path.abspath(__file__)), "profiles", name)
     try:
         for line in open(path):
             if line.startswith("TRAFFIC_BYTES_PER_LAUNCH="):
@@ -118,16 +119,39 @@ def main():
     lw = dev(synth.normal((64, 64, 3, 3), 4101, float(np.sqrt(2.0 / 576))))
     lb = dev(synth.uniform((64,), 4103, -0.1, 0.1))
     ly = torch.empty((batch, 64, 56, 56), device="cuda")
-    conv_ms = _event_time_ms(torch, lambda: pkg.conv2d(lx, lw, lb, None, 1, 1, 1, True, out=ly), 30, 5)
-    conv_flop = 2.0 * batch * 64 * 56 * 56 * 64 * 9
-    conv_tflops = conv_flop / (conv_ms * 1e-3) / 1e12
-    roofline = {"bound": "mfma", "kernel": "conv_mfma_kernel<3,3> (layer1: [%d,64,56,56]x[64,64,3,3] s1 p1 +bias+relu)" % batch,
-                "variant": pkg.conv2d_variant((batch, 64, 56, 56), (64, 64, 3, 3), 1, 1),
-                "achieved": round(conv_tflops, 3), "peak": PEAK_FP32_MFMA_TFLOPS, "unit": "TFLOP/s",
-                "frac": round(conv_tflops / PEAK_FP32_MFMA_TFLOPS, 4), "avg_launch_ms": round(conv_ms, 4),
-                "flop_per_launch": conv_flop, "traffic": _profiled_traffic_bytes() if batch == 64 else None,
-                "traffic_unit": "bytes per launch (FETCH_SIZE + WRITE_SIZE, calibrated on a copy; from profiles/)",
-                "algorithmic_bytes_per_launch": 4 * (2 * batch * 64 * 56 * 56 + 64 * 64 * 9 + 64)}
+    conv_flop = 2.0 * batch * 64 * 56 * 56 * 64 * 9          # multiply-adds of the direct definition, x2
+    gemm_ms = _event_time_ms(torch, lambda: pkg.conv2d(lx, lw, lb, None, 1, 1, 1, True, out=ly), 30, 5)
+    gemm_tflops = conv_flop / (gemm_ms * 1e-3) / 1e12
+    gemm_row = {"kernel": "conv_mfma_kernel<3,3> (implicit GEMM)", "variant": pkg.conv2d_variant((batch, 64, 56, 56), (64, 64, 3, 3), 1, 1),
+                "avg_launch_ms": round(gemm_ms, 4), "achieved": round(gemm_tflops, 3), "frac": round(gemm_tflops / PEAK_FP32_MFMA_TFLOPS, 4),
+                "traffic": _profiled_traffic_bytes("conv3x3_layer1_bs64_counters.md") if batch == 64 else None}
+    algorithmic_bytes = 4 * (2 * batch * 64 * 56 * 56 + 64 * 64 * 9 + 64)
+    if pkg.conv2d_winograd_preferred((batch, 64, 56, 56), (64, 64, 3, 3)) and os.environ.get("KXC_HIP_WINOGRAD", "1") != "0":
+        # the launch plan runs this layer as Winograd F(2x2,3x3): 16 multiplies per 2x2 outputs instead of 36.
+        # `achieved` is the ALGORITHMIC rate (direct-definition FLOP / time); `matrix_core_*` is what the matrix
+        # cores actually execute (4/9 of it), i.e. how busy the MFMA pipe is.
+        lu = pkg.conv2d_winograd_transform_weights(lx.shape, lw, 1)
+        conv_ms = _event_time_ms(torch, lambda: pkg.conv2d_winograd(lx, lu, lw.shape, lb, None, 1, True, out=ly), 30, 5)
+        conv_tflops = conv_flop / (conv_ms * 1e-3) / 1e12
+        executed = conv_flop * 16.0 / 36.0
+        roofline = {"bound": "mfma", "kernel": "wino_kernel (layer1: [%d,64,56,56]x[64,64,3,3] s1 p1 +bias+relu, Winograd F(2x2,3x3))" % batch,
+                    "variant": pkg.conv2d_winograd_variant(lx.shape, lw.shape),
+                    "achieved": round(conv_tflops, 3), "peak": PEAK_FP32_MFMA_TFLOPS, "unit": "TFLOP/s",
+                    "frac": round(conv_tflops / PEAK_FP32_MFMA_TFLOPS, 4), "avg_launch_ms": round(conv_ms, 4),
+                    "flop_per_launch": conv_flop,
+                    "matrix_core_flop_per_launch": executed,
+                    "matrix_core_tflops": round(executed / (conv_ms * 1e-3) / 1e12, 3),
+                    "matrix_core_frac": round(executed / (conv_ms * 1e-3) / 1e12 / PEAK_FP32_MFMA_TFLOPS, 4),
+                    "traffic": _profiled_traffic_bytes("winograd_layer1_bs64_counters.md") if batch == 64 else None,
+                    "traffic_unit": "bytes per launch (FETCH_SIZE + WRITE_SIZE, calibrated on a copy; from profiles/)",
+                    "algorithmic_bytes_per_launch": algorithmic_bytes, "same_layer_implicit_gemm": gemm_row}
+    else:
+        roofline = {"bound": "mfma", "kernel": "conv_mfma_kernel<3,3> (layer1: [%d,64,56,56]x[64,64,3,3] s1 p1 +bias+relu)" % batch,
+                    "variant": gemm_row["variant"], "achieved": gemm_row["achieved"], "peak": PEAK_FP32_MFMA_TFLOPS,
+                    "unit": "TFLOP/s", "frac": gemm_row["frac"], "avg_launch_ms": gemm_row["avg_launch_ms"],
+                    "flop_per_launch": conv_flop, "traffic": gemm_row["traffic"],
+                    "traffic_unit": "bytes per launch (FETCH_SIZE + WRITE_SIZE, calibrated on a copy; from profiles/)",
+                    "algorithmic_bytes_per_launch": algorithmic_bytes}
 
     result = {
         "metric": "resnet18_fp32_bs64_img_per_s", "value": round(img_s, 2), "unit": "img/s",
@@ -183,9 +207,18 @@ def bench_conv_layers(torch, pkg, synth, dev, batch):
         skip = torch.zeros_like(y) if res else None
         ms = _event_time_ms(torch, lambda: pkg.conv2d(x, w, b, skip, s, p, 1, True, out=y), 20, 3)
         flop = 2.0 * batch * o * oh * oh * c * k * k
-        rows.append({"layer": name, "variant": pkg.conv2d_variant((batch, c, h, h), (o, c, k, k), s, p), "count": count,
-                     "ms": round(ms, 4), "tflops": round(flop / (ms * 1e-3) / 1e12, 2),
-                     "frac_fp32_mfma_peak": round(flop / (ms * 1e-3) / 1e12 / PEAK_FP32_MFMA_TFLOPS, 4)})
+        row = {"layer": name, "variant": pkg.conv2d_variant((batch, c, h, h), (o, c, k, k), s, p), "count": count,
+               "ms": round(ms, 4), "tflops": round(flop / (ms * 1e-3) / 1e12, 2),
+               "frac_fp32_mfma_peak": round(flop / (ms * 1e-3) / 1e12 / PEAK_FP32_MFMA_TFLOPS, 4)}
+        if k == 3 and s == 1 and pkg.conv2d_winograd_preferred((batch, c, h, h), (o, c, k, k), s, p):
+            # what the launch plan uses for this layer; tflops = direct-definition FLOP / time
+            u = pkg.conv2d_winograd_transform_weights(x.shape, w, p)
+            wms = _event_time_ms(torch, lambda: pkg.conv2d_winograd(x, u, w.shape, b, skip, p, True, out=y), 20, 3)
+            row["winograd"] = {"variant": pkg.conv2d_winograd_variant(x.shape, w.shape, s, p), "ms": round(wms, 4),
+                               "tflops": round(flop / (wms * 1e-3) / 1e12, 2),
+                               "frac_fp32_mfma_peak": round(flop / (wms * 1e-3) / 1e12 / PEAK_FP32_MFMA_TFLOPS, 4),
+                               "matrix_core_frac": round(flop * 16.0 / 36.0 / (wms * 1e-3) / 1e12 / PEAK_FP32_MFMA_TFLOPS, 4)}
+        rows.append(row)
     return rows
 
 

@@ -190,21 +190,11 @@ wino_kernel(const WinoArgs a) {
         for (int i = 0; i < ITEMS; ++i)
 #pragma unroll
             for (int q = 0; q < 12; ++q) d[i][q] = load_f32(xr, goff[i][q], soff);
-#ifdef KXC_WDBG_NO_RAW
-#pragma unroll
-        for (int i = 0; i < ITEMS; ++i)
-#pragma unroll
-            for (int q = 0; q < 12; ++q) d[i][q] = (float)(goff[i][q] + soff);
-#endif
     };
     auto issue_u = [&](int s, float* buf) {
 #pragma unroll
         for (int j = 0; j < ULOADS; ++j)
-#ifndef KXC_WDBG_NO_U
             load16_to_lds(ur, (lds_ptr_t)(buf + (j * NTH + wave * 64) * 4), uoff[j], static_cast<uint32_t>(s) * 8192u);
-#else
-            ;
-#endif
     };
     auto transform = [&](float* buf) {
 #pragma unroll
@@ -235,13 +225,8 @@ wino_kernel(const WinoArgs a) {
     auto mm = [&](int fg, int set) {
 #pragma unroll
         for (int f = 0; f < 4; ++f) {
-#ifdef KXC_WDBG_NO_MFMA
-            acc[fg * 4 + f][0][0] += ra[set][0][f] + rb[set][f];
-            acc[fg * 4 + f][1][0] += ra[set][1][f];
-#else
             acc[fg * 4 + f][0] = __builtin_amdgcn_mfma_f32_16x16x4f32(ra[set][0][f], rb[set][f], acc[fg * 4 + f][0], 0, 0, 0);
             acc[fg * 4 + f][1] = __builtin_amdgcn_mfma_f32_16x16x4f32(ra[set][1][f], rb[set][f], acc[fg * 4 + f][1], 0, 0, 0);
-#endif
         }
     };
 
@@ -303,9 +288,6 @@ wino_kernel(const WinoArgs a) {
     // ---- epilogue: accumulator register g of block kb holds output channel 16*kb + 4*(lane/16) + g, tile lane%16
     const int tile = t0 + wave_t * 16 + (lane & 15);
     if (tile >= a.NT) return;
-#ifdef KXC_WDBG_NO_EPI
-    if (acc[0][0][0] != 123456.789f) return;
-#endif
     const int n = fast_div(tile, a.div_ti), rem = tile - n * a.TI;
     const int ty = fast_div(rem, a.div_tw), tx = rem - ty * a.TW;
     const int oh = 2 * ty, ow = 2 * tx;
@@ -392,11 +374,21 @@ bool Supported(const kxc_hip_conv2d_desc* d) {
     return x_bytes < (1LL << 31) && y_elems < (1LL << 31) && u_bytes < (1LL << 31) && tiles < (1LL << 30);
 }
 
+int64_t Tiles(const kxc_hip_conv2d_desc* d) {
+    const int64_t oh = static_cast<int64_t>(d->h) + 2 * d->pad_h - 2, ow = static_cast<int64_t>(d->w) + 2 * d->pad_w - 2;
+    return static_cast<int64_t>(d->n) * CeilDiv(oh, 2) * CeilDiv(ow, 2);
+}
+
+// Measured on MI355X: 64 x 32 workgroups (four waves) are the fastest shape once there is one per compute unit;
+// smaller launches run faster as twice as many 64 x 16 workgroups of two waves.
 const WinoVariant* SelectWino(const kxc_hip_conv2d_desc* d) {
     if (const char* e = std::getenv("KXC_HIP_WINOGRAD_VARIANT")) {
         for (int i = 0; i < kNumWino; ++i)
             if (std::strcmp(e, kWino[i].name) == 0) return &kWino[i];
     }
+    const int64_t units = CeilDiv(Tiles(d), 32) * CeilDiv(d->o, 64);
+    for (int i = 0; i < kNumWino; ++i)
+        if (kWino[i].wk == 2 && kWino[i].wt == (units < 256 ? 1 : 2)) return &kWino[i];
     return &kWino[0];
 }
 
@@ -408,13 +400,12 @@ int32_t kxc_hip_conv2d_winograd_supported(const kxc_hip_conv2d_desc* desc) { ret
 
 int32_t kxc_hip_conv2d_winograd_preferred(const kxc_hip_conv2d_desc* desc) {
     if (!Supported(desc)) return 0;
-    const WinoVariant* v = SelectWino(desc);
-    const int64_t oh = static_cast<int64_t>(desc->h) + 2 * desc->pad_h - 2, ow = static_cast<int64_t>(desc->w) + 2 * desc->pad_w - 2;
-    const int64_t tiles = static_cast<int64_t>(desc->n) * CeilDiv(oh, 2) * CeilDiv(ow, 2);
-    const int64_t units = CeilDiv(tiles, 16 * v->wt) * CeilDiv(desc->o, 32 * v->wk);
-    int64_t min_units = 256;                     // one workgroup per compute unit
-    if (const char* e = std::getenv("KXC_HIP_WINOGRAD_MIN_UNITS")) min_units = std::atoll(e);
-    return units >= min_units ? 1 : 0;
+    // A workgroup walks all input channels (c / 4 steps of ~0.7 us) whatever the launch size, while the
+    // implicit-GEMM kernel splits a long reduction over workgroups when the launch is small: Winograd pays from
+    // tiles * o >= 512 * c on (measured: batch 4 at 64 channels, batch 32 at 512 channels of ResNet-18).
+    int64_t factor = 512;
+    if (const char* e = std::getenv("KXC_HIP_WINOGRAD_MIN_WORK")) factor = std::atoll(e);
+    return Tiles(desc) * desc->o >= factor * desc->c ? 1 : 0;
 }
 
 const char* kxc_hip_conv2d_winograd_variant(const kxc_hip_conv2d_desc* desc) {

@@ -132,7 +132,7 @@ int32_t kxc_hip_conv2d_winograd_nchw_f32(const kxc_hip_conv2d_desc* desc, const 
                                          const float* bias, const float* residual, float* y, void* stream);
 const char* kxc_hip_conv2d_winograd_variant(const kxc_hip_conv2d_desc* desc);
 /* 1 when the shape qualifies and the launch is large enough for this path to beat kxc_hip_conv2d_nchw_f32
- * (measured on MI355X: at least one workgroup per compute unit), else 0. */
+ * (measured on MI355X: 2x2 output blocks * o >= 512 * c), else 0. */
 int32_t kxc_hip_conv2d_winograd_preferred(const kxc_hip_conv2d_desc* desc);
 
 /* nn_relu: ReluCompute (src/relay/op/nn/activation.cc:14-19). */

@@ -210,7 +210,8 @@ def test_conv_winograd_unsupported_shapes_are_refused(pkg):
     assert not pkg.conv2d_winograd_supported((1, 8, 8, 8), (16, 8, 1, 1), 1, 0)        # filter size
     assert not pkg.conv2d_winograd_supported((1, 6, 8, 8), (16, 6, 3, 3), 1, 1)        # channels not a multiple of 4
     assert not pkg.conv2d_winograd_supported((1, 8, 8, 8), (16, 8, 3, 3), 1, 1, 2)     # dilation
-    assert not pkg.conv2d_winograd_preferred((1, 64, 56, 56), (64, 64, 3, 3))          # batch 1: direct path is faster
+    assert not pkg.conv2d_winograd_preferred((1, 512, 7, 7), (512, 512, 3, 3))         # small launch, long reduction
+    assert pkg.conv2d_winograd_variant((1, 64, 56, 56), (64, 64, 3, 3)).endswith("_t1")  # small launches: smaller groups
     assert pkg.conv2d_winograd_preferred((64, 64, 56, 56), (64, 64, 3, 3))
     x = torch.zeros((1, 6, 8, 8), device="cuda"); u = torch.zeros((1024,), device="cuda")
     with pytest.raises(pkg.KxcHipError):

@@ -90,7 +90,8 @@ def test_resnet18_hip_plan_without_gpu():
     with tempfile.TemporaryDirectory() as d:
         run("resnet18", "hip", d, "1", "224")
         one = json.load(open(os.path.join(d, "plan.json")))
-    assert not any("winograd" in n["kernel_symbol"] for n in one["nodes"])     # batch 1: too small to pay
+    # batch 1: only the 56x56 layer has enough 2x2 blocks per input channel for Winograd to pay
+    assert sum("winograd" in n["kernel_symbol"] for n in one["nodes"]) == 4
 
 
 # ------------------------------------------------------------------ GPU
@@ -124,7 +125,7 @@ def test_resnet18_hip_winograd_matches_oracle(synth):
     from gpu_util import assert_close
     with tempfile.TemporaryDirectory() as d:
         x, consts = _write_resnet_inputs(synth, d, 3, 2, 224)
-        out = run("resnet18", "hip", d, "2", "224", env={"KXC_HIP_WINOGRAD_MIN_UNITS": "0"})
+        out = run("resnet18", "hip", d, "2", "224", env={"KXC_HIP_WINOGRAD_MIN_WORK": "0"})
         assert "execution plan replayed: 23 launches, identical output" in out
         plan = json.load(open(os.path.join(d, "plan.json")))
         assert sum(".winograd_f2k3" in n["kernel_symbol"] for n in plan["nodes"]) == 13
