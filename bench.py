@@ -59,6 +59,7 @@ def main():
     ap.add_argument("--steps", type=int, default=20)
     ap.add_argument("--warmup", type=int, default=5)
     ap.add_argument("--batch", type=int, default=64)
+    ap.add_argument("--eager", action="store_true", help="time only eager plan runs (no HIP graph replay)")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--no-layers", action="store_true", help="skip the per-layer / per-operator timings")
     ap.add_argument("--int8-only", action="store_true",
@@ -98,17 +99,30 @@ def main():
     packed = module.packed(tensors)
     stream = torch.cuda.current_stream().cuda_stream
 
-    def step():
-        module.run_packed(packed, stream)
+    def timed(run_step):
+        for _ in range(args.warmup):
+            run_step()
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        for _ in range(args.steps):
+            run_step()
+        torch.cuda.synchronize()
+        return (time.perf_counter() - t0) * 1e3 / args.steps
 
-    for _ in range(args.warmup):
-        step()
-    torch.cuda.synchronize()
-    t0 = time.perf_counter()
-    for _ in range(args.steps):
-        step()
-    torch.cuda.synchronize()
-    t1 = time.perf_counter()
+    # eager: 23 launches per step enqueued one by one; then the same plan replayed as one captured HIP graph per
+    # step (needs a stream other than the null stream; the first run on it is eager, the second is captured)
+    eager_ms = timed(lambda: module.run_packed(packed, stream))
+    graph_ms = None
+    if not args.eager:
+        side = torch.cuda.Stream()
+        with torch.cuda.stream(side):
+            module.enable_graph_replay(True)
+            for _ in range(3):
+                module.run_packed(packed, side.cuda_stream)
+            graph_ms = timed(lambda: module.run_packed(packed, side.cuda_stream))
+        torch.cuda.synchronize()
+        module.enable_graph_replay(False)
+    t1, t0 = (min(eager_ms, graph_ms) if graph_ms is not None else eager_ms) * args.steps * 1e-3, 0.0
     ms_per_step = (t1 - t0) * 1e3 / args.steps
     img_s = batch / (ms_per_step * 1e-3)
     flop_step = r18.flops_per_image() * batch
@@ -164,6 +178,7 @@ def main():
         "end_to_end_tflops": round(flop_step / (ms_per_step * 1e-3) / 1e12, 3),
         "end_to_end_frac_of_fp32_mfma_peak": round(flop_step / (ms_per_step * 1e-3) / 1e12 / PEAK_FP32_MFMA_TFLOPS, 4),
         "logits_finite": logits_ok,
+        "eager_ms_per_step": round(eager_ms, 4), "hip_graph_replay_ms_per_step": round(graph_ms, 4) if graph_ms is not None else None,
         "device": {"name": attrs.device_name.decode(), "arch": attrs.arch.decode(), "cus": int(attrs.multi_processor_count),
                    "clock_khz": int(attrs.max_clock_rate_khz)},
         "roofline": roofline,

@@ -35,6 +35,7 @@ namespace {
 
 typedef float floatx4 __attribute__((ext_vector_type(4)));
 typedef float floatx2 __attribute__((ext_vector_type(2)));
+typedef uint32_t uintx2 __attribute__((ext_vector_type(2)));
 typedef __attribute__((address_space(3))) void* lds_ptr_t;
 
 constexpr uint32_t kOob = 0x80000000u;     // beyond any buffer this kernel accepts (< 2 GiB): reads as 0
@@ -285,10 +286,14 @@ wino_kernel(const WinoArgs a) {
     }
     asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
 
-    // ---- epilogue: accumulator register g of block kb holds output channel 16*kb + 4*(lane/16) + g, tile lane%16
+    // ---- epilogue: accumulator register g of block kb holds output channel 16*kb + 4*(lane/16) + g, tile lane%16.
+    // Everything goes through buffer descriptors: an offset beyond the buffer makes a load return 0 and drops a
+    // store, so absent channels, tiles past the end and the odd last row / column need no branches, and all loads
+    // (bias, residual) are issued before the first store -- a wait for a load would otherwise also wait for every
+    // store issued before it.
     const int tile = t0 + wave_t * 16 + (lane & 15);
-    if (tile >= a.NT) return;
-    const int n = fast_div(tile, a.div_ti), rem = tile - n * a.TI;
+    const int tile_c = min(tile, a.NT - 1);
+    const int n = fast_div(tile_c, a.div_ti), rem = tile_c - n * a.TI;
     const int ty = fast_div(rem, a.div_tw), tx = rem - ty * a.TW;
     const int oh = 2 * ty, ow = 2 * tx;
     const bool row1 = oh + 1 < a.OH, col1 = ow + 1 < a.OW;
@@ -296,12 +301,52 @@ wino_kernel(const WinoArgs a) {
     const bool has_bias = (a.flags & KXC_HIP_CONV_BIAS) != 0;
     const bool has_res = (a.flags & KXC_HIP_CONV_RESIDUAL) != 0;
     const bool do_relu = (a.flags & KXC_HIP_CONV_RELU) != 0;
+    const uint32_t y_bytes = static_cast<uint32_t>(a.N) * static_cast<uint32_t>(a.O) * static_cast<uint32_t>(a.OHW) * 4u;
+    const __amdgpu_buffer_rsrc_t yr = make_rsrc(a.y, y_bytes);
+    const __amdgpu_buffer_rsrc_t rr = make_rsrc(has_res ? a.res : a.y, has_res ? y_bytes : 0u);
+    const __amdgpu_buffer_rsrc_t br = make_rsrc(has_bias ? a.bias : a.y, has_bias ? static_cast<uint32_t>(a.O) * 4u : 0u);
+    const uint32_t rowb = static_cast<uint32_t>(a.OW) * 4u;
+    const uint32_t rowmask = row1 ? 0u : kOob, colmask = col1 ? 0u : kOob;   // OR-ed into an offset: beyond the buffer
+
+    uint32_t off00[2][4];
+    float bv[2][4];
+    float q[2][4][4];
+#pragma unroll
+    for (int kb = 0; kb < 2; ++kb)
+#pragma unroll
+        for (int g = 0; g < 4; ++g) {
+            const int o = (kg * WK + wave_k) * 32 + kb * 16 + 4 * (lane >> 4) + g;
+            const bool ok = tile < a.NT && o < a.O;
+            off00[kb][g] = ok ? static_cast<uint32_t>(((n * a.O + o) * a.OH + oh) * a.OW + ow) * 4u : kOob;
+            bv[kb][g] = load_f32(br, ok ? static_cast<uint32_t>(o) * 4u : kOob, 0);
+        }
+    if (has_res && vec2) {
+#pragma unroll
+        for (int kb = 0; kb < 2; ++kb)
+#pragma unroll
+            for (int g = 0; g < 4; ++g) {
+                const uint32_t o0 = off00[kb][g], o1 = (o0 + rowb) | rowmask;
+                // (two 4-byte loads per row: the 8-byte buffer-load builtin of this toolchain fetches only 4 bytes)
+                q[kb][g][0] = load_f32(rr, o0, 0); q[kb][g][1] = load_f32(rr, o0 + 4u, 0);
+                q[kb][g][2] = load_f32(rr, o1, 0); q[kb][g][3] = load_f32(rr, o1 + 4u, 0);
+            }
+    } else if (has_res) {
+#pragma unroll
+        for (int kb = 0; kb < 2; ++kb)
+#pragma unroll
+            for (int g = 0; g < 4; ++g) {
+                const uint32_t o0 = off00[kb][g], o1 = (o0 + rowb) | rowmask;
+                q[kb][g][0] = load_f32(rr, o0, 0);
+                q[kb][g][1] = load_f32(rr, (o0 + 4u) | colmask, 0);
+                q[kb][g][2] = load_f32(rr, o1, 0);
+                q[kb][g][3] = load_f32(rr, (o1 + 4u) | colmask, 0);
+            }
+    }
+    float yv[2][4][4];
 #pragma unroll
     for (int kb = 0; kb < 2; ++kb) {
 #pragma unroll
         for (int g = 0; g < 4; ++g) {
-            const int o = (kg * WK + wave_k) * 32 + kb * 16 + 4 * (lane >> 4) + g;
-            if (o >= a.O) continue;
             // A^T M A with A^T = [1 1 1 0; 0 1 -1 -1]
             float r0[4], r1[4];
 #pragma unroll
@@ -312,37 +357,39 @@ wino_kernel(const WinoArgs a) {
             }
             float y00 = (r0[0] + r0[1]) + r0[2], y01 = (r0[1] - r0[2]) - r0[3];
             float y10 = (r1[0] + r1[1]) + r1[2], y11 = (r1[1] - r1[2]) - r1[3];
-            const int off = ((n * a.O + o) * a.OH + oh) * a.OW + ow;
             if (has_bias) {
-                const float bval = a.bias[o];
+                const float bval = bv[kb][g];
                 y00 = __fadd_rn(y00, bval); y01 = __fadd_rn(y01, bval); y10 = __fadd_rn(y10, bval); y11 = __fadd_rn(y11, bval);
             }
-            if (vec2) {
-                if (has_res) {
-                    const floatx2 q0 = *reinterpret_cast<const floatx2*>(a.res + off);
-                    y00 = __fadd_rn(y00, q0[0]); y01 = __fadd_rn(y01, q0[1]);
-                    if (row1) {
-                        const floatx2 q1 = *reinterpret_cast<const floatx2*>(a.res + off + a.OW);
-                        y10 = __fadd_rn(y10, q1[0]); y11 = __fadd_rn(y11, q1[1]);
-                    }
-                }
-                if (do_relu) { y00 = relu_sel(y00); y01 = relu_sel(y01); y10 = relu_sel(y10); y11 = relu_sel(y11); }
-                *reinterpret_cast<floatx2*>(a.y + off) = floatx2{y00, y01};
-                if (row1) *reinterpret_cast<floatx2*>(a.y + off + a.OW) = floatx2{y10, y11};
-            } else {
-                if (has_res) {
-                    y00 = __fadd_rn(y00, a.res[off]);
-                    if (col1) y01 = __fadd_rn(y01, a.res[off + 1]);
-                    if (row1) y10 = __fadd_rn(y10, a.res[off + a.OW]);
-                    if (row1 && col1) y11 = __fadd_rn(y11, a.res[off + a.OW + 1]);
-                }
-                if (do_relu) { y00 = relu_sel(y00); y01 = relu_sel(y01); y10 = relu_sel(y10); y11 = relu_sel(y11); }
-                a.y[off] = y00;
-                if (col1) a.y[off + 1] = y01;
-                if (row1) a.y[off + a.OW] = y10;
-                if (row1 && col1) a.y[off + a.OW + 1] = y11;
+            if (has_res) {
+                y00 = __fadd_rn(y00, q[kb][g][0]); y01 = __fadd_rn(y01, q[kb][g][1]);
+                y10 = __fadd_rn(y10, q[kb][g][2]); y11 = __fadd_rn(y11, q[kb][g][3]);
             }
+            if (do_relu) { y00 = relu_sel(y00); y01 = relu_sel(y01); y10 = relu_sel(y10); y11 = relu_sel(y11); }
+            yv[kb][g][0] = y00; yv[kb][g][1] = y01; yv[kb][g][2] = y10; yv[kb][g][3] = y11;
         }
+    }
+    auto bits = [](float v) { return __builtin_bit_cast(uint32_t, v); };
+    if (vec2) {
+#pragma unroll
+        for (int kb = 0; kb < 2; ++kb)
+#pragma unroll
+            for (int g = 0; g < 4; ++g) {
+                const uint32_t o0 = off00[kb][g], o1 = (o0 + rowb) | rowmask;
+                __builtin_amdgcn_raw_buffer_store_b64(uintx2{bits(yv[kb][g][0]), bits(yv[kb][g][1])}, yr, o0, 0, 0);
+                __builtin_amdgcn_raw_buffer_store_b64(uintx2{bits(yv[kb][g][2]), bits(yv[kb][g][3])}, yr, o1, 0, 0);
+            }
+    } else {
+#pragma unroll
+        for (int kb = 0; kb < 2; ++kb)
+#pragma unroll
+            for (int g = 0; g < 4; ++g) {
+                const uint32_t o0 = off00[kb][g], o1 = (o0 + rowb) | rowmask;
+                __builtin_amdgcn_raw_buffer_store_b32(bits(yv[kb][g][0]), yr, o0, 0, 0);
+                __builtin_amdgcn_raw_buffer_store_b32(bits(yv[kb][g][1]), yr, (o0 + 4u) | colmask, 0, 0);
+                __builtin_amdgcn_raw_buffer_store_b32(bits(yv[kb][g][2]), yr, o1, 0, 0);
+                __builtin_amdgcn_raw_buffer_store_b32(bits(yv[kb][g][3]), yr, (o1 + 4u) | colmask, 0, 0);
+            }
     }
 }
 
@@ -371,7 +418,7 @@ bool Supported(const kxc_hip_conv2d_desc* d) {
     const int64_t y_elems = static_cast<int64_t>(d->n) * d->o * oh * ow;
     const int64_t u_bytes = CeilDiv(d->o, 32) * 32 * static_cast<int64_t>(d->c) * 64;
     const int64_t tiles = static_cast<int64_t>(d->n) * CeilDiv(oh, 2) * CeilDiv(ow, 2);
-    return x_bytes < (1LL << 31) && y_elems < (1LL << 31) && u_bytes < (1LL << 31) && tiles < (1LL << 30);
+    return x_bytes < (1LL << 31) && y_elems * 4 < (1LL << 31) && u_bytes < (1LL << 31) && tiles < (1LL << 30);
 }
 
 int64_t Tiles(const kxc_hip_conv2d_desc* d) {
