@@ -371,28 +371,64 @@ conv_mfma_kernel(const ConvArgs a) {
         }
         return;
     }
+    // Bias, residual and output go through buffer descriptors: an offset beyond the buffer makes a load return 0
+    // and drops a store, so absent channels and pixels past the end need no branches, and every load is issued
+    // before the first store (a wait for a load also waits for all stores issued before it: with loads and stores
+    // interleaved each of the 16 rows would cost a full memory round trip).
     const bool has_bias = (a.flags & KXC_HIP_CONV_BIAS) != 0;
     const bool has_res = (a.flags & KXC_HIP_CONV_RESIDUAL) != 0;
     const bool do_relu = (a.flags & KXC_HIP_CONV_RELU) != 0;
+    const uint32_t y_bytes = static_cast<uint32_t>(a.out_elems) * 4u;
+    const __amdgpu_buffer_rsrc_t yr = make_rsrc(a.y, y_bytes);
+    const __amdgpu_buffer_rsrc_t rr = make_rsrc(has_res ? a.res : a.y, has_res ? y_bytes : 0u);
+    const __amdgpu_buffer_rsrc_t br = make_rsrc(has_bias ? a.bias : a.y, has_bias ? static_cast<uint32_t>(a.O) * 4u : 0u);
+    const uint32_t plane = static_cast<uint32_t>(a.OHW) * 4u;
+    uint32_t yb[RP];
 #pragma unroll
-    for (int i = 0; i < RO; ++i) {
+    for (int j = 0; j < RP; ++j) yb[j] = ybase[j] >= 0 ? static_cast<uint32_t>(ybase[j]) * 4u : kOobOffset;
+    auto channel = [&](int i, int g) { return o0 + (wave_o * RO + i) * 32 + 8 * (g / 4) + 4 * half + (g % 4); };
+    auto out_off = [&](int i, int g, int j) {
+        const int o = channel(i, g);
+        return o < a.O ? yb[j] + static_cast<uint32_t>(o) * plane : kOobOffset;
+    };
+    float bv[RO][16];
+#pragma unroll
+    for (int i = 0; i < RO; ++i)
 #pragma unroll
         for (int g = 0; g < 16; ++g) {
-            const int o = o0 + (wave_o * RO + i) * 32 + 8 * (g / 4) + 4 * half + (g % 4);
-            if (o >= a.O) continue;
-            const float bval = has_bias ? a.bias[o] : 0.0f;
+            const int o = channel(i, g);
+            bv[i][g] = __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(br, o < a.O ? static_cast<uint32_t>(o) * 4u : kOobOffset, 0, 0));
+        }
+    // rows (accumulator registers) per batch of residual loads: the whole block when one block per wave, fewer
+    // for register-blocked tiles so that the staged residual never needs more than 16 registers
+    constexpr int GC = 16 / (RO * RP) < 4 ? 4 : 16 / (RO * RP);
 #pragma unroll
-            for (int j = 0; j < RP; ++j) {
-                if (ybase[j] < 0) continue;
-                const int off = ybase[j] + o * a.OHW;
-                float v = acc[i][j][g];
-                if (has_bias) v = __fadd_rn(v, bval);
-                if (has_res) v = __fadd_rn(v, a.res[off]);
-                if (do_relu) v = relu_sel(v);
+    for (int gc = 0; gc < 16; gc += GC) {
+        float q[RO][RP][GC];
+        if (has_res) {
+#pragma unroll
+            for (int i = 0; i < RO; ++i)
+#pragma unroll
+                for (int g = 0; g < GC; ++g)
+#pragma unroll
+                    for (int j = 0; j < RP; ++j)
+                        q[i][j][g] = __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(rr, out_off(i, gc + g, j), 0, 0));
+        }
+#pragma unroll
+        for (int i = 0; i < RO; ++i) {
+#pragma unroll
+            for (int g = 0; g < GC; ++g) {
+#pragma unroll
+                for (int j = 0; j < RP; ++j) {
+                    float v = acc[i][j][gc + g];
+                    if (has_bias) v = __fadd_rn(v, bv[i][gc + g]);
+                    if (has_res) v = __fadd_rn(v, q[i][j][g]);
+                    if (do_relu) v = relu_sel(v);
 #ifdef KXC_DBG_NO_STORE
-                if (v == 123456.789f)
+                    if (v == 123456.789f)
 #endif
-                a.y[off] = v;
+                    __builtin_amdgcn_raw_buffer_store_b32(__builtin_bit_cast(uint32_t, v), yr, out_off(i, gc + g, j), 0, 0);
+                }
             }
         }
     }
@@ -569,7 +605,7 @@ void Select(const ConvArgs& a, int kh, int kw, Choice* choice) {
     const int64_t y_elems = static_cast<int64_t>(a.N) * a.O * a.OHW;
     const int64_t w_bytes = static_cast<int64_t>(a.O) * a.C * kh * kw * 4;
     const int64_t q_rows = static_cast<int64_t>(a.N + 1) * a.Hp + kh * a.dh;
-    if (x_bytes >= (1LL << 31) || y_elems >= (1LL << 31) || w_bytes >= (1LL << 31) || q_rows * a.Wp >= (1LL << 31)) return;
+    if (x_bytes >= (1LL << 31) || y_elems * 4 >= (1LL << 31) || w_bytes >= (1LL << 31) || q_rows * a.Wp >= (1LL << 31)) return;
     const char* forced = std::getenv("KXC_HIP_CONV_VARIANT");
     // Shape rules on top of the table order (measured, see the table's comment).
     const char* preferred = nullptr;

@@ -116,7 +116,7 @@ __global__ void __launch_bounds__(256) wino_weight_kernel(const float* __restric
 // One step = 4 input channels.  LDS per buffer: U [WK][c4][o/16: 2][f/4: 4][o%16][f%4] and
 // V [c4][WT][f/4: 4][tile%16][f%4]; two of each.
 // ------------------------------------------------------------------------------------------
-template <int WK, int WT>
+template <int WK, int WT, bool SKEW>
 __global__ void __launch_bounds__(64 * WK * WT) __attribute__((amdgpu_waves_per_eu(2)))
 wino_kernel(const WinoArgs a) {
     constexpr int NTH = 64 * WK * WT;
@@ -231,6 +231,72 @@ wino_kernel(const WinoArgs a) {
         }
     };
 
+    const int last = a.csteps - 1;
+    if constexpr (SKEW) {
+        // Three LDS tiles (weights + transformed input of one step each) and the barrier in the MIDDLE of a step:
+        // between two barriers a wave multiplies the second half of step p (groups 2, 3) and the first half of
+        // step p+1 (groups 0, 1), while tile p+2 is being filled.  The operands of the first group after a barrier
+        // come from a tile that was already visible before it, so they are fetched ahead of the barrier and no
+        // wave waits for LDS right after one.
+        constexpr int BUF = U_FLOATS + V_FLOATS;
+        auto ubuf = [&](int i) { return lds + i * BUF; };
+        auto vbuf = [&](int i) { return lds + i * BUF + U_FLOATS; };
+        issue_u(0, ubuf(0));
+        load_raw(0);
+        transform(vbuf(0));
+        load_raw(min(1, last));
+        __builtin_amdgcn_sched_barrier(0);
+        __syncthreads();                                    // tile 0 visible
+        issue_u(min(1, last), ubuf(1));
+        fetch(ubuf(0), vbuf(0), 0, 0);
+        fetch(ubuf(0), vbuf(0), 1, 1);
+        __builtin_amdgcn_sched_barrier(0);
+        mm(0, 0);
+        transform(vbuf(1));
+        __builtin_amdgcn_sched_barrier(0);
+        fetch(ubuf(0), vbuf(0), 2, 0);
+        mm(1, 1);
+        load_raw(min(2, last));
+        __builtin_amdgcn_sched_barrier(0);
+        __syncthreads();                                    // tile 1 visible
+        int i0 = 0, i1 = 1, i2 = 2;                         // buffers of tiles p, p+1, p+2
+        for (int p = 0; p < last; ++p) {
+            const float* const u0 = ubuf(i0); const float* const v0 = vbuf(i0);
+            const float* const u1 = ubuf(i1); const float* const v1 = vbuf(i1);
+            issue_u(min(p + 2, last), ubuf(i2));
+            fetch(u0, v0, 3, 1);
+            __builtin_amdgcn_sched_barrier(0);
+            mm(2, 0);
+            __builtin_amdgcn_sched_barrier(0);
+            fetch(u1, v1, 0, 0);
+            mm(3, 1);
+            __builtin_amdgcn_sched_barrier(0);
+            fetch(u1, v1, 1, 1);
+            mm(0, 0);
+            transform(vbuf(i2));                            // raw input of step p+2, requested one window ago
+#pragma unroll
+            for (int q = 0; q < 8; ++q) {
+                __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+                __builtin_amdgcn_sched_group_barrier(0x002, 6, 0);
+            }
+            __builtin_amdgcn_sched_barrier(0);
+            fetch(u1, v1, 2, 0);
+            mm(1, 1);
+            load_raw(min(p + 3, last));
+#pragma unroll
+            for (int q = 0; q < 8; ++q) {
+                __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+                __builtin_amdgcn_sched_group_barrier(0x020, 2, 0);
+            }
+            __builtin_amdgcn_sched_barrier(0);
+            __syncthreads();                                // tile p+2 visible
+            const int t = i0; i0 = i1; i1 = i2; i2 = t;
+        }
+        // second half of the last step
+        fetch(ubuf(i0), vbuf(i0), 3, 1);
+        mm(2, 0);
+        mm(3, 1);
+    } else {
     // LDS: two weight tiles and two transformed-input tiles.  The compiler orders every barrier after the
     // LDS-writing loads issued before it, so a weight tile is requested at the top of the step before the one that
     // uses it and has that whole step to arrive; the raw input (registers) is requested two steps ahead.
@@ -238,7 +304,6 @@ wino_kernel(const WinoArgs a) {
     float* const ub1 = lds + U_FLOATS;
     float* const vb0 = lds + 2 * U_FLOATS;
     float* const vb1 = vb0 + V_FLOATS;
-    const int last = a.csteps - 1;
 
     // ---- prologue: weight tile and transformed input of step 0; raw input of step 1 in flight
     issue_u(0, ub0);
@@ -283,6 +348,7 @@ wino_kernel(const WinoArgs a) {
         mm(3, 1);
         __builtin_amdgcn_sched_barrier(0);
         __syncthreads();
+    }
     }
     asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
 
@@ -395,17 +461,20 @@ wino_kernel(const WinoArgs a) {
 
 struct WinoVariant {
     const char* name;
-    int wk, wt;
+    int wk, wt, bufs;
     void (*kernel)(const WinoArgs);
 };
-#define KXC_WINO(WK, WT) {"winograd_f2k3_o" #WK "_t" #WT, WK, WT, wino_kernel<WK, WT>}
-// name = winograd_f2k3_o<waves along output channels (32 each)>_t<waves along tiles (16 each)>
+#define KXC_WINO(WK, WT) {"winograd_f2k3_o" #WK "_t" #WT, WK, WT, 2, wino_kernel<WK, WT, false>}
+#define KXC_WINO_S3(WK, WT) {"winograd_f2k3_o" #WK "_t" #WT "_s3", WK, WT, 3, wino_kernel<WK, WT, true>}
+// name = winograd_f2k3_o<waves along output channels (32 each)>_t<waves along tiles (16 each)>[_s3: three LDS tiles]
 const WinoVariant kWino[] = {
     KXC_WINO(2, 2),   // 64 channels x 32 tiles, 4 waves, 48 KiB of LDS (default)
     KXC_WINO(2, 4),   // 64 x 64, 8 waves
     KXC_WINO(1, 4),   // 32 x 64, 4 waves
     KXC_WINO(2, 1),   // 64 x 16, 2 waves
     KXC_WINO(1, 2),   // 32 x 32, 2 waves
+    KXC_WINO_S3(2, 2),   // three LDS tiles, barrier in the middle of a step
+    KXC_WINO_S3(2, 1),
 };
 constexpr int kNumWino = sizeof(kWino) / sizeof(kWino[0]);
 
@@ -508,7 +577,7 @@ int32_t kxc_hip_conv2d_winograd_nchw_f32(const kxc_hip_conv2d_desc* desc, const 
     if (const char* e = std::getenv("KXC_HIP_WINOGRAD_KFAST")) a.k_fastest = std::atoi(e);
     a.div_ti = MakeFastDiv(a.TI); a.div_tw = MakeFastDiv(a.TW);
     a.div_kgroups = MakeFastDiv(a.k_groups); a.div_tgroups = MakeFastDiv(a.t_groups);
-    const size_t lds_bytes = 2 * static_cast<size_t>(2048 * v->wk + 1024 * v->wt) * sizeof(float);
+    const size_t lds_bytes = v->bufs * static_cast<size_t>(2048 * v->wk + 1024 * v->wt) * sizeof(float);
     if (lds_bytes > 64 * 1024) {
         KXC_HIP_CALL(hipFuncSetAttribute(reinterpret_cast<const void*>(v->kernel), hipFuncAttributeMaxDynamicSharedMemorySize,
                                          static_cast<int>(lds_bytes)),
