@@ -90,30 +90,56 @@ __device__ __forceinline__ void epilogue_c16(const intx16 (&acc)[RO], const QArg
     const bool has_bias = (a.flags & KXC_HIP_CONV_BIAS) != 0;
     const bool has_res = (a.flags & KXC_HIP_CONV_RESIDUAL) != 0;
     const bool do_relu = (a.flags & KXC_HIP_CONV_RELU) != 0;
+    // All loads (residual word, 4 multipliers, 4 biases per group of 4 channels) are issued before the first store:
+    // a wait for a load also waits for every store issued before it, so interleaving them would cost one memory
+    // round trip per group.  Absent channel groups load group 0 and store nothing.
+    auto group = [&](int i, int j) { return (ob0 + i) * 32 + 8 * j + 4 * half; };       // first of 4 consecutive channels
+    auto offset = [&](int o) { return (static_cast<int64_t>(ypix) + static_cast<int64_t>(o >> 4) * a.OHW) * 16 + (o & 15); };
+    uint32_t resw[RO][4];
+    float4 mv[RO][4];
+    int4 bv[RO][4];
 #pragma unroll
-    for (int i = 0; i < RO; ++i) {
-        const int obase = (ob0 + i) * 32;
-        if (obase >= a.O) continue;
+    for (int i = 0; i < RO; ++i)
 #pragma unroll
         for (int j = 0; j < 4; ++j) {
-            const int o = obase + 8 * j + 4 * half;                 // first of 4 consecutive channels
-            if (o >= a.O) continue;
-            const int64_t off = (static_cast<int64_t>(ypix) + static_cast<int64_t>(o >> 4) * a.OHW) * 16 + (o & 15);
-            uint32_t resw = 0;
-            if (has_res) resw = *reinterpret_cast<const uint32_t*>(a.res + off);
-            const float4 mv = *reinterpret_cast<const float4*>(a.mult + o);
-            int4 bv = make_int4(0, 0, 0, 0);
-            if (has_bias) bv = *reinterpret_cast<const int4*>(a.bias + o);
-            const float ms[4] = {mv.x, mv.y, mv.z, mv.w};
-            const int bs[4] = {bv.x, bv.y, bv.z, bv.w};
+            const int o = group(i, j), oc = o < a.O ? o : 0;
+            mv[i][j] = *reinterpret_cast<const float4*>(a.mult + oc);
+            bv[i][j] = make_int4(0, 0, 0, 0);
+            resw[i][j] = 0;
+        }
+    if (has_bias) {
+#pragma unroll
+        for (int i = 0; i < RO; ++i)
+#pragma unroll
+            for (int j = 0; j < 4; ++j) {
+                const int o = group(i, j);
+                bv[i][j] = *reinterpret_cast<const int4*>(a.bias + (o < a.O ? o : 0));
+            }
+    }
+    if (has_res) {
+#pragma unroll
+        for (int i = 0; i < RO; ++i)
+#pragma unroll
+            for (int j = 0; j < 4; ++j) {
+                const int o = group(i, j);
+                resw[i][j] = *reinterpret_cast<const uint32_t*>(a.res + offset(o < a.O ? o : 0));
+            }
+    }
+#pragma unroll
+    for (int i = 0; i < RO; ++i) {
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+            const int o = group(i, j);
+            const float ms[4] = {mv[i][j].x, mv[i][j].y, mv[i][j].z, mv[i][j].w};
+            const int bs[4] = {bv[i][j].x, bv[i][j].y, bv[i][j].z, bv[i][j].w};
             uint32_t outw = 0;
 #pragma unroll
             for (int e = 0; e < 4; ++e) {
-                const int32_t rq = static_cast<int32_t>(static_cast<int8_t>((resw >> (8 * e)) & 0xff));
+                const int32_t rq = static_cast<int32_t>(static_cast<int8_t>((resw[i][j] >> (8 * e)) & 0xff));
                 const int32_t q = requant_i32(acc[i][4 * j + e] + bs[e], ms[e], has_res, rq, a.res_mult, do_relu);
                 outw |= (static_cast<uint32_t>(q) & 0xffu) << (8 * e);
             }
-            *reinterpret_cast<uint32_t*>(a.y + off) = outw;
+            if (o < a.O) *reinterpret_cast<uint32_t*>(a.y + offset(o)) = outw;
         }
     }
 }

@@ -34,6 +34,7 @@ struct CompileConfigNode {
     bool hip_concurrent_branches{true};   // run a block's downsample convolution beside its first 3x3 convolution
     bool hip_winograd{true};              // 3x3 stride-1 convolutions with constant weights as Winograd F(2x2,3x3) where faster
     bool sync_after_run{true};
+    int background_threads{0};         // adaptive runtime: compile workers (0 = half the hardware threads)
 };
 class CompileConfig : public Ref<CompileConfigNode> {
 public:

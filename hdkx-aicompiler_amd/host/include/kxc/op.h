@@ -159,6 +159,19 @@ KXC_ATTRS_REF(ReduceMeanAttrs)
     static ReduceMeanAttrs Create(std::vector<int64_t> axes, int keepdims);
 };
 
+// softmax (src/relay/op/nn/softmax.cc): axis may be negative
+struct SoftmaxAttrsNode : AttrsNode { int64_t axis = -1; };
+KXC_ATTRS_REF(SoftmaxAttrs)
+    static SoftmaxAttrs Create(int64_t axis = -1);
+};
+
+// cast (src/relay/op/tensor/transform.cc:84-104): `to` is a dtype code -- 0 float32, 1 int32, 2 int64, 3 float64,
+// 4 bool, 5 int8, 6 uint8
+struct CastAttrsNode : AttrsNode { int to = 0; };
+KXC_ATTRS_REF(CastAttrs)
+    static CastAttrs Create(int to);
+};
+
 #define KXC_SIMPLE_ATTRS(TypeName)                \
     struct TypeName##Node : AttrsNode {};         \
     KXC_ATTRS_REF(TypeName)                       \
@@ -181,6 +194,10 @@ Type FlattenInferType(const Attrs& attrs, const Array<Type>& inputs);
 Type ReshapeInferType(const Attrs& attrs, const Array<Type>& inputs);
 Type TransposeInferType(const Attrs& attrs, const Array<Type>& inputs);
 Type ReduceMeanInferType(const Attrs& attrs, const Array<Type>& inputs);
+Type SoftmaxInferType(const Attrs& attrs, const Array<Type>& inputs);
+Type CastInferType(const Attrs& attrs, const Array<Type>& inputs);
+// dtype string of a cast code; throws "cast has unsupported dtype code: N"
+std::string CastDTypeFromCode(int code);
 
 // InferTypePass (src/relay/transforms/infer_type.cc:41-222): fills checked_type_ of every node.
 Function InferTypePass(const Function& f);

@@ -45,6 +45,11 @@ Tensor reshape(const Tensor& x, std::vector<int64_t> new_shape, std::string name
 Tensor transpose(const Tensor& x, std::vector<int> axes, std::string name);
 // mean over trailing/selected axes: sum then division by the element count
 Tensor reduce_mean(const Tensor& x, std::vector<int> axes, bool keepdims, std::string name);
+// exp(x) / sum over `axis` of exp(x), as three stages named <name>_exp, <name>_sum (axis kept with extent 1) and
+// <name> (src/relay/op/nn/softmax.cc: no max subtraction, like the reference)
+Tensor softmax(const Tensor& x, int axis, std::string name);
+// Call(dtype, "cast", {x}) per element (include/te/topi/elemwise.h:113-122): C conversion rules
+Tensor cast(const Tensor& x, tir::DataType dtype, std::string name);
 
 }  // namespace topi
 }  // namespace te

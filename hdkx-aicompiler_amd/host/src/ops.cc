@@ -355,6 +355,34 @@ void EnsureBuiltinOpsRegistered() {
                 for (auto v : a->axes) axes.push_back(static_cast<int>(v));
                 return te::topi::reduce_mean(in[0], axes, a->keepdims != 0, "T_reduce_mean");
             });
+        OpRegEntry::Register("softmax")
+            .describe("Computes softmax along one tensor axis.")
+            .set_num_inputs(1)
+            .add_argument("data", "Tensor", "The input tensor.")
+            .set_attr<std::string>("TAttrs", "SoftmaxAttrs")
+            .set_attr<FInferType>("FInferType", SoftmaxInferType)
+            .set_attr<FRelayToTE>("FRelayToTE", [](const Attrs& attrs, const Array<te::Tensor>& in, const Type&) {
+                if (in.size() != 1) throw std::runtime_error("softmax expects exactly 1 input(s)");
+                if (in[0]->dtype.code != 2) throw std::runtime_error("softmax lowering requires floating-point input");
+                const auto* a = attrs.As<SoftmaxAttrsNode>();
+                const int nd = static_cast<int>(in[0]->shape.size());
+                int64_t axis = a ? a->axis : -1;
+                if (axis < 0) axis += nd;
+                if (axis < 0 || axis >= nd) throw std::runtime_error("softmax axis out of range");
+                return te::topi::softmax(in[0], static_cast<int>(axis), "T_softmax");
+            });
+        OpRegEntry::Register("cast")
+            .describe("Converts the elements to another dtype.")
+            .set_num_inputs(1)
+            .add_argument("data", "Tensor", "The input tensor.")
+            .set_attr<std::string>("TAttrs", "CastAttrs")
+            .set_attr<FInferType>("FInferType", CastInferType)
+            .set_attr<FRelayToTE>("FRelayToTE", [](const Attrs& attrs, const Array<te::Tensor>& in, const Type&) {
+                if (in.size() != 1) throw std::runtime_error("cast expects exactly 1 input(s)");
+                const auto* a = attrs.As<CastAttrsNode>();
+                if (!a) throw std::runtime_error("cast expects CastAttrs");
+                return te::topi::cast(in[0], tir::DTypeFromString(CastDTypeFromCode(a->to)), "T_cast");
+            });
         return true;
     }();
     (void)done;

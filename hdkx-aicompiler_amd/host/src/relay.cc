@@ -125,6 +125,22 @@ ReduceMeanAttrs ReduceMeanAttrs::Create(std::vector<int64_t> axes, int keepdims)
     return ReduceMeanAttrs(n);
 }
 
+SoftmaxAttrs SoftmaxAttrs::Create(int64_t axis) {
+    auto n = std::make_shared<SoftmaxAttrsNode>();
+    n->axis = axis;
+    return SoftmaxAttrs(n);
+}
+CastAttrs CastAttrs::Create(int to) {
+    auto n = std::make_shared<CastAttrsNode>();
+    n->to = to;
+    return CastAttrs(n);
+}
+std::string CastDTypeFromCode(int code) {
+    static const char* const names[] = {"float32", "int32", "int64", "float64", "bool", "int8", "uint8"};
+    if (code < 0 || code > 6) throw std::runtime_error("cast has unsupported dtype code: " + std::to_string(code));
+    return names[code];
+}
+
 // ------------------------------------------------------------------ shape rules
 namespace {
 const TensorTypeNode* RequireTensor(const std::string& op, const Type& t, const char* what) {
@@ -345,6 +361,24 @@ Type ReduceMeanInferType(const Attrs& attrs, const Array<Type>& in) {
         else if (a->keepdims) shape.push_back(1);
     }
     return TensorType(shape, x->dtype);
+}
+
+Type SoftmaxInferType(const Attrs& attrs, const Array<Type>& in) {
+    RequireArity("softmax", in, 1);
+    const auto* x = RequireTensor("softmax", in[0], "data");
+    const auto* a = attrs.As<SoftmaxAttrsNode>();
+    const int nd = static_cast<int>(x->shape.size());
+    int64_t axis = a ? a->axis : -1;
+    if (axis < 0) axis += nd;
+    if (axis < 0 || axis >= nd) throw std::runtime_error("softmax axis out of range");
+    return TensorType(x->shape, x->dtype);
+}
+
+Type CastInferType(const Attrs& attrs, const Array<Type>& in) {
+    RequireArity("cast", in, 1);
+    const auto* x = RequireTensor("cast", in[0], "data");
+    const auto* a = attrs.As<CastAttrsNode>();
+    return TensorType(x->shape, a ? CastDTypeFromCode(a->to) : x->dtype);
 }
 
 // ------------------------------------------------------------------ InferType

@@ -275,6 +275,29 @@ Tensor reduce_mean(const Tensor& x, std::vector<int> axes, bool keepdims, std::s
                    kInjective);
 }
 
+Tensor softmax(const Tensor& x, int axis, std::string name) {
+    std::vector<int64_t> in_shape = x.const_shape();
+    const int nd = static_cast<int>(in_shape.size());
+    Tensor e = unary_call(x, "exp", name + "_exp");
+    IterVar r = reduce_axis(0, I64(in_shape[axis]), "k");
+    std::vector<PrimExpr> sshape;
+    for (int d = 0; d < nd; ++d) sshape.push_back(I64(d == axis ? 1 : in_shape[d]));
+    Tensor s = compute(sshape, [&](const Array<Var>& i) {
+        std::vector<PrimExpr> idx;
+        for (int d = 0; d < nd; ++d) idx.push_back(d == axis ? PrimExpr(r.var) : PrimExpr(i[d]));
+        return sum(e(idx), {r});
+    }, name + "_sum", kInjective);
+    return compute(x->shape, [&](const Array<Var>& i) {
+        std::vector<PrimExpr> den;
+        for (int d = 0; d < nd; ++d) den.push_back(d == axis ? I64(0) : PrimExpr(i[d]));
+        return e(i) / s(den);
+    }, name, kInjective);
+}
+
+Tensor cast(const Tensor& x, tir::DataType dtype, std::string name) {
+    return compute(x->shape, [&](const Array<Var>& i) { return tir::Call(dtype, "cast", {x(i)}); }, name, kElementWise);
+}
+
 }  // namespace topi
 }  // namespace te
 }  // namespace kxc

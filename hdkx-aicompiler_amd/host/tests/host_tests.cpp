@@ -16,11 +16,16 @@
 #include <fstream>
 #include <functional>
 #include <iostream>
+#include <condition_variable>
+#include <mutex>
+#include <thread>
+#include <atomic>
 
 #include "kxc/compiler.h"
 #include "kxc/models.h"
 #include "kxc/onnx_importer.h"
 #include "kxc/profiling.h"
+#include "kxc/runtime_session.h"
 #include "kxc/topi.h"
 
 namespace {
@@ -202,6 +207,51 @@ void TestReduceMean() {
     ExpectNear(out, {2.0f, 5.0f});
 }
 
+// softmax over the last axis against the formula (test/op_numeric_llvm_test.cpp:271-293)
+void TestSoftmax() {
+    kxc::Var data("data", kxc::TensorType({2, 3}, "float32"));
+    kxc::Function func({data}, kxc::Call(Op::Get("softmax"), {data}, kxc::relay::SoftmaxAttrs::Create(1)));
+    std::vector<float> d = {1, 2, 3, 1, 3, 5}, out(6, 0.0f), expect(6, 0.0f);
+    CompileAndRun("softmax", func, {In(d), Out(out)});
+    for (int row = 0; row < 2; ++row) {
+        float denom = 0.0f;
+        for (int col = 0; col < 3; ++col) denom += std::exp(d[row * 3 + col]);
+        for (int col = 0; col < 3; ++col) expect[row * 3 + col] = std::exp(d[row * 3 + col]) / denom;
+    }
+    ExpectNear(out, expect);
+    // axis 0 of a rank-3 tensor, negative axis spelling: every column of the leading axis sums to 1
+    kxc::Var t("t", kxc::TensorType({3, 2, 2}, "float32"));
+    kxc::Function f2({t}, kxc::Call(Op::Get("softmax"), {t}, kxc::relay::SoftmaxAttrs::Create(-3)));
+    std::vector<float> td = {0.5f, -1, 2, 0, 1, 1, -2, 3, 0.25f, 0, 1, -1}, to(12, 0.0f);
+    CompileAndRun("softmax axis 0", f2, {In(td), Out(to)});
+    for (int i = 0; i < 4; ++i) {
+        float denom = std::exp(td[i]) + std::exp(td[4 + i]) + std::exp(td[8 + i]);
+        ExpectNear({to[i], to[4 + i], to[8 + i]}, {std::exp(td[i]) / denom, std::exp(td[4 + i]) / denom, std::exp(td[8 + i]) / denom});
+    }
+}
+
+// float32 -> int32 truncates toward zero (test/op_numeric_llvm_test.cpp:295-305)
+void TestCast() {
+    kxc::Var data("data", kxc::TensorType({4}, "float32"));
+    kxc::Function func({data}, kxc::Call(Op::Get("cast"), {data}, kxc::relay::CastAttrs::Create(1)));
+    std::vector<float> d = {1.9f, -2.2f, 3.0f, 4.8f};
+    std::vector<int32_t> out(4, 0);
+    CompileAndRun("cast", func, {In(d), Buf{out.data(), out.size() * sizeof(int32_t), true}});
+    if (out != std::vector<int32_t>({1, -2, 3, 4})) throw std::runtime_error("cast: wrong result");
+    // int32 -> float32 and back through a chain
+    kxc::Var iv("iv", kxc::TensorType({3}, "int32"));
+    kxc::Function f2({iv}, kxc::Call(Op::Get("cast"), {iv}, kxc::relay::CastAttrs::Create(0)));
+    std::vector<int32_t> id = {-7, 0, 12};
+    std::vector<float> fo(3, 0.0f);
+    CompileAndRun("cast to float", f2, {Buf{id.data(), id.size() * sizeof(int32_t), false}, Out(fo)});
+    ExpectNear(fo, {-7.0f, 0.0f, 12.0f});
+    bool threw = false;
+    try { kxc::relay::CastAttrs::Create(9); kxc::relay::CastDTypeFromCode(9); } catch (const std::exception& e) {
+        threw = std::string(e.what()) == "cast has unsupported dtype code: 9";
+    }
+    if (!threw) throw std::runtime_error("cast: bad dtype code was not refused");
+}
+
 void TestModelAddChain() {
     kxc::Var x("x", kxc::TensorType({4}, "float32"));
     kxc::Var y("y", kxc::TensorType({4}, "float32"));
@@ -283,7 +333,8 @@ int RunOpNumeric() {
         {"matmul", TestMatmul}, {"nn_dense", TestDense}, {"nn_gemm", TestGemm}, {"nn_relu", TestRelu},
         {"nn_conv2d", TestConv2D}, {"nn_max_pool2d", TestMaxPool2D}, {"nn_avg_pool2d", TestAvgPool2D},
         {"nn_global_avg_pool2d", TestGlobalAvgPool2D}, {"nn_flatten", TestFlatten}, {"reshape", TestReshape},
-        {"transpose", TestTranspose}, {"reduce_mean", TestReduceMean}, {"model_add_chain", TestModelAddChain},
+        {"transpose", TestTranspose}, {"reduce_mean", TestReduceMean}, {"softmax", TestSoftmax}, {"cast", TestCast},
+        {"model_add_chain", TestModelAddChain},
         {"model_mlp", TestModelMLP}, {"model_cnn", TestModelCNN}, {"errors", TestErrors},
     };
     for (const auto& t : tests) {
@@ -527,6 +578,196 @@ int RunOnnxErrors(const std::string& dir) {
     return 0;
 }
 
+// adaptive <cpu|hip|hipgen> [bundle dir]: the adaptive runtime (kxc/runtime_session.h) -- cache rules, shape
+// statistics, priority order of the background compiler, a session that goes miss -> fuzzy hit -> background
+// compile -> exact hit, and compiles on worker threads concurrent with runs on this thread.
+struct StagedArgs {                     // host vectors staged through DeviceAPI buffers when the target is the GPU
+    std::vector<Buf> bufs;
+    std::vector<void*> args;
+    explicit StagedArgs(std::vector<Buf> b) : bufs(std::move(b)) {
+        if (g_mode == "cpu") { for (auto& x : bufs) args.push_back(x.host); return; }
+        kxc::DeviceAPI* api = kxc::GetDeviceAPI(kxc::kGPU);
+        kxc::Device dev(kxc::kGPU, 0), cpu(kxc::kCPU, 0);
+        for (auto& x : bufs) {
+            void* d = api->AllocDataSpace(dev, x.bytes, 256);
+            if (!x.out) api->CopyDataFromTo(cpu, x.host, dev, d, x.bytes);
+            args.push_back(d);
+        }
+    }
+    void Fetch() {
+        if (g_mode == "cpu") return;
+        kxc::DeviceAPI* api = kxc::GetDeviceAPI(kxc::kGPU);
+        kxc::Device dev(kxc::kGPU, 0), cpu(kxc::kCPU, 0);
+        for (size_t i = 0; i < bufs.size(); ++i)
+            if (bufs[i].out) api->CopyDataFromTo(dev, args[i], cpu, bufs[i].host, bufs[i].bytes);
+    }
+    ~StagedArgs() {
+        if (g_mode == "cpu") return;
+        kxc::DeviceAPI* api = kxc::GetDeviceAPI(kxc::kGPU);
+        for (void* d : args) api->FreeDataSpace(kxc::Device(kxc::kGPU, 0), d);
+    }
+};
+
+int RunAdaptive(const std::string& bundle_dir) {
+    using namespace kxc::runtime;
+    // ---- KernelCache::ShapeDistance (kernel_cache.cc:54-73)
+    auto sig = [](std::vector<std::vector<int64_t>> s) { return MakeShapeSignature(s); };
+    Check(KernelCache::ShapeDistance(sig({{2, 3}}), sig({{2, 3}})) == 0, "identical shapes are at distance 0");
+    Check(KernelCache::ShapeDistance(sig({{2, 3}}), sig({{4, 8}})) == 7, "distance is the summed difference");
+    Check(KernelCache::ShapeDistance(sig({{2, 3}}), sig({{4, 2}})) == -1, "a smaller cached dimension cannot serve");
+    Check(KernelCache::ShapeDistance(sig({{2, 3}}), sig({{2, 3, 1}})) == -1, "rank must agree");
+    Check(KernelCache::ShapeDistance(sig({{2, 3}}), sig({{2, 3}, {1}})) == -1, "input count must agree");
+    Check(sig({{2, 3}}).Hash() == sig({{2, 3}}).Hash() && !(sig({{2, 3}}) == sig({{3, 2}})), "signature equality / hash");
+    // ---- ShapePredictor (shape_predictor.cc:17-66)
+    {
+        ShapePredictor p;
+        for (int i = 0; i < 3; ++i) p.Record(sig({{8}}));
+        p.Record(sig({{4}}));
+        for (int i = 0; i < 2; ++i) p.Record(sig({{2}}));
+        Check(p.TotalCount() == 6 && p.GetCount(sig({{8}})) == 3 && p.GetCount(sig({{9}})) == 0, "counts");
+        auto top = p.PredictTopK(2);
+        Check(top.size() == 2 && top[0] == sig({{8}}) && top[1] == sig({{2}}), "top-k is ordered by frequency");
+        Check(p.ShouldCompile(sig({{2}})) && !p.ShouldCompile(sig({{4}})) && !p.ShouldCompile(sig({{9}})), "seen at least twice");
+        Check(p.ShouldCompile(sig({{4}}), 1), "count threshold argument");
+    }
+    // ---- KernelRunner (kernel_runner.cc:13-34)
+    {
+        KernelRunner r;
+        bool threw = false;
+        try { r.Run({}); } catch (const std::exception& e) { threw = std::string(e.what()) == "KernelRunner: no kernel available"; }
+        Check(threw && !r.HasKernel(), "an empty runner refuses to run");
+    }
+
+    auto make_add = [](int64_t rows) {
+        kxc::Var x("x", kxc::TensorType({rows, 3}, "float32"));
+        kxc::Var y("y", kxc::TensorType({3}, "float32"));
+        return kxc::Function({x, y}, kxc::Call(Op::Get("add"), {x, y}));
+    };
+    // ---- BackgroundCompiler: one worker; while it is held inside the first task's callback four more tasks are
+    // queued -- they must complete highest priority first (background_compiler.h:36, background_compiler.cc:54-58)
+    {
+        BackgroundCompiler bg(1);
+        std::mutex mu;
+        std::condition_variable cv;
+        bool release = false;
+        std::vector<int> order;
+        auto task = [&](int priority, bool hold) {
+            BackgroundCompiler::CompileTask t;
+            t.relay_func = make_add(2);
+            t.config = MakeConfig();
+            t.priority = priority;
+            t.on_complete = [&, priority, hold](kxc::api::CompiledModule m) {
+                Check(m.IsReady() || g_mode == "cpu", "background module ready");
+                std::unique_lock<std::mutex> lock(mu);
+                if (hold) cv.wait(lock, [&] { return release; });
+                order.push_back(priority);
+            };
+            return t;
+        };
+        bg.Submit(task(100, true));
+        while (bg.PendingCount() != 0) std::this_thread::yield();          // the worker has taken it
+        for (int p : {1, 7, 3, 5}) bg.Submit(task(p, false));
+        Check(bg.PendingCount() == 4, "four tasks queued behind the running one");
+        { std::lock_guard<std::mutex> lock(mu); release = true; }
+        cv.notify_all();
+        bg.WaitAll();
+        Check(order == std::vector<int>({100, 7, 5, 3, 1}), "tasks complete in priority order");
+        Check(bg.CompletedCount() == 5 && bg.PendingCount() == 0 && bg.FailedCount() == 0, "completed count");
+        // a task whose compilation throws is counted as failed and does not stop the worker
+        BackgroundCompiler::CompileTask bad;
+        kxc::Var v("v", kxc::TensorType({2, 3}, "float32"));
+        kxc::Var w("w", kxc::TensorType({4}, "float32"));
+        bad.relay_func = kxc::Function({v, w}, kxc::Call(Op::Get("add"), {v, w}));     // shapes do not broadcast
+        bad.config = MakeConfig();
+        bg.Submit(bad);
+        bg.WaitAll();
+        Check(bg.FailedCount() == 1 && bg.CompletedCount() == 5, "a failing compile is contained");
+    }
+
+    // ---- RuntimeSession: warm up a larger shape, then ask for a smaller one three times
+    std::shared_ptr<kxc::profiling::ProfileContext> ctx;
+    if (!bundle_dir.empty()) {
+        kxc::profiling::ProfileOptions options;
+        options.enabled = true;
+        options.bundle_dir = bundle_dir;
+        ctx = kxc::profiling::ProfileContext::Create(options);
+    }
+    {
+        std::unique_ptr<kxc::profiling::ActivationScope> scope;
+        if (ctx) scope = std::make_unique<kxc::profiling::ActivationScope>(ctx, ctx->NextRunId("adaptive"));
+        auto config = MakeConfig();
+        config->background_threads = 2;
+        RuntimeSession session(make_add(2), config, ctx);
+        Check(session.CachedKernelCount() == 0 && session.GetStatus() == "RuntimeSession{cached=0, pending=0, completed=0, total_runs=0}",
+              "fresh session status: " + session.GetStatus());
+        session.WarmUp({{4, 3}, {3}});
+        session.WarmUp({{4, 3}, {3}});                                    // second warm-up of a cached shape is a no-op
+        Check(session.CachedKernelCount() == 1, "warm-up caches one module");
+        std::vector<float> xd = {1, 2, 3, 4, 5, 6}, yd = {10, 20, 30}, out(6, 0.0f);
+        StagedArgs staged({In(xd), In(yd), Out(out)});
+        const std::vector<std::vector<int64_t>> small = {{2, 3}, {3}};
+        session.Run(staged.args, small);                                  // fuzzy hit, seen once: nothing scheduled
+        session.WaitAll();
+        Check(session.CachedKernelCount() == 1, "first fuzzy hit schedules nothing");
+        session.Run(staged.args, small);                                  // fuzzy hit, seen twice: background compile
+        session.WaitAll();
+        Check(session.CachedKernelCount() == 2, "second fuzzy hit compiles the exact shape in the background");
+        session.Run(staged.args, small);                                  // exact hit
+        session.Run(staged.args, small);
+        session.WaitAll();
+        staged.Fetch();
+        ExpectNear(out, {11, 22, 33, 14, 25, 36});
+        Check(session.GetStatus() == "RuntimeSession{cached=2, pending=0, completed=1, total_runs=4}", "status: " + session.GetStatus());
+        Check(session.PendingCompileCount() == 0, "nothing pending");
+        // a shape nothing cached can serve: compiled on the calling thread
+        RuntimeSession cold(make_add(2), config, ctx);
+        cold.Run(staged.args, small);
+        Check(cold.CachedKernelCount() == 1 && cold.GetStatus() == "RuntimeSession{cached=1, pending=0, completed=0, total_runs=1}",
+              "cold miss compiles synchronously: " + cold.GetStatus());
+    }
+
+    // ---- compiles on worker threads while this thread runs: the small CNN of the known-answer tests, compiled
+    // eight times on four workers, each module run by the worker that built it, with the session above's kind of
+    // run going on here in between
+    {
+        BackgroundCompiler bg(4);
+        std::atomic<int> good{0};
+        std::mutex print_mu;
+        for (int i = 0; i < 8; ++i) {
+            BackgroundCompiler::CompileTask t;
+            t.relay_func = make_add(2 + i);
+            t.config = MakeConfig();
+            t.priority = i;
+            const int rows = 2 + i;
+            t.on_complete = [&, rows](kxc::api::CompiledModule m) {
+                std::vector<float> xd(static_cast<size_t>(rows) * 3), yd = {1, 2, 3}, out(xd.size(), 0.0f);
+                for (size_t k = 0; k < xd.size(); ++k) xd[k] = static_cast<float>(k);
+                StagedArgs staged({In(xd), In(yd), Out(out)});
+                m.Run(staged.args);
+                staged.Fetch();
+                bool ok = true;
+                for (size_t k = 0; k < xd.size(); ++k) ok = ok && out[k] == xd[k] + yd[k % 3];
+                if (ok) ++good;
+            };
+            bg.Submit(std::move(t));
+        }
+        auto module = kxc::api::Compiler::Compile(make_add(2), MakeConfig());
+        std::vector<float> xd = {1, 2, 3, 4, 5, 6}, yd = {10, 20, 30}, out(6, 0.0f);
+        StagedArgs staged({In(xd), In(yd), Out(out)});
+        for (int it = 0; it < 50; ++it) module.Run(staged.args);
+        bg.WaitAll();
+        staged.Fetch();
+        ExpectNear(out, {11, 22, 33, 14, 25, 36});
+        Check(good.load() == 8 && bg.CompletedCount() == 8, "eight concurrent compiles ran correctly: " + std::to_string(good.load()));
+    }
+    if (ctx) {
+        ctx->Flush();
+        std::cout << "profile bundle: " << ctx->bundle_dir() << " events=" << ctx->event_count() << "\n";
+    }
+    std::cout << "adaptive runtime ok (" << g_mode << ")\n";
+    return 0;
+}
+
 // profile <cpu|hip|hipgen> <bundle dir>: the CNN known-answer model under an active profiling context; the
 // bundle lands in <bundle dir> (the Python tests read it back).
 int RunProfile(const std::string& dir) {
@@ -556,6 +797,7 @@ int main(int argc, char** argv) {
         const std::string cmd = argc > 1 ? argv[1] : "";
         if (cmd == "op_numeric") { g_mode = argc > 2 ? argv[2] : "cpu"; return RunOpNumeric(); }
         if (cmd == "device_info") return RunDeviceInfo();
+        if (cmd == "adaptive") { g_mode = argc > 2 ? argv[2] : "cpu"; return RunAdaptive(argc > 3 ? argv[3] : ""); }
         if (cmd == "codegen") return RunCodegen();
         if (cmd == "onnx" && argc >= 4) { g_mode = argv[2]; return RunOnnx(argv[3]); }
         if (cmd == "onnx_errors" && argc >= 3) return RunOnnxErrors(argv[2]);

@@ -45,7 +45,7 @@ def bits(a):
 def test_op_numeric_known_answers_cpu():
     out = run("op_numeric", "cpu")
     assert "All operator numeric tests passed (cpu)" in out
-    assert out.count("[PASS]") == 21
+    assert out.count("[PASS]") == 23          # 19 operators (softmax and cast included), 3 small models, the error cases
 
 
 def test_device_info_contract():
@@ -180,6 +180,44 @@ def test_profiling_bundle_cpu_target():
         infer = [e for e in events if e["pass_name"] == "InferType"][0]
         assert spans[infer["parent_span_id"]]["event_type"] == "compile"       # nesting follows the call stack
         assert os.path.exists(os.path.join(d, "artifacts", "kernel_main.c"))
+
+
+# ------------------------------------------------------------------ adaptive runtime
+def _adaptive_events(d):
+    events, _, _ = _read_bundle(d)
+    return [(e["component"], e["event_type"]) for e in events], events
+
+
+def test_adaptive_runtime_cpu_target():
+    """RuntimeSession / KernelCache / ShapePredictor / BackgroundCompiler / KernelRunner with the reference's rules
+    (cache miss -> fuzzy hit -> background compile -> exact hit, priority order, status text), and the profiling
+    events a session leaves."""
+    with tempfile.TemporaryDirectory() as d:
+        assert "adaptive runtime ok (cpu)" in run("adaptive", "cpu", d)
+        kinds, events = _adaptive_events(d)
+    for want in ("runtime_session_warmup", "runtime_session_run", "cache_fuzzy_hit", "cache_exact_hit",
+                 "cache_miss_sync_compile", "background_compile_submitted", "background_compile_completed",
+                 "runtime_session_wait_all"):
+        assert ("runtime_session", want) in kinds, want
+    assert ("background_compiler", "background_compile_task") in kinds
+    assert kinds.count(("runtime_session", "cache_fuzzy_hit")) == 2 and kinds.count(("runtime_session", "cache_exact_hit")) == 2
+    assert kinds.count(("runtime_session", "background_compile_submitted")) == 1
+    runs = [e for e in events if e["event_type"] == "runtime_session_run"]
+    assert all(e["shape_signature"] == "[[2,3],[3]]" or "2" in e["shape_signature"] for e in runs)
+    task = [e for e in events if e["event_type"] == "background_compile_task"][0]
+    submit = [e for e in events if e["event_type"] == "background_compile_submitted"][0]
+    assert task["run_id"] == submit["run_id"]                  # the worker thread reports under the caller's run
+
+
+@pytest.mark.gpu
+def test_adaptive_runtime_hip_target():
+    """The same on the GPU: worker threads build launch plans (and, for generated kernels, compile with hipRTC
+    and load modules) while the calling thread keeps running."""
+    assert "adaptive runtime ok (hip)" in run("adaptive", "hip")
+    with tempfile.TemporaryDirectory() as d:
+        assert "adaptive runtime ok (hipgen)" in run("adaptive", "hipgen", d)
+        kinds, _ = _adaptive_events(d)
+    assert ("runtime_session", "background_compile_completed") in kinds
 
 
 @pytest.mark.gpu
