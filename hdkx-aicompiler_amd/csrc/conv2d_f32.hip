@@ -289,12 +289,6 @@ conv_mfma_kernel(const ConvArgs a) {
             for (int i = 0; i < RO; ++i) av[i] = ws[wbase[i] + koff_w];
 #pragma unroll
             for (int j = 0; j < RP; ++j) bv[j] = xs[xbase[j] + koff_x];
-#ifdef KXC_DBG_NO_LDS_READS
-#pragma unroll
-            for (int i = 0; i < RO; ++i) av[i] = (float)(wbase[i] + koff_w);
-#pragma unroll
-            for (int j = 0; j < RP; ++j) bv[j] = (float)(xbase[j] + koff_x);
-#endif
         };
         float av[PF + 1][RO], bv[PF + 1][RP];
 #pragma unroll
@@ -321,10 +315,8 @@ conv_mfma_kernel(const ConvArgs a) {
         }
         }
 
-#ifndef KXC_DBG_NO_BARRIER
         asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
         __syncthreads();
-#endif
     }
 
     // ---- combine the reduction groups: groups 1.. park their accumulators in LDS (the tiles are dead after
@@ -424,9 +416,6 @@ conv_mfma_kernel(const ConvArgs a) {
                     if (has_bias) v = __fadd_rn(v, bv[i][gc + g]);
                     if (has_res) v = __fadd_rn(v, q[i][j][g]);
                     if (do_relu) v = relu_sel(v);
-#ifdef KXC_DBG_NO_STORE
-                    if (v == 123456.789f)
-#endif
                     __builtin_amdgcn_raw_buffer_store_b32(__builtin_bit_cast(uint32_t, v), yr, out_off(i, gc + g, j), 0, 0);
                 }
             }
