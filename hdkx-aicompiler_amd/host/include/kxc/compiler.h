@@ -19,6 +19,9 @@
 #include "kxc/lower.h"
 
 namespace kxc {
+namespace runtime {
+class RuntimeSession;       // kxc/runtime_session.h
+}
 namespace api {
 
 enum class CompileMode { kAOT, kJIT, kAdaptive };
@@ -34,7 +37,10 @@ struct CompileConfigNode {
     bool hip_concurrent_branches{true};   // run a block's downsample convolution beside its first 3x3 convolution
     bool hip_winograd{true};              // 3x3 stride-1 convolutions with constant weights as Winograd F(2x2,3x3) where faster
     bool sync_after_run{true};
-    int background_threads{0};         // adaptive runtime: compile workers (0 = half the hardware threads)
+    // Adaptive mode (include/api/compile_config.h:40-45)
+    std::vector<std::vector<int64_t>> suggested_input_shapes;   // each is warmed up at Compile
+    int background_threads{0};         // compile workers (0 = half the hardware threads)
+    bool enable_hot_swap{true};
 };
 class CompileConfig : public Ref<CompileConfigNode> {
 public:
@@ -42,6 +48,9 @@ public:
     explicit CompileConfig(std::shared_ptr<CompileConfigNode> n) : Ref<CompileConfigNode>(std::move(n)) {}
     static CompileConfig AOT(Target target, int opt_level = 3);
     static CompileConfig JIT(Target target);
+    // Compile returns a module backed by a runtime::RuntimeSession: Run(args, input_shapes) goes through its shape
+    // cache and background compiler (src/api/compile_config.cc:38-49, src/api/compiler.cc:64-80).
+    static CompileConfig Adaptive(Target target, std::vector<std::vector<int64_t>> suggested_shapes = {});
 };
 
 // One launch of a compiled module, as an execution-plan node would describe it
@@ -60,6 +69,11 @@ public:
     CompiledModule() = default;
     explicit CompiledModule(std::shared_ptr<CompiledModuleImpl> impl) : impl_(std::move(impl)) {}
     void Run(const std::vector<void*>& packed_args);
+    // Adaptive modules run only through this overload (the plain one throws "Adaptive mode requires
+    // Run(args, input_shapes)..."); for other modules the shapes are ignored (src/api/compiler.cc:146-191).
+    void Run(const std::vector<void*>& packed_args, const std::vector<std::vector<int64_t>>& input_shapes);
+    void WarmUp(const std::vector<std::vector<int64_t>>& input_shapes);     // adaptive: compile for a shape now
+    void WaitAll();                                                          // adaptive: drain background compiles
     bool IsReady() const;
     std::string GetStatus() const;
     const tir::PrimFunc& GetPrimFunc() const;
@@ -81,7 +95,9 @@ public:
     void EnableGraphReplay(bool enable);
 
 private:
+    friend class Compiler;
     std::shared_ptr<CompiledModuleImpl> impl_;
+    std::shared_ptr<runtime::RuntimeSession> session_;     // adaptive mode only
 };
 
 class Compiler {

@@ -1,5 +1,6 @@
 // compiler.cc -- Compiler::Compile and CompiledModule (see compiler.h).
 #include "kxc/compiler.h"
+#include "kxc/runtime_session.h"
 #include "kxc/profiling.h"
 #include "json_reader.h"
 
@@ -35,6 +36,15 @@ CompileConfig CompileConfig::JIT(Target target) {
     n->mode = CompileMode::kJIT;
     n->opt_level = 1;
     n->target = target;
+    n->enable_hot_swap = false;
+    return CompileConfig(n);
+}
+CompileConfig CompileConfig::Adaptive(Target target, std::vector<std::vector<int64_t>> suggested_shapes) {
+    auto n = std::make_shared<CompileConfigNode>();
+    n->mode = CompileMode::kAdaptive;
+    n->opt_level = 2;
+    n->target = target;
+    n->suggested_input_shapes = std::move(suggested_shapes);
     return CompileConfig(n);
 }
 
@@ -502,6 +512,14 @@ private:
 
 CompiledModule Compiler::Compile(Function func, CompileConfig config) {
     if (!config.defined() || !config->target.defined()) throw std::runtime_error("Compiler::Compile: config has no target");
+    if (config->mode == CompileMode::kAdaptive) {
+        // the session compiles (ahead-of-time mode) on demand; every suggested shape is warmed up now, each as the
+        // shape of a single input (src/api/compiler.cc:64-80)
+        CompiledModule adaptive;
+        adaptive.session_ = std::make_shared<runtime::RuntimeSession>(func, config, profiling::CurrentContext());
+        for (const auto& shape : config->suggested_input_shapes) adaptive.session_->WarmUp({shape});
+        return adaptive;
+    }
     auto impl = std::make_shared<CompiledModuleImpl>();
     impl->config = config;
     profiling::EventSpec cspec;
@@ -555,7 +573,19 @@ CompiledModule Compiler::Compile(Function func, CompileConfig config) {
     return module;
 }
 
+void CompiledModule::Run(const std::vector<void*>& packed_args, const std::vector<std::vector<int64_t>>& input_shapes) {
+    if (session_) { session_->Run(packed_args, input_shapes); return; }
+    Run(packed_args);
+}
+void CompiledModule::WarmUp(const std::vector<std::vector<int64_t>>& input_shapes) {
+    if (session_) session_->WarmUp(input_shapes);
+}
+void CompiledModule::WaitAll() {
+    if (session_) session_->WaitAll();
+}
+
 void CompiledModule::Run(const std::vector<void*>& packed_args) {
+    if (session_) throw std::runtime_error("Adaptive mode requires Run(args, input_shapes). Use the overload with input_shapes.");
     if (!impl_ || !impl_->ready) throw std::runtime_error("CompiledModule::Run: module is not ready: " + GetStatus());
     const size_t expect = static_cast<size_t>(impl_->input_count + impl_->constant_count + 1);
     if (packed_args.size() != expect)
@@ -612,8 +642,8 @@ void CompiledModule::Run(const std::vector<void*>& packed_args) {
     }
 }
 
-bool CompiledModule::IsReady() const { return impl_ && impl_->ready; }
-std::string CompiledModule::GetStatus() const { return impl_ ? impl_->status : "empty"; }
+bool CompiledModule::IsReady() const { return session_ || (impl_ && impl_->ready); }
+std::string CompiledModule::GetStatus() const { return session_ ? session_->GetStatus() : impl_ ? impl_->status : "empty"; }
 const tir::PrimFunc& CompiledModule::GetPrimFunc() const { return impl_->prim_func; }
 const std::string& CompiledModule::GetSource() const { return impl_->source; }
 void CompiledModule::SaveCSource(const std::string& path) const {

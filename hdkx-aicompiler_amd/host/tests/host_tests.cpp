@@ -726,6 +726,45 @@ int RunAdaptive(const std::string& bundle_dir) {
               "cold miss compiles synchronously: " + cold.GetStatus());
     }
 
+    // ---- the same through the user-visible entry: CompileConfig::Adaptive + Compiler::Compile
+    // (include/api/compile_config.h:62-68, src/api/compiler.cc:64-80,146-191)
+    {
+        auto base = MakeConfig();
+        auto config = kxc::api::CompileConfig::Adaptive(base->target, {{4, 3}});
+        config->hip_use_handwritten = base->hip_use_handwritten;
+        config->hip_fuse = base->hip_fuse;
+        config->background_threads = 1;
+        Check(config->mode == kxc::api::CompileMode::kAdaptive && config->opt_level == 2 && config->enable_hot_swap, "Adaptive config");
+        kxc::Var x("x", kxc::TensorType({2, 3}, "float32"));
+        kxc::Function relu({x}, kxc::Call(Op::Get("nn_relu"), {x}));
+        auto module = kxc::api::Compiler::Compile(relu, config);
+        Check(module.IsReady(), "an adaptive module is ready at once");
+        Check(module.GetStatus() == "RuntimeSession{cached=1, pending=0, completed=0, total_runs=0}",
+              "the suggested shape was warmed up: " + module.GetStatus());
+        std::vector<float> xd = {-1, 2, -3, 4, -5, 6}, out(6, 0.0f);
+        StagedArgs staged({In(xd), Out(out)});
+        bool threw = false;
+        try { module.Run(staged.args); } catch (const std::exception& e) {
+            threw = std::string(e.what()) == "Adaptive mode requires Run(args, input_shapes). Use the overload with input_shapes.";
+        }
+        Check(threw, "the plain Run of an adaptive module is refused");
+        module.Run(staged.args, {{2, 3}});
+        module.Run(staged.args, {{2, 3}});
+        module.WaitAll();
+        module.WarmUp({{8, 3}});
+        staged.Fetch();
+        ExpectNear(out, {0, 2, 0, 4, 0, 6});
+        Check(module.GetStatus() == "RuntimeSession{cached=3, pending=0, completed=1, total_runs=2}", "adaptive module status: " + module.GetStatus());
+        // a non-adaptive module accepts the shape overload and ignores the shapes
+        auto plain = kxc::api::Compiler::Compile(relu, MakeConfig());
+        std::fill(out.begin(), out.end(), 0.0f);
+        StagedArgs staged2({In(xd), Out(out)});
+        plain.Run(staged2.args, {{2, 3}});
+        plain.WaitAll();
+        staged2.Fetch();
+        ExpectNear(out, {0, 2, 0, 4, 0, 6});
+    }
+
     // ---- compiles on worker threads while this thread runs: the small CNN of the known-answer tests, compiled
     // eight times on four workers, each module run by the worker that built it, with the session above's kind of
     // run going on here in between
