@@ -116,10 +116,11 @@ __global__ void __launch_bounds__(256) wino_weight_kernel(const float* __restric
 // One step = 4 input channels.  LDS per buffer: U [WK][c4][o/16: 2][f/4: 4][o%16][f%4] and
 // V [c4][WT][f/4: 4][tile%16][f%4]; two of each.
 // ------------------------------------------------------------------------------------------
-template <int WK, int WT, bool SKEW>
-__global__ void __launch_bounds__(64 * WK * WT) __attribute__((amdgpu_waves_per_eu(2)))
+template <int WK, int WT, int KS>
+__global__ void __launch_bounds__(64 * WK * WT * KS) __attribute__((amdgpu_waves_per_eu(2)))
 wino_kernel(const WinoArgs a) {
-    constexpr int NTH = 64 * WK * WT;
+    constexpr int NW = WK * WT;                     // waves of one reduction group
+    constexpr int NTH = 64 * NW;                    // threads of one reduction group
     constexpr int TT = 16 * WT;
     constexpr int U_FLOATS = 2048 * WK;
     constexpr int V_FLOATS = 1024 * WT;
@@ -127,11 +128,14 @@ wino_kernel(const WinoArgs a) {
     constexpr int ITEMS = 2 / WK;                   // (tile, channel, half) items per thread and step
     static_assert(WK == 1 || WK == 2, "a thread transforms one or two input items per step");
     static_assert((U_FLOATS / 4) % NTH == 0, "weight tile must divide over the threads");
+    static_assert(KS == 1 || KS == 2, "the input channels are split over at most two groups of waves");
 
     extern __shared__ float lds[];
-    const int tid = threadIdx.x;
-    const int lane = tid & 63;
-    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int lane = threadIdx.x & 63;
+    const int wave_all = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    const int kgroup = wave_all / NW;               // which share of the input channels this wave reduces
+    const int wave = wave_all - kgroup * NW;
+    const int tid = static_cast<int>(threadIdx.x) - kgroup * NTH;
     const int wave_k = wave / WT, wave_t = wave % WT;
     // Consecutive workgroups go to the 8 XCDs round-robin; each XCD (own L2) takes a contiguous run of units.
     const int unit = (blockIdx.x & 7) * a.units_per_xcd + (blockIdx.x >> 3);
@@ -231,93 +235,33 @@ wino_kernel(const WinoArgs a) {
         }
     };
 
-    const int last = a.csteps - 1;
-    if constexpr (SKEW) {
-        // Three LDS tiles (weights + transformed input of one step each) and the barrier in the MIDDLE of a step:
-        // between two barriers a wave multiplies the second half of step p (groups 2, 3) and the first half of
-        // step p+1 (groups 0, 1), while tile p+2 is being filled.  The operands of the first group after a barrier
-        // come from a tile that was already visible before it, so they are fetched ahead of the barrier and no
-        // wave waits for LDS right after one.
-        constexpr int BUF = U_FLOATS + V_FLOATS;
-        auto ubuf = [&](int i) { return lds + i * BUF; };
-        auto vbuf = [&](int i) { return lds + i * BUF + U_FLOATS; };
-        issue_u(0, ubuf(0));
-        load_raw(0);
-        transform(vbuf(0));
-        load_raw(min(1, last));
-        __builtin_amdgcn_sched_barrier(0);
-        __syncthreads();                                    // tile 0 visible
-        issue_u(min(1, last), ubuf(1));
-        fetch(ubuf(0), vbuf(0), 0, 0);
-        fetch(ubuf(0), vbuf(0), 1, 1);
-        __builtin_amdgcn_sched_barrier(0);
-        mm(0, 0);
-        transform(vbuf(1));
-        __builtin_amdgcn_sched_barrier(0);
-        fetch(ubuf(0), vbuf(0), 2, 0);
-        mm(1, 1);
-        load_raw(min(2, last));
-        __builtin_amdgcn_sched_barrier(0);
-        __syncthreads();                                    // tile 1 visible
-        int i0 = 0, i1 = 1, i2 = 2;                         // buffers of tiles p, p+1, p+2
-        for (int p = 0; p < last; ++p) {
-            const float* const u0 = ubuf(i0); const float* const v0 = vbuf(i0);
-            const float* const u1 = ubuf(i1); const float* const v1 = vbuf(i1);
-            issue_u(min(p + 2, last), ubuf(i2));
-            fetch(u0, v0, 3, 1);
-            __builtin_amdgcn_sched_barrier(0);
-            mm(2, 0);
-            __builtin_amdgcn_sched_barrier(0);
-            fetch(u1, v1, 0, 0);
-            mm(3, 1);
-            __builtin_amdgcn_sched_barrier(0);
-            fetch(u1, v1, 1, 1);
-            mm(0, 0);
-            transform(vbuf(i2));                            // raw input of step p+2, requested one window ago
-#pragma unroll
-            for (int q = 0; q < 8; ++q) {
-                __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
-                __builtin_amdgcn_sched_group_barrier(0x002, 6, 0);
-            }
-            __builtin_amdgcn_sched_barrier(0);
-            fetch(u1, v1, 2, 0);
-            mm(1, 1);
-            load_raw(min(p + 3, last));
-#pragma unroll
-            for (int q = 0; q < 8; ++q) {
-                __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
-                __builtin_amdgcn_sched_group_barrier(0x020, 2, 0);
-            }
-            __builtin_amdgcn_sched_barrier(0);
-            __syncthreads();                                // tile p+2 visible
-            const int t = i0; i0 = i1; i1 = i2; i2 = t;
-        }
-        // second half of the last step
-        fetch(ubuf(i0), vbuf(i0), 3, 1);
-        mm(2, 0);
-        mm(3, 1);
-    } else {
     // LDS: two weight tiles and two transformed-input tiles.  The compiler orders every barrier after the
     // LDS-writing loads issued before it, so a weight tile is requested at the top of the step before the one that
     // uses it and has that whole step to arrive; the raw input (registers) is requested two steps ahead.
-    float* const ub0 = lds;
-    float* const ub1 = lds + U_FLOATS;
-    float* const vb0 = lds + 2 * U_FLOATS;
+    // KS == 2 (launches with too few units to give every SIMD two waves): the two groups of waves own their own
+    // tiles and reduce one half of the input channels each, in lock step (the barriers are shared); their
+    // accumulators are added through LDS after the loop.  The host passes a step count divisible by KS.
+    float* const ub0 = lds + kgroup * 2 * (U_FLOATS + V_FLOATS);
+    float* const ub1 = ub0 + U_FLOATS;
+    float* const vb0 = ub0 + 2 * U_FLOATS;
     float* const vb1 = vb0 + V_FLOATS;
+    const int s_lo = kgroup * (a.csteps / KS), s_hi = s_lo + a.csteps / KS;
+    const int last = s_hi - 1;
 
-    // ---- prologue: weight tile and transformed input of step 0; raw input of step 1 in flight
-    issue_u(0, ub0);
-    load_raw(0);
+    // ---- prologue: weight tile and transformed input of the first step; raw input of the second in flight
+    issue_u(s_lo, ub0);
+    load_raw(s_lo);
     transform(vb0);
-    load_raw(min(1, last));
+    load_raw(min(s_lo + 1, last));
     __builtin_amdgcn_sched_barrier(0);
     __syncthreads();
 
-    for (int s = 0; s < a.csteps; ++s) {
-        const float* const ucur = (s & 1) ? ub1 : ub0;
-        const float* const vcur = (s & 1) ? vb1 : vb0;
-        float* const unxt = (s & 1) ? ub0 : ub1;
-        float* const vnxt = (s & 1) ? vb0 : vb1;
+    for (int s = s_lo; s < s_hi; ++s) {
+        const bool odd = ((s - s_lo) & 1) != 0;
+        const float* const ucur = odd ? ub1 : ub0;
+        const float* const vcur = odd ? vb1 : vb0;
+        float* const unxt = odd ? ub0 : ub1;
+        float* const vnxt = odd ? vb0 : vb1;
         // Steps past the end re-load the last step (never used), which keeps the loop free of branches.
         issue_u(min(s + 1, last), unxt);
         fetch(ucur, vcur, 0, 0);
@@ -349,8 +293,31 @@ wino_kernel(const WinoArgs a) {
         __builtin_amdgcn_sched_barrier(0);
         __syncthreads();
     }
+        asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+
+    if (KS > 1) {
+        // group 1 parks its accumulators in LDS (the tiles are dead after the loop's last barrier), one
+        // output-channel block at a time ([f][g][thread]: 16 KiB per wave), group 0 adds them to its own
+        float* const red = lds;
+#pragma unroll
+        for (int kb = 0; kb < 2; ++kb) {
+            if (kgroup == 1) {
+#pragma unroll
+                for (int f = 0; f < 16; ++f)
+#pragma unroll
+                    for (int g = 0; g < 4; ++g) red[(f * 4 + g) * NTH + tid] = acc[f][kb][g];
+            }
+            __syncthreads();
+            if (kgroup == 0) {
+#pragma unroll
+                for (int f = 0; f < 16; ++f)
+#pragma unroll
+                    for (int g = 0; g < 4; ++g) acc[f][kb][g] += red[(f * 4 + g) * NTH + tid];
+            }
+            __syncthreads();
+        }
+        if (kgroup != 0) return;
     }
-    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
 
     // ---- epilogue: accumulator register g of block kb holds output channel 16*kb + 4*(lane/16) + g, tile lane%16.
     // Everything goes through buffer descriptors: an offset beyond the buffer makes a load return 0 and drops a
@@ -461,20 +428,20 @@ wino_kernel(const WinoArgs a) {
 
 struct WinoVariant {
     const char* name;
-    int wk, wt, bufs;
+    int wk, wt, ks;
     void (*kernel)(const WinoArgs);
 };
-#define KXC_WINO(WK, WT) {"winograd_f2k3_o" #WK "_t" #WT, WK, WT, 2, wino_kernel<WK, WT, false>}
-#define KXC_WINO_S3(WK, WT) {"winograd_f2k3_o" #WK "_t" #WT "_s3", WK, WT, 3, wino_kernel<WK, WT, true>}
-// name = winograd_f2k3_o<waves along output channels (32 each)>_t<waves along tiles (16 each)>[_s3: three LDS tiles]
+#define KXC_WINO(WK, WT) {"winograd_f2k3_o" #WK "_t" #WT, WK, WT, 1, wino_kernel<WK, WT, 1>}
+#define KXC_WINO_KS2(WK, WT) {"winograd_f2k3_o" #WK "_t" #WT "_ks2", WK, WT, 2, wino_kernel<WK, WT, 2>}
+// name = winograd_f2k3_o<waves along output channels (32 each)>_t<waves along tiles (16 each)>[_ks2: input channels split over two groups of waves]
 const WinoVariant kWino[] = {
     KXC_WINO(2, 2),   // 64 channels x 32 tiles, 4 waves, 48 KiB of LDS (default)
     KXC_WINO(2, 4),   // 64 x 64, 8 waves
     KXC_WINO(1, 4),   // 32 x 64, 4 waves
     KXC_WINO(2, 1),   // 64 x 16, 2 waves
     KXC_WINO(1, 2),   // 32 x 32, 2 waves
-    KXC_WINO_S3(2, 2),   // three LDS tiles, barrier in the middle of a step
-    KXC_WINO_S3(2, 1),
+    KXC_WINO_KS2(2, 2),  // 64 x 32, input channels split over two groups of 4 waves (96 KiB of LDS)
+    KXC_WINO_KS2(2, 1),  // 64 x 16, two groups of 2 waves
 };
 constexpr int kNumWino = sizeof(kWino) / sizeof(kWino[0]);
 
@@ -500,11 +467,17 @@ int64_t Tiles(const kxc_hip_conv2d_desc* d) {
 const WinoVariant* SelectWino(const kxc_hip_conv2d_desc* d) {
     if (const char* e = std::getenv("KXC_HIP_WINOGRAD_VARIANT")) {
         for (int i = 0; i < kNumWino; ++i)
-            if (std::strcmp(e, kWino[i].name) == 0) return &kWino[i];
+            if (std::strcmp(e, kWino[i].name) == 0 && (kWino[i].ks == 1 || (d->c / 4) % kWino[i].ks == 0)) return &kWino[i];
     }
+    // 64 x 32 groups from one per compute unit on; below that twice as many 64 x 16 groups.  A launch that cannot
+    // give every SIMD two waves (at most one 64 x 32 group per compute unit) and has a long reduction splits the
+    // input channels over two groups of waves inside the workgroup instead.
     const int64_t units = CeilDiv(Tiles(d), 32) * CeilDiv(d->o, 64);
+    const int csteps = d->c / 4;
+    const int wt = units < 256 ? 1 : 2;
+    const int ks = (units <= 256 && csteps % 2 == 0 && csteps >= 32) ? 2 : 1;
     for (int i = 0; i < kNumWino; ++i)
-        if (kWino[i].wk == 2 && kWino[i].wt == (units < 256 ? 1 : 2)) return &kWino[i];
+        if (kWino[i].wk == 2 && kWino[i].wt == wt && kWino[i].ks == ks) return &kWino[i];
     return &kWino[0];
 }
 
@@ -577,14 +550,14 @@ int32_t kxc_hip_conv2d_winograd_nchw_f32(const kxc_hip_conv2d_desc* desc, const 
     if (const char* e = std::getenv("KXC_HIP_WINOGRAD_KFAST")) a.k_fastest = std::atoi(e);
     a.div_ti = MakeFastDiv(a.TI); a.div_tw = MakeFastDiv(a.TW);
     a.div_kgroups = MakeFastDiv(a.k_groups); a.div_tgroups = MakeFastDiv(a.t_groups);
-    const size_t lds_bytes = v->bufs * static_cast<size_t>(2048 * v->wk + 1024 * v->wt) * sizeof(float);
+    const size_t lds_bytes = v->ks * 2 * static_cast<size_t>(2048 * v->wk + 1024 * v->wt) * sizeof(float);
     if (lds_bytes > 64 * 1024) {
         KXC_HIP_CALL(hipFuncSetAttribute(reinterpret_cast<const void*>(v->kernel), hipFuncAttributeMaxDynamicSharedMemorySize,
                                          static_cast<int>(lds_bytes)),
                      "hipFuncSetAttribute(MaxDynamicSharedMemorySize)");
     }
     hipLaunchKernelGGL(v->kernel, NoteGrid(dim3(static_cast<unsigned>(a.units_per_xcd * 8))),
-                       NoteBlock(dim3(64 * v->wk * v->wt)), NoteLds(lds_bytes), ResolveStream(stream), a);
+                       NoteBlock(dim3(64 * v->wk * v->wt * v->ks)), NoteLds(lds_bytes), ResolveStream(stream), a);
     return CheckLaunch(v->name);
 }
 

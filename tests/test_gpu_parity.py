@@ -205,6 +205,29 @@ def test_conv_winograd_exact_on_small_integers(pkg, orc):
         assert_bit_exact(host(pkg.conv2d_winograd(dev(x), u, wt.shape, dev(b), None, p, True)), want, str((n, c, h, w, o, p)))
 
 
+@pytest.mark.parametrize("variant", ["winograd_f2k3_o2_t2_ks2", "winograd_f2k3_o2_t1_ks2", "winograd_f2k3_o2_t4", "winograd_f2k3_o1_t2"])
+def test_conv_winograd_variants(pkg, fast_orc, orc, synth, monkeypatch, variant):
+    """Every workgroup shape of the Winograd kernel, forced: the two-group channel split (accumulators added through
+    LDS) and the larger / smaller tiles, on a ragged shape against the oracle and bit-exact on small integers."""
+    monkeypatch.setenv("KXC_HIP_WINOGRAD_VARIANT", variant)
+    n, c, h, w, o, p = 3, 24, 13, 10, 80, 1
+    assert pkg.conv2d_winograd_variant((n, c, h, w), (o, c, 3, 3), 1, p) == variant
+    x = synth.uniform((n, c, h, w), 7300)
+    wt = synth.normal((o, c, 3, 3), 7301, float(np.sqrt(2.0 / (c * 9))))
+    b = synth.uniform((o,), 7302, -0.1, 0.1)
+    skip = synth.uniform((n, o, h, w), 7303)
+    u = pkg.conv2d_winograd_transform_weights((n, c, h, w), dev(wt), p)
+    got = host(pkg.conv2d_winograd(dev(x), u, wt.shape, dev(b), dev(skip), p, True))
+    assert_close(got, fast_orc.conv_chain(x, wt, b, 1, p, skip, True), what=variant)
+    rng = np.random.default_rng(13)
+    xi = rng.integers(-3, 4, (2, 16, 9, 8)).astype(np.float32)
+    wi = (4 * rng.integers(-2, 3, (64, 16, 3, 3))).astype(np.float32)
+    bi = rng.integers(-5, 6, (64,)).astype(np.float32)
+    ui = pkg.conv2d_winograd_transform_weights(xi.shape, dev(wi), 1)
+    assert_bit_exact(host(pkg.conv2d_winograd(dev(xi), ui, wi.shape, dev(bi), None, 1, True)),
+                     orc.conv_chain(xi, wi, bi, 1, 1, None, True), variant + " on small integers")
+
+
 def test_conv_winograd_unsupported_shapes_are_refused(pkg):
     assert not pkg.conv2d_winograd_supported((1, 8, 8, 8), (16, 8, 3, 3), 2, 1)        # stride
     assert not pkg.conv2d_winograd_supported((1, 8, 8, 8), (16, 8, 1, 1), 1, 0)        # filter size
