@@ -26,6 +26,9 @@
 // ResNet-sized reductions), not bit for bit.
 #include <cstdlib>
 #include <cstring>
+#include <mutex>
+#include <utility>
+#include <vector>
 
 #include "common.h"
 
@@ -552,9 +555,20 @@ int32_t kxc_hip_conv2d_winograd_nchw_f32(const kxc_hip_conv2d_desc* desc, const 
     a.div_kgroups = MakeFastDiv(a.k_groups); a.div_tgroups = MakeFastDiv(a.t_groups);
     const size_t lds_bytes = v->ks * 2 * static_cast<size_t>(2048 * v->wk + 1024 * v->wt) * sizeof(float);
     if (lds_bytes > 64 * 1024) {
-        KXC_HIP_CALL(hipFuncSetAttribute(reinterpret_cast<const void*>(v->kernel), hipFuncAttributeMaxDynamicSharedMemorySize,
-                                         static_cast<int>(lds_bytes)),
-                     "hipFuncSetAttribute(MaxDynamicSharedMemorySize)");
+        // above the default 64 KiB the dynamic LDS size has to be granted per kernel and device (once)
+        static std::mutex mu;
+        static std::vector<std::pair<int, const void*>> granted;
+        int dev = 0;
+        KXC_HIP_CALL(hipGetDevice(&dev), "hipGetDevice");
+        const void* fn = reinterpret_cast<const void*>(v->kernel);
+        std::lock_guard<std::mutex> lock(mu);
+        bool have = false;
+        for (const auto& g : granted) have = have || (g.first == dev && g.second == fn);
+        if (!have) {
+            KXC_HIP_CALL(hipFuncSetAttribute(fn, hipFuncAttributeMaxDynamicSharedMemorySize, static_cast<int>(lds_bytes)),
+                         "hipFuncSetAttribute(MaxDynamicSharedMemorySize)");
+            granted.emplace_back(dev, fn);
+        }
     }
     hipLaunchKernelGGL(v->kernel, NoteGrid(dim3(static_cast<unsigned>(a.units_per_xcd * 8))),
                        NoteBlock(dim3(64 * v->wk * v->wt * v->ks)), NoteLds(lds_bytes), ResolveStream(stream), a);

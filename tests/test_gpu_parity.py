@@ -228,6 +228,27 @@ def test_conv_winograd_variants(pkg, fast_orc, orc, synth, monkeypatch, variant)
                      orc.conv_chain(xi, wi, bi, 1, 1, None, True), variant + " on small integers")
 
 
+def test_conv_winograd_random_shapes_against_direct_kernel(pkg):
+    """Seeded random geometries (batch, channels, height, width, output channels, padding; every epilogue mix):
+    the Winograd kernel against the reference-order direct kernel on the same GPU tensors."""
+    rng = np.random.default_rng(20240601)
+    for case in range(24):
+        n = int(rng.integers(1, 6)); c = 4 * int(rng.integers(1, 24)); o = int(rng.integers(1, 150))
+        h = int(rng.integers(1, 40)); w = int(rng.integers(1, 40)); p = int(rng.integers(0, 3))
+        if h + 2 * p < 3 or w + 2 * p < 3:
+            continue
+        x = torch.from_numpy(rng.uniform(-1, 1, (n, c, h, w)).astype(np.float32)).cuda()
+        wt = torch.from_numpy((rng.standard_normal((o, c, 3, 3)) * np.sqrt(2.0 / (9 * c))).astype(np.float32)).cuda()
+        b = torch.from_numpy(rng.uniform(-0.1, 0.1, (o,)).astype(np.float32)).cuda() if case % 2 == 0 else None
+        oh, ow = h + 2 * p - 2, w + 2 * p - 2
+        r = torch.from_numpy(rng.uniform(-1, 1, (n, o, oh, ow)).astype(np.float32)).cuda() if case % 3 == 0 else None
+        relu = case % 4 != 3
+        u = pkg.conv2d_winograd_transform_weights(x.shape, wt, p)
+        got = pkg.conv2d_winograd(x, u, wt.shape, b, r, p, relu)
+        want = pkg.conv2d(x, wt, b, r, 1, p, 1, relu, force_direct=True)
+        assert_close(host(got), host(want), what="case %d: n=%d c=%d h=%d w=%d o=%d p=%d" % (case, n, c, h, w, o, p))
+
+
 def test_conv_winograd_unsupported_shapes_are_refused(pkg):
     assert not pkg.conv2d_winograd_supported((1, 8, 8, 8), (16, 8, 3, 3), 2, 1)        # stride
     assert not pkg.conv2d_winograd_supported((1, 8, 8, 8), (16, 8, 1, 1), 1, 0)        # filter size
