@@ -168,11 +168,11 @@ def main():
                     "algorithmic_bytes_per_launch": algorithmic_bytes}
 
     result = {
-        "metric": "resnet18_fp32_bs64_img_per_s", "value": round(img_s, 2), "unit": "img/s",
+        "metric": "resnet18_fp32_bs%d_img_per_s" % batch, "value": round(img_s, 2), "unit": "img/s",
         "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "ms_per_step": round(ms_per_step, 4),
         "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "f32", "data": "synthetic",
         "config": {"workload": "ResNet-18 fp32 inference, batch %d, input [%d,3,224,224], BN folded, seeded Kaiming weights "
-                               "(BASELINE configs[3])" % (batch, batch),
+                               "(BASELINE configs[%d])" % (batch, batch, 3 if batch == 64 else 2),
                    "compiled_by": "C++ host layer, Compiler::Compile(Relay graph, target hip)",
                    "launches_per_step": len(info["launches"]), "workspace_bytes": info["workspace_bytes"]},
         "end_to_end_tflops": round(flop_step / (ms_per_step * 1e-3) / 1e12, 3),
