@@ -129,27 +129,40 @@ __global__ void __launch_bounds__(kBlock) maxpool3x3s2_kernel(const float* __res
 }
 
 // ---------------------------------------------------------------- global average pool
-// One wave per 64 consecutive planes.  The 64*HW contiguous floats are staged through LDS with
-// coalesced loads; each lane then adds up its own plane in row-major order (LDS row stride is
-// odd, so the 64 lanes hit distinct banks).
-constexpr int kGapPlanes = 64;
-__global__ void __launch_bounds__(kGapPlanes) gap_lds_kernel(const float* __restrict__ x, float* __restrict__ y,
-                                                             int64_t planes, int32_t hw, int32_t hw_pad) {
+// Small planes (HW <= 128): a workgroup of 256 threads takes 16 consecutive planes.  Their 16*HW contiguous
+// floats are fetched with coalesced loads that are all in flight together and staged through LDS; one lane per
+// plane then adds its plane up in row-major order, as the CPU loop does (LDS row stride is odd, so the lanes hit
+// distinct banks).  16 planes per group keeps a batch-1 launch (512 planes) spread over 32 compute units.
+constexpr int kGapPlanes = 16;       // planes per workgroup
+constexpr int kGapThreads = 256;
+constexpr int kGapMaxHw = 128;       // 16 planes x 128 elements = 8 loads per thread
+__global__ void __launch_bounds__(kGapThreads) gap_lds_kernel(const float* __restrict__ x, float* __restrict__ y,
+                                                              int64_t planes, int32_t hw, int32_t hw_pad, FastDiv div_hw) {
     extern __shared__ float tile[];
     const int64_t plane0 = static_cast<int64_t>(blockIdx.x) * kGapPlanes;
     const int64_t remaining = planes - plane0;
     const int32_t np = remaining < kGapPlanes ? static_cast<int32_t>(remaining) : kGapPlanes;
     const int32_t count = np * hw;
     const float* src = x + plane0 * hw;
-    for (int32_t e = threadIdx.x; e < count; e += kGapPlanes) {
-        const int32_t p = e / hw;
-        const int32_t i = e - p * hw;
-        tile[p * hw_pad + i] = src[e];
+    constexpr int kLoads = kGapPlanes * kGapMaxHw / kGapThreads;
+    float v[kLoads];
+    // every load is issued before the first value is used
+#pragma unroll
+    for (int k = 0; k < kLoads; ++k) {
+        const int32_t e = static_cast<int32_t>(threadIdx.x) + k * kGapThreads;
+        v[k] = e < count ? src[e] : 0.0f;
+    }
+#pragma unroll
+    for (int k = 0; k < kLoads; ++k) {
+        const int32_t e = static_cast<int32_t>(threadIdx.x) + k * kGapThreads;
+        const int32_t p = fast_div(e, div_hw);
+        if (e < count) tile[p * hw_pad + (e - p * hw)] = v[k];
     }
     __syncthreads();
     if (static_cast<int32_t>(threadIdx.x) < np) {
         float acc = 0.0f;
         const float* row = tile + threadIdx.x * hw_pad;
+#pragma unroll 8
         for (int32_t i = 0; i < hw; ++i) acc = __fadd_rn(acc, row[i]);
         y[plane0 + threadIdx.x] = __fdiv_rn(acc, static_cast<float>(hw));
     }
@@ -273,12 +286,13 @@ int32_t kxc_hip_global_avg_pool2d_f32(const float* x, float* y, int64_t n, int64
     KXC_HIP_REQUIRE(x && y, "kxc_hip_global_avg_pool2d_f32: NULL pointer");
     hipStream_t s = ResolveStream(stream);
     const int64_t hw = h * w;
-    if (hw <= 128) {
+    if (hw <= kGapMaxHw) {
         const int32_t hw_pad = static_cast<int32_t>(hw | 1);
         const int64_t blocks = CeilDiv(planes, kGapPlanes);
         KXC_HIP_REQUIRE(blocks <= kMaxGridX, "kxc_hip_global_avg_pool2d_f32: tensor too large");
-        const size_t lds = static_cast<size_t>(kGapPlanes) * hw_pad * sizeof(float);   // <= 33 KiB
-        gap_lds_kernel<<<NoteGrid(static_cast<int>(blocks)), NoteBlock(kGapPlanes), NoteLds(lds), s>>>(x, y, planes, static_cast<int32_t>(hw), hw_pad);
+        const size_t lds = static_cast<size_t>(kGapPlanes) * hw_pad * sizeof(float);   // <= 8.1 KiB
+        gap_lds_kernel<<<NoteGrid(static_cast<int>(blocks)), NoteBlock(kGapThreads), NoteLds(lds), s>>>(
+            x, y, planes, static_cast<int32_t>(hw), hw_pad, MakeFastDiv(static_cast<int32_t>(hw)));
         return CheckLaunch("global_avg_pool2d");
     }
     KXC_HIP_REQUIRE(planes <= kMaxGridX, "kxc_hip_global_avg_pool2d_f32: tensor too large");

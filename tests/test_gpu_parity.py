@@ -391,6 +391,12 @@ def test_gap_full_size(pkg, fast_orc, synth):
     assert_bit_exact(host(pkg.global_avg_pool2d(dev(x))), fast_orc.gap(x), "gap 2x2")
     x = synth.uniform((2, 3, 40, 40), 2022)            # large plane: wave reduction, different order
     assert_close(host(pkg.global_avg_pool2d(dev(x))), fast_orc.gap(x), what="gap 40x40")
+    # the staged kernel's limits: plane counts that do not fill a workgroup, planes of 1 and of 128 elements
+    for i, shape in enumerate([(1, 17, 1, 1), (3, 11, 8, 16), (1, 33, 9, 14), (2, 16, 1, 127), (1, 5, 2, 64)]):
+        x = synth.uniform(shape, 2030 + i)
+        assert_bit_exact(host(pkg.global_avg_pool2d(dev(x))), fast_orc.gap(x), "gap %s" % (shape,))
+    x = synth.uniform((1, 5, 3, 43), 2036)             # 129 elements: the first plane size of the wave reduction
+    assert_close(host(pkg.global_avg_pool2d(dev(x))), fast_orc.gap(x), what="gap 3x43")
 
 
 def test_dense_full_size(pkg, fast_orc, synth):
