@@ -120,12 +120,13 @@ def test_resnet18_hip_matches_oracle(synth):
 
 @pytest.mark.gpu
 def test_resnet18_hip_winograd_matches_oracle(synth):
-    """The same network with every 3x3 stride-1 convolution on the Winograd kernel (forced at this small batch):
-    logits within the fp32 tolerance, and the saved plan replays to the identical output."""
+    """The same network with every 3x3 stride-1 convolution on the Winograd kernel and every downsample on the
+    side lane (both forced at this small batch): logits within the fp32 tolerance, and the saved plan replays to
+    the identical output."""
     from gpu_util import assert_close
     with tempfile.TemporaryDirectory() as d:
         x, consts = _write_resnet_inputs(synth, d, 3, 2, 224)
-        out = run("resnet18", "hip", d, "2", "224", env={"KXC_HIP_WINOGRAD_MIN_WORK": "0"})
+        out = run("resnet18", "hip", d, "2", "224", env={"KXC_HIP_WINOGRAD_MIN_WORK": "0", "KXC_HIP_CONCURRENT_MIN_ELEMS": "0"})
         assert "execution plan replayed: 23 launches, identical output" in out
         plan = json.load(open(os.path.join(d, "plan.json")))
         assert sum(".winograd_f2k3" in n["kernel_symbol"] for n in plan["nodes"]) == 13
