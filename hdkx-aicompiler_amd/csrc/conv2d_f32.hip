@@ -426,12 +426,25 @@ conv_mfma_kernel(const ConvArgs a) {
 // Second half of a layer whose reduction was split over workgroups: y = relu(((p0 + p1) + ... ) + bias + residual),
 // the partial sums added in split order (deterministic), then the same epilogue as the unsplit kernel.
 __global__ void __launch_bounds__(256) conv_split_reduce_kernel(const ConvArgs a) {
-    const int64_t e = static_cast<int64_t>(blockIdx.x) * 256 + threadIdx.x;
-    if (e >= a.out_elems) return;
-    float v = a.partial[e];
-    for (int s = 1; s < a.gsplit; ++s) v = __fadd_rn(v, a.partial[static_cast<int64_t>(s) * a.out_elems + e]);
-    if (a.flags & KXC_HIP_CONV_BIAS) v = __fadd_rn(v, a.bias[(e / a.OHW) % a.O]);
-    if (a.flags & KXC_HIP_CONV_RESIDUAL) v = __fadd_rn(v, a.res[e]);
+    // (the matrix-core path takes outputs below 2 GiB only, so 32-bit element indices do)
+    const int32_t e = static_cast<int32_t>(blockIdx.x) * 256 + static_cast<int32_t>(threadIdx.x);
+    const int32_t total = static_cast<int32_t>(a.out_elems);
+    if (e >= total) return;
+    const float* const p = a.partial + e;
+    // every load of a batch of eight splits, the bias and the residual are in flight before the first addition
+    float bias = 0.0f, res = 0.0f;
+    if (a.flags & KXC_HIP_CONV_BIAS) { const int32_t plane = fast_div(e, a.div_ohw); bias = a.bias[plane % a.O]; }
+    if (a.flags & KXC_HIP_CONV_RESIDUAL) res = a.res[e];
+    float v = p[0];
+    for (int32_t s0 = 1; s0 < a.gsplit; s0 += 8) {
+        float t[8];
+#pragma unroll
+        for (int i = 0; i < 8; ++i) t[i] = s0 + i < a.gsplit ? p[static_cast<int64_t>(s0 + i) * total] : 0.0f;
+#pragma unroll
+        for (int i = 0; i < 8; ++i) v = s0 + i < a.gsplit ? __fadd_rn(v, t[i]) : v;
+    }
+    if (a.flags & KXC_HIP_CONV_BIAS) v = __fadd_rn(v, bias);
+    if (a.flags & KXC_HIP_CONV_RESIDUAL) v = __fadd_rn(v, res);
     if (a.flags & KXC_HIP_CONV_RELU) v = relu_sel(v);
     a.y[e] = v;
 }
