@@ -616,6 +616,13 @@ void Select(const ConvArgs& a, int kh, int kw, Choice* choice) {
     if (kh == 3 && a.sh == 2 && a.W >= 28 && a.W < 56 && a.O % 64 == 0 && a.M >= 8192) preferred = "mfma_k3x3_c4_o2x1_p8x1";
     if (kh == 3 && a.sh == 1 && a.W >= 56 && a.O % 64 == 0 && a.M >= 65536) preferred = "mfma_k3x3_c4_o1x2_p4x1";
     if (kh == 1 && a.W >= 56 && a.O % 64 == 0 && a.M >= 32768) preferred = "mfma_k1x1_c8_o1x2_p4x2";
+    if (kh == 7 && kw == 7) {
+        // first layer at small batch: fewer than 128 of the 64 x 256 tiles leave half the compute units idle
+        // (batch 1: 17.5 us; 32 x 128 tiles 10.8 us; batch 2: 18.1 us; 32 x 256 tiles 12.9 us; equal from batch 4 on)
+        const int64_t big_tiles = CeilDiv(a.M, 256) * CeilDiv(a.O, 64);
+        if (big_tiles < 64) preferred = "mfma_k7x7_t1_o1x1_p4x1";
+        else if (big_tiles < 128) preferred = "mfma_k7x7_t1_o1x1_p8x1";
+    }
     // Pass 0 takes the rule's variant (or the forced one).  Pass 1 takes the first table entry that fits,
     // unless that launch would leave most SIMDs idle (fewer than three waves per SIMD): then the reduction is
     // split inside the workgroup -- two ways on the 32x128 tile if that is enough, else four or eight ways on

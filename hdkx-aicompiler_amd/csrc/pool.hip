@@ -263,14 +263,21 @@ int32_t kxc_hip_pool2d_f32(const kxc_hip_pool2d_desc* desc, const float* x, floa
                       (d.h % 2) == 0 && d.ow == d.w / 2 && d.oh == d.h / 2 &&
                       (reinterpret_cast<uintptr_t>(x) & 15u) == 0 && (reinterpret_cast<uintptr_t>(y) & 15u) == 0;
     if (fast) {
-        constexpr int kRows = 4;
+        // four output rows per thread share input rows between them; a launch too small to give every compute
+        // unit a workgroup that way (batch 1) takes one row per thread and four times the threads instead
         const int32_t col_groups = d.ow / 4;
-        const int32_t row_groups = (d.oh + kRows - 1) / kRows;
+        const bool small = planes * ((d.oh + 3) / 4) * col_groups < 256LL * kBlock;   // 256 compute units
+        const int32_t rows = small ? 1 : 4;
+        const int32_t row_groups = (d.oh + rows - 1) / rows;
         const int64_t threads = planes * row_groups * col_groups;
         const int64_t blocks = CeilDiv(threads, kBlock);
         KXC_HIP_REQUIRE(blocks <= kMaxGridX, "kxc_hip_pool2d_f32: tensor too large");
-        maxpool3x3s2_kernel<kRows><<<NoteGrid(static_cast<int>(blocks)), NoteBlock(kBlock), NoteLds(0), s>>>(x, y, d.h, d.w, d.oh, d.ow, col_groups,
-                                                                               row_groups, threads);
+        if (small)
+            maxpool3x3s2_kernel<1><<<NoteGrid(static_cast<int>(blocks)), NoteBlock(kBlock), NoteLds(0), s>>>(
+                x, y, d.h, d.w, d.oh, d.ow, col_groups, row_groups, threads);
+        else
+            maxpool3x3s2_kernel<4><<<NoteGrid(static_cast<int>(blocks)), NoteBlock(kBlock), NoteLds(0), s>>>(
+                x, y, d.h, d.w, d.oh, d.ow, col_groups, row_groups, threads);
         return CheckLaunch("maxpool3x3s2");
     }
     if (desc->is_avg) pool_generic_kernel<true><<<NoteGrid(GridFor(total)), NoteBlock(kBlock), NoteLds(0), s>>>(x, y, d, total);

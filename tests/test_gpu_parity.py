@@ -357,6 +357,10 @@ def test_maxpool_full_size_bit_exact(pkg, fast_orc, synth):
     # every image against torch's max pool (exact for inputs above -1e30)
     want = torch.nn.functional.max_pool2d(xd, 3, 2, 1)
     assert torch.equal(got, want)
+    # small launches take one output row per thread instead of four: a batch-1 map and a ragged small one
+    for i, shape in enumerate([(1, 64, 112, 112), (2, 3, 14, 24), (1, 5, 2, 8)]):
+        xs = synth.uniform(shape, 2040 + i)
+        assert_bit_exact(host(pkg.pool2d(dev(xs), 3, 2, 1)), fast_orc.pool2d(xs, 3, 2, 1), "maxpool %s" % (shape,))
     # idempotence-like property: pooling a constant plane returns the constant
     c = torch.full((2, 3, 16, 16), -7.5, device="cuda")
     assert torch.equal(pkg.pool2d(c, 3, 2, 1), torch.full((2, 3, 8, 8), -7.5, device="cuda"))
