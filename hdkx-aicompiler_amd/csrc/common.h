@@ -69,6 +69,23 @@ __device__ __forceinline__ int fast_div(int x, FastDiv f) {
     return static_cast<int>((static_cast<uint64_t>(static_cast<uint32_t>(x)) * f.mul) >> f.shift);
 }
 
+// Reductions split over workgroups (both convolution kernels): every part writes raw partial outputs to
+// partial[split][total]; SplitReduce adds them in split order (deterministic) and applies the layer's epilogue,
+// y = relu(((p0 + p1) + ...) + bias[channel] + residual).
+struct SplitReduceArgs {
+    const float* partial;
+    const float* bias;
+    const float* res;
+    float* y;
+    int32_t gsplit, total, O;
+    uint32_t flags;            // KXC_HIP_CONV_BIAS | _RESIDUAL | _RELU
+    FastDiv div_ohw;
+};
+// Scratch for the partial outputs: one grow-only buffer per (device, stream), so that launches on different
+// streams never share one.  In steady state no call allocates.
+int32_t SplitScratch(hipStream_t stream, size_t bytes, float** out);
+int32_t LaunchSplitReduce(hipStream_t stream, const SplitReduceArgs& a);
+
 constexpr int64_t kMaxGridX = 2147483647LL;
 
 inline int64_t CeilDiv(int64_t a, int64_t b) { return (a + b - 1) / b; }

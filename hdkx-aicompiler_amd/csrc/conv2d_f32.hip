@@ -423,32 +423,6 @@ conv_mfma_kernel(const ConvArgs a) {
     }
 }
 
-// Second half of a layer whose reduction was split over workgroups: y = relu(((p0 + p1) + ... ) + bias + residual),
-// the partial sums added in split order (deterministic), then the same epilogue as the unsplit kernel.
-__global__ void __launch_bounds__(256) conv_split_reduce_kernel(const ConvArgs a) {
-    // (the matrix-core path takes outputs below 2 GiB only, so 32-bit element indices do)
-    const int32_t e = static_cast<int32_t>(blockIdx.x) * 256 + static_cast<int32_t>(threadIdx.x);
-    const int32_t total = static_cast<int32_t>(a.out_elems);
-    if (e >= total) return;
-    const float* const p = a.partial + e;
-    // every load of a batch of eight splits, the bias and the residual are in flight before the first addition
-    float bias = 0.0f, res = 0.0f;
-    if (a.flags & KXC_HIP_CONV_BIAS) { const int32_t plane = fast_div(e, a.div_ohw); bias = a.bias[plane % a.O]; }
-    if (a.flags & KXC_HIP_CONV_RESIDUAL) res = a.res[e];
-    float v = p[0];
-    for (int32_t s0 = 1; s0 < a.gsplit; s0 += 8) {
-        float t[8];
-#pragma unroll
-        for (int i = 0; i < 8; ++i) t[i] = s0 + i < a.gsplit ? p[static_cast<int64_t>(s0 + i) * total] : 0.0f;
-#pragma unroll
-        for (int i = 0; i < 8; ++i) v = s0 + i < a.gsplit ? __fadd_rn(v, t[i]) : v;
-    }
-    if (a.flags & KXC_HIP_CONV_BIAS) v = __fadd_rn(v, bias);
-    if (a.flags & KXC_HIP_CONV_RESIDUAL) v = __fadd_rn(v, res);
-    if (a.flags & KXC_HIP_CONV_RELU) v = relu_sel(v);
-    a.y[e] = v;
-}
-
 // ------------------------------------------------------------------------------------------
 // Direct kernel: the CPU loop nest, one thread per output element.
 // ------------------------------------------------------------------------------------------
@@ -665,31 +639,6 @@ void Select(const ConvArgs& a, int kh, int kw, Choice* choice) {
     }
 }
 
-// Scratch for the partial sums of a workgroup-split reduction: one grow-only buffer per (device, stream), so
-// that launches on different streams never share one.  Growing frees the old buffer (hipFree waits for the
-// device) and allocates a larger one; in steady state no call allocates.
-int32_t SplitScratch(hipStream_t stream, size_t bytes, float** out) {
-    struct Entry { int device; hipStream_t stream; float* ptr; size_t bytes; };
-    static std::mutex mu;
-    static std::vector<Entry> entries;
-    int dev = 0;
-    KXC_HIP_CALL(hipGetDevice(&dev), "hipGetDevice");
-    std::lock_guard<std::mutex> lock(mu);
-    Entry* e = nullptr;
-    for (Entry& it : entries)
-        if (it.device == dev && it.stream == stream) e = &it;
-    if (!e) { entries.push_back({dev, stream, nullptr, 0}); e = &entries.back(); }
-    if (e->bytes < bytes) {
-        if (e->ptr) KXC_HIP_CALL(hipFree(e->ptr), "hipFree(split scratch)");
-        e->ptr = nullptr; e->bytes = 0;
-        const size_t want = (bytes + (1u << 20) - 1) & ~static_cast<size_t>((1u << 20) - 1);
-        KXC_HIP_CALL(hipMalloc(reinterpret_cast<void**>(&e->ptr), want), "hipMalloc(split scratch)");
-        e->bytes = want;
-    }
-    *out = e->ptr;
-    return KXC_HIP_OK;
-}
-
 int32_t FillArgs(const kxc_hip_conv2d_desc* d, ConvArgs* a, const char* who) {
     KXC_HIP_REQUIRE(d != nullptr, "%s: desc is NULL", who);
     KXC_HIP_REQUIRE(d->n >= 0 && d->c > 0 && d->h > 0 && d->w > 0 && d->o > 0 && d->kh > 0 && d->kw > 0,
@@ -807,8 +756,10 @@ int32_t kxc_hip_conv2d_nchw_f32(const kxc_hip_conv2d_desc* desc, const float* x,
         hipLaunchKernelGGL(c.v->kernel, NoteGrid(grid), NoteBlock(dim3(64 * c.v->nw * c.v->ks)), NoteLds(c.lds_bytes), s, a);
         if (int32_t rc = CheckLaunch(c.v->name)) return rc;
         if (a.gsplit > 1) {
-            conv_split_reduce_kernel<<<NoteGrid(static_cast<int>(CeilDiv(total, 256))), NoteBlock(256), NoteLds(0), s>>>(a);
-            return CheckLaunch("conv_split_reduce");
+            SplitReduceArgs r;
+            r.partial = a.partial; r.bias = a.bias; r.res = a.res; r.y = a.y;
+            r.gsplit = a.gsplit; r.total = static_cast<int32_t>(total); r.O = a.O; r.flags = a.flags; r.div_ohw = a.div_ohw;
+            return LaunchSplitReduce(s, r);
         }
         return KXC_HIP_OK;
     }

@@ -55,7 +55,11 @@ struct WinoArgs {
     int32_t csteps;                  // C / 4
     int32_t t_groups, k_groups, num_units, units_per_xcd, k_fastest;
     uint32_t x_bytes, u_bytes, flags;
-    FastDiv div_ti, div_tw, div_kgroups, div_tgroups;
+    // gsplit > 1: the input channels are split over gsplit workgroups per tile (steps_per_split steps each), which
+    // write raw partial outputs to partial[split][N*O*OH*OW]; a second kernel adds them and applies the epilogue
+    int32_t gsplit, steps_per_split;
+    float* partial;
+    FastDiv div_ti, div_tw, div_kgroups, div_tgroups, div_gsplit;
 };
 
 __device__ __forceinline__ __amdgpu_buffer_rsrc_t make_rsrc(const void* p, uint32_t bytes) {
@@ -141,8 +145,10 @@ wino_kernel(const WinoArgs a) {
     const int tid = static_cast<int>(threadIdx.x) - kgroup * NTH;
     const int wave_k = wave / WT, wave_t = wave % WT;
     // Consecutive workgroups go to the 8 XCDs round-robin; each XCD (own L2) takes a contiguous run of units.
-    const int unit = (blockIdx.x & 7) * a.units_per_xcd + (blockIdx.x >> 3);
-    if (unit >= a.num_units || static_cast<int>(blockIdx.x >> 3) >= a.units_per_xcd) return;
+    const int slot = (blockIdx.x & 7) * a.units_per_xcd + (blockIdx.x >> 3);
+    if (slot >= a.num_units * a.gsplit || static_cast<int>(blockIdx.x >> 3) >= a.units_per_xcd) return;
+    const int unit = a.gsplit > 1 ? fast_div(slot, a.div_gsplit) : slot;
+    const int split = slot - unit * a.gsplit;
     int kg, tg;
     if (a.k_fastest) { tg = fast_div(unit, a.div_kgroups); kg = unit - tg * a.k_groups; }
     else { kg = fast_div(unit, a.div_tgroups); tg = unit - kg * a.t_groups; }
@@ -247,7 +253,9 @@ wino_kernel(const WinoArgs a) {
     float* const ub1 = ub0 + U_FLOATS;
     float* const vb0 = ub0 + 2 * U_FLOATS;
     float* const vb1 = vb0 + V_FLOATS;
-    const int s_lo = kgroup * (a.csteps / KS), s_hi = s_lo + a.csteps / KS;
+    // (the host never combines the split over workgroups with the split over wave groups)
+    const int s_lo = a.gsplit > 1 ? split * a.steps_per_split : kgroup * (a.csteps / KS);
+    const int s_hi = a.gsplit > 1 ? min(s_lo + a.steps_per_split, a.csteps) : s_lo + a.csteps / KS;
     const int last = s_hi - 1;
 
     // ---- prologue: weight tile and transformed input of the first step; raw input of the second in flight
@@ -333,13 +341,16 @@ wino_kernel(const WinoArgs a) {
     const int oh = 2 * ty, ow = 2 * tx;
     const bool row1 = oh + 1 < a.OH, col1 = ow + 1 < a.OW;
     const bool vec2 = (a.OW & 1) == 0;
-    const bool has_bias = (a.flags & KXC_HIP_CONV_BIAS) != 0;
-    const bool has_res = (a.flags & KXC_HIP_CONV_RESIDUAL) != 0;
-    const bool do_relu = (a.flags & KXC_HIP_CONV_RELU) != 0;
+    // (a part of a split reduction stores its raw output transform; the adding kernel applies the epilogue)
+    const uint32_t flags = a.gsplit > 1 ? 0u : a.flags;
+    const bool has_bias = (flags & KXC_HIP_CONV_BIAS) != 0;
+    const bool has_res = (flags & KXC_HIP_CONV_RESIDUAL) != 0;
+    const bool do_relu = (flags & KXC_HIP_CONV_RELU) != 0;
     const uint32_t y_bytes = static_cast<uint32_t>(a.N) * static_cast<uint32_t>(a.O) * static_cast<uint32_t>(a.OHW) * 4u;
-    const __amdgpu_buffer_rsrc_t yr = make_rsrc(a.y, y_bytes);
-    const __amdgpu_buffer_rsrc_t rr = make_rsrc(has_res ? a.res : a.y, has_res ? y_bytes : 0u);
-    const __amdgpu_buffer_rsrc_t br = make_rsrc(has_bias ? a.bias : a.y, has_bias ? static_cast<uint32_t>(a.O) * 4u : 0u);
+    float* const y_out = a.gsplit > 1 ? a.partial + static_cast<int64_t>(split) * (y_bytes / 4u) : a.y;
+    const __amdgpu_buffer_rsrc_t yr = make_rsrc(y_out, y_bytes);
+    const __amdgpu_buffer_rsrc_t rr = make_rsrc(has_res ? a.res : y_out, has_res ? y_bytes : 0u);
+    const __amdgpu_buffer_rsrc_t br = make_rsrc(has_bias ? a.bias : y_out, has_bias ? static_cast<uint32_t>(a.O) * 4u : 0u);
     const uint32_t rowb = static_cast<uint32_t>(a.OW) * 4u;
     const uint32_t rowmask = row1 ? 0u : kOob, colmask = col1 ? 0u : kOob;   // OR-ed into an offset: beyond the buffer
 
@@ -466,6 +477,17 @@ int64_t Tiles(const kxc_hip_conv2d_desc* d) {
     return static_cast<int64_t>(d->n) * CeilDiv(oh, 2) * CeilDiv(ow, 2);
 }
 
+// Launches that leave most compute units idle split the input channels over workgroups: the number of parts for
+// `units` workgroups of `csteps` steps.  Every part keeps at least four steps, the parts together stay below one
+// workgroup per compute unit, and the partial outputs stay small next to the caches (they are read back once).
+int GroupSplit(int64_t units, int csteps, int64_t out_elems) {
+    int split = 1;
+    while (split < 32 && units * split * 2 <= 256 && csteps / (split * 2) >= 4 &&
+           out_elems * static_cast<int64_t>(sizeof(float)) * split * 2 <= (8LL << 20))
+        split *= 2;
+    return split;
+}
+
 // Measured on MI355X: 64 x 32 workgroups (four waves) are the fastest shape once there is one per compute unit;
 // smaller launches run faster as twice as many 64 x 16 workgroups of two waves.
 const WinoVariant* SelectWino(const kxc_hip_conv2d_desc* d) {
@@ -473,11 +495,20 @@ const WinoVariant* SelectWino(const kxc_hip_conv2d_desc* d) {
         for (int i = 0; i < kNumWino; ++i)
             if (std::strcmp(e, kWino[i].name) == 0 && (kWino[i].ks == 1 || (d->c / 4) % kWino[i].ks == 0)) return &kWino[i];
     }
+    const int csteps = d->c / 4;
+    const int64_t oh = static_cast<int64_t>(d->h) + 2 * d->pad_h - 2, ow = static_cast<int64_t>(d->w) + 2 * d->pad_w - 2;
+    // Small launches (batch 1-8 of ResNet-18): 64 x 16 groups with the channels split over workgroups beat both
+    // the split inside the workgroup and the implicit-GEMM kernel (batch 1, 512 channels: 14.7 against 62.9 and
+    // 20.0 us).
+    const int64_t units_t1 = CeilDiv(Tiles(d), 16) * CeilDiv(d->o, 64);
+    if (GroupSplit(units_t1, csteps, static_cast<int64_t>(d->n) * d->o * oh * ow) > 1) {
+        for (int i = 0; i < kNumWino; ++i)
+            if (kWino[i].wk == 2 && kWino[i].wt == 1 && kWino[i].ks == 1) return &kWino[i];
+    }
     // 64 x 32 groups from one per compute unit on; below that twice as many 64 x 16 groups.  A launch that cannot
     // give every SIMD two waves (at most one 64 x 32 group per compute unit) and has a long reduction splits the
     // input channels over two groups of waves inside the workgroup instead.
     const int64_t units = CeilDiv(Tiles(d), 32) * CeilDiv(d->o, 64);
-    const int csteps = d->c / 4;
     const int wt = units < 256 ? 1 : 2;
     const int ks = (units <= 256 && csteps % 2 == 0 && csteps >= 32) ? 2 : 1;
     for (int i = 0; i < kNumWino; ++i)
@@ -493,10 +524,10 @@ int32_t kxc_hip_conv2d_winograd_supported(const kxc_hip_conv2d_desc* desc) { ret
 
 int32_t kxc_hip_conv2d_winograd_preferred(const kxc_hip_conv2d_desc* desc) {
     if (!Supported(desc)) return 0;
-    // A workgroup walks all input channels (c / 4 steps of ~0.7 us) whatever the launch size, while the
-    // implicit-GEMM kernel splits a long reduction over workgroups when the launch is small: Winograd pays from
-    // tiles * o >= 512 * c on (measured: batch 4 at 64 channels, batch 32 at 512 channels of ResNet-18).
-    int64_t factor = 512;
+    // Measured against the implicit-GEMM kernel on the ResNet-18 layers from batch 1 to 64: faster or equal
+    // everywhere once small launches split their channels over workgroups, so every supported shape takes it.
+    // KXC_HIP_WINOGRAD_MIN_WORK = f restricts it to tiles * o >= f * c.
+    int64_t factor = 0;
     if (const char* e = std::getenv("KXC_HIP_WINOGRAD_MIN_WORK")) factor = std::atoll(e);
     return Tiles(desc) * desc->o >= factor * desc->c ? 1 : 0;
 }
@@ -530,6 +561,7 @@ int32_t kxc_hip_conv2d_winograd_nchw_f32(const kxc_hip_conv2d_desc* desc, const 
     KXC_HIP_REQUIRE(!(desc->flags & KXC_HIP_CONV_RESIDUAL) || residual,
                     "kxc_hip_conv2d_winograd_nchw_f32: residual flag without residual");
     const WinoVariant* v = SelectWino(desc);
+    hipStream_t s = ResolveStream(stream);
     WinoArgs a;
     std::memset(&a, 0, sizeof(a));
     a.x = x; a.u = u; a.bias = bias; a.res = residual; a.y = y;
@@ -548,7 +580,27 @@ int32_t kxc_hip_conv2d_winograd_nchw_f32(const kxc_hip_conv2d_desc* desc, const 
     a.t_groups = static_cast<int32_t>(CeilDiv(a.NT, 16 * v->wt));
     a.k_groups = static_cast<int32_t>(CeilDiv(a.O, 32 * v->wk));
     a.num_units = a.t_groups * a.k_groups;
-    a.units_per_xcd = static_cast<int32_t>(CeilDiv(a.num_units, 8));
+    // Small launches split the input channels over workgroups (GroupSplit): each part writes its raw output
+    // transform (the transform is linear) to a scratch buffer, and a second kernel adds the parts in order and
+    // applies the epilogue.
+    a.gsplit = 1;
+    a.steps_per_split = a.csteps;
+    const int64_t out_elems = static_cast<int64_t>(a.N) * a.O * a.OHW;
+    if (v->ks == 1) {
+        int split = GroupSplit(a.num_units, a.csteps, out_elems);
+        if (const char* e = std::getenv("KXC_HIP_WINOGRAD_GSPLIT")) { const int f = std::atoi(e); if (f >= 1 && f <= a.csteps) split = f; }
+        if (split > 1) {
+            a.steps_per_split = static_cast<int32_t>(CeilDiv(a.csteps, split));
+            a.gsplit = static_cast<int32_t>(CeilDiv(a.csteps, a.steps_per_split));      // no empty part
+            if (a.gsplit > 1) {
+                if (int32_t rc = SplitScratch(s, static_cast<size_t>(a.gsplit) * out_elems * sizeof(float), &a.partial)) return rc;
+            } else {
+                a.steps_per_split = a.csteps;
+            }
+        }
+    }
+    a.div_gsplit = MakeFastDiv(a.gsplit);
+    a.units_per_xcd = static_cast<int32_t>(CeilDiv(static_cast<int64_t>(a.num_units) * a.gsplit, 8));
     // transformed weights of all output channels small next to an L2: neighbouring units share the input tile
     a.k_fastest = a.u_bytes <= (2u << 20) ? 1 : 0;
     if (const char* e = std::getenv("KXC_HIP_WINOGRAD_KFAST")) a.k_fastest = std::atoi(e);
@@ -572,8 +624,16 @@ int32_t kxc_hip_conv2d_winograd_nchw_f32(const kxc_hip_conv2d_desc* desc, const 
         }
     }
     hipLaunchKernelGGL(v->kernel, NoteGrid(dim3(static_cast<unsigned>(a.units_per_xcd * 8))),
-                       NoteBlock(dim3(64 * v->wk * v->wt * v->ks)), NoteLds(lds_bytes), ResolveStream(stream), a);
-    return CheckLaunch(v->name);
+                       NoteBlock(dim3(64 * v->wk * v->wt * v->ks)), NoteLds(lds_bytes), s, a);
+    if (int32_t rc = CheckLaunch(v->name)) return rc;
+    if (a.gsplit > 1) {
+        SplitReduceArgs r;
+        r.partial = a.partial; r.bias = bias; r.res = residual; r.y = y;
+        r.gsplit = a.gsplit; r.total = static_cast<int32_t>(out_elems); r.O = a.O; r.flags = a.flags;
+        r.div_ohw = MakeFastDiv(a.OHW);
+        return LaunchSplitReduce(s, r);
+    }
+    return KXC_HIP_OK;
 }
 
 }  // extern "C"

@@ -1,0 +1,71 @@
+// split_reduce.hip -- second half of a convolution whose reduction was split over workgroups, shared by the
+// implicit-GEMM and the Winograd kernel: the partial outputs of the parts are added in split order and the
+// layer's epilogue (bias, residual, ReLU) is applied; plus the scratch buffers the parts write to.
+#include <mutex>
+#include <vector>
+
+#include "common.h"
+
+namespace kxc_hip {
+
+namespace {
+
+__device__ __forceinline__ float relu_sel(float v) { return (v > 0.0f) ? v : 0.0f; }
+
+__global__ void __launch_bounds__(256) conv_split_reduce_kernel(const SplitReduceArgs a) {
+    const int32_t e = static_cast<int32_t>(blockIdx.x) * 256 + static_cast<int32_t>(threadIdx.x);
+    if (e >= a.total) return;
+    const float* const p = a.partial + e;
+    // every load of a batch of eight splits, the bias and the residual are in flight before the first addition
+    float bias = 0.0f, res = 0.0f;
+    if (a.flags & KXC_HIP_CONV_BIAS) { const int32_t plane = fast_div(e, a.div_ohw); bias = a.bias[plane % a.O]; }
+    if (a.flags & KXC_HIP_CONV_RESIDUAL) res = a.res[e];
+    float v = p[0];
+    for (int32_t s0 = 1; s0 < a.gsplit; s0 += 8) {
+        float t[8];
+#pragma unroll
+        for (int i = 0; i < 8; ++i) t[i] = s0 + i < a.gsplit ? p[static_cast<int64_t>(s0 + i) * a.total] : 0.0f;
+#pragma unroll
+        for (int i = 0; i < 8; ++i) v = s0 + i < a.gsplit ? __fadd_rn(v, t[i]) : v;
+    }
+    if (a.flags & KXC_HIP_CONV_BIAS) v = __fadd_rn(v, bias);
+    if (a.flags & KXC_HIP_CONV_RESIDUAL) v = __fadd_rn(v, res);
+    if (a.flags & KXC_HIP_CONV_RELU) v = relu_sel(v);
+    a.y[e] = v;
+}
+
+}  // namespace
+
+// A buffer that has been handed out stays allocated until the process ends, also after a larger one replaced it:
+// a captured graph may still hold its address.  Buffers double, so the retired ones add up to less than the
+// current one.
+int32_t SplitScratch(hipStream_t stream, size_t bytes, float** out) {
+    struct Entry { int device; hipStream_t stream; float* ptr; size_t bytes; };
+    static std::mutex mu;
+    static std::vector<Entry> entries;
+    int dev = 0;
+    KXC_HIP_CALL(hipGetDevice(&dev), "hipGetDevice");
+    std::lock_guard<std::mutex> lock(mu);
+    Entry* e = nullptr;
+    for (Entry& it : entries)
+        if (it.device == dev && it.stream == stream) e = &it;
+    if (!e) { entries.push_back({dev, stream, nullptr, 0}); e = &entries.back(); }
+    if (e->bytes < bytes) {
+        size_t want = e->bytes ? 2 * e->bytes : (static_cast<size_t>(1) << 20);
+        while (want < bytes) want *= 2;
+        float* fresh = nullptr;
+        KXC_HIP_CALL(hipMalloc(reinterpret_cast<void**>(&fresh), want), "hipMalloc(split scratch)");
+        e->ptr = fresh;          // the previous buffer is left allocated on purpose
+        e->bytes = want;
+    }
+    *out = e->ptr;
+    return KXC_HIP_OK;
+}
+
+int32_t LaunchSplitReduce(hipStream_t stream, const SplitReduceArgs& a) {
+    KXC_HIP_REQUIRE(a.gsplit >= 1 && a.total > 0 && a.O > 0 && a.partial && a.y, "split reduction: bad arguments");
+    conv_split_reduce_kernel<<<NoteGrid(static_cast<int>(CeilDiv(a.total, 256))), NoteBlock(256), NoteLds(0), stream>>>(a);
+    return CheckLaunch("conv_split_reduce");
+}
+
+}  // namespace kxc_hip

@@ -5,6 +5,8 @@ convolution / gemm kernels, all int8), within 1e-3 for the matrix-core kernels w
 differs.  Large (BASELINE-size) cases use properties that need no CPU run: agreement between the
 matrix-core kernel and the bit-exact direct kernel, linearity, batch independence.
 """
+import os
+
 import numpy as np
 import pytest
 import torch
@@ -228,6 +230,35 @@ def test_conv_winograd_variants(pkg, fast_orc, orc, synth, monkeypatch, variant)
                      orc.conv_chain(xi, wi, bi, 1, 1, None, True), variant + " on small integers")
 
 
+@pytest.mark.parametrize("forced", [None, "2", "3", "5"])
+def test_conv_winograd_channel_split_over_workgroups(pkg, fast_orc, orc, synth, monkeypatch, forced):
+    """Small launches split the input channels over workgroups (partial output transforms in a scratch buffer,
+    added in order by a second kernel that applies the epilogue): batch-1 ResNet layers with the automatic split,
+    a ragged shape with forced splits that leave a shorter last part, and small integers bit for bit."""
+    if forced:
+        monkeypatch.setenv("KXC_HIP_WINOGRAD_GSPLIT", forced)
+    shapes = [(1, 512, 7, 7, 512, 1), (1, 128, 28, 28, 128, 1)] if forced is None else [(2, 44, 9, 11, 72, 1), (1, 64, 6, 5, 40, 0)]
+    for (n, c, h, w, o, p) in shapes:
+        x = synth.uniform((n, c, h, w), 7400)
+        wt = synth.normal((o, c, 3, 3), 7401, float(np.sqrt(2.0 / (c * 9))))
+        b = synth.uniform((o,), 7402, -0.1, 0.1)
+        oh, ow = h + 2 * p - 2, w + 2 * p - 2
+        skip = synth.uniform((n, o, oh, ow), 7403)
+        assert pkg.conv2d_winograd_variant((n, c, h, w), (o, c, 3, 3), 1, p) == "winograd_f2k3_o2_t1"
+        u = pkg.conv2d_winograd_transform_weights((n, c, h, w), dev(wt), p)
+        got = host(pkg.conv2d_winograd(dev(x), u, wt.shape, dev(b), dev(skip), p, True))
+        assert_close(got, fast_orc.conv_chain(x, wt, b, 1, p, skip, True), what="split %s %s" % (forced, (n, c, h, w, o, p)))
+        got = host(pkg.conv2d_winograd(dev(x), u, wt.shape, None, None, p, False))
+        assert_close(got, fast_orc.conv_chain(x, wt, None, 1, p, None, False), what="split, no epilogue")
+    rng = np.random.default_rng(17)
+    xi = rng.integers(-3, 4, (1, 64, 9, 8)).astype(np.float32)
+    wi = (4 * rng.integers(-2, 3, (64, 64, 3, 3))).astype(np.float32)
+    bi = rng.integers(-5, 6, (64,)).astype(np.float32)
+    ui = pkg.conv2d_winograd_transform_weights(xi.shape, dev(wi), 1)
+    assert_bit_exact(host(pkg.conv2d_winograd(dev(xi), ui, wi.shape, dev(bi), None, 1, True)),
+                     orc.conv_chain(xi, wi, bi, 1, 1, None, True), "split on small integers")
+
+
 def test_conv_winograd_random_shapes_against_direct_kernel(pkg):
     """Seeded random geometries (batch, channels, height, width, output channels, padding; every epilogue mix):
     the Winograd kernel against the reference-order direct kernel on the same GPU tensors."""
@@ -254,7 +285,12 @@ def test_conv_winograd_unsupported_shapes_are_refused(pkg):
     assert not pkg.conv2d_winograd_supported((1, 8, 8, 8), (16, 8, 1, 1), 1, 0)        # filter size
     assert not pkg.conv2d_winograd_supported((1, 6, 8, 8), (16, 6, 3, 3), 1, 1)        # channels not a multiple of 4
     assert not pkg.conv2d_winograd_supported((1, 8, 8, 8), (16, 8, 3, 3), 1, 1, 2)     # dilation
-    assert not pkg.conv2d_winograd_preferred((1, 512, 7, 7), (512, 512, 3, 3))         # small launch, long reduction
+    assert pkg.conv2d_winograd_preferred((1, 512, 7, 7), (512, 512, 3, 3))             # small launches split their channels
+    os.environ["KXC_HIP_WINOGRAD_MIN_WORK"] = "512"
+    try:
+        assert not pkg.conv2d_winograd_preferred((1, 512, 7, 7), (512, 512, 3, 3))     # 16 blocks * 512 < 512 * 512
+    finally:
+        del os.environ["KXC_HIP_WINOGRAD_MIN_WORK"]
     assert pkg.conv2d_winograd_variant((1, 64, 56, 56), (64, 64, 3, 3)).endswith("_t1")  # small launches: smaller groups
     assert pkg.conv2d_winograd_preferred((64, 64, 56, 56), (64, 64, 3, 3))
     x = torch.zeros((1, 6, 8, 8), device="cuda"); u = torch.zeros((1024,), device="cuda")

@@ -90,8 +90,13 @@ def test_resnet18_hip_plan_without_gpu():
     with tempfile.TemporaryDirectory() as d:
         run("resnet18", "hip", d, "1", "224")
         one = json.load(open(os.path.join(d, "plan.json")))
-    # batch 1: only the 56x56 layer has enough 2x2 blocks per input channel for Winograd to pay
-    assert sum("winograd" in n["kernel_symbol"] for n in one["nodes"]) == 4
+    # batch 1: the same thirteen layers (small launches split their input channels over workgroups)
+    assert sum("winograd" in n["kernel_symbol"] for n in one["nodes"]) == 13
+    with tempfile.TemporaryDirectory() as d:
+        run("resnet18", "hip", d, "1", "224", env={"KXC_HIP_WINOGRAD_MIN_WORK": "512"})
+        few = json.load(open(os.path.join(d, "plan.json")))
+    # with the work threshold only the 56x56 layers have enough 2x2 blocks per input channel
+    assert sum("winograd" in n["kernel_symbol"] for n in few["nodes"]) == 4
 
 
 # ------------------------------------------------------------------ GPU
