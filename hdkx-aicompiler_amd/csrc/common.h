@@ -6,6 +6,7 @@
 #include <cstdarg>
 #include <cstdint>
 #include <cstdio>
+#include <mutex>
 #include <string>
 
 #include "kxc_hip.h"
@@ -82,8 +83,13 @@ struct SplitReduceArgs {
     FastDiv div_ohw;
 };
 // Scratch for the partial outputs: one grow-only buffer per (device, stream), so that launches on different
-// streams never share one.  In steady state no call allocates.
-int32_t SplitScratch(hipStream_t stream, size_t bytes, float** out);
+// streams never share one.  In steady state no call allocates.  The lease keeps other host threads that enqueue
+// on the same stream out until the adding kernel has been enqueued behind the parts (release it after that).
+struct SplitScratchLease {
+    float* ptr = nullptr;
+    std::unique_lock<std::mutex> lock;
+};
+int32_t AcquireSplitScratch(hipStream_t stream, size_t bytes, SplitScratchLease* lease);
 int32_t LaunchSplitReduce(hipStream_t stream, const SplitReduceArgs& a);
 
 constexpr int64_t kMaxGridX = 2147483647LL;

@@ -719,6 +719,7 @@ int32_t kxc_hip_conv2d_nchw_f32(const kxc_hip_conv2d_desc* desc, const float* x,
         a.gsplit = 1;
         a.cps = a.nchunks;
         a.out_elems = total;
+        SplitScratchLease lease;      // held until the adding kernel is enqueued
         {
             const int64_t waves = tiles * c.v->nw * c.v->ks;
             int split = 1;
@@ -731,7 +732,8 @@ int32_t kxc_hip_conv2d_nchw_f32(const kxc_hip_conv2d_desc* desc, const float* x,
                 a.cps = static_cast<int32_t>(CeilDiv(a.nchunks, split));
                 a.gsplit = static_cast<int32_t>(CeilDiv(a.nchunks, a.cps));      // no empty split
                 if (a.gsplit > 1) {
-                    if (int32_t rc = SplitScratch(s, static_cast<size_t>(a.gsplit) * total * sizeof(float), &a.partial)) return rc;
+                    if (int32_t rc = AcquireSplitScratch(s, static_cast<size_t>(a.gsplit) * total * sizeof(float), &lease)) return rc;
+                    a.partial = lease.ptr;
                 } else {
                     a.cps = a.nchunks;
                 }

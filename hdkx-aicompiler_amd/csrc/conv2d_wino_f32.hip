@@ -585,6 +585,7 @@ int32_t kxc_hip_conv2d_winograd_nchw_f32(const kxc_hip_conv2d_desc* desc, const 
     // applies the epilogue.
     a.gsplit = 1;
     a.steps_per_split = a.csteps;
+    SplitScratchLease lease;      // held until the adding kernel is enqueued
     const int64_t out_elems = static_cast<int64_t>(a.N) * a.O * a.OHW;
     if (v->ks == 1) {
         int split = GroupSplit(a.num_units, a.csteps, out_elems);
@@ -593,7 +594,8 @@ int32_t kxc_hip_conv2d_winograd_nchw_f32(const kxc_hip_conv2d_desc* desc, const 
             a.steps_per_split = static_cast<int32_t>(CeilDiv(a.csteps, split));
             a.gsplit = static_cast<int32_t>(CeilDiv(a.csteps, a.steps_per_split));      // no empty part
             if (a.gsplit > 1) {
-                if (int32_t rc = SplitScratch(s, static_cast<size_t>(a.gsplit) * out_elems * sizeof(float), &a.partial)) return rc;
+                if (int32_t rc = AcquireSplitScratch(s, static_cast<size_t>(a.gsplit) * out_elems * sizeof(float), &lease)) return rc;
+                a.partial = lease.ptr;
             } else {
                 a.steps_per_split = a.csteps;
             }

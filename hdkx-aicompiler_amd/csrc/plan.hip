@@ -59,9 +59,11 @@ struct kxc_hip_plan {
     // captured; later runs with the same argument pointers launch the instantiated graph
     bool graph_enabled = false;
     int eager_runs = 0;
+    hipStream_t eager_stream = nullptr;   // stream of the last eager run (scratch buffers are per stream)
     hipGraph_t graph = nullptr;
     hipGraphExec_t graph_exec = nullptr;
     std::vector<void*> graph_args;
+    hipStream_t graph_stream = nullptr;   // the graph is replayed only on the stream it was captured on
 };
 
 namespace {
@@ -642,6 +644,7 @@ void DropGraph(kxc_hip_plan* plan) {
     plan->graph_exec = nullptr;
     plan->graph = nullptr;
     plan->graph_args.clear();
+    plan->graph_stream = nullptr;
 }
 
 }  // namespace
@@ -653,14 +656,17 @@ int32_t kxc_hip_plan_run(kxc_hip_plan* plan, void** args, void* stream) {
     hipStream_t main_stream = reinterpret_cast<hipStream_t>(stream ? stream : static_cast<void*>(CurrentStream()));
     // Graph replay needs a real stream (the null stream cannot be captured) and one eager run before the
     // capture, so that everything that allocates lazily (split-reduction scratch, function attributes) exists.
+    // The captured kernels hold the addresses of that stream's scratch buffers, so a run on another stream
+    // captures again.
     if (!plan->graph_enabled || main_stream == nullptr) return EnqueueAll(plan, args, main_stream);
     const std::vector<void*> now(args, args + plan->num_args);
-    if (plan->graph_exec && now == plan->graph_args) {
+    if (plan->graph_exec && now == plan->graph_args && plan->graph_stream == main_stream) {
         KXC_HIP_CALL(hipGraphLaunch(plan->graph_exec, main_stream), "hipGraphLaunch");
         return KXC_HIP_OK;
     }
-    if (plan->eager_runs < 1) {
-        ++plan->eager_runs;
+    if (plan->eager_runs < 1 || plan->eager_stream != main_stream) {
+        plan->eager_runs = 1;
+        plan->eager_stream = main_stream;
         return EnqueueAll(plan, args, main_stream);
     }
     DropGraph(plan);
@@ -681,6 +687,7 @@ int32_t kxc_hip_plan_run(kxc_hip_plan* plan, void** args, void* stream) {
         return Fail(KXC_HIP_ERR_RUNTIME, "kxc_hip_plan_run: hipGraphInstantiate failed: %s", hipGetErrorString(inst));
     }
     plan->graph_args = now;
+    plan->graph_stream = main_stream;
     KXC_HIP_CALL(hipGraphLaunch(plan->graph_exec, main_stream), "hipGraphLaunch");     // the capture itself ran nothing
     return KXC_HIP_OK;
 }

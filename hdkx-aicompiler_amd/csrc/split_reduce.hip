@@ -1,6 +1,7 @@
 // split_reduce.hip -- second half of a convolution whose reduction was split over workgroups, shared by the
 // implicit-GEMM and the Winograd kernel: the partial outputs of the parts are added in split order and the
 // layer's epilogue (bias, residual, ReLU) is applied; plus the scratch buffers the parts write to.
+#include <memory>
 #include <mutex>
 #include <vector>
 
@@ -39,17 +40,23 @@ __global__ void __launch_bounds__(256) conv_split_reduce_kernel(const SplitReduc
 // A buffer that has been handed out stays allocated until the process ends, also after a larger one replaced it:
 // a captured graph may still hold its address.  Buffers double, so the retired ones add up to less than the
 // current one.
-int32_t SplitScratch(hipStream_t stream, size_t bytes, float** out) {
-    struct Entry { int device; hipStream_t stream; float* ptr; size_t bytes; };
+int32_t AcquireSplitScratch(hipStream_t stream, size_t bytes, SplitScratchLease* lease) {
+    struct Entry { int device; hipStream_t stream; float* ptr; size_t bytes; std::mutex in_use; };
     static std::mutex mu;
-    static std::vector<Entry> entries;
+    static std::vector<std::unique_ptr<Entry>> entries;      // entries are never removed: their addresses are stable
     int dev = 0;
     KXC_HIP_CALL(hipGetDevice(&dev), "hipGetDevice");
-    std::lock_guard<std::mutex> lock(mu);
     Entry* e = nullptr;
-    for (Entry& it : entries)
-        if (it.device == dev && it.stream == stream) e = &it;
-    if (!e) { entries.push_back({dev, stream, nullptr, 0}); e = &entries.back(); }
+    {
+        std::lock_guard<std::mutex> lock(mu);
+        for (auto& it : entries)
+            if (it->device == dev && it->stream == stream) e = it.get();
+        if (!e) {
+            entries.emplace_back(new Entry{dev, stream, nullptr, 0, {}});
+            e = entries.back().get();
+        }
+    }
+    std::unique_lock<std::mutex> in_use(e->in_use);
     if (e->bytes < bytes) {
         size_t want = e->bytes ? 2 * e->bytes : (static_cast<size_t>(1) << 20);
         while (want < bytes) want *= 2;
@@ -58,7 +65,8 @@ int32_t SplitScratch(hipStream_t stream, size_t bytes, float** out) {
         e->ptr = fresh;          // the previous buffer is left allocated on purpose
         e->bytes = want;
     }
-    *out = e->ptr;
+    lease->ptr = e->ptr;
+    lease->lock = std::move(in_use);
     return KXC_HIP_OK;
 }
 

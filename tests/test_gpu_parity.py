@@ -575,6 +575,16 @@ def test_plan_hip_graph_replay(pkg):
             plan.run([x] + consts + [other], stream.cuda_stream)
             stream.synchronize()
             assert_bit_exact(host(other), eager, "graph replay with a new output buffer %d" % replay)
+    # another stream: the captured kernels hold the first stream's scratch addresses, so the plan runs eagerly
+    # once and captures again there
+    second = torch.cuda.Stream()
+    with torch.cuda.stream(second):
+        for replay in range(4):
+            other.zero_()
+            second.synchronize()
+            plan.run([x] + consts + [other], second.cuda_stream)
+            second.synchronize()
+            assert_bit_exact(host(other), eager, "graph replay on a second stream %d" % replay)
     plan.enable_graph(False)
     plan.run([x] + consts + [out])
     torch.cuda.synchronize()
