@@ -207,7 +207,8 @@ def test_conv_winograd_exact_on_small_integers(pkg, orc):
         assert_bit_exact(host(pkg.conv2d_winograd(dev(x), u, wt.shape, dev(b), None, p, True)), want, str((n, c, h, w, o, p)))
 
 
-@pytest.mark.parametrize("variant", ["winograd_f2k3_o2_t2_ks2", "winograd_f2k3_o2_t1_ks2", "winograd_f2k3_o2_t4", "winograd_f2k3_o1_t2"])
+@pytest.mark.parametrize("variant", ["winograd_f2k3_o2_t2_ks2", "winograd_f2k3_o2_t1_ks2", "winograd_f2k3_o2_t4", "winograd_f2k3_o1_t4",
+                                     "winograd_f2k3_o1_t2", "winograd_f2k3_o2_t2"])
 def test_conv_winograd_variants(pkg, fast_orc, orc, synth, monkeypatch, variant):
     """Every workgroup shape of the Winograd kernel, forced: the two-group channel split (accumulators added through
     LDS) and the larger / smaller tiles, on a ragged shape against the oracle and bit-exact on small integers."""
