@@ -14,7 +14,10 @@ namespace {
 __device__ __forceinline__ float relu_sel(float v) { return (v > 0.0f) ? v : 0.0f; }
 
 __global__ void __launch_bounds__(256) conv_split_reduce_kernel(const SplitReduceArgs a) {
-    const int32_t e = static_cast<int32_t>(blockIdx.x) * 256 + static_cast<int32_t>(threadIdx.x);
+    // XCD x (blockIdx % 8) takes the x-th eighth of the elements, like the kernels that wrote the parts
+    const int32_t per_xcd = static_cast<int32_t>(gridDim.x >> 3);
+    const int32_t block = static_cast<int32_t>(blockIdx.x & 7) * per_xcd + static_cast<int32_t>(blockIdx.x >> 3);
+    const int32_t e = block * 256 + static_cast<int32_t>(threadIdx.x);
     if (e >= a.total) return;
     const float* const p = a.partial + e;
     // every load of a batch of eight splits, the bias and the residual are in flight before the first addition
@@ -72,7 +75,7 @@ int32_t AcquireSplitScratch(hipStream_t stream, size_t bytes, SplitScratchLease*
 
 int32_t LaunchSplitReduce(hipStream_t stream, const SplitReduceArgs& a) {
     KXC_HIP_REQUIRE(a.gsplit >= 1 && a.total > 0 && a.O > 0 && a.partial && a.y, "split reduction: bad arguments");
-    conv_split_reduce_kernel<<<NoteGrid(static_cast<int>(CeilDiv(a.total, 256))), NoteBlock(256), NoteLds(0), stream>>>(a);
+    conv_split_reduce_kernel<<<NoteGrid(static_cast<int>(CeilDiv(CeilDiv(a.total, 256), 8) * 8)), NoteBlock(256), NoteLds(0), stream>>>(a);
     return CheckLaunch("conv_split_reduce");
 }
 
