@@ -46,15 +46,24 @@ __global__ void __launch_bounds__(kBlock) relu_scalar_kernel(const float* __rest
 template <int OP, bool RELU>
 __global__ void __launch_bounds__(kBlock) same_shape_kernel(const float* __restrict__ a, const float* __restrict__ b,
                                                             float* __restrict__ y, int64_t n4, int64_t n) {
+    // two 16-byte vectors of each operand per thread and trip, all four loads issued before the first use
     const int64_t stride = static_cast<int64_t>(gridDim.x) * kBlock;
-    for (int64_t i = static_cast<int64_t>(blockIdx.x) * kBlock + threadIdx.x; i < n4; i += stride) {
-        const float4 va = reinterpret_cast<const float4*>(a)[i];
-        const float4 vb = reinterpret_cast<const float4*>(b)[i];
+    auto op4 = [](const float4& va, const float4& vb) {
         float4 r;
         r.x = binop<OP>(va.x, vb.x); r.y = binop<OP>(va.y, vb.y);
         r.z = binop<OP>(va.z, vb.z); r.w = binop<OP>(va.w, vb.w);
         if (RELU) { r.x = relu_sel(r.x); r.y = relu_sel(r.y); r.z = relu_sel(r.z); r.w = relu_sel(r.w); }
-        reinterpret_cast<float4*>(y)[i] = r;
+        return r;
+    };
+    for (int64_t i = static_cast<int64_t>(blockIdx.x) * kBlock + threadIdx.x; i < n4; i += 2 * stride) {
+        const int64_t j = i + stride;
+        const bool second = j < n4;
+        const float4 va0 = reinterpret_cast<const float4*>(a)[i];
+        const float4 vb0 = reinterpret_cast<const float4*>(b)[i];
+        const float4 va1 = second ? reinterpret_cast<const float4*>(a)[j] : va0;
+        const float4 vb1 = second ? reinterpret_cast<const float4*>(b)[j] : vb0;
+        reinterpret_cast<float4*>(y)[i] = op4(va0, vb0);
+        if (second) reinterpret_cast<float4*>(y)[j] = op4(va1, vb1);
     }
     const int64_t tail = n4 * 4 + static_cast<int64_t>(blockIdx.x) * kBlock + threadIdx.x;
     if (blockIdx.x == 0 && tail < n) {
@@ -150,7 +159,7 @@ inline bool Aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 
 template <int OP>
 int32_t LaunchSameShape(const float* a, const float* b, float* y, int64_t n, bool relu, hipStream_t s) {
     const int64_t n4 = (Aligned16(a) && Aligned16(b) && Aligned16(y)) ? n / 4 : 0;
-    const int grid = GridFor(n4 > 0 ? n4 : n);
+    const int grid = GridFor(n4 > 0 ? (n4 + 1) / 2 : n);      // the vector kernel takes two vectors per thread
     if (n4 == 0) {
         // unaligned: go through the generic kernel with a flat 1-d description
         BroadcastDims d{};

@@ -199,11 +199,14 @@ def relu(x):
     return y
 
 
-def binary(op, a, b, relu=False):
+def binary(op, a, b, relu=False, out=None):
     import torch
     _need(a, torch.float32, "a"); _need(b, torch.float32, "b")
     shape = torch.broadcast_shapes(a.shape, b.shape)
-    y = torch.empty(shape, dtype=torch.float32, device=a.device)
+    y = out if out is not None else torch.empty(shape, dtype=torch.float32, device=a.device)
+    _need(y, torch.float32, "out")
+    if tuple(y.shape) != tuple(shape):
+        raise ValueError("binary: out has shape %s, expected %s" % (tuple(y.shape), tuple(shape)))
     sa = (C.c_int64 * max(1, a.dim()))(*a.shape); sb = (C.c_int64 * max(1, b.dim()))(*b.shape)
     _check(lib().kxc_hip_broadcast_binary_f32(C.c_int32(op), _p(a), sa, C.c_int32(a.dim()), _p(b), sb,
                                               C.c_int32(b.dim()), _p(y), C.c_int32(int(relu)), _stream()))
@@ -245,22 +248,28 @@ def pool2d(x, k, s, pad, ceil_mode=False, avg=False, out=None):
     return y
 
 
-def global_avg_pool2d(x):
+def global_avg_pool2d(x, out=None):
     import torch
     _need(x, torch.float32, "x")
     n, c, h, w = x.shape
-    y = torch.empty((n, c, 1, 1), dtype=torch.float32, device=x.device)
+    y = out if out is not None else torch.empty((n, c, 1, 1), dtype=torch.float32, device=x.device)
+    _need(y, torch.float32, "out")
+    if y.numel() != n * c:
+        raise ValueError("global_avg_pool2d: out has %d elements, expected %d" % (y.numel(), n * c))
     _check(lib().kxc_hip_global_avg_pool2d_f32(_p(x), _p(y), C.c_int64(n), C.c_int64(c), C.c_int64(h), C.c_int64(w),
                                                _stream()))
     return y
 
 
-def gemm(a, b, c=None, alpha=1.0, beta=1.0, transB=1):
+def gemm(a, b, c=None, alpha=1.0, beta=1.0, transB=1, out=None):
     import torch
     _need(a, torch.float32, "a"); _need(b, torch.float32, "b"); _need(c, torch.float32, "c")
     m, k = a.shape
     n = b.shape[0] if transB else b.shape[1]
-    y = torch.empty((m, n), dtype=torch.float32, device=a.device)
+    y = out if out is not None else torch.empty((m, n), dtype=torch.float32, device=a.device)
+    _need(y, torch.float32, "out")
+    if y.numel() != m * n:
+        raise ValueError("gemm: out has %d elements, expected %d" % (y.numel(), m * n))
     _check(lib().kxc_hip_gemm_f32(_p(a), _p(b), _p(c), _p(y), C.c_int64(m), C.c_int64(n), C.c_int64(k),
                                   C.c_float(alpha), C.c_float(beta), C.c_int32(transB),
                                   C.c_int64(c.numel() if c is not None else 0), _stream()))
