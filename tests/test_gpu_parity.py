@@ -345,6 +345,31 @@ def test_plan_winograd_node_transforms_constants_once(pkg, synth, fast_orc):
     assert_bit_exact(host(y2), host(y), "deserialised winograd plan")
 
 
+@pytest.mark.parametrize("shape", [(1, 64, 56, 56, 128, 2), (1, 256, 14, 14, 512, 2), (2, 8, 5, 7, 40, 1), (3, 24, 9, 6, 33, 2),
+                                   (1, 40, 7, 7, 100, 3), (2, 272, 6, 6, 48, 1)], ids=lambda s: "x".join(map(str, s)))
+def test_conv1x1_small_launch_kernel(pkg, fast_orc, orc, synth, shape):
+    """Unpadded 1x1 filters on small launches (the downsample convolutions at batch 1-16) take a kernel of their
+    own: four or eight waves split the input channels and feed the matrix cores straight from memory.  Channel
+    counts that leave a short last batch of loads, output channels and pixels that do not fill a 32 x 32 tile,
+    strides 1-3, every epilogue mix."""
+    n, c, h, w, o, stride = shape
+    assert pkg.conv2d_variant((n, c, h, w), (o, c, 1, 1), stride, 0) == "mfma_k1x1_small"
+    x = synth.uniform((n, c, h, w), 7500)
+    wt = synth.normal((o, c, 1, 1), 7501, float(np.sqrt(2.0 / c)))
+    b = synth.uniform((o,), 7502, -0.1, 0.1)
+    oh, ow = (h - 1) // stride + 1, (w - 1) // stride + 1
+    skip = synth.uniform((n, o, oh, ow), 7503)
+    for (bias, res, relu) in [(b, None, False), (b, skip, True), (None, None, True), (None, skip, False)]:
+        got = host(pkg.conv2d(dev(x), dev(wt), None if bias is None else dev(bias), None if res is None else dev(res),
+                              stride, 0, 1, relu))
+        assert_close(got, fast_orc.conv_chain(x, wt, bias, stride, 0, res, relu), what="1x1 small %s" % (shape,))
+    rng = np.random.default_rng(19)
+    xi = rng.integers(-3, 4, (n, c, h, w)).astype(np.float32)
+    wi = rng.integers(-2, 3, (o, c, 1, 1)).astype(np.float32)
+    assert_bit_exact(host(pkg.conv2d(dev(xi), dev(wi), None, None, stride, 0, 1, False)),
+                     orc.conv_chain(xi, wi, None, stride, 0, None, False), "1x1 small on small integers")
+
+
 def test_conv_dilation(pkg, orc, synth):
     x = synth.uniform((1, 8, 20, 20), 300); w = synth.uniform((32, 8, 3, 3), 301)
     want = orc.conv2d(x, w, 1, 2, 2)
