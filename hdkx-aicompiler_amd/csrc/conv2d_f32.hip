@@ -702,6 +702,10 @@ void Select(const ConvArgs& a, int kh, int kw, Choice* choice) {
                     if (!split[k].v) continue;
                     *choice = split[k];
                     if (split_waves[k] >= 2560) break;      // enough waves: stop splitting further
+                    // stride 2: the 32 x 64 tiles of the deeper splits stage their patches badly; two wave groups
+                    // on the 32 x 128 tile plus the split over workgroups win from batch 1 to 16 (batch 8,
+                    // 128 -> 256 channels at 28 x 28: 20.5 against 31.5 us)
+                    if (kh == 3 && a.sh == 2) break;
                 }
             }
         }
