@@ -477,14 +477,26 @@ int64_t Tiles(const kxc_hip_conv2d_desc* d) {
     return static_cast<int64_t>(d->n) * CeilDiv(oh, 2) * CeilDiv(ow, 2);
 }
 
-// Launches that leave most compute units idle split the input channels over workgroups: the number of parts for
-// `units` workgroups of `csteps` steps.  Every part keeps at least four steps, the parts together stay below one
-// workgroup per compute unit, and the partial outputs stay small next to the caches (they are read back once).
+// Launches that leave compute units idle split the input channels over workgroups: the number of parts for
+// `units` 64 x 16 workgroups of `csteps` steps.  Two regimes, both measured on the ResNet-18 layers:
+//  * tiny launches (batch 1-4): parts of at least four steps while all parts together stay below one workgroup
+//    per compute unit (batch 1, 512 channels: 8 units -> 32 parts, 62.9 -> 14.7 us);
+//  * up to 256 units with a long reduction (64 steps and more; batch 8-32 of the 256- and 512-channel layers):
+//    parts of at least sixteen steps up to four workgroups per compute unit, which is what fills every SIMD with
+//    two waves (batch 16, 512 channels: 128 units -> 8 parts, 55.7 -> 39.6 us; the split inside the workgroup: 66).
+// The partial outputs (read back once by the adding kernel) stay below 16 MiB.
 int GroupSplit(int64_t units, int csteps, int64_t out_elems) {
     int split = 1;
-    while (split < 32 && units * split * 2 <= 256 && csteps / (split * 2) >= 4 &&
-           out_elems * static_cast<int64_t>(sizeof(float)) * split * 2 <= (8LL << 20))
-        split *= 2;
+    while (split < 32) {
+        const int next = split * 2;
+        const int64_t groups = units * next;
+        const int steps = csteps / next;
+        const bool tiny = groups <= 256 && steps >= 4;
+        const bool filling = units <= 256 && groups <= 1024 && csteps >= 64 && steps >= 16;
+        if (!(tiny || filling)) break;
+        if (out_elems * static_cast<int64_t>(sizeof(float)) * next > (16LL << 20)) break;
+        split = next;
+    }
     return split;
 }
 
