@@ -166,15 +166,19 @@ wino_kernel(const WinoArgs a) {
         const int tile = t0 + tile_l;
         const int n = fast_div(tile, a.div_ti), rem = tile - n * a.TI;
         const int ty = fast_div(rem, a.div_tw), tx = rem - ty * a.TW;
+        // (row and column validity are tested once each and combined per element: no per-element products)
+        const int iw0 = 2 * tx - a.pw;
+        uint32_t colmask[4];
+#pragma unroll
+        for (int j = 0; j < 4; ++j) colmask[j] = (iw0 + j >= 0 && iw0 + j < a.W) ? 0u : kOob;
+        const uint32_t plane = static_cast<uint32_t>((n * a.C + cl) * a.H);
 #pragma unroll
         for (int r = 0; r < 3; ++r) {
             const int ih = 2 * ty - a.ph + half + r;
+            const uint32_t rowmask = (tile < a.NT && ih >= 0 && ih < a.H) ? 0u : kOob;
+            const uint32_t row = ((plane + static_cast<uint32_t>(ih)) * static_cast<uint32_t>(a.W) + static_cast<uint32_t>(iw0)) * 4u;
 #pragma unroll
-            for (int j = 0; j < 4; ++j) {
-                const int iw = 2 * tx - a.pw + j;
-                const bool ok = tile < a.NT && ih >= 0 && ih < a.H && iw >= 0 && iw < a.W;
-                goff[i][r * 4 + j] = ok ? static_cast<uint32_t>(((n * a.C + cl) * a.H + ih) * a.W + iw) * 4u : kOob;
-            }
+            for (int j = 0; j < 4; ++j) goff[i][r * 4 + j] = (rowmask | colmask[j]) != 0u ? kOob : row + 4u * j;
         }
         vdst[i] = ((cl * WT + tile_l / 16) * 4 + 2 * half) * 64 + (tile_l % 16) * 4;
     }
