@@ -195,7 +195,7 @@ def main():
         "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "ms_per_step": round(ms_per_step, 4),
         "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "f32", "data": "synthetic",
         "config": {"workload": "ResNet-18 fp32 inference, batch %d, input [%d,3,224,224], BN folded, seeded Kaiming weights "
-                               "(BASELINE configs[%d])" % (batch, batch, 3 if batch == 64 else 2),
+                               "(benchmark configuration %d)" % (batch, batch, 4 if batch == 64 else 3),
                    "compiled_by": "C++ host layer, Compiler::Compile(Relay graph, target hip)",
                    "launches_per_step": len(info["launches"]), "workspace_bytes": info["workspace_bytes"]},
         "end_to_end_tflops": round(flop_step / (ms_per_step * 1e-3) / 1e12, 3),
@@ -261,7 +261,7 @@ def bench_conv_layers(torch, pkg, synth, dev, batch):
 
 
 def bench_ops(torch, pkg, synth, dev):
-    """BASELINE configs[1]: the bandwidth-bound operators at ResNet-18 shapes, algorithmic bytes / time."""
+    """Benchmark configuration 2: the bandwidth-bound operators at ResNet-18 shapes, algorithmic bytes / time."""
     rows = []
     x = dev(synth.uniform((64, 64, 112, 112), 2000))
     y = torch.empty((64, 64, 56, 56), device="cuda")
@@ -317,7 +317,7 @@ def bench_batch1(torch, pkg, hostapi, synth, dev):
 
 
 def bench_int8(torch, pkg, synth, dev, np, batch):
-    """BASELINE configs[4]: quantised ResNet-18, batch 64, int8 matrix cores (calibrated on the same batch)."""
+    """Benchmark configuration 5: quantised ResNet-18, batch 64, int8 matrix cores (calibrated on the same batch)."""
     qr = importlib.import_module("hdkx-aicompiler_amd.qresnet18")
     consts = synth.resnet18_consts(5)
     x = dev(synth.resnet18_input(5, batch))

@@ -148,7 +148,7 @@ int main(int argc, char** argv) {
         all << "#include <stdint.h>\n#include <math.h>\n";
         struct Case { std::string name; Function f; };
         std::vector<Case> cases;
-        // BASELINE config 1
+        // benchmark configuration 1
         cases.push_back({"kxc_ref_conv_cfg1", ConvCase(1, 64, 56, 56, 64, 3, 1, 1, true, true)});
         // the reference test's own tiny shapes (test/op_numeric_llvm_test.cpp)
         cases.push_back({"kxc_ref_conv_kat", ConvCase(1, 1, 3, 3, 1, 2, 1, 0, false, false)});

@@ -3,7 +3,7 @@ them (test/onnx_importer_test.cpp:146-179) and host<->device shuttling."""
 import numpy as np
 import torch
 
-FP32_TOL = 1e-3     # BASELINE: max relative error 1e-3 for fp32 operators and end-to-end logits
+FP32_TOL = 1e-3     # the stated tolerance: max relative error 1e-3 for fp32 operators and end-to-end logits
 
 
 def dev(a):

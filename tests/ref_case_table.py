@@ -42,7 +42,7 @@ CASES = {
 def case_inputs(name):
     shapes, _ = CASES[name]
     base = 7000 + 10 * sorted(CASES).index(name)
-    if name == "kxc_ref_conv_cfg1":  # BASELINE configuration 1, seeds 1000..1002
+    if name == "kxc_ref_conv_cfg1":  # benchmark configuration 1, seeds 1000..1002
         return [synth.uniform(shapes[0], 1000), synth.normal(shapes[1], 1001, float(np.sqrt(2.0 / 576))),
                 synth.uniform(shapes[2], 1002, -0.1, 0.1)]
     return [synth.uniform(s, base + t) for t, s in enumerate(shapes)]

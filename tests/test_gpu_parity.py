@@ -2,7 +2,7 @@
 
 Bit-exact where the arithmetic allows it (max pool, global average pool, elementwise, the direct
 convolution / gemm kernels, all int8), within 1e-3 for the matrix-core kernels whose reduction order
-differs.  Large (BASELINE-size) cases use properties that need no CPU run: agreement between the
+differs.  Large (full-size) cases use properties that need no CPU run: agreement between the
 matrix-core kernel and the bit-exact direct kernel, linearity, batch independence.
 """
 import os
@@ -300,7 +300,7 @@ def test_conv_winograd_unsupported_shapes_are_refused(pkg):
 
 
 def test_conv_winograd_full_batch_properties(pkg, synth):
-    """BASELINE-size layers (batch 64): Winograd vs the implicit-GEMM kernel on the GPU, linearity in the weights
+    """Full-size layers (batch 64): Winograd vs the implicit-GEMM kernel on the GPU, linearity in the weights
     and batch independence."""
     for (c, hw, o) in [(64, 56, 64), (512, 7, 512)]:
         x = dev(synth.uniform((64, c, hw, hw), 7100))
@@ -392,7 +392,7 @@ def test_conv_exact_on_small_integers(pkg, orc):
 
 
 def test_conv_full_batch_properties(pkg, synth):
-    """BASELINE-size layer (batch 64): matrix-core kernel vs the bit-exact direct kernel on the GPU,
+    """Full-size layer (batch 64): matrix-core kernel vs the bit-exact direct kernel on the GPU,
     plus linearity in the weights and batch independence."""
     x = dev(synth.uniform((64, 64, 56, 56), 4100))
     w1 = dev(synth.normal((64, 64, 3, 3), 4101, float(np.sqrt(2.0 / 576))))
@@ -408,7 +408,7 @@ def test_conv_full_batch_properties(pkg, synth):
     assert_close(host(one), host(fast[17:18]), tol=1e-4, what="batch independence")
 
 
-# ------------------------------------------------------------------ pooling / elementwise at BASELINE sizes
+# ------------------------------------------------------------------ pooling / elementwise at full sizes
 def test_maxpool_full_size_bit_exact(pkg, fast_orc, synth):
     x = synth.uniform((64, 64, 112, 112), 2000)
     xd = dev(x)
@@ -549,7 +549,7 @@ def test_resnet18_small_image(pkg, fast_orc):
 
 
 def test_resnet18_batch1_224(pkg, fast_orc):
-    """BASELINE configuration 3: full ResNet-18 at batch 1, logits within 1e-3 of the CPU path."""
+    """Benchmark configuration 3: full ResNet-18 at batch 1, logits within 1e-3 of the CPU path."""
     x, consts, got, info = _run_plan(pkg, 1, 224, 3)
     want = fast_orc.resnet18(x, consts)
     assert_close(got, want, what="resnet18 224 logits", floor="scale")
@@ -557,7 +557,7 @@ def test_resnet18_batch1_224(pkg, fast_orc):
 
 
 def test_resnet18_batch64_properties(pkg, fast_orc):
-    """BASELINE configuration 4 at full size: image 0 and image 63 of the batch against the CPU path
+    """Benchmark configuration 4 at full size: image 0 and image 63 of the batch against the CPU path
     run on those images alone (the graph is independent per image)."""
     import importlib
     synth = importlib.import_module("hdkx-aicompiler_amd.synth")
