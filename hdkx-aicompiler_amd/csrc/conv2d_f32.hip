@@ -702,10 +702,11 @@ void Select(const ConvArgs& a, int kh, int kw, Choice* choice) {
                     if (!split[k].v) continue;
                     *choice = split[k];
                     if (split_waves[k] >= 2560) break;      // enough waves: stop splitting further
-                    // stride 2: the 32 x 64 tiles of the deeper splits stage their patches badly; two wave groups
-                    // on the 32 x 128 tile plus the split over workgroups win from batch 1 to 16 (batch 8,
-                    // 128 -> 256 channels at 28 x 28: 20.5 against 31.5 us)
-                    if (kh == 3 && a.sh == 2) break;
+                    // 3x3: two wave groups on the 32 x 128 tile plus the split over workgroups beat the deeper
+                    // splits on 32 x 64 tiles from batch 1 to 16, at stride 2 (batch 8, 128 -> 256 channels at
+                    // 28 x 28: 20.5 against 31.5 us) and at stride 1 (batch 1, 256 channels at 14 x 14: 12.6
+                    // against 19.8 us with the adding kernel; batch 4, 512 channels at 7 x 7: 23.8 against 37.9)
+                    if (kh == 3) break;
                 }
             }
         }
