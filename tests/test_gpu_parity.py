@@ -281,6 +281,35 @@ def test_conv_winograd_random_shapes_against_direct_kernel(pkg):
         assert_close(host(got), host(want), what="case %d: n=%d c=%d h=%d w=%d o=%d p=%d" % (case, n, c, h, w, o, p))
 
 
+def test_conv_random_shapes_against_direct_kernel(pkg):
+    """Seeded random geometries over every filter size the matrix-core kernels take (1x1, 3x3, 7x7; strides 1-3,
+    paddings 0-3, dilations 1-2; ragged channel, output-channel and pixel counts; every epilogue mix): whatever
+    kernel the library selects -- tiled, split over wave groups or workgroups, the small-launch 1x1 kernel --
+    against the reference-order direct kernel on the same GPU tensors."""
+    rng = np.random.default_rng(20240707)
+    seen = set()
+    for case in range(60):
+        k = int(rng.choice([1, 1, 3, 3, 3, 7]))
+        n = int(rng.integers(1, 5)); c = int(rng.choice([3, 8, 16, 24, 40, 64, 96, 128, 200, 256])); o = int(rng.integers(8, 200))
+        h = int(rng.integers(4, 40)); w = int(rng.integers(4, 40))
+        stride = int(rng.integers(1, 4)); p = int(rng.integers(0, 4)); dil = int(rng.integers(1, 3)) if k == 3 else 1
+        if k == 1:
+            p = int(rng.choice([0, 0, 1]))
+        if h + 2 * p < dil * (k - 1) + 1 or w + 2 * p < dil * (k - 1) + 1:
+            continue
+        x = torch.from_numpy(rng.uniform(-1, 1, (n, c, h, w)).astype(np.float32)).cuda()
+        wt = torch.from_numpy((rng.standard_normal((o, c, k, k)) * np.sqrt(2.0 / (k * k * c))).astype(np.float32)).cuda()
+        b = torch.from_numpy(rng.uniform(-0.1, 0.1, (o,)).astype(np.float32)).cuda() if case % 2 == 0 else None
+        oh = (h + 2 * p - (dil * (k - 1) + 1)) // stride + 1; ow = (w + 2 * p - (dil * (k - 1) + 1)) // stride + 1
+        r = torch.from_numpy(rng.uniform(-1, 1, (n, o, oh, ow)).astype(np.float32)).cuda() if case % 3 == 0 else None
+        relu = case % 4 != 3
+        seen.add(pkg.conv2d_variant((n, c, h, w), (o, c, k, k), stride, p, dil))
+        got = pkg.conv2d(x, wt, b, r, stride, p, dil, relu)
+        want = pkg.conv2d(x, wt, b, r, stride, p, dil, relu, force_direct=True)
+        assert_close(host(got), host(want), what="case %d: k=%d n=%d c=%d h=%d w=%d o=%d s=%d p=%d d=%d" % (case, k, n, c, h, w, o, stride, p, dil))
+    assert "mfma_k1x1_small" in seen and any(v.startswith("mfma_k3x3") for v in seen) and any(v.startswith("mfma_k7x7") for v in seen), seen
+
+
 def test_conv_winograd_unsupported_shapes_are_refused(pkg):
     assert not pkg.conv2d_winograd_supported((1, 8, 8, 8), (16, 8, 3, 3), 2, 1)        # stride
     assert not pkg.conv2d_winograd_supported((1, 8, 8, 8), (16, 8, 1, 1), 1, 0)        # filter size
