@@ -457,6 +457,24 @@ def test_maxpool_full_size_bit_exact(pkg, fast_orc, synth):
     assert torch.equal(pkg.pool2d(c, 3, 2, 1), torch.full((2, 3, 8, 8), -7.5, device="cuda"))
 
 
+def test_pool_random_shapes_against_oracle(pkg, fast_orc):
+    """Seeded random pooling geometries (window 1-4, stride 1-3, padding below the window) through the generic
+    kernel, and 3x3/2/1 maps of every size class through the row-reusing kernel: max bit for bit against the CPU
+    checker, average within the fp32 tolerance."""
+    rng = np.random.default_rng(20240808)
+    for case in range(24):
+        k = int(rng.integers(1, 5)); s_ = int(rng.integers(1, 4)); p = int(rng.integers(0, (k + 1) // 2 + 1))
+        p = min(p, k - 1) if k > 1 else 0
+        n = int(rng.integers(1, 4)); c = int(rng.integers(1, 20)); h = int(rng.integers(k, 30)); w = int(rng.integers(k, 30))
+        x = rng.uniform(-1, 1, (n, c, h, w)).astype(np.float32)
+        what = "case %d: k=%d s=%d p=%d shape=%s" % (case, k, s_, p, (n, c, h, w))
+        assert_bit_exact(host(pkg.pool2d(dev(x), k, s_, p)), fast_orc.pool2d(x, k, s_, p), what)
+        assert_close(host(pkg.pool2d(dev(x), k, s_, p, avg=True)), fast_orc.pool2d(x, k, s_, p, avg=True), what=what + " avg")
+    for shape in [(1, 3, 8, 8), (2, 5, 6, 16), (1, 64, 56, 56), (3, 7, 30, 24), (4, 64, 112, 112), (9, 128, 28, 32)]:
+        x = rng.uniform(-1, 1, shape).astype(np.float32)
+        assert_bit_exact(host(pkg.pool2d(dev(x), 3, 2, 1)), fast_orc.pool2d(x, 3, 2, 1), "3x3/2 %s" % (shape,))
+
+
 def test_maxpool_edge_semantics(pkg, orc):
     x = np.full((1, 1, 8, 8), -3e30, np.float32)            # below the -1e30 pad candidate
     assert_bit_exact(host(pkg.pool2d(dev(x), 3, 2, 1)), orc.pool2d(x, 3, 2, 1), "pad candidate")
