@@ -497,6 +497,29 @@ def test_add_relu_full_size(pkg, fast_orc, synth):
     assert_bit_exact(host(pkg.relu(dev(x)[1:])), fast_orc.relu(x[1:]), "relu unaligned")   # 4-byte aligned view
 
 
+def test_broadcast_binary_random_shapes(pkg):
+    """add / subtract / multiply / divide over seeded random right-aligned broadcast shapes (size-1 and missing
+    leading dimensions on either side, lengths that leave a vector tail), with and without the fused ReLU: one
+    rounded fp32 operation per element, so bit for bit against numpy."""
+    rng = np.random.default_rng(20240909)
+    ops = [np.add, np.subtract, np.multiply, np.divide]
+    for case in range(40):
+        nd = int(rng.integers(1, 5))
+        full = [int(rng.integers(1, 9)) for _ in range(nd)]
+        sa = [d if rng.random() < 0.7 else 1 for d in full][int(rng.integers(0, nd)):]
+        sb = [d if rng.random() < 0.7 else 1 for d in full][int(rng.integers(0, nd)):]
+        if case % 5 == 0:                       # same shape, long enough for the vector kernel and its tail
+            sa = sb = [int(rng.integers(1, 4)), int(rng.integers(1000, 5000))]
+        a = rng.uniform(-2, 2, sa).astype(np.float32); b = rng.uniform(0.5, 2, sb).astype(np.float32) * rng.choice([-1, 1], sb).astype(np.float32)
+        op = case % 4; relu = case % 3 == 0
+        want = ops[op](a, b).astype(np.float32)
+        if relu:
+            want = np.where(want > 0, want, np.float32(0))
+        got = host(pkg.binary(op, dev(a), dev(b), relu=relu))
+        assert got.shape == want.shape, (case, sa, sb)
+        assert_bit_exact(got, want, "case %d: op %d %s %s relu=%s" % (case, op, sa, sb, relu))
+
+
 def test_gap_full_size(pkg, fast_orc, synth):
     x = synth.uniform((64, 512, 7, 7), 2020)
     assert_bit_exact(host(pkg.global_avg_pool2d(dev(x))), fast_orc.gap(x), "gap 7x7")
