@@ -547,6 +547,26 @@ def test_dense_full_size(pkg, fast_orc, synth):
     assert_bit_exact(host(pkg.gemm(dev(ai), dev(np.eye(64, dtype=np.float32)))), ai, "identity weight (mfma)")
 
 
+def test_gemm_random_shapes(pkg):
+    """nn_dense / nn_gemm over seeded random sizes (k a multiple of 32 takes the matrix-core kernel, anything
+    else the reference-order kernel), both layouts of the second operand, alpha / beta scaling, bias of length n
+    or 1: against a float64 evaluation within the fp32 tolerance."""
+    rng = np.random.default_rng(20241010)
+    for case in range(30):
+        m = int(rng.integers(1, 70)); n = int(rng.integers(1, 130))
+        k = 32 * int(rng.integers(1, 10)) if case % 2 == 0 else int(rng.integers(1, 200))
+        trans_b = 1 if case % 3 != 2 else 0
+        a = rng.uniform(-1, 1, (m, k)).astype(np.float32)
+        b = rng.uniform(-1, 1, (n, k) if trans_b else (k, n)).astype(np.float32)
+        c = None if case % 4 == 3 else rng.uniform(-1, 1, (1,) if case % 4 == 2 else (n,)).astype(np.float32)
+        alpha = 1.0 if case % 5 else 0.5; beta = 1.0 if case % 7 else 2.0
+        want = alpha * (a.astype(np.float64) @ (b.astype(np.float64).T if trans_b else b.astype(np.float64)))
+        if c is not None:
+            want = want + beta * c.astype(np.float64)
+        got = host(pkg.gemm(dev(a), dev(b), None if c is None else dev(c), alpha, beta, trans_b))
+        assert_close(got, want.astype(np.float32), what="case %d: m=%d n=%d k=%d transB=%d" % (case, m, n, k, trans_b))
+
+
 def test_bias_add_and_flatten(pkg, orc, synth):
     x = synth.uniform((3, 6, 5, 7), 2040); b = synth.uniform((6,), 2041)
     assert_bit_exact(host(pkg.bias_add(dev(x), dev(b))), orc.bias_add(x, b), "bias_add")
