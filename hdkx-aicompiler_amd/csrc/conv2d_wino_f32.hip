@@ -195,10 +195,6 @@ wino_kernel(const WinoArgs a) {
     const int b_base = ((lane >> 4) * WT + wave_t) * 256 + (lane & 15) * 4;
 
     floatx4 acc[16][2];
-#pragma unroll
-    for (int f = 0; f < 16; ++f)
-#pragma unroll
-        for (int kb = 0; kb < 2; ++kb) acc[f][kb] = floatx4{0.0f, 0.0f, 0.0f, 0.0f};
 
     float d[ITEMS][12];
     auto load_raw = [&](int s) {
@@ -265,6 +261,13 @@ wino_kernel(const WinoArgs a) {
     // ---- prologue: weight tile and transformed input of the first step; raw input of the second in flight
     issue_u(s_lo, ub0);
     load_raw(s_lo);
+    __builtin_amdgcn_sched_barrier(0);
+    // (the 128 accumulator registers are cleared while the first loads are on their way)
+#pragma unroll
+    for (int f = 0; f < 16; ++f)
+#pragma unroll
+        for (int kb = 0; kb < 2; ++kb) acc[f][kb] = floatx4{0.0f, 0.0f, 0.0f, 0.0f};
+    __builtin_amdgcn_sched_barrier(0);
     transform(vb0);
     load_raw(min(s_lo + 1, last));
     __builtin_amdgcn_sched_barrier(0);
