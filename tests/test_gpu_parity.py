@@ -260,6 +260,44 @@ def test_conv_winograd_channel_split_over_workgroups(pkg, fast_orc, orc, synth, 
                      orc.conv_chain(xi, wi, bi, 1, 1, None, True), "split on small integers")
 
 
+def test_split_reduction_from_two_host_threads(pkg, synth):
+    """Two host threads enqueue split convolutions (parts + adding kernel, sharing the stream's scratch buffer) on
+    the same stream at the same time: the pair of launches of one call is never interleaved with another call's,
+    so every result equals the single-threaded one."""
+    import threading
+    shapes = [(1, 512, 7, 7, 512), (1, 128, 28, 28, 128)]
+    cases = []
+    for i, (n, c, h, w, o) in enumerate(shapes):
+        x = dev(synth.uniform((n, c, h, w), 7600 + i))
+        wt = dev(synth.normal((o, c, 3, 3), 7610 + i, float(np.sqrt(2.0 / (c * 9)))))
+        u = pkg.conv2d_winograd_transform_weights((n, c, h, w), wt, 1)
+        want_w = pkg.conv2d_winograd(x, u, wt.shape, None, None, 1, True).clone()
+        want_g = pkg.conv2d(x, wt, None, None, 1, 1, 1, True).clone()
+        cases.append((x, wt, u, want_w, want_g))
+    torch.cuda.synchronize()
+    stream = torch.cuda.current_stream()
+    errors = []
+
+    def worker(idx):
+        x, wt, u, want_w, want_g = cases[idx]
+        with torch.cuda.stream(stream):
+            for it in range(40):
+                got_w = pkg.conv2d_winograd(x, u, wt.shape, None, None, 1, True)
+                got_g = pkg.conv2d(x, wt, None, None, 1, 1, 1, True)
+                if it % 10 == 9:
+                    stream.synchronize()
+                    if not (torch.equal(got_w, want_w) and torch.equal(got_g, want_g)):
+                        errors.append((idx, it))
+
+    threads = [threading.Thread(target=worker, args=(i,)) for i in range(2)]
+    for t in threads:
+        t.start()
+    for t in threads:
+        t.join()
+    torch.cuda.synchronize()
+    assert not errors, errors
+
+
 def test_conv_winograd_random_shapes_against_direct_kernel(pkg):
     """Seeded random geometries (batch, channels, height, width, output channels, padding; every epilogue mix):
     the Winograd kernel against the reference-order direct kernel on the same GPU tensors."""
