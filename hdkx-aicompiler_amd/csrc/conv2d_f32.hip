@@ -825,7 +825,11 @@ int32_t kxc_hip_conv2d_nchw_f32(const kxc_hip_conv2d_desc* desc, const float* x,
             while (split < 16 && waves * split < 2048 && a.nchunks / (split * 2) >= 2 * c.v->ks &&
                    total * static_cast<int64_t>(sizeof(float)) * split * 2 <= (8LL << 20))
                 split *= 2;
-            if (const char* e = std::getenv("KXC_HIP_CONV_GSPLIT")) { const int f = std::atoi(e); if (f >= 1 && f <= a.nchunks) split = f; }
+            if (const char* e = std::getenv("KXC_HIP_CONV_GSPLIT")) {
+                // (a forced split is honoured while its partial sums stay below 256 MiB)
+                const int f = std::atoi(e);
+                if (f >= 1 && f <= a.nchunks && total * static_cast<int64_t>(sizeof(float)) * f <= (256LL << 20)) split = f;
+            }
             if (split > 1) {
                 a.cps = static_cast<int32_t>(CeilDiv(a.nchunks, split));
                 a.gsplit = static_cast<int32_t>(CeilDiv(a.nchunks, a.cps));      // no empty split

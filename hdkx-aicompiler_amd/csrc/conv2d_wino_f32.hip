@@ -608,7 +608,11 @@ int32_t kxc_hip_conv2d_winograd_nchw_f32(const kxc_hip_conv2d_desc* desc, const 
     const int64_t out_elems = static_cast<int64_t>(a.N) * a.O * a.OHW;
     if (v->ks == 1) {
         int split = GroupSplit(a.num_units, a.csteps, out_elems);
-        if (const char* e = std::getenv("KXC_HIP_WINOGRAD_GSPLIT")) { const int f = std::atoi(e); if (f >= 1 && f <= a.csteps) split = f; }
+        if (const char* e = std::getenv("KXC_HIP_WINOGRAD_GSPLIT")) {
+            // (a forced split is honoured while its partial outputs stay below 256 MiB)
+            const int f = std::atoi(e);
+            if (f >= 1 && f <= a.csteps && out_elems * static_cast<int64_t>(sizeof(float)) * f <= (256LL << 20)) split = f;
+        }
         if (split > 1) {
             a.steps_per_split = static_cast<int32_t>(CeilDiv(a.csteps, split));
             a.gsplit = static_cast<int32_t>(CeilDiv(a.csteps, a.steps_per_split));      // no empty part
