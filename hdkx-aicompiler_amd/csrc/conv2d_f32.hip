@@ -757,31 +757,62 @@ bool UseSmall1x1(const kxc_hip_conv2d_desc* d, const ConvArgs& a) {
     return a.M <= 16384;
 }
 
-}  // namespace
-
-extern "C" {
-
-const char* kxc_hip_conv2d_variant(const kxc_hip_conv2d_desc* desc) {
-    ConvArgs a;
-    if (FillArgs(desc, &a, "kxc_hip_conv2d_variant") != KXC_HIP_OK) return "invalid";
-    if (desc->flags & KXC_HIP_CONV_FORCE_DIRECT) return "direct";
-    if (UseSmall1x1(desc, a)) return "mfma_k1x1_small";
-    ApplyRowView(&a, desc->kh);
-    Choice c;
-    Select(a, desc->kh, desc->kw, &c);
-    return c.v ? c.v->name : "direct";
+// Launches that still leave most SIMDs idle (batch 1, deep layers: a handful of tiles, a long reduction) split
+// the reduction over workgroups as well; every workgroup keeps at least two chunks per wave group, and the partial
+// sums stay small next to the caches (the split re-reads them once): at most 8 MiB.
+void SplitOverWorkgroups(const Choice& c, int32_t nchunks, int64_t tiles, int64_t total, int* out_split) {
+    const int64_t waves = tiles * c.v->nw * c.v->ks;
+    int split = 1;
+    while (split < 16 && waves * split < 2048 && nchunks / (split * 2) >= 2 * c.v->ks &&
+           total * static_cast<int64_t>(sizeof(float)) * split * 2 <= (8LL << 20))
+        split *= 2;
+    if (const char* e = std::getenv("KXC_HIP_CONV_GSPLIT")) {
+        // (a forced split is honoured while its partial sums stay below 256 MiB)
+        const int f = std::atoi(e);
+        if (f >= 1 && f <= nchunks && total * static_cast<int64_t>(sizeof(float)) * f <= (256LL << 20)) split = f;
+    }
+    *out_split = split;
 }
 
-int32_t kxc_hip_conv2d_nchw_f32(const kxc_hip_conv2d_desc* desc, const float* x, const float* w, const float* bias,
-                                const float* residual, float* y, void* stream) {
+// ------------------------------------------------------------------------------------------
+// Scratch of the entry point that allocates nothing (kxc_hip_conv2d_nchw_f32_noalloc): the raw partial sums of a
+// reduction split over workgroups live in this file-scope device array instead of a hipMalloc'ed buffer.  Every
+// GPU the library runs on holds its own copy (8 MiB) until the process ends.  The array's name is only a host-side
+// handle; its device address is asked for once per device (with that device current) and kernels get that address.
+// ------------------------------------------------------------------------------------------
+constexpr size_t kNoAllocScratchBytes = static_cast<size_t>(8) << 20;
+static __device__ __align__(256) float scratch[kNoAllocScratchBytes / sizeof(float)];
+
+constexpr int kMaxDevices = 64;
+int32_t NoAllocScratch(float** out) {
+    static std::mutex mu;
+    static float* addr[kMaxDevices] = {};
+    int dev = 0;
+    KXC_HIP_CALL(hipGetDevice(&dev), "hipGetDevice");
+    KXC_HIP_REQUIRE(dev >= 0 && dev < kMaxDevices, "kxc_hip_conv2d_nchw_f32_noalloc: device %d out of range", dev);
+    std::lock_guard<std::mutex> lock(mu);
+    if (!addr[dev]) {
+        float* p = nullptr;
+        KXC_HIP_CALL(hipGetSymbolAddress(reinterpret_cast<void**>(&p), HIP_SYMBOL(scratch)), "hipGetSymbolAddress(scratch)");
+        KXC_HIP_REQUIRE(p != nullptr, "kxc_hip_conv2d_nchw_f32_noalloc: no device address for the scratch array");
+        addr[dev] = p;
+    }
+    *out = addr[dev];
+    return KXC_HIP_OK;
+}
+
+// The operator behind both entry points.  no_alloc: the partial sums of a split reduction go to the file-scope
+// scratch array instead of the grow-only per-stream buffer, and a launch that would need more is refused.
+int32_t Conv2dRun(const kxc_hip_conv2d_desc* desc, const float* x, const float* w, const float* bias,
+                  const float* residual, float* y, void* stream, bool no_alloc) {
+    const char* const who = no_alloc ? "kxc_hip_conv2d_nchw_f32_noalloc" : "kxc_hip_conv2d_nchw_f32";
     ConvArgs a;
-    if (int32_t rc = FillArgs(desc, &a, "kxc_hip_conv2d_nchw_f32")) return rc;
+    if (int32_t rc = FillArgs(desc, &a, who)) return rc;
     const int64_t total = static_cast<int64_t>(a.N) * a.O * a.OHW;
     if (total == 0) return KXC_HIP_OK;
-    KXC_HIP_REQUIRE(x && w && y, "kxc_hip_conv2d_nchw_f32: NULL pointer");
-    KXC_HIP_REQUIRE(!(desc->flags & KXC_HIP_CONV_BIAS) || bias, "kxc_hip_conv2d_nchw_f32: bias flag without bias");
-    KXC_HIP_REQUIRE(!(desc->flags & KXC_HIP_CONV_RESIDUAL) || residual,
-                    "kxc_hip_conv2d_nchw_f32: residual flag without residual");
+    KXC_HIP_REQUIRE(x && w && y, "%s: NULL pointer", who);
+    KXC_HIP_REQUIRE(!(desc->flags & KXC_HIP_CONV_BIAS) || bias, "%s: bias flag without bias", who);
+    KXC_HIP_REQUIRE(!(desc->flags & KXC_HIP_CONV_RESIDUAL) || residual, "%s: residual flag without residual", who);
     a.x = x; a.w = w; a.bias = bias; a.res = residual; a.y = y;
     a.x_bytes = static_cast<uint32_t>(static_cast<int64_t>(a.N) * a.C * a.H * a.W * 4);       // < 2 GiB on the MFMA path
     a.w_bytes = static_cast<uint32_t>(static_cast<int64_t>(a.O) * a.C * desc->kh * desc->kw * 4);
@@ -810,7 +841,7 @@ int32_t kxc_hip_conv2d_nchw_f32(const kxc_hip_conv2d_desc* desc, const float* x,
         a.p_tiles = static_cast<int32_t>(CeilDiv(a.M, c.v->tp));
         a.o_tiles = static_cast<int32_t>(CeilDiv(a.O, c.v->to));
         const int64_t tiles = static_cast<int64_t>(a.p_tiles) * a.o_tiles;
-        KXC_HIP_REQUIRE(tiles < (1LL << 30), "kxc_hip_conv2d_nchw_f32: too many tiles");
+        KXC_HIP_REQUIRE(tiles < (1LL << 30), "%s: too many tiles", who);
         a.num_tiles = static_cast<int32_t>(tiles);
         // Launches that still leave most SIMDs idle (batch 1, deep layers: a handful of tiles, a long reduction)
         // split the reduction over workgroups as well; every workgroup keeps at least two chunks per wave group.
@@ -819,23 +850,23 @@ int32_t kxc_hip_conv2d_nchw_f32(const kxc_hip_conv2d_desc* desc, const float* x,
         a.out_elems = total;
         SplitScratchLease lease;      // held until the adding kernel is enqueued
         {
-            const int64_t waves = tiles * c.v->nw * c.v->ks;
             int split = 1;
-            // (only while the partial sums stay small next to the caches: the split re-reads them once)
-            while (split < 16 && waves * split < 2048 && a.nchunks / (split * 2) >= 2 * c.v->ks &&
-                   total * static_cast<int64_t>(sizeof(float)) * split * 2 <= (8LL << 20))
-                split *= 2;
-            if (const char* e = std::getenv("KXC_HIP_CONV_GSPLIT")) {
-                // (a forced split is honoured while its partial sums stay below 256 MiB)
-                const int f = std::atoi(e);
-                if (f >= 1 && f <= a.nchunks && total * static_cast<int64_t>(sizeof(float)) * f <= (256LL << 20)) split = f;
-            }
+            SplitOverWorkgroups(c, a.nchunks, tiles, total, &split);
             if (split > 1) {
                 a.cps = static_cast<int32_t>(CeilDiv(a.nchunks, split));
                 a.gsplit = static_cast<int32_t>(CeilDiv(a.nchunks, a.cps));      // no empty split
                 if (a.gsplit > 1) {
-                    if (int32_t rc = AcquireSplitScratch(s, static_cast<size_t>(a.gsplit) * total * sizeof(float), &lease)) return rc;
-                    a.partial = lease.ptr;
+                    const size_t need = static_cast<size_t>(a.gsplit) * total * sizeof(float);
+                    if (no_alloc) {
+                        // every kernel of the pair overwrites what it reads later, nothing has to start at zero
+                        KXC_HIP_REQUIRE(need <= kNoAllocScratchBytes,
+                                        "%s: the split reduction needs %zu bytes of scratch, the built-in array holds %zu",
+                                        who, need, kNoAllocScratchBytes);
+                        if (int32_t rc = NoAllocScratch(&a.partial)) return rc;
+                    } else {
+                        if (int32_t rc = AcquireSplitScratch(s, need, &lease)) return rc;
+                        a.partial = lease.ptr;
+                    }
                 } else {
                     a.cps = a.nchunks;
                 }
@@ -871,6 +902,54 @@ int32_t kxc_hip_conv2d_nchw_f32(const kxc_hip_conv2d_desc* desc, const float* x,
     if (g > 256 * 64) g = 256 * 64;
     conv_direct_kernel<<<NoteGrid(static_cast<int>(g)), NoteBlock(256), NoteLds(0), s>>>(direct_args, desc->kh, desc->kw, total);
     return CheckLaunch("conv_direct");
+}
+
+}  // namespace
+
+extern "C" {
+
+const char* kxc_hip_conv2d_variant(const kxc_hip_conv2d_desc* desc) {
+    ConvArgs a;
+    if (FillArgs(desc, &a, "kxc_hip_conv2d_variant") != KXC_HIP_OK) return "invalid";
+    if (desc->flags & KXC_HIP_CONV_FORCE_DIRECT) return "direct";
+    if (UseSmall1x1(desc, a)) return "mfma_k1x1_small";
+    ApplyRowView(&a, desc->kh);
+    Choice c;
+    Select(a, desc->kh, desc->kw, &c);
+    return c.v ? c.v->name : "direct";
+}
+
+int32_t kxc_hip_conv2d_nchw_f32(const kxc_hip_conv2d_desc* desc, const float* x, const float* w, const float* bias,
+                                const float* residual, float* y, void* stream) {
+    return Conv2dRun(desc, x, w, bias, residual, y, stream, false);
+}
+
+int32_t kxc_hip_conv2d_nchw_f32_noalloc(const kxc_hip_conv2d_desc* desc, const float* x, const float* w, const float* bias,
+                                        const float* residual, float* y, void* stream) {
+    return Conv2dRun(desc, x, w, bias, residual, y, stream, true);
+}
+
+size_t kxc_hip_conv2d_noalloc_scratch_bytes(void) { return kNoAllocScratchBytes; }
+
+int32_t kxc_hip_conv2d_scratch_needed(const kxc_hip_conv2d_desc* desc, size_t* out_bytes) {
+    KXC_HIP_REQUIRE(out_bytes != nullptr, "kxc_hip_conv2d_scratch_needed: out_bytes is NULL");
+    *out_bytes = 0;
+    ConvArgs a;
+    if (int32_t rc = FillArgs(desc, &a, "kxc_hip_conv2d_scratch_needed")) return rc;
+    const int64_t total = static_cast<int64_t>(a.N) * a.O * a.OHW;
+    if (total == 0 || (desc->flags & KXC_HIP_CONV_FORCE_DIRECT) || UseSmall1x1(desc, a) || a.M <= 0) return KXC_HIP_OK;
+    ApplyRowView(&a, desc->kh);
+    Choice c;
+    Select(a, desc->kh, desc->kw, &c);
+    if (!c.v) return KXC_HIP_OK;
+    const int32_t nchunks = (a.C + c.v->cc - 1) / c.v->cc;
+    int split = 1;
+    SplitOverWorkgroups(c, nchunks, CeilDiv(a.M, c.v->tp) * CeilDiv(a.O, c.v->to), total, &split);
+    if (split > 1) {
+        const int64_t parts = CeilDiv(nchunks, CeilDiv(nchunks, split));
+        if (parts > 1) *out_bytes = static_cast<size_t>(parts) * total * sizeof(float);
+    }
+    return KXC_HIP_OK;
 }
 
 }  // extern "C"

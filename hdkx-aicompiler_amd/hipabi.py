@@ -83,6 +83,7 @@ def lib():
         _lib.kxc_hip_qconv2d_c16_variant.restype = C.c_char_p
         _lib.kxc_hip_plan_node_symbol.restype = C.c_char_p
         _lib.kxc_hip_plan_workspace.restype = C.c_void_p
+        _lib.kxc_hip_conv2d_noalloc_scratch_bytes.restype = C.c_size_t
     return _lib
 
 
@@ -131,7 +132,10 @@ def conv2d_variant(x_shape, w_shape, stride, pad, dil=1, flags=0):
     return lib().kxc_hip_conv2d_variant(C.byref(d)).decode()
 
 
-def conv2d(x, w, bias=None, residual=None, stride=1, pad=0, dil=1, relu=False, force_direct=False, out=None):
+def conv2d(x, w, bias=None, residual=None, stride=1, pad=0, dil=1, relu=False, force_direct=False, out=None,
+           no_alloc=False):
+    """nn_conv2d through kxc_hip_conv2d_nchw_f32, or (no_alloc, with `out` given) through the entry point that
+    allocates nothing."""
     import torch
     _need(x, torch.float32, "x"); _need(w, torch.float32, "w")
     _need(bias, torch.float32, "bias"); _need(residual, torch.float32, "residual")
@@ -141,7 +145,8 @@ def conv2d(x, w, bias=None, residual=None, stride=1, pad=0, dil=1, relu=False, f
             (CONV_RELU if relu else 0) | (CONV_FORCE_DIRECT if force_direct else 0)
     d = conv_desc(tuple(x.shape), tuple(w.shape), stride, pad, dil, flags)
     y = out if out is not None else torch.empty(conv_out_shape(d), dtype=torch.float32, device=x.device)
-    _check(lib().kxc_hip_conv2d_nchw_f32(C.byref(d), _p(x), _p(w), _p(bias), _p(residual), _p(y), _stream()))
+    entry = lib().kxc_hip_conv2d_nchw_f32_noalloc if no_alloc else lib().kxc_hip_conv2d_nchw_f32
+    _check(entry(C.byref(d), _p(x), _p(w), _p(bias), _p(residual), _p(y), _stream()))
     return y
 
 

@@ -116,6 +116,21 @@ int32_t kxc_hip_conv2d_nchw_f32(const kxc_hip_conv2d_desc* desc, const float* x,
                                 const float* bias, const float* residual, float* y, void* stream);
 /* Name of the kernel variant the library would launch for this shape ("mfma_..." or "direct"). */
 const char* kxc_hip_conv2d_variant(const kxc_hip_conv2d_desc* desc);
+/* The same operator for callers that cannot allocate device memory (code under HIP graph capture, tight serving
+ * loops, harnesses that forbid hipMalloc).  No counterpart in the reference.  Same arguments, kernels and results
+ * as kxc_hip_conv2d_nchw_f32, but it calls no hipMalloc / hipFree or allocating library routine: the partial sums
+ * of a reduction split over workgroups (small launches with long reductions, e.g. batch-1 512-channel layers) go
+ * to a device array built into the library, kxc_hip_conv2d_noalloc_scratch_bytes() = 8 MiB per GPU, held until the
+ * process ends.  A launch whose partial sums would not fit fails with KXC_HIP_ERR_INVALID and launches nothing
+ * (the library's own choice of split never exceeds the array; only a forced split can).  All calls on one GPU
+ * share that array: two calls whose kernels may overlap on that GPU (different streams, different threads) race;
+ * calls enqueued on one stream are safe. */
+int32_t kxc_hip_conv2d_nchw_f32_noalloc(const kxc_hip_conv2d_desc* desc, const float* x, const float* w,
+                                        const float* bias, const float* residual, float* y, void* stream);
+size_t kxc_hip_conv2d_noalloc_scratch_bytes(void);
+/* Bytes of scratch (partial sums) a launch for this shape uses, 0 when its reduction is not split over workgroups:
+ * lets a caller see beforehand whether kxc_hip_conv2d_nchw_f32_noalloc takes the shape. */
+int32_t kxc_hip_conv2d_scratch_needed(const kxc_hip_conv2d_desc* desc, size_t* out_bytes);
 
 /* nn_conv2d with a 3x3 filter, stride 1, dilation 1 and c % 4 == 0 as Winograd F(2x2, 3x3) on the matrix cores:
  * same operator and epilogue as kxc_hip_conv2d_nchw_f32 (convolution.cc:38-75, nn.h:107-158) with 2.25x fewer
