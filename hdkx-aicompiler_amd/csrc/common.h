@@ -92,6 +92,14 @@ struct SplitScratchLease {
 int32_t AcquireSplitScratch(hipStream_t stream, size_t bytes, SplitScratchLease* lease);
 int32_t LaunchSplitReduce(hipStream_t stream, const SplitReduceArgs& a);
 
+// The filter transforms of several Winograd layers in one launch (conv2d_wino_f32.hip).
+struct WinoWeightJob {
+    const kxc_hip_conv2d_desc* desc;
+    const float* w;      // OIHW weights
+    float* u;            // kxc_hip_conv2d_winograd_weight_bytes(desc) bytes
+};
+int32_t LaunchWinogradWeightTransforms(const WinoWeightJob* jobs, int32_t count, hipStream_t stream);
+
 constexpr int64_t kMaxGridX = 2147483647LL;
 
 inline int64_t CeilDiv(int64_t a, int64_t b) { return (a + b - 1) / b; }

@@ -24,6 +24,7 @@
 // The sums are formed in a different order than the direct loop nest (and G introduces factors 1/2, 1/4), so
 // results agree with the CPU backend within the fp32 tolerance of the operator (about 1e-6 relative on
 // ResNet-sized reductions), not bit for bit.
+#include <algorithm>
 #include <cstdlib>
 #include <cstring>
 #include <mutex>
@@ -86,9 +87,8 @@ __device__ __forceinline__ float relu_sel(float v) { return (v > 0.0f) ? v : 0.0
 // Filter transform.  One thread per (o, c), o < 32*ceil(O/32) (absent output channels give zero blocks).
 // packed index: ((o/32 * csteps + c/4) * 2048) + (((c%4)*2 + (o%32)/16)*4 + i)*64 + (o%16)*4 + j  for U[i][j]
 // ------------------------------------------------------------------------------------------
-__global__ void __launch_bounds__(256) wino_weight_kernel(const float* __restrict__ w, float* __restrict__ u, int32_t O,
-                                                          int32_t C, int32_t o_padded) {
-    const int e = blockIdx.x * 256 + threadIdx.x;
+__device__ __forceinline__ void wino_weight_one(const float* __restrict__ w, float* __restrict__ u, int32_t O, int32_t C,
+                                                int32_t o_padded, int e) {
     if (e >= o_padded * C) return;
     const int o = e / C, c = e - o * C;
     float g[3][3];
@@ -116,6 +116,26 @@ __global__ void __launch_bounds__(256) wino_weight_kernel(const float* __restric
         v[3] = t[i][2];
         *reinterpret_cast<floatx4*>(dst + i * 64) = v;
     }
+}
+
+__global__ void __launch_bounds__(256) wino_weight_kernel(const float* __restrict__ w, float* __restrict__ u, int32_t O,
+                                                          int32_t C, int32_t o_padded) {
+    wino_weight_one(w, u, O, C, o_padded, blockIdx.x * 256 + threadIdx.x);
+}
+
+// The filter transforms of several layers in one launch (a launch plan transforms all its Winograd layers' weights
+// at the start of a run): block b belongs to the job whose [first_block, next first_block) range holds it.
+constexpr int kMaxWeightJobs = 32;
+struct WinoWeightBatch {
+    const float* w[kMaxWeightJobs];
+    float* u[kMaxWeightJobs];
+    int32_t O[kMaxWeightJobs], C[kMaxWeightJobs], o_padded[kMaxWeightJobs], first_block[kMaxWeightJobs + 1];
+    int32_t count;
+};
+__global__ void __launch_bounds__(256) wino_weight_batch_kernel(const WinoWeightBatch b) {
+    int j = 0;
+    while (j + 1 < b.count && static_cast<int32_t>(blockIdx.x) >= b.first_block[j + 1]) ++j;
+    wino_weight_one(b.w[j], b.u[j], b.O[j], b.C[j], b.o_padded[j], (static_cast<int>(blockIdx.x) - b.first_block[j]) * 256 + threadIdx.x);
 }
 
 // ------------------------------------------------------------------------------------------
@@ -536,6 +556,33 @@ const WinoVariant* SelectWino(const kxc_hip_conv2d_desc* d) {
 }
 
 }  // namespace
+
+namespace kxc_hip {
+
+int32_t LaunchWinogradWeightTransforms(const WinoWeightJob* jobs, int32_t count, hipStream_t stream) {
+    for (int32_t base = 0; base < count; base += kMaxWeightJobs) {
+        WinoWeightBatch b;
+        std::memset(&b, 0, sizeof(b));
+        b.count = std::min<int32_t>(kMaxWeightJobs, count - base);
+        int64_t blocks = 0;
+        for (int32_t j = 0; j < b.count; ++j) {
+            const WinoWeightJob& job = jobs[base + j];
+            KXC_HIP_REQUIRE(job.desc && Supported(job.desc) && job.w && job.u, "winograd weight transform: bad job %d", base + j);
+            b.w[j] = job.w; b.u[j] = job.u;
+            b.O[j] = job.desc->o; b.C[j] = job.desc->c;
+            b.o_padded[j] = static_cast<int32_t>(CeilDiv(job.desc->o, 32) * 32);
+            b.first_block[j] = static_cast<int32_t>(blocks);
+            blocks += CeilDiv(static_cast<int64_t>(b.o_padded[j]) * b.C[j], 256);
+            KXC_HIP_REQUIRE(blocks < kMaxGridX, "winograd weight transform: too many blocks");
+        }
+        b.first_block[b.count] = static_cast<int32_t>(blocks);
+        wino_weight_batch_kernel<<<NoteGrid(static_cast<int>(blocks)), NoteBlock(256), NoteLds(0), stream>>>(b);
+        if (int32_t rc = CheckLaunch("wino_weight_batch_kernel")) return rc;
+    }
+    return KXC_HIP_OK;
+}
+
+}  // namespace kxc_hip
 
 extern "C" {
 

@@ -64,6 +64,15 @@ struct kxc_hip_plan {
     hipGraphExec_t graph_exec = nullptr;
     std::vector<void*> graph_args;
     hipStream_t graph_stream = nullptr;   // the graph is replayed only on the stream it was captured on
+    // Constants of Winograd nodes.  Default: the filter transforms of all such nodes run at the start of EVERY
+    // run (one launch), so weights rewritten in place -- or another tensor at the same address -- are seen, as
+    // with the CPU backend, which re-reads every constant on every call.  Frozen (kxc_hip_plan_freeze_constants):
+    // transformed when first seen or when another pointer arrives; constants_ready orders runs on other streams
+    // after the stream the transforms were enqueued on.
+    bool constants_frozen = false;
+    hipEvent_t constants_ready = nullptr;
+    bool constants_recorded = false;
+    hipStream_t constants_stream = nullptr;
 };
 
 namespace {
@@ -123,6 +132,7 @@ int32_t kxc_hip_plan_destroy(kxc_hip_plan* plan) {
         if (n.done_event) (void)hipEventDestroy(n.done_event);
     }
     if (plan->side_stream) (void)hipStreamDestroy(plan->side_stream);
+    if (plan->constants_ready) (void)hipEventDestroy(plan->constants_ready);
     if (plan->graph_exec) (void)hipGraphExecDestroy(plan->graph_exec);
     if (plan->graph) (void)hipGraphDestroy(plan->graph);
     delete plan;
@@ -172,6 +182,19 @@ int32_t kxc_hip_plan_add_conv2d_winograd(kxc_hip_plan* plan, const kxc_hip_conv2
 int32_t kxc_hip_plan_invalidate_constants(kxc_hip_plan* plan) {
     KXC_HIP_REQUIRE(plan != nullptr, "kxc_hip_plan_invalidate_constants: plan is NULL");
     for (Node& n : plan->nodes) n.transformed_from = nullptr;
+    return KXC_HIP_OK;
+}
+
+int32_t kxc_hip_plan_freeze_constants(kxc_hip_plan* plan, int32_t frozen) {
+    KXC_HIP_REQUIRE(plan != nullptr, "kxc_hip_plan_freeze_constants: plan is NULL");
+    plan->constants_frozen = frozen != 0;
+    for (Node& n : plan->nodes) n.transformed_from = nullptr;      // the next run transforms what it is given
+    if (plan->graph_exec) {       // a captured graph holds the other mode's launches
+        (void)hipGraphExecDestroy(plan->graph_exec); plan->graph_exec = nullptr;
+        if (plan->graph) { (void)hipGraphDestroy(plan->graph); plan->graph = nullptr; }
+        plan->graph_args.clear();
+        plan->graph_stream = nullptr;
+    }
     return KXC_HIP_OK;
 }
 
@@ -483,6 +506,39 @@ int32_t CheckRunArgs(kxc_hip_plan* plan, void** args, const char* who) {
     return KXC_HIP_OK;
 }
 
+// The filter transforms of the plan's Winograd nodes, all in one launch on `stream`: every node's (only_changed:
+// those whose weight pointer differs from the one last transformed).  *launched tells whether anything ran.
+int32_t TransformConstants(kxc_hip_plan* plan, void** args, hipStream_t stream, bool only_changed, bool* launched) {
+    std::vector<WinoWeightJob> jobs;
+    for (Node& n : plan->nodes) {
+        if (n.kind != NodeKind::kConv2D || n.i32[0] != 1) continue;
+        const void* w = Resolve(plan, n.bufs[1], args);
+        if (only_changed && n.transformed_from == w) continue;
+        jobs.push_back({&n.conv, static_cast<const float*>(w), static_cast<float*>(Resolve(plan, n.bufs[5], args))});
+        n.transformed_from = w;
+    }
+    *launched = !jobs.empty();
+    if (jobs.empty()) return KXC_HIP_OK;
+    return LaunchWinogradWeightTransforms(jobs.data(), static_cast<int32_t>(jobs.size()), stream);
+}
+
+// Frozen constants: transform what has not been seen yet (outside any stream capture), and order a run on another
+// stream after the transforms.
+int32_t EnsureFrozenConstants(kxc_hip_plan* plan, void** args, hipStream_t stream) {
+    bool launched = false;
+    if (int32_t rc = TransformConstants(plan, args, stream, true, &launched)) return rc;
+    if (launched) {
+        if (!plan->constants_ready)
+            KXC_HIP_CALL(hipEventCreateWithFlags(&plan->constants_ready, hipEventDisableTiming), "plan event");
+        KXC_HIP_CALL(hipEventRecord(plan->constants_ready, stream), "hipEventRecord");
+        plan->constants_recorded = true;
+        plan->constants_stream = stream;
+    } else if (plan->constants_recorded && plan->constants_stream != stream) {
+        KXC_HIP_CALL(hipStreamWaitEvent(stream, plan->constants_ready, 0), "hipStreamWaitEvent");
+    }
+    return KXC_HIP_OK;
+}
+
 // Enqueues one node on stream s.
 int32_t RunNode(kxc_hip_plan* plan, Node& n, void** args, void* s) {
     {
@@ -491,13 +547,7 @@ int32_t RunNode(kxc_hip_plan* plan, Node& n, void** args, void* s) {
         switch (n.kind) {
             case NodeKind::kConv2D:
                 if (n.i32[0] == 1) {
-                    // weights are module constants: transformed when first seen (or when another tensor is passed)
-                    if (n.transformed_from != B(1)) {
-                        rc = kxc_hip_conv2d_winograd_transform_weights(&n.conv, static_cast<const float*>(B(1)),
-                                                                       static_cast<float*>(B(5)), s);
-                        if (rc) break;
-                        n.transformed_from = B(1);
-                    }
+                    // (the transformed weights in B(5) were written by TransformConstants at the start of the run)
                     rc = kxc_hip_conv2d_winograd_nchw_f32(&n.conv, static_cast<const float*>(B(0)), static_cast<const float*>(B(5)),
                                                           static_cast<const float*>(B(2)), static_cast<const float*>(B(3)),
                                                           static_cast<float*>(B(4)), s);
@@ -616,6 +666,10 @@ namespace {
 // join event (also the pattern stream capture records as parallel graph branches).
 int32_t EnqueueAll(kxc_hip_plan* plan, void** args, hipStream_t main_stream) {
     void* s = static_cast<void*>(main_stream);
+    if (!plan->constants_frozen) {
+        bool launched = false;
+        if (int32_t rc = TransformConstants(plan, args, main_stream, false, &launched)) return rc;
+    }
     std::vector<Node*> unjoined;      // side-lane nodes the main lane has not waited for yet
     for (Node& n : plan->nodes) {
         if (n.lane == 1 && plan->side_stream) {
@@ -654,6 +708,8 @@ extern "C" {
 int32_t kxc_hip_plan_run(kxc_hip_plan* plan, void** args, void* stream) {
     if (int32_t rc = CheckRunArgs(plan, args, "kxc_hip_plan_run")) return rc;
     hipStream_t main_stream = reinterpret_cast<hipStream_t>(stream ? stream : static_cast<void*>(CurrentStream()));
+    if (plan->constants_frozen)
+        if (int32_t rc = EnsureFrozenConstants(plan, args, main_stream)) return rc;
     // Graph replay needs a real stream (the null stream cannot be captured) and one eager run before the
     // capture, so that everything that allocates lazily (split-reduction scratch, function attributes) exists.
     // The captured kernels hold the addresses of that stream's scratch buffers, so a run on another stream
@@ -723,6 +779,11 @@ int32_t kxc_hip_plan_run_profiled(kxc_hip_plan* plan, void** args, void* stream,
     // one event before every node and one after the last: node i ran between events i and i+1
     std::vector<hipEvent_t> ev(static_cast<size_t>(nodes) + 1, nullptr);
     int32_t rc = KXC_HIP_OK;
+    {
+        bool launched = false;
+        rc = plan->constants_frozen ? EnsureFrozenConstants(plan, args, hs) : TransformConstants(plan, args, hs, false, &launched);
+        if (rc != KXC_HIP_OK) return rc;
+    }
     for (auto& e : ev)
         if (hipEventCreate(&e) != hipSuccess) { rc = Fail(KXC_HIP_ERR_RUNTIME, "%s: hipEventCreate failed", who); break; }
     for (int32_t i = 0; rc == KXC_HIP_OK && i < nodes; ++i) {

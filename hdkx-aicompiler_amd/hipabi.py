@@ -510,6 +510,9 @@ class Plan:
     def invalidate_constants(self):
         _check(lib().kxc_hip_plan_invalidate_constants(self._h))
 
+    def freeze_constants(self, frozen=True):
+        _check(lib().kxc_hip_plan_freeze_constants(self._h, C.c_int32(1 if frozen else 0)))
+
     def add_pool2d(self, desc, x, y):
         _check(lib().kxc_hip_plan_add_pool2d(self._h, C.byref(desc), x, y))
 

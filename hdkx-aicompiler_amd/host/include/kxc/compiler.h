@@ -36,6 +36,11 @@ struct CompileConfigNode {
     bool hip_fuse{true};               // fold bias / residual add / ReLU into convolution launches
     bool hip_concurrent_branches{true};   // run a block's downsample convolution beside its first 3x3 convolution
     bool hip_winograd{true};              // 3x3 stride-1 convolutions with constant weights as Winograd F(2x2,3x3) where faster
+    // Winograd layers transform their (constant) filters on the GPU.  false (default): at the start of every Run, from
+    // the pointers passed to that Run, so a Run always sees the constants' current contents, like the CPU back end.
+    // true: once, when a pointer is first seen -- the caller promises not to change the weights behind the module's
+    // back (serving); CompiledModule::InvalidateConstants() announces an in-place update.
+    bool hip_constants_frozen{false};
     bool sync_after_run{true};
     // Adaptive mode (include/api/compile_config.h:40-45)
     std::vector<std::vector<int64_t>> suggested_input_shapes;   // each is warmed up at Compile
@@ -93,6 +98,9 @@ public:
     // hip target: later runs on a non-null stream with unchanged argument pointers replay a captured HIP graph
     // (one launch call per Run instead of one per kernel; for launch-bound, small-batch functions).
     void EnableGraphReplay(bool enable);
+    // hip target: see CompileConfigNode::hip_constants_frozen.
+    void FreezeConstants(bool frozen);
+    void InvalidateConstants();
 
 private:
     friend class Compiler;

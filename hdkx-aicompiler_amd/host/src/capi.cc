@@ -60,6 +60,26 @@ int kxc_host_module_enable_graph(void* module, int enable) {
     }
 }
 
+int kxc_host_module_freeze_constants(void* module, int frozen) {
+    try {
+        static_cast<ModuleHandle*>(module)->module.FreezeConstants(frozen != 0);
+        return 0;
+    } catch (const std::exception& e) {
+        g_error = e.what();
+        return 1;
+    }
+}
+
+int kxc_host_module_invalidate_constants(void* module) {
+    try {
+        static_cast<ModuleHandle*>(module)->module.InvalidateConstants();
+        return 0;
+    } catch (const std::exception& e) {
+        g_error = e.what();
+        return 1;
+    }
+}
+
 int kxc_host_module_is_ready(void* module) { return static_cast<ModuleHandle*>(module)->module.IsReady() ? 1 : 0; }
 const char* kxc_host_module_status(void* module) {
     g_error = static_cast<ModuleHandle*>(module)->module.GetStatus();

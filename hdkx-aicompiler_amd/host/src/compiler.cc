@@ -187,6 +187,7 @@ public:
         if (!dry_) {
             if (kxc_hip_plan_finalize(m_->plan, m_->workspace_bytes))
                 throw std::runtime_error(std::string("plan finalize failed: ") + kxc_hip_last_error());
+            if (cfg_->hip_constants_frozen) kxc_hip_plan_freeze_constants(m_->plan, 1);
             m_->ready = true;
             m_->status = "ready (hip back end, " + std::to_string(m_->execs.size()) + " launches)";
         } else {
@@ -669,6 +670,15 @@ void CompiledModule::EnableGraphReplay(bool enable) {
     if (kxc_hip_plan_enable_graph(impl_->plan, enable ? 1 : 0)) throw std::runtime_error(std::string("EnableGraphReplay: ") + kxc_hip_last_error());
 }
 
+void CompiledModule::FreezeConstants(bool frozen) {
+    if (!impl_ || !impl_->plan) throw std::runtime_error("FreezeConstants: not a loaded hip module");
+    if (kxc_hip_plan_freeze_constants(impl_->plan, frozen ? 1 : 0)) throw std::runtime_error(std::string("FreezeConstants: ") + kxc_hip_last_error());
+}
+void CompiledModule::InvalidateConstants() {
+    if (!impl_ || !impl_->plan) throw std::runtime_error("InvalidateConstants: not a loaded hip module");
+    if (kxc_hip_plan_invalidate_constants(impl_->plan)) throw std::runtime_error(std::string("InvalidateConstants: ") + kxc_hip_last_error());
+}
+
 std::string CompiledModule::ExecutionPlanJSON() const {
     std::ostringstream os;
     os << "{\"schema_version\":1,\"num_values\":" << impl_->num_values << ",\"output_value\":" << impl_->output_value
@@ -754,6 +764,7 @@ CompiledModule Compiler::LoadExecutionPlan(const std::string& plan_json, Compile
     if (kxc_hip_plan_num_nodes(impl->plan) != static_cast<int32_t>(impl->execs.size()))
         throw std::runtime_error("LoadExecutionPlan: node list and launch plan disagree");
     impl->workspace_bytes = static_cast<size_t>(hip.at("workspace_bytes").integer);
+    if (config->hip_constants_frozen) kxc_hip_plan_freeze_constants(impl->plan, 1);
     impl->ready = true;
     impl->status = "loaded from an execution plan";
     return CompiledModule(impl);

@@ -234,6 +234,7 @@ RuntimeSession::RuntimeSession(Function relay_func, api::CompileConfig config,
     internal_config_->hip_fuse = config->hip_fuse;
     internal_config_->hip_concurrent_branches = config->hip_concurrent_branches;
     internal_config_->hip_winograd = config->hip_winograd;
+    internal_config_->hip_constants_frozen = config->hip_constants_frozen;
     internal_config_->sync_after_run = config->sync_after_run;
 }
 
@@ -257,7 +258,21 @@ void RuntimeSession::Run(const std::vector<void*>& args, const std::vector<std::
         exact->Run(args);
         return;
     }
-    if (api::CompiledModule* fuzzy = cache_.GetFuzzy(sig)) {
+    // A fuzzy candidate was compiled for other (larger) extents.  On the host back end the reference runs it on
+    // the caller's buffers (src/runtime/runtime_session.cc:63-75); on the hip target that would make device kernels
+    // read and write past allocations sized for the smaller shape, so there a fuzzy candidate counts as a miss and
+    // the exact shape is compiled on the calling thread.
+    const bool device_buffers = config_->target.defined() && config_->target->kind == "hip";
+    api::CompiledModule* fuzzy = cache_.GetFuzzy(sig);
+    if (fuzzy && device_buffers) {
+        if (profile_context_) {
+            profiling::EventSpec skipped = SessionEvent("cache_fuzzy_skipped_device_buffers");
+            skipped.fields["shape_hash"] = hash;
+            profile_context_->RecordInstant(std::move(skipped), profiling::CurrentRunId(), profiling::CurrentSpanId());
+        }
+        fuzzy = nullptr;
+    }
+    if (fuzzy) {
         {
             profiling::ScopedSpan hit(profile_context_, SessionEvent("cache_fuzzy_hit"));
             hit.AddField("shape_hash", hash);

@@ -706,9 +706,12 @@ int RunAdaptive(const std::string& bundle_dir) {
         std::vector<float> xd = {1, 2, 3, 4, 5, 6}, yd = {10, 20, 30}, out(6, 0.0f);
         StagedArgs staged({In(xd), In(yd), Out(out)});
         const std::vector<std::vector<int64_t>> small = {{2, 3}, {3}};
+        const bool device = g_mode != "cpu";
         session.Run(staged.args, small);                                  // fuzzy hit, seen once: nothing scheduled
         session.WaitAll();
-        Check(session.CachedKernelCount() == 1, "first fuzzy hit schedules nothing");
+        // (on the hip target a module compiled for larger extents never runs on the caller's device buffers: the
+        //  fuzzy candidate counts as a miss and the exact shape is compiled at once)
+        Check(session.CachedKernelCount() == (device ? 2 : 1), "first run of the smaller shape");
         session.Run(staged.args, small);                                  // fuzzy hit, seen twice: background compile
         session.WaitAll();
         Check(session.CachedKernelCount() == 2, "second fuzzy hit compiles the exact shape in the background");
@@ -717,7 +720,9 @@ int RunAdaptive(const std::string& bundle_dir) {
         session.WaitAll();
         staged.Fetch();
         ExpectNear(out, {11, 22, 33, 14, 25, 36});
-        Check(session.GetStatus() == "RuntimeSession{cached=2, pending=0, completed=1, total_runs=4}", "status: " + session.GetStatus());
+        Check(session.GetStatus() == (device ? "RuntimeSession{cached=2, pending=0, completed=0, total_runs=4}"
+                                             : "RuntimeSession{cached=2, pending=0, completed=1, total_runs=4}"),
+              "status: " + session.GetStatus());
         Check(session.PendingCompileCount() == 0, "nothing pending");
         // a shape nothing cached can serve: compiled on the calling thread
         RuntimeSession cold(make_add(2), config, ctx);
@@ -754,7 +759,9 @@ int RunAdaptive(const std::string& bundle_dir) {
         module.WarmUp({{8, 3}});
         staged.Fetch();
         ExpectNear(out, {0, 2, 0, 4, 0, 6});
-        Check(module.GetStatus() == "RuntimeSession{cached=3, pending=0, completed=1, total_runs=2}", "adaptive module status: " + module.GetStatus());
+        Check(module.GetStatus() == (g_mode != "cpu" ? "RuntimeSession{cached=3, pending=0, completed=0, total_runs=2}"
+                                                     : "RuntimeSession{cached=3, pending=0, completed=1, total_runs=2}"),
+              "adaptive module status: " + module.GetStatus());
         // a non-adaptive module accepts the shape overload and ignores the shapes
         auto plain = kxc::api::Compiler::Compile(relu, MakeConfig());
         std::fill(out.begin(), out.end(), 0.0f);

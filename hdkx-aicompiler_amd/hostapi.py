@@ -73,6 +73,16 @@ class CompiledResNet18:
         if lib().kxc_host_module_enable_graph(self._h, 1 if enable else 0) != 0:
             raise hipabi.KxcHipError(lib().kxc_host_last_error().decode())
 
+    def freeze_constants(self, frozen=True):
+        """Serving mode: the weights will not change behind the module's back, so Winograd layers transform their
+        filters once instead of at the start of every run."""
+        if lib().kxc_host_module_freeze_constants(self._h, 1 if frozen else 0) != 0:
+            raise hipabi.KxcHipError(lib().kxc_host_last_error().decode())
+
+    def invalidate_constants(self):
+        if lib().kxc_host_module_invalidate_constants(self._h) != 0:
+            raise hipabi.KxcHipError(lib().kxc_host_last_error().decode())
+
     def close(self):
         if self._h:
             lib().kxc_host_module_free(self._h)

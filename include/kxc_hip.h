@@ -296,13 +296,19 @@ int32_t kxc_hip_plan_add_conv2d(kxc_hip_plan* plan, const kxc_hip_conv2d_desc* d
                                 kxc_hip_buf w, kxc_hip_buf bias, kxc_hip_buf residual, kxc_hip_buf y);
 /* The same operator through kxc_hip_conv2d_winograd_nchw_f32.  `w` is the OIHW weight tensor as the reference
  * passes it (a module constant among the packed arguments); `u` is a workspace region of
- * kxc_hip_conv2d_winograd_weight_bytes bytes that no other node uses.  The node transforms w into u on the first
- * run and again whenever a different pointer arrives for w; a caller that rewrites the weights in place calls
- * kxc_hip_plan_invalidate_constants. */
+ * kxc_hip_conv2d_winograd_weight_bytes bytes that no other node uses.
+ * By default every run starts with ONE launch that transforms the weights of all the plan's Winograd nodes from
+ * the pointers passed to that run, so a run always sees the current contents of its constants, like the CPU
+ * backend, which re-reads every constant on every call (src/codegen/compiled_kernel.cc:41-55).
+ * kxc_hip_plan_freeze_constants(plan, 1) is the serving mode: the caller promises that the weight tensors do not
+ * change; they are transformed when first seen and again only when a different pointer arrives (a run on another
+ * stream is ordered after the transforms), and kxc_hip_plan_invalidate_constants forces a new transform after an
+ * in-place update. */
 int32_t kxc_hip_plan_add_conv2d_winograd(kxc_hip_plan* plan, const kxc_hip_conv2d_desc* desc, kxc_hip_buf x,
                                          kxc_hip_buf w, kxc_hip_buf bias, kxc_hip_buf residual, kxc_hip_buf y,
                                          kxc_hip_buf u);
 int32_t kxc_hip_plan_invalidate_constants(kxc_hip_plan* plan);
+int32_t kxc_hip_plan_freeze_constants(kxc_hip_plan* plan, int32_t frozen);
 int32_t kxc_hip_plan_add_pool2d(kxc_hip_plan* plan, const kxc_hip_pool2d_desc* desc, kxc_hip_buf x,
                                 kxc_hip_buf y);
 int32_t kxc_hip_plan_add_global_avg_pool2d(kxc_hip_plan* plan, int64_t n, int64_t c, int64_t h,

@@ -385,9 +385,12 @@ def test_conv_winograd_full_batch_properties(pkg, synth):
         assert_close(host(one), host(fast[17:18]), tol=1e-4, what="batch independence")
 
 
-def test_plan_winograd_node_transforms_constants_once(pkg, synth, fast_orc):
-    """A plan's Winograd node takes the OIHW weights as a packed argument, transforms them on the first run and when
-    another tensor is passed; the serialised plan keeps the node."""
+def test_plan_winograd_node_constants(pkg, synth, fast_orc):
+    """A plan's Winograd node takes the OIHW weights as a packed argument.  By default every run transforms them
+    again (one launch per plan), so weights rewritten in place at the same address are seen, as the CPU backend
+    would see them; with frozen constants they are transformed when a pointer is first seen, an in-place update
+    needs invalidate_constants, and a run on another stream is ordered after the transform.  The serialised plan
+    keeps the node."""
     n, c, h, o = 4, 16, 12, 64
     x = synth.uniform((n, c, h, h), 7200)
     w1 = synth.normal((o, c, 3, 3), 7201, 0.1); w2 = synth.normal((o, c, 3, 3), 7202, 0.1)
@@ -400,16 +403,45 @@ def test_plan_winograd_node_transforms_constants_once(pkg, synth, fast_orc):
     assert "winograd" in plan.node_symbol(0)
     xd, w1d, w2d, bd = dev(x), dev(w1), dev(w2), dev(b)
     y = torch.empty((n, o, h, h), device="cuda")
-    for wd, wh in ((w1d, w1), (w1d, w1), (w2d, w2)):
+    want1 = fast_orc.conv_chain(x, w1, b, 1, 1, None, True)
+    want2 = fast_orc.conv_chain(x, w2, b, 1, 1, None, True)
+    for wd, want in ((w1d, want1), (w1d, want1), (w2d, want2)):
         plan.run([xd, wd, bd, y]); torch.cuda.synchronize()
-        assert_close(host(y), fast_orc.conv_chain(x, wh, b, 1, 1, None, True), what="plan winograd")
-    w2d.copy_(w1d); plan.invalidate_constants()          # rewritten in place: the caller says so
+        assert_close(host(y), want, what="plan winograd")
+    # default: rewritten in place at the same pointer, nothing said -- the next run uses the new contents
+    w2d.copy_(w1d)
     plan.run([xd, w2d, bd, y]); torch.cuda.synchronize()
-    assert_close(host(y), fast_orc.conv_chain(x, w1, b, 1, 1, None, True), what="plan winograd after invalidate")
-    again = pkg.Plan.deserialize(plan.serialize(), 0)
+    assert_close(host(y), want1, what="plan winograd after an in-place update")
+    # the same through a captured graph: the transform is part of the replay
+    stream = torch.cuda.Stream()
+    plan.enable_graph(True)
+    with torch.cuda.stream(stream):
+        for k, (src, want) in enumerate(((w2, want2), (w2, want2), (w1, want1), (w2, want2))):
+            w2d.copy_(dev(src)); y.zero_()
+            plan.run([xd, w2d, bd, y], stream.cuda_stream); stream.synchronize()
+            assert_close(host(y), want, what="graph replay %d sees the current weights" % k)
+    plan.enable_graph(False)
+    # frozen: transformed once per pointer
+    plan.freeze_constants(True)
+    w2d.copy_(dev(w2))
+    plan.run([xd, w2d, bd, y]); torch.cuda.synchronize()
+    assert_close(host(y), want2, what="frozen: first run transforms")
+    w2d.copy_(w1d)                                        # behind the plan's back: stale by contract
+    plan.run([xd, w2d, bd, y]); torch.cuda.synchronize()
+    assert_close(host(y), want2, what="frozen: an unannounced in-place update is not seen")
+    plan.invalidate_constants()
+    other = torch.cuda.Stream()
+    with torch.cuda.stream(other):                        # transform enqueued on this stream ...
+        plan.run([xd, w2d, bd, y], other.cuda_stream)
     y2 = torch.empty_like(y)
-    again.run([xd, w1d, bd, y2]); torch.cuda.synchronize()
-    assert_bit_exact(host(y2), host(y), "deserialised winograd plan")
+    plan.run([xd, w2d, bd, y2])                           # ... and a run on another stream waits for it
+    torch.cuda.synchronize()
+    assert_close(host(y), want1, what="frozen: after invalidate")
+    assert_bit_exact(host(y2), host(y), "frozen: run on a second stream after the transform")
+    again = pkg.Plan.deserialize(plan.serialize(), 0)
+    y3 = torch.empty_like(y)
+    again.run([xd, w1d, bd, y3]); torch.cuda.synchronize()
+    assert_bit_exact(host(y3), host(y), "deserialised winograd plan")
 
 
 @pytest.mark.parametrize("shape", [(1, 64, 56, 56, 128, 2), (1, 256, 14, 14, 512, 2), (2, 8, 5, 7, 40, 1), (3, 24, 9, 6, 33, 2),
