@@ -32,6 +32,7 @@
 #include <cstring>
 #include <type_traits>
 #include <mutex>
+#include <string>
 #include <vector>
 
 #include "common.h"
@@ -65,6 +66,15 @@ struct ConvArgs {
     int32_t p_tiles, o_tiles, num_tiles, tiles_per_xcd, o_fastest;
     uint32_t flags;
     FastDiv div_wp, div_hp, div_ohw, div_ow, div_otiles, div_ptiles, div_gsplit;
+    // Second output of the DS kernels: a 1x1 convolution with the same strides and no padding on the same input,
+    // y2[n,o,oh,ow] = sum_c x[n,c,oh*sh,ow*sw] * w2[o,c] (+ bias2[o]).  Its operand is one tap of this
+    // convolution's window (the centre tap of a 3x3 window with padding 1), which the staged patch already holds;
+    // ds_off is that tap's offset inside a channel's patch.
+    const float* w2;
+    const float* bias2;
+    float* y2;
+    uint32_t w2_bytes;
+    int32_t ds_off;
 };
 
 __device__ __forceinline__ float relu_sel(float v) { return (v > 0.0f) ? v : 0.0f; }
@@ -97,9 +107,14 @@ typedef __attribute__((address_space(3))) void* lds_ptr_t;
 // TPAIR: how the two k values of one matrix instruction are chosen.  false: the same filter tap of two adjacent
 // channels (CC even).  true: two consecutive taps of ONE channel (an odd tap count gets a zero-weight partner):
 // for a 3-channel 7x7 first layer that is 75 k-steps instead of the 98 that pairing channels 2 and "3" costs.
-template <int KH, int KW, int CC, int WO, int WP, int RO, int RP, int PPT, int KS, bool TPAIR = false>
+//
+// DS: the workgroup also produces the second output described in ConvArgs (a residual block's 1x1 downsample next
+// to the block's first 3x3 convolution): per chunk CC/2 more k-steps that read the window's centre tap and a
+// second, small weight tile [2 planes][TO][CC/2], into a second set of accumulators.
+template <int KH, int KW, int CC, int WO, int WP, int RO, int RP, int PPT, int KS, bool TPAIR = false, bool DS = false>
 __global__ void __launch_bounds__(64 * WO * WP * KS) __attribute__((amdgpu_waves_per_eu(2)))
 conv_mfma_kernel(const ConvArgs a) {
+    static_assert(!(DS && TPAIR), "the second output pairs channels");
     constexpr int NW = WO * WP;                               // waves per reduction group
     constexpr int TO = 32 * RO * WO;
     constexpr int TP = 32 * RP * WP;
@@ -112,6 +127,14 @@ conv_mfma_kernel(const ConvArgs a) {
     constexpr int WSEG = WSZ / 64;                            // 64-float segments of the weight tile
     constexpr int WPT = (WSEG + NW - 1) / NW;                 // weight segments per wave
     constexpr int PF = (RO * RP >= 4) ? 1 : (RO * RP == 2 ? 2 : 3);   // operand prefetch distance in k-steps
+    // second weight tile (DS): element L = plane*PLB + row*KS2B + pair, channel = 2*pair + plane
+    constexpr int NS2 = DS ? CC / 2 : 0;                      // k-steps of the second output per chunk
+    constexpr int KS2B = (CC / 2) | 1;
+    constexpr int PLB = (TO * KS2B + 63) / 64 * 64 + 32;
+    constexpr int WSZB = DS ? 2 * PLB : 0;
+    constexpr int WSEGB = WSZB / 64;
+    constexpr int WPTB = (WSEGB + NW - 1) / NW;
+    constexpr int NST = NS + NS2;                             // all k-steps of a chunk
 
     extern __shared__ float lds[];
     const int tid = threadIdx.x;
@@ -132,10 +155,11 @@ conv_mfma_kernel(const ConvArgs a) {
     const int c_lo = split * a.cps;                           // this workgroup's chunks: [c_lo, c_hi)
     const int c_hi = min(a.nchunks, c_lo + a.cps);
     const int iters = (c_hi - c_lo + KS - 1) / KS;            // chunk steps of every reduction group
-    // per group: [xs0][ws0][xs1][ws1]; the second pair exists only when a group has more than one chunk
-    float* const xs0 = lds + kgroup * (iters > 1 ? 2 : 1) * (xs_size + WSZ);
-    float* const ws0 = xs0 + xs_size;
-    float* const xs1 = ws0 + WSZ;
+    // per group: [xs0][ws0][vs0][xs1][ws1][vs1] (vs: the second output's weight tile); the second set exists only
+    // when a group has more than one chunk
+    float* const xs0 = lds + kgroup * (iters > 1 ? 2 : 1) * (xs_size + WSZ + WSZB);
+    float* const ws0 = xs0 + xs_size;                 // (vs0 = ws0 + WSZ)
+    float* const xs1 = ws0 + WSZ + WSZB;
     float* const ws1 = xs1 + xs_size;
 
     const int wave_o = wave / WP;
@@ -164,6 +188,7 @@ conv_mfma_kernel(const ConvArgs a) {
 
     const __amdgpu_buffer_rsrc_t xr = make_rsrc(a.x, a.x_bytes);
     const __amdgpu_buffer_rsrc_t wr = make_rsrc(a.w, a.w_bytes);
+    const __amdgpu_buffer_rsrc_t w2r = make_rsrc(DS ? a.w2 : a.w, DS ? a.w2_bytes : 0u);
 
     // ---- per-thread load tables (byte offsets; kOobOffset reads as 0)
     uint32_t goff[PPT];
@@ -179,7 +204,20 @@ conv_mfma_kernel(const ConvArgs a) {
     // weight tile element L = plane*PL + row*KS2 + col; col = pair*KHW + tap with channel = 2*pair + plane, or
     // (TPAIR) col = channel*TPS + s with tap = 2*s + plane
     uint32_t woff[WPT];
+    uint32_t woff2[WPTB > 0 ? WPTB : 1];
     auto weight_table = [&](int channels_left) {
+        if (DS) {
+#pragma unroll
+            for (int i = 0; i < WPTB; ++i) {
+                const int L = (wave + i * NW) * 64 + lane;
+                const int plane = L >= PLB ? 1 : 0;
+                const int rem = L - plane * PLB;
+                const int row = rem / KS2B, pair = rem - row * KS2B;
+                const int cl = 2 * pair + plane;
+                const bool ok = L < WSZB && row < TO && pair < NS2 && (o0 + row) < a.O && cl < channels_left;
+                woff2[i] = ok ? static_cast<uint32_t>((o0 + row) * a.C + cl) * 4u : kOobOffset;
+            }
+        }
 #pragma unroll
         for (int i = 0; i < WPT; ++i) {
             const int L = (wave + i * NW) * 64 + lane;
@@ -208,24 +246,38 @@ conv_mfma_kernel(const ConvArgs a) {
         ybase[j] = (m < a.M) ? n * a.O * a.OHW + rem : -1;
     }
     int wbase[RO];
+    int wbase2[RO];
 #pragma unroll
-    for (int i = 0; i < RO; ++i) wbase[i] = half * PL + ((wave_o * RO + i) * 32 + r) * KS2;
+    for (int i = 0; i < RO; ++i) {
+        wbase[i] = half * PL + ((wave_o * RO + i) * 32 + r) * KS2;
+        wbase2[i] = half * PLB + ((wave_o * RO + i) * 32 + r) * KS2B;
+    }
 
     floatx16 acc[RO][RP];
+    floatx16 acc2[DS ? RO : 1][DS ? RP : 1];
 #pragma unroll
     for (int i = 0; i < RO; ++i)
 #pragma unroll
         for (int j = 0; j < RP; ++j)
 #pragma unroll
-            for (int g = 0; g < 16; ++g) acc[i][j][g] = 0.0f;
+            for (int g = 0; g < 16; ++g) {
+                acc[i][j][g] = 0.0f;
+                if constexpr (DS) acc2[i][j][g] = 0.0f;
+            }
 
     // The loads of one chunk as NOPS separate operations (CC*PPT patch segments, then WPT weight segments), so
     // that the main loop can issue them a few at a time between matrix instructions instead of in one burst
     // during which the wave feeds nothing to the matrix pipe.
-    constexpr int NOPS = CC * PPT + WPT;
+    constexpr int NOPS = CC * PPT + WPT + WPTB;
     auto issue_op = [&](int j, int chunk, float* xs, float* ws) {
         const int c0 = chunk * CC;
-        if (j < CC * PPT) {
+        if (DS && j >= CC * PPT + WPT) {
+            const int i = j - CC * PPT - WPT;
+            const int seg = wave + i * NW;
+            if (seg < WSEGB)
+                __builtin_amdgcn_raw_ptr_buffer_load_lds(w2r, (lds_ptr_t)(ws + WSZ + seg * 64), 4, woff2[i < WPTB ? i : 0],
+                                                         static_cast<uint32_t>(c0) * 4u, 0, 0);
+        } else if (j < CC * PPT) {
             const int cl = j / PPT, i = j - cl * PPT;
             const int seg = wave + i * NW;
             if (seg < xsegs) {
@@ -265,13 +317,23 @@ conv_mfma_kernel(const ConvArgs a) {
         float* const nws = (it & 1) ? ws0 : ws1;
         if (has_next && (chunk + KS) * CC + CC > a.C) weight_table(a.C - (chunk + KS) * CC);   // partial last chunk (rare)
         if (chunk < c_hi) {
-        constexpr int OPS_PER_STEP = (NOPS + NS - 1) / NS;
+        constexpr int OPS_PER_STEP = (NOPS + NST - 1) / NST;
 
         // k-steps of this chunk: step = pair * KHW + tap.  Operands are fetched from LDS PF steps ahead of
         // the matrix instruction that consumes them (rotating register sets; all indices are compile-time
         // after unrolling), so the LDS latency is covered by the PF matrix instructions in between.
         auto fetch = [&](int step, float (&av)[RO], float (&bv)[RP]) {
             int koff_x, koff_w;
+            if (DS && step >= NS) {
+                // second output: the window's centre tap of channel pair step - NS, weights from the second tile
+                const int cp = step - NS;
+                koff_x = (2 * cp) * a.chs + a.ds_off;
+#pragma unroll
+                for (int i = 0; i < RO; ++i) av[i] = ws[WSZ + wbase2[i] + cp];
+#pragma unroll
+                for (int j = 0; j < RP; ++j) bv[j] = xs[xbase[j] + koff_x];
+                return;
+            }
             if (TPAIR) {
                 // lane half h reads tap 2*s + h of channel c; a tap past the end (zero weight) re-reads the last one
                 const int c = step / TPS, s2 = 2 * (step - c * TPS);
@@ -294,17 +356,25 @@ conv_mfma_kernel(const ConvArgs a) {
         float av[PF + 1][RO], bv[PF + 1][RP];
 #pragma unroll
         for (int p = 0; p < PF; ++p)
-            if (p < NS) fetch(p, av[p % (PF + 1)], bv[p % (PF + 1)]);
+            if (p < NST) fetch(p, av[p % (PF + 1)], bv[p % (PF + 1)]);
 #pragma unroll
-        for (int step = 0; step < NS; ++step) {
-            if (step + PF < NS) fetch(step + PF, av[(step + PF) % (PF + 1)], bv[(step + PF) % (PF + 1)]);
+        for (int step = 0; step < NST; ++step) {
+            if (step + PF < NST) fetch(step + PF, av[(step + PF) % (PF + 1)], bv[(step + PF) % (PF + 1)]);
             __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
             for (int i = 0; i < RO; ++i)
 #pragma unroll
-                for (int j = 0; j < RP; ++j)
+                for (int j = 0; j < RP; ++j) {
+                    if constexpr (DS) {
+                        if (step >= NS) {
+                            acc2[i][j] = __builtin_amdgcn_mfma_f32_32x32x2f32(av[step % (PF + 1)][i], bv[step % (PF + 1)][j],
+                                                                              acc2[i][j], 0, 0, 0);
+                            continue;
+                        }
+                    }
                     acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x2f32(av[step % (PF + 1)][i], bv[step % (PF + 1)][j],
                                                                      acc[i][j], 0, 0, 0);
+                }
             __builtin_amdgcn_sched_barrier(0);
             // next chunk's loads, a few per k-step, issued while this step's matrix instructions execute
             if (has_next) {
@@ -321,34 +391,44 @@ conv_mfma_kernel(const ConvArgs a) {
     }
 
     // ---- combine the reduction groups: groups 1.. park their accumulators in LDS (the tiles are dead after
-    // the loop's last barrier), group 0 adds them in group order
+    // the loop's last barrier), group 0 adds them in group order; the second output's accumulators follow in a
+    // second round through the same LDS
     if (KS > 1) {
         float* const red = lds;
-        if (kgroup > 0) {
+        auto combine = [&](auto& accs) {
+            if (kgroup > 0) {
 #pragma unroll
-            for (int i = 0; i < RO; ++i)
+                for (int i = 0; i < RO; ++i)
 #pragma unroll
-                for (int j = 0; j < RP; ++j)
+                    for (int j = 0; j < RP; ++j)
 #pragma unroll
-                    for (int g = 0; g < 16; ++g)
-                        red[((((kgroup - 1) * NW + wave) * RO * RP + i * RP + j) * 16 + g) * 64 + lane] = acc[i][j][g];
+                        for (int g = 0; g < 16; ++g)
+                            red[((((kgroup - 1) * NW + wave) * RO * RP + i * RP + j) * 16 + g) * 64 + lane] = accs[i][j][g];
+            }
+            __syncthreads();
+            if (kgroup == 0) {
+#pragma unroll
+                for (int kg = 1; kg < KS; ++kg)
+#pragma unroll
+                    for (int i = 0; i < RO; ++i)
+#pragma unroll
+                        for (int j = 0; j < RP; ++j)
+#pragma unroll
+                            for (int g = 0; g < 16; ++g)
+                                accs[i][j][g] += red[((((kg - 1) * NW + wave) * RO * RP + i * RP + j) * 16 + g) * 64 + lane];
+            }
+        };
+        combine(acc);
+        if constexpr (DS) {
+            __syncthreads();
+            combine(acc2);
         }
-        __syncthreads();
         if (kgroup > 0) return;
-#pragma unroll
-        for (int kg = 1; kg < KS; ++kg)
-#pragma unroll
-            for (int i = 0; i < RO; ++i)
-#pragma unroll
-                for (int j = 0; j < RP; ++j)
-#pragma unroll
-                    for (int g = 0; g < 16; ++g)
-                        acc[i][j][g] += red[((((kg - 1) * NW + wave) * RO * RP + i * RP + j) * 16 + g) * 64 + lane];
     }
 
     // ---- epilogue: accumulator register g of a block holds row 8*(g/4) + 4*half + g%4, column r
     if (a.gsplit > 1) {
-        // raw partial sums of this split; conv_split_reduce_kernel finishes the layer
+        // raw partial sums of this split; conv_split_reduce_kernel finishes the layer (never with a second output)
         float* const part = a.partial + static_cast<int64_t>(split) * a.out_elems;
         if (KS == 1 || kgroup == 0) {
 #pragma unroll
@@ -368,13 +448,7 @@ conv_mfma_kernel(const ConvArgs a) {
     // and drops a store, so absent channels and pixels past the end need no branches, and every load is issued
     // before the first store (a wait for a load also waits for all stores issued before it: with loads and stores
     // interleaved each of the 16 rows would cost a full memory round trip).
-    const bool has_bias = (a.flags & KXC_HIP_CONV_BIAS) != 0;
-    const bool has_res = (a.flags & KXC_HIP_CONV_RESIDUAL) != 0;
-    const bool do_relu = (a.flags & KXC_HIP_CONV_RELU) != 0;
     const uint32_t y_bytes = static_cast<uint32_t>(a.out_elems) * 4u;
-    const __amdgpu_buffer_rsrc_t yr = make_rsrc(a.y, y_bytes);
-    const __amdgpu_buffer_rsrc_t rr = make_rsrc(has_res ? a.res : a.y, has_res ? y_bytes : 0u);
-    const __amdgpu_buffer_rsrc_t br = make_rsrc(has_bias ? a.bias : a.y, has_bias ? static_cast<uint32_t>(a.O) * 4u : 0u);
     const uint32_t plane = static_cast<uint32_t>(a.OHW) * 4u;
     uint32_t yb[RP];
 #pragma unroll
@@ -384,44 +458,59 @@ conv_mfma_kernel(const ConvArgs a) {
         const int o = channel(i, g);
         return o < a.O ? yb[j] + static_cast<uint32_t>(o) * plane : kOobOffset;
     };
-    float bv[RO][16];
+    auto load_bias = [&](float (&bv)[RO][16], const float* bias, bool has_bias) {
+        const __amdgpu_buffer_rsrc_t br = make_rsrc(has_bias ? bias : a.y, has_bias ? static_cast<uint32_t>(a.O) * 4u : 0u);
 #pragma unroll
-    for (int i = 0; i < RO; ++i)
+        for (int i = 0; i < RO; ++i)
 #pragma unroll
-        for (int g = 0; g < 16; ++g) {
-            const int o = channel(i, g);
-            bv[i][g] = __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(br, o < a.O ? static_cast<uint32_t>(o) * 4u : kOobOffset, 0, 0));
-        }
-    // rows (accumulator registers) per batch of residual loads: the whole block when one block per wave, fewer
-    // for register-blocked tiles so that the staged residual never needs more than 16 registers
-    constexpr int GC = 16 / (RO * RP) < 4 ? 4 : 16 / (RO * RP);
+            for (int g = 0; g < 16; ++g) {
+                const int o = channel(i, g);
+                bv[i][g] = __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(br, o < a.O ? static_cast<uint32_t>(o) * 4u : kOobOffset, 0, 0));
+            }
+    };
+    auto finish = [&](auto& accs, const float (&bv)[RO][16], bool has_bias, const float* res, bool has_res, bool do_relu, float* y) {
+        const __amdgpu_buffer_rsrc_t yr = make_rsrc(y, y_bytes);
+        const __amdgpu_buffer_rsrc_t rr = make_rsrc(has_res ? res : y, has_res ? y_bytes : 0u);
+        // rows (accumulator registers) per batch of residual loads: the whole block when one block per wave, fewer
+        // for register-blocked tiles so that the staged residual never needs more than 16 registers
+        constexpr int GC = 16 / (RO * RP) < 4 ? 4 : 16 / (RO * RP);
 #pragma unroll
-    for (int gc = 0; gc < 16; gc += GC) {
-        float q[RO][RP][GC];
-        if (has_res) {
+        for (int gc = 0; gc < 16; gc += GC) {
+            float q[RO][RP][GC];
+            if (has_res) {
 #pragma unroll
-            for (int i = 0; i < RO; ++i)
+                for (int i = 0; i < RO; ++i)
 #pragma unroll
-                for (int g = 0; g < GC; ++g)
+                    for (int g = 0; g < GC; ++g)
 #pragma unroll
-                    for (int j = 0; j < RP; ++j)
-                        q[i][j][g] = __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(rr, out_off(i, gc + g, j), 0, 0));
-        }
+                        for (int j = 0; j < RP; ++j)
+                            q[i][j][g] = __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(rr, out_off(i, gc + g, j), 0, 0));
+            }
 #pragma unroll
-        for (int i = 0; i < RO; ++i) {
+            for (int i = 0; i < RO; ++i) {
 #pragma unroll
-            for (int g = 0; g < GC; ++g) {
+                for (int g = 0; g < GC; ++g) {
 #pragma unroll
-                for (int j = 0; j < RP; ++j) {
-                    float v = acc[i][j][gc + g];
-                    if (has_bias) v = __fadd_rn(v, bv[i][gc + g]);
-                    if (has_res) v = __fadd_rn(v, q[i][j][g]);
-                    if (do_relu) v = relu_sel(v);
-                    __builtin_amdgcn_raw_buffer_store_b32(__builtin_bit_cast(uint32_t, v), yr, out_off(i, gc + g, j), 0, 0);
+                    for (int j = 0; j < RP; ++j) {
+                        float v = accs[i][j][gc + g];
+                        if (has_bias) v = __fadd_rn(v, bv[i][gc + g]);
+                        if (has_res) v = __fadd_rn(v, q[i][j][g]);
+                        if (do_relu) v = relu_sel(v);
+                        __builtin_amdgcn_raw_buffer_store_b32(__builtin_bit_cast(uint32_t, v), yr, out_off(i, gc + g, j), 0, 0);
+                    }
                 }
             }
         }
-    }
+    };
+    // both outputs' bias values are loaded before anything is stored; the second output has no other loads, so its
+    // stores simply follow the main output's
+    const bool has_bias = (a.flags & KXC_HIP_CONV_BIAS) != 0;
+    float bias_main[RO][16];
+    float bias_second[DS ? RO : 1][16];
+    load_bias(bias_main, a.bias, has_bias);
+    if constexpr (DS) load_bias(bias_second, a.bias2, a.bias2 != nullptr);
+    finish(acc, bias_main, has_bias, a.res, (a.flags & KXC_HIP_CONV_RESIDUAL) != 0, (a.flags & KXC_HIP_CONV_RELU) != 0, a.y);
+    if constexpr (DS) finish(acc2, bias_second, a.bias2 != nullptr, nullptr, false, false, a.y2);
 }
 
 // ------------------------------------------------------------------------------------------
@@ -534,17 +623,27 @@ struct Variant {
     const char* name;
     int kh, kw, cc, to, tp, nw, ppt, ks, tpair;
     void (*kernel)(const ConvArgs);
+    void (*ds_kernel)(const ConvArgs);      // the same tile with the second (1x1 downsample) output, or nullptr
 };
 
 #define KXC_VARIANT(KH, KW, CC, WO, WP, RO, RP, PPT)                                                   \
     {"mfma_k" #KH "x" #KW "_c" #CC "_o" #WO "x" #RO "_p" #WP "x" #RP, KH, KW, CC, 32 * RO * WO, 32 * RP * WP, \
-     WO * WP, PPT, 1, 0, conv_mfma_kernel<KH, KW, CC, WO, WP, RO, RP, PPT, 1>}
+     WO * WP, PPT, 1, 0, conv_mfma_kernel<KH, KW, CC, WO, WP, RO, RP, PPT, 1>, nullptr}
 #define KXC_VARIANT_KS(KH, KW, CC, WO, WP, RO, RP, PPT, KS)                                            \
     {"mfma_k" #KH "x" #KW "_c" #CC "_o" #WO "x" #RO "_p" #WP "x" #RP "_ks" #KS, KH, KW, CC, 32 * RO * WO,   \
-     32 * RP * WP, WO * WP, PPT, KS, 0, conv_mfma_kernel<KH, KW, CC, WO, WP, RO, RP, PPT, KS>}
+     32 * RP * WP, WO * WP, PPT, KS, 0, conv_mfma_kernel<KH, KW, CC, WO, WP, RO, RP, PPT, KS>, nullptr}
 #define KXC_VARIANT_TP(KH, KW, CC, WO, WP, RO, RP, PPT)                                                \
     {"mfma_k" #KH "x" #KW "_t" #CC "_o" #WO "x" #RO "_p" #WP "x" #RP, KH, KW, CC, 32 * RO * WO, 32 * RP * WP, \
-     WO * WP, PPT, 1, 1, conv_mfma_kernel<KH, KW, CC, WO, WP, RO, RP, PPT, 1, true>}
+     WO * WP, PPT, 1, 1, conv_mfma_kernel<KH, KW, CC, WO, WP, RO, RP, PPT, 1, true>, nullptr}
+// (tiles that also exist with the second output)
+#define KXC_VARIANT_DS(KH, KW, CC, WO, WP, RO, RP, PPT)                                                \
+    {"mfma_k" #KH "x" #KW "_c" #CC "_o" #WO "x" #RO "_p" #WP "x" #RP, KH, KW, CC, 32 * RO * WO, 32 * RP * WP, \
+     WO * WP, PPT, 1, 0, conv_mfma_kernel<KH, KW, CC, WO, WP, RO, RP, PPT, 1>,                          \
+     conv_mfma_kernel<KH, KW, CC, WO, WP, RO, RP, PPT, 1, false, true>}
+#define KXC_VARIANT_KS_DS(KH, KW, CC, WO, WP, RO, RP, PPT, KS)                                         \
+    {"mfma_k" #KH "x" #KW "_c" #CC "_o" #WO "x" #RO "_p" #WP "x" #RP "_ks" #KS, KH, KW, CC, 32 * RO * WO,   \
+     32 * RP * WP, WO * WP, PPT, KS, 0, conv_mfma_kernel<KH, KW, CC, WO, WP, RO, RP, PPT, KS>,          \
+     conv_mfma_kernel<KH, KW, CC, WO, WP, RO, RP, PPT, KS, false, true>}
 
 // name = mfma_k<filter>_c<channels per chunk>_o<waves x blocks along output channels>_p<waves x blocks
 // along pixels>; tile = 32*blocks*waves in each direction.
@@ -556,18 +655,18 @@ struct Variant {
 // entry that fits the shape, except that launches too small to fill the GPU take the entry with
 // the most workgroups.
 const Variant kVariants[] = {
-    KXC_VARIANT(3, 3, 4, 1, 4, 1, 1, 4),   // 32 x 128, 4 waves            (default)
-    KXC_VARIANT(3, 3, 4, 1, 8, 1, 1, 2),   // 32 x 256, 8 waves            (14x14 maps: fewer weight refills)
-    KXC_VARIANT(3, 3, 2, 1, 4, 1, 1, 4),   // 32 x 128, 2-channel chunks   (stride-2 56->28: smaller patch)
-    KXC_VARIANT(3, 3, 4, 1, 2, 1, 1, 8),   // 32 x 64, 2 waves             (small launches)
+    KXC_VARIANT_DS(3, 3, 4, 1, 4, 1, 1, 4),   // 32 x 128, 4 waves            (default)
+    KXC_VARIANT_DS(3, 3, 4, 1, 8, 1, 1, 2),   // 32 x 256, 8 waves            (14x14 maps: fewer weight refills)
+    KXC_VARIANT_DS(3, 3, 2, 1, 4, 1, 1, 4),   // 32 x 128, 2-channel chunks   (stride-2 56->28: smaller patch)
+    KXC_VARIANT_DS(3, 3, 4, 1, 2, 1, 1, 8),   // 32 x 64, 2 waves             (small launches)
     KXC_VARIANT(3, 3, 4, 2, 4, 1, 1, 4),   // 64 x 128, 8 waves
-    KXC_VARIANT(3, 3, 4, 2, 8, 1, 1, 2),   // 64 x 256, 16 waves
+    KXC_VARIANT_DS(3, 3, 4, 2, 8, 1, 1, 2),   // 64 x 256, 16 waves
     KXC_VARIANT(3, 3, 4, 1, 4, 2, 1, 4),   // 64 x 128, 4 waves of 64x32
     KXC_VARIANT(3, 3, 4, 1, 4, 2, 2, 4),   // 64 x 256, 4 waves of 64x64
     KXC_VARIANT(3, 3, 8, 1, 8, 1, 1, 2),   // 8-channel chunks
-    KXC_VARIANT_KS(3, 3, 4, 1, 4, 1, 1, 4, 2),   // 32 x 128, reduction split 2 ways (8 waves)
-    KXC_VARIANT_KS(3, 3, 4, 1, 2, 1, 1, 8, 4),   // 32 x 64, split 4 ways (8 waves)
-    KXC_VARIANT_KS(3, 3, 4, 1, 2, 1, 1, 8, 8),   // 32 x 64, split 8 ways (16 waves)
+    KXC_VARIANT_KS_DS(3, 3, 4, 1, 4, 1, 1, 4, 2),   // 32 x 128, reduction split 2 ways (8 waves)
+    KXC_VARIANT_KS_DS(3, 3, 4, 1, 2, 1, 1, 8, 4),   // 32 x 64, split 4 ways (8 waves)
+    KXC_VARIANT_KS_DS(3, 3, 4, 1, 2, 1, 1, 8, 8),   // 32 x 64, split 8 ways (16 waves)
     KXC_VARIANT(1, 1, 8, 1, 4, 2, 1, 4),   // 64 x 128
     KXC_VARIANT(1, 1, 8, 1, 4, 2, 2, 6),   // 64 x 256
     KXC_VARIANT(1, 1, 8, 2, 2, 1, 1, 6),   // 64 x 64
@@ -613,7 +712,8 @@ int32_t MaxTileRows(const ConvArgs& a, int kh, int tp) {
 constexpr size_t kMaxLdsBytes = 160 * 1024;  // LDS of one gfx950 compute unit
 constexpr int kNumCUs = 256;
 
-bool Fits(const Variant& v, const ConvArgs& a, Choice* out) {
+bool Fits(const Variant& v, const ConvArgs& a, Choice* out, bool ds = false) {
+    if (ds && !v.ds_kernel) return false;
     const int32_t rows = MaxTileRows(a, v.kh, v.tp);
     const int64_t P = static_cast<int64_t>(rows) * a.Wp;
     const int64_t segs = (P + 63) / 64;
@@ -631,7 +731,8 @@ bool Fits(const Variant& v, const ConvArgs& a, Choice* out) {
     if (v.ks > 1 && nchunks < 2 * v.ks) return false;          // not enough reduction to split
     const int buffers = (nchunks + v.ks - 1) / v.ks > 1 ? 2 : 1;   // a single chunk step needs no second buffer
     const size_t xs_size = (static_cast<size_t>(v.cc) * chs + 31) & ~static_cast<size_t>(31);
-    size_t lds = static_cast<size_t>(v.ks) * buffers * (xs_size + 2 * static_cast<size_t>(pl)) * sizeof(float);
+    const int plb = (v.to * ((v.cc / 2) | 1) + 63) / 64 * 64 + 32;                 // second output's weight planes
+    size_t lds = static_cast<size_t>(v.ks) * buffers * (xs_size + 2 * static_cast<size_t>(pl) + (ds ? 2 * static_cast<size_t>(plb) : 0)) * sizeof(float);
     const size_t red = static_cast<size_t>(v.ks - 1) * v.to * v.tp * sizeof(float);   // partial accumulators
     if (red > lds) lds = red;
     if (lds > kMaxLdsBytes) return false;
@@ -642,7 +743,7 @@ bool Fits(const Variant& v, const ConvArgs& a, Choice* out) {
 }
 
 // Picks the MFMA variant for a shape, or leaves choice.v == nullptr for the direct kernel.
-void Select(const ConvArgs& a, int kh, int kw, Choice* choice) {
+void Select(const ConvArgs& a, int kh, int kw, Choice* choice, bool ds = false) {
     choice->v = nullptr;
     if (a.O < 32 || a.M < 32) return;
     // 32-bit byte offsets inside the kernel
@@ -688,7 +789,7 @@ void Select(const ConvArgs& a, int kh, int kw, Choice* choice) {
             if (pass == 0 && !(forced && *forced) && (!preferred || std::strcmp(preferred, v.name) != 0)) continue;
             if (v.to > a.O && v.to > 32) continue;    // do not spend matrix work on absent output channels
             Choice c;
-            if (!Fits(v, a, &c)) continue;
+            if (!Fits(v, a, &c, ds)) continue;
             if (pass == 0 || (forced && *forced)) { *choice = c; return; }
             const int64_t waves = CeilDiv(a.M, v.tp) * CeilDiv(a.O, v.to) * v.nw * v.ks;
             if (!first_fit.v && v.ks == 1) { first_fit = c; first_waves = waves; }
@@ -803,9 +904,24 @@ int32_t NoAllocScratch(float** out) {
 
 // The operator behind both entry points.  no_alloc: the partial sums of a split reduction go to the file-scope
 // scratch array instead of the grow-only per-stream buffer, and a launch that would need more is refused.
+// The second output of kxc_hip_conv2d_pair_nchw_f32 (see ConvArgs).
+struct SecondOutput {
+    const float* w2 = nullptr;
+    const float* bias2 = nullptr;
+    float* y2 = nullptr;
+};
+
+// Whether a convolution can carry the second output: the 1x1 convolution's operand x[n,c,oh*sh,ow*sw] must be a tap
+// of this window, i.e. the padding is a multiple of the dilation and lies inside the filter.
+bool PairTap(const kxc_hip_conv2d_desc* d, int* rh, int* rw) {
+    if (d->pad_h % d->dil_h != 0 || d->pad_w % d->dil_w != 0) return false;
+    *rh = d->pad_h / d->dil_h; *rw = d->pad_w / d->dil_w;
+    return *rh < d->kh && *rw < d->kw;
+}
+
 int32_t Conv2dRun(const kxc_hip_conv2d_desc* desc, const float* x, const float* w, const float* bias,
-                  const float* residual, float* y, void* stream, bool no_alloc) {
-    const char* const who = no_alloc ? "kxc_hip_conv2d_nchw_f32_noalloc" : "kxc_hip_conv2d_nchw_f32";
+                  const float* residual, float* y, void* stream, bool no_alloc, const SecondOutput* second = nullptr) {
+    const char* const who = second ? "kxc_hip_conv2d_pair_nchw_f32" : no_alloc ? "kxc_hip_conv2d_nchw_f32_noalloc" : "kxc_hip_conv2d_nchw_f32";
     ConvArgs a;
     if (int32_t rc = FillArgs(desc, &a, who)) return rc;
     const int64_t total = static_cast<int64_t>(a.N) * a.O * a.OHW;
@@ -821,7 +937,7 @@ int32_t Conv2dRun(const kxc_hip_conv2d_desc* desc, const float* x, const float* 
     // A filter one row high with a vertical stride touches only every stride-th input row (the 1x1/2
     // downsample convolutions): the matrix kernel then sees an image of OH rows that are stride rows apart, so
     // the skipped rows are neither loaded nor staged.
-    if (UseSmall1x1(desc, a)) {
+    if (!second && UseSmall1x1(desc, a)) {
         a.div_ohw = MakeFastDiv(a.OHW); a.div_ow = MakeFastDiv(a.OW);
         const dim3 grid(static_cast<unsigned>(CeilDiv(a.O, 32)), static_cast<unsigned>(CeilDiv(a.M, 32)));
         // eight waves split a long reduction (each keeps an even number of channels)
@@ -834,7 +950,15 @@ int32_t Conv2dRun(const kxc_hip_conv2d_desc* desc, const float* x, const float* 
     ConvArgs direct_args = a;
     ApplyRowView(&a, desc->kh);
     Choice c;
-    if (!(desc->flags & KXC_HIP_CONV_FORCE_DIRECT) && a.M > 0) Select(a, desc->kh, desc->kw, &c);
+    if (!(desc->flags & KXC_HIP_CONV_FORCE_DIRECT) && a.M > 0) Select(a, desc->kh, desc->kw, &c, second != nullptr);
+    if (second) {
+        int rh = 0, rw = 0;
+        KXC_HIP_REQUIRE(c.v && c.v->ds_kernel && PairTap(desc, &rh, &rw), "%s: no kernel with a second output covers this shape", who);
+        KXC_HIP_REQUIRE(second->w2 && second->y2, "%s: NULL pointer", who);
+        a.w2 = second->w2; a.bias2 = second->bias2; a.y2 = second->y2;
+        a.w2_bytes = static_cast<uint32_t>(static_cast<int64_t>(a.O) * a.C * 4);
+        a.ds_off = rh * a.dh * a.Wp + rw * a.dw;
+    }
     if (c.v) {
         a.chs = c.chs;
         a.nchunks = (a.C + c.v->cc - 1) / c.v->cc;
@@ -851,7 +975,7 @@ int32_t Conv2dRun(const kxc_hip_conv2d_desc* desc, const float* x, const float* 
         SplitScratchLease lease;      // held until the adding kernel is enqueued
         {
             int split = 1;
-            SplitOverWorkgroups(c, a.nchunks, tiles, total, &split);
+            if (!second) SplitOverWorkgroups(c, a.nchunks, tiles, total, &split);      // (a second output is never split)
             if (split > 1) {
                 a.cps = static_cast<int32_t>(CeilDiv(a.nchunks, split));
                 a.gsplit = static_cast<int32_t>(CeilDiv(a.nchunks, a.cps));      // no empty split
@@ -883,12 +1007,13 @@ int32_t Conv2dRun(const kxc_hip_conv2d_desc* desc, const float* x, const float* 
         dim3 grid(static_cast<unsigned>(a.tiles_per_xcd * 8));
         if (c.lds_bytes > 64 * 1024) {
             // above the default 64 KiB the dynamic LDS size has to be granted per kernel
-            KXC_HIP_CALL(hipFuncSetAttribute(reinterpret_cast<const void*>(c.v->kernel),
+            KXC_HIP_CALL(hipFuncSetAttribute(reinterpret_cast<const void*>(second ? c.v->ds_kernel : c.v->kernel),
                                              hipFuncAttributeMaxDynamicSharedMemorySize,
                                              static_cast<int>(c.lds_bytes)),
                          "hipFuncSetAttribute(MaxDynamicSharedMemorySize)");
         }
-        hipLaunchKernelGGL(c.v->kernel, NoteGrid(grid), NoteBlock(dim3(64 * c.v->nw * c.v->ks)), NoteLds(c.lds_bytes), s, a);
+        void (*const kernel)(const ConvArgs) = second ? c.v->ds_kernel : c.v->kernel;
+        hipLaunchKernelGGL(kernel, NoteGrid(grid), NoteBlock(dim3(64 * c.v->nw * c.v->ks)), NoteLds(c.lds_bytes), s, a);
         if (int32_t rc = CheckLaunch(c.v->name)) return rc;
         if (a.gsplit > 1) {
             SplitReduceArgs r;
@@ -930,6 +1055,46 @@ int32_t kxc_hip_conv2d_nchw_f32_noalloc(const kxc_hip_conv2d_desc* desc, const f
 }
 
 size_t kxc_hip_conv2d_noalloc_scratch_bytes(void) { return kNoAllocScratchBytes; }
+
+// Variant of the pair kernel for a shape, or nullptr.
+static const Variant* PairVariant(const kxc_hip_conv2d_desc* desc) {
+    ConvArgs a;
+    if (!desc || FillArgs(desc, &a, "kxc_hip_conv2d_pair_supported") != KXC_HIP_OK) return nullptr;
+    int rh = 0, rw = 0;
+    if ((desc->flags & KXC_HIP_CONV_FORCE_DIRECT) || a.M <= 0 || !PairTap(desc, &rh, &rw)) return nullptr;
+    if (desc->kh == 1 && desc->kw == 1) return nullptr;
+    Choice c;
+    Select(a, desc->kh, desc->kw, &c, true);
+    if (!c.v || !c.v->ds_kernel) return nullptr;
+    // A launch small enough to split its reduction over workgroups (batch 1-4 of the deep layers) gains more from
+    // that split than from the shared input, and a second output is never split: such shapes keep two launches.
+    if (!std::getenv("KXC_HIP_CONV_VARIANT")) {
+        const int32_t nchunks = (a.C + c.v->cc - 1) / c.v->cc;
+        int split = 1;
+        SplitOverWorkgroups(c, nchunks, CeilDiv(a.M, c.v->tp) * CeilDiv(a.O, c.v->to), static_cast<int64_t>(a.N) * a.O * a.OHW, &split);
+        if (split > 1) return nullptr;
+    }
+    return c.v;
+}
+
+int32_t kxc_hip_conv2d_pair_supported(const kxc_hip_conv2d_desc* desc) { return PairVariant(desc) ? 1 : 0; }
+
+const char* kxc_hip_conv2d_pair_variant(const kxc_hip_conv2d_desc* desc) {
+    // static storage: one name per table entry
+    static std::once_flag once;
+    static std::vector<std::string> names;
+    std::call_once(once, [] { for (int i = 0; i < kNumVariants; ++i) names.push_back(std::string(kVariants[i].name) + "_ds"); });
+    const Variant* v = PairVariant(desc);
+    return v ? names[static_cast<size_t>(v - kVariants)].c_str() : "unsupported";
+}
+
+int32_t kxc_hip_conv2d_pair_nchw_f32(const kxc_hip_conv2d_desc* desc, const float* x, const float* w, const float* bias,
+                                     const float* residual, float* y, const float* w2, const float* bias2, float* y2,
+                                     void* stream) {
+    SecondOutput second;
+    second.w2 = w2; second.bias2 = bias2; second.y2 = y2;
+    return Conv2dRun(desc, x, w, bias, residual, y, stream, false, &second);
+}
 
 int32_t kxc_hip_conv2d_scratch_needed(const kxc_hip_conv2d_desc* desc, size_t* out_bytes) {
     KXC_HIP_REQUIRE(out_bytes != nullptr, "kxc_hip_conv2d_scratch_needed: out_bytes is NULL");

@@ -179,6 +179,27 @@ int32_t kxc_hip_plan_add_conv2d_winograd(kxc_hip_plan* plan, const kxc_hip_conv2
     return KXC_HIP_OK;
 }
 
+int32_t kxc_hip_plan_add_conv2d_pair(kxc_hip_plan* plan, const kxc_hip_conv2d_desc* desc, kxc_hip_buf x, kxc_hip_buf w,
+                                     kxc_hip_buf bias, kxc_hip_buf residual, kxc_hip_buf y, kxc_hip_buf w2, kxc_hip_buf bias2,
+                                     kxc_hip_buf y2) {
+    const char* who = "kxc_hip_plan_add_conv2d_pair";
+    KXC_PLAN_BEGIN(who);
+    KXC_HIP_REQUIRE(desc != nullptr, "%s: desc is NULL", who);
+    KXC_HIP_REQUIRE(kxc_hip_conv2d_pair_supported(desc), "%s: no kernel with a second output covers this shape", who);
+    KXC_PLAN_BUF(w2, false, who); KXC_PLAN_BUF(bias2, true, who); KXC_PLAN_BUF(y2, false, who);
+    if (int32_t rc = kxc_hip_plan_add_conv2d(plan, desc, x, w, bias, residual, y)) return rc;
+    Node& n = plan->nodes.back();
+    n.i32[0] = 2;                      // params = {w2, bias2, y2}
+    n.params = {w2, bias2, y2};
+    n.symbol = std::string("kxc_conv2d_nchw_f32.") + kxc_hip_conv2d_pair_variant(desc);
+    if (desc->flags & KXC_HIP_CONV_BIAS) n.symbol += "+bias";
+    if (desc->flags & KXC_HIP_CONV_RESIDUAL) n.symbol += "+add";
+    if (desc->flags & KXC_HIP_CONV_RELU) n.symbol += "+relu";
+    n.symbol += "|conv1x1";
+    if (bias2.kind != KXC_HIP_BUF_NONE) n.symbol += "+bias";
+    return KXC_HIP_OK;
+}
+
 int32_t kxc_hip_plan_invalidate_constants(kxc_hip_plan* plan) {
     KXC_HIP_REQUIRE(plan != nullptr, "kxc_hip_plan_invalidate_constants: plan is NULL");
     for (Node& n : plan->nodes) n.transformed_from = nullptr;
@@ -551,6 +572,15 @@ int32_t RunNode(kxc_hip_plan* plan, Node& n, void** args, void* s) {
                     rc = kxc_hip_conv2d_winograd_nchw_f32(&n.conv, static_cast<const float*>(B(0)), static_cast<const float*>(B(5)),
                                                           static_cast<const float*>(B(2)), static_cast<const float*>(B(3)),
                                                           static_cast<float*>(B(4)), s);
+                    break;
+                }
+                if (n.i32[0] == 2) {
+                    rc = kxc_hip_conv2d_pair_nchw_f32(&n.conv, static_cast<const float*>(B(0)), static_cast<const float*>(B(1)),
+                                                      static_cast<const float*>(B(2)), static_cast<const float*>(B(3)),
+                                                      static_cast<float*>(B(4)),
+                                                      static_cast<const float*>(Resolve(plan, n.params[0], args)),
+                                                      static_cast<const float*>(Resolve(plan, n.params[1], args)),
+                                                      static_cast<float*>(Resolve(plan, n.params[2], args)), s);
                     break;
                 }
                 rc = kxc_hip_conv2d_nchw_f32(&n.conv, static_cast<const float*>(B(0)), static_cast<const float*>(B(1)),
@@ -936,6 +966,10 @@ int32_t kxc_hip_plan_deserialize(const char* text, int32_t device_id, kxc_hip_mo
         if (n.kind == NodeKind::kConv2D && n.i32[0] == 1 &&
             (!kxc_hip_conv2d_winograd_supported(&n.conv) || n.bufs[5].kind != KXC_HIP_BUF_WORKSPACE))
             return fail("bad Winograd convolution node");
+        if (n.kind == NodeKind::kConv2D && n.i32[0] == 2 &&
+            (!kxc_hip_conv2d_pair_supported(&n.conv) || n.params.size() != 3 || n.params[0].kind == KXC_HIP_BUF_NONE ||
+             n.params[2].kind == KXC_HIP_BUF_NONE))
+            return fail("bad convolution-pair node");
         if (n.kind == NodeKind::kModuleKernel) {
             // generated kernels are found by name in the modules the caller compiled from the saved source
             for (int32_t m = 0; m < num_modules && !n.function; ++m) {

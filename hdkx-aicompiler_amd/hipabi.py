@@ -80,6 +80,7 @@ def lib():
         _lib.kxc_hip_target_kind.restype = C.c_char_p
         _lib.kxc_hip_conv2d_variant.restype = C.c_char_p
         _lib.kxc_hip_conv2d_winograd_variant.restype = C.c_char_p
+        _lib.kxc_hip_conv2d_pair_variant.restype = C.c_char_p
         _lib.kxc_hip_qconv2d_c16_variant.restype = C.c_char_p
         _lib.kxc_hip_plan_node_symbol.restype = C.c_char_p
         _lib.kxc_hip_plan_workspace.restype = C.c_void_p
@@ -144,10 +145,45 @@ def conv2d(x, w, bias=None, residual=None, stride=1, pad=0, dil=1, relu=False, f
     flags = (CONV_BIAS if bias is not None else 0) | (CONV_RESIDUAL if residual is not None else 0) | \
             (CONV_RELU if relu else 0) | (CONV_FORCE_DIRECT if force_direct else 0)
     d = conv_desc(tuple(x.shape), tuple(w.shape), stride, pad, dil, flags)
+    if out is not None:
+        _check_out(out, conv_out_shape(d))
     y = out if out is not None else torch.empty(conv_out_shape(d), dtype=torch.float32, device=x.device)
     entry = lib().kxc_hip_conv2d_nchw_f32_noalloc if no_alloc else lib().kxc_hip_conv2d_nchw_f32
     _check(entry(C.byref(d), _p(x), _p(w), _p(bias), _p(residual), _p(y), _stream()))
     return y
+
+
+def _check_out(out, shape, name="out"):
+    import torch
+    _need(out, torch.float32, name)
+    if tuple(out.shape) != tuple(shape):
+        raise KxcHipError("%s has shape %s, the operator writes %s" % (name, tuple(out.shape), tuple(shape)))
+
+
+def conv2d_pair_supported(x_shape, w_shape, stride, pad, dil=1):
+    d = conv_desc(x_shape, w_shape, stride, pad, dil, 0)
+    return bool(lib().kxc_hip_conv2d_pair_supported(C.byref(d)))
+
+
+def conv2d_pair_variant(x_shape, w_shape, stride, pad, dil=1):
+    d = conv_desc(x_shape, w_shape, stride, pad, dil, 0)
+    return lib().kxc_hip_conv2d_pair_variant(C.byref(d)).decode()
+
+
+def conv2d_pair(x, w, bias, residual, w2, bias2, stride=1, pad=0, dil=1, relu=False):
+    """(conv(x, w) [+bias] [+residual] [relu], conv1x1(x, w2, same stride, no padding) [+bias2]) in one launch."""
+    import torch
+    for t, nm in ((x, "x"), (w, "w"), (bias, "bias"), (residual, "residual"), (w2, "w2"), (bias2, "bias2")):
+        _need(t, torch.float32, nm)
+    if x.shape[1] != w.shape[1] or tuple(w2.shape) != (w.shape[0], w.shape[1], 1, 1):
+        raise KxcHipError("conv2d_pair: w2 must be [o, c, 1, 1] for w [o, c, kh, kw]")
+    flags = (CONV_BIAS if bias is not None else 0) | (CONV_RESIDUAL if residual is not None else 0) | (CONV_RELU if relu else 0)
+    d = conv_desc(tuple(x.shape), tuple(w.shape), stride, pad, dil, flags)
+    y = torch.empty(conv_out_shape(d), dtype=torch.float32, device=x.device)
+    y2 = torch.empty_like(y)
+    _check(lib().kxc_hip_conv2d_pair_nchw_f32(C.byref(d), _p(x), _p(w), _p(bias), _p(residual), _p(y), _p(w2), _p(bias2), _p(y2),
+                                              _stream()))
+    return y, y2
 
 
 def conv2d_winograd_supported(x_shape, w_shape, stride, pad, dil=1):
@@ -191,6 +227,8 @@ def conv2d_winograd(x, u, w_shape, bias=None, residual=None, pad=1, relu=False, 
     flags = (CONV_BIAS if bias is not None else 0) | (CONV_RESIDUAL if residual is not None else 0) | \
             (CONV_RELU if relu else 0)
     d = conv_desc(tuple(x.shape), tuple(w_shape), 1, pad, 1, flags)
+    if out is not None:
+        _check_out(out, conv_out_shape(d))
     y = out if out is not None else torch.empty(conv_out_shape(d), dtype=torch.float32, device=x.device)
     _check(lib().kxc_hip_conv2d_winograd_nchw_f32(C.byref(d), _p(x), _p(u), _p(bias), _p(residual), _p(y), _stream()))
     return y
@@ -248,6 +286,8 @@ def pool2d(x, k, s, pad, ceil_mode=False, avg=False, out=None):
     import torch
     _need(x, torch.float32, "x")
     d = pool_desc(tuple(x.shape), k, s, pad, ceil_mode, avg)
+    if out is not None:
+        _check_out(out, pool_out_shape(d))
     y = out if out is not None else torch.empty(pool_out_shape(d), dtype=torch.float32, device=x.device)
     _check(lib().kxc_hip_pool2d_f32(C.byref(d), _p(x), _p(y), _stream()))
     return y
@@ -506,6 +546,9 @@ class Plan:
 
     def add_conv2d_winograd(self, desc, x, w, bias, residual, y, u):
         _check(lib().kxc_hip_plan_add_conv2d_winograd(self._h, C.byref(desc), x, w, bias, residual, y, u))
+
+    def add_conv2d_pair(self, desc, x, w, bias, residual, y, w2, bias2, y2):
+        _check(lib().kxc_hip_plan_add_conv2d_pair(self._h, C.byref(desc), x, w, bias, residual, y, w2, bias2, y2))
 
     def invalidate_constants(self):
         _check(lib().kxc_hip_plan_invalidate_constants(self._h))

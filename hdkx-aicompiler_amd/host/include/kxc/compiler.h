@@ -35,6 +35,7 @@ struct CompileConfigNode {
     bool hip_use_handwritten{true};    // false: every operator goes through the TIR -> HIP generator
     bool hip_fuse{true};               // fold bias / residual add / ReLU into convolution launches
     bool hip_concurrent_branches{true};   // run a block's downsample convolution beside its first 3x3 convolution
+    bool hip_pair_convolutions{true};     // a block's 1x1 downsample as a second output of its first convolution's launch
     bool hip_winograd{true};              // 3x3 stride-1 convolutions with constant weights as Winograd F(2x2,3x3) where faster
     // Winograd layers transform their (constant) filters on the GPU.  false (default): at the start of every Run, from
     // the pointers passed to that Run, so a Run always sees the constants' current contents, like the CPU back end.
@@ -101,6 +102,9 @@ public:
     // hip target: see CompileConfigNode::hip_constants_frozen.
     void FreezeConstants(bool frozen);
     void InvalidateConstants();
+    // hip target: one Run with a HIP event between consecutive launches; returns each launch's duration in
+    // nanoseconds, in the order of GetKernelExecs() (waits for the last launch).
+    std::vector<int64_t> RunTimed(const std::vector<void*>& packed_args);
 
 private:
     friend class Compiler;

@@ -66,7 +66,19 @@ struct HIPDispatchContext {
     // empty when the configuration rules that out.
     std::vector<bool> input_constant;
     std::function<HIPBuffer(int64_t)> alloc_persistent;
+    // A second call of the same operator on the same first input whose value this launch produces as well (offered
+    // only after the operator's "FHIPPairQuery" said yes for the two calls): its attributes, input types, inputs
+    // (the first one equals inputs[0]) and output.
+    bool has_pair = false;
+    Attrs pair_attrs;
+    Array<Type> pair_input_types;
+    Array<HIPBuffer> pair_inputs;
+    HIPBuffer pair_output;
 };
+// Whether one launch of call A (attrs, input types, and whether a ReLU / residual is fused behind it is irrelevant)
+// can also produce call B, an unfused call of the same operator on the same first input.
+using FHIPPairQuery = std::function<bool(const Attrs& a_attrs, const Array<Type>& a_inputs, const std::vector<bool>& a_constant,
+                                         const Attrs& b_attrs, const Array<Type>& b_inputs)>;
 // Appends the launch(es) for one call to the plan; returns the kernel_symbol, or "" to decline (the
 // call is then compiled through the code generator).
 using FHIPDispatch = std::function<std::string(const HIPDispatchContext&, kxc_hip_plan*)>;

@@ -80,6 +80,21 @@ int kxc_host_module_invalidate_constants(void* module) {
     }
 }
 
+// durations_ns[i] = duration of launch i (order of kxc_host_module_symbols); *count = number of launches.
+int kxc_host_module_run_timed(void* module, void** packed_args, int num_args, long long* durations_ns, int capacity, int* count) {
+    try {
+        const std::vector<int64_t> d =
+            static_cast<ModuleHandle*>(module)->module.RunTimed(std::vector<void*>(packed_args, packed_args + num_args));
+        *count = static_cast<int>(d.size());
+        if (capacity < *count) { g_error = "kxc_host_module_run_timed: capacity too small"; return 1; }
+        for (size_t i = 0; i < d.size(); ++i) durations_ns[i] = d[i];
+        return 0;
+    } catch (const std::exception& e) {
+        g_error = e.what();
+        return 1;
+    }
+}
+
 int kxc_host_module_is_ready(void* module) { return static_cast<ModuleHandle*>(module)->module.IsReady() ? 1 : 0; }
 const char* kxc_host_module_status(void* module) {
     g_error = static_cast<ModuleHandle*>(module)->module.GetStatus();

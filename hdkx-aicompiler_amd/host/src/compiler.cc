@@ -301,6 +301,52 @@ private:
             auto it = group_of_tail_.find(c);
             if (it != group_of_tail_.end()) order.push_back(it->second);
         }
+        // Pairs: a call B whose launch can ride on an earlier call A of the same operator on the same input (the
+        // operator's FHIPPairQuery decides: a block's 1x1 downsample on its first convolution).  B's group leaves
+        // the emission order; A's launch writes both values.  B's other inputs must exist before A runs (function
+        // parameters or constants), and B is unfused and comes after A, so nothing between them reads B's value.
+        std::vector<int> carries(groups_.size(), -1);
+        const char* pair_env = std::getenv("KXC_HIP_PAIR");                     // "0" switches pairing off
+        if (cfg_->hip_fuse && cfg_->hip_use_handwritten && cfg_->hip_pair_convolutions && !(pair_env && pair_env[0] == '0')) {
+            std::vector<bool> merged(groups_.size(), false);
+            for (size_t sb = 1; sb < order.size(); ++sb) {
+                const Group& gb = groups_[order[sb]];
+                const auto* opb = gb.head->op.As<OpNode>();
+                const auto* query = OpAttr<relay::FHIPPairQuery>(opb, "FHIPPairQuery");
+                if (!query || gb.head != gb.tail || gb.residual || gb.fused_relu || !IsF32(gb.head->checked_type_)) continue;
+                if (gb.tail == f_->body.get() || !OpAttr<relay::FHIPDispatch>(opb, "FHIPDispatch")) continue;
+                bool inputs_ready = true;
+                for (size_t i = 1; i < gb.head->args.size(); ++i)
+                    inputs_ready = inputs_ready && arg_index_.count(Resolve(gb.head->args[i].get())) > 0;
+                if (!inputs_ready) continue;
+                Array<Type> b_types;
+                for (const auto& a : gb.head->args) b_types.push_back(a.checked_type());
+                for (size_t sa = 0; sa < sb; ++sa) {
+                    const size_t ia = order[sa];
+                    const Group& ga = groups_[ia];
+                    if (merged[ia] || carries[ia] >= 0 || ga.head->op.get() != gb.head->op.get()) continue;
+                    if (ga.tail == f_->body.get() || !IsF32(ga.head->checked_type_)) continue;
+                    if (Resolve(ga.head->args[0].get()) != Resolve(gb.head->args[0].get())) continue;
+                    if (TT(ga.tail->checked_type_)->shape != TT(gb.tail->checked_type_)->shape) continue;
+                    Array<Type> a_types;
+                    std::vector<bool> a_const;
+                    for (const auto& a : ga.head->args) {
+                        a_types.push_back(a.checked_type());
+                        a_const.push_back(dynamic_cast<const ConstantNode*>(Resolve(a.get())) != nullptr);
+                    }
+                    const char* wino_env = std::getenv("KXC_HIP_WINOGRAD");
+                    if (!cfg_->hip_winograd || (wino_env && wino_env[0] == '0')) a_const.assign(a_const.size(), false);
+                    if (!(*query)(ga.head->attrs, a_types, a_const, gb.head->attrs, b_types)) continue;
+                    carries[ia] = static_cast<int>(order[sb]);
+                    merged[order[sb]] = true;
+                    break;
+                }
+            }
+            std::vector<size_t> kept;
+            for (size_t g : order)
+                if (!merged[g]) kept.push_back(g);
+            order.swap(kept);
+        }
         // Independent branches: a hand-written convolution whose value is only the residual operand of a later
         // fused convolution (a block's 1x1 downsample) and that does not depend on the group emitted just before
         // it moves in front of that group and runs on the plan's side lane, concurrently with it; the consumer
@@ -351,6 +397,8 @@ private:
             if (is_alias[order[step]]) continue;
             for (const auto& a : g.head->args) last_use[Resolve(a.get())] = static_cast<int>(step);
             if (g.residual) last_use[Resolve(g.residual)] = static_cast<int>(step);
+            if (carries[order[step]] >= 0)
+                for (const auto& a : groups_[carries[order[step]]].head->args) last_use[Resolve(a.get())] = static_cast<int>(step);
         }
         last_use[Resolve(f_->body.get())] = static_cast<int>(order.size());
         // a side-lane launch may still be reading its operands until the join has been enqueued
@@ -393,6 +441,17 @@ private:
                     arena_.top += (std::max<int64_t>(bytes, 1) + 255) / 256 * 256;
                     return relay::HIPBuffer{KXC_HIP_BUF_WORKSPACE, off};
                 };
+            const Group* carried = carries[order[step]] >= 0 ? &groups_[carries[order[step]]] : nullptr;
+            if (carried) {
+                slot_[carried->tail] = arena_.Alloc(TypeBytes(carried->tail->checked_type_));
+                ctx.has_pair = true;
+                ctx.pair_attrs = carried->head->attrs;
+                for (const auto& a : carried->head->args) {
+                    ctx.pair_input_types.push_back(a.checked_type());
+                    ctx.pair_inputs.push_back(BufferOf(a.get()));
+                }
+                ctx.pair_output = {KXC_HIP_BUF_WORKSPACE, slot_[carried->tail].first};
+            }
             ctx.out_type = g.tail->checked_type_;
             ctx.output = out;
             ctx.fused_relu = g.fused_relu;
@@ -404,6 +463,10 @@ private:
             for (const auto& a : g.head->args) info.input_values.push_back(value_id_.at(a.get()));
             if (g.residual) info.input_values.push_back(value_id_.at(g.residual));
             info.output_values.push_back(value_id_.at(g.tail));
+            if (carried) {
+                for (size_t i = 1; i < carried->head->args.size(); ++i) info.input_values.push_back(value_id_.at(carried->head->args[i].get()));
+                info.output_values.push_back(value_id_.at(carried->tail));
+            }
 
             std::string symbol;
             const int32_t first_node = kxc_hip_plan_num_nodes(m_->plan);
@@ -426,7 +489,7 @@ private:
                     kxc_hip_plan_set_concurrency(m_->plan, first_node, side ? 1 : 0, joins[order[step]] ? 1 : 0))
                     throw std::runtime_error(std::string("plan_set_concurrency failed: ") + kxc_hip_last_error());
             } else {
-                if (g.fused_relu || g.residual) throw std::runtime_error("hip back end: operator declined a fused launch: " + op->name);
+                if (g.fused_relu || g.residual || carried) throw std::runtime_error("hip back end: operator declined a fused launch: " + op->name);
                 EmitGenerated(g, ctx, info, static_cast<int>(step));
             }
             // release everything whose last reader has now been enqueued
@@ -668,6 +731,20 @@ size_t CompiledModule::workspace_bytes() const { return impl_->workspace_bytes; 
 void CompiledModule::EnableGraphReplay(bool enable) {
     if (!impl_ || !impl_->plan) throw std::runtime_error("EnableGraphReplay: not a loaded hip module");
     if (kxc_hip_plan_enable_graph(impl_->plan, enable ? 1 : 0)) throw std::runtime_error(std::string("EnableGraphReplay: ") + kxc_hip_last_error());
+}
+
+std::vector<int64_t> CompiledModule::RunTimed(const std::vector<void*>& packed_args) {
+    if (!impl_ || !impl_->plan || !impl_->ready) throw std::runtime_error("RunTimed: not a loaded hip module");
+    const size_t expect = static_cast<size_t>(impl_->input_count + impl_->constant_count + 1);
+    if (packed_args.size() != expect) throw std::runtime_error("RunTimed: expected " + std::to_string(expect) + " packed arguments");
+    std::vector<kxc_hip_launch_record> records(static_cast<size_t>(kxc_hip_plan_num_nodes(impl_->plan)) + 1);
+    int32_t count = 0;
+    if (kxc_hip_plan_run_profiled(impl_->plan, const_cast<void**>(packed_args.data()), nullptr, records.data(),
+                                  static_cast<int32_t>(records.size()), &count))
+        throw std::runtime_error(std::string("RunTimed: ") + kxc_hip_last_error());
+    std::vector<int64_t> out;
+    for (int32_t i = 0; i < count; ++i) out.push_back(records[i].duration_ns);
+    return out;
 }
 
 void CompiledModule::FreezeConstants(bool frozen) {

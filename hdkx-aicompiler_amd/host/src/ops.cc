@@ -49,11 +49,12 @@ te::Tensor Conv2DCompute(const Attrs& attrs, const Array<te::Tensor>& in, const 
     return te::compute(conv->shape, [&](const Array<tir::Var>& ax) { return conv(ax) + bias(ax[1]); }, "T_conv2d_bias_add");
 }
 
-std::string Conv2DDispatch(const HIPDispatchContext& c, kxc_hip_plan* plan) {
-    const auto* p = c.attrs.As<Conv2DAttrsNode>();
-    if (!p || !IsF32(c.input_types[0]) || !IsF32(c.out_type)) return "";
-    const auto* x = TT(c.input_types[0]);
-    const auto* w = TT(c.input_types[1]);
+bool ConvDesc(const Attrs& attrs, const Array<Type>& input_types, kxc_hip_conv2d_desc* out) {
+    const auto* p = attrs.As<Conv2DAttrsNode>();
+    if (!p || input_types.size() < 2 || !IsF32(input_types[0]) || !IsF32(input_types[1])) return false;
+    const auto* x = TT(input_types[0]);
+    const auto* w = TT(input_types[1]);
+    if (x->shape.size() != 4 || w->shape.size() != 4) return false;
     kxc_hip_conv2d_desc d{};
     d.n = static_cast<int32_t>(x->shape[0]); d.c = static_cast<int32_t>(x->shape[1]);
     d.h = static_cast<int32_t>(x->shape[2]); d.w = static_cast<int32_t>(x->shape[3]);
@@ -61,10 +62,39 @@ std::string Conv2DDispatch(const HIPDispatchContext& c, kxc_hip_plan* plan) {
     d.stride_h = Read2D(p->strides, 0, 1); d.stride_w = Read2D(p->strides, 1, 1);
     d.pad_h = Read2D(p->padding, 0, 0); d.pad_w = Read2D(p->padding, 1, 0);
     d.dil_h = Read2D(p->dilation, 0, 1); d.dil_w = Read2D(p->dilation, 1, 1);
+    *out = d;
+    return true;
+}
+
+// A residual block's first convolution (A) and its 1x1 downsample (B: same input, same strides, no padding, same
+// number of output channels) run as one launch when the library has a kernel with a second output for A's shape
+// and A would not rather run as Winograd.
+bool Conv2DPairQuery(const Attrs& a_attrs, const Array<Type>& a_inputs, const std::vector<bool>& a_constant, const Attrs& b_attrs,
+                     const Array<Type>& b_inputs) {
+    kxc_hip_conv2d_desc a{}, b{};
+    if (!ConvDesc(a_attrs, a_inputs, &a) || !ConvDesc(b_attrs, b_inputs, &b)) return false;
+    if (b.kh != 1 || b.kw != 1 || b.pad_h != 0 || b.pad_w != 0 || b.o != a.o || b.c != a.c) return false;
+    if (b.stride_h != a.stride_h || b.stride_w != a.stride_w) return false;
+    if (a_constant.size() > 1 && a_constant[1] && kxc_hip_conv2d_winograd_preferred(&a)) return false;
+    return kxc_hip_conv2d_pair_supported(&a) != 0;
+}
+
+std::string Conv2DDispatch(const HIPDispatchContext& c, kxc_hip_plan* plan) {
+    kxc_hip_conv2d_desc d{};
+    if (!ConvDesc(c.attrs, c.input_types, &d) || !IsF32(c.out_type)) return "";
     const bool has_bias = c.inputs.size() == 3;
     d.flags = (has_bias ? KXC_HIP_CONV_BIAS : 0u) | (c.has_residual ? KXC_HIP_CONV_RESIDUAL : 0u) |
               (c.fused_relu ? KXC_HIP_CONV_RELU : 0u);
     const kxc_hip_buf none{KXC_HIP_BUF_NONE, 0};
+    if (c.has_pair) {
+        const bool bias2 = c.pair_inputs.size() == 3;
+        Check(kxc_hip_plan_add_conv2d_pair(plan, &d, B(c.inputs[0]), B(c.inputs[1]), has_bias ? B(c.inputs[2]) : none,
+                                           c.has_residual ? B(c.residual) : none, B(c.output), B(c.pair_inputs[1]),
+                                           bias2 ? B(c.pair_inputs[2]) : none, B(c.pair_output)),
+              "nn_conv2d pair dispatch");
+        return std::string("kxc_conv2d_nchw_f32.") + kxc_hip_conv2d_pair_variant(&d) + (has_bias ? "+bias" : "") +
+               (c.has_residual ? "+add" : "") + (c.fused_relu ? "+relu" : "") + "|conv1x1" + (bias2 ? "+bias" : "");
+    }
     // 3x3 stride-1 convolutions with constant weights run as Winograd F(2x2,3x3) when the library expects that to
     // be faster for the shape; the transformed weights get a workspace region of their own.
     if (c.alloc_persistent && c.input_constant.size() > 1 && c.input_constant[1] && kxc_hip_conv2d_winograd_preferred(&d)) {
@@ -207,7 +237,8 @@ void EnsureBuiltinOpsRegistered() {
             .set_attr<FInferType>("FInferType", Conv2DInferType)
             .set_attr<FRelayToTE>("FRelayToTE", Conv2DCompute)
             .set_attr<bool>("THIPFusable", true)
-            .set_attr<FHIPDispatch>("FHIPDispatch", Conv2DDispatch);
+            .set_attr<FHIPDispatch>("FHIPDispatch", Conv2DDispatch)
+            .set_attr<FHIPPairQuery>("FHIPPairQuery", Conv2DPairQuery);
         OpRegEntry::Register("nn_relu")
             .describe("Rectified Linear Unit activation")
             .set_num_inputs(1)

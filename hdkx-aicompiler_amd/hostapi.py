@@ -73,6 +73,21 @@ class CompiledResNet18:
         if lib().kxc_host_module_enable_graph(self._h, 1 if enable else 0) != 0:
             raise hipabi.KxcHipError(lib().kxc_host_last_error().decode())
 
+    def run_timed(self, args, stream=None):
+        """One run with a HIP event between consecutive launches: [(kernel symbol, microseconds)] per launch."""
+        n = len(self.launches())
+        buf = (C.c_longlong * (n + 8))()
+        count = C.c_int(0)
+        if stream is not None:
+            hipabi.lib().kxc_hip_set_stream(0, C.c_void_p(stream))
+        try:
+            if lib().kxc_host_module_run_timed(self._h, args, len(args), buf, n + 8, C.byref(count)) != 0:
+                raise hipabi.KxcHipError(lib().kxc_host_last_error().decode())
+        finally:
+            if stream is not None:
+                hipabi.lib().kxc_hip_set_stream(0, C.c_void_p(0))
+        return [(self.launches()[i], buf[i] / 1e3) for i in range(count.value)]
+
     def freeze_constants(self, frozen=True):
         """Serving mode: the weights will not change behind the module's back, so Winograd layers transform their
         filters once instead of at the start of every run."""

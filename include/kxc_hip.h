@@ -132,6 +132,21 @@ size_t kxc_hip_conv2d_noalloc_scratch_bytes(void);
  * lets a caller see beforehand whether kxc_hip_conv2d_nchw_f32_noalloc takes the shape. */
 int32_t kxc_hip_conv2d_scratch_needed(const kxc_hip_conv2d_desc* desc, size_t* out_bytes);
 
+/* Two nn_conv2d calls on the same input in one launch: the convolution `desc` describes (convolution.cc:38-75, with
+ * its fused epilogue as above) and a 1x1 convolution with the same strides, no padding and the same number of
+ * output channels, y2[n,o,oh,ow] = sum_c x[n,c,oh*stride_h,ow*stride_w] * w2[o,c] (+ bias2[o], NULL = none) -- a
+ * residual block's first 3x3/2 convolution and its 1x1/2 downsample (test/resnet18_ir_dump.cpp:330-352).  The 1x1
+ * operand is the tap (pad/dilation) of the first convolution's window, which its staged input already holds, so
+ * the input is read once and the second launch disappears.  Both outputs equal what the two separate calls give
+ * (the second one bit for bit: same kernel arithmetic).
+ *   ..._supported: 1 when a matrix-core kernel with a second output covers the shape (padding a multiple of the
+ *   dilation and inside the filter, no 1x1 first filter), else 0; ..._variant names it ("unsupported" otherwise). */
+int32_t kxc_hip_conv2d_pair_supported(const kxc_hip_conv2d_desc* desc);
+const char* kxc_hip_conv2d_pair_variant(const kxc_hip_conv2d_desc* desc);
+int32_t kxc_hip_conv2d_pair_nchw_f32(const kxc_hip_conv2d_desc* desc, const float* x, const float* w,
+                                     const float* bias, const float* residual, float* y, const float* w2,
+                                     const float* bias2, float* y2, void* stream);
+
 /* nn_conv2d with a 3x3 filter, stride 1, dilation 1 and c % 4 == 0 as Winograd F(2x2, 3x3) on the matrix cores:
  * same operator and epilogue as kxc_hip_conv2d_nchw_f32 (convolution.cc:38-75, nn.h:107-158) with 2.25x fewer
  * multiplies; the sums are formed in a different order, results agree within the operator's fp32 tolerance.
@@ -307,6 +322,10 @@ int32_t kxc_hip_plan_add_conv2d(kxc_hip_plan* plan, const kxc_hip_conv2d_desc* d
 int32_t kxc_hip_plan_add_conv2d_winograd(kxc_hip_plan* plan, const kxc_hip_conv2d_desc* desc, kxc_hip_buf x,
                                          kxc_hip_buf w, kxc_hip_buf bias, kxc_hip_buf residual, kxc_hip_buf y,
                                          kxc_hip_buf u);
+/* Both convolutions of kxc_hip_conv2d_pair_nchw_f32 as one node. */
+int32_t kxc_hip_plan_add_conv2d_pair(kxc_hip_plan* plan, const kxc_hip_conv2d_desc* desc, kxc_hip_buf x,
+                                     kxc_hip_buf w, kxc_hip_buf bias, kxc_hip_buf residual, kxc_hip_buf y,
+                                     kxc_hip_buf w2, kxc_hip_buf bias2, kxc_hip_buf y2);
 int32_t kxc_hip_plan_invalidate_constants(kxc_hip_plan* plan);
 int32_t kxc_hip_plan_freeze_constants(kxc_hip_plan* plan, int32_t frozen);
 int32_t kxc_hip_plan_add_pool2d(kxc_hip_plan* plan, const kxc_hip_pool2d_desc* desc, kxc_hip_buf x,

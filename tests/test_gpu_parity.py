@@ -159,6 +159,108 @@ def test_conv_reduction_split_over_workgroups(pkg, fast_orc, synth, monkeypatch,
     assert_bit_exact(got2, got1, "split reduction is deterministic")
 
 
+# ------------------------------------------------------------------ convolution pair (3x3 + 1x1 downsample)
+PAIR_SHAPES = [
+    # n, c, h, w, o, k, s, p
+    (2, 64, 56, 56, 128, 3, 2, 1),     # layer2.0: conv1 + downsample
+    (2, 128, 28, 28, 256, 3, 2, 1),    # layer3.0
+    (3, 256, 14, 14, 512, 3, 2, 1),    # layer4.0 (tiles cross image boundaries)
+    (8, 64, 56, 56, 128, 3, 2, 1),     # enough work for the unsplit tiles
+    (16, 256, 14, 14, 512, 3, 2, 1),
+    (1, 30, 17, 19, 96, 3, 2, 1),      # ragged: odd sizes, channels not a multiple of the chunk
+    (2, 7, 9, 33, 40, 3, 1, 1),        # stride 1, output channels not a multiple of the tile
+    (1, 12, 20, 20, 64, 5, 2, 2),      # no 5x5 matrix kernel: refused
+]
+
+
+@pytest.mark.parametrize("shape", PAIR_SHAPES, ids=lambda s: "x".join(map(str, s)))
+def test_conv_pair_against_oracle(pkg, fast_orc, synth, monkeypatch, shape):
+    """A block's first convolution and its 1x1 downsample in one launch: both outputs against the CPU path's two
+    separate convolutions, and the first output bit for bit what the separate matrix-core launch gives."""
+    n, c, h, w, o, k, s, p = shape
+    if k == 5:
+        assert not pkg.conv2d_pair_supported((n, c, h, w), (o, c, k, k), s, p)
+        assert pkg.conv2d_pair_variant((n, c, h, w), (o, c, k, k), s, p) == "unsupported"
+        return
+    if not pkg.conv2d_pair_supported((n, c, h, w), (o, c, k, k), s, p):
+        # a launch this small would rather split its reduction over workgroups: not paired unless that is ruled out
+        assert _scratch_needed(pkg, (n, c, h, w), (o, c, k, k), s, p) > 0
+        monkeypatch.setenv("KXC_HIP_CONV_GSPLIT", "1")
+    assert pkg.conv2d_pair_supported((n, c, h, w), (o, c, k, k), s, p)
+    variant = pkg.conv2d_pair_variant((n, c, h, w), (o, c, k, k), s, p)
+    assert variant.endswith("_ds"), variant
+    seed = 6300 + PAIR_SHAPES.index(shape) * 11
+    x = synth.uniform((n, c, h, w), seed)
+    w1 = synth.normal((o, c, k, k), seed + 1, float(np.sqrt(2.0 / (c * k * k))))
+    b1 = synth.uniform((o,), seed + 2, -0.1, 0.1)
+    w2 = synth.normal((o, c, 1, 1), seed + 3, float(np.sqrt(2.0 / c)))
+    b2 = synth.uniform((o,), seed + 4, -0.1, 0.1)
+    oh, ow = (h + 2 * p - k) // s + 1, (w + 2 * p - k) // s + 1
+    skip = synth.uniform((n, o, oh, ow), seed + 5)
+    want1 = fast_orc.conv_chain(x, w1, b1, s, p, None, True)
+    want2 = fast_orc.conv_chain(x, w2, b2, s, 0, None, False)
+    y1, y2 = pkg.conv2d_pair(dev(x), dev(w1), dev(b1), None, dev(w2), dev(b2), s, p, 1, True)
+    assert_close(host(y1), want1, what=variant + " first output")
+    assert_close(host(y2), want2, what=variant + " second output")
+    # the first output is the single launch's, bit for bit (same tile, same order of sums)
+    alone = pkg.conv2d(dev(x), dev(w1), dev(b1), None, s, p, 1, True)
+    if pkg.conv2d_variant((n, c, h, w), (o, c, k, k), s, p) + "_ds" == variant and _scratch_needed(pkg, (n, c, h, w), (o, c, k, k), s, p) == 0:
+        assert_bit_exact(host(y1), host(alone), "first output of the pair equals the single launch")
+    # residual on the first output, no biases
+    want1 = fast_orc.conv_chain(x, w1, None, s, p, skip, False)
+    want2 = fast_orc.conv2d(x, w2, s, 0)
+    y1, y2 = pkg.conv2d_pair(dev(x), dev(w1), None, dev(skip), dev(w2), None, s, p, 1, False)
+    assert_close(host(y1), want1, what=variant + " first output (+residual)")
+    assert_close(host(y2), want2, what=variant + " second output (bare)")
+
+
+def _scratch_needed(pkg, xs, ws, s, p):
+    import ctypes as C
+    d = pkg.conv_desc(xs, ws, s, p, 1, 0)
+    n = C.c_size_t(0)
+    assert pkg.lib().kxc_hip_conv2d_scratch_needed(C.byref(d), C.byref(n)) == 0
+    return n.value
+
+
+@pytest.mark.parametrize("variant", ["mfma_k3x3_c4_o1x1_p4x1", "mfma_k3x3_c4_o1x1_p8x1", "mfma_k3x3_c2_o1x1_p4x1",
+                                     "mfma_k3x3_c4_o1x1_p2x1", "mfma_k3x3_c4_o2x1_p8x1", "mfma_k3x3_c4_o1x1_p4x1_ks2",
+                                     "mfma_k3x3_c4_o1x1_p2x1_ks4", "mfma_k3x3_c4_o1x1_p2x1_ks8"])
+def test_conv_pair_every_tile(pkg, fast_orc, synth, monkeypatch, variant):
+    """Every tile shape that exists with a second output, forced once (128 -> 256 channels)."""
+    monkeypatch.setenv("KXC_HIP_CONV_VARIANT", variant)
+    # (a forced tile must hold the shape's input patch: the first candidate shape it accepts is used)
+    for n, c, h, o, s, p in ((2, 128, 28, 256, 2, 1), (3, 128, 12, 256, 1, 1)):
+        if pkg.conv2d_pair_variant((n, c, h, h), (o, c, 3, 3), s, p) == variant + "_ds":
+            break
+    else:
+        raise AssertionError("no candidate shape fits " + variant)
+    x = synth.uniform((n, c, h, h), 6500)
+    w1 = synth.normal((o, c, 3, 3), 6501, float(np.sqrt(2.0 / (c * 9))))
+    b1 = synth.uniform((o,), 6502, -0.1, 0.1)
+    w2 = synth.normal((o, c, 1, 1), 6503, float(np.sqrt(2.0 / c)))
+    b2 = synth.uniform((o,), 6504, -0.1, 0.1)
+    y1, y2 = pkg.conv2d_pair(dev(x), dev(w1), dev(b1), None, dev(w2), dev(b2), s, p, 1, True)
+    assert_close(host(y1), fast_orc.conv_chain(x, w1, b1, s, p, None, True), what=variant + " first output")
+    assert_close(host(y2), fast_orc.conv_chain(x, w2, b2, s, 0, None, False), what=variant + " second output")
+
+
+def test_conv_pair_full_batch_properties(pkg, synth):
+    """Batch 64 at the three ResNet-18 shapes: the pair launch against the two separate launches."""
+    for c, h, o in ((64, 56, 128), (128, 28, 256), (256, 14, 512)):
+        x = dev(synth.uniform((64, c, h, h), 6600 + c))
+        w1 = dev(synth.normal((o, c, 3, 3), 6601 + c, float(np.sqrt(2.0 / (c * 9)))))
+        b1 = dev(synth.uniform((o,), 6602 + c, -0.1, 0.1))
+        w2 = dev(synth.normal((o, c, 1, 1), 6603 + c, float(np.sqrt(2.0 / c))))
+        b2 = dev(synth.uniform((o,), 6604 + c, -0.1, 0.1))
+        y1, y2 = pkg.conv2d_pair(x, w1, b1, None, w2, b2, 2, 1, 1, True)
+        a1 = pkg.conv2d(x, w1, b1, None, 2, 1, 1, True)
+        a2 = pkg.conv2d(x, w2, b2, None, 2, 0, 1, False)
+        assert_close(host(y1), host(a1), tol=1e-4, what="pair vs single launch, first output, %d channels" % c)
+        assert_close(host(y2), host(a2), tol=1e-4, what="pair vs single launch, second output, %d channels" % c)
+        d2 = pkg.conv2d(x[5:6].contiguous(), w2, b2, None, 2, 0, 1, False, force_direct=True)
+        assert_close(host(y2[5:6]), host(d2), what="second output vs the reference-order kernel, image 5")
+
+
 # ------------------------------------------------------------------ Winograd F(2x2,3x3)
 WINOGRAD_SHAPES = [
     (2, 64, 56, 56, 64, 1),       # layer1
