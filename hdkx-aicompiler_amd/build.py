@@ -16,7 +16,7 @@ LIBDIR = os.path.join(PKG, "lib")
 OBJDIR = os.path.join(PKG, "build")
 LIB = os.path.join(LIBDIR, "libkxc_hip.so")
 
-SOURCES = ["device_api.hip", "eltwise.hip", "pool.hip", "gemm.hip", "conv2d_f32.hip", "conv2d_wino_f32.hip", "split_reduce.hip", "qconv_i8.hip", "qconv_c16_i8.hip",
+SOURCES = ["device_api.hip", "activity.hip", "eltwise.hip", "pool.hip", "gemm.hip", "conv2d_f32.hip", "conv2d_wino_f32.hip", "split_reduce.hip", "qconv_i8.hip", "qconv_c16_i8.hip",
            "module.hip", "plan.hip"]
 
 HIPCC = os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")

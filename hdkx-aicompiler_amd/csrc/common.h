@@ -6,6 +6,7 @@
 #include <cstdarg>
 #include <cstdint>
 #include <cstdio>
+#include <cstring>
 #include <mutex>
 #include <string>
 
@@ -99,6 +100,43 @@ struct WinoWeightJob {
     float* u;            // kxc_hip_conv2d_winograd_weight_bytes(desc) bytes
 };
 int32_t LaunchWinogradWeightTransforms(const WinoWeightJob* jobs, int32_t count, hipStream_t stream);
+
+// Activity recording (activity.hip).  ApiScope times one HIP runtime call on the host; DeviceScope brackets the
+// copy / fill / kernel that call enqueues with two HIP events on its stream.  Both do nothing while recording is off.
+bool ActivityOn();
+struct ActivitySuppress {      // the calling thread records nothing while one of these lives (a profiled plan run
+    ActivitySuppress();        // times its launches itself)
+    ~ActivitySuppress();
+};
+class ApiScope {
+public:
+    explicit ApiScope(const char* name);
+    ~ApiScope();
+    void SetResult(hipError_t e) { result_ = static_cast<int32_t>(e); }
+    uint64_t correlation() const { return correlation_; }
+private:
+    bool on_;
+    const char* name_;
+    uint64_t correlation_ = 0;
+    int64_t start_ns_ = 0;
+    int32_t result_ = 0;
+};
+class DeviceScope {
+public:
+    DeviceScope(int32_t kind, const char* name, hipStream_t stream, uint64_t correlation);
+    ~DeviceScope();
+    int64_t bytes = 0;
+    int32_t value = 0, copy_kind = 0;
+    uint32_t grid[3] = {0, 0, 0}, block[3] = {0, 0, 0}, dynamic_shared_memory = 0;
+private:
+    bool on_;
+    int32_t kind_;
+    const char* name_;
+    hipStream_t stream_;
+    uint64_t correlation_;
+    int64_t host_start_ns_ = 0;
+    hipEvent_t start_ = nullptr, stop_ = nullptr;
+};
 
 constexpr int64_t kMaxGridX = 2147483647LL;
 

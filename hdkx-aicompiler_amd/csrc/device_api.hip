@@ -23,6 +23,17 @@ hipStream_t& CurrentStream() {
 
 using namespace kxc_hip;
 
+namespace {
+// One HIP runtime call, recorded as a RUNTIME_API activity while recording is on.
+template <typename F>
+hipError_t Api(const char* name, F&& call) {
+    ApiScope scope(name);
+    const hipError_t e = call();
+    scope.SetResult(e);
+    return e;
+}
+}  // namespace
+
 extern "C" {
 
 const char* kxc_hip_last_error(void) { return LastError().c_str(); }
@@ -106,14 +117,14 @@ int32_t kxc_hip_alloc(int32_t device_id, size_t nbytes, size_t alignment, void**
     KXC_HIP_REQUIRE(alignment <= 256, "kxc_hip_alloc: alignment %zu > 256 is not supported", alignment);
     *out_ptr = nullptr;
     KXC_HIP_CALL(hipSetDevice(device_id), "HIP SetDevice");
-    KXC_HIP_CALL(hipMalloc(out_ptr, nbytes ? nbytes : 1), "HIP AllocDataSpace");
+    KXC_HIP_CALL(Api("hipMalloc", [&] { return hipMalloc(out_ptr, nbytes ? nbytes : 1); }), "HIP AllocDataSpace");
     return KXC_HIP_OK;
 }
 
 int32_t kxc_hip_free(int32_t device_id, void* ptr) {
     if (!ptr) return KXC_HIP_OK;
     KXC_HIP_CALL(hipSetDevice(device_id), "HIP SetDevice");
-    KXC_HIP_CALL(hipFree(ptr), "HIP FreeDataSpace");
+    KXC_HIP_CALL(Api("hipFree", [&] { return hipFree(ptr); }), "HIP FreeDataSpace");
     return KXC_HIP_OK;
 }
 
@@ -128,11 +139,34 @@ int32_t kxc_hip_copy(const void* from, size_t from_offset, void* to, size_t to_o
     const uint8_t* src = static_cast<const uint8_t*>(from) + from_offset;
     uint8_t* dst = static_cast<uint8_t*>(to) + to_offset;
     hipStream_t s = ResolveStream(stream);
-    if (s == nullptr) {
-        KXC_HIP_CALL(hipMemcpy(dst, src, nbytes, kinds[kind]), "HIP CopyDataFromTo");
-    } else {
-        KXC_HIP_CALL(hipMemcpyAsync(dst, src, nbytes, kinds[kind], s), "HIP CopyDataFromTo");
+    hipError_t e = hipSuccess;
+    {
+        ApiScope api(s ? "hipMemcpyAsync" : "hipMemcpy");
+        DeviceScope dev(KXC_HIP_ACTIVITY_MEMCPY, s ? "hipMemcpyAsync" : "hipMemcpy", s, api.correlation());
+        dev.bytes = static_cast<int64_t>(nbytes);
+        dev.copy_kind = kind;
+        e = s ? hipMemcpyAsync(dst, src, nbytes, kinds[kind], s) : hipMemcpy(dst, src, nbytes, kinds[kind]);
+        api.SetResult(e);
     }
+    KXC_HIP_CALL(e, "HIP CopyDataFromTo");
+    return KXC_HIP_OK;
+}
+
+int32_t kxc_hip_memset(void* ptr, int32_t value, size_t nbytes, int32_t device_id, void* stream) {
+    if (nbytes == 0) return KXC_HIP_OK;
+    KXC_HIP_REQUIRE(ptr != nullptr, "kxc_hip_memset: NULL pointer");
+    KXC_HIP_CALL(hipSetDevice(device_id), "HIP SetDevice");
+    hipStream_t s = ResolveStream(stream);
+    hipError_t e = hipSuccess;
+    {
+        ApiScope api(s ? "hipMemsetAsync" : "hipMemset");
+        DeviceScope dev(KXC_HIP_ACTIVITY_MEMSET, s ? "hipMemsetAsync" : "hipMemset", s, api.correlation());
+        dev.bytes = static_cast<int64_t>(nbytes);
+        dev.value = value & 0xff;
+        e = s ? hipMemsetAsync(ptr, value, nbytes, s) : hipMemset(ptr, value, nbytes);
+        api.SetResult(e);
+    }
+    KXC_HIP_CALL(e, "HIP Memset");
     return KXC_HIP_OK;
 }
 
@@ -140,7 +174,7 @@ int32_t kxc_hip_stream_create(int32_t device_id, void** out_stream) {
     KXC_HIP_REQUIRE(out_stream != nullptr, "kxc_hip_stream_create: out_stream is NULL");
     KXC_HIP_CALL(hipSetDevice(device_id), "HIP SetDevice");
     hipStream_t s = nullptr;
-    KXC_HIP_CALL(hipStreamCreate(&s), "HIP StreamCreate");   // default priority only
+    KXC_HIP_CALL(Api("hipStreamCreate", [&] { return hipStreamCreate(&s); }), "HIP StreamCreate");   // default priority only
     *out_stream = s;
     return KXC_HIP_OK;
 }
@@ -149,7 +183,7 @@ int32_t kxc_hip_stream_destroy(int32_t device_id, void* stream) {
     if (!stream) return KXC_HIP_OK;
     KXC_HIP_CALL(hipSetDevice(device_id), "HIP SetDevice");
     hipStream_t s = reinterpret_cast<hipStream_t>(stream);
-    KXC_HIP_CALL(hipStreamDestroy(s), "HIP StreamDestroy");
+    KXC_HIP_CALL(Api("hipStreamDestroy", [&] { return hipStreamDestroy(s); }), "HIP StreamDestroy");
     if (CurrentStream() == s) CurrentStream() = nullptr;
     return KXC_HIP_OK;
 }
@@ -171,9 +205,9 @@ int32_t kxc_hip_stream_sync(int32_t device_id, void* stream) {
     KXC_HIP_CALL(hipSetDevice(device_id), "HIP SetDevice");
     hipStream_t s = ResolveStream(stream);
     if (s == nullptr) {
-        KXC_HIP_CALL(hipDeviceSynchronize(), "HIP StreamSync");
+        KXC_HIP_CALL(Api("hipDeviceSynchronize", [&] { return hipDeviceSynchronize(); }), "HIP StreamSync");
     } else {
-        KXC_HIP_CALL(hipStreamSynchronize(s), "HIP StreamSync");
+        KXC_HIP_CALL(Api("hipStreamSynchronize", [&] { return hipStreamSynchronize(s); }), "HIP StreamSync");
     }
     return KXC_HIP_OK;
 }

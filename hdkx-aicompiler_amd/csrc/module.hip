@@ -8,6 +8,8 @@
 
 #include <cstring>
 #include <mutex>
+#include <string>
+#include <unordered_map>
 #include <vector>
 
 #include "common.h"
@@ -24,6 +26,11 @@ namespace {
 std::mutex& LoadMutex() {
     static std::mutex m;
     return m;
+}
+
+std::unordered_map<hipFunction_t, std::string>& FunctionNames() {      // guarded by LoadMutex()
+    static std::unordered_map<hipFunction_t, std::string> names;
+    return names;
 }
 
 void CopyLog(const std::string& text, char* log, size_t cap) {
@@ -124,6 +131,10 @@ int32_t kxc_hip_module_get_function(kxc_hip_module* module, const char* symbol, 
     hipError_t e = hipModuleGetFunction(&f, module->module, symbol);
     if (e != hipSuccess)
         return Fail(KXC_HIP_ERR_RUNTIME, "hipModuleGetFunction(%s) failed: %s", symbol, hipGetErrorString(e));
+    {
+        std::lock_guard<std::mutex> lock(LoadMutex());
+        FunctionNames()[f] = symbol;        // launch records name their kernel
+    }
     *out_function = f;
     return KXC_HIP_OK;
 }
@@ -138,9 +149,27 @@ int32_t kxc_hip_module_launch(void* function, const uint32_t grid[3], const uint
     NoteGrid(dim3(grid[0], grid[1], grid[2]));
     NoteBlock(dim3(block[0], block[1], block[2]));
     NoteLds(shared_bytes);
-    KXC_HIP_CALL(hipModuleLaunchKernel(reinterpret_cast<hipFunction_t>(function), grid[0], grid[1], grid[2], block[0],
-                                       block[1], block[2], shared_bytes, ResolveStream(stream), kernel_params, nullptr),
-                 "hipModuleLaunchKernel");
+    hipStream_t s = ResolveStream(stream);
+    hipError_t e = hipSuccess;
+    if (ActivityOn()) {
+        std::string name = "kxc_module_kernel";
+        {
+            std::lock_guard<std::mutex> lock(LoadMutex());
+            auto it = FunctionNames().find(reinterpret_cast<hipFunction_t>(function));
+            if (it != FunctionNames().end()) name = it->second;
+        }
+        ApiScope api("hipModuleLaunchKernel");
+        DeviceScope dev(KXC_HIP_ACTIVITY_KERNEL, name.c_str(), s, api.correlation());
+        for (int i = 0; i < 3; ++i) { dev.grid[i] = grid[i]; dev.block[i] = block[i]; }
+        dev.dynamic_shared_memory = shared_bytes;
+        e = hipModuleLaunchKernel(reinterpret_cast<hipFunction_t>(function), grid[0], grid[1], grid[2], block[0], block[1],
+                                  block[2], shared_bytes, s, kernel_params, nullptr);
+        api.SetResult(e);
+    } else {
+        e = hipModuleLaunchKernel(reinterpret_cast<hipFunction_t>(function), grid[0], grid[1], grid[2], block[0], block[1],
+                                  block[2], shared_bytes, s, kernel_params, nullptr);
+    }
+    KXC_HIP_CALL(e, "hipModuleLaunchKernel");
     return KXC_HIP_OK;
 }
 

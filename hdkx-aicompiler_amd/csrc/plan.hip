@@ -806,6 +806,7 @@ int32_t kxc_hip_plan_run_profiled(kxc_hip_plan* plan, void** args, void* stream,
     KXC_HIP_REQUIRE(capacity >= nodes, "%s: %d records needed, room for %d", who, nodes, capacity);
     void* s = stream ? stream : static_cast<void*>(CurrentStream());
     hipStream_t hs = reinterpret_cast<hipStream_t>(s);
+    ActivitySuppress no_activity_records;      // this run times its launches itself
     // one event before every node and one after the last: node i ran between events i and i+1
     std::vector<hipEvent_t> ev(static_cast<size_t>(nodes) + 1, nullptr);
     int32_t rc = KXC_HIP_OK;

@@ -1,0 +1,5 @@
+// Forwarding header: code written against the reference's include/relay/op.h compiles against the host layer
+// with -I<host>/include/compat -I<host>/include.
+#pragma once
+#include "kxc/relay.h"
+#include "kxc/op.h"

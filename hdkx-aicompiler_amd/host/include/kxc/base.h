@@ -13,10 +13,17 @@
 #include <memory>
 #include <stdexcept>
 #include <string>
+#include <type_traits>
 #include <utility>
 #include <vector>
 
 namespace kxc {
+
+// Common base of every node a handle points to, so that code written against the reference can key maps by
+// `const Object*` and pass any handle where an ObjectRef is expected (include/base/object.h:68-183).
+struct Object {
+    virtual ~Object() = default;
+};
 
 // Shared, nullable handle to an immutable-by-convention node.  `defined()`, `get()`, `As<T>()` and
 // `operator->` follow the reference's ObjectRef vocabulary (include/base/object.h:115-183).
@@ -35,6 +42,14 @@ public:
 
 protected:
     std::shared_ptr<NodeT> ptr_;
+};
+
+// Handle to any node: every Ref<T> with T derived from Object converts to it.
+class ObjectRef : public Ref<Object> {
+public:
+    ObjectRef() = default;
+    template <typename U, typename = typename std::enable_if<std::is_base_of<Object, U>::value>::type>
+    ObjectRef(const Ref<U>& other) : Ref<Object>(std::shared_ptr<Object>(other.shared())) {}
 };
 
 // Array<T>: a value-semantics vector with the reference's push_back/size/[] surface

@@ -48,6 +48,41 @@ struct HIPModuleSource {
     std::vector<HIPKernelSpec> kernels;      // in execution order
 };
 
+// One compiled function behind the Run ABI `int32_t f(void** packed_args)`: what the reference's CompiledKernelNode
+// is for its LLVM JIT and C back ends (include/codegen/compiled_kernel.h:19-41), with the HIP back end's resources
+// beside them.  Host back ends: func_ptr is the entry point of a library opened from so_path (lib_handle).  HIP back
+// end: jit_resource owns the launch plan and func_ptr is non-null exactly while that plan can be run, so
+// IsReady() keeps its meaning; hip_modules are the run-time compiled modules whose kernels the plan launches.
+// The destructor releases everything (dlclose, plan, modules), as the reference's does for its back ends
+// (src/codegen/compiled_kernel.cc:21-39).
+class CompiledKernelNode : public Object {
+public:
+    std::string kernel_name;
+    CodeGenBackend backend{CodeGenBackend::kC};
+    void* func_ptr{nullptr};
+    void* jit_resource{nullptr};
+    std::string so_path;
+    void* lib_handle{nullptr};
+    std::vector<tir::BufferInfo> param_buffers;      // signature of the packed arguments, in order
+    // HIP back end
+    std::vector<void*> hip_modules;                  // kxc_hip_module*
+    int device_id{0};
+    bool sync_after_run{true};                       // wait for the stream after enqueueing (callers read outputs at once)
+    ~CompiledKernelNode() override;
+};
+
+class CompiledKernel : public Ref<CompiledKernelNode> {
+public:
+    CompiledKernel() = default;
+    explicit CompiledKernel(std::shared_ptr<CompiledKernelNode> n) : Ref<CompiledKernelNode>(std::move(n)) {}
+    // Calls the function with packed_args = inputs, constants, outputs.  Throws "CompiledKernel: not ready or
+    // func_ptr is null", or "Kernel <name> returned error code N" (src/codegen/compiled_kernel.cc:41-55; the HIP back
+    // end appends the library's message).  HIP: every pointer is a device pointer; the launches go to the calling
+    // thread's current stream.
+    void operator()(const std::vector<void*>& args) const;
+    bool IsReady() const;
+};
+
 class CodeGenHIP {
 public:
     // prefix: made part of every kernel symbol so several PrimFuncs can share one module

@@ -17,6 +17,7 @@
 #include "kxc/codegen.h"
 #include "kxc/device_api.h"
 #include "kxc/lower.h"
+#include "kxc/profiling.h"
 
 namespace kxc {
 namespace runtime {
@@ -47,6 +48,11 @@ struct CompileConfigNode {
     std::vector<std::vector<int64_t>> suggested_input_shapes;   // each is warmed up at Compile
     int background_threads{0};         // compile workers (0 = half the hardware threads)
     bool enable_hot_swap{true};
+    std::string cache_dir;             // empty = cache in memory (the only kind either implementation has)
+    // When enabled and no context is active on the calling thread, Compile creates a ProfileContext from these
+    // options; the module keeps it, activates it around every Run and names its bundle in GetProfileBundlePath()
+    // (include/api/compile_config.h:47, src/api/compiler.cc:32-40).
+    profiling::ProfileOptions profile_options;
 };
 class CompileConfig : public Ref<CompileConfigNode> {
 public:
@@ -82,6 +88,10 @@ public:
     void WaitAll();                                                          // adaptive: drain background compiles
     bool IsReady() const;
     std::string GetStatus() const;
+    // Directory of the profiling bundle; empty when profiling was not enabled (include/api/compiler.h:88).
+    std::string GetProfileBundlePath() const;
+    // The compiled function behind Run (include/api/compiler.h:96-105 holds a codegen::CompiledKernel likewise).
+    const codegen::CompiledKernel& GetKernel() const;
     const tir::PrimFunc& GetPrimFunc() const;
     // Generated source: C for the host back end, HIP for the GPU back end.
     const std::string& GetSource() const;
@@ -110,6 +120,7 @@ private:
     friend class Compiler;
     std::shared_ptr<CompiledModuleImpl> impl_;
     std::shared_ptr<runtime::RuntimeSession> session_;     // adaptive mode only
+    std::shared_ptr<profiling::ProfileContext> session_profile_;
 };
 
 class Compiler {

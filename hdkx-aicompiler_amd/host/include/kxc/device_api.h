@@ -25,6 +25,25 @@ private:
 
 using StreamHandle = void*;
 
+// Single-attribute query keys (include/base/device_api.h:19-39).
+enum class DeviceAttrKind : int {
+    kExist = 0, kMaxThreadsPerBlock = 1, kWarpSize = 2, kMaxSharedMemoryPerBlock = 3, kComputeVersion = 4, kDeviceName = 5,
+    kMaxClockRate = 6, kMultiProcessorCount = 7, kMaxRegistersPerBlock = 8, kApiVersion = 9, kDriverVersion = 10,
+    kL2CacheSizeBytes = 11, kTotalGlobalMemory = 12, kAvailableGlobalMemory = 13, kMaxSharedMemoryPerMultiprocessor = 14,
+    kMaxRegistersPerMultiprocessor = 15, kMaxThreadsPerMultiprocessor = 16, kComputeVersionMajor = 17, kComputeVersionMinor = 18,
+};
+// What GetAttr returns: an integer, or text for kComputeVersion / kDeviceName (the reference's RetValue holds either).
+struct RetValue {
+    int64_t v_int64{0};
+    std::string v_str;
+    bool is_str{false};
+    RetValue& operator=(int64_t v) { v_int64 = v; is_str = false; return *this; }
+    RetValue& operator=(int v) { v_int64 = v; is_str = false; return *this; }
+    RetValue& operator=(const std::string& s) { v_str = s; is_str = true; return *this; }
+    operator int64_t() const { return v_int64; }
+    operator std::string() const { return v_str; }
+};
+
 struct DeviceAttributes {
     int exists{0};
     int64_t max_threads_per_block{1};
@@ -70,6 +89,8 @@ public:
                                 const Device& from_dev, const Device& to_dev, StreamHandle stream);
     virtual DeviceAttributes GetDeviceAttributes(const Device& device) = 0;
     virtual std::string GetTargetKind(const Device& device) const = 0;
+    // One attribute of GetDeviceAttributes (src/base/device_api.cc:198-262); never throws for an absent device.
+    virtual void GetAttr(const Device& device, DeviceAttrKind kind, RetValue* rv);
     virtual StreamHandle CreateStream(const Device& device);
     virtual void FreeStream(const Device& device, StreamHandle stream);
     virtual void SetStream(const Device& device, StreamHandle stream);
@@ -78,7 +99,24 @@ public:
     virtual void SyncStreamFromTo(const Device& device, StreamHandle src, StreamHandle dst);
     virtual void* AllocWorkspace(const Device& device, size_t nbytes, size_t alignment);
     virtual void FreeWorkspace(const Device& device, void* ptr);
+    // Whether host code may do address arithmetic on this back end's device pointers (true for HIP and the CPU).
+    virtual bool SupportsDevicePointerArithmeticsOnHost(const Device& device) const { return true; }
+    // Whether SetDevice must be called before using a device of this type (src/base/device_api.cc:184-186).
+    static bool NeedSetDevice(DeviceTypeCode type) { return type != kCPU; }
 };
+
+// Registry of the back ends by device type (include/base/device_api.h:126-135, src/base/device_api.cc:159-182): kCPU ->
+// the host API, kGPU -> the HIP API; anything else throws "Device API not supported".
+class DeviceAPIManager {
+public:
+    static DeviceAPIManager* Global();
+    DeviceAPI* GetAPI(DeviceTypeCode type);
+
+private:
+    DeviceAPIManager() = default;
+};
+void GetDeviceAttr(const Device& device, DeviceAttrKind kind, RetValue* rv);
+int64_t GetDeviceAttr(const Device& device, DeviceAttrKind kind);
 
 DeviceAPI* GetCPUDeviceAPI();
 DeviceAPI* GetHIPDeviceAPI();

@@ -134,6 +134,15 @@ public:
                    StringMap fields = {}, MetricMap metrics = {}, const std::string& run_id = "");
     std::string WriteArtifact(const std::string& relative_path, const std::string& content);
     void PublishDiagnostics(const std::vector<DiagnosticEntry>& diagnostics);
+    // Fetches the GPU-side activity the HIP library has recorded since the last call (runtime API calls, copies,
+    // fills, kernel launches) and adds it as "backend.hip" events: hip_runtime_api / hip_memcpy / hip_memset /
+    // hip_kernel, with the metric keys the reference's CUPTI adapter uses for their CUDA counterparts
+    // (src/base/profiling.cc:537-651).  Flush calls it; a caller synchronises its streams first.
+    void CollectGpuActivity();
+    // The device-side diagnosis rules the reference's offline analyser applies to a bundle (kernel_launch_overhead,
+    // copy_dominance, sync_overhead: python/kxc_agent/services/diagnosis_engine.py:233-297, thresholds
+    // rule_library.py:22-24), evaluated on the recorded events.
+    std::vector<DiagnosticEntry> DiagnoseDeviceOverheads() const;
     void Flush();
     std::size_t event_count() const;
 
@@ -146,6 +155,13 @@ private:
     std::string trace_id_, session_id_, bundle_dir_;
     std::int64_t start_wall_ns_{0}, start_mono_ns_{0};
     std::vector<std::string> event_lines_, trace_events_;
+    struct EventDigest {            // what the diagnosis rules read
+        std::string component, event_type;
+        std::int64_t duration_ns;
+    };
+    std::vector<EventDigest> digests_;
+    bool gpu_activity_on_{false};
+    bool auto_diagnosed_{false};     // diagnostics_ came from DiagnoseDeviceOverheads, not from PublishDiagnostics
     std::vector<DiagnosticEntry> diagnostics_;
     std::uint64_t run_counter_{0}, span_counter_{0};
     bool layout_done_{false};

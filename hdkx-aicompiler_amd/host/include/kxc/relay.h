@@ -10,9 +10,7 @@
 namespace kxc {
 
 // ------------------------------------------------------------------ types
-struct TypeNode {
-    virtual ~TypeNode() = default;
-};
+struct TypeNode : Object {};
 struct TensorTypeNode : TypeNode {
     std::vector<int64_t> shape;
     std::string dtype;
@@ -36,10 +34,24 @@ public:
 std::string TypeToString(const Type& t);
 
 // ------------------------------------------------------------------ host tensor
+}  // namespace kxc
+// Element type of a host tensor as the reference's NDArray exposes it (include/base/ndarray.h:19-31).
+extern "C" {
+typedef enum { kDLInt = 0U, kDLUint = 1U, kDLFloat = 2U, kDLBfloat = 4U, kDLComplex = 5U } DLDataTypeCode;
+typedef struct {
+    uint8_t code;
+    uint8_t bits;
+    uint16_t lanes;
+} DLDataType;
+}
+namespace kxc {
 namespace runtime {
-struct NDArrayNode {
+struct NDArrayNode : Object {
     std::vector<int64_t> shape;
     std::string dtype;
+    struct {
+        DLDataType dtype;
+    } dl_tensor;                   // dtype as {code, bits, lanes}, filled on construction
     std::vector<char> bytes;       // zero-filled on construction (src/base/ndarray.cc:35-62)
     void* data() { return bytes.data(); }
     const void* data() const { return bytes.data(); }
@@ -55,8 +67,7 @@ public:
 }  // namespace runtime
 
 // ------------------------------------------------------------------ expressions
-struct RelayExprNode {
-    virtual ~RelayExprNode() = default;
+struct RelayExprNode : Object {
     mutable Type checked_type_;     // filled by InferType
 };
 class Expr : public Ref<RelayExprNode> {
@@ -98,9 +109,7 @@ public:
     const ConstantNode* operator->() const { return static_cast<const ConstantNode*>(ptr_.get()); }
 };
 
-struct AttrsNode {
-    virtual ~AttrsNode() = default;
-};
+struct AttrsNode : Object {};
 class Attrs : public Ref<AttrsNode> {
 public:
     Attrs() = default;

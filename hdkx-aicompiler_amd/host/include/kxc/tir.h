@@ -8,6 +8,8 @@
 // The representation is one tagged node type per family rather than a class per node.
 #pragma once
 
+#include <ostream>
+
 #include <functional>
 #include <limits>
 
@@ -178,6 +180,19 @@ std::string ToString(const PrimFunc& f);
 PrimExpr FoldAndSimplify(const PrimExpr& e);
 Stmt FoldAndSimplify(const Stmt& s);
 PrimFunc RunTIRPassPipeline(const PrimFunc& f, const std::vector<std::string>& passes);
+
+// Structured text dump of a PrimFunc under the reference's names (include/tir/pass/print_ir.h:14-27).
+namespace pass {
+class IRPrinterPass {
+public:
+    explicit IRPrinterPass(int indent_spaces = 2) : indent_spaces_(indent_spaces) {}
+    void Run(const PrimFunc& func, std::ostream& os) const;
+
+private:
+    int indent_spaces_;
+};
+void DumpPrimFunc(const PrimFunc& func, std::ostream& os, int indent_spaces = 2);
+}  // namespace pass
 
 // The type two operands are promoted to before a binary operation.
 DataType PromoteTypes(DataType a, DataType b);

@@ -60,22 +60,41 @@ public:
     int num_values = 0;
     std::vector<int> input_value_ids, constant_value_ids;
     int output_value = -1;
-    // host back end
-    void* dl_handle = nullptr;
-    int32_t (*fn)(void**) = nullptr;
-    std::string so_path;
-    // hip back end
+    // The compiled function (include/api/compiler.h:96-105 keeps a codegen::CompiledKernel the same way): owns the
+    // generated library of the host back end, or the launch plan and run-time compiled modules of the hip back end.
+    codegen::CompiledKernel kernel;
+    // hip back end: the plan the kernel owns (alias), and what a dry build (no GPU) keeps instead
     kxc_hip_plan* plan = nullptr;
-    std::vector<kxc_hip_module*> modules;
-    std::vector<std::string> module_sources;     // one per entry of modules (dry builds keep the sources only)
+    std::vector<kxc_hip_module*> modules;        // moved into the kernel node once the plan is loaded
+    std::vector<std::string> module_sources;     // one per generated module (dry builds keep the sources only)
     size_t workspace_bytes = 0;
     bool ready = false;
+    std::shared_ptr<profiling::ProfileContext> profile_context;      // from config->profile_options, when enabled
 
+    // Hands the plan and the modules to a kernel node (callable = the plan was finalized on a GPU).
+    void AdoptHipKernel(bool callable) {
+        auto node = std::make_shared<codegen::CompiledKernelNode>();
+        node->kernel_name = "kxc_kernel_main";
+        node->backend = codegen::CodeGenBackend::kHIP;
+        node->jit_resource = plan;
+        node->func_ptr = callable ? static_cast<void*>(plan) : nullptr;
+        for (auto* m : modules) node->hip_modules.push_back(m);
+        modules.clear();
+        node->device_id = config->target->device.device_id();
+        node->sync_after_run = config->sync_after_run;
+        if (prim_func.defined())
+            for (const auto& v : prim_func->params) {
+                auto it = prim_func->buffer_map.find(v.get());
+                if (it != prim_func->buffer_map.end()) node->param_buffers.push_back(it->second);
+            }
+        kernel = codegen::CompiledKernel(node);
+    }
     ~CompiledModuleImpl() {
-        if (plan) kxc_hip_plan_destroy(plan);
-        for (auto* m : modules) kxc_hip_module_free(m);
-        if (dl_handle) dlclose(dl_handle);
-        if (!so_path.empty()) std::remove(so_path.c_str());
+        // (before a kernel node adopted them)
+        if (!kernel.defined()) {
+            if (plan) kxc_hip_plan_destroy(plan);
+            for (auto* m : modules) kxc_hip_module_free(m);
+        }
     }
 };
 
@@ -95,7 +114,7 @@ void CompileHost(const Function& typed, const CompileConfig& config, CompiledMod
     const std::string base = std::string(tmp && *tmp ? tmp : "/tmp") + "/kxc_jit_" + std::to_string(getpid()) + "_" +
                              std::to_string(counter.fetch_add(1));
     const std::string c_path = base + ".c";
-    m->so_path = base + ".so";
+    const std::string so_path = base + ".so";
     {
         std::ofstream out(c_path);
         out << m->source;
@@ -103,7 +122,7 @@ void CompileHost(const Function& typed, const CompileConfig& config, CompiledMod
     const int level = config->opt_level < 0 ? 0 : config->opt_level > 3 ? 3 : config->opt_level;
     // strict fp32: no contraction, no fast-math -- results do not depend on the optimisation level
     const std::string cmd = "cc -std=gnu11 -O" + std::to_string(level) +
-                            " -fno-fast-math -ffp-contract=off -shared -fPIC -w -o " + m->so_path + " " + c_path + " -lm 2>&1";
+                            " -fno-fast-math -ffp-contract=off -shared -fPIC -w -o " + so_path + " " + c_path + " -lm 2>&1";
     FILE* pipe = popen(cmd.c_str(), "r");
     if (!pipe) throw std::runtime_error("host compiler could not be started");
     std::string log;
@@ -112,10 +131,19 @@ void CompileHost(const Function& typed, const CompileConfig& config, CompiledMod
     const int rc = pclose(pipe);
     std::remove(c_path.c_str());
     if (rc != 0) throw std::runtime_error("host compilation of the generated C failed:\n" + log);
-    m->dl_handle = dlopen(m->so_path.c_str(), RTLD_NOW | RTLD_LOCAL);
-    if (!m->dl_handle) throw std::runtime_error(std::string("dlopen failed: ") + dlerror());
-    m->fn = reinterpret_cast<int32_t (*)(void**)>(dlsym(m->dl_handle, kKernelEntrySymbol));
-    if (!m->fn) throw std::runtime_error("generated library lacks kxc_kernel_main");
+    auto node = std::make_shared<codegen::CompiledKernelNode>();
+    node->kernel_name = kKernelEntrySymbol;
+    node->backend = codegen::CodeGenBackend::kC;
+    node->so_path = so_path;
+    node->lib_handle = dlopen(so_path.c_str(), RTLD_NOW | RTLD_LOCAL);
+    if (!node->lib_handle) throw std::runtime_error(std::string("dlopen failed: ") + dlerror());
+    node->func_ptr = dlsym(node->lib_handle, kKernelEntrySymbol);
+    if (!node->func_ptr) throw std::runtime_error("generated library lacks kxc_kernel_main");
+    for (const auto& v : m->prim_func->params) {
+        auto it = m->prim_func->buffer_map.find(v.get());
+        if (it != m->prim_func->buffer_map.end()) node->param_buffers.push_back(it->second);
+    }
+    m->kernel = codegen::CompiledKernel(node);
     KernelExecInfo e;
     e.op_name = "main";
     e.kernel_symbol = kKernelEntrySymbol;
@@ -188,9 +216,11 @@ public:
             if (kxc_hip_plan_finalize(m_->plan, m_->workspace_bytes))
                 throw std::runtime_error(std::string("plan finalize failed: ") + kxc_hip_last_error());
             if (cfg_->hip_constants_frozen) kxc_hip_plan_freeze_constants(m_->plan, 1);
+            m_->AdoptHipKernel(true);
             m_->ready = true;
             m_->status = "ready (hip back end, " + std::to_string(m_->execs.size()) + " launches)";
         } else {
+            m_->AdoptHipKernel(false);
             m_->status = "compiled without loading (no GPU): " + std::to_string(m_->execs.size()) + " launches";
         }
     }
@@ -582,18 +612,40 @@ private:
 
 }  // namespace
 
+namespace {
+// The caller's active context, else one made from the configuration's profile_options when those are enabled
+// (src/api/compiler.cc:32-40).
+std::shared_ptr<profiling::ProfileContext> MaybeCreateProfileContext(const CompileConfig& config) {
+    if (profiling::CurrentContext()) return profiling::CurrentContext();
+    if (!config.defined() || !config->profile_options.enabled) return nullptr;
+    return profiling::ProfileContext::Create(config->profile_options);
+}
+}  // namespace
+
 CompiledModule Compiler::Compile(Function func, CompileConfig config) {
     if (!config.defined() || !config->target.defined()) throw std::runtime_error("Compiler::Compile: config has no target");
+    std::shared_ptr<profiling::ProfileContext> own_context;
+    std::unique_ptr<profiling::ActivationScope> own_activation;
+    if (!profiling::CurrentContext()) {
+        own_context = MaybeCreateProfileContext(config);
+        if (own_context) own_activation = std::make_unique<profiling::ActivationScope>(own_context, own_context->NextRunId("compile"));
+    }
+    struct FlushOnExit {
+        std::shared_ptr<profiling::ProfileContext> ctx;
+        ~FlushOnExit() { if (ctx) ctx->Flush(); }
+    } flush{own_context};
     if (config->mode == CompileMode::kAdaptive) {
         // the session compiles (ahead-of-time mode) on demand; every suggested shape is warmed up now, each as the
         // shape of a single input (src/api/compiler.cc:64-80)
         CompiledModule adaptive;
         adaptive.session_ = std::make_shared<runtime::RuntimeSession>(func, config, profiling::CurrentContext());
         for (const auto& shape : config->suggested_input_shapes) adaptive.session_->WarmUp({shape});
+        adaptive.session_profile_ = own_context;
         return adaptive;
     }
     auto impl = std::make_shared<CompiledModuleImpl>();
     impl->config = config;
+    impl->profile_context = own_context;
     profiling::EventSpec cspec;
     cspec.component = "compiler";
     cspec.event_type = "compile";
@@ -663,9 +715,22 @@ void CompiledModule::Run(const std::vector<void*>& packed_args) {
     if (packed_args.size() != expect)
         throw std::runtime_error("CompiledModule::Run: expected " + std::to_string(expect) + " packed arguments, got " +
                                  std::to_string(packed_args.size()));
-    if (impl_->fn) {
-        const int32_t rc = impl_->fn(const_cast<void**>(packed_args.data()));
-        if (rc != 0) throw std::runtime_error("Kernel kxc_kernel_main returned error code " + std::to_string(rc));
+    // a module compiled with profile_options carries its own context (src/api/compiler.cc:149-168)
+    std::unique_ptr<profiling::ActivationScope> activation;
+    if (impl_->profile_context && !profiling::CurrentContext())
+        activation = std::make_unique<profiling::ActivationScope>(impl_->profile_context, impl_->profile_context->NextRunId("execute"));
+    struct FlushOnExit {
+        std::shared_ptr<profiling::ProfileContext> ctx;
+        ~FlushOnExit() { if (ctx) ctx->Flush(); }
+    } flush{activation ? impl_->profile_context : nullptr};
+    // (src/api/compiler.cc:158-163: one "compiled_module_run" span per call, carrying the kernel's name)
+    profiling::EventSpec mspec;
+    mspec.component = "runtime";
+    mspec.event_type = "compiled_module_run";
+    mspec.kernel_symbol = impl_->kernel->kernel_name;
+    profiling::ScopedSpan module_span = profiling::CurrentSpan(mspec);
+    if (impl_->kernel->backend != codegen::CodeGenBackend::kHIP) {
+        impl_->kernel(packed_args);
         return;
     }
     auto ctx = profiling::CurrentContext();
@@ -706,15 +771,18 @@ void CompiledModule::Run(const std::vector<void*>& packed_args) {
         run_span.AddMetric("launches", count);
         return;     // the profiled run has already waited for the last launch
     }
-    if (kxc_hip_plan_run(impl_->plan, const_cast<void**>(packed_args.data()), nullptr))
-        throw std::runtime_error(std::string("Kernel kxc_kernel_main failed: ") + kxc_hip_last_error());
-    if (impl_->config->sync_after_run) {
-        if (kxc_hip_stream_sync(impl_->config->target->device.device_id(), nullptr))
-            throw std::runtime_error(std::string("HIP StreamSync failed: ") + kxc_hip_last_error());
-    }
+    impl_->kernel(packed_args);
 }
 
-bool CompiledModule::IsReady() const { return session_ || (impl_ && impl_->ready); }
+bool CompiledModule::IsReady() const { return session_ || (impl_ && impl_->ready && impl_->kernel.IsReady()); }
+const codegen::CompiledKernel& CompiledModule::GetKernel() const {
+    if (!impl_) throw std::runtime_error("GetKernel: empty module");
+    return impl_->kernel;
+}
+std::string CompiledModule::GetProfileBundlePath() const {
+    if (session_) return session_profile_ ? session_profile_->bundle_dir() : "";
+    return impl_ && impl_->profile_context ? impl_->profile_context->bundle_dir() : "";
+}
 std::string CompiledModule::GetStatus() const { return session_ ? session_->GetStatus() : impl_ ? impl_->status : "empty"; }
 const tir::PrimFunc& CompiledModule::GetPrimFunc() const { return impl_->prim_func; }
 const std::string& CompiledModule::GetSource() const { return impl_->source; }
@@ -842,6 +910,7 @@ CompiledModule Compiler::LoadExecutionPlan(const std::string& plan_json, Compile
         throw std::runtime_error("LoadExecutionPlan: node list and launch plan disagree");
     impl->workspace_bytes = static_cast<size_t>(hip.at("workspace_bytes").integer);
     if (config->hip_constants_frozen) kxc_hip_plan_freeze_constants(impl->plan, 1);
+    impl->AdoptHipKernel(true);
     impl->ready = true;
     impl->status = "loaded from an execution plan";
     return CompiledModule(impl);

@@ -94,7 +94,11 @@ public:
         const bool fg = from_dev.device_type() == kGPU, tg = to_dev.device_type() == kGPU;
         const int kind = (!fg && tg) ? 0 : (fg && !tg) ? 1 : (fg && tg) ? 2 : 3;
         const int dev = tg ? to_dev.device_id() : from_dev.device_id();
-        profiling::ScopedSpan span = ApiSpan("copy_data_from_to", tg ? to_dev : from_dev, static_cast<double>(nbytes));
+        // event_type "copy" and the "from->to" device tag are what the reference records (cuda_device_api.cc:124-129),
+        // and what its bundle analyser sums for the copy_dominance rule
+        profiling::ScopedSpan span = ApiSpan("copy", tg ? to_dev : from_dev, static_cast<double>(nbytes));
+        span.AddField("device_api.route", std::string(fg ? "hip:" : "cpu:") + std::to_string(from_dev.device_id()) + "->" +
+                                              (tg ? "hip:" : "cpu:") + std::to_string(to_dev.device_id()));
         span.AddField("device_api.copy_kind", kind == 0 ? "host_to_device" : kind == 1 ? "device_to_host" : kind == 2 ? "device_to_device" : "host_to_host");
         if (kxc_hip_copy(from_ptr, from_offset, to_ptr, to_offset, nbytes, kind, dev, stream)) ThrowHip("CopyDataFromTo");
     }
@@ -160,12 +164,51 @@ DeviceAPI* GetHIPDeviceAPI() {
     static HIPDeviceAPI api;
     return &api;
 }
-DeviceAPI* GetDeviceAPI(DeviceTypeCode type) {
+DeviceAPIManager* DeviceAPIManager::Global() {
+    static DeviceAPIManager instance;
+    return &instance;
+}
+DeviceAPI* DeviceAPIManager::GetAPI(DeviceTypeCode type) {
     switch (type) {
         case kCPU: return GetCPUDeviceAPI();
         case kGPU: return GetHIPDeviceAPI();
-        default: throw std::runtime_error("Device type not supported");
+        default: throw std::runtime_error("Device API not supported");
     }
+}
+DeviceAPI* GetDeviceAPI(DeviceTypeCode type) { return DeviceAPIManager::Global()->GetAPI(type); }
+
+void DeviceAPI::GetAttr(const Device& device, DeviceAttrKind kind, RetValue* rv) {
+    const DeviceAttributes a = GetDeviceAttributes(device);
+    switch (kind) {
+        case DeviceAttrKind::kExist: *rv = a.exists; return;
+        case DeviceAttrKind::kMaxThreadsPerBlock: *rv = a.max_threads_per_block; return;
+        case DeviceAttrKind::kWarpSize: *rv = a.warp_size; return;
+        case DeviceAttrKind::kMaxSharedMemoryPerBlock: *rv = a.max_shared_memory_per_block; return;
+        case DeviceAttrKind::kComputeVersion: *rv = a.compute_version; return;
+        case DeviceAttrKind::kDeviceName: *rv = a.device_name; return;
+        case DeviceAttrKind::kMaxClockRate: *rv = a.max_clock_rate_khz; return;
+        case DeviceAttrKind::kMultiProcessorCount: *rv = a.multi_processor_count; return;
+        case DeviceAttrKind::kMaxRegistersPerBlock: *rv = a.max_registers_per_block; return;
+        case DeviceAttrKind::kApiVersion: *rv = a.api_version; return;
+        case DeviceAttrKind::kDriverVersion: *rv = a.driver_version; return;
+        case DeviceAttrKind::kL2CacheSizeBytes: *rv = a.l2_cache_size_bytes; return;
+        case DeviceAttrKind::kTotalGlobalMemory: *rv = a.total_global_memory; return;
+        case DeviceAttrKind::kAvailableGlobalMemory: *rv = a.available_global_memory; return;
+        case DeviceAttrKind::kMaxSharedMemoryPerMultiprocessor: *rv = a.max_shared_memory_per_multiprocessor; return;
+        case DeviceAttrKind::kMaxRegistersPerMultiprocessor: *rv = a.max_registers_per_block; return;
+        case DeviceAttrKind::kMaxThreadsPerMultiprocessor: *rv = a.max_threads_per_multiprocessor; return;
+        case DeviceAttrKind::kComputeVersionMajor: *rv = a.compute_version_major; return;
+        case DeviceAttrKind::kComputeVersionMinor: *rv = a.compute_version_minor; return;
+    }
+    throw std::runtime_error("Unknown device attribute kind");
+}
+void GetDeviceAttr(const Device& device, DeviceAttrKind kind, RetValue* rv) {
+    GetDeviceAPI(device.device_type())->GetAttr(device, kind, rv);
+}
+int64_t GetDeviceAttr(const Device& device, DeviceAttrKind kind) {
+    RetValue rv;
+    GetDeviceAttr(device, kind, &rv);
+    return rv.v_int64;
 }
 
 std::vector<DeviceInfo> GetAllDeviceInfo() {

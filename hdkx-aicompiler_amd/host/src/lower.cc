@@ -166,8 +166,11 @@ Stmt LowerCompute(const Tensor& t, const std::unordered_map<const tir::TensorNod
 
 }  // namespace
 
-LoweredFunc LowerToTIRDetailed(const Function& f) {
-    if (!f.defined()) throw std::runtime_error("LowerToTIR: undefined function");
+LoweredFunc LowerToTIRDetailed(const Function& untyped) {
+    if (!untyped.defined()) throw std::runtime_error("LowerToTIR expects a defined function");
+    // types are inferred here as well (src/relay/backend/lower.cc:470-477), so an untyped graph can be lowered
+    const Function f = InferTypePass(untyped);
+    if (!f->body.defined()) throw std::runtime_error("LowerToTIR expects function body to be defined");
     Converter conv(f);
     Tensor out_tensor = conv.Visit(f->body);
 

@@ -1,6 +1,8 @@
 // profiling.cc -- bundle writer and thread-local span stack (see kxc/profiling.h).
 #include "kxc/profiling.h"
 
+#include "kxc_hip.h"
+
 #include <dlfcn.h>
 #include <unistd.h>
 
@@ -301,14 +303,104 @@ ProfileContext::ProfileContext(ProfileOptions options) : options_(std::move(opti
                       ? (std::filesystem::temp_directory_path() / ("kxc_profile_" + HashText(seed))).string()
                       : options_.bundle_dir;
 }
+namespace {
+std::mutex g_activity_mu;
+int g_activity_users = 0;      // contexts that asked the HIP library to record activity
+}  // namespace
+
 ProfileContext::~ProfileContext() {
     try {
         if (options_.enabled && !event_lines_.empty()) Flush();
     } catch (...) {
     }
+    if (gpu_activity_on_) {
+        std::lock_guard<std::mutex> lock(g_activity_mu);
+        if (--g_activity_users == 0) kxc_hip_activity_enable(0);
+    }
 }
 std::shared_ptr<ProfileContext> ProfileContext::Create(const ProfileOptions& options) {
-    return std::shared_ptr<ProfileContext>(new ProfileContext(options));
+    std::shared_ptr<ProfileContext> ctx(new ProfileContext(options));
+    if (options.enabled && options.enable_gpu_activity) {
+        int32_t devices = 0;
+        if (kxc_hip_device_count(&devices) == 0 && devices > 0) {
+            std::lock_guard<std::mutex> lock(g_activity_mu);
+            if (kxc_hip_activity_enable(1) == 0) {
+                ++g_activity_users;
+                ctx->gpu_activity_on_ = true;
+            }
+        }
+    }
+    return ctx;
+}
+
+void ProfileContext::CollectGpuActivity() {
+    if (!gpu_activity_on_) return;
+    int32_t count = 0;
+    if (kxc_hip_activity_drain(nullptr, 0, &count) != 0 || count == 0) return;
+    std::vector<kxc_hip_activity_record> records(static_cast<size_t>(count) + 64);
+    if (kxc_hip_activity_drain(records.data(), static_cast<int32_t>(records.size()), &count) != 0) return;
+    // the library's clock -> this context's time base
+    const std::int64_t offset = NowNs() - kxc_hip_activity_now_ns();
+    static const char* const kTypes[4] = {"hip_runtime_api", "hip_memcpy", "hip_memset", "hip_kernel"};
+    for (int32_t i = 0; i < count; ++i) {
+        const kxc_hip_activity_record& r = records[static_cast<size_t>(i)];
+        if (r.kind < 0 || r.kind > 3) continue;
+        EventSpec e;
+        e.component = "backend.hip";
+        e.event_type = kTypes[r.kind];
+        e.device = r.kind == KXC_HIP_ACTIVITY_RUNTIME_API ? "hip" : "hip:" + std::to_string(r.device_id);
+        e.fields["backend.hip.correlation_id"] = std::to_string(r.correlation_id);
+        e.fields["backend.hip.thread_id"] = std::to_string(r.thread_id);
+        if (r.kind == KXC_HIP_ACTIVITY_RUNTIME_API) {
+            e.fields["backend.hip.api"] = r.name;
+            e.fields["backend.hip.return_value"] = std::to_string(r.return_value);
+            if (r.return_value != 0) { e.status = "error"; e.severity = LogSeverity::kWarn; }
+        } else {
+            e.fields["backend.hip.stream_id"] = std::to_string(r.stream);
+            e.fields["backend.hip.timing_source"] = r.timed_on_gpu ? "hip_events" : "host_clock";
+        }
+        if (r.kind == KXC_HIP_ACTIVITY_MEMCPY) {
+            e.fields["backend.hip.copy_kind"] = std::to_string(r.copy_kind);
+            e.metrics["bytes"] = static_cast<double>(r.bytes);
+            e.metrics["copy_count"] = 1.0;
+        } else if (r.kind == KXC_HIP_ACTIVITY_MEMSET) {
+            e.metrics["bytes"] = static_cast<double>(r.bytes);
+            e.metrics["value"] = static_cast<double>(r.value);
+        } else if (r.kind == KXC_HIP_ACTIVITY_KERNEL) {
+            e.kernel_symbol = r.name;
+            e.metrics["grid_x"] = r.grid[0]; e.metrics["grid_y"] = r.grid[1]; e.metrics["grid_z"] = r.grid[2];
+            e.metrics["block_x"] = r.block[0]; e.metrics["block_y"] = r.block[1]; e.metrics["block_z"] = r.block[2];
+            e.metrics["dynamic_shared_memory"] = r.dynamic_shared_memory;
+        }
+        RecordCompletedSpan(e, CurrentRunId(), NextSpanId(), "", r.start_ns + offset, r.end_ns + offset);
+    }
+}
+
+std::vector<DiagnosticEntry> ProfileContext::DiagnoseDeviceOverheads() const {
+    constexpr double kCopyDominanceRatio = 0.40, kSyncDominanceRatio = 0.25;
+    constexpr std::int64_t kSmallKernelRunNs = 200000;
+    std::int64_t copy = 0, device = 0, sync = 0, total = 0;
+    int tiny_runs = 0;
+    {
+        std::lock_guard<std::mutex> lock(mu_);
+        for (const EventDigest& d : digests_) {
+            total += d.duration_ns;
+            if (d.component == "device_api") {
+                device += d.duration_ns;
+                if (d.event_type == "copy") copy += d.duration_ns;
+            }
+            if (d.event_type == "stream_sync" || d.event_type == "execute_barrier_node") sync += d.duration_ns;
+            if ((d.event_type == "compiled_module_run" || d.event_type == "adaptive_module_run") && d.duration_ns < kSmallKernelRunNs) ++tiny_runs;
+        }
+    }
+    std::vector<DiagnosticEntry> out;
+    if (device > 0 && static_cast<double>(copy) / static_cast<double>(device) >= kCopyDominanceRatio)
+        out.push_back({"copy_dominance", "warn", "device_api", "Device copy time dominates device API activity."});
+    if (total > 0 && static_cast<double>(sync) / static_cast<double>(total) >= kSyncDominanceRatio)
+        out.push_back({"sync_overhead", "warn", "runtime", "Synchronization overhead is a large portion of the run."});
+    if (tiny_runs >= 5)
+        out.push_back({"kernel_launch_overhead", "info", "runtime", "Many very short module runs suggest launch overhead may dominate."});
+    return out;
 }
 std::int64_t ProfileContext::NowNs() const { return SteadyNs() - start_mono_ns_; }
 std::string ProfileContext::NextRunId(const std::string& prefix) {
@@ -330,6 +422,7 @@ void ProfileContext::RecordCompletedSpan(const EventSpec& spec, const std::strin
     std::lock_guard<std::mutex> lock(mu_);
     event_lines_.push_back(EventLine(trace_id_, session_id_, run_id, span_id, parent, spec, start_ns, dur));
     trace_events_.push_back(TraceEvent(spec, start_ns, dur, spec.component == "backend.hip"));
+    digests_.push_back({spec.component, spec.event_type, dur});
 }
 void ProfileContext::RecordInstant(EventSpec spec, const std::string& run_id, const std::string& parent) {
     if (!options_.enabled || static_cast<int>(spec.severity) < static_cast<int>(options_.log_level)) return;
@@ -370,11 +463,25 @@ std::string ProfileContext::WriteArtifact(const std::string& relative_path, cons
 void ProfileContext::PublishDiagnostics(const std::vector<DiagnosticEntry>& diagnostics) {
     std::lock_guard<std::mutex> lock(mu_);
     diagnostics_ = diagnostics;
+    auto_diagnosed_ = false;
     EnsureLayoutLocked();
     WriteAllLocked();
 }
 void ProfileContext::Flush() {
+    CollectGpuActivity();
+    // unless a caller published a diagnosis of its own, the device-side rules are evaluated on what was recorded
+    bool published = false;
+    {
+        std::lock_guard<std::mutex> lock(mu_);
+        published = !diagnostics_.empty() && !auto_diagnosed_;
+    }
+    std::vector<DiagnosticEntry> found;
+    if (!published) found = DiagnoseDeviceOverheads();
     std::lock_guard<std::mutex> lock(mu_);
+    if (!published) {
+        diagnostics_ = found;
+        auto_diagnosed_ = true;
+    }
     EnsureLayoutLocked();
     WriteAllLocked();
 }
@@ -421,7 +528,8 @@ void ProfileContext::WriteAllLocked() {
     {
         std::vector<DiagnosticEntry> items = diagnostics_;
         if (items.empty())
-            items.push_back({"not_analyzed", "info", "analysis", "Bundle created; no analysis has been run on it."});
+            items.push_back({"no_findings", "info", "analysis",
+                             "The device-side rules (kernel_launch_overhead, copy_dominance, sync_overhead) found nothing."});
         std::ofstream f(dir / "diagnosis.json", std::ios::out | std::ios::trunc);
         f << "{\"trace_id\":\"" << Escape(trace_id_) << "\",\"diagnostics\":[";
         for (size_t i = 0; i < items.size(); ++i) {

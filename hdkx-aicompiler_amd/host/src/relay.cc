@@ -27,7 +27,11 @@ NDArray::NDArray(Array<int64_t> shape, std::string dtype) {
     n->shape = shape;
     n->dtype = dtype;
     const int64_t count = Product(n->shape);
-    n->bytes.assign(static_cast<size_t>(count) * tir::DTypeFromString(dtype).bytes(), 0);
+    const tir::DataType dt = tir::DTypeFromString(dtype);
+    n->bytes.assign(static_cast<size_t>(count) * dt.bytes(), 0);
+    n->dl_tensor.dtype.code = static_cast<uint8_t>(dt.code);       // 0 int, 1 uint (bool: 1 bit), 2 float
+    n->dl_tensor.dtype.bits = static_cast<uint8_t>(dt.bits);
+    n->dl_tensor.dtype.lanes = 1;
     ptr_ = n;
 }
 void NDArray::CopyFromBytes(const void* src, size_t nbytes) {

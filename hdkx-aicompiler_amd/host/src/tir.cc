@@ -145,6 +145,30 @@ Stmt Evaluate(PrimExpr value) {
     return s;
 }
 
+namespace pass {
+void IRPrinterPass::Run(const PrimFunc& func, std::ostream& os) const {
+    os << "================ TIR PrimFunc ================\n";
+    if (!func.defined()) { os << "<undefined>\n"; return; }
+    const std::string pad(static_cast<size_t>(indent_spaces_ < 0 ? 0 : indent_spaces_), ' ');
+    os << "params(" << func->params.size() << "):\n";
+    for (size_t i = 0; i < func->params.size(); ++i) {
+        os << pad << "[" << i << "] " << func->params[i].name_hint();
+        auto it = func->buffer_map.find(func->params[i].get());
+        if (it != func->buffer_map.end()) {
+            os << " : buffer " << it->second.name << " " << DTypeToString(it->second.dtype) << "[";
+            for (size_t d = 0; d < it->second.shape.size(); ++d) os << (d ? ", " : "") << it->second.shape[d];
+            os << "]";
+        }
+        os << "\n";
+    }
+    os << "attrs:\n";
+    for (const auto& kv : func->int_attrs) os << pad << kv.first << " = " << kv.second << "\n";
+    for (const auto& kv : func->str_attrs) os << pad << kv.first << " = \"" << kv.second << "\"\n";
+    os << "body:\n" << ToString(func->body, indent_spaces_ < 0 ? 0 : indent_spaces_);
+}
+void DumpPrimFunc(const PrimFunc& func, std::ostream& os, int indent_spaces) { IRPrinterPass(indent_spaces).Run(func, os); }
+}  // namespace pass
+
 DataType PromoteTypes(DataType a, DataType b) {
     if (a == b) return a;
     if (a.is_float() || b.is_float()) {

@@ -27,6 +27,7 @@
 #include "kxc/profiling.h"
 #include "kxc/runtime_session.h"
 #include "kxc/topi.h"
+#include "kxc_hip.h"
 
 namespace {
 
@@ -838,6 +839,216 @@ int RunProfile(const std::string& dir) {
     return 0;
 }
 
+// HIP counterpart of the reference's only GPU test (test/cupti_smoke_test.cpp:95-267): device API allocation,
+// stream and copies, a fill, the kernel `scale_add` (y[i] = x[i] * alpha + 1, n = 64, block 128, grid 1, multiply and
+// add rounded separately) compiled at run time and launched on the device API's stream, all inside a profiling
+// context; the bundle must then hold backend.hip events of every kind: hip_runtime_api, hip_memcpy, hip_memset,
+// hip_kernel.
+int RunHipSmoke(const std::string& dir) {
+    namespace profiling = kxc::profiling;
+    auto target = kxc::BuildTarget(kxc::kGPU);
+    Check(target->attrs.exists == 1, "hip_smoke needs a GPU: " + target->attrs.status);
+    profiling::ProfileOptions options;
+    options.enabled = true;
+    options.bundle_dir = dir;
+    options.enable_gpu_activity = true;
+    auto ctx = profiling::ProfileContext::Create(options);
+    const std::string run_id = ctx->NextRunId("hip-smoke");
+    {
+        profiling::ActivationScope activation(ctx, run_id);
+        profiling::EventSpec root_spec;
+        root_spec.component = "test";
+        root_spec.event_type = "hip_smoke";
+        profiling::ScopedSpan root_span(ctx, std::move(root_spec), run_id);
+
+        kxc::DeviceAPI* api = kxc::DeviceAPIManager::Global()->GetAPI(kxc::kGPU);
+        const kxc::Device gpu(kxc::kGPU, 0), cpu(kxc::kCPU, 0);
+        std::vector<float> host_in(64, 3.5f), host_out(64, -1.0f);
+        const size_t nbytes = host_in.size() * sizeof(float);
+        api->SetDevice(gpu);
+        void* gpu_buf = api->AllocDataSpace(gpu, nbytes, 64);
+        void* gpu_out = api->AllocDataSpace(gpu, nbytes, 64);
+        kxc::StreamHandle stream = api->CreateStream(gpu);
+        api->SetStream(gpu, stream);
+        api->CopyDataFromTo(cpu, host_in.data(), gpu, gpu_buf, nbytes);
+        Check(kxc_hip_memset(gpu_buf, 0, nbytes, 0, stream) == 0, std::string("memset: ") + kxc_hip_last_error());
+        api->CopyDataFromTo(host_in.data(), 0, gpu_buf, 0, nbytes, cpu, gpu, stream);
+
+        const char* source = R"(
+extern "C" __global__ void scale_add(const float* x, float* y, float alpha, int n) {
+  int i = blockIdx.x * blockDim.x + threadIdx.x;
+  if (i < n) {
+    y[i] = x[i] * alpha + 1.0f;
+  }
+}
+)";
+        kxc_hip_module* module = nullptr;
+        std::vector<char> log(4096, 0);
+        Check(kxc_hip_module_compile(source, "scale_add.hip", &module, log.data(), log.size()) == 0,
+              std::string("compile: ") + kxc_hip_last_error());
+        void* kernel = nullptr;
+        Check(kxc_hip_module_get_function(module, "scale_add", &kernel) == 0, std::string("get_function: ") + kxc_hip_last_error());
+        float alpha = 2.0f;
+        int n = static_cast<int>(host_in.size());
+        void* kernel_args[] = {&gpu_buf, &gpu_out, &alpha, &n};
+        const uint32_t block[3] = {128, 1, 1};
+        const uint32_t grid[3] = {static_cast<uint32_t>((n + 127) / 128), 1, 1};
+        Check(kxc_hip_module_launch(kernel, grid, block, 0, stream, kernel_args) == 0, std::string("launch: ") + kxc_hip_last_error());
+        api->CopyDataFromTo(gpu_out, 0, host_out.data(), 0, nbytes, gpu, cpu, stream);
+        api->StreamSync(gpu, stream);
+        kxc_hip_module_free(module);
+        for (float v : host_out) Check(v == 8.0f, "Kernel output verification failed");
+        api->SetStream(gpu, nullptr);
+        api->FreeStream(gpu, stream);
+        api->FreeDataSpace(gpu, gpu_out);
+        api->FreeDataSpace(gpu, gpu_buf);
+        // single-attribute queries of the same back end
+        Check(kxc::GetDeviceAttr(gpu, kxc::DeviceAttrKind::kWarpSize) == 64 && kxc::GetDeviceAttr(gpu, kxc::DeviceAttrKind::kExist) == 1,
+              "GetAttr");
+        Check(kxc::DeviceAPI::NeedSetDevice(kxc::kGPU) && !kxc::DeviceAPI::NeedSetDevice(kxc::kCPU), "NeedSetDevice");
+    }
+    ctx->Flush();
+    std::ifstream manifest(dir + "/manifest.json");
+    std::string manifest_text((std::istreambuf_iterator<char>(manifest)), std::istreambuf_iterator<char>());
+    Check(manifest_text.find("\"enable_gpu_activity\":true") != std::string::npos, "manifest marks GPU activity as on");
+    bool saw_runtime = false, saw_memcpy = false, saw_memset = false, saw_kernel = false;
+    std::ifstream events(dir + "/events.jsonl");
+    std::string line;
+    while (std::getline(events, line)) {
+        if (line.find("\"component\":\"backend.hip\"") == std::string::npos) continue;
+        saw_runtime = saw_runtime || line.find("\"event_type\":\"hip_runtime_api\"") != std::string::npos;
+        saw_memcpy = saw_memcpy || line.find("\"event_type\":\"hip_memcpy\"") != std::string::npos;
+        saw_memset = saw_memset || line.find("\"event_type\":\"hip_memset\"") != std::string::npos;
+        saw_kernel = saw_kernel || (line.find("\"event_type\":\"hip_kernel\"") != std::string::npos &&
+                                    line.find("\"kernel_symbol\":\"scale_add\"") != std::string::npos);
+    }
+    Check(saw_runtime && saw_memcpy && saw_memset && saw_kernel, "Missing expected HIP activity events");
+    std::cout << "HIP bundle generated at: " << dir << "\n";
+    return 0;
+}
+
+// The device-side diagnosis rules on synthetic events: six module runs of 50 us, copies that make up most of the
+// device API time, and synchronisation that makes up a third of everything.
+int RunDiagnosis(const std::string& dir) {
+    namespace profiling = kxc::profiling;
+    profiling::ProfileOptions options;
+    options.enabled = true;
+    options.bundle_dir = dir;
+    options.enable_gpu_activity = false;
+    auto ctx = profiling::ProfileContext::Create(options);
+    Check(ctx->DiagnoseDeviceOverheads().empty(), "an empty context has no findings");
+    auto add = [&](const char* component, const char* type, std::int64_t start, std::int64_t dur) {
+        profiling::EventSpec e;
+        e.component = component;
+        e.event_type = type;
+        ctx->RecordCompletedSpan(e, "run-1", ctx->NextSpanId(), "", start, start + dur);
+    };
+    for (int i = 0; i < 6; ++i) add("runtime", "compiled_module_run", 1000 * i, 50000);
+    add("device_api", "copy", 400000, 900000);
+    add("device_api", "alloc_data_space", 1400000, 100000);
+    add("device_api", "stream_sync", 1500000, 700000);
+    const auto found = ctx->DiagnoseDeviceOverheads();
+    auto has = [&](const char* c) { for (const auto& d : found) if (d.category == c) return true; return false; };
+    Check(has("kernel_launch_overhead") && has("copy_dominance") && has("sync_overhead"), "all three rules fire");
+    ctx->Flush();
+    // one long module run and little copying: nothing fires
+    auto calm = profiling::ProfileContext::Create(options);
+    {
+        profiling::EventSpec e;
+        e.component = "runtime";
+        e.event_type = "compiled_module_run";
+        calm->RecordCompletedSpan(e, "run-1", calm->NextSpanId(), "", 0, 5000000);
+        e.component = "device_api"; e.event_type = "alloc_data_space";
+        calm->RecordCompletedSpan(e, "run-1", calm->NextSpanId(), "", 0, 1000);
+    }
+    Check(calm->DiagnoseDeviceOverheads().empty(), "a calm run has no findings");
+    // (what a caller publishes is kept)
+    ctx->PublishDiagnostics({{"pass_regression", "warn", "tir.transform", "published by a caller"}});
+    ctx->Flush();
+    std::ifstream f(dir + "/diagnosis.json");
+    std::string text((std::istreambuf_iterator<char>(f)), std::istreambuf_iterator<char>());
+    Check(text.find("pass_regression") != std::string::npos && text.find("copy_dominance") == std::string::npos, "published diagnosis is kept");
+    ctx->PublishDiagnostics({});
+    ctx->Flush();
+    std::cout << "diagnosis rules ok\n";
+    return 0;
+}
+
+// The compiled-kernel object and the compile-configuration surface (include/codegen/compiled_kernel.h:19-56,
+// include/api/compile_config.h:40-50, include/api/compiler.h:88): fields, IsReady, the call operator with the
+// reference's error texts, profile_options -> a module-owned context, GetProfileBundlePath.
+int RunKernelObject(const std::string& dir) {
+    using kxc::codegen::CodeGenBackend;
+    kxc::Var x("x", kxc::TensorType({2, 3}, "float32"));
+    kxc::Var y("y", kxc::TensorType({3}, "float32"));
+    kxc::Function add({x, y}, kxc::Call(Op::Get("add"), {x, y}));
+    auto config = MakeConfig();
+    config->profile_options.enabled = !dir.empty();
+    config->profile_options.bundle_dir = dir;
+    config->cache_dir = "";
+    auto module = kxc::api::Compiler::Compile(add, config);
+    const kxc::codegen::CompiledKernel kernel = module.GetKernel();
+    Check(kernel.defined() && kernel.IsReady() && module.IsReady(), "kernel is ready");
+    Check(kernel->kernel_name == "kxc_kernel_main", "kernel name: " + kernel->kernel_name);
+    Check(kernel->backend == (g_mode == "cpu" ? CodeGenBackend::kC : CodeGenBackend::kHIP), "kernel backend");
+    Check(kernel->func_ptr != nullptr, "IsReady <=> func_ptr");
+    Check(kernel->param_buffers.size() == 3 && kernel->param_buffers[0].shape == std::vector<int64_t>({2, 3}),
+          "param_buffers carries the packed-argument signature");
+    if (g_mode == "cpu") Check(kernel->lib_handle != nullptr && !kernel->so_path.empty(), "host back end owns its library");
+    else Check(kernel->jit_resource != nullptr && kernel->lib_handle == nullptr, "hip back end owns its launch plan");
+    std::vector<float> xd = {1, 2, 3, 4, 5, 6}, yd = {10, 20, 30}, out(6, 0.0f);
+    {
+        StagedArgs staged({In(xd), In(yd), Out(out)});
+        kernel(staged.args);                                   // the kernel object is callable by itself
+        staged.Fetch();
+        ExpectNear(out, {11, 22, 33, 14, 25, 36});
+    }
+    {
+        std::fill(out.begin(), out.end(), 0.0f);
+        StagedArgs staged({In(xd), In(yd), Out(out)});
+        module.Run(staged.args);
+        staged.Fetch();
+        ExpectNear(out, {11, 22, 33, 14, 25, 36});
+    }
+    bool threw = false;
+    try { kxc::codegen::CompiledKernel()(std::vector<void*>{}); } catch (const std::exception& e) {
+        threw = std::string(e.what()) == "CompiledKernel: not ready or func_ptr is null";
+    }
+    Check(threw, "an empty kernel refuses to run with the reference's message");
+    Check(!kxc::codegen::CompiledKernel().IsReady(), "an empty kernel is not ready");
+    if (g_mode != "cpu") {
+        // a failing launch surfaces as the Run ABI's error: "Kernel <name> returned error code N"
+        threw = false;
+        try { kernel(std::vector<void*>{nullptr, nullptr, nullptr}); } catch (const std::exception& e) {
+            threw = std::string(e.what()).rfind("Kernel kxc_kernel_main returned error code ", 0) == 0;
+        }
+        Check(threw, "kernel error text");
+    }
+    // a copy of the kernel handle keeps the resources alive after the module is gone
+    module = kxc::api::CompiledModule();
+    {
+        std::fill(out.begin(), out.end(), 0.0f);
+        StagedArgs staged({In(xd), In(yd), Out(out)});
+        kernel(staged.args);
+        staged.Fetch();
+        ExpectNear(out, {11, 22, 33, 14, 25, 36});
+    }
+    if (!dir.empty()) {
+        auto again = kxc::api::Compiler::Compile(add, config);
+        Check(again.GetProfileBundlePath() == dir, "GetProfileBundlePath: " + again.GetProfileBundlePath());
+        StagedArgs staged({In(xd), In(yd), Out(out)});
+        again.Run(staged.args);
+        std::ifstream events(dir + "/events.jsonl");
+        std::string all((std::istreambuf_iterator<char>(events)), std::istreambuf_iterator<char>());
+        Check(all.find("\"event_type\":\"compile\"") != std::string::npos, "the module's own context recorded the compile");
+        Check(all.find("\"run_id\":\"execute") != std::string::npos, "Run activates the module's context under an execute run id");
+        auto plain = MakeConfig();
+        Check(kxc::api::Compiler::Compile(add, plain).GetProfileBundlePath().empty(), "no profiling: empty bundle path");
+    }
+    std::cout << "kernel object ok (" << g_mode << ")\n";
+    return 0;
+}
+
 int main(int argc, char** argv) {
     try {
         const std::string cmd = argc > 1 ? argv[1] : "";
@@ -847,6 +1058,9 @@ int main(int argc, char** argv) {
         if (cmd == "codegen") return RunCodegen();
         if (cmd == "onnx" && argc >= 4) { g_mode = argv[2]; return RunOnnx(argv[3]); }
         if (cmd == "onnx_errors" && argc >= 3) return RunOnnxErrors(argv[2]);
+        if (cmd == "hip_smoke" && argc >= 3) return RunHipSmoke(argv[2]);
+        if (cmd == "diagnosis" && argc >= 3) return RunDiagnosis(argv[2]);
+        if (cmd == "kernel_object") { g_mode = argc > 2 ? argv[2] : "cpu"; return RunKernelObject(argc > 3 ? argv[3] : ""); }
         if (cmd == "profile" && argc >= 4) { g_mode = argv[2]; return RunProfile(argv[3]); }
         if (cmd == "resnet18" && argc >= 6) { g_mode = argv[2]; return RunResNet18(argv[3], std::atoll(argv[4]), std::atoll(argv[5])); }
         std::cerr << "usage: host_tests op_numeric <cpu|hip|hipgen> | device_info | codegen | resnet18 <cpu|hip|hipgen> <dir> <batch> <hw>\n";

@@ -89,6 +89,42 @@ int32_t kxc_hip_get_stream(int32_t device_id, void** out_stream);
 int32_t kxc_hip_stream_sync(int32_t device_id, void* stream);
 int32_t kxc_hip_stream_wait(int32_t device_id, void* src_stream, void* dst_stream);
 
+/* Fill (the reference's only GPU test uses cudaMemsetAsync beside the device API, test/cupti_smoke_test.cpp:113-118):
+ * every byte of [ptr, ptr + nbytes) = value & 0xff; stream NULL and no current stream: synchronous. */
+int32_t kxc_hip_memset(void* ptr, int32_t value, size_t nbytes, int32_t device_id, void* stream);
+
+/* Activity records for the profiling bundle: what the reference's CUPTI adapter collects for CUDA
+ * (src/base/profiling.cc:537-651: runtime API calls, memcpy, memset, kernels, each with start and end), taken at
+ * the library's own call sites.  While enabled, every HIP runtime call made by section 1 (device API) and section 3
+ * (module loader) leaves a RUNTIME_API record timed on the host, and every copy, fill and kernel launch they enqueue
+ * leaves a MEMCPY / MEMSET / KERNEL record timed on the GPU by two HIP events on its stream (timed_on_gpu = 1;
+ * synchronous copies are timed on the host).  Times are nanoseconds of the clock kxc_hip_activity_now_ns() reads.
+ * correlation_id ties a device record to the API record of the call that enqueued it.  kxc_hip_activity_drain
+ * hands over and forgets the finished records, waiting for device records still in flight; capacity 0 only counts. */
+#define KXC_HIP_ACTIVITY_RUNTIME_API 0
+#define KXC_HIP_ACTIVITY_MEMCPY 1
+#define KXC_HIP_ACTIVITY_MEMSET 2
+#define KXC_HIP_ACTIVITY_KERNEL 3
+typedef struct kxc_hip_activity_record {
+    int32_t kind;                    /* KXC_HIP_ACTIVITY_* */
+    char name[96];                   /* HIP runtime call, or kernel symbol */
+    int64_t start_ns, end_ns;
+    int64_t bytes;                   /* copies and fills */
+    int32_t value;                   /* fills */
+    int32_t copy_kind;               /* copies: 0 host->device, 1 device->host, 2 device->device, 3 host->host */
+    uint32_t grid[3], block[3];      /* kernels */
+    uint32_t dynamic_shared_memory;
+    uint64_t correlation_id;
+    int32_t return_value;            /* RUNTIME_API: hipError_t of the call */
+    int32_t device_id;
+    uint64_t stream;
+    uint64_t thread_id;
+    int32_t timed_on_gpu;
+} kxc_hip_activity_record;
+int32_t kxc_hip_activity_enable(int32_t enable);
+int32_t kxc_hip_activity_drain(kxc_hip_activity_record* records, int32_t capacity, int32_t* count);
+int64_t kxc_hip_activity_now_ns(void);
+
 /* ========================================================================
  * 2. Hand-written operators.  Each is the GPU implementation of one
  *    FRelayToTE compute definition (the CPU definition stays the fallback).

@@ -52,6 +52,22 @@ def test_device_info_contract():
     assert "device info ok" in run("device_info")
 
 
+def test_compiled_kernel_object_and_compile_config_surface_cpu():
+    """codegen::CompiledKernel (fields, IsReady, call operator, error text), CompileConfig::profile_options / cache_dir
+    and CompiledModule::GetProfileBundlePath on the host back end."""
+    with tempfile.TemporaryDirectory() as d:
+        assert "kernel object ok (cpu)" in run("kernel_object", "cpu", d)
+
+
+@pytest.mark.gpu
+def test_compiled_kernel_object_hip():
+    """The same object owning a launch plan: ready exactly while the plan can run, "Kernel <name> returned error code
+    N" when a launch is refused, resources alive as long as any handle."""
+    with tempfile.TemporaryDirectory() as d:
+        assert "kernel object ok (hip)" in run("kernel_object", "hip", d)
+    assert "kernel object ok (hipgen)" in run("kernel_object", "hipgen")
+
+
 def test_lowering_and_code_generators():
     assert "codegen ok" in run("codegen")
 
@@ -337,9 +353,61 @@ def test_profiling_bundle_hip_events():
                    for k in kernels)
         starts = [k["ts_ns"] for k in kernels]
         assert starts == sorted(starts)
-        copies = [e for e in events if e["component"] == "device_api" and e["event_type"] == "copy_data_from_to"]
+        copies = [e for e in events if e["component"] == "device_api" and e["event_type"] == "copy"]
         assert copies and all(c["metrics"]["bytes"] > 0 for c in copies)
         assert summary["component_counts"]["backend.hip"] >= len(kernels)
+
+
+@pytest.mark.gpu
+def test_hip_smoke_bundle_has_every_activity_kind():
+    """The HIP counterpart of the reference's only GPU test (test/cupti_smoke_test.cpp:95-267): device API calls, a
+    fill, the run-time compiled `scale_add` kernel launched with hipModuleLaunchKernel on a device-API stream.  The
+    bundle holds backend.hip events of all four kinds with the metric keys of the reference's CUDA records
+    (src/base/profiling.cc:537-651), device_api spans the bundle analyser's rules read, and a diagnosis."""
+    with tempfile.TemporaryDirectory() as d:
+        assert "HIP bundle generated at:" in run("hip_smoke", d)
+        events, manifest, summary = _read_bundle(d)
+        diagnosis = json.load(open(os.path.join(d, "diagnosis.json")))
+    hip = [e for e in events if e["component"] == "backend.hip"]
+    by_type = {}
+    for e in hip:
+        by_type.setdefault(e["event_type"], []).append(e)
+    assert set(by_type) == {"hip_runtime_api", "hip_memcpy", "hip_memset", "hip_kernel"}
+    apis = {e["fields"]["backend.hip.api"] for e in by_type["hip_runtime_api"]}
+    assert {"hipMalloc", "hipStreamCreate", "hipMemsetAsync", "hipMemcpyAsync", "hipModuleLaunchKernel",
+            "hipStreamSynchronize", "hipFree"} <= apis
+    assert all(e["fields"]["backend.hip.return_value"] == "0" for e in by_type["hip_runtime_api"])
+    (kernel,) = by_type["hip_kernel"]
+    assert kernel["kernel_symbol"] == "scale_add" and kernel["device"] == "hip:0"
+    m = kernel["metrics"]
+    assert (m["grid_x"], m["grid_y"], m["grid_z"], m["block_x"], m["block_y"], m["block_z"]) == (1, 1, 1, 128, 1, 1)
+    assert m["dynamic_shared_memory"] == 0 and kernel["duration_ns"] > 0
+    assert kernel["fields"]["backend.hip.timing_source"] == "hip_events"
+    (fill,) = by_type["hip_memset"]
+    assert fill["metrics"]["bytes"] == 256 and fill["metrics"]["value"] == 0
+    copies = by_type["hip_memcpy"]
+    assert len(copies) == 3 and all(c["metrics"]["bytes"] == 256 and c["metrics"]["copy_count"] == 1 for c in copies)
+    assert sorted(c["fields"]["backend.hip.copy_kind"] for c in copies) == ["0", "0", "1"]
+    # every device record is tied to the API call that enqueued it
+    api_ids = {e["fields"]["backend.hip.correlation_id"] for e in by_type["hip_runtime_api"]}
+    assert all(e["fields"]["backend.hip.correlation_id"] in api_ids for e in copies + [fill, kernel])
+    # on the stream (the thread's current one): copy in, fill, copy in again, the kernel, the copy out
+    order = sorted([fill, kernel] + copies, key=lambda e: e["ts_ns"])
+    assert [e["event_type"] for e in order] == ["hip_memcpy", "hip_memset", "hip_memcpy", "hip_kernel", "hip_memcpy"]
+    assert len({e["fields"]["backend.hip.stream_id"] for e in order}) == 1
+    device_api = [e for e in events if e["component"] == "device_api"]
+    assert {"alloc_data_space", "copy", "stream_sync", "free_data_space"} <= {e["event_type"] for e in device_api}
+    assert manifest["enable_gpu_activity"] is True
+    assert diagnosis["diagnostics"] and all({"category", "severity", "component", "summary"} <= set(x) for x in diagnosis["diagnostics"])
+
+
+def test_bundle_diagnosis_rules_cpu():
+    """kernel_launch_overhead / copy_dominance / sync_overhead as the reference's bundle analyser defines them
+    (python/kxc_agent/services/diagnosis_engine.py:233-297), evaluated when a bundle is written."""
+    with tempfile.TemporaryDirectory() as d:
+        assert "diagnosis rules ok" in run("diagnosis", d)
+        cats = {x["category"] for x in json.load(open(os.path.join(d, "diagnosis.json")))["diagnostics"]}
+    assert {"kernel_launch_overhead", "copy_dominance", "sync_overhead"} <= cats
 
 
 # ------------------------------------------------------------------ ONNX import wire format
