@@ -23,7 +23,9 @@
 // Both are written by LDS-direct buffer loads of 16 bytes per lane and double buffered.
 // A k-step is 32 reduction values: lane half h takes linear index q = 2*step + h of the chunk's
 // (tap, channel block) pairs, q = tap*CBC + cb_local; indices past the end carry zero weights.
+#include <cstdlib>
 #include <cstring>
+#include <type_traits>
 #include <vector>
 
 #include "common.h"
@@ -125,30 +127,55 @@ __device__ __forceinline__ void epilogue_c16(const intx16 (&acc)[RO], const QArg
                 resw[i][j] = *reinterpret_cast<const uint32_t*>(a.res + offset(o < a.O ? o : 0));
             }
     }
+    // These kernels are bound by instruction issue around the (very fast) int8 matrix instructions, so the
+    // requantisation is kept short: the ReLU form needs no NaN select (the clamp's lower bound 0 is also what a NaN
+    // maps to: a median-of-three with a NaN operand returns the smaller of the other two), the clamp is one
+    // median instruction, and four results are packed with three byte permutes.
+    auto finish = [&](auto relu_c, auto res_c) {
+        constexpr bool kRelu = decltype(relu_c)::value, kRes = decltype(res_c)::value;
 #pragma unroll
-    for (int i = 0; i < RO; ++i) {
+        for (int i = 0; i < RO; ++i) {
 #pragma unroll
-        for (int j = 0; j < 4; ++j) {
-            const int o = group(i, j);
-            const float ms[4] = {mv[i][j].x, mv[i][j].y, mv[i][j].z, mv[i][j].w};
-            const int bs[4] = {bv[i][j].x, bv[i][j].y, bv[i][j].z, bv[i][j].w};
-            uint32_t outw = 0;
+            for (int j = 0; j < 4; ++j) {
+                const int o = group(i, j);
+                const float ms[4] = {mv[i][j].x, mv[i][j].y, mv[i][j].z, mv[i][j].w};
+                const int bs[4] = {bv[i][j].x, bv[i][j].y, bv[i][j].z, bv[i][j].w};
+                int32_t q[4];
 #pragma unroll
-            for (int e = 0; e < 4; ++e) {
-                const int32_t rq = static_cast<int32_t>(static_cast<int8_t>((resw[i][j] >> (8 * e)) & 0xff));
-                const int32_t q = requant_i32(acc[i][4 * j + e] + bs[e], ms[e], has_res, rq, a.res_mult, do_relu);
-                outw |= (static_cast<uint32_t>(q) & 0xffu) << (8 * e);
+                for (int e = 0; e < 4; ++e) {
+                    float v = __fmul_rn(static_cast<float>(acc[i][4 * j + e] + bs[e]), ms[e]);
+                    if (kRes) {
+                        const int32_t rq = static_cast<int32_t>(static_cast<int8_t>((resw[i][j] >> (8 * e)) & 0xff));
+                        v = __fadd_rn(v, __fmul_rn(static_cast<float>(rq), a.res_mult));
+                    }
+                    float r = rintf(v);
+                    if (!kRelu) r = (v == v) ? r : 0.0f;
+                    r = __builtin_amdgcn_fmed3f(r, kRelu ? 0.0f : -128.0f, 127.0f);
+                    q[e] = static_cast<int32_t>(r);
+                }
+                const uint32_t lo = __builtin_amdgcn_perm(static_cast<uint32_t>(q[1]), static_cast<uint32_t>(q[0]), 0x0c0c0400u);
+                const uint32_t hi = __builtin_amdgcn_perm(static_cast<uint32_t>(q[3]), static_cast<uint32_t>(q[2]), 0x0c0c0400u);
+                const uint32_t outw = __builtin_amdgcn_perm(hi, lo, 0x05040100u);
+                if (o < a.O) *reinterpret_cast<uint32_t*>(a.y + offset(o)) = outw;
             }
-            if (o < a.O) *reinterpret_cast<uint32_t*>(a.y + offset(o)) = outw;
         }
-    }
+    };
+    using T = std::true_type;
+    using F = std::false_type;
+    if (do_relu) { if (has_res) finish(T{}, T{}); else finish(T{}, F{}); }
+    else { if (has_res) finish(F{}, T{}); else finish(F{}, F{}); }
 }
 
-template <int KH, int KW, int CBC, int WP, int RO, int PPT>
+// RP: 32-pixel blocks per wave (a wave computes RO x RP blocks; a weight operand then feeds RP matrix
+// instructions and a pixel operand RO of them).  These kernels are bound by the latency chain of a workgroup
+// (set-up, first loads, one weight fetch per k-step, epilogue), not by the matrix pipe, so a launch runs fastest
+// when all its waves are resident at once: larger per-wave tiles trade idle matrix cycles for fewer waves.
+// WD: depth of the weight ring in k-steps (must divide the k-steps of a chunk).
+template <int KH, int KW, int CBC, int WP, int RO, int PPT, int RP = 1, int WD = 0>
 __global__ void __launch_bounds__(64 * WP) __attribute__((amdgpu_waves_per_eu(2))) qconv_mfma_kernel(const QArgs a) {
     constexpr int KHW = KH * KW;
     constexpr int NS = (KHW * CBC + 1) / 2;          // matrix k-steps per chunk
-    constexpr int TP = 32 * WP;
+    constexpr int TP = 32 * WP * RP;
 
     extern __shared__ __attribute__((aligned(16))) char lds[];
     const int tid = threadIdx.x;
@@ -195,24 +222,27 @@ __global__ void __launch_bounds__(64 * WP) __attribute__((amdgpu_waves_per_eu(2)
         goff[i] = ok ? (static_cast<uint32_t>(n) * a.CB * a.H * a.W + static_cast<uint32_t>(ih * a.W + iw)) * 16u : kOob;
     }
 
-    // per-lane operand base: byte address of the pixel's (tap 0, channel block 0) position
-    const int m = m0 + wave * 32 + r;
-    int xbase;
-    int ypix;            // position index (n*OB16*OHW + pixel) of this lane's output pixel for block 0, or -1
-    {
+    // per-lane operand bases: byte address of each pixel's (tap 0, channel block 0) position
+    int xbase[RP];
+    int ypix[RP];        // position index (n*OB16*OHW + pixel) of this lane's output pixel for block 0, or -1
+#pragma unroll
+    for (int j = 0; j < RP; ++j) {
+        const int m = m0 + (wave * RP + j) * 32 + r;
         const int mc = min(m, a.M - 1);
         const int n = fast_div(mc, a.div_ohw), rem = mc - n * a.OHW;
         const int oh = fast_div(rem, a.div_ow), ow = rem - oh * a.OW;
-        xbase = ((n * a.Hp + oh * a.sh - qmin) * a.Wp + ow * a.sw) * 16;
-        if (CBC > 1) xbase += half * a.chs * 16;
-        ypix = (m < a.M) ? n * (a.O >> 4) * a.OHW + rem : -1;
+        xbase[j] = ((n * a.Hp + oh * a.sh - qmin) * a.Wp + ow * a.sw) * 16;
+        if (CBC > 1) xbase[j] += half * a.chs * 16;
+        ypix[j] = (m < a.M) ? n * (a.O >> 4) * a.OHW + rem : -1;
     }
 
-    intx16 acc[RO];
+    intx16 acc[RP][RO];
 #pragma unroll
-    for (int i = 0; i < RO; ++i)
+    for (int j = 0; j < RP; ++j)
 #pragma unroll
-        for (int g = 0; g < 16; ++g) acc[i][g] = 0;
+        for (int i = 0; i < RO; ++i)
+#pragma unroll
+            for (int g = 0; g < 16; ++g) acc[j][i][g] = 0;
 
     auto issue_loads = [&](int chunk, char* buf) {
 #pragma unroll
@@ -237,7 +267,8 @@ __global__ void __launch_bounds__(64 * WP) __attribute__((amdgpu_waves_per_eu(2)
     // through the vector cache.  A ring of D steps is kept in flight across chunk boundaries; loads past the
     // last step fall outside the buffer and return 0 without a branch.  With the weights out of LDS a workgroup
     // needs only the patch (12 KiB per buffer for a 56-wide map), which triples the resident workgroups per CU.
-    constexpr int D = (NS % 3 == 0) ? 3 : (NS % 5 == 0 ? 5 : (NS % 2 == 0 ? 2 : 1));
+    constexpr int D = WD > 0 ? WD : ((NS % 3 == 0) ? 3 : (NS % 5 == 0 ? 5 : (NS % 2 == 0 ? 2 : 1)));
+    static_assert(NS % D == 0, "the weight ring must divide the k-steps of a chunk");
     const uint32_t total_steps = static_cast<uint32_t>(a.nchunks) * NS;
     uint32_t wvoff[RO];
 #pragma unroll
@@ -263,7 +294,7 @@ __global__ void __launch_bounds__(64 * WP) __attribute__((amdgpu_waves_per_eu(2)
             const int rh = t / KW, rw = t - rh * KW;
             return (rh * a.Wp + rw) * 16;
         };
-        auto fetch_b = [&](int step) -> intx4 {
+        auto fetch_b = [&](int step, intx4 (&b)[RP]) {
             int off;
             if constexpr (CBC == 1) {
                 off = half ? tap_off(2 * step + 1) : tap_off(2 * step);
@@ -271,28 +302,35 @@ __global__ void __launch_bounds__(64 * WP) __attribute__((amdgpu_waves_per_eu(2)
                 constexpr int H2 = CBC / 2;
                 off = tap_off(step / H2) + 2 * (step % H2) * a.chs * 16;
             }
-            return *reinterpret_cast<const intx4*>(buf + xbase + off);
+#pragma unroll
+            for (int j = 0; j < RP; ++j) b[j] = *reinterpret_cast<const intx4*>(buf + xbase[j] + off);
         };
         const uint32_t t0 = static_cast<uint32_t>(chunk) * NS;
-        intx4 bcur = fetch_b(0);
+        intx4 bcur[RP], bnext[RP];
+        fetch_b(0, bcur);
 #pragma unroll
         for (int step = 0; step < NS; ++step) {
-            intx4 bnext = bcur;
-            if (step + 1 < NS) bnext = fetch_b(step + 1);
+            if (step + 1 < NS) fetch_b(step + 1, bnext);
 #pragma unroll
-            for (int i = 0; i < RO; ++i)
-                acc[i] = __builtin_amdgcn_mfma_i32_32x32x32_i8(ring[step % D][i], bcur, acc[i], 0, 0, 0);
+            for (int j = 0; j < RP; ++j)
+#pragma unroll
+                for (int i = 0; i < RO; ++i)
+                    acc[j][i] = __builtin_amdgcn_mfma_i32_32x32x32_i8(ring[step % D][i], bcur[j], acc[j][i], 0, 0, 0);
 #pragma unroll
             for (int i = 0; i < RO; ++i) ring[step % D][i] = load_a(i, t0 + step + D);
-            bcur = bnext;
+            if (step + 1 < NS) {
+#pragma unroll
+                for (int j = 0; j < RP; ++j) bcur[j] = bnext[j];
+            }
         }
         // every load older than the D*RO ring refills just issued has completed: that includes the next patch
         asm volatile("s_waitcnt vmcnt(%0)" ::"n"(D * RO) : "memory");
         __syncthreads();
     }
 
-    if (ypix < 0) return;
-    epilogue_c16<RO>(acc, a, ypix, ob0, half);
+#pragma unroll
+    for (int j = 0; j < RP; ++j)
+        if (ypix[j] >= 0) epilogue_c16<RO>(acc[j], a, ypix[j], ob0, half);
 }
 
 // ------------------------------------------------------------------------------------------------
@@ -579,13 +617,17 @@ __global__ void __launch_bounds__(kBlock) gap_c16_kernel(const int8_t* __restric
 // ------------------------------------------------------------------ host side
 struct QVariant {
     const char* name;
-    int kh, kw, cbc, wp, ro, ppt;
+    int kh, kw, cbc, wp, ro, ppt, rp;
     void (*kernel)(const QArgs);
 };
 
 #define KXC_QV(KH, KW, CBC, WP, RO, PPT)                                                             \
-    { "qmfma_k" #KH "x" #KW "_cb" #CBC "_p" #WP "_o" #RO, KH, KW, CBC, WP, RO, PPT,                      \
+    { "qmfma_k" #KH "x" #KW "_cb" #CBC "_p" #WP "_o" #RO, KH, KW, CBC, WP, RO, PPT, 1,                   \
       qconv_mfma_kernel<KH, KW, CBC, WP, RO, PPT> }
+// (RP pixel blocks per wave, weight ring of WD k-steps)
+#define KXC_QV2(KH, KW, CBC, WP, RO, PPT, RP, WD)                                                    \
+    { "qmfma_k" #KH "x" #KW "_cb" #CBC "_p" #WP "x" #RP "_o" #RO "_d" #WD, KH, KW, CBC, WP, RO, PPT, RP,  \
+      qconv_mfma_kernel<KH, KW, CBC, WP, RO, PPT, RP, WD> }
 
 const QVariant kQVariants[] = {
     KXC_QV(3, 3, 2, 4, 2, 4),
@@ -600,8 +642,17 @@ const QVariant kQVariants[] = {
     KXC_QV(1, 1, 1, 2, 1, 6),
     KXC_QV(7, 7, 1, 4, 2, 12),
     KXC_QV(7, 7, 1, 2, 2, 12),
+    // two pixel blocks per wave (chosen by the shape rules in PrepareUncached, or by name); a deeper weight ring (nine
+    // k-steps instead of three) was measured too and changed nothing
+    KXC_QV2(3, 3, 2, 4, 2, 8, 2, 3),
+    KXC_QV2(3, 3, 2, 4, 1, 8, 2, 3),
+    KXC_QV2(3, 3, 2, 2, 2, 8, 2, 3),
+    KXC_QV2(3, 3, 2, 2, 1, 8, 2, 3),
 };
 
+// Channel blocks (of 16 channels) per LDS chunk.  Larger chunks (64 or 128 channels) were measured on the ResNet-18
+// layers at batch 64 and were slower everywhere (512 -> 512 channels at 7 x 7: 14.3 -> 15-20 us; 256 -> 512 with
+// stride 2: 11 -> 23 us): with few chunks the first, large patch load is exposed and nothing overlaps it.
 int CbcFor(int c, int kh, int kw) {
     const int cb = (c + 15) / 16;
     if (cb == 1) return 1;
@@ -638,6 +689,8 @@ int32_t Prepare(const kxc_hip_qconv2d_desc* d, QLaunch* L, const char* who) {
     KXC_HIP_REQUIRE(d != nullptr, "%s: desc is NULL", who);
     struct Entry { kxc_hip_qconv2d_desc desc; QLaunch launch; };
     thread_local std::vector<Entry> cache;
+    if (const char* f = std::getenv("KXC_HIP_QCONV_VARIANT"))
+        if (*f) return PrepareUncached(d, L, who);          // forced variants are not cached
     for (const Entry& e : cache)
         if (std::memcmp(&e.desc, d, sizeof(*d)) == 0) { *L = e.launch; return KXC_HIP_OK; }
     if (int32_t rc = PrepareUncached(d, L, who)) return rc;
@@ -682,10 +735,27 @@ int32_t PrepareUncached(const kxc_hip_qconv2d_desc* d, QLaunch* L, const char* w
     // pick the first variant that fits, preferring enough workgroups to fill 256 CUs a few times over
     const QVariant* best = nullptr;
     int best_chs = 0;
+    const char* forced = std::getenv("KXC_HIP_QCONV_VARIANT");        // a variant by name (kernel experiments, tests)
+    // Shape rules, from a sweep of every 3x3 variant over the ResNet-18 layers at batch 64 (the kernels are bound by
+    // instruction issue around the matrix instructions, so fewer, larger per-wave tiles win while there are enough
+    // pixels): stride 1 with at least 8192 output pixels takes two pixel blocks per wave (64 -> 64 channels at 56 x 56:
+    // 21.4 -> 17.7 us; 128 at 28 x 28: 17.8 -> 13.6; 256 at 14 x 14: 15.4 -> 12.4), stride 2 two output-channel
+    // blocks per wave (128 -> 256 at 28 -> 14: 11.7 -> 10.2 us); the small 7 x 7 maps keep one block per wave.
+    if (!(forced && *forced) && d->kh == 3 && d->kw == 3 && cbc == 2) {
+        if (d->stride_h == 1 && d->stride_w == 1 && M >= 8192) forced = M >= 100000 ? "qmfma_k3x3_cb2_p4x2_o1_d3" : "qmfma_k3x3_cb2_p2x2_o1_d3";
+        else if (d->stride_h == 2 && d->stride_w == 2 && (a.O / 32) % 2 == 0 && M >= 2048) forced = "qmfma_k3x3_cb2_p4_o2";
+    }
+    const bool by_rule = forced && *forced && !(std::getenv("KXC_HIP_QCONV_VARIANT") && *std::getenv("KXC_HIP_QCONV_VARIANT"));
+    for (int pass = 0; pass < 2 && best == nullptr; ++pass) {
+    if (pass == 1) {
+        if (!by_rule) break;
+        forced = nullptr;           // the rule's variant does not hold this shape's patch: walk the table
+    }
     for (const QVariant& v : kQVariants) {
         if (v.kh != d->kh || v.kw != d->kw || v.cbc != cbc) continue;
         if ((a.O / 32) % v.ro != 0) continue;
-        const int TP = 32 * v.wp;
+        if (forced && *forced ? std::strcmp(forced, v.name) != 0 : v.rp != 1 || std::strstr(v.name, "_d") != nullptr) continue;
+        const int TP = 32 * v.wp * v.rp;
         const int rows = MaxRows(a, v.kh, TP);
         const int positions = rows * a.Wp;
         const int segs = (positions + 63) / 64;
@@ -696,11 +766,12 @@ int32_t PrepareUncached(const kxc_hip_qconv2d_desc* d, QLaunch* L, const char* w
         if (lds > 160 * 1024) continue;
         const int64_t tiles = CeilDiv(M, TP) * ((a.O / 32) / v.ro);
         if (best == nullptr) { best = &v; best_chs = chs; L->lds_bytes = lds; }
-        if (tiles >= 2 * 256) { best = &v; best_chs = chs; L->lds_bytes = lds; break; }
+        if (tiles >= 2 * 256 || (forced && *forced)) { best = &v; best_chs = chs; L->lds_bytes = lds; break; }
+    }
     }
     KXC_HIP_REQUIRE(best != nullptr, "%s: no matrix-core variant for a %dx%d filter on this shape", who, d->kh, d->kw);
     a.chs = best_chs;
-    a.p_tiles = static_cast<int32_t>(CeilDiv(M, 32 * best->wp));
+    a.p_tiles = static_cast<int32_t>(CeilDiv(M, 32 * best->wp * best->rp));
     a.o_tiles = (a.O / 32) / best->ro;
     a.num_tiles = a.p_tiles * a.o_tiles;
     a.tiles_per_xcd = (a.num_tiles + 7) / 8;

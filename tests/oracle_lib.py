@@ -252,8 +252,8 @@ class Oracle:
 class RefCases:
     """oracle/_ref/libkxc_ref_cases.so: the reference's own lowering + C code generator output.
 
-    Present only where it was built from the reference checkout (the built library is carried
-    along to GPU machines; its sources are not)."""
+    Present only where it was built from the reference checkout (the build container); GPU machines get the
+    committed fixtures written from it instead."""
 
     PATH = os.path.join(ORACLE_DIR, "_ref", "libkxc_ref_cases.so")
 
