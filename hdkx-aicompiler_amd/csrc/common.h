@@ -88,10 +88,44 @@ struct SplitReduceArgs {
 // on the same stream out until the adding kernel has been enqueued behind the parts (release it after that).
 struct SplitScratchLease {
     float* ptr = nullptr;
+    uint32_t* counters = nullptr;      // kSplitCounters arrival counters, all zero between launches
     std::unique_lock<std::mutex> lock;
 };
 int32_t AcquireSplitScratch(hipStream_t stream, size_t bytes, SplitScratchLease* lease);
 int32_t LaunchSplitReduce(hipStream_t stream, const SplitReduceArgs& a);
+
+// A split reduction without the adding kernel: every part stores its raw partial outputs as before, then counts
+// itself in at its tile's arrival counter; the part that arrives last adds all parts in split order (the same
+// order, hence the same bits, as the adding kernel) and applies the epilogue.  The counters sit in front of the
+// partial outputs, start at zero and are set back to zero by the last arrival, so a launch (or the replay of a
+// captured one) leaves them as it found them.  Launches that share a scratch buffer are ordered by their stream.
+constexpr int32_t kSplitCounters = 16384;
+constexpr size_t kSplitCounterBytes = static_cast<size_t>(kSplitCounters) * sizeof(uint32_t);
+// Largest number of parts the last arrival finishes itself (0: the adding kernel always does; see split_reduce.hip).
+int32_t SplitFuseMaxParts();
+
+#if defined(__HIPCC__)
+// Cache policy of the parts' stores and of the last part's loads of partial outputs: device scope (sc1), i.e.
+// written through to and read from the level all XCDs share.  With it no cache-wide write-back or invalidate is
+// needed around the counter (a release fence at device scope writes back the whole L2 of the XCD: measured at about
+// 20 us per launch of 200 workgroups).
+constexpr int kDeviceScopeAux = 0x10;
+// True for the workgroup that arrives last of `parts` at `counter`.  Every thread of the workgroup calls it after
+// its device-scope stores of partial outputs; `flag` is a word of LDS nobody else uses until the call returns.
+// The counter is bumped by a vector memory atomic at device scope once every wave's stores have been acknowledged.
+__device__ __forceinline__ bool split_arrive_last(uint32_t* counter, int32_t parts, uint32_t* flag) {
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+    __syncthreads();
+    if (threadIdx.x == 0) {
+        const uint32_t prev = __hip_atomic_fetch_add(counter, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        const bool last = prev + 1u == static_cast<uint32_t>(parts);
+        if (last) __hip_atomic_store(counter, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        *flag = last ? 1u : 0u;
+    }
+    __syncthreads();
+    return *flag != 0u;
+}
+#endif
 
 // The filter transforms of several Winograd layers in one launch (conv2d_wino_f32.hip).
 struct WinoWeightJob {

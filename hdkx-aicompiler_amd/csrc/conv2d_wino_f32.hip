@@ -28,6 +28,7 @@
 #include <cstdlib>
 #include <cstring>
 #include <mutex>
+#include <type_traits>
 #include <utility>
 #include <vector>
 
@@ -60,6 +61,7 @@ struct WinoArgs {
     // write raw partial outputs to partial[split][N*O*OH*OW]; a second kernel adds them and applies the epilogue
     int32_t gsplit, steps_per_split;
     float* partial;
+    uint32_t* counters;              // FUSE kernels: arrival counter of unit i at counters[i], zero between launches
     FastDiv div_ti, div_tw, div_kgroups, div_tgroups, div_gsplit;
 };
 
@@ -143,9 +145,12 @@ __global__ void __launch_bounds__(256) wino_weight_batch_kernel(const WinoWeight
 // One step = 4 input channels.  LDS per buffer: U [WK][c4][o/16: 2][f/4: 4][o%16][f%4] and
 // V [c4][WT][f/4: 4][tile%16][f%4]; two of each.
 // ------------------------------------------------------------------------------------------
-template <int WK, int WT, int KS>
+// FUSE: a reduction split over workgroups is finished by the part that arrives last (see split_arrive_last)
+// instead of the adding kernel.
+template <int WK, int WT, int KS, bool FUSE = false>
 __global__ void __launch_bounds__(64 * WK * WT * KS) __attribute__((amdgpu_waves_per_eu(2)))
 wino_kernel(const WinoArgs a) {
+    static_assert(!FUSE || KS == 1, "the split over workgroups is never combined with the split over wave groups");
     constexpr int NW = WK * WT;                     // waves of one reduction group
     constexpr int NTH = 64 * NW;                    // threads of one reduction group
     constexpr int TT = 16 * WT;
@@ -368,22 +373,11 @@ wino_kernel(const WinoArgs a) {
     const int oh = 2 * ty, ow = 2 * tx;
     const bool row1 = oh + 1 < a.OH, col1 = ow + 1 < a.OW;
     const bool vec2 = (a.OW & 1) == 0;
-    // (a part of a split reduction stores its raw output transform; the adding kernel applies the epilogue)
-    const uint32_t flags = a.gsplit > 1 ? 0u : a.flags;
-    const bool has_bias = (flags & KXC_HIP_CONV_BIAS) != 0;
-    const bool has_res = (flags & KXC_HIP_CONV_RESIDUAL) != 0;
-    const bool do_relu = (flags & KXC_HIP_CONV_RELU) != 0;
     const uint32_t y_bytes = static_cast<uint32_t>(a.N) * static_cast<uint32_t>(a.O) * static_cast<uint32_t>(a.OHW) * 4u;
-    float* const y_out = a.gsplit > 1 ? a.partial + static_cast<int64_t>(split) * (y_bytes / 4u) : a.y;
-    const __amdgpu_buffer_rsrc_t yr = make_rsrc(y_out, y_bytes);
-    const __amdgpu_buffer_rsrc_t rr = make_rsrc(has_res ? a.res : y_out, has_res ? y_bytes : 0u);
-    const __amdgpu_buffer_rsrc_t br = make_rsrc(has_bias ? a.bias : y_out, has_bias ? static_cast<uint32_t>(a.O) * 4u : 0u);
     const uint32_t rowb = static_cast<uint32_t>(a.OW) * 4u;
     const uint32_t rowmask = row1 ? 0u : kOob, colmask = col1 ? 0u : kOob;   // OR-ed into an offset: beyond the buffer
 
-    uint32_t off00[2][4];
-    float bv[2][4];
-    float q[2][4][4];
+    uint32_t off00[2][4], boff[2][4];
 #pragma unroll
     for (int kb = 0; kb < 2; ++kb)
 #pragma unroll
@@ -391,88 +385,145 @@ wino_kernel(const WinoArgs a) {
             const int o = (kg * WK + wave_k) * 32 + kb * 16 + 4 * (lane >> 4) + g;
             const bool ok = tile < a.NT && o < a.O;
             off00[kb][g] = ok ? static_cast<uint32_t>(((n * a.O + o) * a.OH + oh) * a.OW + ow) * 4u : kOob;
-            bv[kb][g] = load_f32(br, ok ? static_cast<uint32_t>(o) * 4u : kOob, 0);
+            boff[kb][g] = ok ? static_cast<uint32_t>(o) * 4u : kOob;
         }
-    if (has_res && vec2) {
-#pragma unroll
-        for (int kb = 0; kb < 2; ++kb)
-#pragma unroll
-            for (int g = 0; g < 4; ++g) {
-                const uint32_t o0 = off00[kb][g], o1 = (o0 + rowb) | rowmask;
-                // (two 4-byte loads per row: the 8-byte buffer-load builtin of this toolchain fetches only 4 bytes)
-                q[kb][g][0] = load_f32(rr, o0, 0); q[kb][g][1] = load_f32(rr, o0 + 4u, 0);
-                q[kb][g][2] = load_f32(rr, o1, 0); q[kb][g][3] = load_f32(rr, o1 + 4u, 0);
-            }
-    } else if (has_res) {
-#pragma unroll
-        for (int kb = 0; kb < 2; ++kb)
-#pragma unroll
-            for (int g = 0; g < 4; ++g) {
-                const uint32_t o0 = off00[kb][g], o1 = (o0 + rowb) | rowmask;
-                q[kb][g][0] = load_f32(rr, o0, 0);
-                q[kb][g][1] = load_f32(rr, (o0 + 4u) | colmask, 0);
-                q[kb][g][2] = load_f32(rr, o1, 0);
-                q[kb][g][3] = load_f32(rr, (o1 + 4u) | colmask, 0);
-            }
-    }
-    float yv[2][4][4];
-#pragma unroll
-    for (int kb = 0; kb < 2; ++kb) {
-#pragma unroll
-        for (int g = 0; g < 4; ++g) {
-            // A^T M A with A^T = [1 1 1 0; 0 1 -1 -1]
-            float r0[4], r1[4];
-#pragma unroll
-            for (int j = 0; j < 4; ++j) {
-                const float m0 = acc[j][kb][g], m1 = acc[4 + j][kb][g], m2 = acc[8 + j][kb][g], m3 = acc[12 + j][kb][g];
-                r0[j] = (m0 + m1) + m2;
-                r1[j] = (m1 - m2) - m3;
-            }
-            float y00 = (r0[0] + r0[1]) + r0[2], y01 = (r0[1] - r0[2]) - r0[3];
-            float y10 = (r1[0] + r1[1]) + r1[2], y11 = (r1[1] - r1[2]) - r1[3];
-            if (has_bias) {
-                const float bval = bv[kb][g];
-                y00 = __fadd_rn(y00, bval); y01 = __fadd_rn(y01, bval); y10 = __fadd_rn(y10, bval); y11 = __fadd_rn(y11, bval);
-            }
-            if (has_res) {
-                y00 = __fadd_rn(y00, q[kb][g][0]); y01 = __fadd_rn(y01, q[kb][g][1]);
-                y10 = __fadd_rn(y10, q[kb][g][2]); y11 = __fadd_rn(y11, q[kb][g][3]);
-            }
-            if (do_relu) { y00 = relu_sel(y00); y01 = relu_sel(y01); y10 = relu_sel(y10); y11 = relu_sel(y11); }
-            yv[kb][g][0] = y00; yv[kb][g][1] = y01; yv[kb][g][2] = y10; yv[kb][g][3] = y11;
-        }
-    }
+    // the four outputs of a tile from / to a tensor of the output's shape (also a part's raw outputs)
+    // (aux: cache policy of the access, a compile-time constant passed as a type)
+    auto load4 = [&](const __amdgpu_buffer_rsrc_t r, int kb, int g, float (&v)[4], auto aux) {
+        constexpr int AUX = decltype(aux)::value;
+        const uint32_t o0 = off00[kb][g], o1 = (o0 + rowb) | rowmask;
+        auto ld = [&](uint32_t off) { return __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(r, off, 0, AUX)); };
+        // (two 4-byte loads per row: the 8-byte buffer-load builtin of this toolchain fetches only 4 bytes)
+        v[0] = ld(o0);
+        v[1] = ld((o0 + 4u) | colmask);      // (an even row length has no odd last column: the mask is 0)
+        v[2] = ld(o1);
+        v[3] = ld((o1 + 4u) | colmask);
+    };
+    using Cached = std::integral_constant<int, 0>;
+    using DeviceScope = std::integral_constant<int, kDeviceScopeAux>;
     auto bits = [](float v) { return __builtin_bit_cast(uint32_t, v); };
-    if (vec2) {
+    auto store_all = [&](const __amdgpu_buffer_rsrc_t yr, const float (&yv)[2][4][4], auto aux) {
+        constexpr int AUX = decltype(aux)::value;
+        if (vec2) {
+#pragma unroll
+            for (int kb = 0; kb < 2; ++kb)
+#pragma unroll
+                for (int g = 0; g < 4; ++g) {
+                    const uint32_t o0 = off00[kb][g], o1 = (o0 + rowb) | rowmask;
+                    __builtin_amdgcn_raw_buffer_store_b64(uintx2{bits(yv[kb][g][0]), bits(yv[kb][g][1])}, yr, o0, 0, AUX);
+                    __builtin_amdgcn_raw_buffer_store_b64(uintx2{bits(yv[kb][g][2]), bits(yv[kb][g][3])}, yr, o1, 0, AUX);
+                }
+        } else {
+#pragma unroll
+            for (int kb = 0; kb < 2; ++kb)
+#pragma unroll
+                for (int g = 0; g < 4; ++g) {
+                    const uint32_t o0 = off00[kb][g], o1 = (o0 + rowb) | rowmask;
+                    __builtin_amdgcn_raw_buffer_store_b32(bits(yv[kb][g][0]), yr, o0, 0, AUX);
+                    __builtin_amdgcn_raw_buffer_store_b32(bits(yv[kb][g][1]), yr, (o0 + 4u) | colmask, 0, AUX);
+                    __builtin_amdgcn_raw_buffer_store_b32(bits(yv[kb][g][2]), yr, o1, 0, AUX);
+                    __builtin_amdgcn_raw_buffer_store_b32(bits(yv[kb][g][3]), yr, (o1 + 4u) | colmask, 0, AUX);
+                }
+        }
+    };
+    // A^T M A with A^T = [1 1 1 0; 0 1 -1 -1]
+    auto output_transform = [&](float (&yv)[2][4][4]) {
 #pragma unroll
         for (int kb = 0; kb < 2; ++kb)
 #pragma unroll
             for (int g = 0; g < 4; ++g) {
-                const uint32_t o0 = off00[kb][g], o1 = (o0 + rowb) | rowmask;
-                __builtin_amdgcn_raw_buffer_store_b64(uintx2{bits(yv[kb][g][0]), bits(yv[kb][g][1])}, yr, o0, 0, 0);
-                __builtin_amdgcn_raw_buffer_store_b64(uintx2{bits(yv[kb][g][2]), bits(yv[kb][g][3])}, yr, o1, 0, 0);
+                float r0[4], r1[4];
+#pragma unroll
+                for (int j = 0; j < 4; ++j) {
+                    const float m0 = acc[j][kb][g], m1 = acc[4 + j][kb][g], m2 = acc[8 + j][kb][g], m3 = acc[12 + j][kb][g];
+                    r0[j] = (m0 + m1) + m2;
+                    r1[j] = (m1 - m2) - m3;
+                }
+                yv[kb][g][0] = (r0[0] + r0[1]) + r0[2]; yv[kb][g][1] = (r0[1] - r0[2]) - r0[3];
+                yv[kb][g][2] = (r1[0] + r1[1]) + r1[2]; yv[kb][g][3] = (r1[1] - r1[2]) - r1[3];
             }
-    } else {
+    };
+    float bv[2][4];
+    float q[2][4][4];
+    // bias and residual of the layer's epilogue: issued early, used by finish()
+    auto issue_epilogue_loads = [&](bool has_bias, bool has_res, const float* any) {
+        const __amdgpu_buffer_rsrc_t rr = make_rsrc(has_res ? a.res : any, has_res ? y_bytes : 0u);
+        const __amdgpu_buffer_rsrc_t br = make_rsrc(has_bias ? a.bias : any, has_bias ? static_cast<uint32_t>(a.O) * 4u : 0u);
 #pragma unroll
         for (int kb = 0; kb < 2; ++kb)
 #pragma unroll
-            for (int g = 0; g < 4; ++g) {
-                const uint32_t o0 = off00[kb][g], o1 = (o0 + rowb) | rowmask;
-                __builtin_amdgcn_raw_buffer_store_b32(bits(yv[kb][g][0]), yr, o0, 0, 0);
-                __builtin_amdgcn_raw_buffer_store_b32(bits(yv[kb][g][1]), yr, (o0 + 4u) | colmask, 0, 0);
-                __builtin_amdgcn_raw_buffer_store_b32(bits(yv[kb][g][2]), yr, o1, 0, 0);
-                __builtin_amdgcn_raw_buffer_store_b32(bits(yv[kb][g][3]), yr, (o1 + 4u) | colmask, 0, 0);
+            for (int g = 0; g < 4; ++g) bv[kb][g] = load_f32(br, boff[kb][g], 0);
+        if (has_res) {
+#pragma unroll
+            for (int kb = 0; kb < 2; ++kb)
+#pragma unroll
+                for (int g = 0; g < 4; ++g) load4(rr, kb, g, q[kb][g], Cached{});
+        }
+    };
+    auto finish = [&](float (&yv)[2][4][4], bool has_bias, bool has_res, bool do_relu) {
+#pragma unroll
+        for (int kb = 0; kb < 2; ++kb)
+#pragma unroll
+            for (int g = 0; g < 4; ++g)
+#pragma unroll
+                for (int e = 0; e < 4; ++e) {
+                    float v = yv[kb][g][e];
+                    if (has_bias) v = __fadd_rn(v, bv[kb][g]);
+                    if (has_res) v = __fadd_rn(v, q[kb][g][e]);
+                    if (do_relu) v = relu_sel(v);
+                    yv[kb][g][e] = v;
+                }
+    };
+    const bool has_bias = (a.flags & KXC_HIP_CONV_BIAS) != 0;
+    const bool has_res = (a.flags & KXC_HIP_CONV_RESIDUAL) != 0;
+    const bool do_relu = (a.flags & KXC_HIP_CONV_RELU) != 0;
+    float yv[2][4][4];
+    if (a.gsplit > 1) {
+        // a part of a split reduction stores its raw output transform (the transform is linear)
+        float* const part = a.partial + static_cast<int64_t>(split) * (y_bytes / 4u);
+        output_transform(yv);
+        if constexpr (FUSE) {
+            // ... and the part that arrives last adds all of them in split order and finishes the layer; without
+            // FUSE the adding kernel does.  Parts are stored and re-loaded at device scope (see kDeviceScopeAux).
+            store_all(make_rsrc(part, y_bytes), yv, DeviceScope{});
+            if (!split_arrive_last(a.counters + unit, a.gsplit, reinterpret_cast<uint32_t*>(lds))) return;
+            issue_epilogue_loads(has_bias, has_res, a.y);
+#pragma unroll 2
+            for (int s = 0; s < a.gsplit; ++s) {
+                const __amdgpu_buffer_rsrc_t pr = make_rsrc(a.partial + static_cast<int64_t>(s) * (y_bytes / 4u), y_bytes);
+                float p[2][4][4];
+#pragma unroll
+                for (int kb = 0; kb < 2; ++kb)
+#pragma unroll
+                    for (int g = 0; g < 4; ++g) load4(pr, kb, g, p[kb][g], DeviceScope{});
+#pragma unroll
+                for (int kb = 0; kb < 2; ++kb)
+#pragma unroll
+                    for (int g = 0; g < 4; ++g)
+#pragma unroll
+                        for (int e = 0; e < 4; ++e) yv[kb][g][e] = s == 0 ? p[kb][g][e] : __fadd_rn(yv[kb][g][e], p[kb][g][e]);
             }
+            finish(yv, has_bias, has_res, do_relu);
+            store_all(make_rsrc(a.y, y_bytes), yv, Cached{});
+        } else {
+            store_all(make_rsrc(part, y_bytes), yv, Cached{});
+        }
+        return;
     }
+    issue_epilogue_loads(has_bias, has_res, a.y);
+    output_transform(yv);
+    finish(yv, has_bias, has_res, do_relu);
+    store_all(make_rsrc(a.y, y_bytes), yv, Cached{});
 }
 
 struct WinoVariant {
     const char* name;
     int wk, wt, ks;
     void (*kernel)(const WinoArgs);
+    void (*fuse_kernel)(const WinoArgs);      // the last part finishes a split reduction (nullptr: none)
 };
-#define KXC_WINO(WK, WT) {"winograd_f2k3_o" #WK "_t" #WT, WK, WT, 1, wino_kernel<WK, WT, 1>}
-#define KXC_WINO_KS2(WK, WT) {"winograd_f2k3_o" #WK "_t" #WT "_ks2", WK, WT, 2, wino_kernel<WK, WT, 2>}
+#define KXC_WINO(WK, WT) {"winograd_f2k3_o" #WK "_t" #WT, WK, WT, 1, wino_kernel<WK, WT, 1>, wino_kernel<WK, WT, 1, true>}
+#define KXC_WINO_KS2(WK, WT) {"winograd_f2k3_o" #WK "_t" #WT "_ks2", WK, WT, 2, wino_kernel<WK, WT, 2>, nullptr}
 // name = winograd_f2k3_o<waves along output channels (32 each)>_t<waves along tiles (16 each)>[_ks2: input channels split over two groups of waves]
 const WinoVariant kWino[] = {
     KXC_WINO(2, 2),   // 64 channels x 32 tiles, 4 waves, 48 KiB of LDS (default)
@@ -652,6 +703,7 @@ int32_t kxc_hip_conv2d_winograd_nchw_f32(const kxc_hip_conv2d_desc* desc, const 
     a.gsplit = 1;
     a.steps_per_split = a.csteps;
     SplitScratchLease lease;      // held until the adding kernel is enqueued
+    bool fuse = false;            // the part that arrives last adds the parts: no adding kernel
     const int64_t out_elems = static_cast<int64_t>(a.N) * a.O * a.OHW;
     if (v->ks == 1) {
         int split = GroupSplit(a.num_units, a.csteps, out_elems);
@@ -666,6 +718,8 @@ int32_t kxc_hip_conv2d_winograd_nchw_f32(const kxc_hip_conv2d_desc* desc, const 
             if (a.gsplit > 1) {
                 if (int32_t rc = AcquireSplitScratch(s, static_cast<size_t>(a.gsplit) * out_elems * sizeof(float), &lease)) return rc;
                 a.partial = lease.ptr;
+                a.counters = lease.counters;
+                fuse = v->fuse_kernel && a.gsplit <= SplitFuseMaxParts() && a.num_units <= kSplitCounters;
             } else {
                 a.steps_per_split = a.csteps;
             }
@@ -685,7 +739,7 @@ int32_t kxc_hip_conv2d_winograd_nchw_f32(const kxc_hip_conv2d_desc* desc, const 
         static std::vector<std::pair<int, const void*>> granted;
         int dev = 0;
         KXC_HIP_CALL(hipGetDevice(&dev), "hipGetDevice");
-        const void* fn = reinterpret_cast<const void*>(v->kernel);
+        const void* fn = reinterpret_cast<const void*>(fuse ? v->fuse_kernel : v->kernel);
         std::lock_guard<std::mutex> lock(mu);
         bool have = false;
         for (const auto& g : granted) have = have || (g.first == dev && g.second == fn);
@@ -695,10 +749,10 @@ int32_t kxc_hip_conv2d_winograd_nchw_f32(const kxc_hip_conv2d_desc* desc, const 
             granted.emplace_back(dev, fn);
         }
     }
-    hipLaunchKernelGGL(v->kernel, NoteGrid(dim3(static_cast<unsigned>(a.units_per_xcd * 8))),
+    hipLaunchKernelGGL(fuse ? v->fuse_kernel : v->kernel, NoteGrid(dim3(static_cast<unsigned>(a.units_per_xcd * 8))),
                        NoteBlock(dim3(64 * v->wk * v->wt * v->ks)), NoteLds(lds_bytes), s, a);
     if (int32_t rc = CheckLaunch(v->name)) return rc;
-    if (a.gsplit > 1) {
+    if (a.gsplit > 1 && !fuse) {
         SplitReduceArgs r;
         r.partial = a.partial; r.bias = bias; r.res = residual; r.y = y;
         r.gsplit = a.gsplit; r.total = static_cast<int32_t>(out_elems); r.O = a.O; r.flags = a.flags;

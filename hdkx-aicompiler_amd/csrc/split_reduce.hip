@@ -1,6 +1,7 @@
 // split_reduce.hip -- second half of a convolution whose reduction was split over workgroups, shared by the
 // implicit-GEMM and the Winograd kernel: the partial outputs of the parts are added in split order and the
 // layer's epilogue (bias, residual, ReLU) is applied; plus the scratch buffers the parts write to.
+#include <cstdlib>
 #include <memory>
 #include <mutex>
 #include <vector>
@@ -38,13 +39,28 @@ __global__ void __launch_bounds__(256) conv_split_reduce_kernel(const SplitReduc
     a.y[e] = v;
 }
 
+__global__ void __launch_bounds__(256) split_counters_clear_kernel(uint32_t* counters, int32_t n) {
+    const int32_t i = static_cast<int32_t>(blockIdx.x) * 256 + static_cast<int32_t>(threadIdx.x);
+    if (i < n) counters[i] = 0u;
+}
+
 }  // namespace
+
+// Off by default.  Measured on MI355X, ResNet-18 at batch 1 (13 split Winograd layers, graph replay): the last
+// part's tail is three dependent round trips beyond the XCD's own L2 (stores acknowledged, counter, parts read back)
+// and costs more than the adding kernel with its launch: 0.226 ms per image with the adding kernel everywhere,
+// 0.240 with the four 4-part layers finished by the last part, 0.263 up to 8 parts, 0.309 up to 16, 0.373 up to 32.
+// KXC_HIP_SPLIT_FUSE_MAX=<parts> turns it on for reductions split into at most that many parts.
+int32_t SplitFuseMaxParts() {
+    const char* e = std::getenv("KXC_HIP_SPLIT_FUSE_MAX");
+    return e ? static_cast<int32_t>(std::atoi(e)) : 0;
+}
 
 // A buffer that has been handed out stays allocated until the process ends, also after a larger one replaced it:
 // a captured graph may still hold its address.  Buffers double, so the retired ones add up to less than the
 // current one.
 int32_t AcquireSplitScratch(hipStream_t stream, size_t bytes, SplitScratchLease* lease) {
-    struct Entry { int device; hipStream_t stream; float* ptr; size_t bytes; std::mutex in_use; };
+    struct Entry { int device; hipStream_t stream; float* ptr; uint32_t* counters; size_t bytes; std::mutex in_use; };
     static std::mutex mu;
     static std::vector<std::unique_ptr<Entry>> entries;      // entries are never removed: their addresses are stable
     int dev = 0;
@@ -55,7 +71,7 @@ int32_t AcquireSplitScratch(hipStream_t stream, size_t bytes, SplitScratchLease*
         for (auto& it : entries)
             if (it->device == dev && it->stream == stream) e = it.get();
         if (!e) {
-            entries.emplace_back(new Entry{dev, stream, nullptr, 0, {}});
+            entries.emplace_back(new Entry{dev, stream, nullptr, nullptr, 0, {}});
             e = entries.back().get();
         }
     }
@@ -63,12 +79,18 @@ int32_t AcquireSplitScratch(hipStream_t stream, size_t bytes, SplitScratchLease*
     if (e->bytes < bytes) {
         size_t want = e->bytes ? 2 * e->bytes : (static_cast<size_t>(1) << 20);
         while (want < bytes) want *= 2;
-        float* fresh = nullptr;
-        KXC_HIP_CALL(hipMalloc(reinterpret_cast<void**>(&fresh), want), "hipMalloc(split scratch)");
-        e->ptr = fresh;          // the previous buffer is left allocated on purpose
+        char* fresh = nullptr;
+        KXC_HIP_CALL(hipMalloc(reinterpret_cast<void**>(&fresh), kSplitCounterBytes + want), "hipMalloc(split scratch)");
+        // the arrival counters in front start at zero: a fill kernel on the caller's stream, ahead of the first
+        // launch that counts (under stream capture it becomes a node of the graph, which is harmless)
+        split_counters_clear_kernel<<<kSplitCounters / 256, 256, 0, stream>>>(reinterpret_cast<uint32_t*>(fresh), kSplitCounters);
+        if (int32_t rc = CheckLaunch("split_counters_clear")) { (void)hipFree(fresh); return rc; }
+        e->counters = reinterpret_cast<uint32_t*>(fresh);
+        e->ptr = reinterpret_cast<float*>(fresh + kSplitCounterBytes);          // the previous buffer is left allocated on purpose
         e->bytes = want;
     }
     lease->ptr = e->ptr;
+    lease->counters = e->counters;
     lease->lock = std::move(in_use);
     return KXC_HIP_OK;
 }

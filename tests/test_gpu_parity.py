@@ -362,6 +362,34 @@ def test_conv_winograd_channel_split_over_workgroups(pkg, fast_orc, orc, synth, 
                      orc.conv_chain(xi, wi, bi, 1, 1, None, True), "split on small integers")
 
 
+@pytest.mark.parametrize("shape", [(1, 64, 56, 56, 64), (1, 128, 28, 28, 128), (1, 256, 14, 14, 256), (1, 512, 7, 7, 512), (2, 44, 9, 11, 72)])
+def test_conv_winograd_last_part_finishes_the_reduction(pkg, synth, monkeypatch, shape):
+    """KXC_HIP_SPLIT_FUSE_MAX lets the part that arrives last at its tile's counter add the parts and apply the
+    epilogue instead of the adding kernel (off by default: measured slower).  Same order of additions, so the
+    result equals the adding kernel's bit for bit -- on every one of 30 launches into an output pre-filled with NaN
+    (a tile nobody finished, or one finished before all parts were visible, would show), with the counters left at
+    zero for the next launch."""
+    n, c, h, w, o = shape
+    x = dev(synth.uniform((n, c, h, w), 7500))
+    wt = dev(synth.normal((o, c, 3, 3), 7501, float(np.sqrt(2.0 / (c * 9)))))
+    b = dev(synth.uniform((o,), 7502, -0.1, 0.1))
+    skip = dev(synth.uniform((n, o, h, w), 7503))
+    if n == 2:
+        monkeypatch.setenv("KXC_HIP_WINOGRAD_GSPLIT", "3")
+    u = pkg.conv2d_winograd_transform_weights((n, c, h, w), wt, 1)
+    monkeypatch.setenv("KXC_HIP_SPLIT_FUSE_MAX", "0")
+    want = pkg.conv2d_winograd(x, u, wt.shape, b, skip, 1, True).clone()
+    want_plain = pkg.conv2d_winograd(x, u, wt.shape, None, None, 1, False).clone()
+    monkeypatch.setenv("KXC_HIP_SPLIT_FUSE_MAX", "32")
+    out = torch.empty_like(want)
+    for it in range(30):
+        out.fill_(float("nan"))
+        got = pkg.conv2d_winograd(x, u, wt.shape, b, skip, 1, True, out=out)
+        assert torch.equal(got, want), "launch %d of %s" % (it, shape)
+    out.fill_(float("nan"))
+    assert torch.equal(pkg.conv2d_winograd(x, u, wt.shape, None, None, 1, False, out=out), want_plain)
+
+
 def test_split_reduction_from_two_host_threads(pkg, synth):
     """Two host threads enqueue split convolutions (parts + adding kernel, sharing the stream's scratch buffer) on
     the same stream at the same time: the pair of launches of one call is never interleaved with another call's,
