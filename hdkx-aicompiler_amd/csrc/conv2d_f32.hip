@@ -75,6 +75,12 @@ struct ConvArgs {
     float* y2;
     uint32_t w2_bytes;
     int32_t ds_off;
+    // Stride 2 in both directions (phase != 0): a channel's patch is kept as four phase planes -- (row parity,
+    // column parity) of the padded position, plane (2*rp + cp) at cp_plane*(2*rp + cp), row pitch Wp/2 -- so that
+    // the 32 pixels a half-wave reads for one tap are neighbours in LDS (dense banks) instead of every other float
+    // of every other row.  plane = ceil(rows/2) * Wp/2 floats for the tallest tile of the launch; needs Hp, Wp even.
+    int32_t phase, plane, halfw;
+    FastDiv div_plane, div_halfw;
 };
 
 __device__ __forceinline__ float relu_sel(float v) { return (v > 0.0f) ? v : 0.0f; }
@@ -183,7 +189,7 @@ conv_mfma_kernel(const ConvArgs a) {
         qlast = n2 * a.Hp + fast_div(rem2, a.div_ow) * a.sh + (KH - 1) * a.dh;
     }
     const int P = (qlast - qmin + 1) * a.Wp;      // patch positions per channel (<= chs - 32)
-    const int xsegs = (P + 63) >> 6;              // 64-float segments per channel
+    const int xsegs = ((a.phase ? 4 * a.plane : P) + 63) >> 6;              // 64-float segments per channel
     const int HW = a.H * a.W;
 
     const __amdgpu_buffer_rsrc_t xr = make_rsrc(a.x, a.x_bytes);
@@ -195,10 +201,18 @@ conv_mfma_kernel(const ConvArgs a) {
 #pragma unroll
     for (int i = 0; i < PPT; ++i) {
         const int pos = (wave + i * NW) * 64 + lane;
-        const int q = fast_div(pos, a.div_wp), col = pos - q * a.Wp;
+        int q, col;
+        if (a.phase) {
+            // LDS position -> plane, row and column inside the plane -> padded row and column
+            const int pl = fast_div(pos, a.div_plane), rem = pos - pl * a.plane;
+            const int qr = fast_div(rem, a.div_halfw), qc = rem - qr * a.halfw;
+            q = 2 * qr + (pl >> 1); col = 2 * qc + (pl & 1);
+        } else {
+            q = fast_div(pos, a.div_wp); col = pos - q * a.Wp;
+        }
         const int Q = qmin + q;
         const int n = fast_div(Q, a.div_hp), ih = Q - n * a.Hp - a.ph, iw = col - a.pw;
-        const bool ok = pos < P && n < a.N && ih >= 0 && ih < a.Hv && iw >= 0 && iw < a.W;
+        const bool ok = (a.phase ? (pos < 4 * a.plane && Q <= qlast) : pos < P) && n < a.N && ih >= 0 && ih < a.Hv && iw >= 0 && iw < a.W;
         goff[i] = ok ? static_cast<uint32_t>(((n * a.C) * a.H + ih * a.row_step) * a.W + iw) * 4u : kOobOffset;
     }
     // weight tile element L = plane*PL + row*KS2 + col; col = pair*KHW + tap with channel = 2*pair + plane, or
@@ -242,7 +256,9 @@ conv_mfma_kernel(const ConvArgs a) {
         const int mc = min(m, a.M - 1);
         const int n = fast_div(mc, a.div_ohw), rem = mc - n * a.OHW;
         const int oh = fast_div(rem, a.div_ow), ow = rem - oh * a.OW;
-        xbase[j] = (n * a.Hp + oh * a.sh - qmin) * a.Wp + ow * a.sw + (TPAIR ? 0 : half * a.chs);
+        // (phase planes: the window's first row is an even row of the patch, its first column an even column)
+        xbase[j] = a.phase ? ((n * a.Hp + oh * 2 - qmin) >> 1) * a.halfw + ow + (TPAIR ? 0 : half * a.chs)
+                           : (n * a.Hp + oh * a.sh - qmin) * a.Wp + ow * a.sw + (TPAIR ? 0 : half * a.chs);
         ybase[j] = (m < a.M) ? n * a.O * a.OHW + rem : -1;
     }
     int wbase[RO];
@@ -251,6 +267,15 @@ conv_mfma_kernel(const ConvArgs a) {
     for (int i = 0; i < RO; ++i) {
         wbase[i] = half * PL + ((wave_o * RO + i) * 32 + r) * KS2;
         wbase2[i] = half * PLB + ((wave_o * RO + i) * 32 + r) * KS2B;
+    }
+
+    // offset of filter tap (rh, rw) from the window's first element inside a channel's patch
+    int toff[KHW];
+#pragma unroll
+    for (int t = 0; t < KHW; ++t) {
+        const int rh = t / KW, rw = t % KW;
+        toff[t] = a.phase ? ((rh & 1) * 2 + (rw & 1)) * a.plane + (rh >> 1) * a.halfw + (rw >> 1)
+                          : rh * a.dh * a.Wp + rw * a.dw;
     }
 
     floatx16 acc[RO][RP];
@@ -338,14 +363,12 @@ conv_mfma_kernel(const ConvArgs a) {
                 // lane half h reads tap 2*s + h of channel c; a tap past the end (zero weight) re-reads the last one
                 const int c = step / TPS, s2 = 2 * (step - c * TPS);
                 const int t0 = s2, t1 = s2 + 1 < KHW ? s2 + 1 : KHW - 1;
-                const int off0 = (t0 / KW) * a.dh * a.Wp + (t0 % KW) * a.dw;
-                const int off1 = (t1 / KW) * a.dh * a.Wp + (t1 % KW) * a.dw;
+                const int off0 = toff[t0], off1 = toff[t1];
                 koff_x = c * a.chs + (half ? off1 : off0);
                 koff_w = step;
             } else {
                 const int cp = step / KHW, tap = step - cp * KHW;
-                const int rh = tap / KW, rw = tap - rh * KW;
-                koff_x = (2 * cp) * a.chs + rh * a.dh * a.Wp + rw * a.dw;
+                koff_x = (2 * cp) * a.chs + toff[tap];
                 koff_w = cp * KHW + tap;
             }
 #pragma unroll
@@ -661,10 +684,12 @@ const Variant kVariants[] = {
     KXC_VARIANT_DS(3, 3, 4, 1, 2, 1, 1, 8),   // 32 x 64, 2 waves             (small launches)
     KXC_VARIANT(3, 3, 4, 2, 4, 1, 1, 4),   // 64 x 128, 8 waves
     KXC_VARIANT_DS(3, 3, 4, 2, 8, 1, 1, 2),   // 64 x 256, 16 waves
+    KXC_VARIANT_DS(3, 3, 4, 2, 7, 1, 1, 2),   // 64 x 224, 14 waves
     KXC_VARIANT(3, 3, 4, 1, 4, 2, 1, 4),   // 64 x 128, 4 waves of 64x32
     KXC_VARIANT(3, 3, 4, 1, 4, 2, 2, 4),   // 64 x 256, 4 waves of 64x64
     KXC_VARIANT(3, 3, 8, 1, 8, 1, 1, 2),   // 8-channel chunks
     KXC_VARIANT_KS_DS(3, 3, 4, 1, 4, 1, 1, 4, 2),   // 32 x 128, reduction split 2 ways (8 waves)
+    KXC_VARIANT_KS_DS(3, 3, 4, 1, 7, 1, 1, 4, 2),   // 32 x 224, split 2 ways (14 waves)
     KXC_VARIANT_KS_DS(3, 3, 4, 1, 2, 1, 1, 8, 4),   // 32 x 64, split 4 ways (8 waves)
     KXC_VARIANT_KS_DS(3, 3, 4, 1, 2, 1, 1, 8, 8),   // 32 x 64, split 8 ways (16 waves)
     KXC_VARIANT(1, 1, 8, 1, 4, 2, 1, 4),   // 64 x 128
@@ -692,8 +717,18 @@ constexpr int kNumVariants = sizeof(kVariants) / sizeof(kVariants[0]);
 struct Choice {
     const Variant* v = nullptr;
     int32_t chs = 0;
+    int32_t plane = 0;      // > 0: phase-plane patch layout with planes of this many floats (see ConvArgs)
     size_t lds_bytes = 0;
 };
+
+// Stride 2 both ways, no dilation, even padded extents: the patch is staged as four phase planes.
+// KXC_HIP_CONV_PHASE=0 keeps the row-major patch (for comparison).
+bool UsePhasePlanes(const ConvArgs& a, const Variant& v) {
+    if (a.sh != 2 || a.sw != 2 || a.dh != 1 || a.dw != 1 || (a.Hp & 1) || (a.Wp & 1)) return false;
+    const char* e = std::getenv("KXC_HIP_CONV_PHASE");
+    const int mode = e ? std::atoi(e) : 1;
+    return mode == 2 || (mode == 1 && !v.tpair);
+}
 
 // Largest padded-row span any pixel tile of size tp touches.
 int32_t MaxTileRows(const ConvArgs& a, int kh, int tp) {
@@ -715,14 +750,17 @@ constexpr int kNumCUs = 256;
 bool Fits(const Variant& v, const ConvArgs& a, Choice* out, bool ds = false) {
     if (ds && !v.ds_kernel) return false;
     const int32_t rows = MaxTileRows(a, v.kh, v.tp);
-    const int64_t P = static_cast<int64_t>(rows) * a.Wp;
+    const bool phase = UsePhasePlanes(a, v);
+    const int64_t plane = phase ? static_cast<int64_t>((rows + 1) / 2) * (a.Wp / 2) : 0;
+    const int64_t P = phase ? 4 * plane : static_cast<int64_t>(rows) * a.Wp;
     const int64_t segs = (P + 63) / 64;
     if (segs > static_cast<int64_t>(v.ppt) * v.nw) return false;
     // Channel stride: a multiple of 64 floats plus 32, so the two half-waves (which read channels
     // c and c+1 at the same position) fall into different halves of the LDS banks.
     // With a horizontal stride of 2 the lanes of a half-wave already use every other bank, so the second
     // half-wave is skewed by one more float to land on the odd banks.
-    const int32_t chs = static_cast<int32_t>(segs * 64 + 32) + ((a.sw % 2 == 0 && !v.tpair) ? 1 : 0);
+    // (Phase planes are read densely: no skew.)
+    const int32_t chs = static_cast<int32_t>(segs * 64 + 32) + ((a.sw % 2 == 0 && !v.tpair && !phase) ? 1 : 0);
     const int khw = v.kh * v.kw;
     if (v.tpair && a.C % 2 == 0) return false;     // pairing taps pays when channels cannot be paired evenly
     const int ks2 = (v.tpair ? v.cc * ((khw + 1) / 2) : (v.cc / 2) * khw) | 1;
@@ -738,6 +776,7 @@ bool Fits(const Variant& v, const ConvArgs& a, Choice* out, bool ds = false) {
     if (lds > kMaxLdsBytes) return false;
     out->v = &v;
     out->chs = chs;
+    out->plane = static_cast<int32_t>(plane);
     out->lds_bytes = lds;
     return true;
 }
@@ -808,6 +847,23 @@ void Select(const ConvArgs& a, int kh, int kw, Choice* choice, bool ds = false) 
                     // 28 x 28: 20.5 against 31.5 us) and at stride 1 (batch 1, 256 channels at 14 x 14: 12.6
                     // against 19.8 us with the adding kernel; batch 4, 512 channels at 7 x 7: 23.8 against 37.9)
                     if (kh == 3) break;
+                }
+            }
+            // Every workgroup of a launch does the same work, so the launch takes as long as the compute unit with
+            // the most workgroups: 400 of the 32 x 128 two-group tiles (batch 64, 256 -> 512 channels at 14 x 14,
+            // stride 2) are two on 144 compute units and one on the rest (measured: 256 tiles 77 us, 400 tiles 109,
+            // 512 tiles 116).  The 32 x 224 tile makes 224 workgroups of 14 waves, one per compute unit: 106 us
+            // against 118 in the same process.  Taken when it fills the compute units better.
+            if (kh == 3 && choice->v && std::strcmp(choice->v->name, "mfma_k3x3_c4_o1x1_p4x1_ks2") == 0 && a.M >= 2048) {
+                auto fill = [&](const Variant& v) {
+                    const int64_t wgs = CeilDiv(a.M, v.tp) * CeilDiv(a.O, v.to);
+                    return static_cast<double>(wgs) / static_cast<double>(CeilDiv(wgs, kNumCUs) * kNumCUs);
+                };
+                for (int i = 0; i < kNumVariants; ++i) {
+                    const Variant& v = kVariants[i];
+                    Choice c;
+                    if (std::strcmp(v.name, "mfma_k3x3_c4_o1x1_p7x1_ks2") != 0 || !Fits(v, a, &c, ds)) continue;
+                    if (CeilDiv(a.M, v.tp) * CeilDiv(a.O, v.to) <= kNumCUs && fill(v) > fill(*choice->v) + 0.05) *choice = c;
                 }
             }
         }
@@ -957,10 +1013,16 @@ int32_t Conv2dRun(const kxc_hip_conv2d_desc* desc, const float* x, const float* 
         KXC_HIP_REQUIRE(second->w2 && second->y2, "%s: NULL pointer", who);
         a.w2 = second->w2; a.bias2 = second->bias2; a.y2 = second->y2;
         a.w2_bytes = static_cast<uint32_t>(static_cast<int64_t>(a.O) * a.C * 4);
-        a.ds_off = rh * a.dh * a.Wp + rw * a.dw;
+        a.ds_off = c.plane > 0 ? ((rh & 1) * 2 + (rw & 1)) * c.plane + (rh >> 1) * (a.Wp / 2) + (rw >> 1)
+                               : rh * a.dh * a.Wp + rw * a.dw;
     }
     if (c.v) {
         a.chs = c.chs;
+        a.phase = c.plane > 0 ? 1 : 0;
+        a.plane = c.plane;
+        a.halfw = a.Wp / 2;
+        a.div_plane = MakeFastDiv(a.plane);
+        a.div_halfw = MakeFastDiv(a.halfw);
         a.nchunks = (a.C + c.v->cc - 1) / c.v->cc;
         a.p_tiles = static_cast<int32_t>(CeilDiv(a.M, c.v->tp));
         a.o_tiles = static_cast<int32_t>(CeilDiv(a.O, c.v->to));
