@@ -721,12 +721,16 @@ struct Choice {
     size_t lds_bytes = 0;
 };
 
-// Stride 2 both ways, no dilation, even padded extents: the patch is staged as four phase planes.
-// KXC_HIP_CONV_PHASE=0 keeps the row-major patch (for comparison).
+// Stride 2 both ways, no dilation, even padded extents: the patch can be staged as four phase planes
+// (KXC_HIP_CONV_PHASE=1; 2: also for the tap-pairing 7x7 kernels).  Off by default.  Measured on MI355X, batch 64,
+// the three 3x3/2 + 1x1/2 launches of ResNet-18: SQ_LDS_BANK_CONFLICT drops from 7.5M / 4.5M / 16.1M cycles per
+// launch to 4.0M each, and the launch times do not move (98 / 95 / 108 us; the 56 -> 28 layer gets 3 % slower
+// because its planes round up to one more 64-float segment per channel): LDS bank conflicts are not what limits
+// these kernels -- how evenly the workgroups fill the compute units is (see Select()).
 bool UsePhasePlanes(const ConvArgs& a, const Variant& v) {
     if (a.sh != 2 || a.sw != 2 || a.dh != 1 || a.dw != 1 || (a.Hp & 1) || (a.Wp & 1)) return false;
     const char* e = std::getenv("KXC_HIP_CONV_PHASE");
-    const int mode = e ? std::atoi(e) : 1;
+    const int mode = e ? std::atoi(e) : 0;
     return mode == 2 || (mode == 1 && !v.tpair);
 }
 

@@ -262,6 +262,32 @@ def test_conv_pair_full_batch_properties(pkg, synth):
 
 
 # ------------------------------------------------------------------ Winograd F(2x2,3x3)
+@pytest.mark.parametrize("shape", [(4, 64, 56, 56, 128, 3, 1), (3, 128, 28, 28, 256, 3, 1), (5, 256, 14, 14, 512, 3, 1),
+                                   (2, 3, 64, 64, 64, 7, 3), (2, 8, 13, 17, 32, 3, 1), (2, 6, 12, 18, 40, 5, 2)])
+def test_conv_stride2_phase_plane_layout_is_bit_identical(pkg, synth, monkeypatch, shape):
+    """KXC_HIP_CONV_PHASE stages a stride-2 patch as four (row parity, column parity) planes.  Only where the patch
+    sits in LDS changes, not the order of the products, so every output equals the default layout's bit for bit
+    (the pair kernel's second output included); odd padded extents fall back to the default layout by themselves."""
+    n, c, h, w, o, k, p = shape
+    x = dev(synth.uniform((n, c, h, w), 7700))
+    wt = dev(synth.normal((o, c, k, k), 7701, float(np.sqrt(2.0 / (c * k * k)))))
+    b = dev(synth.uniform((o,), 7702, -0.1, 0.1))
+    w2 = dev(synth.normal((o, c, 1, 1), 7703, float(np.sqrt(2.0 / c))))
+    pair = k == 3 and pkg.conv2d_pair_supported((n, c, h, w), (o, c, k, k), 2, p)
+    def run():
+        outs = [pkg.conv2d(x, wt, b, None, 2, p, 1, True).clone()]
+        if pair:
+            outs += [t.clone() for t in pkg.conv2d_pair(x, wt, b, None, w2, None, 2, p, 1, True)]
+        return outs
+    monkeypatch.setenv("KXC_HIP_CONV_PHASE", "0")
+    want = run()
+    monkeypatch.setenv("KXC_HIP_CONV_PHASE", "2")
+    got = run()
+    assert len(got) == len(want)
+    for g, t in zip(got, want):
+        assert torch.equal(g, t), shape
+
+
 WINOGRAD_SHAPES = [
     (2, 64, 56, 56, 64, 1),       # layer1
     (3, 128, 28, 28, 128, 1),     # layer2
