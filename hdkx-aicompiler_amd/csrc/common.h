@@ -127,6 +127,21 @@ __device__ __forceinline__ bool split_arrive_last(uint32_t* counter, int32_t par
 }
 #endif
 
+// A convolution launch resolved ahead of time (a launch plan's node): kernel, tile shape, grid, the split of the
+// reduction and every environment switch are decided once, from the descriptor; a launch combines them with the
+// operand pointers and the stream.  conv2d_f32.hip (implicit GEMM, one or two outputs) and conv2d_wino_f32.hip.
+struct PreparedConv;
+int32_t PrepareConv2d(const kxc_hip_conv2d_desc* desc, bool second_output, PreparedConv** out);
+int32_t LaunchPreparedConv2d(const PreparedConv* p, const float* x, const float* w, const float* bias, const float* residual,
+                             float* y, const float* w2, const float* bias2, float* y2, hipStream_t stream);
+const char* PreparedConvName(const PreparedConv* p);
+void FreePreparedConv(PreparedConv* p);
+struct PreparedWinograd;
+int32_t PrepareWinograd(const kxc_hip_conv2d_desc* desc, PreparedWinograd** out);
+int32_t LaunchPreparedWinograd(const PreparedWinograd* p, const float* x, const float* u, const float* bias,
+                               const float* residual, float* y, hipStream_t stream);
+void FreePreparedWinograd(PreparedWinograd* p);
+
 // The filter transforms of several Winograd layers in one launch (conv2d_wino_f32.hip).
 struct WinoWeightJob {
     const kxc_hip_conv2d_desc* desc;

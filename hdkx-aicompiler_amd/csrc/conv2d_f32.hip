@@ -30,9 +30,11 @@
 //    cover (output channels not a multiple of 32, very wide rows) and on request.
 #include <cstdlib>
 #include <cstring>
+#include <memory>
 #include <type_traits>
 #include <mutex>
 #include <string>
+#include <utility>
 #include <vector>
 
 #include "common.h"
@@ -962,15 +964,6 @@ int32_t NoAllocScratch(float** out) {
     return KXC_HIP_OK;
 }
 
-// The operator behind both entry points.  no_alloc: the partial sums of a split reduction go to the file-scope
-// scratch array instead of the grow-only per-stream buffer, and a launch that would need more is refused.
-// The second output of kxc_hip_conv2d_pair_nchw_f32 (see ConvArgs).
-struct SecondOutput {
-    const float* w2 = nullptr;
-    const float* bias2 = nullptr;
-    float* y2 = nullptr;
-};
-
 // Whether a convolution can carry the second output: the 1x1 convolution's operand x[n,c,oh*sh,ow*sw] must be a tap
 // of this window, i.e. the padding is a multiple of the dilation and lies inside the filter.
 bool PairTap(const kxc_hip_conv2d_desc* d, int* rh, int* rw) {
@@ -979,123 +972,223 @@ bool PairTap(const kxc_hip_conv2d_desc* d, int* rh, int* rw) {
     return *rh < d->kh && *rw < d->kw;
 }
 
-int32_t Conv2dRun(const kxc_hip_conv2d_desc* desc, const float* x, const float* w, const float* bias,
-                  const float* residual, float* y, void* stream, bool no_alloc, const SecondOutput* second = nullptr) {
-    const char* const who = second ? "kxc_hip_conv2d_pair_nchw_f32" : no_alloc ? "kxc_hip_conv2d_nchw_f32_noalloc" : "kxc_hip_conv2d_nchw_f32";
-    ConvArgs a;
+// Everything about a launch that the descriptor alone decides (kernel, tile shape, grid, the split of the reduction,
+// the switches read from the environment): resolved once per call by the entry points, once per node by a launch
+// plan (kxc_hip::PreparedConv), and combined with the operand pointers and the stream at launch time.
+struct ConvLaunch {
+    enum Path { kEmpty, kSmall1x1, kMfma, kDirect };
+    Path path = kEmpty;
+    ConvArgs a;                     // without operand pointers and partial-sum buffer
+    ConvArgs direct_args;
+    void (*kernel)(const ConvArgs) = nullptr;
+    const char* name = "";
+    dim3 grid, block;
+    size_t lds_bytes = 0;
+    size_t scratch_bytes = 0;       // partial sums of a reduction split over workgroups (0: none)
+    int32_t kh = 0, kw = 0;
+    int64_t total = 0;
+    bool second = false;
+};
+
+int32_t Conv2dResolve(const kxc_hip_conv2d_desc* desc, bool second, const char* who, ConvLaunch* L) {
+    ConvArgs& a = L->a;
     if (int32_t rc = FillArgs(desc, &a, who)) return rc;
-    const int64_t total = static_cast<int64_t>(a.N) * a.O * a.OHW;
-    if (total == 0) return KXC_HIP_OK;
-    KXC_HIP_REQUIRE(x && w && y, "%s: NULL pointer", who);
-    KXC_HIP_REQUIRE(!(desc->flags & KXC_HIP_CONV_BIAS) || bias, "%s: bias flag without bias", who);
-    KXC_HIP_REQUIRE(!(desc->flags & KXC_HIP_CONV_RESIDUAL) || residual, "%s: residual flag without residual", who);
-    a.x = x; a.w = w; a.bias = bias; a.res = residual; a.y = y;
+    L->second = second;
+    L->kh = desc->kh; L->kw = desc->kw;
+    L->total = static_cast<int64_t>(a.N) * a.O * a.OHW;
+    if (L->total == 0) { L->path = ConvLaunch::kEmpty; return KXC_HIP_OK; }
+    const int64_t total = L->total;
     a.x_bytes = static_cast<uint32_t>(static_cast<int64_t>(a.N) * a.C * a.H * a.W * 4);       // < 2 GiB on the MFMA path
     a.w_bytes = static_cast<uint32_t>(static_cast<int64_t>(a.O) * a.C * desc->kh * desc->kw * 4);
-    hipStream_t s = ResolveStream(stream);
 
     // A filter one row high with a vertical stride touches only every stride-th input row (the 1x1/2
     // downsample convolutions): the matrix kernel then sees an image of OH rows that are stride rows apart, so
     // the skipped rows are neither loaded nor staged.
     if (!second && UseSmall1x1(desc, a)) {
         a.div_ohw = MakeFastDiv(a.OHW); a.div_ow = MakeFastDiv(a.OW);
-        const dim3 grid(static_cast<unsigned>(CeilDiv(a.O, 32)), static_cast<unsigned>(CeilDiv(a.M, 32)));
+        L->path = ConvLaunch::kSmall1x1;
+        L->grid = dim3(static_cast<unsigned>(CeilDiv(a.O, 32)), static_cast<unsigned>(CeilDiv(a.M, 32)));
         // eight waves split a long reduction (each keeps an even number of channels)
-        if (a.C >= 256 && a.C % 16 == 0)
-            hipLaunchKernelGGL(conv1x1_small_kernel<8>, NoteGrid(grid), NoteBlock(dim3(512)), NoteLds(0), s, a);
-        else
-            hipLaunchKernelGGL(conv1x1_small_kernel<4>, NoteGrid(grid), NoteBlock(dim3(256)), NoteLds(0), s, a);
-        return CheckLaunch("mfma_k1x1_small");
+        const bool eight = a.C >= 256 && a.C % 16 == 0;
+        L->kernel = eight ? conv1x1_small_kernel<8> : conv1x1_small_kernel<4>;
+        L->block = dim3(eight ? 512 : 256);
+        L->name = "mfma_k1x1_small";
+        return KXC_HIP_OK;
     }
-    ConvArgs direct_args = a;
+    L->direct_args = a;
     ApplyRowView(&a, desc->kh);
     Choice c;
-    if (!(desc->flags & KXC_HIP_CONV_FORCE_DIRECT) && a.M > 0) Select(a, desc->kh, desc->kw, &c, second != nullptr);
+    if (!(desc->flags & KXC_HIP_CONV_FORCE_DIRECT) && a.M > 0) Select(a, desc->kh, desc->kw, &c, second);
     if (second) {
         int rh = 0, rw = 0;
         KXC_HIP_REQUIRE(c.v && c.v->ds_kernel && PairTap(desc, &rh, &rw), "%s: no kernel with a second output covers this shape", who);
-        KXC_HIP_REQUIRE(second->w2 && second->y2, "%s: NULL pointer", who);
-        a.w2 = second->w2; a.bias2 = second->bias2; a.y2 = second->y2;
         a.w2_bytes = static_cast<uint32_t>(static_cast<int64_t>(a.O) * a.C * 4);
         a.ds_off = c.plane > 0 ? ((rh & 1) * 2 + (rw & 1)) * c.plane + (rh >> 1) * (a.Wp / 2) + (rw >> 1)
                                : rh * a.dh * a.Wp + rw * a.dw;
     }
-    if (c.v) {
-        a.chs = c.chs;
-        a.phase = c.plane > 0 ? 1 : 0;
-        a.plane = c.plane;
-        a.halfw = a.Wp / 2;
-        a.div_plane = MakeFastDiv(a.plane);
-        a.div_halfw = MakeFastDiv(a.halfw);
-        a.nchunks = (a.C + c.v->cc - 1) / c.v->cc;
-        a.p_tiles = static_cast<int32_t>(CeilDiv(a.M, c.v->tp));
-        a.o_tiles = static_cast<int32_t>(CeilDiv(a.O, c.v->to));
-        const int64_t tiles = static_cast<int64_t>(a.p_tiles) * a.o_tiles;
-        KXC_HIP_REQUIRE(tiles < (1LL << 30), "%s: too many tiles", who);
-        a.num_tiles = static_cast<int32_t>(tiles);
-        // Launches that still leave most SIMDs idle (batch 1, deep layers: a handful of tiles, a long reduction)
-        // split the reduction over workgroups as well; every workgroup keeps at least two chunks per wave group.
-        a.gsplit = 1;
-        a.cps = a.nchunks;
-        a.out_elems = total;
-        SplitScratchLease lease;      // held until the adding kernel is enqueued
-        {
-            int split = 1;
-            if (!second) SplitOverWorkgroups(c, a.nchunks, tiles, total, &split);      // (a second output is never split)
-            if (split > 1) {
-                a.cps = static_cast<int32_t>(CeilDiv(a.nchunks, split));
-                a.gsplit = static_cast<int32_t>(CeilDiv(a.nchunks, a.cps));      // no empty split
-                if (a.gsplit > 1) {
-                    const size_t need = static_cast<size_t>(a.gsplit) * total * sizeof(float);
-                    if (no_alloc) {
-                        // every kernel of the pair overwrites what it reads later, nothing has to start at zero
-                        KXC_HIP_REQUIRE(need <= kNoAllocScratchBytes,
-                                        "%s: the split reduction needs %zu bytes of scratch, the built-in array holds %zu",
-                                        who, need, kNoAllocScratchBytes);
-                        if (int32_t rc = NoAllocScratch(&a.partial)) return rc;
-                    } else {
-                        if (int32_t rc = AcquireSplitScratch(s, need, &lease)) return rc;
-                        a.partial = lease.ptr;
-                    }
-                } else {
-                    a.cps = a.nchunks;
-                }
-            }
-        }
-        a.div_gsplit = MakeFastDiv(a.gsplit);
-        a.tiles_per_xcd = static_cast<int32_t>(CeilDiv(tiles * a.gsplit, 8));
-        a.div_wp = MakeFastDiv(a.Wp); a.div_hp = MakeFastDiv(a.Hp); a.div_ohw = MakeFastDiv(a.OHW);
-        a.div_ow = MakeFastDiv(a.OW); a.div_otiles = MakeFastDiv(a.o_tiles); a.div_ptiles = MakeFastDiv(a.p_tiles);
-        // weights of one output-channel tile: to * C * kh * kw * 4 bytes; keep the larger operand resident
-        const int64_t w_tile_bytes = static_cast<int64_t>(c.v->to) * a.C * desc->kh * desc->kw * 4;
-        a.o_fastest = w_tile_bytes * a.o_tiles <= (2 << 20) ? 1 : 0;
-        if (const char* e = std::getenv("KXC_HIP_CONV_OFAST")) a.o_fastest = std::atoi(e);
-        dim3 grid(static_cast<unsigned>(a.tiles_per_xcd * 8));
-        if (c.lds_bytes > 64 * 1024) {
-            // above the default 64 KiB the dynamic LDS size has to be granted per kernel
-            KXC_HIP_CALL(hipFuncSetAttribute(reinterpret_cast<const void*>(second ? c.v->ds_kernel : c.v->kernel),
-                                             hipFuncAttributeMaxDynamicSharedMemorySize,
-                                             static_cast<int>(c.lds_bytes)),
-                         "hipFuncSetAttribute(MaxDynamicSharedMemorySize)");
-        }
-        void (*const kernel)(const ConvArgs) = second ? c.v->ds_kernel : c.v->kernel;
-        hipLaunchKernelGGL(kernel, NoteGrid(grid), NoteBlock(dim3(64 * c.v->nw * c.v->ks)), NoteLds(c.lds_bytes), s, a);
-        if (int32_t rc = CheckLaunch(c.v->name)) return rc;
-        if (a.gsplit > 1) {
-            SplitReduceArgs r;
-            r.partial = a.partial; r.bias = a.bias; r.res = a.res; r.y = a.y;
-            r.gsplit = a.gsplit; r.total = static_cast<int32_t>(total); r.O = a.O; r.flags = a.flags; r.div_ohw = a.div_ohw;
-            return LaunchSplitReduce(s, r);
-        }
+    if (!c.v) {
+        int64_t g = CeilDiv(total, 256);
+        if (g > 256 * 64) g = 256 * 64;
+        L->path = ConvLaunch::kDirect;
+        L->grid = dim3(static_cast<unsigned>(g));
+        L->block = dim3(256);
+        L->name = "conv_direct";
         return KXC_HIP_OK;
     }
-    int64_t g = CeilDiv(total, 256);
-    if (g > 256 * 64) g = 256 * 64;
-    conv_direct_kernel<<<NoteGrid(static_cast<int>(g)), NoteBlock(256), NoteLds(0), s>>>(direct_args, desc->kh, desc->kw, total);
-    return CheckLaunch("conv_direct");
+    a.chs = c.chs;
+    a.phase = c.plane > 0 ? 1 : 0;
+    a.plane = c.plane;
+    a.halfw = a.Wp / 2;
+    a.div_plane = MakeFastDiv(a.plane);
+    a.div_halfw = MakeFastDiv(a.halfw);
+    a.nchunks = (a.C + c.v->cc - 1) / c.v->cc;
+    a.p_tiles = static_cast<int32_t>(CeilDiv(a.M, c.v->tp));
+    a.o_tiles = static_cast<int32_t>(CeilDiv(a.O, c.v->to));
+    const int64_t tiles = static_cast<int64_t>(a.p_tiles) * a.o_tiles;
+    KXC_HIP_REQUIRE(tiles < (1LL << 30), "%s: too many tiles", who);
+    a.num_tiles = static_cast<int32_t>(tiles);
+    // Launches that still leave most SIMDs idle (batch 1, deep layers: a handful of tiles, a long reduction)
+    // split the reduction over workgroups as well; every workgroup keeps at least two chunks per wave group.
+    a.gsplit = 1;
+    a.cps = a.nchunks;
+    a.out_elems = total;
+    int split = 1;
+    if (!second) SplitOverWorkgroups(c, a.nchunks, tiles, total, &split);      // (a second output is never split)
+    if (split > 1) {
+        a.cps = static_cast<int32_t>(CeilDiv(a.nchunks, split));
+        a.gsplit = static_cast<int32_t>(CeilDiv(a.nchunks, a.cps));      // no empty split
+        if (a.gsplit > 1) L->scratch_bytes = static_cast<size_t>(a.gsplit) * total * sizeof(float);
+        else a.cps = a.nchunks;
+    }
+    a.div_gsplit = MakeFastDiv(a.gsplit);
+    a.tiles_per_xcd = static_cast<int32_t>(CeilDiv(tiles * a.gsplit, 8));
+    a.div_wp = MakeFastDiv(a.Wp); a.div_hp = MakeFastDiv(a.Hp); a.div_ohw = MakeFastDiv(a.OHW);
+    a.div_ow = MakeFastDiv(a.OW); a.div_otiles = MakeFastDiv(a.o_tiles); a.div_ptiles = MakeFastDiv(a.p_tiles);
+    // weights of one output-channel tile: to * C * kh * kw * 4 bytes; keep the larger operand resident
+    const int64_t w_tile_bytes = static_cast<int64_t>(c.v->to) * a.C * desc->kh * desc->kw * 4;
+    a.o_fastest = w_tile_bytes * a.o_tiles <= (2 << 20) ? 1 : 0;
+    if (const char* e = std::getenv("KXC_HIP_CONV_OFAST")) a.o_fastest = std::atoi(e);
+    L->path = ConvLaunch::kMfma;
+    L->kernel = second ? c.v->ds_kernel : c.v->kernel;
+    L->name = c.v->name;
+    L->grid = dim3(static_cast<unsigned>(a.tiles_per_xcd * 8));
+    L->block = dim3(64 * c.v->nw * c.v->ks);
+    L->lds_bytes = c.lds_bytes;
+    return KXC_HIP_OK;
+}
+
+// Above the default 64 KiB the dynamic LDS size has to be granted per kernel and device (once).
+int32_t GrantLds(void (*kernel)(const ConvArgs), size_t lds_bytes) {
+    static std::mutex mu;
+    static std::vector<std::pair<int, const void*>> granted;
+    int dev = 0;
+    KXC_HIP_CALL(hipGetDevice(&dev), "hipGetDevice");
+    const void* fn = reinterpret_cast<const void*>(kernel);
+    std::lock_guard<std::mutex> lock(mu);
+    for (const auto& g : granted)
+        if (g.first == dev && g.second == fn) return KXC_HIP_OK;
+    KXC_HIP_CALL(hipFuncSetAttribute(fn, hipFuncAttributeMaxDynamicSharedMemorySize, static_cast<int>(kMaxLdsBytes)),
+                 "hipFuncSetAttribute(MaxDynamicSharedMemorySize)");
+    granted.emplace_back(dev, fn);
+    return KXC_HIP_OK;
+}
+
+// The second output of kxc_hip_conv2d_pair_nchw_f32 (see ConvArgs).
+struct SecondOutput {
+    const float* w2 = nullptr;
+    const float* bias2 = nullptr;
+    float* y2 = nullptr;
+};
+
+// no_alloc: the partial sums of a split reduction go to the file-scope scratch array instead of the grow-only
+// per-stream buffer, and a launch that would need more is refused.
+int32_t Conv2dLaunch(const ConvLaunch& L, const char* who, const float* x, const float* w, const float* bias,
+                     const float* residual, float* y, void* stream, bool no_alloc, const SecondOutput* second) {
+    if (L.path == ConvLaunch::kEmpty) return KXC_HIP_OK;
+    KXC_HIP_REQUIRE(x && w && y, "%s: NULL pointer", who);
+    KXC_HIP_REQUIRE(!(L.a.flags & KXC_HIP_CONV_BIAS) || bias, "%s: bias flag without bias", who);
+    KXC_HIP_REQUIRE(!(L.a.flags & KXC_HIP_CONV_RESIDUAL) || residual, "%s: residual flag without residual", who);
+    KXC_HIP_REQUIRE(L.second == (second != nullptr), "%s: launch resolved for a different number of outputs", who);
+    hipStream_t s = ResolveStream(stream);
+    if (L.path == ConvLaunch::kDirect) {
+        ConvArgs d = L.direct_args;
+        d.x = x; d.w = w; d.bias = bias; d.res = residual; d.y = y;
+        conv_direct_kernel<<<NoteGrid(L.grid), NoteBlock(L.block), NoteLds(0), s>>>(d, L.kh, L.kw, L.total);
+        return CheckLaunch("conv_direct");
+    }
+    ConvArgs a = L.a;
+    a.x = x; a.w = w; a.bias = bias; a.res = residual; a.y = y;
+    if (L.path == ConvLaunch::kSmall1x1) {
+        hipLaunchKernelGGL(L.kernel, NoteGrid(L.grid), NoteBlock(L.block), NoteLds(0), s, a);
+        return CheckLaunch(L.name);
+    }
+    if (second) {
+        KXC_HIP_REQUIRE(second->w2 && second->y2, "%s: NULL pointer", who);
+        a.w2 = second->w2; a.bias2 = second->bias2; a.y2 = second->y2;
+    }
+    SplitScratchLease lease;      // held until the adding kernel is enqueued
+    if (L.scratch_bytes > 0) {
+        if (no_alloc) {
+            // every kernel of the pair overwrites what it reads later, nothing has to start at zero
+            KXC_HIP_REQUIRE(L.scratch_bytes <= kNoAllocScratchBytes,
+                            "%s: the split reduction needs %zu bytes of scratch, the built-in array holds %zu",
+                            who, L.scratch_bytes, kNoAllocScratchBytes);
+            if (int32_t rc = NoAllocScratch(&a.partial)) return rc;
+        } else {
+            if (int32_t rc = AcquireSplitScratch(s, L.scratch_bytes, &lease)) return rc;
+            a.partial = lease.ptr;
+        }
+    }
+    if (L.lds_bytes > 64 * 1024)
+        if (int32_t rc = GrantLds(L.kernel, L.lds_bytes)) return rc;
+    hipLaunchKernelGGL(L.kernel, NoteGrid(L.grid), NoteBlock(L.block), NoteLds(L.lds_bytes), s, a);
+    if (int32_t rc = CheckLaunch(L.name)) return rc;
+    if (a.gsplit > 1) {
+        SplitReduceArgs r;
+        r.partial = a.partial; r.bias = a.bias; r.res = a.res; r.y = a.y;
+        r.gsplit = a.gsplit; r.total = static_cast<int32_t>(L.total); r.O = a.O; r.flags = a.flags; r.div_ohw = a.div_ohw;
+        return LaunchSplitReduce(s, r);
+    }
+    return KXC_HIP_OK;
+}
+
+int32_t Conv2dRun(const kxc_hip_conv2d_desc* desc, const float* x, const float* w, const float* bias,
+                  const float* residual, float* y, void* stream, bool no_alloc, const SecondOutput* second = nullptr) {
+    const char* const who = second ? "kxc_hip_conv2d_pair_nchw_f32" : no_alloc ? "kxc_hip_conv2d_nchw_f32_noalloc" : "kxc_hip_conv2d_nchw_f32";
+    ConvLaunch L;
+    if (int32_t rc = Conv2dResolve(desc, second != nullptr, who, &L)) return rc;
+    return Conv2dLaunch(L, who, x, w, bias, residual, y, stream, no_alloc, second);
 }
 
 }  // namespace
+
+namespace kxc_hip {
+
+struct PreparedConv {
+    ConvLaunch launch;
+    std::string who;
+};
+
+int32_t PrepareConv2d(const kxc_hip_conv2d_desc* desc, bool second_output, PreparedConv** out) {
+    std::unique_ptr<PreparedConv> p(new PreparedConv);
+    p->who = second_output ? "kxc_hip_conv2d_pair_nchw_f32 (plan node)" : "kxc_hip_conv2d_nchw_f32 (plan node)";
+    if (int32_t rc = Conv2dResolve(desc, second_output, p->who.c_str(), &p->launch)) return rc;
+    *out = p.release();
+    return KXC_HIP_OK;
+}
+
+int32_t LaunchPreparedConv2d(const PreparedConv* p, const float* x, const float* w, const float* bias, const float* residual,
+                             float* y, const float* w2, const float* bias2, float* y2, hipStream_t stream) {
+    SecondOutput second;
+    second.w2 = w2; second.bias2 = bias2; second.y2 = y2;
+    return Conv2dLaunch(p->launch, p->who.c_str(), x, w, bias, residual, y, stream, false, p->launch.second ? &second : nullptr);
+}
+
+const char* PreparedConvName(const PreparedConv* p) { return p->launch.name; }
+
+void FreePreparedConv(PreparedConv* p) { delete p; }
+
+}  // namespace kxc_hip
 
 extern "C" {
 

@@ -627,9 +627,140 @@ const WinoVariant* SelectWino(const kxc_hip_conv2d_desc* d) {
     return &kWino[0];
 }
 
+// What the descriptor alone decides about a launch (variant, grid, the split over workgroups, the switches read
+// from the environment): resolved once per call by the entry point, once per node by a launch plan.
+struct WinoLaunch {
+    const WinoVariant* v = nullptr;
+    WinoArgs a;                 // without operand pointers, partial outputs and counters
+    int64_t out_elems = 0;
+    size_t scratch_bytes = 0;   // partial outputs of a split over workgroups (0: none)
+    size_t lds_bytes = 0;
+    bool fuse = false;          // the part that arrives last adds the parts: no adding kernel
+};
+
+int32_t WinoResolve(const kxc_hip_conv2d_desc* desc, WinoLaunch* L) {
+    KXC_HIP_REQUIRE(desc && Supported(desc), "kxc_hip_conv2d_winograd_nchw_f32: unsupported shape");
+    const WinoVariant* v = SelectWino(desc);
+    L->v = v;
+    WinoArgs& a = L->a;
+    std::memset(&a, 0, sizeof(a));
+    a.N = static_cast<int32_t>(desc->n); a.C = static_cast<int32_t>(desc->c); a.H = static_cast<int32_t>(desc->h);
+    a.W = static_cast<int32_t>(desc->w); a.O = static_cast<int32_t>(desc->o);
+    a.ph = static_cast<int32_t>(desc->pad_h); a.pw = static_cast<int32_t>(desc->pad_w);
+    a.OH = a.H + 2 * a.ph - 2; a.OW = a.W + 2 * a.pw - 2;
+    a.TW = (a.OW + 1) / 2;
+    a.TI = ((a.OH + 1) / 2) * a.TW;
+    a.NT = a.N * a.TI;
+    a.HW = a.H * a.W; a.OHW = a.OH * a.OW;
+    a.csteps = a.C / 4;
+    a.x_bytes = static_cast<uint32_t>(static_cast<int64_t>(a.N) * a.C * a.HW * 4);
+    a.u_bytes = static_cast<uint32_t>(CeilDiv(a.O, 32) * 32 * static_cast<int64_t>(a.C) * 64);
+    a.flags = desc->flags;
+    a.t_groups = static_cast<int32_t>(CeilDiv(a.NT, 16 * v->wt));
+    a.k_groups = static_cast<int32_t>(CeilDiv(a.O, 32 * v->wk));
+    a.num_units = a.t_groups * a.k_groups;
+    // Small launches split the input channels over workgroups (GroupSplit): each part writes its raw output
+    // transform (the transform is linear) to a scratch buffer, and a second kernel adds the parts in order and
+    // applies the epilogue.
+    a.gsplit = 1;
+    a.steps_per_split = a.csteps;
+    const int64_t out_elems = static_cast<int64_t>(a.N) * a.O * a.OHW;
+    L->out_elems = out_elems;
+    if (v->ks == 1) {
+        int split = GroupSplit(a.num_units, a.csteps, out_elems);
+        if (const char* e = std::getenv("KXC_HIP_WINOGRAD_GSPLIT")) {
+            // (a forced split is honoured while its partial outputs stay below 256 MiB)
+            const int f = std::atoi(e);
+            if (f >= 1 && f <= a.csteps && out_elems * static_cast<int64_t>(sizeof(float)) * f <= (256LL << 20)) split = f;
+        }
+        if (split > 1) {
+            a.steps_per_split = static_cast<int32_t>(CeilDiv(a.csteps, split));
+            a.gsplit = static_cast<int32_t>(CeilDiv(a.csteps, a.steps_per_split));      // no empty part
+            if (a.gsplit > 1) {
+                L->scratch_bytes = static_cast<size_t>(a.gsplit) * out_elems * sizeof(float);
+                L->fuse = v->fuse_kernel && a.gsplit <= SplitFuseMaxParts() && a.num_units <= kSplitCounters;
+            } else {
+                a.steps_per_split = a.csteps;
+            }
+        }
+    }
+    a.div_gsplit = MakeFastDiv(a.gsplit);
+    a.units_per_xcd = static_cast<int32_t>(CeilDiv(static_cast<int64_t>(a.num_units) * a.gsplit, 8));
+    // transformed weights of all output channels small next to an L2: neighbouring units share the input tile
+    a.k_fastest = a.u_bytes <= (2u << 20) ? 1 : 0;
+    if (const char* e = std::getenv("KXC_HIP_WINOGRAD_KFAST")) a.k_fastest = std::atoi(e);
+    a.div_ti = MakeFastDiv(a.TI); a.div_tw = MakeFastDiv(a.TW);
+    a.div_kgroups = MakeFastDiv(a.k_groups); a.div_tgroups = MakeFastDiv(a.t_groups);
+    L->lds_bytes = v->ks * 2 * static_cast<size_t>(2048 * v->wk + 1024 * v->wt) * sizeof(float);
+    return KXC_HIP_OK;
+}
+
+int32_t WinoRun(const WinoLaunch& L, const float* x, const float* u, const float* bias, const float* residual, float* y,
+                hipStream_t s) {
+    const WinoVariant* v = L.v;
+    KXC_HIP_REQUIRE(x && u && y, "kxc_hip_conv2d_winograd_nchw_f32: NULL pointer");
+    KXC_HIP_REQUIRE(!(L.a.flags & KXC_HIP_CONV_BIAS) || bias, "kxc_hip_conv2d_winograd_nchw_f32: bias flag without bias");
+    KXC_HIP_REQUIRE(!(L.a.flags & KXC_HIP_CONV_RESIDUAL) || residual,
+                    "kxc_hip_conv2d_winograd_nchw_f32: residual flag without residual");
+    WinoArgs a = L.a;
+    a.x = x; a.u = u; a.bias = bias; a.res = residual; a.y = y;
+    SplitScratchLease lease;      // held until the adding kernel is enqueued
+    if (L.scratch_bytes > 0) {
+        if (int32_t rc = AcquireSplitScratch(s, L.scratch_bytes, &lease)) return rc;
+        a.partial = lease.ptr;
+        a.counters = lease.counters;
+    }
+    void (*const kernel)(const WinoArgs) = L.fuse ? v->fuse_kernel : v->kernel;
+    if (L.lds_bytes > 64 * 1024) {
+        // above the default 64 KiB the dynamic LDS size has to be granted per kernel and device (once)
+        static std::mutex mu;
+        static std::vector<std::pair<int, const void*>> granted;
+        int dev = 0;
+        KXC_HIP_CALL(hipGetDevice(&dev), "hipGetDevice");
+        const void* fn = reinterpret_cast<const void*>(kernel);
+        std::lock_guard<std::mutex> lock(mu);
+        bool have = false;
+        for (const auto& g : granted) have = have || (g.first == dev && g.second == fn);
+        if (!have) {
+            KXC_HIP_CALL(hipFuncSetAttribute(fn, hipFuncAttributeMaxDynamicSharedMemorySize, static_cast<int>(L.lds_bytes)),
+                         "hipFuncSetAttribute(MaxDynamicSharedMemorySize)");
+            granted.emplace_back(dev, fn);
+        }
+    }
+    hipLaunchKernelGGL(kernel, NoteGrid(dim3(static_cast<unsigned>(a.units_per_xcd * 8))),
+                       NoteBlock(dim3(64 * v->wk * v->wt * v->ks)), NoteLds(L.lds_bytes), s, a);
+    if (int32_t rc = CheckLaunch(v->name)) return rc;
+    if (a.gsplit > 1 && !L.fuse) {
+        SplitReduceArgs r;
+        r.partial = a.partial; r.bias = bias; r.res = residual; r.y = y;
+        r.gsplit = a.gsplit; r.total = static_cast<int32_t>(L.out_elems); r.O = a.O; r.flags = a.flags;
+        r.div_ohw = MakeFastDiv(a.OHW);
+        return LaunchSplitReduce(s, r);
+    }
+    return KXC_HIP_OK;
+}
+
 }  // namespace
 
 namespace kxc_hip {
+
+struct PreparedWinograd {
+    WinoLaunch launch;
+};
+
+int32_t PrepareWinograd(const kxc_hip_conv2d_desc* desc, PreparedWinograd** out) {
+    PreparedWinograd* p = new PreparedWinograd;
+    if (int32_t rc = WinoResolve(desc, &p->launch)) { delete p; return rc; }
+    *out = p;
+    return KXC_HIP_OK;
+}
+
+int32_t LaunchPreparedWinograd(const PreparedWinograd* p, const float* x, const float* u, const float* bias,
+                               const float* residual, float* y, hipStream_t stream) {
+    return WinoRun(p->launch, x, u, bias, residual, y, stream);
+}
+
+void FreePreparedWinograd(PreparedWinograd* p) { delete p; }
 
 int32_t LaunchWinogradWeightTransforms(const WinoWeightJob* jobs, int32_t count, hipStream_t stream) {
     for (int32_t base = 0; base < count; base += kMaxWeightJobs) {
@@ -692,94 +823,9 @@ int32_t kxc_hip_conv2d_winograd_transform_weights(const kxc_hip_conv2d_desc* des
 
 int32_t kxc_hip_conv2d_winograd_nchw_f32(const kxc_hip_conv2d_desc* desc, const float* x, const float* u, const float* bias,
                                          const float* residual, float* y, void* stream) {
-    KXC_HIP_REQUIRE(desc && Supported(desc), "kxc_hip_conv2d_winograd_nchw_f32: unsupported shape");
-    KXC_HIP_REQUIRE(x && u && y, "kxc_hip_conv2d_winograd_nchw_f32: NULL pointer");
-    KXC_HIP_REQUIRE(!(desc->flags & KXC_HIP_CONV_BIAS) || bias, "kxc_hip_conv2d_winograd_nchw_f32: bias flag without bias");
-    KXC_HIP_REQUIRE(!(desc->flags & KXC_HIP_CONV_RESIDUAL) || residual,
-                    "kxc_hip_conv2d_winograd_nchw_f32: residual flag without residual");
-    const WinoVariant* v = SelectWino(desc);
-    hipStream_t s = ResolveStream(stream);
-    WinoArgs a;
-    std::memset(&a, 0, sizeof(a));
-    a.x = x; a.u = u; a.bias = bias; a.res = residual; a.y = y;
-    a.N = static_cast<int32_t>(desc->n); a.C = static_cast<int32_t>(desc->c); a.H = static_cast<int32_t>(desc->h);
-    a.W = static_cast<int32_t>(desc->w); a.O = static_cast<int32_t>(desc->o);
-    a.ph = static_cast<int32_t>(desc->pad_h); a.pw = static_cast<int32_t>(desc->pad_w);
-    a.OH = a.H + 2 * a.ph - 2; a.OW = a.W + 2 * a.pw - 2;
-    a.TW = (a.OW + 1) / 2;
-    a.TI = ((a.OH + 1) / 2) * a.TW;
-    a.NT = a.N * a.TI;
-    a.HW = a.H * a.W; a.OHW = a.OH * a.OW;
-    a.csteps = a.C / 4;
-    a.x_bytes = static_cast<uint32_t>(static_cast<int64_t>(a.N) * a.C * a.HW * 4);
-    a.u_bytes = static_cast<uint32_t>(CeilDiv(a.O, 32) * 32 * static_cast<int64_t>(a.C) * 64);
-    a.flags = desc->flags;
-    a.t_groups = static_cast<int32_t>(CeilDiv(a.NT, 16 * v->wt));
-    a.k_groups = static_cast<int32_t>(CeilDiv(a.O, 32 * v->wk));
-    a.num_units = a.t_groups * a.k_groups;
-    // Small launches split the input channels over workgroups (GroupSplit): each part writes its raw output
-    // transform (the transform is linear) to a scratch buffer, and a second kernel adds the parts in order and
-    // applies the epilogue.
-    a.gsplit = 1;
-    a.steps_per_split = a.csteps;
-    SplitScratchLease lease;      // held until the adding kernel is enqueued
-    bool fuse = false;            // the part that arrives last adds the parts: no adding kernel
-    const int64_t out_elems = static_cast<int64_t>(a.N) * a.O * a.OHW;
-    if (v->ks == 1) {
-        int split = GroupSplit(a.num_units, a.csteps, out_elems);
-        if (const char* e = std::getenv("KXC_HIP_WINOGRAD_GSPLIT")) {
-            // (a forced split is honoured while its partial outputs stay below 256 MiB)
-            const int f = std::atoi(e);
-            if (f >= 1 && f <= a.csteps && out_elems * static_cast<int64_t>(sizeof(float)) * f <= (256LL << 20)) split = f;
-        }
-        if (split > 1) {
-            a.steps_per_split = static_cast<int32_t>(CeilDiv(a.csteps, split));
-            a.gsplit = static_cast<int32_t>(CeilDiv(a.csteps, a.steps_per_split));      // no empty part
-            if (a.gsplit > 1) {
-                if (int32_t rc = AcquireSplitScratch(s, static_cast<size_t>(a.gsplit) * out_elems * sizeof(float), &lease)) return rc;
-                a.partial = lease.ptr;
-                a.counters = lease.counters;
-                fuse = v->fuse_kernel && a.gsplit <= SplitFuseMaxParts() && a.num_units <= kSplitCounters;
-            } else {
-                a.steps_per_split = a.csteps;
-            }
-        }
-    }
-    a.div_gsplit = MakeFastDiv(a.gsplit);
-    a.units_per_xcd = static_cast<int32_t>(CeilDiv(static_cast<int64_t>(a.num_units) * a.gsplit, 8));
-    // transformed weights of all output channels small next to an L2: neighbouring units share the input tile
-    a.k_fastest = a.u_bytes <= (2u << 20) ? 1 : 0;
-    if (const char* e = std::getenv("KXC_HIP_WINOGRAD_KFAST")) a.k_fastest = std::atoi(e);
-    a.div_ti = MakeFastDiv(a.TI); a.div_tw = MakeFastDiv(a.TW);
-    a.div_kgroups = MakeFastDiv(a.k_groups); a.div_tgroups = MakeFastDiv(a.t_groups);
-    const size_t lds_bytes = v->ks * 2 * static_cast<size_t>(2048 * v->wk + 1024 * v->wt) * sizeof(float);
-    if (lds_bytes > 64 * 1024) {
-        // above the default 64 KiB the dynamic LDS size has to be granted per kernel and device (once)
-        static std::mutex mu;
-        static std::vector<std::pair<int, const void*>> granted;
-        int dev = 0;
-        KXC_HIP_CALL(hipGetDevice(&dev), "hipGetDevice");
-        const void* fn = reinterpret_cast<const void*>(fuse ? v->fuse_kernel : v->kernel);
-        std::lock_guard<std::mutex> lock(mu);
-        bool have = false;
-        for (const auto& g : granted) have = have || (g.first == dev && g.second == fn);
-        if (!have) {
-            KXC_HIP_CALL(hipFuncSetAttribute(fn, hipFuncAttributeMaxDynamicSharedMemorySize, static_cast<int>(lds_bytes)),
-                         "hipFuncSetAttribute(MaxDynamicSharedMemorySize)");
-            granted.emplace_back(dev, fn);
-        }
-    }
-    hipLaunchKernelGGL(fuse ? v->fuse_kernel : v->kernel, NoteGrid(dim3(static_cast<unsigned>(a.units_per_xcd * 8))),
-                       NoteBlock(dim3(64 * v->wk * v->wt * v->ks)), NoteLds(lds_bytes), s, a);
-    if (int32_t rc = CheckLaunch(v->name)) return rc;
-    if (a.gsplit > 1 && !fuse) {
-        SplitReduceArgs r;
-        r.partial = a.partial; r.bias = bias; r.res = residual; r.y = y;
-        r.gsplit = a.gsplit; r.total = static_cast<int32_t>(out_elems); r.O = a.O; r.flags = a.flags;
-        r.div_ohw = MakeFastDiv(a.OHW);
-        return LaunchSplitReduce(s, r);
-    }
-    return KXC_HIP_OK;
+    WinoLaunch L;
+    if (int32_t rc = WinoResolve(desc, &L)) return rc;
+    return WinoRun(L, x, u, bias, residual, y, ResolveStream(stream));
 }
 
 }  // extern "C"

@@ -9,6 +9,8 @@
 #include <cstring>
 #include <sstream>
 #include <string>
+#include <memory>
+#include <utility>
 #include <vector>
 
 #include "common.h"
@@ -39,11 +41,86 @@ struct Node {
     hipEvent_t fork_event = nullptr, done_event = nullptr;
     // Winograd convolution (i32[0] == 1 on a kConv2D node): the weight pointer whose transform bufs[5] holds
     const void* transformed_from = nullptr;
+    // convolution launches resolved at finalize (kernel, tile shape, grid, split, environment switches)
+    std::shared_ptr<kxc_hip::PreparedConv> prepared_conv;
+    std::shared_ptr<kxc_hip::PreparedWinograd> prepared_wino;
     // module kernel
     void* function = nullptr;
     uint32_t grid[3], block[3], shared_bytes = 0;
     std::vector<kxc_hip_buf> params;
 };
+
+// Bytes of every operand whose size follows from the node's geometry (fp32 operators; the int8 nodes' blocked
+// layouts and module kernels' parameters are checked by offset only).
+void OperandExtents(const Node& n, std::vector<std::pair<kxc_hip_buf, size_t>>* out) {
+    auto add = [&](const kxc_hip_buf& b, int64_t elems, size_t elem_bytes = 4) {
+        if (b.kind != KXC_HIP_BUF_NONE && elems > 0) out->emplace_back(b, static_cast<size_t>(elems) * elem_bytes);
+    };
+    switch (n.kind) {
+        case NodeKind::kConv2D: {
+            const kxc_hip_conv2d_desc& d = n.conv;
+            const int64_t oh = (static_cast<int64_t>(d.h) + 2 * d.pad_h - (static_cast<int64_t>(d.dil_h) * (d.kh - 1) + 1)) / d.stride_h + 1;
+            const int64_t ow = (static_cast<int64_t>(d.w) + 2 * d.pad_w - (static_cast<int64_t>(d.dil_w) * (d.kw - 1) + 1)) / d.stride_w + 1;
+            const int64_t y = static_cast<int64_t>(d.n) * d.o * oh * ow;
+            add(n.bufs[0], static_cast<int64_t>(d.n) * d.c * d.h * d.w);
+            add(n.bufs[1], static_cast<int64_t>(d.o) * d.c * d.kh * d.kw);
+            add(n.bufs[2], d.o);
+            add(n.bufs[3], y);
+            add(n.bufs[4], y);
+            if (n.i32[0] == 1) {
+                size_t u = 0;
+                if (kxc_hip_conv2d_winograd_weight_bytes(&d, &u) == KXC_HIP_OK) add(n.bufs[5], static_cast<int64_t>(u), 1);
+            }
+            if (n.i32[0] == 2 && n.params.size() == 3) {
+                add(n.params[0], static_cast<int64_t>(d.o) * d.c);
+                add(n.params[1], d.o);
+                add(n.params[2], y);
+            }
+            break;
+        }
+        case NodeKind::kPool2D: {
+            const kxc_hip_pool2d_desc& d = n.pool;
+            auto dim = [&](int64_t in, int64_t k, int64_t s, int64_t p0, int64_t p1) {
+                const int64_t span = in + p0 + p1 - k;
+                if (span < 0 || s <= 0) return static_cast<int64_t>(0);
+                return (d.ceil_mode ? (span + s - 1) / s : span / s) + 1;      // as kxc_hip_pool2d_f32 sizes its output
+            };
+            add(n.bufs[0], static_cast<int64_t>(d.n) * d.c * d.h * d.w);
+            add(n.bufs[1], static_cast<int64_t>(d.n) * d.c * dim(d.h, d.kh, d.stride_h, d.pad_top, d.pad_bottom) *
+                               dim(d.w, d.kw, d.stride_w, d.pad_left, d.pad_right));
+            break;
+        }
+        case NodeKind::kGlobalAvgPool:
+            add(n.bufs[0], n.dims[0] * n.dims[1] * n.dims[2] * n.dims[3]);
+            add(n.bufs[1], n.dims[0] * n.dims[1]);
+            break;
+        case NodeKind::kGemm:
+            add(n.bufs[0], n.dims[0] * n.dims[2]);
+            add(n.bufs[1], n.dims[1] * n.dims[2]);
+            add(n.bufs[2], n.dims[3]);
+            add(n.bufs[3], n.dims[0] * n.dims[1]);
+            break;
+        case NodeKind::kBinary: {
+            int64_t a = 1, b = 1;
+            for (int i = 0; i < n.i32[1]; ++i) a *= n.a_shape[i];
+            for (int i = 0; i < n.i32[2]; ++i) b *= n.b_shape[i];
+            add(n.bufs[0], a);
+            add(n.bufs[1], b);
+            add(n.bufs[2], a > b ? a : b);      // (the broadcast result is at least as large as either operand)
+            break;
+        }
+        case NodeKind::kRelu:
+            add(n.bufs[0], n.dims[0]);
+            add(n.bufs[1], n.dims[0]);
+            break;
+        case NodeKind::kCopy:
+            add(n.bufs[0], n.dims[0], 1);
+            add(n.bufs[1], n.dims[0], 1);
+            break;
+        default:
+            break;
+    }
+}
 
 }  // namespace
 
@@ -481,6 +558,18 @@ int32_t kxc_hip_plan_add_module_kernel(kxc_hip_plan* plan, void* function, const
 int32_t kxc_hip_plan_finalize(kxc_hip_plan* plan, size_t workspace_bytes) {
     KXC_HIP_REQUIRE(plan != nullptr, "kxc_hip_plan_finalize: plan is NULL");
     KXC_HIP_REQUIRE(!plan->finalized, "kxc_hip_plan_finalize: plan is already finalized");
+    // every workspace operand whose size the node's geometry fixes must end inside the workspace
+    for (const Node& n : plan->nodes) {
+        std::vector<std::pair<kxc_hip_buf, size_t>> extents;
+        OperandExtents(n, &extents);
+        for (const auto& e : extents) {
+            if (e.first.kind != KXC_HIP_BUF_WORKSPACE) continue;
+            const size_t off = static_cast<size_t>(e.first.index_or_offset);
+            KXC_HIP_REQUIRE(off <= workspace_bytes && e.second <= workspace_bytes - off,
+                            "kxc_hip_plan_finalize: node %s: an operand of %zu bytes at workspace offset %zu does not fit the "
+                            "%zu-byte workspace", n.symbol.c_str(), e.second, off, workspace_bytes);
+        }
+    }
     for (const Node& n : plan->nodes) {
         auto check = [&](kxc_hip_buf b) {
             return !(b.kind == KXC_HIP_BUF_WORKSPACE && static_cast<size_t>(b.index_or_offset) >= workspace_bytes &&
@@ -509,6 +598,20 @@ int32_t kxc_hip_plan_finalize(kxc_hip_plan* plan, size_t workspace_bytes) {
         }
         KXC_HIP_CALL(hipEventCreateWithFlags(&n.fork_event, hipEventDisableTiming), "plan event");
         KXC_HIP_CALL(hipEventCreateWithFlags(&n.done_event, hipEventDisableTiming), "plan event");
+    }
+    // Resolve every convolution launch now: the runs only add the operand pointers and the stream.
+    for (Node& n : plan->nodes) {
+        if (n.kind != NodeKind::kConv2D) continue;
+        KXC_HIP_CALL(hipSetDevice(plan->device_id), "HIP SetDevice");
+        if (n.i32[0] == 1) {
+            kxc_hip::PreparedWinograd* p = nullptr;
+            if (int32_t rc = kxc_hip::PrepareWinograd(&n.conv, &p)) return rc;
+            n.prepared_wino.reset(p, kxc_hip::FreePreparedWinograd);
+        } else {
+            kxc_hip::PreparedConv* p = nullptr;
+            if (int32_t rc = kxc_hip::PrepareConv2d(&n.conv, n.i32[0] == 2, &p)) return rc;
+            n.prepared_conv.reset(p, kxc_hip::FreePreparedConv);
+        }
     }
     plan->finalized = true;
     return KXC_HIP_OK;
@@ -567,25 +670,24 @@ int32_t RunNode(kxc_hip_plan* plan, Node& n, void** args, void* s) {
         auto B = [&](int i) { return Resolve(plan, n.bufs[i], args); };
         switch (n.kind) {
             case NodeKind::kConv2D:
+                // (launches resolved at finalize; s is never NULL here)
                 if (n.i32[0] == 1) {
                     // (the transformed weights in B(5) were written by TransformConstants at the start of the run)
-                    rc = kxc_hip_conv2d_winograd_nchw_f32(&n.conv, static_cast<const float*>(B(0)), static_cast<const float*>(B(5)),
-                                                          static_cast<const float*>(B(2)), static_cast<const float*>(B(3)),
-                                                          static_cast<float*>(B(4)), s);
+                    rc = kxc_hip::LaunchPreparedWinograd(n.prepared_wino.get(), static_cast<const float*>(B(0)),
+                                                         static_cast<const float*>(B(5)), static_cast<const float*>(B(2)),
+                                                         static_cast<const float*>(B(3)), static_cast<float*>(B(4)),
+                                                         kxc_hip::ResolveStream(s));
                     break;
                 }
-                if (n.i32[0] == 2) {
-                    rc = kxc_hip_conv2d_pair_nchw_f32(&n.conv, static_cast<const float*>(B(0)), static_cast<const float*>(B(1)),
-                                                      static_cast<const float*>(B(2)), static_cast<const float*>(B(3)),
-                                                      static_cast<float*>(B(4)),
-                                                      static_cast<const float*>(Resolve(plan, n.params[0], args)),
-                                                      static_cast<const float*>(Resolve(plan, n.params[1], args)),
-                                                      static_cast<float*>(Resolve(plan, n.params[2], args)), s);
-                    break;
+                {
+                    const bool pair = n.i32[0] == 2;
+                    rc = kxc_hip::LaunchPreparedConv2d(
+                        n.prepared_conv.get(), static_cast<const float*>(B(0)), static_cast<const float*>(B(1)),
+                        static_cast<const float*>(B(2)), static_cast<const float*>(B(3)), static_cast<float*>(B(4)),
+                        pair ? static_cast<const float*>(Resolve(plan, n.params[0], args)) : nullptr,
+                        pair ? static_cast<const float*>(Resolve(plan, n.params[1], args)) : nullptr,
+                        pair ? static_cast<float*>(Resolve(plan, n.params[2], args)) : nullptr, kxc_hip::ResolveStream(s));
                 }
-                rc = kxc_hip_conv2d_nchw_f32(&n.conv, static_cast<const float*>(B(0)), static_cast<const float*>(B(1)),
-                                             static_cast<const float*>(B(2)), static_cast<const float*>(B(3)),
-                                             static_cast<float*>(B(4)), s);
                 break;
             case NodeKind::kPool2D:
                 rc = kxc_hip_pool2d_f32(&n.pool, static_cast<const float*>(B(0)), static_cast<float*>(B(1)), s);

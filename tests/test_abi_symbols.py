@@ -81,6 +81,24 @@ def test_plan_builder_validates_on_the_host(pkg):
     plan.add_relu(4, pkg.Buf.arg(0), pkg.Buf.arg(2))
     assert plan.symbols() == ["kxc_relu_f32"]
     plan.close()
+    # finalize checks every workspace operand's extent, not only where it starts, before it allocates anything
+    plan = pkg.Plan(3)
+    plan.add_relu(1000, pkg.Buf.arg(0), pkg.Buf.ws(256))                    # 4000 bytes at offset 256
+    try:
+        plan.finalize(4096)
+        raise AssertionError("operand past the end of the workspace accepted")
+    except pkg.KxcHipError as e:
+        assert "does not fit" in str(e) and "4000 bytes" in str(e)
+    plan.close()
+    plan = pkg.Plan(3)
+    d = pkg.ConvDesc(1, 4, 8, 8, 8, 3, 3, 1, 1, 1, 1, 1, 1, 0)             # y: 1 x 8 x 8 x 8 floats = 2048 bytes
+    plan.add_conv2d(d, pkg.Buf.arg(0), pkg.Buf.arg(1), pkg.Buf.none(), pkg.Buf.none(), pkg.Buf.ws(1024))
+    try:
+        plan.finalize(2048)
+        raise AssertionError("convolution output past the end of the workspace accepted")
+    except pkg.KxcHipError as e:
+        assert "does not fit" in str(e)
+    plan.close()
 
 
 def test_resnet18_plan_shape(pkg):
