@@ -599,10 +599,21 @@ int32_t kxc_hip_plan_finalize(kxc_hip_plan* plan, size_t workspace_bytes) {
         KXC_HIP_CALL(hipEventCreateWithFlags(&n.fork_event, hipEventDisableTiming), "plan event");
         KXC_HIP_CALL(hipEventCreateWithFlags(&n.done_event, hipEventDisableTiming), "plan event");
     }
-    // Resolve every convolution launch now: the runs only add the operand pointers and the stream.
+    // Resolve every convolution launch now: the runs only add the operand pointers and the stream.  The node's
+    // symbol names the variant resolved here (the one chosen when the node was added may have been picked under
+    // other environment switches).
     for (Node& n : plan->nodes) {
         if (n.kind != NodeKind::kConv2D) continue;
         KXC_HIP_CALL(hipSetDevice(plan->device_id), "HIP SetDevice");
+        {
+            const std::string prefix = "kxc_conv2d_nchw_f32.";
+            const char* variant = n.i32[0] == 1   ? kxc_hip_conv2d_winograd_variant(&n.conv)
+                                  : n.i32[0] == 2 ? kxc_hip_conv2d_pair_variant(&n.conv)
+                                                  : kxc_hip_conv2d_variant(&n.conv);
+            const size_t end = n.symbol.find_first_of("+|", prefix.size());
+            if (n.symbol.compare(0, prefix.size(), prefix) == 0)
+                n.symbol = prefix + variant + (end == std::string::npos ? std::string() : n.symbol.substr(end));
+        }
         if (n.i32[0] == 1) {
             kxc_hip::PreparedWinograd* p = nullptr;
             if (int32_t rc = kxc_hip::PrepareWinograd(&n.conv, &p)) return rc;

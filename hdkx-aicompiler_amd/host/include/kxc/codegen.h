@@ -18,7 +18,9 @@
 //   * LDS staging: a reduction whose source rows are contiguous in memory (global average pool,
 //     reduce_mean over trailing axes, row sums) is scheduled as a cooperative, coalesced load of the
 //     workgroup's rows into LDS followed by per-thread sequential sums from LDS (odd row stride, no
-//     bank conflicts), which keeps the order and removes the strided global reads.
+//     bank conflicts), which keeps the order and removes the strided global reads; a reduction whose innermost
+//     axis walks an operand contiguously per thread (dense / matmul against a transposed operand, long rows) stages
+//     that operand a chunk of the axis at a time the same way ("lds_k_stage"), again adding in the CPU order.
 #pragma once
 
 #include "kxc/tir.h"
@@ -40,7 +42,7 @@ struct HIPKernelSpec {
     uint32_t shared_bytes = 0;
     // kernel parameters: the buffer variables of the PrimFunc (parameters or Allocate'd intermediates)
     std::vector<const tir::ExprNode*> buffers;
-    std::string schedule;     // "flat" or "lds_row_reduce"
+    std::string schedule;     // "flat", "lds_row_reduce" or "lds_k_stage"
 };
 
 struct HIPModuleSource {

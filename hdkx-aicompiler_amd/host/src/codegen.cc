@@ -61,9 +61,15 @@ private:
 // to the wider / floating type, which is the reference's promotion rule
 // (src/codegen/codegen_llvm.cc:189-217,266-273); Min/Max are compare + select with an ordered compare
 // (:317-334), Select is a conditional (:391-442).
-std::string EmitExpr(const PrimExpr& e, Names* names) {
+// overrides: text to emit in place of given nodes (the LDS-staged loads of a scheduled reduction)
+using ExprOverrides = std::map<const ExprNode*, std::string>;
+std::string EmitExpr(const PrimExpr& e, Names* names, const ExprOverrides* overrides = nullptr) {
     if (!e.defined()) return "0";
-    auto A = [&](int i) { return EmitExpr(e->args[i], names); };
+    if (overrides) {
+        auto it = overrides->find(e.get());
+        if (it != overrides->end()) return it->second;
+    }
+    auto A = [&](int i) { return EmitExpr(e->args[i], names, overrides); };
     char buf[64];
     switch (e->kind) {
         case ExprKind::kIntImm:
@@ -333,12 +339,82 @@ bool MatchRowReduce(const LoopNest& data, Stmt* init_out, PrimExpr* src_load, in
     return true;
 }
 
+// Recognises  for data axes { out[o] = init; for reduce axes { out[o] = out[o] + EXPR } }  where the innermost
+// reduce axis k has a constant extent of at least 16 and EXPR holds fp32 loads that walk memory contiguously along k
+// (dense / matmul with a transposed operand, long row sums): every thread reads a run of consecutive floats, so the
+// lanes of a wave read addresses a whole row apart.  Such loads are staged through LDS a chunk of k at a time.
+struct KStage {
+    Stmt init, upd;
+    LoopNest red;
+    PrimExpr expr;                       // EXPR
+    std::vector<PrimExpr> staged;        // the load nodes that go through LDS
+    int64_t extent = 0;                  // of the innermost reduce axis
+    int chunk = 0;                       // floats of a row staged at a time
+};
+
+void CollectLoads(const PrimExpr& e, std::vector<PrimExpr>* out) {
+    if (!e.defined()) return;
+    if (e->kind == ExprKind::kLoad) out->push_back(e);
+    for (const auto& a : e->args) CollectLoads(a, out);
+}
+
+bool MatchKStage(const LoopNest& data, KStage* m) {
+    const Stmt& b = data.body;
+    if (!b.defined() || b->kind != StmtKind::kSeqStmt || b->body.size() != 2 || data.vars.empty()) return false;
+    const Stmt& init = b->body[0];
+    if (init->kind != StmtKind::kStore) return false;
+    LoopNest red = PeelLoops(b->body[1], false);
+    if (red.vars.empty() || !red.body.defined() || red.body->kind != StmtKind::kStore) return false;
+    const Stmt& upd = red.body;
+    if (upd->var.get() != init->var.get()) return false;
+    if (!upd->a.defined() || upd->a->kind != ExprKind::kAdd) return false;       // sums only: the order is kept
+    const PrimExpr& old = upd->a->args[0];
+    if (old->kind != ExprKind::kLoad || old->args[0].get() != init->var.get()) return false;
+    Affine oi = AnalyzeAffine(init->b), ui = AnalyzeAffine(upd->b), li = AnalyzeAffine(old->args[1]);
+    if (!oi.ok || !ui.ok || !li.ok || oi.coef != ui.coef || oi.constant != ui.constant || oi.coef != li.coef ||
+        oi.constant != li.constant)
+        return false;
+    for (const auto& v : red.vars)
+        if (oi.coef.count(v.get()) && oi.coef.at(v.get()) != 0) return false;     // the output does not move with the reduction
+    if (!init->a.defined() || !init->a.dtype().is_float() || init->a.dtype().bits != 32) return false;
+    const tir::Var& rk = red.vars.back();
+    const int64_t extent = red.extents.back();
+    if (extent < 16) return false;
+    std::vector<PrimExpr> loads;
+    CollectLoads(upd->a->args[1], &loads);
+    const tir::Var& lane_var = data.vars.back();
+    const int64_t lane_extent = data.extents.back();
+    for (const auto& l : loads) {
+        if (l->args[0].get() == init->var.get()) return false;                  // EXPR reads the output: not a plain sum
+        if (!l.dtype().is_float() || l.dtype().bits != 32) continue;
+        Affine ai = AnalyzeAffine(l->args[1]);
+        if (!ai.ok || !ai.coef.count(rk.get()) || ai.coef.at(rk.get()) != 1) continue;
+        bool thread_dependent = false;
+        for (const auto& v : data.vars)
+            if (ai.coef.count(v.get()) && ai.coef.at(v.get()) != 0) thread_dependent = true;
+        if (!thread_dependent) continue;
+        // the same row for (nearly) every lane of a wave is a broadcast load already
+        const int64_t lane_coef = ai.coef.count(lane_var.get()) ? ai.coef.at(lane_var.get()) : 0;
+        if (lane_coef == 0 && lane_extent >= 64) continue;
+        m->staged.push_back(l);
+    }
+    if (m->staged.empty() || m->staged.size() > 2) return false;
+    m->init = init; m->upd = upd; m->red = red; m->expr = upd->a->args[1];
+    m->extent = extent;
+    m->chunk = m->staged.size() == 1 ? 32 : 16;      // 256 rows x (chunk + 1) floats per staged load: 33 / 2 x 17 KiB
+    return true;
+}
+
 }  // namespace
 
 HIPModuleSource CodeGenHIP::Generate(const tir::PrimFunc& func, const std::string& prefix) {
     HIPModuleSource out;
     Names names;
     names.builtin_types = true;
+    // identifiers the schedules below declare themselves: no buffer or loop variable may take them
+    for (const char* id : {"tile", "tile0", "tile1", "rowbase0", "rowbase1", "total", "base", "rows", "row", "e", "k", "kk",
+                           "k0", "kend", "acc", "gid", "rem", "valid", "r"})
+        names.Reserve(id);
     std::ostringstream os;
     os << "// generated by kxc CodeGenHIP for gfx950 (wave64)\n";
     os << "#ifndef INFINITY\n#define INFINITY __builtin_inff()\n#endif\n#ifndef NAN\n#define NAN __builtin_nanf(\"\")\n#endif\n\n";
@@ -397,6 +473,68 @@ HIPModuleSource CodeGenHIP::Generate(const tir::PrimFunc& func, const std::strin
             os << "      for (int r = 0; r < " << R << "; ++r) acc = acc + tile[threadIdx.x * " << rp << " + r];\n";
             os << "      " << o << "[base + threadIdx.x] = acc;\n";
             os << "    }\n    __syncthreads();\n  }\n";
+        } else if (KStage ks; MatchKStage(data, &ks)) {
+            // ---- reduction whose k-contiguous operands are staged through LDS, a chunk of k at a time; every
+            // thread still adds its products in the CPU order (acc = acc + EXPR for k = 0, 1, ...)
+            spec.schedule = "lds_k_stage";
+            const int KC = ks.chunk, KP = KC + 1;
+            const std::string o = names.Get(ks.init->var.get());
+            const std::string rk = names.Get(ks.red.vars.back().get());
+            for (size_t j = 0; j < ks.staged.size(); ++j) {
+                os << "  __shared__ float tile" << j << "[" << 256 * KP << "];\n";
+                os << "  __shared__ long long rowbase" << j << "[256];\n";
+            }
+            os << "  const long long total = " << total << "LL;\n";
+            os << "  for (long long base = (long long)blockIdx.x * 256; base < total; base += (long long)gridDim.x * 256) {\n";
+            os << "    const long long gid = base + threadIdx.x;\n";
+            os << "    const bool valid = gid < total;\n";
+            os << "    long long rem = valid ? gid : total - 1;      // threads past the end help with the loads only\n";
+            for (int i = static_cast<int>(data.vars.size()) - 1; i >= 0; --i) {
+                const std::string v = names.Get(data.vars[i].get());
+                if (i == 0) os << "    const int " << v << " = (int)rem;\n";
+                else {
+                    os << "    const int " << v << " = (int)(rem % " << data.extents[i] << "LL);\n";
+                    os << "    rem /= " << data.extents[i] << "LL;\n";
+                }
+            }
+            os << "    float acc = " << EmitExpr(ks.init->a, &names) << ";\n";
+            std::string pad = "    ";
+            for (size_t i = 0; i + 1 < ks.red.vars.size(); ++i) {
+                const std::string v = names.Get(ks.red.vars[i].get());
+                os << pad << "for (int " << v << " = 0; " << v << " < " << ks.red.extents[i] << "; ++" << v << ") {\n";
+                pad += "  ";
+            }
+            os << pad << "{ const int " << rk << " = 0;\n";
+            for (size_t j = 0; j < ks.staged.size(); ++j)
+                os << pad << "  rowbase" << j << "[threadIdx.x] = (long long)(" << EmitExpr(ks.staged[j]->args[1], &names) << ");\n";
+            os << pad << "}\n";
+            os << pad << "for (int k0 = 0; k0 < " << ks.extent << "; k0 += " << KC << ") {\n";
+            os << pad << "  __syncthreads();\n";
+            os << pad << "  for (int e = threadIdx.x; e < " << 256 * KC << "; e += 256) {\n";
+            os << pad << "    const int row = e / " << KC << ", k = e - row * " << KC << ";\n";
+            os << pad << "    if (k0 + k < " << ks.extent << ") {\n";
+            ExprOverrides overrides;
+            for (size_t j = 0; j < ks.staged.size(); ++j) {
+                os << pad << "      tile" << j << "[row * " << KP << " + k] = " << names.Get(ks.staged[j]->args[0].get())
+                   << "[rowbase" << j << "[row] + k0 + k];\n";
+                overrides[ks.staged[j].get()] = "tile" + std::to_string(j) + "[threadIdx.x * " + std::to_string(KP) + " + kk]";
+            }
+            os << pad << "    }\n";
+            os << pad << "  }\n";
+            os << pad << "  __syncthreads();\n";
+            os << pad << "  const int kend = (" << ks.extent << " - k0) < " << KC << " ? (" << ks.extent << " - k0) : " << KC << ";\n";
+            os << pad << "  for (int kk = 0; kk < kend; ++kk) {\n";
+            os << pad << "    const int " << rk << " = k0 + kk;\n";
+            os << pad << "    (void)" << rk << ";\n";
+            os << pad << "    acc = acc + " << EmitExpr(ks.expr, &names, &overrides) << ";\n";
+            os << pad << "  }\n";
+            os << pad << "}\n";
+            for (size_t i = 0; i + 1 < ks.red.vars.size(); ++i) {
+                pad.resize(pad.size() - 2);
+                os << pad << "}\n";
+            }
+            os << "    if (valid) " << o << "[" << EmitExpr(ks.init->b, &names) << "] = acc;\n";
+            os << "  }\n";
         } else {
             // ---- flat schedule: one output element per thread per grid-stride step
             spec.schedule = "flat";

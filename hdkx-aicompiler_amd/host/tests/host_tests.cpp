@@ -484,6 +484,22 @@ int RunCodegen() {
     Check(gap_hip.kernels.size() == 2 && gap_hip.kernels[0].schedule == "lds_row_reduce", "gap sum is LDS staged");
     Check(gap_hip.source.find("__shared__ float tile[") != std::string::npos, "LDS tile declared");
     Check(gap_hip.source.find("/ ((long long)49LL)") != std::string::npos || gap_hip.source.find("49") != std::string::npos, "division by H*W");
+    // dense against a [units, k] weight: every thread walks a row of the weight -> staged through LDS in chunks of k,
+    // still added in k order; a short reduction (k = 8) stays flat
+    {
+        kxc::Var dx("x", kxc::TensorType({8, 64}, "float32")), dw("w", kxc::TensorType({40, 64}, "float32"));
+        kxc::Function dense({dx, dw}, kxc::Call(Op::Get("nn_dense"), {dx, dw}, kxc::relay::DenseAttrs::Create(40, "")));
+        auto dense_hip = cgh.Generate(kxc::relay::LowerToTIR(kxc::relay::InferTypePass(dense)), "kxc_dense");
+        Check(dense_hip.kernels.size() == 1 && dense_hip.kernels[0].schedule == "lds_k_stage",
+              "dense is LDS staged along k, got " + dense_hip.kernels[0].schedule);
+        Check(dense_hip.source.find("__shared__ float tile0[") != std::string::npos &&
+                  dense_hip.source.find("acc = acc + ") != std::string::npos, "staged tile and ordered accumulation");
+        if (const char* dump = std::getenv("KXC_DUMP_DENSE_HIP")) std::ofstream(dump) << dense_hip.source;
+        kxc::Var sx("x", kxc::TensorType({8, 8}, "float32")), sw("w", kxc::TensorType({4, 8}, "float32"));
+        kxc::Function small({sx, sw}, kxc::Call(Op::Get("nn_dense"), {sx, sw}, kxc::relay::DenseAttrs::Create(4, "")));
+        auto small_hip = cgh.Generate(kxc::relay::LowerToTIR(kxc::relay::InferTypePass(small)), "kxc_small");
+        Check(small_hip.kernels[0].schedule == "flat", "a reduction of 8 stays flat");
+    }
     // a ResNet-18 compile for the hip target without a GPU: plan and fusion are built, nothing is loaded
     g_mode = "hip";
     auto module = kxc::api::Compiler::Compile(kxc::models::BuildResNet18(1, 224), MakeConfig());

@@ -248,7 +248,8 @@ def test_resnet18_generated_kernels_equal_oracle_bit_for_bit(synth):
         x, consts = _write_resnet_inputs(synth, d, 3, 1, 64)
         out = run("resnet18", "hipgen", d, "1", "64")
         assert "execution plan replayed:" in out and "identical output" in out      # generated kernels recompiled from the saved source
-        assert "lds_row_reduce" in out
+        assert "lds_row_reduce" in out          # global average pool: whole rows staged through LDS
+        assert "lds_k_stage" in out             # the FC layer: rows of the weight staged a chunk of k at a time
         got = np.fromfile(os.path.join(d, "logits.bin"), np.float32).reshape(1, 1000)
     want = Oracle(fast=True).resnet18(x, consts)
     assert np.array_equal(bits(got), bits(want))
