@@ -1,0 +1,4 @@
+// Forwarding header: code written against the reference's include/base/registry.h compiles against the host layer
+// with -I<host>/include/compat -I<host>/include.
+#pragma once
+#include "kxc/packed_func.h"

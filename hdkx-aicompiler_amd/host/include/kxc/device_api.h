@@ -32,16 +32,43 @@ enum class DeviceAttrKind : int {
     kL2CacheSizeBytes = 11, kTotalGlobalMemory = 12, kAvailableGlobalMemory = 13, kMaxSharedMemoryPerMultiprocessor = 14,
     kMaxRegistersPerMultiprocessor = 15, kMaxThreadsPerMultiprocessor = 16, kComputeVersionMajor = 17, kComputeVersionMinor = 18,
 };
-// What GetAttr returns: an integer, or text for kComputeVersion / kDeviceName (the reference's RetValue holds either).
+// What a packed function returns (include/base/packedfunc.h:110-230): nothing, an integer, a double, text or an object
+// handle.  GetAttr gives an integer, or text for kComputeVersion / kDeviceName.
 struct RetValue {
     int64_t v_int64{0};
+    double v_float{0.0};
     std::string v_str;
-    bool is_str{false};
-    RetValue& operator=(int64_t v) { v_int64 = v; is_str = false; return *this; }
-    RetValue& operator=(int v) { v_int64 = v; is_str = false; return *this; }
-    RetValue& operator=(const std::string& s) { v_str = s; is_str = true; return *this; }
-    operator int64_t() const { return v_int64; }
-    operator std::string() const { return v_str; }
+    ObjectRef v_object;
+    bool is_str{false}, is_float{false}, is_object{false}, is_set{false};
+    RetValue& operator=(int64_t v) { Clear(); v_int64 = v; return *this; }
+    RetValue& operator=(int v) { return *this = static_cast<int64_t>(v); }
+    RetValue& operator=(bool v) { return *this = static_cast<int64_t>(v); }
+    RetValue& operator=(double v) { Clear(); v_float = v; is_float = true; return *this; }
+    RetValue& operator=(const std::string& s) { Clear(); v_str = s; is_str = true; return *this; }
+    RetValue& operator=(const char* s) { return *this = std::string(s ? s : ""); }
+    RetValue& operator=(const ObjectRef& o) { Clear(); v_object = o; is_object = true; return *this; }
+    // conversions throw the reference's "Type mismatch: expected ..." when the held kind does not fit
+    operator int64_t() const {
+        if (is_float) return static_cast<int64_t>(v_float);
+        if (is_str || is_object) throw std::runtime_error("Type mismatch: expected int");
+        return v_int64;
+    }
+    operator double() const {
+        if (is_float) return v_float;
+        if (is_str || is_object) throw std::runtime_error("Type mismatch: expected double");
+        return static_cast<double>(v_int64);
+    }
+    operator std::string() const {
+        if (!is_str && is_set) throw std::runtime_error("Type mismatch: expected string");
+        return v_str;
+    }
+    operator ObjectRef() const {
+        if (!is_object && is_set) throw std::runtime_error("Type mismatch: expected ObjectRef");
+        return v_object;
+    }
+
+private:
+    void Clear() { v_int64 = 0; v_float = 0.0; v_str.clear(); v_object = ObjectRef(); is_str = is_float = is_object = false; is_set = true; }
 };
 
 struct DeviceAttributes {
@@ -123,8 +150,9 @@ DeviceAPI* GetHIPDeviceAPI();
 DeviceAPI* GetDeviceAPI(DeviceTypeCode type);
 std::vector<DeviceInfo> GetAllDeviceInfo();
 std::string GetAllDeviceInfoJSON();
+std::string ListDevicesJSON();      // the available ones only
 
-struct TargetNode {
+struct TargetNode : Object {
     std::string kind;            // "llvm" for the CPU (the reference's name), "hip" for the GPU
     Device device;
     DeviceAttributes attrs;

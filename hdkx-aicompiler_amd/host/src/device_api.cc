@@ -232,11 +232,25 @@ std::vector<DeviceInfo> GetAllDeviceInfo() {
     return out;
 }
 
-std::string GetAllDeviceInfoJSON() {
+namespace {
+std::string DeviceInfosToJSON(const std::vector<DeviceInfo>& infos);
+}
+std::string GetAllDeviceInfoJSON() { return DeviceInfosToJSON(GetAllDeviceInfo()); }
+
+// Only the devices that can be used (src/base/device_api.cc:363-371).
+std::string ListDevicesJSON() {
+    std::vector<DeviceInfo> available;
+    for (const auto& info : GetAllDeviceInfo())
+        if (info.available) available.push_back(info);
+    return DeviceInfosToJSON(available);
+}
+
+namespace {
+std::string DeviceInfosToJSON(const std::vector<DeviceInfo>& infos) {
     std::ostringstream os;
     os << "[";
     bool first = true;
-    for (const auto& d : GetAllDeviceInfo()) {
+    for (const auto& d : infos) {
         os << (first ? "" : ",") << "{\"device_type\":" << static_cast<int>(d.device_type) << ",\"device_id\":" << d.device_id
            << ",\"device_type_name\":\"" << d.device_type_name << "\",\"target_kind\":\"" << d.target_kind
            << "\",\"available\":" << (d.available ? "true" : "false") << ",\"arch\":\"" << d.attrs.arch
@@ -246,6 +260,7 @@ std::string GetAllDeviceInfoJSON() {
     os << "]";
     return os.str();
 }
+}  // namespace
 
 Target BuildTarget(DeviceTypeCode type, int device_id) {
     auto n = std::make_shared<TargetNode>();

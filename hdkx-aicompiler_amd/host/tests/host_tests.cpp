@@ -22,6 +22,7 @@
 #include <atomic>
 
 #include "kxc/compiler.h"
+#include "kxc/packed_func.h"
 #include "kxc/models.h"
 #include "kxc/onnx_importer.h"
 #include "kxc/profiling.h"
@@ -1065,6 +1066,87 @@ int RunKernelObject(const std::string& dir) {
     return 0;
 }
 
+// The registry face of the device API and of the plan functions (include/base/registry.h, src/base/device_api.cc:442-658).
+int RunPackedFunc(const std::string& mode) {
+    using kxc::PackedFunc; using kxc::Registry; using kxc::RetValue;
+    Registry& reg = Registry::Global();
+    Check(!reg.Get("no.such.function").defined(), "an absent name gives an empty function");
+    bool threw = false;
+    try { RetValue rv; reg.Get("no.such.function")(kxc::Args(), &rv); } catch (const std::runtime_error& e) { threw = std::string(e.what()) == "PackedFunc is empty"; }
+    Check(threw, "calling an empty function throws");
+    threw = false;
+    try { reg.Set("device_api.GetAttr", PackedFunc()); } catch (const std::runtime_error& e) {
+        threw = std::string(e.what()) == "Function device_api.GetAttr is already registered.";
+    }
+    Check(threw, "a name registers once");
+    for (const char* name : {"device_api.AllocDataSpace", "device_api.FreeDataSpace", "device_api.AllocWorkspace", "device_api.FreeWorkspace",
+                             "device_api.CopyDataFromTo", "device_api.CopyDataFromToEx", "device_api.GetAttr", "device_api.CreateStream",
+                             "device_api.FreeStream", "device_api.StreamSync", "device_api.SyncStreamFromTo", "device_api.SetStream",
+                             "device_api.GetCurrentStream", "device_api.NeedSetDevice", "device_api.ListDevices", "device_api.ListDevicesJSON",
+                             "device_api.GetAllDeviceInfo", "device_api.GetAllDeviceInfoJSON", "device_api.GetTargetKind",
+                             "device_api.GetTargetArch", "target.Build", "device.DetectAndRegister",
+                             "kxc.relay.transform.lower_to_exec_plan_json", "kxc.relay.transform.lower_to_exec_plan_json_file",
+                             "kxc.hip.execute_plan_json", "kxc.hip.execute_plan_json_file"})
+        Check(reg.Get(name).defined(), std::string(name) + " is registered");
+    const kxc::Device cpu(kxc::kCPU, 0), gpu(kxc::kGPU, 0);
+    Check(static_cast<int64_t>(reg.Get("device_api.NeedSetDevice")(0)) == 0 && static_cast<int64_t>(reg.Get("device_api.NeedSetDevice")(1)) == 1,
+          "NeedSetDevice: every type but the CPU");
+    Check(static_cast<std::string>(reg.Get("device_api.GetTargetKind")(cpu)) == "llvm", "CPU target kind");
+    Check(static_cast<std::string>(reg.Get("device_api.ListDevicesJSON")()).find("\"cpu\"") != std::string::npos, "the CPU is always listed");
+    threw = false;
+    try { reg.Get("device_api.AllocDataSpace")(std::string("cpu"), 16, 16); } catch (const std::runtime_error& e) {
+        threw = std::string(e.what()).find("Type mismatch") == 0;
+    }
+    Check(threw, "a wrong argument type is refused");
+    // allocate, copy and free through the registry on the host back end
+    std::vector<float> src = {1.5f, -2.0f, 3.25f, 4.0f}, dst(4, 0.0f);
+    auto I = [](const void* p) { return static_cast<int64_t>(reinterpret_cast<uintptr_t>(p)); };
+    const int64_t hbuf = reg.Get("device_api.AllocDataSpace")(cpu, 16, 64);
+    Check(hbuf != 0, "host allocation");
+    reg.Get("device_api.CopyDataFromTo")(cpu, I(src.data()), cpu, hbuf, 16);
+    reg.Get("device_api.CopyDataFromTo")(cpu, hbuf, cpu, I(dst.data()), 16);
+    Check(dst == src, "host copy round trip");
+    reg.Get("device_api.FreeDataSpace")(cpu, hbuf);
+    if (mode == "hip") {
+        Check(static_cast<std::string>(reg.Get("device_api.GetTargetKind")(gpu)) == "hip" &&
+                  static_cast<std::string>(reg.Get("device_api.GetTargetArch")(gpu)).find("gfx") == 0, "GPU target kind and arch");
+        Check(static_cast<int64_t>(reg.Get("device_api.GetAttr")(gpu, static_cast<int>(kxc::DeviceAttrKind::kWarpSize))) == 64, "wave size 64");
+        kxc::ObjectRef target = reg.Get("target.Build")(gpu);
+        Check(target.defined() && target.As<kxc::TargetNode>() && target.As<kxc::TargetNode>()->kind == "hip", "target.Build gives a Target");
+        reg.Get("device.DetectAndRegister")();
+        // (the marketing name comes from the driver's id table and may be empty where that table is not installed)
+        Check(reg.Get("device_info.hip.0.name").defined() && static_cast<int64_t>(reg.Get("device_info.hip.0.memory")()) > (1LL << 30) &&
+                  !static_cast<std::string>(reg.Get("device_info.hip.0.compute_capability")()).empty(), "device_info.hip.0.*");
+        (void)static_cast<std::string>(reg.Get("device_info.hip.0.name")());
+        const int64_t stream = reg.Get("device_api.CreateStream")(gpu);
+        const int64_t dbuf = reg.Get("device_api.AllocDataSpace")(gpu, 16, 256);
+        std::fill(dst.begin(), dst.end(), 0.0f);
+        reg.Get("device_api.CopyDataFromToEx")(cpu, I(src.data()), 0, gpu, dbuf, 0, 16, stream);
+        reg.Get("device_api.CopyDataFromToEx")(gpu, dbuf, 8, cpu, I(dst.data()), 8, 8, stream);      // the second half only
+        reg.Get("device_api.StreamSync")(gpu, stream);
+        Check(dst[0] == 0.0f && dst[1] == 0.0f && dst[2] == src[2] && dst[3] == src[3], "device copy with offsets on a stream");
+        // a Relay function -> plan JSON -> run from the JSON, all through the registry
+        kxc::Var a("a", kxc::TensorType({2, 3}, "float32")), b("b", kxc::TensorType({2, 3}, "float32"));
+        kxc::Function func({a, b}, kxc::Call(Op::Get("add"), {a, b}));
+        const std::string json = reg.Get("kxc.relay.transform.lower_to_exec_plan_json")(func);
+        Check(json.find("\"kernel_symbol\"") != std::string::npos && json.find("\"kxc_hip\"") != std::string::npos, "plan JSON from the registry");
+        std::vector<float> av = {1, 2, 3, 4, 5, 6}, bv = {10, 20, 30, 40, 50, 60}, out(6, 0.0f);
+        const int64_t da = reg.Get("device_api.AllocDataSpace")(gpu, 24, 256), db = reg.Get("device_api.AllocDataSpace")(gpu, 24, 256),
+                      dout = reg.Get("device_api.AllocDataSpace")(gpu, 24, 256);
+        reg.Get("device_api.CopyDataFromTo")(cpu, I(av.data()), gpu, da, 24);
+        reg.Get("device_api.CopyDataFromTo")(cpu, I(bv.data()), gpu, db, 24);
+        void* packed[3] = {reinterpret_cast<void*>(da), reinterpret_cast<void*>(db), reinterpret_cast<void*>(dout)};
+        Check(static_cast<int64_t>(reg.Get("kxc.hip.execute_plan_json")(json, static_cast<void*>(packed), 3)) == 0, "plan run");
+        reg.Get("device_api.StreamSync")(gpu, 0);
+        reg.Get("device_api.CopyDataFromTo")(gpu, dout, cpu, I(out.data()), 24);
+        Check(out == std::vector<float>({11, 22, 33, 44, 55, 66}), "plan run from JSON adds");
+        for (int64_t p : {da, db, dout, dbuf}) reg.Get("device_api.FreeDataSpace")(gpu, p);
+        reg.Get("device_api.FreeStream")(gpu, stream);
+    }
+    std::cout << "packed functions ok (" << mode << ")\n";
+    return 0;
+}
+
 int main(int argc, char** argv) {
     try {
         const std::string cmd = argc > 1 ? argv[1] : "";
@@ -1072,6 +1154,7 @@ int main(int argc, char** argv) {
         if (cmd == "device_info") return RunDeviceInfo();
         if (cmd == "adaptive") { g_mode = argc > 2 ? argv[2] : "cpu"; return RunAdaptive(argc > 3 ? argv[3] : ""); }
         if (cmd == "codegen") return RunCodegen();
+        if (cmd == "packed_func") return RunPackedFunc(argc > 2 ? argv[2] : "cpu");
         if (cmd == "onnx" && argc >= 4) { g_mode = argv[2]; return RunOnnx(argv[3]); }
         if (cmd == "onnx_errors" && argc >= 3) return RunOnnxErrors(argv[2]);
         if (cmd == "hip_smoke" && argc >= 3) return RunHipSmoke(argv[2]);

@@ -52,6 +52,19 @@ def test_device_info_contract():
     assert "device info ok" in run("device_info")
 
 
+def test_packed_function_registry_cpu():
+    """Registry::Global().Get / Set, KXC_REGISTER_GLOBAL, Args / RetValue conversions and the device_api.* functions on
+    the host back end (include/base/registry.h:13-61, src/base/device_api.cc:442-658)."""
+    assert "packed functions ok (cpu)" in run("packed_func", "cpu")
+
+
+@pytest.mark.gpu
+def test_packed_function_registry_hip():
+    """The same registry on the GPU: allocation, copies with offsets on a stream, attributes, target.Build,
+    device_info.hip.0.*, and a Relay function lowered to plan JSON and run from that JSON."""
+    assert "packed functions ok (hip)" in run("packed_func", "hip")
+
+
 def test_compiled_kernel_object_and_compile_config_surface_cpu():
     """codegen::CompiledKernel (fields, IsReady, call operator, error text), CompileConfig::profile_options / cache_dir
     and CompiledModule::GetProfileBundlePath on the host back end."""
