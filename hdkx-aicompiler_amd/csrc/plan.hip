@@ -478,6 +478,25 @@ int32_t kxc_hip_plan_add_qconv2d_c16(kxc_hip_plan* plan, const kxc_hip_qconv2d_d
     return KXC_HIP_OK;
 }
 
+// i32[0] = 3: the c16 convolution with a second output; params = {w2_packed, bias2, mult2, y2}
+int32_t kxc_hip_plan_add_qconv2d_c16_pair(kxc_hip_plan* plan, const kxc_hip_qconv2d_desc* desc, kxc_hip_buf x,
+                                          kxc_hip_buf w_packed, kxc_hip_buf bias, kxc_hip_buf mult, kxc_hip_buf residual,
+                                          kxc_hip_buf y, kxc_hip_buf w2_packed, kxc_hip_buf bias2, kxc_hip_buf mult2,
+                                          kxc_hip_buf y2) {
+    const char* who = "kxc_hip_plan_add_qconv2d_c16_pair";
+    KXC_PLAN_BEGIN(who);
+    KXC_HIP_REQUIRE(desc != nullptr, "%s: desc is NULL", who);
+    KXC_HIP_REQUIRE(kxc_hip_qconv2d_c16_pair_supported(desc), "%s: no kernel with a second output covers this shape", who);
+    KXC_PLAN_BUF(w2_packed, false, who); KXC_PLAN_BUF(bias2, true, who); KXC_PLAN_BUF(mult2, false, who); KXC_PLAN_BUF(y2, false, who);
+    if (int32_t rc = kxc_hip_plan_add_qconv2d_c16(plan, desc, x, w_packed, bias, mult, residual, y)) return rc;
+    Node& n = plan->nodes.back();
+    n.i32[0] = 3;
+    n.params = {w2_packed, bias2, mult2, y2};
+    n.symbol += "|qconv1x1";
+    if (bias2.kind != KXC_HIP_BUF_NONE) n.symbol += "+bias";
+    return KXC_HIP_OK;
+}
+
 int32_t kxc_hip_plan_add_qconv2d_c4(kxc_hip_plan* plan, const kxc_hip_qconv2d_desc* desc, kxc_hip_buf x_c4,
                                     kxc_hip_buf w_packed, kxc_hip_buf bias, kxc_hip_buf mult, kxc_hip_buf y_c16) {
     const char* who = "kxc_hip_plan_add_qconv2d_c4";
@@ -731,6 +750,16 @@ int32_t RunNode(kxc_hip_plan* plan, Node& n, void** args, void* s) {
                     rc = kxc_hip_qconv2d_c4_i8(&n.qconv, static_cast<const int8_t*>(B(0)), static_cast<const int8_t*>(B(1)),
                                                static_cast<const int32_t*>(B(2)), static_cast<const float*>(B(3)),
                                                static_cast<int8_t*>(B(5)), s);
+                    break;
+                }
+                if (n.i32[0] == 3) {
+                    rc = kxc_hip_qconv2d_c16_pair_i8(&n.qconv, static_cast<const int8_t*>(B(0)), static_cast<const int8_t*>(B(1)),
+                                                     static_cast<const int32_t*>(B(2)), static_cast<const float*>(B(3)),
+                                                     static_cast<const int8_t*>(B(4)), static_cast<int8_t*>(B(5)),
+                                                     static_cast<const int8_t*>(Resolve(plan, n.params[0], args)),
+                                                     static_cast<const int32_t*>(Resolve(plan, n.params[1], args)),
+                                                     static_cast<const float*>(Resolve(plan, n.params[2], args)),
+                                                     static_cast<int8_t*>(Resolve(plan, n.params[3], args)), s);
                     break;
                 }
                 if (n.i32[0] == 1) {
@@ -1084,6 +1113,10 @@ int32_t kxc_hip_plan_deserialize(const char* text, int32_t device_id, kxc_hip_mo
             (!kxc_hip_conv2d_pair_supported(&n.conv) || n.params.size() != 3 || n.params[0].kind == KXC_HIP_BUF_NONE ||
              n.params[2].kind == KXC_HIP_BUF_NONE))
             return fail("bad convolution-pair node");
+        if (n.kind == NodeKind::kQConv2D && n.i32[0] == 3 &&
+            (!kxc_hip_qconv2d_c16_pair_supported(&n.qconv) || n.params.size() != 4 || n.params[0].kind == KXC_HIP_BUF_NONE ||
+             n.params[2].kind == KXC_HIP_BUF_NONE || n.params[3].kind == KXC_HIP_BUF_NONE))
+            return fail("bad int8 convolution-pair node");
         if (n.kind == NodeKind::kModuleKernel) {
             // generated kernels are found by name in the modules the caller compiled from the saved source
             for (int32_t m = 0; m < num_modules && !n.function; ++m) {

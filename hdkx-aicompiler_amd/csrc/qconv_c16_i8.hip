@@ -82,6 +82,16 @@ struct QArgs {
     float res_mult;
     uint32_t flags;
     FastDiv div_wp, div_hp, div_ohw, div_ow, div_otiles;   // div_wp: positions per LDS row (pixels, or pixel quads on c4)
+    // Second output of the DS kernels: a 1x1 convolution with the same strides and no padding on the same input
+    // (a residual block's downsample beside the block's first 3x3 convolution).  Its operand x[n, c, oh*sh, ow*sw] is
+    // the tap (rh, rw) = (pad_h, pad_w) of this convolution's window, which the staged patch already holds at byte
+    // offset ds_off; wp2 is packed like wp with one tap ([o block][chunk][k-step][lane][16]); bias + requantise, no ReLU.
+    const int8_t* wp2;
+    const int32_t* bias2;
+    const float* mult2;
+    int8_t* y2;
+    uint32_t w2_bytes;
+    int32_t ds_off;
 };
 
 // Epilogue shared by the matrix-core kernels.  Accumulator register g of a 32x32 block is output channel
@@ -171,10 +181,13 @@ __device__ __forceinline__ void epilogue_c16(const intx16 (&acc)[RO], const QArg
 // (set-up, first loads, one weight fetch per k-step, epilogue), not by the matrix pipe, so a launch runs fastest
 // when all its waves are resident at once: larger per-wave tiles trade idle matrix cycles for fewer waves.
 // WD: depth of the weight ring in k-steps (must divide the k-steps of a chunk).
-template <int KH, int KW, int CBC, int WP, int RO, int PPT, int RP = 1, int WD = 0>
+// DS: the workgroup also produces the second output described in QArgs: per chunk (CBC + 1) / 2 more k-steps that read
+// the window's tap at ds_off against the second packed weights, into a second set of accumulators.
+template <int KH, int KW, int CBC, int WP, int RO, int PPT, int RP = 1, int WD = 0, bool DS = false>
 __global__ void __launch_bounds__(64 * WP) __attribute__((amdgpu_waves_per_eu(2))) qconv_mfma_kernel(const QArgs a) {
     constexpr int KHW = KH * KW;
     constexpr int NS = (KHW * CBC + 1) / 2;          // matrix k-steps per chunk
+    constexpr int NS2 = DS ? (CBC + 1) / 2 : 0;      // ... of the second output
     constexpr int TP = 32 * WP * RP;
 
     extern __shared__ __attribute__((aligned(16))) char lds[];
@@ -277,6 +290,17 @@ __global__ void __launch_bounds__(64 * WP) __attribute__((amdgpu_waves_per_eu(2)
         return __builtin_amdgcn_raw_buffer_load_b128(wr, wvoff[i] + (t < total_steps ? t * 1024u : kOob), 0, 0);
     };
     intx4 ring[D][RO];
+    // second output: its few weight fragments of a chunk are requested at the top of the chunk
+    const __amdgpu_buffer_rsrc_t wr2 = make_rsrc(DS ? a.wp2 : a.wp, DS ? a.w2_bytes : 0u);
+    intx16 acc2[DS ? RP : 1][DS ? RO : 1];
+    if constexpr (DS) {
+#pragma unroll
+        for (int j = 0; j < RP; ++j)
+#pragma unroll
+            for (int i = 0; i < RO; ++i)
+#pragma unroll
+                for (int g = 0; g < 16; ++g) acc2[j][i][g] = 0;
+    }
 
     issue_loads(0, buf0);
 #pragma unroll
@@ -288,6 +312,18 @@ __global__ void __launch_bounds__(64 * WP) __attribute__((amdgpu_waves_per_eu(2)
 
     for (int chunk = 0; chunk < a.nchunks; ++chunk) {
         const char* buf = (chunk & 1) ? buf1 : buf0;
+        intx4 a2[DS ? NS2 : 1][RO];
+        if constexpr (DS) {
+#pragma unroll
+            for (int s2 = 0; s2 < NS2; ++s2)
+#pragma unroll
+                for (int i = 0; i < RO; ++i)
+                    a2[s2][i] = __builtin_amdgcn_raw_buffer_load_b128(
+                        wr2, (static_cast<uint32_t>(ob0 + i) * static_cast<uint32_t>(a.nchunks) * NS2 + static_cast<uint32_t>(chunk) * NS2 + s2) * 1024u +
+                                 static_cast<uint32_t>(lane) * 16u, 0, 0);
+            __builtin_amdgcn_sched_barrier(0);
+            asm volatile("" ::: "memory");      // ahead of the next patch's loads in program order
+        }
         if (chunk + 1 < a.nchunks) issue_loads(chunk + 1, (chunk & 1) ? buf0 : buf1);
         auto tap_off = [&](int tap) {
             const int t = tap < KHW ? tap : KHW - 1;
@@ -323,6 +359,19 @@ __global__ void __launch_bounds__(64 * WP) __attribute__((amdgpu_waves_per_eu(2)
                 for (int j = 0; j < RP; ++j) bcur[j] = bnext[j];
             }
         }
+        if constexpr (DS) {
+            // lane half h takes channel block 2*s2 + h of the chunk at the second output's tap
+#pragma unroll
+            for (int s2 = 0; s2 < NS2; ++s2) {
+                const int off = a.ds_off + (CBC > 1 ? 2 * s2 * a.chs * 16 : 0);
+#pragma unroll
+                for (int j = 0; j < RP; ++j) {
+                    const intx4 b2 = *reinterpret_cast<const intx4*>(buf + xbase[j] + off);
+#pragma unroll
+                    for (int i = 0; i < RO; ++i) acc2[j][i] = __builtin_amdgcn_mfma_i32_32x32x32_i8(a2[s2][i], b2, acc2[j][i], 0, 0, 0);
+                }
+            }
+        }
         // every load older than the D*RO ring refills just issued has completed: that includes the next patch
         asm volatile("s_waitcnt vmcnt(%0)" ::"n"(D * RO) : "memory");
         __syncthreads();
@@ -331,6 +380,14 @@ __global__ void __launch_bounds__(64 * WP) __attribute__((amdgpu_waves_per_eu(2)
 #pragma unroll
     for (int j = 0; j < RP; ++j)
         if (ypix[j] >= 0) epilogue_c16<RO>(acc[j], a, ypix[j], ob0, half);
+    if constexpr (DS) {
+        QArgs second = a;
+        second.bias = a.bias2; second.mult = a.mult2; second.res = nullptr; second.y = a.y2;
+        second.flags = a.bias2 ? KXC_HIP_CONV_BIAS : 0u;
+#pragma unroll
+        for (int j = 0; j < RP; ++j)
+            if (ypix[j] >= 0) epilogue_c16<RO>(acc2[j], second, ypix[j], ob0, half);
+    }
 }
 
 // ------------------------------------------------------------------------------------------------
@@ -619,25 +676,29 @@ struct QVariant {
     const char* name;
     int kh, kw, cbc, wp, ro, ppt, rp;
     void (*kernel)(const QArgs);
+    void (*ds_kernel)(const QArgs);     // with the second output (nullptr: none)
 };
 
 #define KXC_QV(KH, KW, CBC, WP, RO, PPT)                                                             \
     { "qmfma_k" #KH "x" #KW "_cb" #CBC "_p" #WP "_o" #RO, KH, KW, CBC, WP, RO, PPT, 1,                   \
-      qconv_mfma_kernel<KH, KW, CBC, WP, RO, PPT> }
+      qconv_mfma_kernel<KH, KW, CBC, WP, RO, PPT>, nullptr }
+#define KXC_QV_DS(KH, KW, CBC, WP, RO, PPT)                                                          \
+    { "qmfma_k" #KH "x" #KW "_cb" #CBC "_p" #WP "_o" #RO, KH, KW, CBC, WP, RO, PPT, 1,                   \
+      qconv_mfma_kernel<KH, KW, CBC, WP, RO, PPT>, qconv_mfma_kernel<KH, KW, CBC, WP, RO, PPT, 1, 0, true> }
 // (RP pixel blocks per wave, weight ring of WD k-steps)
 #define KXC_QV2(KH, KW, CBC, WP, RO, PPT, RP, WD)                                                    \
     { "qmfma_k" #KH "x" #KW "_cb" #CBC "_p" #WP "x" #RP "_o" #RO "_d" #WD, KH, KW, CBC, WP, RO, PPT, RP,  \
-      qconv_mfma_kernel<KH, KW, CBC, WP, RO, PPT, RP, WD> }
+      qconv_mfma_kernel<KH, KW, CBC, WP, RO, PPT, RP, WD>, nullptr }
 
 const QVariant kQVariants[] = {
-    KXC_QV(3, 3, 2, 4, 2, 4),
-    KXC_QV(3, 3, 2, 4, 1, 4),
-    KXC_QV(3, 3, 2, 2, 1, 4),
+    KXC_QV_DS(3, 3, 2, 4, 2, 4),
+    KXC_QV_DS(3, 3, 2, 4, 1, 4),
+    KXC_QV_DS(3, 3, 2, 2, 1, 4),
     KXC_QV(1, 1, 4, 4, 2, 6),
     KXC_QV(1, 1, 4, 4, 1, 6),
     KXC_QV(1, 1, 4, 2, 1, 6),
-    KXC_QV(3, 3, 1, 4, 1, 4),      // at most 16 input channels: k-steps pair filter taps
-    KXC_QV(3, 3, 1, 2, 1, 4),
+    KXC_QV_DS(3, 3, 1, 4, 1, 4),      // at most 16 input channels: k-steps pair filter taps
+    KXC_QV_DS(3, 3, 1, 2, 1, 4),
     KXC_QV(1, 1, 1, 4, 1, 6),
     KXC_QV(1, 1, 1, 2, 1, 6),
     KXC_QV(7, 7, 1, 4, 2, 12),
@@ -839,6 +900,65 @@ int32_t kxc_hip_qconv2d_c16_i8(const kxc_hip_qconv2d_desc* d, const int8_t* x, c
                      "hipFuncSetAttribute");
     }
     hipLaunchKernelGGL(L.v->kernel, NoteGrid(dim3(L.grid)), NoteBlock(dim3(64 * L.v->wp)), NoteLds(L.lds_bytes), ResolveStream(stream), a);
+    return CheckLaunch(L.v->name);
+}
+
+// ---- two outputs from one launch: the convolution and a 1x1 convolution with the same strides, no padding
+int32_t kxc_hip_qconv2d_c16_pair_supported(const kxc_hip_qconv2d_desc* d) {
+    QLaunch L;
+    if (!d || d->pad_h >= d->kh || d->pad_w >= d->kw) return 0;
+    if (Prepare(d, &L, "kxc_hip_qconv2d_c16_pair_supported") != KXC_HIP_OK) { LastError().clear(); return 0; }
+    return (L.v && L.v->ds_kernel) ? 1 : 0;
+}
+
+int32_t kxc_hip_qconv2d_c16_pair_packed_bytes(const kxc_hip_qconv2d_desc* d, size_t* out_bytes) {
+    KXC_HIP_REQUIRE(d != nullptr && out_bytes != nullptr, "kxc_hip_qconv2d_c16_pair_packed_bytes: NULL argument");
+    KXC_HIP_REQUIRE(d->c > 0 && d->o > 0 && d->kh > 0 && d->kw > 0 && d->o % 32 == 0,
+                    "kxc_hip_qconv2d_c16_pair_packed_bytes: bad shape (output channels must be a multiple of 32)");
+    const int cbc = CbcFor(d->c, d->kh, d->kw);
+    const int64_t nchunks = ((d->c + 15) / 16 + cbc - 1) / cbc;
+    *out_bytes = static_cast<size_t>((d->o / 32) * nchunks * ((cbc + 1) / 2) * 1024);
+    return KXC_HIP_OK;
+}
+
+// w2_oihw: [o, c, 1, 1] int8; packed in the chunking of the convolution `d` describes
+int32_t kxc_hip_qconv2d_c16_pair_pack_weights(const kxc_hip_qconv2d_desc* d, const int8_t* w2_oihw, int8_t* packed, void* stream) {
+    size_t bytes = 0;
+    if (int32_t rc = kxc_hip_qconv2d_c16_pair_packed_bytes(d, &bytes)) return rc;
+    KXC_HIP_REQUIRE(w2_oihw && packed, "kxc_hip_qconv2d_c16_pair_pack_weights: NULL pointer");
+    PackArgs p;
+    p.w = w2_oihw; p.wp = packed; p.O = d->o; p.C = d->c; p.KHW = 1;
+    p.CBC = CbcFor(d->c, d->kh, d->kw);
+    p.NS = (p.CBC + 1) / 2;
+    p.nchunks = ((d->c + 15) / 16 + p.CBC - 1) / p.CBC;
+    p.oblocks = d->o / 32;
+    const int64_t slots = static_cast<int64_t>(bytes / 16);
+    pack_weights_kernel<<<NoteGrid(static_cast<int>(CeilDiv(slots, kBlock))), NoteBlock(kBlock), NoteLds(0), ResolveStream(stream)>>>(p, slots);
+    return CheckLaunch("qconv2d_c16_pair_pack_weights");
+}
+
+int32_t kxc_hip_qconv2d_c16_pair_i8(const kxc_hip_qconv2d_desc* d, const int8_t* x, const int8_t* w_packed, const int32_t* bias,
+                                    const float* mult, const int8_t* residual, int8_t* y, const int8_t* w2_packed,
+                                    const int32_t* bias2, const float* mult2, int8_t* y2, void* stream) {
+    const char* who = "kxc_hip_qconv2d_c16_pair_i8";
+    QLaunch L;
+    if (int32_t rc = Prepare(d, &L, who)) return rc;
+    KXC_HIP_REQUIRE(L.v && L.v->ds_kernel && d->pad_h < d->kh && d->pad_w < d->kw, "%s: no kernel with a second output covers this shape", who);
+    if (L.args.M == 0) return KXC_HIP_OK;
+    KXC_HIP_REQUIRE(x && w_packed && mult && y && w2_packed && mult2 && y2, "%s: NULL pointer", who);
+    KXC_HIP_REQUIRE(!(d->flags & KXC_HIP_CONV_BIAS) || bias, "%s: bias flag without bias", who);
+    KXC_HIP_REQUIRE(!(d->flags & KXC_HIP_CONV_RESIDUAL) || residual, "%s: residual flag without residual", who);
+    QArgs& a = L.args;
+    a.x = x; a.wp = w_packed; a.bias = bias; a.mult = mult; a.res = residual; a.y = y;
+    a.wp2 = w2_packed; a.bias2 = bias2; a.mult2 = mult2; a.y2 = y2;
+    a.w2_bytes = static_cast<uint32_t>(static_cast<int64_t>(a.O / 32) * a.nchunks * ((L.v->cbc + 1) / 2) * 1024);
+    a.ds_off = (d->pad_h * a.Wp + d->pad_w) * 16;
+    if (L.lds_bytes > 64 * 1024) {
+        KXC_HIP_CALL(hipFuncSetAttribute(reinterpret_cast<const void*>(L.v->ds_kernel),
+                                         hipFuncAttributeMaxDynamicSharedMemorySize, static_cast<int>(L.lds_bytes)),
+                     "hipFuncSetAttribute");
+    }
+    hipLaunchKernelGGL(L.v->ds_kernel, NoteGrid(dim3(L.grid)), NoteBlock(dim3(64 * L.v->wp)), NoteLds(L.lds_bytes), ResolveStream(stream), a);
     return CheckLaunch(L.v->name);
 }
 

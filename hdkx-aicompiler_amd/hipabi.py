@@ -463,6 +463,44 @@ def qconv2d_c16(x, c, w_packed, w_shape, bias, mult, residual=None, res_mult=0.0
     return y
 
 
+def qconv2d_c16_pair_supported(n, c, h, w, o, k, stride, pad):
+    d = qconv_desc(n, c, h, w, o, k, k, stride, pad, 0)
+    return bool(lib().kxc_hip_qconv2d_c16_pair_supported(C.byref(d)))
+
+
+def qconv2d_c16_pair_pack_weights(w2, k):
+    """[o, c, 1, 1] int8 weights (GPU) of the second output -> packed in the chunking of the k x k convolution."""
+    import torch
+    _need(w2, torch.int8, "w2")
+    o, c = w2.shape[0], w2.shape[1]
+    d = qconv_desc(1, c, k, k, o, k, k, 1, 0)
+    nbytes = C.c_size_t()
+    _check(lib().kxc_hip_qconv2d_c16_pair_packed_bytes(C.byref(d), C.byref(nbytes)))
+    packed = torch.empty((nbytes.value,), dtype=torch.int8, device=w2.device)
+    _check(lib().kxc_hip_qconv2d_c16_pair_pack_weights(C.byref(d), _p(w2), _p(packed), _stream()))
+    return packed
+
+
+def qconv2d_c16_pair(x, c, w_packed, w_shape, bias, mult, w2_packed, bias2, mult2, residual=None, res_mult=0.0, stride=1,
+                     pad=0, relu=True):
+    """(qconv2d_c16(x, w ...), the 1x1 convolution with the same strides and no padding, bias2 + requantise) in one launch."""
+    import torch
+    _need(x, torch.int8, "x"); _need(w_packed, torch.int8, "w_packed"); _need(bias, torch.int32, "bias")
+    _need(mult, torch.float32, "mult"); _need(residual, torch.int8, "residual")
+    _need(w2_packed, torch.int8, "w2_packed"); _need(bias2, torch.int32, "bias2"); _need(mult2, torch.float32, "mult2")
+    n, cb, h, wd, _ = x.shape
+    o, _, kh, kw = w_shape
+    flags = (CONV_BIAS if bias is not None else 0) | (CONV_RESIDUAL if residual is not None else 0) | \
+            (CONV_RELU if relu else 0)
+    d = qconv_desc(n, c, h, wd, o, kh, kw, stride, pad, flags, res_mult)
+    oh = (h + 2 * pad - kh) // stride + 1; ow = (wd + 2 * pad - kw) // stride + 1
+    y = torch.empty(c16_shape(n, o, oh, ow), dtype=torch.int8, device=x.device)
+    y2 = torch.empty_like(y)
+    _check(lib().kxc_hip_qconv2d_c16_pair_i8(C.byref(d), _p(x), _p(w_packed), _p(bias), _p(mult), _p(residual), _p(y),
+                                             _p(w2_packed), _p(bias2), _p(mult2), _p(y2), _stream()))
+    return y, y2
+
+
 def quantize_to_c4(x, scale):
     """fp32 NCHW (at most 4 channels) -> int8 [N][H][W][4]."""
     import torch
@@ -592,6 +630,10 @@ class Plan:
 
     def add_qconv2d_c16(self, desc, x, w_packed, bias, mult, residual, y):
         _check(lib().kxc_hip_plan_add_qconv2d_c16(self._h, C.byref(desc), x, w_packed, bias, mult, residual, y))
+
+    def add_qconv2d_c16_pair(self, desc, x, w_packed, bias, mult, residual, y, w2_packed, bias2, mult2, y2):
+        _check(lib().kxc_hip_plan_add_qconv2d_c16_pair(self._h, C.byref(desc), x, w_packed, bias, mult, residual, y,
+                                                       w2_packed, bias2, mult2, y2))
 
     def add_qconv2d_c4(self, desc, x, w_packed, bias, mult, y):
         _check(lib().kxc_hip_plan_add_qconv2d_c4(self._h, C.byref(desc), x, w_packed, bias, mult, y))

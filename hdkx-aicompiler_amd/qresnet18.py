@@ -13,6 +13,8 @@ Activations live in the channel-blocked c16 layout between layers; the input is 
 
 Host-side preparation (numpy) happens once per model; the per-batch work is one launch plan.
 """
+import os
+
 import numpy as np
 
 from . import hipabi as H
@@ -161,6 +163,31 @@ class QuantizedResNet18:
                                  residual["buf"] if residual is not None else Buf.none(), y["buf"])
             return y
 
+        def conv_pair(x, name, down_name):
+            # a block's first 3x3/2 convolution and its 1x1/2 downsample in one launch (two outputs); the
+            # downsample's weights are re-packed in the chunking of the 3x3 kernel
+            i, L = by_name[name]
+            j, D = by_name[down_name]
+            n, c, h, w = x["shape"]
+            d = H.qconv_desc(n, c, h, w, L["cout"], L["k"], L["k"], L["stride"], L["pad"], CONV_BIAS | CONV_RELU, 0.0)
+            oh = (h + 2 * L["pad"] - L["k"]) // L["stride"] + 1
+            ow = (w + 2 * L["pad"] - L["k"]) // L["stride"] + 1
+            self.consts[3 * j] = H.qconv2d_c16_pair_pack_weights(dev(D["wq"]), L["k"])
+            y = new_act(n, L["cout"], oh, ow)
+            y2 = new_act(n, L["cout"], oh, ow)
+            plan.add_qconv2d_c16_pair(d, x["buf"], arg(1 + 3 * i), arg(2 + 3 * i), arg(3 + 3 * i), Buf.none(), y["buf"],
+                                      arg(1 + 3 * j), arg(2 + 3 * j), arg(3 + 3 * j), y2["buf"])
+            return y, y2
+
+        def can_pair(x, name, down_name):
+            if os.environ.get("KXC_HIP_QPAIR", "1") == "0":
+                return False
+            _, L = by_name[name]
+            _, D = by_name[down_name]
+            n, c, h, w = x["shape"]
+            return (D["k"] == 1 and D["pad"] == 0 and D["stride"] == L["stride"] and D["cout"] == L["cout"] and not D["relu"]
+                    and H.qconv2d_c16_pair_supported(n, c, h, w, L["cout"], L["k"], L["stride"], L["pad"]))
+
         if self.first_c4:
             L0 = model["layers"][0]
             off, size = arena.alloc(batch * hw * hw * 4)
@@ -185,8 +212,11 @@ class QuantizedResNet18:
             for blk in range(2):
                 first = blk == 0 and stage > 0
                 name = "l%d.%d" % (stage + 1, blk)
-                a = conv(cur, name + ".conv1")
-                idn = conv(cur, name + ".down") if first else cur
+                if first and can_pair(cur, name + ".conv1", name + ".down"):
+                    a, idn = conv_pair(cur, name + ".conv1", name + ".down")
+                else:
+                    a = conv(cur, name + ".conv1")
+                    idn = conv(cur, name + ".down") if first else cur
                 out = conv(a, name + ".conv2", residual=idn)
                 free_act(a)
                 if first:

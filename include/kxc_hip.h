@@ -280,6 +280,19 @@ const char* kxc_hip_qconv2d_c16_variant(const kxc_hip_qconv2d_desc* desc);
 int32_t kxc_hip_qconv2d_c16_i8(const kxc_hip_qconv2d_desc* desc, const int8_t* x, const int8_t* w_packed,
                                const int32_t* bias, const float* mult, const int8_t* residual, int8_t* y,
                                void* stream);
+/* Two outputs from one launch (a residual block's first 3x3/2 convolution and its 1x1/2 downsample): y as above, and
+ * y2[n,o,oh,ow] = requantise(sum_c x[n,c,oh*stride,ow*stride] * w2[o,c] + bias2[o], mult2[o]) without ReLU -- the 1x1
+ * convolution with the same strides and no padding, whose operand is the tap (pad_h, pad_w) of the first one's window
+ * (needs pad < filter size).  w2_packed comes from kxc_hip_qconv2d_c16_pair_pack_weights (w2 is [o,c,1,1], packed in
+ * the chunking of `desc`); bias2 may be NULL.  Bit-identical to the two separate launches. */
+int32_t kxc_hip_qconv2d_c16_pair_supported(const kxc_hip_qconv2d_desc* desc);
+int32_t kxc_hip_qconv2d_c16_pair_packed_bytes(const kxc_hip_qconv2d_desc* desc, size_t* out_bytes);
+int32_t kxc_hip_qconv2d_c16_pair_pack_weights(const kxc_hip_qconv2d_desc* desc, const int8_t* w2_oihw, int8_t* packed,
+                                              void* stream);
+int32_t kxc_hip_qconv2d_c16_pair_i8(const kxc_hip_qconv2d_desc* desc, const int8_t* x, const int8_t* w_packed,
+                                    const int32_t* bias, const float* mult, const int8_t* residual, int8_t* y,
+                                    const int8_t* w2_packed, const int32_t* bias2, const float* mult2, int8_t* y2,
+                                    void* stream);
 /* Layout converters and the quantising converter (fp32 NCHW -> int8 c16, same rounding as kxc_hip_quantize_f32_i8). */
 int32_t kxc_hip_i8_nchw_to_c16(const int8_t* x, int8_t* y, int64_t n, int64_t c, int64_t hw, void* stream);
 int32_t kxc_hip_i8_c16_to_nchw(const int8_t* x, int8_t* y, int64_t n, int64_t c, int64_t hw, void* stream);
@@ -387,6 +400,11 @@ int32_t kxc_hip_plan_add_global_avg_pool2d_i8(kxc_hip_plan* plan, int64_t n, int
 int32_t kxc_hip_plan_add_qconv2d_c16(kxc_hip_plan* plan, const kxc_hip_qconv2d_desc* desc, kxc_hip_buf x,
                                      kxc_hip_buf w_packed, kxc_hip_buf bias, kxc_hip_buf mult,
                                      kxc_hip_buf residual, kxc_hip_buf y);
+/* The c16 convolution with the second output of kxc_hip_qconv2d_c16_pair_i8 as one node. */
+int32_t kxc_hip_plan_add_qconv2d_c16_pair(kxc_hip_plan* plan, const kxc_hip_qconv2d_desc* desc, kxc_hip_buf x,
+                                          kxc_hip_buf w_packed, kxc_hip_buf bias, kxc_hip_buf mult,
+                                          kxc_hip_buf residual, kxc_hip_buf y, kxc_hip_buf w2_packed,
+                                          kxc_hip_buf bias2, kxc_hip_buf mult2, kxc_hip_buf y2);
 int32_t kxc_hip_plan_add_qconv2d_c4(kxc_hip_plan* plan, const kxc_hip_qconv2d_desc* desc, kxc_hip_buf x_c4,
                                     kxc_hip_buf w_packed, kxc_hip_buf bias, kxc_hip_buf mult, kxc_hip_buf y_c16);
 int32_t kxc_hip_plan_add_quantize_c4(kxc_hip_plan* plan, int64_t n, int64_t c, int64_t hw, float scale,

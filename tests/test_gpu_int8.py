@@ -97,6 +97,44 @@ def test_qconv_c16_against_cpu(pkg, orc, shape, residual):
     assert len(np.unique(want)) > 20
 
 
+QPAIR_SHAPES = [
+    # n, c, h, w, o, stride: the three ResNet-18 blocks, a ragged shape with a partial channel block and an odd block count
+    (2, 64, 56, 56, 128, 2), (64, 64, 56, 56, 128, 2), (3, 128, 28, 28, 256, 2), (5, 256, 14, 14, 512, 2),
+    (2, 40, 13, 17, 64, 2), (1, 10, 9, 9, 32, 2), (2, 48, 12, 10, 96, 1),
+]
+
+
+@pytest.mark.parametrize("shape", QPAIR_SHAPES, ids=lambda s: "x".join(map(str, s)))
+def test_qconv_c16_pair_against_cpu(pkg, orc, shape):
+    """A 3x3 convolution (bias, ReLU) and the 1x1 convolution with the same strides and no padding (bias, no ReLU)
+    from one launch: both outputs bit-exact against the CPU int8 operators and against the two separate launches."""
+    n, c, h, w, o, s = shape
+    rng = np.random.default_rng(hash(shape) % (2 ** 31))
+    x = rng.integers(-128, 128, (n, c, h, w), dtype=np.int8)
+    wq = rng.integers(-127, 128, (o, c, 3, 3), dtype=np.int8)
+    w2 = rng.integers(-127, 128, (o, c, 1, 1), dtype=np.int8)
+    bias = rng.integers(-20000, 20000, (o,), dtype=np.int32)
+    bias2 = rng.integers(-2000, 2000, (o,), dtype=np.int32)
+    mult = rng.uniform(0.5, 2.0, (o,)).astype(np.float32) * np.float32(1.0 / (8.0 * np.sqrt(c * 9) * 64))
+    mult2 = rng.uniform(0.5, 2.0, (o,)).astype(np.float32) * np.float32(1.0 / (8.0 * np.sqrt(c) * 64))
+    assert pkg.qconv2d_c16_pair_supported(n, c, h, w, o, 3, s, 1)
+    xc = to_c16(pkg, x)
+    packed = pkg.qconv2d_c16_pack_weights(dev(wq))
+    packed2 = pkg.qconv2d_c16_pair_pack_weights(dev(w2), 3)
+    y, y2 = pkg.qconv2d_c16_pair(xc, c, packed, wq.shape, dev(bias), dev(mult), packed2, dev(bias2), dev(mult2), None, 0.0, s, 1, True)
+    if n <= 8:
+        assert_bit_exact(from_c16(pkg, y, o), orc.qconv(x, wq, bias, mult, s, 1, None, 0.0, True), "pair, main output %s" % (shape,))
+        want2 = orc.qconv(x, w2, bias2, mult2, s, 0, None, 0.0, False)
+        assert_bit_exact(from_c16(pkg, y2, o), want2, "pair, second output %s" % (shape,))
+        assert len(np.unique(want2)) > 20
+    alone = pkg.qconv2d_c16(xc, c, packed, wq.shape, dev(bias), dev(mult), None, 0.0, s, 1, True)
+    alone2 = pkg.qconv2d_c16(xc, c, pkg.qconv2d_c16_pack_weights(dev(w2)), w2.shape, dev(bias2), dev(mult2), None, 0.0, s, 0, False)
+    assert torch.equal(y, alone) and torch.equal(y2, alone2)
+    # no bias on the second output
+    _, y2n = pkg.qconv2d_c16_pair(xc, c, packed, wq.shape, dev(bias), dev(mult), packed2, None, dev(mult2), None, 0.0, s, 1, True)
+    assert torch.equal(y2n, pkg.qconv2d_c16(xc, c, pkg.qconv2d_c16_pack_weights(dev(w2)), w2.shape, None, dev(mult2), None, 0.0, s, 0, False))
+
+
 @pytest.mark.parametrize("shape", [(2, 3, 224, 224, 64), (1, 3, 64, 64, 64), (3, 4, 20, 36, 32), (2, 1, 9, 8, 96)],
                          ids=lambda s: "x".join(map(str, s)))
 def test_qconv_first_layer_c4_against_cpu(pkg, orc, shape):
@@ -213,7 +251,9 @@ def test_qresnet18_small_every_layer(pkg, orc):
     assert_bit_exact(host(out), want_logits, "quantised logits (plan)")
     # the quantisation must be meaningful: logits close to the fp32 network's in the large
     assert np.isfinite(want_logits).all() and np.abs(want_logits).max() > 0
-    assert len(net.launches) == 24 and net.launches[1].startswith("kxc_qconv2d_c4_i8:qmfma")
+    # 24 operators, 21 launches: the three downsamples are second outputs of their block's first convolution
+    assert len(net.launches) == 21 and net.launches[1].startswith("kxc_qconv2d_c4_i8:qmfma")
+    assert sum("|qconv1x1+bias" in s for s in net.launches) == 3
     assert net.launches[3].startswith("kxc_qconv2d_c16_i8:qmfma")
 
 
