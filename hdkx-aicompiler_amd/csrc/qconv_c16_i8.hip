@@ -94,81 +94,110 @@ struct QArgs {
     int32_t ds_off;
 };
 
-// Epilogue shared by the matrix-core kernels.  Accumulator register g of a 32x32 block is output channel
-// 8*(g/4) + 4*half + g%4 (within the block of 32) at the lane's pixel: registers 4j..4j+3 are four
-// consecutive channels = one dword of the pixel's c16 word.  ypix = n*(O/16)*OHW + pixel index.
+typedef unsigned int uintx2 __attribute__((ext_vector_type(2)));
+typedef unsigned int uintx4 __attribute__((ext_vector_type(4)));
+
+// v_permlane32_swap: a's lanes 32-63 change places with b's lanes 0-31 (gfx950).  The host pass of the compiler
+// does not know the instruction and sees an empty body.
+__device__ __forceinline__ void swap_halves(uint32_t& a, uint32_t& b) {
+#if defined(__HIP_DEVICE_COMPILE__)
+    const uintx2 r = __builtin_amdgcn_permlane32_swap(a, b, false, false);
+    a = r[0]; b = r[1];
+#endif
+}
+
+// Accumulator register g of a 32x32 block is output channel 8*(g/4) + 4*half + g%4 (within the block of 32) at the
+// lane's pixel: registers 4j..4j+3 ("group j") are four consecutive channels = one dword of the pixel's c16 word.
+// The accumulators START at the bias (int32 addition wraps the same way in any order), so the epilogue has no add.
 template <int RO>
-__device__ __forceinline__ void epilogue_c16(const intx16 (&acc)[RO], const QArgs& a, int ypix, int ob0, int half) {
-    const bool has_bias = (a.flags & KXC_HIP_CONV_BIAS) != 0;
-    const bool has_res = (a.flags & KXC_HIP_CONV_RESIDUAL) != 0;
-    const bool do_relu = (a.flags & KXC_HIP_CONV_RELU) != 0;
-    // All loads (residual word, 4 multipliers, 4 biases per group of 4 channels) are issued before the first store:
-    // a wait for a load also waits for every store issued before it, so interleaving them would cost one memory
-    // round trip per group.  Absent channel groups load group 0 and store nothing.
-    auto group = [&](int i, int j) { return (ob0 + i) * 32 + 8 * j + 4 * half; };       // first of 4 consecutive channels
-    auto offset = [&](int o) { return (static_cast<int64_t>(ypix) + static_cast<int64_t>(o >> 4) * a.OHW) * 16 + (o & 15); };
-    uint32_t resw[RO][4];
-    float4 mv[RO][4];
-    int4 bv[RO][4];
+__device__ __forceinline__ void init_acc_with_bias(intx16 (&acc)[RO], const int32_t* bias, bool has_bias, int32_t O, int ob0, int half) {
 #pragma unroll
     for (int i = 0; i < RO; ++i)
 #pragma unroll
         for (int j = 0; j < 4; ++j) {
-            const int o = group(i, j), oc = o < a.O ? o : 0;
-            mv[i][j] = *reinterpret_cast<const float4*>(a.mult + oc);
-            bv[i][j] = make_int4(0, 0, 0, 0);
-            resw[i][j] = 0;
+            const int o = (ob0 + i) * 32 + 8 * j + 4 * half;
+            int4 b = make_int4(0, 0, 0, 0);
+            if (has_bias) b = *reinterpret_cast<const int4*>(bias + (o < O ? o : 0));
+            acc[i][4 * j + 0] = b.x; acc[i][4 * j + 1] = b.y; acc[i][4 * j + 2] = b.z; acc[i][4 * j + 3] = b.w;
         }
-    if (has_bias) {
+}
+
+// Epilogue shared by the matrix-core kernels: requantise RP x RO blocks whose accumulators already hold the bias.
+// These kernels are bound by instruction issue around the (very fast) int8 matrix instructions, so it is kept short:
+//  * rounding and conversion are one addition: v + 1.5*2^23 rounds v to an integer (ties to even) and leaves its two's
+//    complement in the low mantissa bits, so after the clamp (one median instruction; with ReLU its lower bound 0 is
+//    also what a NaN maps to, without ReLU a NaN is replaced by 0 first) the low byte of the sum IS the int8 result;
+//  * four results are packed with three byte permutes, and two lane-half swaps per block turn the four packed dwords
+//    of a lane (channel groups 0, 2, 4, 6 or 1, 3, 5, 7 of the block) into the 16 consecutive channels of one c16
+//    word: lane r stores channels 0-15 and lane r + 32 channels 16-31 of pixel r with ONE 16-byte store each (and
+//    reads the residual with one 16-byte load) instead of four 4-byte ones;
+//  * the multipliers are loaded once for all pixel blocks of the wave, and every load is issued before the first
+//    store (a wait for a load also waits for every store issued before it).
+// ypix[j] = n*(O/16)*OHW + pixel index of the lane's pixel in block j, or -1 past the end.
+template <int RO, int RP>
+__device__ __forceinline__ void epilogue_c16(const intx16 (&acc)[RP][RO], const QArgs& a, const int (&ypix)[RP], int ob0, int half) {
+    const bool has_res = (a.flags & KXC_HIP_CONV_RESIDUAL) != 0;
+    const bool do_relu = (a.flags & KXC_HIP_CONV_RELU) != 0;
+    // this lane's c16 word of block (i, j): channels (ob0 + i)*32 + 16*half .. + 15
+    auto word = [&](int i, int j) {
+        return (static_cast<int64_t>(ypix[j]) + static_cast<int64_t>((ob0 + i) * 2 + half) * a.OHW) * 16;
+    };
+    float4 mv[RO][4];
 #pragma unroll
-        for (int i = 0; i < RO; ++i)
+    for (int i = 0; i < RO; ++i)
 #pragma unroll
-            for (int j = 0; j < 4; ++j) {
-                const int o = group(i, j);
-                bv[i][j] = *reinterpret_cast<const int4*>(a.bias + (o < a.O ? o : 0));
-            }
-    }
+        for (int j = 0; j < 4; ++j) {
+            const int o = (ob0 + i) * 32 + 8 * j + 4 * half;
+            mv[i][j] = *reinterpret_cast<const float4*>(a.mult + (o < a.O ? o : 0));
+        }
+    // residual words, brought from "16 consecutive channels per lane" to the accumulators' channel groups
+    uint32_t resw[RP][RO][4];
     if (has_res) {
 #pragma unroll
-        for (int i = 0; i < RO; ++i)
+        for (int j = 0; j < RP; ++j)
 #pragma unroll
-            for (int j = 0; j < 4; ++j) {
-                const int o = group(i, j);
-                resw[i][j] = *reinterpret_cast<const uint32_t*>(a.res + offset(o < a.O ? o : 0));
+            for (int i = 0; i < RO; ++i) {
+                uintx4 q = {0u, 0u, 0u, 0u};
+                if (ypix[j] >= 0) q = *reinterpret_cast<const uintx4*>(a.res + word(i, j));
+                uint32_t q0 = q[0], q1 = q[1], q2 = q[2], q3 = q[3];
+                swap_halves(q0, q1);      // (the inverse of the stores' swaps below)
+                swap_halves(q2, q3);
+                resw[j][i][0] = q0; resw[j][i][2] = q1; resw[j][i][1] = q2; resw[j][i][3] = q3;
             }
     }
-    // These kernels are bound by instruction issue around the (very fast) int8 matrix instructions, so the
-    // requantisation is kept short: the ReLU form needs no NaN select (the clamp's lower bound 0 is also what a NaN
-    // maps to: a median-of-three with a NaN operand returns the smaller of the other two), the clamp is one
-    // median instruction, and four results are packed with three byte permutes.
     auto finish = [&](auto relu_c, auto res_c) {
         constexpr bool kRelu = decltype(relu_c)::value, kRes = decltype(res_c)::value;
+        constexpr float kMagic = 12582912.0f;      // 1.5 * 2^23
 #pragma unroll
-        for (int i = 0; i < RO; ++i) {
+        for (int j = 0; j < RP; ++j)
 #pragma unroll
-            for (int j = 0; j < 4; ++j) {
-                const int o = group(i, j);
-                const float ms[4] = {mv[i][j].x, mv[i][j].y, mv[i][j].z, mv[i][j].w};
-                const int bs[4] = {bv[i][j].x, bv[i][j].y, bv[i][j].z, bv[i][j].w};
-                int32_t q[4];
+            for (int i = 0; i < RO; ++i) {
+                uint32_t w[4];
 #pragma unroll
-                for (int e = 0; e < 4; ++e) {
-                    float v = __fmul_rn(static_cast<float>(acc[i][4 * j + e] + bs[e]), ms[e]);
-                    if (kRes) {
-                        const int32_t rq = static_cast<int32_t>(static_cast<int8_t>((resw[i][j] >> (8 * e)) & 0xff));
-                        v = __fadd_rn(v, __fmul_rn(static_cast<float>(rq), a.res_mult));
+                for (int gq = 0; gq < 4; ++gq) {
+                    const float ms[4] = {mv[i][gq].x, mv[i][gq].y, mv[i][gq].z, mv[i][gq].w};
+                    uint32_t t[4];
+#pragma unroll
+                    for (int e = 0; e < 4; ++e) {
+                        float v = __fmul_rn(static_cast<float>(acc[j][i][4 * gq + e]), ms[e]);
+                        if (kRes) {
+                            const int32_t rq = static_cast<int32_t>(static_cast<int8_t>((resw[j][i][gq] >> (8 * e)) & 0xff));
+                            v = __fadd_rn(v, __fmul_rn(static_cast<float>(rq), a.res_mult));
+                        }
+                        if (!kRelu) v = (v == v) ? v : 0.0f;
+                        v = __builtin_amdgcn_fmed3f(v, kRelu ? 0.0f : -128.0f, 127.0f);
+                        t[e] = __builtin_bit_cast(uint32_t, __fadd_rn(v, kMagic));
                     }
-                    float r = rintf(v);
-                    if (!kRelu) r = (v == v) ? r : 0.0f;
-                    r = __builtin_amdgcn_fmed3f(r, kRelu ? 0.0f : -128.0f, 127.0f);
-                    q[e] = static_cast<int32_t>(r);
+                    const uint32_t lo = __builtin_amdgcn_perm(t[1], t[0], 0x0c0c0400u);
+                    const uint32_t hi = __builtin_amdgcn_perm(t[3], t[2], 0x0c0c0400u);
+                    w[gq] = __builtin_amdgcn_perm(hi, lo, 0x05040100u);
                 }
-                const uint32_t lo = __builtin_amdgcn_perm(static_cast<uint32_t>(q[1]), static_cast<uint32_t>(q[0]), 0x0c0c0400u);
-                const uint32_t hi = __builtin_amdgcn_perm(static_cast<uint32_t>(q[3]), static_cast<uint32_t>(q[2]), 0x0c0c0400u);
-                const uint32_t outw = __builtin_amdgcn_perm(hi, lo, 0x05040100u);
-                if (o < a.O) *reinterpret_cast<uint32_t*>(a.y + offset(o)) = outw;
+                // lane half 0 holds channel groups 0, 2, 4, 6 (channels 0-3, 8-11, 16-19, 24-27), half 1 the odd ones:
+                // after the swaps half 0 has channels 0-15 as (w0, w2, w1, w3) and half 1 channels 16-31 likewise
+                swap_halves(w[0], w[2]);
+                swap_halves(w[1], w[3]);
+                if (ypix[j] >= 0) *reinterpret_cast<uintx4*>(a.y + word(i, j)) = uintx4{w[0], w[2], w[1], w[3]};
             }
-        }
     };
     using T = std::true_type;
     using F = std::false_type;
@@ -251,11 +280,7 @@ __global__ void __launch_bounds__(64 * WP) __attribute__((amdgpu_waves_per_eu(2)
 
     intx16 acc[RP][RO];
 #pragma unroll
-    for (int j = 0; j < RP; ++j)
-#pragma unroll
-        for (int i = 0; i < RO; ++i)
-#pragma unroll
-            for (int g = 0; g < 16; ++g) acc[j][i][g] = 0;
+    for (int j = 0; j < RP; ++j) init_acc_with_bias<RO>(acc[j], a.bias, (a.flags & KXC_HIP_CONV_BIAS) != 0, a.O, ob0, half);
 
     auto issue_loads = [&](int chunk, char* buf) {
 #pragma unroll
@@ -295,11 +320,7 @@ __global__ void __launch_bounds__(64 * WP) __attribute__((amdgpu_waves_per_eu(2)
     intx16 acc2[DS ? RP : 1][DS ? RO : 1];
     if constexpr (DS) {
 #pragma unroll
-        for (int j = 0; j < RP; ++j)
-#pragma unroll
-            for (int i = 0; i < RO; ++i)
-#pragma unroll
-                for (int g = 0; g < 16; ++g) acc2[j][i][g] = 0;
+        for (int j = 0; j < RP; ++j) init_acc_with_bias<RO>(acc2[j], a.bias2, a.bias2 != nullptr, a.O, ob0, half);
     }
 
     issue_loads(0, buf0);
@@ -377,16 +398,12 @@ __global__ void __launch_bounds__(64 * WP) __attribute__((amdgpu_waves_per_eu(2)
         __syncthreads();
     }
 
-#pragma unroll
-    for (int j = 0; j < RP; ++j)
-        if (ypix[j] >= 0) epilogue_c16<RO>(acc[j], a, ypix[j], ob0, half);
+    epilogue_c16<RO, RP>(acc, a, ypix, ob0, half);
     if constexpr (DS) {
         QArgs second = a;
-        second.bias = a.bias2; second.mult = a.mult2; second.res = nullptr; second.y = a.y2;
-        second.flags = a.bias2 ? KXC_HIP_CONV_BIAS : 0u;
-#pragma unroll
-        for (int j = 0; j < RP; ++j)
-            if (ypix[j] >= 0) epilogue_c16<RO>(acc2[j], second, ypix[j], ob0, half);
+        second.mult = a.mult2; second.res = nullptr; second.y = a.y2;
+        second.flags = 0u;      // (its bias is in the accumulators already; no residual, no ReLU)
+        epilogue_c16<RO, RP>(acc2, second, ypix, ob0, half);
     }
 }
 
@@ -453,19 +470,17 @@ __global__ void __launch_bounds__(64 * WP) __attribute__((amdgpu_waves_per_eu(2)
         }
     }
     const int m = m0 + wave * 32 + r;
-    int xbase, ypix;
+    int xbase;
+    int ypix[1];
     {
         const int mc = min(m, a.M - 1);
         const int n = fast_div(mc, a.div_ohw), rem = mc - n * a.OHW;
         const int oh = fast_div(rem, a.div_ow), ow = rem - oh * a.OW;
         xbase = (n * a.Hp + oh * 2 - qmin) * W4 * 16 + ow * 8 + half * 16;
-        ypix = (m < a.M) ? n * (a.O >> 4) * a.OHW + rem : -1;
+        ypix[0] = (m < a.M) ? n * (a.O >> 4) * a.OHW + rem : -1;
     }
-    intx16 acc[RO];
-#pragma unroll
-    for (int i = 0; i < RO; ++i)
-#pragma unroll
-        for (int g = 0; g < 16; ++g) acc[i][g] = 0;
+    intx16 acc[1][RO];
+    init_acc_with_bias<RO>(acc[0], a.bias, (a.flags & KXC_HIP_CONV_BIAS) != 0, a.O, ob0, half);
     asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
     __syncthreads();
     const char* ws = lds + xs_bytes + lane * 16;
@@ -478,11 +493,10 @@ __global__ void __launch_bounds__(64 * WP) __attribute__((amdgpu_waves_per_eu(2)
 #pragma unroll
         for (int i = 0; i < RO; ++i) {
             const intx4 wv = *reinterpret_cast<const intx4*>(ws + (i * KH + kh) * 1024);
-            acc[i] = __builtin_amdgcn_mfma_i32_32x32x32_i8(wv, b, acc[i], 0, 0, 0);
+            acc[0][i] = __builtin_amdgcn_mfma_i32_32x32x32_i8(wv, b, acc[0][i], 0, 0, 0);
         }
     }
-    if (ypix < 0) return;
-    epilogue_c16<RO>(acc, a, ypix, ob0, half);
+    epilogue_c16<RO, 1>(acc, a, ypix, ob0, half);
 }
 
 // Weights of the first-layer kernel: [o block][kh][lane][16]; lane (o, half), byte j = pixel j/4, channel j%4,
