@@ -311,8 +311,11 @@ __global__ void __launch_bounds__(64 * WP) __attribute__((amdgpu_waves_per_eu(2)
     uint32_t wvoff[RO];
 #pragma unroll
     for (int i = 0; i < RO; ++i) wvoff[i] = static_cast<uint32_t>(ob0 + i) * total_steps * 1024u + static_cast<uint32_t>(lane) * 16u;
+    // (the step index is uniform: it goes into the instruction's scalar offset, clamped to the last step -- a ring
+    // entry past the end is never used -- which costs two scalar instructions per load and no vector one)
     auto load_a = [&](int i, uint32_t t) -> intx4 {
-        return __builtin_amdgcn_raw_buffer_load_b128(wr, wvoff[i] + (t < total_steps ? t * 1024u : kOob), 0, 0);
+        const uint32_t tc = t < total_steps ? t : total_steps - 1u;
+        return __builtin_amdgcn_raw_buffer_load_b128(wr, wvoff[i], tc * 1024u, 0);
     };
     intx4 ring[D][RO];
     // second output: its few weight fragments of a chunk are requested at the top of the chunk
@@ -718,7 +721,8 @@ const QVariant kQVariants[] = {
     KXC_QV(7, 7, 1, 4, 2, 12),
     KXC_QV(7, 7, 1, 2, 2, 12),
     // two pixel blocks per wave (chosen by the shape rules in PrepareUncached, or by name); a deeper weight ring (nine
-    // k-steps instead of three) was measured too and changed nothing
+    // k-steps, a whole chunk, instead of three) was measured twice on all seven ResNet-18 layer shapes and was never
+    // faster (e.g. 512 -> 512 channels at 7 x 7: 14.1 against 13.2 us)
     KXC_QV2(3, 3, 2, 4, 2, 8, 2, 3),
     KXC_QV2(3, 3, 2, 4, 1, 8, 2, 3),
     KXC_QV2(3, 3, 2, 2, 2, 8, 2, 3),
