@@ -254,6 +254,13 @@ def test_qresnet18_small_every_layer(pkg, orc):
     # 24 operators, 21 launches: the three downsamples are second outputs of their block's first convolution
     assert len(net.launches) == 21 and net.launches[1].startswith("kxc_qconv2d_c4_i8:qmfma")
     assert sum("|qconv1x1+bias" in s for s in net.launches) == 3
+    # the plan as text and back (the two-output nodes carry four more operands): same logits
+    again = pkg.Plan.deserialize(net.plan.serialize(), 0)
+    out2 = torch.zeros_like(out)
+    again.run([dev(x)] + net.consts + [out2])
+    torch.cuda.synchronize()
+    assert_bit_exact(host(out2), want_logits, "quantised logits (plan rebuilt from its text)")
+    assert again.symbols() == net.launches
     assert net.launches[3].startswith("kxc_qconv2d_c16_i8:qmfma")
 
 
