@@ -969,7 +969,12 @@ int32_t NoAllocScratch(float** out) {
 bool PairTap(const kxc_hip_conv2d_desc* d, int* rh, int* rw) {
     if (d->pad_h % d->dil_h != 0 || d->pad_w % d->dil_w != 0) return false;
     *rh = d->pad_h / d->dil_h; *rw = d->pad_w / d->dil_w;
-    return *rh < d->kh && *rw < d->kw;
+    if (*rh >= d->kh || *rw >= d->kw) return false;
+    // ... and the unpadded 1x1 convolution must have this convolution's output extent (true for "same" padding,
+    // 2*pad = dil*(k-1)): otherwise the second output would have rows or columns the 1x1 convolution does not have
+    const int64_t oh = (static_cast<int64_t>(d->h) + 2 * d->pad_h - (static_cast<int64_t>(d->dil_h) * (d->kh - 1) + 1)) / d->stride_h + 1;
+    const int64_t ow = (static_cast<int64_t>(d->w) + 2 * d->pad_w - (static_cast<int64_t>(d->dil_w) * (d->kw - 1) + 1)) / d->stride_w + 1;
+    return oh == (d->h - 1) / d->stride_h + 1 && ow == (d->w - 1) / d->stride_w + 1;
 }
 
 // Everything about a launch that the descriptor alone decides (kernel, tile shape, grid, the split of the reduction,

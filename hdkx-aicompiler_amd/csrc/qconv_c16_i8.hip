@@ -922,9 +922,18 @@ int32_t kxc_hip_qconv2d_c16_i8(const kxc_hip_qconv2d_desc* d, const int8_t* x, c
 }
 
 // ---- two outputs from one launch: the convolution and a 1x1 convolution with the same strides, no padding
+// The second output's operand must be a tap of the window (pad < filter size) and the unpadded 1x1 convolution must
+// have this convolution's output extent (true for "same" padding, 2*pad = k-1).
+static bool PairGeometry(const kxc_hip_qconv2d_desc* d) {
+    if (!d || d->pad_h >= d->kh || d->pad_w >= d->kw || d->stride_h <= 0 || d->stride_w <= 0) return false;
+    const int64_t oh = (static_cast<int64_t>(d->h) + 2 * d->pad_h - d->kh) / d->stride_h + 1;
+    const int64_t ow = (static_cast<int64_t>(d->w) + 2 * d->pad_w - d->kw) / d->stride_w + 1;
+    return oh == (d->h - 1) / d->stride_h + 1 && ow == (d->w - 1) / d->stride_w + 1;
+}
+
 int32_t kxc_hip_qconv2d_c16_pair_supported(const kxc_hip_qconv2d_desc* d) {
     QLaunch L;
-    if (!d || d->pad_h >= d->kh || d->pad_w >= d->kw) return 0;
+    if (!PairGeometry(d)) return 0;
     if (Prepare(d, &L, "kxc_hip_qconv2d_c16_pair_supported") != KXC_HIP_OK) { LastError().clear(); return 0; }
     return (L.v && L.v->ds_kernel) ? 1 : 0;
 }
@@ -961,7 +970,7 @@ int32_t kxc_hip_qconv2d_c16_pair_i8(const kxc_hip_qconv2d_desc* d, const int8_t*
     const char* who = "kxc_hip_qconv2d_c16_pair_i8";
     QLaunch L;
     if (int32_t rc = Prepare(d, &L, who)) return rc;
-    KXC_HIP_REQUIRE(L.v && L.v->ds_kernel && d->pad_h < d->kh && d->pad_w < d->kw, "%s: no kernel with a second output covers this shape", who);
+    KXC_HIP_REQUIRE(L.v && L.v->ds_kernel && PairGeometry(d), "%s: no kernel with a second output covers this shape", who);
     if (L.args.M == 0) return KXC_HIP_OK;
     KXC_HIP_REQUIRE(x && w_packed && mult && y && w2_packed && mult2 && y2, "%s: NULL pointer", who);
     KXC_HIP_REQUIRE(!(d->flags & KXC_HIP_CONV_BIAS) || bias, "%s: bias flag without bias", who);

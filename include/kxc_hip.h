@@ -176,7 +176,8 @@ int32_t kxc_hip_conv2d_scratch_needed(const kxc_hip_conv2d_desc* desc, size_t* o
  * the input is read once and the second launch disappears.  Both outputs equal what the two separate calls give
  * (the second one bit for bit: same kernel arithmetic).
  *   ..._supported: 1 when a matrix-core kernel with a second output covers the shape (padding a multiple of the
- *   dilation and inside the filter, no 1x1 first filter), else 0; ..._variant names it ("unsupported" otherwise). */
+ *   dilation and inside the filter, and "same" padding -- 2*pad = dilation*(k-1) -- so that the unpadded 1x1
+ *   convolution has the first one's output extent; no 1x1 first filter), else 0; ..._variant names it ("unsupported" otherwise). */
 int32_t kxc_hip_conv2d_pair_supported(const kxc_hip_conv2d_desc* desc);
 const char* kxc_hip_conv2d_pair_variant(const kxc_hip_conv2d_desc* desc);
 int32_t kxc_hip_conv2d_pair_nchw_f32(const kxc_hip_conv2d_desc* desc, const float* x, const float* w,
@@ -283,7 +284,7 @@ int32_t kxc_hip_qconv2d_c16_i8(const kxc_hip_qconv2d_desc* desc, const int8_t* x
 /* Two outputs from one launch (a residual block's first 3x3/2 convolution and its 1x1/2 downsample): y as above, and
  * y2[n,o,oh,ow] = requantise(sum_c x[n,c,oh*stride,ow*stride] * w2[o,c] + bias2[o], mult2[o]) without ReLU -- the 1x1
  * convolution with the same strides and no padding, whose operand is the tap (pad_h, pad_w) of the first one's window
- * (needs pad < filter size).  w2_packed comes from kxc_hip_qconv2d_c16_pair_pack_weights (w2 is [o,c,1,1], packed in
+ * (needs "same" padding, 2*pad = k-1, so that both convolutions have the same output extent).  w2_packed comes from kxc_hip_qconv2d_c16_pair_pack_weights (w2 is [o,c,1,1], packed in
  * the chunking of `desc`); bias2 may be NULL.  Bit-identical to the two separate launches. */
 int32_t kxc_hip_qconv2d_c16_pair_supported(const kxc_hip_qconv2d_desc* desc);
 int32_t kxc_hip_qconv2d_c16_pair_packed_bytes(const kxc_hip_qconv2d_desc* desc, size_t* out_bytes);

@@ -135,6 +135,42 @@ def test_qconv_c16_pair_against_cpu(pkg, orc, shape):
     assert torch.equal(y2n, pkg.qconv2d_c16(xc, c, pkg.qconv2d_c16_pack_weights(dev(w2)), w2.shape, None, dev(mult2), None, 0.0, s, 0, False))
 
 
+def test_qconv_c16_pair_random_shapes(pkg):
+    """Seeded random geometries for the int8 two-output kernel (strides 1-3, padding 1 (0 and 2 are refused: the outputs' extents would differ), ragged channel and pixel
+    counts, residual on the main output): both outputs equal the two separate launches byte for byte."""
+    rng = np.random.default_rng(20250102)
+    ran = 0
+    for case in range(40):
+        n = int(rng.integers(1, 5)); c = int(rng.choice([3, 10, 16, 24, 40, 64, 100, 128])); o = int(rng.choice([32, 64, 96, 128]))
+        h = int(rng.integers(5, 30)); w = int(rng.integers(5, 30)); s = int(rng.integers(1, 4)); p = int(rng.choice([0, 1, 1, 1, 1, 2]))
+        if p != 1:
+            assert not pkg.qconv2d_c16_pair_supported(n, c, h, w, o, 3, s, p)      # the two outputs would differ in extent
+        if h + 2 * p < 3 or w + 2 * p < 3 or not pkg.qconv2d_c16_pair_supported(n, c, h, w, o, 3, s, p):
+            continue
+        ran += 1
+        x = torch.from_numpy(rng.integers(-128, 128, (n, c, h, w), dtype=np.int8)).cuda()
+        wq = torch.from_numpy(rng.integers(-127, 128, (o, c, 3, 3), dtype=np.int8)).cuda()
+        w2 = torch.from_numpy(rng.integers(-127, 128, (o, c, 1, 1), dtype=np.int8)).cuda()
+        bias = torch.from_numpy(rng.integers(-20000, 20000, (o,), dtype=np.int32)).cuda()
+        bias2 = torch.from_numpy(rng.integers(-2000, 2000, (o,), dtype=np.int32)).cuda() if case % 2 else None
+        mult = torch.from_numpy((rng.uniform(0.5, 2.0, (o,)) / (8.0 * np.sqrt(c * 9) * 64)).astype(np.float32)).cuda()
+        mult2 = torch.from_numpy((rng.uniform(0.5, 2.0, (o,)) / (8.0 * np.sqrt(c) * 64)).astype(np.float32)).cuda()
+        oh = (h + 2 * p - 3) // s + 1; ow = (w + 2 * p - 3) // s + 1
+        xc = pkg.i8_nchw_to_c16(x)
+        res = pkg.i8_nchw_to_c16(torch.from_numpy(rng.integers(-128, 128, (n, o, oh, ow), dtype=np.int8)).cuda()) if case % 3 == 0 else None
+        relu = case % 4 != 3
+        packed = pkg.qconv2d_c16_pack_weights(wq)
+        y, y2 = pkg.qconv2d_c16_pair(xc, c, packed, wq.shape, bias, mult, pkg.qconv2d_c16_pair_pack_weights(w2, 3), bias2, mult2,
+                                     res, 0.37 if res is not None else 0.0, s, p, relu)
+        alone = pkg.qconv2d_c16(xc, c, packed, wq.shape, bias, mult, res, 0.37 if res is not None else 0.0, s, p, relu)
+        # the second output: the 1x1 convolution on the tap (p, p) of the window = on x sampled with the stride, unpadded
+        xs = pkg.i8_nchw_to_c16(x[:, :, 0:(oh - 1) * s + 1:s, 0:(ow - 1) * s + 1:s].contiguous())
+        alone2 = pkg.qconv2d_c16(xs, c, pkg.qconv2d_c16_pack_weights(w2), w2.shape, bias2, mult2, None, 0.0, 1, 0, False)
+        assert torch.equal(y, alone), "case %d main" % case
+        assert torch.equal(y2, alone2), "case %d second: n=%d c=%d h=%d w=%d o=%d s=%d p=%d" % (case, n, c, h, w, o, s, p)
+    assert ran >= 20, ran
+
+
 @pytest.mark.parametrize("shape", [(2, 3, 224, 224, 64), (1, 3, 64, 64, 64), (3, 4, 20, 36, 32), (2, 1, 9, 8, 96)],
                          ids=lambda s: "x".join(map(str, s)))
 def test_qconv_first_layer_c4_against_cpu(pkg, orc, shape):

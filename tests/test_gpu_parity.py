@@ -504,6 +504,39 @@ def test_conv_random_shapes_against_direct_kernel(pkg):
     assert "mfma_k1x1_small" in seen and any(v.startswith("mfma_k3x3") for v in seen) and any(v.startswith("mfma_k7x7") for v in seen), seen
 
 
+def test_conv_pair_random_shapes_against_direct_kernel(pkg):
+    """Seeded random geometries for the two-output kernel (3x3 filters, strides 1-3, padding 1 (0 and 2 are refused: the outputs' extents would differ), ragged channel,
+    output-channel and pixel counts, with and without either bias, residual and ReLU on the main output): both
+    outputs against the reference-order direct kernel run twice on the same GPU tensors."""
+    rng = np.random.default_rng(20250101)
+    ran = 0
+    for case in range(90):
+        n = int(rng.integers(1, 6)); c = int(rng.choice([4, 8, 16, 24, 40, 64, 96, 128])); o = int(rng.choice([32, 40, 64, 96, 128, 200]))
+        h = int(rng.integers(5, 34)); w = int(rng.integers(5, 34)); stride = int(rng.integers(1, 4)); p = int(rng.choice([0, 1, 1, 1, 1, 2]))
+        if p != 1:
+            assert not pkg.conv2d_pair_supported((n, c, h, w), (o, c, 3, 3), stride, p)      # the two outputs would differ in extent
+        if h + 2 * p < 3 or w + 2 * p < 3 or not pkg.conv2d_pair_supported((n, c, h, w), (o, c, 3, 3), stride, p):
+            continue
+        ran += 1
+        x = torch.from_numpy(rng.uniform(-1, 1, (n, c, h, w)).astype(np.float32)).cuda()
+        wt = torch.from_numpy((rng.standard_normal((o, c, 3, 3)) * np.sqrt(2.0 / (9 * c))).astype(np.float32)).cuda()
+        w2 = torch.from_numpy((rng.standard_normal((o, c, 1, 1)) * np.sqrt(2.0 / c)).astype(np.float32)).cuda()
+        b = torch.from_numpy(rng.uniform(-0.1, 0.1, (o,)).astype(np.float32)).cuda() if case % 2 == 0 else None
+        b2 = torch.from_numpy(rng.uniform(-0.1, 0.1, (o,)).astype(np.float32)).cuda() if case % 3 != 0 else None
+        oh = (h + 2 * p - 3) // stride + 1; ow = (w + 2 * p - 3) // stride + 1
+        r = torch.from_numpy(rng.uniform(-1, 1, (n, o, oh, ow)).astype(np.float32)).cuda() if case % 4 == 0 else None
+        relu = case % 5 != 4
+        # the 1x1 convolution reads x[oh*stride + p - p, ...]: same strides, no padding, on the window's tap (p, p)
+        y, y2 = pkg.conv2d_pair(x, wt, b, r, w2, b2, stride, p, 1, relu)
+        want = pkg.conv2d(x, wt, b, r, stride, p, 1, relu, force_direct=True)
+        xs = x[:, :, 0:(oh - 1) * stride + 1:stride, 0:(ow - 1) * stride + 1:stride].contiguous()
+        want2 = pkg.conv2d(xs, w2, b2, None, 1, 0, 1, False, force_direct=True)
+        what = "case %d: n=%d c=%d h=%d w=%d o=%d s=%d p=%d" % (case, n, c, h, w, o, stride, p)
+        assert_close(host(y), host(want), what=what + " (main)")
+        assert_close(host(y2), host(want2), what=what + " (second)")
+    assert ran >= 20, ran
+
+
 def test_conv_winograd_unsupported_shapes_are_refused(pkg):
     assert not pkg.conv2d_winograd_supported((1, 8, 8, 8), (16, 8, 3, 3), 2, 1)        # stride
     assert not pkg.conv2d_winograd_supported((1, 8, 8, 8), (16, 8, 1, 1), 1, 0)        # filter size
