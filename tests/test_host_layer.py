@@ -59,6 +59,14 @@ def test_packed_function_registry_cpu():
 
 
 @pytest.mark.gpu
+def test_generated_kernels_lds_schedules_bit_exact():
+    """dense / matmul / reduce_mean shapes that take the generator's LDS-staged schedules (ragged chunks, fewer outputs
+    than a workgroup, an operand that is not contiguous along the reduce axis): bit-identical to the host back end."""
+    out = run("generated_numeric")
+    assert "generated kernels ok" in out and out.count("[PASS]") == 5
+
+
+@pytest.mark.gpu
 def test_packed_function_registry_hip():
     """The same registry on the GPU: allocation, copies with offsets on a stream, attributes, target.Build,
     device_info.hip.0.*, and a Relay function lowered to plan JSON and run from that JSON."""
