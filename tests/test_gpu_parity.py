@@ -224,7 +224,8 @@ def _scratch_needed(pkg, xs, ws, s, p):
 
 @pytest.mark.parametrize("variant", ["mfma_k3x3_c4_o1x1_p4x1", "mfma_k3x3_c4_o1x1_p8x1", "mfma_k3x3_c2_o1x1_p4x1",
                                      "mfma_k3x3_c4_o1x1_p2x1", "mfma_k3x3_c4_o2x1_p8x1", "mfma_k3x3_c4_o1x1_p4x1_ks2",
-                                     "mfma_k3x3_c4_o1x1_p2x1_ks4", "mfma_k3x3_c4_o1x1_p2x1_ks8"])
+                                     "mfma_k3x3_c4_o1x1_p2x1_ks4", "mfma_k3x3_c4_o1x1_p2x1_ks8", "mfma_k3x3_c4_o1x1_p7x1_ks2",
+                                     "mfma_k3x3_c4_o2x1_p7x1"])
 def test_conv_pair_every_tile(pkg, fast_orc, synth, monkeypatch, variant):
     """Every tile shape that exists with a second output, forced once (128 -> 256 channels)."""
     monkeypatch.setenv("KXC_HIP_CONV_VARIANT", variant)
