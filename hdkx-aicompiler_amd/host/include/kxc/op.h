@@ -179,6 +179,27 @@ KXC_ATTRS_REF(SoftmaxAttrs)
 
 // cast (src/relay/op/tensor/transform.cc:84-104): `to` is a dtype code -- 0 float32, 1 int32, 2 int64, 3 float64,
 // 4 bool, 5 int8, 6 uint8
+// Quantised operators.  The reference has no int8 operator (grep for int8 / quant finds dtype plumbing only); these
+// follow its rules for adding one (docs/relay-op-integration/04-lowering-backend.md:142-152: attributes, type rule,
+// TOPI compute with a tir::Call for the new intrinsic `rint`, code-generator mapping, numeric test):
+//   qnn_quantize(x f32)                                   -> int8  clamp(rint(x / scale), -127, 127), NaN -> 0
+//   qnn_conv2d(x i8, w i8, bias i32, mult f32[, res i8])  -> int8  acc = sum x*w in int32 + bias[o];
+//        v = (float)acc * mult[o] [+ (float)res * res_mult];  clamp(rint(v), relu ? 0 : -128, 127), NaN -> 0
+//   qnn_dense(x i8 [M,K], w i8 [N,K], bias i32, mult f32) -> float32  (float)(acc + bias[j]) * mult[j]
+// rint rounds to nearest, ties to even; every float operation is rounded separately.
+struct QnnConv2DAttrsNode : AttrsNode {
+    std::vector<int64_t> strides, padding;      // {h, w}; padding symmetric {h, w}
+    bool relu = true;
+    double res_mult = 0.0;
+};
+KXC_ATTRS_REF(QnnConv2DAttrs)
+    static QnnConv2DAttrs Create(std::vector<int64_t> strides, std::vector<int64_t> padding, bool relu, double res_mult = 0.0);
+};
+struct QnnQuantizeAttrsNode : AttrsNode { double scale = 1.0; };
+KXC_ATTRS_REF(QnnQuantizeAttrs)
+    static QnnQuantizeAttrs Create(double scale);
+};
+
 struct CastAttrsNode : AttrsNode { int to = 0; };
 KXC_ATTRS_REF(CastAttrs)
     static CastAttrs Create(int to);
@@ -198,6 +219,9 @@ Type Conv2DInferType(const Attrs& attrs, const Array<Type>& inputs);
 Type Pool2DInferType(const Attrs& attrs, const Array<Type>& inputs);
 Type GlobalAvgPool2DInferType(const Attrs& attrs, const Array<Type>& inputs);
 Type DenseInferType(const Attrs& attrs, const Array<Type>& inputs);
+Type QnnConv2DInferType(const Attrs& attrs, const Array<Type>& inputs);
+Type QnnDenseInferType(const Attrs& attrs, const Array<Type>& inputs);
+Type QnnQuantizeInferType(const Attrs& attrs, const Array<Type>& inputs);
 Type GemmInferType(const Attrs& attrs, const Array<Type>& inputs);
 Type MatmulInferType(const Attrs& attrs, const Array<Type>& inputs);
 Type UnarySameInferType(const Attrs& attrs, const Array<Type>& inputs);

@@ -51,6 +51,12 @@ Tensor softmax(const Tensor& x, int axis, std::string name);
 // Call(dtype, "cast", {x}) per element (include/te/topi/elemwise.h:113-122): C conversion rules
 Tensor cast(const Tensor& x, tir::DataType dtype, std::string name);
 
+// Quantised operators (see QnnConv2DAttrsNode in op.h for the arithmetic).  residual may be an undefined Tensor.
+Tensor qnn_quantize(const Tensor& x, double scale, std::string name);
+Tensor qnn_conv2d_nchw(const Tensor& data, const Tensor& kernel, const Tensor& bias, const Tensor& mult, const Tensor& residual,
+                       int stride_h, int stride_w, int pad_h, int pad_w, bool relu, double res_mult, std::string name);
+Tensor qnn_dense(const Tensor& A, const Tensor& B, const Tensor& bias, const Tensor& mult, std::string name);
+
 }  // namespace topi
 }  // namespace te
 }  // namespace kxc

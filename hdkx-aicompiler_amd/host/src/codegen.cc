@@ -101,7 +101,9 @@ std::string EmitExpr(const PrimExpr& e, Names* names, const ExprOverrides* overr
         case ExprKind::kCall: {
             if (e->name == "cast") return "((" + CType(e->dtype, names->builtin_types) + ")(" + A(0) + "))";
             static const std::map<std::string, std::string> f32 = {{"exp", "expf"}, {"log", "logf"}, {"sqrt", "sqrtf"},
-                {"floor", "floorf"}, {"ceil", "ceilf"}, {"fabs", "fabsf"}, {"tanh", "tanhf"}};
+                {"floor", "floorf"}, {"ceil", "ceilf"}, {"fabs", "fabsf"}, {"tanh", "tanhf"},
+                // round to nearest, ties to even (the default rounding mode): the quantised operators' rounding
+                {"rint", "rintf"}};
             std::string name = e->name;
             if (name.rfind("tir.", 0) == 0) name = name.substr(4);
             auto it = f32.find(name);

@@ -193,6 +193,59 @@ std::string DenseDispatch(bool transB, const HIPDispatchContext& c, kxc_hip_plan
     return "kxc_gemm_f32";
 }
 
+// ---------------------------------------------------------------- quantised operators (no counterpart in the reference)
+bool IsDType(const Type& t, const char* dtype) { return TT(t) && TT(t)->dtype == dtype; }
+
+te::Tensor QnnConv2DCompute(const Attrs& attrs, const Array<te::Tensor>& in, const Type&) {
+    const auto* p = attrs.As<QnnConv2DAttrsNode>();
+    if (!p) throw std::runtime_error("qnn_conv2d expects QnnConv2DAttrs");
+    if (in.size() != 4 && in.size() != 5) throw std::runtime_error("qnn_conv2d expects data, weight, bias, mult[, residual]");
+    const auto st = ReadPair(p->strides, 1), pd = ReadPair(p->padding, 0);
+    return te::topi::qnn_conv2d_nchw(in[0], in[1], in[2], in[3], in.size() == 5 ? in[4] : te::Tensor(), static_cast<int>(st[0]),
+                                     static_cast<int>(st[1]), static_cast<int>(pd[0]), static_cast<int>(pd[1]), p->relu, p->res_mult,
+                                     "T_qnn_conv2d");
+}
+
+std::string QnnConv2DDispatch(const HIPDispatchContext& c, kxc_hip_plan* plan) {
+    const auto* p = c.attrs.As<QnnConv2DAttrsNode>();
+    if (!p || c.inputs.size() < 4 || !IsDType(c.input_types[0], "int8") || !IsDType(c.out_type, "int8")) return "";
+    const auto* x = TT(c.input_types[0]);
+    const auto* w = TT(c.input_types[1]);
+    const auto st = ReadPair(p->strides, 1), pd = ReadPair(p->padding, 0);
+    kxc_hip_qconv2d_desc d{};
+    d.n = static_cast<int32_t>(x->shape[0]); d.c = static_cast<int32_t>(x->shape[1]);
+    d.h = static_cast<int32_t>(x->shape[2]); d.w = static_cast<int32_t>(x->shape[3]);
+    d.o = static_cast<int32_t>(w->shape[0]); d.kh = static_cast<int32_t>(w->shape[2]); d.kw = static_cast<int32_t>(w->shape[3]);
+    d.stride_h = static_cast<int32_t>(st[0]); d.stride_w = static_cast<int32_t>(st[1]);
+    d.pad_h = static_cast<int32_t>(pd[0]); d.pad_w = static_cast<int32_t>(pd[1]);
+    const bool has_res = c.inputs.size() == 5;
+    d.flags = KXC_HIP_CONV_BIAS | (has_res ? KXC_HIP_CONV_RESIDUAL : 0u) | (p->relu ? KXC_HIP_CONV_RELU : 0u);
+    d.res_mult = has_res ? static_cast<float>(p->res_mult) : 0.0f;
+    const kxc_hip_buf none{KXC_HIP_BUF_NONE, 0};
+    Check(kxc_hip_plan_add_qconv2d(plan, &d, B(c.inputs[0]), B(c.inputs[1]), B(c.inputs[2]), B(c.inputs[3]),
+                                   has_res ? B(c.inputs[4]) : none, B(c.output)),
+          "qnn_conv2d dispatch");
+    return "kxc_qconv2d_nchw_i8";
+}
+
+std::string QnnDenseDispatch(const HIPDispatchContext& c, kxc_hip_plan* plan) {
+    if (c.inputs.size() != 4 || !IsDType(c.input_types[0], "int8") || !IsF32(c.out_type)) return "";
+    const auto* a = TT(c.input_types[0]);
+    const auto* o = TT(c.out_type);
+    Check(kxc_hip_plan_add_qdense(plan, o->shape[0], o->shape[1], a->shape[1], B(c.inputs[0]), B(c.inputs[1]), B(c.inputs[2]),
+                                  B(c.inputs[3]), B(c.output)),
+          "qnn_dense dispatch");
+    return "kxc_qdense_i8";
+}
+
+std::string QnnQuantizeDispatch(const HIPDispatchContext& c, kxc_hip_plan* plan) {
+    const auto* p = c.attrs.As<QnnQuantizeAttrsNode>();
+    if (!p || !IsF32(c.input_types[0])) return "";
+    Check(kxc_hip_plan_add_quantize(plan, Product(TT(c.input_types[0])->shape), static_cast<float>(p->scale), B(c.inputs[0]), B(c.output)),
+          "qnn_quantize dispatch");
+    return "kxc_quantize_f32_i8";
+}
+
 // ---------------------------------------------------------------- elementwise
 std::string BinaryDispatch(int op, const HIPDispatchContext& c, kxc_hip_plan* plan) {
     if (!IsF32(c.input_types[0]) || !IsF32(c.input_types[1])) return "";
@@ -294,6 +347,42 @@ void EnsureBuiltinOpsRegistered() {
                 return te::topi::dense(in[0], in[1], "T_dense");
             })
             .set_attr<FHIPDispatch>("FHIPDispatch", [](const HIPDispatchContext& c, kxc_hip_plan* p) { return DenseDispatch(true, c, p); });
+        OpRegEntry::Register("qnn_conv2d")
+            .describe("int8 2D convolution with int32 accumulation and per-output-channel requantisation (NCHW / OIHW).")
+            .set_num_inputs(-1)
+            .add_argument("data", "Tensor", "int8 input.")
+            .add_argument("weight", "Tensor", "int8 weights.")
+            .add_argument("bias", "Tensor", "int32 bias per output channel.")
+            .add_argument("mult", "Tensor", "float32 requantisation multiplier per output channel.")
+            .set_attr<std::string>("TAttrs", "QnnConv2DAttrs")
+            .set_attr<FInferType>("FInferType", QnnConv2DInferType)
+            .set_attr<FRelayToTE>("FRelayToTE", QnnConv2DCompute)
+            .set_attr<FHIPDispatch>("FHIPDispatch", QnnConv2DDispatch);
+        OpRegEntry::Register("qnn_dense")
+            .describe("int8 dense layer with int32 accumulation; float32 output (acc + bias) * mult.")
+            .set_num_inputs(4)
+            .add_argument("data", "Tensor", "int8 input [M, K].")
+            .add_argument("weight", "Tensor", "int8 weights [N, K].")
+            .add_argument("bias", "Tensor", "int32 bias [N].")
+            .add_argument("mult", "Tensor", "float32 multiplier [N].")
+            .set_attr<FInferType>("FInferType", QnnDenseInferType)
+            .set_attr<FRelayToTE>("FRelayToTE", [](const Attrs&, const Array<te::Tensor>& in, const Type&) {
+                if (in.size() != 4) throw std::runtime_error("qnn_dense expects data, weight, bias, mult");
+                return te::topi::qnn_dense(in[0], in[1], in[2], in[3], "T_qnn_dense");
+            })
+            .set_attr<FHIPDispatch>("FHIPDispatch", QnnDenseDispatch);
+        OpRegEntry::Register("qnn_quantize")
+            .describe("float32 -> int8 with a per-tensor scale: clamp(rint(x / scale), -127, 127).")
+            .set_num_inputs(1)
+            .add_argument("data", "Tensor", "float32 input.")
+            .set_attr<std::string>("TAttrs", "QnnQuantizeAttrs")
+            .set_attr<FInferType>("FInferType", QnnQuantizeInferType)
+            .set_attr<FRelayToTE>("FRelayToTE", [](const Attrs& attrs, const Array<te::Tensor>& in, const Type&) {
+                const auto* p = attrs.As<QnnQuantizeAttrsNode>();
+                if (!p || in.size() != 1) throw std::runtime_error("qnn_quantize expects one input and QnnQuantizeAttrs");
+                return te::topi::qnn_quantize(in[0], p->scale, "T_qnn_quantize");
+            })
+            .set_attr<FHIPDispatch>("FHIPDispatch", QnnQuantizeDispatch);
         OpRegEntry::Register("matmul")
             .describe("Matrix multiplication [M,K] x [K,N]")
             .set_num_inputs(2)

@@ -134,6 +134,16 @@ SoftmaxAttrs SoftmaxAttrs::Create(int64_t axis) {
     n->axis = axis;
     return SoftmaxAttrs(n);
 }
+QnnConv2DAttrs QnnConv2DAttrs::Create(std::vector<int64_t> strides, std::vector<int64_t> padding, bool relu, double res_mult) {
+    auto n = std::make_shared<QnnConv2DAttrsNode>();
+    n->strides = std::move(strides); n->padding = std::move(padding); n->relu = relu; n->res_mult = res_mult;
+    return QnnConv2DAttrs(n);
+}
+QnnQuantizeAttrs QnnQuantizeAttrs::Create(double scale) {
+    auto n = std::make_shared<QnnQuantizeAttrsNode>();
+    n->scale = scale;
+    return QnnQuantizeAttrs(n);
+}
 CastAttrs CastAttrs::Create(int to) {
     auto n = std::make_shared<CastAttrsNode>();
     n->to = to;
@@ -224,6 +234,67 @@ Type Conv2DInferType(const Attrs& attrs, const Array<Type>& in) {
     const int64_t ow = WindowOutputDim("nn_conv2d", data->shape[3], weight->shape[3], padding[1], padding[3], strides[1], dilation[1], false);
     const std::string dtype = a && !a->out_dtype.empty() ? a->out_dtype : data->dtype;
     return TensorType({data->shape[0], channels, oh, ow}, dtype);
+}
+
+namespace {
+void RequireDType(const char* op, const TensorTypeNode* t, const char* what, const char* dtype) {
+    if (t->dtype != dtype) throw std::runtime_error(std::string(op) + " expects " + what + " of dtype " + dtype + ", got " + t->dtype);
+}
+void RequireChannelVector(const char* op, const TensorTypeNode* t, const char* what, int64_t channels) {
+    if (t->shape.size() != 1 || t->shape[0] != channels)
+        throw std::runtime_error(std::string(op) + " " + what + " must be rank-1 with one entry per output channel");
+}
+}  // namespace
+
+Type QnnConv2DInferType(const Attrs& attrs, const Array<Type>& in) {
+    if (in.size() != 4 && in.size() != 5) throw std::runtime_error("qnn_conv2d expects data, weight, bias, mult[, residual]");
+    const auto* a = attrs.As<QnnConv2DAttrsNode>();
+    if (!a) throw std::runtime_error("qnn_conv2d expects QnnConv2DAttrs");
+    const auto* data = RequireTensor("qnn_conv2d", in[0], "data");
+    const auto* weight = RequireTensor("qnn_conv2d", in[1], "weight");
+    const auto* bias = RequireTensor("qnn_conv2d", in[2], "bias");
+    const auto* mult = RequireTensor("qnn_conv2d", in[3], "mult");
+    RequireDType("qnn_conv2d", data, "data", "int8"); RequireDType("qnn_conv2d", weight, "weight", "int8");
+    RequireDType("qnn_conv2d", bias, "bias", "int32"); RequireDType("qnn_conv2d", mult, "mult", "float32");
+    if (data->shape.size() != 4 || weight->shape.size() != 4) throw std::runtime_error("qnn_conv2d expects NCHW/OIHW rank-4 tensors");
+    if (data->shape[1] != weight->shape[1]) throw std::runtime_error("qnn_conv2d input channel mismatch");
+    RequireChannelVector("qnn_conv2d", bias, "bias", weight->shape[0]);
+    RequireChannelVector("qnn_conv2d", mult, "mult", weight->shape[0]);
+    const auto strides = ReadPair(a->strides, 1);
+    const auto pads = ReadPair(a->padding, 0);
+    const int64_t oh = WindowOutputDim("qnn_conv2d", data->shape[2], weight->shape[2], pads[0], pads[0], strides[0], 1, false);
+    const int64_t ow = WindowOutputDim("qnn_conv2d", data->shape[3], weight->shape[3], pads[1], pads[1], strides[1], 1, false);
+    const std::vector<int64_t> oshape = {data->shape[0], weight->shape[0], oh, ow};
+    if (in.size() == 5) {
+        const auto* res = RequireTensor("qnn_conv2d", in[4], "residual");
+        RequireDType("qnn_conv2d", res, "residual", "int8");
+        if (res->shape != oshape) throw std::runtime_error("qnn_conv2d residual must have the output's shape");
+    }
+    return TensorType(oshape, "int8");
+}
+
+Type QnnDenseInferType(const Attrs&, const Array<Type>& in) {
+    RequireArity("qnn_dense", in, 4);
+    const auto* data = RequireTensor("qnn_dense", in[0], "data");
+    const auto* weight = RequireTensor("qnn_dense", in[1], "weight");
+    const auto* bias = RequireTensor("qnn_dense", in[2], "bias");
+    const auto* mult = RequireTensor("qnn_dense", in[3], "mult");
+    RequireDType("qnn_dense", data, "data", "int8"); RequireDType("qnn_dense", weight, "weight", "int8");
+    RequireDType("qnn_dense", bias, "bias", "int32"); RequireDType("qnn_dense", mult, "mult", "float32");
+    if (data->shape.size() != 2 || weight->shape.size() != 2) throw std::runtime_error("qnn_dense expects rank-2 data and weight");
+    if (data->shape[1] != weight->shape[1]) throw std::runtime_error("qnn_dense input dimension mismatch");
+    RequireChannelVector("qnn_dense", bias, "bias", weight->shape[0]);
+    RequireChannelVector("qnn_dense", mult, "mult", weight->shape[0]);
+    return TensorType({data->shape[0], weight->shape[0]}, "float32");
+}
+
+Type QnnQuantizeInferType(const Attrs& attrs, const Array<Type>& in) {
+    RequireArity("qnn_quantize", in, 1);
+    const auto* a = attrs.As<QnnQuantizeAttrsNode>();
+    if (!a || !(a->scale > 0.0)) throw std::runtime_error("qnn_quantize expects QnnQuantizeAttrs with a positive scale");
+    const auto* x = RequireTensor("qnn_quantize", in[0], "data");
+    RequireDType("qnn_quantize", x, "data", "float32");
+    return TensorType(x->shape, "int8");
 }
 
 Type Pool2DInferType(const Attrs& attrs, const Array<Type>& in) {

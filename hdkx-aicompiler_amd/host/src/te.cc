@@ -298,6 +298,57 @@ Tensor cast(const Tensor& x, tir::DataType dtype, std::string name) {
     return compute(x->shape, [&](const Array<Var>& i) { return tir::Call(dtype, "cast", {x(i)}); }, name, kElementWise);
 }
 
+// ---- quantised operators: int32 accumulation, one rounded fp32 multiply (and add) per output, rint = round to
+// nearest with ties to even, NaN -> 0, clamp, convert
+namespace {
+PrimExpr RintClampToI8(PrimExpr v, double lo, double hi) {
+    const DataType f32 = DataType::Float(32);
+    PrimExpr r = tir::Call(f32, "rint", {v});
+    r = tir::Select(tir::EQ(v, v), r, make_const(f32, 0.0));
+    r = tir::Min(tir::Max(r, make_const(f32, lo)), make_const(f32, hi));
+    return tir::Call(DataType::Int(8), "cast", {r});
+}
+}  // namespace
+
+Tensor qnn_quantize(const Tensor& x, double scale, std::string name) {
+    return compute(x->shape, [&](const Array<Var>& i) { return RintClampToI8(x(i) / make_const(x->dtype, scale), -127.0, 127.0); },
+                   name, kElementWise);
+}
+
+Tensor qnn_conv2d_nchw(const Tensor& data, const Tensor& kernel, const Tensor& bias, const Tensor& mult, const Tensor& residual,
+                       int stride_h, int stride_w, int pad_h, int pad_w, bool relu, double res_mult, std::string name) {
+    const DataType i32 = DataType::Int(32), f32 = DataType::Float(32);
+    const int64_t H = ConstDim(data->shape[2]), W = ConstDim(data->shape[3]);
+    const int64_t KH = ConstDim(kernel->shape[2]), KW = ConstDim(kernel->shape[3]);
+    const int64_t OH = (H + 2 * pad_h - KH) / stride_h + 1, OW = (W + 2 * pad_w - KW) / stride_w + 1;
+    IterVar rc = reduce_axis(0, data->shape[1], "rc");
+    IterVar rh = reduce_axis(0, kernel->shape[2], "rh");
+    IterVar rw = reduce_axis(0, kernel->shape[3], "rw");
+    const std::vector<PrimExpr> oshape = {data->shape[0], kernel->shape[0], I64(OH), I64(OW)};
+    Tensor acc = compute(oshape, [&](const Array<Var>& i) {
+        PrimExpr h_in = i[2] * stride_h + rh.var - pad_h;
+        PrimExpr w_in = i[3] * stride_w + rw.var - pad_w;
+        PrimExpr x = tir::Select((h_in >= 0) && (h_in < data->shape[2]) && (w_in >= 0) && (w_in < data->shape[3]),
+                                 tir::Call(i32, "cast", {data(i[0], rc.var, h_in, w_in)}), make_const(i32, 0));
+        return sum(x * tir::Call(i32, "cast", {kernel(i[1], rc.var, rh.var, rw.var)}), {rc, rh, rw});
+    }, name + "_acc", kConv2d);
+    return compute(oshape, [&](const Array<Var>& i) {
+        PrimExpr v = tir::Call(f32, "cast", {acc(i) + bias(i[1])}) * mult(i[1]);
+        if (residual.defined()) v = v + tir::Call(f32, "cast", {residual(i)}) * make_const(f32, static_cast<double>(static_cast<float>(res_mult)));
+        return RintClampToI8(v, relu ? 0.0 : -128.0, 127.0);
+    }, name, kElementWise);
+}
+
+Tensor qnn_dense(const Tensor& A, const Tensor& B, const Tensor& bias, const Tensor& mult, std::string name) {
+    const DataType i32 = DataType::Int(32), f32 = DataType::Float(32);
+    IterVar k = reduce_axis(0, A->shape[1], "k");
+    Tensor acc = compute({A->shape[0], B->shape[0]}, [&](const Array<Var>& i) {
+        return sum(tir::Call(i32, "cast", {A(i[0], k.var)}) * tir::Call(i32, "cast", {B(i[1], k.var)}), {k});
+    }, name + "_acc", kMatMul);
+    return compute(acc->shape, [&](const Array<Var>& i) { return tir::Call(f32, "cast", {acc(i) + bias(i[1])}) * mult(i[1]); },
+                   name, kElementWise);
+}
+
 }  // namespace topi
 }  // namespace te
 }  // namespace kxc

@@ -9,6 +9,8 @@
 //   host_tests resnet18 <cpu|hip|hipgen> <dir> <batch> <hw>
 //                                            builds the ResNet-18 graph, reads input.bin and const_<k>.bin
 //                                            from <dir>, runs, writes logits.bin and plan.json
+#include <dlfcn.h>
+#include <array>
 #include <cmath>
 #include <sstream>
 #include <cstdio>
@@ -1125,6 +1127,184 @@ int RunGeneratedNumeric() {
     return 0;
 }
 
+// Quantised operators (qnn_quantize, qnn_conv2d, qnn_dense) through the compiler, bit-exact against hand-worked answers
+// and against the C oracle loaded from the path given (its functions are bound by name, nothing else is linked).
+int RunQnn(const std::string& oracle_path) {
+    auto I8 = [](std::vector<int8_t>& v, bool out) { return Buf{v.data(), v.size(), out}; };
+    auto I32 = [](std::vector<int32_t>& v) { return Buf{v.data(), v.size() * sizeof(int32_t), false}; };
+    // ---- rounding: ties go to the even integer, NaN gives 0, saturation at +-127
+    {
+        kxc::Var x("x", kxc::TensorType({12}, "float32"));
+        kxc::Function f({x}, kxc::Call(Op::Get("qnn_quantize"), {x}, kxc::relay::QnnQuantizeAttrs::Create(0.5)));
+        std::vector<float> xd = {0.25f, 0.75f, 1.25f, -0.25f, -0.75f, 0.26f, 0.24f, 500.0f, -500.0f, std::nanf(""), 63.5f, -63.75f};
+        std::vector<int8_t> q(12, 99);
+        CompileAndRun("qnn_quantize", f, {In(xd), I8(q, true)});
+        const std::vector<int8_t> expect = {0, 2, 2, 0, -2, 1, 0, 127, -127, 0, 127, -127};
+        for (size_t i = 0; i < q.size(); ++i)
+            Check(q[i] == expect[i], "qnn_quantize[" + std::to_string(i) + "] = " + std::to_string(q[i]) + ", expected " + std::to_string(expect[i]));
+        std::cout << "[PASS] qnn_quantize rounding\n";
+    }
+    // ---- a 1x1x3x3 convolution worked by hand: 2x2 window of ones, bias 1, mult 0.25, residual weight 0.5
+    {
+        kxc::Var d("d", kxc::TensorType({1, 1, 3, 3}, "int8")), w("w", kxc::TensorType({1, 1, 2, 2}, "int8"));
+        kxc::Var b("b", kxc::TensorType({1}, "int32")), m("m", kxc::TensorType({1}, "float32")), r("r", kxc::TensorType({1, 1, 2, 2}, "int8"));
+        kxc::Function f({d, w, b, m, r}, kxc::Call(Op::Get("qnn_conv2d"), {d, w, b, m, r}, kxc::relay::QnnConv2DAttrs::Create({1, 1}, {0, 0}, true, 0.5)));
+        std::vector<int8_t> dd = {1, 2, 3, 4, 5, 6, 7, 8, -100}, wd = {1, 1, 1, 1}, rd = {1, -20, 3, 0}, y(4, 99);
+        std::vector<int32_t> bd = {1};
+        std::vector<float> md = {0.25f};
+        CompileAndRun("qnn_conv2d", f, {I8(dd, false), I8(wd, false), I32(bd), In(md), I8(rd, false), I8(y, true)});
+        // sums 12 16 24 -81; +1 -> 13 17 25 -80; *0.25 -> 3.25 4.25 6.25 -20; + residual*0.5 -> 3.75 -5.75 7.75 -20; rint, relu
+        const std::vector<int8_t> expect = {4, 0, 8, 0};
+        Check(y == expect, "qnn_conv2d hand-worked case differs");
+        std::cout << "[PASS] qnn_conv2d hand-worked\n";
+    }
+    void* lib = dlopen(oracle_path.c_str(), RTLD_NOW | RTLD_LOCAL);
+    Check(lib != nullptr, "cannot load the oracle: " + oracle_path);
+    using ConvFn = void (*)(const int8_t*, const int8_t*, const int32_t*, const float*, const int8_t*, float, int8_t*, int64_t, int64_t,
+                            int64_t, int64_t, int64_t, int64_t, int64_t, int, int, int, int, int);
+    using DenseFn = void (*)(const int8_t*, const int8_t*, const int32_t*, const float*, float*, int64_t, int64_t, int64_t);
+    using QuantFn = void (*)(const float*, int8_t*, int64_t, float);
+    auto oracle_conv = reinterpret_cast<ConvFn>(dlsym(lib, "kxc_oracle_qconv2d_nchw_i8"));
+    auto oracle_dense = reinterpret_cast<DenseFn>(dlsym(lib, "kxc_oracle_qdense_i8"));
+    auto oracle_quant = reinterpret_cast<QuantFn>(dlsym(lib, "kxc_oracle_quantize_f32_i8"));
+    Check(oracle_conv && oracle_dense && oracle_quant, "oracle symbols missing");
+    uint32_t seed = 2024;
+    auto next = [&seed]() { seed = seed * 1664525u + 1013904223u; return seed >> 8; };
+    auto fill_i8 = [&](std::vector<int8_t>& v) { for (auto& e : v) e = static_cast<int8_t>(static_cast<int>(next() % 255) - 127); };
+    // ---- convolutions against the oracle: with and without residual / relu, strides 1 and 2, 1x1 / 3x3 / 7x7 windows
+    struct CS { int64_t n, c, h, w, o, k; int s, p; bool relu, res; };
+    const std::vector<CS> shapes = {{2, 5, 9, 7, 6, 3, 1, 1, true, true},   {1, 3, 8, 8, 4, 1, 2, 0, false, false},
+                                    {1, 4, 10, 11, 8, 3, 2, 1, true, false}, {1, 3, 20, 20, 5, 7, 2, 3, false, true},
+                                    {2, 16, 6, 6, 16, 3, 1, 1, true, true}};
+    for (const auto& c : shapes) {
+        const int64_t oh = (c.h + 2 * c.p - c.k) / c.s + 1, ow = (c.w + 2 * c.p - c.k) / c.s + 1;
+        std::vector<int8_t> x(c.n * c.c * c.h * c.w), w(c.o * c.c * c.k * c.k), res(c.n * c.o * oh * ow), y(res.size(), 99), want(res.size(), 77);
+        std::vector<int32_t> bias(c.o);
+        std::vector<float> mult(c.o);
+        fill_i8(x); fill_i8(w); fill_i8(res);
+        for (auto& b : bias) b = static_cast<int32_t>(next() % 4001) - 2000;
+        // multipliers sized so that outputs spread over the int8 range and some saturate
+        for (auto& m : mult) m = (0.5f + static_cast<float>(next() % 1000) / 1000.0f) * 3.0f / (64.0f * std::sqrt(static_cast<float>(c.c * c.k * c.k)));
+        const float res_mult = 0.37f;
+        kxc::Var d("d", kxc::TensorType({c.n, c.c, c.h, c.w}, "int8")), wv("w", kxc::TensorType({c.o, c.c, c.k, c.k}, "int8"));
+        kxc::Var b("b", kxc::TensorType({c.o}, "int32")), m("m", kxc::TensorType({c.o}, "float32")), r("r", kxc::TensorType({c.n, c.o, oh, ow}, "int8"));
+        auto attrs = kxc::relay::QnnConv2DAttrs::Create({c.s, c.s}, {c.p, c.p}, c.relu, c.res ? res_mult : 0.0);
+        std::vector<Buf> bufs = {I8(x, false), I8(w, false), I32(bias), In(mult)};
+        kxc::Function f = c.res ? kxc::Function({d, wv, b, m, r}, kxc::Call(Op::Get("qnn_conv2d"), {d, wv, b, m, r}, attrs))
+                                : kxc::Function({d, wv, b, m}, kxc::Call(Op::Get("qnn_conv2d"), {d, wv, b, m}, attrs));
+        if (c.res) bufs.push_back(I8(res, false));
+        bufs.push_back(I8(y, true));
+        const std::string name = "qnn_conv2d " + std::to_string(c.c) + "x" + std::to_string(c.h) + "x" + std::to_string(c.w) + " k" +
+                                 std::to_string(c.k) + " s" + std::to_string(c.s);
+        CompileAndRun(name, f, bufs);
+        oracle_conv(x.data(), w.data(), bias.data(), mult.data(), c.res ? res.data() : nullptr, res_mult, want.data(), c.n, c.c, c.h, c.w,
+                    c.o, c.k, c.k, c.s, c.s, c.p, c.p, c.relu ? 1 : 0);
+        int64_t saturated = 0, distinct[256] = {0}, kinds = 0;
+        for (size_t i = 0; i < y.size(); ++i) {
+            Check(y[i] == want[i], name + ": element " + std::to_string(i) + " = " + std::to_string(y[i]) + ", oracle " + std::to_string(want[i]));
+            saturated += want[i] == 127;
+            distinct[static_cast<uint8_t>(want[i])]++;
+        }
+        for (int64_t cnt : distinct) kinds += cnt > 0;
+        Check(kinds > 20, name + ": the case does not spread over the int8 range");
+        std::cout << "[PASS] " << name << " (" << kinds << " distinct values, " << saturated << " at +127)\n";
+    }
+    // ---- dense: float32 result compared as bits
+    for (const auto& s : std::vector<std::array<int64_t, 3>>{{3, 10, 64}, {5, 7, 33}, {1, 1000, 512}}) {
+        const int64_t M = s[0], N = s[1], K = s[2];
+        std::vector<int8_t> a(M * K), bw(N * K);
+        std::vector<int32_t> bias(N);
+        std::vector<float> mult(N), y(M * N, -1.0f), want(M * N, -2.0f);
+        fill_i8(a); fill_i8(bw);
+        for (auto& b : bias) b = static_cast<int32_t>(next() % 20001) - 10000;
+        for (auto& m : mult) m = static_cast<float>(1 + next() % 1000) / 65536.0f;
+        kxc::Var av("a", kxc::TensorType({M, K}, "int8")), bv("b", kxc::TensorType({N, K}, "int8"));
+        kxc::Var cv("c", kxc::TensorType({N}, "int32")), mv("m", kxc::TensorType({N}, "float32"));
+        kxc::Function f({av, bv, cv, mv}, kxc::Call(Op::Get("qnn_dense"), {av, bv, cv, mv}));
+        const std::string name = "qnn_dense " + std::to_string(M) + "x" + std::to_string(K) + " . " + std::to_string(N) + "x" + std::to_string(K);
+        CompileAndRun(name, f, {I8(a, false), I8(bw, false), I32(bias), In(mult), Out(y)});
+        oracle_dense(a.data(), bw.data(), bias.data(), mult.data(), want.data(), M, N, K);
+        Check(std::memcmp(y.data(), want.data(), y.size() * sizeof(float)) == 0, name + " differs from the oracle");
+        std::cout << "[PASS] " << name << "\n";
+    }
+    // ---- quantize against the oracle on values around every tie
+    {
+        const int64_t n = 4096;
+        std::vector<float> x(n);
+        for (int64_t i = 0; i < n; ++i) x[i] = (static_cast<float>(i) - 2048.0f) * 0.0625f * 0.0123f + (i % 3 == 0 ? 0.5f * 0.0123f : 0.0f);
+        std::vector<int8_t> q(n, 99), want(n, 77);
+        kxc::Var xv("x", kxc::TensorType({n}, "float32"));
+        kxc::Function f({xv}, kxc::Call(Op::Get("qnn_quantize"), {xv}, kxc::relay::QnnQuantizeAttrs::Create(0.0123f)));
+        CompileAndRun("qnn_quantize 4096", f, {In(x), I8(q, true)});
+        oracle_quant(x.data(), want.data(), n, 0.0123f);
+        Check(q == want, "qnn_quantize differs from the oracle");
+        std::cout << "[PASS] qnn_quantize 4096\n";
+    }
+    // ---- a quantised chain: quantize -> conv (+relu) -> conv with the first as residual, each stage against the oracle
+    {
+        const int64_t C = 8, H = 12, W = 12;
+        std::vector<float> x(C * H * W), m1(C), m2(C);
+        for (auto& v : x) v = static_cast<float>(static_cast<int>(next() % 2001) - 1000) / 400.0f;
+        std::vector<int8_t> w1(C * C * 9), w2(C * C * 9), y(C * H * W, 99);
+        std::vector<int32_t> b1(C), b2(C);
+        fill_i8(w1); fill_i8(w2);
+        for (int64_t i = 0; i < C; ++i) { b1[i] = static_cast<int32_t>(next() % 801) - 400; b2[i] = static_cast<int32_t>(next() % 801) - 400;
+                                           m1[i] = 0.002f + 0.0001f * static_cast<float>(i); m2[i] = 0.003f - 0.0001f * static_cast<float>(i); }
+        kxc::Var xv("x", kxc::TensorType({1, C, H, W}, "float32")), w1v("w1", kxc::TensorType({C, C, 3, 3}, "int8")), w2v("w2", kxc::TensorType({C, C, 3, 3}, "int8"));
+        kxc::Var b1v("b1", kxc::TensorType({C}, "int32")), b2v("b2", kxc::TensorType({C}, "int32")), m1v("m1", kxc::TensorType({C}, "float32")), m2v("m2", kxc::TensorType({C}, "float32"));
+        kxc::Call q(Op::Get("qnn_quantize"), {xv}, kxc::relay::QnnQuantizeAttrs::Create(0.02));
+        kxc::Call c1(Op::Get("qnn_conv2d"), {q, w1v, b1v, m1v}, kxc::relay::QnnConv2DAttrs::Create({1, 1}, {1, 1}, true));
+        kxc::Call c2(Op::Get("qnn_conv2d"), {c1, w2v, b2v, m2v, q}, kxc::relay::QnnConv2DAttrs::Create({1, 1}, {1, 1}, true, 0.75));
+        kxc::Function f({xv, w1v, b1v, m1v, w2v, b2v, m2v}, c2);
+        CompileAndRun("qnn chain", f, {In(x), I8(w1, false), I32(b1), In(m1), I8(w2, false), I32(b2), In(m2), I8(y, true)});
+        std::vector<int8_t> xq(x.size()), t1(x.size()), want(x.size());
+        oracle_quant(x.data(), xq.data(), static_cast<int64_t>(x.size()), 0.02f);
+        oracle_conv(xq.data(), w1.data(), b1.data(), m1.data(), nullptr, 0.0f, t1.data(), 1, C, H, W, C, 3, 3, 1, 1, 1, 1, 1);
+        oracle_conv(t1.data(), w2.data(), b2.data(), m2.data(), xq.data(), 0.75f, want.data(), 1, C, H, W, C, 3, 3, 1, 1, 1, 1, 1);
+        Check(y == want, "qnn chain differs from the oracle");
+        if (g_mode != "cpu") {
+            // hip: the three operators dispatch to the hand-written int8 launches; hipgen: to generated kernels only
+            int quant = 0, conv = 0;
+            auto module = kxc::api::Compiler::Compile(f, MakeConfig());
+            for (const auto& k : module.GetKernelExecs()) {
+                quant += k.kernel_symbol.find("kxc_quantize_f32_i8") != std::string::npos;
+                conv += k.kernel_symbol.find("kxc_qconv2d_nchw_i8") != std::string::npos;
+            }
+            Check(g_mode == "hip" ? (quant == 1 && conv == 2) : (quant == 0 && conv == 0),
+                  "qnn chain: unexpected dispatch, quantize launches " + std::to_string(quant) + ", conv launches " + std::to_string(conv));
+        }
+        std::cout << "[PASS] qnn chain (quantize, conv, conv + residual)\n";
+    }
+    // ---- type rules
+    {
+        auto expect_throw = [](const std::function<void()>& fn, const std::string& needle) {
+            try { fn(); } catch (const std::exception& e) {
+                Check(std::string(e.what()).find(needle) != std::string::npos, std::string("unexpected message: ") + e.what());
+                return;
+            }
+            throw std::runtime_error("no exception, expected: " + needle);
+        };
+        expect_throw([] {
+            kxc::Var d("d", kxc::TensorType({1, 4, 8, 8}, "float32")), w("w", kxc::TensorType({8, 4, 3, 3}, "int8"));
+            kxc::Var b("b", kxc::TensorType({8}, "int32")), m("m", kxc::TensorType({8}, "float32"));
+            kxc::relay::InferTypePass(kxc::Function({d, w, b, m}, kxc::Call(Op::Get("qnn_conv2d"), {d, w, b, m}, kxc::relay::QnnConv2DAttrs::Create({1, 1}, {1, 1}, false))));
+        }, "int8");
+        expect_throw([] {
+            kxc::Var d("d", kxc::TensorType({1, 4, 8, 8}, "int8")), w("w", kxc::TensorType({8, 4, 3, 3}, "int8"));
+            kxc::Var b("b", kxc::TensorType({7}, "int32")), m("m", kxc::TensorType({8}, "float32"));
+            kxc::relay::InferTypePass(kxc::Function({d, w, b, m}, kxc::Call(Op::Get("qnn_conv2d"), {d, w, b, m}, kxc::relay::QnnConv2DAttrs::Create({1, 1}, {1, 1}, false))));
+        }, "bias");
+        expect_throw([] {
+            kxc::Var d("d", kxc::TensorType({4}, "int8"));
+            kxc::relay::InferTypePass(kxc::Function({d}, kxc::Call(Op::Get("qnn_quantize"), {d}, kxc::relay::QnnQuantizeAttrs::Create(1.0))));
+        }, "float32");
+        std::cout << "[PASS] qnn type rules\n";
+    }
+    dlclose(lib);
+    std::cout << "quantised operators ok (" << g_mode << ")\n";
+    return 0;
+}
+
 // The registry face of the device API and of the plan functions (include/base/registry.h, src/base/device_api.cc:442-658).
 int RunPackedFunc(const std::string& mode) {
     using kxc::PackedFunc; using kxc::Registry; using kxc::RetValue;
@@ -1215,6 +1395,7 @@ int main(int argc, char** argv) {
         if (cmd == "codegen") return RunCodegen();
         if (cmd == "packed_func") return RunPackedFunc(argc > 2 ? argv[2] : "cpu");
         if (cmd == "generated_numeric") return RunGeneratedNumeric();
+        if (cmd == "qnn" && argc >= 4) { g_mode = argv[2]; return RunQnn(argv[3]); }
         if (cmd == "onnx" && argc >= 4) { g_mode = argv[2]; return RunOnnx(argv[3]); }
         if (cmd == "onnx_errors" && argc >= 3) return RunOnnxErrors(argv[2]);
         if (cmd == "hip_smoke" && argc >= 3) return RunHipSmoke(argv[2]);

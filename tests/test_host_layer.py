@@ -58,6 +58,27 @@ def test_packed_function_registry_cpu():
     assert "packed functions ok (cpu)" in run("packed_func", "cpu")
 
 
+def _oracle_so():
+    from oracle_lib import _build_if_missing
+    return _build_if_missing("libkxc_oracle.so")
+
+
+def test_quantised_operators_cpu():
+    """qnn_quantize / qnn_conv2d / qnn_dense as graph operators (type rule, TE compute with the rint intrinsic, host
+    back end): hand-worked answers, and the C oracle on seeded cases, element for element."""
+    out = run("qnn", "cpu", _oracle_so())
+    assert "quantised operators ok (cpu)" in out and out.count("[PASS]") == 13
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("mode", ["hip", "hipgen"])
+def test_quantised_operators_gpu(mode):
+    """The same cases through the hand-written int8 launches (hip) and through kernels generated from the operators'
+    TE compute (hipgen)."""
+    out = run("qnn", mode, _oracle_so())
+    assert "quantised operators ok (%s)" % mode in out and out.count("[PASS]") == 13
+
+
 @pytest.mark.gpu
 def test_generated_kernels_lds_schedules_bit_exact():
     """dense / matmul / reduce_mean shapes that take the generator's LDS-staged schedules (ragged chunks, fewer outputs
