@@ -103,6 +103,9 @@ constexpr int32_t kSplitCounters = 16384;
 constexpr size_t kSplitCounterBytes = static_cast<size_t>(kSplitCounters) * sizeof(uint32_t);
 // Largest number of parts the last arrival finishes itself (0: the adding kernel always does; see split_reduce.hip).
 int32_t SplitFuseMaxParts();
+// Number of equal launches expected to run beside this one on other streams (1: the launch has the GPU to itself).
+// Variant selection sizes its fill rules for that many times the launch's workgroups.
+int32_t SelectLanes();
 
 #if defined(__HIPCC__)
 // Cache policy of the parts' stores and of the last part's loads of partial outputs: device scope (sc1), i.e.

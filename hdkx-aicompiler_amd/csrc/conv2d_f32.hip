@@ -788,9 +788,12 @@ bool Fits(const Variant& v, const ConvArgs& a, Choice* out, bool ds = false) {
 }
 
 // Picks the MFMA variant for a shape, or leaves choice.v == nullptr for the direct kernel.
-void Select(const ConvArgs& a, int kh, int kw, Choice* choice, bool ds = false) {
+void Select(const ConvArgs& real, int kh, int kw, Choice* choice, bool ds = false) {
     choice->v = nullptr;
-    if (a.O < 32 || a.M < 32) return;
+    if (real.O < 32 || real.M < 32) return;
+    // the rules below see the pixels of all launches expected to run side by side
+    ConvArgs a = real;
+    if (static_cast<int64_t>(a.M) * SelectLanes() < (1LL << 31)) a.M *= SelectLanes();
     // 32-bit byte offsets inside the kernel
     const int64_t x_bytes = static_cast<int64_t>(a.N) * a.C * a.H * a.W * 4;
     const int64_t y_elems = static_cast<int64_t>(a.N) * a.O * a.OHW;
@@ -1058,7 +1061,7 @@ int32_t Conv2dResolve(const kxc_hip_conv2d_desc* desc, bool second, const char* 
     a.cps = a.nchunks;
     a.out_elems = total;
     int split = 1;
-    if (!second) SplitOverWorkgroups(c, a.nchunks, tiles, total, &split);      // (a second output is never split)
+    if (!second) SplitOverWorkgroups(c, a.nchunks, tiles * SelectLanes(), total, &split);      // (a second output is never split)
     if (split > 1) {
         a.cps = static_cast<int32_t>(CeilDiv(a.nchunks, split));
         a.gsplit = static_cast<int32_t>(CeilDiv(a.nchunks, a.cps));      // no empty split

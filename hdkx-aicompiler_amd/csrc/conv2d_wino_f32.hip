@@ -83,7 +83,8 @@ __device__ __forceinline__ float load_f32(__amdgpu_buffer_rsrc_t rsrc, uint32_t 
     return __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(rsrc, voffset, soffset, 0));
 }
 
-__device__ __forceinline__ float relu_sel(float v) { return (v > 0.0f) ? v : 0.0f; }
+// max(v, 0) with NaN -> 0, as (v > 0 ? v : 0) gives; one instruction instead of a compare and a select
+__device__ __forceinline__ float relu_sel(float v) { return __builtin_fmaxf(v, 0.0f); }
 
 // ------------------------------------------------------------------------------------------
 // Filter transform, for o < 32*ceil(O/32) (absent output channels give zero blocks).
@@ -204,7 +205,7 @@ wino_kernel(const WinoArgs a) {
 
     // ---- input items: item = tid + i*NTH -> tile = item % TT, channel = (item / TT) % 4, half = item / (4*TT)
     uint32_t goff[ITEMS][12];
-    int vdst[ITEMS];
+    int vdst_a[ITEMS], vdst_b[ITEMS];
 #pragma unroll
     for (int i = 0; i < ITEMS; ++i) {
         const int item = tid + i * NTH;
@@ -224,9 +225,14 @@ wino_kernel(const WinoArgs a) {
             const uint32_t rowmask = (tile < a.NT && ih >= 0 && ih < a.H) ? 0u : kOob;
             const uint32_t row = ((plane + static_cast<uint32_t>(ih)) * static_cast<uint32_t>(a.W) + static_cast<uint32_t>(iw0)) * 4u;
 #pragma unroll
-            for (int j = 0; j < 4; ++j) goff[i][r * 4 + j] = (rowmask | colmask[j]) != 0u ? kOob : row + 4u * j;
+            // (an offset with the top bit set lies beyond the buffer whatever its other bits are)
+            for (int j = 0; j < 4; ++j) goff[i][r * 4 + j] = (row + 4u * j) | rowmask | colmask[j];
         }
-        vdst[i] = ((cl * WT + tile_l / 16) * 4 + 2 * half) * 64 + (tile_l % 16) * 4;
+        // transform rows 2*half and 2*half + 1 of the tile; for half 1 the transform below produces them in the
+        // order (3, 2)
+        const int vrow = ((cl * WT + tile_l / 16) * 4 + 2 * half) * 64 + (tile_l % 16) * 4;
+        vdst_a[i] = vrow + (half ? 64 : 0);
+        vdst_b[i] = vrow + (half ? 0 : 64);
     }
     // ---- weight tile loads: 16-byte unit idx = j*NTH + tid of the tile; block h = idx / 512 is k32 group kg*WK + h
     uint32_t uoff[ULOADS];
@@ -255,22 +261,29 @@ wino_kernel(const WinoArgs a) {
         for (int j = 0; j < ULOADS; ++j)
             load16_to_lds(ur, (lds_ptr_t)(buf + (j * NTH + wave * 64) * 4), uoff[j], static_cast<uint32_t>(s) * 8192u);
     };
+    // On gfx950 the fp32 matrix instructions and the vector ALU share a datapath (measured: an independent v_add_f32
+    // between two v_mfma_f32_16x16x4_f32 costs 4.3 cycles plus about 8 per change of kind; one issued by the other
+    // wave of the SIMD costs 4.8), so every vector instruction of this kernel is paid for in matrix time.
+    // Rows e0, e1, e2 of the patch are rows 0-2 (half 0) or 1-3 (half 1) of the 4x4 input patch d:
+    //   half 0: t0 = d0 - d2 = e0 - e2,  t1 = d1 + d2 = e1 + e2
+    //   half 1: t3 = d1 - d3 = e0 - e2,  t2 = d2 - d1 = e1 - e0
+    // i.e. ta = e0 - e2 and tb = e1 + (half ? -e0 : e2): one select per column instead of both variants and two.
     auto transform = [&](float* buf) {
 #pragma unroll
         for (int i = 0; i < ITEMS; ++i) {
-            const int half = (tid + i * NTH) / (4 * TT);        // uniform over the wave
+            const bool half = (tid + i * NTH) / (4 * TT) != 0;        // uniform over the wave
             float ta[4], tb[4];
 #pragma unroll
             for (int j = 0; j < 4; ++j) {
                 const float e0 = d[i][j], e1 = d[i][4 + j], e2 = d[i][8 + j];
-                ta[j] = half == 0 ? e0 - e2 : e1 - e0;
-                tb[j] = half == 0 ? e1 + e2 : e0 - e2;
+                ta[j] = e0 - e2;
+                tb[j] = e1 + (half ? -e0 : e2);
             }
             floatx4 va, vb;
             va[0] = ta[0] - ta[2]; va[1] = ta[1] + ta[2]; va[2] = ta[2] - ta[1]; va[3] = ta[1] - ta[3];
             vb[0] = tb[0] - tb[2]; vb[1] = tb[1] + tb[2]; vb[2] = tb[2] - tb[1]; vb[3] = tb[1] - tb[3];
-            *reinterpret_cast<floatx4*>(buf + vdst[i]) = va;
-            *reinterpret_cast<floatx4*>(buf + vdst[i] + 64) = vb;
+            *reinterpret_cast<floatx4*>(buf + vdst_a[i]) = va;
+            *reinterpret_cast<floatx4*>(buf + vdst_b[i]) = vb;
         }
     };
     // Operands of one group of four f values: two 16-byte reads of U (output-channel blocks 0 and 1) and one of V.
@@ -281,11 +294,17 @@ wino_kernel(const WinoArgs a) {
         ra[set][1] = *reinterpret_cast<const floatx4*>(ub + a_base + 256 + fg * 64);
         rb[set] = *reinterpret_cast<const floatx4*>(vb + b_base + fg * 64);
     };
-    auto mm = [&](int fg, int set) {
+    // first: the step that starts the accumulators -- C is a constant (0, or the bias for f = 5: m11 has the
+    // coefficient +1 in all four outputs of A^T M A) instead of 128 registers cleared beforehand
+    floatx4 bias4[2];
+    auto mm = [&](int fg, int set, auto first) {
+        constexpr bool FIRST = decltype(first)::value;
+        const floatx4 zero = {0.0f, 0.0f, 0.0f, 0.0f};
 #pragma unroll
         for (int f = 0; f < 4; ++f) {
-            acc[fg * 4 + f][0] = __builtin_amdgcn_mfma_f32_16x16x4f32(ra[set][0][f], rb[set][f], acc[fg * 4 + f][0], 0, 0, 0);
-            acc[fg * 4 + f][1] = __builtin_amdgcn_mfma_f32_16x16x4f32(ra[set][1][f], rb[set][f], acc[fg * 4 + f][1], 0, 0, 0);
+            const int ff = fg * 4 + f;
+            acc[ff][0] = __builtin_amdgcn_mfma_f32_16x16x4f32(ra[set][0][f], rb[set][f], FIRST ? (ff == 5 ? bias4[0] : zero) : acc[ff][0], 0, 0, 0);
+            acc[ff][1] = __builtin_amdgcn_mfma_f32_16x16x4f32(ra[set][1][f], rb[set][f], FIRST ? (ff == 5 ? bias4[1] : zero) : acc[ff][1], 0, 0, 0);
         }
     };
 
@@ -307,56 +326,63 @@ wino_kernel(const WinoArgs a) {
     // ---- prologue: weight tile and transformed input of the first step; raw input of the second in flight
     issue_u(s_lo, ub0);
     load_raw(s_lo);
-    __builtin_amdgcn_sched_barrier(0);
-    // (the 128 accumulator registers are cleared while the first loads are on their way)
+    {
+        // the bias enters through the accumulators (a part of a split reduction adds none: the descriptor is empty)
+        // (of two groups of waves whose accumulators are added, the first brings it)
+        const bool in_acc = a.gsplit == 1 && kgroup == 0 && (a.flags & KXC_HIP_CONV_BIAS) != 0;
+        const __amdgpu_buffer_rsrc_t br = make_rsrc(in_acc ? a.bias : a.x, in_acc ? static_cast<uint32_t>(a.O) * 4u : 0u);
 #pragma unroll
-    for (int f = 0; f < 16; ++f)
+        for (int kb = 0; kb < 2; ++kb)
 #pragma unroll
-        for (int kb = 0; kb < 2; ++kb) acc[f][kb] = floatx4{0.0f, 0.0f, 0.0f, 0.0f};
+            for (int g = 0; g < 4; ++g)
+                bias4[kb][g] = load_f32(br, static_cast<uint32_t>((kg * WK + wave_k) * 32 + kb * 16 + 4 * (lane >> 4) + g) * 4u, 0);
+    }
     __builtin_amdgcn_sched_barrier(0);
     transform(vb0);
     load_raw(min(s_lo + 1, last));
     __builtin_amdgcn_sched_barrier(0);
     __syncthreads();
 
-    for (int s = s_lo; s < s_hi; ++s) {
-        const bool odd = ((s - s_lo) & 1) != 0;
-        const float* const ucur = odd ? ub1 : ub0;
-        const float* const vcur = odd ? vb1 : vb0;
-        float* const unxt = odd ? ub0 : ub1;
-        float* const vnxt = odd ? vb0 : vb1;
-        // Steps past the end re-load the last step (never used), which keeps the loop free of branches.
+    // One step: the tiles of step s are multiplied while those of step s + 1 are made.  A scheduling barrier after
+    // every fetch: left free, the compiler sinks one of the three reads below the matrix instructions of the group
+    // before, to share its registers, and the wave then waits out that read's LDS latency at every change of group.
+    // The transform runs in one block between two groups of matrix instructions (spreading it between them gains
+    // nothing, see transform, and costs a change of kind per piece).
+    auto step = [&](int s, const float* ucur, const float* vcur, float* unxt, float* vnxt, auto first) {
+        // Steps past the end re-load the last step (never used), which keeps the step free of branches.
         issue_u(min(s + 1, last), unxt);
         fetch(ucur, vcur, 0, 0);
         __builtin_amdgcn_sched_barrier(0);
         fetch(ucur, vcur, 1, 1);
-        mm(0, 0);
         __builtin_amdgcn_sched_barrier(0);
-        // group 1 multiplies while the raw input of step s+1 (requested one step ago) is transformed: the vector
-        // instructions are spread between the matrix instructions, which run 8 passes each
+        mm(0, 0, first);
+        __builtin_amdgcn_sched_barrier(0);
         fetch(ucur, vcur, 2, 0);
-        mm(1, 1);
-        transform(vnxt);
-#pragma unroll
-        for (int q = 0; q < 8; ++q) {
-            __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);      // one matrix instruction
-            __builtin_amdgcn_sched_group_barrier(0x002, 6, 0);      // six vector ALU instructions
-        }
+        __builtin_amdgcn_sched_barrier(0);
+        transform(vnxt);       // raw input of step s + 1, requested one step ago
+        __builtin_amdgcn_sched_barrier(0);
+        mm(1, 1, first);
         __builtin_amdgcn_sched_barrier(0);
         fetch(ucur, vcur, 3, 1);
-        mm(2, 0);
+        __builtin_amdgcn_sched_barrier(0);
+        mm(2, 0, first);
         load_raw(min(s + 2, last));
 #pragma unroll
         for (int q = 0; q < 8; ++q) {
-            __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+            __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);      // one matrix instruction
             __builtin_amdgcn_sched_group_barrier(0x020, 2, 0);      // two vector memory reads
         }
         __builtin_amdgcn_sched_barrier(0);
-        mm(3, 1);
+        mm(3, 1, first);
         __builtin_amdgcn_sched_barrier(0);
         __syncthreads();
+    };
+    step(s_lo, ub0, vb0, ub1, vb1, std::true_type{});
+    for (int s = s_lo + 1; s < s_hi; ++s) {
+        const bool odd = ((s - s_lo) & 1) != 0;
+        step(s, odd ? ub1 : ub0, odd ? vb1 : vb0, odd ? ub0 : ub1, odd ? vb0 : vb1, std::false_type{});
     }
-        asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
 
     if (KS > 1) {
         // group 1 parks its accumulators in LDS (the tiles are dead after the loop's last barrier), one
@@ -531,9 +557,9 @@ wino_kernel(const WinoArgs a) {
         }
         return;
     }
-    issue_epilogue_loads(has_bias, has_res, a.y);
+    issue_epilogue_loads(false, has_res, a.y);          // (the bias came in through the accumulators)
     output_transform(yv);
-    finish(yv, has_bias, has_res, do_relu);
+    finish(yv, false, has_res, do_relu);
     store_all(make_rsrc(a.y, y_bytes), yv, Cached{});
 }
 
@@ -611,7 +637,8 @@ const WinoVariant* SelectWino(const kxc_hip_conv2d_desc* d) {
     // Small launches (batch 1-8 of ResNet-18): 64 x 16 groups with the channels split over workgroups beat both
     // the split inside the workgroup and the implicit-GEMM kernel (batch 1, 512 channels: 14.7 against 62.9 and
     // 20.0 us).
-    const int64_t units_t1 = CeilDiv(Tiles(d), 16) * CeilDiv(d->o, 64);
+    const int64_t lanes = SelectLanes();
+    const int64_t units_t1 = CeilDiv(Tiles(d), 16) * CeilDiv(d->o, 64) * lanes;
     if (GroupSplit(units_t1, csteps, static_cast<int64_t>(d->n) * d->o * oh * ow) > 1) {
         for (int i = 0; i < kNumWino; ++i)
             if (kWino[i].wk == 2 && kWino[i].wt == 1 && kWino[i].ks == 1) return &kWino[i];
@@ -619,7 +646,7 @@ const WinoVariant* SelectWino(const kxc_hip_conv2d_desc* d) {
     // 64 x 32 groups from one per compute unit on; below that twice as many 64 x 16 groups.  A launch that cannot
     // give every SIMD two waves (at most one 64 x 32 group per compute unit) and has a long reduction splits the
     // input channels over two groups of waves inside the workgroup instead.
-    const int64_t units = CeilDiv(Tiles(d), 32) * CeilDiv(d->o, 64);
+    const int64_t units = CeilDiv(Tiles(d), 32) * CeilDiv(d->o, 64) * lanes;
     const int wt = units < 256 ? 1 : 2;
     const int ks = (units <= 256 && csteps % 2 == 0 && csteps >= 32) ? 2 : 1;
     for (int i = 0; i < kNumWino; ++i)
@@ -667,7 +694,7 @@ int32_t WinoResolve(const kxc_hip_conv2d_desc* desc, WinoLaunch* L) {
     const int64_t out_elems = static_cast<int64_t>(a.N) * a.O * a.OHW;
     L->out_elems = out_elems;
     if (v->ks == 1) {
-        int split = GroupSplit(a.num_units, a.csteps, out_elems);
+        int split = GroupSplit(static_cast<int64_t>(a.num_units) * SelectLanes(), a.csteps, out_elems);
         if (const char* e = std::getenv("KXC_HIP_WINOGRAD_GSPLIT")) {
             // (a forced split is honoured while its partial outputs stay below 256 MiB)
             const int f = std::atoi(e);

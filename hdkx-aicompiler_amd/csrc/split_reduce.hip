@@ -56,6 +56,12 @@ int32_t SplitFuseMaxParts() {
     return e ? static_cast<int32_t>(std::atoi(e)) : 0;
 }
 
+int32_t SelectLanes() {
+    const char* e = std::getenv("KXC_HIP_SELECT_LANES");
+    const int v = e ? std::atoi(e) : 1;
+    return v >= 1 && v <= 16 ? v : 1;
+}
+
 // A buffer that has been handed out stays allocated until the process ends, also after a larger one replaced it:
 // a captured graph may still hold its address.  Buffers double, so the retired ones add up to less than the
 // current one.
