@@ -118,6 +118,8 @@ def main():
     # The ResNet-18 Relay graph, compiled by the C++ host layer's Compiler::Compile for the "hip" target.
     module = hostapi.CompiledResNet18(batch, 224, "hip", sync_after_run=False)
     info = {"launches": module.launches(), "workspace_bytes": module.workspace_bytes()}
+    # shares of the batch the plan runs side by side on streams of their own (launches of share k end in " @share<k>")
+    shares = 1 + max([int(l.rsplit("@share", 1)[1]) for l in info["launches"] if "@share" in l], default=0)
     tensors = [x] + consts + [out]
     packed = module.packed(tensors)
     stream = torch.cuda.current_stream().cuda_stream
@@ -197,6 +199,35 @@ def main():
                     "traffic": _profiled_traffic_bytes("winograd_layer1_bs64_counters.md") if batch == 64 else None,
                     "traffic_unit": "bytes per launch (FETCH_SIZE + WRITE_SIZE, calibrated on a copy; from profiles/)",
                     "algorithmic_bytes_per_launch": algorithmic_bytes, "same_layer_implicit_gemm": gemm_row}
+        if shares > 1 and batch % shares == 0:
+            # what the plan does with this layer: one launch per share of the batch, side by side on streams of
+            # their own between a fork and a join on the timed stream (variants chosen for `shares` equal launches)
+            part = batch // shares
+            side = [torch.cuda.Stream() for _ in range(shares - 1)]
+            fork = torch.cuda.Event()
+            done = [torch.cuda.Event() for _ in side]
+            prev = pkg.set_select_lanes(shares)
+            try:
+                def pair():
+                    cur = torch.cuda.current_stream()
+                    fork.record(cur)
+                    pkg.conv2d_winograd(lx[:part], lu, lw.shape, lb, None, 1, True, out=ly[:part])
+                    for k, st in enumerate(side):
+                        st.wait_event(fork)
+                        with torch.cuda.stream(st):
+                            lo = (k + 1) * part
+                            pkg.conv2d_winograd(lx[lo:lo + part], lu, lw.shape, lb, None, 1, True, out=ly[lo:lo + part])
+                        done[k].record(st)
+                        cur.wait_event(done[k])
+                pair_ms = _event_time_ms(torch, pair, 30, 5)
+                part_variant = pkg.conv2d_winograd_variant(lx[:part].shape, lw.shape)
+            finally:
+                pkg.set_select_lanes(prev)
+            roofline["side_by_side"] = {
+                "what": "%d launches of [%d,64,56,56] on %d streams, fork to join: the layer as the timed plan runs it" % (shares, part, shares),
+                "variant": part_variant, "ms": round(pair_ms, 4), "achieved": round(conv_flop / (pair_ms * 1e-3) / 1e12, 3),
+                "frac": round(conv_flop / (pair_ms * 1e-3) / 1e12 / PEAK_FP32_MFMA_TFLOPS, 4),
+                "matrix_core_frac": round(executed / (pair_ms * 1e-3) / 1e12 / PEAK_FP32_MFMA_TFLOPS, 4)}
     else:
         roofline = {"bound": "mfma", "kernel": "conv_mfma_kernel<3,3> (layer1: [%d,64,56,56]x[64,64,3,3] s1 p1 +bias+relu)" % batch,
                     "variant": gemm_row["variant"], "achieved": gemm_row["achieved"], "peak": PEAK_FP32_MFMA_TFLOPS,
@@ -214,7 +245,7 @@ def main():
                    "compiled_by": "C++ host layer, Compiler::Compile(Relay graph, target hip)",
                    "constants": "frozen (serving mode: Winograd filter transforms run once, in the warm-up; "
                                 "eager_unfrozen_ms_per_step re-transforms them in every step)",
-                   "launches_per_step": len(info["launches"]), "workspace_bytes": info["workspace_bytes"]},
+                   "batch_shares": shares, "launches_per_step": len(info["launches"]), "workspace_bytes": info["workspace_bytes"]},
         "end_to_end_tflops": round(flop_step / (ms_per_step * 1e-3) / 1e12, 3),
         "end_to_end_frac_of_fp32_mfma_peak": round(flop_step / (ms_per_step * 1e-3) / 1e12 / PEAK_FP32_MFMA_TFLOPS, 4),
         "logits_finite": logits_ok,

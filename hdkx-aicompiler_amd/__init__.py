@@ -14,6 +14,6 @@ from .hipabi import (  # noqa: F401
     conv2d_winograd_supported, conv2d_winograd_preferred, conv2d_winograd_weight_bytes, conv2d_winograd_variant, conv2d_winograd_transform_weights, conv2d_winograd,
     absmax, quantize_to_c4, qconv2d_c4_pack_weights, qconv2d_c4, i8_nchw_to_c16, i8_c16_to_nchw, quantize_to_c16, qconv_desc, qconv2d_c16_variant, qconv2d_c16_pack_weights, qconv2d_c16_pair_supported, qconv2d_c16_pair_pack_weights, qconv2d_c16_pair,
     qconv2d_c16, maxpool2d_c16_i8, global_avg_pool2d_c16_i8, c16_shape, pool_desc, pool_out_shape,
-    device_attributes, Plan, Buf, ConvDesc, PoolDesc, QConvDesc, conv_desc, conv_out_shape,
+    device_attributes, set_select_lanes, Plan, Buf, ConvDesc, PoolDesc, QConvDesc, conv_desc, conv_out_shape,
     CONV_BIAS, CONV_RESIDUAL, CONV_RELU, CONV_FORCE_DIRECT,
 )

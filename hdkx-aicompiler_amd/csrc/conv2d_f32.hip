@@ -927,7 +927,7 @@ bool UseSmall1x1(const kxc_hip_conv2d_desc* d, const ConvArgs& a) {
 // the reduction over workgroups as well; every workgroup keeps at least two chunks per wave group, and the partial
 // sums stay small next to the caches (the split re-reads them once): at most 8 MiB.
 void SplitOverWorkgroups(const Choice& c, int32_t nchunks, int64_t tiles, int64_t total, int* out_split) {
-    const int64_t waves = tiles * c.v->nw * c.v->ks;
+    const int64_t waves = tiles * SelectLanes() * c.v->nw * c.v->ks;      // of all launches expected side by side
     int split = 1;
     while (split < 16 && waves * split < 2048 && nchunks / (split * 2) >= 2 * c.v->ks &&
            total * static_cast<int64_t>(sizeof(float)) * split * 2 <= (8LL << 20))
@@ -1061,7 +1061,7 @@ int32_t Conv2dResolve(const kxc_hip_conv2d_desc* desc, bool second, const char* 
     a.cps = a.nchunks;
     a.out_elems = total;
     int split = 1;
-    if (!second) SplitOverWorkgroups(c, a.nchunks, tiles * SelectLanes(), total, &split);      // (a second output is never split)
+    if (!second) SplitOverWorkgroups(c, a.nchunks, tiles, total, &split);      // (a second output is never split)
     if (split > 1) {
         a.cps = static_cast<int32_t>(CeilDiv(a.nchunks, split));
         a.gsplit = static_cast<int32_t>(CeilDiv(a.nchunks, a.cps));      // no empty split

@@ -39,6 +39,9 @@ struct Node {
     // after it; `join` = this (main-lane) node first waits for every side-lane node enqueued before it
     int32_t lane = 0, join = 0;
     hipEvent_t fork_event = nullptr, done_event = nullptr;
+    // chain > 0: the node belongs to an independent chain of nodes (one share of the batch) that runs on its own
+    // stream from the start of the run to its end, in plan order, beside the main lane and the other chains
+    int32_t chain = 0;
     // Winograd convolution (i32[0] == 1 on a kConv2D node): the weight pointer whose transform bufs[5] holds
     const void* transformed_from = nullptr;
     // convolution launches resolved at finalize (kernel, tile shape, grid, split, environment switches)
@@ -124,6 +127,8 @@ void OperandExtents(const Node& n, std::vector<std::pair<kxc_hip_buf, size_t>>* 
 
 }  // namespace
 
+constexpr int32_t kMaxChains = 7;
+
 struct kxc_hip_plan {
     int32_t device_id = 0;
     int32_t num_args = 0;
@@ -132,6 +137,13 @@ struct kxc_hip_plan {
     size_t workspace_bytes = 0;
     bool finalized = false;
     hipStream_t side_stream = nullptr;     // created at finalize when a node uses lane 1 (default priority)
+    // chains (kxc_hip_plan_set_chain): one stream and one end-of-chain event each, one fork event for all
+    hipStream_t chain_streams[kMaxChains] = {};
+    hipEvent_t chain_done[kMaxChains] = {};
+    hipEvent_t chain_fork = nullptr;
+    int32_t num_chains = 0;
+    // number of equal launches the convolution variants were chosen for (the chains run side by side)
+    int32_t select_lanes = 1;
     // HIP graph replay (kxc_hip_plan_enable_graph): the run after the first one on a capturable stream is
     // captured; later runs with the same argument pointers launch the instantiated graph
     bool graph_enabled = false;
@@ -165,6 +177,13 @@ int32_t CheckBuf(const kxc_hip_plan* p, kxc_hip_buf b, bool optional, const char
                         static_cast<long long>(b.index_or_offset), p->num_args);
         return KXC_HIP_OK;
     }
+    if (b.kind == KXC_HIP_BUF_ARG_OFFSET) {
+        const int64_t arg = b.index_or_offset >> 48, off = b.index_or_offset & ((int64_t{1} << 48) - 1);
+        KXC_HIP_REQUIRE(b.index_or_offset >= 0 && arg < p->num_args, "%s: packed argument index %lld out of range [0,%d)", who,
+                        static_cast<long long>(arg), p->num_args);
+        KXC_HIP_REQUIRE(off % 16 == 0, "%s: the byte offset into a packed argument must be a multiple of 16", who);
+        return KXC_HIP_OK;
+    }
     KXC_HIP_REQUIRE(b.kind == KXC_HIP_BUF_WORKSPACE, "%s: bad buffer kind %d", who, b.kind);
     KXC_HIP_REQUIRE(b.index_or_offset >= 0 && (b.index_or_offset % 256) == 0,
                     "%s: workspace offsets must be non-negative multiples of 256", who);
@@ -174,6 +193,8 @@ int32_t CheckBuf(const kxc_hip_plan* p, kxc_hip_buf b, bool optional, const char
 inline void* Resolve(const kxc_hip_plan* p, kxc_hip_buf b, void** args) {
     if (b.kind == KXC_HIP_BUF_ARG) return args[b.index_or_offset];
     if (b.kind == KXC_HIP_BUF_WORKSPACE) return static_cast<char*>(p->workspace) + b.index_or_offset;
+    if (b.kind == KXC_HIP_BUF_ARG_OFFSET)
+        return static_cast<char*>(args[b.index_or_offset >> 48]) + (b.index_or_offset & ((int64_t{1} << 48) - 1));
     return nullptr;
 }
 
@@ -209,6 +230,11 @@ int32_t kxc_hip_plan_destroy(kxc_hip_plan* plan) {
         if (n.done_event) (void)hipEventDestroy(n.done_event);
     }
     if (plan->side_stream) (void)hipStreamDestroy(plan->side_stream);
+    for (int32_t c = 0; c < kMaxChains; ++c) {
+        if (plan->chain_streams[c]) (void)hipStreamDestroy(plan->chain_streams[c]);
+        if (plan->chain_done[c]) (void)hipEventDestroy(plan->chain_done[c]);
+    }
+    if (plan->chain_fork) (void)hipEventDestroy(plan->chain_fork);
     if (plan->constants_ready) (void)hipEventDestroy(plan->constants_ready);
     if (plan->graph_exec) (void)hipGraphExecDestroy(plan->graph_exec);
     if (plan->graph) (void)hipGraphDestroy(plan->graph);
@@ -618,6 +644,21 @@ int32_t kxc_hip_plan_finalize(kxc_hip_plan* plan, size_t workspace_bytes) {
         KXC_HIP_CALL(hipEventCreateWithFlags(&n.fork_event, hipEventDisableTiming), "plan event");
         KXC_HIP_CALL(hipEventCreateWithFlags(&n.done_event, hipEventDisableTiming), "plan event");
     }
+    for (const Node& n : plan->nodes) plan->num_chains = std::max(plan->num_chains, n.chain);
+    if (plan->num_chains > 0) {
+        KXC_HIP_CALL(hipSetDevice(plan->device_id), "HIP SetDevice");
+        KXC_HIP_CALL(hipEventCreateWithFlags(&plan->chain_fork, hipEventDisableTiming), "plan event");
+        for (int32_t c = 0; c < plan->num_chains; ++c) {
+            KXC_HIP_CALL(hipStreamCreateWithFlags(&plan->chain_streams[c], hipStreamNonBlocking), "plan chain stream");
+            KXC_HIP_CALL(hipEventCreateWithFlags(&plan->chain_done[c], hipEventDisableTiming), "plan event");
+        }
+    }
+    // the variants below are chosen for select_lanes equal launches side by side
+    struct LanesScope {
+        int32_t prev;
+        explicit LanesScope(int32_t lanes) : prev(kxc_hip_set_select_lanes(lanes)) {}
+        ~LanesScope() { kxc_hip_set_select_lanes(prev); }
+    } lanes_scope(plan->select_lanes);
     // Resolve every convolution launch now: the runs only add the operand pointers and the stream.  The node's
     // symbol names the variant resolved here (the one chosen when the node was added may have been picked under
     // other environment switches).
@@ -668,8 +709,12 @@ int32_t TransformConstants(kxc_hip_plan* plan, void** args, hipStream_t stream, 
         if (n.kind != NodeKind::kConv2D || n.i32[0] != 1) continue;
         const void* w = Resolve(plan, n.bufs[1], args);
         if (only_changed && n.transformed_from == w) continue;
-        jobs.push_back({&n.conv, static_cast<const float*>(w), static_cast<float*>(Resolve(plan, n.bufs[5], args))});
         n.transformed_from = w;
+        // (nodes of different chains that share a transformed-weight buffer: one transform)
+        float* const u = static_cast<float*>(Resolve(plan, n.bufs[5], args));
+        bool have = false;
+        for (const WinoWeightJob& j : jobs) have = have || (j.u == u && j.w == w);
+        if (!have) jobs.push_back({&n.conv, static_cast<const float*>(w), u});
     }
     *launched = !jobs.empty();
     if (jobs.empty()) return KXC_HIP_OK;
@@ -842,8 +887,18 @@ int32_t EnqueueAll(kxc_hip_plan* plan, void** args, hipStream_t main_stream) {
         bool launched = false;
         if (int32_t rc = TransformConstants(plan, args, main_stream, false, &launched)) return rc;
     }
+    // chains: everything enqueued on the main stream so far happens before their first node
+    if (plan->num_chains > 0) {
+        KXC_HIP_CALL(hipEventRecord(plan->chain_fork, main_stream), "hipEventRecord");
+        for (int32_t c = 0; c < plan->num_chains; ++c)
+            KXC_HIP_CALL(hipStreamWaitEvent(plan->chain_streams[c], plan->chain_fork, 0), "hipStreamWaitEvent");
+    }
     std::vector<Node*> unjoined;      // side-lane nodes the main lane has not waited for yet
     for (Node& n : plan->nodes) {
+        if (n.chain > 0) {
+            if (int32_t rc = RunNode(plan, n, args, plan->chain_streams[n.chain - 1])) return rc;
+            continue;
+        }
         if (n.lane == 1 && plan->side_stream) {
             // everything enqueued so far on the main lane happens before the side node; the side node then runs
             // concurrently with the main-lane nodes that follow, until a node marked `join`
@@ -861,6 +916,11 @@ int32_t EnqueueAll(kxc_hip_plan* plan, void** args, hipStream_t main_stream) {
         if (int32_t rc = RunNode(plan, n, args, s)) return rc;
     }
     for (Node* side : unjoined) KXC_HIP_CALL(hipStreamWaitEvent(main_stream, side->done_event, 0), "hipStreamWaitEvent");
+    // ... and whatever follows on the main stream happens after their last
+    for (int32_t c = 0; c < plan->num_chains; ++c) {
+        KXC_HIP_CALL(hipEventRecord(plan->chain_done[c], plan->chain_streams[c]), "hipEventRecord");
+        KXC_HIP_CALL(hipStreamWaitEvent(main_stream, plan->chain_done[c], 0), "hipStreamWaitEvent");
+    }
     return KXC_HIP_OK;
 }
 
@@ -938,6 +998,25 @@ int32_t kxc_hip_plan_set_concurrency(kxc_hip_plan* plan, int32_t node, int32_t l
     return KXC_HIP_OK;
 }
 
+int32_t kxc_hip_plan_set_chain(kxc_hip_plan* plan, int32_t node, int32_t chain) {
+    const char* who = "kxc_hip_plan_set_chain";
+    KXC_PLAN_BEGIN(who);
+    KXC_HIP_REQUIRE(node >= 0 && node < static_cast<int32_t>(plan->nodes.size()), "%s: node %d out of range", who, node);
+    KXC_HIP_REQUIRE(chain >= 0 && chain <= kMaxChains, "%s: chain must be in [0, %d]", who, kMaxChains);
+    KXC_HIP_REQUIRE(chain == 0 || (plan->nodes[node].lane == 0 && plan->nodes[node].join == 0),
+                    "%s: a node of a chain takes no part in the side lane", who);
+    plan->nodes[node].chain = chain;
+    return KXC_HIP_OK;
+}
+
+int32_t kxc_hip_plan_set_select_lanes(kxc_hip_plan* plan, int32_t lanes) {
+    const char* who = "kxc_hip_plan_set_select_lanes";
+    KXC_PLAN_BEGIN(who);
+    KXC_HIP_REQUIRE(lanes >= 1 && lanes <= 16, "%s: lanes must be in [1, 16]", who);
+    plan->select_lanes = lanes;
+    return KXC_HIP_OK;
+}
+
 int32_t kxc_hip_plan_run_profiled(kxc_hip_plan* plan, void** args, void* stream, kxc_hip_launch_record* records,
                                   int32_t capacity, int32_t* count) {
     const char* who = "kxc_hip_plan_run_profiled";
@@ -1001,8 +1080,10 @@ int32_t kxc_hip_plan_serialize(const kxc_hip_plan* plan, char* buffer, size_t ca
     char tmp[96];
     auto I = [&](long long v) { std::snprintf(tmp, sizeof(tmp), " %lld", v); out += tmp; };
     auto F = [&](float v) { std::snprintf(tmp, sizeof(tmp), " %a", static_cast<double>(v)); out += tmp; };
-    out += "kxc_hip_plan 1";
+    // (version 2 added the plan's select_lanes and every node's chain)
+    out += "kxc_hip_plan 2";
     I(plan->num_args); I(static_cast<long long>(plan->workspace_bytes)); I(static_cast<long long>(plan->nodes.size()));
+    I(plan->select_lanes);
     out += "\n";
     for (const Node& n : plan->nodes) {
         KXC_HIP_REQUIRE(n.symbol.find_first_of(" \n\t") == std::string::npos,
@@ -1032,7 +1113,7 @@ int32_t kxc_hip_plan_serialize(const kxc_hip_plan* plan, char* buffer, size_t ca
         for (uint32_t v : n.grid) I(v);
         for (uint32_t v : n.block) I(v);
         I(n.shared_bytes);
-        I(n.lane); I(n.join);
+        I(n.lane); I(n.join); I(n.chain);
         I(static_cast<long long>(n.params.size()));
         for (const kxc_hip_buf& b : n.params) { I(b.kind); I(b.index_or_offset); }
         out += "\n";
@@ -1051,12 +1132,16 @@ int32_t kxc_hip_plan_deserialize(const char* text, int32_t device_id, kxc_hip_mo
     std::istringstream in{std::string(text)};
     std::string magic;
     long long version = 0, num_args = 0, workspace = 0, count = 0;
+    long long select_lanes = 1;
     in >> magic >> version >> num_args >> workspace >> count;
-    KXC_HIP_REQUIRE(in && magic == "kxc_hip_plan" && version == 1, "%s: not a version-1 plan", who);
+    if (in && version == 2) in >> select_lanes;
+    KXC_HIP_REQUIRE(in && magic == "kxc_hip_plan" && (version == 1 || version == 2), "%s: not a version-1 or version-2 plan", who);
+    KXC_HIP_REQUIRE(select_lanes >= 1 && select_lanes <= 16, "%s: implausible header", who);
     KXC_HIP_REQUIRE(num_args >= 0 && num_args < (1 << 20) && workspace >= 0 && count >= 0 && count < (1 << 24),
                     "%s: implausible header", who);
     kxc_hip_plan* plan = nullptr;
     if (int32_t rc = kxc_hip_plan_create(device_id, static_cast<int32_t>(num_args), &plan)) return rc;
+    plan->select_lanes = static_cast<int32_t>(select_lanes);
     auto fail = [&](const char* what) {
         kxc_hip_plan_destroy(plan);
         return Fail(KXC_HIP_ERR_INVALID, "%s: %s", who, what);
@@ -1090,7 +1175,10 @@ int32_t kxc_hip_plan_deserialize(const char* text, int32_t device_id, kxc_hip_mo
         for (uint32_t& b : n.block) b = static_cast<uint32_t>(I());
         n.shared_bytes = static_cast<uint32_t>(I());
         n.lane = static_cast<int32_t>(I()); n.join = static_cast<int32_t>(I());
-        if (n.lane < 0 || n.lane > 1 || n.join < 0 || n.join > 1) return fail("bad concurrency flags");
+        if (version >= 2) n.chain = static_cast<int32_t>(I());
+        if (n.lane < 0 || n.lane > 1 || n.join < 0 || n.join > 1 || n.chain < 0 || n.chain > kMaxChains ||
+            (n.chain > 0 && (n.lane || n.join)))
+            return fail("bad concurrency flags");
         const long long np = I();
         if (!in || np < 0 || np > 4096) return fail("bad parameter count");
         for (long long i = 0; i < np; ++i) {
@@ -1102,6 +1190,8 @@ int32_t kxc_hip_plan_deserialize(const char* text, int32_t device_id, kxc_hip_mo
         auto buf_ok = [&](const kxc_hip_buf& b) {
             if (b.kind == KXC_HIP_BUF_ARG) return b.index_or_offset >= 0 && b.index_or_offset < num_args;
             if (b.kind == KXC_HIP_BUF_WORKSPACE) return b.index_or_offset >= 0 && b.index_or_offset < workspace;
+            if (b.kind == KXC_HIP_BUF_ARG_OFFSET)
+                return b.index_or_offset >= 0 && (b.index_or_offset >> 48) < num_args && (b.index_or_offset & 15) == 0;
             return b.kind == KXC_HIP_BUF_NONE;
         };
         for (const kxc_hip_buf& b : n.bufs) if (!buf_ok(b)) return fail("buffer operand out of range");

@@ -56,10 +56,15 @@ int32_t SplitFuseMaxParts() {
     return e ? static_cast<int32_t>(std::atoi(e)) : 0;
 }
 
+// Set per thread (kxc_hip_set_select_lanes: a launch plan sets it while it resolves its launches, a graph builder
+// while it asks which variant a shape would take); KXC_HIP_SELECT_LANES overrides it for measurements.
+thread_local int32_t g_select_lanes = 1;
 int32_t SelectLanes() {
-    const char* e = std::getenv("KXC_HIP_SELECT_LANES");
-    const int v = e ? std::atoi(e) : 1;
-    return v >= 1 && v <= 16 ? v : 1;
+    if (const char* e = std::getenv("KXC_HIP_SELECT_LANES")) {
+        const int v = std::atoi(e);
+        if (v >= 1 && v <= 16) return v;
+    }
+    return g_select_lanes;
 }
 
 // A buffer that has been handed out stays allocated until the process ends, also after a larger one replaced it:
@@ -108,3 +113,9 @@ int32_t LaunchSplitReduce(hipStream_t stream, const SplitReduceArgs& a) {
 }
 
 }  // namespace kxc_hip
+
+extern "C" int32_t kxc_hip_set_select_lanes(int32_t lanes) {
+    const int32_t prev = kxc_hip::g_select_lanes;
+    kxc_hip::g_select_lanes = lanes < 1 ? 1 : (lanes > 16 ? 16 : lanes);
+    return prev;
+}

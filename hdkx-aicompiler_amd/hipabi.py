@@ -14,7 +14,7 @@ _LIB_PATH = os.environ.get("KXC_HIP_LIB") or os.path.join(PKG, "lib", "libkxc_hi
 _lib = None
 
 CONV_BIAS, CONV_RESIDUAL, CONV_RELU, CONV_FORCE_DIRECT = 1, 2, 4, 0x100
-BUF_ARG, BUF_WORKSPACE, BUF_NONE = 0, 1, 2
+BUF_ARG, BUF_WORKSPACE, BUF_NONE, BUF_ARG_OFFSET = 0, 1, 2, 3
 
 
 class KxcHipError(RuntimeError):
@@ -50,6 +50,11 @@ class Buf(C.Structure):
     @staticmethod
     def none():
         return Buf(BUF_NONE, 0)
+
+    @staticmethod
+    def arg_offset(i, nbytes):
+        """packed argument i plus a byte offset (a multiple of 16): one share of a batched argument"""
+        return Buf(BUF_ARG_OFFSET, (i << 48) | nbytes)
 
 
 class DeviceAttrs(C.Structure):
@@ -201,6 +206,12 @@ def conv2d_winograd_weight_bytes(x_shape, w_shape, pad=1):
     nbytes = C.c_size_t(0)
     _check(lib().kxc_hip_conv2d_winograd_weight_bytes(C.byref(d), C.byref(nbytes)))
     return nbytes.value
+
+
+def set_select_lanes(lanes):
+    """Variant selection of this thread's stand-alone launches and queries assumes `lanes` equal launches side by
+    side (kxc_hip_set_select_lanes); returns the previous value."""
+    return int(lib().kxc_hip_set_select_lanes(C.c_int32(lanes)))
 
 
 def conv2d_winograd_variant(x_shape, w_shape, stride=1, pad=1, dil=1):
@@ -656,6 +667,16 @@ class Plan:
 
     def enable_graph(self, enable=True):
         _check(lib().kxc_hip_plan_enable_graph(self._h, C.c_int32(1 if enable else 0)))
+
+    def set_chain(self, node, chain):
+        """Node `node` runs on the plan's chain stream `chain` (1-7), beside the main lane (kxc_hip_plan_set_chain)."""
+        _check(lib().kxc_hip_plan_set_chain(self._h, C.c_int32(node), C.c_int32(chain)))
+
+    def set_select_lanes(self, lanes):
+        _check(lib().kxc_hip_plan_set_select_lanes(self._h, C.c_int32(lanes)))
+
+    def num_nodes(self):
+        return int(lib().kxc_hip_plan_num_nodes(self._h))
 
     def finalize(self, workspace_bytes):
         _check(lib().kxc_hip_plan_finalize(self._h, C.c_size_t(workspace_bytes)))

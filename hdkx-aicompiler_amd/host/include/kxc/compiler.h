@@ -38,6 +38,11 @@ struct CompileConfigNode {
     bool hip_concurrent_branches{true};   // run a block's downsample convolution beside its first 3x3 convolution
     bool hip_pair_convolutions{true};     // a block's 1x1 downsample as a second output of its first convolution's launch
     bool hip_winograd{true};              // 3x3 stride-1 convolutions with constant weights as Winograd F(2x2,3x3) where faster
+    // Shares of the batch that run side by side on streams of their own inside one launch plan (each share is the
+    // whole graph on batch / lanes samples; the kernels of one share fill the compute units the other's leave idle
+    // at the end of every launch).  0: two for batches of 64 samples and more when the graph is separable along the
+    // batch (relay::SplitBatch), else one; 1: never; 2..8: that many (Compile throws when the graph does not allow it).
+    int hip_batch_lanes{0};
     // Winograd layers transform their (constant) filters on the GPU.  false (default): at the start of every Run, from
     // the pointers passed to that Run, so a Run always sees the constants' current contents, like the CPU back end.
     // true: once, when a pointer is first seen -- the caller promises not to change the weights behind the module's

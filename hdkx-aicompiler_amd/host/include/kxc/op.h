@@ -237,6 +237,15 @@ std::string CastDTypeFromCode(int code);
 
 // InferTypePass (src/relay/transforms/infer_type.cc:41-222): fills checked_type_ of every node.
 Function InferTypePass(const Function& f);
+// The same function on 1/lanes of the batch: parameter 0 (the only parameter that may carry the batch) gets a
+// leading extent divided by `lanes`, constants are shared, every call keeps its operator and attributes.  Returns an
+// undefined Function when the graph cannot be proven separable along the batch: every operator between parameter 0
+// and the result must treat the leading axis of a batched operand as independent samples (convolutions, pools,
+// dense / gemm / matmul on the left operand, element-wise operators with broadcast operands that have no batch
+// axis, flatten, softmax / reduce_mean / transpose that leave axis 0 alone, cast, the quantised operators), the
+// result must carry the batch, and the batch must divide.  `f` must be typed; the result is typed.  (No counterpart
+// in the reference; used by the hip back end to run the shares of a batch side by side.)
+Function SplitBatch(const Function& f, int lanes);
 
 }  // namespace relay
 }  // namespace kxc

@@ -203,14 +203,43 @@ int64_t TypeBytes(const Type& t) { return Product(TT(t)->shape) * tir::DTypeFrom
 
 class HipBuilder {
 public:
-    HipBuilder(const Function& f, const CompileConfig& cfg, CompiledModuleImpl* m, bool dry) : f_(f), cfg_(cfg), m_(m), dry_(dry) {}
+    // lanes > 1: `f` is one share of the batch (relay::SplitBatch) and is emitted `lanes` times into the one plan,
+    // share k as chain k of the plan, on the k-th part of parameter 0 and of the result
+    HipBuilder(const Function& f, const CompileConfig& cfg, CompiledModuleImpl* m, bool dry, int lanes = 1)
+        : f_(f), cfg_(cfg), m_(m), dry_(dry), lanes_(lanes) {}
 
     void Build() {
         Number();
         FormGroups();
         if (kxc_hip_plan_create(cfg_->target->device.device_id(), static_cast<int32_t>(num_args_), &m_->plan))
             throw std::runtime_error(std::string("plan creation failed: ") + kxc_hip_last_error());
-        Emit();
+        // variants are chosen for `lanes` equal launches side by side: by the queries made while the plan is built
+        // (this thread) and by the plan when it is finalized
+        struct LanesScope {
+            int32_t prev;
+            explicit LanesScope(int32_t lanes) : prev(kxc_hip_set_select_lanes(lanes)) {}
+            ~LanesScope() { kxc_hip_set_select_lanes(prev); }
+        } lanes_scope(lanes_);
+        if (lanes_ > 1) {
+            if (kxc_hip_plan_set_select_lanes(m_->plan, lanes_)) throw std::runtime_error(std::string("plan_set_select_lanes failed: ") + kxc_hip_last_error());
+            in_share_bytes_ = TypeBytes(f_->params[0].checked_type());
+            out_share_bytes_ = TypeBytes(f_->body.checked_type());
+        }
+        for (lane_ = 0; lane_ < lanes_; ++lane_) {
+            // a share's activations live in workspace regions of its own (the shares run at the same time)
+            arena_.free_list.clear();
+            slot_.clear();
+            alias_.clear();
+            persistent_cursor_ = 0;
+            const int32_t first_node = kxc_hip_plan_num_nodes(m_->plan);
+            const size_t first_exec = m_->execs.size();
+            Emit();
+            if (lane_ == 0) continue;
+            for (int32_t node = first_node; node < kxc_hip_plan_num_nodes(m_->plan); ++node)
+                if (kxc_hip_plan_set_chain(m_->plan, node, lane_))
+                    throw std::runtime_error(std::string("plan_set_chain failed: ") + kxc_hip_last_error());
+            for (size_t e = first_exec; e < m_->execs.size(); ++e) m_->execs[e].kernel_symbol += " @share" + std::to_string(lane_);
+        }
         m_->workspace_bytes = static_cast<size_t>(arena_.top);
         if (!dry_) {
             if (kxc_hip_plan_finalize(m_->plan, m_->workspace_bytes))
@@ -308,7 +337,11 @@ private:
     relay::HIPBuffer BufferOf(const RelayExprNode* e) {
         e = Resolve(e);
         auto a = arg_index_.find(e);
-        if (a != arg_index_.end()) return {KXC_HIP_BUF_ARG, a->second};
+        if (a != arg_index_.end()) {
+            if (lanes_ > 1 && e == f_->params[0].get())
+                return {KXC_HIP_BUF_ARG_OFFSET, KXC_HIP_ARG_OFFSET(a->second, lane_ * in_share_bytes_)};
+            return {KXC_HIP_BUF_ARG, a->second};
+        }
         auto s = slot_.find(e);
         if (s == slot_.end()) {
             const auto* c = dynamic_cast<const CallNode*>(e);
@@ -384,7 +417,9 @@ private:
         std::vector<int> side_join(groups_.size(), -1);
         std::vector<bool> joins(groups_.size(), false);
         const char* conc_env = std::getenv("KXC_HIP_CONCURRENT_BRANCHES");     // "0" switches the side lane off
-        if (cfg_->hip_fuse && cfg_->hip_use_handwritten && cfg_->hip_concurrent_branches && !dry_ && !(conc_env && conc_env[0] == '0')) {
+        // (the shares of a batch already overlap: no side lane inside a share)
+        if (cfg_->hip_fuse && cfg_->hip_use_handwritten && cfg_->hip_concurrent_branches && !dry_ && lanes_ == 1 &&
+            !(conc_env && conc_env[0] == '0')) {
             for (size_t step = 1; step < order.size(); ++step) {
                 const Group& g = groups_[order[step]];
                 const Group& prev = groups_[order[step - 1]];
@@ -451,6 +486,7 @@ private:
             relay::HIPBuffer out;
             if (g.tail == f_->body.get()) {
                 out = {KXC_HIP_BUF_ARG, num_args_ - 1};
+                if (lanes_ > 1) out = {KXC_HIP_BUF_ARG_OFFSET, KXC_HIP_ARG_OFFSET(num_args_ - 1, lane_ * out_share_bytes_)};
             } else {
                 slot_[g.tail] = arena_.Alloc(TypeBytes(g.tail->checked_type_));
                 out = {KXC_HIP_BUF_WORKSPACE, slot_[g.tail].first};
@@ -465,11 +501,15 @@ private:
             const char* wino_env = std::getenv("KXC_HIP_WINOGRAD");                 // "0" switches Winograd off
             if (cfg_->hip_winograd && !(wino_env && wino_env[0] == '0'))
                 ctx.alloc_persistent = [this](int64_t bytes) {
+                    // (the shares of a batch ask in the same order and share what the first one got: transformed
+                    // weights do not depend on the batch)
+                    if (lane_ > 0 && persistent_cursor_ < persistent_.size()) return persistent_[persistent_cursor_++];
                     // above everything handed out so far and never released: no activation of an earlier or later
                     // step ever shares the region, so what the first run wrote there is still valid in the next
                     const int64_t off = arena_.top;
                     arena_.top += (std::max<int64_t>(bytes, 1) + 255) / 256 * 256;
-                    return relay::HIPBuffer{KXC_HIP_BUF_WORKSPACE, off};
+                    persistent_.push_back(relay::HIPBuffer{KXC_HIP_BUF_WORKSPACE, off});
+                    return persistent_.back();
                 };
             const Group* carried = carries[order[step]] >= 0 ? &groups_[carries[order[step]]] : nullptr;
             if (carried) {
@@ -550,7 +590,7 @@ private:
         tir::PrimFunc pf = tir::RunTIRPassPipeline(lowered.func, {"fold_constant", "simplify_expr"});
         codegen::CodeGenHIP cg;
         codegen::HIPModuleSource src = cg.Generate(pf, "kxc_g" + std::to_string(step));
-        m_->source += src.source;
+        if (!compiled_.count(src.source)) m_->source += src.source;
         // buffers: mini-function parameters map to the group's operands, intermediates to scratch slots
         std::unordered_map<const tir::ExprNode*, relay::HIPBuffer> buf;
         for (size_t i = 0; i < g.head->args.size(); ++i) buf[pf->params[i].get()] = ctx.inputs[i];
@@ -562,15 +602,22 @@ private:
         }
         kxc_hip_module* module = nullptr;
         std::vector<char> log(16384, 0);
-        m_->module_sources.push_back(src.source);
-        if (dry_) {
-            size_t size = 0;
-            if (kxc_hip_module_compile_only(src.source.c_str(), "kxc_generated.hip", &size, log.data(), log.size()))
-                throw std::runtime_error(std::string("generated HIP source does not compile: ") + kxc_hip_last_error());
+        // (the shares of a batch generate the same source for the same step: compiled once)
+        auto cached = compiled_.find(src.source);
+        if (cached != compiled_.end()) {
+            module = cached->second;
         } else {
-            if (kxc_hip_module_compile(src.source.c_str(), "kxc_generated.hip", &module, log.data(), log.size()))
-                throw std::runtime_error(std::string("generated HIP source does not compile: ") + kxc_hip_last_error());
-            m_->modules.push_back(module);
+            m_->module_sources.push_back(src.source);
+            if (dry_) {
+                size_t size = 0;
+                if (kxc_hip_module_compile_only(src.source.c_str(), "kxc_generated.hip", &size, log.data(), log.size()))
+                    throw std::runtime_error(std::string("generated HIP source does not compile: ") + kxc_hip_last_error());
+            } else {
+                if (kxc_hip_module_compile(src.source.c_str(), "kxc_generated.hip", &module, log.data(), log.size()))
+                    throw std::runtime_error(std::string("generated HIP source does not compile: ") + kxc_hip_last_error());
+                m_->modules.push_back(module);
+            }
+            compiled_[src.source] = module;
         }
         for (const auto& k : src.kernels) {
             KernelExecInfo e = info;
@@ -597,6 +644,11 @@ private:
     const CompileConfig& cfg_;
     CompiledModuleImpl* m_;
     bool dry_;
+    int lanes_ = 1, lane_ = 0;
+    int64_t in_share_bytes_ = 0, out_share_bytes_ = 0;
+    std::vector<relay::HIPBuffer> persistent_;
+    size_t persistent_cursor_ = 0;
+    std::unordered_map<std::string, kxc_hip_module*> compiled_;
     int next_value_ = 0, num_inputs_ = 0, num_args_ = 0;
     std::unordered_map<const RelayExprNode*, int> value_id_, arg_index_;
     std::vector<const RelayExprNode*> constants_;
@@ -673,8 +725,28 @@ CompiledModule Compiler::Compile(Function func, CompileConfig config) {
             e.event_type = "build_plan";
             e.device = "hip:" + std::to_string(config->target->device.device_id());
             profiling::ScopedSpan span = profiling::CurrentSpan(e);
-            HipBuilder builder(typed, config, impl.get(), dry);
+            // shares of the batch side by side (CompileConfigNode::hip_batch_lanes; KXC_HIP_BATCH_LANES overrides)
+            int want = config->hip_batch_lanes;
+            if (const char* e = std::getenv("KXC_HIP_BATCH_LANES")) want = std::atoi(e);
+            if (want < 0 || want > 8) throw std::runtime_error("hip_batch_lanes must be in [0, 8]");
+            Function share;
+            int lanes = 1;
+            if (want != 1 && config->hip_use_handwritten && !typed->params.empty()) {
+                const auto* t0 = typed->params[0].checked_type().As<TensorTypeNode>();
+                const int64_t batch = t0 && !t0->shape.empty() ? t0->shape[0] : 0;
+                const int ask = want == 0 ? (batch >= 64 ? 2 : 1) : want;
+                if (ask > 1) {
+                    share = relay::SplitBatch(typed, ask);
+                    if (share.defined() && (TypeBytes(share->params[0].checked_type()) % 16 != 0 || TypeBytes(share->body.checked_type()) % 16 != 0))
+                        share = Function();       // a share of an argument must start on a 16-byte boundary
+                    if (share.defined()) lanes = ask;
+                    else if (want > 1)
+                        throw std::runtime_error("hip_batch_lanes = " + std::to_string(want) + ": the graph cannot be split along the batch of parameter 0");
+                }
+            }
+            HipBuilder builder(lanes > 1 ? share : typed, config, impl.get(), dry, lanes);
             builder.Build();
+            span.AddMetric("batch_lanes", static_cast<double>(lanes));
             span.AddMetric("launches", static_cast<double>(impl->execs.size()));
             span.AddMetric("workspace_bytes", static_cast<double>(impl->workspace_bytes));
         }

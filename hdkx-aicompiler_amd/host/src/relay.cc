@@ -499,5 +499,142 @@ Function InferTypePass(const Function& f) {
     return f;
 }
 
+// ---------------------------------------------------------------- SplitBatch
+namespace {
+struct SplitState {
+    int64_t batch = 0;
+    std::unordered_map<const RelayExprNode*, bool> batched;     // value carries the batch on axis 0
+    std::unordered_map<const RelayExprNode*, Expr> clone;
+};
+
+const TensorTypeNode* TTy(const Expr& e) { return e.checked_type().As<TensorTypeNode>(); }
+
+// an operand without the batch beside a batched one of rank `rank`: it must broadcast along axis 0
+bool BroadcastsOverBatch(const Expr& shared, size_t rank) {
+    const auto* t = TTy(shared);
+    return t && (t->shape.size() < rank || (t->shape.size() == rank && t->shape[0] == 1));
+}
+
+// Clones `e` for one share of the batch; false when the graph is not separable.
+bool SplitExpr(const Expr& e, SplitState* st, Expr* out) {
+    auto it = st->clone.find(e.get());
+    if (it != st->clone.end()) { *out = it->second; return true; }
+    if (e.As<ConstantNode>()) {
+        st->batched[e.get()] = false;
+        st->clone[e.get()] = e;          // shared between the shares
+        *out = e;
+        return true;
+    }
+    const auto* call = e.As<CallNode>();
+    const auto* op = call ? call->op.As<OpNode>() : nullptr;
+    if (!op || !TTy(e)) return false;
+    Array<Expr> args;
+    std::vector<bool> b;
+    for (const auto& a : call->args) {
+        Expr c;
+        if (!SplitExpr(a, st, &c)) return false;
+        args.push_back(c);
+        b.push_back(st->batched.at(a.get()));
+    }
+    const std::string& name = op->name;
+    const size_t n = b.size();
+    bool any = false;
+    for (bool x : b) any = any || x;
+    bool result_batched = false;
+    if (!any) {
+        result_batched = false;        // no operand depends on the batch: every share computes the same value
+    } else {
+        const auto* t0 = TTy(call->args[0]);
+        if (!t0 || t0->shape.empty()) return false;
+        const size_t rank0 = t0->shape.size();
+        auto only_first = [&]() -> bool { for (size_t i = 1; i < n; ++i) if (b[i]) return false; return b[0]; };
+        if (name == "nn_conv2d" || name == "nn_dense" || name == "matmul" || name == "qnn_dense") {
+            if (!only_first()) return false;
+        } else if (name == "qnn_conv2d") {
+            // data [, weight, bias, mult] [, residual of the output's shape]
+            for (size_t i = 1; i < n; ++i) if (b[i] && i != 4) return false;
+            if (!b[0] || (n == 5 && !b[4])) return false;
+        } else if (name == "nn_gemm") {
+            const auto* g = call->attrs.As<GemmAttrsNode>();
+            if (!only_first() || (g && g->transA != 0)) return false;
+            if (n == 3 && !BroadcastsOverBatch(call->args[2], 2)) return false;
+        } else if (name == "nn_relu" || name == "sqrt" || name == "exp" || name == "log" || name == "cast" ||
+                   name == "qnn_quantize" || name == "nn_max_pool2d" || name == "nn_avg_pool2d" ||
+                   name == "nn_global_avg_pool2d") {
+            if (n != 1) return false;
+        } else if (name == "add" || name == "subtract" || name == "mul" || name == "multiply" || name == "divide") {
+            if (n != 2) return false;
+            const auto* t1 = TTy(call->args[1]);
+            if (!t1) return false;
+            if (b[0] && b[1]) {
+                if (rank0 != t1->shape.size() || t0->shape[0] != st->batch || t1->shape[0] != st->batch) return false;
+            } else {
+                const Expr& shared = b[0] ? call->args[1] : call->args[0];
+                const size_t rank = b[0] ? rank0 : t1->shape.size();
+                if (!BroadcastsOverBatch(shared, rank)) return false;
+            }
+        } else if (name == "nn_flatten") {
+            const auto* a = call->attrs.As<FlattenAttrsNode>();
+            if (!a || a->axis < 1) return false;
+        } else if (name == "softmax") {
+            const auto* a = call->attrs.As<SoftmaxAttrsNode>();
+            const int64_t axis = a ? (a->axis < 0 ? a->axis + static_cast<int64_t>(rank0) : a->axis) : static_cast<int64_t>(rank0) - 1;
+            if (axis == 0) return false;
+        } else if (name == "reduce_mean") {
+            const auto* a = call->attrs.As<ReduceMeanAttrsNode>();
+            if (!a || a->axes.empty()) return false;
+            for (int64_t ax : a->axes) if (ax == 0 || ax + static_cast<int64_t>(rank0) == 0) return false;
+        } else if (name == "transpose") {
+            const auto* a = call->attrs.As<TransposeAttrsNode>();
+            if (!a || a->axes.empty() || a->axes[0] != 0) return false;
+        } else {
+            return false;      // (reshape and operators this list does not know keep the batch whole)
+        }
+        const auto* to = TTy(e);
+        if (to->shape.empty() || to->shape[0] != st->batch) return false;
+        result_batched = true;
+    }
+    Call c(call->op, args, call->attrs);
+    st->batched[e.get()] = result_batched;
+    st->clone[e.get()] = c;
+    *out = c;
+    return true;
+}
+}  // namespace
+
+Function SplitBatch(const Function& f, int lanes) {
+    if (!f.defined() || lanes < 2 || f->params.empty()) return Function();
+    const auto* t0 = f->params[0].checked_type().As<TensorTypeNode>();
+    if (!t0 || t0->shape.empty() || t0->shape[0] < lanes || t0->shape[0] % lanes != 0) return Function();
+    SplitState st;
+    st.batch = t0->shape[0];
+    Array<Var> params;
+    for (size_t i = 0; i < f->params.size(); ++i) {
+        const Var& p = f->params[i];
+        const auto* t = p.checked_type().As<TensorTypeNode>();
+        if (!t) return Function();
+        std::vector<int64_t> shape = t->shape;
+        if (i == 0) shape[0] /= lanes;
+        Var v(p->vid->name_hint, TensorType(shape, t->dtype));
+        params.push_back(v);
+        st.batched[p.get()] = i == 0;
+        st.clone[p.get()] = v;
+    }
+    Expr body;
+    if (!SplitExpr(f->body, &st, &body) || !st.batched.at(f->body.get())) return Function();
+    Function share(params, body);
+    try {
+        share = InferTypePass(share);
+    } catch (const std::exception&) {
+        return Function();
+    }
+    const auto* full = f->body.checked_type().As<TensorTypeNode>();
+    const auto* part = share->body.checked_type().As<TensorTypeNode>();
+    if (!full || !part || full->shape.size() != part->shape.size() || part->shape[0] * lanes != full->shape[0]) return Function();
+    for (size_t i = 1; i < full->shape.size(); ++i)
+        if (full->shape[i] != part->shape[i]) return Function();
+    return share;
+}
+
 }  // namespace relay
 }  // namespace kxc

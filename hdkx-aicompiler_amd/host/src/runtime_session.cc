@@ -234,6 +234,7 @@ RuntimeSession::RuntimeSession(Function relay_func, api::CompileConfig config,
     internal_config_->hip_fuse = config->hip_fuse;
     internal_config_->hip_concurrent_branches = config->hip_concurrent_branches;
     internal_config_->hip_winograd = config->hip_winograd;
+    internal_config_->hip_batch_lanes = config->hip_batch_lanes;
     internal_config_->hip_pair_convolutions = config->hip_pair_convolutions;
     internal_config_->hip_constants_frozen = config->hip_constants_frozen;
     internal_config_->sync_after_run = config->sync_after_run;

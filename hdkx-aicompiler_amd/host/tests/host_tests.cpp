@@ -12,6 +12,7 @@
 #include <dlfcn.h>
 #include <array>
 #include <cmath>
+#include <set>
 #include <sstream>
 #include <cstdio>
 #include <cstring>
@@ -1305,6 +1306,88 @@ int RunQnn(const std::string& oracle_path) {
     return 0;
 }
 
+// relay::SplitBatch: graphs whose samples are independent split into shares, everything else is refused.
+int RunSplitBatch() {
+    using kxc::relay::SplitBatch; using kxc::relay::InferTypePass;
+    auto shape0 = [](const kxc::Function& f) { return f->body.checked_type().As<kxc::TensorTypeNode>()->shape; };
+    // ---- the ResNet-18 graph at batch 8 splits into 2 and 4 shares, not into 3
+    {
+        kxc::Function net = InferTypePass(kxc::models::BuildResNet18(8, 64));
+        kxc::Function half = SplitBatch(net, 2), quarter = SplitBatch(net, 4);
+        Check(half.defined() && quarter.defined(), "ResNet-18 should split along the batch");
+        Check(shape0(half) == std::vector<int64_t>({4, 1000}) && shape0(quarter) == std::vector<int64_t>({2, 1000}), "share output shape");
+        Check(half->params.size() == net->params.size(), "a share keeps the parameters");
+        Check(!SplitBatch(net, 3).defined(), "8 samples do not divide into 3 shares");
+        Check(!SplitBatch(net, 16).defined(), "more shares than samples");
+        // constants are shared, calls are cloned
+        std::set<const kxc::RelayExprNode*> c_full, c_half;
+        std::function<void(const kxc::Expr&, std::set<const kxc::RelayExprNode*>*)> walk = [&](const kxc::Expr& e, std::set<const kxc::RelayExprNode*>* out) {
+            if (e.As<kxc::ConstantNode>()) { out->insert(e.get()); return; }
+            if (const auto* c = e.As<kxc::CallNode>()) for (const auto& a : c->args) walk(a, out);
+        };
+        walk(net->body, &c_full); walk(half->body, &c_half);
+        Check(!c_full.empty() && c_full == c_half, "the shares read the graph's own constants");
+        std::cout << "[PASS] ResNet-18 splits into shares\n";
+    }
+    auto var = [](const char* n, std::vector<int64_t> shape, const char* dt = "float32") { return kxc::Var(n, kxc::TensorType(shape, dt)); };
+    auto splits = [&](kxc::Function f) { return SplitBatch(InferTypePass(f), 2).defined(); };
+    // ---- accepted
+    {
+        kxc::Var x = var("x", {4, 6}), w = var("w", {5, 6}), b = var("b", {5});
+        Check(splits(kxc::Function({x, w}, kxc::Call(Op::Get("nn_dense"), {x, w}, kxc::relay::DenseAttrs::Create(5, "")))), "dense");
+        Check(splits(kxc::Function({x, w, b}, kxc::Call(Op::Get("nn_gemm"), {x, w, b}, kxc::relay::GemmAttrs::Create(1, 1, 0, 1)))), "gemm");
+        Check(splits(kxc::Function({x}, kxc::Call(Op::Get("softmax"), {x}, kxc::relay::SoftmaxAttrs::Create(-1)))), "softmax over the last axis");
+        Check(splits(kxc::Function({x}, kxc::Call(Op::Get("reduce_mean"), {x}, kxc::relay::ReduceMeanAttrs::Create({1}, 0)))), "reduce_mean over axis 1");
+        kxc::Var y = var("y", {6});
+        Check(splits(kxc::Function({x, y}, kxc::Call(Op::Get("add"), {x, y}))), "add with a broadcast row");
+        Check(splits(kxc::Function({x}, kxc::Call(Op::Get("add"), {x, x}))), "add of two batched values");
+        kxc::Var t = var("t", {4, 2, 3});
+        Check(splits(kxc::Function({t}, kxc::Call(Op::Get("transpose"), {t}, kxc::relay::TransposeAttrs::Create({0, 2, 1})))), "transpose that keeps axis 0");
+        kxc::Var q = var("q", {4, 3, 8, 8});
+        Check(splits(kxc::Function({q}, kxc::Call(Op::Get("qnn_quantize"), {q}, kxc::relay::QnnQuantizeAttrs::Create(0.5)))), "qnn_quantize");
+        std::cout << "[PASS] separable graphs are accepted\n";
+    }
+    // ---- refused: an operator that mixes samples, or a value that would have to be cut without being parameter 0
+    {
+        kxc::Var x = var("x", {4, 6}), w = var("w", {5, 6});
+        Check(!splits(kxc::Function({x}, kxc::Call(Op::Get("softmax"), {x}, kxc::relay::SoftmaxAttrs::Create(0)))), "softmax over the batch");
+        Check(!splits(kxc::Function({x}, kxc::Call(Op::Get("softmax"), {x}, kxc::relay::SoftmaxAttrs::Create(-2)))), "softmax over the batch, negative axis");
+        Check(!splits(kxc::Function({x}, kxc::Call(Op::Get("reduce_mean"), {x}, kxc::relay::ReduceMeanAttrs::Create({0}, 0)))), "reduce_mean over the batch");
+        Check(!splits(kxc::Function({x}, kxc::Call(Op::Get("transpose"), {x}, kxc::relay::TransposeAttrs::Create({1, 0})))), "transpose moves the batch");
+        Check(!splits(kxc::Function({x}, kxc::Call(Op::Get("reshape"), {x}, kxc::relay::ReshapeAttrs::Create({2, 12})))), "reshape");
+        Check(!splits(kxc::Function({x}, kxc::Call(Op::Get("nn_flatten"), {x}, kxc::relay::FlattenAttrs::Create(0)))), "flatten from axis 0");
+        // the batch on the right-hand operand of a product
+        kxc::Var w4 = var("w4", {4, 6});
+        Check(!splits(kxc::Function({w4, x}, kxc::Call(Op::Get("nn_dense"), {x, w4}, kxc::relay::DenseAttrs::Create(4, "")))), "batched weight");
+        kxc::Var a = var("a", {4, 4}), b2 = var("b", {4, 4});
+        Check(!splits(kxc::Function({a, b2}, kxc::Call(Op::Get("matmul"), {b2, a}))), "matmul with the batch on the right");
+        // a second operand of the batch's full shape that is not derived from parameter 0
+        kxc::Var y = var("y", {4, 6});
+        Check(!splits(kxc::Function({x, y}, kxc::Call(Op::Get("add"), {x, y}))), "add with an unbatched operand of batch extent");
+        // the result does not carry the batch
+        Check(!splits(kxc::Function({x, w}, kxc::Call(Op::Get("nn_relu"), {w}, kxc::relay::ReluAttrs::Create()))), "result independent of parameter 0");
+        // shares must divide
+        kxc::Var odd = var("odd", {5, 6});
+        Check(!splits(kxc::Function({odd}, kxc::Call(Op::Get("nn_relu"), {odd}, kxc::relay::ReluAttrs::Create()))), "5 samples in 2 shares");
+        std::cout << "[PASS] inseparable graphs are refused\n";
+    }
+    // ---- an explicit request the graph does not allow makes Compile throw (dry hip target: no GPU needed up to loading)
+    {
+        kxc::Var x = var("x", {4, 8});
+        kxc::Function f({x}, kxc::Call(Op::Get("softmax"), {x}, kxc::relay::SoftmaxAttrs::Create(0)));
+        auto cfg = kxc::api::CompileConfig::JIT(kxc::BuildTarget(kxc::kGPU));
+        cfg->hip_batch_lanes = 2;
+        bool threw = false;
+        try { kxc::api::Compiler::Compile(f, cfg); } catch (const std::exception& e) {
+            threw = std::string(e.what()).find("cannot be split along the batch") != std::string::npos;
+        }
+        Check(threw, "hip_batch_lanes = 2 on an inseparable graph should throw");
+        std::cout << "[PASS] explicit request on an inseparable graph throws\n";
+    }
+    std::cout << "split batch ok\n";
+    return 0;
+}
+
 // The registry face of the device API and of the plan functions (include/base/registry.h, src/base/device_api.cc:442-658).
 int RunPackedFunc(const std::string& mode) {
     using kxc::PackedFunc; using kxc::Registry; using kxc::RetValue;
@@ -1395,6 +1478,7 @@ int main(int argc, char** argv) {
         if (cmd == "codegen") return RunCodegen();
         if (cmd == "packed_func") return RunPackedFunc(argc > 2 ? argv[2] : "cpu");
         if (cmd == "generated_numeric") return RunGeneratedNumeric();
+        if (cmd == "split_batch") return RunSplitBatch();
         if (cmd == "qnn" && argc >= 4) { g_mode = argv[2]; return RunQnn(argv[3]); }
         if (cmd == "onnx" && argc >= 4) { g_mode = argv[2]; return RunOnnx(argv[3]); }
         if (cmd == "onnx_errors" && argc >= 3) return RunOnnxErrors(argv[2]);

@@ -345,7 +345,9 @@ int32_t kxc_hip_module_free(kxc_hip_module* module);
 typedef struct kxc_hip_plan kxc_hip_plan;       /* opaque */
 
 /* A buffer operand: packed_args[index] (kind 0), byte offset into the plan
- * workspace (kind 1), or absent (kind 2, e.g. no bias). */
+ * workspace (kind 1), absent (kind 2, e.g. no bias), or packed_args[index] plus a byte offset that is a
+ * multiple of 16 (kind 3, index_or_offset = KXC_HIP_ARG_OFFSET(index, bytes): one share of a batched
+ * argument). */
 typedef struct kxc_hip_buf {
     int32_t kind;
     int64_t index_or_offset;
@@ -353,6 +355,8 @@ typedef struct kxc_hip_buf {
 #define KXC_HIP_BUF_ARG 0
 #define KXC_HIP_BUF_WORKSPACE 1
 #define KXC_HIP_BUF_NONE 2
+#define KXC_HIP_BUF_ARG_OFFSET 3
+#define KXC_HIP_ARG_OFFSET(index, bytes) (((int64_t)(index) << 48) | (int64_t)(bytes))   /* index < 32768, bytes < 2^48 */
 
 int32_t kxc_hip_plan_create(int32_t device_id, int32_t num_packed_args, kxc_hip_plan** out);
 int32_t kxc_hip_plan_destroy(kxc_hip_plan* plan);
@@ -438,6 +442,20 @@ int32_t kxc_hip_plan_deserialize(const char* text, int32_t device_id, kxc_hip_mo
  * overwrites a buffer the side node uses.  Without a join the plan run ends with one.  (Independent branches of
  * a graph -- a residual block's 1x1 downsample next to its 3x3 convolution -- overlap this way.) */
 int32_t kxc_hip_plan_set_concurrency(kxc_hip_plan* plan, int32_t node, int32_t lane, int32_t join);
+/* Chains: independent runs of nodes inside one plan, e.g. the same network on the two halves of a batch (their
+ * operands are workspace regions of their own and KXC_HIP_BUF_ARG_OFFSET shares of the arguments).  Nodes with
+ * chain k in [1, 7] run on the plan's k-th chain stream in the order they were added, from the start of a plan
+ * run (after everything enqueued before it on the caller's stream) to its end (the caller's stream then waits for
+ * every chain); nodes with chain 0 run on the caller's stream as before.  Under graph replay the chains are
+ * parallel branches of the captured graph.  A launch on a machine that other launches fill needs no split
+ * reduction or small tile of its own to fill it: kxc_hip_plan_set_select_lanes(plan, n) makes finalize choose
+ * every convolution variant as for n equal launches side by side, and kxc_hip_set_select_lanes(n) does the same
+ * for the calling thread's variant queries (kxc_hip_conv2d_variant, _pair_supported, _winograd_preferred ...)
+ * and stand-alone launches; it returns the previous value.  No counterpart in the reference, whose executor runs
+ * one node after the other (src/base/disco/executor.cc:59-90). */
+int32_t kxc_hip_plan_set_chain(kxc_hip_plan* plan, int32_t node, int32_t chain);
+int32_t kxc_hip_plan_set_select_lanes(kxc_hip_plan* plan, int32_t lanes);
+int32_t kxc_hip_set_select_lanes(int32_t lanes);
 /* Allocate the workspace (bytes = the largest offset + size the nodes use). */
 int32_t kxc_hip_plan_finalize(kxc_hip_plan* plan, size_t workspace_bytes);
 /* Enqueue every node on `stream`; returns after enqueue (no synchronisation). */

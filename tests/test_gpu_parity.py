@@ -918,6 +918,92 @@ def test_resnet18_batch64_properties(pkg, fast_orc):
         assert_close(got[n:n + 1], want, what="resnet18 batch 64, image %d" % n, floor="scale")
 
 
+def test_plan_chains_run_shares_of_a_batch_side_by_side(pkg, synth, fast_orc):
+    """Two chains of one plan run the same three launches (Winograd convolution + bias + ReLU with shared transformed
+    weights, max pool, convolution with a residual) on the two halves of a batch, each on a stream of its own, on
+    KXC_HIP_BUF_ARG_OFFSET shares of the arguments: bit-identical to the same nodes in one lane, to the plan rebuilt
+    from its text (version 2 keeps chain and select_lanes) and to every replay of the captured graph; within the
+    operator tolerance of the CPU path.  Wrong uses are refused."""
+    n, c, h, o = 8, 16, 24, 64
+    x = synth.uniform((n, c, h, h), 9100)
+    w = synth.normal((o, c, 3, 3), 9101, 0.1); b = synth.uniform((o,), 9102, -0.1, 0.1)
+    w2 = synth.normal((o, o, 3, 3), 9103, 0.05)
+    half = n // 2
+    d1 = pkg.ConvDesc(half, c, h, h, o, 3, 3, 1, 1, 1, 1, 1, 1, pkg.CONV_BIAS | pkg.CONV_RELU)
+    dp = pkg.pool_desc((half, o, h, h), 3, 1, 1)
+    d2 = pkg.ConvDesc(half, o, h, h, o, 3, 3, 1, 1, 1, 1, 1, 1, pkg.CONV_RESIDUAL)
+    ubytes = pkg.conv2d_winograd_weight_bytes((half, c, h, h), (o, c, 3, 3))
+    ubytes = (ubytes + 255) // 256 * 256
+    act = half * o * h * h * 4                                       # bytes of one share's activation
+    x_share, y_share = half * c * h * h * 4, act
+
+    def build(chains):
+        plan = pkg.Plan(5)                                           # x, w, b, w2, y
+        plan.set_select_lanes(2)
+        for k in range(2):
+            xk, yk = pkg.Buf.arg_offset(0, k * x_share), pkg.Buf.arg_offset(4, k * y_share)
+            t0, t1 = pkg.Buf.ws(ubytes + (2 * k) * act), pkg.Buf.ws(ubytes + (2 * k + 1) * act)
+            first = plan.num_nodes()
+            plan.add_conv2d_winograd(d1, xk, pkg.Buf.arg(1), pkg.Buf.arg(2), pkg.Buf.none(), t0, pkg.Buf.ws(0))
+            plan.add_pool2d(dp, t0, t1)
+            plan.add_conv2d(d2, t1, pkg.Buf.arg(3), pkg.Buf.none(), t0, yk)
+            if chains and k == 1:
+                for node in range(first, plan.num_nodes()):
+                    plan.set_chain(node, 1)
+        plan.finalize(ubytes + 4 * act)
+        return plan
+
+    tensors = [dev(x), dev(w), dev(b), dev(w2)]
+    y_line, y_chain = torch.zeros((n, o, h, h), device="cuda"), torch.zeros((n, o, h, h), device="cuda")
+    in_line, chained = build(False), build(True)
+    in_line.run(tensors + [y_line]); torch.cuda.synchronize()
+    chained.run(tensors + [y_chain]); torch.cuda.synchronize()
+    assert_bit_exact(host(y_chain), host(y_line), "chains against the same nodes in one lane")
+    t = fast_orc.conv_chain(x, w, b, 1, 1, None, True)
+    t1 = fast_orc.pool2d(t, 3, 1, 1)
+    want = fast_orc.conv_chain(t1, w2, None, 1, 1, t, False)
+    assert_close(host(y_chain), want, what="two chains, conv / pool / conv + residual")
+    # the text form keeps the chains; the rebuilt plan gives the same bits
+    text = chained.serialize()
+    assert text.startswith("kxc_hip_plan 2 5 ") and text.splitlines()[0].split()[-1] == "2"
+    again = pkg.Plan.deserialize(text, 0)
+    assert again.serialize() == text
+    y2 = torch.zeros_like(y_chain)
+    again.run(tensors + [y2]); torch.cuda.synchronize()
+    assert_bit_exact(host(y2), host(y_line), "deserialised plan with chains")
+    # graph replay: the chains are parallel branches of the captured graph
+    stream = torch.cuda.Stream()
+    chained.enable_graph(True)
+    with torch.cuda.stream(stream):
+        for replay in range(5):
+            y_chain.zero_()
+            chained.run(tensors + [y_chain], stream.cuda_stream)
+            stream.synchronize()
+            assert_bit_exact(host(y_chain), host(y_line), "graph replay %d of a plan with chains" % replay)
+            z = pkg.relu(tensors[0]); torch.cuda.synchronize()          # eager work between the replays
+            assert torch.isfinite(z).all()
+    # back-to-back runs without waiting in between: a run's chains start after the previous run's end
+    chained.enable_graph(False)
+    for _ in range(4):
+        chained.run(tensors + [y_chain])
+    torch.cuda.synchronize()
+    assert_bit_exact(host(y_chain), host(y_line), "four runs enqueued back to back")
+    for p in (in_line, chained, again):
+        p.close()
+    # refused: a chain beyond the seventh, an offset that is not a multiple of 16, a chain on a side-lane node
+    plan = pkg.Plan(2)
+    plan.add_relu(64, pkg.Buf.arg(0), pkg.Buf.arg(1))
+    with pytest.raises(pkg.KxcHipError, match="chain must be in"):
+        plan.set_chain(0, 8)
+    with pytest.raises(pkg.KxcHipError, match="multiple of 16"):
+        plan.add_relu(64, pkg.Buf.arg_offset(0, 8), pkg.Buf.arg(1))
+    with pytest.raises(pkg.KxcHipError, match="out of range"):
+        plan.add_relu(64, pkg.Buf.arg_offset(2, 0), pkg.Buf.arg(1))
+    with pytest.raises(pkg.KxcHipError, match="lanes must be in"):
+        plan.set_select_lanes(0)
+    plan.close()
+
+
 def test_plan_hip_graph_replay(pkg):
     """A launch plan replayed as a captured HIP graph gives the eager result on every replay, with eager work and
     synchronisations in between, and re-captures when an argument pointer changes.  Batch 1 exercises the

@@ -63,6 +63,15 @@ def _oracle_so():
     return _build_if_missing("libkxc_oracle.so")
 
 
+def test_split_batch_accepts_only_separable_graphs():
+    """relay::SplitBatch (the shares of a batch the hip back end runs side by side): ResNet-18 splits, constants are
+    shared; softmax / reduce_mean / transpose / flatten over the batch axis, reshape, a batched right-hand operand, an
+    unbatched operand of batch extent and a batch that does not divide are refused; an explicit hip_batch_lanes on
+    such a graph makes Compile throw."""
+    out = run("split_batch")
+    assert "split batch ok" in out and out.count("[PASS]") == 4
+
+
 def test_quantised_operators_cpu():
     """qnn_quantize / qnn_conv2d / qnn_dense as graph operators (type rule, TE compute with the rint intrinsic, host
     back end): hand-worked answers, and the C oracle on seeded cases, element for element."""
@@ -128,10 +137,18 @@ def test_resnet18_cpu_backend_equals_oracle_bit_for_bit(synth):
 
 def test_resnet18_hip_plan_without_gpu():
     """Compiling for the hip target needs no GPU up to loading: 49 Relay calls become 20 launches at batch 64
-    (23 at small batches, where a block's downsample keeps a launch of its own)."""
+    (23 at small batches, where a block's downsample keeps a launch of its own).  By default a batch of 64 runs as
+    two shares of 32 side by side, each those 20 launches; KXC_HIP_BATCH_LANES=1 keeps the batch whole."""
     with tempfile.TemporaryDirectory() as d:
         out = run("resnet18", "hip", d, "64", "224")
+        shares = json.load(open(os.path.join(d, "plan.json")))
+    assert "launches: 40" in out and len(shares["nodes"]) == 40
+    assert [n["kernel_symbol"] + " @share1" for n in shares["nodes"][:20]] == [n["kernel_symbol"] for n in shares["nodes"][20:]]
+    assert [n["output_values"] for n in shares["nodes"][:20]] == [n["output_values"] for n in shares["nodes"][20:]]
+    with tempfile.TemporaryDirectory() as d:
+        out = run("resnet18", "hip", d, "64", "224", env={"KXC_HIP_BATCH_LANES": "1"})
         plan = json.load(open(os.path.join(d, "plan.json")))
+    assert [n["kernel_symbol"] for n in plan["nodes"]] == [n["kernel_symbol"] for n in shares["nodes"][:20]]
     assert "launches: 20" in out
     assert len(plan["nodes"]) == 20 and plan["schema_version"] == 1
     syms = [n["kernel_symbol"] for n in plan["nodes"]]
@@ -145,12 +162,12 @@ def test_resnet18_hip_plan_without_gpu():
     # at batch 64 every 3x3 stride-1 convolution (constant weights) takes the Winograd kernel, the rest do not
     assert sum(".winograd_f2k3" in s for s in syms) == 13 and sum(".mfma_" in s for s in syms) == 4
     with tempfile.TemporaryDirectory() as d:
-        run("resnet18", "hip", d, "64", "224", env={"KXC_HIP_PAIR": "0"})
+        run("resnet18", "hip", d, "64", "224", env={"KXC_HIP_PAIR": "0", "KXC_HIP_BATCH_LANES": "1"})
         unpaired = json.load(open(os.path.join(d, "plan.json")))
     assert len(unpaired["nodes"]) == 23
     assert sum(n["kernel_symbol"].startswith("kxc_conv2d") and n["kernel_symbol"].endswith("+bias") for n in unpaired["nodes"]) == 3
     with tempfile.TemporaryDirectory() as d:
-        run("resnet18", "hip", d, "64", "224", env={"KXC_HIP_WINOGRAD": "0"})
+        run("resnet18", "hip", d, "64", "224", env={"KXC_HIP_WINOGRAD": "0", "KXC_HIP_BATCH_LANES": "1"})
         off = json.load(open(os.path.join(d, "plan.json")))
     assert not any("winograd" in n["kernel_symbol"] for n in off["nodes"])
     with tempfile.TemporaryDirectory() as d:
@@ -207,22 +224,36 @@ def test_resnet18_hip_winograd_matches_oracle(synth):
 
 
 def _lanes(plan_json):
-    """(lane, join) of every node of the serialised launch plan (the two fields before the parameter count)."""
+    """(lane, join, chain) of every node of the serialised launch plan (the three fields before the parameter count)."""
     text = json.loads(plan_json)["kxc_hip"]["launch_plan"]
     lines = [line.split() for line in text.splitlines() if line.startswith("node")]
     base = min(len(t) for t in lines)            # a node without parameters; each parameter adds two fields
     out = []
     for t in lines:
         assert (len(t) - base) % 2 == 0 and int(t[base - 1]) == (len(t) - base) // 2
-        out.append((int(t[base - 3]), int(t[base - 2])))
+        out.append((int(t[base - 4]), int(t[base - 3]), int(t[base - 2])))
     return out
 
 
-def _compiled_resnet18_logits(synth, config, batch, module=None):
+def _compiled_resnet18_logits(synth, config, batch, module=None, env=None):
     """The plan bench.py times: ResNet-18 compiled by the C++ host layer with its DEFAULT configuration, run once
-    eagerly and then replayed as a captured HIP graph; returns inputs, logits of both, and the module facts."""
+    eagerly and then replayed as a captured HIP graph; returns inputs, logits of both, and the module facts.
+    env: switches the compiler reads from the environment, set for the compilation only."""
     import importlib
     import torch
+    saved = {k: os.environ.get(k) for k in (env or {})}
+    os.environ.update(env or {})
+    try:
+        return _compiled_resnet18_logits_now(synth, config, batch, importlib, torch)
+    finally:
+        for k, v in saved.items():
+            if v is None:
+                os.environ.pop(k, None)
+            else:
+                os.environ[k] = v
+
+
+def _compiled_resnet18_logits_now(synth, config, batch, importlib, torch):
     hostapi = importlib.import_module("hdkx-aicompiler_amd.hostapi")
     consts_h = synth.resnet18_consts(config)
     x_h = synth.resnet18_input(config, batch)
@@ -259,9 +290,16 @@ def test_resnet18_benchmarked_plan_batch64_matches_oracle(synth):
     from gpu_util import assert_close, assert_bit_exact
     x, consts, eager, replay, facts = _compiled_resnet18_logits(synth, 4, 64)
     syms = facts["launches"]
-    assert len(syms) == 20 and sum(".winograd_f2k3" in s for s in syms) == 13 and sum("_ds+" in s for s in syms) == 3, syms
-    assert set(facts["lanes"]) == {(0, 0)}           # one stream: nothing forks
+    # two shares of 32 images, each the whole network in 20 launches with the variants of the batch-64 launches
+    assert len(syms) == 40 and sum(".winograd_f2k3" in s for s in syms) == 26 and sum("_ds+" in s for s in syms) == 6, syms
+    assert [s + " @share1" for s in syms[:20]] == syms[20:]
+    assert facts["lanes"] == [(0, 0, 0)] * 20 + [(0, 0, 1)] * 20      # the second share is a chain on a stream of its own
     assert_bit_exact(replay, eager, "graph replay of the batch-64 plan")
+    # the whole batch in one share (20 launches, one stream): every launch computes a sample the same way
+    _, _, whole, whole_replay, whole_facts = _compiled_resnet18_logits(synth, 4, 64, env={"KXC_HIP_BATCH_LANES": "1"})
+    assert whole_facts["launches"] == syms[:20] and set(whole_facts["lanes"]) == {(0, 0, 0)}
+    assert_bit_exact(eager, whole, "two shares of the batch against the batch in one share")
+    assert_bit_exact(whole_replay, whole, "graph replay of the one-share plan")
     orc = Oracle(fast=True)
     for n in (0, 63):
         want = orc.resnet18(x[n:n + 1], consts)
