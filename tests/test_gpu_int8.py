@@ -314,6 +314,18 @@ def test_qresnet18_batch64_images(pkg, orc):
     for n in (0, 63):
         want, _ = orc.qresnet18(x[n:n + 1], model, net.gap_mult)
         assert_bit_exact(first[n:n + 1], want, "quantised resnet18 batch 64, image %d" % n)
+    # the same batch as two shares side by side (chains of the one plan on halves of the input and of the logits)
+    two = qr.QuantizedResNet18(model, 64, 224, shares=2)
+    assert two.shares == 2 and len(two.launches) == 2 * len(net.launches)
+    out2 = torch.zeros((64, 1000), device="cuda")
+    stream = torch.cuda.Stream()
+    two.plan.enable_graph(True)
+    with torch.cuda.stream(stream):
+        for replay in range(4):
+            out2.zero_()
+            two.run(xd, out2, stream.cuda_stream)
+            stream.synchronize()
+            assert_bit_exact(host(out2), first, "two shares of the batch, run %d" % replay)
 
 
 @pytest.mark.parametrize("m,n,k", [(64, 1000, 512), (70, 37, 1056), (33, 65, 32), (70, 37, 1040), (1, 5, 16), (9, 12, 24)])
