@@ -1388,6 +1388,68 @@ int RunSplitBatch() {
     return 0;
 }
 
+// Shares of a batch on the GPU for a graph that mixes hand-written launches and generated kernels (softmax has no
+// hand-written kernel): the shares reuse one compiled module per step, and give the one-share result bit for bit.
+int RunSharesGenerated() {
+    g_mode = "hip";
+    const int64_t N = 8, C = 4, H = 6, O = 8;
+    kxc::Var x("x", kxc::TensorType({N, C, H, H}, "float32"));
+    kxc::Var w("w", kxc::TensorType({O, C, 3, 3}, "float32"));
+    auto attrs = kxc::relay::Conv2DAttrs::Create({1, 1}, {1, 1, 1, 1}, {1, 1}, 1, O, {3, 3}, "NCHW", "OIHW", "", "");
+    kxc::Call conv(Op::Get("nn_conv2d"), {x, w}, attrs);
+    kxc::Call relu(Op::Get("nn_relu"), {conv}, kxc::relay::ReluAttrs::Create());
+    kxc::Call gap(Op::Get("nn_global_avg_pool2d"), {relu}, kxc::relay::GlobalAvgPool2DAttrs::Create());
+    kxc::Call flat(Op::Get("nn_flatten"), {gap}, kxc::relay::FlattenAttrs::Create(1));
+    kxc::Call sm(Op::Get("softmax"), {flat}, kxc::relay::SoftmaxAttrs::Create(-1));
+    kxc::Function f({x, w}, sm);
+    std::vector<float> xd(N * C * H * H), wd(O * C * 9);
+    uint32_t seed = 99;
+    for (auto* v : {&xd, &wd})
+        for (float& e : *v) { seed = seed * 1664525u + 1013904223u; e = static_cast<float>(static_cast<int32_t>(seed >> 8) % 2001 - 1000) / 1000.0f; }
+    std::vector<std::vector<float>> outs;
+    for (int lanes : {1, 2, 4}) {
+        auto cfg = MakeConfig();
+        cfg->hip_batch_lanes = lanes;
+        auto module = kxc::api::Compiler::Compile(f, cfg);
+        Check(module.IsReady(), "module should be ready: " + module.GetStatus());
+        const auto& execs = module.GetKernelExecs();
+        const size_t per_share = execs.size() / static_cast<size_t>(lanes);
+        Check(execs.size() == per_share * static_cast<size_t>(lanes), "launch count is a multiple of the shares");
+        size_t generated = 0;
+        for (const auto& e : execs) generated += e.kernel_symbol.find("[generated:") != std::string::npos;
+        Check(generated >= static_cast<size_t>(lanes), "softmax runs through generated kernels in every share");
+        if (lanes > 1) Check(execs.back().kernel_symbol.find(" @share" + std::to_string(lanes - 1)) != std::string::npos, "last launch belongs to the last share");
+        kxc::DeviceAPI* api = kxc::GetDeviceAPI(kxc::kGPU);
+        kxc::Device dev(kxc::kGPU, 0), cpu(kxc::kCPU, 0);
+        std::vector<float> out(N * O, -1.0f);
+        void* dx = api->AllocDataSpace(dev, xd.size() * 4, 256);
+        void* dw = api->AllocDataSpace(dev, wd.size() * 4, 256);
+        void* dy = api->AllocDataSpace(dev, out.size() * 4, 256);
+        api->CopyDataFromTo(cpu, xd.data(), dev, dx, xd.size() * 4);
+        api->CopyDataFromTo(cpu, wd.data(), dev, dw, wd.size() * 4);
+        for (int rep = 0; rep < 3; ++rep) module.Run({dx, dw, dy});
+        api->CopyDataFromTo(dev, dy, cpu, out.data(), out.size() * 4);
+        // the saved plan rebuilds (generated modules compiled again from the saved source, once per distinct source)
+        auto again = kxc::api::Compiler::LoadExecutionPlan(module.ExecutionPlanJSON(), cfg);
+        std::vector<float> out2(N * O, -2.0f);
+        again.Run({dx, dw, dy});
+        api->CopyDataFromTo(dev, dy, cpu, out2.data(), out2.size() * 4);
+        Check(std::memcmp(out.data(), out2.data(), out.size() * 4) == 0, "rebuilt plan differs");
+        for (void* p : {dx, dw, dy}) api->FreeDataSpace(dev, p);
+        for (int64_t n = 0; n < N; ++n) {
+            float sum = 0.0f;
+            for (int64_t o = 0; o < O; ++o) sum += out[n * O + o];
+            Check(std::fabs(sum - 1.0f) < 1e-5f, "softmax rows sum to 1");
+        }
+        outs.push_back(out);
+        std::cout << "[PASS] " << lanes << " share(s): " << execs.size() << " launches\n";
+    }
+    Check(std::memcmp(outs[0].data(), outs[1].data(), outs[0].size() * 4) == 0, "two shares differ from one");
+    Check(std::memcmp(outs[0].data(), outs[2].data(), outs[0].size() * 4) == 0, "four shares differ from one");
+    std::cout << "shares with generated kernels ok\n";
+    return 0;
+}
+
 // The registry face of the device API and of the plan functions (include/base/registry.h, src/base/device_api.cc:442-658).
 int RunPackedFunc(const std::string& mode) {
     using kxc::PackedFunc; using kxc::Registry; using kxc::RetValue;
@@ -1479,6 +1541,7 @@ int main(int argc, char** argv) {
         if (cmd == "packed_func") return RunPackedFunc(argc > 2 ? argv[2] : "cpu");
         if (cmd == "generated_numeric") return RunGeneratedNumeric();
         if (cmd == "split_batch") return RunSplitBatch();
+        if (cmd == "shares_generated") return RunSharesGenerated();
         if (cmd == "qnn" && argc >= 4) { g_mode = argv[2]; return RunQnn(argv[3]); }
         if (cmd == "onnx" && argc >= 4) { g_mode = argv[2]; return RunOnnx(argv[3]); }
         if (cmd == "onnx_errors" && argc >= 3) return RunOnnxErrors(argv[2]);

@@ -89,6 +89,15 @@ def test_quantised_operators_gpu(mode):
 
 
 @pytest.mark.gpu
+def test_shares_of_a_batch_with_generated_kernels():
+    """conv -> relu -> global average pool -> flatten -> softmax at batch 8 in 1, 2 and 4 shares: the hand-written
+    launches and the generated softmax kernels of every share give the one-share result bit for bit, and the saved
+    plan rebuilds."""
+    out = run("shares_generated")
+    assert "shares with generated kernels ok" in out and out.count("[PASS]") == 3
+
+
+@pytest.mark.gpu
 def test_generated_kernels_lds_schedules_bit_exact():
     """dense / matmul / reduce_mean shapes that take the generator's LDS-staged schedules (ragged chunks, fewer outputs
     than a workgroup, an operand that is not contiguous along the reduce axis): bit-identical to the host back end."""
@@ -305,6 +314,29 @@ def test_resnet18_benchmarked_plan_batch64_matches_oracle(synth):
         want = orc.resnet18(x[n:n + 1], consts)
         assert_close(eager[n:n + 1], want, what="host-layer plan, batch 64, image %d" % n, floor="scale")
         assert int(np.argmax(eager[n])) == int(np.argmax(want[0]))
+
+
+@pytest.mark.gpu
+def test_resnet18_two_shares_replay_from_saved_plan(synth):
+    """Four images as two shares of two (forced at this size): the saved execution plan -- 2 x 23 launches, the
+    second share's as a chain on argument offsets -- rebuilds into a module that reproduces the compiled one bit for
+    bit.  Against one share of four the logits agree within the operator tolerance (at this size the reductions of
+    the small launches are split over different numbers of workgroups; at batch 64 the two plans take the same
+    variants and agree bit for bit, see the batch-64 test)."""
+    from gpu_util import assert_close
+    logits = {}
+    for lanes in ("1", "2"):
+        with tempfile.TemporaryDirectory() as d:
+            _write_resnet_inputs(synth, d, 3, 4, 224)
+            out = run("resnet18", "hip", d, "4", "224", env={"KXC_HIP_BATCH_LANES": lanes})
+            n = 23 * int(lanes)
+            assert "execution plan replayed: %d launches, identical output" % n in out, out[-2000:]
+            plan = json.load(open(os.path.join(d, "plan.json")))
+            assert len(plan["nodes"]) == n
+            logits[lanes] = np.fromfile(os.path.join(d, "logits.bin"), np.float32).reshape(4, 1000)
+    assert_close(logits["2"], logits["1"], what="two shares of two images against one share of four", floor="scale")
+    want = Oracle(fast=True).resnet18(synth.resnet18_input(3, 4, 224), synth.resnet18_consts(3))
+    assert_close(logits["2"], want, what="two shares of two images against the CPU path", floor="scale")
 
 
 @pytest.mark.gpu
