@@ -126,14 +126,14 @@ class QuantizedResNet18:
     def __init__(self, model, batch, hw=224, device="cuda", shares=None):
         """shares: parts of the batch that run side by side as chains of the one plan (each the whole network on
         batch / shares images, on its own stream between the fork at the start of a run and the join at its end, so
-        that the launches of one fill the compute units the other's leave idle).  None: one, unless
-        KXC_HIP_BATCH_LANES says otherwise -- measured at batch 64: 0.314 ms in one share, 0.317 in two, 0.413 in four
-        (these launches are 7-15 us each; a fork and a join cost as much as the tails they would fill), unlike the fp32
-        network, which gains 9 %."""
+        that the launches of one fill the compute units the other's leave idle).  None: two from 128 images on, else
+        one (KXC_HIP_BATCH_LANES overrides) -- measured: batch 64 0.311 ms in one share, 0.308-0.317 in two, 0.413 in
+        four (these launches are 7-15 us each; a fork and a join cost as much as the tails they would fill); batch
+        128 0.461 ms in one share, 0.430 in two (298 against 277 k img/s).  The fp32 network gains 9 % at batch 64."""
         import torch
         self.batch, self.hw = batch, hw
         if shares is None:
-            shares = int(os.environ.get("KXC_HIP_BATCH_LANES", "0")) or 1
+            shares = int(os.environ.get("KXC_HIP_BATCH_LANES", "0")) or (2 if batch >= 128 else 1)
         if shares < 1 or shares > 8 or batch % shares != 0 or (batch // shares) % 4 != 0:
             shares = 1           # (a share of the fp32 logits and of the input must start on a 16-byte boundary)
         self.shares = shares
