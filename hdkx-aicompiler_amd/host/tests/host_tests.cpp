@@ -1243,15 +1243,15 @@ int RunQnn(const std::string& oracle_path) {
     }
     // ---- a quantised chain: quantize -> conv (+relu) -> conv with the first as residual, each stage against the oracle
     {
-        const int64_t C = 8, H = 12, W = 12;
-        std::vector<float> x(C * H * W), m1(C), m2(C);
+        const int64_t N = 4, C = 8, H = 12, W = 12;
+        std::vector<float> x(N * C * H * W), m1(C), m2(C);
         for (auto& v : x) v = static_cast<float>(static_cast<int>(next() % 2001) - 1000) / 400.0f;
-        std::vector<int8_t> w1(C * C * 9), w2(C * C * 9), y(C * H * W, 99);
+        std::vector<int8_t> w1(C * C * 9), w2(C * C * 9), y(N * C * H * W, 99);
         std::vector<int32_t> b1(C), b2(C);
         fill_i8(w1); fill_i8(w2);
         for (int64_t i = 0; i < C; ++i) { b1[i] = static_cast<int32_t>(next() % 801) - 400; b2[i] = static_cast<int32_t>(next() % 801) - 400;
                                            m1[i] = 0.002f + 0.0001f * static_cast<float>(i); m2[i] = 0.003f - 0.0001f * static_cast<float>(i); }
-        kxc::Var xv("x", kxc::TensorType({1, C, H, W}, "float32")), w1v("w1", kxc::TensorType({C, C, 3, 3}, "int8")), w2v("w2", kxc::TensorType({C, C, 3, 3}, "int8"));
+        kxc::Var xv("x", kxc::TensorType({N, C, H, W}, "float32")), w1v("w1", kxc::TensorType({C, C, 3, 3}, "int8")), w2v("w2", kxc::TensorType({C, C, 3, 3}, "int8"));
         kxc::Var b1v("b1", kxc::TensorType({C}, "int32")), b2v("b2", kxc::TensorType({C}, "int32")), m1v("m1", kxc::TensorType({C}, "float32")), m2v("m2", kxc::TensorType({C}, "float32"));
         kxc::Call q(Op::Get("qnn_quantize"), {xv}, kxc::relay::QnnQuantizeAttrs::Create(0.02));
         kxc::Call c1(Op::Get("qnn_conv2d"), {q, w1v, b1v, m1v}, kxc::relay::QnnConv2DAttrs::Create({1, 1}, {1, 1}, true));
@@ -1260,9 +1260,22 @@ int RunQnn(const std::string& oracle_path) {
         CompileAndRun("qnn chain", f, {In(x), I8(w1, false), I32(b1), In(m1), I8(w2, false), I32(b2), In(m2), I8(y, true)});
         std::vector<int8_t> xq(x.size()), t1(x.size()), want(x.size());
         oracle_quant(x.data(), xq.data(), static_cast<int64_t>(x.size()), 0.02f);
-        oracle_conv(xq.data(), w1.data(), b1.data(), m1.data(), nullptr, 0.0f, t1.data(), 1, C, H, W, C, 3, 3, 1, 1, 1, 1, 1);
-        oracle_conv(t1.data(), w2.data(), b2.data(), m2.data(), xq.data(), 0.75f, want.data(), 1, C, H, W, C, 3, 3, 1, 1, 1, 1, 1);
+        oracle_conv(xq.data(), w1.data(), b1.data(), m1.data(), nullptr, 0.0f, t1.data(), N, C, H, W, C, 3, 3, 1, 1, 1, 1, 1);
+        oracle_conv(t1.data(), w2.data(), b2.data(), m2.data(), xq.data(), 0.75f, want.data(), N, C, H, W, C, 3, 3, 1, 1, 1, 1, 1);
         Check(y == want, "qnn chain differs from the oracle");
+        if (g_mode == "hip") {
+            // the same graph as two shares of two images side by side (chains of the plan on halves of x and y)
+            setenv("KXC_HIP_BATCH_LANES", "2", 1);
+            std::vector<int8_t> y2(y.size(), 55);
+            try {
+                CompileAndRun("qnn chain in two shares", f, {In(x), I8(w1, false), I32(b1), In(m1), I8(w2, false), I32(b2), In(m2), I8(y2, true)});
+                auto shares = kxc::api::Compiler::Compile(f, MakeConfig());
+                Check(shares.GetKernelExecs().size() == 6 && shares.GetKernelExecs().back().kernel_symbol.find(" @share1") != std::string::npos,
+                      "qnn chain: two shares expected");
+            } catch (...) { unsetenv("KXC_HIP_BATCH_LANES"); throw; }
+            unsetenv("KXC_HIP_BATCH_LANES");
+            Check(y2 == want, "qnn chain in two shares differs from the oracle");
+        }
         if (g_mode != "cpu") {
             // hip: the three operators dispatch to the hand-written int8 launches; hipgen: to generated kernels only
             int quant = 0, conv = 0;
