@@ -606,9 +606,12 @@ int64_t Tiles(const kxc_hip_conv2d_desc* d) {
 // `units` 64 x 16 workgroups of `csteps` steps.  Two regimes, both measured on the ResNet-18 layers:
 //  * tiny launches (batch 1-4): parts of at least four steps while all parts together stay below one workgroup
 //    per compute unit (batch 1, 512 channels: 8 units -> 32 parts, 62.9 -> 14.7 us);
-//  * up to 256 units with a long reduction (64 steps and more; batch 8-32 of the 256- and 512-channel layers):
-//    parts of at least sixteen steps up to four workgroups per compute unit, which is what fills every SIMD with
-//    two waves (batch 16, 512 channels: 128 units -> 8 parts, 55.7 -> 39.6 us; the split inside the workgroup: 66).
+//  * up to 400 units (of the 512 workgroups the GPU holds at once) with a long reduction (64 steps and more; batch
+//    8-32 of the 256- and 512-channel layers): parts of at least sixteen steps up to four workgroups per compute
+//    unit, which is what fills every SIMD with two waves (batch 16, 512 channels: 128 units -> 8 parts, 55.7 -> 39.6
+//    us; the split inside the workgroup: 66).  The bound was 256 units; 392 (the 256-channel layers at batch 64,
+//    counting both shares of the batch) gain from two parts as well: ResNet-18 1.587 -> 1.574 ms at batch 64 in two
+//    shares, 1.025 -> 1.014 at batch 32, no change in one share of 64 or at batch 128; a bound of 800 loses 4 %.
 // The partial outputs (read back once by the adding kernel) stay below 16 MiB.
 int GroupSplit(int64_t units, int csteps, int64_t out_elems) {
     int split = 1;
@@ -617,7 +620,7 @@ int GroupSplit(int64_t units, int csteps, int64_t out_elems) {
         const int64_t groups = units * next;
         const int steps = csteps / next;
         const bool tiny = groups <= 256 && steps >= 4;
-        const bool filling = units <= 256 && groups <= 1024 && csteps >= 64 && steps >= 16;
+        const bool filling = units <= 400 && groups <= 1024 && csteps >= 64 && steps >= 16;
         if (!(tiny || filling)) break;
         if (out_elems * static_cast<int64_t>(sizeof(float)) * next > (16LL << 20)) break;
         split = next;

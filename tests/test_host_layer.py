@@ -304,10 +304,12 @@ def test_resnet18_benchmarked_plan_batch64_matches_oracle(synth):
     assert [s + " @share1" for s in syms[:20]] == syms[20:]
     assert facts["lanes"] == [(0, 0, 0)] * 20 + [(0, 0, 1)] * 20      # the second share is a chain on a stream of its own
     assert_bit_exact(replay, eager, "graph replay of the batch-64 plan")
-    # the whole batch in one share (20 launches, one stream): every launch computes a sample the same way
+    # the whole batch in one share (20 launches, one stream): the same kernels; the 256-channel Winograd layers split
+    # their reduction over two workgroups in the two-share plan only, so the logits agree to rounding, not bit for bit
     _, _, whole, whole_replay, whole_facts = _compiled_resnet18_logits(synth, 4, 64, env={"KXC_HIP_BATCH_LANES": "1"})
     assert whole_facts["launches"] == syms[:20] and set(whole_facts["lanes"]) == {(0, 0, 0)}
-    assert_bit_exact(eager, whole, "two shares of the batch against the batch in one share")
+    assert_close(eager, whole, what="two shares of the batch against the batch in one share", floor="scale")
+    assert float(np.max(np.abs(eager - whole))) <= 1e-4 * float(np.max(np.abs(whole)))
     assert_bit_exact(whole_replay, whole, "graph replay of the one-share plan")
     orc = Oracle(fast=True)
     for n in (0, 63):
