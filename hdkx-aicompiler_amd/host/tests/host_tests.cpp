@@ -1463,6 +1463,120 @@ int RunSharesGenerated() {
     return 0;
 }
 
+// Random small convolutional graphs (plain and strided convolutions, pools, residual blocks with and without a
+// downsample branch, a dense head, sometimes a softmax) at batch 4 or 8: the hip back end in one share and in two
+// shares of the batch against the host back end (operator tolerance) and against each other.
+int RunSharesRandom() {
+    uint32_t seed = 4242;
+    auto next = [&seed]() { seed = seed * 1664525u + 1013904223u; return seed >> 8; };
+    auto uniform = [&](float lo, float hi) { return lo + (hi - lo) * static_cast<float>(next() % 100001) / 100000.0f; };
+    auto constant = [&](std::vector<int64_t> shape, float scale) {
+        kxc::runtime::NDArray a(shape, "float32");
+        std::vector<float> v(static_cast<size_t>(kxc::Product(shape)));
+        for (float& e : v) e = uniform(-scale, scale);
+        a.CopyFromBytes(v.data(), v.size() * sizeof(float));
+        return kxc::Constant(a);
+    };
+    auto conv = [&](kxc::Expr x, int64_t c, int64_t o, int k, int s, int p, bool bias) {
+        auto attrs = kxc::relay::Conv2DAttrs::Create({s, s}, {p, p, p, p}, {1, 1}, 1, static_cast<int>(o), {k, k}, "NCHW", "OIHW", "", "");
+        const float scale = std::sqrt(3.0f / static_cast<float>(c * k * k));
+        if (bias) return kxc::Expr(kxc::Call(Op::Get("nn_conv2d"), {x, constant({o, c, k, k}, scale), constant({o}, 0.1f)}, attrs));
+        return kxc::Expr(kxc::Call(Op::Get("nn_conv2d"), {x, constant({o, c, k, k}, scale)}, attrs));
+    };
+    auto relu = [](kxc::Expr x) { return kxc::Expr(kxc::Call(Op::Get("nn_relu"), {x}, kxc::relay::ReluAttrs::Create())); };
+    auto add = [](kxc::Expr a, kxc::Expr b) { return kxc::Expr(kxc::Call(Op::Get("add"), {a, b})); };
+    const int trials = 8;
+    for (int trial = 0; trial < trials; ++trial) {
+        const int64_t N = (trial % 2) ? 8 : 4;
+        int64_t c = 3 + static_cast<int64_t>(next() % 6), h = 12 + 4 * static_cast<int64_t>(next() % 4);
+        kxc::Var x("x", kxc::TensorType({N, c, h, h}, "float32"));
+        std::vector<float> xd(static_cast<size_t>(N * c * h * h));
+        for (float& e : xd) e = uniform(-1.0f, 1.0f);
+        kxc::Expr e = x;
+        std::string recipe;
+        const int layers = 4 + static_cast<int>(next() % 4);
+        for (int l = 0; l < layers; ++l) {
+            const int kind = static_cast<int>(next() % 5);
+            if (kind == 0) {
+                const int64_t o = 8 * (1 + static_cast<int64_t>(next() % 4));
+                e = conv(e, c, o, 3, 1, 1, next() % 2 == 0);
+                if (next() % 2) e = relu(e);
+                c = o; recipe += "c";
+            } else if (kind == 1 && h >= 8) {
+                const int64_t o = 8 * (1 + static_cast<int64_t>(next() % 4));
+                e = relu(conv(e, c, o, 3, 2, 1, true));
+                c = o; h = (h + 2 - 3) / 2 + 1; recipe += "s";
+            } else if (kind == 2 && h >= 8) {
+                const bool is_max = next() % 2 == 0;
+                auto attrs = kxc::relay::MaxPool2DAttrs::Create({2, 2}, {1, 1, 1, 1}, {1, 1}, {3, 3}, "NCHW", false);
+                e = kxc::Expr(kxc::Call(Op::Get(is_max ? "nn_max_pool2d" : "nn_avg_pool2d"), {e}, attrs));
+                h = (h + 2 - 3) / 2 + 1; recipe += is_max ? "m" : "a";
+            } else if (kind == 3) {
+                kxc::Expr a = relu(conv(e, c, c, 3, 1, 1, true));
+                e = relu(add(conv(a, c, c, 3, 1, 1, true), e));
+                recipe += "r";
+            } else if (h >= 8) {
+                const int64_t o = 2 * c;
+                kxc::Expr a = relu(conv(e, c, o, 3, 2, 1, true));
+                kxc::Expr id = conv(e, c, o, 1, 2, 0, true);
+                e = relu(add(conv(a, o, o, 3, 1, 1, true), id));
+                c = o; h = (h + 2 - 3) / 2 + 1; recipe += "d";
+            }
+        }
+        e = kxc::Expr(kxc::Call(Op::Get("nn_global_avg_pool2d"), {e}, kxc::relay::GlobalAvgPool2DAttrs::Create()));
+        e = kxc::Expr(kxc::Call(Op::Get("nn_flatten"), {e}, kxc::relay::FlattenAttrs::Create(1)));
+        const int64_t classes = 12;
+        e = kxc::Expr(kxc::Call(Op::Get("nn_gemm"), {e, constant({classes, c}, 0.3f), constant({classes}, 0.1f)}, kxc::relay::GemmAttrs::Create(1.0f, 1.0f, 0, 1)));
+        if (trial % 3 == 0) { e = kxc::Expr(kxc::Call(Op::Get("softmax"), {e}, kxc::relay::SoftmaxAttrs::Create(-1))); recipe += "+softmax"; }
+        kxc::Function f({x}, e);
+        auto run = [&](bool gpu, int lanes, size_t* launches) {
+            auto cfg = kxc::api::CompileConfig::JIT(kxc::BuildTarget(gpu ? kxc::kGPU : kxc::kCPU));
+            cfg->opt_level = 0;
+            cfg->hip_batch_lanes = lanes;
+            auto module = kxc::api::Compiler::Compile(f, cfg);
+            Check(module.IsReady(), "module should be ready: " + module.GetStatus());
+            *launches = module.GetKernelExecs().size();
+            std::vector<float> out(static_cast<size_t>(N * classes), -7.0f);
+            const auto& consts = module.GetConstants();
+            std::vector<void*> args;
+            if (!gpu) {
+                args.push_back(xd.data());
+                for (const auto& k : consts) args.push_back(const_cast<void*>(k->data()));
+                args.push_back(out.data());
+                module.Run(args);
+                return out;
+            }
+            kxc::DeviceAPI* api = kxc::GetDeviceAPI(kxc::kGPU);
+            kxc::Device dev(kxc::kGPU, 0), cpu(kxc::kCPU, 0);
+            auto up = [&](const void* src, size_t bytes) {
+                void* d = api->AllocDataSpace(dev, bytes, 256);
+                api->CopyDataFromTo(cpu, const_cast<void*>(src), dev, d, bytes);
+                return d;
+            };
+            args.push_back(up(xd.data(), xd.size() * 4));
+            for (const auto& k : consts) args.push_back(up(k->data(), k.nbytes()));
+            args.push_back(api->AllocDataSpace(dev, out.size() * 4, 256));
+            for (int rep = 0; rep < 2; ++rep) module.Run(args);      // twice: the workspace is reused
+            api->CopyDataFromTo(dev, args.back(), cpu, out.data(), out.size() * 4);
+            for (void* p : args) api->FreeDataSpace(dev, p);
+            return out;
+        };
+        size_t l_cpu = 0, l_one = 0, l_two = 0;
+        const std::vector<float> want = run(false, 1, &l_cpu), one = run(true, 1, &l_one), two = run(true, 2, &l_two);
+        Check(l_two == 2 * l_one, "two shares should hold twice the launches of one (" + std::to_string(l_two) + " vs " + std::to_string(l_one) + ")");
+        float scale = 0.0f;
+        for (float v : want) scale = std::max(scale, std::fabs(v));
+        Check(scale > 0.0f && std::isfinite(scale), "degenerate case");
+        for (size_t i = 0; i < want.size(); ++i) {
+            Check(std::fabs(one[i] - want[i]) <= 1e-3f * std::max(scale, 1.0f), "trial " + std::to_string(trial) + " [" + recipe + "]: one share differs from the host back end at " + std::to_string(i));
+            Check(std::fabs(two[i] - one[i]) <= 1e-4f * std::max(scale, 1.0f), "trial " + std::to_string(trial) + " [" + recipe + "]: two shares differ from one at " + std::to_string(i));
+        }
+        std::cout << "[PASS] trial " << trial << " batch " << N << " [" << recipe << "]: " << l_one << " launches per share\n";
+    }
+    std::cout << "random graphs in shares ok\n";
+    return 0;
+}
+
 // The registry face of the device API and of the plan functions (include/base/registry.h, src/base/device_api.cc:442-658).
 int RunPackedFunc(const std::string& mode) {
     using kxc::PackedFunc; using kxc::Registry; using kxc::RetValue;
@@ -1555,6 +1669,7 @@ int main(int argc, char** argv) {
         if (cmd == "generated_numeric") return RunGeneratedNumeric();
         if (cmd == "split_batch") return RunSplitBatch();
         if (cmd == "shares_generated") return RunSharesGenerated();
+        if (cmd == "shares_random") return RunSharesRandom();
         if (cmd == "qnn" && argc >= 4) { g_mode = argv[2]; return RunQnn(argv[3]); }
         if (cmd == "onnx" && argc >= 4) { g_mode = argv[2]; return RunOnnx(argv[3]); }
         if (cmd == "onnx_errors" && argc >= 3) return RunOnnxErrors(argv[2]);

@@ -98,6 +98,15 @@ def test_shares_of_a_batch_with_generated_kernels():
 
 
 @pytest.mark.gpu
+def test_random_graphs_in_one_and_two_shares():
+    """Eight seeded random convolutional graphs (plain / strided convolutions, pools, residual blocks with and without a
+    downsample branch, dense head, softmax) at batch 4 and 8: hip back end in one share within the operator tolerance
+    of the host back end, two shares within 1e-4 of one share, run twice over the same workspace."""
+    out = run("shares_random")
+    assert "random graphs in shares ok" in out and out.count("[PASS]") == 8
+
+
+@pytest.mark.gpu
 def test_generated_kernels_lds_schedules_bit_exact():
     """dense / matmul / reduce_mean shapes that take the generator's LDS-staged schedules (ragged chunks, fewer outputs
     than a workgroup, an operand that is not contiguous along the reduce axis): bit-identical to the host back end."""
