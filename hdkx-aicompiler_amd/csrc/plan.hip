@@ -1009,6 +1009,28 @@ int32_t kxc_hip_plan_set_chain(kxc_hip_plan* plan, int32_t node, int32_t chain) 
     return KXC_HIP_OK;
 }
 
+int32_t kxc_hip_plan_interleave_chains(kxc_hip_plan* plan, int32_t* new_index, int32_t capacity) {
+    const char* who = "kxc_hip_plan_interleave_chains";
+    KXC_PLAN_BEGIN(who);
+    const int32_t n = static_cast<int32_t>(plan->nodes.size());
+    KXC_HIP_REQUIRE(new_index == nullptr || capacity >= n, "%s: room for %d indices, %d nodes", who, capacity, n);
+    // round k takes the k-th node of the main lane, then the k-th node of every chain: each stream keeps its order
+    std::vector<std::vector<int32_t>> by_chain(kMaxChains + 1);
+    for (int32_t i = 0; i < n; ++i) by_chain[plan->nodes[i].chain].push_back(i);
+    std::vector<int32_t> order;
+    for (size_t k = 0; static_cast<int32_t>(order.size()) < n; ++k)
+        for (const auto& c : by_chain)
+            if (k < c.size()) order.push_back(c[k]);
+    std::vector<Node> moved;
+    moved.reserve(plan->nodes.size());
+    for (int32_t pos = 0; pos < n; ++pos) {
+        moved.push_back(std::move(plan->nodes[order[pos]]));
+        if (new_index) new_index[order[pos]] = pos;
+    }
+    plan->nodes.swap(moved);
+    return KXC_HIP_OK;
+}
+
 int32_t kxc_hip_plan_set_select_lanes(kxc_hip_plan* plan, int32_t lanes) {
     const char* who = "kxc_hip_plan_set_select_lanes";
     KXC_PLAN_BEGIN(who);

@@ -672,6 +672,14 @@ class Plan:
         """Node `node` runs on the plan's chain stream `chain` (1-7), beside the main lane (kxc_hip_plan_set_chain)."""
         _check(lib().kxc_hip_plan_set_chain(self._h, C.c_int32(node), C.c_int32(chain)))
 
+    def interleave_chains(self):
+        """Reorders the nodes so that the streams are fed at the same pace (kxc_hip_plan_interleave_chains); returns
+        the new index of every old node index."""
+        n = self.num_nodes()
+        idx = (C.c_int32 * max(n, 1))()
+        _check(lib().kxc_hip_plan_interleave_chains(self._h, idx, C.c_int32(n)))
+        return [int(idx[i]) for i in range(n)]
+
     def set_select_lanes(self, lanes):
         _check(lib().kxc_hip_plan_set_select_lanes(self._h, C.c_int32(lanes)))
 

@@ -240,6 +240,17 @@ public:
                     throw std::runtime_error(std::string("plan_set_chain failed: ") + kxc_hip_last_error());
             for (size_t e = first_exec; e < m_->execs.size(); ++e) m_->execs[e].kernel_symbol += " @share" + std::to_string(lane_);
         }
+        if (lanes_ > 1 && !(std::getenv("KXC_HIP_INTERLEAVE") && std::getenv("KXC_HIP_INTERLEAVE")[0] == '0')) {
+            // the shares' launches alternate in the plan, so that a run feeds every stream at the same pace
+            std::vector<int32_t> new_index(static_cast<size_t>(kxc_hip_plan_num_nodes(m_->plan)));
+            if (kxc_hip_plan_interleave_chains(m_->plan, new_index.data(), static_cast<int32_t>(new_index.size())))
+                throw std::runtime_error(std::string("plan_interleave_chains failed: ") + kxc_hip_last_error());
+            if (new_index.size() == m_->execs.size()) {
+                std::vector<KernelExecInfo> moved(m_->execs.size());
+                for (size_t i = 0; i < new_index.size(); ++i) moved[static_cast<size_t>(new_index[i])] = m_->execs[i];
+                m_->execs.swap(moved);
+            }
+        }
         m_->workspace_bytes = static_cast<size_t>(arena_.top);
         if (!dry_) {
             if (kxc_hip_plan_finalize(m_->plan, m_->workspace_bytes))

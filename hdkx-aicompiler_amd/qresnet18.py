@@ -210,6 +210,8 @@ class QuantizedResNet18:
             for node in range(first_node, plan.num_nodes()):
                 if share > 0:
                     plan.set_chain(node, share)
+        if shares > 1:
+            plan.interleave_chains()          # a run feeds every share's stream at the same pace
         plan.finalize(arena.top)
         self.plan = plan
         self.workspace_bytes = arena.top

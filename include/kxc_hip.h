@@ -454,6 +454,11 @@ int32_t kxc_hip_plan_set_concurrency(kxc_hip_plan* plan, int32_t node, int32_t l
  * and stand-alone launches; it returns the previous value.  No counterpart in the reference, whose executor runs
  * one node after the other (src/base/disco/executor.cc:59-90). */
 int32_t kxc_hip_plan_set_chain(kxc_hip_plan* plan, int32_t node, int32_t chain);
+/* Reorders the nodes so that a run enqueues the k-th node of the main lane, then the k-th node of every chain, then
+ * the (k+1)-th ...: every stream keeps its own order, and all of them are fed at the same pace (a host that enqueues
+ * one chain after the other starts the second one a whole chain's worth of launch calls late).  new_index (may be
+ * NULL) receives, for every old node index, the node's new index. */
+int32_t kxc_hip_plan_interleave_chains(kxc_hip_plan* plan, int32_t* new_index, int32_t capacity);
 int32_t kxc_hip_plan_set_select_lanes(kxc_hip_plan* plan, int32_t lanes);
 int32_t kxc_hip_set_select_lanes(int32_t lanes);
 /* Allocate the workspace (bytes = the largest offset + size the nodes use). */

@@ -937,7 +937,7 @@ def test_plan_chains_run_shares_of_a_batch_side_by_side(pkg, synth, fast_orc):
     act = half * o * h * h * 4                                       # bytes of one share's activation
     x_share, y_share = half * c * h * h * 4, act
 
-    def build(chains):
+    def build(chains, interleave=False):
         plan = pkg.Plan(5)                                           # x, w, b, w2, y
         plan.set_select_lanes(2)
         for k in range(2):
@@ -950,6 +950,10 @@ def test_plan_chains_run_shares_of_a_batch_side_by_side(pkg, synth, fast_orc):
             if chains and k == 1:
                 for node in range(first, plan.num_nodes()):
                     plan.set_chain(node, 1)
+        if interleave:
+            # main lane and chain alternate; every stream keeps its own order
+            assert plan.interleave_chains() == [0, 2, 4, 1, 3, 5]
+            assert ["winograd" in plan.node_symbol(i) for i in range(6)] == [True, True, False, False, False, False]
         plan.finalize(ubytes + 4 * act)
         return plan
 
@@ -959,6 +963,12 @@ def test_plan_chains_run_shares_of_a_batch_side_by_side(pkg, synth, fast_orc):
     in_line.run(tensors + [y_line]); torch.cuda.synchronize()
     chained.run(tensors + [y_chain]); torch.cuda.synchronize()
     assert_bit_exact(host(y_chain), host(y_line), "chains against the same nodes in one lane")
+    mixed = build(True, interleave=True)
+    y_mixed = torch.zeros_like(y_chain)
+    mixed.run(tensors + [y_mixed]); torch.cuda.synchronize()
+    assert_bit_exact(host(y_mixed), host(y_line), "chains with their launches interleaved")
+    assert pkg.Plan.deserialize(mixed.serialize(), 0).serialize() == mixed.serialize()
+    mixed.close()
     t = fast_orc.conv_chain(x, w, b, 1, 1, None, True)
     t1 = fast_orc.pool2d(t, 3, 1, 1)
     want = fast_orc.conv_chain(t1, w2, None, 1, 1, t, False)

@@ -161,12 +161,13 @@ def test_resnet18_hip_plan_without_gpu():
         out = run("resnet18", "hip", d, "64", "224")
         shares = json.load(open(os.path.join(d, "plan.json")))
     assert "launches: 40" in out and len(shares["nodes"]) == 40
-    assert [n["kernel_symbol"] + " @share1" for n in shares["nodes"][:20]] == [n["kernel_symbol"] for n in shares["nodes"][20:]]
-    assert [n["output_values"] for n in shares["nodes"][:20]] == [n["output_values"] for n in shares["nodes"][20:]]
+    # the two shares' launches alternate
+    assert [n["kernel_symbol"] + " @share1" for n in shares["nodes"][0::2]] == [n["kernel_symbol"] for n in shares["nodes"][1::2]]
+    assert [n["output_values"] for n in shares["nodes"][0::2]] == [n["output_values"] for n in shares["nodes"][1::2]]
     with tempfile.TemporaryDirectory() as d:
         out = run("resnet18", "hip", d, "64", "224", env={"KXC_HIP_BATCH_LANES": "1"})
         plan = json.load(open(os.path.join(d, "plan.json")))
-    assert [n["kernel_symbol"] for n in plan["nodes"]] == [n["kernel_symbol"] for n in shares["nodes"][:20]]
+    assert [n["kernel_symbol"] for n in plan["nodes"]] == [n["kernel_symbol"] for n in shares["nodes"][0::2]]
     assert "launches: 20" in out
     assert len(plan["nodes"]) == 20 and plan["schema_version"] == 1
     syms = [n["kernel_symbol"] for n in plan["nodes"]]
@@ -310,13 +311,13 @@ def test_resnet18_benchmarked_plan_batch64_matches_oracle(synth):
     syms = facts["launches"]
     # two shares of 32 images, each the whole network in 20 launches with the variants of the batch-64 launches
     assert len(syms) == 40 and sum(".winograd_f2k3" in s for s in syms) == 26 and sum("_ds+" in s for s in syms) == 6, syms
-    assert [s + " @share1" for s in syms[:20]] == syms[20:]
-    assert facts["lanes"] == [(0, 0, 0)] * 20 + [(0, 0, 1)] * 20      # the second share is a chain on a stream of its own
+    assert [s + " @share1" for s in syms[0::2]] == syms[1::2]       # the shares' launches alternate in the plan
+    assert facts["lanes"] == [(0, 0, 0), (0, 0, 1)] * 20              # the second share is a chain on a stream of its own
     assert_bit_exact(replay, eager, "graph replay of the batch-64 plan")
     # the whole batch in one share (20 launches, one stream): the same kernels; the 256-channel Winograd layers split
     # their reduction over two workgroups in the two-share plan only, so the logits agree to rounding, not bit for bit
     _, _, whole, whole_replay, whole_facts = _compiled_resnet18_logits(synth, 4, 64, env={"KXC_HIP_BATCH_LANES": "1"})
-    assert whole_facts["launches"] == syms[:20] and set(whole_facts["lanes"]) == {(0, 0, 0)}
+    assert whole_facts["launches"] == syms[0::2] and set(whole_facts["lanes"]) == {(0, 0, 0)}
     assert_close(eager, whole, what="two shares of the batch against the batch in one share", floor="scale")
     assert float(np.max(np.abs(eager - whole))) <= 1e-4 * float(np.max(np.abs(whole)))
     assert_bit_exact(whole_replay, whole, "graph replay of the one-share plan")
