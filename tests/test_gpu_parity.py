@@ -1014,6 +1014,45 @@ def test_plan_chains_run_shares_of_a_batch_side_by_side(pkg, synth, fast_orc):
     plan.close()
 
 
+def test_plan_text_version_1_still_loads(pkg, synth):
+    """The plan text gained a select_lanes field in the header and a chain field per node (version 2); a version-1
+    text -- the same plan written without them -- still loads and gives the same bits."""
+    n, c, h, o = 2, 8, 10, 32
+    x = synth.uniform((n, c, h, h), 9300); w = synth.normal((o, c, 3, 3), 9301, 0.1); b = synth.uniform((o,), 9302, -0.1, 0.1)
+    d = pkg.ConvDesc(n, c, h, h, o, 3, 3, 1, 1, 1, 1, 1, 1, pkg.CONV_BIAS | pkg.CONV_RELU)
+    plan = pkg.Plan(4)
+    plan.add_conv2d(d, pkg.Buf.arg(0), pkg.Buf.arg(1), pkg.Buf.arg(2), pkg.Buf.none(), pkg.Buf.ws(0))
+    plan.add_pool2d(pkg.pool_desc((n, o, h, h), 2, 2, 0), pkg.Buf.ws(0), pkg.Buf.arg(3))
+    plan.finalize(n * o * h * h * 4)
+    tensors = [dev(x), dev(w), dev(b)]
+    y2 = torch.zeros((n, o, h // 2, h // 2), device="cuda")
+    plan.run(tensors + [y2]); torch.cuda.synchronize()
+    lines = plan.serialize().splitlines()
+    head = lines[0].split()
+    assert head[:2] == ["kxc_hip_plan", "2"] and head[-1] == "1"
+    old_lines = [" ".join(["kxc_hip_plan", "1"] + head[2:-1])]
+    for line in lines[1:]:
+        t = line.split()
+        if not t or t[0] != "node":
+            old_lines.append(line)
+            continue
+        # the node ends "... lane join chain np [kind offset]*np"; find np by walking back
+        k = len(t) - 1
+        while True:
+            cand = int(t[k])
+            if len(t) - 1 - k == 2 * cand:
+                break
+            k -= 2
+        assert t[k - 1] == "0"                                   # chain
+        old_lines.append(" ".join(t[:k - 1] + t[k:]))
+    y1 = torch.zeros_like(y2)
+    old = pkg.Plan.deserialize("\n".join(old_lines) + "\n", 0)
+    old.run(tensors + [y1]); torch.cuda.synchronize()
+    assert_bit_exact(host(y1), host(y2), "plan rebuilt from a version-1 text")
+    assert old.serialize() == plan.serialize()                   # written back as version 2
+    plan.close(); old.close()
+
+
 def test_plan_hip_graph_replay(pkg):
     """A launch plan replayed as a captured HIP graph gives the eager result on every replay, with eager work and
     synchronisations in between, and re-captures when an argument pointer changes.  Batch 1 exercises the
