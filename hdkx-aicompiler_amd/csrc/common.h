@@ -82,6 +82,11 @@ struct SplitReduceArgs {
     int32_t gsplit, total, O;
     uint32_t flags;            // KXC_HIP_CONV_BIAS | _RESIDUAL | _RELU
     FastDiv div_ohw;
+    // second output of a two-output launch (same shape; y2 == nullptr: none): its parts, bias and flags
+    const float* partial2 = nullptr;
+    const float* bias2 = nullptr;
+    float* y2 = nullptr;
+    uint32_t flags2 = 0;
 };
 // Scratch for the partial outputs: one grow-only buffer per (device, stream), so that launches on different
 // streams never share one.  In steady state no call allocates.  The lease keeps other host threads that enqueue

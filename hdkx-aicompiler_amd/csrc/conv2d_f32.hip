@@ -453,7 +453,8 @@ conv_mfma_kernel(const ConvArgs a) {
 
     // ---- epilogue: accumulator register g of a block holds row 8*(g/4) + 4*half + g%4, column r
     if (a.gsplit > 1) {
-        // raw partial sums of this split; conv_split_reduce_kernel finishes the layer (never with a second output)
+        // raw partial sums of this split; conv_split_reduce_kernel finishes the layer.  The parts of a second output
+        // follow those of the first: partial[gsplit + split][...].
         float* const part = a.partial + static_cast<int64_t>(split) * a.out_elems;
         if (KS == 1 || kgroup == 0) {
 #pragma unroll
@@ -464,7 +465,10 @@ conv_mfma_kernel(const ConvArgs a) {
                     if (o >= a.O) continue;
 #pragma unroll
                     for (int j = 0; j < RP; ++j)
-                        if (ybase[j] >= 0) part[ybase[j] + o * a.OHW] = acc[i][j][g];
+                        if (ybase[j] >= 0) {
+                            part[ybase[j] + o * a.OHW] = acc[i][j][g];
+                            if constexpr (DS) part[static_cast<int64_t>(a.gsplit) * a.out_elems + ybase[j] + o * a.OHW] = acc2[i][j][g];
+                        }
                 }
         }
         return;
@@ -1061,11 +1065,11 @@ int32_t Conv2dResolve(const kxc_hip_conv2d_desc* desc, bool second, const char* 
     a.cps = a.nchunks;
     a.out_elems = total;
     int split = 1;
-    if (!second) SplitOverWorkgroups(c, a.nchunks, tiles, total, &split);      // (a second output is never split)
+    SplitOverWorkgroups(c, a.nchunks, tiles, total * (second ? 2 : 1), &split);      // (a second output has parts of its own)
     if (split > 1) {
         a.cps = static_cast<int32_t>(CeilDiv(a.nchunks, split));
         a.gsplit = static_cast<int32_t>(CeilDiv(a.nchunks, a.cps));      // no empty split
-        if (a.gsplit > 1) L->scratch_bytes = static_cast<size_t>(a.gsplit) * total * sizeof(float);
+        if (a.gsplit > 1) L->scratch_bytes = static_cast<size_t>(a.gsplit) * total * sizeof(float) * (second ? 2 : 1);
         else a.cps = a.nchunks;
     }
     a.div_gsplit = MakeFastDiv(a.gsplit);
@@ -1155,6 +1159,10 @@ int32_t Conv2dLaunch(const ConvLaunch& L, const char* who, const float* x, const
         SplitReduceArgs r;
         r.partial = a.partial; r.bias = a.bias; r.res = a.res; r.y = a.y;
         r.gsplit = a.gsplit; r.total = static_cast<int32_t>(L.total); r.O = a.O; r.flags = a.flags; r.div_ohw = a.div_ohw;
+        if (second) {
+            r.partial2 = a.partial + static_cast<int64_t>(a.gsplit) * L.total;
+            r.bias2 = a.bias2; r.y2 = a.y2; r.flags2 = a.bias2 ? KXC_HIP_CONV_BIAS : 0u;
+        }
         return LaunchSplitReduce(s, r);
     }
     return KXC_HIP_OK;
@@ -1233,9 +1241,10 @@ static const Variant* PairVariant(const kxc_hip_conv2d_desc* desc) {
     Choice c;
     Select(a, desc->kh, desc->kw, &c, true);
     if (!c.v || !c.v->ds_kernel) return nullptr;
-    // A launch small enough to split its reduction over workgroups (batch 1-4 of the deep layers) gains more from
-    // that split than from the shared input, and a second output is never split: such shapes keep two launches.
-    if (!std::getenv("KXC_HIP_CONV_VARIANT")) {
+    // KXC_HIP_PAIR_SPLIT=0: a launch small enough to split its reduction over workgroups (batch 1-4 of the deep
+    // layers) keeps two launches instead of a two-output launch whose outputs both have parts.
+    const char* ps = std::getenv("KXC_HIP_PAIR_SPLIT");
+    if (ps && std::atoi(ps) == 0 && !std::getenv("KXC_HIP_CONV_VARIANT")) {
         const int32_t nchunks = (a.C + c.v->cc - 1) / c.v->cc;
         int split = 1;
         SplitOverWorkgroups(c, nchunks, CeilDiv(a.M, c.v->tp) * CeilDiv(a.O, c.v->to), static_cast<int64_t>(a.N) * a.O * a.OHW, &split);

@@ -18,13 +18,17 @@ __global__ void __launch_bounds__(256) conv_split_reduce_kernel(const SplitReduc
     // XCD x (blockIdx % 8) takes the x-th eighth of the elements, like the kernels that wrote the parts
     const int32_t per_xcd = static_cast<int32_t>(gridDim.x >> 3);
     const int32_t block = static_cast<int32_t>(blockIdx.x & 7) * per_xcd + static_cast<int32_t>(blockIdx.x >> 3);
-    const int32_t e = block * 256 + static_cast<int32_t>(threadIdx.x);
+    int32_t e = block * 256 + static_cast<int32_t>(threadIdx.x);
+    // elements total .. 2 * total - 1 are the second output of a two-output launch
+    const bool second = a.y2 != nullptr && e >= a.total;
+    if (second) e -= a.total;
     if (e >= a.total) return;
-    const float* const p = a.partial + e;
+    const float* const p = (second ? a.partial2 : a.partial) + e;
+    const uint32_t flags = second ? a.flags2 : a.flags;
     // every load of a batch of eight splits, the bias and the residual are in flight before the first addition
     float bias = 0.0f, res = 0.0f;
-    if (a.flags & KXC_HIP_CONV_BIAS) { const int32_t plane = fast_div(e, a.div_ohw); bias = a.bias[plane % a.O]; }
-    if (a.flags & KXC_HIP_CONV_RESIDUAL) res = a.res[e];
+    if (flags & KXC_HIP_CONV_BIAS) { const int32_t plane = fast_div(e, a.div_ohw); bias = (second ? a.bias2 : a.bias)[plane % a.O]; }
+    if (flags & KXC_HIP_CONV_RESIDUAL) res = a.res[e];
     float v = p[0];
     for (int32_t s0 = 1; s0 < a.gsplit; s0 += 8) {
         float t[8];
@@ -33,10 +37,10 @@ __global__ void __launch_bounds__(256) conv_split_reduce_kernel(const SplitReduc
 #pragma unroll
         for (int i = 0; i < 8; ++i) v = s0 + i < a.gsplit ? __fadd_rn(v, t[i]) : v;
     }
-    if (a.flags & KXC_HIP_CONV_BIAS) v = __fadd_rn(v, bias);
-    if (a.flags & KXC_HIP_CONV_RESIDUAL) v = __fadd_rn(v, res);
-    if (a.flags & KXC_HIP_CONV_RELU) v = relu_sel(v);
-    a.y[e] = v;
+    if (flags & KXC_HIP_CONV_BIAS) v = __fadd_rn(v, bias);
+    if (flags & KXC_HIP_CONV_RESIDUAL) v = __fadd_rn(v, res);
+    if (flags & KXC_HIP_CONV_RELU) v = relu_sel(v);
+    (second ? a.y2 : a.y)[e] = v;
 }
 
 __global__ void __launch_bounds__(256) split_counters_clear_kernel(uint32_t* counters, int32_t n) {
@@ -108,7 +112,9 @@ int32_t AcquireSplitScratch(hipStream_t stream, size_t bytes, SplitScratchLease*
 
 int32_t LaunchSplitReduce(hipStream_t stream, const SplitReduceArgs& a) {
     KXC_HIP_REQUIRE(a.gsplit >= 1 && a.total > 0 && a.O > 0 && a.partial && a.y, "split reduction: bad arguments");
-    conv_split_reduce_kernel<<<NoteGrid(static_cast<int>(CeilDiv(CeilDiv(a.total, 256), 8) * 8)), NoteBlock(256), NoteLds(0), stream>>>(a);
+    KXC_HIP_REQUIRE(!a.y2 || (a.partial2 && a.total < (1 << 30)), "split reduction: bad second output");
+    const int64_t elems = static_cast<int64_t>(a.total) * (a.y2 ? 2 : 1);
+    conv_split_reduce_kernel<<<NoteGrid(static_cast<int>(CeilDiv(CeilDiv(elems, 256), 8) * 8)), NoteBlock(256), NoteLds(0), stream>>>(a);
     return CheckLaunch("conv_split_reduce");
 }
 

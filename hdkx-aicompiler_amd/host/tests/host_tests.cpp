@@ -507,7 +507,7 @@ int RunCodegen() {
     // a ResNet-18 compile for the hip target without a GPU: plan and fusion are built, nothing is loaded
     g_mode = "hip";
     auto module = kxc::api::Compiler::Compile(kxc::models::BuildResNet18(1, 224), MakeConfig());
-    Check(module.GetKernelExecs().size() == 23, "49 Relay calls become 23 launches, got " + std::to_string(module.GetKernelExecs().size()));
+    Check(module.GetKernelExecs().size() == 20, "49 Relay calls become 20 launches, got " + std::to_string(module.GetKernelExecs().size()));
     int fused_add = 0, fused_relu = 0;
     for (const auto& e : module.GetKernelExecs()) {
         if (e.kernel_symbol.find("kxc_conv2d") == 0 && e.input_values.size() == 4) ++fused_add;

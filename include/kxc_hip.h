@@ -174,7 +174,9 @@ int32_t kxc_hip_conv2d_scratch_needed(const kxc_hip_conv2d_desc* desc, size_t* o
  * residual block's first 3x3/2 convolution and its 1x1/2 downsample (test/resnet18_ir_dump.cpp:330-352).  The 1x1
  * operand is the tap (pad/dilation) of the first convolution's window, which its staged input already holds, so
  * the input is read once and the second launch disappears.  Both outputs equal what the two separate calls give
- * (the second one bit for bit: same kernel arithmetic).
+ * (the second one bit for bit: same kernel arithmetic) unless the launch is small enough to split its reduction
+ * over workgroups: then the parts of both outputs are added in split order by one adding launch, within the fp32
+ * tolerance of the separate calls (KXC_HIP_PAIR_SPLIT=0: such shapes are reported unsupported instead).
  *   ..._supported: 1 when a matrix-core kernel with a second output covers the shape (padding a multiple of the
  *   dilation and inside the filter, and "same" padding -- 2*pad = dilation*(k-1) -- so that the unpadded 1x1
  *   convolution has the first one's output extent; no 1x1 first filter), else 0; ..._variant names it ("unsupported" otherwise). */

@@ -214,6 +214,40 @@ def test_conv_pair_against_oracle(pkg, fast_orc, synth, monkeypatch, shape):
     assert_close(host(y2), want2, what=variant + " second output (bare)")
 
 
+@pytest.mark.parametrize("shape", [(1, 64, 56, 56, 128), (1, 128, 28, 28, 256), (1, 256, 14, 14, 512), (2, 256, 14, 14, 512)],
+                         ids=["l2.0", "l3.0", "l4.0", "l4.0-n2"])
+def test_conv_pair_with_both_reductions_split_over_workgroups(pkg, fast_orc, synth, monkeypatch, shape):
+    """The ResNet-18 stride-2 blocks at batch 1-2: the launch splits its input channels over workgroups, every part
+    writes raw sums of both outputs and ONE adding launch finishes both (bias + ReLU on the first, bias on the
+    second).  Both outputs against the CPU path's separate convolutions, run to run bit-identical (the parts are
+    added in split order), and refused with KXC_HIP_PAIR_SPLIT=0."""
+    n, c, h, w, o = shape
+    xs, ws = (n, c, h, w), (o, c, 3, 3)
+    assert _scratch_needed(pkg, xs, ws, 2, 1) > 0                  # the single-output launch of this shape splits
+    assert pkg.conv2d_pair_supported(xs, ws, 2, 1)
+    seed = 6800 + 13 * c + n
+    x = synth.uniform(xs, seed)
+    w1 = synth.normal(ws, seed + 1, float(np.sqrt(2.0 / (c * 9))))
+    b1 = synth.uniform((o,), seed + 2, -0.1, 0.1)
+    w2 = synth.normal((o, c, 1, 1), seed + 3, float(np.sqrt(2.0 / c)))
+    b2 = synth.uniform((o,), seed + 4, -0.1, 0.1)
+    want1 = fast_orc.conv_chain(x, w1, b1, 2, 1, None, True)
+    want2 = fast_orc.conv_chain(x, w2, b2, 2, 0, None, False)
+    y1, y2 = pkg.conv2d_pair(dev(x), dev(w1), dev(b1), None, dev(w2), dev(b2), 2, 1, 1, True)
+    assert_close(host(y1), want1, what="split pair, first output")
+    assert_close(host(y2), want2, what="split pair, second output")
+    z1, z2 = pkg.conv2d_pair(dev(x), dev(w1), dev(b1), None, dev(w2), dev(b2), 2, 1, 1, True)
+    assert_bit_exact(host(z1), host(y1), "first output, second run")
+    assert_bit_exact(host(z2), host(y2), "second output, second run")
+    # no bias on the second output, a residual on the first
+    skip = synth.uniform(want1.shape, seed + 5)
+    y1, y2 = pkg.conv2d_pair(dev(x), dev(w1), None, dev(skip), dev(w2), None, 2, 1, 1, False)
+    assert_close(host(y1), fast_orc.conv_chain(x, w1, None, 2, 1, skip, False), what="split pair, first output (+residual)")
+    assert_close(host(y2), fast_orc.conv2d(x, w2, 2, 0), what="split pair, second output (bare)")
+    monkeypatch.setenv("KXC_HIP_PAIR_SPLIT", "0")
+    assert not pkg.conv2d_pair_supported(xs, ws, 2, 1)
+
+
 def _scratch_needed(pkg, xs, ws, s, p):
     import ctypes as C
     d = pkg.conv_desc(xs, ws, s, p, 1, 0)

@@ -154,8 +154,10 @@ def test_resnet18_cpu_backend_equals_oracle_bit_for_bit(synth):
 
 
 def test_resnet18_hip_plan_without_gpu():
-    """Compiling for the hip target needs no GPU up to loading: 49 Relay calls become 20 launches at batch 64
-    (23 at small batches, where a block's downsample keeps a launch of its own).  By default a batch of 64 runs as
+    """Compiling for the hip target needs no GPU up to loading: 49 Relay calls become 20 launches (each block's
+    downsample is the second output of the block's first convolution, at small batches with the reductions of both
+    outputs split over workgroups; KXC_HIP_PAIR_SPLIT=0 gives such a downsample a launch of its own: 23).  By
+    default a batch of 64 runs as
     two shares of 32 side by side, each those 20 launches; KXC_HIP_BATCH_LANES=1 keeps the batch whole."""
     with tempfile.TemporaryDirectory() as d:
         out = run("resnet18", "hip", d, "64", "224")
@@ -218,11 +220,20 @@ def test_resnet18_hip_matches_oracle(synth):
     with tempfile.TemporaryDirectory() as d:
         x, consts = _write_resnet_inputs(synth, d, 3, 2, 224)
         out = run("resnet18", "hip", d, "2", "224")
-        assert "execution plan replayed: 23 launches, identical output" in out
-        assert "launches: 23" in out
+        assert "execution plan replayed: 20 launches, identical output" in out
+        assert "launches: 20" in out
         got = np.fromfile(os.path.join(d, "logits.bin"), np.float32).reshape(2, 1000)
+        plan = json.load(open(os.path.join(d, "plan.json")))
+        assert sum(n["kernel_symbol"].endswith("_ds+bias+relu|conv1x1+bias") for n in plan["nodes"]) == 3
     want = Oracle(fast=True).resnet18(x, consts)
     assert_close(got, want, what="C++ host layer, ResNet-18 logits", floor="scale")
+    # a downsample of a launch that splits its reduction over workgroups as a launch of its own
+    with tempfile.TemporaryDirectory() as d:
+        _write_resnet_inputs(synth, d, 3, 2, 224)
+        out = run("resnet18", "hip", d, "2", "224", env={"KXC_HIP_PAIR_SPLIT": "0"})
+        assert "execution plan replayed: 23 launches, identical output" in out
+        apart = np.fromfile(os.path.join(d, "logits.bin"), np.float32).reshape(2, 1000)
+    assert_close(apart, want, what="C++ host layer, ResNet-18 logits, downsamples apart", floor="scale")
 
 
 @pytest.mark.gpu
@@ -233,7 +244,7 @@ def test_resnet18_hip_winograd_matches_oracle(synth):
     from gpu_util import assert_close
     with tempfile.TemporaryDirectory() as d:
         x, consts = _write_resnet_inputs(synth, d, 3, 2, 224)
-        out = run("resnet18", "hip", d, "2", "224", env={"KXC_HIP_WINOGRAD_MIN_WORK": "0", "KXC_HIP_CONCURRENT_MIN_ELEMS": "0"})
+        out = run("resnet18", "hip", d, "2", "224", env={"KXC_HIP_WINOGRAD_MIN_WORK": "0", "KXC_HIP_CONCURRENT_MIN_ELEMS": "0", "KXC_HIP_PAIR_SPLIT": "0"})
         assert "execution plan replayed: 23 launches, identical output" in out
         plan = json.load(open(os.path.join(d, "plan.json")))
         assert sum(".winograd_f2k3" in n["kernel_symbol"] for n in plan["nodes"]) == 13
@@ -330,7 +341,7 @@ def test_resnet18_benchmarked_plan_batch64_matches_oracle(synth):
 
 @pytest.mark.gpu
 def test_resnet18_two_shares_replay_from_saved_plan(synth):
-    """Four images as two shares of two (forced at this size): the saved execution plan -- 2 x 23 launches, the
+    """Four images as two shares of two (forced at this size): the saved execution plan -- 2 x 20 launches, the
     second share's as a chain on argument offsets -- rebuilds into a module that reproduces the compiled one bit for
     bit.  Against one share of four the logits agree within the operator tolerance (at this size the reductions of
     the small launches are split over different numbers of workgroups; at batch 64 the two plans take the same
@@ -341,7 +352,7 @@ def test_resnet18_two_shares_replay_from_saved_plan(synth):
         with tempfile.TemporaryDirectory() as d:
             _write_resnet_inputs(synth, d, 3, 4, 224)
             out = run("resnet18", "hip", d, "4", "224", env={"KXC_HIP_BATCH_LANES": lanes})
-            n = 23 * int(lanes)
+            n = 20 * int(lanes)
             assert "execution plan replayed: %d launches, identical output" % n in out, out[-2000:]
             plan = json.load(open(os.path.join(d, "plan.json")))
             assert len(plan["nodes"]) == n
@@ -583,7 +594,7 @@ def test_onnx_import_runs_on_hip(synth):
     with tempfile.TemporaryDirectory() as d:
         consts, x, _ = _onnx_case(synth, d, 2, 224)
         out = run("onnx", "hip", d)
-        assert "launches: 23" in out
+        assert "launches: 20" in out
         got = np.fromfile(os.path.join(d, "logits.bin"), np.float32).reshape(2, 1000)
         want = Oracle(fast=True).resnet18(x, consts)
         abs_err = np.abs(got - want)
