@@ -203,6 +203,34 @@ wino_kernel(const WinoArgs a) {
     const __amdgpu_buffer_rsrc_t xr = make_rsrc(a.x, a.x_bytes);
     const __amdgpu_buffer_rsrc_t ur = make_rsrc(a.u, a.u_bytes);
 
+    // ---- weight tile loads: 16-byte unit idx = j*NTH + tid of the tile; block h = idx / 512 is k32 group kg*WK + h
+    uint32_t uoff[ULOADS];
+#pragma unroll
+    for (int j = 0; j < ULOADS; ++j) {
+        const int idx = j * NTH + tid;
+        const int h = idx / 512, within = idx - h * 512;
+        uoff[j] = static_cast<uint32_t>((kg * WK + h) * a.csteps) * 8192u + static_cast<uint32_t>(within) * 16u;
+    }
+
+    float* const ub0 = lds + kgroup * 2 * (U_FLOATS + V_FLOATS);
+    float* const ub1 = ub0 + U_FLOATS;
+    float* const vb0 = ub0 + 2 * U_FLOATS;
+    float* const vb1 = vb0 + V_FLOATS;
+    // (the host never combines the split over workgroups with the split over wave groups)
+    const int s_lo = a.gsplit > 1 ? split * a.steps_per_split : kgroup * (a.csteps / KS);
+    const int s_hi = a.gsplit > 1 ? min(s_lo + a.steps_per_split, a.csteps) : s_lo + a.csteps / KS;
+    const int last = s_hi - 1;
+
+    auto issue_u = [&](int s, float* buf) {
+#pragma unroll
+        for (int j = 0; j < ULOADS; ++j)
+            load16_to_lds(ur, (lds_ptr_t)(buf + (j * NTH + wave * 64) * 4), uoff[j], static_cast<uint32_t>(s) * 8192u);
+    };
+    // The first weight tile is requested before anything else is computed: at small batches it comes from beyond
+    // the L2 and its latency then overlaps the gather offsets below.
+    issue_u(s_lo, ub0);
+    __builtin_amdgcn_sched_barrier(0);
+
     // ---- input items: item = tid + i*NTH -> tile = item % TT, channel = (item / TT) % 4, half = item / (4*TT)
     uint32_t goff[ITEMS][12];
     int vdst_a[ITEMS], vdst_b[ITEMS];
@@ -234,15 +262,6 @@ wino_kernel(const WinoArgs a) {
         vdst_a[i] = vrow + (half ? 64 : 0);
         vdst_b[i] = vrow + (half ? 0 : 64);
     }
-    // ---- weight tile loads: 16-byte unit idx = j*NTH + tid of the tile; block h = idx / 512 is k32 group kg*WK + h
-    uint32_t uoff[ULOADS];
-#pragma unroll
-    for (int j = 0; j < ULOADS; ++j) {
-        const int idx = j * NTH + tid;
-        const int h = idx / 512, within = idx - h * 512;
-        uoff[j] = static_cast<uint32_t>((kg * WK + h) * a.csteps) * 8192u + static_cast<uint32_t>(within) * 16u;
-    }
-
     const int a_base = wave_k * 2048 + (lane >> 4) * 512 + (lane & 15) * 4;
     const int b_base = ((lane >> 4) * WT + wave_t) * 256 + (lane & 15) * 4;
 
@@ -255,11 +274,6 @@ wino_kernel(const WinoArgs a) {
         for (int i = 0; i < ITEMS; ++i)
 #pragma unroll
             for (int q = 0; q < 12; ++q) d[i][q] = load_f32(xr, goff[i][q], soff);
-    };
-    auto issue_u = [&](int s, float* buf) {
-#pragma unroll
-        for (int j = 0; j < ULOADS; ++j)
-            load16_to_lds(ur, (lds_ptr_t)(buf + (j * NTH + wave * 64) * 4), uoff[j], static_cast<uint32_t>(s) * 8192u);
     };
     // On gfx950 the fp32 matrix instructions and the vector ALU share a datapath (measured: an independent v_add_f32
     // between two v_mfma_f32_16x16x4_f32 costs 4.3 cycles plus about 8 per change of kind; one issued by the other
@@ -314,17 +328,7 @@ wino_kernel(const WinoArgs a) {
     // KS == 2 (launches with too few units to give every SIMD two waves): the two groups of waves own their own
     // tiles and reduce one half of the input channels each, in lock step (the barriers are shared); their
     // accumulators are added through LDS after the loop.  The host passes a step count divisible by KS.
-    float* const ub0 = lds + kgroup * 2 * (U_FLOATS + V_FLOATS);
-    float* const ub1 = ub0 + U_FLOATS;
-    float* const vb0 = ub0 + 2 * U_FLOATS;
-    float* const vb1 = vb0 + V_FLOATS;
-    // (the host never combines the split over workgroups with the split over wave groups)
-    const int s_lo = a.gsplit > 1 ? split * a.steps_per_split : kgroup * (a.csteps / KS);
-    const int s_hi = a.gsplit > 1 ? min(s_lo + a.steps_per_split, a.csteps) : s_lo + a.csteps / KS;
-    const int last = s_hi - 1;
-
     // ---- prologue: weight tile and transformed input of the first step; raw input of the second in flight
-    issue_u(s_lo, ub0);
     load_raw(s_lo);
     {
         // the bias enters through the accumulators (a part of a split reduction adds none: the descriptor is empty)
