@@ -79,6 +79,56 @@ __global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2))) g
     }
 }
 
+// A handful of rows (batch 1-4 of a classifier layer): the matrix-core tile above would be 32 rows of which at
+// most 4 are real, and its k loop is a chain of dependent load latencies.  Here a wave owns four output columns for
+// every row; its lanes split k (a lane takes 4 consecutive floats of every 256), all loads of a 256-chunk are in
+// flight together, and the lanes' sums are added across the wave at the end (a tree: not the CPU order, within the
+// fp32 tolerance like the matrix-core kernel).  Measured on MI355X inside ResNet-18 (FC 512 -> 1000): batch 1
+// 0.2068 -> 0.2040 ms per pass, batch 2 0.2511 -> 0.2480, batch 4 equal, batch 8 slower (0.4643 -> 0.4728).
+constexpr int kGemvRows = 4;
+constexpr int kGemvCols = 4;
+template <int ROWS>
+__global__ void __launch_bounds__(256) gemv_nt_kernel(const float* __restrict__ a, const float* __restrict__ b,
+                                                      const float* __restrict__ c, float* __restrict__ y,
+                                                      int32_t N, int32_t K, float alpha, float beta, int64_t c_len,
+                                                      int scale_a, int scale_c) {
+    const int lane = threadIdx.x & 63;
+    const int n0 = (static_cast<int>(blockIdx.x) * 4 + static_cast<int>(threadIdx.x >> 6)) * kGemvCols;
+    if (n0 >= N) return;
+    float acc[ROWS][kGemvCols];
+#pragma unroll
+    for (int i = 0; i < ROWS; ++i)
+#pragma unroll
+        for (int j = 0; j < kGemvCols; ++j) acc[i][j] = 0.0f;
+    for (int k0 = lane * 4; k0 < K; k0 += 256) {
+        float4 vb[kGemvCols], va[ROWS];
+#pragma unroll
+        for (int j = 0; j < kGemvCols; ++j)
+            vb[j] = *reinterpret_cast<const float4*>(b + static_cast<int64_t>(min(n0 + j, N - 1)) * K + k0);
+#pragma unroll
+        for (int i = 0; i < ROWS; ++i) va[i] = *reinterpret_cast<const float4*>(a + static_cast<int64_t>(i) * K + k0);
+#pragma unroll
+        for (int i = 0; i < ROWS; ++i)
+#pragma unroll
+            for (int j = 0; j < kGemvCols; ++j) {
+                acc[i][j] = fmaf(va[i].x, vb[j].x, acc[i][j]);
+                acc[i][j] = fmaf(va[i].y, vb[j].y, acc[i][j]);
+                acc[i][j] = fmaf(va[i].z, vb[j].z, acc[i][j]);
+                acc[i][j] = fmaf(va[i].w, vb[j].w, acc[i][j]);
+            }
+    }
+#pragma unroll
+    for (int i = 0; i < ROWS; ++i)
+#pragma unroll
+        for (int j = 0; j < kGemvCols; ++j) {
+            float v = acc[i][j];
+#pragma unroll
+            for (int d = 32; d >= 1; d >>= 1) v += __shfl_xor(v, d, 64);
+            if (lane == 0 && n0 + j < N)
+                y[static_cast<int64_t>(i) * N + n0 + j] = epilogue(v, alpha, beta, c, n0 + j, c_len, scale_a != 0, scale_c != 0);
+        }
+}
+
 // Reference-order kernel: k ascending from 0.0f, multiply and add rounded separately.
 template <bool TRANS_B>
 __global__ void __launch_bounds__(256) gemm_direct_kernel(const float* __restrict__ a, const float* __restrict__ b,
@@ -234,6 +284,20 @@ int32_t kxc_hip_gemm_f32(const float* a, const float* b, const float* c, float* 
     const int scale_a = (static_cast<double>(alpha) != 1.0) ? 1 : 0;   // ScaleTensor, src/relay/op/nn/dense.cc:17-24
     const int scale_c = (static_cast<double>(beta) != 1.0) ? 1 : 0;
     const bool aligned = ((reinterpret_cast<uintptr_t>(a) | reinterpret_cast<uintptr_t>(b)) & 15u) == 0;
+    // (the same shapes as the matrix-core kernel below: whatever took the reference-order kernel still does)
+    if (transB && k > 0 && (k % 32) == 0 && aligned && m <= kGemvRows && n < (1 << 20) && k < (1 << 30)) {
+        const unsigned grid = static_cast<unsigned>(CeilDiv(n, 4 * kGemvCols));
+        const int32_t n32 = static_cast<int32_t>(n), k32 = static_cast<int32_t>(k);
+#define KXC_GEMV(R) gemv_nt_kernel<R><<<NoteGrid(grid), NoteBlock(256), NoteLds(0), s>>>(a, b, c, y, n32, k32, alpha, beta, c_len, scale_a, scale_c)
+        switch (m) {
+            case 1: KXC_GEMV(1); break;
+            case 2: KXC_GEMV(2); break;
+            case 3: KXC_GEMV(3); break;
+            default: KXC_GEMV(4); break;
+        }
+#undef KXC_GEMV
+        return CheckLaunch("gemv_nt");
+    }
     if (transB && k > 0 && (k % 32) == 0 && aligned && m < (1 << 20) && n < (1 << 20) && k < (1 << 30)) {
         dim3 grid(static_cast<unsigned>(CeilDiv(n, 32)), static_cast<unsigned>(CeilDiv(m, 32)));
         KXC_HIP_REQUIRE(grid.y <= 65535u, "kxc_hip_gemm_f32: m too large");

@@ -841,6 +841,25 @@ def test_dense_full_size(pkg, fast_orc, synth):
     assert_bit_exact(host(pkg.gemm(dev(ai), dev(np.eye(64, dtype=np.float32)))), ai, "identity weight (mfma)")
 
 
+@pytest.mark.parametrize("m", [1, 2, 3, 4, 5])
+def test_gemm_few_rows(pkg, m):
+    """Up to four rows (a classifier at batch 1-4) take the kernel whose waves split k over their lanes; five take
+    the matrix-core tile.  Against a float64 evaluation, with alpha / beta, a scalar bias and a column count that
+    leaves the last wave's columns partly empty; run to run bit-identical."""
+    rng = np.random.default_rng(4100 + m)
+    for (n, k, alpha, beta, clen) in [(1000, 512, 1.0, 1.0, 1000), (1001, 96, 0.5, 2.0, 1), (3, 32, 1.0, 1.0, 0), (130, 2048, 1.0, 1.0, 130)]:
+        a = rng.uniform(-1, 1, (m, k)).astype(np.float32)
+        b = rng.uniform(-1, 1, (n, k)).astype(np.float32)
+        c = None if clen == 0 else rng.uniform(-1, 1, (clen,)).astype(np.float32)
+        want = alpha * (a.astype(np.float64) @ b.astype(np.float64).T)
+        if c is not None:
+            want = want + beta * c.astype(np.float64)
+        got = host(pkg.gemm(dev(a), dev(b), None if c is None else dev(c), alpha, beta, 1))
+        assert_close(got, want.astype(np.float32), what="m=%d n=%d k=%d" % (m, n, k))
+        again = host(pkg.gemm(dev(a), dev(b), None if c is None else dev(c), alpha, beta, 1))
+        assert_bit_exact(again, got, "second run")
+
+
 def test_gemm_random_shapes(pkg):
     """nn_dense / nn_gemm over seeded random sizes (k a multiple of 32 takes the matrix-core kernel, anything
     else the reference-order kernel), both layouts of the second operand, alpha / beta scaling, bias of length n
