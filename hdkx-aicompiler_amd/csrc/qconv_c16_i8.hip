@@ -544,6 +544,33 @@ __global__ void __launch_bounds__(kBlock) quantize_to_c4_kernel(const float* __r
     reinterpret_cast<uint32_t*>(y)[s] = word;
 }
 
+// The same for four consecutive pixels per thread (plane size a multiple of 4, 16-byte aligned tensors): one 16-byte
+// load per channel, one 16-byte store, a quarter of the index arithmetic.  Same arithmetic per element.
+__global__ void __launch_bounds__(kBlock) quantize_to_c4_x4_kernel(const float* __restrict__ x, int8_t* __restrict__ y,
+                                                                   int32_t C, int32_t HW4, int64_t total4, float scale) {
+    const int64_t s = static_cast<int64_t>(blockIdx.x) * kBlock + threadIdx.x;
+    if (s >= total4) return;
+    const int64_t n = s / HW4;
+    const int32_t p4 = static_cast<int32_t>(s - n * HW4);
+    uint32_t word[4] = {0u, 0u, 0u, 0u};
+#pragma unroll
+    for (int c = 0; c < 4; ++c) {
+        if (c < C) {
+            const float4 v4 = reinterpret_cast<const float4*>(x)[(n * C + c) * HW4 + p4];
+            const float e[4] = {v4.x, v4.y, v4.z, v4.w};
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+                const float v = __fdiv_rn(e[i], scale);
+                float rr = rintf(v);
+                rr = (v == v) ? rr : 0.0f;
+                rr = fminf(fmaxf(rr, -127.0f), 127.0f);
+                word[i] |= (static_cast<uint32_t>(static_cast<int32_t>(rr)) & 0xffu) << (8 * c);
+            }
+        }
+    }
+    reinterpret_cast<uint4*>(y)[s] = make_uint4(word[0], word[1], word[2], word[3]);
+}
+
 // ------------------------------------------------------------------ weight packing
 struct PackArgs {
     const int8_t* w;      // OIHW
@@ -1174,6 +1201,11 @@ int32_t kxc_hip_quantize_f32_nchw_to_c4_i8(const float* x, int8_t* y, int64_t n,
     if (total == 0) return KXC_HIP_OK;
     KXC_HIP_REQUIRE(x && y, "kxc_hip_quantize_f32_nchw_to_c4_i8: NULL pointer");
     KXC_HIP_REQUIRE(CeilDiv(total, kBlock) <= kMaxGridX, "kxc_hip_quantize_f32_nchw_to_c4_i8: tensor too large");
+    if (hw % 4 == 0 && hw / 4 < (1LL << 31) && ((reinterpret_cast<uintptr_t>(x) | reinterpret_cast<uintptr_t>(y)) & 15u) == 0) {
+        quantize_to_c4_x4_kernel<<<NoteGrid(static_cast<int>(CeilDiv(total / 4, kBlock))), NoteBlock(kBlock), NoteLds(0),
+                                   ResolveStream(stream)>>>(x, y, static_cast<int32_t>(c), static_cast<int32_t>(hw / 4), total / 4, scale);
+        return CheckLaunch("quantize_f32_nchw_to_c4_i8");
+    }
     quantize_to_c4_kernel<<<NoteGrid(static_cast<int>(CeilDiv(total, kBlock))), NoteBlock(kBlock), NoteLds(0),
                             ResolveStream(stream)>>>(x, y, static_cast<int32_t>(c), hw, total, scale);
     return CheckLaunch("quantize_f32_nchw_to_c4_i8");

@@ -189,12 +189,18 @@ def test_qconv_first_layer_c4_against_cpu(pkg, orc, shape):
     assert len(np.unique(want)) > 20
 
 
-def test_quantize_to_c4(pkg, orc, synth):
-    x = synth.normal((2, 3, 12, 16), 902, 1.0)
+@pytest.mark.parametrize("shape", [(2, 3, 12, 16), (2, 3, 7, 9), (1, 4, 8, 8), (3, 1, 5, 4), (1, 2, 3, 3)],
+                         ids=["planes-of-4", "odd-planes", "four-channels", "one-channel", "two-channels-odd"])
+def test_quantize_to_c4(pkg, orc, synth, shape):
+    """Plane sizes that are multiples of four take the kernel with four pixels per thread, others one pixel per
+    thread: the same bytes, ties, saturation and NaN included."""
+    x = synth.normal(shape, 902 + shape[1] * 10 + shape[3], 1.0)
+    x.reshape(-1)[:6] = [0.5 * 0.0171, 1.5 * 0.0171, -2.5 * 0.0171, 1000.0, -1000.0, np.nan]
     q = host(pkg.quantize_to_c4(dev(x), 0.0171))
     want = orc.quantize(x, 0.0171)
-    assert_bit_exact(q[..., :3], want.transpose(0, 2, 3, 1), "quantize to c4")
-    assert (q[..., 3] == 0).all()
+    c = shape[1]
+    assert_bit_exact(q[..., :c], want.transpose(0, 2, 3, 1), "quantize to c4")
+    assert (q[..., c:] == 0).all()
 
 
 def test_qconv_c16_closed_forms(pkg):
