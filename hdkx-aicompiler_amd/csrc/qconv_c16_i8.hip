@@ -694,6 +694,56 @@ __global__ void __launch_bounds__(kBlock) maxpool_c16_kernel(const int8_t* __res
     *reinterpret_cast<int4*>(y + s * 16) = make_int4(o[0], o[1], o[2], o[3]);
 }
 
+// The same for a compile-time window every one of whose placements meets the input (the host checks): a tap
+// outside the input re-reads the nearest row / column inside it, which lies in the same window and cannot change the
+// maximum, so all KH*KW loads are issued at once, without branches.  The signed byte maxima are taken two at a time:
+// bytes 0 and 2 of a dword are moved to the high bytes of its 16-bit halves, bytes 1 and 3 are there already, and a
+// packed 16-bit signed max of such halves orders them like the bytes.
+typedef short shortx2 __attribute__((ext_vector_type(2)));
+template <int KH, int KW>
+__global__ void __launch_bounds__(kBlock) maxpool_c16_window_kernel(const int8_t* __restrict__ x, int8_t* __restrict__ y,
+                                                                    const PoolArgs d, int32_t total) {
+    const int32_t s = static_cast<int32_t>(blockIdx.x) * kBlock + static_cast<int32_t>(threadIdx.x);
+    if (s >= total) return;
+    const int32_t t = s / d.OW;
+    const int ow = s - t * d.OW;
+    const int32_t plane = t / d.OH;                  // n*CB + cb
+    const int oh = t - plane * d.OH;
+    const int4* xp = reinterpret_cast<const int4*>(x) + static_cast<int64_t>(plane) * d.H * d.W;
+    int4 v[KH][KW];
+#pragma unroll
+    for (int rh = 0; rh < KH; ++rh) {
+        const int ih = min(max(oh * d.sh + rh - d.pt, 0), d.H - 1);
+#pragma unroll
+        for (int rw = 0; rw < KW; ++rw) {
+            const int iw = min(max(ow * d.sw + rw - d.pl, 0), d.W - 1);
+            v[rh][rw] = xp[ih * d.W + iw];
+        }
+    }
+    uint32_t even[4], odd[4];
+#pragma unroll
+    for (int j = 0; j < 4; ++j) even[j] = odd[j] = 0x80008000u;
+    auto pk_max = [](uint32_t a, uint32_t b) {
+        return __builtin_bit_cast(uint32_t, __builtin_elementwise_max(__builtin_bit_cast(shortx2, a), __builtin_bit_cast(shortx2, b)));
+    };
+#pragma unroll
+    for (int rh = 0; rh < KH; ++rh)
+#pragma unroll
+        for (int rw = 0; rw < KW; ++rw) {
+            const uint32_t w[4] = {static_cast<uint32_t>(v[rh][rw].x), static_cast<uint32_t>(v[rh][rw].y),
+                                   static_cast<uint32_t>(v[rh][rw].z), static_cast<uint32_t>(v[rh][rw].w)};
+#pragma unroll
+            for (int j = 0; j < 4; ++j) {
+                even[j] = pk_max(even[j], (w[j] << 8) & 0xff00ff00u);
+                odd[j] = pk_max(odd[j], w[j] & 0xff00ff00u);
+            }
+        }
+    uint32_t o[4];
+#pragma unroll
+    for (int j = 0; j < 4; ++j) o[j] = ((even[j] >> 8) & 0x00ff00ffu) | (odd[j] & 0xff00ff00u);
+    reinterpret_cast<int4*>(y)[s] = make_int4(static_cast<int>(o[0]), static_cast<int>(o[1]), static_cast<int>(o[2]), static_cast<int>(o[3]));
+}
+
 // Four threads per (n, channel block) plane, each summing one dword (4 channels) of every position; output
 // [N][CB*16] (= c16 with H = W = 1).
 __global__ void __launch_bounds__(kBlock) gap_c16_kernel(const int8_t* __restrict__ x, int8_t* __restrict__ y,
@@ -1070,6 +1120,15 @@ int32_t kxc_hip_maxpool2d_c16_i8(const kxc_hip_pool2d_desc* p, const int8_t* x, 
     if (total == 0) return KXC_HIP_OK;
     KXC_HIP_REQUIRE(x && y, "kxc_hip_maxpool2d_c16_i8: NULL pointer");
     KXC_HIP_REQUIRE(CeilDiv(total, kBlock) <= kMaxGridX, "kxc_hip_maxpool2d_c16_i8: tensor too large");
+    // every placement of a 3x3 window meets the input (first window's last row / column, last window's first)
+    const bool meets = d.pt <= d.KH - 1 && d.pl <= d.KW - 1 && (d.OH - 1) * d.sh - d.pt <= d.H - 1 && (d.OW - 1) * d.sw - d.pl <= d.W - 1;
+    const int64_t in_words = static_cast<int64_t>(d.N) * d.CB * d.H * d.W;
+    if (d.KH == 3 && d.KW == 3 && meets && total < (1LL << 31) && in_words < (1LL << 31) &&
+        ((reinterpret_cast<uintptr_t>(x) | reinterpret_cast<uintptr_t>(y)) & 15u) == 0) {
+        maxpool_c16_window_kernel<3, 3><<<NoteGrid(static_cast<int>(CeilDiv(total, kBlock))), NoteBlock(kBlock), NoteLds(0), ResolveStream(stream)>>>(
+            x, y, d, static_cast<int32_t>(total));
+        return CheckLaunch("maxpool2d_c16_i8");
+    }
     maxpool_c16_kernel<<<NoteGrid(static_cast<int>(CeilDiv(total, kBlock))), NoteBlock(kBlock), NoteLds(0), ResolveStream(stream)>>>(x, y, d, total);
     return CheckLaunch("maxpool2d_c16_i8");
 }

@@ -241,6 +241,14 @@ def test_pools_c16(pkg, orc):
     x = rng.integers(-128, 128, (2, 40, 17, 16), dtype=np.int8)
     got = pkg.maxpool2d_c16_i8(to_c16(pkg, x), 40, 3, 2, 1)
     assert_bit_exact(from_c16(pkg, got, 40), orc.qmaxpool(x, 3, 2, 1), "maxpool c16")
+    # 3x3 windows take the kernel that loads all nine taps at once (taps outside the input re-read the edge), other
+    # windows the general one: strides 1-3, padding 0-2, a one-row input, extreme values at the borders
+    for (shape, k, st, pad) in [((1, 16, 9, 11), 3, 1, 1), ((2, 17, 8, 8), 3, 2, 0), ((1, 32, 1, 7), 3, 2, 1), ((1, 16, 12, 5), 3, 3, 2),
+                                ((2, 16, 10, 10), 2, 2, 0), ((1, 16, 7, 7), 5, 2, 2)]:
+        x = rng.integers(-128, 128, shape, dtype=np.int8)
+        x[:, :, 0, :] = -128; x[:, :, -1, -1] = 127
+        got = pkg.maxpool2d_c16_i8(to_c16(pkg, x), shape[1], k, st, pad)
+        assert_bit_exact(from_c16(pkg, got, shape[1]), orc.qmaxpool(x, k, st, pad), "maxpool c16 %s k%d s%d p%d" % (shape, k, st, pad))
     x = rng.integers(-128, 128, (3, 64, 7, 7), dtype=np.int8)
     got = host(pkg.global_avg_pool2d_c16_i8(to_c16(pkg, x), 64, 0.0173))
     assert_bit_exact(got, orc.qgap(x, 0.0173).reshape(3, 64), "gap c16")
