@@ -158,6 +158,16 @@ struct WinoWeightJob {
 };
 int32_t LaunchWinogradWeightTransforms(const WinoWeightJob* jobs, int32_t count, hipStream_t stream);
 
+// The int8 weight tensors of several convolutions packed by one launch (qconv_c16_i8.hip); kind = KXC_HIP_QPACK_*.
+struct QPackJob {
+    int32_t kind;
+    const kxc_hip_qconv2d_desc* desc;
+    const int8_t* w;     // OIHW
+    int8_t* wp;          // QPackedBytes(job) bytes
+};
+int32_t QPackedBytes(const QPackJob& job, size_t* out_bytes);
+int32_t LaunchQWeightPacks(const QPackJob* jobs, int32_t count, hipStream_t stream);
+
 // Activity recording (activity.hip).  ApiScope times one HIP runtime call on the host; DeviceScope brackets the
 // copy / fill / kernel that call enqueues with two HIP events on its stream.  Both do nothing while recording is off.
 bool ActivityOn();

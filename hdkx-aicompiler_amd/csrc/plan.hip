@@ -21,8 +21,9 @@ namespace {
 
 enum class NodeKind {
     kConv2D, kPool2D, kGlobalAvgPool, kGemm, kBinary, kRelu, kCopy,
-    kQConv2D, kQuantize, kMaxPoolI8, kGlobalAvgPoolI8, kQDense, kModuleKernel
+    kQConv2D, kQuantize, kMaxPoolI8, kGlobalAvgPoolI8, kQDense, kModuleKernel, kI8Layout
 };
+constexpr NodeKind kLastNodeKind = NodeKind::kI8Layout;
 
 struct Node {
     NodeKind kind;
@@ -53,8 +54,23 @@ struct Node {
     std::vector<kxc_hip_buf> params;
 };
 
-// Bytes of every operand whose size follows from the node's geometry (fp32 operators; the int8 nodes' blocked
-// layouts and module kernels' parameters are checked by offset only).
+// A weight tensor that is packed for its kernel at the start of a run (kxc_hip_plan_add_qconv_weight_pack).
+struct PackJob {
+    int32_t kind = 0;                     // KXC_HIP_QPACK_*
+    kxc_hip_qconv2d_desc desc;
+    kxc_hip_buf w, wp;
+    int32_t every_run = 0;
+    const void* packed_from = nullptr;    // the weight pointer whose packed form wp holds
+};
+
+int64_t PoolOutDim(const kxc_hip_pool2d_desc& d, int64_t in, int64_t k, int64_t s, int64_t p0, int64_t p1) {
+    const int64_t span = in + p0 + p1 - k;
+    if (span < 0 || s <= 0) return 0;
+    return (d.ceil_mode ? (span + s - 1) / s : span / s) + 1;      // as the pooling entry points size their output
+}
+
+// Bytes of every operand whose size follows from the node's geometry (module kernels' parameters are checked by
+// offset only).
 void OperandExtents(const Node& n, std::vector<std::pair<kxc_hip_buf, size_t>>* out) {
     auto add = [&](const kxc_hip_buf& b, int64_t elems, size_t elem_bytes = 4) {
         if (b.kind != KXC_HIP_BUF_NONE && elems > 0) out->emplace_back(b, static_cast<size_t>(elems) * elem_bytes);
@@ -83,14 +99,76 @@ void OperandExtents(const Node& n, std::vector<std::pair<kxc_hip_buf, size_t>>* 
         }
         case NodeKind::kPool2D: {
             const kxc_hip_pool2d_desc& d = n.pool;
-            auto dim = [&](int64_t in, int64_t k, int64_t s, int64_t p0, int64_t p1) {
-                const int64_t span = in + p0 + p1 - k;
-                if (span < 0 || s <= 0) return static_cast<int64_t>(0);
-                return (d.ceil_mode ? (span + s - 1) / s : span / s) + 1;      // as kxc_hip_pool2d_f32 sizes its output
-            };
             add(n.bufs[0], static_cast<int64_t>(d.n) * d.c * d.h * d.w);
-            add(n.bufs[1], static_cast<int64_t>(d.n) * d.c * dim(d.h, d.kh, d.stride_h, d.pad_top, d.pad_bottom) *
-                               dim(d.w, d.kw, d.stride_w, d.pad_left, d.pad_right));
+            add(n.bufs[1], static_cast<int64_t>(d.n) * d.c * PoolOutDim(d, d.h, d.kh, d.stride_h, d.pad_top, d.pad_bottom) *
+                               PoolOutDim(d, d.w, d.kw, d.stride_w, d.pad_left, d.pad_right));
+            break;
+        }
+        case NodeKind::kMaxPoolI8: {
+            // i32[0] == 1: channel-blocked (16 bytes per position and block of 16 channels)
+            const kxc_hip_pool2d_desc& d = n.pool;
+            const int64_t cbytes = n.i32[0] == 1 ? (static_cast<int64_t>(d.c) + 15) / 16 * 16 : d.c;
+            add(n.bufs[0], static_cast<int64_t>(d.n) * cbytes * d.h * d.w, 1);
+            add(n.bufs[1], static_cast<int64_t>(d.n) * cbytes * PoolOutDim(d, d.h, d.kh, d.stride_h, d.pad_top, d.pad_bottom) *
+                               PoolOutDim(d, d.w, d.kw, d.stride_w, d.pad_left, d.pad_right), 1);
+            break;
+        }
+        case NodeKind::kGlobalAvgPoolI8: {
+            const int64_t cbytes = n.i32[0] == 1 ? (n.dims[1] + 15) / 16 * 16 : n.dims[1];
+            add(n.bufs[0], n.dims[0] * cbytes * n.dims[2] * n.dims[3], 1);
+            add(n.bufs[1], n.dims[0] * cbytes, 1);
+            break;
+        }
+        case NodeKind::kQuantize:
+            if (n.i32[0] == 0) {
+                add(n.bufs[0], n.dims[0]);
+                add(n.bufs[1], n.dims[0], 1);
+            } else {
+                // dims = {n, c, h*w}; i32[0] == 1: c16 output, 2: c4 output
+                add(n.bufs[0], n.dims[0] * n.dims[1] * n.dims[2]);
+                add(n.bufs[1], n.dims[0] * (n.i32[0] == 1 ? (n.dims[1] + 15) / 16 * 16 : 4) * n.dims[2], 1);
+            }
+            break;
+        case NodeKind::kI8Layout: {
+            // dims = {n, c, h*w}; i32[0] != 0: NCHW -> c16
+            const int64_t plain = n.dims[0] * n.dims[1] * n.dims[2], blocked = n.dims[0] * ((n.dims[1] + 15) / 16 * 16) * n.dims[2];
+            add(n.bufs[0], n.i32[0] ? plain : blocked, 1);
+            add(n.bufs[1], n.i32[0] ? blocked : plain, 1);
+            break;
+        }
+        case NodeKind::kQDense:
+            add(n.bufs[0], n.dims[0] * n.dims[2], 1);
+            add(n.bufs[1], n.dims[1] * n.dims[2], 1);
+            add(n.bufs[2], n.dims[1]);
+            add(n.bufs[3], n.dims[1]);
+            add(n.bufs[4], n.dims[0] * n.dims[1]);
+            break;
+        case NodeKind::kQConv2D: {
+            // i32[0]: 0 NCHW, 1 c16, 2 c4 input / c16 output, 3 c16 with a second output (params)
+            const kxc_hip_qconv2d_desc& d = n.qconv;
+            if (d.stride_h <= 0 || d.stride_w <= 0) break;
+            const int64_t oh = (static_cast<int64_t>(d.h) + 2 * d.pad_h - d.kh) / d.stride_h + 1;
+            const int64_t ow = (static_cast<int64_t>(d.w) + 2 * d.pad_w - d.kw) / d.stride_w + 1;
+            const int mode = n.i32[0];
+            const int64_t ob = mode == 0 ? d.o : (static_cast<int64_t>(d.o) + 15) / 16 * 16;
+            const int64_t y = static_cast<int64_t>(d.n) * ob * oh * ow;
+            const int64_t xc = mode == 0 ? d.c : mode == 2 ? 4 : (static_cast<int64_t>(d.c) + 15) / 16 * 16;
+            add(n.bufs[0], static_cast<int64_t>(d.n) * xc * d.h * d.w, 1);
+            size_t wbytes = static_cast<size_t>(d.o) * d.c * d.kh * d.kw;
+            if (mode == 1 || mode == 3) { if (kxc_hip_qconv2d_c16_packed_bytes(&d, &wbytes) != KXC_HIP_OK) wbytes = 0; }
+            if (mode == 2) { if (kxc_hip_qconv2d_c4_packed_bytes(&d, &wbytes) != KXC_HIP_OK) wbytes = 0; }
+            add(n.bufs[1], static_cast<int64_t>(wbytes), 1);
+            add(n.bufs[2], d.o);
+            add(n.bufs[3], d.o);
+            add(n.bufs[4], y, 1);
+            add(n.bufs[5], y, 1);
+            if (mode == 3 && n.params.size() == 4) {
+                size_t w2 = 0;
+                if (kxc_hip_qconv2d_c16_pair_packed_bytes(&d, &w2) == KXC_HIP_OK) add(n.params[0], static_cast<int64_t>(w2), 1);
+                add(n.params[1], d.o);
+                add(n.params[2], d.o);
+                add(n.params[3], y, 1);
+            }
             break;
         }
         case NodeKind::kGlobalAvgPool:
@@ -133,6 +211,7 @@ struct kxc_hip_plan {
     int32_t device_id = 0;
     int32_t num_args = 0;
     std::vector<Node> nodes;
+    std::vector<PackJob> packs;
     void* workspace = nullptr;
     size_t workspace_bytes = 0;
     bool finalized = false;
@@ -153,8 +232,8 @@ struct kxc_hip_plan {
     hipGraphExec_t graph_exec = nullptr;
     std::vector<void*> graph_args;
     hipStream_t graph_stream = nullptr;   // the graph is replayed only on the stream it was captured on
-    // Constants of Winograd nodes.  Default: the filter transforms of all such nodes run at the start of EVERY
-    // run (one launch), so weights rewritten in place -- or another tensor at the same address -- are seen, as
+    // Constants of Winograd nodes and of the int8 matrix-core convolutions (packs).  Default: the filter transforms
+    // of all such nodes run at the start of EVERY run (one launch each kind), so weights rewritten in place -- or another tensor at the same address -- are seen, as
     // with the CPU backend, which re-reads every constant on every call.  Frozen (kxc_hip_plan_freeze_constants):
     // transformed when first seen or when another pointer arrives; constants_ready orders runs on other streams
     // after the stream the transforms were enqueued on.
@@ -306,6 +385,7 @@ int32_t kxc_hip_plan_add_conv2d_pair(kxc_hip_plan* plan, const kxc_hip_conv2d_de
 int32_t kxc_hip_plan_invalidate_constants(kxc_hip_plan* plan) {
     KXC_HIP_REQUIRE(plan != nullptr, "kxc_hip_plan_invalidate_constants: plan is NULL");
     for (Node& n : plan->nodes) n.transformed_from = nullptr;
+    for (PackJob& j : plan->packs) j.packed_from = nullptr;
     return KXC_HIP_OK;
 }
 
@@ -313,6 +393,7 @@ int32_t kxc_hip_plan_freeze_constants(kxc_hip_plan* plan, int32_t frozen) {
     KXC_HIP_REQUIRE(plan != nullptr, "kxc_hip_plan_freeze_constants: plan is NULL");
     plan->constants_frozen = frozen != 0;
     for (Node& n : plan->nodes) n.transformed_from = nullptr;      // the next run transforms what it is given
+    for (PackJob& j : plan->packs) j.packed_from = nullptr;
     if (plan->graph_exec) {       // a captured graph holds the other mode's launches
         (void)hipGraphExecDestroy(plan->graph_exec); plan->graph_exec = nullptr;
         if (plan->graph) { (void)hipGraphDestroy(plan->graph); plan->graph = nullptr; }
@@ -577,6 +658,42 @@ int32_t kxc_hip_plan_add_global_avg_pool2d_c16_i8(kxc_hip_plan* plan, int64_t nn
     return KXC_HIP_OK;
 }
 
+int32_t kxc_hip_plan_add_i8_layout(kxc_hip_plan* plan, int32_t to_c16, int64_t nn, int64_t c, int64_t hw, kxc_hip_buf x,
+                                   kxc_hip_buf y) {
+    const char* who = "kxc_hip_plan_add_i8_layout";
+    KXC_PLAN_BEGIN(who);
+    KXC_HIP_REQUIRE(nn >= 0 && c > 0 && hw >= 0, "%s: bad shape", who);
+    KXC_PLAN_BUF(x, false, who); KXC_PLAN_BUF(y, false, who);
+    Node n{};
+    n.kind = NodeKind::kI8Layout;
+    n.dims[0] = nn; n.dims[1] = c; n.dims[2] = hw;
+    n.i32[0] = to_c16 ? 1 : 0;
+    n.bufs[0] = x; n.bufs[1] = y;
+    n.symbol = to_c16 ? "kxc_i8_nchw_to_c16" : "kxc_i8_c16_to_nchw";
+    plan->nodes.push_back(n);
+    return KXC_HIP_OK;
+}
+
+int32_t kxc_hip_plan_add_qconv_weight_pack(kxc_hip_plan* plan, int32_t kind, const kxc_hip_qconv2d_desc* desc,
+                                           kxc_hip_buf w_oihw, kxc_hip_buf w_packed, int32_t every_run) {
+    const char* who = "kxc_hip_plan_add_qconv_weight_pack";
+    KXC_PLAN_BEGIN(who);
+    KXC_HIP_REQUIRE(desc != nullptr, "%s: desc is NULL", who);
+    KXC_HIP_REQUIRE(w_oihw.kind == KXC_HIP_BUF_ARG || w_oihw.kind == KXC_HIP_BUF_ARG_OFFSET,
+                    "%s: the weights must be a packed argument (they are read before the first node runs)", who);
+    KXC_HIP_REQUIRE(w_packed.kind == KXC_HIP_BUF_WORKSPACE, "%s: the packed weights live in the plan workspace", who);
+    KXC_PLAN_BUF(w_oihw, false, who); KXC_PLAN_BUF(w_packed, false, who);
+    PackJob j;
+    j.kind = kind; j.desc = *desc; j.w = w_oihw; j.wp = w_packed; j.every_run = every_run ? 1 : 0;
+    size_t bytes = 0;
+    const QPackJob probe{kind, desc, nullptr, nullptr};
+    if (int32_t rc = QPackedBytes(probe, &bytes)) return rc;
+    plan->packs.push_back(j);
+    return KXC_HIP_OK;
+}
+
+int32_t kxc_hip_plan_num_weight_packs(const kxc_hip_plan* plan) { return plan ? static_cast<int32_t>(plan->packs.size()) : 0; }
+
 int32_t kxc_hip_plan_add_module_kernel(kxc_hip_plan* plan, void* function, const char* symbol, const uint32_t grid[3],
                                        const uint32_t block[3], uint32_t shared_bytes, const kxc_hip_buf* params,
                                        int32_t num_params) {
@@ -630,28 +747,14 @@ int32_t kxc_hip_plan_finalize(kxc_hip_plan* plan, size_t workspace_bytes) {
                             "kxc_hip_plan_finalize: node %s uses a workspace offset beyond %zu bytes", n.symbol.c_str(),
                             workspace_bytes);
     }
-    if (workspace_bytes > 0) {
-        KXC_HIP_CALL(hipSetDevice(plan->device_id), "HIP SetDevice");
-        KXC_HIP_CALL(hipMalloc(&plan->workspace, workspace_bytes), "plan workspace allocation");
-    }
-    plan->workspace_bytes = workspace_bytes;
-    for (Node& n : plan->nodes) {
-        if (n.lane != 1) continue;
-        if (!plan->side_stream) {
-            KXC_HIP_CALL(hipSetDevice(plan->device_id), "HIP SetDevice");
-            KXC_HIP_CALL(hipStreamCreateWithFlags(&plan->side_stream, hipStreamNonBlocking), "plan side stream");
-        }
-        KXC_HIP_CALL(hipEventCreateWithFlags(&n.fork_event, hipEventDisableTiming), "plan event");
-        KXC_HIP_CALL(hipEventCreateWithFlags(&n.done_event, hipEventDisableTiming), "plan event");
-    }
-    for (const Node& n : plan->nodes) plan->num_chains = std::max(plan->num_chains, n.chain);
-    if (plan->num_chains > 0) {
-        KXC_HIP_CALL(hipSetDevice(plan->device_id), "HIP SetDevice");
-        KXC_HIP_CALL(hipEventCreateWithFlags(&plan->chain_fork, hipEventDisableTiming), "plan event");
-        for (int32_t c = 0; c < plan->num_chains; ++c) {
-            KXC_HIP_CALL(hipStreamCreateWithFlags(&plan->chain_streams[c], hipStreamNonBlocking), "plan chain stream");
-            KXC_HIP_CALL(hipEventCreateWithFlags(&plan->chain_done[c], hipEventDisableTiming), "plan event");
-        }
+    for (const PackJob& j : plan->packs) {
+        size_t bytes = 0;
+        const QPackJob probe{j.kind, &j.desc, nullptr, nullptr};
+        if (int32_t rc = QPackedBytes(probe, &bytes)) return rc;
+        const size_t off = static_cast<size_t>(j.wp.index_or_offset);
+        KXC_HIP_REQUIRE(off <= workspace_bytes && bytes <= workspace_bytes - off,
+                        "kxc_hip_plan_finalize: packed weights of %zu bytes at workspace offset %zu do not fit the %zu-byte workspace",
+                        bytes, off, workspace_bytes);
     }
     // the variants below are chosen for select_lanes equal launches side by side
     struct LanesScope {
@@ -661,7 +764,7 @@ int32_t kxc_hip_plan_finalize(kxc_hip_plan* plan, size_t workspace_bytes) {
     } lanes_scope(plan->select_lanes);
     // Resolve every convolution launch now: the runs only add the operand pointers and the stream.  The node's
     // symbol names the variant resolved here (the one chosen when the node was added may have been picked under
-    // other environment switches).
+    // other environment switches).  (Before anything is allocated: a failure here leaves nothing behind.)
     for (Node& n : plan->nodes) {
         if (n.kind != NodeKind::kConv2D) continue;
         KXC_HIP_CALL(hipSetDevice(plan->device_id), "HIP SetDevice");
@@ -684,6 +787,32 @@ int32_t kxc_hip_plan_finalize(kxc_hip_plan* plan, size_t workspace_bytes) {
             n.prepared_conv.reset(p, kxc_hip::FreePreparedConv);
         }
     }
+    // Streams, events and the workspace: what a failed call has created so far is kept by the plan and reused by a
+    // second call (kxc_hip_plan_destroy releases it either way).
+    for (Node& n : plan->nodes) {
+        if (n.lane != 1) continue;
+        if (!plan->side_stream) {
+            KXC_HIP_CALL(hipSetDevice(plan->device_id), "HIP SetDevice");
+            KXC_HIP_CALL(hipStreamCreateWithFlags(&plan->side_stream, hipStreamNonBlocking), "plan side stream");
+        }
+        if (!n.fork_event) KXC_HIP_CALL(hipEventCreateWithFlags(&n.fork_event, hipEventDisableTiming), "plan event");
+        if (!n.done_event) KXC_HIP_CALL(hipEventCreateWithFlags(&n.done_event, hipEventDisableTiming), "plan event");
+    }
+    for (const Node& n : plan->nodes) plan->num_chains = std::max(plan->num_chains, n.chain);
+    if (plan->num_chains > 0) {
+        KXC_HIP_CALL(hipSetDevice(plan->device_id), "HIP SetDevice");
+        if (!plan->chain_fork) KXC_HIP_CALL(hipEventCreateWithFlags(&plan->chain_fork, hipEventDisableTiming), "plan event");
+        for (int32_t c = 0; c < plan->num_chains; ++c) {
+            if (!plan->chain_streams[c])
+                KXC_HIP_CALL(hipStreamCreateWithFlags(&plan->chain_streams[c], hipStreamNonBlocking), "plan chain stream");
+            if (!plan->chain_done[c]) KXC_HIP_CALL(hipEventCreateWithFlags(&plan->chain_done[c], hipEventDisableTiming), "plan event");
+        }
+    }
+    if (workspace_bytes > 0 && !plan->workspace) {
+        KXC_HIP_CALL(hipSetDevice(plan->device_id), "HIP SetDevice");
+        KXC_HIP_CALL(hipMalloc(&plan->workspace, workspace_bytes), "plan workspace allocation");
+    }
+    plan->workspace_bytes = workspace_bytes;
     plan->finalized = true;
     return KXC_HIP_OK;
 }
@@ -701,24 +830,45 @@ int32_t CheckRunArgs(kxc_hip_plan* plan, void** args, const char* who) {
     return KXC_HIP_OK;
 }
 
-// The filter transforms of the plan's Winograd nodes, all in one launch on `stream`: every node's (only_changed:
-// those whose weight pointer differs from the one last transformed).  *launched tells whether anything ran.
+// The filter transforms of the plan's Winograd nodes and the weight packs of its int8 convolutions, each kind in one
+// launch on `stream`: every one (only_changed: those whose weight pointer differs from the one last prepared, and the
+// packs marked every_run).  *launched tells whether anything ran.  What was prepared is recorded only after its
+// launch has been enqueued without error, so a failed run is repeated by the next one.
 int32_t TransformConstants(kxc_hip_plan* plan, void** args, hipStream_t stream, bool only_changed, bool* launched) {
     std::vector<WinoWeightJob> jobs;
+    std::vector<std::pair<Node*, const void*>> touched;
     for (Node& n : plan->nodes) {
         if (n.kind != NodeKind::kConv2D || n.i32[0] != 1) continue;
         const void* w = Resolve(plan, n.bufs[1], args);
         if (only_changed && n.transformed_from == w) continue;
-        n.transformed_from = w;
+        touched.emplace_back(&n, w);
         // (nodes of different chains that share a transformed-weight buffer: one transform)
         float* const u = static_cast<float*>(Resolve(plan, n.bufs[5], args));
         bool have = false;
         for (const WinoWeightJob& j : jobs) have = have || (j.u == u && j.w == w);
         if (!have) jobs.push_back({&n.conv, static_cast<const float*>(w), u});
     }
-    *launched = !jobs.empty();
-    if (jobs.empty()) return KXC_HIP_OK;
-    return LaunchWinogradWeightTransforms(jobs.data(), static_cast<int32_t>(jobs.size()), stream);
+    std::vector<QPackJob> packs;
+    std::vector<std::pair<PackJob*, const void*>> packed;
+    for (PackJob& j : plan->packs) {
+        const void* w = Resolve(plan, j.w, args);
+        if (only_changed && !j.every_run && j.packed_from == w) continue;
+        packed.emplace_back(&j, w);
+        int8_t* const wp = static_cast<int8_t*>(Resolve(plan, j.wp, args));
+        bool have = false;
+        for (const QPackJob& q : packs) have = have || (q.wp == wp && q.w == w && q.kind == j.kind);
+        if (!have) packs.push_back({j.kind, &j.desc, static_cast<const int8_t*>(w), wp});
+    }
+    *launched = !jobs.empty() || !packs.empty();
+    if (!jobs.empty()) {
+        if (int32_t rc = LaunchWinogradWeightTransforms(jobs.data(), static_cast<int32_t>(jobs.size()), stream)) return rc;
+        for (auto& t : touched) t.first->transformed_from = t.second;
+    }
+    if (!packs.empty()) {
+        if (int32_t rc = LaunchQWeightPacks(packs.data(), static_cast<int32_t>(packs.size()), stream)) return rc;
+        for (auto& t : packed) t.first->packed_from = t.second;
+    }
+    return KXC_HIP_OK;
 }
 
 // Frozen constants: transform what has not been seen yet (outside any stream capture), and order a run on another
@@ -850,6 +1000,12 @@ int32_t RunNode(kxc_hip_plan* plan, Node& n, void** args, void* s) {
                 rc = kxc_hip_qdense_i8(static_cast<const int8_t*>(B(0)), static_cast<const int8_t*>(B(1)),
                                        static_cast<const int32_t*>(B(2)), static_cast<const float*>(B(3)),
                                        static_cast<float*>(B(4)), n.dims[0], n.dims[1], n.dims[2], s);
+                break;
+            case NodeKind::kI8Layout:
+                rc = n.i32[0] ? kxc_hip_i8_nchw_to_c16(static_cast<const int8_t*>(B(0)), static_cast<int8_t*>(B(1)), n.dims[0],
+                                                       n.dims[1], n.dims[2], s)
+                              : kxc_hip_i8_c16_to_nchw(static_cast<const int8_t*>(B(0)), static_cast<int8_t*>(B(1)), n.dims[0],
+                                                       n.dims[1], n.dims[2], s);
                 break;
             case NodeKind::kModuleKernel: {
                 // every parameter is a device pointer; hipModuleLaunchKernel wants the address of each
@@ -1102,10 +1258,11 @@ int32_t kxc_hip_plan_serialize(const kxc_hip_plan* plan, char* buffer, size_t ca
     char tmp[96];
     auto I = [&](long long v) { std::snprintf(tmp, sizeof(tmp), " %lld", v); out += tmp; };
     auto F = [&](float v) { std::snprintf(tmp, sizeof(tmp), " %a", static_cast<double>(v)); out += tmp; };
-    // (version 2 added the plan's select_lanes and every node's chain)
-    out += "kxc_hip_plan 2";
+    // (version 2 added the plan's select_lanes and every node's chain, version 3 the weight packs)
+    out += "kxc_hip_plan 3";
     I(plan->num_args); I(static_cast<long long>(plan->workspace_bytes)); I(static_cast<long long>(plan->nodes.size()));
     I(plan->select_lanes);
+    I(static_cast<long long>(plan->packs.size()));
     out += "\n";
     for (const Node& n : plan->nodes) {
         KXC_HIP_REQUIRE(n.symbol.find_first_of(" \n\t") == std::string::npos,
@@ -1140,6 +1297,17 @@ int32_t kxc_hip_plan_serialize(const kxc_hip_plan* plan, char* buffer, size_t ca
         for (const kxc_hip_buf& b : n.params) { I(b.kind); I(b.index_or_offset); }
         out += "\n";
     }
+    for (const PackJob& j : plan->packs) {
+        out += "pack";
+        I(j.kind); I(j.every_run);
+        I(j.w.kind); I(j.w.index_or_offset); I(j.wp.kind); I(j.wp.index_or_offset);
+        const kxc_hip_qconv2d_desc& q = j.desc;
+        for (long long v : {(long long)q.n, (long long)q.c, (long long)q.h, (long long)q.w, (long long)q.o, (long long)q.kh,
+                            (long long)q.kw, (long long)q.stride_h, (long long)q.stride_w, (long long)q.pad_h, (long long)q.pad_w,
+                            (long long)q.flags}) I(v);
+        F(q.res_mult);
+        out += "\n";
+    }
     *needed = out.size() + 1;
     if (buffer == nullptr || capacity == 0) return KXC_HIP_OK;
     KXC_HIP_REQUIRE(capacity >= *needed, "kxc_hip_plan_serialize: %zu bytes needed, room for %zu", *needed, capacity);
@@ -1154,10 +1322,12 @@ int32_t kxc_hip_plan_deserialize(const char* text, int32_t device_id, kxc_hip_mo
     std::istringstream in{std::string(text)};
     std::string magic;
     long long version = 0, num_args = 0, workspace = 0, count = 0;
-    long long select_lanes = 1;
+    long long select_lanes = 1, num_packs = 0;
     in >> magic >> version >> num_args >> workspace >> count;
-    if (in && version == 2) in >> select_lanes;
-    KXC_HIP_REQUIRE(in && magic == "kxc_hip_plan" && (version == 1 || version == 2), "%s: not a version-1 or version-2 plan", who);
+    if (in && version >= 2) in >> select_lanes;
+    if (in && version >= 3) in >> num_packs;
+    KXC_HIP_REQUIRE(in && magic == "kxc_hip_plan" && version >= 1 && version <= 3, "%s: not a version-1, -2 or -3 plan", who);
+    KXC_HIP_REQUIRE(num_packs >= 0 && num_packs < (1 << 20), "%s: implausible header", who);
     KXC_HIP_REQUIRE(select_lanes >= 1 && select_lanes <= 16, "%s: implausible header", who);
     KXC_HIP_REQUIRE(num_args >= 0 && num_args < (1 << 20) && workspace >= 0 && count >= 0 && count < (1 << 24),
                     "%s: implausible header", who);
@@ -1173,7 +1343,7 @@ int32_t kxc_hip_plan_deserialize(const char* text, int32_t device_id, kxc_hip_mo
         long long kind = -1;
         Node n{};
         in >> tag >> kind >> n.symbol;
-        if (!in || tag != "node" || kind < 0 || kind > static_cast<long long>(NodeKind::kModuleKernel)) return fail("bad node line");
+        if (!in || tag != "node" || kind < 0 || kind > static_cast<long long>(kLastNodeKind)) return fail("bad node line");
         n.kind = static_cast<NodeKind>(kind);
         long long v = 0;
         auto I = [&]() { in >> v; return v; };
@@ -1240,6 +1410,34 @@ int32_t kxc_hip_plan_deserialize(const char* text, int32_t device_id, kxc_hip_mo
                 return fail("bad launch geometry");
         }
         plan->nodes.push_back(n);
+    }
+    for (long long k = 0; k < num_packs; ++k) {
+        std::string tag;
+        PackJob j;
+        long long v = 0;
+        auto I = [&]() { in >> v; return v; };
+        in >> tag;
+        if (!in || tag != "pack") return fail("bad pack line");
+        j.kind = static_cast<int32_t>(I()); j.every_run = static_cast<int32_t>(I());
+        j.w.kind = static_cast<int32_t>(I()); j.w.index_or_offset = I();
+        j.wp.kind = static_cast<int32_t>(I()); j.wp.index_or_offset = I();
+        kxc_hip_qconv2d_desc& q = j.desc;
+        q.n = I(); q.c = I(); q.h = I(); q.w = I(); q.o = I(); q.kh = I(); q.kw = I(); q.stride_h = I(); q.stride_w = I();
+        q.pad_h = I(); q.pad_w = I(); q.flags = static_cast<uint32_t>(I());
+        std::string t;
+        in >> t;
+        q.res_mult = static_cast<float>(std::strtod(t.c_str(), nullptr));
+        if (!in) return fail("truncated pack line");
+        const bool w_ok = (j.w.kind == KXC_HIP_BUF_ARG && j.w.index_or_offset >= 0 && j.w.index_or_offset < num_args) ||
+                          (j.w.kind == KXC_HIP_BUF_ARG_OFFSET && j.w.index_or_offset >= 0 && (j.w.index_or_offset >> 48) < num_args &&
+                           (j.w.index_or_offset & 15) == 0);
+        if (!w_ok || j.wp.kind != KXC_HIP_BUF_WORKSPACE || j.wp.index_or_offset < 0 || j.wp.index_or_offset >= workspace ||
+            j.wp.index_or_offset % 256 != 0)
+            return fail("pack operand out of range");
+        size_t bytes = 0;
+        const QPackJob probe{j.kind, &j.desc, nullptr, nullptr};
+        if (QPackedBytes(probe, &bytes) != KXC_HIP_OK) return fail("bad pack descriptor");
+        plan->packs.push_back(j);
     }
     if (int32_t rc = kxc_hip_plan_finalize(plan, static_cast<size_t>(workspace))) {
         kxc_hip_plan_destroy(plan);

@@ -504,10 +504,7 @@ __global__ void __launch_bounds__(64 * WP) __attribute__((amdgpu_waves_per_eu(2)
 
 // Weights of the first-layer kernel: [o block][kh][lane][16]; lane (o, half), byte j = pixel j/4, channel j%4,
 // tap kw = 4*half + j/4 - 1.
-__global__ void __launch_bounds__(kBlock) pack_weights_k7_c4_kernel(const int8_t* __restrict__ w, int8_t* __restrict__ wp,
-                                                                    int32_t O, int32_t C, int64_t total_slots) {
-    const int64_t s = static_cast<int64_t>(blockIdx.x) * kBlock + threadIdx.x;
-    if (s >= total_slots) return;
+__device__ __forceinline__ void pack_k7_c4_slot(const int8_t* __restrict__ w, int8_t* __restrict__ wp, int32_t O, int32_t C, int64_t s) {
     const int lane = static_cast<int>(s & 63);
     const int64_t t = s >> 6;
     const int kh = static_cast<int>(t % 7);
@@ -520,6 +517,13 @@ __global__ void __launch_bounds__(kBlock) pack_weights_k7_c4_kernel(const int8_t
         out[j] = (kw >= 0 && kw < 7 && c < C && o < O) ? w[((static_cast<int64_t>(o) * C + c) * 7 + kh) * 7 + kw] : 0;
     }
     *reinterpret_cast<int4*>(wp + s * 16) = *reinterpret_cast<const int4*>(out);
+}
+
+__global__ void __launch_bounds__(kBlock) pack_weights_k7_c4_kernel(const int8_t* __restrict__ w, int8_t* __restrict__ wp,
+                                                                    int32_t O, int32_t C, int64_t total_slots) {
+    const int64_t s = static_cast<int64_t>(blockIdx.x) * kBlock + threadIdx.x;
+    if (s >= total_slots) return;
+    pack_k7_c4_slot(w, wp, O, C, s);
 }
 
 // fp32 NCHW -> int8 c4 ([N][H][W][4]); one thread per pixel.
@@ -578,9 +582,7 @@ struct PackArgs {
     int32_t O, C, KHW, CBC, NS, nchunks, oblocks;
 };
 
-__global__ void __launch_bounds__(kBlock) pack_weights_kernel(const PackArgs a, int64_t total_slots) {
-    const int64_t s = static_cast<int64_t>(blockIdx.x) * kBlock + threadIdx.x;
-    if (s >= total_slots) return;
+__device__ __forceinline__ void pack_slot(const PackArgs& a, int64_t s) {
     const int lane = static_cast<int>(s & 63);
     int64_t t = s >> 6;
     const int step = static_cast<int>(t % a.NS); t /= a.NS;
@@ -597,6 +599,32 @@ __global__ void __launch_bounds__(kBlock) pack_weights_kernel(const PackArgs a, 
         out[j] = (tap < a.KHW && c < a.C && o < a.O) ? a.w[(static_cast<int64_t>(o) * a.C + c) * a.KHW + tap] : 0;
     }
     *reinterpret_cast<int4*>(a.wp + s * 16) = *reinterpret_cast<const int4*>(out);
+}
+
+__global__ void __launch_bounds__(kBlock) pack_weights_kernel(const PackArgs a, int64_t total_slots) {
+    const int64_t s = static_cast<int64_t>(blockIdx.x) * kBlock + threadIdx.x;
+    if (s >= total_slots) return;
+    pack_slot(a, s);
+}
+
+// The weight tensors of several layers in one launch (a launch plan packs the constants of a whole network at the
+// start of a run).  Job j owns the blocks first_block[j] .. first_block[j + 1] - 1; NS == 0 marks the first-layer
+// (c4) order.
+constexpr int kMaxPackJobs = 24;
+struct PackBatch {
+    PackArgs job[kMaxPackJobs];
+    int64_t slots[kMaxPackJobs];
+    int32_t first_block[kMaxPackJobs + 1];
+    int32_t count;
+};
+__global__ void __launch_bounds__(kBlock) pack_weights_batch_kernel(const PackBatch b) {
+    int j = 0;
+    while (j + 1 < b.count && static_cast<int32_t>(blockIdx.x) >= b.first_block[j + 1]) ++j;
+    const int64_t s = static_cast<int64_t>(static_cast<int32_t>(blockIdx.x) - b.first_block[j]) * kBlock + threadIdx.x;
+    if (s >= b.slots[j]) return;
+    const PackArgs& a = b.job[j];
+    if (a.NS == 0) pack_k7_c4_slot(a.w, a.wp, a.O, a.C, s);
+    else pack_slot(a, s);
 }
 
 // ------------------------------------------------------------------ layout conversion and quantisation
@@ -1268,6 +1296,75 @@ int32_t kxc_hip_quantize_f32_nchw_to_c4_i8(const float* x, int8_t* y, int64_t n,
     quantize_to_c4_kernel<<<NoteGrid(static_cast<int>(CeilDiv(total, kBlock))), NoteBlock(kBlock), NoteLds(0),
                             ResolveStream(stream)>>>(x, y, static_cast<int32_t>(c), hw, total, scale);
     return CheckLaunch("quantize_f32_nchw_to_c4_i8");
+}
+
+}  // extern "C"
+
+// ---- the weight tensors of several layers packed by one launch
+namespace kxc_hip {
+
+int32_t QPackedBytes(const QPackJob& job, size_t* out_bytes) {
+    KXC_HIP_REQUIRE(job.desc != nullptr, "weight pack: desc is NULL");
+    switch (job.kind) {
+        case KXC_HIP_QPACK_C16: return kxc_hip_qconv2d_c16_packed_bytes(job.desc, out_bytes);
+        case KXC_HIP_QPACK_C4: return kxc_hip_qconv2d_c4_packed_bytes(job.desc, out_bytes);
+        case KXC_HIP_QPACK_C16_PAIR: return kxc_hip_qconv2d_c16_pair_packed_bytes(job.desc, out_bytes);
+        default: return Fail(KXC_HIP_ERR_INVALID, "weight pack: unknown kind %d", job.kind);
+    }
+}
+
+int32_t LaunchQWeightPacks(const QPackJob* jobs, int32_t count, hipStream_t stream) {
+    for (int32_t base = 0; base < count; base += kMaxPackJobs) {
+        PackBatch b;
+        std::memset(&b, 0, sizeof(b));
+        b.count = std::min<int32_t>(kMaxPackJobs, count - base);
+        int64_t blocks = 0;
+        for (int32_t j = 0; j < b.count; ++j) {
+            const QPackJob& job = jobs[base + j];
+            size_t bytes = 0;
+            if (int32_t rc = QPackedBytes(job, &bytes)) return rc;
+            KXC_HIP_REQUIRE(job.w && job.wp, "weight pack: NULL pointer in job %d", base + j);
+            const kxc_hip_qconv2d_desc* d = job.desc;
+            PackArgs& p = b.job[j];
+            p.w = job.w; p.wp = job.wp; p.O = d->o; p.C = d->c;
+            if (job.kind == KXC_HIP_QPACK_C4) {
+                p.NS = 0;                                   // first-layer order
+            } else {
+                const bool pair = job.kind == KXC_HIP_QPACK_C16_PAIR;
+                p.KHW = pair ? 1 : d->kh * d->kw;
+                p.CBC = CbcFor(d->c, d->kh, d->kw);
+                p.NS = pair ? (p.CBC + 1) / 2 : (p.KHW * p.CBC + 1) / 2;
+                p.nchunks = ((d->c + 15) / 16 + p.CBC - 1) / p.CBC;
+                p.oblocks = d->o / 32;
+            }
+            b.slots[j] = static_cast<int64_t>(bytes / 16);
+            b.first_block[j] = static_cast<int32_t>(blocks);
+            blocks += CeilDiv(b.slots[j], kBlock);
+            KXC_HIP_REQUIRE(blocks < kMaxGridX, "weight pack: too many blocks");
+        }
+        b.first_block[b.count] = static_cast<int32_t>(blocks);
+        if (blocks == 0) continue;
+        pack_weights_batch_kernel<<<NoteGrid(static_cast<int>(blocks)), NoteBlock(kBlock), NoteLds(0), stream>>>(b);
+        if (int32_t rc = CheckLaunch("pack_weights_batch_kernel")) return rc;
+    }
+    return KXC_HIP_OK;
+}
+
+}  // namespace kxc_hip
+
+extern "C" {
+
+int32_t kxc_hip_qconv2d_c4_supported(const kxc_hip_qconv2d_desc* d) {
+    QLaunch L;
+    const K7Variant* v = nullptr;
+    if (PrepareK7(d, &L, &v, "kxc_hip_qconv2d_c4_supported") != KXC_HIP_OK) { LastError().clear(); return 0; }
+    return 1;
+}
+
+int32_t kxc_hip_qconv2d_c16_supported(const kxc_hip_qconv2d_desc* d) {
+    QLaunch L;
+    if (Prepare(d, &L, "kxc_hip_qconv2d_c16_supported") != KXC_HIP_OK) { LastError().clear(); return 0; }
+    return 1;
 }
 
 }  // extern "C"

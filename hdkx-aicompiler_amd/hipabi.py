@@ -571,6 +571,9 @@ def global_avg_pool2d_c16_i8(x, c, mult):
     return y
 
 
+QPACK_C16, QPACK_C4, QPACK_C16_PAIR = 1, 2, 3
+
+
 class Plan:
     """kxc_hip_plan: a list of launches over packed arguments and one workspace."""
 
@@ -661,6 +664,17 @@ class Plan:
     def add_global_avg_pool2d_c16_i8(self, n, c, h, w, mult, x, y):
         _check(lib().kxc_hip_plan_add_global_avg_pool2d_c16_i8(self._h, C.c_int64(n), C.c_int64(c), C.c_int64(h),
                                                                C.c_int64(w), C.c_float(mult), x, y))
+
+    def add_i8_layout(self, to_c16, n, c, hw, x, y):
+        _check(lib().kxc_hip_plan_add_i8_layout(self._h, C.c_int32(1 if to_c16 else 0), C.c_int64(n), C.c_int64(c), C.c_int64(hw), x, y))
+
+    def add_qconv_weight_pack(self, kind, desc, w_oihw, w_packed, every_run=False):
+        """kind: QPACK_C16 / QPACK_C4 / QPACK_C16_PAIR.  w_oihw must be a packed argument, w_packed a workspace region."""
+        _check(lib().kxc_hip_plan_add_qconv_weight_pack(self._h, C.c_int32(kind), C.byref(desc), w_oihw, w_packed,
+                                                        C.c_int32(1 if every_run else 0)))
+
+    def num_weight_packs(self):
+        return int(lib().kxc_hip_plan_num_weight_packs(self._h))
 
     def add_qdense(self, m, n, k, a, b, bias, mult, y):
         _check(lib().kxc_hip_plan_add_qdense(self._h, C.c_int64(m), C.c_int64(n), C.c_int64(k), a, b, bias, mult, y))

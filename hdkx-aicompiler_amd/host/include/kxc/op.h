@@ -51,19 +51,45 @@ struct HIPBuffer {
     int kind = 2;            // KXC_HIP_BUF_ARG / _WORKSPACE / _NONE
     int64_t index_or_offset = 0;
 };
+// How a rank-4 int8 activation lies in memory between two launches.  kHIPLayoutPlain is the tensor type's own
+// row-major (NCHW) layout, the only one function parameters, constants and the result ever have; kHIPLayoutC16
+// stores [N][ceil(C/16)][H][W][16] (one pixel's 16 channels contiguous: the operand slice of the int8 matrix
+// instruction), kHIPLayoutC4 [N][H][W][4] (inputs of at most four channels).  An operator's "FHIPLayoutQuery" says
+// which layouts its hand-written kernel takes and writes for a call; the graph pass places a converter on every
+// edge whose two ends disagree.  kHIPLayoutAny (in `offered` only) marks an input whose producer writes whatever
+// its consumers ask for.
+enum HIPLayout : int { kHIPLayoutAny = -1, kHIPLayoutPlain = 0, kHIPLayoutC16 = 1, kHIPLayoutC4 = 2 };
+struct HIPLayoutChoice {
+    std::vector<int> inputs;             // one per input; empty = all plain
+    int output = kHIPLayoutPlain;
+};
+// offered[i]: the layout input i exists in (kHIPLayoutAny: the producer follows this call).  input_argument[i]: the
+// input is a packed argument (a parameter or a constant), i.e. readable before the first launch of a run.
+using FHIPLayoutQuery = std::function<HIPLayoutChoice(const Attrs& attrs, const Array<Type>& input_types, const Type& out_type,
+                                                      const std::vector<int>& offered, const std::vector<bool>& input_argument)>;
+// Bytes of a tensor of type `t` in layout `layout`.
+int64_t HIPLayoutBytes(const Type& t, int layout);
+
 struct HIPDispatchContext {
     Attrs attrs;
     Array<Type> input_types;
     Type out_type;
     Array<HIPBuffer> inputs;
     HIPBuffer output;
+    // the layouts the inputs arrive in and the output is expected in: what the operator's FHIPLayoutQuery chose
+    // (all plain for operators without one)
+    std::vector<int> input_layouts;
+    int output_layout = kHIPLayoutPlain;
+    int pair_output_layout = kHIPLayoutPlain;
+    // input_argument[i]: input i is a packed argument of the run; input_constant[i]: it is a module constant
+    std::vector<bool> input_argument;
+    bool winograd_allowed = false;
     // what the graph pass fused behind this call (only offered to operators that declare "THIPFusable")
     bool fused_relu = false;
     bool has_residual = false;
     HIPBuffer residual;
     // input_constant[i]: input i is a module constant (same tensor on every run).  alloc_persistent(bytes) hands
-    // out a workspace region that lives as long as the module, for a re-laid-out copy of such a constant; it is
-    // empty when the configuration rules that out.
+    // out a workspace region that lives as long as the module, for a re-laid-out copy of such a constant.
     std::vector<bool> input_constant;
     std::function<HIPBuffer(int64_t)> alloc_persistent;
     // A second call of the same operator on the same first input whose value this launch produces as well (offered
@@ -199,6 +225,12 @@ struct QnnQuantizeAttrsNode : AttrsNode { double scale = 1.0; };
 KXC_ATTRS_REF(QnnQuantizeAttrs)
     static QnnQuantizeAttrs Create(double scale);
 };
+//   qnn_global_avg_pool2d(x i8 [N,C,H,W]) -> int8 [N,C,1,1]  clamp(rint((float)(sum over H, W in int32) * mult), -128, 127)
+//        (mult = s_in / (H * W * s_out), computed by whoever quantised the model)
+struct QnnRequantAttrsNode : AttrsNode { double mult = 1.0; };
+KXC_ATTRS_REF(QnnRequantAttrs)
+    static QnnRequantAttrs Create(double mult);
+};
 
 struct CastAttrsNode : AttrsNode { int to = 0; };
 KXC_ATTRS_REF(CastAttrs)
@@ -222,6 +254,7 @@ Type DenseInferType(const Attrs& attrs, const Array<Type>& inputs);
 Type QnnConv2DInferType(const Attrs& attrs, const Array<Type>& inputs);
 Type QnnDenseInferType(const Attrs& attrs, const Array<Type>& inputs);
 Type QnnQuantizeInferType(const Attrs& attrs, const Array<Type>& inputs);
+Type QnnGlobalAvgPool2DInferType(const Attrs& attrs, const Array<Type>& inputs);
 Type GemmInferType(const Attrs& attrs, const Array<Type>& inputs);
 Type MatmulInferType(const Attrs& attrs, const Array<Type>& inputs);
 Type UnarySameInferType(const Attrs& attrs, const Array<Type>& inputs);

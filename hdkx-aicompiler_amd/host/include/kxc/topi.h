@@ -56,6 +56,7 @@ Tensor qnn_quantize(const Tensor& x, double scale, std::string name);
 Tensor qnn_conv2d_nchw(const Tensor& data, const Tensor& kernel, const Tensor& bias, const Tensor& mult, const Tensor& residual,
                        int stride_h, int stride_w, int pad_h, int pad_w, bool relu, double res_mult, std::string name);
 Tensor qnn_dense(const Tensor& A, const Tensor& B, const Tensor& bias, const Tensor& mult, std::string name);
+Tensor qnn_global_avg_pool2d(const Tensor& data, double mult, std::string name);
 
 }  // namespace topi
 }  // namespace te

@@ -2,6 +2,7 @@
 // a graph for a target and run it with device pointers.  Errors are returned as codes; the message is
 // kept per thread.
 #include <cstring>
+#include <memory>
 
 #include "kxc/compiler.h"
 #include "kxc/models.h"
@@ -12,6 +13,7 @@ struct ModuleHandle {
     kxc::api::CompiledModule module;
     std::string symbols;     // newline-separated kernel symbols
     std::string plan_json;
+    std::string constant_names;     // newline-separated, packed-argument order (graphs whose builder names its constants)
 };
 }  // namespace
 
@@ -33,6 +35,37 @@ int kxc_host_compile_resnet18(const char* target, long long batch, long long hw,
         for (const auto& e : h->module.GetKernelExecs()) h->symbols += e.op_name + " " + e.kernel_symbol + "\n";
         h->plan_json = h->module.ExecutionPlanJSON();
         *out_module = h;
+        return 0;
+    } catch (const std::exception& e) {
+        g_error = e.what();
+        return 1;
+    }
+}
+
+// The quantised ResNet-18 (kxc::models::BuildQResNet18): res_mult = 8 residual multipliers, one per block.
+// lanes: CompileConfigNode::hip_batch_lanes (0 = the back end decides).
+// result: "" for the logits, or the name of an int8 activation to return instead (see BuildQResNet18).
+int kxc_host_compile_qresnet18(const char* target, long long batch, long long hw, double input_scale, const double* res_mult,
+                               double gap_mult, int lanes, int sync_after_run, const char* result, void** out_module) {
+    try {
+        const bool gpu = std::strcmp(target, "cpu") != 0;
+        auto config = kxc::api::CompileConfig::AOT(kxc::BuildTarget(gpu ? kxc::kGPU : kxc::kCPU));
+        config->sync_after_run = sync_after_run != 0;
+        config->hip_batch_lanes = lanes;
+        kxc::models::QResNet18Scales scales;
+        scales.input_scale = input_scale;
+        for (int i = 0; i < 8; ++i) scales.res_mult[i] = res_mult[i];
+        scales.gap_mult = gap_mult;
+        std::unique_ptr<ModuleHandle> h(new ModuleHandle());
+        std::vector<kxc::runtime::NDArray> consts;
+        std::vector<std::string> names;
+        h->module = kxc::api::Compiler::Compile(kxc::models::BuildQResNet18(batch, hw, scales, &consts, &names, result ? result : ""), config);
+        for (const auto& c : h->module.GetConstants())
+            for (size_t i = 0; i < consts.size(); ++i)
+                if (consts[i].get() == c.get()) h->constant_names += names[i] + "\n";
+        for (const auto& e : h->module.GetKernelExecs()) h->symbols += e.op_name + " " + e.kernel_symbol + "\n";
+        h->plan_json = h->module.ExecutionPlanJSON();
+        *out_module = h.release();
         return 0;
     } catch (const std::exception& e) {
         g_error = e.what();
@@ -101,6 +134,7 @@ const char* kxc_host_module_status(void* module) {
     return g_error.c_str();
 }
 const char* kxc_host_module_symbols(void* module) { return static_cast<ModuleHandle*>(module)->symbols.c_str(); }
+const char* kxc_host_module_constant_names(void* module) { return static_cast<ModuleHandle*>(module)->constant_names.c_str(); }
 const char* kxc_host_module_plan_json(void* module) { return static_cast<ModuleHandle*>(module)->plan_json.c_str(); }
 long long kxc_host_module_workspace_bytes(void* module) {
     return static_cast<long long>(static_cast<ModuleHandle*>(module)->module.workspace_bytes());

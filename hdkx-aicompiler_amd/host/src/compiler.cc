@@ -211,6 +211,7 @@ public:
     void Build() {
         Number();
         FormGroups();
+        AssignLayouts();
         if (kxc_hip_plan_create(cfg_->target->device.device_id(), static_cast<int32_t>(num_args_), &m_->plan))
             throw std::runtime_error(std::string("plan creation failed: ") + kxc_hip_last_error());
         // variants are chosen for `lanes` equal launches side by side: by the queries made while the plan is built
@@ -344,6 +345,88 @@ private:
         }
     }
 
+    // ---- layouts of int8 activations between launches (relay::HIPLayout).  Every call whose operator has an
+    // "FHIPLayoutQuery" says, in topological order, which layouts its kernel takes and writes given the layouts its
+    // inputs exist in; a value whose producer writes any layout ("THIPLayoutFollowsConsumers": qnn_quantize) takes
+    // the layout its consumers agree on (a first pass collects their wishes, a second one runs with the decision).
+    // Edges whose ends disagree get a converter when the call is emitted.
+    void AssignLayouts() {
+        if (!cfg_->hip_use_handwritten) return;
+        std::unordered_map<const RelayExprNode*, int> decided;       // follows-consumers values, after pass 0
+        for (int pass = 0; pass < 2; ++pass) {
+            layout_.clear();
+            choice_.clear();
+            std::unordered_map<const RelayExprNode*, std::vector<int>> wishes;
+            for (const CallNode* c : topo_) {
+                const auto* op = c->op.As<OpNode>();
+                const auto* query = OpAttr<relay::FHIPDispatch>(op, "FHIPDispatch") ? OpAttr<relay::FHIPLayoutQuery>(op, "FHIPLayoutQuery") : nullptr;
+                relay::HIPLayoutChoice choice;
+                choice.inputs.assign(c->args.size(), relay::kHIPLayoutPlain);
+                if (query) {
+                    Array<Type> types;
+                    std::vector<int> offered;
+                    std::vector<bool> is_arg;
+                    for (const auto& a : c->args) {
+                        types.push_back(a.checked_type());
+                        auto it = layout_.find(a.get());
+                        offered.push_back(it == layout_.end() ? relay::kHIPLayoutPlain : it->second);
+                        is_arg.push_back(arg_index_.count(a.get()) > 0);
+                    }
+                    choice = (*query)(c->attrs, types, c->checked_type_, offered, is_arg);
+                    if (choice.inputs.size() != c->args.size()) choice.inputs.assign(c->args.size(), relay::kHIPLayoutPlain);
+                }
+                for (size_t i = 0; i < c->args.size(); ++i) {
+                    auto it = layout_.find(c->args[i].get());
+                    if (it != layout_.end() && it->second == relay::kHIPLayoutAny) wishes[c->args[i].get()].push_back(choice.inputs[i]);
+                }
+                choice_[c] = choice;
+                if (OpFlag(op, "THIPLayoutFollowsConsumers") && OpAttr<relay::FHIPDispatch>(op, "FHIPDispatch")) {
+                    auto d = decided.find(c);
+                    layout_[c] = pass == 0 || d == decided.end() ? static_cast<int>(relay::kHIPLayoutAny) : d->second;
+                } else {
+                    layout_[c] = choice.output;
+                }
+            }
+            if (pass == 0) {
+                bool any = false;
+                for (const auto& kv : layout_) {
+                    if (kv.second != relay::kHIPLayoutAny) continue;
+                    any = true;
+                    int agreed = relay::kHIPLayoutPlain;
+                    const auto w = wishes.find(kv.first);
+                    if (w != wishes.end() && !w->second.empty() && kv.first != f_->body.get()) {
+                        agreed = w->second[0];
+                        for (int l : w->second) if (l != agreed) agreed = relay::kHIPLayoutPlain;
+                    }
+                    decided[kv.first] = agreed;
+                }
+                if (!any) break;       // no value's layout was left open: the first pass is final
+            }
+        }
+        for (auto& kv : layout_) if (kv.second == relay::kHIPLayoutAny) kv.second = relay::kHIPLayoutPlain;
+    }
+    int LayoutOf(const RelayExprNode* e) const {
+        auto it = layout_.find(Resolve(e));
+        return it == layout_.end() ? static_cast<int>(relay::kHIPLayoutPlain) : it->second;
+    }
+    int64_t ValueBytes(const RelayExprNode* e) const { return relay::HIPLayoutBytes(e->checked_type_, LayoutOf(e)); }
+    // One converter launch between the plain and the channel-blocked layout of an int8 value.
+    void EmitLayoutConvert(const RelayExprNode* value, int from, int to, relay::HIPBuffer src, relay::HIPBuffer dst) {
+        const auto* t = TT(value->checked_type_);
+        const bool ok = t && t->dtype == "int8" && t->shape.size() == 4 &&
+                        ((from == relay::kHIPLayoutPlain && to == relay::kHIPLayoutC16) || (from == relay::kHIPLayoutC16 && to == relay::kHIPLayoutPlain));
+        if (!ok) throw std::runtime_error("hip back end: no converter between activation layouts " + std::to_string(from) + " and " + std::to_string(to));
+        if (kxc_hip_plan_add_i8_layout(m_->plan, to == relay::kHIPLayoutC16 ? 1 : 0, t->shape[0], t->shape[1], t->shape[2] * t->shape[3],
+                                       {src.kind, src.index_or_offset}, {dst.kind, dst.index_or_offset}))
+            throw std::runtime_error(std::string("plan layout converter failed: ") + kxc_hip_last_error());
+        KernelExecInfo info;
+        info.op_name = "layout_convert";
+        info.kernel_symbol = to == relay::kHIPLayoutC16 ? "kxc_i8_nchw_to_c16" : "kxc_i8_c16_to_nchw";
+        info.input_values.push_back(value_id_.at(value));
+        info.output_values.push_back(value_id_.at(value));
+        m_->execs.push_back(info);
+    }
+
     // ---- buffers
     relay::HIPBuffer BufferOf(const RelayExprNode* e) {
         e = Resolve(e);
@@ -387,7 +470,7 @@ private:
                 const Group& gb = groups_[order[sb]];
                 const auto* opb = gb.head->op.As<OpNode>();
                 const auto* query = OpAttr<relay::FHIPPairQuery>(opb, "FHIPPairQuery");
-                if (!query || gb.head != gb.tail || gb.residual || gb.fused_relu || !IsF32(gb.head->checked_type_)) continue;
+                if (!query || gb.head != gb.tail || gb.residual || gb.fused_relu) continue;
                 if (gb.tail == f_->body.get() || !OpAttr<relay::FHIPDispatch>(opb, "FHIPDispatch")) continue;
                 bool inputs_ready = true;
                 for (size_t i = 1; i < gb.head->args.size(); ++i)
@@ -399,8 +482,10 @@ private:
                     const size_t ia = order[sa];
                     const Group& ga = groups_[ia];
                     if (merged[ia] || carries[ia] >= 0 || ga.head->op.get() != gb.head->op.get()) continue;
-                    if (ga.tail == f_->body.get() || !IsF32(ga.head->checked_type_)) continue;
+                    if (ga.tail == f_->body.get() || TT(ga.head->checked_type_)->dtype != TT(gb.head->checked_type_)->dtype) continue;
                     if (Resolve(ga.head->args[0].get()) != Resolve(gb.head->args[0].get())) continue;
+                    // both launches must read the shared input and write their results in the same layouts
+                    if (LayoutOf(ga.tail) != LayoutOf(gb.tail) || choice_.at(ga.head).inputs[0] != choice_.at(gb.head).inputs[0]) continue;
                     if (TT(ga.tail->checked_type_)->shape != TT(gb.tail->checked_type_)->shape) continue;
                     Array<Type> a_types;
                     std::vector<bool> a_const;
@@ -463,7 +548,8 @@ private:
         for (size_t step = 0; step < order.size(); ++step) {
             const Group& g = groups_[order[step]];
             const auto* op = g.head->op.As<OpNode>();
-            if (OpFlag(op, "THIPAlias") && g.tail != f_->body.get() && g.head == g.tail) {
+            if (OpFlag(op, "THIPAlias") && g.tail != f_->body.get() && g.head == g.tail &&
+                LayoutOf(g.head->args[0].get()) == relay::kHIPLayoutPlain) {
                 is_alias[order[step]] = true;
                 alias_[g.head] = g.head->args[0].get();
             }
@@ -493,45 +579,75 @@ private:
             const Group& g = groups_[order[step]];
             if (is_alias[order[step]]) continue;
             const auto* op = g.head->op.As<OpNode>();
-            // output buffer
-            relay::HIPBuffer out;
+            // output buffer (a result that is not produced in the function's own layout goes through a slot and a converter)
+            relay::HIPBuffer out, final_out;
+            std::vector<std::pair<int64_t, int64_t>> temps;        // slots that live for this step only
+            const int out_layout = LayoutOf(g.tail);
+            const bool convert_result = g.tail == f_->body.get() && out_layout != relay::kHIPLayoutPlain;
             if (g.tail == f_->body.get()) {
                 out = {KXC_HIP_BUF_ARG, num_args_ - 1};
                 if (lanes_ > 1) out = {KXC_HIP_BUF_ARG_OFFSET, KXC_HIP_ARG_OFFSET(num_args_ - 1, lane_ * out_share_bytes_)};
+                if (convert_result) {
+                    final_out = out;
+                    temps.push_back(arena_.Alloc(ValueBytes(g.tail)));
+                    out = {KXC_HIP_BUF_WORKSPACE, temps.back().first};
+                }
             } else {
-                slot_[g.tail] = arena_.Alloc(TypeBytes(g.tail->checked_type_));
+                slot_[g.tail] = arena_.Alloc(ValueBytes(g.tail));
                 out = {KXC_HIP_BUF_WORKSPACE, slot_[g.tail].first};
             }
             relay::HIPDispatchContext ctx;
             ctx.attrs = g.head->attrs;
-            for (const auto& a : g.head->args) {
-                ctx.input_types.push_back(a.checked_type());
-                ctx.inputs.push_back(BufferOf(a.get()));
+            const relay::HIPLayoutChoice* choice = nullptr;
+            {
+                auto ch = choice_.find(g.head);
+                if (ch != choice_.end()) choice = &ch->second;
             }
-            for (const auto& a : g.head->args) ctx.input_constant.push_back(dynamic_cast<const ConstantNode*>(Resolve(a.get())) != nullptr);
+            for (size_t i = 0; i < g.head->args.size(); ++i) {
+                const auto& a = g.head->args[i];
+                ctx.input_types.push_back(a.checked_type());
+                const int have = LayoutOf(a.get()), want = choice ? choice->inputs[i] : static_cast<int>(relay::kHIPLayoutPlain);
+                ctx.input_layouts.push_back(want);
+                if (have == want) {
+                    ctx.inputs.push_back(BufferOf(a.get()));
+                } else {
+                    temps.push_back(arena_.Alloc(relay::HIPLayoutBytes(a.checked_type(), want)));
+                    const relay::HIPBuffer converted{KXC_HIP_BUF_WORKSPACE, temps.back().first};
+                    EmitLayoutConvert(a.get(), have, want, BufferOf(a.get()), converted);
+                    ctx.inputs.push_back(converted);
+                }
+            }
+            ctx.output_layout = out_layout;
+            for (const auto& a : g.head->args) {
+                ctx.input_constant.push_back(dynamic_cast<const ConstantNode*>(Resolve(a.get())) != nullptr);
+                ctx.input_argument.push_back(arg_index_.count(Resolve(a.get())) > 0);
+            }
             const char* wino_env = std::getenv("KXC_HIP_WINOGRAD");                 // "0" switches Winograd off
-            if (cfg_->hip_winograd && !(wino_env && wino_env[0] == '0'))
-                ctx.alloc_persistent = [this](int64_t bytes) {
-                    // (the shares of a batch ask in the same order and share what the first one got: transformed
-                    // weights do not depend on the batch)
-                    if (lane_ > 0 && persistent_cursor_ < persistent_.size()) return persistent_[persistent_cursor_++];
-                    // above everything handed out so far and never released: no activation of an earlier or later
-                    // step ever shares the region, so what the first run wrote there is still valid in the next
-                    const int64_t off = arena_.top;
-                    arena_.top += (std::max<int64_t>(bytes, 1) + 255) / 256 * 256;
-                    persistent_.push_back(relay::HIPBuffer{KXC_HIP_BUF_WORKSPACE, off});
-                    return persistent_.back();
-                };
+            ctx.winograd_allowed = cfg_->hip_winograd && !(wino_env && wino_env[0] == '0');
+            ctx.alloc_persistent = [this](int64_t bytes) {
+                // (the shares of a batch ask in the same order and share what the first one got: transformed or
+                // packed weights do not depend on the batch)
+                if (lane_ > 0 && persistent_cursor_ < persistent_.size()) return persistent_[persistent_cursor_++];
+                // above everything handed out so far and never released: no activation of an earlier or later
+                // step ever shares the region, so what the first run wrote there is still valid in the next
+                const int64_t off = arena_.top;
+                arena_.top += (std::max<int64_t>(bytes, 1) + 255) / 256 * 256;
+                persistent_.push_back(relay::HIPBuffer{KXC_HIP_BUF_WORKSPACE, off});
+                return persistent_.back();
+            };
             const Group* carried = carries[order[step]] >= 0 ? &groups_[carries[order[step]]] : nullptr;
             if (carried) {
-                slot_[carried->tail] = arena_.Alloc(TypeBytes(carried->tail->checked_type_));
+                slot_[carried->tail] = arena_.Alloc(ValueBytes(carried->tail));
                 ctx.has_pair = true;
                 ctx.pair_attrs = carried->head->attrs;
-                for (const auto& a : carried->head->args) {
+                for (size_t i = 0; i < carried->head->args.size(); ++i) {
+                    const auto& a = carried->head->args[i];
                     ctx.pair_input_types.push_back(a.checked_type());
-                    ctx.pair_inputs.push_back(BufferOf(a.get()));
+                    // (input 0 is the first call's; the others are packed arguments, which are always plain)
+                    ctx.pair_inputs.push_back(i == 0 ? ctx.inputs[0] : BufferOf(a.get()));
                 }
                 ctx.pair_output = {KXC_HIP_BUF_WORKSPACE, slot_[carried->tail].first};
+                ctx.pair_output_layout = LayoutOf(carried->tail);
             }
             ctx.out_type = g.tail->checked_type_;
             ctx.output = out;
@@ -571,8 +687,13 @@ private:
                     throw std::runtime_error(std::string("plan_set_concurrency failed: ") + kxc_hip_last_error());
             } else {
                 if (g.fused_relu || g.residual || carried) throw std::runtime_error("hip back end: operator declined a fused launch: " + op->name);
+                for (int l : ctx.input_layouts)
+                    if (l != relay::kHIPLayoutPlain) throw std::runtime_error("hip back end: operator declined the layout it asked for: " + op->name);
+                if (out_layout != relay::kHIPLayoutPlain) throw std::runtime_error("hip back end: operator declined the layout it asked for: " + op->name);
                 EmitGenerated(g, ctx, info, static_cast<int>(step));
             }
+            if (convert_result) EmitLayoutConvert(g.tail, out_layout, relay::kHIPLayoutPlain, out, final_out);
+            for (auto& t : temps) arena_.Release(t);
             // release everything whose last reader has now been enqueued
             for (auto it = slot_.begin(); it != slot_.end();) {
                 auto lu = last_use.find(it->first);
@@ -669,6 +790,8 @@ private:
     std::vector<Group> groups_;
     std::unordered_map<const CallNode*, size_t> group_of_tail_;
     std::unordered_map<const RelayExprNode*, const RelayExprNode*> alias_;
+    std::unordered_map<const RelayExprNode*, int> layout_;                       // how each value lies in memory (HIPLayout)
+    std::unordered_map<const CallNode*, relay::HIPLayoutChoice> choice_;         // what each call's kernel takes and writes
     std::unordered_map<const RelayExprNode*, std::pair<int64_t, int64_t>> slot_;
     Arena arena_;
 };
@@ -676,6 +799,22 @@ private:
 }  // namespace
 
 namespace {
+bool HasQuantisedCalls(const Expr& body) {
+    std::unordered_set<const RelayExprNode*> seen;
+    std::vector<const RelayExprNode*> stack{body.get()};
+    while (!stack.empty()) {
+        const RelayExprNode* e = stack.back();
+        stack.pop_back();
+        if (!e || !seen.insert(e).second) continue;
+        const auto* call = dynamic_cast<const CallNode*>(e);
+        if (!call) continue;
+        const auto* op = call->op.As<OpNode>();
+        if (op && op->name.compare(0, 4, "qnn_") == 0) return true;
+        for (const auto& a : call->args) stack.push_back(a.get());
+    }
+    return false;
+}
+
 // The caller's active context, else one made from the configuration's profile_options when those are enabled
 // (src/api/compiler.cc:32-40).
 std::shared_ptr<profiling::ProfileContext> MaybeCreateProfileContext(const CompileConfig& config) {
@@ -745,7 +884,9 @@ CompiledModule Compiler::Compile(Function func, CompileConfig config) {
             if (want != 1 && config->hip_use_handwritten && !typed->params.empty()) {
                 const auto* t0 = typed->params[0].checked_type().As<TensorTypeNode>();
                 const int64_t batch = t0 && !t0->shape.empty() ? t0->shape[0] : 0;
-                const int ask = want == 0 ? (batch >= 64 ? 2 : 1) : want;
+                // (measured on ResNet-18: the fp32 network gains from two shares from batch 64 on, the quantised one,
+                // whose launches are 7-15 us each, from batch 128 on)
+                const int ask = want == 0 ? (batch >= (HasQuantisedCalls(typed->body) ? 128 : 64) ? 2 : 1) : want;
                 if (ask > 1) {
                     share = relay::SplitBatch(typed, ask);
                     if (share.defined() && (TypeBytes(share->params[0].checked_type()) % 16 != 0 || TypeBytes(share->body.checked_type()) % 16 != 0))

@@ -40,6 +40,10 @@ PrimExpr ReduceIdentity(int rtype, DataType t) {
         const double inf = std::numeric_limits<double>::infinity();
         return tir::FloatImm(is_max ? -inf : inf, t);
     }
+    // (the reference hands every integer type the 64-bit extremes, src/relay/backend/lower.cc:80-95; a narrower type
+    // takes its own, since the 64-bit ones truncate to 0 and -1 there)
+    if (t.is_uint()) return tir::IntImm(is_max ? 0 : (t.bits >= 63 ? std::numeric_limits<int64_t>::max() : (int64_t{1} << t.bits) - 1), t);
+    if (t.bits < 64) return tir::IntImm(is_max ? -(int64_t{1} << (t.bits - 1)) : (int64_t{1} << (t.bits - 1)) - 1, t);
     return tir::IntImm(is_max ? std::numeric_limits<int64_t>::min() : std::numeric_limits<int64_t>::max(), t);
 }
 

@@ -2,6 +2,7 @@
 // definition, src/relay/op/nn/*.cc and src/relay/op/tensor/*.cc of the reference) and, where a
 // hand-written gfx950 kernel exists, the FHIPDispatch hook that adds its launch to a plan.
 #include <algorithm>
+#include <cstdlib>
 
 #include "kxc/op.h"
 #include "kxc/topi.h"
@@ -97,7 +98,8 @@ std::string Conv2DDispatch(const HIPDispatchContext& c, kxc_hip_plan* plan) {
     }
     // 3x3 stride-1 convolutions with constant weights run as Winograd F(2x2,3x3) when the library expects that to
     // be faster for the shape; the transformed weights get a workspace region of their own.
-    if (c.alloc_persistent && c.input_constant.size() > 1 && c.input_constant[1] && kxc_hip_conv2d_winograd_preferred(&d)) {
+    if (c.winograd_allowed && c.alloc_persistent && c.input_constant.size() > 1 && c.input_constant[1] &&
+        kxc_hip_conv2d_winograd_preferred(&d)) {
         size_t u_bytes = 0;
         Check(kxc_hip_conv2d_winograd_weight_bytes(&d, &u_bytes), "nn_conv2d dispatch");
         const HIPBuffer u = c.alloc_persistent(static_cast<int64_t>(u_bytes));
@@ -127,7 +129,8 @@ te::Tensor PoolCompute(const char* op, const char* type, const char* tname, cons
 
 std::string PoolDispatch(bool is_avg, const HIPDispatchContext& c, kxc_hip_plan* plan) {
     const auto* p = c.attrs.As<MaxPool2DAttrsNode>();
-    if (!p || !IsF32(c.input_types[0])) return "";
+    const bool i8 = !is_avg && TT(c.input_types[0]) && TT(c.input_types[0])->dtype == "int8";
+    if (!p || !(IsF32(c.input_types[0]) || i8)) return "";
     const auto* x = TT(c.input_types[0]);
     const auto ks = ReadPair(p->pool_size, 1), st = ReadPair(p->strides, 1), pd = ReadPad4(p->padding);
     kxc_hip_pool2d_desc d{};
@@ -137,6 +140,15 @@ std::string PoolDispatch(bool is_avg, const HIPDispatchContext& c, kxc_hip_plan*
     d.pad_top = pd[0]; d.pad_left = pd[1]; d.pad_bottom = pd[2]; d.pad_right = pd[3];
     d.ceil_mode = p->ceil_mode ? 1 : 0;
     d.is_avg = is_avg ? 1 : 0;
+    if (i8) {
+        // int8 max pool (the padding candidate is -128, the dtype's lowest value): channel-blocked or NCHW
+        const bool blocked = !c.input_layouts.empty() && c.input_layouts[0] == kHIPLayoutC16;
+        if (blocked != (c.output_layout == kHIPLayoutC16)) return "";
+        Check(blocked ? kxc_hip_plan_add_maxpool2d_c16_i8(plan, &d, B(c.inputs[0]), B(c.output))
+                      : kxc_hip_plan_add_maxpool2d_i8(plan, &d, B(c.inputs[0]), B(c.output)),
+              "int8 max pool dispatch");
+        return blocked ? "kxc_max_pool2d_c16_i8" : "kxc_max_pool2d_i8";
+    }
     Check(kxc_hip_plan_add_pool2d(plan, &d, B(c.inputs[0]), B(c.output)), "pool2d dispatch");
     return is_avg ? "kxc_avg_pool2d_f32" : "kxc_max_pool2d_f32";
 }
@@ -206,11 +218,12 @@ te::Tensor QnnConv2DCompute(const Attrs& attrs, const Array<te::Tensor>& in, con
                                      "T_qnn_conv2d");
 }
 
-std::string QnnConv2DDispatch(const HIPDispatchContext& c, kxc_hip_plan* plan) {
-    const auto* p = c.attrs.As<QnnConv2DAttrsNode>();
-    if (!p || c.inputs.size() < 4 || !IsDType(c.input_types[0], "int8") || !IsDType(c.out_type, "int8")) return "";
-    const auto* x = TT(c.input_types[0]);
-    const auto* w = TT(c.input_types[1]);
+bool QnnConvDesc(const Attrs& attrs, const Array<Type>& input_types, kxc_hip_qconv2d_desc* out) {
+    const auto* p = attrs.As<QnnConv2DAttrsNode>();
+    if (!p || input_types.size() < 4 || !IsDType(input_types[0], "int8") || !IsDType(input_types[1], "int8")) return false;
+    const auto* x = TT(input_types[0]);
+    const auto* w = TT(input_types[1]);
+    if (x->shape.size() != 4 || w->shape.size() != 4) return false;
     const auto st = ReadPair(p->strides, 1), pd = ReadPair(p->padding, 0);
     kxc_hip_qconv2d_desc d{};
     d.n = static_cast<int32_t>(x->shape[0]); d.c = static_cast<int32_t>(x->shape[1]);
@@ -218,14 +231,100 @@ std::string QnnConv2DDispatch(const HIPDispatchContext& c, kxc_hip_plan* plan) {
     d.o = static_cast<int32_t>(w->shape[0]); d.kh = static_cast<int32_t>(w->shape[2]); d.kw = static_cast<int32_t>(w->shape[3]);
     d.stride_h = static_cast<int32_t>(st[0]); d.stride_w = static_cast<int32_t>(st[1]);
     d.pad_h = static_cast<int32_t>(pd[0]); d.pad_w = static_cast<int32_t>(pd[1]);
-    const bool has_res = c.inputs.size() == 5;
+    const bool has_res = input_types.size() == 5;
     d.flags = KXC_HIP_CONV_BIAS | (has_res ? KXC_HIP_CONV_RESIDUAL : 0u) | (p->relu ? KXC_HIP_CONV_RELU : 0u);
     d.res_mult = has_res ? static_cast<float>(p->res_mult) : 0.0f;
+    *out = d;
+    return true;
+}
+
+bool MatrixCoresDisabled() {
+    const char* e = std::getenv("KXC_HIP_QNN_MFMA");       // "0": every quantised operator keeps NCHW and its scalar kernel
+    return e && e[0] == '0';
+}
+
+// The matrix-core kernels read channel-blocked activations and weights packed for them.  The weights must be
+// readable before the first launch of a run (a parameter or a constant) because they are packed at its start.
+HIPLayoutChoice QnnConv2DLayout(const Attrs& attrs, const Array<Type>& in, const Type&, const std::vector<int>& offered,
+                                const std::vector<bool>& input_argument) {
+    HIPLayoutChoice plain;
+    plain.inputs.assign(in.size(), kHIPLayoutPlain);
+    kxc_hip_qconv2d_desc d{};
+    if (MatrixCoresDisabled() || !QnnConvDesc(attrs, in, &d) || input_argument.size() < 2 || !input_argument[1]) return plain;
+    HIPLayoutChoice blocked = plain;
+    blocked.output = kHIPLayoutC16;
+    if (in.size() == 5) blocked.inputs[4] = kHIPLayoutC16;
+    // the 4-channel input layout only ever comes from a producer that follows this call (qnn_quantize)
+    if ((offered[0] == kHIPLayoutAny || offered[0] == kHIPLayoutC4) && in.size() == 4 && kxc_hip_qconv2d_c4_supported(&d)) {
+        blocked.inputs[0] = kHIPLayoutC4;
+        return blocked;
+    }
+    if (!kxc_hip_qconv2d_c16_supported(&d)) return plain;
+    blocked.inputs[0] = kHIPLayoutC16;
+    return blocked;
+}
+
+// A residual block's first convolution (A: ReLU, no residual) and its 1x1 downsample (B: same input and strides, no
+// padding, no ReLU, no residual, same number of output channels) as one launch on the matrix cores.
+bool QnnConv2DPairQuery(const Attrs& a_attrs, const Array<Type>& a_inputs, const std::vector<bool>&, const Attrs& b_attrs,
+                        const Array<Type>& b_inputs) {
+    kxc_hip_qconv2d_desc a{}, b{};
+    if (MatrixCoresDisabled() || !QnnConvDesc(a_attrs, a_inputs, &a) || !QnnConvDesc(b_attrs, b_inputs, &b)) return false;
+    if (a_inputs.size() != 4 || b_inputs.size() != 4) return false;
+    if (b.kh != 1 || b.kw != 1 || b.pad_h != 0 || b.pad_w != 0 || b.o != a.o || b.c != a.c) return false;
+    if (b.stride_h != a.stride_h || b.stride_w != a.stride_w || (b.flags & KXC_HIP_CONV_RELU)) return false;
+    const char* e = std::getenv("KXC_HIP_QPAIR");
+    if (e && e[0] == '0') return false;
+    return kxc_hip_qconv2d_c16_pair_supported(&a) != 0;
+}
+
+std::string QnnConv2DDispatch(const HIPDispatchContext& c, kxc_hip_plan* plan) {
+    kxc_hip_qconv2d_desc d{};
+    if (!QnnConvDesc(c.attrs, c.input_types, &d) || !IsDType(c.out_type, "int8")) return "";
+    const bool has_res = c.inputs.size() == 5;
     const kxc_hip_buf none{KXC_HIP_BUF_NONE, 0};
-    Check(kxc_hip_plan_add_qconv2d(plan, &d, B(c.inputs[0]), B(c.inputs[1]), B(c.inputs[2]), B(c.inputs[3]),
-                                   has_res ? B(c.inputs[4]) : none, B(c.output)),
+    const int in_layout = c.input_layouts.empty() ? kHIPLayoutPlain : c.input_layouts[0];
+    if (in_layout == kHIPLayoutPlain) {
+        if (c.output_layout != kHIPLayoutPlain || c.has_pair) return "";
+        Check(kxc_hip_plan_add_qconv2d(plan, &d, B(c.inputs[0]), B(c.inputs[1]), B(c.inputs[2]), B(c.inputs[3]),
+                                       has_res ? B(c.inputs[4]) : none, B(c.output)),
+              "qnn_conv2d dispatch");
+        return "kxc_qconv2d_nchw_i8";
+    }
+    // matrix cores: the weights are packed into a region of the module's own at the start of a run (every run when
+    // they are a parameter rather than a constant)
+    if (c.output_layout != kHIPLayoutC16 || !c.alloc_persistent || (has_res && c.input_layouts[4] != kHIPLayoutC16)) return "";
+    if (c.has_pair && (in_layout != kHIPLayoutC16 || c.pair_inputs.size() != 4 || c.pair_output_layout != kHIPLayoutC16)) return "";
+    const int every_run = c.input_constant.size() > 1 && c.input_constant[1] ? 0 : 1;
+    size_t bytes = 0;
+    if (in_layout == kHIPLayoutC4) {
+        Check(kxc_hip_qconv2d_c4_packed_bytes(&d, &bytes), "qnn_conv2d dispatch");
+        const HIPBuffer wp = c.alloc_persistent(static_cast<int64_t>(bytes));
+        Check(kxc_hip_plan_add_qconv_weight_pack(plan, KXC_HIP_QPACK_C4, &d, B(c.inputs[1]), B(wp), every_run), "qnn_conv2d weight pack");
+        Check(kxc_hip_plan_add_qconv2d_c4(plan, &d, B(c.inputs[0]), B(wp), B(c.inputs[2]), B(c.inputs[3]), B(c.output)),
+              "qnn_conv2d dispatch");
+        return std::string("kxc_qconv2d_c4_i8:qmfma_k7x7s2_c4") + ((d.flags & KXC_HIP_CONV_RELU) ? "+relu" : "");
+    }
+    Check(kxc_hip_qconv2d_c16_packed_bytes(&d, &bytes), "qnn_conv2d dispatch");
+    const HIPBuffer wp = c.alloc_persistent(static_cast<int64_t>(bytes));
+    Check(kxc_hip_plan_add_qconv_weight_pack(plan, KXC_HIP_QPACK_C16, &d, B(c.inputs[1]), B(wp), every_run), "qnn_conv2d weight pack");
+    const std::string tail = std::string(has_res ? "+add" : "") + ((d.flags & KXC_HIP_CONV_RELU) ? "+relu" : "");
+    if (c.has_pair) {
+        size_t bytes2 = 0;
+        Check(kxc_hip_qconv2d_c16_pair_packed_bytes(&d, &bytes2), "qnn_conv2d pair dispatch");
+        const HIPBuffer wp2 = c.alloc_persistent(static_cast<int64_t>(bytes2));
+        Check(kxc_hip_plan_add_qconv_weight_pack(plan, KXC_HIP_QPACK_C16_PAIR, &d, B(c.pair_inputs[1]), B(wp2), every_run),
+              "qnn_conv2d pair weight pack");
+        Check(kxc_hip_plan_add_qconv2d_c16_pair(plan, &d, B(c.inputs[0]), B(wp), B(c.inputs[2]), B(c.inputs[3]),
+                                                has_res ? B(c.inputs[4]) : none, B(c.output), B(wp2), B(c.pair_inputs[2]),
+                                                B(c.pair_inputs[3]), B(c.pair_output)),
+              "qnn_conv2d pair dispatch");
+        return std::string("kxc_qconv2d_c16_i8:") + kxc_hip_qconv2d_c16_variant(&d) + tail + "|qconv1x1+bias";
+    }
+    Check(kxc_hip_plan_add_qconv2d_c16(plan, &d, B(c.inputs[0]), B(wp), B(c.inputs[2]), B(c.inputs[3]),
+                                       has_res ? B(c.inputs[4]) : none, B(c.output)),
           "qnn_conv2d dispatch");
-    return "kxc_qconv2d_nchw_i8";
+    return std::string("kxc_qconv2d_c16_i8:") + kxc_hip_qconv2d_c16_variant(&d) + tail;
 }
 
 std::string QnnDenseDispatch(const HIPDispatchContext& c, kxc_hip_plan* plan) {
@@ -241,9 +340,55 @@ std::string QnnDenseDispatch(const HIPDispatchContext& c, kxc_hip_plan* plan) {
 std::string QnnQuantizeDispatch(const HIPDispatchContext& c, kxc_hip_plan* plan) {
     const auto* p = c.attrs.As<QnnQuantizeAttrsNode>();
     if (!p || !IsF32(c.input_types[0])) return "";
-    Check(kxc_hip_plan_add_quantize(plan, Product(TT(c.input_types[0])->shape), static_cast<float>(p->scale), B(c.inputs[0]), B(c.output)),
+    const auto* x = TT(c.input_types[0]);
+    if (c.output_layout == kHIPLayoutPlain) {
+        Check(kxc_hip_plan_add_quantize(plan, Product(x->shape), static_cast<float>(p->scale), B(c.inputs[0]), B(c.output)),
+              "qnn_quantize dispatch");
+        return "kxc_quantize_f32_i8";
+    }
+    if (x->shape.size() != 4) return "";
+    const int64_t hw = x->shape[2] * x->shape[3];
+    if (c.output_layout == kHIPLayoutC4) {
+        Check(kxc_hip_plan_add_quantize_c4(plan, x->shape[0], x->shape[1], hw, static_cast<float>(p->scale), B(c.inputs[0]), B(c.output)),
+              "qnn_quantize dispatch");
+        return "kxc_quantize_f32_nchw_to_c4_i8";
+    }
+    Check(kxc_hip_plan_add_quantize_c16(plan, x->shape[0], x->shape[1], hw, static_cast<float>(p->scale), B(c.inputs[0]), B(c.output)),
           "qnn_quantize dispatch");
-    return "kxc_quantize_f32_i8";
+    return "kxc_quantize_f32_nchw_to_c16_i8";
+}
+
+// int8 max pool and the requantising global average pool keep whatever layout their input has.
+HIPLayoutChoice Int8PoolLayout(const Attrs&, const Array<Type>& in, const Type&, const std::vector<int>& offered,
+                               const std::vector<bool>&) {
+    HIPLayoutChoice choice;
+    choice.inputs.assign(in.size(), kHIPLayoutPlain);
+    if (!MatrixCoresDisabled() && IsDType(in[0], "int8") && TT(in[0])->shape.size() == 4 && offered[0] == kHIPLayoutC16) {
+        choice.inputs[0] = kHIPLayoutC16;
+        choice.output = kHIPLayoutC16;
+    }
+    return choice;
+}
+HIPLayoutChoice QnnGapLayout(const Attrs&, const Array<Type>& in, const Type&, const std::vector<int>& offered,
+                             const std::vector<bool>&) {
+    // [N][C/16][1][1][16] is plain [N, C, 1, 1] when the channels fill their blocks
+    HIPLayoutChoice choice;
+    choice.inputs.assign(in.size(), kHIPLayoutPlain);
+    if (!MatrixCoresDisabled() && offered[0] == kHIPLayoutC16 && TT(in[0])->shape[1] % 16 == 0) choice.inputs[0] = kHIPLayoutC16;
+    return choice;
+}
+
+std::string QnnGapDispatch(const HIPDispatchContext& c, kxc_hip_plan* plan) {
+    const auto* p = c.attrs.As<QnnRequantAttrsNode>();
+    if (!p || !IsDType(c.input_types[0], "int8") || c.output_layout != kHIPLayoutPlain) return "";
+    const auto* x = TT(c.input_types[0]);
+    const bool blocked = !c.input_layouts.empty() && c.input_layouts[0] == kHIPLayoutC16;
+    Check(blocked ? kxc_hip_plan_add_global_avg_pool2d_c16_i8(plan, x->shape[0], x->shape[1], x->shape[2], x->shape[3],
+                                                              static_cast<float>(p->mult), B(c.inputs[0]), B(c.output))
+                  : kxc_hip_plan_add_global_avg_pool2d_i8(plan, x->shape[0], x->shape[1], x->shape[2], x->shape[3],
+                                                          static_cast<float>(p->mult), B(c.inputs[0]), B(c.output)),
+          "qnn_global_avg_pool2d dispatch");
+    return blocked ? "kxc_global_avg_pool2d_c16_i8" : "kxc_global_avg_pool2d_i8";
 }
 
 // ---------------------------------------------------------------- elementwise
@@ -312,6 +457,7 @@ void EnsureBuiltinOpsRegistered() {
             .set_attr<FRelayToTE>("FRelayToTE", [](const Attrs& a, const Array<te::Tensor>& in, const Type&) {
                 return PoolCompute("nn_max_pool2d", "max", "T_max_pool2d", a, in);
             })
+            .set_attr<FHIPLayoutQuery>("FHIPLayoutQuery", Int8PoolLayout)
             .set_attr<FHIPDispatch>("FHIPDispatch", [](const HIPDispatchContext& c, kxc_hip_plan* p) { return PoolDispatch(false, c, p); });
         OpRegEntry::Register("nn_avg_pool2d")
             .describe("2D average pooling operation.")
@@ -357,6 +503,8 @@ void EnsureBuiltinOpsRegistered() {
             .set_attr<std::string>("TAttrs", "QnnConv2DAttrs")
             .set_attr<FInferType>("FInferType", QnnConv2DInferType)
             .set_attr<FRelayToTE>("FRelayToTE", QnnConv2DCompute)
+            .set_attr<FHIPLayoutQuery>("FHIPLayoutQuery", QnnConv2DLayout)
+            .set_attr<FHIPPairQuery>("FHIPPairQuery", QnnConv2DPairQuery)
             .set_attr<FHIPDispatch>("FHIPDispatch", QnnConv2DDispatch);
         OpRegEntry::Register("qnn_dense")
             .describe("int8 dense layer with int32 accumulation; float32 output (acc + bias) * mult.")
@@ -382,7 +530,21 @@ void EnsureBuiltinOpsRegistered() {
                 if (!p || in.size() != 1) throw std::runtime_error("qnn_quantize expects one input and QnnQuantizeAttrs");
                 return te::topi::qnn_quantize(in[0], p->scale, "T_qnn_quantize");
             })
+            .set_attr<bool>("THIPLayoutFollowsConsumers", true)      // its kernels write NCHW, c16 or c4
             .set_attr<FHIPDispatch>("FHIPDispatch", QnnQuantizeDispatch);
+        OpRegEntry::Register("qnn_global_avg_pool2d")
+            .describe("int8 global average pool: the int32 sum over H and W, requantised with one multiplier, as int8 [N,C,1,1].")
+            .set_num_inputs(1)
+            .add_argument("data", "Tensor", "int8 input [N, C, H, W].")
+            .set_attr<std::string>("TAttrs", "QnnRequantAttrs")
+            .set_attr<FInferType>("FInferType", QnnGlobalAvgPool2DInferType)
+            .set_attr<FRelayToTE>("FRelayToTE", [](const Attrs& attrs, const Array<te::Tensor>& in, const Type&) {
+                const auto* p = attrs.As<QnnRequantAttrsNode>();
+                if (!p || in.size() != 1) throw std::runtime_error("qnn_global_avg_pool2d expects one input and QnnRequantAttrs");
+                return te::topi::qnn_global_avg_pool2d(in[0], p->mult, "T_qnn_global_avg_pool2d");
+            })
+            .set_attr<FHIPLayoutQuery>("FHIPLayoutQuery", QnnGapLayout)
+            .set_attr<FHIPDispatch>("FHIPDispatch", QnnGapDispatch);
         OpRegEntry::Register("matmul")
             .describe("Matrix multiplication [M,K] x [K,N]")
             .set_num_inputs(2)

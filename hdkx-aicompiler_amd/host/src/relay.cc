@@ -144,6 +144,11 @@ QnnQuantizeAttrs QnnQuantizeAttrs::Create(double scale) {
     n->scale = scale;
     return QnnQuantizeAttrs(n);
 }
+QnnRequantAttrs QnnRequantAttrs::Create(double mult) {
+    auto n = std::make_shared<QnnRequantAttrsNode>();
+    n->mult = mult;
+    return QnnRequantAttrs(n);
+}
 CastAttrs CastAttrs::Create(int to) {
     auto n = std::make_shared<CastAttrsNode>();
     n->to = to;
@@ -286,6 +291,27 @@ Type QnnDenseInferType(const Attrs&, const Array<Type>& in) {
     RequireChannelVector("qnn_dense", bias, "bias", weight->shape[0]);
     RequireChannelVector("qnn_dense", mult, "mult", weight->shape[0]);
     return TensorType({data->shape[0], weight->shape[0]}, "float32");
+}
+
+Type QnnGlobalAvgPool2DInferType(const Attrs& attrs, const Array<Type>& in) {
+    RequireArity("qnn_global_avg_pool2d", in, 1);
+    const auto* a = attrs.As<QnnRequantAttrsNode>();
+    if (!a || !(a->mult > 0.0)) throw std::runtime_error("qnn_global_avg_pool2d expects QnnRequantAttrs with a positive multiplier");
+    const auto* x = RequireTensor("qnn_global_avg_pool2d", in[0], "data");
+    RequireDType("qnn_global_avg_pool2d", x, "data", "int8");
+    if (x->shape.size() != 4) throw std::runtime_error("qnn_global_avg_pool2d expects an NCHW rank-4 input");
+    return TensorType({x->shape[0], x->shape[1], 1, 1}, "int8");
+}
+
+int64_t HIPLayoutBytes(const Type& t, int layout) {
+    const auto* tt = t.As<TensorTypeNode>();
+    if (!tt) throw std::runtime_error("HIPLayoutBytes: not a tensor type");
+    const int64_t elem = tir::DTypeFromString(tt->dtype).bytes();
+    if (layout == kHIPLayoutPlain || layout == kHIPLayoutAny) return Product(tt->shape) * elem;
+    if (tt->shape.size() != 4 || elem != 1) throw std::runtime_error("a channel-blocked layout needs a rank-4 int8 tensor");
+    const int64_t cbytes = layout == kHIPLayoutC16 ? (tt->shape[1] + 15) / 16 * 16 : 4;
+    if (layout == kHIPLayoutC4 && tt->shape[1] > 4) throw std::runtime_error("the 4-channel layout holds at most four channels");
+    return tt->shape[0] * cbytes * tt->shape[2] * tt->shape[3];
 }
 
 Type QnnQuantizeInferType(const Attrs& attrs, const Array<Type>& in) {
@@ -560,7 +586,7 @@ bool SplitExpr(const Expr& e, SplitState* st, Expr* out) {
             if (n == 3 && !BroadcastsOverBatch(call->args[2], 2)) return false;
         } else if (name == "nn_relu" || name == "sqrt" || name == "exp" || name == "log" || name == "cast" ||
                    name == "qnn_quantize" || name == "nn_max_pool2d" || name == "nn_avg_pool2d" ||
-                   name == "nn_global_avg_pool2d") {
+                   name == "nn_global_avg_pool2d" || name == "qnn_global_avg_pool2d") {
             if (n != 1) return false;
         } else if (name == "add" || name == "subtract" || name == "mul" || name == "multiply" || name == "divide") {
             if (n != 2) return false;

@@ -163,8 +163,12 @@ Tensor pool2d(const Tensor& data, std::vector<int> kernel_size, std::vector<int>
                            data(i[0], i[1], h_in, w_in), make_const(data->dtype, pad_value));
     };
     std::vector<PrimExpr> oshape = {data->shape[0], data->shape[1], I64(OH), I64(OW)};
+    // (the padding candidate of the reference, nn.h:225, is the float -1e30; an integer tensor takes its dtype's
+    // smallest value instead -- the reference converts -1e30 out of range there, which is undefined)
+    const double lowest = data->dtype.is_float() ? -1e30
+                          : data->dtype.is_uint() ? 0.0 : -static_cast<double>(int64_t{1} << (data->dtype.bits - 1));
     if (is_max)
-        return compute(oshape, [&](const Array<Var>& i) { return max(window(i, -1e30), {rh, rw}); }, name, kPool);
+        return compute(oshape, [&](const Array<Var>& i) { return max(window(i, lowest), {rh, rw}); }, name, kPool);
     Tensor sum_out = compute(oshape, [&](const Array<Var>& i) { return sum(window(i, 0), {rh, rw}); }, name + "_sum", kPool);
     return compute(oshape, [&](const Array<Var>& i) { return sum_out(i) / make_const(sum_out->dtype, KH * KW); }, name,
                    kPool);
@@ -336,6 +340,18 @@ Tensor qnn_conv2d_nchw(const Tensor& data, const Tensor& kernel, const Tensor& b
         PrimExpr v = tir::Call(f32, "cast", {acc(i) + bias(i[1])}) * mult(i[1]);
         if (residual.defined()) v = v + tir::Call(f32, "cast", {residual(i)}) * make_const(f32, static_cast<double>(static_cast<float>(res_mult)));
         return RintClampToI8(v, relu ? 0.0 : -128.0, 127.0);
+    }, name, kElementWise);
+}
+
+Tensor qnn_global_avg_pool2d(const Tensor& data, double mult, std::string name) {
+    const DataType i32 = DataType::Int(32), f32 = DataType::Float(32);
+    IterVar rh = reduce_axis(0, data->shape[2], "rh");
+    IterVar rw = reduce_axis(0, data->shape[3], "rw");
+    Tensor acc = compute({data->shape[0], data->shape[1], I64(1), I64(1)},
+                         [&](const Array<Var>& i) { return sum(tir::Call(i32, "cast", {data(i[0], i[1], rh.var, rw.var)}), {rh, rw}); },
+                         name + "_sum", kPool);
+    return compute(acc->shape, [&](const Array<Var>& i) {
+        return RintClampToI8(tir::Call(f32, "cast", {acc(i)}) * make_const(f32, static_cast<double>(static_cast<float>(mult))), -128.0, 127.0);
     }, name, kElementWise);
 }
 

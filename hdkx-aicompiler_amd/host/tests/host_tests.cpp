@@ -1289,6 +1289,101 @@ int RunQnn(const std::string& oracle_path) {
         }
         std::cout << "[PASS] qnn chain (quantize, conv, conv + residual)\n";
     }
+    // ---- int8 max pool (padding candidate and reduce identity are the dtype's lowest value) and the requantising
+    // global average pool, against the oracle; negative inputs everywhere so that a zero identity would show
+    {
+        using PoolFn = void (*)(const int8_t*, int8_t*, int64_t, int64_t, int64_t, int64_t, int, int, int, int, int, int, int, int);
+        using GapFn = void (*)(const int8_t*, int8_t*, int64_t, int64_t, int64_t, int64_t, float);
+        auto oracle_pool = reinterpret_cast<PoolFn>(dlsym(lib, "kxc_oracle_maxpool2d_i8"));
+        auto oracle_gap = reinterpret_cast<GapFn>(dlsym(lib, "kxc_oracle_global_avg_pool2d_i8"));
+        Check(oracle_pool && oracle_gap, "oracle pooling symbols missing");
+        const int64_t N = 2, C = 5, H = 9, W = 11;
+        std::vector<int8_t> x(N * C * H * W);
+        for (auto& e : x) e = static_cast<int8_t>(-128 + static_cast<int>(next() % 100));       // all negative
+        const int64_t OH = (H + 2 - 3) / 2 + 1, OW = (W + 2 - 3) / 2 + 1;
+        std::vector<int8_t> y(N * C * OH * OW, 99), want(y.size(), 77);
+        kxc::Var xv("x", kxc::TensorType({N, C, H, W}, "int8"));
+        kxc::Function fp({xv}, kxc::Call(Op::Get("nn_max_pool2d"), {xv},
+                                         kxc::relay::MaxPool2DAttrs::Create({2, 2}, {1, 1, 1, 1}, {1, 1}, {3, 3}, "NCHW", false)));
+        CompileAndRun("int8 max pool", fp, {I8(x, false), I8(y, true)});
+        oracle_pool(x.data(), want.data(), N, C, H, W, 3, 3, 2, 2, 1, 1, 1, 1);
+        Check(y == want, "int8 nn_max_pool2d differs from the oracle");
+        std::cout << "[PASS] int8 nn_max_pool2d on negative data\n";
+        fill_i8(x);
+        std::vector<int8_t> g(N * C, 99), gw(N * C, 77);
+        const float mult = 0.0173f;
+        kxc::Function fg({xv}, kxc::Call(Op::Get("qnn_global_avg_pool2d"), {xv}, kxc::relay::QnnRequantAttrs::Create(mult)));
+        CompileAndRun("qnn_global_avg_pool2d", fg, {I8(x, false), I8(g, true)});
+        oracle_gap(x.data(), gw.data(), N, C, H, W, mult);
+        Check(g == gw, "qnn_global_avg_pool2d differs from the oracle");
+        std::cout << "[PASS] qnn_global_avg_pool2d\n";
+    }
+    // ---- a chain wide enough for the int8 matrix cores: on the hip target the convolutions, the pool and the average
+    // run channel-blocked with the weights packed by the plan, and converters appear only where NCHW tensors enter
+    // (the int8 parameter, the residual parameter) -- same bytes as the oracle either way
+    {
+        using PoolFn = void (*)(const int8_t*, int8_t*, int64_t, int64_t, int64_t, int64_t, int, int, int, int, int, int, int, int);
+        using GapFn = void (*)(const int8_t*, int8_t*, int64_t, int64_t, int64_t, int64_t, float);
+        auto oracle_pool = reinterpret_cast<PoolFn>(dlsym(lib, "kxc_oracle_maxpool2d_i8"));
+        auto oracle_gap = reinterpret_cast<GapFn>(dlsym(lib, "kxc_oracle_global_avg_pool2d_i8"));
+        const int64_t N = 3, C = 24, H = 14, W = 10, O = 64;
+        std::vector<int8_t> x(N * C * H * W), w1(O * C * 9), w2(O * O * 9), wd(O * C), res(N * O * 7 * 5);
+        std::vector<int32_t> b1(O), b2(O), bd(O);
+        std::vector<float> m1(O), m2(O), md(O);
+        fill_i8(x); fill_i8(w1); fill_i8(w2); fill_i8(wd); fill_i8(res);
+        for (int64_t i = 0; i < O; ++i) {
+            b1[i] = static_cast<int32_t>(next() % 2001) - 1000; b2[i] = static_cast<int32_t>(next() % 2001) - 1000; bd[i] = static_cast<int32_t>(next() % 201) - 100;
+            m1[i] = (0.5f + static_cast<float>(next() % 1000) / 1000.0f) / (64.0f * std::sqrt(static_cast<float>(C * 9)));
+            m2[i] = (0.5f + static_cast<float>(next() % 1000) / 1000.0f) / (24.0f * std::sqrt(static_cast<float>(O * 9)));
+            md[i] = (0.5f + static_cast<float>(next() % 1000) / 1000.0f) / (64.0f * std::sqrt(static_cast<float>(C)));
+        }
+        kxc::Var xv("x", kxc::TensorType({N, C, H, W}, "int8")), rv("r", kxc::TensorType({N, O, 7, 5}, "int8"));
+        kxc::Var w1v("w1", kxc::TensorType({O, C, 3, 3}, "int8")), w2v("w2", kxc::TensorType({O, O, 3, 3}, "int8")), wdv("wd", kxc::TensorType({O, C, 1, 1}, "int8"));
+        kxc::Var b1v("b1", kxc::TensorType({O}, "int32")), b2v("b2", kxc::TensorType({O}, "int32")), bdv("bd", kxc::TensorType({O}, "int32"));
+        kxc::Var m1v("m1", kxc::TensorType({O}, "float32")), m2v("m2", kxc::TensorType({O}, "float32")), mdv("md", kxc::TensorType({O}, "float32"));
+        // block: a = conv3x3/2(x) relu; idn = conv1x1/2(x); s = conv3x3(a) + idn, relu; t = conv3x3(s) + r (a parameter), relu;
+        // p = maxpool(t); g = gap(p)
+        kxc::Call a(Op::Get("qnn_conv2d"), {xv, w1v, b1v, m1v}, kxc::relay::QnnConv2DAttrs::Create({2, 2}, {1, 1}, true));
+        kxc::Call idn(Op::Get("qnn_conv2d"), {xv, wdv, bdv, mdv}, kxc::relay::QnnConv2DAttrs::Create({2, 2}, {0, 0}, false));
+        kxc::Call sum(Op::Get("qnn_conv2d"), {a, w2v, b2v, m2v, idn}, kxc::relay::QnnConv2DAttrs::Create({1, 1}, {1, 1}, true, 0.6));
+        kxc::Call t(Op::Get("qnn_conv2d"), {sum, w2v, b2v, m2v, rv}, kxc::relay::QnnConv2DAttrs::Create({1, 1}, {1, 1}, true, 0.4));
+        kxc::Call pool(Op::Get("nn_max_pool2d"), {t}, kxc::relay::MaxPool2DAttrs::Create({2, 2}, {1, 1, 1, 1}, {1, 1}, {3, 3}, "NCHW", false));
+        kxc::Call gap(Op::Get("qnn_global_avg_pool2d"), {pool}, kxc::relay::QnnRequantAttrs::Create(0.21));
+        std::vector<int8_t> ya(N * O * 7 * 5), yi(ya.size()), ys(ya.size()), yt(ya.size()), yp(N * O * 4 * 3), yg(N * O);
+        oracle_conv(x.data(), w1.data(), b1.data(), m1.data(), nullptr, 0.0f, ya.data(), N, C, H, W, O, 3, 3, 2, 2, 1, 1, 1);
+        oracle_conv(x.data(), wd.data(), bd.data(), md.data(), nullptr, 0.0f, yi.data(), N, C, H, W, O, 1, 1, 2, 2, 0, 0, 0);
+        oracle_conv(ya.data(), w2.data(), b2.data(), m2.data(), yi.data(), 0.6f, ys.data(), N, O, 7, 5, O, 3, 3, 1, 1, 1, 1, 1);
+        oracle_conv(ys.data(), w2.data(), b2.data(), m2.data(), res.data(), 0.4f, yt.data(), N, O, 7, 5, O, 3, 3, 1, 1, 1, 1, 1);
+        oracle_pool(yt.data(), yp.data(), N, O, 7, 5, 3, 3, 2, 2, 1, 1, 1, 1);
+        oracle_gap(yp.data(), yg.data(), N, O, 4, 3, 0.21f);
+        const std::vector<kxc::Var> params = {xv, rv, w1v, b1v, m1v, w2v, b2v, m2v, wdv, bdv, mdv};
+        auto bufs = [&](std::vector<int8_t>& out) {
+            return std::vector<Buf>{I8(x, false), I8(res, false), I8(w1, false), I32(b1), In(m1), I8(w2, false), I32(b2), In(m2), I8(wd, false), I32(bd), In(md), I8(out, true)};
+        };
+        struct Cut { const char* name; kxc::Expr value; std::vector<int8_t>* want; };
+        for (const Cut& c : {Cut{"t", t, &yt}, Cut{"pool", pool, &yp}, Cut{"gap", gap, &yg}, Cut{"idn", idn, &yi}}) {
+            std::vector<int8_t> got(c.want->size(), 99);
+            kxc::Function f(params, c.value);
+            CompileAndRun(std::string("wide qnn chain cut at ") + c.name, f, bufs(got));
+            Check(got == *c.want, std::string("wide qnn chain cut at ") + c.name + " differs from the oracle");
+        }
+        if (g_mode == "hip") {
+            auto module = kxc::api::Compiler::Compile(kxc::Function(params, gap), MakeConfig());
+            std::string all;
+            int c16 = 0, to_c16 = 0, to_nchw = 0;
+            for (const auto& k : module.GetKernelExecs()) {
+                all += k.kernel_symbol + "; ";
+                c16 += k.kernel_symbol.find("kxc_qconv2d_c16_i8") != std::string::npos;
+                to_c16 += k.kernel_symbol == "kxc_i8_nchw_to_c16";
+                to_nchw += k.kernel_symbol == "kxc_i8_c16_to_nchw";
+            }
+            // pair (a + idn), sum, t on the matrix cores; x and r converted on the way in; the pool and the average blocked
+            Check(c16 == 3 && to_c16 == 2 && to_nchw == 0 && all.find("|qconv1x1+bias") != std::string::npos &&
+                      all.find("kxc_max_pool2d_c16_i8") != std::string::npos && all.find("kxc_global_avg_pool2d_c16_i8") != std::string::npos,
+                  "wide qnn chain: unexpected launches: " + all);
+        }
+        std::cout << "[PASS] wide qnn chain (matrix-core layouts on hip)\n";
+    }
     // ---- type rules
     {
         auto expect_throw = [](const std::function<void()>& fn, const std::string& needle) {

@@ -279,6 +279,8 @@ int32_t kxc_hip_qconv2d_c16_pack_weights(const kxc_hip_qconv2d_desc* desc, const
                                          void* stream);
 /* Name of the kernel variant the shape selects ("none" when no matrix-core variant covers it). */
 const char* kxc_hip_qconv2d_c16_variant(const kxc_hip_qconv2d_desc* desc);
+/* 1 when a matrix-core variant covers the shape (what an operator hook asks before it chooses the layout). */
+int32_t kxc_hip_qconv2d_c16_supported(const kxc_hip_qconv2d_desc* desc);
 /* x, residual, y in c16; w_packed from kxc_hip_qconv2d_c16_pack_weights; bias int32[O], mult float[O]. */
 int32_t kxc_hip_qconv2d_c16_i8(const kxc_hip_qconv2d_desc* desc, const int8_t* x, const int8_t* w_packed,
                                const int32_t* bias, const float* mult, const int8_t* residual, int8_t* y,
@@ -304,6 +306,7 @@ int32_t kxc_hip_quantize_f32_nchw_to_c16_i8(const float* x, int8_t* y, int64_t n
 /* First layer (7x7, stride 2, padding 3, at most 4 input channels, width a multiple of 4) on the "c4" input
  * layout [N][H][W][4] (4 bytes per pixel, channels >= C zero): a k-step of the matrix instruction is one
  * filter row of 8 taps x 4 channels.  Output is c16.  Weights are packed by the _c4_pack_weights call. */
+int32_t kxc_hip_qconv2d_c4_supported(const kxc_hip_qconv2d_desc* desc);
 int32_t kxc_hip_qconv2d_c4_packed_bytes(const kxc_hip_qconv2d_desc* desc, size_t* out_bytes);
 int32_t kxc_hip_qconv2d_c4_pack_weights(const kxc_hip_qconv2d_desc* desc, const int8_t* w_oihw, int8_t* packed,
                                         void* stream);
@@ -424,6 +427,24 @@ int32_t kxc_hip_plan_add_global_avg_pool2d_c16_i8(kxc_hip_plan* plan, int64_t n,
                                                   int64_t w, float mult, kxc_hip_buf x, kxc_hip_buf y);
 int32_t kxc_hip_plan_add_qdense(kxc_hip_plan* plan, int64_t m, int64_t n, int64_t k, kxc_hip_buf a,
                                 kxc_hip_buf b, kxc_hip_buf bias, kxc_hip_buf mult, kxc_hip_buf y);
+/* kxc_hip_i8_nchw_to_c16 (to_c16 != 0) or kxc_hip_i8_c16_to_nchw as a node: what a graph compiler places on an edge
+ * between an operator that keeps int8 activations in NCHW and one that keeps them channel-blocked. */
+int32_t kxc_hip_plan_add_i8_layout(kxc_hip_plan* plan, int32_t to_c16, int64_t n, int64_t c, int64_t hw,
+                                   kxc_hip_buf x, kxc_hip_buf y);
+/* Constant preparation: the OIHW int8 weights `w_oihw` of a convolution (a packed argument: a module constant,
+ * include/relay/relay.h:120-134, which the caller passes again on every run, test/onnx_importer_test.cpp:249-255)
+ * are packed into the workspace region `w_packed` in the order kind's kernel reads them --
+ * KXC_HIP_QPACK_C16: kxc_hip_qconv2d_c16_pack_weights, _C4: kxc_hip_qconv2d_c4_pack_weights, _C16_PAIR:
+ * kxc_hip_qconv2d_c16_pair_pack_weights (desc = the first convolution, w_oihw = the second one's [o,c,1,1]).
+ * Like the Winograd filter transforms, all packs of a plan run as ONE launch at the start of every run, so a run
+ * sees the current contents of its constants; with kxc_hip_plan_freeze_constants a tensor is packed when its
+ * pointer is first seen (every_run != 0 keeps a pack on every run even then: weights that are not constants). */
+#define KXC_HIP_QPACK_C16 1
+#define KXC_HIP_QPACK_C4 2
+#define KXC_HIP_QPACK_C16_PAIR 3
+int32_t kxc_hip_plan_add_qconv_weight_pack(kxc_hip_plan* plan, int32_t kind, const kxc_hip_qconv2d_desc* desc,
+                                           kxc_hip_buf w_oihw, kxc_hip_buf w_packed, int32_t every_run);
+int32_t kxc_hip_plan_num_weight_packs(const kxc_hip_plan* plan);
 /* A run-time compiled kernel (section 3): params[i] is a buffer operand, passed as a pointer. */
 int32_t kxc_hip_plan_add_module_kernel(kxc_hip_plan* plan, void* function, const char* symbol,
                                        const uint32_t grid[3], const uint32_t block[3],

@@ -353,3 +353,166 @@ def test_qdense_shapes(pkg, orc, m, n, k):
     mult = rng.uniform(1e-4, 1e-3, (n,)).astype(np.float32)
     assert_bit_exact(host(pkg.qdense(dev(a), dev(b), dev(bias), dev(mult))), orc.qdense(a, b, bias, mult),
                      "qdense %dx%dx%d" % (m, n, k))
+
+
+# ---------------------------------------------------------------- the same network compiled from its Relay graph
+def _compiled(pkg, model, batch, hw, **kw):
+    ha = importlib.import_module("hdkx-aicompiler_amd.hostapi")
+    mod = ha.CompiledQResNet18(model, batch, hw, **kw)
+    consts = [dev(c) for c in mod.constants(model)]
+    return mod, consts
+
+
+def _run_compiled(mod, x_dev, consts, out):
+    mod.run_packed(mod.packed([x_dev] + consts + [out]))
+    torch.cuda.synchronize()
+
+
+def test_compiled_qresnet18_plan_is_the_matrix_core_plan(pkg):
+    """Compiler::Compile on the quantised graph chooses the channel-blocked layout itself: 21 launches, the first
+    convolution on the 4-channel input layout, every other one on c16, the three downsamples as second outputs,
+    weights packed by the plan from the OIHW constants (20 packs, one per convolution), no layout converter anywhere."""
+    qr, x, model = _quantised_model(pkg, 2, 64, 5)
+    mod, _ = _compiled(pkg, model, 2, 64)
+    sym = mod.launches()
+    assert len(sym) == 21
+    assert sym[0] == "qnn_quantize kxc_quantize_f32_nchw_to_c4_i8"
+    assert sym[1].startswith("qnn_conv2d kxc_qconv2d_c4_i8:qmfma")
+    assert sym[2] == "nn_max_pool2d kxc_max_pool2d_c16_i8"
+    assert all(s.startswith("qnn_conv2d kxc_qconv2d_c16_i8:qmfma") for s in sym[3:19])
+    assert sum("|qconv1x1+bias" in s for s in sym) == 3
+    assert sym[19] == "qnn_global_avg_pool2d kxc_global_avg_pool2d_c16_i8" and sym[20] == "qnn_dense kxc_qdense_i8"
+    assert not any("layout_convert" in s for s in sym)
+    plan_text = mod.plan_json()
+    assert plan_text.count("\\npack ") == 20 and "kxc_hip_plan 3" in plan_text
+
+
+def test_compiled_qresnet18_small_every_layer(pkg, orc):
+    """Batch 2, 64x64 input, through Compiler::Compile: the logits, and every quantised tensor of the network as the
+    result of the graph cut at that layer (which also exercises the converter back to NCHW), bit-exact against the
+    CPU int8 chain."""
+    qr, x, model = _quantised_model(pkg, 2, 64, 5)
+    mod, consts = _compiled(pkg, model, 2, 64)
+    out = torch.empty((2, 1000), device="cuda")
+    _run_compiled(mod, dev(x), consts, out)
+    want_logits, taps = orc.qresnet18(x, model, mod.gap_mult)
+    assert_bit_exact(host(out), want_logits, "compiled quantised logits")
+    # a second run and a run after the weights were updated in place see the current constants
+    _run_compiled(mod, dev(x), consts, out)
+    assert_bit_exact(host(out), want_logits, "compiled quantised logits, second run")
+    for name, want in taps.items():
+        cut, cc = _compiled(pkg, model, 2, 64, result=name)
+        got = torch.empty(want.shape, dtype=torch.int8, device="cuda")
+        _run_compiled(cut, dev(x), cc, got)
+        assert_bit_exact(host(got), want, "compiled graph cut at %s" % name)
+        cut.close()
+    mod.close()
+
+
+def test_compiled_qresnet18_constants_are_read_on_every_run(pkg, orc):
+    """The CPU backend re-reads every constant on every call; so does the compiled module unless its constants are
+    frozen: an in-place update of a weight tensor shows in the next run, a frozen module keeps the packed copy until
+    it is told."""
+    qr, x, model = _quantised_model(pkg, 2, 64, 5)
+    mod, consts = _compiled(pkg, model, 2, 64)
+    out = torch.empty((2, 1000), device="cuda")
+    _run_compiled(mod, dev(x), consts, out)
+    before = host(out).copy()
+    k = mod.constant_names.index("l3.1.conv1.w")
+    saved = consts[k].clone()
+    consts[k].neg_()
+    changed = dict(model)
+    changed["layers"] = [dict(L, wq=-L["wq"]) if L["name"] == "l3.1.conv1" else L for L in model["layers"]]
+    want, _ = orc.qresnet18(x, changed, mod.gap_mult)
+    _run_compiled(mod, dev(x), consts, out)
+    assert_bit_exact(host(out), want, "logits after an in-place weight update")
+    assert not np.array_equal(host(out), before)
+    mod.freeze_constants(True)
+    _run_compiled(mod, dev(x), consts, out)                   # packs what it is given now
+    consts[k].copy_(saved)
+    _run_compiled(mod, dev(x), consts, out)                   # frozen: still the packed copy of the negated weights
+    assert_bit_exact(host(out), want, "frozen module keeps its packed weights")
+    mod.invalidate_constants()
+    _run_compiled(mod, dev(x), consts, out)
+    assert_bit_exact(host(out), before, "after invalidate_constants the restored weights are packed again")
+    mod.close()
+
+
+def test_compiled_qresnet18_batch64_images(pkg, orc):
+    """BASELINE configuration 5 through Compiler::Compile: images 0 and 63 of the batch against the CPU int8 chain,
+    the hand-assembled plan of the same launches, graph replay, and two shares of the batch side by side."""
+    qr, x, model = _quantised_model(pkg, 64, 224, 5)
+    mod, consts = _compiled(pkg, model, 64, 224)
+    assert len(mod.launches()) == 21
+    xd = dev(x)
+    out = torch.empty((64, 1000), device="cuda")
+    _run_compiled(mod, xd, consts, out)
+    first = host(out).copy()
+    for n in (0, 63):
+        want, _ = orc.qresnet18(x[n:n + 1], model, mod.gap_mult)
+        assert_bit_exact(first[n:n + 1], want, "compiled quantised resnet18 batch 64, image %d" % n)
+    mod.freeze_constants(True)
+    mod.enable_graph_replay(True)
+    stream = torch.cuda.Stream()
+    args = mod.packed([xd] + consts + [out])
+    with torch.cuda.stream(stream):
+        for replay in range(4):
+            out.zero_()
+            mod.run_packed(args, stream.cuda_stream)
+            stream.synchronize()
+            assert_bit_exact(host(out), first, "frozen module, graph replay %d" % replay)
+    two, _ = _compiled(pkg, model, 64, 224, lanes=2)
+    assert len(two.launches()) == 42
+    out2 = torch.zeros((64, 1000), device="cuda")
+    _run_compiled(two, xd, consts, out2)
+    assert_bit_exact(host(out2), first, "two shares of the batch")
+    two.close()
+    mod.close()
+
+
+def test_plan_weight_pack_and_layout_nodes(pkg, orc):
+    """C ABI: a plan that is handed OIHW weights packs them itself at the start of a run (one launch for all packs)
+    and converts between NCHW and c16 with layout nodes; its text form round-trips."""
+    H = pkg
+    rng = np.random.default_rng(17)
+    n, c, h, w, o = 2, 40, 13, 17, 64
+    x = rng.integers(-128, 128, (n, c, h, w), dtype=np.int8)
+    wq = rng.integers(-127, 128, (o, c, 3, 3), dtype=np.int8)
+    bias = rng.integers(-20000, 20000, (o,), dtype=np.int32)
+    mult = rng.uniform(0.5, 2.0, (o,)).astype(np.float32) * np.float32(1.0 / (8.0 * np.sqrt(c * 9) * 64))
+    want = orc.qconv(x, wq, bias, mult, 1, 1, None, 0.0, True)
+    d = H.qconv_desc(n, c, h, w, o, 3, 3, 1, 1, H.CONV_BIAS | H.CONV_RELU)
+    Buf = H.Buf
+    cb, ob = (c + 15) // 16, o // 16
+    off_x = 0
+    off_y = off_x + (n * cb * h * w * 16 + 255) // 256 * 256
+    off_w = off_y + (n * ob * h * w * 16 + 255) // 256 * 256
+    plan = H.Plan(5)
+    plan.add_i8_layout(True, n, c, h * w, Buf.arg(0), Buf.ws(off_x))
+    plan.add_qconv_weight_pack(H.QPACK_C16, d, Buf.arg(1), Buf.ws(off_w))
+    plan.add_qconv2d_c16(d, Buf.ws(off_x), Buf.ws(off_w), Buf.arg(2), Buf.arg(3), Buf.none(), Buf.ws(off_y))
+    plan.add_i8_layout(False, n, o, h * w, Buf.ws(off_y), Buf.arg(4))
+    assert plan.num_weight_packs() == 1
+    packed_bytes = int(H.qconv2d_c16_pack_weights(dev(wq)).numel())
+    with pytest.raises(H.KxcHipError):
+        plan.finalize(off_w + packed_bytes - 1)          # the packed weights must fit the workspace
+    plan.finalize(off_w + packed_bytes)
+    out = torch.zeros((n, o, h, w), dtype=torch.int8, device="cuda")
+    wd = dev(wq)
+    plan.run([dev(x), wd, dev(bias), dev(mult), out])
+    torch.cuda.synchronize()
+    assert_bit_exact(host(out), want, "plan with its own weight pack")
+    again = H.Plan.deserialize(plan.serialize(), 0)
+    assert again.num_weight_packs() == 1 and again.symbols() == plan.symbols()
+    out.zero_()
+    again.run([dev(x), wd, dev(bias), dev(mult), out])
+    torch.cuda.synchronize()
+    assert_bit_exact(host(out), want, "the same plan rebuilt from its text")
+    # the weights must be a packed argument, the packed copy a workspace region
+    bad = H.Plan(5)
+    with pytest.raises(H.KxcHipError):
+        bad.add_qconv_weight_pack(H.QPACK_C16, d, Buf.ws(0), Buf.ws(256))
+    with pytest.raises(H.KxcHipError):
+        bad.add_qconv_weight_pack(H.QPACK_C16, d, Buf.arg(1), Buf.arg(2))
+    with pytest.raises(H.KxcHipError):
+        bad.add_qconv_weight_pack(9, d, Buf.arg(1), Buf.ws(0))

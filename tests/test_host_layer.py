@@ -76,7 +76,7 @@ def test_quantised_operators_cpu():
     """qnn_quantize / qnn_conv2d / qnn_dense as graph operators (type rule, TE compute with the rint intrinsic, host
     back end): hand-worked answers, and the C oracle on seeded cases, element for element."""
     out = run("qnn", "cpu", _oracle_so())
-    assert "quantised operators ok (cpu)" in out and out.count("[PASS]") == 13
+    assert "quantised operators ok (cpu)" in out and out.count("[PASS]") == 16
 
 
 @pytest.mark.gpu
@@ -85,7 +85,7 @@ def test_quantised_operators_gpu(mode):
     """The same cases through the hand-written int8 launches (hip) and through kernels generated from the operators'
     TE compute (hipgen)."""
     out = run("qnn", mode, _oracle_so())
-    assert "quantised operators ok (%s)" % mode in out and out.count("[PASS]") == 13
+    assert "quantised operators ok (%s)" % mode in out and out.count("[PASS]") == 16
 
 
 @pytest.mark.gpu
@@ -201,6 +201,52 @@ def test_resnet18_hip_plan_without_gpu():
         few = json.load(open(os.path.join(d, "plan.json")))
     # with the work threshold only the 56x56 layers have enough 2x2 blocks per input channel
     assert sum("winograd" in n["kernel_symbol"] for n in few["nodes"]) == 4
+
+
+def test_quantised_resnet18_hip_plan_without_gpu():
+    """The quantised ResNet-18 graph (qnn_quantize, qnn_conv2d, int8 max pool, qnn_global_avg_pool2d, qnn_dense)
+    compiled for the hip target: the operators' layout hooks put every activation between the first convolution and
+    the average pool into the channel-blocked layout of the int8 matrix cores, the input into the 4-channel layout,
+    and pair each downsample with its block's first convolution -- 24 calls, 21 launches, no converter.  With
+    KXC_HIP_QNN_MFMA=0 every operator keeps NCHW and its reference-order kernel."""
+    import importlib
+    ha = importlib.import_module("hdkx-aicompiler_amd.hostapi")
+    qr = importlib.import_module("hdkx-aicompiler_amd.qresnet18")
+    layers = [{"name": n, "res_mult": 0.37 if n.endswith(".conv2") else 0.0} for (n, *_rest) in qr.layer_table()]
+    model = {"layers": layers, "scale": {"last": 0.02}, "input_scale": 0.02, "gap_scale_out": 0.01, "last": "last"}
+    mod = ha.CompiledQResNet18(model, 64, 224)
+    sym = mod.launches()
+    plan = json.loads(mod.plan_json())
+    assert len(sym) == 21 and len(plan["nodes"]) == 21 and len(plan["constant_value_ids"]) == 63 and mod.num_args == 65
+    assert sym[0] == "qnn_quantize kxc_quantize_f32_nchw_to_c4_i8" and sym[1].startswith("qnn_conv2d kxc_qconv2d_c4_i8:qmfma")
+    assert sym[2] == "nn_max_pool2d kxc_max_pool2d_c16_i8"
+    assert all(s.startswith("qnn_conv2d kxc_qconv2d_c16_i8:qmfma") for s in sym[3:19])
+    assert sum(s.endswith("+relu|qconv1x1+bias") for s in sym) == 3 and sum(s.endswith("+add+relu") for s in sym) == 8
+    pairs = [n for n in plan["nodes"] if "|qconv1x1" in n["kernel_symbol"]]
+    assert all(len(n["output_values"]) == 2 and len(n["input_values"]) == 7 for n in pairs)
+    assert sym[19:] == ["qnn_global_avg_pool2d kxc_global_avg_pool2d_c16_i8", "qnn_dense kxc_qdense_i8"]
+    assert mod.constant_names[:3] == ["conv1.w", "conv1.b", "conv1.m"] and mod.constant_names[-3:] == ["fc.w", "fc.b", "fc.m"]
+    # constants in depth-first argument order: a block's second convolution before its downsample
+    k = mod.constant_names.index("l2.0.conv2.w")
+    assert mod.constant_names[k - 3] == "l2.0.conv1.w" and mod.constant_names[k + 3] == "l2.0.down.w"
+    mod.close()
+    # a batch of 128 runs as two shares side by side; a graph cut at a convolution converts its result back to NCHW
+    two = ha.CompiledQResNet18(model, 128, 224)
+    assert len(two.launches()) == 42 and two.launches()[1].endswith(" @share1")
+    two.close()
+    cut = ha.CompiledQResNet18(model, 2, 64, result="l2.0.down")
+    assert cut.launches()[-1] == "layout_convert kxc_i8_c16_to_nchw" and "qmfma_k1x1" in cut.launches()[-2]
+    assert cut.constant_names[-1] == "l2.0.down.m" and "l2.0.conv1.w" not in cut.constant_names
+    cut.close()
+    os.environ["KXC_HIP_QNN_MFMA"] = "0"
+    try:
+        plain = ha.CompiledQResNet18(model, 2, 64)
+        names = [s.split(" ", 1)[1] for s in plain.launches()]
+        assert len(names) == 24 and names.count("kxc_qconv2d_nchw_i8") == 20 and names[0] == "kxc_quantize_f32_i8"
+        assert "kxc_max_pool2d_i8" in names and "kxc_global_avg_pool2d_i8" in names
+        plain.close()
+    finally:
+        del os.environ["KXC_HIP_QNN_MFMA"]
 
 
 # ------------------------------------------------------------------ GPU
