@@ -87,6 +87,8 @@ def main():
     ap.add_argument("--no-layers", action="store_true", help="skip the per-layer / per-operator timings")
     ap.add_argument("--int8-only", action="store_true",
                     help="run only the quantised ResNet-18 leg (for profiling its kernels) and print its JSON")
+    ap.add_argument("--cpu-full", action="store_true",
+                    help="also time the CPU path on the whole batch once (minutes on one core) -> cpu_baseline.batch_seconds")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py: this build runs on exactly one GPU (no collectives, no sharding); "
@@ -134,12 +136,15 @@ def main():
         torch.cuda.synchronize()
         return (time.perf_counter() - t0) * 1e3 / args.steps
 
-    # eager: 23 launches per step enqueued one by one; then the same plan replayed as one captured HIP graph per
-    # step (needs a stream other than the null stream; the first run on it is eager, the second is captured)
-    # Default mode first: every run re-transforms the Winograd filters from the weight pointers it is given (one
-    # extra launch).  Then the serving mode the headline number is quoted on: the caller declares the weights
-    # fixed, the filters are transformed once (in the warm-up) and the timed steps are the 23 launches of the pass.
+    # Three modes, all named in `config`:
+    #  * default: what a caller who only switched the target gets -- every run re-transforms the Winograd filters
+    #    from the weight pointers it is given (one extra launch), launches enqueued one by one;
+    #  * frozen (the mode `value` is quoted on): the caller declares the weights fixed (FreezeConstants), the filters
+    #    are transformed once, in the warm-up; timed eagerly and as one captured HIP graph per step (needs a stream
+    #    other than the null stream; the first run on it is eager, the second is captured), the faster one counts;
+    #  * one stream: the frozen plan compiled with hip_batch_lanes = 1, i.e. without the second share's stream.
     unfrozen_ms = timed(lambda: module.run_packed(packed, stream))
+    logits_default_mode = out.detach().cpu().numpy().copy()
     module.freeze_constants(True)
     eager_ms = timed(lambda: module.run_packed(packed, stream))
     graph_ms = None
@@ -152,12 +157,38 @@ def main():
             graph_ms = timed(lambda: module.run_packed(packed, side.cuda_stream))
         torch.cuda.synchronize()
         module.enable_graph_replay(False)
-    t1, t0 = (min(eager_ms, graph_ms) if graph_ms is not None else eager_ms) * args.steps * 1e-3, 0.0
-    ms_per_step = (t1 - t0) * 1e3 / args.steps
+    ms_per_step = min(eager_ms, graph_ms) if graph_ms is not None else eager_ms
+    timed_mode = "graph" if graph_ms is not None and graph_ms < eager_ms else "eager"
     img_s = batch / (ms_per_step * 1e-3)
     flop_step = r18.flops_per_image() * batch
     logits_ok = bool(torch.isfinite(out).all().item())
     logits_timed_plan = out.detach().cpu().numpy().copy()        # what the timed plan computed (checked below)
+    default_equals_timed = bool(np.array_equal(logits_default_mode.view(np.uint32), logits_timed_plan.view(np.uint32)))
+    one_stream_ms = None
+    if shares > 1:
+        prev = os.environ.get("KXC_HIP_BATCH_LANES")
+        os.environ["KXC_HIP_BATCH_LANES"] = "1"
+        try:
+            single = hostapi.CompiledResNet18(batch, 224, "hip", sync_after_run=False)
+        finally:
+            if prev is None:
+                del os.environ["KXC_HIP_BATCH_LANES"]
+            else:
+                os.environ["KXC_HIP_BATCH_LANES"] = prev
+        out1 = torch.empty_like(out)
+        packed1 = single.packed([x] + consts + [out1])
+        single.freeze_constants(True)
+        one_stream_ms = timed(lambda: single.run_packed(packed1, stream))
+        if not args.eager:
+            side1 = torch.cuda.Stream()
+            with torch.cuda.stream(side1):
+                single.enable_graph_replay(True)
+                for _ in range(3):
+                    single.run_packed(packed1, side1.cuda_stream)
+                one_stream_ms = min(one_stream_ms, timed(lambda: single.run_packed(packed1, side1.cuda_stream)))
+            torch.cuda.synchronize()
+        single.close()
+        del out1
     # per-launch durations inside the network (HIP events between consecutive launches, average of 5 passes)
     in_network = None
     if not args.no_layers:
@@ -243,8 +274,14 @@ def main():
         "config": {"workload": "ResNet-18 fp32 inference, batch %d, input [%d,3,224,224], BN folded, seeded Kaiming weights "
                                "(benchmark configuration %d)" % (batch, batch, 4 if batch == 64 else 3),
                    "compiled_by": "C++ host layer, Compiler::Compile(Relay graph, target hip)",
-                   "constants": "frozen (serving mode: Winograd filter transforms run once, in the warm-up; "
-                                "eager_unfrozen_ms_per_step re-transforms them in every step)",
+                   "constants": "frozen (serving mode: Winograd filter transforms run once, in the warm-up); "
+                                "default_mode_ms_per_step is what an unchanged caller gets",
+                   "timed_mode": timed_mode,
+                   "default_mode_ms_per_step": round(unfrozen_ms, 4),
+                   "default_mode": "constants re-read (filters re-transformed) in every run, eager launches, %d share(s) of the batch" % shares,
+                   "default_mode_logits_equal_timed_bit_for_bit": default_equals_timed,
+                   "one_stream_ms_per_step": round(one_stream_ms, 4) if one_stream_ms is not None else round(ms_per_step, 4),
+                   "one_stream": "hip_batch_lanes = 1 (no second stream inside the plan), frozen constants, faster of eager and graph",
                    "batch_shares": shares, "launches_per_step": len(info["launches"]), "workspace_bytes": info["workspace_bytes"]},
         "end_to_end_tflops": round(flop_step / (ms_per_step * 1e-3) / 1e12, 3),
         "end_to_end_frac_of_fp32_mfma_peak": round(flop_step / (ms_per_step * 1e-3) / 1e12 / PEAK_FP32_MFMA_TFLOPS, 4),
@@ -267,6 +304,17 @@ def main():
     if not args.no_cpu:
         result["cpu_baseline"], want0 = cpu_baseline(np, synth)
         result["gpu_over_cpu"] = round(img_s / result["cpu_baseline"]["value"], 1)
+        result["gpu_over_cpu_note"] = "GPU batch-%d throughput over the CPU path's one-image rate (the CPU path has no batch effect: one scalar thread)" % batch
+        if args.cpu_full:
+            from oracle_lib import Oracle as _Oracle
+            t0 = time.perf_counter()
+            full = _Oracle(fast=True).resnet18(x_h, consts_h)
+            secs = time.perf_counter() - t0
+            result["cpu_baseline"]["batch_seconds"] = round(secs, 2)
+            result["cpu_baseline"]["batch_img_per_s"] = round(batch / secs, 4)
+            result["gpu_over_cpu_same_batch"] = round(img_s / (batch / secs), 1)
+            g, w = logits_timed_plan.astype(np.float64), full.astype(np.float64)
+            result["parity_whole_batch_max_scaled_err"] = float(np.max(np.abs(g - w) / np.maximum(1.0, np.abs(w))))
         # parity of the TIMED plan at its real size: its logits for the first and the last image of the batch against
         # the CPU path on those images (the reference's acceptance metric, max |a-r| / max(1,|r|), and the plain
         # relative error over logits above 1 % of the largest)
@@ -404,24 +452,44 @@ def bench_batch1(torch, pkg, hostapi, synth, dev):
 
 
 def bench_int8(torch, pkg, synth, dev, np, batch):
-    """Benchmark configuration 5: quantised ResNet-18, batch 64, int8 matrix cores (calibrated on the same batch)."""
+    """Benchmark configuration 5: quantised ResNet-18, batch 64, int8 matrix cores (calibrated on the same batch).
+    The network is the quantised Relay graph compiled by Compiler::Compile for the hip target."""
     qr = importlib.import_module("hdkx-aicompiler_amd.qresnet18")
+    hostapi = importlib.import_module("hdkx-aicompiler_amd.hostapi")
     consts = synth.resnet18_consts(5)
     x = dev(synth.resnet18_input(5, batch))
     amax = qr.calibrate(x, [dev(c) for c in consts])
     model = qr.prepare(consts, amax)
-    net = qr.QuantizedResNet18(model, batch, 224)
+    module = hostapi.CompiledQResNet18(model, batch, 224, "hip", sync_after_run=False)
+    qconsts = [dev(c) for c in module.constants(model)]
     out = torch.empty((batch, 1000), device="cuda")
-    packed = net.packed(x, out)
+    packed = module.packed([x] + qconsts + [out])
     stream = torch.cuda.current_stream().cuda_stream
-    ms = _event_time_ms(torch, lambda: net.plan.run_packed(packed, stream), 50, 10)
+    # default mode: every run packs the int8 weights again from the pointers it is given (one extra launch)
+    unfrozen_ms = _event_time_ms(torch, lambda: module.run_packed(packed, stream), 50, 10)
+    module.freeze_constants(True)
+    eager_ms = _event_time_ms(torch, lambda: module.run_packed(packed, stream), 50, 10)
+    side = torch.cuda.Stream()
+    with torch.cuda.stream(side):
+        module.enable_graph_replay(True)
+        graph_ms = _event_time_ms(torch, lambda: module.run_packed(packed, side.cuda_stream), 50, 10)
+    torch.cuda.synchronize()
+    ms = min(eager_ms, graph_ms)
     r18 = importlib.import_module("hdkx-aicompiler_amd.resnet18")
     ops = float(r18.flops_per_image()) * batch          # 2 integer operations per multiply-accumulate
-    return {"metric": "resnet18_int8_bs%d_img_per_s" % batch, "value": round(batch / (ms * 1e-3), 1), "ms_per_step": round(ms, 4),
-            "int8_tops": round(ops / (ms * 1e-3) / 1e12, 1), "frac_int8_mfma_peak": round(ops / (ms * 1e-3) / 1e12 / 5000.0, 4),
-            "launches_per_step": len(net.launches), "workspace_bytes": net.workspace_bytes,
-            "logits_finite": bool(torch.isfinite(out).all().item()),
-            "parity": "bit-exact against the CPU int8 chain (tests/test_gpu_int8.py); definition is this build's own"}
+    launches = module.launches()
+    result = {"metric": "resnet18_int8_bs%d_img_per_s" % batch, "value": round(batch / (ms * 1e-3), 1), "ms_per_step": round(ms, 4),
+              "compiled_by": "C++ host layer, Compiler::Compile(quantised Relay graph, target hip)",
+              "timed_mode": "frozen constants, " + ("graph replay" if graph_ms < eager_ms else "eager"),
+              "eager_ms_per_step": round(eager_ms, 4), "hip_graph_replay_ms_per_step": round(graph_ms, 4),
+              "default_mode_ms_per_step": round(unfrozen_ms, 4),
+              "int8_tops": round(ops / (ms * 1e-3) / 1e12, 1), "frac_int8_mfma_peak": round(ops / (ms * 1e-3) / 1e12 / 5000.0, 4),
+              "launches_per_step": len(launches), "matrix_core_launches": sum("qmfma" in l for l in launches),
+              "workspace_bytes": module.workspace_bytes(),
+              "logits_finite": bool(torch.isfinite(out).all().item()),
+              "parity": "bit-exact against the CPU int8 chain (tests/test_gpu_int8.py); definition is this build's own"}
+    module.close()
+    return result
 
 
 def cpu_baseline(np, synth):

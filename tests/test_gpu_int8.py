@@ -267,13 +267,11 @@ def _quantised_model(pkg, batch, hw, config):
 
 
 def test_qresnet18_small_every_layer(pkg, orc):
-    """Batch 2, 64x64 input: every quantised tensor of the network and the logits, bit-exact."""
+    """Batch 2, 64x64 input: every quantised tensor of the network through the operator entry points of the C ABI
+    (the compiled graph runs the same launches: test_compiled_qresnet18_small_every_layer), bit-exact."""
     qr, x, model = _quantised_model(pkg, 2, 64, 5)
-    net = qr.QuantizedResNet18(model, 2, 64)
-    out = torch.empty((2, 1000), device="cuda")
-    net.run(dev(x), out)
-    want_logits, taps = orc.qresnet18(x, model, net.gap_mult)
-    # layer by layer through the operator entry points
+    gap_mult = float(np.float32(model["scale"][model["last"]]) / (np.float32(4) * np.float32(model["gap_scale_out"])))
+    want_logits, taps = orc.qresnet18(x, model, gap_mult)
     by = {L["name"]: L for L in model["layers"]}
     q = pkg.quantize_to_c16(dev(x), model["input_scale"])
     assert_bit_exact(from_c16(pkg, q, 3), taps["input"], "quantised input")
@@ -298,48 +296,12 @@ def test_qresnet18_small_every_layer(pkg, orc):
             idn = conv(cur, cin, name + ".down") if first else cur
             cur = conv(a, ch, name + ".conv2", idn)
             cin = ch
-    assert_bit_exact(host(out), want_logits, "quantised logits (plan)")
-    # the quantisation must be meaningful: logits close to the fp32 network's in the large
+    g = pkg.global_avg_pool2d_c16_i8(cur, 512, gap_mult)
+    fc = model["fc"]
+    logits = pkg.qdense(g, dev(fc["wq"]), dev(fc["bias_q"]), dev(fc["mult"]))
+    assert_bit_exact(host(logits), want_logits, "quantised logits (operator by operator)")
+    # the quantisation must be meaningful
     assert np.isfinite(want_logits).all() and np.abs(want_logits).max() > 0
-    # 24 operators, 21 launches: the three downsamples are second outputs of their block's first convolution
-    assert len(net.launches) == 21 and net.launches[1].startswith("kxc_qconv2d_c4_i8:qmfma")
-    assert sum("|qconv1x1+bias" in s for s in net.launches) == 3
-    # the plan as text and back (the two-output nodes carry four more operands): same logits
-    again = pkg.Plan.deserialize(net.plan.serialize(), 0)
-    out2 = torch.zeros_like(out)
-    again.run([dev(x)] + net.consts + [out2])
-    torch.cuda.synchronize()
-    assert_bit_exact(host(out2), want_logits, "quantised logits (plan rebuilt from its text)")
-    assert again.symbols() == net.launches
-    assert net.launches[3].startswith("kxc_qconv2d_c16_i8:qmfma")
-
-
-def test_qresnet18_batch64_images(pkg, orc):
-    """Full size (batch 64, 224x224): images 0 and 63 of the batch against the CPU chain on those images
-    alone (every operator is independent per image), plus determinism of a second run."""
-    qr, x, model = _quantised_model(pkg, 64, 224, 5)
-    net = qr.QuantizedResNet18(model, 64, 224)
-    xd = dev(x)
-    out = torch.empty((64, 1000), device="cuda")
-    net.run(xd, out)
-    first = host(out).copy()
-    net.run(xd, out)
-    assert_bit_exact(host(out), first, "second run")
-    for n in (0, 63):
-        want, _ = orc.qresnet18(x[n:n + 1], model, net.gap_mult)
-        assert_bit_exact(first[n:n + 1], want, "quantised resnet18 batch 64, image %d" % n)
-    # the same batch as two shares side by side (chains of the one plan on halves of the input and of the logits)
-    two = qr.QuantizedResNet18(model, 64, 224, shares=2)
-    assert two.shares == 2 and len(two.launches) == 2 * len(net.launches)
-    out2 = torch.zeros((64, 1000), device="cuda")
-    stream = torch.cuda.Stream()
-    two.plan.enable_graph(True)
-    with torch.cuda.stream(stream):
-        for replay in range(4):
-            out2.zero_()
-            two.run(xd, out2, stream.cuda_stream)
-            stream.synchronize()
-            assert_bit_exact(host(out2), first, "two shares of the batch, run %d" % replay)
 
 
 @pytest.mark.parametrize("m,n,k", [(64, 1000, 512), (70, 37, 1056), (33, 65, 32), (70, 37, 1040), (1, 5, 16), (9, 12, 24)])
@@ -440,7 +402,8 @@ def test_compiled_qresnet18_constants_are_read_on_every_run(pkg, orc):
 
 def test_compiled_qresnet18_batch64_images(pkg, orc):
     """BASELINE configuration 5 through Compiler::Compile: images 0 and 63 of the batch against the CPU int8 chain,
-    the hand-assembled plan of the same launches, graph replay, and two shares of the batch side by side."""
+    determinism, graph replay, the launch plan rebuilt from the text inside the module's execution-plan JSON, and two
+    shares of the batch side by side."""
     qr, x, model = _quantised_model(pkg, 64, 224, 5)
     mod, consts = _compiled(pkg, model, 64, 224)
     assert len(mod.launches()) == 21
@@ -451,6 +414,14 @@ def test_compiled_qresnet18_batch64_images(pkg, orc):
     for n in (0, 63):
         want, _ = orc.qresnet18(x[n:n + 1], model, mod.gap_mult)
         assert_bit_exact(first[n:n + 1], want, "compiled quantised resnet18 batch 64, image %d" % n)
+    import json
+    again = pkg.Plan.deserialize(json.loads(mod.plan_json())["kxc_hip"]["launch_plan"], 0)
+    assert again.num_weight_packs() == 20 and len(again.symbols()) == 21
+    out_again = torch.zeros_like(out)
+    again.run([xd] + consts + [out_again])
+    torch.cuda.synchronize()
+    assert_bit_exact(host(out_again), first, "launch plan rebuilt from its text (two-output nodes, weight packs)")
+    again.close()
     mod.freeze_constants(True)
     mod.enable_graph_replay(True)
     stream = torch.cuda.Stream()
