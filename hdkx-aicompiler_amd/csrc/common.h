@@ -18,6 +18,8 @@ namespace kxc_hip {
 std::string& LastError();
 // Per-thread current stream (DeviceAPI::SetStream semantics: thread local).
 hipStream_t& CurrentStream();
+// Counts every device allocation the library makes (kxc_hip_debug_device_allocations): call next to each hipMalloc.
+void NoteDeviceAllocation();
 
 inline int32_t Fail(int32_t code, const char* fmt, ...) {
     char buf[1024];

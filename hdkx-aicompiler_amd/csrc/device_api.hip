@@ -4,6 +4,8 @@
 // device-wide sync, attribute query that never fails).
 #include <cstring>
 
+#include <atomic>
+
 #include "common.h"
 
 namespace kxc_hip {
@@ -34,7 +36,32 @@ hipError_t Api(const char* name, F&& call) {
 }
 }  // namespace
 
+namespace {
+// Byte fill, 16 bytes per thread (whole aligned chunks as one store).
+__global__ void __launch_bounds__(256) fill_bytes_kernel(uint8_t* __restrict__ p, uint8_t v, size_t n) {
+    const size_t chunk = static_cast<size_t>(blockIdx.x) * 256 + threadIdx.x;
+    const size_t lo = chunk * 16;
+    if (lo >= n) return;
+    const size_t hi = lo + 16 < n ? lo + 16 : n;
+    if (hi - lo == 16 && (reinterpret_cast<uintptr_t>(p + lo) & 15u) == 0) {
+        const uint32_t w = 0x01010101u * v;
+        *reinterpret_cast<uint4*>(p + lo) = make_uint4(w, w, w, w);
+        return;
+    }
+    for (size_t i = lo; i < hi; ++i) p[i] = v;
+}
+std::atomic<int64_t> g_device_allocations{0};
+}  // namespace
+
+namespace kxc_hip {
+void NoteDeviceAllocation() { g_device_allocations.fetch_add(1, std::memory_order_relaxed); }
+}  // namespace kxc_hip
+
 extern "C" {
+
+int64_t kxc_hip_debug_device_allocations(void) { return g_device_allocations.load(std::memory_order_relaxed); }
+
+
 
 const char* kxc_hip_last_error(void) { return LastError().c_str(); }
 int32_t kxc_hip_abi_version(void) { return 1; }
@@ -118,6 +145,7 @@ int32_t kxc_hip_alloc(int32_t device_id, size_t nbytes, size_t alignment, void**
     *out_ptr = nullptr;
     KXC_HIP_CALL(hipSetDevice(device_id), "HIP SetDevice");
     KXC_HIP_CALL(Api("hipMalloc", [&] { return hipMalloc(out_ptr, nbytes ? nbytes : 1); }), "HIP AllocDataSpace");
+    NoteDeviceAllocation();
     return KXC_HIP_OK;
 }
 
@@ -158,6 +186,16 @@ int32_t kxc_hip_memset(void* ptr, int32_t value, size_t nbytes, int32_t device_i
     KXC_HIP_CALL(hipSetDevice(device_id), "HIP SetDevice");
     hipStream_t s = ResolveStream(stream);
     hipError_t e = hipSuccess;
+    hipStreamCaptureStatus capture = hipStreamCaptureStatusNone;
+    if (s != nullptr && hipStreamIsCapturing(s, &capture) == hipSuccess && capture == hipStreamCaptureStatusActive) {
+        // a stream that is being captured records a kernel, never a memset node (replays of memset nodes have
+        // produced wrong contents on this platform)
+        const size_t chunks = (nbytes + 15) / 16;
+        KXC_HIP_REQUIRE(chunks <= static_cast<size_t>(kMaxGridX) * 256, "kxc_hip_memset: region too large for one fill launch");
+        fill_bytes_kernel<<<NoteGrid(static_cast<int>((chunks + 255) / 256)), NoteBlock(256), NoteLds(0), s>>>(
+            static_cast<uint8_t*>(ptr), static_cast<uint8_t>(value & 0xff), nbytes);
+        return CheckLaunch("fill_bytes_kernel");
+    }
     {
         ApiScope api(s ? "hipMemsetAsync" : "hipMemset");
         DeviceScope dev(KXC_HIP_ACTIVITY_MEMSET, s ? "hipMemsetAsync" : "hipMemset", s, api.correlation());

@@ -811,6 +811,7 @@ int32_t kxc_hip_plan_finalize(kxc_hip_plan* plan, size_t workspace_bytes) {
     if (workspace_bytes > 0 && !plan->workspace) {
         KXC_HIP_CALL(hipSetDevice(plan->device_id), "HIP SetDevice");
         KXC_HIP_CALL(hipMalloc(&plan->workspace, workspace_bytes), "plan workspace allocation");
+        NoteDeviceAllocation();
     }
     plan->workspace_bytes = workspace_bytes;
     plan->finalized = true;

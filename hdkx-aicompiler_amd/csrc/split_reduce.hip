@@ -96,6 +96,7 @@ int32_t AcquireSplitScratch(hipStream_t stream, size_t bytes, SplitScratchLease*
         while (want < bytes) want *= 2;
         char* fresh = nullptr;
         KXC_HIP_CALL(hipMalloc(reinterpret_cast<void**>(&fresh), kSplitCounterBytes + want), "hipMalloc(split scratch)");
+        NoteDeviceAllocation();
         // the arrival counters in front start at zero: a fill kernel on the caller's stream, ahead of the first
         // launch that counts (under stream capture it becomes a node of the graph, which is harmless)
         split_counters_clear_kernel<<<kSplitCounters / 256, 256, 0, stream>>>(reinterpret_cast<uint32_t*>(fresh), kSplitCounters);

@@ -354,10 +354,17 @@ struct KStage {
     int chunk = 0;                       // floats of a row staged at a time
 };
 
-void CollectLoads(const PrimExpr& e, std::vector<PrimExpr>* out) {
+// Every load of `e` with whether it is evaluated unconditionally.  A load in a branch of a select, or in the right
+// operand of a short-circuit `and` / `or`, runs only when its guard lets it (a padded window reads the input only
+// inside the image); staging such a load for a whole tile of rows would read addresses the guard excludes, before
+// the buffer or past its end.
+void CollectLoads(const PrimExpr& e, bool guarded, std::vector<std::pair<PrimExpr, bool>>* out) {
     if (!e.defined()) return;
-    if (e->kind == ExprKind::kLoad) out->push_back(e);
-    for (const auto& a : e->args) CollectLoads(a, out);
+    if (e->kind == ExprKind::kLoad) out->emplace_back(e, guarded);
+    for (size_t i = 0; i < e->args.size(); ++i) {
+        const bool lazy = (e->kind == ExprKind::kSelect && i >= 1) || ((e->kind == ExprKind::kAnd || e->kind == ExprKind::kOr) && i >= 1);
+        CollectLoads(e->args[i], guarded || lazy, out);
+    }
 }
 
 bool MatchKStage(const LoopNest& data, KStage* m) {
@@ -382,12 +389,14 @@ bool MatchKStage(const LoopNest& data, KStage* m) {
     const tir::Var& rk = red.vars.back();
     const int64_t extent = red.extents.back();
     if (extent < 16) return false;
-    std::vector<PrimExpr> loads;
-    CollectLoads(upd->a->args[1], &loads);
+    std::vector<std::pair<PrimExpr, bool>> loads;
+    CollectLoads(upd->a->args[1], false, &loads);
     const tir::Var& lane_var = data.vars.back();
     const int64_t lane_extent = data.extents.back();
-    for (const auto& l : loads) {
+    for (const auto& entry : loads) {
+        const PrimExpr& l = entry.first;
         if (l->args[0].get() == init->var.get()) return false;                  // EXPR reads the output: not a plain sum
+        if (entry.second) continue;                                             // guarded: stays a lazy global load
         if (!l.dtype().is_float() || l.dtype().bits != 32) continue;
         Affine ai = AnalyzeAffine(l->args[1]);
         if (!ai.ok || !ai.coef.count(rk.get()) || ai.coef.at(rk.get()) != 1) continue;

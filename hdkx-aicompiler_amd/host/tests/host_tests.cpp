@@ -481,6 +481,21 @@ int RunCodegen() {
     Check(hip.kernels.size() == 3, "one kernel per compute stage");
     Check(hip.source.find("extern \"C\" __global__ void __launch_bounds__(256) kxc_t_s0_T_conv2d(") != std::string::npos, "kernel symbol");
     Check(hip.kernels[0].schedule == "flat", "conv stage is a flat schedule");
+    {
+        // a padded window at least 16 taps wide: the input load sits behind the padding select and must stay a lazy
+        // global load (staged for a whole tile of rows it would read before the buffer and past its end); the weight
+        // load, unguarded and contiguous along rw, may be staged
+        kxc::Var xd("x", kxc::TensorType({1, 2, 4, 40}, "float32")), wd("w", kxc::TensorType({3, 2, 1, 17}, "float32"));
+        auto wide = kxc::relay::Conv2DAttrs::Create({1, 1}, {0, 8, 0, 8}, {1, 1}, 1, 3, {1, 17}, "NCHW", "OIHW", "", "");
+        kxc::Function fw({xd, wd}, kxc::Call(Op::Get("nn_conv2d"), {xd, wd}, wide));
+        auto wide_hip = cgh.Generate(kxc::relay::LowerToTIR(kxc::relay::InferTypePass(fw)), "kxc_wide");
+        Check(wide_hip.kernels.size() == 1, "one stage for a convolution without bias");
+        const std::string& src = wide_hip.source;
+        Check(src.find("= x[rowbase") == std::string::npos, "the padded input is never staged by row base:\n" + src);
+        if (wide_hip.kernels[0].schedule == "lds_k_stage")
+            Check(src.find("= w[rowbase") != std::string::npos && src.find("? x[") != std::string::npos,
+                  "only the weights are staged; the input stays behind its select:\n" + src);
+    }
     // global average pool: contiguous rows -> LDS staged reduction
     kxc::Var x("x", kxc::TensorType({4, 32, 7, 7}, "float32"));
     kxc::Function gap({x}, kxc::Call(Op::Get("nn_global_avg_pool2d"), {x}, kxc::relay::GlobalAvgPool2DAttrs::Create()));
@@ -1101,6 +1116,13 @@ int RunGeneratedNumeric() {
         kxc::Var d("d", kxc::TensorType({600, 40}, "float32"));
         cases.push_back({"reduce_mean 600x40", kxc::Function({d}, kxc::Call(Op::Get("reduce_mean"), {d}, kxc::relay::ReduceMeanAttrs::Create({1}, 0))),
                          {{600, 40}}, 600, "lds_row_reduce"});
+    }
+    {
+        // a window 17 taps wide with padding 8: the weights are staged along rw, the padded input stays behind its select
+        kxc::Var d("d", kxc::TensorType({1, 2, 4, 40}, "float32")), w("w", kxc::TensorType({3, 2, 1, 17}, "float32"));
+        auto attrs = kxc::relay::Conv2DAttrs::Create({1, 1}, {0, 8, 0, 8}, {1, 1}, 1, 3, {1, 17}, "NCHW", "OIHW", "", "");
+        cases.push_back({"conv2d 1x17 window, padding 8", kxc::Function({d, w}, kxc::Call(Op::Get("nn_conv2d"), {d, w}, attrs)),
+                         {{1, 2, 4, 40}, {3, 2, 1, 17}}, 480, "lds_k_stage"});
     }
     for (auto& c : cases) {
         std::vector<std::vector<float>> ins;

@@ -90,8 +90,13 @@ int32_t kxc_hip_stream_sync(int32_t device_id, void* stream);
 int32_t kxc_hip_stream_wait(int32_t device_id, void* src_stream, void* dst_stream);
 
 /* Fill (the reference's only GPU test uses cudaMemsetAsync beside the device API, test/cupti_smoke_test.cpp:113-118):
- * every byte of [ptr, ptr + nbytes) = value & 0xff; stream NULL and no current stream: synchronous. */
+ * every byte of [ptr, ptr + nbytes) = value & 0xff; stream NULL and no current stream: synchronous.  On a stream
+ * that is being captured into a graph the fill is a small kernel, not a memset node. */
 int32_t kxc_hip_memset(void* ptr, int32_t value, size_t nbytes, int32_t device_id, void* stream);
+/* Number of device allocations (hipMalloc: data spaces, plan workspaces, split-reduction scratch) this library has
+ * made in the process so far.  No counterpart in the reference; lets a caller that must not allocate -- and the test
+ * of the entry point that allocates nothing -- check that a call did not. */
+int64_t kxc_hip_debug_device_allocations(void);
 
 /* Activity records for the profiling bundle: what the reference's CUPTI adapter collects for CUDA
  * (src/base/profiling.cc:537-651: runtime API calls, memcpy, memset, kernels, each with start and end), taken at

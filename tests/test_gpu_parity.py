@@ -1028,7 +1028,8 @@ def test_plan_chains_run_shares_of_a_batch_side_by_side(pkg, synth, fast_orc):
     assert_close(host(y_chain), want, what="two chains, conv / pool / conv + residual")
     # the text form keeps the chains; the rebuilt plan gives the same bits
     text = chained.serialize()
-    assert text.startswith("kxc_hip_plan 2 5 ") and text.splitlines()[0].split()[-1] == "2"
+    # header: version, arguments, workspace bytes, nodes, select lanes, weight packs
+    assert text.startswith("kxc_hip_plan 3 5 ") and text.splitlines()[0].split()[-2:] == ["2", "0"]
     again = pkg.Plan.deserialize(text, 0)
     assert again.serialize() == text
     y2 = torch.zeros_like(y_chain)
@@ -1067,9 +1068,10 @@ def test_plan_chains_run_shares_of_a_batch_side_by_side(pkg, synth, fast_orc):
     plan.close()
 
 
-def test_plan_text_version_1_still_loads(pkg, synth):
-    """The plan text gained a select_lanes field in the header and a chain field per node (version 2); a version-1
-    text -- the same plan written without them -- still loads and gives the same bits."""
+def test_plan_text_versions_1_and_2_still_load(pkg, synth):
+    """The plan text gained a select_lanes field in the header and a chain field per node (version 2), then a count
+    of weight packs in the header and a line per pack (version 3); a version-2 and a version-1 text -- the same plan
+    written without them -- still load and give the same bits."""
     n, c, h, o = 2, 8, 10, 32
     x = synth.uniform((n, c, h, h), 9300); w = synth.normal((o, c, 3, 3), 9301, 0.1); b = synth.uniform((o,), 9302, -0.1, 0.1)
     d = pkg.ConvDesc(n, c, h, h, o, 3, 3, 1, 1, 1, 1, 1, 1, pkg.CONV_BIAS | pkg.CONV_RELU)
@@ -1082,8 +1084,14 @@ def test_plan_text_version_1_still_loads(pkg, synth):
     plan.run(tensors + [y2]); torch.cuda.synchronize()
     lines = plan.serialize().splitlines()
     head = lines[0].split()
-    assert head[:2] == ["kxc_hip_plan", "2"] and head[-1] == "1"
-    old_lines = [" ".join(["kxc_hip_plan", "1"] + head[2:-1])]
+    assert head[:2] == ["kxc_hip_plan", "3"] and head[-2:] == ["1", "0"]
+    v2 = pkg.Plan.deserialize("\n".join([" ".join(["kxc_hip_plan", "2"] + head[2:-1])] + lines[1:]) + "\n", 0)
+    y0 = torch.zeros_like(y2)
+    v2.run(tensors + [y0]); torch.cuda.synchronize()
+    assert_bit_exact(host(y0), host(y2), "plan rebuilt from a version-2 text")
+    assert v2.serialize() == plan.serialize()
+    v2.close()
+    old_lines = [" ".join(["kxc_hip_plan", "1"] + head[2:-2])]
     for line in lines[1:]:
         t = line.split()
         if not t or t[0] != "node":
@@ -1102,7 +1110,7 @@ def test_plan_text_version_1_still_loads(pkg, synth):
     old = pkg.Plan.deserialize("\n".join(old_lines) + "\n", 0)
     old.run(tensors + [y1]); torch.cuda.synchronize()
     assert_bit_exact(host(y1), host(y2), "plan rebuilt from a version-1 text")
-    assert old.serialize() == plan.serialize()                   # written back as version 2
+    assert old.serialize() == plan.serialize()                   # written back as the current version
     plan.close(); old.close()
 
 

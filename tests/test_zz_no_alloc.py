@@ -41,23 +41,44 @@ def test_noalloc_conv2d_matches_the_allocating_entry_point_twice_in_a_row(pkg, s
     needs = [_needed(pkg, xs, ws, s, p) for xs, ws, s, p, _ in CASES]
     # both launches use scratch, the second less than the first
     assert needs[0] > needs[1] > 0 and needs[0] <= capacity, needs
+    allocations = pkg.lib().kxc_hip_debug_device_allocations
+    allocations.restype = C.c_int64
     for i, (xs, ws, stride, pad, with_res) in enumerate(CASES):
         x, w, b = _tensors(synth, torch, xs, ws, 7100 + 10 * i)
-        want = pkg.conv2d(x, w, b, None, stride, pad, 1, True)
-        res = torch.from_numpy(synth.uniform(tuple(want.shape), 7105 + 10 * i)).cuda() if with_res else None
-        want = pkg.conv2d(x, w, b, res, stride, pad, 1, True)
-        got = torch.full_like(want, float("nan"))
+        oshape = pkg.conv_out_shape(pkg.conv_desc(xs, ws, stride, pad, 1, 0))
+        res = torch.from_numpy(synth.uniform(tuple(oshape), 7105 + 10 * i)).cuda() if with_res else None
+        got = torch.full(tuple(oshape), float("nan"), dtype=torch.float32, device="cuda")
         print("no-alloc conv2d", xs, ws, "stride", stride, "scratch bytes", needs[i], flush=True)
-        before = torch.cuda.memory_allocated()
+        # the entry point that allocates nothing goes FIRST on each shape (a scratch buffer grown lazily for the shape
+        # would show), and the library's own count of device allocations must not move
+        before = allocations()
         pkg.conv2d(x, w, b, res, stride, pad, 1, True, out=got, no_alloc=True)
         torch.cuda.synchronize()
-        assert torch.cuda.memory_allocated() == before
+        assert allocations() == before, "the no-alloc entry point allocated device memory"
+        want = pkg.conv2d(x, w, b, res, stride, pad, 1, True)
+        torch.cuda.synchronize()
         assert torch.equal(got, want), float((got - want).abs().max())
         # and a third time on the same buffers: the array's leftovers from this very shape change nothing
         got.fill_(float("nan"))
         pkg.conv2d(x, w, b, res, stride, pad, 1, True, out=got, no_alloc=True)
         torch.cuda.synchronize()
         assert torch.equal(got, want)
+
+
+def test_allocation_counter_sees_the_allocating_entry_point(pkg, synth):
+    """The counter the test above relies on does move when the library allocates: a split shape on a fresh stream
+    makes the allocating entry point create that stream's scratch buffer."""
+    import torch
+    allocations = pkg.lib().kxc_hip_debug_device_allocations
+    allocations.restype = C.c_int64
+    xs, ws, stride, pad, _ = CASES[0]
+    x, w, b = _tensors(synth, torch, xs, ws, 7150)
+    stream = torch.cuda.Stream()
+    before = allocations()
+    with torch.cuda.stream(stream):
+        pkg.conv2d(x, w, b, None, stride, pad, 1, True)
+        stream.synchronize()
+    assert allocations() > before
 
 
 def test_noalloc_conv2d_takes_launches_without_scratch(pkg, synth):
