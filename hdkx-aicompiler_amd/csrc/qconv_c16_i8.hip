@@ -608,23 +608,75 @@ __global__ void __launch_bounds__(kBlock) pack_weights_kernel(const PackArgs a, 
 }
 
 // The weight tensors of several layers in one launch (a launch plan packs the constants of a whole network at the
-// start of a run).  Job j owns the blocks first_block[j] .. first_block[j + 1] - 1; NS == 0 marks the first-layer
-// (c4) order.
+// start of a run).  Job j owns the blocks first_block[j] .. first_block[j + 1] - 1.  A block of a job with
+// staged != 0 packs one (output block of 32 channels, chunk) unit: the unit's 32 rows of OIHW bytes -- each a
+// contiguous run of CBC*16*KHW bytes -- are read once, coalesced, into LDS, and its NS*64 slots, which are
+// contiguous in the packed tensor, are written from there (one thread per slot gathers bytes KHW apart: from
+// memory that costs a cache line per byte).  Other jobs (the first-layer order, NS == 0; windows too large for the
+// LDS array) take one thread per slot straight from memory.
 constexpr int kMaxPackJobs = 24;
+constexpr int kPackRowBytes = 800;           // room per staged row: CBC*16*KHW bytes + 4
 struct PackBatch {
     PackArgs job[kMaxPackJobs];
     int64_t slots[kMaxPackJobs];
     int32_t first_block[kMaxPackJobs + 1];
+    int32_t staged[kMaxPackJobs];
     int32_t count;
 };
 __global__ void __launch_bounds__(kBlock) pack_weights_batch_kernel(const PackBatch b) {
+    __shared__ __attribute__((aligned(16))) uint8_t raw[32 * kPackRowBytes];
     int j = 0;
     while (j + 1 < b.count && static_cast<int32_t>(blockIdx.x) >= b.first_block[j + 1]) ++j;
-    const int64_t s = static_cast<int64_t>(static_cast<int32_t>(blockIdx.x) - b.first_block[j]) * kBlock + threadIdx.x;
-    if (s >= b.slots[j]) return;
     const PackArgs& a = b.job[j];
-    if (a.NS == 0) pack_k7_c4_slot(a.w, a.wp, a.O, a.C, s);
-    else pack_slot(a, s);
+    const int32_t local = static_cast<int32_t>(blockIdx.x) - b.first_block[j];
+    if (!b.staged[j]) {
+        const int64_t s = static_cast<int64_t>(local) * kBlock + threadIdx.x;
+        if (s >= b.slots[j]) return;
+        if (a.NS == 0) pack_k7_c4_slot(a.w, a.wp, a.O, a.C, s);
+        else pack_slot(a, s);
+        return;
+    }
+    const int ob = local / a.nchunks, chunk = local - ob * a.nchunks;
+    const int c0 = chunk * a.CBC * 16;
+    const int nch = min(a.CBC * 16, a.C - c0);               // channels of this chunk that exist
+    const int row_bytes = nch * a.KHW;                        // contiguous bytes per output channel
+    const int pitch = ((a.CBC * 16 * a.KHW + 3) & ~3) + 4;    // LDS bytes per row: an odd number of words
+    const bool words = ((static_cast<int64_t>(a.C) * a.KHW) & 3) == 0 && (row_bytes & 3) == 0 && ((c0 * a.KHW) & 3) == 0 &&
+                       (reinterpret_cast<uintptr_t>(a.w) & 3u) == 0;
+    if (words) {
+        const int row_words = row_bytes >> 2;
+        for (int e = threadIdx.x; e < 32 * row_words; e += kBlock) {
+            const int r = e / row_words, k = e - r * row_words;
+            const int o = ob * 32 + r;
+            uint32_t v = 0;
+            if (o < a.O) v = reinterpret_cast<const uint32_t*>(a.w + (static_cast<int64_t>(o) * a.C + c0) * a.KHW)[k];
+            *reinterpret_cast<uint32_t*>(raw + r * pitch + 4 * k) = v;
+        }
+    } else {
+        for (int e = threadIdx.x; e < 32 * row_bytes; e += kBlock) {
+            const int r = e / row_bytes, k = e - r * row_bytes;
+            const int o = ob * 32 + r;
+            raw[r * pitch + k] = o < a.O ? static_cast<uint8_t>(a.w[(static_cast<int64_t>(o) * a.C + c0) * a.KHW + k]) : uint8_t{0};
+        }
+    }
+    __syncthreads();
+    int8_t* const out = a.wp + (static_cast<int64_t>(ob) * a.nchunks + chunk) * a.NS * 1024;
+    for (int s = threadIdx.x; s < a.NS * 64; s += kBlock) {
+        const int lane = s & 63, step = s >> 6;
+        const int r = lane & 31, h = lane >> 5;
+        const int q = 2 * step + h;
+        const int tap = q / a.CBC, cbl = q - tap * a.CBC;
+        uint32_t word[4] = {0u, 0u, 0u, 0u};
+        if (tap < a.KHW) {
+#pragma unroll
+            for (int jj = 0; jj < 16; ++jj) {
+                const int cl = cbl * 16 + jj;
+                const uint32_t v = cl < nch ? raw[r * pitch + cl * a.KHW + tap] : 0u;
+                word[jj >> 2] |= v << (8 * (jj & 3));
+            }
+        }
+        *reinterpret_cast<uint4*>(out + s * 16) = make_uint4(word[0], word[1], word[2], word[3]);
+    }
 }
 
 // ------------------------------------------------------------------ layout conversion and quantisation
@@ -1339,7 +1391,8 @@ int32_t LaunchQWeightPacks(const QPackJob* jobs, int32_t count, hipStream_t stre
             }
             b.slots[j] = static_cast<int64_t>(bytes / 16);
             b.first_block[j] = static_cast<int32_t>(blocks);
-            blocks += CeilDiv(b.slots[j], kBlock);
+            b.staged[j] = p.NS != 0 && ((p.CBC * 16 * p.KHW + 3) & ~3) + 4 <= kPackRowBytes ? 1 : 0;
+            blocks += b.staged[j] ? static_cast<int64_t>(p.oblocks) * p.nchunks : CeilDiv(b.slots[j], kBlock);
             KXC_HIP_REQUIRE(blocks < kMaxGridX, "weight pack: too many blocks");
         }
         b.first_block[b.count] = static_cast<int32_t>(blocks);

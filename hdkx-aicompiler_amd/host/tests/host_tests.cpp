@@ -1775,6 +1775,100 @@ int RunPackedFunc(const std::string& mode) {
     return 0;
 }
 
+// Non-finite inputs through a 3x3 stride-1 convolution with constant weights on the hip target.  With
+// CompileConfig::hip_winograd = false the special values spread exactly as in the CPU back end's direct sum (an Inf or
+// NaN reaches the nine outputs per channel whose window holds it, and an Inf stays an Inf of the product's sign); with
+// the default (Winograd F(2x2,3x3)) the input transform forms differences inside 4x4 patches, so a special value may
+// reach up to sixteen outputs per channel (the 2x2 blocks of the four patches that hold it), an Inf may come out as
+// NaN there, and every other output is unaffected.
+int RunNonFinite() {
+    const int64_t C = 8, H = 12, W = 12, O = 32;
+    std::vector<float> x(C * H * W), w(O * C * 9), b(O);
+    uint32_t seed = 99;
+    auto next = [&seed]() { seed = seed * 1664525u + 1013904223u; return static_cast<float>(seed >> 8) / 16777216.0f - 0.5f; };
+    for (auto& v : x) v = next();
+    for (auto& v : w) { v = next(); if (std::fabs(v) < 0.01f) v = 0.25f; }     // no zero weight: Inf * 0 would be NaN on both sides
+    for (auto& v : b) v = 0.1f * next();
+    struct Special { int64_t c, h, w; float value; };
+    const std::vector<Special> specials = {{2, 5, 6, INFINITY}, {5, 9, 2, NAN}};
+    for (const auto& sp : specials) x[(sp.c * H + sp.h) * W + sp.w] = sp.value;
+    kxc::runtime::NDArray wn({O, C, 3, 3}, "float32"), bn({O}, "float32");
+    wn.CopyFromBytes(w.data(), w.size() * sizeof(float));
+    bn.CopyFromBytes(b.data(), b.size() * sizeof(float));
+    kxc::Var xv("x", kxc::TensorType({1, C, H, W}, "float32"));
+    auto attrs = kxc::relay::Conv2DAttrs::Create({1, 1}, {1, 1, 1, 1}, {1, 1}, 1, static_cast<int>(O), {3, 3}, "NCHW", "OIHW", "", "");
+    kxc::Function f({xv}, kxc::Call(Op::Get("nn_conv2d"), {xv, kxc::Constant(wn), kxc::Constant(bn)}, attrs));
+    // the CPU back end's answer
+    std::vector<float> want(O * H * W, 0.0f);
+    {
+        g_mode = "cpu";
+        auto module = kxc::api::Compiler::Compile(f, MakeConfig());
+        module.Run({x.data(), w.data(), b.data(), want.data()});
+    }
+    g_mode = "hip";
+    kxc::DeviceAPI* api = kxc::GetDeviceAPI(kxc::kGPU);
+    kxc::Device dev(kxc::kGPU, 0), cpu(kxc::kCPU, 0);
+    auto run = [&](bool winograd, std::vector<float>* out, std::string* symbol) {
+        auto config = MakeConfig();
+        config->hip_winograd = winograd;
+        auto module = kxc::api::Compiler::Compile(f, config);
+        *symbol = module.GetKernelExecs().at(0).kernel_symbol;
+        std::vector<std::pair<void*, size_t>> host = {{x.data(), x.size() * 4}, {w.data(), w.size() * 4}, {b.data(), b.size() * 4}, {out->data(), out->size() * 4}};
+        std::vector<void*> args;
+        for (auto& h : host) {
+            void* d = api->AllocDataSpace(dev, h.second, 256);
+            api->CopyDataFromTo(cpu, h.first, dev, d, h.second);
+            args.push_back(d);
+        }
+        module.Run(args);
+        api->CopyDataFromTo(dev, args[3], cpu, out->data(), out->size() * 4);
+        for (void* d : args) api->FreeDataSpace(dev, d);
+    };
+    auto close = [](float got, float ref) { return std::fabs(got - ref) <= 1e-3f * std::max(1.0f, std::fabs(ref)); };
+    // ---- switch off: the reference's propagation, value class by value class
+    std::vector<float> direct(want.size(), 0.0f), wino(want.size(), 0.0f);
+    std::string symbol;
+    run(false, &direct, &symbol);
+    Check(symbol.find("winograd") == std::string::npos, "hip_winograd = false still chose " + symbol);
+    int64_t inf_count = 0, nan_count = 0;
+    for (size_t i = 0; i < want.size(); ++i) {
+        if (std::isnan(want[i])) { Check(std::isnan(direct[i]), "direct: NaN expected at " + std::to_string(i)); ++nan_count; }
+        else if (std::isinf(want[i])) { Check(direct[i] == want[i], "direct: Inf of the same sign expected at " + std::to_string(i)); ++inf_count; }
+        else Check(close(direct[i], want[i]), "direct: finite value differs at " + std::to_string(i));
+    }
+    Check(inf_count == 9 * O && nan_count == 9 * O, "the CPU back end spreads each special value over its nine windows per channel");
+    // ---- default: Winograd
+    run(true, &wino, &symbol);
+    Check(symbol.find("winograd") != std::string::npos, "a 3x3 stride-1 convolution with constant weights should take the Winograd kernel: " + symbol);
+    std::vector<int64_t> affected(O, 0);
+    for (int64_t o = 0; o < O; ++o)
+        for (int64_t h = 0; h < H; ++h)
+            for (int64_t ww = 0; ww < W; ++ww) {
+                const size_t i = static_cast<size_t>((o * H + h) * W + ww);
+                // the 2x2 output blocks of the patches that hold a special value: rows / columns 2*floor((p-1)/2) .. +3
+                bool in_reach = false;
+                for (const auto& sp : specials) {
+                    const int64_t h0 = 2 * ((sp.h - 1) / 2), w0 = 2 * ((sp.w - 1) / 2);
+                    in_reach = in_reach || (h >= h0 && h < h0 + 4 && ww >= w0 && ww < w0 + 4);
+                }
+                if (!in_reach) {
+                    Check(std::isfinite(want[i]) && close(wino[i], want[i]),
+                          "winograd: an output outside the patches of the special values differs at " + std::to_string(i));
+                    continue;
+                }
+                if (!std::isfinite(wino[i])) ++affected[o];
+                // where the direct sum is non-finite, so is the Winograd result (an Inf may have become NaN)
+                if (!std::isfinite(want[i])) Check(!std::isfinite(wino[i]), "winograd: a non-finite output came out finite at " + std::to_string(i));
+                else if (std::isfinite(wino[i])) Check(close(wino[i], want[i]), "winograd: finite value differs at " + std::to_string(i));
+            }
+    for (int64_t o = 0; o < O; ++o)
+        Check(affected[o] >= 18 && affected[o] <= 32, "winograd: a special value reaches at most 16 outputs per channel, got " +
+                                                        std::to_string(affected[o]) + " for two of them in channel " + std::to_string(o));
+    std::cout << "[PASS] non-finite inputs: reference propagation with hip_winograd = false, at most 16 outputs per special value with Winograd\n";
+    std::cout << "non-finite ok\n";
+    return 0;
+}
+
 int main(int argc, char** argv) {
     try {
         const std::string cmd = argc > 1 ? argv[1] : "";
@@ -1782,6 +1876,7 @@ int main(int argc, char** argv) {
         if (cmd == "device_info") return RunDeviceInfo();
         if (cmd == "adaptive") { g_mode = argc > 2 ? argv[2] : "cpu"; return RunAdaptive(argc > 3 ? argv[3] : ""); }
         if (cmd == "codegen") return RunCodegen();
+        if (cmd == "nonfinite") return RunNonFinite();
         if (cmd == "packed_func") return RunPackedFunc(argc > 2 ? argv[2] : "cpu");
         if (cmd == "generated_numeric") return RunGeneratedNumeric();
         if (cmd == "split_batch") return RunSplitBatch();

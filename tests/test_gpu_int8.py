@@ -487,3 +487,50 @@ def test_plan_weight_pack_and_layout_nodes(pkg, orc):
         bad.add_qconv_weight_pack(H.QPACK_C16, d, Buf.arg(1), Buf.arg(2))
     with pytest.raises(H.KxcHipError):
         bad.add_qconv_weight_pack(9, d, Buf.arg(1), Buf.ws(0))
+
+
+def test_plan_packs_many_weight_tensors_in_one_launch(pkg):
+    """The plan's batched pack (one launch for every weight tensor, rows staged through LDS) writes exactly the bytes
+    the per-tensor pack entry points write: full and partial channel blocks, odd block counts, 1x1 / 3x3 / 7x7
+    windows, a second-output tensor in its convolution's chunking, the first-layer order, and more tensors than one
+    batch holds."""
+    import ctypes as C
+    H = pkg
+    rng = np.random.default_rng(23)
+    Buf = H.Buf
+    # (kind, o, c, k) ; the pair packs [o, c, 1, 1] weights in the chunking of a 3x3 convolution on c channels
+    cases = [(H.QPACK_C16, 64, 40, 3), (H.QPACK_C16, 32, 10, 3), (H.QPACK_C16, 64, 72, 1), (H.QPACK_C16, 64, 3, 7),
+             (H.QPACK_C16_PAIR, 128, 64, 3), (H.QPACK_C16_PAIR, 64, 40, 3), (H.QPACK_C4, 64, 3, 7), (H.QPACK_C16, 96, 48, 3),
+             (H.QPACK_C16, 64, 16, 1), (H.QPACK_C16, 32, 17, 5)] + [(H.QPACK_C16, 32, 16 * (i + 1), 3) for i in range(18)]
+    assert len(cases) > 24
+    plan = H.Plan(len(cases))
+    weights, expect, offsets = [], [], []
+    top = 0
+    for i, (kind, o, c, k) in enumerate(cases):
+        if kind == H.QPACK_C16_PAIR:
+            w = rng.integers(-127, 128, (o, c, 1, 1), dtype=np.int8)
+            want = H.qconv2d_c16_pair_pack_weights(dev(w), k)
+            d = H.qconv_desc(1, c, 8, 8, o, k, k, 2, 1)
+        elif kind == H.QPACK_C4:
+            w = rng.integers(-127, 128, (o, c, 7, 7), dtype=np.int8)
+            want = H.qconv2d_c4_pack_weights(dev(w))
+            d = H.qconv_desc(1, c, 16, 16, o, 7, 7, 2, 3)
+        else:
+            w = rng.integers(-127, 128, (o, c, k, k), dtype=np.int8)
+            want = H.qconv2d_c16_pack_weights(dev(w))
+            d = H.qconv_desc(1, c, 8, 8, o, k, k, 1, k // 2)
+        plan.add_qconv_weight_pack(kind, d, Buf.arg(i), Buf.ws(top))
+        weights.append(dev(w)); expect.append(host(want)); offsets.append(top)
+        top += (int(want.numel()) + 255) // 256 * 256
+    plan.add_copy(16, Buf.arg(0), Buf.ws(top))          # a plan needs no node to pack, but a run must enqueue something after it
+    plan.finalize(top + 256)
+    plan.run(weights)
+    torch.cuda.synchronize()
+    base = plan.workspace_ptr()
+    for i, (want, off) in enumerate(zip(expect, offsets)):
+        got = np.empty(want.shape, np.int8)
+        pkg.lib().kxc_hip_copy(C.c_void_p(base), C.c_size_t(off), got.ctypes.data_as(C.c_void_p), C.c_size_t(0), C.c_size_t(got.nbytes),
+                               C.c_int32(1), C.c_int32(0), None)
+        torch.cuda.synchronize()
+        assert_bit_exact(got, want, "batched pack of tensor %d %s" % (i, cases[i][1:]))
+    plan.close()

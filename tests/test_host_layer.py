@@ -116,6 +116,14 @@ def test_generated_kernels_lds_schedules_bit_exact():
 
 
 @pytest.mark.gpu
+def test_non_finite_inputs_with_and_without_winograd():
+    """The stated difference of the default path: with CompileConfig::hip_winograd = false an Inf / NaN input spreads
+    exactly as in the CPU back end (nine outputs per channel, Inf stays Inf); with Winograd it reaches at most the
+    sixteen outputs of the patches that hold it, where an Inf may come out as NaN; everything else is unaffected."""
+    assert "non-finite ok" in run("nonfinite")
+
+
+@pytest.mark.gpu
 def test_packed_function_registry_hip():
     """The same registry on the GPU: allocation, copies with offsets on a stream, attributes, target.Build,
     device_info.hip.0.*, and a Relay function lowered to plan JSON and run from that JSON."""
