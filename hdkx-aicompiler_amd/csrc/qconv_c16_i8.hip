@@ -115,9 +115,8 @@ __device__ __forceinline__ void init_acc_with_bias(intx16 (&acc)[RO], const int3
     for (int i = 0; i < RO; ++i)
 #pragma unroll
         for (int j = 0; j < 4; ++j) {
-            const int o = (ob0 + i) * 32 + 8 * j + 4 * half;
             int4 b = make_int4(0, 0, 0, 0);
-            if (has_bias) b = *reinterpret_cast<const int4*>(bias + (o < O ? o : 0));
+            if (has_bias) b = *reinterpret_cast<const int4*>(bias + (ob0 + i) * 32 + 8 * j + 4 * half);
             acc[i][4 * j + 0] = b.x; acc[i][4 * j + 1] = b.y; acc[i][4 * j + 2] = b.z; acc[i][4 * j + 3] = b.w;
         }
 }
@@ -147,8 +146,8 @@ __device__ __forceinline__ void epilogue_c16(const intx16 (&acc)[RP][RO], const 
     for (int i = 0; i < RO; ++i)
 #pragma unroll
         for (int j = 0; j < 4; ++j) {
-            const int o = (ob0 + i) * 32 + 8 * j + 4 * half;
-            mv[i][j] = *reinterpret_cast<const float4*>(a.mult + (o < a.O ? o : 0));
+            // (output channels are a multiple of 32: every block is whole)
+            mv[i][j] = *reinterpret_cast<const float4*>(a.mult + (ob0 + i) * 32 + 8 * j + 4 * half);
         }
     // residual words, brought from "16 consecutive channels per lane" to the accumulators' channel groups
     uint32_t resw[RP][RO][4];
@@ -406,6 +405,288 @@ __global__ void __launch_bounds__(64 * WP) __attribute__((amdgpu_waves_per_eu(2)
         QArgs second = a;
         second.mult = a.mult2; second.res = nullptr; second.y = a.y2;
         second.flags = 0u;      // (its bias is in the accumulators already; no residual, no ReLU)
+        epilogue_c16<RO, RP>(acc2, second, ypix, ob0, half);
+    }
+}
+
+// ------------------------------------------------------------------------------------------------
+// The same convolution with the staged patch on a row pitch of P positions, P a power of two fixed at compile time
+// (16, 32 or 64, the smallest that holds a padded row), and with the reduction optionally split over KS groups of
+// waves inside the workgroup.
+//  * A 64-lane LDS-direct load covers 64 / P whole rows, so a position's (row, column) is a shift and a mask of the
+//    lane number instead of a division by the padded width, and for P = 64 the row -- hence the image, the input row
+//    and its validity -- is uniform: scalar arithmetic, two vector instructions per load.  Every tap's LDS offset
+//    (rh * P + rw) * 16 is an immediate of the ds_read, with the lane half's channel-block plane folded into the
+//    lane's base address once; bias and multipliers need no clamped addresses (output channels are a multiple of 32).
+//  * KS: vector-memory loads complete in order, so a wave that consumes a weight fragment has also waited for every
+//    patch load issued before it: a wave keeps ONE chunk's patch in flight however many buffers it has, and a
+//    workgroup walks its chunks at one memory latency each (512 -> 512 channels at 7 x 7: 16 chunks, ~0.9 us each,
+//    the same 14-16 us from batch 16 to batch 64).  With KS wave groups, group g takes the chunks g, g + KS, ... of
+//    the same pixels and output channels into its own accumulators, patch buffers and weight ring -- KS chunks in
+//    flight, the chain KS times shorter -- and after the loop the groups' accumulators are added through LDS
+//    (integers: any order gives the same bits) and group 0 runs the epilogue.
+// Same tiles, accumulators, epilogue and second output as qconv_mfma_kernel; PPT = load slots per wave.
+template <int KH, int KW, int CBC, int WP, int RO, int PPT, int RP, int P, int KS, bool DS = false>
+__global__ void __launch_bounds__(64 * WP * KS) __attribute__((amdgpu_waves_per_eu(2))) qconv_rows_kernel(const QArgs a) {
+    constexpr int KHW = KH * KW;
+    constexpr int NS = (KHW * CBC + 1) / 2;          // matrix k-steps per chunk
+    constexpr int NS2 = DS ? (CBC + 1) / 2 : 0;      // ... of the second output
+    constexpr int TP = 32 * WP * RP;
+    constexpr int LOGP = P == 64 ? 6 : (P == 32 ? 5 : 4);
+    static_assert(P == 16 || P == 32 || P == 64, "row pitch of 16, 32 or 64 positions");
+    static_assert(KS == 1 || KS == 2 || KS == 4, "one, two or four wave groups");
+
+    extern __shared__ __attribute__((aligned(16))) char lds[];
+    const int tid = threadIdx.x;
+    const int lane = tid & 63;
+    const int wave_all = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int group = KS == 1 ? 0 : wave_all / WP;   // reduction group of this wave
+    const int wave = KS == 1 ? wave_all : wave_all - group * WP;
+    const int half = lane >> 5;
+    const int r = lane & 31;
+
+    const int plane = a.chs * 16;                    // LDS bytes per channel-block plane
+    const int buf_bytes = CBC * plane;
+    const bool two_buffers = a.nchunks > KS;         // a group with a single chunk needs one
+    char* const buf0 = lds + group * buf_bytes * (two_buffers ? 2 : 1);
+    char* const buf1 = buf0 + buf_bytes;
+
+    const int tile = (blockIdx.x & 7) * a.tiles_per_xcd + (blockIdx.x >> 3);
+    if (tile >= a.num_tiles || static_cast<int>(blockIdx.x >> 3) >= a.tiles_per_xcd) return;
+    const int p_tile = fast_div(tile, a.div_otiles), o_tile = tile - p_tile * a.o_tiles;
+    const int m0 = p_tile * TP;
+    const int ob0 = o_tile * RO;
+
+    const int m_last = min(m0 + TP, a.M) - 1;
+    int qmin, qlast;
+    {
+        const int n = fast_div(m0, a.div_ohw), rem = m0 - n * a.OHW;
+        qmin = n * a.Hp + fast_div(rem, a.div_ow) * a.sh;
+        const int n2 = fast_div(m_last, a.div_ohw), rem2 = m_last - n2 * a.OHW;
+        qlast = n2 * a.Hp + fast_div(rem2, a.div_ow) * a.sh + (KH - 1);
+    }
+    const int nslots = ((qlast - qmin + 1) * P + 63) >> 6;       // 64-position load slots per plane (<= chs / 64)
+    const uint32_t plane_bytes = static_cast<uint32_t>(a.H) * a.W * 16u;
+
+    const __amdgpu_buffer_rsrc_t xr = make_rsrc(a.x, a.x_bytes);
+    const __amdgpu_buffer_rsrc_t wr = make_rsrc(a.wp, a.w_bytes);
+
+    // slot s holds rows s * (64 / P) ...; lane -> (row within the slot, column)
+    const int col = lane & (P - 1);
+    const int iw = col - a.pw;
+    const bool col_ok = iw >= 0 && iw < a.W;
+    uint32_t goff[PPT];
+#pragma unroll
+    for (int i = 0; i < PPT; ++i) {
+        const int slot = wave + i * WP;
+        const int Q = qmin + ((slot << 6) >> LOGP) + (lane >> LOGP);
+        const int n = fast_div(Q, a.div_hp), ih = Q - n * a.Hp - a.ph;
+        const bool ok = col_ok && Q <= qlast && n < a.N && ih >= 0 && ih < a.H;
+        goff[i] = ok ? (static_cast<uint32_t>(n) * a.CB * a.H * a.W + static_cast<uint32_t>(ih * a.W + iw)) * 16u : kOob;
+    }
+
+    int xbase[RP];
+    int ypix[RP];
+#pragma unroll
+    for (int j = 0; j < RP; ++j) {
+        const int m = m0 + (wave * RP + j) * 32 + r;
+        const int mc = min(m, a.M - 1);
+        const int n = fast_div(mc, a.div_ohw), rem = mc - n * a.OHW;
+        const int oh = fast_div(rem, a.div_ow), ow = rem - oh * a.OW;
+        xbase[j] = (((n * a.Hp + oh * a.sh - qmin) << LOGP) + ow * a.sw) * 16;
+        if (CBC > 1) xbase[j] += half * plane;
+        ypix[j] = (m < a.M) ? n * (a.O >> 4) * a.OHW + rem : -1;
+    }
+
+    // accumulators start at the bias (group 0) or at zero (the other groups)
+    intx16 acc[RP][RO];
+    {
+        const bool has_bias = (a.flags & KXC_HIP_CONV_BIAS) != 0 && group == 0;
+#pragma unroll
+        for (int i = 0; i < RO; ++i)
+#pragma unroll
+            for (int g = 0; g < 4; ++g) {
+                int4 b = make_int4(0, 0, 0, 0);
+                if (has_bias) b = *reinterpret_cast<const int4*>(a.bias + (ob0 + i) * 32 + 8 * g + 4 * half);
+#pragma unroll
+                for (int j = 0; j < RP; ++j) { acc[j][i][4 * g + 0] = b.x; acc[j][i][4 * g + 1] = b.y; acc[j][i][4 * g + 2] = b.z; acc[j][i][4 * g + 3] = b.w; }
+            }
+    }
+
+    auto issue_loads = [&](int chunk, char* buf) {
+#pragma unroll
+        for (int cl = 0; cl < CBC; ++cl) {
+            const int cb = chunk * CBC + cl;
+            if (cb < a.CB) {
+                const uint32_t soff = static_cast<uint32_t>(cb) * plane_bytes;
+#pragma unroll
+                for (int i = 0; i < PPT; ++i) {
+                    const int slot = wave + i * WP;
+                    if (slot < nslots)
+                        load16_to_lds(xr, (lds_ptr_t)(buf + cl * plane + slot * 1024), goff[i], soff);
+                }
+            }   // a missing channel block keeps stale bytes; its packed weights are zero and integers have no NaN
+        }
+        __builtin_amdgcn_sched_barrier(0);
+        asm volatile("" ::: "memory");      // the weight loads below stay behind these in program order
+    };
+
+    // weight ring: linear step t = chunk * NS + step of THIS group's chunks (group, group + KS, ...); the entry D
+    // steps ahead of step s belongs to the same chunk or to the group's next one
+    constexpr int D = (NS % 3 == 0) ? 3 : (NS % 5 == 0 ? 5 : (NS % 2 == 0 ? 2 : 1));
+    static_assert(NS % D == 0, "the weight ring must divide the k-steps of a chunk");
+    const uint32_t total_steps = static_cast<uint32_t>(a.nchunks) * NS;
+    uint32_t wvoff[RO];
+#pragma unroll
+    for (int i = 0; i < RO; ++i) wvoff[i] = static_cast<uint32_t>(ob0 + i) * total_steps * 1024u + static_cast<uint32_t>(lane) * 16u;
+    auto load_a = [&](int i, uint32_t t) -> intx4 {
+        const uint32_t tc = t < total_steps ? t : total_steps - 1u;
+        return __builtin_amdgcn_raw_buffer_load_b128(wr, wvoff[i], tc * 1024u, 0);
+    };
+    intx4 ring[D][RO];
+    const __amdgpu_buffer_rsrc_t wr2 = make_rsrc(DS ? a.wp2 : a.wp, DS ? a.w2_bytes : 0u);
+    intx16 acc2[DS ? RP : 1][DS ? RO : 1];
+    if constexpr (DS) {
+        const bool has_bias2 = a.bias2 != nullptr && group == 0;
+#pragma unroll
+        for (int i = 0; i < RO; ++i)
+#pragma unroll
+            for (int g = 0; g < 4; ++g) {
+                int4 b = make_int4(0, 0, 0, 0);
+                if (has_bias2) b = *reinterpret_cast<const int4*>(a.bias2 + (ob0 + i) * 32 + 8 * g + 4 * half);
+#pragma unroll
+                for (int j = 0; j < RP; ++j) { acc2[j][i][4 * g + 0] = b.x; acc2[j][i][4 * g + 1] = b.y; acc2[j][i][4 * g + 2] = b.z; acc2[j][i][4 * g + 3] = b.w; }
+            }
+    }
+
+    // every group runs the same number of rounds (a group without a chunk in the last round only keeps the barriers)
+    const int rounds = (a.nchunks + KS - 1) / KS;
+    if (group < a.nchunks) issue_loads(group, buf0);
+#pragma unroll
+    for (int d = 0; d < D; ++d)
+#pragma unroll
+        for (int i = 0; i < RO; ++i) ring[d][i] = load_a(i, static_cast<uint32_t>(group) * NS + d);
+    asm volatile("s_waitcnt vmcnt(%0)" ::"n"(D * RO) : "memory");     // the patch has landed, the ring may still fly
+    __syncthreads();
+
+    for (int round = 0; round < rounds; ++round) {
+        const int chunk = round * KS + group;
+        const char* buf = (round & 1) ? buf1 : buf0;
+        const bool live = chunk < a.nchunks;
+        intx4 a2[DS ? NS2 : 1][RO];
+        if constexpr (DS) {
+#pragma unroll
+            for (int s2 = 0; s2 < NS2; ++s2)
+#pragma unroll
+                for (int i = 0; i < RO; ++i)
+                    a2[s2][i] = __builtin_amdgcn_raw_buffer_load_b128(
+                        live ? wr2 : make_rsrc(a.wp, 0u),
+                        (static_cast<uint32_t>(ob0 + i) * static_cast<uint32_t>(a.nchunks) * NS2 + static_cast<uint32_t>(chunk) * NS2 + s2) * 1024u +
+                            static_cast<uint32_t>(lane) * 16u, 0, 0);
+            __builtin_amdgcn_sched_barrier(0);
+            asm volatile("" ::: "memory");      // ahead of the next patch's loads in program order
+        }
+        if (chunk + KS < a.nchunks) issue_loads(chunk + KS, (round & 1) ? buf0 : buf1);
+        if (live) {
+            // this chunk's operand base per pixel block; the tap offsets below are compile-time constants
+            const char* xb[RP];
+#pragma unroll
+            for (int j = 0; j < RP; ++j) xb[j] = buf + xbase[j];
+            auto tap_imm = [](int tap) constexpr {
+                const int t = tap < KHW ? tap : KHW - 1;
+                return ((t / KW) * P + (t % KW)) * 16;
+            };
+            auto fetch_b = [&](int step, intx4 (&b)[RP]) {
+                if constexpr (CBC == 1) {
+                    const int off = half ? tap_imm(2 * step + 1) : tap_imm(2 * step);
+#pragma unroll
+                    for (int j = 0; j < RP; ++j) b[j] = *reinterpret_cast<const intx4*>(xb[j] + off);
+                } else {
+                    constexpr int H2 = CBC / 2;
+                    const int pl = 2 * (step % H2) * plane;          // 0 when a chunk is two channel blocks
+#pragma unroll
+                    for (int j = 0; j < RP; ++j) b[j] = *reinterpret_cast<const intx4*>(xb[j] + pl + tap_imm(step / H2));
+                }
+            };
+            const uint32_t t0 = static_cast<uint32_t>(chunk) * NS;
+            intx4 bcur[RP], bnext[RP];
+            fetch_b(0, bcur);
+#pragma unroll
+            for (int step = 0; step < NS; ++step) {
+                if (step + 1 < NS) fetch_b(step + 1, bnext);
+#pragma unroll
+                for (int j = 0; j < RP; ++j)
+#pragma unroll
+                    for (int i = 0; i < RO; ++i)
+                        acc[j][i] = __builtin_amdgcn_mfma_i32_32x32x32_i8(ring[step % D][i], bcur[j], acc[j][i], 0, 0, 0);
+                // the ring entry D steps on: in this chunk, or in the group's next one (KS chunks further)
+                const uint32_t tn = step + D < NS ? t0 + step + D : t0 + static_cast<uint32_t>(KS) * NS + (step + D - NS);
+#pragma unroll
+                for (int i = 0; i < RO; ++i) ring[step % D][i] = load_a(i, tn);
+                if (step + 1 < NS) {
+#pragma unroll
+                    for (int j = 0; j < RP; ++j) bcur[j] = bnext[j];
+                }
+            }
+            if constexpr (DS) {
+#pragma unroll
+                for (int s2 = 0; s2 < NS2; ++s2) {
+                    const int off = a.ds_off + (CBC > 1 ? 2 * s2 * plane : 0);
+#pragma unroll
+                    for (int j = 0; j < RP; ++j) {
+                        const intx4 b2 = *reinterpret_cast<const intx4*>(xb[j] + off);
+#pragma unroll
+                        for (int i = 0; i < RO; ++i) acc2[j][i] = __builtin_amdgcn_mfma_i32_32x32x32_i8(a2[s2][i], b2, acc2[j][i], 0, 0, 0);
+                    }
+                }
+            }
+        }
+        // every load older than the ring refills just issued has completed: that includes the next patch.  (A group
+        // that was not live this round issued no refill; its next patch, if any, does not exist either.)
+        if (live) asm volatile("s_waitcnt vmcnt(%0)" ::"n"(D * RO) : "memory");
+        else asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+        __syncthreads();
+    }
+
+    if constexpr (KS > 1) {
+        // groups 1 .. KS-1 hand their accumulators to group 0 through LDS (the patches are done with: the last round
+        // ended with a barrier): [group - 1][wave][block][register][lane], 256 bytes per register and wave
+        constexpr int NACC = RP * RO * (DS ? 2 : 1);
+        int* const xch = reinterpret_cast<int*>(lds);
+        if (group > 0) {
+            int* const mine = xch + ((group - 1) * WP + wave) * NACC * 16 * 64 + lane;
+#pragma unroll
+            for (int j = 0; j < RP; ++j)
+#pragma unroll
+                for (int i = 0; i < RO; ++i)
+#pragma unroll
+                    for (int e = 0; e < 16; ++e) {
+                        mine[((j * RO + i) * 16 + e) * 64] = acc[j][i][e];
+                        if constexpr (DS) mine[(((RP * RO) + j * RO + i) * 16 + e) * 64] = acc2[j][i][e];
+                    }
+        }
+        __syncthreads();
+        if (group > 0) return;
+#pragma unroll
+        for (int g = 1; g < KS; ++g) {
+            const int* const theirs = xch + ((g - 1) * WP + wave) * NACC * 16 * 64 + lane;
+#pragma unroll
+            for (int j = 0; j < RP; ++j)
+#pragma unroll
+                for (int i = 0; i < RO; ++i)
+#pragma unroll
+                    for (int e = 0; e < 16; ++e) {
+                        acc[j][i][e] += theirs[((j * RO + i) * 16 + e) * 64];
+                        if constexpr (DS) acc2[j][i][e] += theirs[(((RP * RO) + j * RO + i) * 16 + e) * 64];
+                    }
+        }
+    }
+
+    epilogue_c16<RO, RP>(acc, a, ypix, ob0, half);
+    if constexpr (DS) {
+        QArgs second = a;
+        second.mult = a.mult2; second.res = nullptr; second.y = a.y2;
+        second.flags = 0u;
         epilogue_c16<RO, RP>(acc2, second, ypix, ob0, half);
     }
 }
@@ -886,6 +1167,37 @@ const QVariant kQVariants[] = {
     KXC_QV2(3, 3, 2, 2, 1, 8, 2, 3),
 };
 
+// The same tiles on a compile-time row pitch (qconv_rows_kernel): chosen in place of the variant above with the same
+// (window, chunk, waves, blocks per wave) when a padded row fits 64 positions.  p = positions per LDS row, ks = wave
+// groups that split the input channels inside the workgroup.
+struct QRowVariant {
+    const char* name;
+    int kh, kw, cbc, wp, ro, ppt, rp, p, ks;
+    void (*kernel)(const QArgs);
+    void (*ds_kernel)(const QArgs);
+};
+#define KXC_QR(KH, KW, CBC, WP, RO, PPT, RP, P, KS)                                                                \
+    { "qrows_k" #KH "x" #KW "_cb" #CBC "_p" #WP "x" #RP "_o" #RO "_w" #P "_ks" #KS, KH, KW, CBC, WP, RO, PPT, RP, P, KS,   \
+      qconv_rows_kernel<KH, KW, CBC, WP, RO, PPT, RP, P, KS>, nullptr }
+#define KXC_QR_DS(KH, KW, CBC, WP, RO, PPT, RP, P, KS)                                                             \
+    { "qrows_k" #KH "x" #KW "_cb" #CBC "_p" #WP "x" #RP "_o" #RO "_w" #P "_ks" #KS, KH, KW, CBC, WP, RO, PPT, RP, P, KS,   \
+      qconv_rows_kernel<KH, KW, CBC, WP, RO, PPT, RP, P, KS>, qconv_rows_kernel<KH, KW, CBC, WP, RO, PPT, RP, P, KS, true> }
+#define KXC_QR_PITCHES(M, KH, KW, CBC, WP, RO, PPT, RP, KS)                                                        \
+    M(KH, KW, CBC, WP, RO, PPT, RP, 64, KS), M(KH, KW, CBC, WP, RO, PPT, RP, 32, KS), M(KH, KW, CBC, WP, RO, PPT, RP, 16, KS)
+const QRowVariant kQRowVariants[] = {
+    KXC_QR_PITCHES(KXC_QR_DS, 3, 3, 2, 4, 2, 4, 1, 1),
+    KXC_QR_PITCHES(KXC_QR_DS, 3, 3, 2, 4, 1, 4, 1, 1),
+    KXC_QR_PITCHES(KXC_QR_DS, 3, 3, 2, 2, 1, 8, 1, 1),
+    KXC_QR_PITCHES(KXC_QR, 3, 3, 2, 4, 2, 4, 2, 1),
+    KXC_QR_PITCHES(KXC_QR, 3, 3, 2, 4, 1, 4, 2, 1),
+    KXC_QR_PITCHES(KXC_QR, 3, 3, 2, 2, 2, 8, 2, 1),
+    KXC_QR_PITCHES(KXC_QR, 3, 3, 2, 2, 1, 8, 2, 1),
+    // the input channels split over two or four wave groups (small maps with long reductions)
+    KXC_QR_DS(3, 3, 2, 4, 2, 4, 1, 32, 2), KXC_QR_DS(3, 3, 2, 4, 2, 4, 1, 16, 2),
+    KXC_QR_DS(3, 3, 2, 2, 1, 8, 1, 16, 2), KXC_QR_DS(3, 3, 2, 2, 1, 8, 1, 16, 4),
+    KXC_QR(3, 3, 2, 2, 1, 8, 2, 16, 2), KXC_QR(3, 3, 2, 2, 1, 8, 2, 16, 4), KXC_QR(3, 3, 2, 2, 1, 8, 2, 32, 2),
+};
+
 // Channel blocks (of 16 channels) per LDS chunk.  Larger chunks (64 or 128 channels) were measured on the ResNet-18
 // layers at batch 64 and were slower everywhere (512 -> 512 channels at 7 x 7: 14.3 -> 15-20 us; 256 -> 512 with
 // stride 2: 11 -> 23 us): with few chunks the first, large patch load is exposed and nothing overlaps it.
@@ -901,6 +1213,11 @@ struct QLaunch {
     QArgs args;
     int grid = 0;
     size_t lds_bytes = 0;
+    // what is launched: the variant's kernels, or those of the row-pitch variant that replaced it
+    const char* name = "";
+    void (*kernel)(const QArgs) = nullptr;
+    void (*ds_kernel)(const QArgs) = nullptr;
+    int threads = 0;
 };
 
 // Largest number of patch rows any pixel tile of TP pixels touches.
@@ -927,6 +1244,7 @@ int32_t Prepare(const kxc_hip_qconv2d_desc* d, QLaunch* L, const char* who) {
     thread_local std::vector<Entry> cache;
     if (const char* f = std::getenv("KXC_HIP_QCONV_VARIANT"))
         if (*f) return PrepareUncached(d, L, who);          // forced variants are not cached
+    if (std::getenv("KXC_HIP_QCONV_ROWS") || std::getenv("KXC_HIP_QCONV_KS")) return PrepareUncached(d, L, who);
     for (const Entry& e : cache)
         if (std::memcmp(&e.desc, d, sizeof(*d)) == 0) { *L = e.launch; return KXC_HIP_OK; }
     if (int32_t rc = PrepareUncached(d, L, who)) return rc;
@@ -1015,8 +1333,42 @@ int32_t PrepareUncached(const kxc_hip_qconv2d_desc* d, QLaunch* L, const char* w
     a.div_ow = MakeFastDiv(a.OW); a.div_otiles = MakeFastDiv(a.o_tiles);
     L->grid = a.tiles_per_xcd * 8;
     L->v = best;
+    L->name = best->name; L->kernel = best->kernel; L->ds_kernel = best->ds_kernel; L->threads = 64 * best->wp;
     const int NS = (best->kh * best->kw * cbc + 1) / 2;
     a.w_bytes = static_cast<uint32_t>(static_cast<int64_t>(a.O / 32) * a.nchunks * NS * 1024);
+    // the same tile on a compile-time row pitch when a padded row fits 64 positions (KXC_HIP_QCONV_ROWS=0: never)
+    const char* rows_env = std::getenv("KXC_HIP_QCONV_ROWS");
+    const int pitch = a.Wp <= 16 ? 16 : a.Wp <= 32 ? 32 : a.Wp <= 64 ? 64 : 0;
+    // Wave groups over the input channels: a launch whose workgroups leave SIMDs idle while each walks a long chain
+    // of chunks (KXC_HIP_QCONV_KS forces 1, 2 or 4 where a variant exists).
+    int want_ks = 1;
+    {
+        const int64_t waves = static_cast<int64_t>(a.num_tiles) * best->wp * SelectLanes();
+        if (a.nchunks >= 8 && waves <= 2 * 1024) want_ks = a.nchunks >= 16 && waves <= 1024 + 512 ? 4 : 2;
+        if (const char* e = std::getenv("KXC_HIP_QCONV_KS")) want_ks = std::atoi(e);
+    }
+    if (pitch != 0 && !(rows_env && rows_env[0] == '0')) {
+        for (int ks = want_ks; ks >= 1 && std::strncmp(L->name, "qrows", 5) != 0; ks >>= 1) {
+            for (const QRowVariant& rv : kQRowVariants) {
+                if (rv.kh != best->kh || rv.kw != best->kw || rv.cbc != cbc || rv.wp != best->wp || rv.ro != best->ro ||
+                    rv.rp != best->rp || rv.p != pitch || rv.ks != ks)
+                    continue;
+                if (best->ds_kernel != nullptr && rv.ds_kernel == nullptr) continue;      // keep the second output available
+                const int rows = MaxRows(a, rv.kh, 32 * rv.wp * rv.rp);
+                const int nslots = (rows * pitch + 63) / 64;
+                if (nslots > rv.ppt * rv.wp) continue;
+                const size_t patches = static_cast<size_t>(cbc) * nslots * 1024 * (a.nchunks > ks ? 2 : 1) * ks;
+                // the groups' accumulators are exchanged through the same LDS after the loop
+                const size_t exchange = static_cast<size_t>(ks - 1) * rv.wp * rv.rp * rv.ro * (rv.ds_kernel ? 2 : 1) * 4096;
+                const size_t lds = std::max(patches, exchange);
+                if (lds > 160 * 1024) continue;
+                a.chs = nslots * 64;
+                L->lds_bytes = lds;
+                L->name = rv.name; L->kernel = rv.kernel; L->ds_kernel = rv.ds_kernel; L->threads = 64 * rv.wp * rv.ks;
+                break;
+            }
+        }
+    }
     return KXC_HIP_OK;
 }
 
@@ -1055,7 +1407,7 @@ int32_t kxc_hip_qconv2d_c16_pack_weights(const kxc_hip_qconv2d_desc* d, const in
 const char* kxc_hip_qconv2d_c16_variant(const kxc_hip_qconv2d_desc* d) {
     QLaunch L;
     if (Prepare(d, &L, "kxc_hip_qconv2d_c16_variant") != KXC_HIP_OK) return "none";
-    return L.v ? L.v->name : "empty";
+    return L.v ? L.name : "empty";
 }
 
 int32_t kxc_hip_qconv2d_c16_i8(const kxc_hip_qconv2d_desc* d, const int8_t* x, const int8_t* w_packed,
@@ -1070,12 +1422,12 @@ int32_t kxc_hip_qconv2d_c16_i8(const kxc_hip_qconv2d_desc* d, const int8_t* x, c
     QArgs& a = L.args;
     a.x = x; a.wp = w_packed; a.bias = bias; a.mult = mult; a.res = residual; a.y = y;
     if (L.lds_bytes > 64 * 1024) {
-        KXC_HIP_CALL(hipFuncSetAttribute(reinterpret_cast<const void*>(L.v->kernel),
+        KXC_HIP_CALL(hipFuncSetAttribute(reinterpret_cast<const void*>(L.kernel),
                                          hipFuncAttributeMaxDynamicSharedMemorySize, static_cast<int>(L.lds_bytes)),
                      "hipFuncSetAttribute");
     }
-    hipLaunchKernelGGL(L.v->kernel, NoteGrid(dim3(L.grid)), NoteBlock(dim3(64 * L.v->wp)), NoteLds(L.lds_bytes), ResolveStream(stream), a);
-    return CheckLaunch(L.v->name);
+    hipLaunchKernelGGL(L.kernel, NoteGrid(dim3(L.grid)), NoteBlock(dim3(L.threads)), NoteLds(L.lds_bytes), ResolveStream(stream), a);
+    return CheckLaunch(L.name);
 }
 
 // ---- two outputs from one launch: the convolution and a 1x1 convolution with the same strides, no padding
@@ -1092,7 +1444,7 @@ int32_t kxc_hip_qconv2d_c16_pair_supported(const kxc_hip_qconv2d_desc* d) {
     QLaunch L;
     if (!PairGeometry(d)) return 0;
     if (Prepare(d, &L, "kxc_hip_qconv2d_c16_pair_supported") != KXC_HIP_OK) { LastError().clear(); return 0; }
-    return (L.v && L.v->ds_kernel) ? 1 : 0;
+    return (L.v && L.ds_kernel) ? 1 : 0;
 }
 
 int32_t kxc_hip_qconv2d_c16_pair_packed_bytes(const kxc_hip_qconv2d_desc* d, size_t* out_bytes) {
@@ -1127,7 +1479,7 @@ int32_t kxc_hip_qconv2d_c16_pair_i8(const kxc_hip_qconv2d_desc* d, const int8_t*
     const char* who = "kxc_hip_qconv2d_c16_pair_i8";
     QLaunch L;
     if (int32_t rc = Prepare(d, &L, who)) return rc;
-    KXC_HIP_REQUIRE(L.v && L.v->ds_kernel && PairGeometry(d), "%s: no kernel with a second output covers this shape", who);
+    KXC_HIP_REQUIRE(L.v && L.ds_kernel && PairGeometry(d), "%s: no kernel with a second output covers this shape", who);
     if (L.args.M == 0) return KXC_HIP_OK;
     KXC_HIP_REQUIRE(x && w_packed && mult && y && w2_packed && mult2 && y2, "%s: NULL pointer", who);
     KXC_HIP_REQUIRE(!(d->flags & KXC_HIP_CONV_BIAS) || bias, "%s: bias flag without bias", who);
@@ -1136,14 +1488,17 @@ int32_t kxc_hip_qconv2d_c16_pair_i8(const kxc_hip_qconv2d_desc* d, const int8_t*
     a.x = x; a.wp = w_packed; a.bias = bias; a.mult = mult; a.res = residual; a.y = y;
     a.wp2 = w2_packed; a.bias2 = bias2; a.mult2 = mult2; a.y2 = y2;
     a.w2_bytes = static_cast<uint32_t>(static_cast<int64_t>(a.O / 32) * a.nchunks * ((L.v->cbc + 1) / 2) * 1024);
-    a.ds_off = (d->pad_h * a.Wp + d->pad_w) * 16;
+    // the second output's tap in the staged patch: rows are Wp positions apart, or the row pitch of a qrows variant
+    int row_positions = a.Wp;
+    if (std::strncmp(L.name, "qrows", 5) == 0) row_positions = a.Wp <= 16 ? 16 : a.Wp <= 32 ? 32 : 64;
+    a.ds_off = (d->pad_h * row_positions + d->pad_w) * 16;
     if (L.lds_bytes > 64 * 1024) {
-        KXC_HIP_CALL(hipFuncSetAttribute(reinterpret_cast<const void*>(L.v->ds_kernel),
+        KXC_HIP_CALL(hipFuncSetAttribute(reinterpret_cast<const void*>(L.ds_kernel),
                                          hipFuncAttributeMaxDynamicSharedMemorySize, static_cast<int>(L.lds_bytes)),
                      "hipFuncSetAttribute");
     }
-    hipLaunchKernelGGL(L.v->ds_kernel, NoteGrid(dim3(L.grid)), NoteBlock(dim3(64 * L.v->wp)), NoteLds(L.lds_bytes), ResolveStream(stream), a);
-    return CheckLaunch(L.v->name);
+    hipLaunchKernelGGL(L.ds_kernel, NoteGrid(dim3(L.grid)), NoteBlock(dim3(L.threads)), NoteLds(L.lds_bytes), ResolveStream(stream), a);
+    return CheckLaunch(L.name);
 }
 
 int32_t kxc_hip_i8_nchw_to_c16(const int8_t* x, int8_t* y, int64_t n, int64_t c, int64_t hw, void* stream) {
