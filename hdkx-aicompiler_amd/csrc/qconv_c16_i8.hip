@@ -411,45 +411,42 @@ __global__ void __launch_bounds__(64 * WP) __attribute__((amdgpu_waves_per_eu(2)
 
 // ------------------------------------------------------------------------------------------------
 // The same convolution with the staged patch on a row pitch of P positions, P a power of two fixed at compile time
-// (16, 32 or 64, the smallest that holds a padded row), and with the reduction optionally split over KS groups of
-// waves inside the workgroup.
+// (64: padded rows of 33 to 64 positions, the 56 x 56 layers of ResNet-18).
 //  * A 64-lane LDS-direct load covers 64 / P whole rows, so a position's (row, column) is a shift and a mask of the
 //    lane number instead of a division by the padded width, and for P = 64 the row -- hence the image, the input row
 //    and its validity -- is uniform: scalar arithmetic, two vector instructions per load.  Every tap's LDS offset
 //    (rh * P + rw) * 16 is an immediate of the ds_read, with the lane half's channel-block plane folded into the
 //    lane's base address once; bias and multipliers need no clamped addresses (output channels are a multiple of 32).
-//  * KS: vector-memory loads complete in order, so a wave that consumes a weight fragment has also waited for every
-//    patch load issued before it: a wave keeps ONE chunk's patch in flight however many buffers it has, and a
-//    workgroup walks its chunks at one memory latency each (512 -> 512 channels at 7 x 7: 16 chunks, ~0.9 us each,
-//    the same 14-16 us from batch 16 to batch 64).  With KS wave groups, group g takes the chunks g, g + KS, ... of
-//    the same pixels and output channels into its own accumulators, patch buffers and weight ring -- KS chunks in
-//    flight, the chain KS times shorter -- and after the loop the groups' accumulators are added through LDS
-//    (integers: any order gives the same bits) and group 0 runs the epilogue.
+// Measured on the ResNet-18 layers at batch 64 (one process, launches captured in a graph): 14.3 against 14.7-15.5 us
+// for 64 -> 64 channels at 56 x 56, no difference for the stride-2 layer on the same input.  Pitches of 16 and 32
+// positions for the narrower layers were built and were SLOWER than the general kernel (512 -> 512 at 7 x 7: 16.6
+// against 14.1 us; rows 256 or 512 bytes apart put the same column of every row into the same LDS banks), so only
+// the 64-position pitch is instantiated.  Also measured and not kept: splitting the input channels over two or four
+// wave groups inside the workgroup (their accumulators added through LDS): 18.0-18.5 against 13.8 us for the 7 x 7
+// layer, 12.6-19.5 against 11.9 for 14 x 14; and a ring of three or four patch buffers: vector-memory loads complete
+// in order, so a wave that consumes a weight fragment has also waited for every patch load issued before it, and one
+// chunk's patch in flight per wave is all a deeper ring can hold.
 // Same tiles, accumulators, epilogue and second output as qconv_mfma_kernel; PPT = load slots per wave.
-template <int KH, int KW, int CBC, int WP, int RO, int PPT, int RP, int P, int KS, bool DS = false>
-__global__ void __launch_bounds__(64 * WP * KS) __attribute__((amdgpu_waves_per_eu(2))) qconv_rows_kernel(const QArgs a) {
+template <int KH, int KW, int CBC, int WP, int RO, int PPT, int RP, int P, bool DS = false>
+__global__ void __launch_bounds__(64 * WP) __attribute__((amdgpu_waves_per_eu(2))) qconv_rows_kernel(const QArgs a) {
     constexpr int KHW = KH * KW;
     constexpr int NS = (KHW * CBC + 1) / 2;          // matrix k-steps per chunk
     constexpr int NS2 = DS ? (CBC + 1) / 2 : 0;      // ... of the second output
     constexpr int TP = 32 * WP * RP;
     constexpr int LOGP = P == 64 ? 6 : (P == 32 ? 5 : 4);
     static_assert(P == 16 || P == 32 || P == 64, "row pitch of 16, 32 or 64 positions");
-    static_assert(KS == 1 || KS == 2 || KS == 4, "one, two or four wave groups");
 
     extern __shared__ __attribute__((aligned(16))) char lds[];
     const int tid = threadIdx.x;
     const int lane = tid & 63;
-    const int wave_all = __builtin_amdgcn_readfirstlane(tid >> 6);
-    const int group = KS == 1 ? 0 : wave_all / WP;   // reduction group of this wave
-    const int wave = KS == 1 ? wave_all : wave_all - group * WP;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int half = lane >> 5;
     const int r = lane & 31;
 
     const int plane = a.chs * 16;                    // LDS bytes per channel-block plane
     const int buf_bytes = CBC * plane;
-    const bool two_buffers = a.nchunks > KS;         // a group with a single chunk needs one
-    char* const buf0 = lds + group * buf_bytes * (two_buffers ? 2 : 1);
-    char* const buf1 = buf0 + buf_bytes;
+    char* const buf0 = lds;
+    char* const buf1 = lds + buf_bytes;              // present only when nchunks > 1
 
     const int tile = (blockIdx.x & 7) * a.tiles_per_xcd + (blockIdx.x >> 3);
     if (tile >= a.num_tiles || static_cast<int>(blockIdx.x >> 3) >= a.tiles_per_xcd) return;
@@ -498,10 +495,10 @@ __global__ void __launch_bounds__(64 * WP * KS) __attribute__((amdgpu_waves_per_
         ypix[j] = (m < a.M) ? n * (a.O >> 4) * a.OHW + rem : -1;
     }
 
-    // accumulators start at the bias (group 0) or at zero (the other groups)
+    // accumulators start at the bias
     intx16 acc[RP][RO];
     {
-        const bool has_bias = (a.flags & KXC_HIP_CONV_BIAS) != 0 && group == 0;
+        const bool has_bias = (a.flags & KXC_HIP_CONV_BIAS) != 0;
 #pragma unroll
         for (int i = 0; i < RO; ++i)
 #pragma unroll
@@ -531,8 +528,7 @@ __global__ void __launch_bounds__(64 * WP * KS) __attribute__((amdgpu_waves_per_
         asm volatile("" ::: "memory");      // the weight loads below stay behind these in program order
     };
 
-    // weight ring: linear step t = chunk * NS + step of THIS group's chunks (group, group + KS, ...); the entry D
-    // steps ahead of step s belongs to the same chunk or to the group's next one
+    // weight ring: see qconv_mfma_kernel
     constexpr int D = (NS % 3 == 0) ? 3 : (NS % 5 == 0 ? 5 : (NS % 2 == 0 ? 2 : 1));
     static_assert(NS % D == 0, "the weight ring must divide the k-steps of a chunk");
     const uint32_t total_steps = static_cast<uint32_t>(a.nchunks) * NS;
@@ -547,7 +543,7 @@ __global__ void __launch_bounds__(64 * WP * KS) __attribute__((amdgpu_waves_per_
     const __amdgpu_buffer_rsrc_t wr2 = make_rsrc(DS ? a.wp2 : a.wp, DS ? a.w2_bytes : 0u);
     intx16 acc2[DS ? RP : 1][DS ? RO : 1];
     if constexpr (DS) {
-        const bool has_bias2 = a.bias2 != nullptr && group == 0;
+        const bool has_bias2 = a.bias2 != nullptr;
 #pragma unroll
         for (int i = 0; i < RO; ++i)
 #pragma unroll
@@ -559,20 +555,16 @@ __global__ void __launch_bounds__(64 * WP * KS) __attribute__((amdgpu_waves_per_
             }
     }
 
-    // every group runs the same number of rounds (a group without a chunk in the last round only keeps the barriers)
-    const int rounds = (a.nchunks + KS - 1) / KS;
-    if (group < a.nchunks) issue_loads(group, buf0);
+    issue_loads(0, buf0);
 #pragma unroll
     for (int d = 0; d < D; ++d)
 #pragma unroll
-        for (int i = 0; i < RO; ++i) ring[d][i] = load_a(i, static_cast<uint32_t>(group) * NS + d);
+        for (int i = 0; i < RO; ++i) ring[d][i] = load_a(i, d);
     asm volatile("s_waitcnt vmcnt(%0)" ::"n"(D * RO) : "memory");     // the patch has landed, the ring may still fly
     __syncthreads();
 
-    for (int round = 0; round < rounds; ++round) {
-        const int chunk = round * KS + group;
-        const char* buf = (round & 1) ? buf1 : buf0;
-        const bool live = chunk < a.nchunks;
+    for (int chunk = 0; chunk < a.nchunks; ++chunk) {
+        const char* buf = (chunk & 1) ? buf1 : buf0;
         intx4 a2[DS ? NS2 : 1][RO];
         if constexpr (DS) {
 #pragma unroll
@@ -580,14 +572,14 @@ __global__ void __launch_bounds__(64 * WP * KS) __attribute__((amdgpu_waves_per_
 #pragma unroll
                 for (int i = 0; i < RO; ++i)
                     a2[s2][i] = __builtin_amdgcn_raw_buffer_load_b128(
-                        live ? wr2 : make_rsrc(a.wp, 0u),
+                        wr2,
                         (static_cast<uint32_t>(ob0 + i) * static_cast<uint32_t>(a.nchunks) * NS2 + static_cast<uint32_t>(chunk) * NS2 + s2) * 1024u +
                             static_cast<uint32_t>(lane) * 16u, 0, 0);
             __builtin_amdgcn_sched_barrier(0);
             asm volatile("" ::: "memory");      // ahead of the next patch's loads in program order
         }
-        if (chunk + KS < a.nchunks) issue_loads(chunk + KS, (round & 1) ? buf0 : buf1);
-        if (live) {
+        if (chunk + 1 < a.nchunks) issue_loads(chunk + 1, (chunk & 1) ? buf0 : buf1);
+        {
             // this chunk's operand base per pixel block; the tap offsets below are compile-time constants
             const char* xb[RP];
 #pragma unroll
@@ -619,10 +611,8 @@ __global__ void __launch_bounds__(64 * WP * KS) __attribute__((amdgpu_waves_per_
 #pragma unroll
                     for (int i = 0; i < RO; ++i)
                         acc[j][i] = __builtin_amdgcn_mfma_i32_32x32x32_i8(ring[step % D][i], bcur[j], acc[j][i], 0, 0, 0);
-                // the ring entry D steps on: in this chunk, or in the group's next one (KS chunks further)
-                const uint32_t tn = step + D < NS ? t0 + step + D : t0 + static_cast<uint32_t>(KS) * NS + (step + D - NS);
 #pragma unroll
-                for (int i = 0; i < RO; ++i) ring[step % D][i] = load_a(i, tn);
+                for (int i = 0; i < RO; ++i) ring[step % D][i] = load_a(i, t0 + step + D);
                 if (step + 1 < NS) {
 #pragma unroll
                     for (int j = 0; j < RP; ++j) bcur[j] = bnext[j];
@@ -641,45 +631,9 @@ __global__ void __launch_bounds__(64 * WP * KS) __attribute__((amdgpu_waves_per_
                 }
             }
         }
-        // every load older than the ring refills just issued has completed: that includes the next patch.  (A group
-        // that was not live this round issued no refill; its next patch, if any, does not exist either.)
-        if (live) asm volatile("s_waitcnt vmcnt(%0)" ::"n"(D * RO) : "memory");
-        else asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+        // every load older than the ring refills just issued has completed: that includes the next patch
+        asm volatile("s_waitcnt vmcnt(%0)" ::"n"(D * RO) : "memory");
         __syncthreads();
-    }
-
-    if constexpr (KS > 1) {
-        // groups 1 .. KS-1 hand their accumulators to group 0 through LDS (the patches are done with: the last round
-        // ended with a barrier): [group - 1][wave][block][register][lane], 256 bytes per register and wave
-        constexpr int NACC = RP * RO * (DS ? 2 : 1);
-        int* const xch = reinterpret_cast<int*>(lds);
-        if (group > 0) {
-            int* const mine = xch + ((group - 1) * WP + wave) * NACC * 16 * 64 + lane;
-#pragma unroll
-            for (int j = 0; j < RP; ++j)
-#pragma unroll
-                for (int i = 0; i < RO; ++i)
-#pragma unroll
-                    for (int e = 0; e < 16; ++e) {
-                        mine[((j * RO + i) * 16 + e) * 64] = acc[j][i][e];
-                        if constexpr (DS) mine[(((RP * RO) + j * RO + i) * 16 + e) * 64] = acc2[j][i][e];
-                    }
-        }
-        __syncthreads();
-        if (group > 0) return;
-#pragma unroll
-        for (int g = 1; g < KS; ++g) {
-            const int* const theirs = xch + ((g - 1) * WP + wave) * NACC * 16 * 64 + lane;
-#pragma unroll
-            for (int j = 0; j < RP; ++j)
-#pragma unroll
-                for (int i = 0; i < RO; ++i)
-#pragma unroll
-                    for (int e = 0; e < 16; ++e) {
-                        acc[j][i][e] += theirs[((j * RO + i) * 16 + e) * 64];
-                        if constexpr (DS) acc2[j][i][e] += theirs[(((RP * RO) + j * RO + i) * 16 + e) * 64];
-                    }
-        }
     }
 
     epilogue_c16<RO, RP>(acc, a, ypix, ob0, half);
@@ -1167,35 +1121,28 @@ const QVariant kQVariants[] = {
     KXC_QV2(3, 3, 2, 2, 1, 8, 2, 3),
 };
 
-// The same tiles on a compile-time row pitch (qconv_rows_kernel): chosen in place of the variant above with the same
-// (window, chunk, waves, blocks per wave) when a padded row fits 64 positions.  p = positions per LDS row, ks = wave
-// groups that split the input channels inside the workgroup.
+// The same tiles on a compile-time row pitch of 64 positions (qconv_rows_kernel): chosen in place of the variant above
+// with the same (window, chunk, waves, blocks per wave) for stride-1 layers whose padded rows take 33 to 64 positions.
 struct QRowVariant {
     const char* name;
-    int kh, kw, cbc, wp, ro, ppt, rp, p, ks;
+    int kh, kw, cbc, wp, ro, ppt, rp, p;
     void (*kernel)(const QArgs);
     void (*ds_kernel)(const QArgs);
 };
-#define KXC_QR(KH, KW, CBC, WP, RO, PPT, RP, P, KS)                                                                \
-    { "qrows_k" #KH "x" #KW "_cb" #CBC "_p" #WP "x" #RP "_o" #RO "_w" #P "_ks" #KS, KH, KW, CBC, WP, RO, PPT, RP, P, KS,   \
-      qconv_rows_kernel<KH, KW, CBC, WP, RO, PPT, RP, P, KS>, nullptr }
-#define KXC_QR_DS(KH, KW, CBC, WP, RO, PPT, RP, P, KS)                                                             \
-    { "qrows_k" #KH "x" #KW "_cb" #CBC "_p" #WP "x" #RP "_o" #RO "_w" #P "_ks" #KS, KH, KW, CBC, WP, RO, PPT, RP, P, KS,   \
-      qconv_rows_kernel<KH, KW, CBC, WP, RO, PPT, RP, P, KS>, qconv_rows_kernel<KH, KW, CBC, WP, RO, PPT, RP, P, KS, true> }
-#define KXC_QR_PITCHES(M, KH, KW, CBC, WP, RO, PPT, RP, KS)                                                        \
-    M(KH, KW, CBC, WP, RO, PPT, RP, 64, KS), M(KH, KW, CBC, WP, RO, PPT, RP, 32, KS), M(KH, KW, CBC, WP, RO, PPT, RP, 16, KS)
+#define KXC_QR(KH, KW, CBC, WP, RO, PPT, RP, P)                                                                    \
+    { "qrows_k" #KH "x" #KW "_cb" #CBC "_p" #WP "x" #RP "_o" #RO "_w" #P, KH, KW, CBC, WP, RO, PPT, RP, P,              \
+      qconv_rows_kernel<KH, KW, CBC, WP, RO, PPT, RP, P>, nullptr }
+#define KXC_QR_DS(KH, KW, CBC, WP, RO, PPT, RP, P)                                                                 \
+    { "qrows_k" #KH "x" #KW "_cb" #CBC "_p" #WP "x" #RP "_o" #RO "_w" #P, KH, KW, CBC, WP, RO, PPT, RP, P,              \
+      qconv_rows_kernel<KH, KW, CBC, WP, RO, PPT, RP, P>, qconv_rows_kernel<KH, KW, CBC, WP, RO, PPT, RP, P, true> }
 const QRowVariant kQRowVariants[] = {
-    KXC_QR_PITCHES(KXC_QR_DS, 3, 3, 2, 4, 2, 4, 1, 1),
-    KXC_QR_PITCHES(KXC_QR_DS, 3, 3, 2, 4, 1, 4, 1, 1),
-    KXC_QR_PITCHES(KXC_QR_DS, 3, 3, 2, 2, 1, 8, 1, 1),
-    KXC_QR_PITCHES(KXC_QR, 3, 3, 2, 4, 2, 4, 2, 1),
-    KXC_QR_PITCHES(KXC_QR, 3, 3, 2, 4, 1, 4, 2, 1),
-    KXC_QR_PITCHES(KXC_QR, 3, 3, 2, 2, 2, 8, 2, 1),
-    KXC_QR_PITCHES(KXC_QR, 3, 3, 2, 2, 1, 8, 2, 1),
-    // the input channels split over two or four wave groups (small maps with long reductions)
-    KXC_QR_DS(3, 3, 2, 4, 2, 4, 1, 32, 2), KXC_QR_DS(3, 3, 2, 4, 2, 4, 1, 16, 2),
-    KXC_QR_DS(3, 3, 2, 2, 1, 8, 1, 16, 2), KXC_QR_DS(3, 3, 2, 2, 1, 8, 1, 16, 4),
-    KXC_QR(3, 3, 2, 2, 1, 8, 2, 16, 2), KXC_QR(3, 3, 2, 2, 1, 8, 2, 16, 4), KXC_QR(3, 3, 2, 2, 1, 8, 2, 32, 2),
+    KXC_QR_DS(3, 3, 2, 4, 2, 4, 1, 64),
+    KXC_QR_DS(3, 3, 2, 4, 1, 4, 1, 64),
+    KXC_QR_DS(3, 3, 2, 2, 1, 8, 1, 64),
+    KXC_QR(3, 3, 2, 4, 2, 4, 2, 64),
+    KXC_QR(3, 3, 2, 4, 1, 4, 2, 64),
+    KXC_QR(3, 3, 2, 2, 2, 8, 2, 64),
+    KXC_QR(3, 3, 2, 2, 1, 8, 2, 64),
 };
 
 // Channel blocks (of 16 channels) per LDS chunk.  Larger chunks (64 or 128 channels) were measured on the ResNet-18
@@ -1244,7 +1191,7 @@ int32_t Prepare(const kxc_hip_qconv2d_desc* d, QLaunch* L, const char* who) {
     thread_local std::vector<Entry> cache;
     if (const char* f = std::getenv("KXC_HIP_QCONV_VARIANT"))
         if (*f) return PrepareUncached(d, L, who);          // forced variants are not cached
-    if (std::getenv("KXC_HIP_QCONV_ROWS") || std::getenv("KXC_HIP_QCONV_KS")) return PrepareUncached(d, L, who);
+    if (std::getenv("KXC_HIP_QCONV_ROWS")) return PrepareUncached(d, L, who);
     for (const Entry& e : cache)
         if (std::memcmp(&e.desc, d, sizeof(*d)) == 0) { *L = e.launch; return KXC_HIP_OK; }
     if (int32_t rc = PrepareUncached(d, L, who)) return rc;
@@ -1336,37 +1283,25 @@ int32_t PrepareUncached(const kxc_hip_qconv2d_desc* d, QLaunch* L, const char* w
     L->name = best->name; L->kernel = best->kernel; L->ds_kernel = best->ds_kernel; L->threads = 64 * best->wp;
     const int NS = (best->kh * best->kw * cbc + 1) / 2;
     a.w_bytes = static_cast<uint32_t>(static_cast<int64_t>(a.O / 32) * a.nchunks * NS * 1024);
-    // the same tile on a compile-time row pitch when a padded row fits 64 positions (KXC_HIP_QCONV_ROWS=0: never)
+    // the same tile on a compile-time row pitch for stride-1 layers whose padded rows take 33 to 64 positions
+    // (KXC_HIP_QCONV_ROWS=0: never)
     const char* rows_env = std::getenv("KXC_HIP_QCONV_ROWS");
-    const int pitch = a.Wp <= 16 ? 16 : a.Wp <= 32 ? 32 : a.Wp <= 64 ? 64 : 0;
-    // Wave groups over the input channels: a launch whose workgroups leave SIMDs idle while each walks a long chain
-    // of chunks (KXC_HIP_QCONV_KS forces 1, 2 or 4 where a variant exists).
-    int want_ks = 1;
-    {
-        const int64_t waves = static_cast<int64_t>(a.num_tiles) * best->wp * SelectLanes();
-        if (a.nchunks >= 8 && waves <= 2 * 1024) want_ks = a.nchunks >= 16 && waves <= 1024 + 512 ? 4 : 2;
-        if (const char* e = std::getenv("KXC_HIP_QCONV_KS")) want_ks = std::atoi(e);
-    }
+    const int pitch = a.Wp > 32 && a.Wp <= 64 && d->stride_h == 1 && d->stride_w == 1 ? 64 : 0;
     if (pitch != 0 && !(rows_env && rows_env[0] == '0')) {
-        for (int ks = want_ks; ks >= 1 && std::strncmp(L->name, "qrows", 5) != 0; ks >>= 1) {
-            for (const QRowVariant& rv : kQRowVariants) {
-                if (rv.kh != best->kh || rv.kw != best->kw || rv.cbc != cbc || rv.wp != best->wp || rv.ro != best->ro ||
-                    rv.rp != best->rp || rv.p != pitch || rv.ks != ks)
-                    continue;
-                if (best->ds_kernel != nullptr && rv.ds_kernel == nullptr) continue;      // keep the second output available
-                const int rows = MaxRows(a, rv.kh, 32 * rv.wp * rv.rp);
-                const int nslots = (rows * pitch + 63) / 64;
-                if (nslots > rv.ppt * rv.wp) continue;
-                const size_t patches = static_cast<size_t>(cbc) * nslots * 1024 * (a.nchunks > ks ? 2 : 1) * ks;
-                // the groups' accumulators are exchanged through the same LDS after the loop
-                const size_t exchange = static_cast<size_t>(ks - 1) * rv.wp * rv.rp * rv.ro * (rv.ds_kernel ? 2 : 1) * 4096;
-                const size_t lds = std::max(patches, exchange);
-                if (lds > 160 * 1024) continue;
-                a.chs = nslots * 64;
-                L->lds_bytes = lds;
-                L->name = rv.name; L->kernel = rv.kernel; L->ds_kernel = rv.ds_kernel; L->threads = 64 * rv.wp * rv.ks;
-                break;
-            }
+        for (const QRowVariant& rv : kQRowVariants) {
+            if (rv.kh != best->kh || rv.kw != best->kw || rv.cbc != cbc || rv.wp != best->wp || rv.ro != best->ro ||
+                rv.rp != best->rp || rv.p != pitch)
+                continue;
+            if (best->ds_kernel != nullptr && rv.ds_kernel == nullptr) continue;      // keep the second output available
+            const int rows = MaxRows(a, rv.kh, 32 * rv.wp * rv.rp);
+            const int nslots = (rows * pitch + 63) / 64;
+            if (nslots > rv.ppt * rv.wp) continue;
+            const size_t lds = static_cast<size_t>(cbc) * nslots * 1024 * (a.nchunks > 1 ? 2 : 1);
+            if (lds > 160 * 1024) continue;
+            a.chs = nslots * 64;
+            L->lds_bytes = lds;
+            L->name = rv.name; L->kernel = rv.kernel; L->ds_kernel = rv.ds_kernel; L->threads = 64 * rv.wp;
+            break;
         }
     }
     return KXC_HIP_OK;
@@ -1490,7 +1425,7 @@ int32_t kxc_hip_qconv2d_c16_pair_i8(const kxc_hip_qconv2d_desc* d, const int8_t*
     a.w2_bytes = static_cast<uint32_t>(static_cast<int64_t>(a.O / 32) * a.nchunks * ((L.v->cbc + 1) / 2) * 1024);
     // the second output's tap in the staged patch: rows are Wp positions apart, or the row pitch of a qrows variant
     int row_positions = a.Wp;
-    if (std::strncmp(L.name, "qrows", 5) == 0) row_positions = a.Wp <= 16 ? 16 : a.Wp <= 32 ? 32 : 64;
+    if (std::strncmp(L.name, "qrows", 5) == 0) row_positions = 64;
     a.ds_off = (d->pad_h * row_positions + d->pad_w) * 16;
     if (L.lds_bytes > 64 * 1024) {
         KXC_HIP_CALL(hipFuncSetAttribute(reinterpret_cast<const void*>(L.ds_kernel),

@@ -98,34 +98,35 @@ def test_qconv_c16_against_cpu(pkg, orc, shape, residual):
 
 
 def test_qconv_c16_row_pitch_kernels_equal_the_general_kernel(pkg, orc, monkeypatch):
-    """Shapes whose padded rows fit 64 positions run on a compile-time row pitch (kernel names qrows_*); with
-    KXC_HIP_QCONV_ROWS=0 the same shapes take the general kernel.  Same bytes either way, and both against the CPU."""
+    """Stride-1 3x3 layers whose padded rows take 33 to 64 positions run on a compile-time row pitch (kernel names
+    qrows_*); with KXC_HIP_QCONV_ROWS=0 the same shapes take the general kernel.  Same bytes either way, and both
+    against the CPU: full and ragged tiles, partial channel blocks, tiles that cross image boundaries."""
     rng = np.random.default_rng(31)
-    for (n, c, h, w, o, k, s, p) in [(2, 64, 56, 56, 64, 3, 1, 1), (3, 128, 28, 28, 128, 3, 1, 1), (5, 256, 14, 14, 256, 3, 1, 1),
-                                     (7, 512, 7, 7, 512, 3, 1, 1), (2, 64, 56, 56, 128, 3, 2, 1), (2, 48, 9, 33, 96, 3, 2, 1),
-                                     (1, 72, 12, 12, 64, 1, 1, 0), (1, 40, 5, 62, 32, 3, 1, 1), (2, 32, 6, 63, 64, 3, 1, 1)]:
+    for (n, c, h, w, o, k, s, p, rows_expected) in [(2, 64, 56, 56, 64, 3, 1, 1, True), (3, 40, 5, 62, 32, 3, 1, 1, True),
+                                                    (2, 32, 6, 61, 64, 3, 1, 1, True), (5, 64, 9, 33, 96, 3, 1, 1, True),
+                                                    (64, 64, 56, 56, 64, 3, 1, 1, True), (2, 64, 56, 56, 128, 3, 2, 1, False),
+                                                    (3, 128, 28, 28, 128, 3, 1, 1, False), (2, 32, 6, 63, 64, 3, 1, 1, False)]:
         x = rng.integers(-128, 128, (n, c, h, w), dtype=np.int8)
         wq = rng.integers(-127, 128, (o, c, k, k), dtype=np.int8)
         bias = rng.integers(-20000, 20000, (o,), dtype=np.int32)
         mult = rng.uniform(0.5, 2.0, (o,)).astype(np.float32) * np.float32(1.0 / (8.0 * np.sqrt(c * k * k) * 64))
         oh, ow = (h + 2 * p - k) // s + 1, (w + 2 * p - k) // s + 1
         res = rng.integers(-128, 128, (n, o, oh, ow), dtype=np.int8)
-        want = orc.qconv(x, wq, bias, mult, s, p, res, 0.41, True)
         packed = pkg.qconv2d_c16_pack_weights(dev(wq))
         d = pkg.qconv_desc(n, c, h, w, o, k, k, s, p)
         args = (to_c16(pkg, x), c, packed, wq.shape, dev(bias), dev(mult), to_c16(pkg, res), 0.41, s, p, True)
         monkeypatch.delenv("KXC_HIP_QCONV_ROWS", raising=False)
         name = pkg.qconv2d_c16_variant(d)
-        # (a tile of the stride-2 33-wide shape spans more rows than its variant has load slots: it stays general)
-        if (h, w) != (9, 33):
-            assert name.startswith("qrows_") == (w + 2 * p <= 64), (name, w, p)
+        assert name.startswith("qrows_") == rows_expected, (name, w, p)
         rows = pkg.qconv2d_c16(*args)
         monkeypatch.setenv("KXC_HIP_QCONV_ROWS", "0")
         assert pkg.qconv2d_c16_variant(d).startswith("qmfma_")
         general = pkg.qconv2d_c16(*args)
         monkeypatch.delenv("KXC_HIP_QCONV_ROWS")
         assert_bit_exact(host(rows), host(general), "row-pitch kernel against the general kernel %s" % ((n, c, h, w, o, k, s, p),))
-        assert_bit_exact(from_c16(pkg, rows, o), want, "row-pitch kernel against the CPU %s" % ((n, c, h, w, o, k, s, p),))
+        if n <= 5:
+            want = orc.qconv(x, wq, bias, mult, s, p, res, 0.41, True)
+            assert_bit_exact(from_c16(pkg, rows, o), want, "row-pitch kernel against the CPU %s" % ((n, c, h, w, o, k, s, p),))
 
 
 QPAIR_SHAPES = [
