@@ -83,6 +83,8 @@ struct ConvArgs {
     // of every other row.  plane = ceil(rows/2) * Wp/2 floats for the tallest tile of the launch; needs Hp, Wp even.
     int32_t phase, plane, halfw;
     FastDiv div_plane, div_halfw;
+    // HP kernels (KXC_HIP_CONV_HPOOL): width of the pooled output, OW / 2
+    int32_t PW;
 };
 
 __device__ __forceinline__ float relu_sel(float v) { return (v > 0.0f) ? v : 0.0f; }
@@ -119,10 +121,16 @@ typedef __attribute__((address_space(3))) void* lds_ptr_t;
 // DS: the workgroup also produces the second output described in ConvArgs (a residual block's 1x1 downsample next
 // to the block's first 3x3 convolution): per chunk CC/2 more k-steps that read the window's centre tap and a
 // second, small weight tile [2 planes][TO][CC/2], into a second set of accumulators.
-template <int KH, int KW, int CC, int WO, int WP, int RO, int RP, int PPT, int KS, bool TPAIR = false, bool DS = false>
+//
+// HP: the result leaves the kernel max-pooled along W (window 3, stride 2, one column of padding on the left; see the
+// epilogue): the first half of a 3x3 / stride-2 max pool that follows the convolution, done while the row is still
+// in registers, so that only half the feature map is written.
+template <int KH, int KW, int CC, int WO, int WP, int RO, int RP, int PPT, int KS, bool TPAIR = false, bool DS = false,
+          bool HP = false>
 __global__ void __launch_bounds__(64 * WO * WP * KS) __attribute__((amdgpu_waves_per_eu(2)))
 conv_mfma_kernel(const ConvArgs a) {
     static_assert(!(DS && TPAIR), "the second output pairs channels");
+    static_assert(!HP || (KS == 1 && !DS), "the pooling epilogue handles one reduction group and one output");
     constexpr int NW = WO * WP;                               // waves per reduction group
     constexpr int TO = 32 * RO * WO;
     constexpr int TP = 32 * RP * WP;
@@ -452,6 +460,73 @@ conv_mfma_kernel(const ConvArgs a) {
     }
 
     // ---- epilogue: accumulator register g of a block holds row 8*(g/4) + 4*half + g%4, column r
+    if constexpr (HP) {
+        // y[n,o,oh,pw] = max over columns 2pw-1 .. 2pw+1 of the (bias, ReLU) result; column -1 does not exist.  The host
+        // guarantees that OW is even, that a tile is a whole number of output rows and that every tile is full, so a
+        // lane's column has the parity of r and the even lanes own the windows: lane r needs lanes r-1 and r+1 of its
+        // half-wave.  The left neighbour of a block's lane 0 is lane 31 of the wave before it (one float per
+        // accumulator register, handed over through LDS -- the tiles are dead after the loop's last barrier); the
+        // first window of a row has no left neighbour.  With ReLU the values are >= +0 and never NaN, so the order
+        // of the comparisons does not matter and a padding candidate would never win.
+        const bool has_bias = (a.flags & KXC_HIP_CONV_BIAS) != 0;
+        const bool do_relu = (a.flags & KXC_HIP_CONV_RELU) != 0;
+        auto channel = [&](int i, int g) { return o0 + (wave_o * RO + i) * 32 + 8 * (g / 4) + 4 * half + (g % 4); };
+        const __amdgpu_buffer_rsrc_t br = make_rsrc(has_bias ? a.bias : a.y, has_bias ? static_cast<uint32_t>(a.O) * 4u : 0u);
+        float bv[RO][16];
+#pragma unroll
+        for (int i = 0; i < RO; ++i)
+#pragma unroll
+            for (int g = 0; g < 16; ++g) {
+                const int o = channel(i, g);
+                bv[i][g] = __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(br, o < a.O ? static_cast<uint32_t>(o) * 4u : kOobOffset, 0, 0));
+            }
+        // edge[block][half][RO][16], block = the wave's 32-pixel blocks in tile order per output-channel group
+        float* const edge = lds;
+        auto edge_at = [&](int block, int i, int g) { return (((wave_o * WP * RP + block) * 2 + half) * RO + i) * 16 + g; };
+#pragma unroll
+        for (int i = 0; i < RO; ++i)
+#pragma unroll
+            for (int j = 0; j < RP; ++j)
+#pragma unroll
+                for (int g = 0; g < 16; ++g) {
+                    float v = acc[i][j][g];
+                    if (has_bias) v = __fadd_rn(v, bv[i][g]);
+                    if (do_relu) v = relu_sel(v);
+                    acc[i][j][g] = v;
+                    if (r == 31) edge[edge_at(wave_p * RP + j, i, g)] = v;
+                }
+        __syncthreads();
+        const uint32_t y_bytes = static_cast<uint32_t>(a.out_elems) * 4u;
+        const uint32_t plane = static_cast<uint32_t>(a.OH * a.PW) * 4u;
+        const __amdgpu_buffer_rsrc_t yr = make_rsrc(a.y, y_bytes);
+#pragma unroll
+        for (int j = 0; j < RP; ++j) {
+            const int block = wave_p * RP + j;
+            const int m = m0 + block * 32 + r;                        // < M: every tile is full
+            const int n = fast_div(m, a.div_ohw), rem = m - n * a.OHW;
+            const int oh = fast_div(rem, a.div_ow), ow = rem - oh * a.OW;
+            const bool row_start = ow == 0;
+            const bool from_edge = r == 0 && !row_start;              // (then block > 0: a tile starts a row)
+            const uint32_t yb = (r & 1) ? kOobOffset : static_cast<uint32_t>((n * a.O * a.OH + oh) * a.PW + (ow >> 1)) * 4u;
+#pragma unroll
+            for (int i = 0; i < RO; ++i)
+#pragma unroll
+                for (int g = 0; g < 16; ++g) {
+                    const float v = acc[i][j][g];
+                    const int bits = __builtin_bit_cast(int, v);
+                    // lane l reads lane l-1 (0x138: whole-wave shift right by one) and lane l+1 (0x130: shift left)
+                    float left = __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(bits, bits, 0x138, 0xf, 0xf, false));
+                    const float right = __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(bits, bits, 0x130, 0xf, 0xf, false));
+                    if (from_edge) left = edge[edge_at(block - 1, i, g)];
+                    if (row_start) left = v;
+                    const float pooled = fmaxf(v, fmaxf(left, right));
+                    const int o = channel(i, g);
+                    __builtin_amdgcn_raw_buffer_store_b32(__builtin_bit_cast(uint32_t, pooled), yr,
+                                                          o < a.O && yb != kOobOffset ? yb + static_cast<uint32_t>(o) * plane : kOobOffset, 0, 0);
+                }
+        }
+        return;
+    }
     if (a.gsplit > 1) {
         // raw partial sums of this split; conv_split_reduce_kernel finishes the layer.  The parts of a second output
         // follow those of the first: partial[gsplit + split][...].
@@ -653,6 +728,7 @@ struct Variant {
     int kh, kw, cc, to, tp, nw, ppt, ks, tpair;
     void (*kernel)(const ConvArgs);
     void (*ds_kernel)(const ConvArgs);      // the same tile with the second (1x1 downsample) output, or nullptr
+    void (*hp_kernel)(const ConvArgs);      // the same tile with the pooling epilogue (KXC_HIP_CONV_HPOOL), or nullptr
 };
 
 #define KXC_VARIANT(KH, KW, CC, WO, WP, RO, RP, PPT)                                                   \
@@ -664,6 +740,10 @@ struct Variant {
 #define KXC_VARIANT_TP(KH, KW, CC, WO, WP, RO, RP, PPT)                                                \
     {"mfma_k" #KH "x" #KW "_t" #CC "_o" #WO "x" #RO "_p" #WP "x" #RP, KH, KW, CC, 32 * RO * WO, 32 * RP * WP, \
      WO * WP, PPT, 1, 1, conv_mfma_kernel<KH, KW, CC, WO, WP, RO, RP, PPT, 1, true>, nullptr}
+#define KXC_VARIANT_TP_HP(KH, KW, CC, WO, WP, RO, RP, PPT)                                             \
+    {"mfma_k" #KH "x" #KW "_t" #CC "_o" #WO "x" #RO "_p" #WP "x" #RP, KH, KW, CC, 32 * RO * WO, 32 * RP * WP, \
+     WO * WP, PPT, 1, 1, conv_mfma_kernel<KH, KW, CC, WO, WP, RO, RP, PPT, 1, true>, nullptr,              \
+     conv_mfma_kernel<KH, KW, CC, WO, WP, RO, RP, PPT, 1, true, false, true>}
 // (tiles that also exist with the second output)
 #define KXC_VARIANT_DS(KH, KW, CC, WO, WP, RO, RP, PPT)                                                \
     {"mfma_k" #KH "x" #KW "_c" #CC "_o" #WO "x" #RO "_p" #WP "x" #RP, KH, KW, CC, 32 * RO * WO, 32 * RP * WP, \
@@ -712,6 +792,12 @@ const Variant kVariants[] = {
     KXC_VARIANT_TP(7, 7, 3, 1, 8, 1, 1, 8),   // 32 x 256, all three channels in one chunk
     KXC_VARIANT_TP(7, 7, 3, 1, 4, 1, 1, 12),  // 32 x 128
     KXC_VARIANT_TP(7, 7, 3, 1, 8, 2, 1, 8),   // 64 x 256
+    // tiles that are whole rows of a 112-wide map, which the pooling epilogue needs.  Seven 32-pixel blocks per
+    // row pair do not divide over eight waves: seven waves of one block each leave a SIMD short (227 us for the
+    // batch-64 first layer against 194 us for the 64 x 256 tile), 14 waves of one block 255 us; four waves that
+    // each keep 32 channels x 224 pixels (seven blocks) in registers reach 192 us.
+    KXC_VARIANT_TP_HP(7, 7, 1, 2, 2, 1, 7, 12),  // 64 x 448, 4 waves of 32 x 224
+    KXC_VARIANT_TP_HP(7, 7, 1, 1, 7, 2, 1, 8),   // 64 x 224, 7 waves of 64 x 32
     KXC_VARIANT(7, 7, 2, 1, 8, 1, 1, 8),   // 32 x 256; 2-channel chunks: two chunks for RGB, loads overlap compute
     KXC_VARIANT(7, 7, 2, 1, 7, 1, 1, 8),   // 32 x 224: two full output rows of a 112-wide map
     KXC_VARIANT(7, 7, 4, 1, 8, 1, 1, 8),   // 32 x 256, one chunk (3 input channels padded to 4)
@@ -883,6 +969,31 @@ void Select(const ConvArgs& real, int kh, int kw, Choice* choice, bool ds = fals
     }
 }
 
+// The variant whose pooling epilogue (KXC_HIP_CONV_HPOOL) covers a shape: ReLU and no residual, an even output
+// width, tiles that are whole output rows and all full.  `a` is the shape after FillArgs.
+bool HpoolChoice(const kxc_hip_conv2d_desc* desc, const ConvArgs& a, Choice* choice) {
+    choice->v = nullptr;
+    if (!(desc->flags & KXC_HIP_CONV_RELU) || (desc->flags & (KXC_HIP_CONV_RESIDUAL | KXC_HIP_CONV_FORCE_DIRECT))) return false;
+    if (a.M <= 0 || a.OW < 2 || (a.OW & 1)) return false;
+    const int64_t x_bytes = static_cast<int64_t>(a.N) * a.C * a.H * a.W * 4;
+    const int64_t y_elems = static_cast<int64_t>(a.N) * a.O * a.OHW;
+    const int64_t w_bytes = static_cast<int64_t>(a.O) * a.C * desc->kh * desc->kw * 4;
+    const int64_t q_rows = static_cast<int64_t>(a.N + 1) * a.Hp + desc->kh * a.dh;
+    if (x_bytes >= (1LL << 31) || y_elems * 4 >= (1LL << 31) || w_bytes >= (1LL << 31) || q_rows * a.Wp >= (1LL << 31)) return false;
+    const char* forced = std::getenv("KXC_HIP_CONV_HPOOL_VARIANT");
+    for (int i = 0; i < kNumVariants; ++i) {
+        const Variant& v = kVariants[i];
+        if (!v.hp_kernel || v.kh != desc->kh || v.kw != desc->kw) continue;
+        if (forced && *forced && std::strcmp(forced, v.name) != 0) continue;
+        if (v.tp % a.OW != 0 || a.M % v.tp != 0) continue;
+        Choice c;
+        if (!Fits(v, a, &c)) continue;
+        *choice = c;
+        return true;
+    }
+    return false;
+}
+
 int32_t FillArgs(const kxc_hip_conv2d_desc* d, ConvArgs* a, const char* who) {
     KXC_HIP_REQUIRE(d != nullptr, "%s: desc is NULL", who);
     KXC_HIP_REQUIRE(d->n >= 0 && d->c > 0 && d->h > 0 && d->w > 0 && d->o > 0 && d->kh > 0 && d->kw > 0,
@@ -1016,7 +1127,8 @@ int32_t Conv2dResolve(const kxc_hip_conv2d_desc* desc, bool second, const char* 
     // A filter one row high with a vertical stride touches only every stride-th input row (the 1x1/2
     // downsample convolutions): the matrix kernel then sees an image of OH rows that are stride rows apart, so
     // the skipped rows are neither loaded nor staged.
-    if (!second && UseSmall1x1(desc, a)) {
+    const bool hpool = (desc->flags & KXC_HIP_CONV_HPOOL) != 0;
+    if (!second && !hpool && UseSmall1x1(desc, a)) {
         a.div_ohw = MakeFastDiv(a.OHW); a.div_ow = MakeFastDiv(a.OW);
         L->path = ConvLaunch::kSmall1x1;
         L->grid = dim3(static_cast<unsigned>(CeilDiv(a.O, 32)), static_cast<unsigned>(CeilDiv(a.M, 32)));
@@ -1030,7 +1142,12 @@ int32_t Conv2dResolve(const kxc_hip_conv2d_desc* desc, bool second, const char* 
     L->direct_args = a;
     ApplyRowView(&a, desc->kh);
     Choice c;
-    if (!(desc->flags & KXC_HIP_CONV_FORCE_DIRECT) && a.M > 0) Select(a, desc->kh, desc->kw, &c, second);
+    if (hpool) {
+        KXC_HIP_REQUIRE(!second && HpoolChoice(desc, a, &c), "%s: no kernel with the pooling epilogue covers this shape", who);
+        a.PW = a.OW / 2;
+    } else if (!(desc->flags & KXC_HIP_CONV_FORCE_DIRECT) && a.M > 0) {
+        Select(a, desc->kh, desc->kw, &c, second);
+    }
     if (second) {
         int rh = 0, rw = 0;
         KXC_HIP_REQUIRE(c.v && c.v->ds_kernel && PairTap(desc, &rh, &rw), "%s: no kernel with a second output covers this shape", who);
@@ -1063,9 +1180,10 @@ int32_t Conv2dResolve(const kxc_hip_conv2d_desc* desc, bool second, const char* 
     // split the reduction over workgroups as well; every workgroup keeps at least two chunks per wave group.
     a.gsplit = 1;
     a.cps = a.nchunks;
-    a.out_elems = total;
+    a.out_elems = hpool ? static_cast<int64_t>(a.N) * a.O * a.OH * a.PW : total;
     int split = 1;
-    SplitOverWorkgroups(c, a.nchunks, tiles, total * (second ? 2 : 1), &split);      // (a second output has parts of its own)
+    // (a second output has parts of its own; the pooling epilogue needs the whole sum in one workgroup)
+    if (!hpool) SplitOverWorkgroups(c, a.nchunks, tiles, total * (second ? 2 : 1), &split);
     if (split > 1) {
         a.cps = static_cast<int32_t>(CeilDiv(a.nchunks, split));
         a.gsplit = static_cast<int32_t>(CeilDiv(a.nchunks, a.cps));      // no empty split
@@ -1081,7 +1199,7 @@ int32_t Conv2dResolve(const kxc_hip_conv2d_desc* desc, bool second, const char* 
     a.o_fastest = w_tile_bytes * a.o_tiles <= (2 << 20) ? 1 : 0;
     if (const char* e = std::getenv("KXC_HIP_CONV_OFAST")) a.o_fastest = std::atoi(e);
     L->path = ConvLaunch::kMfma;
-    L->kernel = second ? c.v->ds_kernel : c.v->kernel;
+    L->kernel = second ? c.v->ds_kernel : hpool ? c.v->hp_kernel : c.v->kernel;
     L->name = c.v->name;
     L->grid = dim3(static_cast<unsigned>(a.tiles_per_xcd * 8));
     L->block = dim3(64 * c.v->nw * c.v->ks);
@@ -1211,6 +1329,10 @@ extern "C" {
 const char* kxc_hip_conv2d_variant(const kxc_hip_conv2d_desc* desc) {
     ConvArgs a;
     if (FillArgs(desc, &a, "kxc_hip_conv2d_variant") != KXC_HIP_OK) return "invalid";
+    if (desc->flags & KXC_HIP_CONV_HPOOL) {
+        Choice hp;
+        return HpoolChoice(desc, a, &hp) ? hp.v->name : "unsupported";
+    }
     if (desc->flags & KXC_HIP_CONV_FORCE_DIRECT) return "direct";
     if (UseSmall1x1(desc, a)) return "mfma_k1x1_small";
     ApplyRowView(&a, desc->kh);
@@ -1236,7 +1358,7 @@ static const Variant* PairVariant(const kxc_hip_conv2d_desc* desc) {
     ConvArgs a;
     if (!desc || FillArgs(desc, &a, "kxc_hip_conv2d_pair_supported") != KXC_HIP_OK) return nullptr;
     int rh = 0, rw = 0;
-    if ((desc->flags & KXC_HIP_CONV_FORCE_DIRECT) || a.M <= 0 || !PairTap(desc, &rh, &rw)) return nullptr;
+    if ((desc->flags & (KXC_HIP_CONV_FORCE_DIRECT | KXC_HIP_CONV_HPOOL)) || a.M <= 0 || !PairTap(desc, &rh, &rw)) return nullptr;
     if (desc->kh == 1 && desc->kw == 1) return nullptr;
     Choice c;
     Select(a, desc->kh, desc->kw, &c, true);
@@ -1254,6 +1376,26 @@ static const Variant* PairVariant(const kxc_hip_conv2d_desc* desc) {
 }
 
 int32_t kxc_hip_conv2d_pair_supported(const kxc_hip_conv2d_desc* desc) { return PairVariant(desc) ? 1 : 0; }
+
+int32_t kxc_hip_conv2d_hpool_supported(const kxc_hip_conv2d_desc* desc) {
+    ConvArgs a;
+    if (!desc || FillArgs(desc, &a, "kxc_hip_conv2d_hpool_supported") != KXC_HIP_OK) return 0;
+    Choice c;
+    return HpoolChoice(desc, a, &c) ? 1 : 0;
+}
+
+// Measured on MI355X, 3 -> 64 channels, 7x7 / 2 on 224 x 224, inside the network (launch + pool, us): batch 64
+// 192 + 27 against 194 + 51, batch 32 114 + 17 against 109 + 26, batch 16 63 + 12 against 65 + 17, batch 8 46 + 8
+// against 37 + 13, batch 4 44 + 7 against 25 + 8: the 64 x 448 tile needs 448 workgroups (16 images) to fill the
+// compute units; below that the smaller tiles of the unpooled kernel win.
+int32_t kxc_hip_conv2d_hpool_preferred(const kxc_hip_conv2d_desc* desc) {
+    ConvArgs a;
+    if (!desc || FillArgs(desc, &a, "kxc_hip_conv2d_hpool_preferred") != KXC_HIP_OK) return 0;
+    Choice c;
+    if (!HpoolChoice(desc, a, &c)) return 0;
+    if (const char* e = std::getenv("KXC_HIP_CONV_HPOOL")) return std::atoi(e) != 0 ? 1 : 0;
+    return CeilDiv(a.M, c.v->tp) * CeilDiv(a.O, c.v->to) >= 448 ? 1 : 0;
+}
 
 const char* kxc_hip_conv2d_pair_variant(const kxc_hip_conv2d_desc* desc) {
     // static storage: one name per table entry
@@ -1278,7 +1420,7 @@ int32_t kxc_hip_conv2d_scratch_needed(const kxc_hip_conv2d_desc* desc, size_t* o
     ConvArgs a;
     if (int32_t rc = FillArgs(desc, &a, "kxc_hip_conv2d_scratch_needed")) return rc;
     const int64_t total = static_cast<int64_t>(a.N) * a.O * a.OHW;
-    if (total == 0 || (desc->flags & KXC_HIP_CONV_FORCE_DIRECT) || UseSmall1x1(desc, a) || a.M <= 0) return KXC_HIP_OK;
+    if (total == 0 || (desc->flags & (KXC_HIP_CONV_FORCE_DIRECT | KXC_HIP_CONV_HPOOL)) || UseSmall1x1(desc, a) || a.M <= 0) return KXC_HIP_OK;
     ApplyRowView(&a, desc->kh);
     Choice c;
     Select(a, desc->kh, desc->kw, &c);

@@ -590,6 +590,7 @@ constexpr int kNumWino = sizeof(kWino) / sizeof(kWino[0]);
 bool Supported(const kxc_hip_conv2d_desc* d) {
     if (!d || d->kh != 3 || d->kw != 3 || d->stride_h != 1 || d->stride_w != 1 || d->dil_h != 1 || d->dil_w != 1) return false;
     if (d->n <= 0 || d->c <= 0 || d->c % 4 != 0 || d->o <= 0 || d->h <= 0 || d->w <= 0) return false;
+    if (d->flags & KXC_HIP_CONV_HPOOL) return false;      // the pooling epilogue exists in the direct-convolution kernels only
     // padding beyond the filter's reach only adds all-zero border tiles; cap it so the sizes below cannot overflow
     if (d->pad_h < 0 || d->pad_w < 0 || d->pad_h > (1 << 20) || d->pad_w > (1 << 20)) return false;
     const int64_t oh = static_cast<int64_t>(d->h) + 2 * d->pad_h - 2, ow = static_cast<int64_t>(d->w) + 2 * d->pad_w - 2;

@@ -80,7 +80,8 @@ void OperandExtents(const Node& n, std::vector<std::pair<kxc_hip_buf, size_t>>* 
             const kxc_hip_conv2d_desc& d = n.conv;
             const int64_t oh = (static_cast<int64_t>(d.h) + 2 * d.pad_h - (static_cast<int64_t>(d.dil_h) * (d.kh - 1) + 1)) / d.stride_h + 1;
             const int64_t ow = (static_cast<int64_t>(d.w) + 2 * d.pad_w - (static_cast<int64_t>(d.dil_w) * (d.kw - 1) + 1)) / d.stride_w + 1;
-            const int64_t y = static_cast<int64_t>(d.n) * d.o * oh * ow;
+            // (KXC_HIP_CONV_HPOOL: the output is pooled along W, half as wide)
+            const int64_t y = static_cast<int64_t>(d.n) * d.o * oh * ((d.flags & KXC_HIP_CONV_HPOOL) ? ow / 2 : ow);
             add(n.bufs[0], static_cast<int64_t>(d.n) * d.c * d.h * d.w);
             add(n.bufs[1], static_cast<int64_t>(d.o) * d.c * d.kh * d.kw);
             add(n.bufs[2], d.o);
@@ -330,6 +331,8 @@ int32_t kxc_hip_plan_add_conv2d(kxc_hip_plan* plan, const kxc_hip_conv2d_desc* d
     KXC_PLAN_BUF(x, false, who); KXC_PLAN_BUF(w, false, who); KXC_PLAN_BUF(y, false, who);
     KXC_PLAN_BUF(bias, !(desc->flags & KXC_HIP_CONV_BIAS), who);
     KXC_PLAN_BUF(residual, !(desc->flags & KXC_HIP_CONV_RESIDUAL), who);
+    KXC_HIP_REQUIRE(!(desc->flags & KXC_HIP_CONV_HPOOL) || kxc_hip_conv2d_hpool_supported(desc),
+                    "%s: no kernel with the pooling epilogue covers this shape", who);
     Node n{};
     n.kind = NodeKind::kConv2D;
     n.conv = *desc;
@@ -338,6 +341,7 @@ int32_t kxc_hip_plan_add_conv2d(kxc_hip_plan* plan, const kxc_hip_conv2d_desc* d
     if (desc->flags & KXC_HIP_CONV_BIAS) n.symbol += "+bias";
     if (desc->flags & KXC_HIP_CONV_RESIDUAL) n.symbol += "+add";
     if (desc->flags & KXC_HIP_CONV_RELU) n.symbol += "+relu";
+    if (desc->flags & KXC_HIP_CONV_HPOOL) n.symbol += "+maxpool3w";
     plan->nodes.push_back(n);
     return KXC_HIP_OK;
 }
@@ -348,6 +352,7 @@ int32_t kxc_hip_plan_add_conv2d_winograd(kxc_hip_plan* plan, const kxc_hip_conv2
     KXC_PLAN_BEGIN(who);
     KXC_HIP_REQUIRE(desc != nullptr, "%s: desc is NULL", who);
     KXC_HIP_REQUIRE(kxc_hip_conv2d_winograd_supported(desc), "%s: not a 3x3 stride-1 convolution with c %% 4 == 0", who);
+    KXC_HIP_REQUIRE(!(desc->flags & KXC_HIP_CONV_HPOOL), "%s: the pooling epilogue belongs to kxc_hip_plan_add_conv2d", who);
     KXC_HIP_REQUIRE(u.kind == KXC_HIP_BUF_WORKSPACE, "%s: the transformed weights live in the plan workspace", who);
     KXC_PLAN_BUF(u, false, who);
     if (int32_t rc = kxc_hip_plan_add_conv2d(plan, desc, x, w, bias, residual, y)) return rc;
@@ -368,6 +373,7 @@ int32_t kxc_hip_plan_add_conv2d_pair(kxc_hip_plan* plan, const kxc_hip_conv2d_de
     KXC_PLAN_BEGIN(who);
     KXC_HIP_REQUIRE(desc != nullptr, "%s: desc is NULL", who);
     KXC_HIP_REQUIRE(kxc_hip_conv2d_pair_supported(desc), "%s: no kernel with a second output covers this shape", who);
+    KXC_HIP_REQUIRE(!(desc->flags & KXC_HIP_CONV_HPOOL), "%s: the pooling epilogue belongs to kxc_hip_plan_add_conv2d", who);
     KXC_PLAN_BUF(w2, false, who); KXC_PLAN_BUF(bias2, true, who); KXC_PLAN_BUF(y2, false, who);
     if (int32_t rc = kxc_hip_plan_add_conv2d(plan, desc, x, w, bias, residual, y)) return rc;
     Node& n = plan->nodes.back();
@@ -1389,6 +1395,9 @@ int32_t kxc_hip_plan_deserialize(const char* text, int32_t device_id, kxc_hip_mo
         };
         for (const kxc_hip_buf& b : n.bufs) if (!buf_ok(b)) return fail("buffer operand out of range");
         for (const kxc_hip_buf& b : n.params) if (!buf_ok(b)) return fail("kernel parameter out of range");
+        if (n.kind == NodeKind::kConv2D && (n.conv.flags & KXC_HIP_CONV_HPOOL) &&
+            (n.i32[0] != 0 || !kxc_hip_conv2d_hpool_supported(&n.conv)))
+            return fail("bad convolution node with the pooling epilogue");
         if (n.kind == NodeKind::kConv2D && n.i32[0] == 1 &&
             (!kxc_hip_conv2d_winograd_supported(&n.conv) || n.bufs[5].kind != KXC_HIP_BUF_WORKSPACE))
             return fail("bad Winograd convolution node");

@@ -128,6 +128,42 @@ __global__ void __launch_bounds__(kBlock) maxpool3x3s2_kernel(const float* __res
     }
 }
 
+// Column max pool: window 3x1, stride (2,1), one row of padding above (and below when the height is even): the
+// second half of a 3x3 / stride-2 max pool whose column maxima the convolution before it already took
+// (KXC_HIP_CONV_HPOOL).  One thread produces a 4-wide strip of ROWS consecutive output rows from 2*ROWS + 1 aligned
+// 16-byte loads; every input row is requested once per strip (plus the one row neighbouring strips share).
+template <int ROWS>
+__global__ void __launch_bounds__(kBlock) maxpool3x1s2_kernel(const float* __restrict__ x, float* __restrict__ y,
+                                                              int32_t h, int32_t w, int32_t oh_total,
+                                                              int32_t col_groups, int32_t row_groups, int64_t total) {
+    const int64_t tid = static_cast<int64_t>(blockIdx.x) * kBlock + threadIdx.x;
+    if (tid >= total) return;
+    const int32_t cg = static_cast<int32_t>(tid % col_groups);
+    const int64_t t2 = tid / col_groups;
+    const int32_t rg = static_cast<int32_t>(t2 % row_groups);
+    const int64_t plane = t2 / row_groups;
+    const float* xp = x + plane * h * w + cg * 4;
+    float* yp = y + plane * oh_total * w + cg * 4;
+    const int32_t oh0 = rg * ROWS;
+    float4 rows[2 * ROWS + 1];
+#pragma unroll
+    for (int k = 0; k < 2 * ROWS + 1; ++k) {
+        const int32_t ih = 2 * oh0 - 1 + k;
+        rows[k] = (ih >= 0 && ih < h) ? *reinterpret_cast<const float4*>(xp + static_cast<int64_t>(ih) * w)
+                                      : make_float4(kPadValue, kPadValue, kPadValue, kPadValue);
+    }
+#pragma unroll
+    for (int r = 0; r < ROWS; ++r) {
+        if (oh0 + r >= oh_total) break;
+        float4 o;
+        o.x = max_sel(max_sel(max_sel(-INFINITY, rows[2 * r].x), rows[2 * r + 1].x), rows[2 * r + 2].x);
+        o.y = max_sel(max_sel(max_sel(-INFINITY, rows[2 * r].y), rows[2 * r + 1].y), rows[2 * r + 2].y);
+        o.z = max_sel(max_sel(max_sel(-INFINITY, rows[2 * r].z), rows[2 * r + 1].z), rows[2 * r + 2].z);
+        o.w = max_sel(max_sel(max_sel(-INFINITY, rows[2 * r].w), rows[2 * r + 1].w), rows[2 * r + 2].w);
+        *reinterpret_cast<float4*>(yp + static_cast<int64_t>(oh0 + r) * w) = o;
+    }
+}
+
 // ---------------------------------------------------------------- global average pool
 // Small planes (HW <= 128): a workgroup of 256 threads takes 16 consecutive planes.  Their 16*HW contiguous
 // floats are fetched with coalesced loads that are all in flight together and staged through LDS; one lane per
@@ -279,6 +315,25 @@ int32_t kxc_hip_pool2d_f32(const kxc_hip_pool2d_desc* desc, const float* x, floa
             maxpool3x3s2_kernel<4><<<NoteGrid(static_cast<int>(blocks)), NoteBlock(kBlock), NoteLds(0), s>>>(
                 x, y, d.h, d.w, d.oh, d.ow, col_groups, row_groups, threads);
         return CheckLaunch("maxpool3x3s2");
+    }
+    const bool columns = !desc->is_avg && d.kh == 3 && d.kw == 1 && d.sh == 2 && d.sw == 1 && d.pt == 1 && d.pl == 0 &&
+                         desc->pad_right == 0 && desc->pad_bottom <= 1 && !desc->ceil_mode && (d.w % 4) == 0 &&
+                         (reinterpret_cast<uintptr_t>(x) & 15u) == 0 && (reinterpret_cast<uintptr_t>(y) & 15u) == 0;
+    if (columns) {
+        const int32_t col_groups = d.w / 4;
+        const bool small = planes * ((d.oh + 3) / 4) * col_groups < 256LL * kBlock;
+        const int32_t rows = small ? 1 : 4;
+        const int32_t row_groups = (d.oh + rows - 1) / rows;
+        const int64_t threads = planes * row_groups * col_groups;
+        const int64_t blocks = CeilDiv(threads, kBlock);
+        KXC_HIP_REQUIRE(blocks <= kMaxGridX, "kxc_hip_pool2d_f32: tensor too large");
+        if (small)
+            maxpool3x1s2_kernel<1><<<NoteGrid(static_cast<int>(blocks)), NoteBlock(kBlock), NoteLds(0), s>>>(
+                x, y, d.h, d.w, d.oh, col_groups, row_groups, threads);
+        else
+            maxpool3x1s2_kernel<4><<<NoteGrid(static_cast<int>(blocks)), NoteBlock(kBlock), NoteLds(0), s>>>(
+                x, y, d.h, d.w, d.oh, col_groups, row_groups, threads);
+        return CheckLaunch("maxpool3x1s2");
     }
     if (desc->is_avg) pool_generic_kernel<true><<<NoteGrid(GridFor(total)), NoteBlock(kBlock), NoteLds(0), s>>>(x, y, d, total);
     else pool_generic_kernel<false><<<NoteGrid(GridFor(total)), NoteBlock(kBlock), NoteLds(0), s>>>(x, y, d, total);

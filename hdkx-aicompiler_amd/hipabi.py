@@ -13,7 +13,7 @@ PKG = os.path.dirname(os.path.abspath(__file__))
 _LIB_PATH = os.environ.get("KXC_HIP_LIB") or os.path.join(PKG, "lib", "libkxc_hip.so")
 _lib = None
 
-CONV_BIAS, CONV_RESIDUAL, CONV_RELU, CONV_FORCE_DIRECT = 1, 2, 4, 0x100
+CONV_BIAS, CONV_RESIDUAL, CONV_RELU, CONV_HPOOL, CONV_FORCE_DIRECT = 1, 2, 4, 0x10, 0x100
 BUF_ARG, BUF_WORKSPACE, BUF_NONE, BUF_ARG_OFFSET = 0, 1, 2, 3
 
 
@@ -130,7 +130,13 @@ def conv_desc(x_shape, w_shape, stride, pad, dil=1, flags=0):
 def conv_out_shape(d):
     oh = (d.h + 2 * d.pad_h - ((d.kh - 1) * d.dil_h + 1)) // d.stride_h + 1
     ow = (d.w + 2 * d.pad_w - ((d.kw - 1) * d.dil_w + 1)) // d.stride_w + 1
-    return (d.n, d.o, oh, ow)
+    return (d.n, d.o, oh, ow // 2 if d.flags & CONV_HPOOL else ow)
+
+
+def conv2d_hpool_supported(x_shape, w_shape, stride, pad, dil=1, flags=CONV_BIAS | CONV_RELU, preferred=False):
+    d = conv_desc(x_shape, w_shape, stride, pad, dil, flags)
+    f = lib().kxc_hip_conv2d_hpool_preferred if preferred else lib().kxc_hip_conv2d_hpool_supported
+    return bool(f(C.byref(d)))
 
 
 def conv2d_variant(x_shape, w_shape, stride, pad, dil=1, flags=0):
@@ -139,16 +145,16 @@ def conv2d_variant(x_shape, w_shape, stride, pad, dil=1, flags=0):
 
 
 def conv2d(x, w, bias=None, residual=None, stride=1, pad=0, dil=1, relu=False, force_direct=False, out=None,
-           no_alloc=False):
+           no_alloc=False, hpool=False):
     """nn_conv2d through kxc_hip_conv2d_nchw_f32, or (no_alloc, with `out` given) through the entry point that
-    allocates nothing."""
+    allocates nothing.  hpool: KXC_HIP_CONV_HPOOL, the result max-pooled along W (window 3, stride 2, padding 1)."""
     import torch
     _need(x, torch.float32, "x"); _need(w, torch.float32, "w")
     _need(bias, torch.float32, "bias"); _need(residual, torch.float32, "residual")
     if x.shape[1] != w.shape[1]:
         raise KxcHipError("nn_conv2d input channel mismatch")
     flags = (CONV_BIAS if bias is not None else 0) | (CONV_RESIDUAL if residual is not None else 0) | \
-            (CONV_RELU if relu else 0) | (CONV_FORCE_DIRECT if force_direct else 0)
+            (CONV_RELU if relu else 0) | (CONV_FORCE_DIRECT if force_direct else 0) | (CONV_HPOOL if hpool else 0)
     d = conv_desc(tuple(x.shape), tuple(w.shape), stride, pad, dil, flags)
     if out is not None:
         _check_out(out, conv_out_shape(d))
@@ -282,7 +288,9 @@ def pool_desc(x_shape, k, s, pad, ceil_mode=False, avg=False):
     n, c, h, w = x_shape
     if isinstance(pad, int):
         pad = (pad, pad, pad, pad)
-    return PoolDesc(n, c, h, w, k, k, s, s, pad[0], pad[1], pad[2], pad[3], int(ceil_mode), int(avg))
+    kh, kw = (k, k) if isinstance(k, int) else k
+    sh, sw = (s, s) if isinstance(s, int) else s
+    return PoolDesc(n, c, h, w, kh, kw, sh, sw, pad[0], pad[1], pad[2], pad[3], int(ceil_mode), int(avg))
 
 
 def pool_out_shape(d):

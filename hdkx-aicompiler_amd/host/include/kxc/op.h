@@ -100,7 +100,18 @@ struct HIPDispatchContext {
     Array<Type> pair_input_types;
     Array<HIPBuffer> pair_inputs;
     HIPBuffer pair_output;
+    // A pooling call that is the sole reader of this launch's value and that the operator's "FHIPPoolQuery" agreed
+    // to produce as well: `output` and `out_type` are then the pooling call's, and alloc_temp(bytes) hands out
+    // workspace that lives until the call's launches have been appended (for what passes between them).
+    bool has_pool = false;
+    std::string pool_op;
+    Attrs pool_attrs;
+    std::function<HIPBuffer(int64_t)> alloc_temp;
 };
+// Whether the launch(es) of a call (attributes, input types, what is fused behind it) can also produce the pooling
+// call `pool_op` (nn_max_pool2d / nn_avg_pool2d, MaxPool2DAttrs) that reads its value.
+using FHIPPoolQuery = std::function<bool(const Attrs& attrs, const Array<Type>& inputs, bool fused_relu, bool has_residual,
+                                         const std::string& pool_op, const Attrs& pool_attrs)>;
 // Whether one launch of call A (attrs, input types, and whether a ReLU / residual is fused behind it is irrelevant)
 // can also produce call B, an unfused call of the same operator on the same first input.
 using FHIPPairQuery = std::function<bool(const Attrs& a_attrs, const Array<Type>& a_inputs, const std::vector<bool>& a_constant,

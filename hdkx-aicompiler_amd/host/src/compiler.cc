@@ -187,6 +187,7 @@ struct Group {
     const CallNode* tail = nullptr;     // the last call folded into it (its value is the group's output)
     const RelayExprNode* residual = nullptr;
     bool fused_relu = false;
+    const CallNode* pool = nullptr;     // a pooling call behind it that the head's launches produce as well (then the tail)
 };
 
 template <typename T>
@@ -335,6 +336,20 @@ private:
                     }
                     n = SoleConsumer(g.tail);
                     if (n && !absorbed.count(n) && IsOp(n, "nn_relu")) { g.fused_relu = true; g.tail = n; absorbed.insert(n); }
+                    // ... -> pooling, when the operator can take part of the window in its own launch
+                    n = SoleConsumer(g.tail);
+                    const auto* pool_query = OpAttr<relay::FHIPPoolQuery>(op, "FHIPPoolQuery");
+                    const char* pool_env = std::getenv("KXC_HIP_FUSE_POOL");            // "0" switches it off
+                    if (n && pool_query && !absorbed.count(n) && g.tail != f_->body.get() && !(pool_env && pool_env[0] == '0') &&
+                        (IsOp(n, "nn_max_pool2d") || IsOp(n, "nn_avg_pool2d")) && IsF32(n->checked_type_)) {
+                        Array<Type> types;
+                        for (const auto& a : c->args) types.push_back(a.checked_type());
+                        if ((*pool_query)(c->attrs, types, g.fused_relu, g.residual != nullptr, n->op.As<OpNode>()->name, n->attrs)) {
+                            g.pool = n;
+                            g.tail = n;
+                            absorbed.insert(n);
+                        }
+                    }
                 } else if (OpFlag(op, "THIPFusableRelu") && TT(c->checked_type_)->shape.size() <= 6) {
                     const CallNode* n = SoleConsumer(g.tail);
                     if (n && !absorbed.count(n) && IsOp(n, "nn_relu")) { g.fused_relu = true; g.tail = n; absorbed.insert(n); }
@@ -481,7 +496,7 @@ private:
                 for (size_t sa = 0; sa < sb; ++sa) {
                     const size_t ia = order[sa];
                     const Group& ga = groups_[ia];
-                    if (merged[ia] || carries[ia] >= 0 || ga.head->op.get() != gb.head->op.get()) continue;
+                    if (merged[ia] || carries[ia] >= 0 || ga.pool || ga.head->op.get() != gb.head->op.get()) continue;
                     if (ga.tail == f_->body.get() || TT(ga.head->checked_type_)->dtype != TT(gb.head->checked_type_)->dtype) continue;
                     if (Resolve(ga.head->args[0].get()) != Resolve(gb.head->args[0].get())) continue;
                     // both launches must read the shared input and write their results in the same layouts
@@ -649,6 +664,15 @@ private:
                 ctx.pair_output = {KXC_HIP_BUF_WORKSPACE, slot_[carried->tail].first};
                 ctx.pair_output_layout = LayoutOf(carried->tail);
             }
+            if (g.pool) {
+                ctx.has_pool = true;
+                ctx.pool_op = g.pool->op.As<OpNode>()->name;
+                ctx.pool_attrs = g.pool->attrs;
+                ctx.alloc_temp = [this, &temps](int64_t bytes) {
+                    temps.push_back(arena_.Alloc(bytes));
+                    return relay::HIPBuffer{KXC_HIP_BUF_WORKSPACE, temps.back().first};
+                };
+            }
             ctx.out_type = g.tail->checked_type_;
             ctx.output = out;
             ctx.fused_relu = g.fused_relu;
@@ -681,12 +705,23 @@ private:
                 info.kernel_symbol = symbol;
                 m_->execs.push_back(info);
                 const int32_t added = kxc_hip_plan_num_nodes(m_->plan) - first_node;
+                if (g.pool) {
+                    // the launches behind the first one finish the pooling call
+                    for (int32_t k = 1; k < added; ++k) {
+                        KernelExecInfo more;
+                        more.op_name = ctx.pool_op;
+                        more.kernel_symbol = kxc_hip_plan_node_symbol(m_->plan, first_node + k);
+                        more.input_values.push_back(value_id_.at(g.tail));
+                        more.output_values.push_back(value_id_.at(g.tail));
+                        m_->execs.push_back(more);
+                    }
+                }
                 const bool side = side_join[order[step]] >= 0 && added == 1;
                 if ((side || joins[order[step]]) && added >= 1 &&
                     kxc_hip_plan_set_concurrency(m_->plan, first_node, side ? 1 : 0, joins[order[step]] ? 1 : 0))
                     throw std::runtime_error(std::string("plan_set_concurrency failed: ") + kxc_hip_last_error());
             } else {
-                if (g.fused_relu || g.residual || carried) throw std::runtime_error("hip back end: operator declined a fused launch: " + op->name);
+                if (g.fused_relu || g.residual || carried || g.pool) throw std::runtime_error("hip back end: operator declined a fused launch: " + op->name);
                 for (int l : ctx.input_layouts)
                     if (l != relay::kHIPLayoutPlain) throw std::runtime_error("hip back end: operator declined the layout it asked for: " + op->name);
                 if (out_layout != relay::kHIPLayoutPlain) throw std::runtime_error("hip back end: operator declined the layout it asked for: " + op->name);

@@ -80,6 +80,23 @@ bool Conv2DPairQuery(const Attrs& a_attrs, const Array<Type>& a_inputs, const st
     return kxc_hip_conv2d_pair_supported(&a) != 0;
 }
 
+// conv -> relu -> max pool (3x3, stride 2, padding 1): the convolution's launch takes the maximum over the three
+// columns of every window while an output row is in registers and writes a map half as wide; a 3x1 / stride (2,1)
+// max pool finishes the window.  Offered when the library has that epilogue for the shape and expects the two
+// launches to beat convolution + 3x3 pool.
+bool Conv2DPoolQuery(const Attrs& attrs, const Array<Type>& inputs, bool fused_relu, bool has_residual, const std::string& pool_op,
+                     const Attrs& pool_attrs) {
+    kxc_hip_conv2d_desc d{};
+    const auto* p = pool_attrs.As<MaxPool2DAttrsNode>();
+    if (pool_op != "nn_max_pool2d" || !p || !fused_relu || has_residual || !ConvDesc(attrs, inputs, &d)) return false;
+    if (!p->layout.empty() && p->layout != "NCHW") return false;
+    const auto ks = ReadPair(p->pool_size, 1), st = ReadPair(p->strides, 1), pd = ReadPad4(p->padding);
+    if (ks[0] != 3 || ks[1] != 3 || st[0] != 2 || st[1] != 2 || pd[0] != 1 || pd[1] != 1 || pd[2] != 1 || pd[3] != 1 || p->ceil_mode)
+        return false;
+    d.flags = (inputs.size() == 3 ? KXC_HIP_CONV_BIAS : 0u) | KXC_HIP_CONV_RELU;
+    return kxc_hip_conv2d_hpool_preferred(&d) != 0;
+}
+
 std::string Conv2DDispatch(const HIPDispatchContext& c, kxc_hip_plan* plan) {
     kxc_hip_conv2d_desc d{};
     if (!ConvDesc(c.attrs, c.input_types, &d) || !IsF32(c.out_type)) return "";
@@ -87,6 +104,22 @@ std::string Conv2DDispatch(const HIPDispatchContext& c, kxc_hip_plan* plan) {
     d.flags = (has_bias ? KXC_HIP_CONV_BIAS : 0u) | (c.has_residual ? KXC_HIP_CONV_RESIDUAL : 0u) |
               (c.fused_relu ? KXC_HIP_CONV_RELU : 0u);
     const kxc_hip_buf none{KXC_HIP_BUF_NONE, 0};
+    if (c.has_pool) {
+        // (Conv2DPoolQuery said yes for exactly this call: 3x3 / stride 2 / padding 1 behind a ReLU)
+        if (c.has_pair || c.has_residual || !c.fused_relu || !c.alloc_temp) return "";
+        d.flags |= KXC_HIP_CONV_HPOOL;
+        const int64_t oh = (d.h + 2 * d.pad_h - (d.dil_h * (d.kh - 1) + 1)) / d.stride_h + 1;
+        const int64_t ow = (d.w + 2 * d.pad_w - (d.dil_w * (d.kw - 1) + 1)) / d.stride_w + 1;
+        const HIPBuffer half = c.alloc_temp(static_cast<int64_t>(d.n) * d.o * oh * (ow / 2) * 4);
+        Check(kxc_hip_plan_add_conv2d(plan, &d, B(c.inputs[0]), B(c.inputs[1]), has_bias ? B(c.inputs[2]) : none, none, B(half)),
+              "nn_conv2d dispatch");
+        kxc_hip_pool2d_desc q{};
+        q.n = d.n; q.c = d.o; q.h = static_cast<int32_t>(oh); q.w = static_cast<int32_t>(ow / 2);
+        q.kh = 3; q.kw = 1; q.stride_h = 2; q.stride_w = 1;
+        q.pad_top = 1; q.pad_bottom = 1;
+        Check(kxc_hip_plan_add_pool2d(plan, &q, B(half), B(c.output)), "nn_conv2d dispatch (column pool)");
+        return std::string("kxc_conv2d_nchw_f32.") + kxc_hip_conv2d_variant(&d) + (has_bias ? "+bias" : "") + "+relu+maxpool3w";
+    }
     if (c.has_pair) {
         const bool bias2 = c.pair_inputs.size() == 3;
         Check(kxc_hip_plan_add_conv2d_pair(plan, &d, B(c.inputs[0]), B(c.inputs[1]), has_bias ? B(c.inputs[2]) : none,
@@ -436,7 +469,8 @@ void EnsureBuiltinOpsRegistered() {
             .set_attr<FRelayToTE>("FRelayToTE", Conv2DCompute)
             .set_attr<bool>("THIPFusable", true)
             .set_attr<FHIPDispatch>("FHIPDispatch", Conv2DDispatch)
-            .set_attr<FHIPPairQuery>("FHIPPairQuery", Conv2DPairQuery);
+            .set_attr<FHIPPairQuery>("FHIPPairQuery", Conv2DPairQuery)
+            .set_attr<FHIPPoolQuery>("FHIPPoolQuery", Conv2DPoolQuery);
         OpRegEntry::Register("nn_relu")
             .describe("Rectified Linear Unit activation")
             .set_num_inputs(1)

@@ -138,6 +138,7 @@ int64_t kxc_hip_activity_now_ns(void);
 #define KXC_HIP_CONV_BIAS 1u       /* + bias[o]              (convolution.cc:72-74)            */
 #define KXC_HIP_CONV_RESIDUAL 2u   /* + residual[n,o,h,w]    (add(conv_out, skip), math.cc:41-47) */
 #define KXC_HIP_CONV_RELU 4u       /* (v > 0) ? v : 0        (nn.h:19-30)                      */
+#define KXC_HIP_CONV_HPOOL 0x10u   /* y is max-pooled along W on the way out; see kxc_hip_conv2d_hpool_supported */
 #define KXC_HIP_CONV_FORCE_DIRECT 0x100u /* use the one-thread-per-output kernel (reference order) */
 
 /* nn_conv2d: Conv2DCompute (src/relay/op/nn/convolution.cc:38-75) ->
@@ -190,6 +191,22 @@ const char* kxc_hip_conv2d_pair_variant(const kxc_hip_conv2d_desc* desc);
 int32_t kxc_hip_conv2d_pair_nchw_f32(const kxc_hip_conv2d_desc* desc, const float* x, const float* w,
                                      const float* bias, const float* residual, float* y, const float* w2,
                                      const float* bias2, float* y2, void* stream);
+
+/* nn_conv2d -> nn_relu -> nn_max_pool2d(3x3, stride 2, padding 1) (test/resnet18_ir_dump.cpp:281-291; MaxPool2DCompute,
+ * src/relay/op/nn/pooling.cc:50-67 -> topi::pool2d, include/te/topi/nn.h:161-258): a maximum over a 3x3 window is
+ * the maximum over three rows of the maxima over three columns, so the convolution kernel can take the column
+ * maxima while an output row is still in registers.  With KXC_HIP_CONV_HPOOL in desc->flags
+ * (kxc_hip_conv2d_nchw_f32 and kxc_hip_plan_add_conv2d) y is [n,o,oh,ow/2] with
+ *   y[n,o,oh,pw] = max(v[2pw-1], v[2pw], v[2pw+1]),  v = relu(conv + bias) of row (n,o,oh),  v[-1] left out,
+ * half the bytes of the unpooled map; kxc_hip_pool2d_f32 with a 3x1 window, stride (2,1) and padding (1,0,1,0)
+ * finishes the pool.  Every value is a ReLU result (>= +0, never NaN), so the pooling pad candidate of the
+ * reference never wins and the two-step maximum equals the 3x3 one bit for bit.
+ *   ..._supported: 1 when a kernel with that epilogue covers the shape: KXC_HIP_CONV_RELU set, no residual, an even
+ *   output width that divides the kernel's 224-pixel tile (7x7 filters: 112, 56, 32, 16 ...), n*oh*ow a multiple of 224.
+ *   ..._preferred: ... and the library expects conv + column pool to beat conv + 3x3 pool (KXC_HIP_CONV_HPOOL=0/1 in
+ *   the environment overrides the rule). */
+int32_t kxc_hip_conv2d_hpool_supported(const kxc_hip_conv2d_desc* desc);
+int32_t kxc_hip_conv2d_hpool_preferred(const kxc_hip_conv2d_desc* desc);
 
 /* nn_conv2d with a 3x3 filter, stride 1, dilation 1 and c % 4 == 0 as Winograd F(2x2, 3x3) on the matrix cores:
  * same operator and epilogue as kxc_hip_conv2d_nchw_f32 (convolution.cc:38-75, nn.h:107-158) with 2.25x fewer
@@ -260,7 +277,7 @@ typedef struct kxc_hip_qconv2d_desc {
     int32_t o, kh, kw;
     int32_t stride_h, stride_w;
     int32_t pad_h, pad_w;
-    uint32_t flags;                  /* KXC_HIP_CONV_BIAS | _RESIDUAL | _RELU | _FORCE_DIRECT */
+    uint32_t flags;                  /* KXC_HIP_CONV_BIAS | _RESIDUAL | _RELU | _HPOOL | _FORCE_DIRECT */
     float res_mult;
 } kxc_hip_qconv2d_desc;
 int32_t kxc_hip_qconv2d_nchw_i8(const kxc_hip_qconv2d_desc* desc, const int8_t* x, const int8_t* w,

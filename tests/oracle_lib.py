@@ -87,12 +87,14 @@ class Oracle:
         N, Cc, H, W = x.shape
         if np.isscalar(pad):
             pad = (pad, pad, pad, pad)
-        hn = H + pad[0] + pad[2] - k; wn = W + pad[1] + pad[3] - k
-        OH = (hn + s - 1) // s + 1 if ceil_mode else hn // s + 1
-        OW = (wn + s - 1) // s + 1 if ceil_mode else wn // s + 1
+        kh, kw = (k, k) if np.isscalar(k) else k                  # (window and stride: one number or (rows, columns))
+        sh, sw = (s, s) if np.isscalar(s) else s
+        hn = H + pad[0] + pad[2] - kh; wn = W + pad[1] + pad[3] - kw
+        OH = (hn + sh - 1) // sh + 1 if ceil_mode else hn // sh + 1
+        OW = (wn + sw - 1) // sw + 1 if ceil_mode else wn // sw + 1
         y = np.empty((N, Cc, OH, OW), np.float32)
         self.lib.kxc_oracle_pool2d_f32(_ptr(x, _f32p), _ptr(y, _f32p), _i64(N), _i64(Cc), _i64(H), _i64(W),
-                                       _int(k), _int(k), _int(s), _int(s),
+                                       _int(kh), _int(kw), _int(sh), _int(sw),
                                        _int(pad[0]), _int(pad[1]), _int(pad[2]), _int(pad[3]),
                                        _int(int(ceil_mode)), _int(int(avg)))
         return y

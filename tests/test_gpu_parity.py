@@ -782,6 +782,87 @@ def test_maxpool_edge_semantics(pkg, orc):
         assert_bit_exact(host(pkg.pool2d(dev(x), k, s, p, avg=True)), orc.pool2d(x, k, s, p, avg=True), "avg")
 
 
+def test_column_maxpool_bit_exact(pkg, fast_orc, orc, synth):
+    """The 3x1 window with stride (2,1) that finishes a 3x3/2 max pool whose column maxima were taken by the
+    convolution before it: bit for bit against the CPU checker, on the first layer's half-width map (four rows per
+    thread), small maps (one row per thread), odd heights, and values below the -1e30 pad candidate."""
+    x = synth.uniform((4, 64, 112, 56), 2100)
+    assert_bit_exact(host(pkg.pool2d(dev(x), (3, 1), (2, 1), (1, 0, 1, 0))), fast_orc.pool2d(x, (3, 1), (2, 1), (1, 0, 1, 0)), "column pool")
+    for i, shape in enumerate([(1, 64, 112, 56), (2, 3, 14, 24), (1, 5, 7, 8), (3, 2, 9, 4), (1, 1, 2, 4)]):
+        xs = synth.uniform(shape, 2110 + i)
+        for pad in ((1, 0, 1, 0), (1, 0, 0, 0)):
+            assert_bit_exact(host(pkg.pool2d(dev(xs), (3, 1), (2, 1), pad)), fast_orc.pool2d(xs, (3, 1), (2, 1), pad), "column pool %s %s" % (shape, pad))
+    x = np.full((1, 2, 8, 8), -3e30, np.float32)
+    x[0, 1, 3, 2] = np.nan
+    assert_bit_exact(host(pkg.pool2d(dev(x), (3, 1), (2, 1), (1, 0, 1, 0))), orc.pool2d(x, (3, 1), (2, 1), (1, 0, 1, 0)), "pad candidate, NaN")
+    # a width that is not a multiple of four takes the generic kernel
+    xs = synth.uniform((2, 3, 10, 6), 2130)
+    assert_bit_exact(host(pkg.pool2d(dev(xs), (3, 1), (2, 1), (1, 0, 1, 0))), fast_orc.pool2d(xs, (3, 1), (2, 1), (1, 0, 1, 0)), "generic")
+
+
+HPOOL_SHAPES = [(2, 3, 224, 224, 64, 7, 2, 3), (2, 3, 112, 112, 48, 7, 2, 3), (7, 3, 64, 64, 64, 7, 2, 3), (1, 5, 31, 56, 80, 7, 2, 3)]
+
+
+@pytest.mark.parametrize("shape", HPOOL_SHAPES, ids=lambda s: "x".join(map(str, s)))
+@pytest.mark.parametrize("variant", ["mfma_k7x7_t1_o2x1_p2x7", "mfma_k7x7_t1_o1x2_p7x1"])
+def test_conv_with_column_maxima_in_the_epilogue(pkg, fast_orc, synth, monkeypatch, shape, variant):
+    """KXC_HIP_CONV_HPOOL: conv -> bias -> relu with the maximum over the three columns of every 3x3/2 pooling window
+    taken in the convolution's epilogue, then the 3x1 column pool: against the CPU checker's
+    pool2d(relu(conv2d + bias)) within the matrix-core tolerance, and bit for bit against the same kernel family
+    without the epilogue followed by the 3x3 pool (the maximum is exact, so only the convolution's rounding is in
+    play and that is the same in both).  Both tiles that have the epilogue."""
+    n, c, h, w, o, k, s, p = shape
+    monkeypatch.setenv("KXC_HIP_CONV_HPOOL_VARIANT", variant)
+    if not pkg.conv2d_hpool_supported((n, c, h, w), (o, c, k, k), s, p):
+        pytest.skip("tile %s does not cover %s" % (variant, shape,))
+    flags = pkg.CONV_BIAS | pkg.CONV_RELU | pkg.CONV_HPOOL
+    assert pkg.conv2d_variant((n, c, h, w), (o, c, k, k), s, p, 1, flags) == variant
+    seed = 2200 + HPOOL_SHAPES.index(shape) * 5
+    x = synth.uniform((n, c, h, w), seed)
+    wt = synth.normal((o, c, k, k), seed + 1, float(np.sqrt(2.0 / (c * k * k))))
+    b = synth.uniform((o,), seed + 2, -0.1, 0.1)
+    half = pkg.conv2d(dev(x), dev(wt), dev(b), None, s, p, 1, True, hpool=True)
+    oh, ow = (h + 2 * p - k) // s + 1, (w + 2 * p - k) // s + 1
+    assert tuple(half.shape) == (n, o, oh, ow // 2)
+    got = pkg.pool2d(half, (3, 1), (2, 1), (1, 0, 1, 0))
+    want = fast_orc.pool2d(fast_orc.conv_chain(x, wt, b, s, p, None, True), 3, 2, 1)
+    assert_close(host(got), want, what=variant)
+    # the same tile without the epilogue, then the whole 3x3 window (a 64-channel tile is not taken for fewer channels)
+    if o < 64:
+        return
+    monkeypatch.setenv("KXC_HIP_CONV_VARIANT", variant)
+    monkeypatch.setenv("KXC_HIP_CONV_GSPLIT", "1")        # (a small unpooled launch would split its reduction over workgroups)
+    assert pkg.conv2d_variant((n, c, h, w), (o, c, k, k), s, p) == variant
+    full = pkg.conv2d(dev(x), dev(wt), dev(b), None, s, p, 1, True)
+    assert torch.equal(half, torch.nn.functional.max_pool2d(full, (1, 3), (1, 2), (0, 1)))
+    assert torch.equal(got, pkg.pool2d(full, 3, 2, 1))
+
+
+def test_conv_column_maxima_refusals_and_full_batch(pkg, synth):
+    """Shapes the epilogue does not cover are reported and refused; at the benchmark's batch the two launches equal
+    convolution + 3x3 pool bit for bit on every image (first-layer shape, both shares' batch)."""
+    w7 = (64, 3, 7, 7)
+    assert pkg.conv2d_hpool_supported((64, 3, 224, 224), w7, 2, 3)
+    assert pkg.conv2d_hpool_supported((64, 3, 224, 224), w7, 2, 3, preferred=True)
+    assert not pkg.conv2d_hpool_supported((2, 3, 224, 224), w7, 2, 3, preferred=True)       # too few tiles to pay
+    assert not pkg.conv2d_hpool_supported((1, 3, 64, 64), w7, 2, 3)                          # 1024 pixels: not whole tiles
+    assert not pkg.conv2d_hpool_supported((2, 3, 222, 222), w7, 2, 3)                        # 111 columns: odd
+    assert not pkg.conv2d_hpool_supported((2, 64, 56, 56), (64, 64, 3, 3), 1, 1)             # no 3x3 kernel has it
+    assert not pkg.conv2d_hpool_supported((2, 3, 224, 224), w7, 2, 3, flags=pkg.CONV_BIAS)   # needs the ReLU
+    assert not pkg.conv2d_hpool_supported((2, 3, 224, 224), w7, 2, 3, flags=pkg.CONV_BIAS | pkg.CONV_RELU | pkg.CONV_RESIDUAL)
+    x = dev(synth.uniform((1, 3, 64, 64), 2300)); w = dev(synth.normal(w7, 2301, 0.1)); b = dev(synth.uniform((64,), 2302))
+    with pytest.raises(pkg.KxcHipError, match="pooling epilogue"):
+        pkg.conv2d(x, w, b, None, 2, 3, 1, True, hpool=True)
+    with pytest.raises(pkg.KxcHipError, match="pooling epilogue"):
+        pkg.conv2d(dev(synth.uniform((2, 3, 224, 224), 2303)), w, b, None, 2, 3, 1, False, hpool=True)
+    for batch in (32, 64):
+        xb = dev(synth.uniform((batch, 3, 224, 224), 2310 + batch))
+        got = pkg.pool2d(pkg.conv2d(xb, w, b, None, 2, 3, 1, True, hpool=True), (3, 1), (2, 1), (1, 0, 1, 0))
+        want = pkg.pool2d(pkg.conv2d(xb, w, b, None, 2, 3, 1, True), 3, 2, 1)
+        assert torch.equal(got, want)
+        del got, want, xb
+
+
 def test_add_relu_full_size(pkg, fast_orc, synth):
     a = synth.uniform((64, 128, 28, 28), 2010); b = synth.uniform((64, 128, 28, 28), 2011)
     got = host(pkg.binary(0, dev(a), dev(b), relu=True))

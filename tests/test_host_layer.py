@@ -183,7 +183,16 @@ def test_resnet18_hip_plan_without_gpu():
     assert len(plan["nodes"]) == 20 and plan["schema_version"] == 1
     syms = [n["kernel_symbol"] for n in plan["nodes"]]
     assert sum("+add+relu" in s for s in syms) == 8          # residual tails folded into convolutions
-    assert sum(s.startswith("kxc_conv2d") and s.endswith("+bias+relu") for s in syms) == 6
+    assert sum(s.startswith("kxc_conv2d") and s.endswith("+bias+relu") for s in syms) == 5
+    # the first convolution takes the column maxima of the 3x3/2 max pool behind it; a 3x1 pool finishes the window
+    assert syms[0].endswith("+bias+relu+maxpool3w") and syms[1] == "kxc_max_pool2d_f32"
+    assert [n["op_name"] for n in plan["nodes"][:2]] == ["nn_conv2d", "nn_max_pool2d"]
+    assert plan["nodes"][0]["output_values"] == plan["nodes"][1]["input_values"] == plan["nodes"][1]["output_values"]
+    with tempfile.TemporaryDirectory() as d:
+        run("resnet18", "hip", d, "64", "224", env={"KXC_HIP_FUSE_POOL": "0", "KXC_HIP_BATCH_LANES": "1"})
+        unfused = json.load(open(os.path.join(d, "plan.json")))
+    assert len(unfused["nodes"]) == 20 and unfused["nodes"][0]["kernel_symbol"].endswith("+bias+relu")
+    assert unfused["nodes"][0]["output_values"] != unfused["nodes"][1]["output_values"]
     # each block's 1x1 downsample is the second output of the block's first 3x3/2 convolution
     pairs = [n for n in plan["nodes"] if n["kernel_symbol"].endswith("_ds+bias+relu|conv1x1+bias")]
     assert len(pairs) == 3 and all(len(n["output_values"]) == 2 and len(n["input_values"]) == 5 for n in pairs)
@@ -203,8 +212,10 @@ def test_resnet18_hip_plan_without_gpu():
     with tempfile.TemporaryDirectory() as d:
         run("resnet18", "hip", d, "1", "224")
         one = json.load(open(os.path.join(d, "plan.json")))
-    # batch 1: the same thirteen layers (small launches split their input channels over workgroups)
+    # batch 1: the same thirteen layers (small launches split their input channels over workgroups); too few tiles
+    # for the first layer's pooling epilogue to pay
     assert sum("winograd" in n["kernel_symbol"] for n in one["nodes"]) == 13
+    assert not any("maxpool3w" in n["kernel_symbol"] for n in one["nodes"])
     with tempfile.TemporaryDirectory() as d:
         run("resnet18", "hip", d, "1", "224", env={"KXC_HIP_WINOGRAD_MIN_WORK": "512"})
         few = json.load(open(os.path.join(d, "plan.json")))
@@ -229,7 +240,9 @@ def test_quantised_resnet18_hip_plan_without_gpu():
     assert len(sym) == 21 and len(plan["nodes"]) == 21 and len(plan["constant_value_ids"]) == 63 and mod.num_args == 65
     assert sym[0] == "qnn_quantize kxc_quantize_f32_nchw_to_c4_i8" and sym[1].startswith("qnn_conv2d kxc_qconv2d_c4_i8:qmfma")
     assert sym[2] == "nn_max_pool2d kxc_max_pool2d_c16_i8"
-    assert all(s.startswith("qnn_conv2d kxc_qconv2d_c16_i8:qmfma") for s in sym[3:19])
+    assert all(s.startswith(("qnn_conv2d kxc_qconv2d_c16_i8:qmfma", "qnn_conv2d kxc_qconv2d_c16_i8:qrows")) for s in sym[3:19])
+    # the four 56 x 56 stride-1 layers take the kernel with the 64-position row pitch
+    assert [":qrows_k3x3" in s for s in sym[3:19]] == [True] * 4 + [False] * 12
     assert sum(s.endswith("+relu|qconv1x1+bias") for s in sym) == 3 and sum(s.endswith("+add+relu") for s in sym) == 8
     pairs = [n for n in plan["nodes"] if "|qconv1x1" in n["kernel_symbol"]]
     assert all(len(n["output_values"]) == 2 and len(n["input_values"]) == 7 for n in pairs)
@@ -387,6 +400,12 @@ def test_resnet18_benchmarked_plan_batch64_matches_oracle(synth):
     assert_close(eager, whole, what="two shares of the batch against the batch in one share", floor="scale")
     assert float(np.max(np.abs(eager - whole))) <= 1e-4 * float(np.max(np.abs(whole)))
     assert_bit_exact(whole_replay, whole, "graph replay of the one-share plan")
+    # the first layer's pooling epilogue: the same logits bit for bit as convolution + 3x3 pool (the maximum is exact
+    # and the 64 x 448 and 64 x 256 tiles add a pixel's products in the same order)
+    assert syms[0].endswith("+bias+relu+maxpool3w")
+    _, _, unfused, _, unfused_facts = _compiled_resnet18_logits(synth, 4, 64, env={"KXC_HIP_FUSE_POOL": "0"})
+    assert not any("maxpool3w" in s for s in unfused_facts["launches"])
+    assert_bit_exact(unfused, eager, "with and without the pooling epilogue")
     orc = Oracle(fast=True)
     for n in (0, 63):
         want = orc.resnet18(x[n:n + 1], consts)
