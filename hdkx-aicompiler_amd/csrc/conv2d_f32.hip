@@ -763,6 +763,12 @@ struct Variant {
 // 256 CUs well.  Per filter size the table is in order of preference; Select() takes the first
 // entry that fits the shape, except that launches too small to fill the GPU take the entry with
 // the most workgroups.
+//
+// Register-blocked tiles for the three 3x3 stride-2 launches with a second output (a wave keeps 32 channels x 64 to
+// 224 pixels of both outputs), forced one layer at a time inside the batch-64 network: every one slower than the
+// table's choice (64 x 128 in four waves of 32 x 64: the 28 x 28 layer's pass 1.567 -> 1.609 ms; 64 x 256 in eight
+// waves of 32 x 64 on the 56 x 56 layer: 1.567 -> 1.579 ms; 32 x 224 per wave: four to ten times slower, the two
+// accumulator sets no longer fit the registers).  Only the 3-channel first layer gains from blocking (see below).
 const Variant kVariants[] = {
     KXC_VARIANT_DS(3, 3, 4, 1, 4, 1, 1, 4),   // 32 x 128, 4 waves            (default)
     KXC_VARIANT_DS(3, 3, 4, 1, 8, 1, 1, 2),   // 32 x 256, 8 waves            (14x14 maps: fewer weight refills)
