@@ -53,7 +53,25 @@ def build(verbose=True):
         raise RuntimeError("link failed:\n" + r.stderr)
     if verbose:
         print("built", LIB)
+    build_rocprof_tool(verbose)
     return LIB
+
+
+def build_rocprof_tool(verbose=True):
+    """libkxc_hip_rocprof.so: the rocprofiler-sdk tool library behind kxc_hip_activity_enable(2).  Host code only;
+    loaded on request, never linked into libkxc_hip.so."""
+    rocm = os.environ.get("ROCM_PATH", "/opt/rocm")
+    out = os.path.join(LIBDIR, "libkxc_hip_rocprof.so")
+    cmd = [os.environ.get("CXX", "g++"), "-std=c++17", "-O2", "-fPIC", "-shared", "-Wall", "-D__HIP_PLATFORM_AMD__",
+           "-I" + os.path.join(ROOT, "include"), "-I" + os.path.join(rocm, "include"),
+           os.path.join(CSRC, "rocprof_tool.cpp"), "-o", out,
+           "-L" + os.path.join(rocm, "lib"), "-lrocprofiler-sdk", "-Wl,-rpath," + os.path.join(rocm, "lib")]
+    r = subprocess.run(cmd, capture_output=True, text=True)
+    if r.returncode != 0:
+        raise RuntimeError("building libkxc_hip_rocprof.so failed:\n" + r.stderr)
+    if verbose:
+        print("built", out)
+    return out
 
 
 if __name__ == "__main__":

@@ -4,6 +4,13 @@
 // from the library's own call sites instead of a tool library: every HIP runtime call of the device API and the
 // module loader is timed on the host, and every copy, fill and kernel launch they enqueue is bracketed by two HIP
 // events on its stream.  Off by default and free while off (one relaxed atomic load per call).
+//
+// Mode 2 takes the records from rocprofiler-sdk instead (libkxc_hip_rocprof.so, rocprof_tool.cpp): buffered tracing
+// of kernel dispatches, memory copies and HIP runtime calls of the WHOLE process, which is what the reference's
+// adapter does with CUPTI.  The tool library is loaded on request only, and it has to be registered before the
+// process makes its first HIP call.
+#include <dlfcn.h>
+
 #include <atomic>
 #include <chrono>
 #include <mutex>
@@ -30,7 +37,12 @@ struct State {
     std::vector<Pending> pending;
     hipEvent_t base = nullptr;      // recorded and waited for at enable: GPU time zero
     int64_t base_host_ns = 0;
+    uint64_t dropped = 0;           // device records not kept because kMaxPending were already waiting for a drain
 };
+constexpr size_t kMaxPending = 1u << 16;
+// hipEventElapsedTime returns float milliseconds: 24 bits of mantissa are a microsecond at 16 s from the base event
+// and worse beyond, so the base is renewed when it is older than this and no record still refers to it
+constexpr int64_t kBaseMaxAgeNs = 4000000000LL;
 State& S() {
     static State* s = new State();  // never destroyed: records may arrive during process exit
     return *s;
@@ -52,6 +64,52 @@ void Fill(kxc_hip_activity_record* r, int32_t kind, const char* name) {
 }
 
 thread_local int t_suppress = 0;
+
+// ---- mode 2: the rocprofiler-sdk tool library, loaded from this library's own directory
+struct SdkTool {
+    void* handle = nullptr;
+    int32_t (*prepare)() = nullptr;
+    int32_t (*start)() = nullptr;
+    int32_t (*stop)() = nullptr;
+    int32_t (*drain)(kxc_hip_activity_record*, int32_t, int32_t*) = nullptr;
+    const char* (*status)() = nullptr;
+    std::string error;
+    bool running = false;
+};
+SdkTool& Sdk() {
+    static SdkTool* t = new SdkTool();
+    return *t;
+}
+
+// (caller holds S().mu or runs before main)
+bool LoadSdkTool() {
+    SdkTool& t = Sdk();
+    if (t.handle) return true;
+    Dl_info info;
+    std::string path = "libkxc_hip_rocprof.so";
+    if (dladdr(reinterpret_cast<const void*>(&LoadSdkTool), &info) && info.dli_fname) {
+        const std::string self = info.dli_fname;
+        const size_t slash = self.rfind('/');
+        if (slash != std::string::npos) path = self.substr(0, slash + 1) + path;
+    }
+    void* h = dlopen(path.c_str(), RTLD_NOW | RTLD_GLOBAL);
+    if (!h) { t.error = std::string("cannot load ") + path + ": " + dlerror(); return false; }
+    t.prepare = reinterpret_cast<int32_t (*)()>(dlsym(h, "kxc_rocprof_prepare"));
+    t.start = reinterpret_cast<int32_t (*)()>(dlsym(h, "kxc_rocprof_start"));
+    t.stop = reinterpret_cast<int32_t (*)()>(dlsym(h, "kxc_rocprof_stop"));
+    t.drain = reinterpret_cast<int32_t (*)(kxc_hip_activity_record*, int32_t, int32_t*)>(dlsym(h, "kxc_rocprof_drain"));
+    t.status = reinterpret_cast<const char* (*)()>(dlsym(h, "kxc_rocprof_status"));
+    if (!t.prepare || !t.start || !t.stop || !t.drain || !t.status) { t.error = path + " lacks the kxc_rocprof_* entry points"; dlclose(h); return false; }
+    t.handle = h;
+    return true;
+}
+
+// KXC_PROFILE_GPU_ACTIVITY=2 in the environment: register the tool while this library is being loaded, which is
+// before any HIP call this library makes (a failure shows when mode 2 is asked for).
+__attribute__((constructor)) void RegisterSdkToolEarly() {
+    const char* e = std::getenv("KXC_PROFILE_GPU_ACTIVITY");
+    if (e && e[0] == '2' && e[1] == 0 && LoadSdkTool()) (void)Sdk().prepare();
+}
 
 }  // namespace
 
@@ -109,6 +167,13 @@ DeviceScope::~DeviceScope() {
         (void)hipGetLastError();
     }
     std::lock_guard<std::mutex> lock(S().mu);
+    if (S().pending.size() >= kMaxPending) {
+        // nobody drains: keep the newest kMaxPending device records' worth of events at most
+        if (p.start) (void)hipEventDestroy(p.start);
+        if (p.stop) (void)hipEventDestroy(p.stop);
+        ++S().dropped;
+        return;
+    }
     S().pending.push_back(p);
 }
 
@@ -121,6 +186,37 @@ extern "C" {
 int32_t kxc_hip_activity_enable(int32_t enable) {
     State& s = S();
     std::lock_guard<std::mutex> lock(s.mu);
+    KXC_HIP_REQUIRE(enable >= 0 && enable <= 2, "kxc_hip_activity_enable: mode %d (0 off, 1 call sites of this library, 2 rocprofiler-sdk)", enable);
+    SdkTool& tool = Sdk();
+    if (enable != 2 && tool.running) {
+        (void)tool.stop();
+        tool.running = false;
+    }
+    if (enable == 2) {
+        // no HIP call before the tool is registered
+        g_on.store(false);
+        KXC_HIP_REQUIRE(LoadSdkTool(), "kxc_hip_activity_enable(2): %s", tool.error.c_str());
+        KXC_HIP_REQUIRE(tool.prepare() == 0, "kxc_hip_activity_enable(2): %s", tool.status());
+        KXC_HIP_REQUIRE(tool.start() == 0, "kxc_hip_activity_enable(2): %s", tool.status());
+        // A tool registered after the HIP runtime initialised is accepted by rocprofiler-sdk and then never hears of
+        // anything.  One harmless runtime call shows which case this is: its record has to come back.
+        int version = 0;
+        (void)hipDriverGetVersion(&version);
+        bool heard = false;
+        for (int tries = 0; tries < 40 && !heard; ++tries) {
+            int32_t m = 0;
+            heard = tool.drain(nullptr, 0, &m) == 0 && m > 0;
+            if (!heard) std::this_thread::sleep_for(std::chrono::milliseconds(5));
+        }
+        if (!heard) {
+            (void)tool.stop();
+            KXC_HIP_REQUIRE(false, "kxc_hip_activity_enable(2): rocprofiler-sdk does not see this process's HIP calls -- the tool was "
+                                   "registered after the HIP runtime had initialised; ask for mode 2 before the first HIP call "
+                                   "(or set KXC_PROFILE_GPU_ACTIVITY=2 in the environment)");
+        }
+        tool.running = true;
+        return KXC_HIP_OK;
+    }
     if (enable) {
         if (!s.base) {
             // GPU time zero: an event that has completed, and the host time at which it was seen complete
@@ -158,6 +254,23 @@ int32_t kxc_hip_activity_drain(kxc_hip_activity_record* records, int32_t capacit
         s.done.push_back(p.rec);
     }
     s.pending.clear();
+    if (s.base && g_on.load() && NowNs() - s.base_host_ns > kBaseMaxAgeNs) {
+        if (hipEventRecord(s.base, nullptr) == hipSuccess && hipEventSynchronize(s.base) == hipSuccess) s.base_host_ns = NowNs();
+        else (void)hipGetLastError();
+    }
+    // mode 2: what rocprofiler-sdk has delivered so far (timed_on_gpu = 2 marks the source)
+    SdkTool& tool = Sdk();
+    if (tool.handle) {
+        int32_t m = 0;
+        if (tool.drain(nullptr, 0, &m) == 0 && m > 0) {
+            std::vector<kxc_hip_activity_record> more(static_cast<size_t>(m) + 256);
+            if (tool.drain(more.data(), static_cast<int32_t>(more.size()), &m) == 0)
+                for (int32_t i = 0; i < m; ++i) {
+                    if (more[static_cast<size_t>(i)].timed_on_gpu) more[static_cast<size_t>(i)].timed_on_gpu = 2;
+                    s.done.push_back(more[static_cast<size_t>(i)]);
+                }
+        }
+    }
     const int32_t n = static_cast<int32_t>(s.done.size());
     *count = n;
     if (capacity == 0) return KXC_HIP_OK;           // size query

@@ -9,6 +9,10 @@
 //     so they need no tool library and cost nothing when profiling is off;
 //   * ProfileOptions::enable_gpu_activity replaces enable_cupti, enable_roctx replaces enable_nvtx
 //     (ranges through the roctx library, looked up at run time; absent library = no ranges).
+//     enable_gpu_activity = 2 takes the activity records from rocprofiler-sdk's buffered tracing instead of the
+//     HIP library's own call sites (every HIP call of the process is then seen, as with CUPTI); the context must
+//     be created before the process's first HIP call for that, or KXC_PROFILE_GPU_ACTIVITY=2 set in the
+//     environment.  If the tool cannot be registered any more the context falls back to 1 and records a warning.
 #pragma once
 
 #include <cstdint>
@@ -51,7 +55,7 @@ struct ProfileOptions {
     LogSeverity log_level{LogSeverity::kInfo};
     IRCaptureMode ir_capture_mode{IRCaptureMode::kChangedOrFailed};
     bool enable_roctx{false};
-    bool enable_gpu_activity{true};
+    int enable_gpu_activity{1};       // 0 off, 1 (true) records at the HIP library's call sites, 2 rocprofiler-sdk
     bool record_pass_ir{true};
     bool record_execution_plan_details{true};
     int schema_version{1};
@@ -139,6 +143,8 @@ public:
     // hip_kernel, with the metric keys the reference's CUPTI adapter uses for their CUDA counterparts
     // (src/base/profiling.cc:537-651).  Flush calls it; a caller synchronises its streams first.
     void CollectGpuActivity();
+    // 0: no device activity records; 1: taken at the HIP library's call sites; 2: from rocprofiler-sdk
+    int gpu_activity_mode() const { return gpu_activity_mode_; }
     // The device-side diagnosis rules the reference's offline analyser applies to a bundle (kernel_launch_overhead,
     // copy_dominance, sync_overhead: python/kxc_agent/services/diagnosis_engine.py:233-297, thresholds
     // rule_library.py:22-24), evaluated on the recorded events.
@@ -161,6 +167,7 @@ private:
     };
     std::vector<EventDigest> digests_;
     bool gpu_activity_on_{false};
+    int gpu_activity_mode_{0};        // what Create could switch on: 0, 1 or 2
     bool auto_diagnosed_{false};     // diagnostics_ came from DiagnoseDeviceOverheads, not from PublishDiagnostics
     std::vector<DiagnosticEntry> diagnostics_;
     std::uint64_t run_counter_{0}, span_counter_{0};

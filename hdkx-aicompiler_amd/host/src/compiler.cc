@@ -993,8 +993,9 @@ void CompiledModule::Run(const std::vector<void*>& packed_args) {
         return;
     }
     auto ctx = profiling::CurrentContext();
-    if (ctx && ctx->options().enabled && ctx->options().enable_gpu_activity) {
+    if (ctx && ctx->options().enabled && ctx->options().enable_gpu_activity && ctx->gpu_activity_mode() != 2) {
         // One "runtime" span for the call, one "backend.hip" event per launch from the plan's HIP events.
+        // (With rocprofiler-sdk as the source every dispatch is recorded by the profiler and the plan runs as usual.)
         profiling::EventSpec rspec;
         rspec.component = "runtime";
         rspec.event_type = "kernel_run";

@@ -219,7 +219,8 @@ ProfileOptions ApplyEnvironmentOverrides(ProfileOptions o) {
         else if (s == "verbose") o.ir_capture_mode = IRCaptureMode::kVerbose;
     }
     o.enable_roctx = EnvBool("KXC_PROFILE_ROCTX", o.enable_roctx);
-    o.enable_gpu_activity = EnvBool("KXC_PROFILE_GPU_ACTIVITY", o.enable_gpu_activity);
+    if (const char* v = std::getenv("KXC_PROFILE_GPU_ACTIVITY"); v && v[0] == '2' && v[1] == 0) o.enable_gpu_activity = 2;
+    else o.enable_gpu_activity = EnvBool("KXC_PROFILE_GPU_ACTIVITY", o.enable_gpu_activity != 0) ? std::max(o.enable_gpu_activity, 1) : 0;
     o.record_pass_ir = EnvBool("KXC_PROFILE_RECORD_PASS_IR", o.record_pass_ir);
     o.record_execution_plan_details = EnvBool("KXC_PROFILE_EXEC_PLAN_DETAILS", o.record_execution_plan_details);
     return o;
@@ -321,13 +322,32 @@ ProfileContext::~ProfileContext() {
 std::shared_ptr<ProfileContext> ProfileContext::Create(const ProfileOptions& options) {
     std::shared_ptr<ProfileContext> ctx(new ProfileContext(options));
     if (options.enabled && options.enable_gpu_activity) {
+        std::lock_guard<std::mutex> lock(g_activity_mu);
+        int mode = options.enable_gpu_activity >= 2 ? 2 : 1;
+        std::string why;
+        // (the rocprofiler-sdk tool has to be registered before the first HIP call: nothing may ask the runtime
+        // anything before this)
+        if (mode == 2 && kxc_hip_activity_enable(2) != 0) {
+            why = kxc_hip_last_error();
+            mode = 1;
+        }
         int32_t devices = 0;
-        if (kxc_hip_device_count(&devices) == 0 && devices > 0) {
-            std::lock_guard<std::mutex> lock(g_activity_mu);
-            if (kxc_hip_activity_enable(1) == 0) {
-                ++g_activity_users;
-                ctx->gpu_activity_on_ = true;
-            }
+        if (kxc_hip_device_count(&devices) == 0 && devices > 0 && (mode == 2 || kxc_hip_activity_enable(1) == 0)) {
+            ++g_activity_users;
+            ctx->gpu_activity_on_ = true;
+            ctx->gpu_activity_mode_ = mode;
+        } else if (mode == 2) {
+            kxc_hip_activity_enable(0);
+        }
+        if (!why.empty()) {
+            EventSpec e;
+            e.component = "backend.hip";
+            e.event_type = "activity_source_fallback";
+            e.status = "degraded";
+            e.severity = LogSeverity::kWarn;
+            e.message = "rocprofiler-sdk tracing not available, recording at the HIP library's call sites: " + why;
+            const std::int64_t now = ctx->NowNs();
+            ctx->RecordCompletedSpan(e, "", ctx->NextSpanId(), "", now, now);
         }
     }
     return ctx;
@@ -357,7 +377,7 @@ void ProfileContext::CollectGpuActivity() {
             if (r.return_value != 0) { e.status = "error"; e.severity = LogSeverity::kWarn; }
         } else {
             e.fields["backend.hip.stream_id"] = std::to_string(r.stream);
-            e.fields["backend.hip.timing_source"] = r.timed_on_gpu ? "hip_events" : "host_clock";
+            e.fields["backend.hip.timing_source"] = r.timed_on_gpu == 2 ? "rocprofiler_sdk" : r.timed_on_gpu ? "hip_events" : "host_clock";
         }
         if (r.kind == KXC_HIP_ACTIVITY_MEMCPY) {
             e.fields["backend.hip.copy_kind"] = std::to_string(r.copy_kind);
@@ -495,7 +515,8 @@ void ProfileContext::WriteAllLocked() {
           << IRCaptureModeToString(options_.ir_capture_mode) << "\",\"enable_roctx\":" << (options_.enable_roctx ? "true" : "false")
           << ",\"roctx_available\":" << (RoctxLib().push ? "true" : "false")
           << ",\"enable_gpu_activity\":" << (options_.enable_gpu_activity ? "true" : "false")
-          << ",\"gpu_activity_source\":\"hip_events\",\"record_execution_plan_details\":"
+          << ",\"gpu_activity_source\":\"" << (gpu_activity_mode_ == 2 ? "rocprofiler_sdk" : "hip_events")
+          << "\",\"record_execution_plan_details\":"
           << (options_.record_execution_plan_details ? "true" : "false") << ",\"event_count\":" << event_lines_.size() << "}";
     }
     {

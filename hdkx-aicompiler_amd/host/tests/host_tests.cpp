@@ -879,15 +879,21 @@ int RunProfile(const std::string& dir) {
 // add rounded separately) compiled at run time and launched on the device API's stream, all inside a profiling
 // context; the bundle must then hold backend.hip events of every kind: hip_runtime_api, hip_memcpy, hip_memset,
 // hip_kernel.
-int RunHipSmoke(const std::string& dir) {
+// sdk: the activity records come from rocprofiler-sdk (ProfileOptions::enable_gpu_activity = 2), and the test itself
+// calls hipMemcpyAsync -- outside the HIP library of this build, whose call sites the default mode instruments --
+// and expects that copy in the bundle too.  The context is created before anything asks the HIP runtime a question:
+// a rocprofiler-sdk tool can only be registered before the runtime initialises.
+int RunHipSmoke(const std::string& dir, bool sdk = false) {
     namespace profiling = kxc::profiling;
-    auto target = kxc::BuildTarget(kxc::kGPU);
-    Check(target->attrs.exists == 1, "hip_smoke needs a GPU: " + target->attrs.status);
     profiling::ProfileOptions options;
     options.enabled = true;
     options.bundle_dir = dir;
-    options.enable_gpu_activity = true;
+    options.enable_gpu_activity = sdk ? 2 : 1;
     auto ctx = profiling::ProfileContext::Create(options);
+    auto target = kxc::BuildTarget(kxc::kGPU);
+    Check(target->attrs.exists == 1, "hip_smoke needs a GPU: " + target->attrs.status);
+    if (sdk) Check(ctx->gpu_activity_mode() == 2, std::string("rocprofiler-sdk tracing is not on: ") + kxc_hip_last_error());
+    constexpr size_t kOutsideBytes = 200;       // a size nothing else in this test copies
     const std::string run_id = ctx->NextRunId("hip-smoke");
     {
         profiling::ActivationScope activation(ctx, run_id);
@@ -930,6 +936,15 @@ extern "C" __global__ void scale_add(const float* x, float* y, float alpha, int 
         const uint32_t grid[3] = {static_cast<uint32_t>((n + 127) / 128), 1, 1};
         Check(kxc_hip_module_launch(kernel, grid, block, 0, stream, kernel_args) == 0, std::string("launch: ") + kxc_hip_last_error());
         api->CopyDataFromTo(gpu_out, 0, host_out.data(), 0, nbytes, gpu, cpu, stream);
+        if (sdk) {
+            // a copy the application enqueues itself, straight through the HIP runtime
+            using MemcpyAsync = int (*)(void*, const void*, size_t, int, void*);
+            void* hip = dlopen("libamdhip64.so", RTLD_NOW);
+            Check(hip != nullptr, "dlopen(libamdhip64.so)");
+            auto copy = reinterpret_cast<MemcpyAsync>(dlsym(hip, "hipMemcpyAsync"));
+            Check(copy != nullptr, "dlsym(hipMemcpyAsync)");
+            Check(copy(gpu_buf, host_in.data(), kOutsideBytes, 1 /* hipMemcpyHostToDevice */, stream) == 0, "hipMemcpyAsync from the test");
+        }
         api->StreamSync(gpu, stream);
         kxc_hip_module_free(module);
         for (float v : host_out) Check(v == 8.0f, "Kernel output verification failed");
@@ -942,11 +957,15 @@ extern "C" __global__ void scale_add(const float* x, float* y, float alpha, int 
               "GetAttr");
         Check(kxc::DeviceAPI::NeedSetDevice(kxc::kGPU) && !kxc::DeviceAPI::NeedSetDevice(kxc::kCPU), "NeedSetDevice");
     }
+    if (sdk) std::this_thread::sleep_for(std::chrono::milliseconds(200));      // completion records are delivered by a profiler thread
     ctx->Flush();
     std::ifstream manifest(dir + "/manifest.json");
     std::string manifest_text((std::istreambuf_iterator<char>(manifest)), std::istreambuf_iterator<char>());
     Check(manifest_text.find("\"enable_gpu_activity\":true") != std::string::npos, "manifest marks GPU activity as on");
+    Check(manifest_text.find(sdk ? "\"gpu_activity_source\":\"rocprofiler_sdk\"" : "\"gpu_activity_source\":\"hip_events\"") != std::string::npos,
+          "manifest names the source of the activity records");
     bool saw_runtime = false, saw_memcpy = false, saw_memset = false, saw_kernel = false;
+    bool saw_outside_call = !sdk, saw_outside_copy = !sdk;
     std::ifstream events(dir + "/events.jsonl");
     std::string line;
     while (std::getline(events, line)) {
@@ -955,9 +974,15 @@ extern "C" __global__ void scale_add(const float* x, float* y, float alpha, int 
         saw_memcpy = saw_memcpy || line.find("\"event_type\":\"hip_memcpy\"") != std::string::npos;
         saw_memset = saw_memset || line.find("\"event_type\":\"hip_memset\"") != std::string::npos;
         saw_kernel = saw_kernel || (line.find("\"event_type\":\"hip_kernel\"") != std::string::npos &&
-                                    line.find("\"kernel_symbol\":\"scale_add\"") != std::string::npos);
+                                    line.find("\"kernel_symbol\":\"scale_add\"") != std::string::npos &&
+                                    (!sdk || line.find("\"backend.hip.timing_source\":\"rocprofiler_sdk\"") != std::string::npos));
+        saw_outside_call = saw_outside_call || (line.find("\"event_type\":\"hip_runtime_api\"") != std::string::npos &&
+                                                line.find("\"backend.hip.api\":\"hipMemcpyAsync\"") != std::string::npos);
+        saw_outside_copy = saw_outside_copy || (line.find("\"event_type\":\"hip_memcpy\"") != std::string::npos &&
+                                                line.find("\"bytes\":200") != std::string::npos);
     }
     Check(saw_runtime && saw_memcpy && saw_memset && saw_kernel, "Missing expected HIP activity events");
+    Check(saw_outside_call && saw_outside_copy, "the copy the test enqueued itself is not in the bundle");
     std::cout << "HIP bundle generated at: " << dir << "\n";
     return 0;
 }
@@ -1886,6 +1911,7 @@ int main(int argc, char** argv) {
         if (cmd == "onnx" && argc >= 4) { g_mode = argv[2]; return RunOnnx(argv[3]); }
         if (cmd == "onnx_errors" && argc >= 3) return RunOnnxErrors(argv[2]);
         if (cmd == "hip_smoke" && argc >= 3) return RunHipSmoke(argv[2]);
+        if (cmd == "hip_smoke_sdk" && argc >= 3) return RunHipSmoke(argv[2], true);
         if (cmd == "diagnosis" && argc >= 3) return RunDiagnosis(argv[2]);
         if (cmd == "kernel_object") { g_mode = argc > 2 ? argv[2] : "cpu"; return RunKernelObject(argc > 3 ? argv[3] : ""); }
         if (cmd == "profile" && argc >= 4) { g_mode = argv[2]; return RunProfile(argv[3]); }

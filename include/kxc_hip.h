@@ -105,7 +105,18 @@ int64_t kxc_hip_debug_device_allocations(void);
  * leaves a MEMCPY / MEMSET / KERNEL record timed on the GPU by two HIP events on its stream (timed_on_gpu = 1;
  * synchronous copies are timed on the host).  Times are nanoseconds of the clock kxc_hip_activity_now_ns() reads.
  * correlation_id ties a device record to the API record of the call that enqueued it.  kxc_hip_activity_drain
- * hands over and forgets the finished records, waiting for device records still in flight; capacity 0 only counts. */
+ * hands over and forgets the finished records, waiting for device records still in flight; capacity 0 only counts.
+ * At most 65536 device records wait for a drain; later ones are dropped until it comes.
+ *
+ * kxc_hip_activity_enable(mode): 0 off; 1 the call sites of this library, as above; 2 the records come from
+ * rocprofiler-sdk's buffered tracing instead (kernel dispatches, memory copies, HIP runtime calls of the WHOLE
+ * process -- also those the application or another library makes -- timed by the profiler: timed_on_gpu = 2; fills
+ * appear as the runtime call and the fill kernel, there is no MEMSET record).  Mode 2 loads
+ * libkxc_hip_rocprof.so from this library's directory, a rocprofiler-sdk tool (it exports rocprofiler_configure),
+ * and registers it with rocprofiler_force_configure; that only works BEFORE the process's first HIP call, so either
+ * call kxc_hip_activity_enable(2) first thing, or set KXC_PROFILE_GPU_ACTIVITY=2 in the environment (the tool is
+ * then registered while this library loads), or list the tool library in ROCP_TOOL_LIBRARIES.  Too late is an
+ * error that says so; mode 1 still works then. */
 #define KXC_HIP_ACTIVITY_RUNTIME_API 0
 #define KXC_HIP_ACTIVITY_MEMCPY 1
 #define KXC_HIP_ACTIVITY_MEMSET 2

@@ -611,6 +611,69 @@ def test_hip_smoke_bundle_has_every_activity_kind():
     assert diagnosis["diagnostics"] and all({"category", "severity", "component", "summary"} <= set(x) for x in diagnosis["diagnostics"])
 
 
+@pytest.mark.gpu
+def test_hip_smoke_bundle_from_rocprofiler_sdk():
+    """The same smoke test with the activity records taken from rocprofiler-sdk's buffered tracing
+    (ProfileOptions::enable_gpu_activity = 2; the tool library registers itself before the process's first HIP
+    call), which is how the reference's adapter uses CUPTI (src/base/profiling.cc:250-695): the profiler sees the
+    whole process, so a copy the TEST enqueues with hipMemcpyAsync -- outside the HIP library of this build -- is in
+    the bundle next to the library's own three copies, the fill and the kernel, every device record tied to the API
+    call that caused it and timed by the profiler."""
+    with tempfile.TemporaryDirectory() as d:
+        assert "HIP bundle generated at:" in run("hip_smoke_sdk", d)
+        events, manifest, summary = _read_bundle(d)
+    assert manifest["gpu_activity_source"] == "rocprofiler_sdk"
+    hip = [e for e in events if e["component"] == "backend.hip"]
+    by_type = {}
+    for e in hip:
+        by_type.setdefault(e["event_type"], []).append(e)
+    assert set(by_type) == {"hip_runtime_api", "hip_memcpy", "hip_memset", "hip_kernel"}
+    apis = [e["fields"]["backend.hip.api"] for e in by_type["hip_runtime_api"]]
+    assert {"hipMalloc", "hipStreamCreate", "hipMemsetAsync", "hipMemcpyAsync", "hipModuleLaunchKernel", "hipStreamSynchronize", "hipFree"} <= set(apis)
+    assert apis.count("hipMemcpyAsync") == 4                    # three by the device API, one by the test
+    (kernel,) = by_type["hip_kernel"]                           # the runtime's own copy / fill kernels are not listed as kernels
+    assert kernel["kernel_symbol"] == "scale_add" and kernel["device"] == "hip:0" and kernel["duration_ns"] > 0
+    m = kernel["metrics"]
+    assert (m["grid_x"], m["grid_y"], m["grid_z"], m["block_x"], m["block_y"], m["block_z"]) == (1, 1, 1, 128, 1, 1)
+    (fill,) = by_type["hip_memset"]
+    assert fill["metrics"]["bytes"] == 256 and fill["metrics"]["value"] == 0
+    copies = by_type["hip_memcpy"]
+    assert sorted(c["metrics"]["bytes"] for c in copies) == [200, 256, 256, 256]
+    assert sorted(c["fields"]["backend.hip.copy_kind"] for c in copies) == ["0", "0", "0", "1"]
+    device_records = copies + [fill, kernel]
+    assert all(e["fields"]["backend.hip.timing_source"] in ("rocprofiler_sdk", "host_clock") for e in device_records)
+    assert kernel["fields"]["backend.hip.timing_source"] == "rocprofiler_sdk"
+    api_ids = {e["fields"]["backend.hip.correlation_id"] for e in by_type["hip_runtime_api"]}
+    assert all(e["fields"]["backend.hip.correlation_id"] in api_ids for e in device_records)
+
+
+@pytest.mark.gpu
+def test_rocprofiler_sdk_source_is_refused_once_hip_has_initialised(pkg):
+    """A rocprofiler-sdk tool registered after the HIP runtime initialised would never receive a record; the library
+    notices (its probe call does not come back) and says what to do, and the default source still works."""
+    import ctypes as C
+    import torch
+    torch.zeros(4, device="cuda")
+    torch.cuda.synchronize()
+    lib = pkg.lib()
+    assert lib.kxc_hip_activity_enable(2) != 0
+    assert "before the first HIP call" in lib.kxc_hip_last_error().decode()
+    assert lib.kxc_hip_activity_enable(1) == 0
+    try:
+        p = C.c_void_p()
+        assert lib.kxc_hip_alloc(0, C.c_size_t(256), C.c_size_t(64), C.byref(p)) == 0
+        assert lib.kxc_hip_free(0, p) == 0
+        n = C.c_int32(0)
+        assert lib.kxc_hip_activity_drain(None, 0, C.byref(n)) == 0 and n.value >= 2
+        room = n.value + 64
+        records = C.create_string_buffer(room * 208)             # sizeof(kxc_hip_activity_record)
+        assert lib.kxc_hip_activity_drain(records, room, C.byref(n)) == 0
+        names = {records.raw[208 * i + 4:208 * i + 100].split(b"\0", 1)[0] for i in range(n.value)}
+        assert {b"hipMalloc", b"hipFree"} <= names
+    finally:
+        assert lib.kxc_hip_activity_enable(0) == 0
+
+
 def test_bundle_diagnosis_rules_cpu():
     """kernel_launch_overhead / copy_dominance / sync_overhead as the reference's bundle analyser defines them
     (python/kxc_agent/services/diagnosis_engine.py:233-297), evaluated when a bundle is written."""
