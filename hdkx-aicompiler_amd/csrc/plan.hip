@@ -145,19 +145,21 @@ void OperandExtents(const Node& n, std::vector<std::pair<kxc_hip_buf, size_t>>* 
             add(n.bufs[4], n.dims[0] * n.dims[1]);
             break;
         case NodeKind::kQConv2D: {
-            // i32[0]: 0 NCHW, 1 c16, 2 c4 input / c16 output, 3 c16 with a second output (params)
+            // i32[0]: 0 NCHW, 1 c16, 2 c4 input / c16 output, 3 c16 with a second output (params),
+            // 4 c4 input / c16 output max-pooled 3x3 / 2 / 1 in the same kernel
             const kxc_hip_qconv2d_desc& d = n.qconv;
             if (d.stride_h <= 0 || d.stride_w <= 0) break;
             const int64_t oh = (static_cast<int64_t>(d.h) + 2 * d.pad_h - d.kh) / d.stride_h + 1;
             const int64_t ow = (static_cast<int64_t>(d.w) + 2 * d.pad_w - d.kw) / d.stride_w + 1;
             const int mode = n.i32[0];
             const int64_t ob = mode == 0 ? d.o : (static_cast<int64_t>(d.o) + 15) / 16 * 16;
-            const int64_t y = static_cast<int64_t>(d.n) * ob * oh * ow;
-            const int64_t xc = mode == 0 ? d.c : mode == 2 ? 4 : (static_cast<int64_t>(d.c) + 15) / 16 * 16;
+            const int64_t y = mode == 4 ? static_cast<int64_t>(d.n) * ob * ((oh - 1) / 2 + 1) * ((ow - 1) / 2 + 1)
+                                        : static_cast<int64_t>(d.n) * ob * oh * ow;
+            const int64_t xc = mode == 0 ? d.c : (mode == 2 || mode == 4) ? 4 : (static_cast<int64_t>(d.c) + 15) / 16 * 16;
             add(n.bufs[0], static_cast<int64_t>(d.n) * xc * d.h * d.w, 1);
             size_t wbytes = static_cast<size_t>(d.o) * d.c * d.kh * d.kw;
             if (mode == 1 || mode == 3) { if (kxc_hip_qconv2d_c16_packed_bytes(&d, &wbytes) != KXC_HIP_OK) wbytes = 0; }
-            if (mode == 2) { if (kxc_hip_qconv2d_c4_packed_bytes(&d, &wbytes) != KXC_HIP_OK) wbytes = 0; }
+            if (mode == 2 || mode == 4) { if (kxc_hip_qconv2d_c4_packed_bytes(&d, &wbytes) != KXC_HIP_OK) wbytes = 0; }
             add(n.bufs[1], static_cast<int64_t>(wbytes), 1);
             add(n.bufs[2], d.o);
             add(n.bufs[3], d.o);
@@ -626,6 +628,18 @@ int32_t kxc_hip_plan_add_qconv2d_c4(kxc_hip_plan* plan, const kxc_hip_qconv2d_de
     return KXC_HIP_OK;
 }
 
+int32_t kxc_hip_plan_add_qconv2d_c4_maxpool(kxc_hip_plan* plan, const kxc_hip_qconv2d_desc* desc, kxc_hip_buf x_c4,
+                                            kxc_hip_buf w_packed, kxc_hip_buf bias, kxc_hip_buf mult, kxc_hip_buf y_c16) {
+    const char* who = "kxc_hip_plan_add_qconv2d_c4_maxpool";
+    KXC_HIP_REQUIRE(desc != nullptr, "%s: desc is NULL", who);
+    KXC_HIP_REQUIRE(kxc_hip_qconv2d_c4_maxpool_supported(desc), "%s: the first-layer kernel with the pool does not cover this shape", who);
+    if (int32_t rc = kxc_hip_plan_add_qconv2d_c4(plan, desc, x_c4, w_packed, bias, mult, y_c16)) return rc;
+    Node& n = plan->nodes.back();
+    n.i32[0] = 4;
+    n.symbol = "kxc_qconv2d_c4_i8:qmfma_k7x7s2_c4+maxpool3x3s2";
+    return KXC_HIP_OK;
+}
+
 int32_t kxc_hip_plan_add_quantize_c4(kxc_hip_plan* plan, int64_t nn, int64_t c, int64_t hw, float scale, kxc_hip_buf x,
                                      kxc_hip_buf q) {
     if (int32_t rc = kxc_hip_plan_add_quantize(plan, nn, scale, x, q)) return rc;
@@ -948,6 +962,12 @@ int32_t RunNode(kxc_hip_plan* plan, Node& n, void** args, void* s) {
                 break;
             }
             case NodeKind::kQConv2D:
+                if (n.i32[0] == 4) {
+                    rc = kxc_hip_qconv2d_c4_maxpool_i8(&n.qconv, static_cast<const int8_t*>(B(0)), static_cast<const int8_t*>(B(1)),
+                                                       static_cast<const int32_t*>(B(2)), static_cast<const float*>(B(3)),
+                                                       static_cast<int8_t*>(B(5)), s);
+                    break;
+                }
                 if (n.i32[0] == 2) {
                     rc = kxc_hip_qconv2d_c4_i8(&n.qconv, static_cast<const int8_t*>(B(0)), static_cast<const int8_t*>(B(1)),
                                                static_cast<const int32_t*>(B(2)), static_cast<const float*>(B(3)),
@@ -1405,6 +1425,8 @@ int32_t kxc_hip_plan_deserialize(const char* text, int32_t device_id, kxc_hip_mo
             (!kxc_hip_conv2d_pair_supported(&n.conv) || n.params.size() != 3 || n.params[0].kind == KXC_HIP_BUF_NONE ||
              n.params[2].kind == KXC_HIP_BUF_NONE))
             return fail("bad convolution-pair node");
+        if (n.kind == NodeKind::kQConv2D && (n.i32[0] < 0 || n.i32[0] > 4 || (n.i32[0] == 4 && !kxc_hip_qconv2d_c4_maxpool_supported(&n.qconv))))
+            return fail("bad int8 convolution node");
         if (n.kind == NodeKind::kQConv2D && n.i32[0] == 3 &&
             (!kxc_hip_qconv2d_c16_pair_supported(&n.qconv) || n.params.size() != 4 || n.params[0].kind == KXC_HIP_BUF_NONE ||
              n.params[2].kind == KXC_HIP_BUF_NONE || n.params[3].kind == KXC_HIP_BUF_NONE))

@@ -92,6 +92,10 @@ struct QArgs {
     int8_t* y2;
     uint32_t w2_bytes;
     int32_t ds_off;
+    // First layer with the 3x3 / stride-2 / padding-1 max pool behind it in the same kernel (qconv_k7s2_c4_pool_kernel):
+    // pooled extents, pooled rows per workgroup, workgroups per image
+    int32_t POH, PW, pool_rows, pool_tiles;
+    FastDiv div_pool_tiles;
 };
 
 typedef unsigned int uintx2 __attribute__((ext_vector_type(2)));
@@ -735,6 +739,165 @@ __global__ void __launch_bounds__(64 * WP) __attribute__((amdgpu_waves_per_eu(2)
         }
     }
     epilogue_c16<RO, 1>(acc, a, ypix, ob0, half);
+}
+
+
+// ------------------------------------------------------------------------------------------
+// First layer AND the max pool behind it (3x3, stride 2, padding 1) in one kernel: int8 c4 input -> the pooled
+// feature map in c16.  The unpooled map (51 MB at batch 64, written once and read once) never exists.
+//
+// A workgroup of four waves owns `pool_rows` pooled rows of one image for RO blocks of 32 output channels and walks
+// the 2*pool_rows + 1 convolution rows they need, top to bottom (neighbouring workgroups compute the row they share
+// twice: 1/(2*pool_rows) more matrix and requantisation work).  Wave w computes convolution columns 30w-1 .. 30w+30
+// of every row -- 32 columns for the 15 pooling windows centred on columns 30w, 30w+2, ..., 30w+28, so that all
+// three columns of a window lie in one wave and no value crosses waves (neighbouring waves overlap by two columns).
+// Per row: seven matrix instructions per channel block, the usual requantisation up to the clamp -- kept as a float
+// because rounding is monotonic: the maximum of the rounded values is the rounded maximum -- the maximum over lanes
+// r-1, r, r+1 (two DPP operands), and the running maximum over rows in registers; after a window's third row the
+// odd lanes round, pack and store their pooled pixel.  Columns and rows outside the convolution's output count as
+// -128, the pooling pad candidate of int8 (the lowest value: it never wins against a real one): a missing column
+// through per-lane clamp bounds, a missing row by not being computed.
+// ------------------------------------------------------------------------------------------
+template <int RO, bool RELU>
+__global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2))) qconv_k7s2_c4_pool_kernel(const QArgs a) {
+    constexpr int KH = 7;
+    constexpr int WP = 4;
+    constexpr int WSEG = RO * KH;
+    extern __shared__ __attribute__((aligned(16))) char lds[];
+    const int tid = threadIdx.x;
+    const int lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int half = lane >> 5;
+    const int r = lane & 31;
+    const int W4 = (a.W >> 2) + 2;                  // 16-byte positions per LDS row
+    const int row_bytes = W4 * 16;
+    const int xs_bytes = a.chs * 16;
+
+    const int tile = (blockIdx.x & 7) * a.tiles_per_xcd + (blockIdx.x >> 3);
+    if (tile >= a.num_tiles || static_cast<int>(blockIdx.x >> 3) >= a.tiles_per_xcd) return;
+    const int p_tile = fast_div(tile, a.div_otiles), o_tile = tile - p_tile * a.o_tiles;
+    const int n = fast_div(p_tile, a.div_pool_tiles), pt = p_tile - n * a.pool_tiles;
+    const int ob0 = o_tile * RO;
+    const int p0 = pt * a.pool_rows, p1 = min(p0 + a.pool_rows, a.POH);       // pooled rows [p0, p1)
+    const int c_lo = max(2 * p0 - 1, 0), c_hi = min(2 * (p1 - 1) + 1, a.OH - 1);   // convolution rows needed
+    const int nrows = 2 * (c_hi - c_lo) + KH;                                 // padded input rows staged
+    const int P = nrows * W4;
+    const int xsegs = (P + 63) >> 6;
+    const __amdgpu_buffer_rsrc_t xr = make_rsrc(a.x, a.x_bytes);
+    const __amdgpu_buffer_rsrc_t wr = make_rsrc(a.wp, a.w_bytes);
+    for (int seg = wave; seg < xsegs; seg += WP) {
+        const int pos = seg * 64 + lane;
+        const int q = fast_div(pos, a.div_wp), c4 = pos - q * W4;
+        const int ih = 2 * c_lo + q - 3;
+        const bool ok = pos < P && ih >= 0 && ih < a.H && c4 >= 1 && c4 <= (a.W >> 2);
+        const uint32_t off = ok ? static_cast<uint32_t>((n * a.H + ih) * a.W + (c4 - 1) * 4) * 4u : kOob;
+        load16_to_lds(xr, (lds_ptr_t)(lds + seg * 1024), off, 0);
+    }
+    for (int seg = wave; seg < WSEG; seg += WP) {
+        const int ro = seg / KH, st = seg - ro * KH;
+        load16_to_lds(wr, (lds_ptr_t)(lds + xs_bytes + seg * 1024), static_cast<uint32_t>(lane) * 16u,
+                      (static_cast<uint32_t>(ob0 + ro) * KH + st) * 1024u);
+    }
+    // this lane's column, its place in an LDS row, and the pooled pixel an odd lane owns
+    const int col = 30 * wave - 1 + r;
+    const bool col_ok = col >= 0 && col < a.OW;
+    const int xcol = min(max(col, 0), a.OW - 1) * 8 + half * 16;
+    const int pw = 15 * wave + (r >> 1);
+    const bool owner = (r & 1) && r <= 29 && pw < a.PW;
+    const bool has_bias = (a.flags & KXC_HIP_CONV_BIAS) != 0;
+    constexpr float kPad = -128.0f;
+    // the clamp's bounds are per lane: a column outside the map clamps to [-128, -128] and so becomes the pad candidate
+    const float lower = col_ok ? (RELU ? 0.0f : -128.0f) : kPad;
+    const float upper = col_ok ? 127.0f : kPad;
+    intx16 bv[RO];
+    float4 mv[RO][4];
+#pragma unroll
+    for (int i = 0; i < RO; ++i)
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+            const int4 b4 = has_bias ? *reinterpret_cast<const int4*>(a.bias + (ob0 + i) * 32 + 8 * j + 4 * half) : make_int4(0, 0, 0, 0);
+            bv[i][4 * j + 0] = b4.x; bv[i][4 * j + 1] = b4.y; bv[i][4 * j + 2] = b4.z; bv[i][4 * j + 3] = b4.w;
+            mv[i][j] = *reinterpret_cast<const float4*>(a.mult + (ob0 + i) * 32 + 8 * j + 4 * half);
+        }
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+    __syncthreads();
+    const char* ws = lds + xs_bytes + lane * 16;
+
+    // One convolution row: for every accumulator register the requantised value before rounding, already the maximum
+    // over the lane's column and its two neighbours, handed to sink(i, g, value).
+    auto conv_row = [&](int c, auto&& sink) {
+        intx16 acc[RO];
+        const char* xrow = lds + 2 * (c - c_lo) * row_bytes + xcol;
+#pragma unroll
+        for (int kh = 0; kh < KH; ++kh) {
+            const int2 lo = *reinterpret_cast<const int2*>(xrow + kh * row_bytes);        // 8-byte aligned
+            const int2 hi = *reinterpret_cast<const int2*>(xrow + kh * row_bytes + 8);
+            intx4 b;
+            b[0] = lo.x; b[1] = lo.y; b[2] = hi.x; b[3] = hi.y;
+#pragma unroll
+            for (int i = 0; i < RO; ++i) {
+                const intx4 wv = *reinterpret_cast<const intx4*>(ws + (i * KH + kh) * 1024);
+                // (the sum starts at the bias: the first instruction takes it as its addend)
+                acc[i] = __builtin_amdgcn_mfma_i32_32x32x32_i8(wv, b, kh == 0 ? bv[i] : acc[i], 0, 0, 0);
+            }
+        }
+#pragma unroll
+        for (int i = 0; i < RO; ++i)
+#pragma unroll
+            for (int gq = 0; gq < 4; ++gq) {
+                const float ms[4] = {mv[i][gq].x, mv[i][gq].y, mv[i][gq].z, mv[i][gq].w};
+#pragma unroll
+                for (int e = 0; e < 4; ++e) {
+                    // (the requantisation of epilogue_c16 up to the clamp)
+                    float v = __fmul_rn(static_cast<float>(acc[i][4 * gq + e]), ms[e]);
+                    if (!RELU) v = (v == v) ? v : 0.0f;
+                    v = __builtin_amdgcn_fmed3f(v, lower, upper);
+                    const int bits = __builtin_bit_cast(int, v);
+                    constexpr int kLowest = static_cast<int>(0xff800000u);      // -inf: what a lane without a neighbour reads
+                    // lane l reads lane l-1 (0x138: whole-wave shift right by one) and lane l+1 (0x130)
+                    const float left = __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(kLowest, bits, 0x138, 0xf, 0xf, false));
+                    const float right = __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(kLowest, bits, 0x130, 0xf, 0xf, false));
+                    sink(i, 4 * gq + e, fmaxf(fmaxf(v, left), right));
+                }
+            }
+    };
+
+    // carry = the row above the next window (row 2p - 1), which is the previous window's last row
+    float carry[RO][16];
+    if (2 * p0 - 1 >= 0) {
+        conv_row(2 * p0 - 1, [&](int i, int g, float v) { carry[i][g] = v; });
+    } else {
+#pragma unroll
+        for (int i = 0; i < RO; ++i)
+#pragma unroll
+            for (int g = 0; g < 16; ++g) carry[i][g] = kPad;
+    }
+    for (int p = p0; p < p1; ++p) {
+        float best[RO][16];
+        conv_row(2 * p, [&](int i, int g, float v) { best[i][g] = fmaxf(carry[i][g], v); });      // (row 2p always exists)
+        if (2 * p + 1 < a.OH)
+            conv_row(2 * p + 1, [&](int i, int g, float v) { best[i][g] = fmaxf(best[i][g], v); carry[i][g] = v; });
+        constexpr float kMagic = 12582912.0f;      // 1.5 * 2^23: the sum's low byte is the rounded value
+#pragma unroll
+        for (int i = 0; i < RO; ++i) {
+            uint32_t w[4];
+#pragma unroll
+            for (int gq = 0; gq < 4; ++gq) {
+                uint32_t t[4];
+#pragma unroll
+                for (int e = 0; e < 4; ++e) t[e] = __builtin_bit_cast(uint32_t, __fadd_rn(best[i][4 * gq + e], kMagic));
+                const uint32_t lo = __builtin_amdgcn_perm(t[1], t[0], 0x0c0c0400u);
+                const uint32_t hi = __builtin_amdgcn_perm(t[3], t[2], 0x0c0c0400u);
+                w[gq] = __builtin_amdgcn_perm(hi, lo, 0x05040100u);
+            }
+            swap_halves(w[0], w[2]);      // (as in epilogue_c16: half 0 ends up with channels 0-15, half 1 with 16-31)
+            swap_halves(w[1], w[3]);
+            if (owner) {
+                const int64_t word = (static_cast<int64_t>((n * (a.O >> 4) + (ob0 + i) * 2 + half) * a.POH + p) * a.PW + pw) * 16;
+                *reinterpret_cast<uintx4*>(a.y + word) = uintx4{w[0], w[2], w[1], w[3]};
+            }
+        }
+    }
 }
 
 // Weights of the first-layer kernel: [o block][kh][lane][16]; lane (o, half), byte j = pixel j/4, channel j%4,
@@ -1580,9 +1743,91 @@ int32_t PrepareK7(const kxc_hip_qconv2d_desc* d, QLaunch* L, const K7Variant** o
     return KXC_HIP_OK;
 }
 
+// The first layer with the max pool in the same kernel: the first-layer conditions, a pooled width the four waves
+// cover (15 windows each), and rows per workgroup chosen so that the launch has about two workgroups per compute
+// unit (KXC_HIP_QPOOL_ROWS forces it).
+struct K7PoolLaunch {
+    QArgs args;
+    void (*kernel)(const QArgs) = nullptr;
+    const char* name = "";
+    int grid = 0;
+    size_t lds_bytes = 0;
+};
+
+int32_t PrepareK7Pool(const kxc_hip_qconv2d_desc* d, K7PoolLaunch* L, const char* who) {
+    QLaunch base;
+    const K7Variant* unused = nullptr;
+    if (int32_t rc = PrepareK7(d, &base, &unused, who)) return rc;
+    QArgs& a = L->args;
+    a = base.args;
+    a.POH = (a.OH - 1) / 2 + 1;       // (OH + 2*1 - 3) / 2 + 1
+    a.PW = (a.OW - 1) / 2 + 1;
+    KXC_HIP_REQUIRE(a.PW <= 60, "%s: the pooled map is %d columns wide, the kernel covers 60", who, a.PW);
+    KXC_HIP_REQUIRE(static_cast<int64_t>(a.N) * a.O * a.POH * a.PW < (1LL << 31), "%s: tensor too large for 32-bit addressing", who);
+    if (a.M == 0) return KXC_HIP_OK;
+    const int ro = (a.O / 32) % 2 == 0 ? 2 : 1;
+    a.o_tiles = (a.O / 32) / ro;
+    const int W4 = a.W / 4 + 2;
+    // measured on the 224 x 224 first layer (us, rows 2 / 3 / 4 / 5 / 7 / 8): batch 16 10.8 / 13.7 / 11.5 / 13.2 / 17.2 /
+    // 19.1, batch 32 19.0 / 19.8 / 17.0 / 20.0 / 17.6 / 19.4, batch 64 30.9 / 30.1 / 30.4 / 29.4 / 27.1 / 29.9, batch 128
+    // 59.1 / 55.9 / 51.2 / 53.8 / 49.8 / 55.3: as many rows as leave about two workgroups per compute unit, at most 7
+    int rows = 1;
+    for (int r = 7; r >= 1; --r) {
+        rows = r;
+        if (static_cast<int64_t>(a.N) * CeilDiv(a.POH, r) * a.o_tiles >= 448) break;
+    }
+    if (const char* e = std::getenv("KXC_HIP_QPOOL_ROWS")) {
+        const int f = std::atoi(e);
+        if (f >= 1 && f <= 16) rows = f;
+    }
+    if (rows > a.POH) rows = a.POH;
+    size_t lds = 0;
+    for (;; --rows) {
+        const int segs = ((4 * rows + 7) * W4 + 63) / 64;
+        lds = static_cast<size_t>(segs) * 1024 + static_cast<size_t>(ro) * 7 * 1024;
+        a.chs = segs * 64;
+        if (lds <= 64 * 1024 || rows == 1) break;
+    }
+    KXC_HIP_REQUIRE(lds <= 64 * 1024, "%s: image rows too wide for the first-layer kernel (width %d)", who, d->w);
+    a.pool_rows = rows;
+    a.pool_tiles = static_cast<int32_t>(CeilDiv(a.POH, rows));
+    a.div_pool_tiles = MakeFastDiv(a.pool_tiles);
+    a.p_tiles = a.N * a.pool_tiles;
+    a.num_tiles = a.p_tiles * a.o_tiles;
+    a.tiles_per_xcd = (a.num_tiles + 7) / 8;
+    a.div_otiles = MakeFastDiv(a.o_tiles);
+    const bool relu = (a.flags & KXC_HIP_CONV_RELU) != 0;
+    L->kernel = ro == 2 ? (relu ? qconv_k7s2_c4_pool_kernel<2, true> : qconv_k7s2_c4_pool_kernel<2, false>)
+                        : (relu ? qconv_k7s2_c4_pool_kernel<1, true> : qconv_k7s2_c4_pool_kernel<1, false>);
+    L->name = ro == 2 ? "qmfma_k7x7s2_c4_o2_maxpool3x3s2" : "qmfma_k7x7s2_c4_o1_maxpool3x3s2";
+    L->grid = a.tiles_per_xcd * 8;
+    L->lds_bytes = lds;
+    return KXC_HIP_OK;
+}
+
 }  // namespace
 
 extern "C" {
+
+int32_t kxc_hip_qconv2d_c4_maxpool_supported(const kxc_hip_qconv2d_desc* d) {
+    if (!d) return 0;
+    K7PoolLaunch L;
+    if (PrepareK7Pool(d, &L, "kxc_hip_qconv2d_c4_maxpool_supported") != KXC_HIP_OK) { LastError().clear(); return 0; }
+    return 1;
+}
+
+int32_t kxc_hip_qconv2d_c4_maxpool_i8(const kxc_hip_qconv2d_desc* d, const int8_t* x_c4, const int8_t* w_packed,
+                                      const int32_t* bias, const float* mult, int8_t* y_c16, void* stream) {
+    K7PoolLaunch L;
+    if (int32_t rc = PrepareK7Pool(d, &L, "kxc_hip_qconv2d_c4_maxpool_i8")) return rc;
+    if (L.args.M == 0) return KXC_HIP_OK;
+    KXC_HIP_REQUIRE(x_c4 && w_packed && mult && y_c16, "kxc_hip_qconv2d_c4_maxpool_i8: NULL pointer");
+    KXC_HIP_REQUIRE(!(d->flags & KXC_HIP_CONV_BIAS) || bias, "kxc_hip_qconv2d_c4_maxpool_i8: bias flag without bias");
+    QArgs& a = L.args;
+    a.x = x_c4; a.wp = w_packed; a.bias = bias; a.mult = mult; a.res = nullptr; a.y = y_c16;
+    hipLaunchKernelGGL(L.kernel, NoteGrid(dim3(L.grid)), NoteBlock(dim3(256)), NoteLds(L.lds_bytes), ResolveStream(stream), a);
+    return CheckLaunch(L.name);
+}
 
 int32_t kxc_hip_qconv2d_c4_packed_bytes(const kxc_hip_qconv2d_desc* d, size_t* out_bytes) {
     KXC_HIP_REQUIRE(d != nullptr && out_bytes != nullptr, "kxc_hip_qconv2d_c4_packed_bytes: NULL argument");

@@ -558,6 +558,27 @@ def qconv2d_c4(x, c, w_packed, w_shape, bias, mult, relu=True):
     return y
 
 
+def qconv2d_c4_maxpool_supported(x_shape, o, c=3, relu=True):
+    n, h, wd, _ = x_shape
+    d = qconv_desc(n, c, h, wd, o, 7, 7, 2, 3, CONV_BIAS | (CONV_RELU if relu else 0))
+    return bool(lib().kxc_hip_qconv2d_c4_maxpool_supported(C.byref(d)))
+
+
+def qconv2d_c4_maxpool(x, c, w_packed, w_shape, bias, mult, relu=True):
+    """First layer and the 3x3 / stride 2 / padding 1 max pool behind it in one kernel; returns the pooled c16 map."""
+    import torch
+    _need(x, torch.int8, "x"); _need(w_packed, torch.int8, "w_packed"); _need(bias, torch.int32, "bias")
+    _need(mult, torch.float32, "mult")
+    n, h, wd, _ = x.shape
+    o = w_shape[0]
+    flags = (CONV_BIAS if bias is not None else 0) | (CONV_RELU if relu else 0)
+    d = qconv_desc(n, c, h, wd, o, 7, 7, 2, 3, flags)
+    oh = (h + 6 - 7) // 2 + 1; ow = (wd + 6 - 7) // 2 + 1
+    y = torch.empty(c16_shape(n, o, (oh - 1) // 2 + 1, (ow - 1) // 2 + 1), dtype=torch.int8, device=x.device)
+    _check(lib().kxc_hip_qconv2d_c4_maxpool_i8(C.byref(d), _p(x), _p(w_packed), _p(bias), _p(mult), _p(y), _stream()))
+    return y
+
+
 def maxpool2d_c16_i8(x, c, k, s, pad):
     import torch
     _need(x, torch.int8, "x")

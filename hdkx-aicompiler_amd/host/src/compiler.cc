@@ -213,6 +213,7 @@ public:
         Number();
         FormGroups();
         AssignLayouts();
+        FusePoolsByLayout();
         if (kxc_hip_plan_create(cfg_->target->device.device_id(), static_cast<int32_t>(num_args_), &m_->plan))
             throw std::runtime_error(std::string("plan creation failed: ") + kxc_hip_last_error());
         // variants are chosen for `lanes` equal launches side by side: by the queries made while the plan is built
@@ -419,6 +420,39 @@ private:
             }
         }
         for (auto& kv : layout_) if (kv.second == relay::kHIPLayoutAny) kv.second = relay::kHIPLayoutPlain;
+    }
+    // Pool fusion that depends on the layouts just assigned (the fp32 one is decided in FormGroups): a call of an
+    // operator with an "FHIPPoolQuery" that stands alone, whose only reader is a pooling call that stands alone, and
+    // whose kernel was given a layout other than plain for its first input -- the int8 first layer on its 4-channel
+    // input.  The pooling call's group dissolves into the convolution's.
+    void FusePoolsByLayout() {
+        if (!cfg_->hip_fuse || !cfg_->hip_use_handwritten) return;
+        const char* pool_env = std::getenv("KXC_HIP_FUSE_POOL");            // "0" switches it off
+        if (pool_env && pool_env[0] == '0') return;
+        for (size_t gi = 0; gi < groups_.size(); ++gi) {
+            Group& g = groups_[gi];
+            if (g.head != g.tail || g.pool || g.residual || g.fused_relu || g.head == f_->body.get()) continue;
+            const auto* op = g.head->op.As<OpNode>();
+            const auto* query = OpAttr<relay::FHIPPoolQuery>(op, "FHIPPoolQuery");
+            auto ch = choice_.find(g.head);
+            if (!query || IsF32(g.head->checked_type_) || ch == choice_.end() || ch->second.inputs.empty() ||
+                ch->second.inputs[0] == relay::kHIPLayoutPlain)
+                continue;
+            const CallNode* n = SoleConsumer(g.head);
+            if (!n || !(IsOp(n, "nn_max_pool2d") || IsOp(n, "nn_avg_pool2d"))) continue;
+            auto pg = group_of_tail_.find(n);
+            if (pg == group_of_tail_.end() || groups_[pg->second].head != n) continue;        // the pool is not on its own
+            auto pch = choice_.find(n);
+            if (pch == choice_.end() || pch->second.inputs.empty() || pch->second.inputs[0] != ch->second.output || LayoutOf(n) != ch->second.output)
+                continue;
+            Array<Type> types;
+            for (const auto& a : g.head->args) types.push_back(a.checked_type());
+            if (!(*query)(g.head->attrs, types, false, false, n->op.As<OpNode>()->name, n->attrs)) continue;
+            group_of_tail_.erase(g.head);
+            group_of_tail_[n] = gi;          // (the pooling call's own group is no longer reachable and is never emitted)
+            g.pool = n;
+            g.tail = n;
+        }
     }
     int LayoutOf(const RelayExprNode* e) const {
         auto it = layout_.find(Resolve(e));

@@ -311,12 +311,26 @@ bool QnnConv2DPairQuery(const Attrs& a_attrs, const Array<Type>& a_inputs, const
     return kxc_hip_qconv2d_c16_pair_supported(&a) != 0;
 }
 
+// The first layer on its 4-channel input followed by nn_max_pool2d(3x3, stride 2, padding 1) as one kernel whose
+// output is the pooled map (asked once the layouts are known: the call's first input is not plain).
+bool QnnConv2DPoolQuery(const Attrs& attrs, const Array<Type>& inputs, bool, bool, const std::string& pool_op, const Attrs& pool_attrs) {
+    kxc_hip_qconv2d_desc d{};
+    const auto* p = pool_attrs.As<MaxPool2DAttrsNode>();
+    if (MatrixCoresDisabled() || pool_op != "nn_max_pool2d" || !p || inputs.size() != 4 || !QnnConvDesc(attrs, inputs, &d)) return false;
+    if (!p->layout.empty() && p->layout != "NCHW") return false;
+    const auto ks = ReadPair(p->pool_size, 1), st = ReadPair(p->strides, 1), pd = ReadPad4(p->padding);
+    if (ks[0] != 3 || ks[1] != 3 || st[0] != 2 || st[1] != 2 || pd[0] != 1 || pd[1] != 1 || pd[2] != 1 || pd[3] != 1 || p->ceil_mode)
+        return false;
+    return kxc_hip_qconv2d_c4_supported(&d) != 0 && kxc_hip_qconv2d_c4_maxpool_supported(&d) != 0;
+}
+
 std::string QnnConv2DDispatch(const HIPDispatchContext& c, kxc_hip_plan* plan) {
     kxc_hip_qconv2d_desc d{};
     if (!QnnConvDesc(c.attrs, c.input_types, &d) || !IsDType(c.out_type, "int8")) return "";
     const bool has_res = c.inputs.size() == 5;
     const kxc_hip_buf none{KXC_HIP_BUF_NONE, 0};
     const int in_layout = c.input_layouts.empty() ? kHIPLayoutPlain : c.input_layouts[0];
+    if (c.has_pool && (in_layout != kHIPLayoutC4 || c.has_pair)) return "";
     if (in_layout == kHIPLayoutPlain) {
         if (c.output_layout != kHIPLayoutPlain || c.has_pair) return "";
         Check(kxc_hip_plan_add_qconv2d(plan, &d, B(c.inputs[0]), B(c.inputs[1]), B(c.inputs[2]), B(c.inputs[3]),
@@ -334,6 +348,11 @@ std::string QnnConv2DDispatch(const HIPDispatchContext& c, kxc_hip_plan* plan) {
         Check(kxc_hip_qconv2d_c4_packed_bytes(&d, &bytes), "qnn_conv2d dispatch");
         const HIPBuffer wp = c.alloc_persistent(static_cast<int64_t>(bytes));
         Check(kxc_hip_plan_add_qconv_weight_pack(plan, KXC_HIP_QPACK_C4, &d, B(c.inputs[1]), B(wp), every_run), "qnn_conv2d weight pack");
+        if (c.has_pool) {
+            Check(kxc_hip_plan_add_qconv2d_c4_maxpool(plan, &d, B(c.inputs[0]), B(wp), B(c.inputs[2]), B(c.inputs[3]), B(c.output)),
+                  "qnn_conv2d dispatch (with the max pool)");
+            return std::string("kxc_qconv2d_c4_i8:qmfma_k7x7s2_c4") + ((d.flags & KXC_HIP_CONV_RELU) ? "+relu" : "") + "+maxpool3x3s2";
+        }
         Check(kxc_hip_plan_add_qconv2d_c4(plan, &d, B(c.inputs[0]), B(wp), B(c.inputs[2]), B(c.inputs[3]), B(c.output)),
               "qnn_conv2d dispatch");
         return std::string("kxc_qconv2d_c4_i8:qmfma_k7x7s2_c4") + ((d.flags & KXC_HIP_CONV_RELU) ? "+relu" : "");
@@ -539,6 +558,7 @@ void EnsureBuiltinOpsRegistered() {
             .set_attr<FRelayToTE>("FRelayToTE", QnnConv2DCompute)
             .set_attr<FHIPLayoutQuery>("FHIPLayoutQuery", QnnConv2DLayout)
             .set_attr<FHIPPairQuery>("FHIPPairQuery", QnnConv2DPairQuery)
+            .set_attr<FHIPPoolQuery>("FHIPPoolQuery", QnnConv2DPoolQuery)
             .set_attr<FHIPDispatch>("FHIPDispatch", QnnConv2DDispatch);
         OpRegEntry::Register("qnn_dense")
             .describe("int8 dense layer with int32 accumulation; float32 output (acc + bias) * mult.")

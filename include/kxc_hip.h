@@ -345,6 +345,14 @@ int32_t kxc_hip_qconv2d_c4_pack_weights(const kxc_hip_qconv2d_desc* desc, const 
                                         void* stream);
 int32_t kxc_hip_qconv2d_c4_i8(const kxc_hip_qconv2d_desc* desc, const int8_t* x_c4, const int8_t* w_packed,
                               const int32_t* bias, const float* mult, int8_t* y_c16, void* stream);
+/* The same first layer followed by nn_max_pool2d with a 3x3 window, stride 2 and padding 1 on all sides (the
+ * chain of test/resnet18_ir_dump.cpp:281-291 in its int8 form) as ONE kernel: y_c16 is the pooled map
+ * [n, o, (oh-1)/2+1, (ow-1)/2+1] in c16, bit for bit what kxc_hip_qconv2d_c4_i8 followed by kxc_hip_maxpool2d_c16_i8
+ * gives (the padding candidate of the int8 pool is -128); the unpooled map is never written.  ..._supported: the
+ * first-layer conditions and a pooled width of at most 60 columns. */
+int32_t kxc_hip_qconv2d_c4_maxpool_supported(const kxc_hip_qconv2d_desc* desc);
+int32_t kxc_hip_qconv2d_c4_maxpool_i8(const kxc_hip_qconv2d_desc* desc, const int8_t* x_c4, const int8_t* w_packed,
+                                      const int32_t* bias, const float* mult, int8_t* y_c16, void* stream);
 int32_t kxc_hip_quantize_f32_nchw_to_c4_i8(const float* x, int8_t* y, int64_t n, int64_t c, int64_t hw,
                                            float scale, void* stream);
 int32_t kxc_hip_maxpool2d_c16_i8(const kxc_hip_pool2d_desc* desc, const int8_t* x, int8_t* y, void* stream);
@@ -450,6 +458,9 @@ int32_t kxc_hip_plan_add_qconv2d_c16_pair(kxc_hip_plan* plan, const kxc_hip_qcon
                                           kxc_hip_buf bias2, kxc_hip_buf mult2, kxc_hip_buf y2);
 int32_t kxc_hip_plan_add_qconv2d_c4(kxc_hip_plan* plan, const kxc_hip_qconv2d_desc* desc, kxc_hip_buf x_c4,
                                     kxc_hip_buf w_packed, kxc_hip_buf bias, kxc_hip_buf mult, kxc_hip_buf y_c16);
+/* kxc_hip_qconv2d_c4_maxpool_i8 as a plan node: y_c16 is the pooled map. */
+int32_t kxc_hip_plan_add_qconv2d_c4_maxpool(kxc_hip_plan* plan, const kxc_hip_qconv2d_desc* desc, kxc_hip_buf x_c4,
+                                            kxc_hip_buf w_packed, kxc_hip_buf bias, kxc_hip_buf mult, kxc_hip_buf y_c16);
 int32_t kxc_hip_plan_add_quantize_c4(kxc_hip_plan* plan, int64_t n, int64_t c, int64_t hw, float scale,
                                      kxc_hip_buf x, kxc_hip_buf q);
 int32_t kxc_hip_plan_add_quantize_c16(kxc_hip_plan* plan, int64_t n, int64_t c, int64_t hw, float scale,

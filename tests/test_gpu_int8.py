@@ -221,6 +221,44 @@ def test_qconv_first_layer_c4_against_cpu(pkg, orc, shape):
     assert len(np.unique(want)) > 20
 
 
+@pytest.mark.parametrize("shape,relu", [((2, 3, 224, 224, 64), True), ((2, 3, 224, 224, 64), False), ((3, 3, 70, 92, 32), True),
+                                        ((1, 4, 64, 64, 96), False), ((2, 3, 33, 240, 64), True), ((2, 1, 9, 8, 32), True),
+                                        ((1, 2, 1, 4, 32), False)],
+                         ids=lambda v: "x".join(map(str, v)) if isinstance(v, tuple) else str(v))
+def test_qconv_first_layer_with_the_max_pool_in_the_kernel(pkg, orc, monkeypatch, shape, relu):
+    """First layer (7x7 / 2 / 3 on the 4-channel layout) and the 3x3 / stride 2 / padding 1 max pool behind it as one
+    kernel: the CPU int8 convolution followed by the CPU int8 max pool, byte for byte -- full-size maps, odd output
+    widths and heights (the last window hangs over the edge), a 60-column pooled map (the widest the four waves
+    cover), one-row inputs, with and without ReLU (without it negative values and the -128 pad candidate meet), and
+    every number of pooled rows per workgroup."""
+    n, c, h, w, o = shape
+    rng = np.random.default_rng(hash(shape) % (2 ** 31))
+    x = rng.integers(-128, 128, (n, c, h, w), dtype=np.int8)
+    wq = rng.integers(-127, 128, (o, c, 7, 7), dtype=np.int8)
+    bias = rng.integers(-20000, 20000, (o,), dtype=np.int32)
+    mult = rng.uniform(0.5, 2.0, (o,)).astype(np.float32) * np.float32(1.0 / (8.0 * np.sqrt(c * 49) * 64))
+    want = orc.qmaxpool(orc.qconv(x, wq, bias, mult, 2, 3, None, 0.0, relu), 3, 2, 1)
+    x4 = np.zeros((n, h, w, 4), np.int8)
+    x4[..., :c] = x.transpose(0, 2, 3, 1)
+    xd, wp = dev(x4), pkg.qconv2d_c4_pack_weights(dev(wq))
+    assert pkg.qconv2d_c4_maxpool_supported(x4.shape, o, c, relu)
+    for rows in (None, "1", "2", "3", "5", "7"):
+        if rows is None:
+            monkeypatch.delenv("KXC_HIP_QPOOL_ROWS", raising=False)
+        else:
+            monkeypatch.setenv("KXC_HIP_QPOOL_ROWS", rows)
+        got = pkg.qconv2d_c4_maxpool(xd, c, wp, wq.shape, dev(bias), dev(mult), relu)
+        assert_bit_exact(from_c16(pkg, got, o), want, "first layer + max pool %s relu=%s rows=%s" % (shape, relu, rows))
+    monkeypatch.delenv("KXC_HIP_QPOOL_ROWS", raising=False)
+    # ... and the two launches it replaces
+    two = pkg.maxpool2d_c16_i8(pkg.qconv2d_c4(xd, c, wp, wq.shape, dev(bias), dev(mult), relu), o, 3, 2, 1)
+    assert torch.equal(got, two)
+    if h > 8:
+        assert len(np.unique(want)) > 20
+    # a map wider than the kernel covers is refused (a 244-pixel row pools to 61 columns)
+    assert not pkg.qconv2d_c4_maxpool_supported((1, 8, 244, 4), 32)
+
+
 @pytest.mark.parametrize("shape", [(2, 3, 12, 16), (2, 3, 7, 9), (1, 4, 8, 8), (3, 1, 5, 4), (1, 2, 3, 3)],
                          ids=["planes-of-4", "odd-planes", "four-channels", "one-channel", "two-channels-odd"])
 def test_quantize_to_c4(pkg, orc, synth, shape):
@@ -363,19 +401,19 @@ def _run_compiled(mod, x_dev, consts, out):
 
 
 def test_compiled_qresnet18_plan_is_the_matrix_core_plan(pkg):
-    """Compiler::Compile on the quantised graph chooses the channel-blocked layout itself: 21 launches, the first
-    convolution on the 4-channel input layout, every other one on c16, the three downsamples as second outputs,
-    weights packed by the plan from the OIHW constants (20 packs, one per convolution), no layout converter anywhere."""
+    """Compiler::Compile on the quantised graph chooses the channel-blocked layout itself: 20 launches, the first
+    convolution on the 4-channel input layout with the max pool in its kernel, every other one on c16, the three
+    downsamples as second outputs, weights packed by the plan from the OIHW constants (20 packs, one per convolution),
+    no layout converter anywhere."""
     qr, x, model = _quantised_model(pkg, 2, 64, 5)
     mod, _ = _compiled(pkg, model, 2, 64)
     sym = mod.launches()
-    assert len(sym) == 21
+    assert len(sym) == 20
     assert sym[0] == "qnn_quantize kxc_quantize_f32_nchw_to_c4_i8"
-    assert sym[1].startswith("qnn_conv2d kxc_qconv2d_c4_i8:qmfma")
-    assert sym[2] == "nn_max_pool2d kxc_max_pool2d_c16_i8"
-    assert all(s.startswith("qnn_conv2d kxc_qconv2d_c16_i8:qmfma") for s in sym[3:19])
+    assert sym[1] == "qnn_conv2d kxc_qconv2d_c4_i8:qmfma_k7x7s2_c4+relu+maxpool3x3s2"
+    assert all(s.startswith("qnn_conv2d kxc_qconv2d_c16_i8:qmfma") for s in sym[2:18])
     assert sum("|qconv1x1+bias" in s for s in sym) == 3
-    assert sym[19] == "qnn_global_avg_pool2d kxc_global_avg_pool2d_c16_i8" and sym[20] == "qnn_dense kxc_qdense_i8"
+    assert sym[18] == "qnn_global_avg_pool2d kxc_global_avg_pool2d_c16_i8" and sym[19] == "qnn_dense kxc_qdense_i8"
     assert not any("layout_convert" in s for s in sym)
     plan_text = mod.plan_json()
     assert plan_text.count("\\npack ") == 20 and "kxc_hip_plan 3" in plan_text
@@ -438,7 +476,7 @@ def test_compiled_qresnet18_batch64_images(pkg, orc):
     shares of the batch side by side."""
     qr, x, model = _quantised_model(pkg, 64, 224, 5)
     mod, consts = _compiled(pkg, model, 64, 224)
-    assert len(mod.launches()) == 21
+    assert len(mod.launches()) == 20
     xd = dev(x)
     out = torch.empty((64, 1000), device="cuda")
     _run_compiled(mod, xd, consts, out)
@@ -448,7 +486,7 @@ def test_compiled_qresnet18_batch64_images(pkg, orc):
         assert_bit_exact(first[n:n + 1], want, "compiled quantised resnet18 batch 64, image %d" % n)
     import json
     again = pkg.Plan.deserialize(json.loads(mod.plan_json())["kxc_hip"]["launch_plan"], 0)
-    assert again.num_weight_packs() == 20 and len(again.symbols()) == 21
+    assert again.num_weight_packs() == 20 and len(again.symbols()) == 20
     out_again = torch.zeros_like(out)
     again.run([xd] + consts + [out_again])
     torch.cuda.synchronize()
@@ -465,7 +503,7 @@ def test_compiled_qresnet18_batch64_images(pkg, orc):
             stream.synchronize()
             assert_bit_exact(host(out), first, "frozen module, graph replay %d" % replay)
     two, _ = _compiled(pkg, model, 64, 224, lanes=2)
-    assert len(two.launches()) == 42
+    assert len(two.launches()) == 40
     out2 = torch.zeros((64, 1000), device="cuda")
     _run_compiled(two, xd, consts, out2)
     assert_bit_exact(host(out2), first, "two shares of the batch")

@@ -227,7 +227,8 @@ def test_quantised_resnet18_hip_plan_without_gpu():
     """The quantised ResNet-18 graph (qnn_quantize, qnn_conv2d, int8 max pool, qnn_global_avg_pool2d, qnn_dense)
     compiled for the hip target: the operators' layout hooks put every activation between the first convolution and
     the average pool into the channel-blocked layout of the int8 matrix cores, the input into the 4-channel layout,
-    and pair each downsample with its block's first convolution -- 24 calls, 21 launches, no converter.  With
+    pair each downsample with its block's first convolution, and fold the max pool into the first convolution's
+    kernel -- 24 calls, 20 launches, no converter (KXC_HIP_FUSE_POOL=0: 21, the pool a launch of its own).  With
     KXC_HIP_QNN_MFMA=0 every operator keeps NCHW and its reference-order kernel."""
     import importlib
     ha = importlib.import_module("hdkx-aicompiler_amd.hostapi")
@@ -237,9 +238,21 @@ def test_quantised_resnet18_hip_plan_without_gpu():
     mod = ha.CompiledQResNet18(model, 64, 224)
     sym = mod.launches()
     plan = json.loads(mod.plan_json())
-    assert len(sym) == 21 and len(plan["nodes"]) == 21 and len(plan["constant_value_ids"]) == 63 and mod.num_args == 65
-    assert sym[0] == "qnn_quantize kxc_quantize_f32_nchw_to_c4_i8" and sym[1].startswith("qnn_conv2d kxc_qconv2d_c4_i8:qmfma")
-    assert sym[2] == "nn_max_pool2d kxc_max_pool2d_c16_i8"
+    assert len(sym) == 20 and len(plan["nodes"]) == 20 and len(plan["constant_value_ids"]) == 63 and mod.num_args == 65
+    assert sym[0] == "qnn_quantize kxc_quantize_f32_nchw_to_c4_i8"
+    assert sym[1] == "qnn_conv2d kxc_qconv2d_c4_i8:qmfma_k7x7s2_c4+relu+maxpool3x3s2"
+    # (the fused node produces the pooling call's value)
+    assert plan["nodes"][1]["output_values"] != plan["nodes"][0]["output_values"] and plan["nodes"][2]["input_values"][0] == plan["nodes"][1]["output_values"][0]
+    os.environ["KXC_HIP_FUSE_POOL"] = "0"
+    try:
+        unfused = ha.CompiledQResNet18(model, 64, 224)
+        usym = unfused.launches()
+        unfused.close()
+    finally:
+        del os.environ["KXC_HIP_FUSE_POOL"]
+    assert len(usym) == 21 and usym[1] == "qnn_conv2d kxc_qconv2d_c4_i8:qmfma_k7x7s2_c4+relu" and usym[2] == "nn_max_pool2d kxc_max_pool2d_c16_i8"
+    assert usym[3:] == sym[2:]
+    sym = [sym[0], sym[1], "(pool)"] + sym[2:]                  # numbered as in the unfused plan below
     assert all(s.startswith(("qnn_conv2d kxc_qconv2d_c16_i8:qmfma", "qnn_conv2d kxc_qconv2d_c16_i8:qrows")) for s in sym[3:19])
     # the four 56 x 56 stride-1 layers take the kernel with the 64-position row pitch
     assert [":qrows_k3x3" in s for s in sym[3:19]] == [True] * 4 + [False] * 12
@@ -254,7 +267,7 @@ def test_quantised_resnet18_hip_plan_without_gpu():
     mod.close()
     # a batch of 128 runs as two shares side by side; a graph cut at a convolution converts its result back to NCHW
     two = ha.CompiledQResNet18(model, 128, 224)
-    assert len(two.launches()) == 42 and two.launches()[1].endswith(" @share1")
+    assert len(two.launches()) == 40 and two.launches()[1].endswith(" @share1")
     two.close()
     cut = ha.CompiledQResNet18(model, 2, 64, result="l2.0.down")
     assert cut.launches()[-1] == "layout_convert kxc_i8_c16_to_nchw" and "qmfma_k1x1" in cut.launches()[-2]
