@@ -1690,7 +1690,8 @@ const K7Variant kK7Variants[] = {
     {"qmfma_k7x7s2_c4_p2_o1", 2, 1, 8, qconv_k7s2_c4_kernel<2, 1, 8>},
 };
 
-int32_t PrepareK7(const kxc_hip_qconv2d_desc* d, QLaunch* L, const K7Variant** out, const char* who) {
+// select_variant = false: only the geometry (the kernel with the pool has its own tiling)
+int32_t PrepareK7(const kxc_hip_qconv2d_desc* d, QLaunch* L, const K7Variant** out, const char* who, bool select_variant = true) {
     KXC_HIP_REQUIRE(d != nullptr, "%s: desc is NULL", who);
     KXC_HIP_REQUIRE(d->kh == 7 && d->kw == 7 && d->stride_h == 2 && d->stride_w == 2 && d->pad_h == 3 && d->pad_w == 3,
                     "%s: only a 7x7 filter with stride 2 and padding 3 runs on the c4 layout", who);
@@ -1719,6 +1720,9 @@ int32_t PrepareK7(const kxc_hip_qconv2d_desc* d, QLaunch* L, const K7Variant** o
     *out = nullptr;
     if (M == 0) return KXC_HIP_OK;
     const int W4 = a.W / 4 + 2;
+    a.div_wp = MakeFastDiv(W4); a.div_hp = MakeFastDiv(a.Hp); a.div_ohw = MakeFastDiv(a.OHW);
+    a.div_ow = MakeFastDiv(a.OW);
+    if (!select_variant) return KXC_HIP_OK;
     for (const K7Variant& v : kK7Variants) {
         if ((a.O / 32) % v.ro != 0) continue;
         const int rows = MaxRows(a, 7, 32 * v.wp);
@@ -1737,8 +1741,7 @@ int32_t PrepareK7(const kxc_hip_qconv2d_desc* d, QLaunch* L, const K7Variant** o
     a.o_tiles = (a.O / 32) / (*out)->ro;
     a.num_tiles = a.p_tiles * a.o_tiles;
     a.tiles_per_xcd = (a.num_tiles + 7) / 8;
-    a.div_wp = MakeFastDiv(W4); a.div_hp = MakeFastDiv(a.Hp); a.div_ohw = MakeFastDiv(a.OHW);
-    a.div_ow = MakeFastDiv(a.OW); a.div_otiles = MakeFastDiv(a.o_tiles);
+    a.div_otiles = MakeFastDiv(a.o_tiles);
     L->grid = a.tiles_per_xcd * 8;
     return KXC_HIP_OK;
 }
@@ -1757,7 +1760,7 @@ struct K7PoolLaunch {
 int32_t PrepareK7Pool(const kxc_hip_qconv2d_desc* d, K7PoolLaunch* L, const char* who) {
     QLaunch base;
     const K7Variant* unused = nullptr;
-    if (int32_t rc = PrepareK7(d, &base, &unused, who)) return rc;
+    if (int32_t rc = PrepareK7(d, &base, &unused, who, false)) return rc;
     QArgs& a = L->args;
     a = base.args;
     a.POH = (a.OH - 1) / 2 + 1;       // (OH + 2*1 - 3) / 2 + 1
