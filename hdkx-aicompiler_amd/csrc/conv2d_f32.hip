@@ -632,7 +632,13 @@ __global__ void __launch_bounds__(64 * NWAVES) conv1x1_small_kernel(const ConvAr
     const int lane = threadIdx.x & 63;
     const int half = lane >> 5;
     const int r = lane & 31;
-    const int o0 = blockIdx.x * 32, p0 = blockIdx.y * 32;
+    // consecutive workgroups go to the 8 XCDs round-robin; every XCD (own L2) gets a contiguous run of pixel tiles with
+    // all their output-channel tiles, so an input tile is fetched into one L2 instead of eight (measured: 16 x the
+    // input bytes fetched for the 14 x 14 / 512-channel downsample with the output-channel tile as blockIdx.x)
+    const int unit = (blockIdx.x & 7) * a.tiles_per_xcd + (blockIdx.x >> 3);
+    if (unit >= a.num_tiles || static_cast<int>(blockIdx.x >> 3) >= a.tiles_per_xcd) return;
+    const int p_tile = fast_div(unit, a.div_otiles), o_tile = unit - p_tile * a.o_tiles;
+    const int o0 = o_tile * 32, p0 = p_tile * 32;
     const int o = min(o0 + r, a.O - 1);                 // clamped rows / pixels are computed and never stored
     const int px = min(p0 + r, a.M - 1);
     const int n = fast_div(px, a.div_ohw), rem = px - n * a.OHW;
@@ -903,7 +909,6 @@ void Select(const ConvArgs& real, int kh, int kw, Choice* choice, bool ds = fals
     if (kh == 3 && a.sh == 2 && a.W >= 56) preferred = "mfma_k3x3_c2_o1x1_p4x1";
     if (kh == 3 && a.sh == 2 && a.W >= 28 && a.W < 56 && a.O % 64 == 0 && a.M >= 8192) preferred = "mfma_k3x3_c4_o2x1_p8x1";
     if (kh == 3 && a.sh == 1 && a.W >= 56 && a.O % 64 == 0 && a.M >= 65536) preferred = "mfma_k3x3_c4_o1x2_p4x1";
-    if (kh == 1 && a.W >= 56 && a.O % 64 == 0 && a.M >= 32768) preferred = "mfma_k1x1_c8_o1x2_p4x2";
     if (kh == 7 && kw == 7) {
         // first layer at small batch: fewer than 128 of the 64 x 256 tiles leave half the compute units idle
         // (batch 1: 17.5 us; 32 x 128 tiles 10.8 us; batch 2: 18.1 us; 32 x 256 tiles 12.9 us; equal from batch 4 on)
@@ -942,7 +947,9 @@ void Select(const ConvArgs& real, int kh, int kw, Choice* choice, bool ds = fals
         }
         if (pass == 1) {
             *choice = first_fit;
-            if (first_fit.v && first_waves < kEnoughWaves) {
+            // (a 1x1 filter's reduction is only as long as its input channels: splitting 64 or 128 of them costs more
+            // than the idle SIMDs -- batch 32, 64 -> 128 channels at 56 x 56, stride 2: 26.6 us split two ways, 21.4 whole)
+            if (first_fit.v && first_waves < kEnoughWaves && !(kh == 1 && a.C < 256)) {
                 for (int k = 0; k < 3; ++k) {
                     if (!split[k].v) continue;
                     *choice = split[k];
@@ -1031,17 +1038,19 @@ void ApplyRowView(ConvArgs* a, int kh) {
     }
 }
 
-// The small-launch 1x1 kernel takes unpadded 1x1 filters with C % 8 == 0 while the whole launch has at most 16384
-// output pixels.  Measured on the three ResNet-18 downsamples: 5.3 / 6.1 / 7.9 us against 10.0 / 12.0 / 15.6 us
-// for the general kernel at batch 1, still ahead or equal at batch 16 (12544 / 3136 / 784 pixels), behind from
-// batch 64 on (45.7 against 32.4 us for the 56 -> 28 layer).
+// The small-launch 1x1 kernel takes unpadded 1x1 filters with C % 8 == 0 while the whole launch has at most 2^21
+// outputs (pixels x channels).  Measured on the three ResNet-18 downsamples: 5.3 / 6.1 / 7.9 us against 10.0 / 12.0 / 15.6 us
+// for the general kernel at batch 1, still ahead at batch 16 (14.1 / 13.3 / 13.2 against 17.6 / 20.9 / 18.3) and, for
+// the two deeper ones, at batch 32 (1.6 M outputs each: 22.4 / 24.2 against 29.5 / 26.2); behind from 3.2 M outputs
+// on (batch 64, 128 -> 256 channels at 28 x 28: 43.4 against 35.2 us for the 64 x 128 tile; batch 32, 64 -> 128 at
+// 56 x 56: 25.7 against 21.3).
 bool UseSmall1x1(const kxc_hip_conv2d_desc* d, const ConvArgs& a) {
     if (d->kh != 1 || d->kw != 1 || d->pad_h != 0 || d->pad_w != 0 || a.C % 8 != 0 || a.M <= 0) return false;
     if (d->flags & KXC_HIP_CONV_FORCE_DIRECT) return false;
     const int64_t x_elems = static_cast<int64_t>(a.N) * a.C * a.H * a.W, y_elems = static_cast<int64_t>(a.N) * a.O * a.OHW;
     if (x_elems >= (1LL << 31) || y_elems >= (1LL << 31) || CeilDiv(a.M, 32) > 65535) return false;
     if (const char* e = std::getenv("KXC_HIP_CONV_VARIANT")) return std::strcmp(e, "mfma_k1x1_small") == 0;
-    return a.M <= 16384;
+    return a.M <= 16384 && static_cast<int64_t>(a.M) * a.O <= (1LL << 21);
 }
 
 // Launches that still leave most SIMDs idle (batch 1, deep layers: a handful of tiles, a long reduction) split
@@ -1137,7 +1146,12 @@ int32_t Conv2dResolve(const kxc_hip_conv2d_desc* desc, bool second, const char* 
     if (!second && !hpool && UseSmall1x1(desc, a)) {
         a.div_ohw = MakeFastDiv(a.OHW); a.div_ow = MakeFastDiv(a.OW);
         L->path = ConvLaunch::kSmall1x1;
-        L->grid = dim3(static_cast<unsigned>(CeilDiv(a.O, 32)), static_cast<unsigned>(CeilDiv(a.M, 32)));
+        a.o_tiles = static_cast<int32_t>(CeilDiv(a.O, 32));
+        a.p_tiles = static_cast<int32_t>(CeilDiv(a.M, 32));
+        a.num_tiles = a.o_tiles * a.p_tiles;
+        a.tiles_per_xcd = (a.num_tiles + 7) / 8;
+        a.div_otiles = MakeFastDiv(a.o_tiles);
+        L->grid = dim3(static_cast<unsigned>(a.tiles_per_xcd * 8));
         // eight waves split a long reduction (each keeps an even number of channels)
         const bool eight = a.C >= 256 && a.C % 16 == 0;
         L->kernel = eight ? conv1x1_small_kernel<8> : conv1x1_small_kernel<4>;
