@@ -484,7 +484,7 @@ def bench_int8(torch, pkg, synth, dev, np, batch):
               "eager_ms_per_step": round(eager_ms, 4), "hip_graph_replay_ms_per_step": round(graph_ms, 4),
               "default_mode_ms_per_step": round(unfrozen_ms, 4),
               "int8_tops": round(ops / (ms * 1e-3) / 1e12, 1), "frac_int8_mfma_peak": round(ops / (ms * 1e-3) / 1e12 / 5000.0, 4),
-              "launches_per_step": len(launches), "matrix_core_launches": sum("qmfma" in l for l in launches),
+              "launches_per_step": len(launches), "matrix_core_launches": sum(("qmfma" in l or "qrows" in l or "kxc_qdense" in l) for l in launches),
               "workspace_bytes": module.workspace_bytes(),
               "logits_finite": bool(torch.isfinite(out).all().item()),
               "parity": "bit-exact against the CPU int8 chain (tests/test_gpu_int8.py); definition is this build's own"}
