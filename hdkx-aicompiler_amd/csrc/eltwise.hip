@@ -43,37 +43,27 @@ __global__ void __launch_bounds__(kBlock) relu_scalar_kernel(const float* __rest
     for (int64_t i = static_cast<int64_t>(blockIdx.x) * kBlock + threadIdx.x; i < n; i += stride) y[i] = relu_sel(x[i]);
 }
 
-// Loads and stores carry the non-temporal hint: every byte is touched once, and keeping it out of the way of what the
-// caches hold is worth 12 % on operands that come from HBM (77 MB add + ReLU: 16.2 -> 14.2 us, 0.68 of 8 TB/s; a plain
-// device copy of the same size reaches 0.67) and 7 % on operands that sit in the last-level cache (12.3 -> 11.4 us).
-// The hint on the loads alone: 14.1 / 13.2 us; on the stores alone: 15.3 / 12.1; four vectors per thread or other
-// grid sizes: no better.
 template <int OP, bool RELU>
 __global__ void __launch_bounds__(kBlock) same_shape_kernel(const float* __restrict__ a, const float* __restrict__ b,
                                                             float* __restrict__ y, int64_t n4, int64_t n) {
     // two 16-byte vectors of each operand per thread and trip, all four loads issued before the first use
     const int64_t stride = static_cast<int64_t>(gridDim.x) * kBlock;
-    typedef float vec4 __attribute__((ext_vector_type(4)));
-    auto op4 = [](const vec4& va, const vec4& vb) {
-        vec4 r;
+    auto op4 = [](const float4& va, const float4& vb) {
+        float4 r;
         r.x = binop<OP>(va.x, vb.x); r.y = binop<OP>(va.y, vb.y);
         r.z = binop<OP>(va.z, vb.z); r.w = binop<OP>(va.w, vb.w);
         if (RELU) { r.x = relu_sel(r.x); r.y = relu_sel(r.y); r.z = relu_sel(r.z); r.w = relu_sel(r.w); }
         return r;
     };
-    const vec4* const a4 = reinterpret_cast<const vec4*>(a);
-    const vec4* const b4 = reinterpret_cast<const vec4*>(b);
-    vec4* const y4 = reinterpret_cast<vec4*>(y);
     for (int64_t i = static_cast<int64_t>(blockIdx.x) * kBlock + threadIdx.x; i < n4; i += 2 * stride) {
         const int64_t j = i + stride;
         const bool second = j < n4;
-        const int64_t jj = second ? j : i;
-        const vec4 va0 = __builtin_nontemporal_load(a4 + i);
-        const vec4 vb0 = __builtin_nontemporal_load(b4 + i);
-        const vec4 va1 = __builtin_nontemporal_load(a4 + jj);
-        const vec4 vb1 = __builtin_nontemporal_load(b4 + jj);
-        __builtin_nontemporal_store(op4(va0, vb0), y4 + i);
-        if (second) __builtin_nontemporal_store(op4(va1, vb1), y4 + j);
+        const float4 va0 = reinterpret_cast<const float4*>(a)[i];
+        const float4 vb0 = reinterpret_cast<const float4*>(b)[i];
+        const float4 va1 = second ? reinterpret_cast<const float4*>(a)[j] : va0;
+        const float4 vb1 = second ? reinterpret_cast<const float4*>(b)[j] : vb0;
+        reinterpret_cast<float4*>(y)[i] = op4(va0, vb0);
+        if (second) reinterpret_cast<float4*>(y)[j] = op4(va1, vb1);
     }
     const int64_t tail = n4 * 4 + static_cast<int64_t>(blockIdx.x) * kBlock + threadIdx.x;
     if (blockIdx.x == 0 && tail < n) {
