@@ -45,6 +45,10 @@ struct Tool {
     std::vector<kxc_hip_activity_record> done;
     uint64_t dropped = 0;
 };
+// Nobody may ever drain: beyond these counts new records are dropped (and counted) instead of kept.
+constexpr size_t kMaxRecords = 1u << 20;
+constexpr size_t kMaxOpenTransfers = 1u << 16;
+
 Tool& T() {
     static Tool* t = new Tool();     // never destroyed: callbacks may arrive during process exit
     return *t;
@@ -187,9 +191,10 @@ void BufferCallback(rocprofiler_context_id_t, rocprofiler_buffer_id_t, rocprofil
         r.correlation_id = p->correlation_id.internal;
         r.thread_id = p->thread_id;
         r.return_value = static_cast<int32_t>(p->retval.hipError_t_retval);
-        t.done.push_back(r);
+        if (t.done.size() < kMaxRecords) t.done.push_back(r);
+        else ++t.dropped;
         Transfer x;
-        if (r.return_value == 0 && TransferOf(*p, &x) && x.bytes > 0) {
+        if (r.return_value == 0 && Transfers().size() < kMaxOpenTransfers && TransferOf(*p, &x) && x.bytes > 0) {
             x.thread_id = p->thread_id; x.api_start_ns = r.start_ns; x.api_end_ns = r.end_ns;
             std::snprintf(x.api, sizeof(x.api), "%s", name);
             Transfers()[r.correlation_id] = x;
@@ -252,7 +257,8 @@ void BufferCallback(rocprofiler_context_id_t, rocprofiler_buffer_id_t, rocprofil
         } else {
             continue;
         }
-        t.done.push_back(r);
+        if (t.done.size() < kMaxRecords) t.done.push_back(r);
+        else ++t.dropped;
     }
 }
 
