@@ -511,6 +511,31 @@ def test_profiling_bundle_cpu_target():
         assert os.path.exists(os.path.join(d, "artifacts", "kernel_main.c"))
 
 
+def _roctx_bundle(target):
+    with tempfile.TemporaryDirectory() as off, tempfile.TemporaryDirectory() as on:
+        run("profile", target, off)
+        run("profile", target, on, env={"KXC_PROFILE_ROCTX": "1"})
+        e_off, m_off, _ = _read_bundle(off)
+        e_on, m_on, _ = _read_bundle(on)
+    assert m_off["enable_roctx"] is False and m_on["enable_roctx"] is True
+    # ROCm ships the marker library in this image: the spans really push and pop their ranges
+    assert m_on["roctx_available"] is True
+    # markers change nothing in the bundle: the same spans in the same order
+    assert [(e["component"], e["event_type"], e["pass_name"]) for e in e_on if e["component"] != "device_api"] == \
+           [(e["component"], e["event_type"], e["pass_name"]) for e in e_off if e["component"] != "device_api"]
+
+
+def test_roctx_ranges_cpu_target():
+    """ProfileOptions::enable_roctx (the reference's enable_nvtx, include/base/profiling.h:65): every ScopedSpan
+    pushes a range named component:event_type into libroctx64, loaded with dlopen, and pops it when it ends."""
+    _roctx_bundle("cpu")
+
+
+@pytest.mark.gpu
+def test_roctx_ranges_hip_target():
+    _roctx_bundle("hip")
+
+
 # ------------------------------------------------------------------ adaptive runtime
 def _adaptive_events(d):
     events, _, _ = _read_bundle(d)
