@@ -1,7 +1,9 @@
 // codegen.cc -- see codegen.h.
 #include "kxc/codegen.h"
 
+#include <algorithm>
 #include <cmath>
+#include <cstdlib>
 #include <cstdio>
 #include <functional>
 #include <map>
@@ -416,6 +418,132 @@ bool MatchKStage(const LoopNest& data, KStage* m) {
     return true;
 }
 
+// Recognises  for data axes { out[o] = init; for reduce axes { out[o] = out[o] + EXPR } }  (fp32) where EXPR's loads
+// split over the data axes: some loads do not move with an axis others move with (a convolution's input window does
+// not depend on the output channel, its weights on nothing else).  A thread then owns a small block of outputs along up
+// to two such axes and every loaded value feeds several accumulators; each output is still summed by one thread
+// in the CPU order.  `tile[i]` is the block extent along `axis[i]` (an index into the data axes; -1 = unused).
+struct RegTile {
+    Stmt init, upd;
+    LoopNest red;
+    PrimExpr expr;
+    int axis[2] = {-1, -1};
+    int tile[2] = {1, 1};
+    int64_t units = 0;                  // threads' worth of work: blocks of outputs
+};
+
+bool MatchRegTile(const LoopNest& data, int64_t min_units, RegTile* m) {
+    const Stmt& b = data.body;
+    if (!b.defined() || b->kind != StmtKind::kSeqStmt || b->body.size() != 2 || data.vars.size() < 2) return false;
+    const Stmt& init = b->body[0];
+    if (init->kind != StmtKind::kStore) return false;
+    LoopNest red = PeelLoops(b->body[1], false);
+    if (red.vars.empty() || !red.body.defined() || red.body->kind != StmtKind::kStore) return false;
+    const Stmt& upd = red.body;
+    if (upd->var.get() != init->var.get()) return false;
+    if (!upd->a.defined() || upd->a->kind != ExprKind::kAdd) return false;
+    const PrimExpr& old = upd->a->args[0];
+    if (old->kind != ExprKind::kLoad || old->args[0].get() != init->var.get()) return false;
+    Affine oi = AnalyzeAffine(init->b), ui = AnalyzeAffine(upd->b), li = AnalyzeAffine(old->args[1]);
+    if (!oi.ok || !ui.ok || !li.ok || oi.coef != ui.coef || oi.constant != ui.constant || oi.coef != li.coef ||
+        oi.constant != li.constant)
+        return false;
+    for (const auto& v : red.vars)
+        if (oi.coef.count(v.get()) && oi.coef.at(v.get()) != 0) return false;
+    if (!init->a.defined() || !init->a.dtype().is_float() || init->a.dtype().bits != 32) return false;
+    int64_t reduce_extent = 1;
+    for (auto e : red.extents) reduce_extent *= e;
+    if (reduce_extent < 4) return false;
+    std::vector<std::pair<PrimExpr, bool>> loads;
+    CollectLoads(upd->a->args[1], false, &loads);
+    CollectLoads(init->a, false, &loads);
+    if (loads.size() < 2) return false;
+    const int nd = static_cast<int>(data.vars.size());
+    // moves[l][a]: load l's address changes with data axis a (an index that is not affine counts as moving with all)
+    std::vector<std::vector<bool>> moves;
+    for (const auto& entry : loads) {
+        if (entry.first->args[0].get() == init->var.get()) return false;        // EXPR reads the output
+        Affine ai = AnalyzeAffine(entry.first->args[1]);
+        std::vector<bool> row(static_cast<size_t>(nd), true);
+        if (ai.ok)
+            for (int a = 0; a < nd; ++a) row[static_cast<size_t>(a)] = ai.coef.count(data.vars[a].get()) && ai.coef.at(data.vars[a].get()) != 0;
+        moves.push_back(row);
+    }
+    const int lane = nd - 1;                                                   // consecutive lanes walk the innermost axis
+    auto shares = [&](int a, bool lane_varying_only) {
+        bool still = false, moving = false;
+        for (const auto& row : moves) {
+            if (row[static_cast<size_t>(a)]) moving = true;
+            else if (!lane_varying_only || row[static_cast<size_t>(lane)]) still = true;
+        }
+        return still && moving;
+    };
+    // first axis: one along which a per-lane load (the expensive kind) is shared; else any axis that shares a load
+    int a1 = -1;
+    for (int pass = 0; pass < 2 && a1 < 0; ++pass)
+        for (int a = 0; a < lane && a1 < 0; ++a)
+            if (data.extents[a] >= 2 && shares(a, pass == 0)) a1 = a;
+    if (a1 < 0) return false;
+    // second axis (innermost candidate first): it must share a load that moves with the first
+    int a2 = -1;
+    for (int a = lane - 1; a >= 0 && a2 < 0; --a) {
+        if (a == a1 || data.extents[a] < 2) continue;
+        for (const auto& row : moves)
+            if (row[static_cast<size_t>(a1)] && !row[static_cast<size_t>(a)]) a2 = a;
+    }
+    int64_t total = 1;
+    for (auto e : data.extents) total *= e;
+    auto units_for = [&](int t1, int t2) {
+        int64_t u = total / data.extents[a1] * ((data.extents[a1] + t1 - 1) / t1);
+        if (a2 >= 0) u = u / data.extents[a2] * ((data.extents[a2] + t2 - 1) / t2);
+        return u;
+    };
+    int t1 = static_cast<int>(std::min<int64_t>(4, data.extents[a1]));
+    int t2 = a2 >= 0 ? static_cast<int>(std::min<int64_t>(4, data.extents[a2])) : 1;
+    // keep the machine full: fewer, fatter threads only while there is at least `min_units` of them
+    while (t2 > 1 && units_for(t1, t2) < min_units) t2 = (t2 + 1) / 2;
+    while (t1 > 1 && units_for(t1, t2) < min_units) t1 = (t1 + 1) / 2;
+    if (t1 * t2 < 2) return false;
+    if (t1 == 1) { a1 = a2; t1 = t2; a2 = -1; t2 = 1; }
+    if (t2 == 1) a2 = -1;
+    m->init = init; m->upd = upd; m->red = red; m->expr = upd->a->args[1];
+    m->axis[0] = a1; m->axis[1] = a2; m->tile[0] = t1; m->tile[1] = t2;
+    m->units = units_for(t1, t2);
+    return true;
+}
+
+// Which of the two tiled axes an expression reads (bit 0: `a`, bit 1: `b`), and whether it loads from memory.
+int TileDeps(const PrimExpr& e, const ExprNode* a, const ExprNode* b) {
+    if (!e.defined()) return 0;
+    if (e->kind == ExprKind::kVar) return (e.get() == a ? 1 : 0) | (b && e.get() == b ? 2 : 0);
+    int d = 0;
+    for (const auto& x : e->args) d |= TileDeps(x, a, b);
+    return d;
+}
+bool HasLoad(const PrimExpr& e) {
+    if (!e.defined()) return false;
+    if (e->kind == ExprKind::kLoad) return true;
+    for (const auto& x : e->args)
+        if (HasLoad(x)) return true;
+    return false;
+}
+// The largest sub-expressions with a load that read only some of the tiled axes: a block of outputs evaluates each once
+// per index of the axes it does read, not once per output.  Nothing is taken out of a branch that is evaluated lazily
+// (a padded window's input load stays behind its bounds test; the whole select moves).
+struct SharedTerm { PrimExpr e; int deps; };
+void CollectSharedTerms(const PrimExpr& e, const ExprNode* a, const ExprNode* b, std::vector<SharedTerm>* out) {
+    if (!e.defined() || out->size() >= 8) return;
+    const int full = 1 | (b ? 2 : 0);
+    const int d = TileDeps(e, a, b);
+    if (d != full) {
+        if (HasLoad(e)) out->push_back({e, d});
+        return;
+    }
+    const bool lazy = e->kind == ExprKind::kSelect || e->kind == ExprKind::kAnd || e->kind == ExprKind::kOr;
+    for (size_t i = 0; i < e->args.size(); ++i)
+        if (!lazy || i == 0) CollectSharedTerms(e->args[i], a, b, out);
+}
+
 }  // namespace
 
 HIPModuleSource CodeGenHIP::Generate(const tir::PrimFunc& func, const std::string& prefix) {
@@ -426,6 +554,19 @@ HIPModuleSource CodeGenHIP::Generate(const tir::PrimFunc& func, const std::strin
     for (const char* id : {"tile", "tile0", "tile1", "rowbase0", "rowbase1", "total", "base", "rows", "row", "e", "k", "kk",
                            "k0", "kend", "acc", "gid", "rem", "valid", "r"})
         names.Reserve(id);
+    for (const char* id : {"ta_base", "tb_base"}) names.Reserve(id);
+    for (int i = 0; i < 4; ++i) {
+        names.Reserve("ta" + std::to_string(i));
+        names.Reserve("tb" + std::to_string(i));
+        for (int j = 0; j < 4; ++j) names.Reserve("acc" + std::to_string(i) + std::to_string(j));
+    }
+    for (int k = 0; k < 8; ++k) {
+        names.Reserve("u" + std::to_string(k));
+        for (int i = 0; i < 4; ++i) names.Reserve("u" + std::to_string(k) + "_" + std::to_string(i));
+    }
+    // threads a register-tiled stage must keep (one workgroup of 256 on each of the 256 compute units)
+    int64_t tile_min_units = 65536;
+    if (const char* v = std::getenv("KXC_HIPGEN_TILE_MIN_UNITS")) tile_min_units = std::max<int64_t>(1, std::atoll(v));
     std::ostringstream os;
     os << "// generated by kxc CodeGenHIP for gfx950 (wave64)\n";
     os << "#ifndef INFINITY\n#define INFINITY __builtin_inff()\n#endif\n#ifndef NAN\n#define NAN __builtin_nanf(\"\")\n#endif\n\n";
@@ -545,6 +686,87 @@ HIPModuleSource CodeGenHIP::Generate(const tir::PrimFunc& func, const std::strin
                 os << pad << "}\n";
             }
             os << "    if (valid) " << o << "[" << EmitExpr(ks.init->b, &names) << "] = acc;\n";
+            os << "  }\n";
+        } else if (RegTile rt; MatchRegTile(data, tile_min_units, &rt)) {
+            // ---- register-tiled reduction: a thread owns tile[0] x tile[1] outputs along two data axes; the loads
+            // that do not move with an axis are shared by the accumulators along it (the compiler merges the equal
+            // loads of the repeated expression); every output is summed by its one thread in the CPU order
+            spec.schedule = "reg_tile";
+            const std::string o = names.Get(rt.init->var.get());
+            const char* base_name[2] = {"ta_base", "tb_base"};
+            const char* value_name[2] = {"ta", "tb"};
+            total = rt.units;
+            os << "  for (long long gid = (long long)blockIdx.x * 256 + threadIdx.x; gid < " << total
+               << "LL; gid += (long long)gridDim.x * 256) {\n";
+            os << "    long long rem = gid;\n";
+            for (int i = static_cast<int>(data.vars.size()) - 1; i >= 0; --i) {
+                const int which = i == rt.axis[0] ? 0 : (i == rt.axis[1] ? 1 : -1);
+                const int64_t steps = which < 0 ? data.extents[i] : (data.extents[i] + rt.tile[which] - 1) / rt.tile[which];
+                const std::string v = which < 0 ? names.Get(data.vars[i].get()) : std::string(base_name[which]);
+                const std::string scale = which < 0 ? "" : " * " + std::to_string(rt.tile[which]);
+                if (i == 0) os << "    const int " << v << " = (int)rem" << scale << ";\n";
+                else {
+                    os << "    const int " << v << " = (int)(rem % " << steps << "LL)" << scale << ";\n";
+                    os << "    rem /= " << steps << "LL;\n";
+                }
+                // a block that hangs over the end of its axis repeats the last index; its stores are skipped below
+                for (int j = 0; which >= 0 && j < rt.tile[which]; ++j)
+                    os << "    const int " << value_name[which] << j << " = " << v << " + " << j << " < " << data.extents[i] << " ? " << v
+                       << " + " << j << " : " << data.extents[i] - 1 << ";\n";
+            }
+            auto at = [&](int i, int j) {
+                ExprOverrides ov;
+                ov[data.vars[static_cast<size_t>(rt.axis[0])].get()] = "ta" + std::to_string(i);
+                if (rt.axis[1] >= 0) ov[data.vars[static_cast<size_t>(rt.axis[1])].get()] = "tb" + std::to_string(j);
+                return ov;
+            };
+            for (int i = 0; i < rt.tile[0]; ++i)
+                for (int j = 0; j < rt.tile[1]; ++j) {
+                    const ExprOverrides ov = at(i, j);
+                    os << "    float acc" << i << j << " = " << EmitExpr(rt.init->a, &names, &ov) << ";\n";
+                }
+            std::string pad = "    ";
+            for (size_t i = 0; i < rt.red.vars.size(); ++i) {
+                const std::string v = names.Get(rt.red.vars[i].get());
+                os << pad << "for (int " << v << " = 0; " << v << " < " << rt.red.extents[i] << "; ++" << v << ") {\n";
+                pad += "  ";
+            }
+            const ExprNode* va = data.vars[static_cast<size_t>(rt.axis[0])].get();
+            const ExprNode* vb = rt.axis[1] >= 0 ? data.vars[static_cast<size_t>(rt.axis[1])].get() : nullptr;
+            std::vector<SharedTerm> shared;
+            CollectSharedTerms(rt.expr, va, vb, &shared);
+            for (size_t k = 0; k < shared.size(); ++k) {
+                const std::string u = "u" + std::to_string(k);
+                if (shared[k].deps == 0) os << pad << "const auto " << u << " = " << EmitExpr(shared[k].e, &names) << ";\n";
+                for (int i = 0; shared[k].deps == 1 && i < rt.tile[0]; ++i) {
+                    const ExprOverrides ov = at(i, 0);
+                    os << pad << "const auto " << u << "_" << i << " = " << EmitExpr(shared[k].e, &names, &ov) << ";\n";
+                }
+                for (int j = 0; shared[k].deps == 2 && j < rt.tile[1]; ++j) {
+                    const ExprOverrides ov = at(0, j);
+                    os << pad << "const auto " << u << "_" << j << " = " << EmitExpr(shared[k].e, &names, &ov) << ";\n";
+                }
+            }
+            for (int i = 0; i < rt.tile[0]; ++i)
+                for (int j = 0; j < rt.tile[1]; ++j) {
+                    ExprOverrides ov = at(i, j);
+                    for (size_t k = 0; k < shared.size(); ++k) {
+                        const std::string u = "u" + std::to_string(k);
+                        ov[shared[k].e.get()] = shared[k].deps == 0 ? u : u + "_" + std::to_string(shared[k].deps == 1 ? i : j);
+                    }
+                    os << pad << "acc" << i << j << " = acc" << i << j << " + " << EmitExpr(rt.expr, &names, &ov) << ";\n";
+                }
+            for (size_t i = 0; i < rt.red.vars.size(); ++i) {
+                pad.resize(pad.size() - 2);
+                os << pad << "}\n";
+            }
+            for (int i = 0; i < rt.tile[0]; ++i)
+                for (int j = 0; j < rt.tile[1]; ++j) {
+                    const ExprOverrides ov = at(i, j);
+                    os << "    if (ta_base + " << i << " < " << data.extents[static_cast<size_t>(rt.axis[0])];
+                    if (rt.axis[1] >= 0) os << " && tb_base + " << j << " < " << data.extents[static_cast<size_t>(rt.axis[1])];
+                    os << ") " << o << "[" << EmitExpr(rt.init->b, &names, &ov) << "] = acc" << i << j << ";\n";
+                }
             os << "  }\n";
         } else {
             // ---- flat schedule: one output element per thread per grid-stride step

@@ -480,7 +480,13 @@ int RunCodegen() {
     auto hip = cgh.Generate(pf, "kxc_t");
     Check(hip.kernels.size() == 3, "one kernel per compute stage");
     Check(hip.source.find("extern \"C\" __global__ void __launch_bounds__(256) kxc_t_s0_T_conv2d(") != std::string::npos, "kernel symbol");
-    Check(hip.kernels[0].schedule == "flat", "conv stage is a flat schedule");
+    // 200 704 outputs: blocks of two output channels still leave 65 536 threads; the input window is read once per block
+    Check(hip.kernels[0].schedule == "reg_tile", "conv stage takes the register-tiled schedule: " + hip.kernels[0].schedule);
+    Check(hip.source.find("acc10 = acc10 + (u0 * weight[") != std::string::npos && hip.source.find("acc01") == std::string::npos &&
+              hip.source.find("acc20") == std::string::npos,
+          "blocks of 2 x 1 outputs sharing the input term");
+    Check(hip.kernels[0].grid[0] == 392, "100 352 threads in workgroups of 256");
+    Check(hip.kernels[1].schedule == "flat" && hip.kernels[2].schedule == "flat", "bias add and relu are flat");
     {
         // a padded window at least 16 taps wide: the input load sits behind the padding select and must stay a lazy
         // global load (staged for a whole tile of rows it would read before the buffer and past its end); the weight
@@ -1116,7 +1122,10 @@ int RunGeneratedNumeric() {
     auto fill = [](std::vector<float>& v, uint32_t seed) {
         for (float& x : v) { seed = seed * 1664525u + 1013904223u; x = static_cast<float>(static_cast<int32_t>(seed >> 8) % 2001 - 1000) / 997.0f; }
     };
-    struct Case { std::string name; kxc::Function func; std::vector<std::vector<int64_t>> in_shapes; int64_t out_elems; std::string schedule; };
+    struct Case {
+        std::string name; kxc::Function func; std::vector<std::vector<int64_t>> in_shapes; int64_t out_elems; std::string schedule;
+        const char* tile_min_units = nullptr;      // KXC_HIPGEN_TILE_MIN_UNITS for this case (small shapes take the tiled schedule)
+    };
     std::vector<Case> cases;
     {
         kxc::Var x("x", kxc::TensorType({5, 70}, "float32")), w("w", kxc::TensorType({37, 70}, "float32"));
@@ -1149,7 +1158,25 @@ int RunGeneratedNumeric() {
         cases.push_back({"conv2d 1x17 window, padding 8", kxc::Function({d, w}, kxc::Call(Op::Get("nn_conv2d"), {d, w}, attrs)),
                          {{1, 2, 4, 40}, {3, 2, 1, 17}}, 480, "lds_k_stage"});
     }
+    // convolution-shaped nests: a thread owns a block of outputs along the output-channel axis and the row axis
+    auto conv_case = [&](const std::string& name, std::vector<int64_t> xs, std::vector<int64_t> ws, std::vector<int64_t> strides,
+                         std::vector<int64_t> pads, std::vector<int64_t> dil, const char* min_units, const std::string& schedule) {
+        kxc::Var d("d", kxc::TensorType(xs, "float32")), w("w", kxc::TensorType(ws, "float32"));
+        auto attrs = kxc::relay::Conv2DAttrs::Create(strides, pads, dil, 1, ws[0], {ws[2], ws[3]}, "NCHW", "OIHW", "", "");
+        kxc::Function f({d, w}, kxc::Call(Op::Get("nn_conv2d"), {d, w}, attrs));
+        const int64_t oh = (xs[2] + pads[0] + pads[2] - dil[0] * (ws[2] - 1) - 1) / strides[0] + 1;
+        const int64_t ow = (xs[3] + pads[1] + pads[3] - dil[1] * (ws[3] - 1) - 1) / strides[1] + 1;
+        cases.push_back({name, f, {xs, ws}, xs[0] * ws[0] * oh * ow, schedule, min_units});
+    };
+    conv_case("conv2d 3x3, 7 channels out, 9 rows (ragged blocks)", {2, 5, 9, 11}, {7, 5, 3, 3}, {1, 1}, {1, 1, 1, 1}, {1, 1}, "1", "reg_tile");
+    conv_case("conv2d 3x3 stride 2 dilation 2", {1, 3, 13, 10}, {6, 3, 3, 3}, {2, 2}, {2, 2, 2, 2}, {2, 2}, "1", "reg_tile");
+    conv_case("conv2d 1x1, two channels out", {3, 4, 5, 6}, {2, 4, 1, 1}, {1, 1}, {0, 0, 0, 0}, {1, 1}, "1", "reg_tile");
+    conv_case("conv2d 5x5, padding 2 x 1, three channels in blocks of 2 x 1", {1, 2, 6, 7}, {3, 2, 5, 5}, {1, 1}, {2, 1, 2, 1}, {1, 1}, "40", "reg_tile");
+    conv_case("conv2d 3x3 large enough for 4 x 4 blocks by default", {4, 8, 64, 64}, {64, 8, 3, 3}, {1, 1}, {1, 1, 1, 1}, {1, 1}, nullptr, "reg_tile");
+    conv_case("conv2d 3x3 too small to give up threads", {1, 8, 14, 14}, {16, 8, 3, 3}, {1, 1}, {1, 1, 1, 1}, {1, 1}, nullptr, "flat");
     for (auto& c : cases) {
+        if (c.tile_min_units) setenv("KXC_HIPGEN_TILE_MIN_UNITS", c.tile_min_units, 1);
+        else unsetenv("KXC_HIPGEN_TILE_MIN_UNITS");
         std::vector<std::vector<float>> ins;
         uint32_t seed = 12345;
         for (const auto& shp : c.in_shapes) { ins.emplace_back(static_cast<size_t>(kxc::Product(shp))); fill(ins.back(), seed); seed += 7919; }

@@ -110,9 +110,11 @@ def test_random_graphs_in_one_and_two_shares():
 def test_generated_kernels_lds_schedules_bit_exact():
     """dense / matmul / reduce_mean shapes that take the generator's LDS-staged schedules (ragged chunks, fewer outputs
     than a workgroup, an operand that is not contiguous along the reduce axis, a padded window whose input load stays
-    behind its select): bit-identical to the host back end."""
+    behind its select), and convolution-shaped nests in the register-tiled schedule (ragged blocks, stride and dilation,
+    a 5x5 window, 1x1, the default block choice at a large and at a small shape): bit-identical to the host back end."""
     out = run("generated_numeric")
-    assert "generated kernels ok" in out and out.count("[PASS]") == 6
+    assert "generated kernels ok" in out and out.count("[PASS]") == 12
+    assert out.count("(reg_tile)") == 5
 
 
 @pytest.mark.gpu
