@@ -1282,6 +1282,8 @@ const QVariant kQVariants[] = {
     KXC_QV2(3, 3, 2, 4, 1, 8, 2, 3),
     KXC_QV2(3, 3, 2, 2, 2, 8, 2, 3),
     KXC_QV2(3, 3, 2, 2, 1, 8, 2, 3),
+    // 64 channels x 128 pixels per wave (128 accumulator registers): the largest maps only
+    KXC_QV2(3, 3, 2, 4, 2, 8, 4, 3),
 };
 
 // The same tiles on a compile-time row pitch of 64 positions (qconv_rows_kernel): chosen in place of the variant above
@@ -1306,6 +1308,7 @@ const QRowVariant kQRowVariants[] = {
     KXC_QR(3, 3, 2, 4, 1, 4, 2, 64),
     KXC_QR(3, 3, 2, 2, 2, 8, 2, 64),
     KXC_QR(3, 3, 2, 2, 1, 8, 2, 64),
+    KXC_QR(3, 3, 2, 4, 2, 4, 4, 64),
 };
 
 // Channel blocks (of 16 channels) per LDS chunk.  Larger chunks (64 or 128 channels) were measured on the ResNet-18
@@ -1354,7 +1357,7 @@ int32_t Prepare(const kxc_hip_qconv2d_desc* d, QLaunch* L, const char* who) {
     thread_local std::vector<Entry> cache;
     if (const char* f = std::getenv("KXC_HIP_QCONV_VARIANT"))
         if (*f) return PrepareUncached(d, L, who);          // forced variants are not cached
-    if (std::getenv("KXC_HIP_QCONV_ROWS")) return PrepareUncached(d, L, who);
+    if (std::getenv("KXC_HIP_QCONV_ROWS") || std::getenv("KXC_HIP_QCONV_BIG_TILE")) return PrepareUncached(d, L, who);
     for (const Entry& e : cache)
         if (std::memcmp(&e.desc, d, sizeof(*d)) == 0) { *L = e.launch; return KXC_HIP_OK; }
     if (int32_t rc = PrepareUncached(d, L, who)) return rc;
@@ -1406,7 +1409,21 @@ int32_t PrepareUncached(const kxc_hip_qconv2d_desc* d, QLaunch* L, const char* w
     // 21.4 -> 17.7 us; 128 at 28 x 28: 17.8 -> 13.6; 256 at 14 x 14: 15.4 -> 12.4), stride 2 two output-channel
     // blocks per wave (128 -> 256 at 28 -> 14: 11.7 -> 10.2 us); the small 7 x 7 maps keep one block per wave.
     if (!(forced && *forced) && d->kh == 3 && d->kw == 3 && cbc == 2) {
-        if (d->stride_h == 1 && d->stride_w == 1 && M >= 8192) forced = M >= 100000 ? "qmfma_k3x3_cb2_p4x2_o1_d3" : "qmfma_k3x3_cb2_p2x2_o1_d3";
+        // (a wave that takes 64 channels x 128 pixels feeds four matrix instructions from every weight fragment and two
+        // from every pixel fragment, but at 210 registers only two such workgroups fit a compute unit: it wins where its
+        // tiles fill those 512 places well -- 64 -> 64 channels at 56 x 56: 14.2 -> 13.8 us at batch 64 (392 tiles) and
+        // 26.7 -> 26.3 at batch 128 (784), the quantised ResNet-18 0.2993 -> 0.2924 ms per batch of 64 -- and loses where
+        // they do not: 8.6 -> 9.4 us at batch 32 (196 tiles), 20.4 -> 21.1 at batch 96 (588); on the 28 x 28 and
+        // smaller maps it is 10-60 % slower than two pixel blocks of one channel block)
+        if (d->stride_h == 1 && d->stride_w == 1 && M >= 8192) {
+            const char* big = std::getenv("KXC_HIP_QCONV_BIG_TILE");       // 0: never the 64 x 128 tile, 1: from 100 000 pixels on
+            bool big_ok = M >= 100000 && (a.O / 32) % 2 == 0 && !(big && big[0] == '0');
+            if (big_ok && !(big && big[0] == '1')) {
+                const int64_t tiles = CeilDiv(M, 512) * (a.O / 64), rounds = CeilDiv(tiles, 512);
+                big_ok = 10 * tiles >= 7 * rounds * 512;
+            }
+            forced = M >= 100000 ? (big_ok ? "qmfma_k3x3_cb2_p4x4_o2_d3" : "qmfma_k3x3_cb2_p4x2_o1_d3") : "qmfma_k3x3_cb2_p2x2_o1_d3";
+        }
         else if (d->stride_h == 2 && d->stride_w == 2 && (a.O / 32) % 2 == 0 && M >= 2048) forced = "qmfma_k3x3_cb2_p4_o2";
     }
     const bool by_rule = forced && *forced && !(std::getenv("KXC_HIP_QCONV_VARIANT") && *std::getenv("KXC_HIP_QCONV_VARIANT"));

@@ -129,6 +129,42 @@ def test_qconv_c16_row_pitch_kernels_equal_the_general_kernel(pkg, orc, monkeypa
             assert_bit_exact(from_c16(pkg, rows, o), want, "row-pitch kernel against the CPU %s" % ((n, c, h, w, o, k, s, p),))
 
 
+def test_qconv_c16_largest_wave_tile_against_cpu(pkg, orc, monkeypatch):
+    """The tile the largest stride-1 maps take (64 channels x 128 pixels per wave, four waves), forced by name onto shapes the CPU finishes quickly: whole and ragged tiles, a partial channel block, tiles
+    that cross image boundaries, with and without residual, on the row pitch and in the general kernel."""
+    rng = np.random.default_rng(77)
+    monkeypatch.setenv("KXC_HIP_QCONV_VARIANT", "qmfma_k3x3_cb2_p4x4_o2_d3")
+    # (the last flag: the row-pitch kernel holds the shape's patch -- 33-wide rows put 22 rows into a tile, over its 16)
+    for (n, c, h, w, o, residual, relu, on_pitch) in [(2, 64, 56, 56, 64, True, True, True), (3, 40, 5, 62, 64, False, True, True),
+                                                      (5, 64, 9, 33, 128, True, False, False), (7, 128, 7, 7, 64, False, False, False),
+                                                      (1, 20, 17, 19, 64, True, True, False)]:
+        x = rng.integers(-128, 128, (n, c, h, w), dtype=np.int8)
+        wq = rng.integers(-127, 128, (o, c, 3, 3), dtype=np.int8)
+        bias = rng.integers(-20000, 20000, (o,), dtype=np.int32)
+        mult = rng.uniform(0.5, 2.0, (o,)).astype(np.float32) * np.float32(1.0 / (8.0 * np.sqrt(c * 9) * 64))
+        res = rng.integers(-128, 128, (n, o, h, w), dtype=np.int8) if residual else None
+        want = orc.qconv(x, wq, bias, mult, 1, 1, res, 0.29 if residual else 0.0, relu)
+        packed = pkg.qconv2d_c16_pack_weights(dev(wq))
+        d = pkg.qconv_desc(n, c, h, w, o, 3, 3, 1, 1)
+        args = (to_c16(pkg, x), c, packed, wq.shape, dev(bias), dev(mult), to_c16(pkg, res) if residual else None,
+                0.29 if residual else 0.0, 1, 1, relu)
+        for rows in (None, "0"):
+            if rows is None:
+                monkeypatch.delenv("KXC_HIP_QCONV_ROWS", raising=False)
+            else:
+                monkeypatch.setenv("KXC_HIP_QCONV_ROWS", rows)
+            name = pkg.qconv2d_c16_variant(d)
+            assert "p4x4_o2" in name and name.startswith("qrows_" if rows is None and on_pitch else "qmfma_"), name
+            got = pkg.qconv2d_c16(*args)
+            assert_bit_exact(from_c16(pkg, got, o), want, "%s %s" % (name, (n, c, h, w, o)))
+    monkeypatch.delenv("KXC_HIP_QCONV_ROWS", raising=False)
+    monkeypatch.delenv("KXC_HIP_QCONV_VARIANT")
+    # the shape rule: 64 -> 64 channels at 56 x 56 takes it where its tiles fill the two workgroup places per compute unit
+    variant = lambda n: pkg.qconv2d_c16_variant(pkg.qconv_desc(n, 64, 56, 56, 64, 3, 3, 1, 1))
+    assert "p4x4_o2" in variant(64) and "p4x4_o2" in variant(128)
+    assert "p4x2_o1" in variant(32) and "p4x2_o1" in variant(96) and "p2x2_o1" in variant(31)
+
+
 QPAIR_SHAPES = [
     # n, c, h, w, o, stride: the three ResNet-18 blocks, a ragged shape with a partial channel block and an odd block count
     (2, 64, 56, 56, 128, 2), (64, 64, 56, 56, 128, 2), (3, 128, 28, 28, 256, 2), (5, 256, 14, 14, 512, 2),
