@@ -76,6 +76,45 @@ def _profiled_traffic_bytes(name):
     return None
 
 
+def bench_generated(torch, pkg, hostapi, synth, dev, np, batch, steps, warmup):
+    """ResNet-18 fp32 through kernels generated from the lowered loop nests only (CompileConfig::hip_use_handwritten =
+    false, no fusion: 70 launches), with the per-launch times of one run grouped by the generator's schedule.  These
+    kernels keep the CPU back end's order of additions; the hand-written plan's logits serve as the check."""
+    consts = [dev(c) for c in synth.resnet18_consts(4)]
+    x = dev(synth.resnet18_input(4, batch))
+    out = torch.empty((batch, 1000), device="cuda")
+    module = hostapi.CompiledResNet18(batch, 224, "hip", use_handwritten=False, fuse=False, sync_after_run=False)
+    packed = module.packed([x] + consts + [out])
+    stream = torch.cuda.current_stream().cuda_stream
+    for _ in range(max(1, warmup)):
+        module.run_packed(packed, stream)
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(steps):
+        module.run_packed(packed, stream)
+    torch.cuda.synchronize()
+    ms = (time.perf_counter() - t0) * 1e3 / steps
+    by_schedule = {}
+    for name, us in module.run_timed(packed, stream):
+        schedule = name.rsplit("[generated:", 1)[1].rstrip("]") if "[generated:" in name else "other"
+        op = name.split()[0]
+        key = "%s/%s" % (op, schedule)
+        e = by_schedule.setdefault(key, {"launches": 0, "us": 0.0})
+        e["launches"] += 1
+        e["us"] = round(e["us"] + us, 1)
+    ref = torch.empty((batch, 1000), device="cuda")
+    hand = hostapi.CompiledResNet18(batch, 224, "hip", sync_after_run=True)
+    hand.run_packed(hand.packed([x] + consts + [ref]), stream)
+    torch.cuda.synchronize()
+    got, want = out.cpu().numpy(), ref.cpu().numpy()
+    err = float(np.max(np.abs(got - want) / np.maximum(1.0, np.abs(want))))
+    return {"metric": "resnet18_fp32_generated_kernels_img_per_s", "value": round(batch / ms * 1e3, 1), "unit": "img/s",
+            "batch": batch, "ms_per_step": round(ms, 4), "steps": steps, "warmup": warmup, "launches_per_step": len(module.launches()),
+            "tile_min_units": os.environ.get("KXC_HIPGEN_TILE_MIN_UNITS", "default (65536)"),
+            "by_operator_and_schedule": by_schedule,
+            "max_scaled_difference_from_the_hand_written_plan": err}
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -87,6 +126,8 @@ def main():
     ap.add_argument("--no-layers", action="store_true", help="skip the per-layer / per-operator timings")
     ap.add_argument("--int8-only", action="store_true",
                     help="run only the quantised ResNet-18 leg (for profiling its kernels) and print its JSON")
+    ap.add_argument("--generated-only", action="store_true",
+                    help="run only the ResNet-18 compiled to kernels generated from its TIR (no hand-written kernel) and print its JSON")
     ap.add_argument("--cpu-full", action="store_true",
                     help="also time the CPU path on the whole batch once (minutes on one core) -> cpu_baseline.batch_seconds")
     args = ap.parse_args()
@@ -111,6 +152,9 @@ def main():
     batch = args.batch
     if args.int8_only:
         print(json.dumps(bench_int8(torch, pkg, synth, dev, np, batch)))
+        return
+    if args.generated_only:
+        print(json.dumps(bench_generated(torch, pkg, hostapi, synth, dev, np, batch, args.steps, args.warmup)))
         return
     consts_h = synth.resnet18_consts(4)
     x_h = synth.resnet18_input(4, batch)
