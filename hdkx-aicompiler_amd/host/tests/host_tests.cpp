@@ -488,6 +488,20 @@ int RunCodegen() {
     Check(hip.kernels[0].grid[0] == 392, "100 352 threads in workgroups of 256");
     Check(hip.kernels[1].schedule == "flat" && hip.kernels[2].schedule == "flat", "bias add and relu are flat");
     {
+        // with no lower bound on the thread count the same stage takes 4 x 4 blocks (output channels x rows): the padded
+        // window term is evaluated once per row of the block, the weight once per channel, 16 accumulators, guarded stores
+        setenv("KXC_HIPGEN_TILE_MIN_UNITS", "1", 1);
+        auto tiled = cgh.Generate(pf, "kxc_t");
+        unsetenv("KXC_HIPGEN_TILE_MIN_UNITS");
+        const std::string& src = tiled.source;
+        Check(tiled.kernels[0].schedule == "reg_tile" && tiled.kernels[0].grid[0] == 49, "4 x 4 blocks: 12 544 threads");
+        for (const char* piece : {"const auto u0_3 = (", "const auto u1_3 = weight[", "acc33 = acc33 + (u0_3 * u1_3);", "float acc00 = ",
+                                  "if (ta_base + 3 < 64 && tb_base + 3 < 56) T_conv2d["})
+            Check(src.find(piece) != std::string::npos, std::string("register-tiled source holds: ") + piece);
+        Check(src.find("? data[") != std::string::npos && src.find("u0_0 = ((((") != std::string::npos,
+              "the input load stays behind its bounds test inside the shared term");
+    }
+    {
         // a padded window at least 16 taps wide: the input load sits behind the padding select and must stay a lazy
         // global load (staged for a whole tile of rows it would read before the buffer and past its end); the weight
         // load, unguarded and contiguous along rw, may be staged
