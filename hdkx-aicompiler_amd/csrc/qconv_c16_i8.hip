@@ -369,22 +369,25 @@ __global__ void __launch_bounds__(64 * WP) __attribute__((amdgpu_waves_per_eu(2)
             for (int j = 0; j < RP; ++j) b[j] = *reinterpret_cast<const intx4*>(buf + xbase[j] + off);
         };
         const uint32_t t0 = static_cast<uint32_t>(chunk) * NS;
-        intx4 bcur[RP], bnext[RP];
-        fetch_b(0, bcur);
+        // Pixel operands are read DB k-steps ahead.  With several pixel blocks per wave every step ends in a scheduling
+        // barrier: left free, the compiler gathers the LDS reads of many steps ahead of their matrix instructions and the
+        // wave then waits for all of them at once (256 -> 256 channels at 14 x 14, batch 64: 12.4 -> 11.6 us; with one
+        // pixel block per wave the barrier changes nothing or costs 1-2 %, so those variants stay as they were).
+        constexpr int DB = RP >= 2 ? 2 : 1;
+        intx4 bring[DB][RP];
+#pragma unroll
+        for (int s0 = 0; s0 < DB; ++s0) fetch_b(s0, bring[s0]);
 #pragma unroll
         for (int step = 0; step < NS; ++step) {
-            if (step + 1 < NS) fetch_b(step + 1, bnext);
 #pragma unroll
             for (int j = 0; j < RP; ++j)
 #pragma unroll
                 for (int i = 0; i < RO; ++i)
-                    acc[j][i] = __builtin_amdgcn_mfma_i32_32x32x32_i8(ring[step % D][i], bcur[j], acc[j][i], 0, 0, 0);
+                    acc[j][i] = __builtin_amdgcn_mfma_i32_32x32x32_i8(ring[step % D][i], bring[step % DB][j], acc[j][i], 0, 0, 0);
 #pragma unroll
             for (int i = 0; i < RO; ++i) ring[step % D][i] = load_a(i, t0 + step + D);
-            if (step + 1 < NS) {
-#pragma unroll
-                for (int j = 0; j < RP; ++j) bcur[j] = bnext[j];
-            }
+            if (step + DB < NS) fetch_b(step + DB, bring[step % DB]);
+            if constexpr (RP >= 2) __builtin_amdgcn_sched_barrier(0);
         }
         if constexpr (DS) {
             // lane half h takes channel block 2*s2 + h of the chunk at the second output's tap
@@ -605,22 +608,23 @@ __global__ void __launch_bounds__(64 * WP) __attribute__((amdgpu_waves_per_eu(2)
                 }
             };
             const uint32_t t0 = static_cast<uint32_t>(chunk) * NS;
-            intx4 bcur[RP], bnext[RP];
-            fetch_b(0, bcur);
+            // (pixel operands two k-steps ahead and a scheduling barrier per step for several pixel blocks per wave: see
+            // qconv_mfma_kernel; 64 -> 64 channels at 56 x 56, batch 64: 13.2-13.7 -> 12.9 us)
+            constexpr int DB = RP >= 2 ? 2 : 1;
+            intx4 bring[DB][RP];
+#pragma unroll
+            for (int s0 = 0; s0 < DB; ++s0) fetch_b(s0, bring[s0]);
 #pragma unroll
             for (int step = 0; step < NS; ++step) {
-                if (step + 1 < NS) fetch_b(step + 1, bnext);
 #pragma unroll
                 for (int j = 0; j < RP; ++j)
 #pragma unroll
                     for (int i = 0; i < RO; ++i)
-                        acc[j][i] = __builtin_amdgcn_mfma_i32_32x32x32_i8(ring[step % D][i], bcur[j], acc[j][i], 0, 0, 0);
+                        acc[j][i] = __builtin_amdgcn_mfma_i32_32x32x32_i8(ring[step % D][i], bring[step % DB][j], acc[j][i], 0, 0, 0);
 #pragma unroll
                 for (int i = 0; i < RO; ++i) ring[step % D][i] = load_a(i, t0 + step + D);
-                if (step + 1 < NS) {
-#pragma unroll
-                    for (int j = 0; j < RP; ++j) bcur[j] = bnext[j];
-                }
+                if (step + DB < NS) fetch_b(step + DB, bring[step % DB]);
+                if constexpr (RP >= 2) __builtin_amdgcn_sched_barrier(0);
             }
             if constexpr (DS) {
 #pragma unroll
