@@ -468,16 +468,21 @@ conv_mfma_kernel(const ConvArgs a) {
         // accumulator register, handed over through LDS -- the tiles are dead after the loop's last barrier); the
         // first window of a row has no left neighbour.  With ReLU the values are >= +0 and never NaN, so the order
         // of the comparisons does not matter and a padding candidate would never win.
+        // The vector ALU shares its datapath with the fp32 matrix instructions, and with 16 x RO x RP values per lane this
+        // epilogue is a tenth of the kernel: the neighbours come through the LDS crossbar (ds_bpermute, no vector-ALU
+        // instruction; a row's first column names itself as its left neighbour), the one float from the block before
+        // is read by every lane and selected, ReLU is one maximum (NaN -> 0 as (v > 0 ? v : 0) gives; the host only
+        // offers this epilogue with ReLU), and the channel part of a store's address rides in its scalar offset.
         const bool has_bias = (a.flags & KXC_HIP_CONV_BIAS) != 0;
-        const bool do_relu = (a.flags & KXC_HIP_CONV_RELU) != 0;
-        auto channel = [&](int i, int g) { return o0 + (wave_o * RO + i) * 32 + 8 * (g / 4) + 4 * half + (g % 4); };
         const __amdgpu_buffer_rsrc_t br = make_rsrc(has_bias ? a.bias : a.y, has_bias ? static_cast<uint32_t>(a.O) * 4u : 0u);
-        float bv[RO][16];
+        // (the host guarantees O % 8 == 0: the eight channels of a register group's two lane halves are all there or all absent)
+        const int ch0 = o0 + wave_o * RO * 32;                 // uniform: channel of (i, g) = ch0 + 32 i + 8 (g / 4) + g % 4 + 4 half
+        float bv[RO][16];                                      // (no bias: the descriptor is empty, loads give 0; v + 0 then ReLU = ReLU(v))
 #pragma unroll
         for (int i = 0; i < RO; ++i)
 #pragma unroll
             for (int g = 0; g < 16; ++g) {
-                const int o = channel(i, g);
+                const int o = ch0 + 32 * i + 8 * (g / 4) + (g % 4) + 4 * half;
                 bv[i][g] = __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(br, o < a.O ? static_cast<uint32_t>(o) * 4u : kOobOffset, 0, 0));
             }
         // edge[block][half][RO][16], block = the wave's 32-pixel blocks in tile order per output-channel group
@@ -488,17 +493,20 @@ conv_mfma_kernel(const ConvArgs a) {
 #pragma unroll
             for (int j = 0; j < RP; ++j)
 #pragma unroll
-                for (int g = 0; g < 16; ++g) {
-                    float v = acc[i][j][g];
-                    if (has_bias) v = __fadd_rn(v, bv[i][g]);
-                    if (do_relu) v = relu_sel(v);
-                    acc[i][j][g] = v;
-                    if (r == 31) edge[edge_at(wave_p * RP + j, i, g)] = v;
-                }
+                for (int g = 0; g < 16; ++g) acc[i][j][g] = __builtin_fmaxf(__fadd_rn(acc[i][j][g], bv[i][g]), 0.0f);
+        if (r == 31) {
+#pragma unroll
+            for (int i = 0; i < RO; ++i)
+#pragma unroll
+                for (int j = 0; j < RP; ++j)
+#pragma unroll
+                    for (int g = 0; g < 16; ++g) edge[edge_at(wave_p * RP + j, i, g)] = acc[i][j][g];
+        }
         __syncthreads();
         const uint32_t y_bytes = static_cast<uint32_t>(a.out_elems) * 4u;
         const uint32_t plane = static_cast<uint32_t>(a.OH * a.PW) * 4u;
         const __amdgpu_buffer_rsrc_t yr = make_rsrc(a.y, y_bytes);
+        const int right_addr = ((lane + 1) & 63) * 4;        // (lane 31 / 63 reads a lane of the other half: an odd column, never stored)
 #pragma unroll
         for (int j = 0; j < RP; ++j) {
             const int block = wave_p * RP + j;
@@ -507,22 +515,30 @@ conv_mfma_kernel(const ConvArgs a) {
             const int oh = fast_div(rem, a.div_ow), ow = rem - oh * a.OW;
             const bool row_start = ow == 0;
             const bool from_edge = r == 0 && !row_start;              // (then block > 0: a tile starts a row)
-            const uint32_t yb = (r & 1) ? kOobOffset : static_cast<uint32_t>((n * a.O * a.OH + oh) * a.PW + (ow >> 1)) * 4u;
+            const int left_addr = (row_start || r == 0 ? lane : lane - 1) * 4;
+            // even columns own the windows; the lane half's four channels per register group are part of the lane's offset
+            const uint32_t yb = (r & 1) ? kOobOffset
+                                        : static_cast<uint32_t>((n * a.O * a.OH + oh) * a.PW + (ow >> 1)) * 4u + static_cast<uint32_t>(4 * half) * plane;
+            const int prev = block > 0 ? block - 1 : 0;
 #pragma unroll
             for (int i = 0; i < RO; ++i)
 #pragma unroll
-                for (int g = 0; g < 16; ++g) {
-                    const float v = acc[i][j][g];
-                    const int bits = __builtin_bit_cast(int, v);
-                    // lane l reads lane l-1 (0x138: whole-wave shift right by one) and lane l+1 (0x130: shift left)
-                    float left = __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(bits, bits, 0x138, 0xf, 0xf, false));
-                    const float right = __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(bits, bits, 0x130, 0xf, 0xf, false));
-                    if (from_edge) left = edge[edge_at(block - 1, i, g)];
-                    if (row_start) left = v;
-                    const float pooled = fmaxf(v, fmaxf(left, right));
-                    const int o = channel(i, g);
-                    __builtin_amdgcn_raw_buffer_store_b32(__builtin_bit_cast(uint32_t, pooled), yr,
-                                                          o < a.O && yb != kOobOffset ? yb + static_cast<uint32_t>(o) * plane : kOobOffset, 0, 0);
+                for (int gq = 0; gq < 4; ++gq) {
+                    const int cg = ch0 + 32 * i + 8 * gq;              // uniform; its channels are cg .. cg + 7
+                    const uint32_t yv = cg + 8 <= a.O ? yb : kOobOffset;
+#pragma unroll
+                    for (int ge = 0; ge < 4; ++ge) {
+                        const int g = 4 * gq + ge;
+                        const float v = acc[i][j][g];
+                        const int bits = __builtin_bit_cast(int, v);
+                        float left = __builtin_bit_cast(float, __builtin_amdgcn_ds_bpermute(left_addr, bits));
+                        const float right = __builtin_bit_cast(float, __builtin_amdgcn_ds_bpermute(right_addr, bits));
+                        const float before = edge[edge_at(prev, i, g)];
+                        left = from_edge ? before : left;
+                        const float pooled = fmaxf(v, fmaxf(left, right));
+                        __builtin_amdgcn_raw_buffer_store_b32(__builtin_bit_cast(uint32_t, pooled), yr, yv,
+                                                              static_cast<uint32_t>(cg + ge) * plane, 0);
+                    }
                 }
         }
         return;
@@ -988,6 +1004,7 @@ bool HpoolChoice(const kxc_hip_conv2d_desc* desc, const ConvArgs& a, Choice* cho
     choice->v = nullptr;
     if (!(desc->flags & KXC_HIP_CONV_RELU) || (desc->flags & (KXC_HIP_CONV_RESIDUAL | KXC_HIP_CONV_FORCE_DIRECT))) return false;
     if (a.M <= 0 || a.OW < 2 || (a.OW & 1)) return false;
+    if (a.O % 8 != 0) return false;      // the epilogue masks absent channels eight at a time
     const int64_t x_bytes = static_cast<int64_t>(a.N) * a.C * a.H * a.W * 4;
     const int64_t y_elems = static_cast<int64_t>(a.N) * a.O * a.OHW;
     const int64_t w_bytes = static_cast<int64_t>(a.O) * a.C * desc->kh * desc->kw * 4;

@@ -212,8 +212,8 @@ int32_t kxc_hip_conv2d_pair_nchw_f32(const kxc_hip_conv2d_desc* desc, const floa
  * half the bytes of the unpooled map; kxc_hip_pool2d_f32 with a 3x1 window, stride (2,1) and padding (1,0,1,0)
  * finishes the pool.  Every value is a ReLU result (>= +0, never NaN), so the pooling pad candidate of the
  * reference never wins and the two-step maximum equals the 3x3 one bit for bit.
- *   ..._supported: 1 when a kernel with that epilogue covers the shape: KXC_HIP_CONV_RELU set, no residual, an even
- *   output width that divides the kernel's 224-pixel tile (7x7 filters: 112, 56, 32, 16 ...), n*oh*ow a multiple of 224.
+ *   ..._supported: 1 when a kernel with that epilogue covers the shape: KXC_HIP_CONV_RELU set, no residual, output
+ *   channels a multiple of 8, an even output width that divides the kernel's 224-pixel tile (7x7 filters: 112, 56, 32, 16 ...), n*oh*ow a multiple of 224.
  *   ..._preferred: ... and the library expects conv + column pool to beat conv + 3x3 pool (KXC_HIP_CONV_HPOOL=0/1 in
  *   the environment overrides the rule). */
 int32_t kxc_hip_conv2d_hpool_supported(const kxc_hip_conv2d_desc* desc);

@@ -847,6 +847,7 @@ def test_conv_column_maxima_refusals_and_full_batch(pkg, synth):
     assert not pkg.conv2d_hpool_supported((2, 3, 224, 224), w7, 2, 3, preferred=True)       # too few tiles to pay
     assert not pkg.conv2d_hpool_supported((1, 3, 64, 64), w7, 2, 3)                          # 1024 pixels: not whole tiles
     assert not pkg.conv2d_hpool_supported((2, 3, 222, 222), w7, 2, 3)                        # 111 columns: odd
+    assert not pkg.conv2d_hpool_supported((2, 3, 224, 224), (60, 3, 7, 7), 2, 3)             # channels are masked eight at a time
     assert not pkg.conv2d_hpool_supported((2, 64, 56, 56), (64, 64, 3, 3), 1, 1)             # no 3x3 kernel has it
     assert not pkg.conv2d_hpool_supported((2, 3, 224, 224), w7, 2, 3, flags=pkg.CONV_BIAS)   # needs the ReLU
     assert not pkg.conv2d_hpool_supported((2, 3, 224, 224), w7, 2, 3, flags=pkg.CONV_BIAS | pkg.CONV_RELU | pkg.CONV_RESIDUAL)
