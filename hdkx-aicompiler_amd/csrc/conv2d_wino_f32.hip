@@ -282,16 +282,19 @@ wino_kernel(const WinoArgs a) {
     //   half 0: t0 = d0 - d2 = e0 - e2,  t1 = d1 + d2 = e1 + e2
     //   half 1: t3 = d1 - d3 = e0 - e2,  t2 = d2 - d1 = e1 - e0
     // i.e. ta = e0 - e2 and tb = e1 + (half ? -e0 : e2): one select per column instead of both variants and two.
-    auto transform = [&](float* buf) {
+    // The half an item transforms is fixed for the whole kernel: with two items per thread item i is half i; with one, a
+    // wave's threads all work on the half `wave_half`, and the main loop below exists once per half (one branch in
+    // front of it), so that tb is one instruction per column instead of a select and an addition.
+    auto transform = [&](float* buf, auto half_c) {
 #pragma unroll
         for (int i = 0; i < ITEMS; ++i) {
-            const bool half = (tid + i * NTH) / (4 * TT) != 0;        // uniform over the wave
+            const bool half = ITEMS == 2 ? i == 1 : decltype(half_c)::value;
             float ta[4], tb[4];
 #pragma unroll
             for (int j = 0; j < 4; ++j) {
                 const float e0 = d[i][j], e1 = d[i][4 + j], e2 = d[i][8 + j];
                 ta[j] = e0 - e2;
-                tb[j] = e1 + (half ? -e0 : e2);
+                tb[j] = half ? e1 - e0 : e1 + e2;
             }
             floatx4 va, vb;
             va[0] = ta[0] - ta[2]; va[1] = ta[1] + ta[2]; va[2] = ta[2] - ta[1]; va[3] = ta[1] - ta[3];
@@ -342,7 +345,8 @@ wino_kernel(const WinoArgs a) {
                 bias4[kb][g] = load_f32(br, static_cast<uint32_t>((kg * WK + wave_k) * 32 + kb * 16 + 4 * (lane >> 4) + g) * 4u, 0);
     }
     __builtin_amdgcn_sched_barrier(0);
-    transform(vb0);
+    auto main_loop = [&](auto half_c) {
+    transform(vb0, half_c);
     load_raw(min(s_lo + 1, last));
     __builtin_amdgcn_sched_barrier(0);
     __syncthreads();
@@ -363,7 +367,7 @@ wino_kernel(const WinoArgs a) {
         __builtin_amdgcn_sched_barrier(0);
         fetch(ucur, vcur, 2, 0);
         __builtin_amdgcn_sched_barrier(0);
-        transform(vnxt);       // raw input of step s + 1, requested one step ago
+        transform(vnxt, half_c);       // raw input of step s + 1, requested one step ago
         __builtin_amdgcn_sched_barrier(0);
         mm(1, 1, first);
         __builtin_amdgcn_sched_barrier(0);
@@ -386,6 +390,9 @@ wino_kernel(const WinoArgs a) {
         const bool odd = ((s - s_lo) & 1) != 0;
         step(s, odd ? ub1 : ub0, odd ? vb1 : vb0, odd ? ub0 : ub1, odd ? vb0 : vb1, std::false_type{});
     }
+    };
+    if (ITEMS == 2 || __builtin_amdgcn_readfirstlane(tid / (4 * TT)) == 0) main_loop(std::false_type{});
+    else main_loop(std::true_type{});
     asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
 
     if (KS > 1) {
