@@ -386,9 +386,10 @@ wino_kernel(const WinoArgs a) {
         __syncthreads();
     };
     step(s_lo, ub0, vb0, ub1, vb1, std::true_type{});
-    for (int s = s_lo + 1; s < s_hi; ++s) {
-        const bool odd = ((s - s_lo) & 1) != 0;
-        step(s, odd ? ub1 : ub0, odd ? vb1 : vb0, odd ? ub0 : ub1, odd ? vb0 : vb1, std::false_type{});
+    // (two steps per trip, so that every call names its buffers: their per-lane addresses stay in registers)
+    for (int s = s_lo + 1; s < s_hi; s += 2) {
+        step(s, ub1, vb1, ub0, vb0, std::false_type{});
+        if (s + 1 < s_hi) step(s + 1, ub0, vb0, ub1, vb1, std::false_type{});
     }
     };
     if (ITEMS == 2 || __builtin_amdgcn_readfirstlane(tid / (4 * TT)) == 0) main_loop(std::false_type{});
