@@ -273,7 +273,10 @@ def main():
                     "matrix_core_frac": round(executed / (conv_ms * 1e-3) / 1e12 / PEAK_FP32_MFMA_TFLOPS, 4),
                     "traffic": _profiled_traffic_bytes("winograd_layer1_bs64_counters.md") if batch == 64 else None,
                     "traffic_unit": "bytes per launch (FETCH_SIZE + WRITE_SIZE, calibrated on a copy; from profiles/)",
-                    "algorithmic_bytes_per_launch": algorithmic_bytes, "same_layer_implicit_gemm": gemm_row}
+                    "algorithmic_bytes_per_launch": algorithmic_bytes, "same_layer_implicit_gemm": gemm_row,
+                    "accounting": "achieved and frac divide the OPERATOR's FLOP (2*N*O*OH*OW*C*9, every output computed) by the measured "
+                                  "time; Winograd F(2x2,3x3) executes 16/36 of those multiplies, so frac can reach or pass 1 while the "
+                                  "matrix cores run at matrix_core_frac of their peak"}
         if shares > 1 and batch % shares == 0:
             # what the plan does with this layer: one launch per share of the batch, side by side on streams of
             # their own between a fork and a join on the timed stream (variants chosen for `shares` equal launches)
